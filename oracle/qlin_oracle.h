@@ -1,0 +1,113 @@
+/*
+ * CPU oracle for the group-affine quantized-linear path -- TEST INFRASTRUCTURE ONLY.
+ *
+ * This is a plain-C restatement of the reference's (1amageek/swift-mlx-lm) packing,
+ * dequantization, GEMV/GEMM and argmax semantics.  It exists so that the HIP kernels can be
+ * checked against it.  Nothing in the shipped library links, loads or calls it; only the test
+ * suite, the smoke check and the benchmark's CPU-baseline leg may.
+ *
+ * Every function names the reference file:line it follows (paths relative to the reference
+ * checkout; MC/ = Sources/MetalCompiler/).
+ *
+ * Parity pinning status (what fixes each function besides its own formula):
+ *   orc_unpack_code            pinned: reference slot formulas + literal byte vectors + brute force
+ *   orc_pack_stream            pinned: literal byte vectors (0x76543210 -> 10 32 54 76), Q6 byte formulas
+ *   orc_repack_mlx_to_staf     pinned: byte-exact layout vectors from the reference's round-trip tests
+ *   orc_dequant_*              pinned: closed-form KATs with power-of-two scales (exact in fp32)
+ *   orc_gemm_f64 / *_ref_f32   pinned: closed-form KATs (192.0 / 320.0, integer dot products)
+ *   orc_bf16_from_f32          pinned: RNE rule + known bit patterns
+ *   orc_f16_from_f32           pinned: exhaustive round trip over all 65536 half patterns vs numpy
+ *   orc_argmax_lowest          PARITY UNPINNED against the reference (it holds no argmax value
+ *                              test); pinned only by brute force against numpy on tiny vectors
+ *   orc_quantize_affine        PARITY UNPINNED (the reference has no weight quantizer; this is an
+ *                              input generator, not part of the path under test)
+ */
+#ifndef QLIN_ORACLE_H
+#define QLIN_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* dtype tags for scale/bias planes and activations */
+enum { ORC_F16 = 0, ORC_BF16 = 1, ORC_F32 = 2 };
+
+typedef struct {
+    int32_t scheme;          /* STAF scheme identifier (MC/STAF/STAFFormat.swift:175-217) */
+    int32_t bits;
+    int32_t group;           /* weights per block == group size */
+    int32_t bytes_per_block; /* 4 + group*bits/8 */
+    int32_t in_reference;    /* 1 if registered by the reference, 0 for q6g64 / q2g64 */
+} orc_format;
+
+/* MC/STAF/QuantizationFormat.swift:1315-1335 (formatForMLXQuantization) + q6g64/q2g64. */
+int orc_format_for_mlx(int bits, int group, orc_format* out);
+/* MC/STAF/QuantizationFormat.swift:1284-1312 (format(for:)). */
+int orc_format_for_scheme(int scheme, orc_format* out);
+
+/* MC/BFloat16.swift:25-32, MC/STAF/STAFPayloadConverter.swift:116-121. */
+uint16_t orc_bf16_from_f32(float v);
+float orc_bf16_to_f32(uint16_t h);
+/* Swift Float16(Float): IEEE binary16 round-to-nearest-even. */
+uint16_t orc_f16_from_f32(float v);
+float orc_f16_to_f32(uint16_t h);
+
+/* MC/STAF/QuantizationFormat.swift:1060-1062,1087-1089,1121-1139,1172-1192,1221-1235,1254-1256 */
+uint32_t orc_unpack_code(const uint8_t* qs, int k, int bits);
+/* Closed form q_k = (stream >> k*bits) & mask over the LSB-first byte stream. */
+uint32_t orc_unpack_code_stream(const uint8_t* qs, size_t k, int bits);
+/* LSB-first bit-stream packer (Tests/MetalCompilerTests/Core/UnifiedGEMVBitLevelTests.swift:303-321). */
+void orc_pack_stream(const uint8_t* codes, size_t n, int bits, uint8_t* out);
+
+/* MC/STAF/STAFPayloadConverter.swift:209-282 (+ :326-368 scale normalisation). */
+int orc_repack_mlx_to_staf(int bits, int group, size_t n_rows, size_t packed_words_per_row,
+                           const uint32_t* codes, const void* scales, const void* biases,
+                           int sb_dtype, uint8_t* out_blocks);
+/* Inverse view: STAF blocks -> MLX planes (codes words, f16 scales, f16 biases). */
+int orc_staf_to_planes(int bits, int group, size_t n_rows, size_t k, const uint8_t* blocks,
+                       uint32_t* codes, uint16_t* scales_f16, uint16_t* biases_f16);
+
+/* Codes only (uint8 per weight), from either layout. */
+int orc_unpack_staf_codes(int bits, int group, size_t n_rows, size_t k, const uint8_t* blocks,
+                          uint8_t* out_codes);
+int orc_unpack_plane_codes(int bits, size_t n_rows, size_t k, const uint32_t* codes,
+                           uint8_t* out_codes);
+
+/* Sources/SwiftLM/CPUWeightStore.swift:141-172: w = scale*float(q) + zero, fp32, unfused. */
+int orc_dequant_staf_f32(int bits, int group, size_t n_rows, size_t k, const uint8_t* blocks,
+                         float* out);
+int orc_dequant_planes_f32(int bits, int group, size_t n_rows, size_t k, const uint32_t* codes,
+                           const void* scales, const void* biases, int sb_dtype, float* out);
+/* MC/Generator/MetalSourceGenerator+Quantized.swift:403-413: bfloat(scale*q+zero). */
+int orc_dequant_staf_bf16(int bits, int group, size_t n_rows, size_t k, const uint8_t* blocks,
+                          uint16_t* out);
+
+/* fp64 accumulation of given fp32 weights [N,K] against activations x [M, x_stride]. */
+void orc_gemm_f64(const float* w, const float* x, size_t m, size_t n, size_t k, size_t x_stride,
+                  double* y);
+
+/* Reference loop nest, fp32 accumulate (MC/Generator/MetalSourceGenerator+Quantized.swift:116-153,
+ * :539-573): for m, for row, for block, for k: sum += (scale*q+zero)*x.  Rows are split over
+ * `threads` pthreads.  Output y[m*N + row]. */
+int orc_qgemm_staf_ref_f32(int bits, int group, const uint8_t* blocks, const float* x, size_t m,
+                           size_t n, size_t k, size_t x_stride, float* y, int threads);
+int orc_qgemm_planes_ref_f32(int bits, int group, const uint32_t* codes, const void* scales,
+                             const void* biases, int sb_dtype, const float* x, size_t m, size_t n,
+                             size_t k, size_t x_stride, float* y, int threads);
+
+/* Strict '>' scan from index 0 (MC/Generator/MetalSourceGenerator+Sampling.swift:80-90):
+ * NaN never wins, ties keep the lowest index, empty / all-NaN input yields 0. */
+int32_t orc_argmax_lowest(const float* v, size_t n);
+
+/* Input generator: per-group affine quantizer (MC/STAF/README.md:102-103; rounding, clamp and
+ * 1e-10 floor as MC/Generator/MetalSourceGenerator+Quantized.swift:427-433). */
+int orc_quantize_affine(const float* w, size_t n_rows, size_t k, int bits, int group, int sb_dtype,
+                        uint32_t* codes, void* scales, void* biases);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
