@@ -1,0 +1,196 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-linear hot path on one MI355X.
+
+Workload (BASELINE config 1 at M=1): one decode pass over the seven 4-bit g64 projections of a
+Llama-3-8B layer (q, k, v, o, gate, up, down).  One "step" = those seven GEMV launches on one
+stream.  `--layers` distinct copies of the layer's weights (default 32, 3.9 GB) are resident in
+HBM and steps rotate through them, so every launch streams its weights from HBM rather than
+from the 256 MB last-level cache.  The headline value is weight bytes / time, the convention of
+the reference's own GB/s figure.
+
+Prints exactly one JSON line on stdout; progress and secondary figures go to stderr.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "tests")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBPS = 8000.0            # MI355X published HBM3E bandwidth
+LAYER_SHAPES = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
+                ("gate", 14336, 4096), ("up", 14336, 4096), ("down", 4096, 14336)]
+BITS, GROUP = 4, 64
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def weight_bytes(n, k, bits=BITS, group=GROUP):
+    return n * (k // group) * (4 + group * bits // 8)
+
+
+def time_region(ctx, fn, reps, stream=0):
+    """Average milliseconds per call of fn over `reps` calls, HIP events on the launch stream."""
+    e0, e1 = ctx.event_create(), ctx.event_create()
+    ctx.event_record(e0, stream)
+    for i in range(reps):
+        fn(i)
+    ctx.event_record(e1, stream)
+    ctx.event_synchronize(e1)
+    ms = ctx.event_elapsed_ms(e0, e1) / reps
+    ctx.event_destroy(e0); ctx.event_destroy(e1)
+    return ms
+
+
+def cpu_baseline(seconds: float):
+    """The reference's loop nest (row -> block -> k, fp32 accumulate) on the host cores, timed on
+    BASELINE config 0 (q4 g64, 2048 -> 8192, M=1) for a bounded number of passes."""
+    import kat
+    import oracle
+    n, k = 8192, 2048
+    words, s, z = oracle.quantize_affine(kat.seeded_weights(11, n, k), BITS, GROUP, oracle.BF16)
+    x = oracle.bf16_to_f32(oracle.bf16_from_f32(kat.seeded_activations(12, 1, k))).reshape(1, k)
+    cores = min(os.cpu_count() or 1, 16)
+    oracle.qgemm_planes_ref_f32(BITS, GROUP, words, s, z, oracle.BF16, x, n, k, threads=cores)  # warm-up
+    passes, t0 = 0, time.perf_counter()
+    while True:
+        oracle.qgemm_planes_ref_f32(BITS, GROUP, words, s, z, oracle.BF16, x, n, k, threads=cores)
+        passes += 1
+        dt = time.perf_counter() - t0
+        if dt >= seconds or passes >= 2000:
+            break
+    gbps = weight_bytes(n, k) * passes / dt / 1e9
+    return {"value": round(gbps, 4), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": f"{passes} passes of config 0 (q4 g64 2048->8192, M=1, 9437184 weight bytes each) "
+                      f"in {dt:.1f} s, rows split over {cores} pthreads"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=320)
+    ap.add_argument("--warmup", type=int, default=32)
+    ap.add_argument("--layers", type=int, default=32, help="distinct weight copies resident in HBM")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--skip-parity", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build runs on exactly one GPU (one process, one device); "
+                 f"--gpus {a.gpus} is not supported")
+
+    import kat
+    import oracle
+    from __graft_entry__ import load_package
+    pkg = load_package()
+    ctx = pkg.Context(0)
+    info = ctx.device_info()
+    log(f"device: {info.name.decode()} {info.arch.decode()} CUs={info.compute_units}")
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(BITS, GROUP)
+
+    # ---- synthetic layer: W ~ N(0, 0.02^2) quantised per group, bf16 scale/bias planes
+    host = {}
+    for i, (name, n, k) in enumerate(LAYER_SHAPES):
+        t0 = time.perf_counter()
+        words, s, z = oracle.quantize_affine(kat.seeded_weights(1000 + i, n, k), BITS, GROUP, oracle.BF16)
+        host[name] = (words, s, z)
+        log(f"  synthesised {name} {k}->{n} in {time.perf_counter() - t0:.1f}s")
+    xs = {k: oracle.bf16_to_f32(oracle.bf16_from_f32(kat.seeded_activations(77 + k, 1, k))).reshape(1, k)
+          for k in (4096, 14336)}
+    xdev = {k: ctx.upload(oracle.bf16_from_f32(v)) for k, v in xs.items()}
+    ydev = {name: ctx.alloc(n * 2) for name, n, _ in LAYER_SHAPES}
+
+    layers = []
+    for _ in range(a.layers):
+        layers.append({name: ctx.weight_prepare_mlx(fmt, *host[name], pkg.BF16, pkg.LAYOUT_PLANES)
+                       for name, _, _ in LAYER_SHAPES})
+    layer_bytes = sum(weight_bytes(n, k) for _, n, k in LAYER_SHAPES)
+    log(f"resident: {a.layers} layers x {layer_bytes} B = {a.layers * layer_bytes / 1e9:.2f} GB")
+
+    # ---- parity gate: no number is reported from a run whose outputs were not verified
+    if not a.skip_parity:
+        for name, n, k in LAYER_SHAPES:
+            words, s, z = host[name]
+            wq = oracle.dequant_planes_f32(BITS, GROUP, n, k, words, s, z, oracle.BF16)
+            want = oracle.gemm_f64(wq, xs[k])[0]
+            y32 = ctx.alloc(n * 4)
+            ctx.qgemv(layers[-1][name], xdev[k], pkg.BF16, y32, pkg.F32, 1)
+            ctx.synchronize()
+            got = y32.download(np.float32)
+            rel = float(np.linalg.norm(got - want) / np.linalg.norm(want))
+            mx = float(np.max(np.abs(got - want)))
+            y32.free()
+            if not (rel <= 1e-3 and mx <= 2e-2):
+                sys.exit(f"bench.py: parity gate failed on {name}: rel-L2 {rel:.3e} max-abs {mx:.3e}")
+            log(f"  parity {name}: rel-L2 {rel:.2e} max-abs {mx:.2e}")
+
+    stream = ctx.stream_create()
+
+    def step(i):
+        L = layers[i % a.layers]
+        for name, n, k in LAYER_SHAPES:
+            ctx.qgemv(L[name], xdev[k], pkg.BF16, ydev[name], pkg.BF16, 1, 0, 0, 0, stream)
+
+    for i in range(a.warmup):
+        step(i)
+    ctx.synchronize(stream)
+    ms_step = time_region(ctx, step, a.steps, stream)
+    ctx.synchronize(stream)
+    value = layer_bytes / (ms_step * 1e-3) / 1e9
+
+    # ---- dominant kernel (gate/up 4096 -> 14336): average launch duration over rotating copies
+    per_shape = {}
+    for name, n, k in [("gate", 14336, 4096), ("down", 4096, 14336), ("q", 4096, 4096), ("k", 1024, 4096)]:
+        def one(i, name=name, k=k):
+            ctx.qgemv(layers[i % a.layers][name], xdev[k], pkg.BF16, ydev[name], pkg.BF16, 1, 0, 0, 0, stream)
+        for i in range(a.layers):
+            one(i)
+        ctx.synchronize(stream)
+        ms = time_region(ctx, one, max(a.steps, 4 * a.layers), stream)
+        per_shape[name] = {"us": round(ms * 1e3, 3), "GBps": round(weight_bytes(n, k) / (ms * 1e-3) / 1e9, 1)}
+        log(f"  {name:5s} {k}->{n}: {ms * 1e3:.2f} us/launch, {per_shape[name]['GBps']} GB/s")
+    gate_ms = per_shape["gate"]["us"] * 1e-3
+    achieved = weight_bytes(14336, 4096) / (gate_ms * 1e-3) / 1e9
+
+    cpu = None if a.no_cpu else cpu_baseline(a.cpu_seconds)
+
+    out = {
+        "metric": "4-bit decode GEMV GB/s (weight bytes / time, M=1)",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": round(ms_step, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16 activations x u4 codes, fp32 accumulate",
+        "data": "synthetic: W~N(0,0.02^2) quantised q4 g64 (bf16 scale/bias planes), x~N(0,1) bf16, seeded; "
+                f"{a.layers} resident copies of one layer's tensors",
+        "config": {"workload": "Llama-3-8B decode layer sweep (BASELINE config 1), M=1: q,k,v,o,gate,up,down "
+                               "GEMVs per step", "bits": BITS, "group_size": GROUP,
+                   "weight_bytes_per_step": layer_bytes, "layers_resident": a.layers,
+                   "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2), "per_shape": per_shape},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "gemv_planes_kernel<4,64> on gate/up 4096->14336 (33030144 weight bytes/launch)"},
+    }
+    if cpu is not None:
+        out["cpu_baseline"] = cpu
+    print(json.dumps(out), flush=True)
+    ctx.close()
+
+
+if __name__ == "__main__":
+    main()

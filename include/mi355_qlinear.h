@@ -1,0 +1,367 @@
+/*
+ * mi355_qlinear.h -- C ABI of the MI355X (gfx950) group-affine quantized-linear library.
+ *
+ * One shared library (libmi355_qlinear.so) replaces the quantized-linear hot path that
+ * swift-lm's MetalCompiler emits as generated Metal kernels over STAF-packed weights:
+ * decode GEMV, prefill GEMM, dequant-to-bf16, LM head + argmax.  The reference has no FFI;
+ * its "plugin API" is the Swift value-type contract between planner and encoder.  Each entry
+ * point below names the reference interface it stands in for (paths relative to the reference
+ * checkout, MC/ = Sources/MetalCompiler/).
+ *
+ * Conventions
+ *   - Every call returns mi355q_status (0 = ok, negative = error).  No exception or unwinding
+ *     crosses this boundary.  mi355q_last_error() returns the message of the last failing call
+ *     on the calling thread.
+ *   - Pointers named *_dev are device pointers (HBM) valid on the context's GPU; *_host are host
+ *     pointers.  Device pointers may come from mi355q_buffer_alloc or from any other HIP
+ *     allocator in the same process (a torch tensor's data_ptr, hipMalloc, ...).
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).  Launch calls are
+ *     asynchronous: they validate, enqueue and return.
+ *   - A context is thread-compatible, not thread-safe: callers serialise calls per context, as
+ *     the reference serialises per MetalSubmissionContext
+ *     (MC/Execution/MetalSubmissionContext.swift:56-120).
+ *   - Shapes follow the reference: a weight is [N = outputDimension, K = inputDimension];
+ *     K % groupSize == 0 is required (MC/Generator/MetalSourceGenerator+Quantized.swift:547);
+ *     activations are [M = sequenceLength, x_row_stride >= K] in elements; outputs are [M, N].
+ *   - There is no CPU fallback anywhere.  If no GPU is usable the context cannot be created and
+ *     every compute entry point fails with MI355Q_ERR_DEVICE.
+ */
+#ifndef MI355_QLINEAR_H
+#define MI355_QLINEAR_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355Q_API __attribute__((visibility("default")))
+#define MI355Q_ABI_VERSION 1
+
+typedef int32_t mi355q_status;
+enum {
+    MI355Q_OK = 0,
+    MI355Q_ERR_INVALID_ARGUMENT = -1,   /* precondition / fatalError in the reference */
+    MI355Q_ERR_UNSUPPORTED_FORMAT = -2, /* STAFConversionError.unsupportedQuantization
+                                           (MC/STAF/STAFConversionPlanner.swift:179-187) */
+    MI355Q_ERR_SHAPE = -3,              /* STAFConversionError.inconsistentQuantizationShape
+                                           (MC/STAF/STAFPayloadConverter.swift:238-243) */
+    MI355Q_ERR_NULL_HANDLE = -4,
+    MI355Q_ERR_DEVICE = -5,             /* MetalCompilerError.deviceSetupFailed */
+    MI355Q_ERR_OUT_OF_MEMORY = -6,
+    MI355Q_ERR_KERNEL_NOT_FOUND = -7,   /* MetalCompilerError.kernelNotFound */
+    MI355Q_ERR_SIZE_MISMATCH = -8       /* payload size != rows*blocksPerRow*bytesPerBlock
+                                           (Sources/SwiftLM/CPUWeightStore.swift:133-138) */
+};
+
+/* BufferPrecision (MC/MetalDispatchTypes.swift:13-37) */
+typedef enum { MI355Q_F16 = 0, MI355Q_BF16 = 1, MI355Q_F32 = 2 } mi355q_dtype;
+
+/* STAFWeightLayout (MC/STAF/STAFWeightAccessRequest.swift:3-7): the canonical row-major STAF
+ * interleaved blocks, or this library's specialized layout (split planes: uint32 code words
+ * [N, K*bits/32] + scales [N, K/g] + biases [N, K/g], i.e. the MLX source planes). */
+typedef enum { MI355Q_LAYOUT_STAF_BLOCKS = 0, MI355Q_LAYOUT_PLANES = 1 } mi355q_layout;
+
+/* Launch flags */
+enum {
+    MI355Q_FLAG_NONE = 0,
+    MI355Q_FLAG_FORCE_GENERIC = 1, /* run the reference-shaped per-code kernel (A/B and tests) */
+    MI355Q_FLAG_FORCE_SMALL_M = 2, /* qgemm: use the small-M GEMV-style kernel whatever M is */
+    MI355Q_FLAG_FORCE_MFMA = 4     /* qgemm: use the MFMA kernel whatever M is */
+};
+
+/* ------------------------------------------------------------------------------------------
+ * Format descriptor: QuantizationFormat protocol (MC/STAF/QuantizationFormat.swift:25-153)
+ * ---------------------------------------------------------------------------------------- */
+typedef struct {
+    uint8_t scheme_identifier;   /* QuantizationSchemeIdentifier (MC/STAF/STAFFormat.swift:175-217) */
+    uint8_t bits;
+    uint8_t is_quantized;
+    uint8_t is_aligned;          /* bits in {2,4,8,16,32} (QuantizationFormat.swift:161-166) */
+    uint32_t group_size;
+    uint32_t weights_per_block;
+    uint32_t bytes_per_block;    /* 4 + group*bits/8 */
+    uint8_t has_direct_gemm;     /* directGEMMKernel() != nil (q4g64,q4g128,q8g32,q8g64) */
+    uint8_t batched_gemm_counts; /* bit c set <=> batchedGEMMKernel(count: c) != nil */
+    uint8_t in_reference_registry; /* 0 for q6g64 / q2g64 (new scheme ids 0x22 / 0x62) */
+    uint8_t reserved0;
+    uint32_t direct_gemm_threadgroup_memory_length; /* max(2g,256)*4 (QuantizationFormat.swift:364-367) */
+    char block_struct_name[32];
+    char gemv_kernel_name[32];          /* "gemv_q4_g64" */
+    char gemm_kernel_name_f32s[32];     /* gemmKernelName(.float32) */
+    char gemm_kernel_name[32];          /* gemmKernelName(decode precision) */
+    char dequant_to_bfloat_kernel_name[32]; /* "dequant_q4_g64_bf16" */
+    char embedding_lookup_token[16];    /* "q4_g64" */
+} mi355q_format;
+
+/* QuantizationFormatRegistry.formatForMLXQuantization(bits:groupSize:)
+ * (QuantizationFormat.swift:1315-1335).  Unknown pair -> MI355Q_ERR_UNSUPPORTED_FORMAT; there
+ * is no silent default (MC/Generator/MetalKernelSourceCatalog.swift:14). */
+MI355Q_API mi355q_status mi355q_format_for_mlx_quantization(int bits, int group_size,
+                                                            mi355q_format* out);
+/* QuantizationFormatRegistry.format(for:) (QuantizationFormat.swift:1284-1312); 0x42 aliases
+ * q4g128.  Dense and rotor schemes are outside this path -> MI355Q_ERR_UNSUPPORTED_FORMAT. */
+MI355Q_API mi355q_status mi355q_format_for_scheme(uint8_t scheme_identifier, mi355q_format* out);
+/* Enumerate the registry (CaseIterable analogue) for contract tests. */
+MI355Q_API int32_t mi355q_format_count(void);
+MI355Q_API mi355q_status mi355q_format_at(int32_t index, mi355q_format* out);
+
+/* bf16 round-to-nearest-even of the host type (MC/BFloat16.swift:25-32). */
+MI355Q_API uint16_t mi355q_bf16_from_f32(float value);
+
+/* STAFPayloadConverter.repackMLXQuantized (MC/STAF/STAFPayloadConverter.swift:209-282) on host
+ * memory: MLX planes -> STAF interleaved blocks, scales/biases normalised to f16 (:326-368).
+ * out_capacity must be >= n_rows * (K/group) * bytes_per_block. */
+MI355Q_API mi355q_status mi355q_repack_mlx_to_staf(uint8_t scheme_identifier, size_t n_rows,
+                                                   size_t packed_words_per_row,
+                                                   const uint32_t* codes_host,
+                                                   const void* scales_host,
+                                                   const void* biases_host, mi355q_dtype sb_dtype,
+                                                   uint8_t* out_blocks_host, size_t out_capacity);
+
+/* ------------------------------------------------------------------------------------------
+ * Context, memory, streams, events  (MTLDevice / MTLBuffer / MTLCommandQueue stand-ins)
+ * ---------------------------------------------------------------------------------------- */
+typedef struct mi355q_context mi355q_context;
+typedef struct mi355q_weight mi355q_weight;
+
+typedef struct {
+    char name[64];
+    char arch[32];              /* "gfx950..." */
+    int32_t compute_units;
+    int32_t wavefront_size;
+    int32_t lds_bytes_per_workgroup;
+    int32_t reserved0;
+    uint64_t hbm_bytes;
+    double hbm_peak_gbps;       /* published: 8000 */
+    double mfma_bf16_peak_tflops; /* published dense: 2500 */
+} mi355q_device_info;
+
+MI355Q_API const char* mi355q_last_error(void);
+MI355Q_API int32_t mi355q_abi_version(void);
+/* MTLCreateSystemDefaultDevice analogue.  Fails with MI355Q_ERR_DEVICE when there is no GPU. */
+MI355Q_API mi355q_status mi355q_context_create(int device_index, mi355q_context** out);
+MI355Q_API mi355q_status mi355q_context_destroy(mi355q_context* ctx);
+MI355Q_API mi355q_status mi355q_device_query(mi355q_context* ctx, mi355q_device_info* out);
+
+MI355Q_API mi355q_status mi355q_buffer_alloc(mi355q_context* ctx, size_t bytes, void** out_dev);
+MI355Q_API mi355q_status mi355q_buffer_free(mi355q_context* ctx, void* dev);
+MI355Q_API mi355q_status mi355q_buffer_upload(mi355q_context* ctx, void* dst_dev,
+                                              const void* src_host, size_t bytes);
+MI355Q_API mi355q_status mi355q_buffer_download(mi355q_context* ctx, void* dst_host,
+                                                const void* src_dev, size_t bytes);
+MI355Q_API mi355q_status mi355q_buffer_fill(mi355q_context* ctx, void* stream, void* dst_dev,
+                                            uint32_t word, size_t n_words);
+
+MI355Q_API mi355q_status mi355q_stream_create(mi355q_context* ctx, void** out_stream);
+MI355Q_API mi355q_status mi355q_stream_destroy(mi355q_context* ctx, void* stream);
+MI355Q_API mi355q_status mi355q_stream_synchronize(mi355q_context* ctx, void* stream);
+MI355Q_API mi355q_status mi355q_event_create(mi355q_context* ctx, void** out_event);
+MI355Q_API mi355q_status mi355q_event_destroy(mi355q_context* ctx, void* event);
+MI355Q_API mi355q_status mi355q_event_record(mi355q_context* ctx, void* event, void* stream);
+MI355Q_API mi355q_status mi355q_event_synchronize(mi355q_context* ctx, void* event);
+MI355Q_API mi355q_status mi355q_event_elapsed_ms(mi355q_context* ctx, void* start, void* stop,
+                                                 float* out_ms);
+
+/* ------------------------------------------------------------------------------------------
+ * Packed weights: STAFWeightStore.resolvedBufferAccess / registeringSpecializedBufferAccess
+ * (MC/STAF/STAFLoader.swift:213-299) and STAFSpecializedWeightStoreBuilder.prepare
+ * (MC/STAF/STAFSpecializedWeightStoreBuilder.swift:15-31).  A handle is immutable after
+ * creation.  "prepare" handles own their device memory; "wrap" handles borrow it.
+ * ---------------------------------------------------------------------------------------- */
+typedef struct {
+    uint8_t scheme_identifier;
+    uint8_t bits;
+    uint8_t layout;             /* mi355q_layout */
+    uint8_t sb_dtype;           /* dtype of scale/bias: F16 for STAF blocks, F16/BF16 for planes */
+    uint32_t group_size;
+    uint64_t n_rows;            /* N */
+    uint64_t k;                 /* K */
+    uint64_t weight_bytes;      /* algorithmic: N*(K/g)*bytes_per_block
+                                   (MC/Compiler/MetalCompilerDiagnostics.swift:192-203) */
+    const void* blocks_dev;     /* STAF layout */
+    const void* codes_dev;      /* planes layout */
+    const void* scales_dev;
+    const void* biases_dev;
+    uint8_t owns_memory;
+    uint8_t reserved[7];
+} mi355q_weight_info;
+
+/* From MLX source planes in host memory (uint32 [N, K*bits/32]; scales/biases [N, K/g] in
+ * sb_dtype; F32 scales are normalised to F16 as the converter does).  `layout` picks the
+ * device layout; STAF_BLOCKS repacks on the host first (the reference's load path). */
+MI355Q_API mi355q_status mi355q_weight_prepare_mlx(mi355q_context* ctx, uint8_t scheme_identifier,
+                                                   uint64_t n_rows, uint64_t k,
+                                                   const uint32_t* codes_host,
+                                                   const void* scales_host,
+                                                   const void* biases_host, mi355q_dtype sb_dtype,
+                                                   mi355q_layout layout, mi355q_weight** out);
+/* From STAF interleaved blocks in host memory (a mapped model.staf payload).  payload_bytes
+ * must equal N*(K/g)*bytes_per_block.  layout = PLANES de-interleaves once, at load time. */
+MI355Q_API mi355q_status mi355q_weight_prepare_staf(mi355q_context* ctx, uint8_t scheme_identifier,
+                                                    uint64_t n_rows, uint64_t k,
+                                                    const uint8_t* blocks_host,
+                                                    size_t payload_bytes, mi355q_layout layout,
+                                                    mi355q_weight** out);
+/* Zero-copy: borrow device memory that already holds the payload -- the (buffer, offset) pair
+ * of STAFWeightBufferAccess.  The caller keeps the memory alive and unchanged. */
+MI355Q_API mi355q_status mi355q_weight_wrap_staf(mi355q_context* ctx, uint8_t scheme_identifier,
+                                                 uint64_t n_rows, uint64_t k,
+                                                 const void* blocks_dev, size_t payload_bytes,
+                                                 mi355q_weight** out);
+MI355Q_API mi355q_status mi355q_weight_wrap_planes(mi355q_context* ctx, uint8_t scheme_identifier,
+                                                   uint64_t n_rows, uint64_t k,
+                                                   const void* codes_dev, const void* scales_dev,
+                                                   const void* biases_dev, mi355q_dtype sb_dtype,
+                                                   mi355q_weight** out);
+MI355Q_API mi355q_status mi355q_weight_query(const mi355q_weight* w, mi355q_weight_info* out);
+MI355Q_API mi355q_status mi355q_weight_destroy(mi355q_weight* w);
+
+/* ------------------------------------------------------------------------------------------
+ * Launches
+ * ---------------------------------------------------------------------------------------- */
+
+/* Decode projection: gemv_q{b}_g{g} (generateUnifiedQuantizedGEMV,
+ * MC/Generator/MetalSourceGenerator+Quantized.swift:496-575; bindings 0=input 1=weight
+ * 2=output 3=inputDimension 4=outputDimension, MC/Compiler/MetalDispatchStepBuilder.swift:679-688)
+ * widened to the sequence signature for small M (5=sequenceLength 6=inputRowStride,
+ * :116-153).  y[m*y_row_stride + n] = sum_k (scale*q + zero) * x[m*x_row_stride + k], fp32
+ * accumulation, result rounded once to y_dtype.  1 <= M <= 8.  y_row_stride 0 means N. */
+MI355Q_API mi355q_status mi355q_qgemv(mi355q_context* ctx, void* stream, const mi355q_weight* w,
+                                      const void* x_dev, mi355q_dtype x_dtype, void* y_dev,
+                                      mi355q_dtype y_dtype, uint32_t m, uint32_t x_row_stride,
+                                      uint32_t y_row_stride, uint32_t flags);
+
+/* Prefill projection: gemm_q4_g64_f32s / gemm_q8_g32_f32s (:22-156) and the two-step
+ * dequant_q*_bf16 + gemm_bf16_f32s path (:361-416, MC/Generator/MetalSourceGenerator+Linear.swift:18-81)
+ * as ONE fused kernel: code tiles are dequantised to bf16 in LDS and contracted on MFMA with
+ * fp32 accumulation.  Any M >= 1; M is a run-time value (the reference rebinds sequenceLength
+ * per call, MC/Compiler/MetalPrefillStepBuilder.swift:728-732).  Small M routes to the
+ * GEMV-style kernel unless flags say otherwise. */
+MI355Q_API mi355q_status mi355q_qgemm(mi355q_context* ctx, void* stream, const mi355q_weight* w,
+                                      const void* x_dev, mi355q_dtype x_dtype, void* y_dev,
+                                      mi355q_dtype y_dtype, uint32_t m, uint32_t x_row_stride,
+                                      uint32_t y_row_stride, uint32_t flags);
+
+/* batched_gemm_q4_g64_{2,3} (:166-338; bindings MC/Compiler/MetalPrefillStepBuilder.swift:928-955):
+ * 2 or 3 projections sharing one input (gate+up, q+k+v) in one launch.  All weights must share
+ * K, scheme and layout.  Outputs are separate [M, N_i] buffers with row stride N_i. */
+MI355Q_API mi355q_status mi355q_batched_qgemm(mi355q_context* ctx, void* stream, uint32_t count,
+                                              const mi355q_weight* const* weights,
+                                              const void* x_dev, mi355q_dtype x_dtype,
+                                              void* const* y_devs, mi355q_dtype y_dtype,
+                                              uint32_t m, uint32_t x_row_stride, uint32_t flags);
+
+/* dequant_q{b}_g{g}_bf16 (generateUnifiedDequantToBFloat, :361-416): whole matrix to row-major
+ * bf16 [N, K], each weight bf16_rne(scale*q + zero). */
+MI355Q_API mi355q_status mi355q_dequant_bf16(mi355q_context* ctx, void* stream,
+                                             const mi355q_weight* w, void* out_bf16_dev);
+
+/* gemm_bf16_f32s (generateMPPGEMM, MC/Generator/MetalSourceGenerator+Linear.swift:18-81):
+ * C[M,N] = A[M, a_row_stride>=K] * B[N,K]^T with B dense bf16 (the dequant scratch), MFMA,
+ * fp32 accumulation. */
+MI355Q_API mi355q_status mi355q_gemm_bf16(mi355q_context* ctx, void* stream, const void* a_dev,
+                                          mi355q_dtype a_dtype, const void* b_bf16_dev,
+                                          void* c_dev, mi355q_dtype c_dtype, uint32_t m,
+                                          uint32_t n, uint32_t k, uint32_t a_row_stride,
+                                          uint32_t c_row_stride);
+
+/* Debug / parity: every code of the matrix as one byte, row-major [N, K]. */
+MI355Q_API mi355q_status mi355q_unpack_codes(mi355q_context* ctx, void* stream,
+                                             const mi355q_weight* w, uint8_t* out_codes_dev);
+
+/* argmax / argmax_f32 (generateArgmax, MC/Generator/MetalSourceGenerator+Sampling.swift:62-107;
+ * bindings 0=logits 1=int* result 2=vocabularySize).  Strict '>' from -inf with index 0 as
+ * the start value: NaN never wins; ties resolve to the LOWEST index (a rule this library adds:
+ * the reference's reduction order does not define ties). */
+MI355Q_API mi355q_status mi355q_argmax(mi355q_context* ctx, void* stream, const void* logits_dev,
+                                       mi355q_dtype dtype, uint32_t vocabulary_size,
+                                       int32_t* token_out_dev);
+
+/* OutputHeadFragment = LinearFragment + ArgmaxFragment (MC/Compilable/OutputHeadFragment.swift:5-8)
+ * fused into one launch: fp32 logits [N] (optional, may be NULL) and the greedy token index.
+ * M = 1 (the reference runs the head in lastToken mode, MC/Compiler/MetalPrefillStepBuilder.swift:493-507). */
+MI355Q_API mi355q_status mi355q_lmhead_argmax(mi355q_context* ctx, void* stream,
+                                              const mi355q_weight* w, const void* x_dev,
+                                              mi355q_dtype x_dtype, float* logits_f32_dev,
+                                              int32_t* token_out_dev, uint32_t flags);
+
+/* ------------------------------------------------------------------------------------------
+ * Planner mirror: launch shapes, kernel selection and the quantization-plan record
+ * ---------------------------------------------------------------------------------------- */
+
+/* DecodeProjectionShapeFamily (MC/Compiler/MetalCompileContext.swift:5-90) */
+typedef enum {
+    MI355Q_FAMILY_GENERIC = 0,
+    MI355Q_FAMILY_LARGE_DENSE = 1,
+    MI355Q_FAMILY_INPUT2048_SQUARE = 2,
+    MI355Q_FAMILY_INPUT2048_6144 = 3,
+    MI355Q_FAMILY_INPUT2048_8192 = 4,
+    MI355Q_FAMILY_INPUT2048_EXPANDED = 5,
+    MI355Q_FAMILY_INPUT8192_TILED = 6,
+    MI355Q_FAMILY_VOCAB_DENSE = 7
+} mi355q_shape_family;
+
+/* MetalQuantizationExecutionPath / FallbackReason (MC/Compiler/MetalQuantizationPlan.swift:22-27,290-298) */
+typedef enum {
+    MI355Q_PATH_PREFILL_PROJECTION = 0,
+    MI355Q_PATH_DECODE_PROJECTION = 1
+} mi355q_execution_path;
+typedef enum {
+    MI355Q_FALLBACK_NONE = 0,
+    MI355Q_FALLBACK_INPUT_STRIDE_MISMATCH = 1,
+    MI355Q_FALLBACK_LAST_TOKEN_USES_DECODE_KERNEL = 2,
+    MI355Q_FALLBACK_DISABLED_BY_ENVIRONMENT = 3,
+    MI355Q_FALLBACK_UNAVAILABLE_ACCELERATION = 4
+} mi355q_fallback_reason;
+
+/* One planned dispatch: MetalDispatchStep / MetalPrefillStep reduced to what a HIP launch
+ * needs (MC/Execution/MetalDecodePlan.swift:6-97, MC/Execution/MetalPrefillPlan.swift:6-140)
+ * together with its MetalQuantizationPlanEntry (MC/Compiler/MetalQuantizationPlan.swift:304-318). */
+typedef struct {
+    char kernel_name[48];        /* reference-compatible name, e.g. "gemv_q4_g64" */
+    char device_kernel[48];      /* the HIP kernel variant that will run */
+    char kernel_family[32];      /* MetalQuantizationKernelFamily.description */
+    uint32_t grid[3];            /* workgroups */
+    uint32_t block[3];           /* threads per workgroup */
+    uint32_t lds_bytes;
+    uint32_t rows_per_workgroup;
+    uint32_t reference_simdgroups;   /* DecodeProjectionShapeFamily.preferredSimdgroups */
+    uint32_t reference_tile_elements;
+    int32_t shape_family;        /* mi355q_shape_family */
+    int32_t path;                /* mi355q_execution_path */
+    uint8_t scheme_identifier;
+    uint8_t layout;
+    uint8_t used_fallback;
+    uint8_t fallback_reason;     /* mi355q_fallback_reason */
+    uint32_t input_dimension;    /* binding 3 */
+    uint32_t output_dimension;   /* binding 4 */
+    uint32_t sequence_length;    /* binding 5 (planned maximum) */
+    uint32_t input_row_stride;   /* binding 6 */
+    uint64_t weight_bytes;       /* blocks * bytesPerBlock */
+    uint64_t flops;              /* 2*M*K*N */
+} mi355q_step;
+
+MI355Q_API mi355q_status mi355q_shape_family_resolve(uint32_t output_dimension,
+                                                     uint32_t input_dimension,
+                                                     int32_t* out_family,
+                                                     uint32_t* out_simdgroups,
+                                                     uint32_t* out_tile_elements,
+                                                     char* out_kernel_base_name, size_t name_cap);
+/* MetalDispatchStepBuilder (decode) for one LinearFragment. */
+MI355Q_API mi355q_status mi355q_plan_decode_step(const mi355q_weight* w, uint32_t m,
+                                                 mi355q_dtype x_dtype, uint32_t flags,
+                                                 mi355q_step* out);
+/* MetalPrefillStepBuilder.buildSteps(LinearFragment): writes 1 or 2 steps (dequant + GEMM when
+ * the two-step path is selected).  `is_last_token` mirrors mode = .lastToken. */
+MI355Q_API mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w,
+                                                   uint32_t maximum_sequence_length,
+                                                   uint32_t input_row_stride, mi355q_dtype x_dtype,
+                                                   int is_last_token, uint32_t flags,
+                                                   mi355q_step* out_steps, uint32_t* out_count);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_QLINEAR_H */

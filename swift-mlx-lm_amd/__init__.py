@@ -1,0 +1,485 @@
+"""Host-side mirror (Python/ctypes) of the quantized-linear interface over libmi355_qlinear.so.
+
+The names follow the reference's planner/encoder contract (QuantizationFormat,
+QuantizationFormatRegistry, STAFWeightLayout, dispatch steps, quantization-plan entries); the
+arithmetic all happens in the HIP library.  There is no CPU fallback: loading fails loudly when
+the shared library is missing, and creating a ``Context`` fails when there is no MI355X.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from dataclasses import dataclass
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libmi355_qlinear.so")
+
+# BufferPrecision
+F16, BF16, F32 = 0, 1, 2
+# STAFWeightLayout
+LAYOUT_STAF_BLOCKS, LAYOUT_PLANES = 0, 1
+# launch flags
+FLAG_NONE, FLAG_FORCE_GENERIC, FLAG_FORCE_SMALL_M, FLAG_FORCE_MFMA = 0, 1, 2, 4
+
+STATUS_NAMES = {0: "OK", -1: "INVALID_ARGUMENT", -2: "UNSUPPORTED_FORMAT", -3: "SHAPE", -4: "NULL_HANDLE",
+                -5: "DEVICE", -6: "OUT_OF_MEMORY", -7: "KERNEL_NOT_FOUND", -8: "SIZE_MISMATCH"}
+FALLBACK_NAMES = {0: None, 1: "inputStrideMismatch", 2: "lastTokenProjectionUsesDecodeKernel",
+                  3: "disabledByEnvironment", 4: "unavailableAcceleration"}
+PATH_NAMES = {0: "prefillProjection", 1: "decodeProjection"}
+FAMILY_NAMES = {0: "generic", 1: "largeDense", 2: "input2048SquareDense", 3: "input20486144Dense",
+                4: "input20488192Dense", 5: "input2048ExpandedDense", 6: "input8192Tiled", 7: "vocabDense"}
+
+
+class MI355QError(RuntimeError):
+    def __init__(self, status: int, message: str):
+        super().__init__(f"[{STATUS_NAMES.get(status, status)}] {message}")
+        self.status = status
+        self.status_name = STATUS_NAMES.get(status, str(status))
+
+
+class _Format(C.Structure):
+    _fields_ = [("scheme_identifier", C.c_uint8), ("bits", C.c_uint8), ("is_quantized", C.c_uint8),
+                ("is_aligned", C.c_uint8), ("group_size", C.c_uint32), ("weights_per_block", C.c_uint32),
+                ("bytes_per_block", C.c_uint32), ("has_direct_gemm", C.c_uint8),
+                ("batched_gemm_counts", C.c_uint8), ("in_reference_registry", C.c_uint8),
+                ("reserved0", C.c_uint8), ("direct_gemm_threadgroup_memory_length", C.c_uint32),
+                ("block_struct_name", C.c_char * 32), ("gemv_kernel_name", C.c_char * 32),
+                ("gemm_kernel_name_f32s", C.c_char * 32), ("gemm_kernel_name", C.c_char * 32),
+                ("dequant_to_bfloat_kernel_name", C.c_char * 32), ("embedding_lookup_token", C.c_char * 16)]
+
+
+class _DeviceInfo(C.Structure):
+    _fields_ = [("name", C.c_char * 64), ("arch", C.c_char * 32), ("compute_units", C.c_int32),
+                ("wavefront_size", C.c_int32), ("lds_bytes_per_workgroup", C.c_int32), ("reserved0", C.c_int32),
+                ("hbm_bytes", C.c_uint64), ("hbm_peak_gbps", C.c_double), ("mfma_bf16_peak_tflops", C.c_double)]
+
+
+class _WeightInfo(C.Structure):
+    _fields_ = [("scheme_identifier", C.c_uint8), ("bits", C.c_uint8), ("layout", C.c_uint8),
+                ("sb_dtype", C.c_uint8), ("group_size", C.c_uint32), ("n_rows", C.c_uint64), ("k", C.c_uint64),
+                ("weight_bytes", C.c_uint64), ("blocks_dev", C.c_void_p), ("codes_dev", C.c_void_p),
+                ("scales_dev", C.c_void_p), ("biases_dev", C.c_void_p), ("owns_memory", C.c_uint8),
+                ("reserved", C.c_uint8 * 7)]
+
+
+class _Step(C.Structure):
+    _fields_ = [("kernel_name", C.c_char * 48), ("device_kernel", C.c_char * 48), ("kernel_family", C.c_char * 32),
+                ("grid", C.c_uint32 * 3), ("block", C.c_uint32 * 3), ("lds_bytes", C.c_uint32),
+                ("rows_per_workgroup", C.c_uint32), ("reference_simdgroups", C.c_uint32),
+                ("reference_tile_elements", C.c_uint32), ("shape_family", C.c_int32), ("path", C.c_int32),
+                ("scheme_identifier", C.c_uint8), ("layout", C.c_uint8), ("used_fallback", C.c_uint8),
+                ("fallback_reason", C.c_uint8), ("input_dimension", C.c_uint32), ("output_dimension", C.c_uint32),
+                ("sequence_length", C.c_uint32), ("input_row_stride", C.c_uint32), ("weight_bytes", C.c_uint64),
+                ("flops", C.c_uint64)]
+
+
+_lib = None
+
+
+def library() -> C.CDLL:
+    """Load the HIP shared library; raise (never fall back) when it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(f"{LIB_PATH} is missing: build it with `python swift-mlx-lm_amd/build.py` "
+                          "(there is no CPU implementation to fall back to)")
+    L = C.CDLL(LIB_PATH)
+    vp, u32, u64, u8, i32, sz = C.c_void_p, C.c_uint32, C.c_uint64, C.c_uint8, C.c_int32, C.c_size_t
+    P = C.POINTER
+    sig = {
+        "mi355q_last_error": (C.c_char_p, []),
+        "mi355q_abi_version": (i32, []),
+        "mi355q_format_for_mlx_quantization": (i32, [C.c_int, C.c_int, P(_Format)]),
+        "mi355q_format_for_scheme": (i32, [u8, P(_Format)]),
+        "mi355q_format_count": (i32, []),
+        "mi355q_format_at": (i32, [i32, P(_Format)]),
+        "mi355q_bf16_from_f32": (C.c_uint16, [C.c_float]),
+        "mi355q_repack_mlx_to_staf": (i32, [u8, sz, sz, vp, vp, vp, C.c_int, vp, sz]),
+        "mi355q_context_create": (i32, [C.c_int, P(vp)]),
+        "mi355q_context_destroy": (i32, [vp]),
+        "mi355q_device_query": (i32, [vp, P(_DeviceInfo)]),
+        "mi355q_buffer_alloc": (i32, [vp, sz, P(vp)]),
+        "mi355q_buffer_free": (i32, [vp, vp]),
+        "mi355q_buffer_upload": (i32, [vp, vp, vp, sz]),
+        "mi355q_buffer_download": (i32, [vp, vp, vp, sz]),
+        "mi355q_buffer_fill": (i32, [vp, vp, vp, u32, sz]),
+        "mi355q_stream_create": (i32, [vp, P(vp)]),
+        "mi355q_stream_destroy": (i32, [vp, vp]),
+        "mi355q_stream_synchronize": (i32, [vp, vp]),
+        "mi355q_event_create": (i32, [vp, P(vp)]),
+        "mi355q_event_destroy": (i32, [vp, vp]),
+        "mi355q_event_record": (i32, [vp, vp, vp]),
+        "mi355q_event_synchronize": (i32, [vp, vp]),
+        "mi355q_event_elapsed_ms": (i32, [vp, vp, vp, P(C.c_float)]),
+        "mi355q_weight_prepare_mlx": (i32, [vp, u8, u64, u64, vp, vp, vp, C.c_int, C.c_int, P(vp)]),
+        "mi355q_weight_prepare_staf": (i32, [vp, u8, u64, u64, vp, sz, C.c_int, P(vp)]),
+        "mi355q_weight_wrap_staf": (i32, [vp, u8, u64, u64, vp, sz, P(vp)]),
+        "mi355q_weight_wrap_planes": (i32, [vp, u8, u64, u64, vp, vp, vp, C.c_int, P(vp)]),
+        "mi355q_weight_query": (i32, [vp, P(_WeightInfo)]),
+        "mi355q_weight_destroy": (i32, [vp]),
+        "mi355q_qgemv": (i32, [vp, vp, vp, vp, C.c_int, vp, C.c_int, u32, u32, u32, u32]),
+        "mi355q_qgemm": (i32, [vp, vp, vp, vp, C.c_int, vp, C.c_int, u32, u32, u32, u32]),
+        "mi355q_batched_qgemm": (i32, [vp, vp, u32, P(vp), vp, C.c_int, P(vp), C.c_int, u32, u32, u32]),
+        "mi355q_dequant_bf16": (i32, [vp, vp, vp, vp]),
+        "mi355q_gemm_bf16": (i32, [vp, vp, vp, C.c_int, vp, vp, C.c_int, u32, u32, u32, u32, u32]),
+        "mi355q_unpack_codes": (i32, [vp, vp, vp, vp]),
+        "mi355q_argmax": (i32, [vp, vp, vp, C.c_int, u32, vp]),
+        "mi355q_lmhead_argmax": (i32, [vp, vp, vp, vp, C.c_int, vp, vp, u32]),
+        "mi355q_shape_family_resolve": (i32, [u32, u32, P(i32), P(u32), P(u32), C.c_char_p, sz]),
+        "mi355q_plan_decode_step": (i32, [vp, u32, C.c_int, u32, P(_Step)]),
+        "mi355q_plan_prefill_steps": (i32, [vp, u32, u32, C.c_int, C.c_int, u32, P(_Step), P(u32)]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(L, name)          # AttributeError here means the ABI and this binding diverged
+        fn.restype, fn.argtypes = res, args
+    _lib = L
+    return L
+
+
+EXPORTED_SYMBOLS = None  # filled lazily by exported_symbols()
+
+
+def exported_symbols():
+    """Names this binding expects the library to export (== every declaration of the C header)."""
+    import re
+    header = os.path.join(_HERE, "..", "include", "mi355_qlinear.h")
+    with open(header) as f:
+        text = f.read()
+    return sorted(set(re.findall(r"MI355Q_API\s+[A-Za-z0-9_ ]+?\**\s*\b(mi355q_[a-z0-9_]+)\s*\(", text)))
+
+
+def _check(status: int):
+    if status != 0:
+        msg = library().mi355q_last_error()
+        raise MI355QError(status, msg.decode() if msg else "")
+
+
+# --------------------------------------------------------------------------------- formats
+@dataclass(frozen=True)
+class QuantizationFormat:
+    scheme_identifier: int
+    bits: int
+    group_size: int
+    weights_per_block: int
+    bytes_per_block: int
+    is_quantized: bool
+    is_aligned: bool
+    has_direct_gemm: bool
+    batched_gemm_counts: tuple
+    in_reference_registry: bool
+    direct_gemm_threadgroup_memory_length: int
+    block_struct_name: str
+    gemv_kernel_name: str
+    gemm_kernel_name_f32s: str
+    gemm_kernel_name: str
+    dequant_to_bfloat_kernel_name: str
+    embedding_lookup_token: str
+
+    @staticmethod
+    def _from(c: _Format) -> "QuantizationFormat":
+        return QuantizationFormat(
+            c.scheme_identifier, c.bits, c.group_size, c.weights_per_block, c.bytes_per_block,
+            bool(c.is_quantized), bool(c.is_aligned), bool(c.has_direct_gemm),
+            tuple(i for i in range(8) if c.batched_gemm_counts >> i & 1), bool(c.in_reference_registry),
+            c.direct_gemm_threadgroup_memory_length, c.block_struct_name.decode(), c.gemv_kernel_name.decode(),
+            c.gemm_kernel_name_f32s.decode(), c.gemm_kernel_name.decode(),
+            c.dequant_to_bfloat_kernel_name.decode(), c.embedding_lookup_token.decode())
+
+    def gemm_kernel_name_for(self, buffer_precision: int) -> str:
+        return self.gemm_kernel_name_f32s if buffer_precision == F32 else self.gemm_kernel_name
+
+    def weight_bytes(self, n: int, k: int) -> int:
+        return n * (k // self.group_size) * self.bytes_per_block
+
+
+class QuantizationFormatRegistry:
+    @staticmethod
+    def format_for_mlx_quantization(bits: int, group_size: int) -> QuantizationFormat:
+        c = _Format()
+        _check(library().mi355q_format_for_mlx_quantization(bits, group_size, C.byref(c)))
+        return QuantizationFormat._from(c)
+
+    @staticmethod
+    def format(scheme_identifier: int) -> QuantizationFormat:
+        c = _Format()
+        _check(library().mi355q_format_for_scheme(scheme_identifier, C.byref(c)))
+        return QuantizationFormat._from(c)
+
+    @staticmethod
+    def all_formats():
+        L = library()
+        out = []
+        for i in range(L.mi355q_format_count()):
+            c = _Format()
+            _check(L.mi355q_format_at(i, C.byref(c)))
+            out.append(QuantizationFormat._from(c))
+        return out
+
+
+def bf16_from_f32(value: float) -> int:
+    return int(library().mi355q_bf16_from_f32(float(np.float32(value))))
+
+
+def _np_sb(a, sb_dtype):
+    return np.ascontiguousarray(a, dtype=np.float32 if sb_dtype == F32 else np.uint16)
+
+
+def repack_mlx_to_staf(fmt: QuantizationFormat, codes, scales, biases, sb_dtype: int) -> np.ndarray:
+    """STAFPayloadConverter.repackMLXQuantized on host memory (no GPU needed)."""
+    codes = np.ascontiguousarray(codes, dtype=np.uint32)
+    n, packed = codes.shape
+    scales, biases = _np_sb(scales, sb_dtype), _np_sb(biases, sb_dtype)
+    k = packed * 32 // fmt.bits
+    out = np.zeros(max(1, n * (k // fmt.group_size) * fmt.bytes_per_block), dtype=np.uint8)
+    _check(library().mi355q_repack_mlx_to_staf(fmt.scheme_identifier, n, packed, codes.ctypes.data,
+                                               scales.ctypes.data, biases.ctypes.data, sb_dtype,
+                                               out.ctypes.data, out.size))
+    return out
+
+
+# ------------------------------------------------------------------------- device objects
+class DeviceBuffer:
+    def __init__(self, ctx: "Context", ptr: int, nbytes: int):
+        self.ctx, self.ptr, self.nbytes = ctx, ptr, nbytes
+
+    def download(self, dtype, shape=None) -> np.ndarray:
+        dtype = np.dtype(dtype)
+        out = np.empty(self.nbytes // dtype.itemsize, dtype=dtype)
+        _check(library().mi355q_buffer_download(self.ctx.handle, out.ctypes.data, self.ptr, out.nbytes))
+        return out.reshape(shape) if shape is not None else out
+
+    def upload(self, array: np.ndarray):
+        a = np.ascontiguousarray(array)
+        assert a.nbytes <= self.nbytes
+        _check(library().mi355q_buffer_upload(self.ctx.handle, self.ptr, a.ctypes.data, a.nbytes))
+
+    def free(self):
+        if self.ptr:
+            _check(library().mi355q_buffer_free(self.ctx.handle, self.ptr))
+            self.ptr = 0
+
+    def offset(self, nbytes: int) -> int:
+        return self.ptr + nbytes
+
+
+@dataclass(frozen=True)
+class DispatchStep:
+    """One planned launch together with its quantization-plan entry."""
+    kernel_name: str
+    device_kernel: str
+    kernel_family: str
+    grid: tuple
+    block: tuple
+    lds_bytes: int
+    rows_per_workgroup: int
+    reference_simdgroups: int
+    reference_tile_elements: int
+    shape_family: str
+    path: str
+    scheme_identifier: int
+    layout: int
+    used_fallback: bool
+    fallback_reason: str | None
+    input_dimension: int
+    output_dimension: int
+    sequence_length: int
+    input_row_stride: int
+    weight_bytes: int
+    flops: int
+
+    @staticmethod
+    def _from(s: _Step) -> "DispatchStep":
+        return DispatchStep(s.kernel_name.decode(), s.device_kernel.decode(), s.kernel_family.decode(),
+                            tuple(s.grid), tuple(s.block), s.lds_bytes, s.rows_per_workgroup,
+                            s.reference_simdgroups, s.reference_tile_elements, FAMILY_NAMES[s.shape_family],
+                            PATH_NAMES[s.path], s.scheme_identifier, s.layout, bool(s.used_fallback),
+                            FALLBACK_NAMES[s.fallback_reason], s.input_dimension, s.output_dimension,
+                            s.sequence_length, s.input_row_stride, s.weight_bytes, s.flops)
+
+
+class PackedWeight:
+    """A prepared (or wrapped) packed weight: the STAFWeightBufferAccess of one tensor."""
+
+    def __init__(self, ctx: "Context", handle: int, keepalive=()):
+        self.ctx, self.handle, self._keep = ctx, handle, keepalive
+
+    @property
+    def info(self) -> _WeightInfo:
+        i = _WeightInfo()
+        _check(library().mi355q_weight_query(self.handle, C.byref(i)))
+        return i
+
+    @property
+    def format(self) -> QuantizationFormat:
+        return QuantizationFormatRegistry.format(self.info.scheme_identifier)
+
+    def plan_decode_step(self, m: int = 1, x_dtype: int = BF16, flags: int = 0) -> DispatchStep:
+        s = _Step()
+        _check(library().mi355q_plan_decode_step(self.handle, m, x_dtype, flags, C.byref(s)))
+        return DispatchStep._from(s)
+
+    def plan_prefill_steps(self, maximum_sequence_length: int, input_row_stride: int = 0, x_dtype: int = BF16,
+                           is_last_token: bool = False, flags: int = 0):
+        steps = (_Step * 2)()
+        n = C.c_uint32(0)
+        _check(library().mi355q_plan_prefill_steps(self.handle, maximum_sequence_length, input_row_stride, x_dtype,
+                                                   int(is_last_token), flags, steps, C.byref(n)))
+        return [DispatchStep._from(steps[i]) for i in range(n.value)]
+
+    def destroy(self):
+        if self.handle:
+            _check(library().mi355q_weight_destroy(self.handle))
+            self.handle = 0
+
+
+def shape_family(output_dimension: int, input_dimension: int):
+    """DecodeProjectionShapeFamily.resolve -> (family, preferredSimdgroups, tileElements, kernelBaseName)."""
+    fam, sg, tile = C.c_int32(), C.c_uint32(), C.c_uint32()
+    name = C.create_string_buffer(48)
+    _check(library().mi355q_shape_family_resolve(output_dimension, input_dimension, C.byref(fam), C.byref(sg),
+                                                 C.byref(tile), name, 48))
+    return FAMILY_NAMES[fam.value], sg.value, tile.value, name.value.decode()
+
+
+class Context:
+    """Device context (the MTLDevice + command queue stand-in).  Raises MI355QError when no GPU."""
+
+    def __init__(self, device_index: int = 0):
+        h = C.c_void_p()
+        _check(library().mi355q_context_create(device_index, C.byref(h)))
+        self.handle = h.value
+
+    def close(self):
+        if self.handle:
+            library().mi355q_context_destroy(self.handle)
+            self.handle = None
+
+    # ---- device info / memory / streams / events
+    def device_info(self) -> _DeviceInfo:
+        i = _DeviceInfo()
+        _check(library().mi355q_device_query(self.handle, C.byref(i)))
+        return i
+
+    def alloc(self, nbytes: int) -> DeviceBuffer:
+        p = C.c_void_p()
+        _check(library().mi355q_buffer_alloc(self.handle, max(1, nbytes), C.byref(p)))
+        return DeviceBuffer(self, p.value, nbytes)
+
+    def upload(self, array: np.ndarray) -> DeviceBuffer:
+        a = np.ascontiguousarray(array)
+        b = self.alloc(a.nbytes)
+        if a.nbytes:
+            b.upload(a)
+        return b
+
+    def fill(self, buf: DeviceBuffer, word: int, stream: int = 0):
+        _check(library().mi355q_buffer_fill(self.handle, stream, buf.ptr, word, buf.nbytes // 4))
+
+    def stream_create(self) -> int:
+        p = C.c_void_p()
+        _check(library().mi355q_stream_create(self.handle, C.byref(p)))
+        return p.value
+
+    def stream_destroy(self, stream: int):
+        _check(library().mi355q_stream_destroy(self.handle, stream))
+
+    def synchronize(self, stream: int = 0):
+        _check(library().mi355q_stream_synchronize(self.handle, stream))
+
+    def event_create(self) -> int:
+        p = C.c_void_p()
+        _check(library().mi355q_event_create(self.handle, C.byref(p)))
+        return p.value
+
+    def event_destroy(self, ev: int):
+        _check(library().mi355q_event_destroy(self.handle, ev))
+
+    def event_record(self, ev: int, stream: int = 0):
+        _check(library().mi355q_event_record(self.handle, ev, stream))
+
+    def event_synchronize(self, ev: int):
+        _check(library().mi355q_event_synchronize(self.handle, ev))
+
+    def event_elapsed_ms(self, start: int, stop: int) -> float:
+        ms = C.c_float()
+        _check(library().mi355q_event_elapsed_ms(self.handle, start, stop, C.byref(ms)))
+        return ms.value
+
+    # ---- packed weights
+    def weight_prepare_mlx(self, fmt: QuantizationFormat, codes, scales, biases, sb_dtype: int,
+                           layout: int = LAYOUT_PLANES, k: int | None = None) -> PackedWeight:
+        codes = np.ascontiguousarray(codes, dtype=np.uint32)
+        n, packed = codes.shape
+        k = packed * 32 // fmt.bits if k is None else k
+        scales, biases = _np_sb(scales, sb_dtype), _np_sb(biases, sb_dtype)
+        h = C.c_void_p()
+        _check(library().mi355q_weight_prepare_mlx(self.handle, fmt.scheme_identifier, n, k, codes.ctypes.data,
+                                                   scales.ctypes.data, biases.ctypes.data, sb_dtype, layout,
+                                                   C.byref(h)))
+        return PackedWeight(self, h.value)
+
+    def weight_prepare_staf(self, fmt: QuantizationFormat, n: int, k: int, blocks,
+                            layout: int = LAYOUT_STAF_BLOCKS) -> PackedWeight:
+        blocks = np.ascontiguousarray(blocks, dtype=np.uint8)
+        h = C.c_void_p()
+        _check(library().mi355q_weight_prepare_staf(self.handle, fmt.scheme_identifier, n, k, blocks.ctypes.data,
+                                                    blocks.size, layout, C.byref(h)))
+        return PackedWeight(self, h.value)
+
+    def weight_wrap_staf(self, fmt: QuantizationFormat, n: int, k: int, blocks: DeviceBuffer,
+                         byte_offset: int = 0, payload_bytes: int | None = None) -> PackedWeight:
+        payload_bytes = fmt.weight_bytes(n, k) if payload_bytes is None else payload_bytes
+        h = C.c_void_p()
+        _check(library().mi355q_weight_wrap_staf(self.handle, fmt.scheme_identifier, n, k,
+                                                 blocks.ptr + byte_offset, payload_bytes, C.byref(h)))
+        return PackedWeight(self, h.value, keepalive=(blocks,))
+
+    def weight_wrap_planes(self, fmt: QuantizationFormat, n: int, k: int, codes: DeviceBuffer,
+                           scales: DeviceBuffer, biases: DeviceBuffer, sb_dtype: int) -> PackedWeight:
+        h = C.c_void_p()
+        _check(library().mi355q_weight_wrap_planes(self.handle, fmt.scheme_identifier, n, k, codes.ptr, scales.ptr,
+                                                   biases.ptr, sb_dtype, C.byref(h)))
+        return PackedWeight(self, h.value, keepalive=(codes, scales, biases))
+
+    # ---- launches (device pointers as ints or DeviceBuffers)
+    @staticmethod
+    def _ptr(b):
+        return b.ptr if isinstance(b, DeviceBuffer) else (0 if b is None else int(b))
+
+    def qgemv(self, w: PackedWeight, x, x_dtype, y, y_dtype, m=1, x_row_stride=0, y_row_stride=0, flags=0,
+              stream=0):
+        _check(library().mi355q_qgemv(self.handle, stream, w.handle, self._ptr(x), x_dtype, self._ptr(y), y_dtype,
+                                      m, x_row_stride, y_row_stride, flags))
+
+    def qgemm(self, w: PackedWeight, x, x_dtype, y, y_dtype, m, x_row_stride=0, y_row_stride=0, flags=0,
+              stream=0):
+        _check(library().mi355q_qgemm(self.handle, stream, w.handle, self._ptr(x), x_dtype, self._ptr(y), y_dtype,
+                                      m, x_row_stride, y_row_stride, flags))
+
+    def batched_qgemm(self, weights, x, x_dtype, ys, y_dtype, m, x_row_stride=0, flags=0, stream=0):
+        n = len(weights)
+        wh = (C.c_void_p * n)(*[w.handle for w in weights])
+        yh = (C.c_void_p * n)(*[self._ptr(y) for y in ys])
+        _check(library().mi355q_batched_qgemm(self.handle, stream, n, wh, self._ptr(x), x_dtype, yh, y_dtype, m,
+                                              x_row_stride, flags))
+
+    def dequant_bf16(self, w: PackedWeight, out, stream=0):
+        _check(library().mi355q_dequant_bf16(self.handle, stream, w.handle, self._ptr(out)))
+
+    def gemm_bf16(self, a, a_dtype, b_bf16, c, c_dtype, m, n, k, a_row_stride=0, c_row_stride=0, stream=0):
+        _check(library().mi355q_gemm_bf16(self.handle, stream, self._ptr(a), a_dtype, self._ptr(b_bf16),
+                                          self._ptr(c), c_dtype, m, n, k, a_row_stride, c_row_stride))
+
+    def unpack_codes(self, w: PackedWeight, out, stream=0):
+        _check(library().mi355q_unpack_codes(self.handle, stream, w.handle, self._ptr(out)))
+
+    def argmax(self, logits, dtype, vocabulary_size, token_out, stream=0):
+        _check(library().mi355q_argmax(self.handle, stream, self._ptr(logits), dtype, vocabulary_size,
+                                       self._ptr(token_out)))
+
+    def lmhead_argmax(self, w: PackedWeight, x, x_dtype, logits_f32, token_out, flags=0, stream=0):
+        _check(library().mi355q_lmhead_argmax(self.handle, stream, w.handle, self._ptr(x), x_dtype,
+                                              self._ptr(logits_f32), self._ptr(token_out), flags))

@@ -1,0 +1,175 @@
+// Launch entry points of the C ABI: argument validation on the host, then kernel selection.
+// Nothing here computes on the CPU; a shape no kernel accepts is an error, never a fallback.
+#include "common.h"
+
+using namespace mi355q;
+
+namespace {
+
+bool dtype_ok(int d) { return d == MI355Q_F16 || d == MI355Q_BF16 || d == MI355Q_F32; }
+
+mi355q_status check_launch(mi355q_context* ctx, const mi355q_weight* w) {
+    if (!ctx) return fail(MI355Q_ERR_NULL_HANDLE, "context is null");
+    if (!w) return fail(MI355Q_ERR_NULL_HANDLE, "weight handle is null");
+    if (w->ctx != ctx) return fail(MI355Q_ERR_INVALID_ARGUMENT, "weight handle belongs to another context");
+    hipError_t e = hipSetDevice(ctx->device);
+    if (e != hipSuccess) return fail(MI355Q_ERR_DEVICE, "hipSetDevice failed: %s", hipGetErrorString(e));
+    return MI355Q_OK;
+}
+
+mi355q_status check_io(const mi355q_weight* w, const void* x, int x_dtype, const void* y, int y_dtype, uint32_t m,
+                       uint32_t& x_stride, uint32_t& y_stride) {
+    if (!x || !y) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null activation or output pointer");
+    if (!dtype_ok(x_dtype) || !dtype_ok(y_dtype)) return fail(MI355Q_ERR_INVALID_ARGUMENT, "bad dtype tag");
+    if (m == 0) return fail(MI355Q_ERR_INVALID_ARGUMENT, "sequence length M must be >= 1");
+    if (x_stride == 0) x_stride = (uint32_t)w->k;
+    if (y_stride == 0) y_stride = (uint32_t)w->n;
+    if (x_stride < w->k)
+        return fail(MI355Q_ERR_SHAPE, "inputRowStride %u < inputDimension %llu", x_stride, (unsigned long long)w->k);
+    if (y_stride < w->n)
+        return fail(MI355Q_ERR_SHAPE, "output row stride %u < outputDimension %llu", y_stride,
+                    (unsigned long long)w->n);
+    const size_t xa = x_dtype == MI355Q_F32 ? 4 : 2, ya = y_dtype == MI355Q_F32 ? 4 : 2;
+    if ((uintptr_t)x % xa || (uintptr_t)y % ya) return fail(MI355Q_ERR_INVALID_ARGUMENT, "misaligned pointer");
+    return MI355Q_OK;
+}
+
+// Small-M path: the split-plane kernel when the shape allows it, else the per-code kernel.
+mi355q_status run_small_m(mi355q_context* ctx, hipStream_t s, const mi355q_weight* w, const void* x, int x_dtype,
+                          void* y, int y_dtype, uint32_t m, uint32_t xs, uint32_t ys, uint32_t flags) {
+    const WView v = w->view();
+    const size_t xsz = x_dtype == MI355Q_F32 ? 4 : 2, ysz = y_dtype == MI355Q_F32 ? 4 : 2;
+    for (uint32_t m0 = 0; m0 < m; m0 += 8) {
+        const uint32_t mm = m - m0 < 8 ? m - m0 : 8;
+        const void* xp = (const char*)x + (size_t)m0 * xs * xsz;
+        void* yp = (char*)y + (size_t)m0 * ys * ysz;
+        mi355q_status st;
+        if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && gemv_fast_eligible(v, x_dtype, mm, xs) && (uintptr_t)xp % 16 == 0)
+            st = launch_gemv_fast(s, ctx, v, xp, yp, y_dtype, mm, xs, ys, nullptr, nullptr, nullptr);
+        else
+            st = launch_gemv_generic(s, v, xp, x_dtype, yp, y_dtype, mm, xs, ys);
+        if (st != MI355Q_OK) return st;
+    }
+    return MI355Q_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+mi355q_status mi355q_qgemv(mi355q_context* ctx, void* stream, const mi355q_weight* w, const void* x_dev,
+                           mi355q_dtype x_dtype, void* y_dev, mi355q_dtype y_dtype, uint32_t m,
+                           uint32_t x_row_stride, uint32_t y_row_stride, uint32_t flags) {
+    if (mi355q_status s = check_launch(ctx, w)) return s;
+    if (mi355q_status s = check_io(w, x_dev, x_dtype, y_dev, y_dtype, m, x_row_stride, y_row_stride)) return s;
+    if (m > 8) return fail(MI355Q_ERR_INVALID_ARGUMENT, "qgemv takes 1 <= M <= 8 (got %u); use qgemm", m);
+    return run_small_m(ctx, (hipStream_t)stream, w, x_dev, x_dtype, y_dev, y_dtype, m, x_row_stride, y_row_stride,
+                       flags);
+}
+
+mi355q_status mi355q_qgemm(mi355q_context* ctx, void* stream, const mi355q_weight* w, const void* x_dev,
+                           mi355q_dtype x_dtype, void* y_dev, mi355q_dtype y_dtype, uint32_t m,
+                           uint32_t x_row_stride, uint32_t y_row_stride, uint32_t flags) {
+    if (mi355q_status s = check_launch(ctx, w)) return s;
+    if (mi355q_status s = check_io(w, x_dev, x_dtype, y_dev, y_dtype, m, x_row_stride, y_row_stride)) return s;
+    if ((flags & MI355Q_FLAG_FORCE_MFMA) && (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)))
+        return fail(MI355Q_ERR_INVALID_ARGUMENT, "contradictory kernel selection flags");
+    const WView v = w->view();
+    const bool mfma_ok = gemm_mfma_eligible(v, x_dtype, m, x_row_stride);
+    if (flags & MI355Q_FLAG_FORCE_MFMA) {
+        if (!mfma_ok)
+            return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the MFMA GEMM does not accept this format, layout or stride");
+        return launch_qgemm_mfma((hipStream_t)stream, ctx, v, x_dev, x_dtype, y_dev, y_dtype, m, x_row_stride,
+                                 y_row_stride);
+    }
+    const bool small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) || m <= 8 || !mfma_ok;
+    if (small)
+        return run_small_m(ctx, (hipStream_t)stream, w, x_dev, x_dtype, y_dev, y_dtype, m, x_row_stride,
+                           y_row_stride, flags);
+    return launch_qgemm_mfma((hipStream_t)stream, ctx, v, x_dev, x_dtype, y_dev, y_dtype, m, x_row_stride,
+                             y_row_stride);
+}
+
+mi355q_status mi355q_batched_qgemm(mi355q_context* ctx, void* stream, uint32_t count,
+                                   const mi355q_weight* const* weights, const void* x_dev, mi355q_dtype x_dtype,
+                                   void* const* y_devs, mi355q_dtype y_dtype, uint32_t m, uint32_t x_row_stride,
+                                   uint32_t flags) {
+    if (!ctx) return fail(MI355Q_ERR_NULL_HANDLE, "context is null");
+    if (count != 2 && count != 3)
+        return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "batched projection count must be 2 or 3 (got %u)", count);
+    if (!weights || !y_devs) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null weight or output array");
+    for (uint32_t i = 0; i < count; i++) {
+        if (!weights[i]) return fail(MI355Q_ERR_NULL_HANDLE, "weight handle %u is null", i);
+        if (weights[i]->k != weights[0]->k || weights[i]->fmt.scheme_identifier != weights[0]->fmt.scheme_identifier ||
+            weights[i]->layout != weights[0]->layout)
+            return fail(MI355Q_ERR_SHAPE, "batched projections must share K, scheme and layout");
+    }
+    // One shared input, `count` outputs with row stride N_i: each projection keeps its own launch;
+    // the launches are independent and queue back to back on the stream.
+    for (uint32_t i = 0; i < count; i++) {
+        mi355q_status st = mi355q_qgemm(ctx, stream, weights[i], x_dev, x_dtype, y_devs[i], y_dtype, m,
+                                        x_row_stride, 0, flags);
+        if (st != MI355Q_OK) return st;
+    }
+    return MI355Q_OK;
+}
+
+mi355q_status mi355q_dequant_bf16(mi355q_context* ctx, void* stream, const mi355q_weight* w, void* out_bf16_dev) {
+    if (mi355q_status s = check_launch(ctx, w)) return s;
+    if (!out_bf16_dev || (uintptr_t)out_bf16_dev % 2) return fail(MI355Q_ERR_INVALID_ARGUMENT, "bad output pointer");
+    return launch_dequant_bf16((hipStream_t)stream, w->view(), (uint16_t*)out_bf16_dev);
+}
+
+mi355q_status mi355q_gemm_bf16(mi355q_context* ctx, void* stream, const void* a_dev, mi355q_dtype a_dtype,
+                               const void* b_bf16_dev, void* c_dev, mi355q_dtype c_dtype, uint32_t m, uint32_t n,
+                               uint32_t k, uint32_t a_row_stride, uint32_t c_row_stride) {
+    if (!ctx) return fail(MI355Q_ERR_NULL_HANDLE, "context is null");
+    if (!a_dev || !b_bf16_dev || !c_dev) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null pointer");
+    if (!dtype_ok(a_dtype) || !dtype_ok(c_dtype)) return fail(MI355Q_ERR_INVALID_ARGUMENT, "bad dtype tag");
+    if (!m || !n || !k) return fail(MI355Q_ERR_SHAPE, "empty GEMM");
+    if (a_row_stride == 0) a_row_stride = k;
+    if (c_row_stride == 0) c_row_stride = n;
+    if (a_row_stride < k || c_row_stride < n) return fail(MI355Q_ERR_SHAPE, "row stride smaller than the row");
+    MI355Q_HIP(hipSetDevice(ctx->device));
+    return launch_gemm_bf16_mfma((hipStream_t)stream, ctx, a_dev, a_dtype, (const uint16_t*)b_bf16_dev, c_dev,
+                                 c_dtype, m, n, k, a_row_stride, c_row_stride);
+}
+
+mi355q_status mi355q_unpack_codes(mi355q_context* ctx, void* stream, const mi355q_weight* w,
+                                  uint8_t* out_codes_dev) {
+    if (mi355q_status s = check_launch(ctx, w)) return s;
+    if (!out_codes_dev) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null output pointer");
+    return launch_unpack_codes((hipStream_t)stream, w->view(), out_codes_dev);
+}
+
+mi355q_status mi355q_argmax(mi355q_context* ctx, void* stream, const void* logits_dev, mi355q_dtype dtype,
+                            uint32_t vocabulary_size, int32_t* token_out_dev) {
+    if (!ctx) return fail(MI355Q_ERR_NULL_HANDLE, "context is null");
+    if (!logits_dev || !token_out_dev) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null pointer");
+    if (!dtype_ok(dtype)) return fail(MI355Q_ERR_INVALID_ARGUMENT, "bad dtype tag");
+    MI355Q_HIP(hipSetDevice(ctx->device));
+    return launch_argmax((hipStream_t)stream, logits_dev, dtype, vocabulary_size, token_out_dev);
+}
+
+mi355q_status mi355q_lmhead_argmax(mi355q_context* ctx, void* stream, const mi355q_weight* w, const void* x_dev,
+                                   mi355q_dtype x_dtype, float* logits_f32_dev, int32_t* token_out_dev,
+                                   uint32_t flags) {
+    if (mi355q_status s = check_launch(ctx, w)) return s;
+    if (!x_dev || !token_out_dev) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null pointer");
+    if (!dtype_ok(x_dtype)) return fail(MI355Q_ERR_INVALID_ARGUMENT, "bad dtype tag");
+    const WView v = w->view();
+    const uint32_t xs = (uint32_t)w->k;
+    if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && gemv_fast_eligible(v, x_dtype, 1, xs) && (uintptr_t)x_dev % 16 == 0)
+        return launch_gemv_fast((hipStream_t)stream, ctx, v, x_dev, nullptr, MI355Q_F32, 1, xs, (uint32_t)w->n,
+                                logits_f32_dev, token_out_dev, ctx->argmax_scratch);
+    // two dispatches, as the reference runs the head: projection to fp32 logits, then argmax
+    if (!logits_f32_dev)
+        return fail(MI355Q_ERR_INVALID_ARGUMENT,
+                    "a logits buffer is required when the fused head kernel does not accept the shape");
+    mi355q_status st = launch_gemv_generic((hipStream_t)stream, v, x_dev, x_dtype, logits_f32_dev, MI355Q_F32, 1, xs,
+                                           (uint32_t)w->n);
+    if (st != MI355Q_OK) return st;
+    return launch_argmax((hipStream_t)stream, logits_f32_dev, MI355Q_F32, (uint32_t)w->n, token_out_dev);
+}
+
+}  // extern "C"

@@ -1,0 +1,120 @@
+// Internal declarations shared by the translation units of libmi355_qlinear.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <string>
+
+#include "../../include/mi355_qlinear.h"
+
+namespace mi355q {
+
+// ---- error plumbing ------------------------------------------------------------------------
+void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+mi355q_status fail(mi355q_status code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define MI355Q_HIP(call)                                                                       \
+    do {                                                                                       \
+        hipError_t _e = (call);                                                                \
+        if (_e != hipSuccess)                                                                  \
+            return ::mi355q::fail(_e == hipErrorOutOfMemory ? MI355Q_ERR_OUT_OF_MEMORY         \
+                                                            : MI355Q_ERR_DEVICE,               \
+                                  "%s failed: %s", #call, hipGetErrorString(_e));              \
+    } while (0)
+
+// ---- format registry (formats.cpp) ---------------------------------------------------------
+const mi355q_format* find_format_mlx(int bits, int group);
+const mi355q_format* find_format_scheme(uint8_t scheme);
+int format_count();
+const mi355q_format* format_at(int i);
+
+// ---- device-side view of one packed weight -------------------------------------------------
+struct WView {
+    const uint8_t* blocks;    // STAF interleaved blocks (layout 0)
+    const uint32_t* codes;    // planes (layout 1)
+    const uint16_t* scales;
+    const uint16_t* biases;
+    uint32_t n, k;
+    uint32_t group, bits;
+    uint32_t bytes_per_block, blocks_per_row, words_per_row;
+    uint32_t layout;          // mi355q_layout
+    uint32_t sb_dtype;        // mi355q_dtype of scale/bias (F16 for STAF)
+};
+
+}  // namespace mi355q
+
+struct mi355q_context {
+    int device;
+    hipDeviceProp_t props;
+    // scratch of the fused LM-head/argmax launch: [0] packed (key,~index) maximum, [1] ticket
+    unsigned long long* argmax_scratch;
+};
+
+struct mi355q_weight {
+    mi355q_context* ctx;
+    mi355q_format fmt;
+    uint64_t n, k;
+    uint8_t layout, sb_dtype, owns;
+    void* blocks;
+    void* codes;
+    void* scales;
+    void* biases;
+    size_t blocks_bytes, codes_bytes, sb_bytes;
+    mi355q::WView view() const {
+        mi355q::WView v;
+        v.blocks = (const uint8_t*)blocks;
+        v.codes = (const uint32_t*)codes;
+        v.scales = (const uint16_t*)scales;
+        v.biases = (const uint16_t*)biases;
+        v.n = (uint32_t)n;
+        v.k = (uint32_t)k;
+        v.group = fmt.group_size;
+        v.bits = fmt.bits;
+        v.bytes_per_block = fmt.bytes_per_block;
+        v.blocks_per_row = (uint32_t)(k / fmt.group_size);
+        v.words_per_row = (uint32_t)(k * fmt.bits / 32);
+        v.layout = layout;
+        v.sb_dtype = sb_dtype;
+        return v;
+    }
+};
+
+namespace mi355q {
+
+// ---- launchers implemented in the kernel translation units ---------------------------------
+// Each returns MI355Q_OK or a launch-time failure; all shape checks happen in api.hip before.
+mi355q_status launch_unpack_codes(hipStream_t s, const WView& w, uint8_t* out);
+mi355q_status launch_dequant_bf16(hipStream_t s, const WView& w, uint16_t* out);
+mi355q_status launch_gemv_generic(hipStream_t s, const WView& w, const void* x, int x_dtype,
+                                  void* y, int y_dtype, uint32_t m, uint32_t x_stride,
+                                  uint32_t y_stride);
+mi355q_status launch_argmax(hipStream_t s, const void* logits, int dtype, uint32_t n,
+                            int32_t* token_out);
+
+// Fast split-plane GEMV (kernels_gemv.hip).  can_* say whether a shape is eligible.
+bool gemv_fast_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
+mi355q_status launch_gemv_fast(hipStream_t s, const mi355q_context* ctx, const WView& w,
+                               const void* x, void* y, int y_dtype, uint32_t m,
+                               uint32_t x_stride, uint32_t y_stride, float* logits_f32,
+                               int32_t* token_out, unsigned long long* argmax_scratch);
+struct GemvLaunchShape {
+    uint32_t grid, block, lds_bytes, rows_per_workgroup;
+    const char* kernel;
+};
+GemvLaunchShape gemv_fast_shape(const mi355q_context* ctx, const WView& w, uint32_t m);
+
+// MFMA GEMM (kernels_gemm.hip)
+bool gemm_mfma_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
+mi355q_status launch_qgemm_mfma(hipStream_t s, const mi355q_context* ctx, const WView& w,
+                                const void* x, int x_dtype, void* y, int y_dtype, uint32_t m,
+                                uint32_t x_stride, uint32_t y_stride);
+mi355q_status launch_gemm_bf16_mfma(hipStream_t s, const mi355q_context* ctx, const void* a,
+                                    int a_dtype, const uint16_t* b, void* c, int c_dtype,
+                                    uint32_t m, uint32_t n, uint32_t k, uint32_t a_stride,
+                                    uint32_t c_stride);
+
+}  // namespace mi355q

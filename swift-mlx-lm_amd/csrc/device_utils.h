@@ -1,0 +1,104 @@
+// Device helpers shared by the kernel translation units (gfx950, wave64).
+#pragma once
+
+#include "common.h"
+
+namespace mi355q {
+
+// ---- number formats ------------------------------------------------------------------------
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+__device__ __forceinline__ float f16_to_f32(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
+
+// bits + 0x7FFF + lsb, >> 16: the reference's host/MSL rule
+// (Sources/MetalCompiler/BFloat16.swift:25-32, Generator/MetalSourceGenerator.swift:50-56).
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
+    const uint32_t u = __float_as_uint(f);
+    return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+}
+__device__ __forceinline__ uint16_t f32_to_f16_rne(float f) {
+    return __builtin_bit_cast(uint16_t, (_Float16)f);
+}
+
+__device__ __forceinline__ float sb_to_f32(uint16_t h, uint32_t sb_dtype) {
+    return sb_dtype == MI355Q_BF16 ? bf16_to_f32(h) : f16_to_f32(h);
+}
+
+template <int D>
+__device__ __forceinline__ float load_act(const void* p, size_t i) {
+    if constexpr (D == MI355Q_F16) return f16_to_f32(((const uint16_t*)p)[i]);
+    else if constexpr (D == MI355Q_BF16) return bf16_to_f32(((const uint16_t*)p)[i]);
+    else return ((const float*)p)[i];
+}
+
+template <int D>
+__device__ __forceinline__ void store_out(void* p, size_t i, float v) {
+    if constexpr (D == MI355Q_F16) ((uint16_t*)p)[i] = f32_to_f16_rne(v);
+    else if constexpr (D == MI355Q_BF16) ((uint16_t*)p)[i] = f32_to_bf16_rne(v);
+    else ((float*)p)[i] = v;
+}
+
+// ---- one code / one block header, either layout ---------------------------------------------
+// q_k = (stream >> k*bits) & mask over the LSB-first bit stream
+// (Sources/MetalCompiler/STAF/QuantizationFormat.swift:1044-1257).
+__device__ __forceinline__ uint32_t load_code(const WView& w, uint32_t row, uint32_t c) {
+    const uint32_t mask = (1u << w.bits) - 1u;
+    if (w.layout == MI355Q_LAYOUT_PLANES) {
+        const uint32_t* rowp = w.codes + (size_t)row * w.words_per_row;
+        const uint64_t bit = (uint64_t)c * w.bits;
+        const uint32_t word = (uint32_t)(bit >> 5), sh = (uint32_t)(bit & 31);
+        uint32_t v = rowp[word] >> sh;
+        if (sh + w.bits > 32) v |= rowp[word + 1] << (32 - sh);
+        return v & mask;
+    }
+    const uint32_t b = c / w.group, e = c - b * w.group;
+    const uint8_t* qs = w.blocks + ((size_t)row * w.blocks_per_row + b) * w.bytes_per_block + 4;
+    const uint32_t bit = e * w.bits, byte = bit >> 3, sh = bit & 7;
+    uint32_t v = qs[byte];
+    if (sh + w.bits > 8) v |= (uint32_t)qs[byte + 1] << 8;
+    return (v >> sh) & mask;
+}
+
+__device__ __forceinline__ void load_scale_zero(const WView& w, uint32_t row, uint32_t b, float& scale,
+                                                float& zero) {
+    if (w.layout == MI355Q_LAYOUT_PLANES) {
+        const size_t g = (size_t)row * w.blocks_per_row + b;
+        scale = sb_to_f32(w.scales[g], w.sb_dtype);
+        zero = sb_to_f32(w.biases[g], w.sb_dtype);
+    } else {
+        const uint16_t* hdr =
+            (const uint16_t*)(w.blocks + ((size_t)row * w.blocks_per_row + b) * w.bytes_per_block);
+        scale = f16_to_f32(hdr[0]);
+        zero = f16_to_f32(hdr[1]);
+    }
+}
+
+// ---- wavefront reductions (all 64 lanes must be active) -------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+
+// Sum over the 64 lanes; every lane returns the total.  Four DPP steps inside each row of 16
+// lanes (quad swap, quad-pair swap, half-row mirror, row mirror), then the four row totals are
+// read with readlane.
+__device__ __forceinline__ float wave_reduce_sum(float v) {
+    v += dpp_f32<0xB1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_f32<0x4E>(v);   // quad_perm [2,3,0,1]
+    v += dpp_f32<0x141>(v);  // row_half_mirror
+    v += dpp_f32<0x140>(v);  // row_mirror
+    const int iv = __float_as_int(v);
+    return (__int_as_float(__builtin_amdgcn_readlane(iv, 0)) + __int_as_float(__builtin_amdgcn_readlane(iv, 16))) +
+           (__int_as_float(__builtin_amdgcn_readlane(iv, 32)) + __int_as_float(__builtin_amdgcn_readlane(iv, 48)));
+}
+
+// (value, index) maximum with "greater, or equal and lower index"; every lane ends with the result.
+__device__ __forceinline__ void wave_argmax(float& v, uint32_t& idx) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(v, off, 64);
+        const uint32_t oi = (uint32_t)__shfl_xor((int)idx, off, 64);
+        if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; }
+    }
+}
+
+}  // namespace mi355q

@@ -1,0 +1,143 @@
+// Reference-shaped kernels: one code at a time, any registered format, either layout, any
+// activation dtype and stride.  They are the always-available path (tiny shapes, odd strides,
+// f16/f32 activations) and the A/B partner of the specialised kernels.
+//
+// Reference kernels these stand in for (Sources/MetalCompiler/Generator/):
+//   generateUnifiedQuantizedGEMV      MetalSourceGenerator+Quantized.swift:496-575
+//   generateQuantizedGEMM_Q4/_Q8      MetalSourceGenerator+Quantized.swift:22-156 (sequence signature)
+//   generateUnifiedDequantToBFloat    MetalSourceGenerator+Quantized.swift:361-416
+//   generateArgmax                    MetalSourceGenerator+Sampling.swift:62-107
+#include "device_utils.h"
+
+namespace mi355q {
+
+// ------------------------------------------------------------------------------ unpack codes
+__global__ __launch_bounds__(256) void unpack_codes_kernel(WView w, uint8_t* __restrict__ out) {
+    const size_t total = (size_t)w.n * w.k;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < total; i += stride) {
+        const uint32_t row = (uint32_t)(i / w.k), c = (uint32_t)(i % w.k);
+        out[i] = (uint8_t)load_code(w, row, c);
+    }
+}
+
+mi355q_status launch_unpack_codes(hipStream_t s, const WView& w, uint8_t* out) {
+    const size_t total = (size_t)w.n * w.k;
+    size_t blocks = (total + 255) / 256;
+    if (blocks > 16384) blocks = 16384;
+    unpack_codes_kernel<<<dim3((unsigned)blocks), dim3(256), 0, s>>>(w, out);
+    MI355Q_HIP(hipGetLastError());
+    return MI355Q_OK;
+}
+
+// ------------------------------------------------------------------------------ dequant bf16
+// One workgroup per row, 256 threads striding over the row, as the reference kernel does.
+// scale*q and +zero are kept as two roundings so the result is bit-identical to an unfused
+// host evaluation.
+__global__ __launch_bounds__(256) void dequant_bf16_kernel(WView w, uint16_t* __restrict__ out) {
+    for (uint32_t row = blockIdx.x; row < w.n; row += gridDim.x) {
+        uint16_t* orow = out + (size_t)row * w.k;
+        for (uint32_t c = threadIdx.x; c < w.k; c += 256) {
+            float scale, zero;
+            load_scale_zero(w, row, c / w.group, scale, zero);
+            const float q = (float)load_code(w, row, c);
+            orow[c] = f32_to_bf16_rne(__fadd_rn(__fmul_rn(scale, q), zero));
+        }
+    }
+}
+
+mi355q_status launch_dequant_bf16(hipStream_t s, const WView& w, uint16_t* out) {
+    unsigned blocks = w.n < 65535u * 16u ? w.n : 65535u * 16u;
+    dequant_bf16_kernel<<<dim3(blocks), dim3(256), 0, s>>>(w, out);
+    MI355Q_HIP(hipGetLastError());
+    return MI355Q_OK;
+}
+
+// ------------------------------------------------------------------------------ generic GEMV
+// grid (ceil(N/4), M); one wavefront per output row, lanes stride over the codes of the row.
+template <int XD, int YD>
+__global__ __launch_bounds__(256) void gemv_generic_kernel(WView w, const void* __restrict__ x,
+                                                           void* __restrict__ y, uint32_t x_stride,
+                                                           uint32_t y_stride) {
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t row = blockIdx.x * 4 + wave;
+    const uint32_t m = blockIdx.y;
+    if (row >= w.n) return;  // whole wavefront leaves together
+    const size_t xoff = (size_t)m * x_stride;
+    float sum = 0.0f;
+    for (uint32_t b = 0; b < w.blocks_per_row; b++) {
+        float scale, zero;
+        load_scale_zero(w, row, b, scale, zero);
+        for (uint32_t e = lane; e < w.group; e += 64) {
+            const uint32_t c = b * w.group + e;
+            const float wt = scale * (float)load_code(w, row, c) + zero;
+            sum += wt * load_act<XD>(x, xoff + c);
+        }
+    }
+    sum = wave_reduce_sum(sum);
+    if (lane == 0) store_out<YD>(y, (size_t)m * y_stride + row, sum);
+}
+
+template <int XD>
+static mi355q_status launch_generic_y(hipStream_t s, const WView& w, const void* x, void* y,
+                                      int y_dtype, uint32_t m, uint32_t xs, uint32_t ys) {
+    dim3 grid((w.n + 3) / 4, m), block(256);
+    switch (y_dtype) {
+    case MI355Q_F16: gemv_generic_kernel<XD, MI355Q_F16><<<grid, block, 0, s>>>(w, x, y, xs, ys); break;
+    case MI355Q_BF16: gemv_generic_kernel<XD, MI355Q_BF16><<<grid, block, 0, s>>>(w, x, y, xs, ys); break;
+    default: gemv_generic_kernel<XD, MI355Q_F32><<<grid, block, 0, s>>>(w, x, y, xs, ys); break;
+    }
+    MI355Q_HIP(hipGetLastError());
+    return MI355Q_OK;
+}
+
+mi355q_status launch_gemv_generic(hipStream_t s, const WView& w, const void* x, int x_dtype, void* y,
+                                  int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride) {
+    if (m > 65535u) return fail(MI355Q_ERR_INVALID_ARGUMENT, "generic kernel supports M <= 65535");
+    switch (x_dtype) {
+    case MI355Q_F16: return launch_generic_y<MI355Q_F16>(s, w, x, y, y_dtype, m, x_stride, y_stride);
+    case MI355Q_BF16: return launch_generic_y<MI355Q_BF16>(s, w, x, y, y_dtype, m, x_stride, y_stride);
+    default: return launch_generic_y<MI355Q_F32>(s, w, x, y, y_dtype, m, x_stride, y_stride);
+    }
+}
+
+// ------------------------------------------------------------------------------------ argmax
+// One workgroup of 1024 threads.  Each thread scans i = tid, tid+1024, ... with a strict '>'
+// from (-inf, index 0); partial results merge with "greater value, or equal value and lower
+// index", so the winner is the lowest index holding the maximum, and NaN never wins.
+template <int D>
+__global__ __launch_bounds__(1024) void argmax_kernel(const void* __restrict__ logits, uint32_t n,
+                                                      int32_t* __restrict__ result) {
+    __shared__ float s_val[16];
+    __shared__ uint32_t s_idx[16];
+    float best = -INFINITY;
+    uint32_t bidx = 0;
+    for (uint32_t i = threadIdx.x; i < n; i += 1024) {
+        const float v = load_act<D>(logits, i);
+        if (v > best) { best = v; bidx = i; }
+    }
+    wave_argmax(best, bidx);
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (lane == 0) { s_val[wave] = best; s_idx[wave] = bidx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float bv = s_val[0];
+        uint32_t bi = s_idx[0];
+        for (int i = 1; i < 16; i++)
+            if (s_val[i] > bv || (s_val[i] == bv && s_idx[i] < bi)) { bv = s_val[i]; bi = s_idx[i]; }
+        result[0] = (int32_t)bi;
+    }
+}
+
+mi355q_status launch_argmax(hipStream_t s, const void* logits, int dtype, uint32_t n, int32_t* token_out) {
+    switch (dtype) {
+    case MI355Q_F16: argmax_kernel<MI355Q_F16><<<dim3(1), dim3(1024), 0, s>>>(logits, n, token_out); break;
+    case MI355Q_BF16: argmax_kernel<MI355Q_BF16><<<dim3(1), dim3(1024), 0, s>>>(logits, n, token_out); break;
+    default: argmax_kernel<MI355Q_F32><<<dim3(1), dim3(1024), 0, s>>>(logits, n, token_out); break;
+    }
+    MI355Q_HIP(hipGetLastError());
+    return MI355Q_OK;
+}
+
+}  // namespace mi355q

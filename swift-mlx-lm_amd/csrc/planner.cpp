@@ -1,0 +1,157 @@
+// Planner mirror: launch-shape families, kernel selection and the quantization-plan record.
+// Reference: Sources/MetalCompiler/Compiler/MetalCompileContext.swift:5-90,246-260 (shape
+// families and GEMV grid), MetalDispatchStepBuilder.swift:640-689 (decode step),
+// MetalPrefillStepBuilder.swift:463-742,1866-1893 (prefill steps and fallback reasons),
+// MetalQuantizationPlan.swift:290-318 (plan entry).
+#include "common.h"
+
+using namespace mi355q;
+
+namespace {
+
+struct Family {
+    int32_t id;
+    uint32_t simdgroups, tile;
+    const char* base;
+};
+
+// DecodeProjectionShapeFamily.resolve + preferredSimdgroups + tileElements + kernelBaseName
+Family resolve_family(uint32_t n, uint32_t k) {
+    if (n >= 65536 && k == 2048) return {MI355Q_FAMILY_VOCAB_DENSE, 16, 2048, "gemv_vocab"};
+    if (k == 2048 && n == 2048) return {MI355Q_FAMILY_INPUT2048_SQUARE, 8, 2048, "gemv_2048_sq"};
+    if (k == 2048 && n == 6144) return {MI355Q_FAMILY_INPUT2048_6144, 4, 2048, "gemv_2048_6144"};
+    if (k == 2048 && n == 8192) return {MI355Q_FAMILY_INPUT2048_8192, 8, 2048, "gemv_2048_8192"};
+    if (k == 2048 && n > 2048 && n < 65536) return {MI355Q_FAMILY_INPUT2048_EXPANDED, 8, 2048, "gemv_2048"};
+    if (k == 8192 && n >= 2048 && n < 65536) return {MI355Q_FAMILY_INPUT8192_TILED, 8, 1024, "gemv_8192_tiled"};
+    if (n >= 32768 && k >= 2048) return {MI355Q_FAMILY_LARGE_DENSE, 8, 512, "gemv_large"};
+    return {MI355Q_FAMILY_GENERIC, 4, 256, "gemv"};
+}
+
+void fill_common(const mi355q_weight* w, uint32_t m, mi355q_step* s) {
+    std::memset(s, 0, sizeof *s);
+    const Family f = resolve_family((uint32_t)w->n, (uint32_t)w->k);
+    s->shape_family = f.id;
+    s->reference_simdgroups = f.simdgroups;
+    s->reference_tile_elements = f.tile;
+    s->scheme_identifier = w->fmt.scheme_identifier;
+    s->layout = w->layout;
+    s->input_dimension = (uint32_t)w->k;
+    s->output_dimension = (uint32_t)w->n;
+    s->sequence_length = m;
+    s->weight_bytes = w->n * (w->k / w->fmt.group_size) * w->fmt.bytes_per_block;
+    s->flops = 2ull * m * w->k * w->n;
+    s->grid[1] = s->grid[2] = s->block[1] = s->block[2] = 1;
+}
+
+void plan_small_m(const mi355q_weight* w, uint32_t m, int x_dtype, uint32_t x_stride, uint32_t flags,
+                  mi355q_step* s) {
+    const WView v = w->view();
+    const bool forced = flags & MI355Q_FLAG_FORCE_GENERIC;
+    if (!forced && gemv_fast_eligible(v, x_dtype, m > 8 ? 8 : m, x_stride)) {
+        const GemvLaunchShape g = gemv_fast_shape(w->ctx, v, m > 8 ? 8 : m);
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_planes_q%u_g%u", (unsigned)w->fmt.bits,
+                      w->fmt.group_size);
+        s->grid[0] = g.grid;
+        s->block[0] = g.block;
+        s->lds_bytes = g.lds_bytes;
+        s->rows_per_workgroup = g.rows_per_workgroup;
+    } else {
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_generic");
+        s->grid[0] = (uint32_t)((w->n + 3) / 4);
+        s->grid[1] = m;
+        s->block[0] = 256;
+        s->rows_per_workgroup = 4;
+        s->used_fallback = 1;
+        s->fallback_reason = forced ? MI355Q_FALLBACK_DISABLED_BY_ENVIRONMENT : MI355Q_FALLBACK_UNAVAILABLE_ACCELERATION;
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+mi355q_status mi355q_shape_family_resolve(uint32_t output_dimension, uint32_t input_dimension, int32_t* out_family,
+                                          uint32_t* out_simdgroups, uint32_t* out_tile_elements,
+                                          char* out_kernel_base_name, size_t name_cap) {
+    const Family f = resolve_family(output_dimension, input_dimension);
+    if (out_family) *out_family = f.id;
+    if (out_simdgroups) *out_simdgroups = f.simdgroups;
+    if (out_tile_elements) *out_tile_elements = f.tile;
+    if (out_kernel_base_name && name_cap) std::snprintf(out_kernel_base_name, name_cap, "%s", f.base);
+    return MI355Q_OK;
+}
+
+mi355q_status mi355q_plan_decode_step(const mi355q_weight* w, uint32_t m, mi355q_dtype x_dtype, uint32_t flags,
+                                      mi355q_step* out) {
+    if (!w) return fail(MI355Q_ERR_NULL_HANDLE, "weight handle is null");
+    if (!out) return fail(MI355Q_ERR_INVALID_ARGUMENT, "out pointer is null");
+    if (m < 1 || m > 8) return fail(MI355Q_ERR_INVALID_ARGUMENT, "decode step takes 1 <= M <= 8");
+    fill_common(w, m, out);
+    out->path = MI355Q_PATH_DECODE_PROJECTION;
+    out->input_row_stride = (uint32_t)w->k;
+    // decode => format.gemvKernelName (MetalKernelNameResolver.swift:85-140)
+    std::snprintf(out->kernel_name, sizeof out->kernel_name, "%s", w->fmt.gemv_kernel_name);
+    std::snprintf(out->kernel_family, sizeof out->kernel_family, "q%uG%uGEMV", (unsigned)w->fmt.bits,
+                  w->fmt.group_size);
+    plan_small_m(w, m, x_dtype, (uint32_t)w->k, flags, out);
+    return MI355Q_OK;
+}
+
+mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w, uint32_t maximum_sequence_length,
+                                        uint32_t input_row_stride, mi355q_dtype x_dtype, int is_last_token,
+                                        uint32_t flags, mi355q_step* out_steps, uint32_t* out_count) {
+    if (!w) return fail(MI355Q_ERR_NULL_HANDLE, "weight handle is null");
+    if (!out_steps || !out_count) return fail(MI355Q_ERR_INVALID_ARGUMENT, "out pointer is null");
+    if (maximum_sequence_length == 0) return fail(MI355Q_ERR_INVALID_ARGUMENT, "maximumSequenceLength must be >= 1");
+    if (input_row_stride == 0) input_row_stride = (uint32_t)w->k;
+    if (input_row_stride < w->k) return fail(MI355Q_ERR_SHAPE, "inputRowStride smaller than inputDimension");
+    *out_count = 1;
+    mi355q_step* s = &out_steps[0];
+    const WView v = w->view();
+
+    if (is_last_token) {
+        // mode = .lastToken: the head runs the decode kernel on one row
+        fill_common(w, 1, s);
+        s->path = MI355Q_PATH_PREFILL_PROJECTION;
+        s->input_row_stride = input_row_stride;
+        std::snprintf(s->kernel_name, sizeof s->kernel_name, "%s", w->fmt.gemv_kernel_name);
+        std::snprintf(s->kernel_family, sizeof s->kernel_family, "q%uG%uGEMV", (unsigned)w->fmt.bits,
+                      w->fmt.group_size);
+        plan_small_m(w, 1, x_dtype, input_row_stride, flags, s);
+        s->used_fallback = 1;
+        s->fallback_reason = MI355Q_FALLBACK_LAST_TOKEN_USES_DECODE_KERNEL;
+        return MI355Q_OK;
+    }
+
+    const uint32_t m = maximum_sequence_length;
+    const bool want_small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) || m <= 8;
+    const bool mfma_ok = gemm_mfma_eligible(v, x_dtype, m, input_row_stride);
+    fill_common(w, m, s);
+    s->path = MI355Q_PATH_PREFILL_PROJECTION;
+    s->input_row_stride = input_row_stride;
+    if (!want_small && mfma_ok) {
+        // fused dequant + matrix-core contraction: the stand-in for dequant_q*_bf16 + gemm_bf16_f32s
+        std::snprintf(s->kernel_name, sizeof s->kernel_name, "%s", w->fmt.gemm_kernel_name_f32s);
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "qgemm_mfma_q%u_g%u", (unsigned)w->fmt.bits,
+                      w->fmt.group_size);
+        std::snprintf(s->kernel_family, sizeof s->kernel_family, "mfmaGEMM");
+        s->block[0] = 256;
+        s->grid[0] = (uint32_t)((w->n + 255) / 256) * ((m + 255) / 256);
+        s->rows_per_workgroup = 256;
+        return MI355Q_OK;
+    }
+    // direct per-row kernel with the sequence signature (gemm_q{b}_g{g}[_f32s])
+    std::snprintf(s->kernel_name, sizeof s->kernel_name, "%s",
+                  x_dtype == MI355Q_F32 ? w->fmt.gemm_kernel_name_f32s : w->fmt.gemm_kernel_name);
+    std::snprintf(s->kernel_family, sizeof s->kernel_family, "q%uG%uGEMM", (unsigned)w->fmt.bits,
+                  w->fmt.group_size);
+    plan_small_m(w, m, x_dtype, input_row_stride, flags, s);
+    if (!want_small && !mfma_ok) {
+        s->used_fallback = 1;
+        s->fallback_reason = (input_row_stride != w->k) ? MI355Q_FALLBACK_INPUT_STRIDE_MISMATCH
+                                                        : MI355Q_FALLBACK_UNAVAILABLE_ACCELERATION;
+    }
+    return MI355Q_OK;
+}
+
+}  // extern "C"
