@@ -361,6 +361,50 @@ MI355Q_API mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w,
                                                    int is_last_token, uint32_t flags,
                                                    mi355q_step* out_steps, uint32_t* out_count);
 
+/* ------------------------------------------------------------------------------------------
+ * Dispatch plan: MetalDispatchPlan (MC/Execution/MetalDecodePlan.swift:6-140) built once at load
+ * time and replayed for every token by MetalDecodeEncoder.encodeSteps
+ * (MC/Execution/MetalDecodeEncoder.swift:18-36).  Steps run in order on one stream, which
+ * satisfies the read/write ordering the reference enforces with barriers
+ * (MC/Compiler/MetalDispatchStepBuilder.swift:276-350).  A plan borrows its weights and
+ * buffers: they must outlive it.
+ * ---------------------------------------------------------------------------------------- */
+typedef struct mi355q_plan mi355q_plan;
+
+MI355Q_API mi355q_status mi355q_plan_create(mi355q_context* ctx, mi355q_plan** out);
+MI355Q_API mi355q_status mi355q_plan_destroy(mi355q_plan* plan);
+/* One LinearFragment step (bindings as mi355q_qgemm).  layer_index and tensor_name are the
+ * step metadata (MetalDispatchStepMetadata); tensor_name may be NULL. */
+MI355Q_API mi355q_status mi355q_plan_add_linear(mi355q_plan* plan, const mi355q_weight* w,
+                                                const void* x_dev, mi355q_dtype x_dtype,
+                                                void* y_dev, mi355q_dtype y_dtype, uint32_t m,
+                                                uint32_t x_row_stride, uint32_t y_row_stride,
+                                                uint32_t flags, int32_t layer_index,
+                                                const char* tensor_name);
+/* One OutputHeadFragment step (bindings as mi355q_lmhead_argmax). */
+MI355Q_API mi355q_status mi355q_plan_add_output_head(mi355q_plan* plan, const mi355q_weight* w,
+                                                     const void* x_dev, mi355q_dtype x_dtype,
+                                                     float* logits_f32_dev, int32_t* token_out_dev,
+                                                     uint32_t flags, const char* tensor_name);
+MI355Q_API int32_t mi355q_plan_step_count(const mi355q_plan* plan);
+/* The planned launch and its quantization-plan entry for step `index`; layer_index_out and
+ * tensor_name_out (capacity name_cap) may be NULL. */
+MI355Q_API mi355q_status mi355q_plan_step_at(const mi355q_plan* plan, int32_t index,
+                                             mi355q_step* out, int32_t* layer_index_out,
+                                             char* tensor_name_out, size_t name_cap);
+/* encodeSteps: enqueue steps [first, first+count) on `stream`; count 0 means "to the end". */
+MI355Q_API mi355q_status mi355q_plan_encode(mi355q_plan* plan, void* stream, uint32_t first,
+                                            uint32_t count);
+/* Capture the whole plan into a HIP graph once, then replay it with one launch per token. */
+MI355Q_API mi355q_status mi355q_plan_graph_build(mi355q_plan* plan, void* stream);
+MI355Q_API mi355q_status mi355q_plan_graph_launch(mi355q_plan* plan, void* stream);
+
+/* Device-to-device copy kernel (prompt-state snapshots copy runtime buffers,
+ * MC/Execution/MetalPromptState.swift:3-19; also the known-size copy that calibrates the HBM
+ * traffic counters).  Both pointers 16-byte aligned, bytes a multiple of 16. */
+MI355Q_API mi355q_status mi355q_buffer_copy(mi355q_context* ctx, void* stream, void* dst_dev,
+                                            const void* src_dev, size_t bytes);
+
 #ifdef __cplusplus
 }
 #endif

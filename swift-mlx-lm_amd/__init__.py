@@ -129,6 +129,16 @@ def library() -> C.CDLL:
         "mi355q_argmax": (i32, [vp, vp, vp, C.c_int, u32, vp]),
         "mi355q_lmhead_argmax": (i32, [vp, vp, vp, vp, C.c_int, vp, vp, u32]),
         "mi355q_shape_family_resolve": (i32, [u32, u32, P(i32), P(u32), P(u32), C.c_char_p, sz]),
+        "mi355q_plan_create": (i32, [vp, P(vp)]),
+        "mi355q_plan_destroy": (i32, [vp]),
+        "mi355q_plan_add_linear": (i32, [vp, vp, vp, C.c_int, vp, C.c_int, u32, u32, u32, u32, i32, C.c_char_p]),
+        "mi355q_plan_add_output_head": (i32, [vp, vp, vp, C.c_int, vp, vp, u32, C.c_char_p]),
+        "mi355q_plan_step_count": (i32, [vp]),
+        "mi355q_plan_step_at": (i32, [vp, i32, P(_Step), P(i32), C.c_char_p, sz]),
+        "mi355q_plan_encode": (i32, [vp, vp, u32, u32]),
+        "mi355q_plan_graph_build": (i32, [vp, vp]),
+        "mi355q_plan_graph_launch": (i32, [vp, vp]),
+        "mi355q_buffer_copy": (i32, [vp, vp, vp, vp, sz]),
         "mi355q_plan_decode_step": (i32, [vp, u32, C.c_int, u32, P(_Step)]),
         "mi355q_plan_prefill_steps": (i32, [vp, u32, u32, C.c_int, C.c_int, u32, P(_Step), P(u32)]),
     }
@@ -335,6 +345,52 @@ class PackedWeight:
             self.handle = 0
 
 
+class DispatchPlan:
+    """Ordered projection steps built once and replayed per token (MetalDispatchPlan + encodeSteps)."""
+
+    def __init__(self, ctx: "Context"):
+        h = C.c_void_p()
+        _check(library().mi355q_plan_create(ctx.handle, C.byref(h)))
+        self.ctx, self.handle, self._keep = ctx, h.value, []
+
+    def add_linear(self, w: "PackedWeight", x, x_dtype, y, y_dtype, m=1, x_row_stride=0, y_row_stride=0, flags=0,
+                   layer_index=-1, tensor_name: str | None = None):
+        _check(library().mi355q_plan_add_linear(self.handle, w.handle, Context._ptr(x), x_dtype, Context._ptr(y),
+                                                y_dtype, m, x_row_stride, y_row_stride, flags, layer_index,
+                                                tensor_name.encode() if tensor_name else None))
+        self._keep.append((w, x, y))
+
+    def add_output_head(self, w: "PackedWeight", x, x_dtype, logits_f32, token_out, flags=0,
+                        tensor_name: str | None = None):
+        _check(library().mi355q_plan_add_output_head(self.handle, w.handle, Context._ptr(x), x_dtype,
+                                                     Context._ptr(logits_f32), Context._ptr(token_out), flags,
+                                                     tensor_name.encode() if tensor_name else None))
+        self._keep.append((w, x, logits_f32, token_out))
+
+    def __len__(self):
+        return library().mi355q_plan_step_count(self.handle)
+
+    def step(self, index: int):
+        s, layer = _Step(), C.c_int32()
+        name = C.create_string_buffer(128)
+        _check(library().mi355q_plan_step_at(self.handle, index, C.byref(s), C.byref(layer), name, 128))
+        return DispatchStep._from(s), layer.value, name.value.decode()
+
+    def encode(self, stream: int = 0, first: int = 0, count: int = 0):
+        _check(library().mi355q_plan_encode(self.handle, stream, first, count))
+
+    def graph_build(self, stream: int):
+        _check(library().mi355q_plan_graph_build(self.handle, stream))
+
+    def graph_launch(self, stream: int):
+        _check(library().mi355q_plan_graph_launch(self.handle, stream))
+
+    def destroy(self):
+        if self.handle:
+            _check(library().mi355q_plan_destroy(self.handle))
+            self.handle = 0
+
+
 def shape_family(output_dimension: int, input_dimension: int):
     """DecodeProjectionShapeFamily.resolve -> (family, preferredSimdgroups, tileElements, kernelBaseName)."""
     fam, sg, tile = C.c_int32(), C.c_uint32(), C.c_uint32()
@@ -374,6 +430,9 @@ class Context:
         if a.nbytes:
             b.upload(a)
         return b
+
+    def copy(self, dst, src, nbytes: int, stream: int = 0):
+        _check(library().mi355q_buffer_copy(self.handle, stream, self._ptr(dst), self._ptr(src), nbytes))
 
     def fill(self, buf: DeviceBuffer, word: int, stream: int = 0):
         _check(library().mi355q_buffer_fill(self.handle, stream, buf.ptr, word, buf.nbytes // 4))

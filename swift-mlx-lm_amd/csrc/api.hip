@@ -1,5 +1,7 @@
 // Launch entry points of the C ABI: argument validation on the host, then kernel selection.
 // Nothing here computes on the CPU; a shape no kernel accepts is an error, never a fallback.
+#include <cstdlib>
+
 #include "common.h"
 
 using namespace mi355q;
@@ -55,39 +57,76 @@ mi355q_status run_small_m(mi355q_context* ctx, hipStream_t s, const mi355q_weigh
 
 }  // namespace
 
+namespace mi355q {
+
+int env_int_cached(const char* name, int fallback) {
+#ifdef MI355Q_GEMV_EXPERIMENT
+    const char* v = std::getenv(name);   // tuning builds re-read the environment at every launch
+    return (v && *v) ? std::atoi(v) : fallback;
+#else
+    (void)name;
+    return fallback;
+#endif
+}
+
+mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_weight* w, const void* x, int x_dtype,
+                              void* y, int y_dtype, uint32_t m, uint32_t xs, uint32_t ys, uint32_t flags,
+                              bool small_m_only) {
+    if (mi355q_status st = check_io(w, x, x_dtype, y, y_dtype, m, xs, ys)) return st;
+    if (small_m_only) {
+        if (m > 8) return fail(MI355Q_ERR_INVALID_ARGUMENT, "qgemv takes 1 <= M <= 8 (got %u); use qgemm", m);
+        return run_small_m(ctx, s, w, x, x_dtype, y, y_dtype, m, xs, ys, flags);
+    }
+    if ((flags & MI355Q_FLAG_FORCE_MFMA) && (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)))
+        return fail(MI355Q_ERR_INVALID_ARGUMENT, "contradictory kernel selection flags");
+    const WView v = w->view();
+    const bool mfma_ok = gemm_mfma_eligible(v, x_dtype, m, xs);
+    if (flags & MI355Q_FLAG_FORCE_MFMA) {
+        if (!mfma_ok)
+            return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the MFMA GEMM does not accept this format, layout or stride");
+        return launch_qgemm_mfma(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
+    }
+    const bool small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) || m <= 8 || !mfma_ok;
+    if (small) return run_small_m(ctx, s, w, x, x_dtype, y, y_dtype, m, xs, ys, flags);
+    return launch_qgemm_mfma(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
+}
+
+mi355q_status dispatch_output_head(mi355q_context* ctx, hipStream_t s, const mi355q_weight* w, const void* x,
+                                   int x_dtype, float* logits, int32_t* token, uint32_t flags) {
+    if (!x || !token) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null pointer");
+    if (!dtype_ok(x_dtype)) return fail(MI355Q_ERR_INVALID_ARGUMENT, "bad dtype tag");
+    const WView v = w->view();
+    const uint32_t xs = (uint32_t)w->k;
+    if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && gemv_fast_eligible(v, x_dtype, 1, xs) && (uintptr_t)x % 16 == 0)
+        return launch_gemv_fast(s, ctx, v, x, nullptr, MI355Q_F32, 1, xs, (uint32_t)w->n, logits, token,
+                                ctx->argmax_scratch);
+    // two dispatches, as the reference runs the head: projection to fp32 logits, then argmax
+    if (!logits)
+        return fail(MI355Q_ERR_INVALID_ARGUMENT,
+                    "a logits buffer is required when the fused head kernel does not accept the shape");
+    mi355q_status st = launch_gemv_generic(s, v, x, x_dtype, logits, MI355Q_F32, 1, xs, (uint32_t)w->n);
+    if (st != MI355Q_OK) return st;
+    return launch_argmax(s, logits, MI355Q_F32, (uint32_t)w->n, token);
+}
+
+}  // namespace mi355q
+
 extern "C" {
 
 mi355q_status mi355q_qgemv(mi355q_context* ctx, void* stream, const mi355q_weight* w, const void* x_dev,
                            mi355q_dtype x_dtype, void* y_dev, mi355q_dtype y_dtype, uint32_t m,
                            uint32_t x_row_stride, uint32_t y_row_stride, uint32_t flags) {
     if (mi355q_status s = check_launch(ctx, w)) return s;
-    if (mi355q_status s = check_io(w, x_dev, x_dtype, y_dev, y_dtype, m, x_row_stride, y_row_stride)) return s;
-    if (m > 8) return fail(MI355Q_ERR_INVALID_ARGUMENT, "qgemv takes 1 <= M <= 8 (got %u); use qgemm", m);
-    return run_small_m(ctx, (hipStream_t)stream, w, x_dev, x_dtype, y_dev, y_dtype, m, x_row_stride, y_row_stride,
-                       flags);
+    return dispatch_linear(ctx, (hipStream_t)stream, w, x_dev, x_dtype, y_dev, y_dtype, m, x_row_stride,
+                           y_row_stride, flags, true);
 }
 
 mi355q_status mi355q_qgemm(mi355q_context* ctx, void* stream, const mi355q_weight* w, const void* x_dev,
                            mi355q_dtype x_dtype, void* y_dev, mi355q_dtype y_dtype, uint32_t m,
                            uint32_t x_row_stride, uint32_t y_row_stride, uint32_t flags) {
     if (mi355q_status s = check_launch(ctx, w)) return s;
-    if (mi355q_status s = check_io(w, x_dev, x_dtype, y_dev, y_dtype, m, x_row_stride, y_row_stride)) return s;
-    if ((flags & MI355Q_FLAG_FORCE_MFMA) && (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)))
-        return fail(MI355Q_ERR_INVALID_ARGUMENT, "contradictory kernel selection flags");
-    const WView v = w->view();
-    const bool mfma_ok = gemm_mfma_eligible(v, x_dtype, m, x_row_stride);
-    if (flags & MI355Q_FLAG_FORCE_MFMA) {
-        if (!mfma_ok)
-            return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the MFMA GEMM does not accept this format, layout or stride");
-        return launch_qgemm_mfma((hipStream_t)stream, ctx, v, x_dev, x_dtype, y_dev, y_dtype, m, x_row_stride,
-                                 y_row_stride);
-    }
-    const bool small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) || m <= 8 || !mfma_ok;
-    if (small)
-        return run_small_m(ctx, (hipStream_t)stream, w, x_dev, x_dtype, y_dev, y_dtype, m, x_row_stride,
-                           y_row_stride, flags);
-    return launch_qgemm_mfma((hipStream_t)stream, ctx, v, x_dev, x_dtype, y_dev, y_dtype, m, x_row_stride,
-                             y_row_stride);
+    return dispatch_linear(ctx, (hipStream_t)stream, w, x_dev, x_dtype, y_dev, y_dtype, m, x_row_stride,
+                           y_row_stride, flags, false);
 }
 
 mi355q_status mi355q_batched_qgemm(mi355q_context* ctx, void* stream, uint32_t count,
@@ -155,21 +194,7 @@ mi355q_status mi355q_lmhead_argmax(mi355q_context* ctx, void* stream, const mi35
                                    mi355q_dtype x_dtype, float* logits_f32_dev, int32_t* token_out_dev,
                                    uint32_t flags) {
     if (mi355q_status s = check_launch(ctx, w)) return s;
-    if (!x_dev || !token_out_dev) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null pointer");
-    if (!dtype_ok(x_dtype)) return fail(MI355Q_ERR_INVALID_ARGUMENT, "bad dtype tag");
-    const WView v = w->view();
-    const uint32_t xs = (uint32_t)w->k;
-    if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && gemv_fast_eligible(v, x_dtype, 1, xs) && (uintptr_t)x_dev % 16 == 0)
-        return launch_gemv_fast((hipStream_t)stream, ctx, v, x_dev, nullptr, MI355Q_F32, 1, xs, (uint32_t)w->n,
-                                logits_f32_dev, token_out_dev, ctx->argmax_scratch);
-    // two dispatches, as the reference runs the head: projection to fp32 logits, then argmax
-    if (!logits_f32_dev)
-        return fail(MI355Q_ERR_INVALID_ARGUMENT,
-                    "a logits buffer is required when the fused head kernel does not accept the shape");
-    mi355q_status st = launch_gemv_generic((hipStream_t)stream, v, x_dev, x_dtype, logits_f32_dev, MI355Q_F32, 1, xs,
-                                           (uint32_t)w->n);
-    if (st != MI355Q_OK) return st;
-    return launch_argmax((hipStream_t)stream, logits_f32_dev, MI355Q_F32, (uint32_t)w->n, token_out_dev);
+    return dispatch_output_head(ctx, (hipStream_t)stream, w, x_dev, x_dtype, logits_f32_dev, token_out_dev, flags);
 }
 
 }  // extern "C"

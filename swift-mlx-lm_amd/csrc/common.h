@@ -38,6 +38,7 @@ struct WView {
     const uint32_t* codes;    // planes (layout 1)
     const uint16_t* scales;
     const uint16_t* biases;
+    const uint32_t* sz;       // planes: scale | bias << 16 per group (packed once at prepare time)
     uint32_t n, k;
     uint32_t group, bits;
     uint32_t bytes_per_block, blocks_per_row, words_per_row;
@@ -63,6 +64,7 @@ struct mi355q_weight {
     void* codes;
     void* scales;
     void* biases;
+    void* sz;                 // owned: packed (scale, bias) words for the planes layout
     size_t blocks_bytes, codes_bytes, sb_bytes;
     mi355q::WView view() const {
         mi355q::WView v;
@@ -70,6 +72,7 @@ struct mi355q_weight {
         v.codes = (const uint32_t*)codes;
         v.scales = (const uint16_t*)scales;
         v.biases = (const uint16_t*)biases;
+        v.sz = (const uint32_t*)sz;
         v.n = (uint32_t)n;
         v.k = (uint32_t)k;
         v.group = fmt.group_size;
@@ -94,6 +97,8 @@ mi355q_status launch_gemv_generic(hipStream_t s, const WView& w, const void* x, 
                                   uint32_t y_stride);
 mi355q_status launch_argmax(hipStream_t s, const void* logits, int dtype, uint32_t n,
                             int32_t* token_out);
+mi355q_status launch_pack_sz(hipStream_t s, const uint16_t* scales, const uint16_t* biases, uint32_t* sz,
+                             size_t groups);
 
 // Fast split-plane GEMV (kernels_gemv.hip).  can_* say whether a shape is eligible.
 bool gemv_fast_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
@@ -106,6 +111,14 @@ struct GemvLaunchShape {
     const char* kernel;
 };
 GemvLaunchShape gemv_fast_shape(const mi355q_context* ctx, const WView& w, uint32_t m);
+
+// Validated dispatch shared by the direct entry points and by plan replay (api.hip)
+mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_weight* w, const void* x, int x_dtype,
+                              void* y, int y_dtype, uint32_t m, uint32_t xs, uint32_t ys, uint32_t flags,
+                              bool small_m_only);
+mi355q_status dispatch_output_head(mi355q_context* ctx, hipStream_t s, const mi355q_weight* w, const void* x,
+                                   int x_dtype, float* logits, int32_t* token, uint32_t flags);
+int env_int_cached(const char* name, int fallback);
 
 // MFMA GEMM (kernels_gemm.hip)
 bool gemm_mfma_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);

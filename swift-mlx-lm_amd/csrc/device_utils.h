@@ -91,6 +91,46 @@ __device__ __forceinline__ float wave_reduce_sum(float v) {
            (__int_as_float(__builtin_amdgcn_readlane(iv, 32)) + __int_as_float(__builtin_amdgcn_readlane(iv, 48)));
 }
 
+// Value of lane (lane ^ MASK).  Quad permutes and the 8-lane rotation are DPP modifiers, 4 and 16
+// go through the swizzle crossbar, 32 through the permute crossbar; none touches LDS memory.
+template <int MASK>
+__device__ __forceinline__ float lane_xor(float v) {
+    if constexpr (MASK == 1) return dpp_f32<0xB1>(v);        // quad_perm [1,0,3,2]
+    else if constexpr (MASK == 2) return dpp_f32<0x4E>(v);   // quad_perm [2,3,0,1]
+    else if constexpr (MASK == 8) return dpp_f32<0x128>(v);  // row_ror:8
+    else if constexpr (MASK == 4) return __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x101F));
+    else if constexpr (MASK == 16) return __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x401F));
+    else return __shfl_xor(v, 32, 64);
+}
+
+// Reduces B per-lane partial sums (B rows, B a power of two <= 64) across the wavefront at once:
+// each stage halves the number of live values by letting the two lanes of a pair each keep one
+// row and hand the other over.  On return, lane l holds the complete sum of row (l & (B-1)).
+// About 3B operations instead of the 12B of B separate reductions.
+template <int B, int MASK = 1>
+__device__ __forceinline__ float transpose_reduce(float (&p)[B], uint32_t lane) {
+    if constexpr (B == 1) {
+        float v = p[0];
+        if constexpr (MASK <= 1) v += lane_xor<1>(v);
+        if constexpr (MASK <= 2) v += lane_xor<2>(v);
+        if constexpr (MASK <= 4) v += lane_xor<4>(v);
+        if constexpr (MASK <= 8) v += lane_xor<8>(v);
+        if constexpr (MASK <= 16) v += lane_xor<16>(v);
+        if constexpr (MASK <= 32) v += lane_xor<32>(v);
+        return v;
+    } else {
+        float q[B / 2];
+        const bool odd = (lane & MASK) != 0;
+#pragma unroll
+        for (int i = 0; i < B / 2; i++) {
+            const float keep = odd ? p[2 * i + 1] : p[2 * i];
+            const float send = odd ? p[2 * i] : p[2 * i + 1];
+            q[i] = keep + lane_xor<MASK>(send);
+        }
+        return transpose_reduce<B / 2, MASK * 2>(q, lane);
+    }
+}
+
 // (value, index) maximum with "greater, or equal and lower index"; every lane ends with the result.
 __device__ __forceinline__ void wave_argmax(float& v, uint32_t& idx) {
 #pragma unroll

@@ -4,7 +4,8 @@
 //   * every lane owns one "lane chunk" of a row per K-step: WPL consecutive code words
 //     (128-bit load for 2/4/8-bit, 96-bit for 3/6-bit, so straddling codes never cross lanes);
 //     a wavefront therefore reads 64*WPL*4 contiguous bytes of one row per load instruction;
-//   * a wavefront carries R rows at once and prefetches the next K-step while it computes;
+//   * a wavefront owns a run of consecutive rows, carries R of them at once and keeps its loads
+//     D pipeline steps ahead of the arithmetic in a register ring;
 //   * activations are staged once per workgroup in LDS, already permuted into the pair order
 //     the unpacker produces, laid out [m][k-step][piece][lane] so reads are conflict-free b128;
 //   * 2/4-bit codes become bf16 pairs (128+q) with one and-or each and go through
@@ -38,8 +39,7 @@ __device__ __forceinline__ void static_for(F&& f) {
 
 struct GemvArgs {
     const uint32_t* codes;
-    const uint16_t* scales;
-    const uint16_t* biases;
+    const uint32_t* sz;      // packed (scale | bias << 16) word per group
     const uint16_t* x;       // bf16 [M, x_stride]
     void* y;                 // [M, y_stride] in y_dtype (may be null when only logits are wanted)
     float* logits;           // optional fp32 [N] copy (M == 1)
@@ -49,8 +49,19 @@ struct GemvArgs {
     uint32_t x_stride, y_stride;
     uint32_t words_per_row, blocks_per_row;
     uint32_t nc;             // K-steps per row = ceil(K / (64*CPL))
-    uint32_t nrb;            // row blocks = ceil(N / (4*R))
+    uint32_t rows_per_wave;  // consecutive rows owned by one wavefront
     uint32_t y_dtype, sb_dtype;
+    uint32_t dbg;            // tuning builds only: bit0 no scale/bias loads, bit1 no arithmetic, bit2 no staging
+};
+
+// Host-side choice of kernel variant and launch shape.
+struct GemvCfg {
+    int r, mt;          // rows per pipeline step, activation rows (1, 2, 4, 8)
+    bool argmax;
+    int waves, depth;   // wavefronts per workgroup, prefetch ring depth
+    int xreg;           // 0: activations read from LDS each step; 1/2: register-resident (K-steps per row)
+    uint32_t grid, rows_per_wave, nc;
+    size_t lds;
 };
 
 template <int BITS> struct GemvGeo;
@@ -88,8 +99,24 @@ __device__ __forceinline__ uint32_t extract_code(const uint32_t (&w)[WPL]) {
     }
 }
 
-template <int BITS, int GROUP, int R, int MT, bool ARGMAX>
-__global__ __launch_bounds__(256) void gemv_planes_kernel(GemvArgs a) {
+// One wavefront owns `rows_per_wave` consecutive rows and walks them R at a time, one K-step
+// (64 lane chunks) per pipeline step.  Every wavefront runs the same number of steps (rows past
+// the end are clamped for loading and masked for storing), so the kernel has no data-dependent
+// control flow around its loads:
+//   1. the activation loads are issued first (vector loads return in issue order, so they must
+//      not queue behind the weight stream),
+//   2. then D steps of weight loads -- for short rows that is the wavefront's whole share --
+//   3. the activations are permuted into LDS behind an LDS-only barrier while the weights are
+//      still in flight,
+//   4. a software pipeline (prologue / steady loop / epilogue over a register ring of D steps)
+//      does the arithmetic as the data lands,
+//   5. row results are parked one per lane and written with a single coalesced store at the end:
+//      a store inside the loop would share the wait counter with the loads and drain the ring.
+// XREG = 1 or 2 means rows are exactly that many K-steps long and the wavefront keeps its
+// activation slice in registers; XREG = 0 re-reads the slice from LDS at every step
+// (conflict-free 128-bit reads shared by the R rows).
+template <int BITS, int GROUP, int R, int MT, bool ARGMAX, int WAVES, int D, int XREG>
+__global__ __launch_bounds__(WAVES * 64) void gemv_planes_kernel(GemvArgs a) {
     using G = GemvGeo<BITS>;
     constexpr int WPL = G::WPL, CPL = G::CPL;
     constexpr int Q = CPL / 8;                          // uint4 pieces (8 codes) per lane chunk
@@ -97,6 +124,9 @@ __global__ __launch_bounds__(256) void gemv_planes_kernel(GemvArgs a) {
     constexpr int NSR = CPL / SR;                       // sub-runs (groups touched) per lane chunk
     constexpr int KC = 64 * CPL;                        // codes per wavefront K-step
     constexpr float OFS = G::PAIRS ? 128.0f : 0.0f;     // magic offset carried by the bf16 codes
+    constexpr int XC = XREG ? XREG : 1;                 // K-steps cached in registers
+    static_assert(XREG == 0 || (MT == 1 && R == 1), "register-resident activations are for M == 1, R == 1");
+    static_assert(XREG == 0 || D % XREG == 0, "ring depth must be a multiple of the K-steps per row");
 
     extern __shared__ uint4 smem[];
     const uint32_t NC = a.nc;
@@ -104,65 +134,59 @@ __global__ __launch_bounds__(256) void gemv_planes_kernel(GemvArgs a) {
     float* sxs = (float*)(smem + (size_t)MT * NC * Q * 64); // [MT][NC][NSR][64]
 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t row0 = (blockIdx.x * WAVES + wave) * a.rows_per_wave;
+    const uint32_t nsteps = (a.rows_per_wave / R) * NC;     // same for every wavefront, >= 1
 
     struct Pref {
         uint32_t w[R][WPL];
-        uint16_t s[R][NSR], z[R][NSR];
+        uint32_t sz[R][NSR];
     };
 
-    auto issue = [&](uint32_t rb, uint32_t c, Pref& p) {
-        const uint32_t chunk = c * 64 + lane;               // lane-chunk index inside the row
-        const bool live = (uint64_t)chunk * CPL < a.k;
+    // Unconditional loads: rows past N and lane chunks past K are clamped to valid addresses.
+    // A clamped lane chunk meets activations staged as zero, a clamped row is never stored.
+    auto issue = [&](uint32_t rg, uint32_t c, Pref& p) {
+        uint32_t chunk = c * 64 + lane;                     // lane-chunk index inside the row
+        chunk = (uint64_t)chunk * CPL < a.k ? chunk : 0;
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            uint32_t row = rb * (4 * R) + wave * R + r;
-            row = row < a.n ? row : a.n - 1;                // clamp: results of such rows are dropped
-            if (live) {
-                const uint32_t* src = a.codes + (size_t)row * a.words_per_row + (size_t)chunk * WPL;
-                if constexpr (WPL == 4) {
-                    const uint4 v = *(const uint4*)src;
-                    p.w[r][0] = v.x; p.w[r][1] = v.y; p.w[r][2] = v.z; p.w[r][3] = v.w;
-                } else {
-#pragma unroll
-                    for (int i = 0; i < WPL; i++) p.w[r][i] = src[i];
-                }
-#pragma unroll
-                for (int sr = 0; sr < NSR; sr++) {
-                    const size_t g = (size_t)row * a.blocks_per_row + ((size_t)chunk * CPL + sr * SR) / GROUP;
-                    p.s[r][sr] = a.scales[g];
-                    p.z[r][sr] = a.biases[g];
-                }
+            uint32_t row = row0 + rg * R + r;
+            row = row < a.n ? row : a.n - 1;
+            const uint32_t* src = a.codes + (size_t)row * a.words_per_row + (size_t)chunk * WPL;
+            if constexpr (WPL == 4) {
+                const uint4 v = *(const uint4*)src;
+                p.w[r][0] = v.x; p.w[r][1] = v.y; p.w[r][2] = v.z; p.w[r][3] = v.w;
             } else {
 #pragma unroll
-                for (int i = 0; i < WPL; i++) p.w[r][i] = 0;
+                for (int i = 0; i < WPL; i++) p.w[r][i] = src[i];
+            }
 #pragma unroll
-                for (int sr = 0; sr < NSR; sr++) { p.s[r][sr] = 0; p.z[r][sr] = 0; }
+            for (int sr = 0; sr < NSR; sr++) {
+                const size_t g = (size_t)row * a.blocks_per_row + ((size_t)chunk * CPL + sr * SR) / GROUP;
+#ifdef MI355Q_GEMV_EXPERIMENT
+                if (a.dbg & 1) { p.sz[r][sr] = 0x38003C00u; continue; }
+#endif
+                p.sz[r][sr] = a.sz[g];
             }
         }
     };
 
-    // ---- first weight loads go out before the activations are staged ------------------------
-    uint32_t rb = blockIdx.x, c = 0;
-    bool have = rb < a.nrb;
-    Pref nxt;
-    if (have) issue(rb, 0, nxt);
-
-    // ---- stage activations: one task = one lane chunk of one activation row -----------------
-    for (uint32_t task = tid; task < (uint32_t)MT * NC * 64; task += 256) {
+    // ---- staging helpers: one task = one lane chunk of one activation row ---------------------
+    const uint32_t ntasks = (uint32_t)MT * NC * 64;
+    auto stage_load = [&](uint32_t task, uint32_t (&d)[CPL / 2]) {
         const uint32_t l = task & 63, cc = (task >> 6) % NC, m = (task >> 6) / NC;
         const uint64_t kbase = (uint64_t)cc * KC + (uint64_t)l * CPL;
-        uint32_t d[CPL / 2];
-        if (m < a.m && kbase < a.k) {
-            const uint4* src = (const uint4*)(a.x + (size_t)m * a.x_stride + kbase);
+        const bool valid = task < ntasks && m < a.m && kbase < a.k;
+        const uint4* src = (const uint4*)(a.x + (valid ? (size_t)m * a.x_stride + kbase : 0));
 #pragma unroll
-            for (int i = 0; i < Q; i++) {
-                const uint4 v = src[i];
-                d[4 * i + 0] = v.x; d[4 * i + 1] = v.y; d[4 * i + 2] = v.z; d[4 * i + 3] = v.w;
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < CPL / 2; i++) d[i] = 0;
+        for (int i = 0; i < Q; i++) {
+            const uint4 v = src[i];                         // clamped address: always readable
+            d[4 * i + 0] = valid ? v.x : 0; d[4 * i + 1] = valid ? v.y : 0;
+            d[4 * i + 2] = valid ? v.z : 0; d[4 * i + 3] = valid ? v.w : 0;
         }
+    };
+    auto stage_store = [&](uint32_t task, const uint32_t (&d)[CPL / 2]) {
+        if (task >= ntasks) return;                         // LDS writes only inside this branch
+        const uint32_t l = task & 63, cc = (task >> 6) % NC, m = (task >> 6) / NC;
         auto elem = [&](int e) -> uint32_t { return (e & 1) ? (d[e >> 1] >> 16) : (d[e >> 1] & 0xFFFFu); };
 #pragma unroll
         for (int i = 0; i < Q; i++) {
@@ -180,24 +204,130 @@ __global__ __launch_bounds__(256) void gemv_planes_kernel(GemvArgs a) {
             for (int e = 0; e < SR; e++) sx += __uint_as_float(elem(sr * SR + e) << 16);
             sxs[((size_t)(m * NC + cc) * NSR + sr) * 64 + l] = sx;
         }
+    };
+
+    // ---- 1. activation loads first ------------------------------------------------------------
+    constexpr int TE = 2;                                   // early staging tasks per thread
+    uint32_t dearly[TE][CPL / 2];
+#pragma unroll
+    for (int t = 0; t < TE; t++) stage_load(tid + t * (WAVES * 64), dearly[t]);
+
+    // ---- 2. the first D steps of weight loads -------------------------------------------------
+    // Steps past the last one repeat it (same addresses, so they hit in L2 and their data is
+    // never used); this keeps every load unconditional.
+    Pref ring[D];
+    uint32_t irg = 0, ic = 0, istep = 0;                    // next step to issue
+    auto advance = [&]() {
+        if (istep + 1 < nsteps) {
+            istep++;
+            if (++ic == NC) { ic = 0; irg++; }
+        }
+    };
+    static_for<D>([&](auto J) {
+        constexpr int j = decltype(J)::value;
+        issue(irg, ic, ring[j]);
+        advance();
+    });
+
+    // ---- 3. permute the activations into LDS (waits only for the loads of step 1) -------------
+#ifdef MI355Q_GEMV_EXPERIMENT
+    if (!(a.dbg & 4))
+#endif
+    {
+#pragma unroll
+        for (int t = 0; t < TE; t++) stage_store(tid + t * (WAVES * 64), dearly[t]);
+        for (uint32_t task = tid + TE * (WAVES * 64); task < ntasks; task += WAVES * 64) {
+            uint32_t dl[CPL / 2];                           // large batches: the remaining tasks
+            stage_load(task, dl);
+            stage_store(task, dl);
+        }
     }
-    __syncthreads();
+    // LDS-only barrier: the weight loads in flight must not be waited for here
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+
+    // ---- optional register-resident activation slice (M == 1, rows of XREG K-steps) -----------
+    uint4 xr[XC][Q];
+    float sxr[XC][NSR];
+    if constexpr (XREG != 0) {
+#pragma unroll
+        for (int cc = 0; cc < XC; cc++) {
+#pragma unroll
+            for (int p = 0; p < Q; p++) xr[cc][p] = xs[((size_t)cc * Q + p) * 64 + lane];
+#pragma unroll
+            for (int sr = 0; sr < NSR; sr++) sxr[cc][sr] = sxs[((size_t)cc * NSR + sr) * 64 + lane];
+        }
+    }
+
+    // The pair mask lives in an SGPR and the bf16 "128.0" pair in a VGPR, both opaque to the
+    // optimiser, so that (w & mask) | magic is one v_and_or_b32 instead of an AND and an OR with
+    // literals (a VOP3 instruction takes no literal and a single scalar operand on this target).
+    uint32_t k_magic = 0x43004300u;
+    uint32_t k_mask = BITS == 4 ? 0x000F000Fu : 0x00030003u;
+    asm volatile("" : "+v"(k_magic));
+    asm volatile("" : "+s"(k_mask));
 
     float acc[R][MT];
+    float res[MT];                   // lane i parks the result of the wavefront's i-th row
 #pragma unroll
-    for (int r = 0; r < R; r++)
+    for (int m = 0; m < MT; m++) {
+        res[m] = 0.0f;
 #pragma unroll
-        for (int m = 0; m < MT; m++) acc[r][m] = 0.0f;
+        for (int r = 0; r < R; r++) acc[r][m] = 0.0f;
+    }
 
-    unsigned long long best = 0ull;  // ARGMAX: packed (ordered value, ~row); 0 = nothing seen
+    unsigned long long best = 0ull;  // ARGMAX, per lane: packed (ordered value, ~row); 0 = nothing seen
+    uint32_t rg = 0, c = 0;          // step being computed
+    constexpr int BR = XREG ? D / XC : 1;   // rows completed per ring pass when rows are XREG steps long
+    float part[BR];                  // their per-lane partial sums, reduced together
+#pragma unroll
+    for (int i = 0; i < BR; i++) part[i] = 0.0f;
 
-    while (have) {
-        Pref cur = nxt;
-        uint32_t c2 = c + 1, rb2 = rb;
-        if (c2 == NC) { c2 = 0; rb2 = rb + gridDim.x; }
-        const bool have2 = rb2 < a.nrb;
-        if (have2) issue(rb2, c2, nxt);
+    auto flush = [&](uint32_t first_local, uint32_t count) {   // rows [first_local, +count) -> memory
+        const uint32_t row = row0 + first_local + lane;
+        if (lane < count && row < a.n) {
+#pragma unroll
+            for (int m = 0; m < MT; m++) {
+                if ((uint32_t)m < a.m) {
+                    if (a.y) {
+                        const size_t o = (size_t)m * a.y_stride + row;
+                        if (a.y_dtype == MI355Q_F32) ((float*)a.y)[o] = res[m];
+                        else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)a.y)[o] = f32_to_bf16_rne(res[m]);
+                        else ((uint16_t*)a.y)[o] = f32_to_f16_rne(res[m]);
+                    }
+                    if (a.logits && m == 0) a.logits[row] = res[m];
+                }
+            }
+            if constexpr (ARGMAX) {
+                const float v = res[0];
+                if (v > -INFINITY) {                         // NaN and -inf never contribute
+                    const uint32_t u = __float_as_uint(v + 0.0f);   // -0 -> +0
+                    const uint32_t key = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+                    const unsigned long long pk =
+                        ((unsigned long long)key << 32) | (unsigned long long)(0xFFFFFFFFu - row);
+                    best = pk > best ? pk : best;
+                }
+            }
+        }
+    };
 
+    // J: ring slot.  When rows are XREG steps long the K-step index of a slot is a compile-time
+    // constant (cj) and so is the slot at which a row completes.
+    auto compute = [&](const Pref& cur, auto J) {
+        constexpr int cj = XREG ? decltype(J)::value % XC : 0;
+#ifdef MI355Q_GEMV_EXPERIMENT
+        if (a.dbg & 2) {
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                uint32_t t = 0;
+#pragma unroll
+                for (int i = 0; i < WPL; i++) t ^= cur.w[r][i];
+                acc[r][0] += __uint_as_float(t & 0x3FFFFFFFu) + __uint_as_float(cur.sz[r][0] & 0x3FFFFFFFu);
+            }
+        } else
+#endif
+        {
         // ---- one K-step of R rows ----------------------------------------------------------
         float dot[R][MT][NSR];
 #pragma unroll
@@ -211,8 +341,12 @@ __global__ __launch_bounds__(256) void gemv_planes_kernel(GemvArgs a) {
             constexpr int p = decltype(P)::value;
             constexpr int sr = (p * 8) / SR;
             uint4 xv[MT];
+            if constexpr (XREG != 0) {
+                xv[0] = xr[cj][p];
+            } else {
 #pragma unroll
-            for (int m = 0; m < MT; m++) xv[m] = xs[((size_t)(m * NC + c) * Q + p) * 64 + lane];
+                for (int m = 0; m < MT; m++) xv[m] = xs[((size_t)(m * NC + c) * Q + p) * 64 + lane];
+            }
 
             if constexpr (G::PAIRS) {
 #pragma unroll
@@ -220,16 +354,16 @@ __global__ __launch_bounds__(256) void gemv_planes_kernel(GemvArgs a) {
                     uint32_t pr[4];
                     if constexpr (BITS == 4) {
                         const uint32_t wv = cur.w[r][p];
-                        pr[0] = (wv & 0x000F000Fu) | 0x43004300u;
-                        pr[1] = ((wv >> 4) & 0x000F000Fu) | 0x43004300u;
-                        pr[2] = ((wv >> 8) & 0x000F000Fu) | 0x43004300u;
-                        pr[3] = ((wv >> 12) & 0x000F000Fu) | 0x43004300u;
+                        pr[0] = (wv & k_mask) | k_magic;
+                        pr[1] = ((wv >> 4) & k_mask) | k_magic;
+                        pr[2] = ((wv >> 8) & k_mask) | k_magic;
+                        pr[3] = ((wv >> 12) & k_mask) | k_magic;
                     } else {  // BITS == 2: word p/2, shifts 2*(4*(p&1) + i)
                         const uint32_t wv = cur.w[r][p >> 1] >> (8 * (p & 1));
-                        pr[0] = (wv & 0x00030003u) | 0x43004300u;
-                        pr[1] = ((wv >> 2) & 0x00030003u) | 0x43004300u;
-                        pr[2] = ((wv >> 4) & 0x00030003u) | 0x43004300u;
-                        pr[3] = ((wv >> 6) & 0x00030003u) | 0x43004300u;
+                        pr[0] = (wv & k_mask) | k_magic;
+                        pr[1] = ((wv >> 2) & k_mask) | k_magic;
+                        pr[2] = ((wv >> 4) & k_mask) | k_magic;
+                        pr[3] = ((wv >> 6) & k_mask) | k_magic;
                     }
 #pragma unroll
                     for (int m = 0; m < MT; m++) {
@@ -276,57 +410,102 @@ __global__ __launch_bounds__(256) void gemv_planes_kernel(GemvArgs a) {
 #pragma unroll
         for (int sr = 0; sr < NSR; sr++) {
             float sx[MT];
+            if constexpr (XREG != 0) {
+                sx[0] = sxr[cj][sr];
+            } else {
 #pragma unroll
-            for (int m = 0; m < MT; m++) sx[m] = sxs[((size_t)(m * NC + c) * NSR + sr) * 64 + lane];
+                for (int m = 0; m < MT; m++) sx[m] = sxs[((size_t)(m * NC + c) * NSR + sr) * 64 + lane];
+            }
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                const float s = sb_to_f32(cur.s[r][sr], a.sb_dtype);
-                const float z = sb_to_f32(cur.z[r][sr], a.sb_dtype);
+                float s, z;
+                const uint32_t szw = cur.sz[r][sr];
+                if (a.sb_dtype == MI355Q_BF16) {            // wavefront-uniform branch
+                    s = __uint_as_float(szw << 16); z = __uint_as_float(szw & 0xFFFF0000u);
+                } else {
+                    s = f16_to_f32((uint16_t)(szw & 0xFFFFu)); z = f16_to_f32((uint16_t)(szw >> 16));
+                }
                 const float zc = z - OFS * s;
 #pragma unroll
                 for (int m = 0; m < MT; m++) acc[r][m] += s * dot[r][m][sr] + zc * sx[m];
             }
         }
-
-        // ---- row block complete: reduce across the wavefront and store ----------------------
-        if (c == NC - 1) {
+        }
+        if constexpr (XREG != 0) {
+            // ---- row complete at a known slot: keep its per-lane partial for the batched reduce -----
+            if constexpr (cj == XC - 1) {
+                part[decltype(J)::value / XC] = acc[0][0];
+                acc[0][0] = 0.0f;
+            }
+        } else {
+            // ---- rows complete: reduce across the wavefront, park the result in its lane ---------
+            if (c == NC - 1) {
 #pragma unroll
-            for (int r = 0; r < R; r++) {
-                const uint32_t row = rb * (4 * R) + wave * R + r;
+                for (int r = 0; r < R; r++) {
+                    const uint32_t local = rg * R + r;
 #pragma unroll
-                for (int m = 0; m < MT; m++) {
-                    const float tot = wave_reduce_sum(acc[r][m]);
-                    acc[r][m] = 0.0f;
-                    if (row < a.n && (uint32_t)m < a.m) {
-                        if (lane == 0) {
-                            if (a.y) {
-                                const size_t o = (size_t)m * a.y_stride + row;
-                                if (a.y_dtype == MI355Q_F32) ((float*)a.y)[o] = tot;
-                                else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)a.y)[o] = f32_to_bf16_rne(tot);
-                                else ((uint16_t*)a.y)[o] = f32_to_f16_rne(tot);
-                            }
-                            if (a.logits && m == 0) a.logits[row] = tot;
-                        }
-                        if constexpr (ARGMAX) {
-                            if (m == 0 && tot > -INFINITY) {  // NaN and -inf never contribute
-                                const uint32_t u = __float_as_uint(tot + 0.0f);  // -0 -> +0
-                                const uint32_t key = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-                                const unsigned long long pk =
-                                    ((unsigned long long)key << 32) | (unsigned long long)(0xFFFFFFFFu - row);
-                                best = pk > best ? pk : best;
-                            }
-                        }
+                    for (int m = 0; m < MT; m++) {
+                        const float tot = wave_reduce_sum(acc[r][m]);
+                        acc[r][m] = 0.0f;
+                        res[m] = (lane == (local & 63u)) ? tot : res[m];
                     }
+                    // a wavefront that owns more than 64 rows empties its lanes every 64 rows
+                    if ((local & 63u) == 63u && local + 1 < a.rows_per_wave) flush(local - 63u, 64u);
                 }
             }
+            if (++c == NC) { c = 0; rg++; }
         }
-        rb = rb2; c = c2; have = have2;
+    };
+
+    // After a ring pass over rows of XREG steps: BR rows are complete; reduce them together and
+    // park row (pass*BR + i) in lane ((pass*BR + i) & 63).
+    auto finish_pass = [&](uint32_t pass) {
+        if constexpr (XREG != 0) {
+            const float v = transpose_reduce<BR>(part, lane);
+            const uint32_t base = (pass * BR) & 63u;
+            res[0] = ((lane & ~(uint32_t)(BR - 1)) == base) ? v : res[0];
+            const uint32_t done = (pass + 1) * BR;
+            if ((done & 63u) == 0u && done < a.rows_per_wave) flush(done - 64u, 64u);
+        }
+    };
+
+    // ---- 4. software pipeline: steady loop (compute a slot, refill it), then drain ------------
+    const uint32_t groups = (nsteps + D - 1) / D;
+    for (uint32_t it = 0; it + 1 < groups; it++) {
+        static_for<D>([&](auto J) {
+            constexpr int j = decltype(J)::value;
+            compute(ring[j], J);
+            issue(irg, ic, ring[j]);
+            advance();
+        });
+        finish_pass(it);
+    }
+    const uint32_t tail = nsteps - (groups - 1) * D;        // 1..D steps left in the ring
+    static_for<D>([&](auto J) {
+        constexpr int j = decltype(J)::value;
+        if ((uint32_t)j < tail) compute(ring[j], J);
+    });
+    finish_pass(groups - 1);
+
+    // ---- 5. one coalesced store of the parked results -----------------------------------------
+    {
+        const uint32_t done = a.rows_per_wave;
+        const uint32_t first = (done - 1) & ~63u;           // start of the last (partial) block of 64
+        flush(first, done - first);
     }
 
     if constexpr (ARGMAX) {
-        // `best` is wavefront-uniform.  One atomic per wavefront, then a ticket: the workgroup that
-        // draws the last ticket publishes the token and leaves the scratch cells zeroed again.
+        // Per-lane candidates -> wavefront maximum (butterfly on the packed 64-bit key), one atomic
+        // per wavefront, then a ticket: the workgroup that draws the last ticket publishes the
+        // token and leaves the scratch cells zeroed again.
         __shared__ uint32_t s_last;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const uint32_t hi = (uint32_t)__shfl_xor((int)(best >> 32), off, 64);
+            const uint32_t lo = (uint32_t)__shfl_xor((int)(best & 0xFFFFFFFFull), off, 64);
+            const unsigned long long o = ((unsigned long long)hi << 32) | lo;
+            best = o > best ? o : best;
+        }
         if (lane == 0 && best) atomicMax(&a.scratch[0], best);
         __threadfence();
         __syncthreads();

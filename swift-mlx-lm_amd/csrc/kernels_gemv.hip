@@ -5,12 +5,12 @@
 
 namespace mi355q {
 
-mi355q_status launch_gemv_planes_q2(hipStream_t, const GemvArgs&, int, int, int, bool, uint32_t, size_t);
-mi355q_status launch_gemv_planes_q3(hipStream_t, const GemvArgs&, int, int, int, bool, uint32_t, size_t);
-mi355q_status launch_gemv_planes_q4(hipStream_t, const GemvArgs&, int, int, int, bool, uint32_t, size_t);
-mi355q_status launch_gemv_planes_q5(hipStream_t, const GemvArgs&, int, int, int, bool, uint32_t, size_t);
-mi355q_status launch_gemv_planes_q6(hipStream_t, const GemvArgs&, int, int, int, bool, uint32_t, size_t);
-mi355q_status launch_gemv_planes_q8(hipStream_t, const GemvArgs&, int, int, int, bool, uint32_t, size_t);
+mi355q_status launch_gemv_planes_q2(hipStream_t, const GemvArgs&, int, const GemvCfg&);
+mi355q_status launch_gemv_planes_q3(hipStream_t, const GemvArgs&, int, const GemvCfg&);
+mi355q_status launch_gemv_planes_q4(hipStream_t, const GemvArgs&, int, const GemvCfg&);
+mi355q_status launch_gemv_planes_q5(hipStream_t, const GemvArgs&, int, const GemvCfg&);
+mi355q_status launch_gemv_planes_q6(hipStream_t, const GemvArgs&, int, const GemvCfg&);
+mi355q_status launch_gemv_planes_q8(hipStream_t, const GemvArgs&, int, const GemvCfg&);
 
 namespace {
 
@@ -38,10 +38,7 @@ size_t lds_bytes(const WView& w, int mt) {
     return (size_t)mt * nc * 64 * ((size_t)(g.cpl / 8) * 16 + nsr * 4);
 }
 
-int env_int(const char* name, int fallback) {
-    const char* v = std::getenv(name);
-    return (v && *v) ? std::atoi(v) : fallback;
-}
+int env_int(const char* name, int fallback) { return env_int_cached(name, fallback); }
 
 // Largest activation batch (1, 2, 4 or 8) whose staged activations fit the LDS budget.
 int max_mt(const WView& w) {
@@ -50,31 +47,46 @@ int max_mt(const WView& w) {
     return 0;
 }
 
-struct Choice { int r, mt; uint32_t grid, nrb, nc; size_t lds; };
-
-Choice choose(const mi355q_context* ctx, const WView& w, uint32_t m, bool argmax) {
-    Choice c{};
+// Variant and launch shape for one call.  In tuning builds (MI355Q_GEMV_EXPERIMENT) environment
+// variables override the heuristics (MI355Q_GEMV_R, _WAVES, _DEPTH, _XREG, _ROWS_PER_WAVE,
+// _WAVES_PER_CU); product builds ignore them.
+GemvCfg choose(const mi355q_context* ctx, const WView& w, uint32_t m, bool argmax) {
+    GemvCfg c{};
+    c.argmax = argmax;
     c.mt = m <= 1 ? 1 : m <= 2 ? 2 : m <= 4 ? 4 : 8;
-    if (c.mt == 1) {
-        // rows per wavefront: more rows in flight per lane once there are enough rows to go round
-        c.r = w.n >= 8192 ? 4 : (w.n >= 2048 ? 2 : 1);
-        const int forced = env_int("MI355Q_GEMV_ROWS_PER_WAVE", 0);
-        if (forced == 1 || forced == 2 || forced == 4) c.r = forced;
-    } else {
-        c.r = c.mt == 8 ? 1 : 2;
-    }
-    (void)argmax;
     const Geo g = geo_for(w.bits);
     const size_t kc = 64 * (size_t)g.cpl;
     c.nc = (uint32_t)((w.k + kc - 1) / kc);
-    c.nrb = (w.n + 4 * c.r - 1) / (4 * c.r);
+    c.waves = 4;
+    if (c.mt == 1) {
+        c.xreg = c.nc <= 2 ? (int)c.nc : 0;     // short rows: activation slice lives in registers
+        c.r = 1;
+    } else {
+        c.xreg = 0;
+        c.r = c.mt == 8 ? 1 : 2;
+    }
+    const int er = env_int("MI355Q_GEMV_R", 0), ew = env_int("MI355Q_GEMV_WAVES", 0),
+              ed = env_int("MI355Q_GEMV_DEPTH", 0), ex = env_int("MI355Q_GEMV_XREG", -1);
+    if (er) c.r = er;
+    if (ew) c.waves = ew;
+    if (ex >= 0) c.xreg = ex ? (int)c.nc : 0;
     c.lds = lds_bytes(w, c.mt);
-    int per_cu = env_int("MI355Q_GEMV_WGS_PER_CU", 4);
-    const size_t fit = c.lds ? (160 * 1024) / c.lds : 8;
-    if ((size_t)per_cu > fit) per_cu = (int)(fit ? fit : 1);
-    if (per_cu < 1) per_cu = 1;
-    const uint32_t cap = (uint32_t)ctx->props.multiProcessorCount * (uint32_t)per_cu;
-    c.grid = c.nrb < cap ? c.nrb : cap;
+    // rows per wavefront: aim for `per_cu` wavefronts on every CU, each owning whole R-row steps
+    const uint32_t per_cu = (uint32_t)env_int("MI355Q_GEMV_WAVES_PER_CU", 16);
+    const uint32_t target = (uint32_t)ctx->props.multiProcessorCount * (per_cu ? per_cu : 16);
+    uint32_t rpw = (w.n + target - 1) / target;
+    const int forced = env_int("MI355Q_GEMV_ROWS_PER_WAVE", 0);
+    if (forced > 0) rpw = (uint32_t)forced;
+    rpw = (rpw + c.r - 1) / c.r * c.r;
+    if (rpw < (uint32_t)c.r) rpw = c.r;
+    c.rows_per_wave = rpw;
+    // ring depth: the whole share of a wavefront when it is short, else 8 steps in flight
+    const uint32_t nsteps = rpw / (uint32_t)c.r * c.nc;
+    if (c.mt == 1) c.depth = nsteps >= 6 ? 8 : nsteps >= 3 ? 4 : 2;
+    else c.depth = c.mt == 2 ? 4 : 2;
+    if (ed) c.depth = ed;
+    const uint32_t rows_per_wg = rpw * (uint32_t)c.waves;
+    c.grid = (w.n + rows_per_wg - 1) / rows_per_wg;
     if (c.grid == 0) c.grid = 1;
     return c;
 }
@@ -89,6 +101,7 @@ bool gemv_fast_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stri
     if (w.k % (uint32_t)g.cpl) return false;       // rows are whole lane chunks
     if (x_stride % 8) return false;                // 128-bit activation loads
     if ((uintptr_t)w.codes % 16) return false;     // 128-bit code loads
+    if (!w.sz) return false;
     if (max_mt(w) == 0) return false;
     return true;
 }
@@ -96,12 +109,12 @@ bool gemv_fast_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stri
 GemvLaunchShape gemv_fast_shape(const mi355q_context* ctx, const WView& w, uint32_t m) {
     const int fit = max_mt(w);
     const uint32_t mm = (fit && m > (uint32_t)fit) ? (uint32_t)fit : m;
-    const Choice c = choose(ctx, w, mm, false);
+    const GemvCfg c = choose(ctx, w, mm, false);
     GemvLaunchShape s;
     s.grid = c.grid;
-    s.block = 256;
+    s.block = (uint32_t)c.waves * 64;
     s.lds_bytes = (uint32_t)c.lds;
-    s.rows_per_workgroup = (uint32_t)(4 * c.r);
+    s.rows_per_workgroup = c.rows_per_wave * (uint32_t)c.waves;
     s.kernel = "gemv_planes_kernel";
     return s;
 }
@@ -118,11 +131,10 @@ mi355q_status launch_gemv_fast(hipStream_t s, const mi355q_context* ctx, const W
     // activation batches larger than what fits in LDS are processed in slices of `fit` rows
     for (uint32_t m0 = 0; m0 < m; m0 += (uint32_t)fit) {
         const uint32_t mm = (m - m0) < (uint32_t)fit ? (m - m0) : (uint32_t)fit;
-        const Choice c = choose(ctx, w, mm, argmax);
+        const GemvCfg c = choose(ctx, w, mm, argmax);
         GemvArgs a{};
         a.codes = w.codes;
-        a.scales = w.scales;
-        a.biases = w.biases;
+        a.sz = w.sz;
         a.x = (const uint16_t*)x + (size_t)m0 * x_stride;
         a.y = y ? (void*)((char*)y + (size_t)m0 * y_stride * ysz) : nullptr;
         a.logits = logits_f32;
@@ -131,16 +143,17 @@ mi355q_status launch_gemv_fast(hipStream_t s, const mi355q_context* ctx, const W
         a.n = w.n; a.k = w.k; a.m = mm;
         a.x_stride = x_stride; a.y_stride = y_stride;
         a.words_per_row = w.words_per_row; a.blocks_per_row = w.blocks_per_row;
-        a.nc = c.nc; a.nrb = c.nrb;
+        a.nc = c.nc; a.rows_per_wave = c.rows_per_wave;
         a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = w.sb_dtype;
+        a.dbg = (uint32_t)env_int("MI355Q_GEMV_DBG", 0);
         mi355q_status st;
         switch (w.bits) {
-        case 2: st = launch_gemv_planes_q2(s, a, (int)w.group, c.r, c.mt, argmax, c.grid, c.lds); break;
-        case 3: st = launch_gemv_planes_q3(s, a, (int)w.group, c.r, c.mt, argmax, c.grid, c.lds); break;
-        case 4: st = launch_gemv_planes_q4(s, a, (int)w.group, c.r, c.mt, argmax, c.grid, c.lds); break;
-        case 5: st = launch_gemv_planes_q5(s, a, (int)w.group, c.r, c.mt, argmax, c.grid, c.lds); break;
-        case 6: st = launch_gemv_planes_q6(s, a, (int)w.group, c.r, c.mt, argmax, c.grid, c.lds); break;
-        case 8: st = launch_gemv_planes_q8(s, a, (int)w.group, c.r, c.mt, argmax, c.grid, c.lds); break;
+        case 2: st = launch_gemv_planes_q2(s, a, (int)w.group, c); break;
+        case 3: st = launch_gemv_planes_q3(s, a, (int)w.group, c); break;
+        case 4: st = launch_gemv_planes_q4(s, a, (int)w.group, c); break;
+        case 5: st = launch_gemv_planes_q5(s, a, (int)w.group, c); break;
+        case 6: st = launch_gemv_planes_q6(s, a, (int)w.group, c); break;
+        case 8: st = launch_gemv_planes_q8(s, a, (int)w.group, c); break;
         default: st = fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no split-plane GEMV for %u-bit codes", w.bits);
         }
         if (st != MI355Q_OK) return st;

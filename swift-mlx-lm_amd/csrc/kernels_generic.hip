@@ -31,6 +31,27 @@ mi355q_status launch_unpack_codes(hipStream_t s, const WView& w, uint8_t* out) {
     return MI355Q_OK;
 }
 
+// ------------------------------------------------------------------- pack (scale, bias) words
+// Split-plane weights keep one 32-bit word per group next to the two 16-bit planes:
+// scale in the low half, bias in the high half, so the GEMV fetches both with one load.
+__global__ __launch_bounds__(256) void pack_sz_kernel(const uint16_t* __restrict__ scales,
+                                                      const uint16_t* __restrict__ biases,
+                                                      uint32_t* __restrict__ sz, size_t groups) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < groups; i += stride) sz[i] = (uint32_t)scales[i] | ((uint32_t)biases[i] << 16);
+}
+
+mi355q_status launch_pack_sz(hipStream_t s, const uint16_t* scales, const uint16_t* biases, uint32_t* sz,
+                             size_t groups) {
+    size_t blocks = (groups + 255) / 256;
+    if (blocks > 8192) blocks = 8192;
+    if (blocks == 0) blocks = 1;
+    pack_sz_kernel<<<dim3((unsigned)blocks), dim3(256), 0, s>>>(scales, biases, sz, groups);
+    MI355Q_HIP(hipGetLastError());
+    return MI355Q_OK;
+}
+
 // ------------------------------------------------------------------------------ dequant bf16
 // One workgroup per row, 256 threads striding over the row, as the reference kernel does.
 // scale*q and +zero are kept as two roundings so the result is bit-identical to an unfused

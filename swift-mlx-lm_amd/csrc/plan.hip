@@ -1,0 +1,215 @@
+// Dispatch plan: an ordered list of projection steps built once and replayed per token, the
+// stand-in for MetalDispatchPlan + MetalDecodeEncoder.encodeSteps
+// (Sources/MetalCompiler/Execution/MetalDecodePlan.swift:6-140, MetalDecodeEncoder.swift:18-36).
+#include <new>
+#include <string>
+#include <vector>
+
+#include "common.h"
+
+using namespace mi355q;
+
+namespace {
+
+enum StepKind { kLinear = 0, kOutputHead = 1 };
+
+struct PlanStep {
+    StepKind kind;
+    const mi355q_weight* w;
+    const void* x;
+    void* y;            // linear: output; head: fp32 logits (may be null)
+    int32_t* token;     // head only
+    int x_dtype, y_dtype;
+    uint32_t m, xs, ys, flags;
+    int32_t layer_index;
+    std::string tensor_name;
+    mi355q_step record;
+};
+
+}  // namespace
+
+struct mi355q_plan {
+    mi355q_context* ctx;
+    std::vector<PlanStep> steps;
+    hipGraph_t graph;
+    hipGraphExec_t graph_exec;
+};
+
+namespace {
+
+mi355q_status encode_range(mi355q_plan* plan, hipStream_t s, uint32_t first, uint32_t count) {
+    const uint32_t n = (uint32_t)plan->steps.size();
+    if (first > n) return fail(MI355Q_ERR_INVALID_ARGUMENT, "first step %u beyond plan length %u", first, n);
+    const uint32_t last = count == 0 ? n : (first + count < n ? first + count : n);
+    for (uint32_t i = first; i < last; i++) {
+        const PlanStep& st = plan->steps[i];
+        mi355q_status rc;
+        if (st.kind == kLinear)
+            rc = dispatch_linear(plan->ctx, s, st.w, st.x, st.x_dtype, st.y, st.y_dtype, st.m, st.xs, st.ys, st.flags,
+                                 false);
+        else
+            rc = dispatch_output_head(plan->ctx, s, st.w, st.x, st.x_dtype, (float*)st.y, st.token, st.flags);
+        if (rc != MI355Q_OK) return rc;
+    }
+    return MI355Q_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+mi355q_status mi355q_plan_create(mi355q_context* ctx, mi355q_plan** out) {
+    if (!ctx) return fail(MI355Q_ERR_NULL_HANDLE, "context is null");
+    if (!out) return fail(MI355Q_ERR_INVALID_ARGUMENT, "plan out pointer is null");
+    mi355q_plan* p = new (std::nothrow) mi355q_plan;
+    if (!p) return fail(MI355Q_ERR_OUT_OF_MEMORY, "host allocation failed");
+    p->ctx = ctx;
+    p->graph = nullptr;
+    p->graph_exec = nullptr;
+    *out = p;
+    return MI355Q_OK;
+}
+
+mi355q_status mi355q_plan_destroy(mi355q_plan* plan) {
+    if (!plan) return fail(MI355Q_ERR_NULL_HANDLE, "plan is null");
+    if (plan->graph_exec) (void)hipGraphExecDestroy(plan->graph_exec);
+    if (plan->graph) (void)hipGraphDestroy(plan->graph);
+    delete plan;
+    return MI355Q_OK;
+}
+
+mi355q_status mi355q_plan_add_linear(mi355q_plan* plan, const mi355q_weight* w, const void* x_dev,
+                                     mi355q_dtype x_dtype, void* y_dev, mi355q_dtype y_dtype, uint32_t m,
+                                     uint32_t x_row_stride, uint32_t y_row_stride, uint32_t flags,
+                                     int32_t layer_index, const char* tensor_name) {
+    if (!plan) return fail(MI355Q_ERR_NULL_HANDLE, "plan is null");
+    if (!w) return fail(MI355Q_ERR_NULL_HANDLE, "weight handle is null");
+    if (w->ctx != plan->ctx) return fail(MI355Q_ERR_INVALID_ARGUMENT, "weight handle belongs to another context");
+    if (!x_dev || !y_dev) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null activation or output pointer");
+    if (m == 0) return fail(MI355Q_ERR_INVALID_ARGUMENT, "sequence length M must be >= 1");
+    if (plan->graph_exec) return fail(MI355Q_ERR_INVALID_ARGUMENT, "plan is frozen: its graph has been built");
+    PlanStep st{};
+    st.kind = kLinear;
+    st.w = w; st.x = x_dev; st.y = y_dev; st.token = nullptr;
+    st.x_dtype = x_dtype; st.y_dtype = y_dtype;
+    st.m = m;
+    st.xs = x_row_stride ? x_row_stride : (uint32_t)w->k;
+    st.ys = y_row_stride ? y_row_stride : (uint32_t)w->n;
+    st.flags = flags;
+    st.layer_index = layer_index;
+    if (tensor_name) st.tensor_name = tensor_name;
+    mi355q_status rc;
+    if (m <= 8) {
+        rc = mi355q_plan_decode_step(w, m, x_dtype, flags, &st.record);
+    } else {
+        mi355q_step two[2];
+        uint32_t cnt = 0;
+        rc = mi355q_plan_prefill_steps(w, m, st.xs, x_dtype, 0, flags, two, &cnt);
+        st.record = two[0];
+    }
+    if (rc != MI355Q_OK) return rc;
+    plan->steps.push_back(st);
+    return MI355Q_OK;
+}
+
+mi355q_status mi355q_plan_add_output_head(mi355q_plan* plan, const mi355q_weight* w, const void* x_dev,
+                                          mi355q_dtype x_dtype, float* logits_f32_dev, int32_t* token_out_dev,
+                                          uint32_t flags, const char* tensor_name) {
+    if (!plan) return fail(MI355Q_ERR_NULL_HANDLE, "plan is null");
+    if (!w) return fail(MI355Q_ERR_NULL_HANDLE, "weight handle is null");
+    if (w->ctx != plan->ctx) return fail(MI355Q_ERR_INVALID_ARGUMENT, "weight handle belongs to another context");
+    if (!x_dev || !token_out_dev) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null pointer");
+    if (plan->graph_exec) return fail(MI355Q_ERR_INVALID_ARGUMENT, "plan is frozen: its graph has been built");
+    PlanStep st{};
+    st.kind = kOutputHead;
+    st.w = w; st.x = x_dev; st.y = logits_f32_dev; st.token = token_out_dev;
+    st.x_dtype = x_dtype; st.y_dtype = MI355Q_F32;
+    st.m = 1; st.xs = (uint32_t)w->k; st.ys = (uint32_t)w->n;
+    st.flags = flags;
+    st.layer_index = -1;
+    if (tensor_name) st.tensor_name = tensor_name;
+    mi355q_step two[2];
+    uint32_t cnt = 0;
+    if (mi355q_status rc = mi355q_plan_prefill_steps(w, 1, 0, x_dtype, 1, flags, two, &cnt)) return rc;
+    st.record = two[0];
+    plan->steps.push_back(st);
+    return MI355Q_OK;
+}
+
+int32_t mi355q_plan_step_count(const mi355q_plan* plan) { return plan ? (int32_t)plan->steps.size() : -1; }
+
+mi355q_status mi355q_plan_step_at(const mi355q_plan* plan, int32_t index, mi355q_step* out, int32_t* layer_index_out,
+                                  char* tensor_name_out, size_t name_cap) {
+    if (!plan) return fail(MI355Q_ERR_NULL_HANDLE, "plan is null");
+    if (index < 0 || (size_t)index >= plan->steps.size() || !out)
+        return fail(MI355Q_ERR_INVALID_ARGUMENT, "step index out of range");
+    const PlanStep& st = plan->steps[(size_t)index];
+    *out = st.record;
+    if (layer_index_out) *layer_index_out = st.layer_index;
+    if (tensor_name_out && name_cap) std::snprintf(tensor_name_out, name_cap, "%s", st.tensor_name.c_str());
+    return MI355Q_OK;
+}
+
+mi355q_status mi355q_plan_encode(mi355q_plan* plan, void* stream, uint32_t first, uint32_t count) {
+    if (!plan) return fail(MI355Q_ERR_NULL_HANDLE, "plan is null");
+    MI355Q_HIP(hipSetDevice(plan->ctx->device));
+    return encode_range(plan, (hipStream_t)stream, first, count);
+}
+
+mi355q_status mi355q_plan_graph_build(mi355q_plan* plan, void* stream) {
+    if (!plan) return fail(MI355Q_ERR_NULL_HANDLE, "plan is null");
+    if (!stream) return fail(MI355Q_ERR_INVALID_ARGUMENT, "graph capture needs an explicit (non-null) stream");
+    if (plan->graph_exec) return MI355Q_OK;
+    MI355Q_HIP(hipSetDevice(plan->ctx->device));
+    hipStream_t s = (hipStream_t)stream;
+    // One eager pass first: kernel attributes are set outside the capture.
+    if (mi355q_status rc = encode_range(plan, s, 0, 0)) return rc;
+    MI355Q_HIP(hipStreamSynchronize(s));
+    MI355Q_HIP(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
+    mi355q_status rc = encode_range(plan, s, 0, 0);
+    hipGraph_t g = nullptr;
+    hipError_t e = hipStreamEndCapture(s, &g);
+    if (rc != MI355Q_OK) {
+        if (g) (void)hipGraphDestroy(g);
+        return rc;
+    }
+    if (e != hipSuccess) return fail(MI355Q_ERR_DEVICE, "hipStreamEndCapture failed: %s", hipGetErrorString(e));
+    plan->graph = g;
+    e = hipGraphInstantiate(&plan->graph_exec, g, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        plan->graph_exec = nullptr;
+        return fail(MI355Q_ERR_DEVICE, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+    }
+    return MI355Q_OK;
+}
+
+mi355q_status mi355q_plan_graph_launch(mi355q_plan* plan, void* stream) {
+    if (!plan) return fail(MI355Q_ERR_NULL_HANDLE, "plan is null");
+    if (!plan->graph_exec) return fail(MI355Q_ERR_INVALID_ARGUMENT, "graph has not been built");
+    MI355Q_HIP(hipGraphLaunch(plan->graph_exec, (hipStream_t)stream));
+    return MI355Q_OK;
+}
+
+__global__ void copy_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src, size_t n_vec) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n_vec; i += stride) dst[i] = src[i];
+}
+
+mi355q_status mi355q_buffer_copy(mi355q_context* ctx, void* stream, void* dst_dev, const void* src_dev, size_t bytes) {
+    if (!ctx) return fail(MI355Q_ERR_NULL_HANDLE, "context is null");
+    if (!dst_dev || !src_dev) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null pointer in buffer_copy");
+    if (bytes % 16 || (uintptr_t)dst_dev % 16 || (uintptr_t)src_dev % 16)
+        return fail(MI355Q_ERR_INVALID_ARGUMENT, "buffer_copy needs 16-byte aligned pointers and size");
+    if (bytes == 0) return MI355Q_OK;
+    MI355Q_HIP(hipSetDevice(ctx->device));
+    const size_t n_vec = bytes / 16;
+    size_t blocks = (n_vec + 255) / 256;
+    if (blocks > 16384) blocks = 16384;
+    copy_kernel<<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>((uint4*)dst_dev, (const uint4*)src_dev,
+                                                                             n_vec);
+    MI355Q_HIP(hipGetLastError());
+    return MI355Q_OK;
+}
+
+}  // extern "C"

@@ -98,6 +98,17 @@ mi355q_status upload_new(void** dev, const void* host, size_t bytes) {
     return MI355Q_OK;
 }
 
+// Packed (scale, bias) plane of a split-plane weight: allocated and filled once, on the device.
+mi355q_status build_sz(mi355q_weight* w) {
+    const size_t groups = (size_t)w->n * (w->k / w->fmt.group_size);
+    MI355Q_HIP(hipMalloc(&w->sz, groups * 4));
+    if (mi355q_status st = launch_pack_sz(nullptr, (const uint16_t*)w->scales, (const uint16_t*)w->biases,
+                                          (uint32_t*)w->sz, groups))
+        return st;
+    MI355Q_HIP(hipStreamSynchronize(nullptr));
+    return MI355Q_OK;
+}
+
 mi355q_status need_ctx(mi355q_context* ctx) {
     if (!ctx) return fail(MI355Q_ERR_NULL_HANDLE, "context is null");
     hipError_t e = hipSetDevice(ctx->device);
@@ -344,6 +355,7 @@ mi355q_status mi355q_weight_prepare_mlx(mi355q_context* ctx, uint8_t scheme_iden
             }
         }
     }
+    if (st == MI355Q_OK && layout == MI355Q_LAYOUT_PLANES) st = build_sz(w);
     if (st != MI355Q_OK) {
         mi355q_weight_destroy(w);
         return st;
@@ -397,6 +409,7 @@ mi355q_status mi355q_weight_prepare_staf(mi355q_context* ctx, uint8_t scheme_ide
         if (st == MI355Q_OK) st = upload_new(&w->scales, s16.data(), w->sb_bytes);
         if (st == MI355Q_OK) st = upload_new(&w->biases, z16.data(), w->sb_bytes);
     }
+    if (st == MI355Q_OK && layout == MI355Q_LAYOUT_PLANES) st = build_sz(w);
     if (st != MI355Q_OK) {
         mi355q_weight_destroy(w);
         return st;
@@ -454,6 +467,16 @@ mi355q_status mi355q_weight_wrap_planes(mi355q_context* ctx, uint8_t scheme_iden
     w->biases = const_cast<void*>(biases_dev);
     w->codes_bytes = (size_t)n_rows * (k * f->bits / 32) * 4;
     w->sb_bytes = (size_t)n_rows * (k / f->group_size) * 2;
+    // the borrowed planes stay where they are; the packed (scale, bias) words are an extra owned buffer
+    if (hipSetDevice(ctx->device) != hipSuccess) {
+        delete w;
+        return fail(MI355Q_ERR_DEVICE, "hipSetDevice failed");
+    }
+    if (mi355q_status st = build_sz(w)) {
+        if (w->sz) (void)hipFree(w->sz);
+        delete w;
+        return st;
+    }
     *out = w;
     return MI355Q_OK;
 }
@@ -480,13 +503,14 @@ mi355q_status mi355q_weight_query(const mi355q_weight* w, mi355q_weight_info* ou
 
 mi355q_status mi355q_weight_destroy(mi355q_weight* w) {
     if (!w) return fail(MI355Q_ERR_NULL_HANDLE, "weight handle is null");
+    (void)hipSetDevice(w->ctx->device);
     if (w->owns) {
-        (void)hipSetDevice(w->ctx->device);
         if (w->blocks) (void)hipFree(w->blocks);
         if (w->codes) (void)hipFree(w->codes);
         if (w->scales) (void)hipFree(w->scales);
         if (w->biases) (void)hipFree(w->biases);
     }
+    if (w->sz) (void)hipFree(w->sz);
     delete w;
     return MI355Q_OK;
 }
