@@ -38,15 +38,17 @@ mi355q_status launch_group(hipStream_t s, const GemvArgs& a, const GemvCfg& c) {
     MI355Q_TRY(1, 1, false, 16, 2, 1) MI355Q_TRY(1, 1, false, 16, 4, 1) MI355Q_TRY(1, 1, false, 16, 8, 1)
     MI355Q_TRY(1, 1, false, 16, 2, 2) MI355Q_TRY(1, 1, false, 16, 4, 2) MI355Q_TRY(1, 1, false, 16, 8, 2)
 #else
-    // M == 1 (decode): register-resident (short rows) and LDS-resident activation variants
-    MI355Q_TRY(1, 1, false, 4, 2, 0) MI355Q_TRY(1, 1, false, 4, 4, 0) MI355Q_TRY(1, 1, false, 4, 8, 0)
-    MI355Q_TRY(1, 1, false, 4, 2, 1) MI355Q_TRY(1, 1, false, 4, 4, 1) MI355Q_TRY(1, 1, false, 4, 8, 1)
-    MI355Q_TRY(1, 1, false, 4, 2, 2) MI355Q_TRY(1, 1, false, 4, 4, 2) MI355Q_TRY(1, 1, false, 4, 8, 2)
+    // M == 1 (decode): register-resident activations for rows of one or two K-steps (4 wavefronts
+    // per workgroup), LDS-resident otherwise (8 wavefronts share one staged copy)
+    MI355Q_TRY(1, 1, false, 4, 2, 1) MI355Q_TRY(1, 1, false, 4, 4, 1)
+    MI355Q_TRY(1, 1, false, 4, 2, 2) MI355Q_TRY(1, 1, false, 4, 4, 2)
+    MI355Q_TRY(1, 1, false, 8, 2, 0) MI355Q_TRY(1, 1, false, 8, 4, 0)
 #endif
-    MI355Q_TRY(1, 1, true, 4, 2, 0) MI355Q_TRY(1, 1, true, 4, 4, 0) MI355Q_TRY(1, 1, true, 4, 8, 0)
-    MI355Q_TRY(1, 1, true, 4, 2, 1) MI355Q_TRY(1, 1, true, 4, 4, 1) MI355Q_TRY(1, 1, true, 4, 8, 1)
-    MI355Q_TRY(1, 1, true, 4, 2, 2) MI355Q_TRY(1, 1, true, 4, 4, 2) MI355Q_TRY(1, 1, true, 4, 8, 2)
-    // small batches
+    // the same with the fused arg-max tail (LM head)
+    MI355Q_TRY(1, 1, true, 4, 2, 1) MI355Q_TRY(1, 1, true, 4, 4, 1)
+    MI355Q_TRY(1, 1, true, 4, 2, 2) MI355Q_TRY(1, 1, true, 4, 4, 2)
+    MI355Q_TRY(1, 1, true, 8, 2, 0) MI355Q_TRY(1, 1, true, 8, 4, 0)
+    // small batches (M = 2, 3-4, 5-8)
     MI355Q_TRY(2, 2, false, 4, 4, 0) MI355Q_TRY(2, 4, false, 4, 2, 0) MI355Q_TRY(1, 8, false, 4, 2, 0)
     return fail(MI355Q_ERR_KERNEL_NOT_FOUND,
                 "no split-plane GEMV variant for q%d g%d R=%d MT=%d argmax=%d waves=%d depth=%d xreg=%d", BITS, GROUP,

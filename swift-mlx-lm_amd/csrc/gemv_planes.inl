@@ -116,7 +116,8 @@ __device__ __forceinline__ uint32_t extract_code(const uint32_t (&w)[WPL]) {
 // activation slice in registers; XREG = 0 re-reads the slice from LDS at every step
 // (conflict-free 128-bit reads shared by the R rows).
 template <int BITS, int GROUP, int R, int MT, bool ARGMAX, int WAVES, int D, int XREG>
-__global__ __launch_bounds__(WAVES * 64) void gemv_planes_kernel(GemvArgs a) {
+__global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(MT == 1 ? 4 : 2)))
+void gemv_planes_kernel(GemvArgs a) {
     using G = GemvGeo<BITS>;
     constexpr int WPL = G::WPL, CPL = G::CPL;
     constexpr int Q = CPL / 8;                          // uint4 pieces (8 codes) per lane chunk
@@ -133,7 +134,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_planes_kernel(GemvArgs a) {
     uint4* xs = smem;                                       // [MT][NC][Q][64]
     float* sxs = (float*)(smem + (size_t)MT * NC * Q * 64); // [MT][NC][NSR][64]
 
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    // the wavefront index is uniform: keep it (and everything derived from it) in scalar registers
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t row0 = (blockIdx.x * WAVES + wave) * a.rows_per_wave;
     const uint32_t nsteps = (a.rows_per_wave / R) * NC;     // same for every wavefront, >= 1
 
@@ -144,29 +147,53 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_planes_kernel(GemvArgs a) {
 
     // Unconditional loads: rows past N and lane chunks past K are clamped to valid addresses.
     // A clamped lane chunk meets activations staged as zero, a clamped row is never stored.
-    auto issue = [&](uint32_t rg, uint32_t c, Pref& p) {
+    // Addresses are "scalar row base + per-lane offset": the row part is wavefront-uniform.
+    auto lane_offsets = [&](uint32_t c, uint32_t& code_off, uint32_t (&sz_off)[NSR]) {
         uint32_t chunk = c * 64 + lane;                     // lane-chunk index inside the row
         chunk = (uint64_t)chunk * CPL < a.k ? chunk : 0;
+        code_off = chunk * WPL;
+#pragma unroll
+        for (int sr = 0; sr < NSR; sr++) sz_off[sr] = (chunk * CPL + sr * SR) / GROUP;
+    };
+    auto issue_at = [&](uint32_t rg, uint32_t code_off, const uint32_t (&sz_off)[NSR], Pref& p) {
 #pragma unroll
         for (int r = 0; r < R; r++) {
             uint32_t row = row0 + rg * R + r;
             row = row < a.n ? row : a.n - 1;
-            const uint32_t* src = a.codes + (size_t)row * a.words_per_row + (size_t)chunk * WPL;
+            const uint32_t* rowp = a.codes + (size_t)row * a.words_per_row;     // scalar
+            const uint32_t* szp = a.sz + (size_t)row * a.blocks_per_row;        // scalar
             if constexpr (WPL == 4) {
-                const uint4 v = *(const uint4*)src;
+                const uint4 v = *(const uint4*)(rowp + code_off);
                 p.w[r][0] = v.x; p.w[r][1] = v.y; p.w[r][2] = v.z; p.w[r][3] = v.w;
             } else {
 #pragma unroll
-                for (int i = 0; i < WPL; i++) p.w[r][i] = src[i];
+                for (int i = 0; i < WPL; i++) p.w[r][i] = rowp[code_off + i];
             }
 #pragma unroll
             for (int sr = 0; sr < NSR; sr++) {
-                const size_t g = (size_t)row * a.blocks_per_row + ((size_t)chunk * CPL + sr * SR) / GROUP;
 #ifdef MI355Q_GEMV_EXPERIMENT
                 if (a.dbg & 1) { p.sz[r][sr] = 0x38003C00u; continue; }
 #endif
-                p.sz[r][sr] = a.sz[g];
+                p.sz[r][sr] = szp[sz_off[sr]];
             }
+        }
+    };
+    // per-lane offsets of the K-steps a ring slot can hold, precomputed when rows are XREG steps long
+    uint32_t pre_code_off[XC];
+    uint32_t pre_sz_off[XC][NSR];
+    if constexpr (XREG != 0) {
+#pragma unroll
+        for (int cc = 0; cc < XC; cc++) lane_offsets((uint32_t)cc, pre_code_off[cc], pre_sz_off[cc]);
+    }
+    // CJ: compile-time K-step of the slot (XREG != 0); c: run-time K-step otherwise
+    auto issue = [&](uint32_t rg, uint32_t c, Pref& p, auto CJ) {
+        if constexpr (XREG != 0) {
+            constexpr int cj = decltype(CJ)::value % XC;
+            issue_at(rg, pre_code_off[cj], pre_sz_off[cj], p);
+        } else {
+            uint32_t code_off, sz_off[NSR];
+            lane_offsets(c, code_off, sz_off);
+            issue_at(rg, code_off, sz_off, p);
         }
     };
 
@@ -225,7 +252,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_planes_kernel(GemvArgs a) {
     };
     static_for<D>([&](auto J) {
         constexpr int j = decltype(J)::value;
-        issue(irg, ic, ring[j]);
+        issue(irg, ic, ring[j], J);
         advance();
     });
 
@@ -420,9 +447,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_planes_kernel(GemvArgs a) {
             for (int r = 0; r < R; r++) {
                 float s, z;
                 const uint32_t szw = cur.sz[r][sr];
-                if (a.sb_dtype == MI355Q_BF16) {            // wavefront-uniform branch
+                if (a.sb_dtype == MI355Q_BF16) {            // wavefront-uniform: keep it a real branch
+                    asm volatile("" ::: "memory");
                     s = __uint_as_float(szw << 16); z = __uint_as_float(szw & 0xFFFF0000u);
                 } else {
+                    asm volatile("" ::: "memory");
                     s = f16_to_f32((uint16_t)(szw & 0xFFFFu)); z = f16_to_f32((uint16_t)(szw >> 16));
                 }
                 const float zc = z - OFS * s;
@@ -475,7 +504,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_planes_kernel(GemvArgs a) {
         static_for<D>([&](auto J) {
             constexpr int j = decltype(J)::value;
             compute(ring[j], J);
-            issue(irg, ic, ring[j]);
+            issue(irg, ic, ring[j], J);
             advance();
         });
         finish_pass(it);

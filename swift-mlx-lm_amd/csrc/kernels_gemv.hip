@@ -57,13 +57,14 @@ GemvCfg choose(const mi355q_context* ctx, const WView& w, uint32_t m, bool argma
     const Geo g = geo_for(w.bits);
     const size_t kc = 64 * (size_t)g.cpl;
     c.nc = (uint32_t)((w.k + kc - 1) / kc);
-    c.waves = 4;
     if (c.mt == 1) {
         c.xreg = c.nc <= 2 ? (int)c.nc : 0;     // short rows: activation slice lives in registers
         c.r = 1;
+        c.waves = c.xreg ? 4 : 8;
     } else {
         c.xreg = 0;
         c.r = c.mt == 8 ? 1 : 2;
+        c.waves = 4;
     }
     const int er = env_int("MI355Q_GEMV_R", 0), ew = env_int("MI355Q_GEMV_WAVES", 0),
               ed = env_int("MI355Q_GEMV_DEPTH", 0), ex = env_int("MI355Q_GEMV_XREG", -1);
@@ -71,8 +72,9 @@ GemvCfg choose(const mi355q_context* ctx, const WView& w, uint32_t m, bool argma
     if (ew) c.waves = ew;
     if (ex >= 0) c.xreg = ex ? (int)c.nc : 0;
     c.lds = lds_bytes(w, c.mt);
-    // rows per wavefront: aim for `per_cu` wavefronts on every CU, each owning whole R-row steps
-    const uint32_t per_cu = (uint32_t)env_int("MI355Q_GEMV_WAVES_PER_CU", 16);
+    // rows per wavefront: aim for `per_cu` wavefronts on every CU (measured best: 32 for M = 1),
+    // each owning a whole number of R-row steps
+    const uint32_t per_cu = (uint32_t)env_int("MI355Q_GEMV_WAVES_PER_CU", c.mt == 1 ? 32 : 16);
     const uint32_t target = (uint32_t)ctx->props.multiProcessorCount * (per_cu ? per_cu : 16);
     uint32_t rpw = (w.n + target - 1) / target;
     const int forced = env_int("MI355Q_GEMV_ROWS_PER_WAVE", 0);
@@ -80,9 +82,9 @@ GemvCfg choose(const mi355q_context* ctx, const WView& w, uint32_t m, bool argma
     rpw = (rpw + c.r - 1) / c.r * c.r;
     if (rpw < (uint32_t)c.r) rpw = c.r;
     c.rows_per_wave = rpw;
-    // ring depth: the whole share of a wavefront when it is short, else 8 steps in flight
+    // ring depth: four pipeline steps in flight, two when a wavefront only has two or three
     const uint32_t nsteps = rpw / (uint32_t)c.r * c.nc;
-    if (c.mt == 1) c.depth = nsteps >= 6 ? 8 : nsteps >= 3 ? 4 : 2;
+    if (c.mt == 1) c.depth = nsteps >= 4 ? 4 : 2;
     else c.depth = c.mt == 2 ? 4 : 2;
     if (ed) c.depth = ed;
     const uint32_t rows_per_wg = rpw * (uint32_t)c.waves;

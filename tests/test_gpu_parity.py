@@ -380,3 +380,83 @@ def test_decode_and_prefill_plan_records(pkg, ctx):
     st2 = ws.plan_decode_step(1)
     assert st2.layout == pkg.LAYOUT_STAF_BLOCKS and st2.kernel_name == "gemv_q4_g64"
     w.destroy(); ws.destroy()
+
+
+# ------------------------------------------------------- dispatch plan replay (boundary b)
+def test_plan_replay_matches_direct_launches(pkg, ctx):
+    """A plan built once (projections of two layers + the output head) replayed from C and as a
+    HIP graph must reproduce the eager launches bit for bit, on every replay."""
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+    shapes = [(512, 1024), (256, 1024), (1024, 512), (2048, 1024)]          # last one: the head
+    ws, xs, ys, eager = [], [], [], []
+    for i, (n, k) in enumerate(shapes):
+        words, s, z, _ = seeded_case(1100 + i, n, k, 4, 64)
+        ws.append(ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, pkg.LAYOUT_PLANES))
+        xs.append(ctx.upload(oracle.bf16_from_f32(kat.seeded_activations(1200 + i, 1, k))))
+        ys.append(ctx.alloc(n * 4))
+    token = ctx.upload(np.array([-9], np.int32))
+    for i in range(3):
+        ctx.qgemv(ws[i], xs[i], pkg.BF16, ys[i], pkg.F32, 1)
+    ctx.lmhead_argmax(ws[3], xs[3], pkg.BF16, ys[3], token)
+    ctx.synchronize()
+    eager = [y.download(np.float32) for y in ys]
+    eager_token = int(token.download(np.int32)[0])
+    assert eager_token == oracle.argmax_lowest(eager[3])
+
+    plan = pkg.DispatchPlan(ctx)
+    for i in range(3):
+        plan.add_linear(ws[i], xs[i], pkg.BF16, ys[i], pkg.F32, 1, layer_index=i // 2, tensor_name=f"t{i}.weight")
+    plan.add_output_head(ws[3], xs[3], pkg.BF16, ys[3], token, tensor_name="lm_head.weight")
+    assert len(plan) == 4
+    st, layer, name = plan.step(1)
+    assert (st.kernel_name, layer, name) == ("gemv_q4_g64", 0, "t1.weight")
+    assert st.path == "decodeProjection" and st.output_dimension == 256
+    head, _, hname = plan.step(3)
+    assert head.fallback_reason == "lastTokenProjectionUsesDecodeKernel" and hname == "lm_head.weight"
+
+    stream = ctx.stream_create()
+
+    def check(label):
+        ctx.synchronize(stream)
+        for y, want in zip(ys, eager):
+            assert np.array_equal(y.download(np.float32), want), label
+        assert int(token.download(np.int32)[0]) == eager_token, label
+
+    def scrub():
+        for y in ys:
+            ctx.fill(y, 0x7FC00000, stream)
+        token.upload(np.array([-9], np.int32))
+
+    for rep in range(3):
+        scrub()
+        plan.encode(stream)
+        check(f"stream replay {rep}")
+    scrub()
+    plan.encode(stream, 1, 2)                                     # a sub-range only touches its outputs
+    ctx.synchronize(stream)
+    assert np.all(np.isnan(ys[0].download(np.float32))) and np.array_equal(ys[1].download(np.float32), eager[1])
+    plan.graph_build(stream)
+    for rep in range(4):                                          # graph replays interleaved with eager work
+        scrub()
+        plan.graph_launch(stream)
+        check(f"graph replay {rep}")
+        ctx.qgemv(ws[0], xs[0], pkg.BF16, ys[0], pkg.F32, 1, stream=stream)
+        ctx.synchronize(stream)
+    with pytest.raises(pkg.MI355QError):                          # a built graph freezes the plan
+        plan.add_linear(ws[0], xs[0], pkg.BF16, ys[0], pkg.F32, 1)
+    plan.destroy()
+    for o in ws:
+        o.destroy()
+    for b in xs + ys + [token]:
+        b.free()
+
+
+def test_buffer_copy_kernel(pkg, ctx):
+    src = np.random.default_rng(3).integers(0, 2**32, size=1 << 18, dtype=np.uint32)
+    a = ctx.upload(src); b = ctx.alloc(src.nbytes)
+    ctx.copy(b, a, src.nbytes)
+    ctx.synchronize()
+    assert np.array_equal(b.download(np.uint32), src)
+    with pytest.raises(pkg.MI355QError):
+        ctx.copy(b.ptr + 4, a, 64)
+    a.free(); b.free()
