@@ -121,6 +121,10 @@ mi355q_status dispatch_output_head(mi355q_context* ctx, hipStream_t s, const mi3
 int env_int_cached(const char* name, int fallback);
 
 // MFMA GEMM (kernels_gemm.hip)
+struct GemmLaunchShape {
+    uint32_t bm, bn, grid, block, lds_bytes;
+};
+GemmLaunchShape gemm_mfma_shape(const mi355q_context* ctx, uint32_t m, uint32_t n);
 bool gemm_mfma_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
 mi355q_status launch_qgemm_mfma(hipStream_t s, const mi355q_context* ctx, const WView& w,
                                 const void* x, int x_dtype, void* y, int y_dtype, uint32_t m,

@@ -1,9 +1,36 @@
 // Device helpers shared by the kernel translation units (gfx950, wave64).
 #pragma once
 
+#include <type_traits>
+#include <utility>
+
 #include "common.h"
 
 namespace mi355q {
+
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+// Calls f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>): a loop whose index is a
+// compile-time constant inside the body.
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+// Code at compile-time bit position POS of a lane chunk held in WPL registers.
+template <int POS, int BITS, int WPL>
+__device__ __forceinline__ uint32_t extract_code(const uint32_t (&w)[WPL]) {
+    constexpr int word = POS >> 5, sh = POS & 31;
+    constexpr uint32_t mask = (1u << BITS) - 1u;
+    if constexpr (sh + BITS <= 32) {
+        return (w[word] >> sh) & mask;
+    } else {
+        return __builtin_amdgcn_alignbit(w[word + 1], w[word], sh) & mask;
+    }
+}
+
 
 // ---- number formats ------------------------------------------------------------------------
 __device__ __forceinline__ float bf16_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }

@@ -26,17 +26,6 @@
 
 namespace mi355q {
 
-template <typename F, int... I>
-__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
-    (f(std::integral_constant<int, I>{}), ...);
-}
-// Calls f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>): a loop whose index is a
-// compile-time constant inside the body.
-template <int N, typename F>
-__device__ __forceinline__ void static_for(F&& f) {
-    static_for_impl(f, std::make_integer_sequence<int, N>{});
-}
-
 struct GemvArgs {
     const uint32_t* codes;
     const uint32_t* sz;      // packed (scale | bias << 16) word per group
@@ -85,18 +74,6 @@ typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
 __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float acc) {
     return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), acc,
                                            false);
-}
-
-// Code at compile-time bit position POS of a lane chunk held in WPL registers.
-template <int POS, int BITS, int WPL>
-__device__ __forceinline__ uint32_t extract_code(const uint32_t (&w)[WPL]) {
-    constexpr int word = POS >> 5, sh = POS & 31;
-    constexpr uint32_t mask = (1u << BITS) - 1u;
-    if constexpr (sh + BITS <= 32) {
-        return (w[word] >> sh) & mask;
-    } else {
-        return __builtin_amdgcn_alignbit(w[word + 1], w[word], sh) & mask;
-    }
 }
 
 // One wavefront owns `rows_per_wave` consecutive rows and walks them R at a time, one K-step

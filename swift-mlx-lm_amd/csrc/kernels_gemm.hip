@@ -1,19 +1,349 @@
-// Prefill GEMM on the matrix cores (placeholder translation unit: selection reports "not
-// eligible" until the MFMA kernels land, so every shape takes the small-M kernels).
-#include "common.h"
+// Prefill GEMM on the matrix cores:  Y[M,N] = X[M,K] * W[N,K]^T  with W either group-affine
+// packed codes (dequantised to bf16 on the way into LDS) or a dense bf16 matrix.
+//
+// Stands in for the reference's two prefill routes in one kernel
+//   gemm_q4_g64_f32s / gemm_q8_g32_f32s                      (direct, scalar FMA)
+//   dequant_q{b}_g{g}_bf16  +  gemm_bf16_f32s (matmul2d)     (two dispatches + a bf16 scratch)
+// (Sources/MetalCompiler/Generator/MetalSourceGenerator+Quantized.swift:22-156,361-416 and
+//  MetalSourceGenerator+Linear.swift:18-81), without the scratch round trip.
+//
+// Shape of the kernel
+//   * workgroup tile BM x BN x 64 (one K-tile = one 64-code run, so every row needs at most a
+//     couple of (scale, bias) words per K-tile), 4 wavefronts in a 2 x 2 arrangement, each
+//     owning a (BM/2) x (BN/2) block of 32x32 accumulators fed by v_mfma_f32_32x32x16_bf16;
+//   * LDS holds two stages of [rows][64] bf16 for both operands; a row is 128 bytes = 8 chunks
+//     of 16 bytes and chunk c of row r lives at position c ^ (r & 7), which makes both the
+//     128-bit stores and the MFMA operand loads (32 rows x one chunk) bank-conflict free;
+//   * the next K-tile is fetched into registers while the current one is multiplied; weight
+//     words are unpacked, scaled (fp32 fma), rounded to bf16 (v_cvt_pk_bf16_f32) and stored to
+//     the other LDS stage, so there is one barrier per K-tile;
+//   * workgroup ids are remapped so that the workgroups of one XCD (id % 8) walk the N-tiles of
+//     the same M-tile: the activation rows they share stay in that XCD's L2;
+//   * fp32 accumulators are rounded once, to the output type, in the epilogue.
+#include "device_utils.h"
 
 namespace mi355q {
 
-bool gemm_mfma_eligible(const WView&, int, uint32_t, uint32_t) { return false; }
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16_t;
+typedef __bf16 bf16x2_v __attribute__((ext_vector_type(2)));
+typedef float float2_v __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-mi355q_status launch_qgemm_mfma(hipStream_t, const mi355q_context*, const WView&, const void*, int, void*, int,
-                                uint32_t, uint32_t, uint32_t) {
-    return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "MFMA GEMM kernel is not built");
+struct GemmArgs {
+    const uint32_t* codes;   // QUANT: [N, K*bits/32]
+    const uint32_t* sz;      // QUANT: packed (scale | bias << 16) per group
+    const uint16_t* bdense;  // !QUANT: bf16 [N, K]
+    const uint16_t* x;       // bf16 [M, xs]
+    void* y;
+    uint32_t m, n, k, xs, ys;
+    uint32_t words_per_row, blocks_per_row;
+    uint32_t y_dtype, sb_dtype;
+    uint32_t tiles_m, tiles_n;
+};
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    float2_v v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_v));
 }
 
-mi355q_status launch_gemm_bf16_mfma(hipStream_t, const mi355q_context*, const void*, int, const uint16_t*, void*,
-                                    int, uint32_t, uint32_t, uint32_t, uint32_t, uint32_t) {
-    return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "MFMA GEMM kernel is not built");
+constexpr int kTileK = 64;            // codes (and bf16 elements) per K-tile
+constexpr int kRowBytes = kTileK * 2; // one LDS row
+
+__device__ __forceinline__ uint32_t lds_off(uint32_t row, uint32_t chunk) {
+    return row * kRowBytes + ((chunk ^ (row & 7u)) << 4);
+}
+
+template <int BITS, int GROUP, int BM, int BN, bool QUANT>
+__global__ __launch_bounds__(256) void qgemm_mfma_kernel(GemmArgs a) {
+    constexpr int TM = BM / 64, TN = BN / 64;             // 32x32 accumulators per wavefront
+    constexpr int A_BYTES = BM * kRowBytes, B_BYTES = BN * kRowBytes, STAGE = A_BYTES + B_BYTES;
+    constexpr int A_PASSES = BM / 32;                     // 16-byte chunks per thread for the X tile
+    constexpr int TPR = 256 / BN;                         // threads per weight row (1 or 2)
+    constexpr int CPT = kTileK / TPR;                     // codes per thread per K-tile
+    constexpr int WPT = QUANT ? CPT * BITS / 32 : 0;      // code words per thread per K-tile
+    constexpr int NGT = QUANT ? (CPT > GROUP ? CPT / GROUP : 1) : 0;   // groups a thread touches
+    constexpr int B_DENSE_PASSES = BN / 32;
+
+    extern __shared__ uint4 smem_q[];
+    char* lds = (char*)smem_q;
+
+    // ---- tile of this workgroup (XCD-aware order) --------------------------------------------
+    const uint32_t total = a.tiles_m * a.tiles_n;
+    const uint32_t per_xcd = (total + 7) / 8;
+    const uint32_t t_id = (blockIdx.x % 8u) * per_xcd + blockIdx.x / 8u;
+    if (t_id >= total) return;
+    const uint32_t tm = t_id / a.tiles_n, tn = t_id % a.tiles_n;
+    const uint32_t m0 = tm * BM, n0 = tn * BN;
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint32_t wm = wave >> 1, wn = wave & 1;
+
+    // ---- global -> register fetch of one K-tile -----------------------------------------------
+    u32x4 xa[A_PASSES];
+    uint32_t wreg[QUANT ? WPT : 1];
+    uint32_t szreg[QUANT ? NGT : 1];
+    u32x4 bd[QUANT ? 1 : B_DENSE_PASSES];
+
+    const uint32_t a_row = tid >> 3, a_chunk = tid & 7;       // X tile: 8 threads per row
+    const uint32_t b_row = tid / TPR, b_part = tid % TPR;     // W tile: TPR threads per row
+    uint32_t b_grow = n0 + b_row;
+    b_grow = b_grow < a.n ? b_grow : a.n - 1;
+
+    auto fetch = [&](uint32_t kt) __attribute__((always_inline)) {
+        const uint32_t k0 = kt * kTileK;
+        static_for<A_PASSES>([&](auto P) __attribute__((always_inline)) {
+            constexpr int p = decltype(P)::value;
+            uint32_t gr = m0 + p * 32 + a_row;
+            gr = gr < a.m ? gr : a.m - 1;
+            xa[p] = *(const u32x4*)(a.x + (size_t)gr * a.xs + k0 + a_chunk * 8);
+        });
+        if constexpr (QUANT) {
+            const uint32_t* src = a.codes + (size_t)b_grow * a.words_per_row + (size_t)kt * (kTileK * BITS / 32) +
+                                  b_part * WPT;
+            if constexpr (WPT % 4 == 0) {
+                static_for<WPT / 4>([&](auto I) __attribute__((always_inline)) {
+                    constexpr int i = decltype(I)::value;
+                    const u32x4 v = ((const u32x4*)src)[i];
+                    wreg[4 * i + 0] = v.x; wreg[4 * i + 1] = v.y; wreg[4 * i + 2] = v.z; wreg[4 * i + 3] = v.w;
+                });
+            } else if constexpr (WPT % 2 == 0) {
+                static_for<WPT / 2>([&](auto I) __attribute__((always_inline)) {
+                    constexpr int i = decltype(I)::value;
+                    const u32x2 v = ((const u32x2*)src)[i];
+                    wreg[2 * i + 0] = v.x; wreg[2 * i + 1] = v.y;
+                });
+            } else {
+                static_for<WPT>([&](auto I) __attribute__((always_inline)) {
+                    constexpr int i = decltype(I)::value;
+                    wreg[i] = src[i];
+                });
+            }
+            static_for<NGT>([&](auto G) __attribute__((always_inline)) {
+                constexpr int g = decltype(G)::value;
+                szreg[g] = a.sz[(size_t)b_grow * a.blocks_per_row + (k0 + b_part * CPT + g * GROUP) / GROUP];
+            });
+        } else {
+            static_for<B_DENSE_PASSES>([&](auto P) __attribute__((always_inline)) {
+                constexpr int p = decltype(P)::value;
+                uint32_t gr = n0 + p * 32 + a_row;
+                gr = gr < a.n ? gr : a.n - 1;
+                bd[p] = *(const u32x4*)(a.bdense + (size_t)gr * a.k + k0 + a_chunk * 8);
+            });
+        }
+    };
+
+    // ---- register -> LDS (with dequantisation of the weight words) ----------------------------
+    auto stash = [&](uint32_t stage) __attribute__((always_inline)) {
+        char* As = lds + stage * STAGE;
+        char* Bs = As + A_BYTES;
+        static_for<A_PASSES>([&](auto P) __attribute__((always_inline)) {
+            constexpr int p = decltype(P)::value;
+            *(u32x4*)(As + lds_off(p * 32 + a_row, a_chunk)) = xa[p];
+        });
+        if constexpr (QUANT) {
+            static_for<CPT / 8>([&](auto C) __attribute__((always_inline)) {
+                constexpr int ci = decltype(C)::value;                 // chunk of 8 codes
+                constexpr int g = NGT > 1 ? (ci * 8) / GROUP : 0;
+                float s, z;
+                const uint32_t szw = szreg[g];
+                if (a.sb_dtype == MI355Q_BF16) {
+                    s = __uint_as_float(szw << 16); z = __uint_as_float(szw & 0xFFFF0000u);
+                } else {
+                    s = f16_to_f32((uint16_t)(szw & 0xFFFFu)); z = f16_to_f32((uint16_t)(szw >> 16));
+                }
+                float f[8];
+                if constexpr (BITS == 4) {
+                    // byte-lane conversion: even codes sit in the low nibbles, odd ones in the high
+                    const uint32_t w = wreg[ci];
+                    const uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;
+                    float q[8];
+                    asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(q[0]) : "v"(lo));
+                    asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(q[1]) : "v"(hi));
+                    asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(q[2]) : "v"(lo));
+                    asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(q[3]) : "v"(hi));
+                    asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(q[4]) : "v"(lo));
+                    asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(q[5]) : "v"(hi));
+                    asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(q[6]) : "v"(lo));
+                    asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(q[7]) : "v"(hi));
+#pragma unroll
+                    for (int e = 0; e < 8; e++) f[e] = __builtin_fmaf(s, q[e], z);
+                } else {
+                    f[0] = __builtin_fmaf(s, (float)extract_code<(ci * 8 + 0) * BITS, BITS, (WPT ? WPT : 1)>(wreg), z);
+                    f[1] = __builtin_fmaf(s, (float)extract_code<(ci * 8 + 1) * BITS, BITS, (WPT ? WPT : 1)>(wreg), z);
+                    f[2] = __builtin_fmaf(s, (float)extract_code<(ci * 8 + 2) * BITS, BITS, (WPT ? WPT : 1)>(wreg), z);
+                    f[3] = __builtin_fmaf(s, (float)extract_code<(ci * 8 + 3) * BITS, BITS, (WPT ? WPT : 1)>(wreg), z);
+                    f[4] = __builtin_fmaf(s, (float)extract_code<(ci * 8 + 4) * BITS, BITS, (WPT ? WPT : 1)>(wreg), z);
+                    f[5] = __builtin_fmaf(s, (float)extract_code<(ci * 8 + 5) * BITS, BITS, (WPT ? WPT : 1)>(wreg), z);
+                    f[6] = __builtin_fmaf(s, (float)extract_code<(ci * 8 + 6) * BITS, BITS, (WPT ? WPT : 1)>(wreg), z);
+                    f[7] = __builtin_fmaf(s, (float)extract_code<(ci * 8 + 7) * BITS, BITS, (WPT ? WPT : 1)>(wreg), z);
+                }
+                u32x4 o;
+                o.x = pack_bf16(f[0], f[1]); o.y = pack_bf16(f[2], f[3]);
+                o.z = pack_bf16(f[4], f[5]); o.w = pack_bf16(f[6], f[7]);
+                *(u32x4*)(Bs + lds_off(b_row, b_part * (CPT / 8) + ci)) = o;
+            });
+        } else {
+            static_for<B_DENSE_PASSES>([&](auto P) __attribute__((always_inline)) {
+                constexpr int p = decltype(P)::value;
+                *(u32x4*)(Bs + lds_off(p * 32 + a_row, a_chunk)) = bd[p];
+            });
+        }
+    };
+
+    floatx16_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+    const uint32_t KT = a.k / kTileK;
+    fetch(0);
+    stash(0);
+    __syncthreads();
+
+    const uint32_t frag_row = lane & 31, frag_half = lane >> 5;
+    for (uint32_t kt = 0; kt < KT; kt++) {
+        const uint32_t stage = kt & 1;
+        if (kt + 1 < KT) fetch(kt + 1);
+        const char* As = lds + stage * STAGE;
+        const char* Bs = As + A_BYTES;
+#pragma unroll
+        for (int kk = 0; kk < kTileK / 16; kk++) {
+            bf16x8_t af[TM], bf[TN];
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+                af[i] = *(const bf16x8_t*)(As + lds_off(wm * (BM / 2) + i * 32 + frag_row, kk * 2 + frag_half));
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+                bf[j] = *(const bf16x8_t*)(Bs + lds_off(wn * (BN / 2) + j * 32 + frag_row, kk * 2 + frag_half));
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+        }
+        if (kt + 1 < KT) stash(stage ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: one rounding, to the output type --------------------------------------------
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const uint32_t col = n0 + wn * (BN / 2) + j * 32 + frag_row;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const uint32_t row = m0 + wm * (BM / 2) + i * 32 + 8 * (r / 4) + 4 * frag_half + (r % 4);
+                if (row < a.m && col < a.n) {
+                    const size_t o = (size_t)row * a.ys + col;
+                    const float v = acc[i][j][r];
+                    if (a.y_dtype == MI355Q_F32) ((float*)a.y)[o] = v;
+                    else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)a.y)[o] = f32_to_bf16_rne(v);
+                    else ((uint16_t*)a.y)[o] = f32_to_f16_rne(v);
+                }
+            }
+        }
+}
+
+// Tile choice: the largest tile that still gives every CU a workgroup.
+GemmLaunchShape gemm_mfma_shape(const mi355q_context* ctx, uint32_t m, uint32_t n) {
+    const uint32_t cus = (uint32_t)ctx->props.multiProcessorCount;
+    auto tiles = [&](uint32_t bm, uint32_t bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
+    GemmLaunchShape g{};
+    if (m > 128 && tiles(256, 256) >= cus) { g.bm = 256; g.bn = 256; }
+    else if (m > 128 && tiles(256, 128) >= cus / 2) { g.bm = 256; g.bn = 128; }
+    else { g.bm = 128; g.bn = 128; }
+    g.grid = (tiles(g.bm, g.bn) + 7) / 8 * 8;
+    g.block = 256;
+    g.lds_bytes = 2 * (g.bm + g.bn) * (uint32_t)kRowBytes;
+    return g;
+}
+
+namespace {
+
+template <int BITS, int GROUP, int BM, int BN, bool QUANT>
+mi355q_status launch_tile(hipStream_t s, GemmArgs a) {
+    a.tiles_m = (a.m + BM - 1) / BM;
+    a.tiles_n = (a.n + BN - 1) / BN;
+    const uint32_t total = a.tiles_m * a.tiles_n;
+    const uint32_t grid = (total + 7) / 8 * 8;
+    constexpr size_t lds = 2 * (size_t)(BM + BN) * kRowBytes;
+    auto kern = qgemm_mfma_kernel<BITS, GROUP, BM, BN, QUANT>;
+    static bool lds_limit_raised = false;      // per instantiation; the library drives one device
+    if (!lds_limit_raised) {
+        MI355Q_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        lds_limit_raised = true;
+    }
+    kern<<<dim3(grid), dim3(256), lds, s>>>(a);
+    MI355Q_HIP(hipGetLastError());
+    return MI355Q_OK;
+}
+
+template <int BITS, int GROUP, bool QUANT>
+mi355q_status launch_shape(hipStream_t s, const mi355q_context* ctx, const GemmArgs& a) {
+    const GemmLaunchShape g = gemm_mfma_shape(ctx, a.m, a.n);
+    if (g.bm == 256 && g.bn == 256) return launch_tile<BITS, GROUP, 256, 256, QUANT>(s, a);
+    if (g.bm == 256 && g.bn == 128) return launch_tile<BITS, GROUP, 256, 128, QUANT>(s, a);
+    return launch_tile<BITS, GROUP, 128, 128, QUANT>(s, a);
+}
+
+}  // namespace
+
+bool gemm_mfma_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
+    if (w.layout != MI355Q_LAYOUT_PLANES || x_dtype != MI355Q_BF16 || !w.sz) return false;
+    if (m < 1) return false;
+    if (w.k % kTileK) return false;
+    if (x_stride % 8) return false;                       // 128-bit activation loads
+    if ((uintptr_t)w.codes % 16) return false;
+    const bool fmt_ok = (w.bits == 4 && (w.group == 64 || w.group == 128)) ||
+                        (w.bits == 8 && (w.group == 32 || w.group == 64)) ||
+                        (w.bits == 6 && w.group == 64) || (w.bits == 3 && w.group == 64) ||
+                        (w.bits == 2 && w.group == 64);
+    return fmt_ok;
+}
+
+mi355q_status launch_qgemm_mfma(hipStream_t s, const mi355q_context* ctx, const WView& w, const void* x, int x_dtype,
+                                void* y, int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride) {
+    if (x_dtype != MI355Q_BF16) return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the MFMA GEMM takes bf16 activations");
+    if ((uintptr_t)x % 16) return fail(MI355Q_ERR_INVALID_ARGUMENT, "activation pointer must be 16-byte aligned");
+    GemmArgs a{};
+    a.codes = w.codes; a.sz = w.sz; a.bdense = nullptr;
+    a.x = (const uint16_t*)x; a.y = y;
+    a.m = m; a.n = w.n; a.k = w.k; a.xs = x_stride; a.ys = y_stride;
+    a.words_per_row = w.words_per_row; a.blocks_per_row = w.blocks_per_row;
+    a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = w.sb_dtype;
+    switch (w.bits * 1000 + w.group) {
+    case 4064: return launch_shape<4, 64, true>(s, ctx, a);
+    case 4128: return launch_shape<4, 128, true>(s, ctx, a);
+    case 8032: return launch_shape<8, 32, true>(s, ctx, a);
+    case 8064: return launch_shape<8, 64, true>(s, ctx, a);
+    case 6064: return launch_shape<6, 64, true>(s, ctx, a);
+    case 3064: return launch_shape<3, 64, true>(s, ctx, a);
+    case 2064: return launch_shape<2, 64, true>(s, ctx, a);
+    default: break;
+    }
+    return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no MFMA GEMM for q%u g%u", w.bits, w.group);
+}
+
+mi355q_status launch_gemm_bf16_mfma(hipStream_t s, const mi355q_context* ctx, const void* a_ptr, int a_dtype,
+                                    const uint16_t* b, void* c, int c_dtype, uint32_t m, uint32_t n, uint32_t k,
+                                    uint32_t a_stride, uint32_t c_stride) {
+    if (a_dtype != MI355Q_BF16) return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the MFMA GEMM takes bf16 activations");
+    if (k % kTileK) return fail(MI355Q_ERR_SHAPE, "K=%u must be a multiple of %d", k, kTileK);
+    if (a_stride % 8 || (uintptr_t)a_ptr % 16 || (uintptr_t)b % 16)
+        return fail(MI355Q_ERR_INVALID_ARGUMENT, "operands must be 16-byte aligned with row strides multiple of 8");
+    GemmArgs a{};
+    a.bdense = b;
+    a.x = (const uint16_t*)a_ptr; a.y = c;
+    a.m = m; a.n = n; a.k = k; a.xs = a_stride; a.ys = c_stride;
+    a.y_dtype = (uint32_t)c_dtype;
+    return launch_shape<4, 64, false>(s, ctx, a);
 }
 
 }  // namespace mi355q

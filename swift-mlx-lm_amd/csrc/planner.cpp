@@ -135,9 +135,11 @@ mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w, uint32_t maximum
         std::snprintf(s->device_kernel, sizeof s->device_kernel, "qgemm_mfma_q%u_g%u", (unsigned)w->fmt.bits,
                       w->fmt.group_size);
         std::snprintf(s->kernel_family, sizeof s->kernel_family, "mfmaGEMM");
-        s->block[0] = 256;
-        s->grid[0] = (uint32_t)((w->n + 255) / 256) * ((m + 255) / 256);
-        s->rows_per_workgroup = 256;
+        const GemmLaunchShape g = gemm_mfma_shape(w->ctx, m, (uint32_t)w->n);
+        s->block[0] = g.block;
+        s->grid[0] = g.grid;
+        s->lds_bytes = g.lds_bytes;
+        s->rows_per_workgroup = g.bn;
         return MI355Q_OK;
     }
     // direct per-row kernel with the sequence signature (gemm_q{b}_g{g}[_f32s])
