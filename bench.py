@@ -29,6 +29,10 @@ HBM_PEAK_GBPS = 8000.0            # MI355X published HBM3E bandwidth
 LAYER_SHAPES = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
                 ("gate", 14336, 4096), ("up", 14336, 4096), ("down", 4096, 14336)]
 BITS, GROUP = 4, 64
+# HBM bytes per gate/up launch from the FETCH_SIZE and WRITE_SIZE counters, each scaled by what the
+# same counter reads for a plain copy of the same size (profiles/gemv_planes_q4_g64_gate_up_hbm_traffic_pmc.md).
+# Measured offline with the profiler; valid for the kernel variant named in `roofline.kernel`.
+GATE_TRAFFIC_BYTES = 33255544
 
 
 def log(*a):
@@ -84,6 +88,7 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-parity", action="store_true")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the secondary prefill-GEMM figure")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (one process, one device); "
@@ -190,6 +195,31 @@ def main():
     achieved = weight_bytes(14336, 4096) / (gate_ms * 1e-3) / 1e9
     gate_step = layers[0]["gate"].plan_decode_step(1)
 
+    # ---- plain copy of the gate tensor's size: the calibration launch for the HBM counters ------
+    gate_bytes = weight_bytes(14336, 4096)
+    csrc, cdst = ctx.alloc(gate_bytes), ctx.alloc(gate_bytes)
+    ctx.fill(csrc, 0x01020304, stream)
+    ctx.copy(cdst, csrc, gate_bytes, stream)
+    ctx.synchronize(stream)
+    ms_copy = time_region(ctx, lambda i: ctx.copy(cdst, csrc, gate_bytes, stream), 8, stream)
+    log(f"  copy  {gate_bytes} B: {ms_copy * 1e3:.2f} us/launch, {2 * gate_bytes / (ms_copy * 1e-3) / 1e9:.1f} GB/s "
+        "read+write")
+
+    # ---- secondary figure: the prefill GEMM of the same layer's gate projection (not the metric)
+    prefill = None
+    if not a.no_prefill:
+        m = 2048
+        xg = ctx.upload(oracle.bf16_from_f32(kat.seeded_activations(5, m, 4096)))
+        yg = ctx.alloc(m * 14336 * 2)
+        wg = layers[0]["gate"]
+        ctx.qgemm(wg, xg, pkg.BF16, yg, pkg.BF16, m, 0, 0, pkg.FLAG_FORCE_MFMA, stream)
+        ctx.synchronize(stream)
+        ms_g = time_region(ctx, lambda i: ctx.qgemm(wg, xg, pkg.BF16, yg, pkg.BF16, m, 0, 0, pkg.FLAG_FORCE_MFMA,
+                                                    stream), 10, stream)
+        prefill = {"m": m, "us": round(ms_g * 1e3, 1), "TFLOPs": round(2.0 * m * 14336 * 4096 / (ms_g * 1e-3) / 1e12, 1)}
+        log(f"  prefill GEMM M={m} 4096->14336: {prefill['us']} us, {prefill['TFLOPs']} TFLOP/s (bf16 MFMA peak 2500)")
+        xg.free(); yg.free()
+
     cpu = None if a.no_cpu else cpu_baseline(a.cpu_seconds)
 
     out = {
@@ -211,9 +241,11 @@ def main():
                    "weight_bytes_per_step": layer_bytes, "layers_resident": a.layers,
                    "replay": mode, "stream_replay_GBps": round(stream_value, 1),
                    "graph_replay_GBps": None if graph_value is None else round(graph_value, 1),
-                   "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2), "per_shape": per_shape},
+                   "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2), "per_shape": per_shape,
+                   "prefill_gemm_gate": prefill},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": GATE_TRAFFIC_BYTES,
+                     "algorithmic_bytes": gate_bytes,
                      "kernel": f"{gate_step.device_kernel} on gate/up 4096->14336 (33030144 weight bytes/launch, "
                                f"grid {gate_step.grid[0]} x {gate_step.block[0]} threads)"},
     }
