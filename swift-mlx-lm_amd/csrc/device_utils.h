@@ -8,6 +8,10 @@
 
 namespace mi355q {
 
+// Native vectors (not the HIP uint4 struct): register arrays of these are reliably kept in VGPRs.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
 template <typename F, int... I>
 __device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
     (f(std::integral_constant<int, I>{}), ...);

@@ -106,9 +106,9 @@ void gemv_planes_kernel(GemvArgs a) {
     static_assert(XREG == 0 || (MT == 1 && R == 1), "register-resident activations are for M == 1, R == 1");
     static_assert(XREG == 0 || D % XREG == 0, "ring depth must be a multiple of the K-steps per row");
 
-    extern __shared__ uint4 smem[];
+    extern __shared__ u32x4 smem[];
     const uint32_t NC = a.nc;
-    uint4* xs = smem;                                       // [MT][NC][Q][64]
+    u32x4* xs = smem;                                      // [MT][NC][Q][64]
     float* sxs = (float*)(smem + (size_t)MT * NC * Q * 64); // [MT][NC][NSR][64]
 
     const uint32_t tid = threadIdx.x, lane = tid & 63;
@@ -140,7 +140,7 @@ void gemv_planes_kernel(GemvArgs a) {
             const uint32_t* rowp = a.codes + (size_t)row * a.words_per_row;     // scalar
             const uint32_t* szp = a.sz + (size_t)row * a.blocks_per_row;        // scalar
             if constexpr (WPL == 4) {
-                const uint4 v = *(const uint4*)(rowp + code_off);
+                const u32x4 v = *(const u32x4*)(rowp + code_off);
                 p.w[r][0] = v.x; p.w[r][1] = v.y; p.w[r][2] = v.z; p.w[r][3] = v.w;
             } else {
 #pragma unroll
@@ -175,46 +175,62 @@ void gemv_planes_kernel(GemvArgs a) {
     };
 
     // ---- staging helpers: one task = one lane chunk of one activation row ---------------------
-    const uint32_t ntasks = (uint32_t)MT * NC * 64;
-    auto stage_load = [&](uint32_t task, uint32_t (&d)[CPL / 2]) {
-        const uint32_t l = task & 63, cc = (task >> 6) % NC, m = (task >> 6) / NC;
-        const uint64_t kbase = (uint64_t)cc * KC + (uint64_t)l * CPL;
-        const bool valid = task < ntasks && m < a.m && kbase < a.k;
-        const uint4* src = (const uint4*)(a.x + (valid ? (size_t)m * a.x_stride + kbase : 0));
+    // Tasks are dealt to wavefronts whole: wave task tw = m * NC + cc covers the 64 lane chunks of
+    // K-step cc of activation row m, so (m, cc) and every bound check on them stay scalar.
+    const uint32_t nwt = (uint32_t)MT * NC;
+    auto task_coords = [&](uint32_t tw, uint32_t& m, uint32_t& cc) {
+        if constexpr (MT == 1) { m = 0; cc = tw; }
+        else { m = tw / NC; cc = tw - m * NC; }
+    };
+    auto stage_load = [&](uint32_t tw, uint32_t (&d)[CPL / 2]) {
+        uint32_t m, cc;
+        task_coords(tw, m, cc);
+        const uint64_t kbase = (uint64_t)cc * KC + (uint64_t)lane * CPL;
+        const bool valid = tw < nwt && m < a.m && kbase < a.k;
+        const u32x4* src = (const u32x4*)(a.x + (valid ? (size_t)m * a.x_stride + kbase : 0));
 #pragma unroll
         for (int i = 0; i < Q; i++) {
-            const uint4 v = src[i];                         // clamped address: always readable
+            const u32x4 v = src[i];                         // clamped address: always readable
             d[4 * i + 0] = valid ? v.x : 0; d[4 * i + 1] = valid ? v.y : 0;
             d[4 * i + 2] = valid ? v.z : 0; d[4 * i + 3] = valid ? v.w : 0;
         }
     };
-    auto stage_store = [&](uint32_t task, const uint32_t (&d)[CPL / 2]) {
-        if (task >= ntasks) return;                         // LDS writes only inside this branch
-        const uint32_t l = task & 63, cc = (task >> 6) % NC, m = (task >> 6) / NC;
-        auto elem = [&](int e) -> uint32_t { return (e & 1) ? (d[e >> 1] >> 16) : (d[e >> 1] & 0xFFFFu); };
-#pragma unroll
-        for (int i = 0; i < Q; i++) {
-            uint4 o;
-            o.x = elem(pair_elem<BITS>(4 * i + 0, 0)) | (elem(pair_elem<BITS>(4 * i + 0, 1)) << 16);
-            o.y = elem(pair_elem<BITS>(4 * i + 1, 0)) | (elem(pair_elem<BITS>(4 * i + 1, 1)) << 16);
-            o.z = elem(pair_elem<BITS>(4 * i + 2, 0)) | (elem(pair_elem<BITS>(4 * i + 2, 1)) << 16);
-            o.w = elem(pair_elem<BITS>(4 * i + 3, 0)) | (elem(pair_elem<BITS>(4 * i + 3, 1)) << 16);
-            xs[((size_t)(m * NC + cc) * Q + i) * 64 + l] = o;
-        }
+    auto stage_store = [&](uint32_t tw, const uint32_t (&d)[CPL / 2]) {
+        if (tw >= nwt) return;                              // LDS writes only inside this (scalar) branch
+        uint32_t m, cc;
+        task_coords(tw, m, cc);
+        // staged pair i = (element e0, element e1) of the lane chunk: one byte permute of two dwords
+        auto pairw = [&](auto I) -> uint32_t {
+            constexpr int i = decltype(I)::value;
+            constexpr int e0 = pair_elem<BITS>(i, 0), e1 = pair_elem<BITS>(i, 1);
+            static_assert((e0 & 1) == (e1 & 1) || e1 == e0 + 1, "pair halves come from the same half-word");
+            if constexpr (e1 == e0 + 1 && (e0 & 1) == 0) return d[e0 >> 1];
+            else return __builtin_amdgcn_perm(d[e1 >> 1], d[e0 >> 1], (e0 & 1) ? 0x07060302u : 0x05040100u);
+        };
+        static_for<Q>([&](auto P) {
+            constexpr int i = decltype(P)::value;
+            u32x4 o;
+            o.x = pairw(std::integral_constant<int, 4 * i + 0>{});
+            o.y = pairw(std::integral_constant<int, 4 * i + 1>{});
+            o.z = pairw(std::integral_constant<int, 4 * i + 2>{});
+            o.w = pairw(std::integral_constant<int, 4 * i + 3>{});
+            xs[((size_t)(m * NC + cc) * Q + i) * 64 + lane] = o;
+        });
+        // sum of the activations of each sub-run: dot2 against the bf16 pair (1.0, 1.0)
 #pragma unroll
         for (int sr = 0; sr < NSR; sr++) {
             float sx = 0.0f;
 #pragma unroll
-            for (int e = 0; e < SR; e++) sx += __uint_as_float(elem(sr * SR + e) << 16);
-            sxs[((size_t)(m * NC + cc) * NSR + sr) * 64 + l] = sx;
+            for (int j = 0; j < SR / 2; j++) sx = dot2_bf16(d[sr * (SR / 2) + j], 0x3F803F80u, sx);
+            sxs[((size_t)(m * NC + cc) * NSR + sr) * 64 + lane] = sx;
         }
     };
 
     // ---- 1. activation loads first ------------------------------------------------------------
-    constexpr int TE = 2;                                   // early staging tasks per thread
+    constexpr int TE = 1;                                   // early staging tasks per wavefront
     uint32_t dearly[TE][CPL / 2];
 #pragma unroll
-    for (int t = 0; t < TE; t++) stage_load(tid + t * (WAVES * 64), dearly[t]);
+    for (int t = 0; t < TE; t++) stage_load(wave + t * WAVES, dearly[t]);
 
     // ---- 2. the first D steps of weight loads -------------------------------------------------
     // Steps past the last one repeat it (same addresses, so they hit in L2 and their data is
@@ -239,11 +255,11 @@ void gemv_planes_kernel(GemvArgs a) {
 #endif
     {
 #pragma unroll
-        for (int t = 0; t < TE; t++) stage_store(tid + t * (WAVES * 64), dearly[t]);
-        for (uint32_t task = tid + TE * (WAVES * 64); task < ntasks; task += WAVES * 64) {
-            uint32_t dl[CPL / 2];                           // large batches: the remaining tasks
-            stage_load(task, dl);
-            stage_store(task, dl);
+        for (int t = 0; t < TE; t++) stage_store(wave + t * WAVES, dearly[t]);
+        for (uint32_t tw = wave + TE * WAVES; tw < nwt; tw += WAVES) {
+            uint32_t dl[CPL / 2];                           // long rows / batches: the remaining tasks
+            stage_load(tw, dl);
+            stage_store(tw, dl);
         }
     }
     // LDS-only barrier: the weight loads in flight must not be waited for here
@@ -252,7 +268,7 @@ void gemv_planes_kernel(GemvArgs a) {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 
     // ---- optional register-resident activation slice (M == 1, rows of XREG K-steps) -----------
-    uint4 xr[XC][Q];
+    u32x4 xr[XC][Q];
     float sxr[XC][NSR];
     if constexpr (XREG != 0) {
 #pragma unroll
@@ -344,7 +360,7 @@ void gemv_planes_kernel(GemvArgs a) {
         static_for<Q>([&](auto P) {
             constexpr int p = decltype(P)::value;
             constexpr int sr = (p * 8) / SR;
-            uint4 xv[MT];
+            u32x4 xv[MT];
             if constexpr (XREG != 0) {
                 xv[0] = xr[cj][p];
             } else {

@@ -28,8 +28,6 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16_t;
 typedef __bf16 bf16x2_v __attribute__((ext_vector_type(2)));
 typedef float float2_v __attribute__((ext_vector_type(2)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 struct GemmArgs {
     const uint32_t* codes;   // QUANT: [N, K*bits/32]
