@@ -122,6 +122,8 @@ def main():
     layer_bytes = sum(weight_bytes(n, k) for _, n, k in LAYER_SHAPES)
     log(f"resident: {a.layers} layers x {layer_bytes} B = {a.layers * layer_bytes / 1e9:.2f} GB")
 
+    stream = ctx.stream_create()
+
     # ---- parity gate: no number is reported from a run whose outputs were not verified
     if not a.skip_parity:
         for name, n, k in LAYER_SHAPES:
@@ -139,44 +141,60 @@ def main():
                 sys.exit(f"bench.py: parity gate failed on {name}: rel-L2 {rel:.3e} max-abs {mx:.3e}")
             log(f"  parity {name}: rel-L2 {rel:.2e} max-abs {mx:.2e}")
 
-    stream = ctx.stream_create()
+    # ---- the decode plans, built once, replayed from C -----------------------------------------
+    #   "7-launch": one launch per projection, the reference's decode schedule
+    #   "4-launch": q+k+v and gate+up share their input and run as one launch each
+    def build_plan(fused):
+        plan = pkg.DispatchPlan(ctx)
+        for li, L in enumerate(layers):
+            def lin(name, k):
+                plan.add_linear(L[name], xdev[k], pkg.BF16, ydev[name], pkg.BF16, 1, layer_index=li,
+                                tensor_name=f"layers.{li}.{name}_proj.weight")
+            if fused:
+                plan.add_batched_linear([L["q"], L["k"], L["v"]], xdev[4096], pkg.BF16,
+                                        [ydev["q"], ydev["k"], ydev["v"]], pkg.BF16, 1, layer_index=li,
+                                        tensor_name=f"layers.{li}.qkv_proj.weight")
+                lin("o", 4096)
+                plan.add_batched_linear([L["gate"], L["up"]], xdev[4096], pkg.BF16, [ydev["gate"], ydev["up"]],
+                                        pkg.BF16, 1, layer_index=li, tensor_name=f"layers.{li}.gate_up_proj.weight")
+                lin("down", 14336)
+            else:
+                for name, n, k in LAYER_SHAPES:
+                    lin(name, k)
+        return plan
 
-    # ---- the decode plan: 7 projection steps per layer, built once, replayed from C ------------
-    plan = pkg.DispatchPlan(ctx)
-    for li, L in enumerate(layers):
-        for name, n, k in LAYER_SHAPES:
-            plan.add_linear(L[name], xdev[k], pkg.BF16, ydev[name], pkg.BF16, 1, layer_index=li,
-                            tensor_name=f"layers.{li}.{name}_proj.weight")
-    per_layer = len(LAYER_SHAPES)
+    results = {}
+    for label, fused in (("7-launch", False), ("4-launch", True)):
+        plan = build_plan(fused)
+        per_layer = len(plan) // a.layers
 
-    def step(i):
-        plan.encode(stream, (i % a.layers) * per_layer, per_layer)
+        def step(i, plan=plan, per_layer=per_layer):
+            plan.encode(stream, (i % a.layers) * per_layer, per_layer)
 
-    for i in range(a.warmup):
-        step(i)
-    ctx.synchronize(stream)
-    ms_step = time_region(ctx, step, a.steps, stream)
-    ctx.synchronize(stream)
+        for i in range(a.warmup):
+            step(i)
+        ctx.synchronize(stream)
+        ms = time_region(ctx, step, a.steps, stream)
+        ctx.synchronize(stream)
+        results[label + " stream"] = ms
+        log(f"{label} stream replay: {ms * 1e3:.2f} us/step, {layer_bytes / (ms * 1e-3) / 1e9:.1f} GB/s")
+        # the same plan captured once into a HIP graph (one launch per pass over all layers)
+        if a.steps % a.layers == 0:
+            plan.graph_build(stream)
+            for _ in range(2):
+                plan.graph_launch(stream)
+            ctx.synchronize(stream)
+            passes = a.steps // a.layers
+            ms_pass = time_region(ctx, lambda i, plan=plan: plan.graph_launch(stream), passes, stream)
+            ctx.synchronize(stream)
+            results[label + " hip-graph"] = ms_pass / a.layers
+            log(f"{label} graph replay:  {ms_pass / a.layers * 1e3:.2f} us/step, "
+                f"{layer_bytes / (ms_pass / a.layers * 1e-3) / 1e9:.1f} GB/s")
+        plan.destroy()
+    mode = min(results, key=results.get)
+    ms_step = results[mode]
     value = layer_bytes / (ms_step * 1e-3) / 1e9
-    stream_value = value
-    log(f"stream replay: {ms_step * 1e3:.2f} us/step, {value:.1f} GB/s")
-
-    # ---- the same plan captured once into a HIP graph (one launch per pass over all layers) ----
-    graph_value = None
-    if a.steps % a.layers == 0:
-        plan.graph_build(stream)
-        for _ in range(2):
-            plan.graph_launch(stream)
-        ctx.synchronize(stream)
-        passes = a.steps // a.layers
-        ms_pass = time_region(ctx, lambda i: plan.graph_launch(stream), passes, stream)
-        ctx.synchronize(stream)
-        ms_step_graph = ms_pass / a.layers
-        graph_value = layer_bytes / (ms_step_graph * 1e-3) / 1e9
-        log(f"graph replay:  {ms_step_graph * 1e3:.2f} us/step, {graph_value:.1f} GB/s")
-    mode = "stream"
-    if graph_value is not None and graph_value > value:
-        value, ms_step, mode = graph_value, ms_step_graph, "hip-graph"
+    replay_gbps = {k: round(layer_bytes / (v * 1e-3) / 1e9, 1) for k, v in results.items()}
 
     # ---- dominant kernel (gate/up 4096 -> 14336): average launch duration over rotating copies
     per_shape = {}
@@ -239,8 +257,7 @@ def main():
         "config": {"workload": "Llama-3-8B decode layer sweep (BASELINE config 1), M=1: q,k,v,o,gate,up,down "
                                "GEMVs per step", "bits": BITS, "group_size": GROUP,
                    "weight_bytes_per_step": layer_bytes, "layers_resident": a.layers,
-                   "replay": mode, "stream_replay_GBps": round(stream_value, 1),
-                   "graph_replay_GBps": None if graph_value is None else round(graph_value, 1),
+                   "replay": mode, "replay_GBps": replay_gbps,
                    "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2), "per_shape": per_shape,
                    "prefill_gemm_gate": prefill},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",

@@ -381,6 +381,18 @@ MI355Q_API mi355q_status mi355q_plan_add_linear(mi355q_plan* plan, const mi355q_
                                                 uint32_t x_row_stride, uint32_t y_row_stride,
                                                 uint32_t flags, int32_t layer_index,
                                                 const char* tensor_name);
+/* One step for 2 or 3 projections that share their input (bindings as mi355q_batched_qgemm):
+ * the decode-time counterpart of the reference's batched prefill kernels
+ * (MC/Generator/MetalSourceGenerator+Quantized.swift:166-338; the entry collector that groups
+ * q/k/v and gate/up is MC/Compiler/MetalEntryCollector.swift:55-95).  For M <= 8 on the
+ * split-plane layout the projections run as one launch. */
+MI355Q_API mi355q_status mi355q_plan_add_batched_linear(mi355q_plan* plan, uint32_t count,
+                                                        const mi355q_weight* const* weights,
+                                                        const void* x_dev, mi355q_dtype x_dtype,
+                                                        void* const* y_devs, mi355q_dtype y_dtype,
+                                                        uint32_t m, uint32_t x_row_stride,
+                                                        uint32_t flags, int32_t layer_index,
+                                                        const char* tensor_name);
 /* One OutputHeadFragment step (bindings as mi355q_lmhead_argmax). */
 MI355Q_API mi355q_status mi355q_plan_add_output_head(mi355q_plan* plan, const mi355q_weight* w,
                                                      const void* x_dev, mi355q_dtype x_dtype,

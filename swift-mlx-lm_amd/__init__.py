@@ -132,6 +132,8 @@ def library() -> C.CDLL:
         "mi355q_plan_create": (i32, [vp, P(vp)]),
         "mi355q_plan_destroy": (i32, [vp]),
         "mi355q_plan_add_linear": (i32, [vp, vp, vp, C.c_int, vp, C.c_int, u32, u32, u32, u32, i32, C.c_char_p]),
+        "mi355q_plan_add_batched_linear": (i32, [vp, u32, vp, vp, C.c_int, vp, C.c_int, u32, u32, u32, i32,
+                                                  C.c_char_p]),
         "mi355q_plan_add_output_head": (i32, [vp, vp, vp, C.c_int, vp, vp, u32, C.c_char_p]),
         "mi355q_plan_step_count": (i32, [vp]),
         "mi355q_plan_step_at": (i32, [vp, i32, P(_Step), P(i32), C.c_char_p, sz]),
@@ -359,6 +361,17 @@ class DispatchPlan:
                                                 y_dtype, m, x_row_stride, y_row_stride, flags, layer_index,
                                                 tensor_name.encode() if tensor_name else None))
         self._keep.append((w, x, y))
+
+    def add_batched_linear(self, weights, x, x_dtype, ys, y_dtype, m=1, x_row_stride=0, flags=0, layer_index=-1,
+                           tensor_name: str | None = None):
+        """2 or 3 projections sharing x (q+k+v, gate+up) as one step; one launch when M <= 8."""
+        n = len(weights)
+        wh = (C.c_void_p * n)(*[w.handle for w in weights])
+        yh = (C.c_void_p * n)(*[Context._ptr(y) for y in ys])
+        _check(library().mi355q_plan_add_batched_linear(self.handle, n, wh, Context._ptr(x), x_dtype, yh, y_dtype, m,
+                                                        x_row_stride, flags, layer_index,
+                                                        tensor_name.encode() if tensor_name else None))
+        self._keep.append((list(weights), x, list(ys)))
 
     def add_output_head(self, w: "PackedWeight", x, x_dtype, logits_f32, token_out, flags=0,
                         tensor_name: str | None = None):

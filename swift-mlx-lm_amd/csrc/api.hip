@@ -91,6 +91,44 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
     return launch_qgemm_mfma(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
 }
 
+// Two or three projections that read the same activations (q+k+v, gate+up).  For M <= 8 on the
+// split-plane layout they run as ONE launch whose rows are the rows of all weights together;
+// otherwise each projection keeps its own launch on the stream.  Output i has row stride N_i
+// (Sources/MetalCompiler/Generator/MetalSourceGenerator+Quantized.swift:166-338).
+mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t count, const mi355q_weight* const* weights,
+                               const void* x, int x_dtype, void* const* ys, int y_dtype, uint32_t m, uint32_t xs,
+                               uint32_t flags) {
+    if (count != 2 && count != 3)
+        return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "batched projection count must be 2 or 3 (got %u)", count);
+    if (!weights || !ys) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null weight or output array");
+    for (uint32_t i = 0; i < count; i++) {
+        if (!weights[i]) return fail(MI355Q_ERR_NULL_HANDLE, "weight handle %u is null", i);
+        if (weights[i]->ctx != ctx)
+            return fail(MI355Q_ERR_INVALID_ARGUMENT, "weight handle %u belongs to another context", i);
+        if (weights[i]->k != weights[0]->k || weights[i]->fmt.scheme_identifier != weights[0]->fmt.scheme_identifier ||
+            weights[i]->layout != weights[0]->layout)
+            return fail(MI355Q_ERR_SHAPE, "batched projections must share K, scheme and layout");
+    }
+    bool fused = m <= 8 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
+    WView views[3];
+    uint32_t strides[3];
+    for (uint32_t i = 0; i < count; i++) {
+        uint32_t x_stride = xs, y_stride = 0;
+        if (mi355q_status st = check_io(weights[i], x, x_dtype, ys[i], y_dtype, m, x_stride, y_stride)) return st;
+        xs = x_stride;
+        strides[i] = y_stride;
+        views[i] = weights[i]->view();
+        fused = fused && gemv_fast_eligible(views[i], x_dtype, m, xs) && views[i].sb_dtype == views[0].sb_dtype;
+    }
+    if (fused && (uintptr_t)x % 16 == 0)
+        return launch_gemv_fast_multi(s, ctx, count, views, x, ys, strides, y_dtype, m, xs, nullptr, nullptr, nullptr);
+    for (uint32_t i = 0; i < count; i++) {
+        mi355q_status st = dispatch_linear(ctx, s, weights[i], x, x_dtype, ys[i], y_dtype, m, xs, 0, flags, false);
+        if (st != MI355Q_OK) return st;
+    }
+    return MI355Q_OK;
+}
+
 mi355q_status dispatch_output_head(mi355q_context* ctx, hipStream_t s, const mi355q_weight* w, const void* x,
                                    int x_dtype, float* logits, int32_t* token, uint32_t flags) {
     if (!x || !token) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null pointer");
@@ -134,23 +172,9 @@ mi355q_status mi355q_batched_qgemm(mi355q_context* ctx, void* stream, uint32_t c
                                    void* const* y_devs, mi355q_dtype y_dtype, uint32_t m, uint32_t x_row_stride,
                                    uint32_t flags) {
     if (!ctx) return fail(MI355Q_ERR_NULL_HANDLE, "context is null");
-    if (count != 2 && count != 3)
-        return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "batched projection count must be 2 or 3 (got %u)", count);
-    if (!weights || !y_devs) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null weight or output array");
-    for (uint32_t i = 0; i < count; i++) {
-        if (!weights[i]) return fail(MI355Q_ERR_NULL_HANDLE, "weight handle %u is null", i);
-        if (weights[i]->k != weights[0]->k || weights[i]->fmt.scheme_identifier != weights[0]->fmt.scheme_identifier ||
-            weights[i]->layout != weights[0]->layout)
-            return fail(MI355Q_ERR_SHAPE, "batched projections must share K, scheme and layout");
-    }
-    // One shared input, `count` outputs with row stride N_i: each projection keeps its own launch;
-    // the launches are independent and queue back to back on the stream.
-    for (uint32_t i = 0; i < count; i++) {
-        mi355q_status st = mi355q_qgemm(ctx, stream, weights[i], x_dev, x_dtype, y_devs[i], y_dtype, m,
-                                        x_row_stride, 0, flags);
-        if (st != MI355Q_OK) return st;
-    }
-    return MI355Q_OK;
+    MI355Q_HIP(hipSetDevice(ctx->device));
+    return dispatch_batched(ctx, (hipStream_t)stream, count, weights, x_dev, x_dtype, y_devs, y_dtype, m,
+                            x_row_stride, flags);
 }
 
 mi355q_status mi355q_dequant_bf16(mi355q_context* ctx, void* stream, const mi355q_weight* w, void* out_bf16_dev) {

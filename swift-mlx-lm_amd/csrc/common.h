@@ -112,7 +112,15 @@ struct GemvLaunchShape {
 };
 GemvLaunchShape gemv_fast_shape(const mi355q_context* ctx, const WView& w, uint32_t m);
 
+mi355q_status launch_gemv_fast_multi(hipStream_t s, const mi355q_context* ctx, uint32_t count, const WView* w,
+                                     const void* x, void* const* y, const uint32_t* y_strides, int y_dtype,
+                                     uint32_t m, uint32_t x_stride, float* logits_f32, int32_t* token_out,
+                                     unsigned long long* argmax_scratch);
+
 // Validated dispatch shared by the direct entry points and by plan replay (api.hip)
+mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t count, const mi355q_weight* const* weights,
+                               const void* x, int x_dtype, void* const* ys, int y_dtype, uint32_t m, uint32_t xs,
+                               uint32_t flags);
 mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_weight* w, const void* x, int x_dtype,
                               void* y, int y_dtype, uint32_t m, uint32_t xs, uint32_t ys, uint32_t flags,
                               bool small_m_only);

@@ -26,16 +26,25 @@
 
 namespace mi355q {
 
+constexpr int kGemvMaxSegments = 3;
+
+// One launch covers up to three weight matrices that share K, format and activations (q+k+v,
+// gate+up).  Wavefronts are dealt to the matrices whole: matrix i owns the wavefronts
+// [wave_end[i-1], wave_end[i]), so a wavefront resolves its matrix once and then runs the
+// single-matrix code on that matrix's rows.
 struct GemvArgs {
-    const uint32_t* codes;
-    const uint32_t* sz;      // packed (scale | bias << 16) word per group
+    const uint32_t* codes[kGemvMaxSegments];
+    const uint32_t* sz[kGemvMaxSegments];      // packed (scale | bias << 16) word per group
+    void* y[kGemvMaxSegments];                 // [M, y_stride[i]] in y_dtype (may be null when only logits are wanted)
+    uint32_t wave_end[kGemvMaxSegments];       // cumulative wavefront counts; unused entries repeat the last
+    uint32_t seg_rows[kGemvMaxSegments];       // N_i
+    uint32_t y_stride[kGemvMaxSegments];
     const uint16_t* x;       // bf16 [M, x_stride]
-    void* y;                 // [M, y_stride] in y_dtype (may be null when only logits are wanted)
-    float* logits;           // optional fp32 [N] copy (M == 1)
+    float* logits;           // optional fp32 [N] copy (M == 1, single segment)
     int32_t* token_out;      // ARGMAX only
     unsigned long long* scratch;  // ARGMAX only: [0] packed max, [1] ticket
-    uint32_t n, k, m;
-    uint32_t x_stride, y_stride;
+    uint32_t k, m;
+    uint32_t x_stride;
     uint32_t words_per_row, blocks_per_row;
     uint32_t nc;             // K-steps per row = ceil(K / (64*CPL))
     uint32_t rows_per_wave;  // consecutive rows owned by one wavefront
@@ -114,7 +123,15 @@ void gemv_planes_kernel(GemvArgs a) {
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     // the wavefront index is uniform: keep it (and everything derived from it) in scalar registers
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
-    const uint32_t row0 = (blockIdx.x * WAVES + wave) * a.rows_per_wave;
+    // matrix of this wavefront (scalar select chain, once), then rows local to that matrix
+    const uint32_t gw = blockIdx.x * WAVES + wave;
+    const bool in1 = gw >= a.wave_end[0], in2 = gw >= a.wave_end[1];
+    const uint32_t* const seg_codes = in2 ? a.codes[2] : in1 ? a.codes[1] : a.codes[0];
+    const uint32_t* const seg_sz = in2 ? a.sz[2] : in1 ? a.sz[1] : a.sz[0];
+    void* const seg_y = in2 ? a.y[2] : in1 ? a.y[1] : a.y[0];
+    const uint32_t seg_ys = in2 ? a.y_stride[2] : in1 ? a.y_stride[1] : a.y_stride[0];
+    const uint32_t seg_n = in2 ? a.seg_rows[2] : in1 ? a.seg_rows[1] : a.seg_rows[0];
+    const uint32_t row0 = (gw - (in2 ? a.wave_end[1] : in1 ? a.wave_end[0] : 0u)) * a.rows_per_wave;
     const uint32_t nsteps = (a.rows_per_wave / R) * NC;     // same for every wavefront, >= 1
 
     struct Pref {
@@ -136,9 +153,9 @@ void gemv_planes_kernel(GemvArgs a) {
 #pragma unroll
         for (int r = 0; r < R; r++) {
             uint32_t row = row0 + rg * R + r;
-            row = row < a.n ? row : a.n - 1;
-            const uint32_t* rowp = a.codes + (size_t)row * a.words_per_row;     // scalar
-            const uint32_t* szp = a.sz + (size_t)row * a.blocks_per_row;        // scalar
+            row = row < seg_n ? row : seg_n - 1;
+            const uint32_t* rowp = seg_codes + (size_t)row * a.words_per_row;   // scalar
+            const uint32_t* szp = seg_sz + (size_t)row * a.blocks_per_row;      // scalar
             if constexpr (WPL == 4) {
                 const u32x4 v = *(const u32x4*)(rowp + code_off);
                 p.w[r][0] = v.x; p.w[r][1] = v.y; p.w[r][2] = v.z; p.w[r][3] = v.w;
@@ -306,15 +323,17 @@ void gemv_planes_kernel(GemvArgs a) {
 
     auto flush = [&](uint32_t first_local, uint32_t count) {   // rows [first_local, +count) -> memory
         const uint32_t row = row0 + first_local + lane;
-        if (lane < count && row < a.n) {
+        if (lane < count && row < seg_n) {
+            void* const yb = seg_y;
+            const uint32_t ys = seg_ys, lrow = row;
 #pragma unroll
             for (int m = 0; m < MT; m++) {
                 if ((uint32_t)m < a.m) {
-                    if (a.y) {
-                        const size_t o = (size_t)m * a.y_stride + row;
-                        if (a.y_dtype == MI355Q_F32) ((float*)a.y)[o] = res[m];
-                        else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)a.y)[o] = f32_to_bf16_rne(res[m]);
-                        else ((uint16_t*)a.y)[o] = f32_to_f16_rne(res[m]);
+                    if (yb) {
+                        const size_t o = (size_t)m * ys + lrow;
+                        if (a.y_dtype == MI355Q_F32) ((float*)yb)[o] = res[m];
+                        else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)yb)[o] = f32_to_bf16_rne(res[m]);
+                        else ((uint16_t*)yb)[o] = f32_to_f16_rne(res[m]);
                     }
                     if (a.logits && m == 0) a.logits[row] = res[m];
                 }

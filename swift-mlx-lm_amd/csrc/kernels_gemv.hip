@@ -121,46 +121,76 @@ GemvLaunchShape gemv_fast_shape(const mi355q_context* ctx, const WView& w, uint3
     return s;
 }
 
-mi355q_status launch_gemv_fast(hipStream_t s, const mi355q_context* ctx, const WView& w, const void* x, void* y,
-                               int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride, float* logits_f32,
-                               int32_t* token_out, unsigned long long* argmax_scratch) {
+// Up to three weights sharing K, format and activations in one launch.  `w[0]` supplies the format;
+// the caller has checked that the others match.
+mi355q_status launch_gemv_fast_multi(hipStream_t s, const mi355q_context* ctx, uint32_t count, const WView* w,
+                                     const void* x, void* const* y, const uint32_t* y_strides, int y_dtype,
+                                     uint32_t m, uint32_t x_stride, float* logits_f32, int32_t* token_out,
+                                     unsigned long long* argmax_scratch) {
+    if (count < 1 || count > (uint32_t)kGemvMaxSegments)
+        return fail(MI355Q_ERR_INVALID_ARGUMENT, "1..%d weights per fused launch", kGemvMaxSegments);
     if ((uintptr_t)x % 16) return fail(MI355Q_ERR_INVALID_ARGUMENT, "activation pointer must be 16-byte aligned");
     const bool argmax = token_out != nullptr;
-    if (argmax && m != 1) return fail(MI355Q_ERR_INVALID_ARGUMENT, "fused argmax needs M == 1");
-    const int fit = max_mt(w);
-    if (!fit) return fail(MI355Q_ERR_SHAPE, "K=%u does not fit the activation staging budget", w.k);
+    if (argmax && (m != 1 || count != 1)) return fail(MI355Q_ERR_INVALID_ARGUMENT, "fused argmax needs M == 1");
+    if (logits_f32 && count != 1) return fail(MI355Q_ERR_INVALID_ARGUMENT, "fp32 logits need a single weight");
+    WView all = w[0];                       // same geometry, rows of every segment together
+    uint64_t total = 0;
+    for (uint32_t i = 0; i < count; i++) total += w[i].n;
+    if (total > 0xFFFFFFFFull) return fail(MI355Q_ERR_SHAPE, "too many rows");
+    all.n = (uint32_t)total;
+    const int fit = max_mt(all);
+    if (!fit) return fail(MI355Q_ERR_SHAPE, "K=%u does not fit the activation staging budget", all.k);
     const size_t ysz = y_dtype == MI355Q_F32 ? 4 : 2;
     // activation batches larger than what fits in LDS are processed in slices of `fit` rows
     for (uint32_t m0 = 0; m0 < m; m0 += (uint32_t)fit) {
         const uint32_t mm = (m - m0) < (uint32_t)fit ? (m - m0) : (uint32_t)fit;
-        const GemvCfg c = choose(ctx, w, mm, argmax);
+        GemvCfg c = choose(ctx, all, mm, argmax);
         GemvArgs a{};
-        a.codes = w.codes;
-        a.sz = w.sz;
+        uint32_t waves = 0;
+        for (uint32_t i = 0; i < (uint32_t)kGemvMaxSegments; i++) {
+            const uint32_t j = i < count ? i : count - 1;
+            if (i < count) waves += (w[i].n + c.rows_per_wave - 1) / c.rows_per_wave;
+            a.codes[i] = w[j].codes;
+            a.sz[i] = w[j].sz;
+            a.y[i] = y[j] ? (void*)((char*)y[j] + (size_t)m0 * y_strides[j] * ysz) : nullptr;
+            a.y_stride[i] = y_strides[j];
+            a.seg_rows[i] = w[j].n;
+            a.wave_end[i] = waves;
+        }
+        const uint32_t grid = (waves + (uint32_t)c.waves - 1) / (uint32_t)c.waves;
         a.x = (const uint16_t*)x + (size_t)m0 * x_stride;
-        a.y = y ? (void*)((char*)y + (size_t)m0 * y_stride * ysz) : nullptr;
         a.logits = logits_f32;
         a.token_out = token_out;
         a.scratch = argmax_scratch;
-        a.n = w.n; a.k = w.k; a.m = mm;
-        a.x_stride = x_stride; a.y_stride = y_stride;
-        a.words_per_row = w.words_per_row; a.blocks_per_row = w.blocks_per_row;
+        a.k = all.k; a.m = mm;
+        a.x_stride = x_stride;
+        a.words_per_row = all.words_per_row; a.blocks_per_row = all.blocks_per_row;
         a.nc = c.nc; a.rows_per_wave = c.rows_per_wave;
-        a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = w.sb_dtype;
+        a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = all.sb_dtype;
         a.dbg = (uint32_t)env_int("MI355Q_GEMV_DBG", 0);
+        c.grid = grid;                        // whole wavefronts per matrix: a few more than rows / rows_per_wave
         mi355q_status st;
-        switch (w.bits) {
-        case 2: st = launch_gemv_planes_q2(s, a, (int)w.group, c); break;
-        case 3: st = launch_gemv_planes_q3(s, a, (int)w.group, c); break;
-        case 4: st = launch_gemv_planes_q4(s, a, (int)w.group, c); break;
-        case 5: st = launch_gemv_planes_q5(s, a, (int)w.group, c); break;
-        case 6: st = launch_gemv_planes_q6(s, a, (int)w.group, c); break;
-        case 8: st = launch_gemv_planes_q8(s, a, (int)w.group, c); break;
-        default: st = fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no split-plane GEMV for %u-bit codes", w.bits);
+        switch (all.bits) {
+        case 2: st = launch_gemv_planes_q2(s, a, (int)all.group, c); break;
+        case 3: st = launch_gemv_planes_q3(s, a, (int)all.group, c); break;
+        case 4: st = launch_gemv_planes_q4(s, a, (int)all.group, c); break;
+        case 5: st = launch_gemv_planes_q5(s, a, (int)all.group, c); break;
+        case 6: st = launch_gemv_planes_q6(s, a, (int)all.group, c); break;
+        case 8: st = launch_gemv_planes_q8(s, a, (int)all.group, c); break;
+        default: st = fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no split-plane GEMV for %u-bit codes", all.bits);
         }
         if (st != MI355Q_OK) return st;
     }
     return MI355Q_OK;
+}
+
+mi355q_status launch_gemv_fast(hipStream_t s, const mi355q_context* ctx, const WView& w, const void* x, void* y,
+                               int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride, float* logits_f32,
+                               int32_t* token_out, unsigned long long* argmax_scratch) {
+    void* ys[1] = {y};
+    const uint32_t strides[1] = {y_stride};
+    return launch_gemv_fast_multi(s, ctx, 1, &w, x, ys, strides, y_dtype, m, x_stride, logits_f32, token_out,
+                                  argmax_scratch);
 }
 
 }  // namespace mi355q

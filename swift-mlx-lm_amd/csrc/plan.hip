@@ -11,7 +11,7 @@ using namespace mi355q;
 
 namespace {
 
-enum StepKind { kLinear = 0, kOutputHead = 1 };
+enum StepKind { kLinear = 0, kOutputHead = 1, kBatched = 2 };
 
 struct PlanStep {
     StepKind kind;
@@ -24,6 +24,10 @@ struct PlanStep {
     int32_t layer_index;
     std::string tensor_name;
     mi355q_step record;
+    // kBatched: 2 or 3 projections sharing x
+    uint32_t count;
+    const mi355q_weight* ws[3];
+    void* ysv[3];
 };
 
 }  // namespace
@@ -47,6 +51,9 @@ mi355q_status encode_range(mi355q_plan* plan, hipStream_t s, uint32_t first, uin
         if (st.kind == kLinear)
             rc = dispatch_linear(plan->ctx, s, st.w, st.x, st.x_dtype, st.y, st.y_dtype, st.m, st.xs, st.ys, st.flags,
                                  false);
+        else if (st.kind == kBatched)
+            rc = dispatch_batched(plan->ctx, s, st.count, st.ws, st.x, st.x_dtype, st.ysv, st.y_dtype, st.m, st.xs,
+                                  st.flags);
         else
             rc = dispatch_output_head(plan->ctx, s, st.w, st.x, st.x_dtype, (float*)st.y, st.token, st.flags);
         if (rc != MI355Q_OK) return rc;
@@ -108,6 +115,52 @@ mi355q_status mi355q_plan_add_linear(mi355q_plan* plan, const mi355q_weight* w, 
         st.record = two[0];
     }
     if (rc != MI355Q_OK) return rc;
+    plan->steps.push_back(st);
+    return MI355Q_OK;
+}
+
+mi355q_status mi355q_plan_add_batched_linear(mi355q_plan* plan, uint32_t count, const mi355q_weight* const* weights,
+                                             const void* x_dev, mi355q_dtype x_dtype, void* const* y_devs,
+                                             mi355q_dtype y_dtype, uint32_t m, uint32_t x_row_stride, uint32_t flags,
+                                             int32_t layer_index, const char* tensor_name) {
+    if (!plan) return fail(MI355Q_ERR_NULL_HANDLE, "plan is null");
+    if (count != 2 && count != 3)
+        return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "batched projection count must be 2 or 3 (got %u)", count);
+    if (!weights || !y_devs || !x_dev) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null pointer");
+    if (m == 0) return fail(MI355Q_ERR_INVALID_ARGUMENT, "sequence length M must be >= 1");
+    if (plan->graph_exec) return fail(MI355Q_ERR_INVALID_ARGUMENT, "plan is frozen: its graph has been built");
+    PlanStep st{};
+    st.kind = kBatched;
+    st.count = count;
+    for (uint32_t i = 0; i < count; i++) {
+        if (!weights[i]) return fail(MI355Q_ERR_NULL_HANDLE, "weight handle %u is null", i);
+        if (weights[i]->ctx != plan->ctx)
+            return fail(MI355Q_ERR_INVALID_ARGUMENT, "weight handle %u belongs to another context", i);
+        if (!y_devs[i]) return fail(MI355Q_ERR_INVALID_ARGUMENT, "output pointer %u is null", i);
+        st.ws[i] = weights[i];
+        st.ysv[i] = y_devs[i];
+    }
+    st.w = weights[0]; st.x = x_dev; st.y = y_devs[0]; st.token = nullptr;
+    st.x_dtype = x_dtype; st.y_dtype = y_dtype;
+    st.m = m;
+    st.xs = x_row_stride ? x_row_stride : (uint32_t)weights[0]->k;
+    st.ys = 0;
+    st.flags = flags;
+    st.layer_index = layer_index;
+    if (tensor_name) st.tensor_name = tensor_name;
+    // the record describes the first projection; the family says that the launch is shared
+    mi355q_status rc;
+    if (m <= 8) {
+        rc = mi355q_plan_decode_step(weights[0], m, x_dtype, flags, &st.record);
+    } else {
+        mi355q_step two[2];
+        uint32_t cnt = 0;
+        rc = mi355q_plan_prefill_steps(weights[0], m, st.xs, x_dtype, 0, flags, two, &cnt);
+        st.record = two[0];
+    }
+    if (rc != MI355Q_OK) return rc;
+    std::snprintf(st.record.kernel_family, sizeof st.record.kernel_family, "batched%uQ%uG%u", count,
+                  (unsigned)weights[0]->fmt.bits, weights[0]->fmt.group_size);
     plan->steps.push_back(st);
     return MI355Q_OK;
 }
