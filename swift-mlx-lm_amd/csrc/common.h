@@ -42,6 +42,8 @@ struct WView {
     uint32_t n, k;
     uint32_t group, bits;
     uint32_t bytes_per_block, blocks_per_row, words_per_row;
+    uint32_t code_stride;     // planes: 32-bit words from one row of codes to the next (>= words_per_row)
+    uint32_t sz_stride;       // planes: 32-bit words from one row of sz to the next (>= blocks_per_row)
     uint32_t layout;          // mi355q_layout
     uint32_t sb_dtype;        // mi355q_dtype of scale/bias (F16 for STAF)
 };
@@ -64,7 +66,13 @@ struct mi355q_weight {
     void* codes;
     void* scales;
     void* biases;
-    void* sz;                 // owned: packed (scale, bias) words for the planes layout
+    void* sz;                 // packed (scale, bias) words for the planes layout
+    // Owned plane weights keep each row's code words and its sz words side by side in ONE buffer
+    // ([codes of row r | sz of row r | pad to 16 bytes]): `codes` points at it, `sz` points
+    // words_per_row further, and both advance by the same stride, so a row is one contiguous
+    // stream in memory.  Borrowed planes (wrap) keep the caller's codes and an owned sz plane.
+    uint32_t code_stride, sz_stride;   // in 32-bit words
+    uint8_t sz_separate;               // sz is an allocation of its own (borrowed planes)
     size_t blocks_bytes, codes_bytes, sb_bytes;
     mi355q::WView view() const {
         mi355q::WView v;
@@ -80,6 +88,8 @@ struct mi355q_weight {
         v.bytes_per_block = fmt.bytes_per_block;
         v.blocks_per_row = (uint32_t)(k / fmt.group_size);
         v.words_per_row = (uint32_t)(k * fmt.bits / 32);
+        v.code_stride = code_stride;
+        v.sz_stride = sz_stride;
         v.layout = layout;
         v.sb_dtype = sb_dtype;
         return v;
@@ -98,7 +108,7 @@ mi355q_status launch_gemv_generic(hipStream_t s, const WView& w, const void* x, 
 mi355q_status launch_argmax(hipStream_t s, const void* logits, int dtype, uint32_t n,
                             int32_t* token_out);
 mi355q_status launch_pack_sz(hipStream_t s, const uint16_t* scales, const uint16_t* biases, uint32_t* sz,
-                             size_t groups);
+                             size_t groups, uint32_t blocks_per_row, uint32_t sz_stride);
 
 // Fast split-plane GEMV (kernels_gemv.hip).  can_* say whether a shape is eligible.
 bool gemv_fast_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);

@@ -74,7 +74,7 @@ __device__ __forceinline__ void store_out(void* p, size_t i, float v) {
 __device__ __forceinline__ uint32_t load_code(const WView& w, uint32_t row, uint32_t c) {
     const uint32_t mask = (1u << w.bits) - 1u;
     if (w.layout == MI355Q_LAYOUT_PLANES) {
-        const uint32_t* rowp = w.codes + (size_t)row * w.words_per_row;
+        const uint32_t* rowp = w.codes + (size_t)row * w.code_stride;
         const uint64_t bit = (uint64_t)c * w.bits;
         const uint32_t word = (uint32_t)(bit >> 5), sh = (uint32_t)(bit & 31);
         uint32_t v = rowp[word] >> sh;

@@ -45,7 +45,7 @@ struct GemvArgs {
     unsigned long long* scratch;  // ARGMAX only: [0] packed max, [1] ticket
     uint32_t k, m;
     uint32_t x_stride;
-    uint32_t words_per_row, blocks_per_row;
+    uint32_t code_stride, sz_stride;   // 32-bit words between consecutive rows
     uint32_t nc;             // K-steps per row = ceil(K / (64*CPL))
     uint32_t rows_per_wave;  // consecutive rows owned by one wavefront
     uint32_t y_dtype, sb_dtype;
@@ -154,8 +154,8 @@ void gemv_planes_kernel(GemvArgs a) {
         for (int r = 0; r < R; r++) {
             uint32_t row = row0 + rg * R + r;
             row = row < seg_n ? row : seg_n - 1;
-            const uint32_t* rowp = seg_codes + (size_t)row * a.words_per_row;   // scalar
-            const uint32_t* szp = seg_sz + (size_t)row * a.blocks_per_row;      // scalar
+            const uint32_t* rowp = seg_codes + (size_t)row * a.code_stride;    // scalar
+            const uint32_t* szp = seg_sz + (size_t)row * a.sz_stride;          // scalar
             if constexpr (WPL == 4) {
                 const u32x4 v = *(const u32x4*)(rowp + code_off);
                 p.w[r][0] = v.x; p.w[r][1] = v.y; p.w[r][2] = v.z; p.w[r][3] = v.w;
@@ -203,7 +203,10 @@ void gemv_planes_kernel(GemvArgs a) {
         uint32_t m, cc;
         task_coords(tw, m, cc);
         const uint64_t kbase = (uint64_t)cc * KC + (uint64_t)lane * CPL;
-        const bool valid = tw < nwt && m < a.m && kbase < a.k;
+        bool valid = tw < nwt && m < a.m && kbase < a.k;
+#ifdef MI355Q_GEMV_EXPERIMENT
+        if (a.dbg & 8) valid = false;                       // every lane reads the same line
+#endif
         const u32x4* src = (const u32x4*)(a.x + (valid ? (size_t)m * a.x_stride + kbase : 0));
 #pragma unroll
         for (int i = 0; i < Q; i++) {
@@ -280,9 +283,14 @@ void gemv_planes_kernel(GemvArgs a) {
         }
     }
     // LDS-only barrier: the weight loads in flight must not be waited for here
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+#ifdef MI355Q_GEMV_EXPERIMENT
+    if (!(a.dbg & 16))
+#endif
+    {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    }
 
     // ---- optional register-resident activation slice (M == 1, rows of XREG K-steps) -----------
     u32x4 xr[XC][Q];

@@ -36,7 +36,7 @@ struct GemmArgs {
     const uint16_t* x;       // bf16 [M, xs]
     void* y;
     uint32_t m, n, k, xs, ys;
-    uint32_t words_per_row, blocks_per_row;
+    uint32_t code_stride, sz_stride;   // 32-bit words between consecutive rows
     uint32_t y_dtype, sb_dtype;
     uint32_t tiles_m, tiles_n;
 };
@@ -99,7 +99,7 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(GemmArgs a) {
             xa[p] = *(const u32x4*)(a.x + (size_t)gr * a.xs + k0 + a_chunk * 8);
         });
         if constexpr (QUANT) {
-            const uint32_t* src = a.codes + (size_t)b_grow * a.words_per_row + (size_t)kt * (kTileK * BITS / 32) +
+            const uint32_t* src = a.codes + (size_t)b_grow * a.code_stride + (size_t)kt * (kTileK * BITS / 32) +
                                   b_part * WPT;
             if constexpr (WPT % 4 == 0) {
                 static_for<WPT / 4>([&](auto I) __attribute__((always_inline)) {
@@ -121,7 +121,7 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(GemmArgs a) {
             }
             static_for<NGT>([&](auto G) __attribute__((always_inline)) {
                 constexpr int g = decltype(G)::value;
-                szreg[g] = a.sz[(size_t)b_grow * a.blocks_per_row + (k0 + b_part * CPT + g * GROUP) / GROUP];
+                szreg[g] = a.sz[(size_t)b_grow * a.sz_stride + (k0 + b_part * CPT + g * GROUP) / GROUP];
             });
         } else {
             static_for<B_DENSE_PASSES>([&](auto P) __attribute__((always_inline)) {
@@ -298,7 +298,7 @@ bool gemm_mfma_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stri
     if (m < 1) return false;
     if (w.k % kTileK) return false;
     if (x_stride % 8) return false;                       // 128-bit activation loads
-    if ((uintptr_t)w.codes % 16) return false;
+    if ((uintptr_t)w.codes % 16 || w.code_stride % 4) return false;
     const bool fmt_ok = (w.bits == 4 && (w.group == 64 || w.group == 128)) ||
                         (w.bits == 8 && (w.group == 32 || w.group == 64)) ||
                         (w.bits == 6 && w.group == 64) || (w.bits == 3 && w.group == 64) ||
@@ -314,7 +314,7 @@ mi355q_status launch_qgemm_mfma(hipStream_t s, const mi355q_context* ctx, const 
     a.codes = w.codes; a.sz = w.sz; a.bdense = nullptr;
     a.x = (const uint16_t*)x; a.y = y;
     a.m = m; a.n = w.n; a.k = w.k; a.xs = x_stride; a.ys = y_stride;
-    a.words_per_row = w.words_per_row; a.blocks_per_row = w.blocks_per_row;
+    a.code_stride = w.code_stride; a.sz_stride = w.sz_stride;
     a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = w.sb_dtype;
     switch (w.bits * 1000 + w.group) {
     case 4064: return launch_shape<4, 64, true>(s, ctx, a);

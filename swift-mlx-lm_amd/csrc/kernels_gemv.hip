@@ -102,7 +102,7 @@ bool gemv_fast_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stri
     if (!g.cpl) return false;
     if (w.k % (uint32_t)g.cpl) return false;       // rows are whole lane chunks
     if (x_stride % 8) return false;                // 128-bit activation loads
-    if ((uintptr_t)w.codes % 16) return false;     // 128-bit code loads
+    if ((uintptr_t)w.codes % 16 || w.code_stride % 4) return false;     // 128-bit code loads
     if (!w.sz) return false;
     if (max_mt(w) == 0) return false;
     return true;
@@ -164,7 +164,7 @@ mi355q_status launch_gemv_fast_multi(hipStream_t s, const mi355q_context* ctx, u
         a.scratch = argmax_scratch;
         a.k = all.k; a.m = mm;
         a.x_stride = x_stride;
-        a.words_per_row = all.words_per_row; a.blocks_per_row = all.blocks_per_row;
+        a.code_stride = all.code_stride; a.sz_stride = all.sz_stride;
         a.nc = c.nc; a.rows_per_wave = c.rows_per_wave;
         a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = all.sb_dtype;
         a.dbg = (uint32_t)env_int("MI355Q_GEMV_DBG", 0);

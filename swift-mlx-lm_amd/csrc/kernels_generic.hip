@@ -36,18 +36,22 @@ mi355q_status launch_unpack_codes(hipStream_t s, const WView& w, uint8_t* out) {
 // scale in the low half, bias in the high half, so the GEMV fetches both with one load.
 __global__ __launch_bounds__(256) void pack_sz_kernel(const uint16_t* __restrict__ scales,
                                                       const uint16_t* __restrict__ biases,
-                                                      uint32_t* __restrict__ sz, size_t groups) {
+                                                      uint32_t* __restrict__ sz, size_t groups,
+                                                      uint32_t blocks_per_row, uint32_t sz_stride) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (; i < groups; i += stride) sz[i] = (uint32_t)scales[i] | ((uint32_t)biases[i] << 16);
+    for (; i < groups; i += stride) {
+        const size_t row = i / blocks_per_row, b = i - row * blocks_per_row;
+        sz[row * sz_stride + b] = (uint32_t)scales[i] | ((uint32_t)biases[i] << 16);
+    }
 }
 
 mi355q_status launch_pack_sz(hipStream_t s, const uint16_t* scales, const uint16_t* biases, uint32_t* sz,
-                             size_t groups) {
+                             size_t groups, uint32_t blocks_per_row, uint32_t sz_stride) {
     size_t blocks = (groups + 255) / 256;
     if (blocks > 8192) blocks = 8192;
     if (blocks == 0) blocks = 1;
-    pack_sz_kernel<<<dim3((unsigned)blocks), dim3(256), 0, s>>>(scales, biases, sz, groups);
+    pack_sz_kernel<<<dim3((unsigned)blocks), dim3(256), 0, s>>>(scales, biases, sz, groups, blocks_per_row, sz_stride);
     MI355Q_HIP(hipGetLastError());
     return MI355Q_OK;
 }

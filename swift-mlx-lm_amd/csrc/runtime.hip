@@ -98,15 +98,43 @@ mi355q_status upload_new(void** dev, const void* host, size_t bytes) {
     return MI355Q_OK;
 }
 
-// Packed (scale, bias) plane of a split-plane weight: allocated and filled once, on the device.
-mi355q_status build_sz(mi355q_weight* w) {
-    const size_t groups = (size_t)w->n * (w->k / w->fmt.group_size);
-    MI355Q_HIP(hipMalloc(&w->sz, groups * 4));
+// Packed (scale, bias) words of a split-plane weight, filled once on the device from the two
+// 16-bit planes.  `dst` is either the sz part of the row-interleaved buffer or a plane of its own.
+mi355q_status fill_sz(mi355q_weight* w) {
+    const uint32_t bpr = (uint32_t)(w->k / w->fmt.group_size);
+    const size_t groups = (size_t)w->n * bpr;
     if (mi355q_status st = launch_pack_sz(nullptr, (const uint16_t*)w->scales, (const uint16_t*)w->biases,
-                                          (uint32_t*)w->sz, groups))
+                                          (uint32_t*)w->sz, groups, bpr, w->sz_stride))
         return st;
     MI355Q_HIP(hipStreamSynchronize(nullptr));
     return MI355Q_OK;
+}
+
+// Borrowed planes: the caller's code plane stays where it is; sz is an owned plane of its own.
+mi355q_status build_sz_plane(mi355q_weight* w) {
+    const uint32_t bpr = (uint32_t)(w->k / w->fmt.group_size);
+    w->code_stride = (uint32_t)(w->k * w->fmt.bits / 32);
+    w->sz_stride = bpr;
+    w->sz_separate = 1;
+    MI355Q_HIP(hipMalloc(&w->sz, (size_t)w->n * bpr * 4));
+    return fill_sz(w);
+}
+
+// Owned planes: one buffer of rows [code words | sz words | pad to 16 bytes].  The host code plane
+// is copied with a pitched copy; scales/biases must already be on the device.
+mi355q_status build_rows(mi355q_weight* w, const void* codes_host) {
+    const uint32_t wpr = (uint32_t)(w->k * w->fmt.bits / 32), bpr = (uint32_t)(w->k / w->fmt.group_size);
+    const uint32_t stride = (wpr + bpr + 3u) & ~3u;
+    w->code_stride = stride;
+    w->sz_stride = stride;
+    w->sz_separate = 0;
+    w->codes_bytes = (size_t)w->n * stride * 4;
+    MI355Q_HIP(hipMalloc(&w->codes, w->codes_bytes));
+    w->sz = (uint32_t*)w->codes + wpr;
+    if (stride != wpr + bpr) MI355Q_HIP(hipMemset(w->codes, 0, w->codes_bytes));   // padding words
+    MI355Q_HIP(hipMemcpy2D(w->codes, (size_t)stride * 4, codes_host, (size_t)wpr * 4, (size_t)wpr * 4, (size_t)w->n,
+                           hipMemcpyHostToDevice));
+    return fill_sz(w);
 }
 
 mi355q_status need_ctx(mi355q_context* ctx) {
@@ -335,10 +363,8 @@ mi355q_status mi355q_weight_prepare_mlx(mi355q_context* ctx, uint8_t scheme_iden
         w->blocks_bytes = blocks.size();
         st = upload_new(&w->blocks, blocks.data(), blocks.size());
     } else {
-        w->codes_bytes = (size_t)n_rows * (k * f->bits / 32) * 4;
         w->sb_bytes = groups * 2;
-        st = upload_new(&w->codes, codes_host, w->codes_bytes);
-        if (st == MI355Q_OK) {
+        {
             if (sb_dtype == MI355Q_F32) {  // normalised to f16 like the converter
                 std::vector<uint16_t> s16(groups), z16(groups);
                 for (size_t i = 0; i < groups; i++) {
@@ -355,7 +381,7 @@ mi355q_status mi355q_weight_prepare_mlx(mi355q_context* ctx, uint8_t scheme_iden
             }
         }
     }
-    if (st == MI355Q_OK && layout == MI355Q_LAYOUT_PLANES) st = build_sz(w);
+    if (st == MI355Q_OK && layout == MI355Q_LAYOUT_PLANES) st = build_rows(w, codes_host);
     if (st != MI355Q_OK) {
         mi355q_weight_destroy(w);
         return st;
@@ -388,13 +414,15 @@ mi355q_status mi355q_weight_prepare_staf(mi355q_context* ctx, uint8_t scheme_ide
     w->layout = (uint8_t)layout;
     w->sb_dtype = MI355Q_F16;
     mi355q_status st;
+    std::vector<uint8_t> planes_codes;           // de-interleaved code plane (host), PLANES only
     if (layout == MI355Q_LAYOUT_STAF_BLOCKS) {
         w->blocks_bytes = payload_bytes;
         st = upload_new(&w->blocks, blocks_host, payload_bytes);
     } else {
         const size_t bpr = k / f->group_size;
         const size_t row_bytes = k * f->bits / 8, group_bytes = (size_t)f->group_size * f->bits / 8;
-        std::vector<uint8_t> codes((size_t)n_rows * row_bytes);
+        std::vector<uint8_t>& codes = planes_codes;
+        codes.resize((size_t)n_rows * row_bytes);
         std::vector<uint16_t> s16(groups), z16(groups);
         for (size_t r = 0; r < n_rows; r++)
             for (size_t b = 0; b < bpr; b++) {
@@ -403,13 +431,11 @@ mi355q_status mi355q_weight_prepare_staf(mi355q_context* ctx, uint8_t scheme_ide
                 std::memcpy(&z16[r * bpr + b], src + 2, 2);
                 std::memcpy(codes.data() + r * row_bytes + b * group_bytes, src + 4, group_bytes);
             }
-        w->codes_bytes = codes.size();
         w->sb_bytes = groups * 2;
-        st = upload_new(&w->codes, codes.data(), codes.size());
-        if (st == MI355Q_OK) st = upload_new(&w->scales, s16.data(), w->sb_bytes);
+        st = upload_new(&w->scales, s16.data(), w->sb_bytes);
         if (st == MI355Q_OK) st = upload_new(&w->biases, z16.data(), w->sb_bytes);
     }
-    if (st == MI355Q_OK && layout == MI355Q_LAYOUT_PLANES) st = build_sz(w);
+    if (st == MI355Q_OK && layout == MI355Q_LAYOUT_PLANES) st = build_rows(w, planes_codes.data());
     if (st != MI355Q_OK) {
         mi355q_weight_destroy(w);
         return st;
@@ -472,7 +498,7 @@ mi355q_status mi355q_weight_wrap_planes(mi355q_context* ctx, uint8_t scheme_iden
         delete w;
         return fail(MI355Q_ERR_DEVICE, "hipSetDevice failed");
     }
-    if (mi355q_status st = build_sz(w)) {
+    if (mi355q_status st = build_sz_plane(w)) {
         if (w->sz) (void)hipFree(w->sz);
         delete w;
         return st;
@@ -510,7 +536,7 @@ mi355q_status mi355q_weight_destroy(mi355q_weight* w) {
         if (w->scales) (void)hipFree(w->scales);
         if (w->biases) (void)hipFree(w->biases);
     }
-    if (w->sz) (void)hipFree(w->sz);
+    if (w->sz && w->sz_separate) (void)hipFree(w->sz);
     delete w;
     return MI355Q_OK;
 }
