@@ -55,6 +55,11 @@ def _compile(src: str, force: bool) -> str:
 def build(force: bool = False, jobs: int | None = None) -> str:
     os.makedirs(OBJ, exist_ok=True)
     os.makedirs(LIBDIR, exist_ok=True)
+    # objects compiled with other flags are stale whatever their age
+    stamp = os.path.join(OBJ, "flags.txt")
+    flags_now = " ".join(FLAGS)
+    if not os.path.exists(stamp) or open(stamp).read() != flags_now:
+        force = True
     jobs = jobs or min(8, os.cpu_count() or 4)
     srcs = sources()
     with ThreadPoolExecutor(max_workers=jobs) as ex:
@@ -64,6 +69,8 @@ def build(force: bool = False, jobs: int | None = None) -> str:
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError("link failed:\n" + r.stderr)
+    with open(stamp, "w") as f:
+        f.write(flags_now)
     return LIB
 
 

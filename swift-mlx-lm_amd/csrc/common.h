@@ -140,7 +140,7 @@ int env_int_cached(const char* name, int fallback);
 
 // MFMA GEMM (kernels_gemm.hip)
 struct GemmLaunchShape {
-    uint32_t bm, bn, grid, block, lds_bytes;
+    uint32_t bm, bn, stages, grid, block, lds_bytes;
 };
 GemmLaunchShape gemm_mfma_shape(const mi355q_context* ctx, uint32_t m, uint32_t n);
 bool gemm_mfma_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);

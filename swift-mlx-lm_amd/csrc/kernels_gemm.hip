@@ -39,6 +39,7 @@ struct GemmArgs {
     uint32_t code_stride, sz_stride;   // 32-bit words between consecutive rows
     uint32_t y_dtype, sb_dtype;
     uint32_t tiles_m, tiles_n;
+    uint32_t dbg;            // tuning builds only: bit0 fetch only the first K-tile, bit1 fill LDS only once
 };
 
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
@@ -49,20 +50,34 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
 constexpr int kTileK = 64;            // codes (and bf16 elements) per K-tile
 constexpr int kRowBytes = kTileK * 2; // one LDS row
 
+// Byte offset of 16-byte chunk `chunk` of tile row `row`.  The LDS has 64 banks of 4 bytes: a row
+// of 128 bytes covers half of them, so two consecutive rows fill all banks and the chunk position
+// is rotated by (row / 2) % 8: any 16 consecutive rows reading (or writing) the same logical chunk
+// touch 16 different bank groups.
 __device__ __forceinline__ uint32_t lds_off(uint32_t row, uint32_t chunk) {
-    return row * kRowBytes + ((chunk ^ (row & 7u)) << 4);
+    return row * kRowBytes + ((chunk ^ ((row >> 1) & 7u)) << 4);
 }
 
-template <int BITS, int GROUP, int BM, int BN, bool QUANT>
-__global__ __launch_bounds__(256) void qgemm_mfma_kernel(GemmArgs a) {
-    constexpr int TM = BM / 64, TN = BN / 64;             // 32x32 accumulators per wavefront
+// STAGES = 2: double-buffered LDS, one barrier per K-tile, one workgroup per CU for the big tiles.
+// STAGES = 1: one LDS stage and two barriers per K-tile, sized so that two workgroups share a CU
+// (and each SIMD holds two wavefronts): one workgroup's matrix-core phase covers the other's
+// dequantisation, LDS fill and barrier.
+// WAVES = 4: wavefronts 2 x 2 over the tile, one per SIMD.  WAVES = 8: 2 x 4, two per SIMD, so that
+// one wavefront's LDS waits and barrier skew are covered by the other's MFMAs.
+template <int BITS, int GROUP, int BM, int BN, bool QUANT, int STAGES, bool SB_BF16, int WAVES>
+__global__ __launch_bounds__(WAVES * 64, (STAGES == 1 ? 2 : 1)) void qgemm_mfma_kernel(GemmArgs a) {
+    constexpr int NT = WAVES * 64;                        // threads
+    constexpr int WN = WAVES / 2;                         // wavefronts along N (2 along M)
+    constexpr int TM = BM / 2 / 32, TN = BN / WN / 32;    // 32x32 accumulators per wavefront
     constexpr int A_BYTES = BM * kRowBytes, B_BYTES = BN * kRowBytes, STAGE = A_BYTES + B_BYTES;
-    constexpr int A_PASSES = BM / 32;                     // 16-byte chunks per thread for the X tile
-    constexpr int TPR = 256 / BN;                         // threads per weight row (1 or 2)
+    constexpr int RPP = NT / 8;                           // tile rows covered by one pass of 16-byte chunks
+    constexpr int A_PASSES = BM / RPP;                    // 16-byte chunks per thread for the X tile
+    constexpr int TPR = NT / BN;                          // threads per weight row
     constexpr int CPT = kTileK / TPR;                     // codes per thread per K-tile
     constexpr int WPT = QUANT ? CPT * BITS / 32 : 0;      // code words per thread per K-tile
     constexpr int NGT = QUANT ? (CPT > GROUP ? CPT / GROUP : 1) : 0;   // groups a thread touches
-    constexpr int B_DENSE_PASSES = BN / 32;
+    constexpr int B_DENSE_PASSES = BN / RPP;
+    static_assert(TPR >= 1 && CPT % 8 == 0, "weight tile does not split over the threads");
 
     extern __shared__ uint4 smem_q[];
     char* lds = (char*)smem_q;
@@ -77,12 +92,18 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(GemmArgs a) {
 
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
-    const uint32_t wm = wave >> 1, wn = wave & 1;
+    const uint32_t wm = wave / WN, wn = wave % WN;
 
-    // ---- global -> register fetch of one K-tile -----------------------------------------------
+    // ---- global -> register fetch and register -> LDS fill of one K-tile, in NP parts -----------
+    // Part p covers X-tile passes [p*AP, (p+1)*AP) and weight chunks [p*BC, (p+1)*BC) (a chunk is 8
+    // codes, 16 bytes of bf16).  The packed weight words of a whole K-tile are fetched together.
+    constexpr int NP = kTileK / 16;                        // one part per MFMA k-step
+    constexpr int AP = A_PASSES / NP;
+    constexpr int BC = QUANT ? (CPT / 8) / NP : B_DENSE_PASSES / NP;
+    static_assert(AP >= 1 && BC >= 1, "tile too small to split into parts");
     u32x4 xa[A_PASSES];
-    uint32_t wreg[QUANT ? WPT : 1];
-    uint32_t szreg[QUANT ? NGT : 1];
+    uint32_t wreg[QUANT ? WPT : 1], wnext[QUANT ? WPT : 1];
+    uint32_t szreg[QUANT ? NGT : 1], sznext[QUANT ? NGT : 1];
     u32x4 bd[QUANT ? 1 : B_DENSE_PASSES];
 
     const uint32_t a_row = tid >> 3, a_chunk = tid & 7;       // X tile: 8 threads per row
@@ -90,64 +111,78 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(GemmArgs a) {
     uint32_t b_grow = n0 + b_row;
     b_grow = b_grow < a.n ? b_grow : a.n - 1;
 
-    auto fetch = [&](uint32_t kt) __attribute__((always_inline)) {
-        const uint32_t k0 = kt * kTileK;
-        static_for<A_PASSES>([&](auto P) __attribute__((always_inline)) {
-            constexpr int p = decltype(P)::value;
-            uint32_t gr = m0 + p * 32 + a_row;
+    auto fetch_x = [&](auto P, uint32_t kt) __attribute__((always_inline)) {
+        constexpr int part = decltype(P)::value;
+        static_for<AP>([&](auto Q) __attribute__((always_inline)) {
+            constexpr int p = part * AP + decltype(Q)::value;
+            uint32_t gr = m0 + p * RPP + a_row;
             gr = gr < a.m ? gr : a.m - 1;
-            xa[p] = *(const u32x4*)(a.x + (size_t)gr * a.xs + k0 + a_chunk * 8);
+            xa[p] = *(const u32x4*)(a.x + (size_t)gr * a.xs + kt * kTileK + a_chunk * 8);
         });
+    };
+    auto fetch_dense = [&](auto P, uint32_t kt) __attribute__((always_inline)) {
+        constexpr int part = decltype(P)::value;
+        if constexpr (!QUANT) {
+            static_for<BC>([&](auto Q) __attribute__((always_inline)) {
+                constexpr int p = part * BC + decltype(Q)::value;
+                uint32_t gr = n0 + p * RPP + a_row;
+                gr = gr < a.n ? gr : a.n - 1;
+                bd[p] = *(const u32x4*)(a.bdense + (size_t)gr * a.k + kt * kTileK + a_chunk * 8);
+            });
+        }
+    };
+    // packed words + (scale, bias) words of K-tile kt into (w, sz)
+    auto fetch_codes = [&](uint32_t kt, uint32_t (&w)[QUANT ? WPT : 1], uint32_t (&sz)[QUANT ? NGT : 1])
+                           __attribute__((always_inline)) {
         if constexpr (QUANT) {
+            const uint32_t k0 = kt * kTileK;
             const uint32_t* src = a.codes + (size_t)b_grow * a.code_stride + (size_t)kt * (kTileK * BITS / 32) +
                                   b_part * WPT;
             if constexpr (WPT % 4 == 0) {
                 static_for<WPT / 4>([&](auto I) __attribute__((always_inline)) {
                     constexpr int i = decltype(I)::value;
                     const u32x4 v = ((const u32x4*)src)[i];
-                    wreg[4 * i + 0] = v.x; wreg[4 * i + 1] = v.y; wreg[4 * i + 2] = v.z; wreg[4 * i + 3] = v.w;
+                    w[4 * i + 0] = v.x; w[4 * i + 1] = v.y; w[4 * i + 2] = v.z; w[4 * i + 3] = v.w;
                 });
             } else if constexpr (WPT % 2 == 0) {
                 static_for<WPT / 2>([&](auto I) __attribute__((always_inline)) {
                     constexpr int i = decltype(I)::value;
                     const u32x2 v = ((const u32x2*)src)[i];
-                    wreg[2 * i + 0] = v.x; wreg[2 * i + 1] = v.y;
+                    w[2 * i + 0] = v.x; w[2 * i + 1] = v.y;
                 });
             } else {
                 static_for<WPT>([&](auto I) __attribute__((always_inline)) {
                     constexpr int i = decltype(I)::value;
-                    wreg[i] = src[i];
+                    w[i] = src[i];
                 });
             }
             static_for<NGT>([&](auto G) __attribute__((always_inline)) {
                 constexpr int g = decltype(G)::value;
-                szreg[g] = a.sz[(size_t)b_grow * a.sz_stride + (k0 + b_part * CPT + g * GROUP) / GROUP];
-            });
-        } else {
-            static_for<B_DENSE_PASSES>([&](auto P) __attribute__((always_inline)) {
-                constexpr int p = decltype(P)::value;
-                uint32_t gr = n0 + p * 32 + a_row;
-                gr = gr < a.n ? gr : a.n - 1;
-                bd[p] = *(const u32x4*)(a.bdense + (size_t)gr * a.k + k0 + a_chunk * 8);
+                sz[g] = a.sz[(size_t)b_grow * a.sz_stride + (k0 + b_part * CPT + g * GROUP) / GROUP];
             });
         }
     };
+    auto fetch = [&](uint32_t kt) __attribute__((always_inline)) {
+        static_for<NP>([&](auto P) __attribute__((always_inline)) { fetch_x(P, kt); fetch_dense(P, kt); });
+        fetch_codes(kt, wreg, szreg);
+    };
 
     // ---- register -> LDS (with dequantisation of the weight words) ----------------------------
-    auto stash = [&](uint32_t stage) __attribute__((always_inline)) {
+    auto stash_part = [&](auto P, uint32_t stage) __attribute__((always_inline)) {
+        constexpr int part = decltype(P)::value;
         char* As = lds + stage * STAGE;
         char* Bs = As + A_BYTES;
-        static_for<A_PASSES>([&](auto P) __attribute__((always_inline)) {
-            constexpr int p = decltype(P)::value;
-            *(u32x4*)(As + lds_off(p * 32 + a_row, a_chunk)) = xa[p];
+        static_for<AP>([&](auto Q) __attribute__((always_inline)) {
+            constexpr int p = part * AP + decltype(Q)::value;
+            *(u32x4*)(As + lds_off(p * RPP + a_row, a_chunk)) = xa[p];
         });
         if constexpr (QUANT) {
-            static_for<CPT / 8>([&](auto C) __attribute__((always_inline)) {
-                constexpr int ci = decltype(C)::value;                 // chunk of 8 codes
+            static_for<BC>([&](auto C) __attribute__((always_inline)) {
+                constexpr int ci = part * BC + decltype(C)::value;     // chunk of 8 codes
                 constexpr int g = NGT > 1 ? (ci * 8) / GROUP : 0;
                 float s, z;
                 const uint32_t szw = szreg[g];
-                if (a.sb_dtype == MI355Q_BF16) {
+                if constexpr (SB_BF16) {     // compile-time: a branch here would split the pipelined loop body
                     s = __uint_as_float(szw << 16); z = __uint_as_float(szw & 0xFFFF0000u);
                 } else {
                     s = f16_to_f32((uint16_t)(szw & 0xFFFFu)); z = f16_to_f32((uint16_t)(szw >> 16));
@@ -184,11 +219,14 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(GemmArgs a) {
                 *(u32x4*)(Bs + lds_off(b_row, b_part * (CPT / 8) + ci)) = o;
             });
         } else {
-            static_for<B_DENSE_PASSES>([&](auto P) __attribute__((always_inline)) {
-                constexpr int p = decltype(P)::value;
-                *(u32x4*)(Bs + lds_off(p * 32 + a_row, a_chunk)) = bd[p];
+            static_for<BC>([&](auto Q) __attribute__((always_inline)) {
+                constexpr int p = part * BC + decltype(Q)::value;
+                *(u32x4*)(Bs + lds_off(p * RPP + a_row, a_chunk)) = bd[p];
             });
         }
+    };
+    auto stash = [&](uint32_t stage) __attribute__((always_inline)) {
+        static_for<NP>([&](auto P) __attribute__((always_inline)) { stash_part(P, stage); });
     };
 
     floatx16_t acc[TM][TN];
@@ -200,33 +238,96 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(GemmArgs a) {
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
     const uint32_t KT = a.k / kTileK;
-    fetch(0);
-    stash(0);
-    __syncthreads();
-
     const uint32_t frag_row = lane & 31, frag_half = lane >> 5;
-    for (uint32_t kt = 0; kt < KT; kt++) {
-        const uint32_t stage = kt & 1;
-        if (kt + 1 < KT) fetch(kt + 1);
+    bf16x8_t af[2][TM], bf[2][TN];
+    auto load_frags = [&](auto KK, uint32_t stage) __attribute__((always_inline)) {
+        constexpr int kk = decltype(KK)::value;
         const char* As = lds + stage * STAGE;
         const char* Bs = As + A_BYTES;
 #pragma unroll
-        for (int kk = 0; kk < kTileK / 16; kk++) {
-            bf16x8_t af[TM], bf[TN];
+        for (int i = 0; i < TM; i++)
+            af[kk & 1][i] = *(const bf16x8_t*)(As + lds_off(wm * (BM / 2) + i * 32 + frag_row, kk * 2 + frag_half));
 #pragma unroll
-            for (int i = 0; i < TM; i++)
-                af[i] = *(const bf16x8_t*)(As + lds_off(wm * (BM / 2) + i * 32 + frag_row, kk * 2 + frag_half));
+        for (int j = 0; j < TN; j++)
+            bf[kk & 1][j] = *(const bf16x8_t*)(Bs + lds_off(wn * (BN / WN) + j * 32 + frag_row, kk * 2 + frag_half));
+    };
+    auto mfmas = [&](auto KK) __attribute__((always_inline)) {
+        constexpr int kk = decltype(KK)::value;
+#pragma unroll
+        for (int i = 0; i < TM; i++)
 #pragma unroll
             for (int j = 0; j < TN; j++)
-                bf[j] = *(const bf16x8_t*)(Bs + lds_off(wn * (BN / 2) + j * 32 + frag_row, kk * 2 + frag_half));
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
-        }
-        if (kt + 1 < KT) stash(stage ^ 1);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][i], bf[kk & 1][j], acc[i][j], 0, 0, 0);
+    };
+    // Matrix-core phase of one K-tile: the operand fragments of k-step kk+1 are read from LDS while
+    // the MFMAs of k-step kk run (two register sets), so only the first read of a K-tile is exposed.
+    auto multiply = [&](uint32_t stage) __attribute__((always_inline)) {
+        load_frags(std::integral_constant<int, 0>{}, stage);
+        static_for<NP>([&](auto KK) __attribute__((always_inline)) {
+            constexpr int kk = decltype(KK)::value;
+            if constexpr (kk + 1 < NP) load_frags(std::integral_constant<int, kk + 1>{}, stage);
+            __builtin_amdgcn_sched_barrier(0);   // keep the reads of kk+1 ahead of the MFMAs of kk
+            mfmas(KK);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+
+    fetch(0);
+    if constexpr (STAGES == 2) {
+        // Software pipeline over K-tiles, all inside one wavefront's instruction stream: while the
+        // MFMAs of K-tile kt run, K-tile kt+1 moves from registers to the other LDS stage (part by
+        // part, dequantising) and K-tile kt+2 is fetched into the registers just freed.  Tile
+        // indices past the end are clamped: the extra fetches and the extra LDS fill are never read.
+        stash(0);
         __syncthreads();
+        fetch(KT > 1 ? 1u : 0u);
+        for (uint32_t kt = 0; kt < KT; kt++) {
+            const uint32_t stage = kt & 1;
+            const uint32_t k2 = kt + 2 < KT ? kt + 2 : KT - 1;
+            load_frags(std::integral_constant<int, 0>{}, stage);
+            static_for<NP>([&](auto KK) __attribute__((always_inline)) {
+                constexpr int kk = decltype(KK)::value;
+                if constexpr (kk + 1 < NP) load_frags(std::integral_constant<int, kk + 1>{}, stage);
+                stash_part(KK, stage ^ 1);
+                fetch_x(KK, k2);
+                fetch_dense(KK, k2);
+                if constexpr (kk == 0) fetch_codes(k2, wnext, sznext);
+                mfmas(KK);
+                // Issue order inside this k-step: the LDS reads for the next k-step first, then the
+                // MFMAs with the fill of the other stage (VALU, LDS writes) and the global loads
+                // spread between them.
+                __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
+#pragma unroll
+                for (int q = 0; q < TM * TN; q++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);     // one MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);     // a few VALU
+                    if (q % 2 == 0) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);   // an LDS write
+                    if (q % 4 == 1) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // a global load
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            });
+            if constexpr (QUANT) {
+#pragma unroll
+                for (int i = 0; i < WPT; i++) wreg[i] = wnext[i];
+#pragma unroll
+                for (int g = 0; g < NGT; g++) szreg[g] = sznext[g];
+            }
+            __syncthreads();
+        }
+    } else {
+        for (uint32_t kt = 0; kt < KT; kt++) {
+#ifdef MI355Q_GEMV_EXPERIMENT
+            if (!(a.dbg & 2) || kt == 0)
+#endif
+            stash(0);
+            __syncthreads();
+#ifdef MI355Q_GEMV_EXPERIMENT
+            if (!(a.dbg & 1))
+#endif
+            if (kt + 1 < KT) fetch(kt + 1);      // in flight during the matrix-core phase
+            multiply(0);
+            __syncthreads();                     // every wavefront is done reading before the next fill
+        }
     }
 
     // ---- epilogue: one rounding, to the output type --------------------------------------------
@@ -234,7 +335,7 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(GemmArgs a) {
     for (int i = 0; i < TM; i++)
 #pragma unroll
         for (int j = 0; j < TN; j++) {
-            const uint32_t col = n0 + wn * (BN / 2) + j * 32 + frag_row;
+            const uint32_t col = n0 + wn * (BN / WN) + j * 32 + frag_row;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const uint32_t row = m0 + wm * (BM / 2) + i * 32 + 8 * (r / 4) + 4 * frag_half + (r % 4);
@@ -249,46 +350,65 @@ __global__ __launch_bounds__(256) void qgemm_mfma_kernel(GemmArgs a) {
         }
 }
 
-// Tile choice: the largest tile that still gives every CU a workgroup.
+// Tile choice.  Problems with at least one 256 x 256 tile per CU take those (eight wavefronts,
+// double-buffered LDS, in-wave software pipeline); smaller ones take 128 x 128 tiles (same
+// pipeline, four wavefronts, two or three workgroups per CU).
 GemmLaunchShape gemm_mfma_shape(const mi355q_context* ctx, uint32_t m, uint32_t n) {
     const uint32_t cus = (uint32_t)ctx->props.multiProcessorCount;
     auto tiles = [&](uint32_t bm, uint32_t bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
     GemmLaunchShape g{};
-    if (m > 128 && tiles(256, 256) >= cus) { g.bm = 256; g.bn = 256; }
-    else if (m > 128 && tiles(256, 128) >= cus / 2) { g.bm = 256; g.bn = 128; }
-    else { g.bm = 128; g.bn = 128; }
+    int pick = env_int_cached("MI355Q_GEMM_TILE", 0);
+    if (pick == 0) pick = (m > 128 && 10 * tiles(256, 256) >= 9 * cus) ? 5 : 3;
+    if (pick == 1) { g.bm = 256; g.bn = 256; g.stages = 2; }
+    else if (pick == 5) { g.bm = 256; g.bn = 256; g.stages = 2; g.block = 512; }
+    else if (pick == 2) { g.bm = 256; g.bn = 128; g.stages = 1; }
+    else if (pick == 4) { g.bm = 128; g.bn = 128; g.stages = 1; }
+    else { g.bm = 128; g.bn = 128; g.stages = 2; }
     g.grid = (tiles(g.bm, g.bn) + 7) / 8 * 8;
-    g.block = 256;
-    g.lds_bytes = 2 * (g.bm + g.bn) * (uint32_t)kRowBytes;
+    if (!g.block) g.block = 256;
+    g.lds_bytes = g.stages * (g.bm + g.bn) * (uint32_t)kRowBytes;
     return g;
 }
 
 namespace {
 
-template <int BITS, int GROUP, int BM, int BN, bool QUANT>
-mi355q_status launch_tile(hipStream_t s, GemmArgs a) {
+template <int BITS, int GROUP, int BM, int BN, bool QUANT, int STAGES, bool SB_BF16, int WAVES>
+mi355q_status launch_tile_sb(hipStream_t s, GemmArgs a) {
     a.tiles_m = (a.m + BM - 1) / BM;
     a.tiles_n = (a.n + BN - 1) / BN;
     const uint32_t total = a.tiles_m * a.tiles_n;
     const uint32_t grid = (total + 7) / 8 * 8;
-    constexpr size_t lds = 2 * (size_t)(BM + BN) * kRowBytes;
-    auto kern = qgemm_mfma_kernel<BITS, GROUP, BM, BN, QUANT>;
+    constexpr size_t lds = (size_t)STAGES * (BM + BN) * kRowBytes;
+    auto kern = qgemm_mfma_kernel<BITS, GROUP, BM, BN, QUANT, STAGES, SB_BF16, WAVES>;
     static bool lds_limit_raised = false;      // per instantiation; the library drives one device
     if (!lds_limit_raised) {
         MI355Q_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         lds_limit_raised = true;
     }
-    kern<<<dim3(grid), dim3(256), lds, s>>>(a);
+    kern<<<dim3(grid), dim3(WAVES * 64), lds, s>>>(a);
     MI355Q_HIP(hipGetLastError());
     return MI355Q_OK;
+}
+
+template <int BITS, int GROUP, int BM, int BN, bool QUANT, int STAGES, int WAVES = 4>
+mi355q_status launch_tile(hipStream_t s, const GemmArgs& a) {
+    if constexpr (QUANT) {
+        if (a.sb_dtype == MI355Q_BF16) return launch_tile_sb<BITS, GROUP, BM, BN, QUANT, STAGES, true, WAVES>(s, a);
+    }
+    return launch_tile_sb<BITS, GROUP, BM, BN, QUANT, STAGES, false, WAVES>(s, a);
 }
 
 template <int BITS, int GROUP, bool QUANT>
 mi355q_status launch_shape(hipStream_t s, const mi355q_context* ctx, const GemmArgs& a) {
     const GemmLaunchShape g = gemm_mfma_shape(ctx, a.m, a.n);
-    if (g.bm == 256 && g.bn == 256) return launch_tile<BITS, GROUP, 256, 256, QUANT>(s, a);
-    if (g.bm == 256 && g.bn == 128) return launch_tile<BITS, GROUP, 256, 128, QUANT>(s, a);
-    return launch_tile<BITS, GROUP, 128, 128, QUANT>(s, a);
+    if (g.bm == 256 && g.bn == 256 && g.block == 512) return launch_tile<BITS, GROUP, 256, 256, QUANT, 2, 8>(s, a);
+#ifdef MI355Q_GEMV_EXPERIMENT
+    // tuning builds: the other tile shapes, selected with MI355Q_GEMM_TILE
+    if (g.bm == 256 && g.bn == 256) return launch_tile<BITS, GROUP, 256, 256, QUANT, 2>(s, a);
+    if (g.bm == 256 && g.bn == 128) return launch_tile<BITS, GROUP, 256, 128, QUANT, 1>(s, a);
+    if (g.stages == 1) return launch_tile<BITS, GROUP, 128, 128, QUANT, 1>(s, a);
+#endif
+    return launch_tile<BITS, GROUP, 128, 128, QUANT, 2>(s, a);
 }
 
 }  // namespace
@@ -316,6 +436,7 @@ mi355q_status launch_qgemm_mfma(hipStream_t s, const mi355q_context* ctx, const 
     a.m = m; a.n = w.n; a.k = w.k; a.xs = x_stride; a.ys = y_stride;
     a.code_stride = w.code_stride; a.sz_stride = w.sz_stride;
     a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = w.sb_dtype;
+    a.dbg = (uint32_t)env_int_cached("MI355Q_GEMM_DBG", 0);
     switch (w.bits * 1000 + w.group) {
     case 4064: return launch_shape<4, 64, true>(s, ctx, a);
     case 4128: return launch_shape<4, 128, true>(s, ctx, a);
@@ -341,6 +462,7 @@ mi355q_status launch_gemm_bf16_mfma(hipStream_t s, const mi355q_context* ctx, co
     a.x = (const uint16_t*)a_ptr; a.y = c;
     a.m = m; a.n = n; a.k = k; a.xs = a_stride; a.ys = c_stride;
     a.y_dtype = (uint32_t)c_dtype;
+    a.dbg = (uint32_t)env_int_cached("MI355Q_GEMM_DBG", 0);
     return launch_shape<4, 64, false>(s, ctx, a);
 }
 

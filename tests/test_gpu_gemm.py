@@ -207,7 +207,7 @@ def test_qgemm_selects_matrix_cores_above_eight_rows(pkg, ctx):
     w = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, pkg.LAYOUT_PLANES)
     step = w.plan_prefill_steps(m)[0]
     assert step.kernel_family == "mfmaGEMM" and not step.used_fallback
-    assert step.block[0] == 256 and step.grid[0] >= 1
+    assert step.block[0] in (256, 512) and step.grid[0] >= 1
     ws = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, pkg.LAYOUT_STAF_BLOCKS)
     step = ws.plan_prefill_steps(m)[0]
     assert step.kernel_family != "mfmaGEMM" and step.used_fallback
