@@ -38,15 +38,14 @@ mi355q_status launch_group(hipStream_t s, const GemvArgs& a, const GemvCfg& c) {
     MI355Q_TRY(1, 1, false, 16, 2, 1) MI355Q_TRY(1, 1, false, 16, 4, 1) MI355Q_TRY(1, 1, false, 16, 8, 1)
     MI355Q_TRY(1, 1, false, 16, 2, 2) MI355Q_TRY(1, 1, false, 16, 4, 2) MI355Q_TRY(1, 1, false, 16, 8, 2)
 #else
-    // M == 1 (decode): register-resident activations for rows of one or two K-steps (4 wavefronts
-    // per workgroup), LDS-resident otherwise (8 wavefronts share one staged copy)
+    // M == 1 (decode): register-resident activations for rows of one K-step, LDS-resident otherwise
     MI355Q_TRY(1, 1, false, 4, 2, 1) MI355Q_TRY(1, 1, false, 4, 4, 1)
-    MI355Q_TRY(1, 1, false, 4, 2, 2) MI355Q_TRY(1, 1, false, 4, 4, 2)
+    MI355Q_TRY(1, 1, false, 4, 2, 0) MI355Q_TRY(1, 1, false, 4, 4, 0)
     MI355Q_TRY(1, 1, false, 8, 2, 0) MI355Q_TRY(1, 1, false, 8, 4, 0)
 #endif
     // the same with the fused arg-max tail (LM head)
     MI355Q_TRY(1, 1, true, 4, 2, 1) MI355Q_TRY(1, 1, true, 4, 4, 1)
-    MI355Q_TRY(1, 1, true, 4, 2, 2) MI355Q_TRY(1, 1, true, 4, 4, 2)
+    MI355Q_TRY(1, 1, true, 4, 2, 0) MI355Q_TRY(1, 1, true, 4, 4, 0)
     MI355Q_TRY(1, 1, true, 8, 2, 0) MI355Q_TRY(1, 1, true, 8, 4, 0)
     // small batches (M = 2, 3-4, 5-8)
     MI355Q_TRY(2, 2, false, 4, 4, 0) MI355Q_TRY(2, 4, false, 4, 2, 0) MI355Q_TRY(1, 8, false, 4, 2, 0)

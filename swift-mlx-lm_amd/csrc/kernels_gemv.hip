@@ -57,10 +57,15 @@ GemvCfg choose(const mi355q_context* ctx, const WView& w, uint32_t m, bool argma
     const Geo g = geo_for(w.bits);
     const size_t kc = 64 * (size_t)g.cpl;
     c.nc = (uint32_t)((w.k + kc - 1) / kc);
+    const uint64_t weight_bytes = (uint64_t)w.n * (w.k / w.group) * (4 + w.group * w.bits / 8);
+    const bool big = weight_bytes >= (24ull << 20);
     if (c.mt == 1) {
-        c.xreg = c.nc <= 2 ? (int)c.nc : 0;     // short rows: activation slice lives in registers
+        // Measured on MI355X (q4 g64): rows of one K-step keep their activation slice in registers;
+        // longer rows read it from LDS.  Large matrices of short rows run best with 4 wavefronts
+        // per workgroup, everything else with 8.
+        c.xreg = c.nc == 1 ? 1 : 0;
         c.r = 1;
-        c.waves = c.xreg ? 4 : 8;
+        c.waves = (c.nc == 1 || (c.nc == 2 && big)) ? 4 : 8;
     } else {
         c.xreg = 0;
         c.r = c.mt == 8 ? 1 : 2;
@@ -84,7 +89,7 @@ GemvCfg choose(const mi355q_context* ctx, const WView& w, uint32_t m, bool argma
     c.rows_per_wave = rpw;
     // ring depth: four pipeline steps in flight, two when a wavefront only has two or three
     const uint32_t nsteps = rpw / (uint32_t)c.r * c.nc;
-    if (c.mt == 1) c.depth = nsteps >= 4 ? 4 : 2;
+    if (c.mt == 1) c.depth = (nsteps >= 4 && (big || c.nc > 2)) ? 4 : 2;
     else c.depth = c.mt == 2 ? 4 : 2;
     if (ed) c.depth = ed;
     const uint32_t rows_per_wg = rpw * (uint32_t)c.waves;
