@@ -61,7 +61,14 @@ typedef enum { MI355Q_F16 = 0, MI355Q_BF16 = 1, MI355Q_F32 = 2 } mi355q_dtype;
 /* STAFWeightLayout (MC/STAF/STAFWeightAccessRequest.swift:3-7): the canonical row-major STAF
  * interleaved blocks, or this library's specialized layout (split planes: uint32 code words
  * [N, K*bits/32] + scales [N, K/g] + biases [N, K/g], i.e. the MLX source planes). */
-typedef enum { MI355Q_LAYOUT_STAF_BLOCKS = 0, MI355Q_LAYOUT_PLANES = 1 } mi355q_layout;
+typedef enum {
+    MI355Q_LAYOUT_STAF_BLOCKS = 0,
+    MI355Q_LAYOUT_PLANES = 1,
+    /* Matrix-core decode layout (4-bit, group 64, K % 128 == 0): records of 16 rows x 128 codes in
+     * the order a wavefront loads them, each followed by its (scale, bias) words.  Serves
+     * 1 <= M <= 16 at the cost of M = 1; prefill on this layout runs in slices of 16 rows. */
+    MI355Q_LAYOUT_TILE16 = 2
+} mi355q_layout;
 
 /* Launch flags */
 enum {

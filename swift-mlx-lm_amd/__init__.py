@@ -19,7 +19,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libmi355_qlinear.so")
 # BufferPrecision
 F16, BF16, F32 = 0, 1, 2
 # STAFWeightLayout
-LAYOUT_STAF_BLOCKS, LAYOUT_PLANES = 0, 1
+LAYOUT_STAF_BLOCKS, LAYOUT_PLANES, LAYOUT_TILE16 = 0, 1, 2
 # launch flags
 FLAG_NONE, FLAG_FORCE_GENERIC, FLAG_FORCE_SMALL_M, FLAG_FORCE_MFMA = 0, 1, 2, 4
 

@@ -36,20 +36,33 @@ mi355q_status check_io(const mi355q_weight* w, const void* x, int x_dtype, const
     return MI355Q_OK;
 }
 
-// Small-M path: the split-plane kernel when the shape allows it, else the per-code kernel.
+// Small-M path: the split-plane kernel or the matrix-core tile kernel when the layout and shape
+// allow it, else the per-code kernel.
 mi355q_status run_small_m(mi355q_context* ctx, hipStream_t s, const mi355q_weight* w, const void* x, int x_dtype,
                           void* y, int y_dtype, uint32_t m, uint32_t xs, uint32_t ys, uint32_t flags) {
     const WView v = w->view();
     const size_t xsz = x_dtype == MI355Q_F32 ? 4 : 2, ysz = y_dtype == MI355Q_F32 ? 4 : 2;
-    for (uint32_t m0 = 0; m0 < m; m0 += 8) {
-        const uint32_t mm = m - m0 < 8 ? m - m0 : 8;
+    const bool generic = flags & MI355Q_FLAG_FORCE_GENERIC;
+    // rows per launch: 16 on the tile layout (fewer when K is so long that 16 staged rows overflow LDS), else 8
+    uint32_t step = 8;
+    if (!generic && v.layout == MI355Q_LAYOUT_TILE16) {
+        step = 16;
+        while (step > 1 && !gemv_tile16_eligible(v, x_dtype, step, xs)) step >>= 1;
+    }
+    for (uint32_t m0 = 0; m0 < m; m0 += step) {
+        const uint32_t mm = m - m0 < step ? m - m0 : step;
         const void* xp = (const char*)x + (size_t)m0 * xs * xsz;
         void* yp = (char*)y + (size_t)m0 * ys * ysz;
         mi355q_status st;
-        if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && gemv_fast_eligible(v, x_dtype, mm, xs) && (uintptr_t)xp % 16 == 0)
+        if (!generic && gemv_tile16_eligible(v, x_dtype, mm, xs) && (uintptr_t)xp % 16 == 0) {
+            void* yv[1] = {yp};
+            const uint32_t strides[1] = {ys};
+            st = launch_gemv_tile16_multi(s, ctx, 1, &v, xp, yv, strides, y_dtype, mm, xs, nullptr, nullptr, nullptr);
+        } else if (!generic && gemv_fast_eligible(v, x_dtype, mm, xs) && (uintptr_t)xp % 16 == 0) {
             st = launch_gemv_fast(s, ctx, v, xp, yp, y_dtype, mm, xs, ys, nullptr, nullptr, nullptr);
-        else
+        } else {
             st = launch_gemv_generic(s, v, xp, x_dtype, yp, y_dtype, mm, xs, ys);
+        }
         if (st != MI355Q_OK) return st;
     }
     return MI355Q_OK;
@@ -110,6 +123,7 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
             return fail(MI355Q_ERR_SHAPE, "batched projections must share K, scheme and layout");
     }
     bool fused = m <= 8 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
+    bool tiled = m <= 16 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
     WView views[3];
     uint32_t strides[3];
     for (uint32_t i = 0; i < count; i++) {
@@ -119,9 +133,13 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
         strides[i] = y_stride;
         views[i] = weights[i]->view();
         fused = fused && gemv_fast_eligible(views[i], x_dtype, m, xs) && views[i].sb_dtype == views[0].sb_dtype;
+        tiled = tiled && gemv_tile16_eligible(views[i], x_dtype, m, xs) && views[i].sb_dtype == views[0].sb_dtype;
     }
     if (fused && (uintptr_t)x % 16 == 0)
         return launch_gemv_fast_multi(s, ctx, count, views, x, ys, strides, y_dtype, m, xs, nullptr, nullptr, nullptr);
+    if (tiled && (uintptr_t)x % 16 == 0)
+        return launch_gemv_tile16_multi(s, ctx, count, views, x, ys, strides, y_dtype, m, xs, nullptr, nullptr,
+                                        nullptr);
     for (uint32_t i = 0; i < count; i++) {
         mi355q_status st = dispatch_linear(ctx, s, weights[i], x, x_dtype, ys[i], y_dtype, m, xs, 0, flags, false);
         if (st != MI355Q_OK) return st;
@@ -138,6 +156,12 @@ mi355q_status dispatch_output_head(mi355q_context* ctx, hipStream_t s, const mi3
     if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && gemv_fast_eligible(v, x_dtype, 1, xs) && (uintptr_t)x % 16 == 0)
         return launch_gemv_fast(s, ctx, v, x, nullptr, MI355Q_F32, 1, xs, (uint32_t)w->n, logits, token,
                                 ctx->argmax_scratch);
+    if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && gemv_tile16_eligible(v, x_dtype, 1, xs) && (uintptr_t)x % 16 == 0) {
+        void* none[1] = {nullptr};
+        const uint32_t strides[1] = {(uint32_t)w->n};
+        return launch_gemv_tile16_multi(s, ctx, 1, &v, x, none, strides, MI355Q_F32, 1, xs, logits, token,
+                                        ctx->argmax_scratch);
+    }
     // two dispatches, as the reference runs the head: projection to fp32 logits, then argmax
     if (!logits)
         return fail(MI355Q_ERR_INVALID_ARGUMENT,

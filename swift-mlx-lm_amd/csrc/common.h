@@ -39,6 +39,7 @@ struct WView {
     const uint16_t* scales;
     const uint16_t* biases;
     const uint32_t* sz;       // planes: scale | bias << 16 per group (packed once at prepare time)
+    const uint32_t* tiles;    // TILE16 records (layout 2)
     uint32_t n, k;
     uint32_t group, bits;
     uint32_t bytes_per_block, blocks_per_row, words_per_row;
@@ -67,6 +68,8 @@ struct mi355q_weight {
     void* scales;
     void* biases;
     void* sz;                 // packed (scale, bias) words for the planes layout
+    void* tiles;              // owned: TILE16 records (layout 2)
+    size_t tiles_bytes;
     // Owned plane weights keep each row's code words and its sz words side by side in ONE buffer
     // ([codes of row r | sz of row r | pad to 16 bytes]): `codes` points at it, `sz` points
     // words_per_row further, and both advance by the same stride, so a row is one contiguous
@@ -81,6 +84,7 @@ struct mi355q_weight {
         v.scales = (const uint16_t*)scales;
         v.biases = (const uint16_t*)biases;
         v.sz = (const uint32_t*)sz;
+        v.tiles = (const uint32_t*)tiles;
         v.n = (uint32_t)n;
         v.k = (uint32_t)k;
         v.group = fmt.group_size;
@@ -126,6 +130,19 @@ mi355q_status launch_gemv_fast_multi(hipStream_t s, const mi355q_context* ctx, u
                                      const void* x, void* const* y, const uint32_t* y_strides, int y_dtype,
                                      uint32_t m, uint32_t x_stride, float* logits_f32, int32_t* token_out,
                                      unsigned long long* argmax_scratch);
+
+// Matrix-core decode kernel over the TILE16 layout (gemv_tile16.hip)
+constexpr int kTile16MaxSegments = 3;
+struct Tile16LaunchShape {
+    uint32_t ksplit, tiles_per_wg, waves, blocks_per_wave, grid, block, lds_bytes;
+};
+bool gemv_tile16_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
+Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_total_tiles, uint32_t k, uint32_t m);
+mi355q_status launch_gemv_tile16_multi(hipStream_t s, const mi355q_context* ctx, uint32_t count, const WView* w,
+                                       const void* x, void* const* y, const uint32_t* y_strides, int y_dtype,
+                                       uint32_t m, uint32_t x_stride, float* logits_f32, int32_t* token_out,
+                                       unsigned long long* argmax_scratch);
+mi355q_status launch_tile16_pack(hipStream_t s, const WView& planes, uint32_t* tiles);
 
 // Validated dispatch shared by the direct entry points and by plan replay (api.hip)
 mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t count, const mi355q_weight* const* weights,

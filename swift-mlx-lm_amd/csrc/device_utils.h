@@ -81,6 +81,14 @@ __device__ __forceinline__ uint32_t load_code(const WView& w, uint32_t row, uint
         if (sh + w.bits > 32) v |= rowp[word + 1] << (32 - sh);
         return v & mask;
     }
+    if (w.layout == MI355Q_LAYOUT_TILE16) {
+        // record (row / 16, c / 128): lane kq*16 + row%16 holds word j = codes (j/2)*64 + kq*16 + (j%2)*8 .. +8
+        // with nibbles stored as (c0,c2,c4,c6,c1,c3,c5,c7)
+        const uint32_t o = c & 127u, g = o >> 6, in_g = o & 63u, kq = in_g >> 4, j = g * 2 + ((in_g >> 3) & 1u);
+        const uint32_t e = in_g & 7u, nib = (e >> 1) + 4u * (e & 1u);
+        const uint32_t* rec = w.tiles + ((size_t)(row >> 4) * (w.k >> 7) + (c >> 7)) * 288u;
+        return (rec[(kq * 16u + (row & 15u)) * 4u + j] >> (4u * nib)) & 0xFu;
+    }
     const uint32_t b = c / w.group, e = c - b * w.group;
     const uint8_t* qs = w.blocks + ((size_t)row * w.blocks_per_row + b) * w.bytes_per_block + 4;
     const uint32_t bit = e * w.bits, byte = bit >> 3, sh = bit & 7;
@@ -95,6 +103,11 @@ __device__ __forceinline__ void load_scale_zero(const WView& w, uint32_t row, ui
         const size_t g = (size_t)row * w.blocks_per_row + b;
         scale = sb_to_f32(w.scales[g], w.sb_dtype);
         zero = sb_to_f32(w.biases[g], w.sb_dtype);
+    } else if (w.layout == MI355Q_LAYOUT_TILE16) {
+        const uint32_t* rec = w.tiles + ((size_t)(row >> 4) * (w.k >> 7) + (b >> 1)) * 288u;
+        const uint32_t szw = rec[256u + (row & 15u) * 2u + (b & 1u)];
+        scale = sb_to_f32((uint16_t)(szw & 0xFFFFu), w.sb_dtype);
+        zero = sb_to_f32((uint16_t)(szw >> 16), w.sb_dtype);
     } else {
         const uint16_t* hdr =
             (const uint16_t*)(w.blocks + ((size_t)row * w.blocks_per_row + b) * w.bytes_per_block);

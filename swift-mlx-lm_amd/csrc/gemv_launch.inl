@@ -47,8 +47,8 @@ mi355q_status launch_group(hipStream_t s, const GemvArgs& a, const GemvCfg& c) {
     MI355Q_TRY(1, 1, true, 4, 2, 1) MI355Q_TRY(1, 1, true, 4, 4, 1)
     MI355Q_TRY(1, 1, true, 4, 2, 0) MI355Q_TRY(1, 1, true, 4, 4, 0)
     MI355Q_TRY(1, 1, true, 8, 2, 0) MI355Q_TRY(1, 1, true, 8, 4, 0)
-    // small batches (M = 2, 3-4, 5-8)
-    MI355Q_TRY(2, 2, false, 4, 4, 0) MI355Q_TRY(2, 4, false, 4, 2, 0) MI355Q_TRY(1, 8, false, 4, 2, 0)
+    // small batches (M = 2, 3-4)
+    MI355Q_TRY(2, 2, false, 4, 4, 0) MI355Q_TRY(2, 4, false, 4, 2, 0)
     return fail(MI355Q_ERR_KERNEL_NOT_FOUND,
                 "no split-plane GEMV variant for q%d g%d R=%d MT=%d argmax=%d waves=%d depth=%d xreg=%d", BITS, GROUP,
                 c.r, c.mt, (int)c.argmax, c.waves, c.depth, c.xreg);

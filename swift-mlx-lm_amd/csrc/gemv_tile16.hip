@@ -1,0 +1,364 @@
+// Decode / small-batch projection on the matrix cores over the TILE16 layout (4-bit codes, groups of
+// 64), 1 <= M <= 16 activation rows per launch.
+//
+// Stands in for gemv_q4_g64 and, at small sequence lengths, gemm_q4_g64
+// (Sources/MetalCompiler/Generator/MetalSourceGenerator+Quantized.swift:496-575 and :22-156):
+//   y[m, n] = sum_g sum_{k in g} (s[n,g] * q[n,k] + z[n,g]) * x[m,k],  fp32 accumulation.
+//
+// TILE16 layout (built once at weight preparation, kernels_generic.hip::tile16_pack_kernel): rows are
+// taken 16 at a time and K 128 codes (two groups) at a time; each (row tile, K-block) is one record
+// of 1152 contiguous bytes:
+//   bytes    0..1023  64 lanes x 16 bytes of codes in the order a wavefront loads them:
+//                     lane = kq*16 + n (n = row in the tile, kq = 0..3); its word j (j = 0..3) holds
+//                     the 8 codes at K-block offset (j/2)*64 + kq*16 + (j%2)*8 .. +8, nibbles stored
+//                     as (c0,c2,c4,c6,c1,c3,c5,c7) so that (w >> 4i) & 0x000F000F is the code pair
+//                     (c2i, c2i+1): the bf16 operand order of the MFMA, with no shuffle;
+//   bytes 1024..1151  16 rows x 2 groups of packed (scale | bias << 16) words, [n][g].
+// A wavefront reads a record with one 128-bit and one 64-bit load per lane and feeds four
+// v_mfma_f32_16x16x32_bf16 per group pair: codes become bf16 (128 + q) with one and-or each, the
+// activations are the A operand straight from LDS (natural order, no permutation), the matrix core
+// does every multiply-add, and a second MFMA against a tile of ones gives sum(x) over the same k.
+// Per group the VALU applies the affine form once per kept output row:
+//   acc += s * D + (z - 128 s) * D1        (D = sum (128+q) x,  D1 = sum x).
+// The accumulator of lane (kq, n) holds output rows m = 4 kq .. 4 kq + 3 of weight row n, so there is
+// no cross-lane reduction at all; the WAVES wavefronts of a workgroup split K and add their partial
+// tiles through LDS at the end.
+#include "device_utils.h"
+
+namespace mi355q {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4_t;
+
+struct T16Args {
+    const uint32_t* tiles[kTile16MaxSegments];   // TILE16 buffers of up to three matrices sharing x
+    void* y[kTile16MaxSegments];
+    uint32_t tile_end[kTile16MaxSegments];       // cumulative row-tile counts; unused entries repeat the last
+    uint32_t seg_rows[kTile16MaxSegments];       // N_i
+    uint32_t y_stride[kTile16MaxSegments];
+    const uint16_t* x;                           // bf16 [M, x_stride]
+    float* logits;                               // optional fp32 [N] copy (M == 1, one matrix)
+    int32_t* token_out;                          // ARGMAX only
+    unsigned long long* scratch;                 // ARGMAX only: [0] packed max, [1] ticket
+    uint32_t k, m, x_stride;
+    uint32_t kblocks;                            // K / 128
+    uint32_t blocks_per_wave;                    // K-blocks per wavefront (K split over the workgroup)
+    uint32_t lds_row_bytes;                      // K*2 + 16: staged activation row pitch
+    uint32_t y_dtype, sb_dtype;
+};
+
+constexpr int kT16RecordWords = 288;             // 1152 bytes
+
+// MR: output rows kept per lane (1, 2 or 4): M <= MR uses lane group 0 only; M > 4 needs MR = 4.
+// A workgroup of KSPLIT * TPW wavefronts covers TPW consecutive row tiles, each split over KSPLIT
+// wavefronts along K; all of them share one staged copy of the activations.
+template <int MR, int KSPLIT, int TPW, int D, bool ARGMAX>
+__global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args a) {
+    constexpr int WAVES = KSPLIT * TPW;
+    extern __shared__ u32x4 smem_t16[];
+    char* lds = (char*)smem_t16;
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint32_t n_in = lane & 15, kq = lane >> 4;
+
+    // ---- matrix and row tile of this wavefront (scalar select chain, once) ----------------------
+    const uint32_t slice = wave % KSPLIT;                   // share of K
+    uint32_t gt = blockIdx.x * TPW + wave / KSPLIT;
+    const bool tile_valid = gt < a.tile_end[kTile16MaxSegments - 1];
+    gt = tile_valid ? gt : a.tile_end[kTile16MaxSegments - 1] - 1;       // idle wavefronts re-read the last tile
+    const bool in1 = gt >= a.tile_end[0], in2 = gt >= a.tile_end[1];
+    const uint32_t* const seg_tiles = in2 ? a.tiles[2] : in1 ? a.tiles[1] : a.tiles[0];
+    void* const seg_y = in2 ? a.y[2] : in1 ? a.y[1] : a.y[0];
+    const uint32_t seg_ys = in2 ? a.y_stride[2] : in1 ? a.y_stride[1] : a.y_stride[0];
+    const uint32_t seg_n = in2 ? a.seg_rows[2] : in1 ? a.seg_rows[1] : a.seg_rows[0];
+    const uint32_t lt = gt - (in2 ? a.tile_end[1] : in1 ? a.tile_end[0] : 0u);
+    const uint32_t n0 = lt * 16;
+
+    // ---- 1. activation loads first (vector loads return in issue order) -------------------------
+    // Raw copy of the M rows into LDS, row pitch K*2 + 16 bytes (the pad spreads the 16 rows of an
+    // A-fragment read over all banks).  Each thread moves up to XC 16-byte chunks per row pass.
+    const uint32_t chunks = a.k / 8;                        // 16-byte chunks per activation row
+    constexpr int XC = 2;
+    u32x4 xe[XC];
+    auto x_row = [&](uint32_t i, uint32_t& m, uint32_t& c) {   // chunk index -> (row, chunk in row)
+        if (a.m == 1) { m = 0; c = i; }                        // uniform: no division on the decode path
+        else { m = i / chunks; c = i - m * chunks; }
+    };
+    auto x_src = [&](uint32_t idx) -> const u32x4* {        // idx over M * chunks, row-major
+        const uint32_t total = a.m * chunks;
+        uint32_t m, c;
+        x_row(idx < total ? idx : 0, m, c);
+        return (const u32x4*)(a.x + (size_t)m * a.x_stride) + c;
+    };
+    auto x_dst = [&](uint32_t idx) -> u32x4* {
+        uint32_t m, c;
+        x_row(idx, m, c);
+        return (u32x4*)(lds + (size_t)m * a.lds_row_bytes) + c;
+    };
+#pragma unroll
+    for (int t = 0; t < XC; t++) xe[t] = *x_src(tid + t * WAVES * 64);
+
+    // ---- 2. the first D K-blocks of this wavefront's share of the row tile ----------------------
+    const uint32_t b_first = slice * a.blocks_per_wave;
+    uint32_t nb = a.kblocks > b_first ? a.kblocks - b_first : 0;          // blocks this wavefront owns
+    nb = nb < a.blocks_per_wave ? nb : a.blocks_per_wave;
+    nb = tile_valid ? nb : 0;
+    const uint32_t b_last = nb ? b_first + nb - 1 : a.kblocks - 1;        // clamp target (always valid)
+    const uint32_t* const tile_base = seg_tiles + (size_t)lt * a.kblocks * kT16RecordWords;
+
+    struct Rec { u32x4 w; u32x2 sz; };
+    Rec ring[D];
+    auto issue = [&](uint32_t b, Rec& r) {
+        b = b < b_last ? b : b_last;                        // unconditional, clamped
+        const uint32_t* rec = tile_base + (size_t)b * kT16RecordWords;   // scalar
+        r.w = *((const u32x4*)rec + lane);
+        r.sz = *((const u32x2*)(rec + 256) + n_in);
+    };
+    static_for<D>([&](auto J) { issue(b_first + decltype(J)::value, ring[decltype(J)::value]); });
+
+    // ---- 3. stage the activations (waits only for the loads of step 1) --------------------------
+    {
+        const uint32_t total = a.m * chunks;
+#pragma unroll
+        for (int t = 0; t < XC; t++) {
+            const uint32_t idx = tid + t * WAVES * 64;
+            if (idx < total) *x_dst(idx) = xe[t];
+        }
+        for (uint32_t idx = tid + XC * WAVES * 64; idx < total; idx += WAVES * 64) *x_dst(idx) = *x_src(idx);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+
+    // ---- 4. K loop --------------------------------------------------------------------------------
+    uint32_t k_mask = 0x000F000Fu, k_magic = 0x43004300u;   // opaque: keeps (w & mask) | magic one v_and_or_b32
+    asm volatile("" : "+s"(k_mask));
+    asm volatile("" : "+v"(k_magic));
+    bf16x8_t ones;
+    {
+        u32x4 o = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
+        ones = __builtin_bit_cast(bf16x8_t, o);
+    }
+    floatx4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+    float acc[MR];
+#pragma unroll
+    for (int r = 0; r < MR; r++) acc[r] = 0.f;
+
+    // A operand: lane (m = lane & 15, kq) reads 8 consecutive bf16 of activation row min(m, M-1)
+    const uint32_t am = n_in < a.m ? n_in : a.m - 1;
+    const char* const a_lane = lds + (size_t)am * a.lds_row_bytes + kq * 32;
+
+    auto unpack = [&](uint32_t w) -> bf16x8_t {
+        u32x4 p;
+        p.x = (w & k_mask) | k_magic;
+        p.y = ((w >> 4) & k_mask) | k_magic;
+        p.z = ((w >> 8) & k_mask) | k_magic;
+        p.w = ((w >> 12) & k_mask) | k_magic;
+        return __builtin_bit_cast(bf16x8_t, p);
+    };
+    auto compute = [&](uint32_t b, const Rec& r) {
+        const char* ab = a_lane + (size_t)b * 256;           // 128 codes = 256 bytes of activations
+        static_for<2>([&](auto G) {
+            constexpr int g = decltype(G)::value;
+            const bf16x8_t a0 = *(const bf16x8_t*)(ab + g * 128);
+            const bf16x8_t a1 = *(const bf16x8_t*)(ab + g * 128 + 16);
+            const bf16x8_t b0 = unpack(g == 0 ? r.w.x : r.w.z);
+            const bf16x8_t b1 = unpack(g == 0 ? r.w.y : r.w.w);
+            floatx4_t d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, b0, zero4, 0, 0, 0);
+            d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b1, d, 0, 0, 0);
+            floatx4_t d1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, ones, zero4, 0, 0, 0);
+            d1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, ones, d1, 0, 0, 0);
+            const uint32_t szw = g == 0 ? r.sz.x : r.sz.y;
+            float s, z;
+            if (a.sb_dtype == MI355Q_BF16) {                // wavefront-uniform
+                asm volatile("" ::: "memory");
+                s = __uint_as_float(szw << 16); z = __uint_as_float(szw & 0xFFFF0000u);
+            } else {
+                asm volatile("" ::: "memory");
+                s = f16_to_f32((uint16_t)(szw & 0xFFFFu)); z = f16_to_f32((uint16_t)(szw >> 16));
+            }
+            const float zc = z - 128.0f * s;
+#pragma unroll
+            for (int q = 0; q < MR; q++) acc[q] += s * d[q] + zc * d1[q];
+        });
+    };
+
+    const uint32_t rounds = (a.blocks_per_wave + D - 1) / D;            // same for every wavefront
+    for (uint32_t it = 0; it < rounds; it++) {
+        static_for<D>([&](auto J) {
+            constexpr int j = decltype(J)::value;
+            const uint32_t idx = it * D + j;                // block index inside this wavefront's share
+            if (idx < nb) compute(b_first + idx, ring[j]);
+            issue(b_first + idx + D, ring[j]);
+        });
+    }
+
+    // ---- 5. add the WAVES partial tiles through LDS, store -------------------------------------
+    // Activations are no longer needed: the reduction buffer overlays them.
+    __syncthreads();
+    float* red = (float*)lds;                               // [WAVES][MR][64]
+#pragma unroll
+    for (int r = 0; r < MR; r++) red[(wave * MR + r) * 64 + lane] = acc[r];
+    __syncthreads();
+    unsigned long long best = 0ull;
+    if (slice == 0 && tile_valid) {                         // the first wavefront of each tile adds and stores
+        const uint32_t row = n0 + n_in;
+#pragma unroll
+        for (int r = 0; r < MR; r++) {
+            float v = 0.f;
+            for (uint32_t w2 = 0; w2 < (uint32_t)KSPLIT; w2++) v += red[((wave + w2) * MR + r) * 64 + lane];
+            const uint32_t m = 4 * kq + r;
+            if (m < a.m && row < seg_n) {
+                if (seg_y) {
+                    const size_t o = (size_t)m * seg_ys + row;
+                    if (a.y_dtype == MI355Q_F32) ((float*)seg_y)[o] = v;
+                    else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)seg_y)[o] = f32_to_bf16_rne(v);
+                    else ((uint16_t*)seg_y)[o] = f32_to_f16_rne(v);
+                }
+                if (a.logits && m == 0) a.logits[row] = v;
+                if constexpr (ARGMAX) {
+                    if (m == 0 && v > -INFINITY) {          // NaN and -inf never contribute
+                        const uint32_t u = __float_as_uint(v + 0.0f);   // -0 -> +0
+                        const uint32_t key = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+                        best = ((unsigned long long)key << 32) | (unsigned long long)(0xFFFFFFFFu - row);
+                    }
+                }
+            }
+        }
+    }
+    if constexpr (ARGMAX) {
+        // wavefront maximum of the packed (ordered value, ~row) key, one atomic per workgroup, then a
+        // ticket: the workgroup that draws the last ticket publishes the token and re-zeroes the cells
+        __shared__ uint32_t s_last;
+        if (slice == 0) {
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+                const uint32_t hi = (uint32_t)__shfl_xor((int)(best >> 32), off, 64);
+                const uint32_t lo = (uint32_t)__shfl_xor((int)(best & 0xFFFFFFFFull), off, 64);
+                const unsigned long long o = ((unsigned long long)hi << 32) | lo;
+                best = o > best ? o : best;
+            }
+            if (lane == 0 && best) atomicMax(&a.scratch[0], best);
+        }
+        __threadfence();
+        __syncthreads();
+        if (tid == 0) {
+            const unsigned long long t = atomicAdd(&a.scratch[1], 1ull);
+            s_last = (t == (unsigned long long)gridDim.x - 1ull) ? 1u : 0u;
+        }
+        __syncthreads();
+        if (s_last && tid == 0) {
+            __threadfence();
+            const unsigned long long pk = atomicExch(&a.scratch[0], 0ull);
+            a.token_out[0] = pk ? (int32_t)(0xFFFFFFFFu - (uint32_t)(pk & 0xFFFFFFFFull)) : 0;
+            atomicExch(&a.scratch[1], 0ull);
+        }
+    }
+}
+
+namespace {
+
+constexpr size_t kT16LdsBudget = 144 * 1024;
+
+template <int MR, int KSPLIT, int TPW, bool ARGMAX>
+mi355q_status launch_t16(hipStream_t s, const T16Args& a, uint32_t grid, size_t lds) {
+    auto kern = gemv_tile16_kernel<MR, KSPLIT, TPW, 4, ARGMAX>;
+    if (lds > 64 * 1024)
+        MI355Q_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    kern<<<dim3(grid), dim3(KSPLIT * TPW * 64), lds, s>>>(a);
+    MI355Q_HIP(hipGetLastError());
+    return MI355Q_OK;
+}
+
+template <int MR, bool ARGMAX>
+mi355q_status launch_t16_shape(hipStream_t s, const T16Args& a, const Tile16LaunchShape& g) {
+    const uint32_t ks = g.ksplit, tpw = g.tiles_per_wg;
+    if (ks == 4 && tpw == 1) return launch_t16<MR, 4, 1, ARGMAX>(s, a, g.grid, g.lds_bytes);
+    if (ks == 4 && tpw == 2) return launch_t16<MR, 4, 2, ARGMAX>(s, a, g.grid, g.lds_bytes);
+    if (ks == 4 && tpw == 4) return launch_t16<MR, 4, 4, ARGMAX>(s, a, g.grid, g.lds_bytes);
+    if (ks == 8 && tpw == 1) return launch_t16<MR, 8, 1, ARGMAX>(s, a, g.grid, g.lds_bytes);
+    if (ks == 8 && tpw == 2) return launch_t16<MR, 8, 2, ARGMAX>(s, a, g.grid, g.lds_bytes);
+    if (ks == 16 && tpw == 1) return launch_t16<MR, 16, 1, ARGMAX>(s, a, g.grid, g.lds_bytes);
+    return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no TILE16 variant for K-split %u x %u tiles per workgroup", ks, tpw);
+}
+
+}  // namespace
+
+bool gemv_tile16_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
+    if (w.layout != MI355Q_LAYOUT_TILE16 || !w.tiles || x_dtype != MI355Q_BF16) return false;
+    if (m < 1 || m > 16) return false;
+    if (w.bits != 4 || w.group != 64 || w.k % 128) return false;
+    if (x_stride % 8) return false;                                   // 128-bit activation loads
+    return (size_t)m * ((size_t)w.k * 2 + 16) <= kT16LdsBudget;       // staged activations fit in LDS
+}
+
+Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_total_tiles, uint32_t k, uint32_t m) {
+    Tile16LaunchShape g{};
+    const uint32_t kblocks = k / 128;
+    const uint32_t cus = (uint32_t)ctx->props.multiProcessorCount;
+    // Measured on MI355X.  K split: the smallest of 4, 8, 16 that puts about eight wavefronts on
+    // every CU (and leaves each wavefront at least two K-blocks).  Row tiles per workgroup: one for
+    // M = 1; more for batches, where the staged activations are the larger share of a workgroup's
+    // traffic, as long as 16 wavefronts hold them and half the CUs still get a workgroup.
+    uint32_t ks = 4;
+    while (ks < 16 && n_total_tiles * ks < cus * 8 && kblocks / (ks * 2) >= 2) ks *= 2;
+    const uint32_t want_tpw = m == 1 ? 1u : m <= 4 ? 2u : 4u;
+    uint32_t tpw = 1;
+    while (tpw < want_tpw && ks * tpw * 2 <= 16 && (n_total_tiles + tpw * 2 - 1) / (tpw * 2) >= cus / 2) tpw *= 2;
+    if ((size_t)m * ((size_t)k * 2 + 16) > 80 * 1024) {
+        // the staged activations leave room for one workgroup per CU: make it as large as possible
+        tpw = 1;
+        while (ks < 16 && kblocks / (ks * 2) >= 2) ks *= 2;
+    }
+    const int eks = env_int_cached("MI355Q_T16_KSPLIT", 0), etpw = env_int_cached("MI355Q_T16_TPW", 0);
+    if (eks) ks = (uint32_t)eks;
+    if (etpw) tpw = (uint32_t)etpw;
+    g.ksplit = ks;
+    g.tiles_per_wg = tpw;
+    g.waves = ks * tpw;
+    g.blocks_per_wave = (kblocks + ks - 1) / ks;
+    g.grid = (n_total_tiles + tpw - 1) / tpw;
+    g.block = g.waves * 64;
+    const size_t x_bytes = (size_t)m * ((size_t)k * 2 + 16);
+    const size_t red_bytes = (size_t)g.waves * 4 * 64 * 4;
+    g.lds_bytes = (uint32_t)(x_bytes > red_bytes ? x_bytes : red_bytes);
+    return g;
+}
+
+mi355q_status launch_gemv_tile16_multi(hipStream_t s, const mi355q_context* ctx, uint32_t count, const WView* w,
+                                       const void* x, void* const* y, const uint32_t* y_strides, int y_dtype,
+                                       uint32_t m, uint32_t x_stride, float* logits_f32, int32_t* token_out,
+                                       unsigned long long* argmax_scratch) {
+    if (count < 1 || count > (uint32_t)kTile16MaxSegments)
+        return fail(MI355Q_ERR_INVALID_ARGUMENT, "1..%d weights per fused launch", kTile16MaxSegments);
+    if ((uintptr_t)x % 16) return fail(MI355Q_ERR_INVALID_ARGUMENT, "activation pointer must be 16-byte aligned");
+    const bool argmax = token_out != nullptr;
+    if (argmax && (m != 1 || count != 1)) return fail(MI355Q_ERR_INVALID_ARGUMENT, "fused argmax needs M == 1");
+    if (logits_f32 && count != 1) return fail(MI355Q_ERR_INVALID_ARGUMENT, "fp32 logits need a single weight");
+    T16Args a{};
+    uint32_t tiles = 0;
+    for (uint32_t i = 0; i < (uint32_t)kTile16MaxSegments; i++) {
+        const uint32_t j = i < count ? i : count - 1;
+        if (i < count) tiles += (w[i].n + 15) / 16;
+        a.tiles[i] = w[j].tiles;
+        a.y[i] = y[j];
+        a.y_stride[i] = y_strides[j];
+        a.seg_rows[i] = w[j].n;
+        a.tile_end[i] = tiles;
+    }
+    const Tile16LaunchShape g = gemv_tile16_shape(ctx, tiles, w[0].k, m);
+    a.x = (const uint16_t*)x;
+    a.logits = logits_f32; a.token_out = token_out; a.scratch = argmax_scratch;
+    a.k = w[0].k; a.m = m; a.x_stride = x_stride;
+    a.kblocks = w[0].k / 128;
+    a.blocks_per_wave = g.blocks_per_wave;
+    a.lds_row_bytes = w[0].k * 2 + 16;
+    a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = w[0].sb_dtype;
+    const int mr = m == 1 ? 1 : m == 2 ? 2 : 4;
+    if (argmax) return launch_t16_shape<1, true>(s, a, g);
+    if (mr == 1) return launch_t16_shape<1, false>(s, a, g);
+    if (mr == 2) return launch_t16_shape<2, false>(s, a, g);
+    return launch_t16_shape<4, false>(s, a, g);
+}
+
+}  // namespace mi355q

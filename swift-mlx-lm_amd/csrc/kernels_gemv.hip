@@ -40,9 +40,11 @@ size_t lds_bytes(const WView& w, int mt) {
 
 int env_int(const char* name, int fallback) { return env_int_cached(name, fallback); }
 
-// Largest activation batch (1, 2, 4 or 8) whose staged activations fit the LDS budget.
+// Largest activation batch per launch (1, 2 or 4) whose staged activations fit the LDS budget.
+// Batches of 5 to 8 rows run as two launches: an 8-row variant of this kernel needs more registers
+// than a wavefront has.
 int max_mt(const WView& w) {
-    for (int mt = 8; mt >= 1; mt >>= 1)
+    for (int mt = 4; mt >= 1; mt >>= 1)
         if (lds_bytes(w, mt) <= kLdsBudget) return mt;
     return 0;
 }
@@ -53,7 +55,7 @@ int max_mt(const WView& w) {
 GemvCfg choose(const mi355q_context* ctx, const WView& w, uint32_t m, bool argmax) {
     GemvCfg c{};
     c.argmax = argmax;
-    c.mt = m <= 1 ? 1 : m <= 2 ? 2 : m <= 4 ? 4 : 8;
+    c.mt = m <= 1 ? 1 : m <= 2 ? 2 : 4;
     const Geo g = geo_for(w.bits);
     const size_t kc = 64 * (size_t)g.cpl;
     c.nc = (uint32_t)((w.k + kc - 1) / kc);
@@ -68,7 +70,7 @@ GemvCfg choose(const mi355q_context* ctx, const WView& w, uint32_t m, bool argma
         c.waves = (c.nc == 1 || (c.nc == 2 && big)) ? 4 : 8;
     } else {
         c.xreg = 0;
-        c.r = c.mt == 8 ? 1 : 2;
+        c.r = 2;
         c.waves = 4;
     }
     const int er = env_int("MI355Q_GEMV_R", 0), ew = env_int("MI355Q_GEMV_WAVES", 0),

@@ -56,6 +56,46 @@ mi355q_status launch_pack_sz(hipStream_t s, const uint16_t* scales, const uint16
     return MI355Q_OK;
 }
 
+// TILE16 records from a split-plane weight (q4, group 64, K % 128 == 0): one thread per output word.
+// Rows past N are zero (codes 0, scale 0, bias 0).  Layout: gemv_tile16.hip.
+__global__ __launch_bounds__(256) void tile16_pack_kernel(WView w, uint32_t* __restrict__ tiles, size_t words) {
+    const uint32_t kblocks = w.k >> 7;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < words; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t recno = i / 288u;
+        const uint32_t o = (uint32_t)(i - recno * 288u);
+        const uint32_t tile = (uint32_t)(recno / kblocks), kb = (uint32_t)(recno - (size_t)tile * kblocks);
+        uint32_t out = 0;
+        if (o < 256u) {
+            const uint32_t lane = o >> 2, j = o & 3u, n = lane & 15u, kq = lane >> 4;
+            const uint32_t row = tile * 16u + n;
+            if (row < w.n) {
+                const uint32_t code0 = kb * 128u + (j >> 1) * 64u + kq * 16u + (j & 1u) * 8u;   // first of 8 codes
+                const uint32_t src = w.codes[(size_t)row * w.code_stride + (code0 >> 3)];
+#pragma unroll
+                for (uint32_t e = 0; e < 8; e++) {
+                    const uint32_t nib = (e >> 1) + 4u * (e & 1u);
+                    out |= ((src >> (4u * e)) & 0xFu) << (4u * nib);
+                }
+            }
+        } else {
+            const uint32_t q = o - 256u, n = q >> 1, g = q & 1u;
+            const uint32_t row = tile * 16u + n;
+            if (row < w.n) out = w.sz[(size_t)row * w.sz_stride + kb * 2u + g];
+        }
+        tiles[i] = out;
+    }
+}
+
+mi355q_status launch_tile16_pack(hipStream_t s, const WView& planes, uint32_t* tiles) {
+    const size_t words = (size_t)((planes.n + 15) / 16) * (planes.k / 128) * 288u;
+    size_t blocks = (words + 255) / 256;
+    if (blocks > 16384) blocks = 16384;
+    if (blocks == 0) blocks = 1;
+    tile16_pack_kernel<<<dim3((unsigned)blocks), dim3(256), 0, s>>>(planes, tiles, words);
+    MI355Q_HIP(hipGetLastError());
+    return MI355Q_OK;
+}
+
 // ------------------------------------------------------------------------------ dequant bf16
 // One workgroup per row, 256 threads striding over the row, as the reference kernel does.
 // scale*q and +zero are kept as two roundings so the result is bit-identical to an unfused

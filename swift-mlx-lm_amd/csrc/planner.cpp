@@ -47,7 +47,15 @@ void plan_small_m(const mi355q_weight* w, uint32_t m, int x_dtype, uint32_t x_st
                   mi355q_step* s) {
     const WView v = w->view();
     const bool forced = flags & MI355Q_FLAG_FORCE_GENERIC;
-    if (!forced && gemv_fast_eligible(v, x_dtype, m > 8 ? 8 : m, x_stride)) {
+    if (!forced && gemv_tile16_eligible(v, x_dtype, m > 16 ? 16 : m, x_stride)) {
+        const Tile16LaunchShape g = gemv_tile16_shape(w->ctx, (uint32_t)((w->n + 15) / 16), (uint32_t)w->k, m > 16 ? 16 : m);
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_tile16_q%u_g%u", (unsigned)w->fmt.bits,
+                      w->fmt.group_size);
+        s->grid[0] = g.grid;
+        s->block[0] = g.block;
+        s->lds_bytes = g.lds_bytes;
+        s->rows_per_workgroup = 16;
+    } else if (!forced && gemv_fast_eligible(v, x_dtype, m > 8 ? 8 : m, x_stride)) {
         const GemvLaunchShape g = gemv_fast_shape(w->ctx, v, m > 8 ? 8 : m);
         std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_planes_q%u_g%u", (unsigned)w->fmt.bits,
                       w->fmt.group_size);

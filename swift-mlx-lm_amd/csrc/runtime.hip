@@ -137,6 +137,29 @@ mi355q_status build_rows(mi355q_weight* w, const void* codes_host) {
     return fill_sz(w);
 }
 
+// TILE16: build the split-plane rows first, re-tile them on the device, drop the rows.
+mi355q_status check_tile16(const mi355q_format* f, uint64_t k) {
+    if (f->bits != 4 || f->group_size != 64)
+        return fail(MI355Q_ERR_UNSUPPORTED_FORMAT, "the TILE16 layout holds 4-bit codes in groups of 64 (got q%u g%u)",
+                    (unsigned)f->bits, f->group_size);
+    if (k % 128) return fail(MI355Q_ERR_SHAPE, "the TILE16 layout needs K %% 128 == 0 (K=%llu)", (unsigned long long)k);
+    return MI355Q_OK;
+}
+
+mi355q_status planes_to_tile16(mi355q_weight* w) {
+    w->layout = MI355Q_LAYOUT_PLANES;
+    const mi355q::WView v = w->view();
+    w->tiles_bytes = (size_t)((w->n + 15) / 16) * (w->k / 128) * 1152;
+    MI355Q_HIP(hipMalloc(&w->tiles, w->tiles_bytes));
+    if (mi355q_status st = launch_tile16_pack(nullptr, v, (uint32_t*)w->tiles)) return st;
+    MI355Q_HIP(hipStreamSynchronize(nullptr));
+    (void)hipFree(w->codes);  w->codes = nullptr; w->sz = nullptr; w->codes_bytes = 0;
+    (void)hipFree(w->scales); w->scales = nullptr;
+    (void)hipFree(w->biases); w->biases = nullptr;
+    w->layout = MI355Q_LAYOUT_TILE16;
+    return MI355Q_OK;
+}
+
 mi355q_status need_ctx(mi355q_context* ctx) {
     if (!ctx) return fail(MI355Q_ERR_NULL_HANDLE, "context is null");
     hipError_t e = hipSetDevice(ctx->device);
@@ -344,9 +367,11 @@ mi355q_status mi355q_weight_prepare_mlx(mi355q_context* ctx, uint8_t scheme_iden
     if (!f) return fail(MI355Q_ERR_UNSUPPORTED_FORMAT, "unsupported scheme 0x%02x", scheme_identifier);
     if (!codes_host || !scales_host || !biases_host) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null plane pointer");
     if ((int)sb_dtype < 0 || (int)sb_dtype > 2) return fail(MI355Q_ERR_INVALID_ARGUMENT, "bad scale dtype");
-    if (layout != MI355Q_LAYOUT_STAF_BLOCKS && layout != MI355Q_LAYOUT_PLANES)
+    if (layout != MI355Q_LAYOUT_STAF_BLOCKS && layout != MI355Q_LAYOUT_PLANES && layout != MI355Q_LAYOUT_TILE16)
         return fail(MI355Q_ERR_INVALID_ARGUMENT, "bad layout");
     if (mi355q_status s = check_shape(f, n_rows, k)) return s;
+    if (layout == MI355Q_LAYOUT_TILE16)
+        if (mi355q_status s = check_tile16(f, k)) return s;
     if ((k * f->bits) % 32)
         return fail(MI355Q_ERR_SHAPE, "MLX planes need K*bits to be a whole number of 32-bit words (K=%llu bits=%u)",
                     (unsigned long long)k, (unsigned)f->bits);
@@ -381,7 +406,8 @@ mi355q_status mi355q_weight_prepare_mlx(mi355q_context* ctx, uint8_t scheme_iden
             }
         }
     }
-    if (st == MI355Q_OK && layout == MI355Q_LAYOUT_PLANES) st = build_rows(w, codes_host);
+    if (st == MI355Q_OK && layout != MI355Q_LAYOUT_STAF_BLOCKS) st = build_rows(w, codes_host);
+    if (st == MI355Q_OK && layout == MI355Q_LAYOUT_TILE16) st = planes_to_tile16(w);
     if (st != MI355Q_OK) {
         mi355q_weight_destroy(w);
         return st;
@@ -399,14 +425,16 @@ mi355q_status mi355q_weight_prepare_staf(mi355q_context* ctx, uint8_t scheme_ide
     const mi355q_format* f = find_format_scheme(scheme_identifier);
     if (!f) return fail(MI355Q_ERR_UNSUPPORTED_FORMAT, "unsupported scheme 0x%02x", scheme_identifier);
     if (!blocks_host) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null block pointer");
-    if (layout != MI355Q_LAYOUT_STAF_BLOCKS && layout != MI355Q_LAYOUT_PLANES)
+    if (layout != MI355Q_LAYOUT_STAF_BLOCKS && layout != MI355Q_LAYOUT_PLANES && layout != MI355Q_LAYOUT_TILE16)
         return fail(MI355Q_ERR_INVALID_ARGUMENT, "bad layout");
     if (mi355q_status s = check_shape(f, n_rows, k)) return s;
+    if (layout == MI355Q_LAYOUT_TILE16)
+        if (mi355q_status s = check_tile16(f, k)) return s;
     const size_t groups = (size_t)n_rows * (k / f->group_size);
     if (payload_bytes != groups * f->bytes_per_block)
         return fail(MI355Q_ERR_SIZE_MISMATCH, "payload is %zu bytes, expected %zu", payload_bytes,
                     groups * f->bytes_per_block);
-    if (layout == MI355Q_LAYOUT_PLANES && (k * f->bits) % 32)
+    if (layout != MI355Q_LAYOUT_STAF_BLOCKS && (k * f->bits) % 32)
         return fail(MI355Q_ERR_SHAPE, "the planes layout needs K*bits to be a whole number of 32-bit words");
     mi355q_weight* w = new_weight(ctx, f, n_rows, k);
     if (!w) return fail(MI355Q_ERR_OUT_OF_MEMORY, "host allocation failed");
@@ -435,7 +463,8 @@ mi355q_status mi355q_weight_prepare_staf(mi355q_context* ctx, uint8_t scheme_ide
         st = upload_new(&w->scales, s16.data(), w->sb_bytes);
         if (st == MI355Q_OK) st = upload_new(&w->biases, z16.data(), w->sb_bytes);
     }
-    if (st == MI355Q_OK && layout == MI355Q_LAYOUT_PLANES) st = build_rows(w, planes_codes.data());
+    if (st == MI355Q_OK && layout != MI355Q_LAYOUT_STAF_BLOCKS) st = build_rows(w, planes_codes.data());
+    if (st == MI355Q_OK && layout == MI355Q_LAYOUT_TILE16) st = planes_to_tile16(w);
     if (st != MI355Q_OK) {
         mi355q_weight_destroy(w);
         return st;
@@ -535,6 +564,7 @@ mi355q_status mi355q_weight_destroy(mi355q_weight* w) {
         if (w->codes) (void)hipFree(w->codes);
         if (w->scales) (void)hipFree(w->scales);
         if (w->biases) (void)hipFree(w->biases);
+        if (w->tiles) (void)hipFree(w->tiles);
     }
     if (w->sz && w->sz_separate) (void)hipFree(w->sz);
     delete w;

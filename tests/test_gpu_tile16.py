@@ -1,0 +1,254 @@
+"""GPU parity tests of the matrix-core decode kernel over the TILE16 layout (4-bit, group 64), through
+the C ABI: the same projections as gemv_q4_g64 / gemm_q4_g64 of the reference
+(MetalSourceGenerator+Quantized.swift:496-575, :22-156) for 1 <= M <= 16 rows per launch.
+
+Bars: unpacked codes and dequantised bf16 bit patterns of the re-tiled weight are bit-exact against
+the CPU oracle; fp32 outputs within relative L2 <= 1e-3 and max-abs <= 2e-2 of an fp64 accumulation
+of the same dequantised weights; bf16 outputs equal bf16_rne(fp32 outputs); token indices exact.
+"""
+import sys
+
+import numpy as np
+import pytest
+
+import kat
+import oracle
+from gpu_util import Case, act_rounded, assert_within_tolerance, out_from_device, seeded_case
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def _fmt(pkg):
+    return pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+
+
+def _run(ctx, pkg, w, x, y_dtype, use_qgemm=False, flags=0):
+    m, k = x.shape
+    n = int(w.info.n_rows)
+    xd = ctx.upload(oracle.bf16_from_f32(x).reshape(x.shape))
+    yd = ctx.alloc(m * n * (4 if y_dtype == pkg.F32 else 2))
+    ctx.fill(yd, 0x7FC00000 if y_dtype == pkg.F32 else 0x7FC07FC0)
+    (ctx.qgemm if use_qgemm else ctx.qgemv)(w, xd, pkg.BF16, yd, y_dtype, m, 0, 0, flags)
+    ctx.synchronize()
+    y = out_from_device(yd, y_dtype, (m, n), pkg)
+    xd.free(); yd.free()
+    return y
+
+
+@pytest.mark.parametrize("n,k", [(16, 128), (37, 256), (1, 128), (130, 1024 + 128), (512, 4096)])
+def test_retiled_weight_unpacks_and_dequantises_bit_exactly(pkg, ctx, n, k):
+    """The device re-tiling (rows -> TILE16 records, nibble permutation included) loses nothing:
+    unpack_codes and dequant_bf16 on the re-tiled weight equal the CPU oracle on the source planes,
+    for both sources (MLX planes with bf16 scales, STAF blocks with f16 scales)."""
+    words, s, z, wq = seeded_case(2000 + n, n, k, 4, 64)
+    want_codes = oracle.unpack_plane_codes(4, n, k, words)
+    w = ctx.weight_prepare_mlx(_fmt(pkg), words, s, z, pkg.BF16, pkg.LAYOUT_TILE16)
+    assert w.info.layout == pkg.LAYOUT_TILE16 and w.info.weight_bytes == n * (k // 64) * 36
+    out = ctx.alloc(n * k); ctx.unpack_codes(w, out); ctx.synchronize()
+    assert np.array_equal(out.download(np.uint8, (n, k)), want_codes)
+    deq = ctx.alloc(n * k * 2); ctx.dequant_bf16(w, deq); ctx.synchronize()
+    assert np.array_equal(deq.download(np.uint16, (n, k)), oracle.bf16_from_f32(wq).reshape(n, k))
+    out.free(); deq.free(); w.destroy()
+    # from STAF blocks (f16 headers)
+    rng = np.random.default_rng(n * 7 + k)
+    codes = rng.integers(0, 16, (n, k), dtype=np.uint8)
+    case = Case(4, 64, codes, rng.choice([0.0625, 0.125, 0.5], (n, k // 64)), rng.integers(-8, 8, (n, k // 64)) * 0.125)
+    blocks = case.staf_blocks()
+    w = ctx.weight_prepare_staf(_fmt(pkg), n, k, blocks, pkg.LAYOUT_TILE16)
+    out = ctx.alloc(n * k); ctx.unpack_codes(w, out); ctx.synchronize()
+    assert np.array_equal(out.download(np.uint8, (n, k)), codes)
+    deq = ctx.alloc(n * k * 2); ctx.dequant_bf16(w, deq); ctx.synchronize()
+    assert np.array_equal(deq.download(np.uint16, (n, k)), oracle.dequant_staf_bf16(4, 64, n, k, blocks).reshape(n, k))
+    out.free(); deq.free(); w.destroy()
+
+
+LLAMA = {"q_o": (4096, 4096), "k_v": (1024, 4096), "gate_up": (14336, 4096), "down": (4096, 14336)}
+
+
+@pytest.mark.parametrize("name", list(LLAMA))
+def test_tile16_llama_shapes_all_batch_sizes(pkg, ctx, name):
+    """BASELINE config 1 shapes, M = 1, 2, 4, 8 (and the sizes in between up to 16)."""
+    n, k = LLAMA[name]
+    words, s, z, wq = seeded_case(2100 + n % 89, n, k, 4, 64)
+    w = ctx.weight_prepare_mlx(_fmt(pkg), words, s, z, pkg.BF16, pkg.LAYOUT_TILE16)
+    for m in (1, 2, 3, 4, 5, 8, 13, 16):
+        if m * (k * 2 + 16) > 144 * 1024:
+            continue                                           # runs as several launches: covered below
+        x = act_rounded(kat.seeded_activations(2200 + m, m, k), pkg.BF16, pkg)
+        say(f"tile16 {name} M={m}")
+        want = oracle.gemm_f64(wq, x)
+        use_qgemm = m > 8
+        y32 = _run(ctx, pkg, w, x, pkg.F32, use_qgemm)
+        rel, _ = assert_within_tolerance(y32, want, f"{name} M={m}")
+        assert rel < 1e-4
+        ybf = _run(ctx, pkg, w, x, pkg.BF16, use_qgemm)
+        assert np.array_equal(oracle.bf16_from_f32(ybf), oracle.bf16_from_f32(y32))
+    w.destroy()
+
+
+def test_tile16_ragged_shapes_and_long_batches(pkg, ctx):
+    """N off the 16-row tile, single row, short and long K, f16 scales, M beyond one launch."""
+    for i, (n, k) in enumerate([(1, 128), (5, 256), (17, 128), (130, 2048 + 128), (4099, 384), (33, 14336)]):
+        words, s, z, wq = seeded_case(2300 + i, n, k, 4, 64)
+        w = ctx.weight_prepare_mlx(_fmt(pkg), words, s, z, pkg.BF16, pkg.LAYOUT_TILE16)
+        for m in (1, 3, 7, 16, 21, 40):
+            x = act_rounded(kat.seeded_activations(2400 + i + m, m, k), pkg.BF16, pkg)
+            say(f"tile16 ragged {k}->{n} M={m}")
+            got = _run(ctx, pkg, w, x, pkg.F32, use_qgemm=m > 8)
+            assert_within_tolerance(got, oracle.gemm_f64(wq, x), f"{k}->{n} M={m}")
+        w.destroy()
+    # f16 scale words (STAF source)
+    rng = np.random.default_rng(5)
+    n, k = 70, 512
+    codes = rng.integers(0, 16, (n, k), dtype=np.uint8)
+    scales = rng.choice([0.0625, 0.125, 0.25], (n, k // 64)); zeros = rng.integers(-8, 8, (n, k // 64)) * 0.0625
+    case = Case(4, 64, codes, scales, zeros)
+    w = ctx.weight_prepare_staf(_fmt(pkg), n, k, case.staf_blocks(), pkg.LAYOUT_TILE16)
+    wq = (scales.repeat(64, axis=1) * codes + zeros.repeat(64, axis=1)).astype(np.float32)
+    for m in (1, 6):
+        x = act_rounded(kat.seeded_activations(2500 + m, m, k), pkg.BF16, pkg)
+        assert_within_tolerance(_run(ctx, pkg, w, x, pkg.F32), oracle.gemm_f64(wq, x), f"f16 scales M={m}")
+    w.destroy()
+
+
+def test_tile16_exact_small_integers_and_scaling(pkg, ctx):
+    """Exactly representable case (every partial sum an integer multiple of 2^-6 below 2^20): the
+    result must be exact whatever the summation order; and y(2x) == 2*y(x) bit for bit at full size."""
+    rng = np.random.default_rng(11)
+    n, k = 100, 1024
+    codes = rng.integers(0, 16, (n, k), dtype=np.uint8)
+    scales = rng.choice([0.125, 0.25, 0.5], (n, k // 64)); zeros = rng.integers(-4, 5, (n, k // 64)) * 0.25
+    case = Case(4, 64, codes, scales, zeros)
+    wq = scales.repeat(64, axis=1) * codes + zeros.repeat(64, axis=1)
+    for sb, w in ((pkg.F16, ctx.weight_prepare_staf(_fmt(pkg), n, k, case.staf_blocks(), pkg.LAYOUT_TILE16)),
+                  (pkg.BF16, ctx.weight_prepare_mlx(_fmt(pkg), *case.planes(pkg.BF16, pkg), pkg.BF16, pkg.LAYOUT_TILE16))):
+        for m in (1, 2, 4, 9):
+            x = rng.integers(-8, 9, (m, k)).astype(np.float32) * 0.125
+            got = _run(ctx, pkg, w, x, pkg.F32, use_qgemm=m > 8)
+            assert np.array_equal(got.astype(np.float64), x.astype(np.float64) @ wq.T), (sb, m)
+        w.destroy()
+    n, k = 14336, 4096
+    words, s, z, _ = seeded_case(2600, n, k, 4, 64)
+    w = ctx.weight_prepare_mlx(_fmt(pkg), words, s, z, pkg.BF16, pkg.LAYOUT_TILE16)
+    x = act_rounded(kat.seeded_activations(2601, 2, k), pkg.BF16, pkg)
+    y1, y2 = _run(ctx, pkg, w, x, pkg.F32), _run(ctx, pkg, w, 2.0 * x, pkg.F32)
+    assert np.array_equal(2.0 * y1, y2)
+    w.destroy()
+
+
+def test_tile16_batched_projections_one_launch(pkg, ctx):
+    for ns, k in [((4096, 1024, 1024), 4096), ((14336, 14336), 4096), ((5, 17, 130), 256)]:
+        ws, wqs = [], []
+        for i, n in enumerate(ns):
+            words, s, z, wq = seeded_case(2700 + i + n % 13, n, k, 4, 64)
+            ws.append(ctx.weight_prepare_mlx(_fmt(pkg), words, s, z, pkg.BF16, pkg.LAYOUT_TILE16)); wqs.append(wq)
+        for m in (1, 4, 11):
+            x = act_rounded(kat.seeded_activations(2750 + m, m, k), pkg.BF16, pkg)
+            xd = ctx.upload(oracle.bf16_from_f32(x).reshape(x.shape))
+            yds = [ctx.alloc(m * n * 4) for n in ns]
+            say(f"tile16 batched {ns} M={m}")
+            ctx.batched_qgemm(ws, xd, pkg.BF16, yds, pkg.F32, m)
+            ctx.synchronize()
+            for i, n in enumerate(ns):
+                assert_within_tolerance(yds[i].download(np.float32, (m, n)), oracle.gemm_f64(wqs[i], x), f"{ns} seg {i}")
+            xd.free()
+            for b in yds:
+                b.free()
+        for w in ws:
+            w.destroy()
+
+
+def test_tile16_lm_head_fused_argmax(pkg, ctx):
+    """BASELINE config 4 (2048 -> 65536): token == lowest-index argmax of the GPU's own fp32 logits and
+    of the CPU reference logits; ties resolve to the lowest index."""
+    n, k = 65536, 2048
+    words, s, z, wq = seeded_case(2800, n, k, 4, 64)
+    w = ctx.weight_prepare_mlx(_fmt(pkg), words, s, z, pkg.BF16, pkg.LAYOUT_TILE16)
+    x = act_rounded(kat.seeded_activations(2801, 1, k), pkg.BF16, pkg)
+    xd = ctx.upload(oracle.bf16_from_f32(x)); logits = ctx.alloc(n * 4); tok = ctx.upload(np.array([-7], np.int32))
+    for rep in range(3):                                     # the scratch cells reset themselves
+        ctx.lmhead_argmax(w, xd, pkg.BF16, logits, tok)
+        ctx.synchronize()
+        got = logits.download(np.float32)
+        assert int(tok.download(np.int32)[0]) == oracle.argmax_lowest(got)
+    want = oracle.gemm_f64(wq, x)[0]
+    assert_within_tolerance(got, want, "lm head logits")
+    assert int(tok.download(np.int32)[0]) == int(np.argmax(want))
+    ctx.lmhead_argmax(w, xd, pkg.BF16, None, tok)            # token only
+    ctx.synchronize()
+    assert int(tok.download(np.int32)[0]) == int(np.argmax(want))
+    w.destroy()
+    # ties: identical rows placed across tile and workgroup boundaries
+    n, k = 4096, 256
+    codes = np.zeros((n, k), np.uint8); codes[[7, 15, 16, 1000, 4095]] = 9
+    case = Case(4, 64, codes, np.full((n, k // 64), 0.25), np.full((n, k // 64), -0.5))
+    w = ctx.weight_prepare_staf(_fmt(pkg), n, k, case.staf_blocks(), pkg.LAYOUT_TILE16)
+    x = np.full((1, k), 0.5, np.float32)
+    xd2 = ctx.upload(oracle.bf16_from_f32(x)); lg2 = ctx.alloc(n * 4)
+    ctx.lmhead_argmax(w, xd2, pkg.BF16, lg2, tok); ctx.synchronize()
+    assert int(tok.download(np.int32)[0]) == 7
+    w.destroy()
+    for b in (xd, logits, tok, xd2, lg2):
+        b.free()
+
+
+def test_tile16_errors_and_plan_records(pkg, ctx):
+    fmt8 = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(8, 32)
+    words, s, z, _ = seeded_case(2900, 16, 128, 8, 32)
+    with pytest.raises(pkg.MI355QError):                      # only q4 g64
+        ctx.weight_prepare_mlx(fmt8, words, s, z, pkg.BF16, pkg.LAYOUT_TILE16)
+    words, s, z, _ = seeded_case(2901, 16, 192, 4, 64)
+    with pytest.raises(pkg.MI355QError):                      # K % 128
+        ctx.weight_prepare_mlx(_fmt(pkg), words, s, z, pkg.BF16, pkg.LAYOUT_TILE16)
+    words, s, z, wq = seeded_case(2902, 256, 512, 4, 64)
+    w = ctx.weight_prepare_mlx(_fmt(pkg), words, s, z, pkg.BF16, pkg.LAYOUT_TILE16)
+    st = w.plan_decode_step(4)
+    assert st.device_kernel == "gemv_tile16_q4_g64" and not st.used_fallback and st.grid[0] == 16
+    # f32 activations are not served by the tile kernel: the per-code kernel runs and agrees
+    x = act_rounded(kat.seeded_activations(2903, 2, 512), pkg.BF16, pkg)
+    xd = ctx.upload(x.astype(np.float32)); yd = ctx.alloc(2 * 256 * 4)
+    ctx.qgemv(w, xd, pkg.F32, yd, pkg.F32, 2); ctx.synchronize()
+    assert_within_tolerance(yd.download(np.float32, (2, 256)), oracle.gemm_f64(wq, x), "f32 activations")
+    got_generic = _run(ctx, pkg, w, x, pkg.F32, flags=pkg.FLAG_FORCE_GENERIC)
+    assert_within_tolerance(got_generic, oracle.gemm_f64(wq, x), "forced generic")
+    xd.free(); yd.free(); w.destroy()
+
+
+def test_tile16_plan_replay_and_graph(pkg, ctx):
+    k = 1024
+    ns = (512, 256, 2048)
+    ws = []
+    for i, n in enumerate(ns):
+        words, s, z, _ = seeded_case(3000 + i, n, k, 4, 64)
+        ws.append(ctx.weight_prepare_mlx(_fmt(pkg), words, s, z, pkg.BF16, pkg.LAYOUT_TILE16))
+    x = ctx.upload(oracle.bf16_from_f32(kat.seeded_activations(3010, 1, k)))
+    ys = [ctx.alloc(n * 4) for n in ns]
+    tok = ctx.upload(np.array([-3], np.int32))
+    ctx.batched_qgemm(ws[:2], x, pkg.BF16, ys[:2], pkg.F32, 1)
+    ctx.lmhead_argmax(ws[2], x, pkg.BF16, ys[2], tok)
+    ctx.synchronize()
+    eager = [y.download(np.float32) for y in ys]; etok = int(tok.download(np.int32)[0])
+    assert etok == oracle.argmax_lowest(eager[2])
+    plan = pkg.DispatchPlan(ctx)
+    plan.add_batched_linear(ws[:2], x, pkg.BF16, ys[:2], pkg.F32, 1)
+    plan.add_output_head(ws[2], x, pkg.BF16, ys[2], tok)
+    stream = ctx.stream_create()
+    plan.graph_build(stream)
+    for rep in range(3):
+        for y in ys:
+            ctx.fill(y, 0x7FC00000, stream)
+        tok.upload(np.array([-3], np.int32))
+        plan.graph_launch(stream) if rep else plan.encode(stream)
+        ctx.synchronize(stream)
+        for y, want in zip(ys, eager):
+            assert np.array_equal(y.download(np.float32), want), rep
+        assert int(tok.download(np.int32)[0]) == etok
+    plan.destroy()
+    for b in ys + [x, tok]:
+        b.free()
+    for w in ws:
+        w.destroy()
