@@ -89,6 +89,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-parity", action="store_true")
     ap.add_argument("--no-prefill", action="store_true", help="skip the secondary prefill-GEMM figure")
+    ap.add_argument("--no-batch-sweep", action="store_true", help="skip the secondary M = 1, 2, 4, 8 figures")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (one process, one device); "
@@ -216,6 +217,43 @@ def main():
         per_shape[label] = {"us": round(ms * 1e3, 3), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1), "weight_bytes": nbytes}
         log(f"  {label:8s}: {ms * 1e3:.2f} us/launch, {per_shape[label]['GBps']} GB/s")
         p1.destroy()
+    # ---- secondary: the same layer step at M = 1, 2, 4, 8 activation rows (BASELINE config 1), on
+    # the split-plane layout and on the matrix-core tile layout (4-launch schedule, stream replay)
+    batch_sweep = None
+    if not a.no_batch_sweep:
+        batch_sweep = {}
+        n_t16 = min(a.layers, 8)                       # 8 x 123 MB: well past the 256 MB last-level cache
+        for lname, layout, pool in (("planes", pkg.LAYOUT_PLANES, layers[:n_t16]), ("tile16", pkg.LAYOUT_TILE16, None)):
+            if pool is None:
+                pool = [{name: ctx.weight_prepare_mlx(fmt, *host[name], pkg.BF16, layout) for name, _, _ in LAYER_SHAPES}
+                        for _ in range(n_t16)]
+            batch_sweep[lname] = {}
+            for m in (1, 2, 4, 8):
+                xm = {k: ctx.alloc(m * k * 2) for k in (4096, 14336)}
+                for k in xm:
+                    ctx.fill(xm[k], 0x3C003C00, stream)
+                ym = {name: ctx.alloc(m * n * 2) for name, n, _ in LAYER_SHAPES}
+                pl = pkg.DispatchPlan(ctx)
+                for L in pool:
+                    pl.add_batched_linear([L["q"], L["k"], L["v"]], xm[4096], pkg.BF16, [ym["q"], ym["k"], ym["v"]],
+                                          pkg.BF16, m)
+                    pl.add_linear(L["o"], xm[4096], pkg.BF16, ym["o"], pkg.BF16, m)
+                    pl.add_batched_linear([L["gate"], L["up"]], xm[4096], pkg.BF16, [ym["gate"], ym["up"]], pkg.BF16, m)
+                    pl.add_linear(L["down"], xm[14336], pkg.BF16, ym["down"], pkg.BF16, m)
+                pl.encode(stream)
+                ctx.synchronize(stream)
+                ms = time_region(ctx, lambda i: pl.encode(stream), 8, stream) / len(pool)
+                batch_sweep[lname][f"M={m}"] = {"us_per_step": round(ms * 1e3, 2),
+                                                "GBps": round(layer_bytes / (ms * 1e-3) / 1e9, 1)}
+                pl.destroy()
+                for b in list(xm.values()) + list(ym.values()):
+                    b.free()
+            log(f"  batch sweep {lname}: " + ", ".join(f"{k} {v['us_per_step']} us" for k, v in batch_sweep[lname].items()))
+            if lname == "tile16":
+                for L in pool:
+                    for w in L.values():
+                        w.destroy()
+
     # the dominant kernel of the reported schedule: the fused gate+up launch, or the gate launch
     dom = "gate_up" if mode.startswith("4-launch") else "gate"
     dom_bytes = per_shape[dom]["weight_bytes"]
@@ -268,7 +306,7 @@ def main():
                    "weight_bytes_per_step": layer_bytes, "layers_resident": a.layers,
                    "replay": mode, "replay_GBps": replay_gbps,
                    "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2), "per_shape": per_shape,
-                   "prefill_gemm_gate": prefill},
+                   "batch_sweep": batch_sweep, "prefill_gemm_gate": prefill},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": TRAFFIC_BYTES[dom],
                      "algorithmic_bytes": dom_bytes,
