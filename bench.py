@@ -29,10 +29,10 @@ HBM_PEAK_GBPS = 8000.0            # MI355X published HBM3E bandwidth
 LAYER_SHAPES = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
                 ("gate", 14336, 4096), ("up", 14336, 4096), ("down", 4096, 14336)]
 BITS, GROUP = 4, 64
-# HBM bytes per gate/up launch from the FETCH_SIZE and WRITE_SIZE counters, each scaled by what the
+# HBM bytes per gate launch and per fused gate+up launch from the FETCH_SIZE and WRITE_SIZE counters, each scaled by what the
 # same counter reads for a plain copy of the same size (profiles/gemv_planes_q4_g64_gate_up_hbm_traffic_pmc.md).
 # Measured offline with the profiler; valid for the kernel variant named in `roofline.kernel`.
-TRAFFIC_BYTES = {"gate": 33255544, "gate_up": None}
+TRAFFIC_BYTES = {"gate": 33243385, "gate_up": 66307175}
 
 
 def log(*a):
