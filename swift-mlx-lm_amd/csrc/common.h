@@ -56,6 +56,9 @@ struct mi355q_context {
     hipDeviceProp_t props;
     // scratch of the fused LM-head/argmax launch: [0] packed (key,~index) maximum, [1] ticket
     unsigned long long* argmax_scratch;
+    // split-K partial results of the prefill GEMM: grown on demand, never shrunk
+    void* workspace;
+    size_t workspace_bytes;
 };
 
 struct mi355q_weight {
@@ -157,14 +160,16 @@ int env_int_cached(const char* name, int fallback);
 
 // MFMA GEMM (kernels_gemm.hip)
 struct GemmLaunchShape {
-    uint32_t bm, bn, stages, grid, block, lds_bytes;
+    uint32_t bm, bn, stages, grid, block, lds_bytes, splits, kt_per_split;
 };
-GemmLaunchShape gemm_mfma_shape(const mi355q_context* ctx, uint32_t m, uint32_t n);
+GemmLaunchShape gemm_mfma_shape(const mi355q_context* ctx, uint32_t m, uint32_t n, uint32_t k);
+// Grows the context's scratch buffer (split-K partials); the buffer is kept until the context goes.
+mi355q_status ensure_workspace(mi355q_context* ctx, size_t bytes);
 bool gemm_mfma_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
-mi355q_status launch_qgemm_mfma(hipStream_t s, const mi355q_context* ctx, const WView& w,
+mi355q_status launch_qgemm_mfma(hipStream_t s, mi355q_context* ctx, const WView& w,
                                 const void* x, int x_dtype, void* y, int y_dtype, uint32_t m,
                                 uint32_t x_stride, uint32_t y_stride);
-mi355q_status launch_gemm_bf16_mfma(hipStream_t s, const mi355q_context* ctx, const void* a,
+mi355q_status launch_gemm_bf16_mfma(hipStream_t s, mi355q_context* ctx, const void* a,
                                     int a_dtype, const uint16_t* b, void* c, int c_dtype,
                                     uint32_t m, uint32_t n, uint32_t k, uint32_t a_stride,
                                     uint32_t c_stride);

@@ -39,6 +39,8 @@ struct GemmArgs {
     uint32_t code_stride, sz_stride;   // 32-bit words between consecutive rows
     uint32_t y_dtype, sb_dtype;
     uint32_t tiles_m, tiles_n;
+    float* partial;          // split-K: fp32 [splits][M][N] partial results (null when K is not split)
+    uint32_t kt_per_split;   // K-tiles per split (blockIdx.y indexes the split)
     uint32_t dbg;            // tuning builds only: bit0 fetch only the first K-tile, bit1 fill LDS only once
 };
 
@@ -237,7 +239,10 @@ __global__ __launch_bounds__(WAVES * 64, (STAGES == 1 ? 2 : 1)) void qgemm_mfma_
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-    const uint32_t KT = a.k / kTileK;
+    // K range of this workgroup: all of K, or one of the splits (blockIdx.y)
+    const uint32_t KT_all = a.k / kTileK;
+    const uint32_t kt0 = blockIdx.y * a.kt_per_split;
+    const uint32_t KT = kt0 + a.kt_per_split < KT_all ? kt0 + a.kt_per_split : KT_all;   // end (exclusive)
     const uint32_t frag_row = lane & 31, frag_half = lane >> 5;
     bf16x8_t af[2][TM], bf[2][TN];
     auto load_frags = [&](auto KK, uint32_t stage) __attribute__((always_inline)) {
@@ -272,7 +277,7 @@ __global__ __launch_bounds__(WAVES * 64, (STAGES == 1 ? 2 : 1)) void qgemm_mfma_
         });
     };
 
-    fetch(0);
+    fetch(kt0);
     if constexpr (STAGES == 2) {
         // Software pipeline over K-tiles, all inside one wavefront's instruction stream: while the
         // MFMAs of K-tile kt run, K-tile kt+1 moves from registers to the other LDS stage (part by
@@ -280,9 +285,9 @@ __global__ __launch_bounds__(WAVES * 64, (STAGES == 1 ? 2 : 1)) void qgemm_mfma_
         // indices past the end are clamped: the extra fetches and the extra LDS fill are never read.
         stash(0);
         __syncthreads();
-        fetch(KT > 1 ? 1u : 0u);
-        for (uint32_t kt = 0; kt < KT; kt++) {
-            const uint32_t stage = kt & 1;
+        fetch(kt0 + 1 < KT ? kt0 + 1 : kt0);
+        for (uint32_t kt = kt0; kt < KT; kt++) {
+            const uint32_t stage = (kt - kt0) & 1;
             const uint32_t k2 = kt + 2 < KT ? kt + 2 : KT - 1;
             load_frags(std::integral_constant<int, 0>{}, stage);
             static_for<NP>([&](auto KK) __attribute__((always_inline)) {
@@ -315,9 +320,9 @@ __global__ __launch_bounds__(WAVES * 64, (STAGES == 1 ? 2 : 1)) void qgemm_mfma_
             __syncthreads();
         }
     } else {
-        for (uint32_t kt = 0; kt < KT; kt++) {
+        for (uint32_t kt = kt0; kt < KT; kt++) {
 #ifdef MI355Q_GEMV_EXPERIMENT
-            if (!(a.dbg & 2) || kt == 0)
+            if (!(a.dbg & 2) || kt == kt0)
 #endif
             stash(0);
             __syncthreads();
@@ -340,8 +345,12 @@ __global__ __launch_bounds__(WAVES * 64, (STAGES == 1 ? 2 : 1)) void qgemm_mfma_
             for (int r = 0; r < 16; r++) {
                 const uint32_t row = m0 + wm * (BM / 2) + i * 32 + 8 * (r / 4) + 4 * frag_half + (r % 4);
                 if (row < a.m && col < a.n) {
-                    const size_t o = (size_t)row * a.ys + col;
                     const float v = acc[i][j][r];
+                    if (a.partial) {                        // split-K: fp32 partial, summed by splitk_reduce_kernel
+                        a.partial[((size_t)blockIdx.y * a.m + row) * a.n + col] = v;
+                        continue;
+                    }
+                    const size_t o = (size_t)row * a.ys + col;
                     if (a.y_dtype == MI355Q_F32) ((float*)a.y)[o] = v;
                     else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)a.y)[o] = f32_to_bf16_rne(v);
                     else ((uint16_t*)a.y)[o] = f32_to_f16_rne(v);
@@ -350,10 +359,26 @@ __global__ __launch_bounds__(WAVES * 64, (STAGES == 1 ? 2 : 1)) void qgemm_mfma_
         }
 }
 
+// Sum of the split-K partials in split order (deterministic), one rounding to the output type.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ partial, void* __restrict__ y,
+                                                            uint32_t m, uint32_t n, uint32_t ys, uint32_t splits,
+                                                            uint32_t y_dtype) {
+    const size_t total = (size_t)m * n;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        float v = 0.f;
+        for (uint32_t s = 0; s < splits; s++) v += partial[(size_t)s * total + i];
+        const size_t row = i / n, col = i - row * n;
+        const size_t o = row * ys + col;
+        if (y_dtype == MI355Q_F32) ((float*)y)[o] = v;
+        else if (y_dtype == MI355Q_BF16) ((uint16_t*)y)[o] = f32_to_bf16_rne(v);
+        else ((uint16_t*)y)[o] = f32_to_f16_rne(v);
+    }
+}
+
 // Tile choice.  Problems with at least one 256 x 256 tile per CU take those (eight wavefronts,
 // double-buffered LDS, in-wave software pipeline); smaller ones take 128 x 128 tiles (same
 // pipeline, four wavefronts, two or three workgroups per CU).
-GemmLaunchShape gemm_mfma_shape(const mi355q_context* ctx, uint32_t m, uint32_t n) {
+GemmLaunchShape gemm_mfma_shape(const mi355q_context* ctx, uint32_t m, uint32_t n, uint32_t k) {
     const uint32_t cus = (uint32_t)ctx->props.multiProcessorCount;
     auto tiles = [&](uint32_t bm, uint32_t bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
     GemmLaunchShape g{};
@@ -366,6 +391,20 @@ GemmLaunchShape gemm_mfma_shape(const mi355q_context* ctx, uint32_t m, uint32_t 
     else { g.bm = 128; g.bn = 128; g.stages = 2; }
     g.grid = (tiles(g.bm, g.bn) + 7) / 8 * 8;
     if (!g.block) g.block = 256;
+    // K is split over workgroups when the tiles alone leave most CUs idle (short M): each split writes
+    // an fp32 partial, a second launch adds them.  At least 8 K-tiles per split.
+    g.splits = 1;
+    const uint32_t kt = k / kTileK;
+    if (g.bm == 128 && tiles(128, 128) * 2 <= cus) {
+        uint32_t want = (2 * cus) / tiles(128, 128);
+        if (want > 16) want = 16;
+        while (want > 1 && kt / want < 8) want--;
+        g.splits = want ? want : 1;
+    }
+    const int es = env_int_cached("MI355Q_GEMM_SPLITK", 0);
+    if (es) g.splits = (uint32_t)es;
+    g.kt_per_split = (kt + g.splits - 1) / g.splits;
+    g.splits = (kt + g.kt_per_split - 1) / g.kt_per_split;
     g.lds_bytes = g.stages * (g.bm + g.bn) * (uint32_t)kRowBytes;
     return g;
 }
@@ -385,8 +424,18 @@ mi355q_status launch_tile_sb(hipStream_t s, GemmArgs a) {
         MI355Q_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         lds_limit_raised = true;
     }
-    kern<<<dim3(grid), dim3(WAVES * 64), lds, s>>>(a);
+    const uint32_t kt = a.k / kTileK;
+    const uint32_t splits = a.partial ? (kt + a.kt_per_split - 1) / a.kt_per_split : 1;
+    if (!a.partial) a.kt_per_split = kt;
+    kern<<<dim3(grid, splits), dim3(WAVES * 64), lds, s>>>(a);
     MI355Q_HIP(hipGetLastError());
+    if (a.partial) {
+        const size_t total = (size_t)a.m * a.n;
+        size_t blocks = (total + 255) / 256;
+        if (blocks > 8192) blocks = 8192;
+        splitk_reduce_kernel<<<dim3((unsigned)blocks), dim3(256), 0, s>>>(a.partial, a.y, a.m, a.n, a.ys, splits, a.y_dtype);
+        MI355Q_HIP(hipGetLastError());
+    }
     return MI355Q_OK;
 }
 
@@ -399,8 +448,14 @@ mi355q_status launch_tile(hipStream_t s, const GemmArgs& a) {
 }
 
 template <int BITS, int GROUP, bool QUANT>
-mi355q_status launch_shape(hipStream_t s, const mi355q_context* ctx, const GemmArgs& a) {
-    const GemmLaunchShape g = gemm_mfma_shape(ctx, a.m, a.n);
+mi355q_status launch_shape(hipStream_t s, mi355q_context* ctx, GemmArgs a) {
+    const GemmLaunchShape g = gemm_mfma_shape(ctx, a.m, a.n, a.k);
+    if (g.splits > 1) {
+        const size_t need = (size_t)g.splits * a.m * a.n * sizeof(float);
+        if (mi355q_status st = ensure_workspace(ctx, need)) return st;
+        a.partial = (float*)ctx->workspace;
+        a.kt_per_split = g.kt_per_split;
+    }
     if (g.bm == 256 && g.bn == 256 && g.block == 512) return launch_tile<BITS, GROUP, 256, 256, QUANT, 2, 8>(s, a);
 #ifdef MI355Q_GEMV_EXPERIMENT
     // tuning builds: the other tile shapes, selected with MI355Q_GEMM_TILE
@@ -426,7 +481,7 @@ bool gemm_mfma_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stri
     return fmt_ok;
 }
 
-mi355q_status launch_qgemm_mfma(hipStream_t s, const mi355q_context* ctx, const WView& w, const void* x, int x_dtype,
+mi355q_status launch_qgemm_mfma(hipStream_t s, mi355q_context* ctx, const WView& w, const void* x, int x_dtype,
                                 void* y, int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride) {
     if (x_dtype != MI355Q_BF16) return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the MFMA GEMM takes bf16 activations");
     if ((uintptr_t)x % 16) return fail(MI355Q_ERR_INVALID_ARGUMENT, "activation pointer must be 16-byte aligned");
@@ -450,7 +505,7 @@ mi355q_status launch_qgemm_mfma(hipStream_t s, const mi355q_context* ctx, const 
     return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no MFMA GEMM for q%u g%u", w.bits, w.group);
 }
 
-mi355q_status launch_gemm_bf16_mfma(hipStream_t s, const mi355q_context* ctx, const void* a_ptr, int a_dtype,
+mi355q_status launch_gemm_bf16_mfma(hipStream_t s, mi355q_context* ctx, const void* a_ptr, int a_dtype,
                                     const uint16_t* b, void* c, int c_dtype, uint32_t m, uint32_t n, uint32_t k,
                                     uint32_t a_stride, uint32_t c_stride) {
     if (a_dtype != MI355Q_BF16) return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the MFMA GEMM takes bf16 activations");

@@ -143,9 +143,10 @@ mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w, uint32_t maximum
         std::snprintf(s->device_kernel, sizeof s->device_kernel, "qgemm_mfma_q%u_g%u", (unsigned)w->fmt.bits,
                       w->fmt.group_size);
         std::snprintf(s->kernel_family, sizeof s->kernel_family, "mfmaGEMM");
-        const GemmLaunchShape g = gemm_mfma_shape(w->ctx, m, (uint32_t)w->n);
+        const GemmLaunchShape g = gemm_mfma_shape(w->ctx, m, (uint32_t)w->n, (uint32_t)w->k);
         s->block[0] = g.block;
         s->grid[0] = g.grid;
+        s->grid[1] = g.splits;
         s->lds_bytes = g.lds_bytes;
         s->rows_per_workgroup = g.bn;
         return MI355Q_OK;

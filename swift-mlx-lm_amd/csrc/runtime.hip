@@ -6,6 +6,23 @@
 
 using namespace mi355q;
 
+namespace mi355q {
+
+mi355q_status ensure_workspace(mi355q_context* ctx, size_t bytes) {
+    if (bytes <= ctx->workspace_bytes) return MI355Q_OK;
+    // launches that still read the old buffer must drain before it is released
+    MI355Q_HIP(hipDeviceSynchronize());
+    if (ctx->workspace) (void)hipFree(ctx->workspace);
+    ctx->workspace = nullptr;
+    ctx->workspace_bytes = 0;
+    const size_t rounded = (bytes + ((size_t)1 << 22) - 1) & ~(((size_t)1 << 22) - 1);
+    MI355Q_HIP(hipMalloc(&ctx->workspace, rounded));
+    ctx->workspace_bytes = rounded;
+    return MI355Q_OK;
+}
+
+}  // namespace mi355q
+
 namespace {
 
 // ---- host float16 <-> float32 (round-to-nearest-even), used only while preparing weights ----
@@ -213,6 +230,7 @@ mi355q_status mi355q_context_destroy(mi355q_context* ctx) {
     (void)hipSetDevice(ctx->device);
     (void)hipDeviceSynchronize();
     if (ctx->argmax_scratch) (void)hipFree(ctx->argmax_scratch);
+    if (ctx->workspace) (void)hipFree(ctx->workspace);
     delete ctx;
     return MI355Q_OK;
 }
