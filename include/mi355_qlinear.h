@@ -274,6 +274,20 @@ MI355Q_API mi355q_status mi355q_gemm_bf16(mi355q_context* ctx, void* stream, con
                                           uint32_t n, uint32_t k, uint32_t a_row_stride,
                                           uint32_t c_row_stride);
 
+/* Quantized embedding gather: embedding_lookup[_seq]_q{b}_g{g}
+ * (MC/Generator/MetalSourceGenerator+Embedding.swift:79-153 for q4, :229-322 for every format; bindings
+ * 0=tokenIDs 1=table 2=output 3=embeddingDim 4=sequenceLength 5=embeddingScale).  `table` is a packed
+ * weight of shape [vocabularySize, embeddingDim] in any layout (a tied LM head can be passed as is);
+ * token ids are int32 in device memory; out[pos*out_row_stride + d] = (float(q)*scale + zero)
+ * [* embedding_scale], rounded once to out_dtype.  sequence_length 1 is the decode variant.  A token
+ * id outside the table gives a row of zeros (the reference reads out of bounds). */
+MI355Q_API mi355q_status mi355q_embedding_lookup(mi355q_context* ctx, void* stream,
+                                                 const mi355q_weight* table,
+                                                 const int32_t* token_ids_dev,
+                                                 uint32_t sequence_length, void* out_dev,
+                                                 mi355q_dtype out_dtype, uint32_t out_row_stride,
+                                                 int has_embedding_scale, float embedding_scale);
+
 /* Debug / parity: every code of the matrix as one byte, row-major [N, K]. */
 MI355Q_API mi355q_status mi355q_unpack_codes(mi355q_context* ctx, void* stream,
                                              const mi355q_weight* w, uint8_t* out_codes_dev);

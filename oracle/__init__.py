@@ -58,6 +58,7 @@ def lib():
         L.orc_dequant_staf_f32.argtypes = [i32, i32, sz, sz, vp, vp]
         L.orc_dequant_planes_f32.argtypes = [i32, i32, sz, sz, vp, vp, vp, i32, vp]
         L.orc_dequant_staf_bf16.argtypes = [i32, i32, sz, sz, vp, vp]
+        L.orc_embedding_lookup_staf_f32.argtypes = [i32, i32, sz, sz, vp, vp, sz, i32, C.c_float, vp]
         L.orc_gemm_f64.argtypes = [vp, vp, sz, sz, sz, sz, vp]; L.orc_gemm_f64.restype = None
         L.orc_qgemm_staf_ref_f32.argtypes = [i32, i32, vp, vp, sz, sz, sz, sz, vp, i32]
         L.orc_qgemm_planes_ref_f32.argtypes = [i32, i32, vp, vp, vp, i32, vp, sz, sz, sz, sz, vp, i32]
@@ -200,6 +201,17 @@ def dequant_staf_bf16(bits, group, n, k, blocks) -> np.ndarray:
 
 
 # --------------------------------------------------------------------- gemm
+def embedding_lookup_staf_f32(bits, group, vocab, dim, table, token_ids, embedding_scale=None) -> np.ndarray:
+    table = _c(table, np.uint8)
+    ids = _c(token_ids, np.int32)
+    out = np.zeros((ids.size, dim), dtype=np.float32)
+    _check(lib().orc_embedding_lookup_staf_f32(bits, group, vocab, dim, _p(table), _p(ids), ids.size,
+                                               0 if embedding_scale is None else 1,
+                                               0.0 if embedding_scale is None else float(embedding_scale), _p(out)),
+           "embedding_lookup_staf_f32")
+    return out
+
+
 def gemm_f64(w, x, x_stride=None) -> np.ndarray:
     """fp64 accumulation of fp32 weights w [N,K] against x [M, x_stride>=K] -> y [M,N] float64."""
     w = _c(w, np.float32); x = _c(x, np.float32)

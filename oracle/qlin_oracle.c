@@ -342,6 +342,34 @@ int orc_dequant_staf_bf16(int bits, int group, size_t n_rows, size_t k, const ui
     return rc;
 }
 
+/* ------------------------------------------------------------------ embedding */
+
+int orc_embedding_lookup_staf_f32(int bits, int group, size_t vocab, size_t dim, const uint8_t* table,
+                                  const int32_t* token_ids, size_t sequence_length, int has_scale,
+                                  float embedding_scale, float* out) {
+    orc_format f;
+    if (orc_format_for_mlx(bits, group, &f)) return -1;
+    if (dim % (size_t)group) return -2;
+    size_t blocks_per_row = dim / (size_t)group;
+    for (size_t pos = 0; pos < sequence_length; pos++) {
+        int32_t tok = token_ids[pos];
+        if (tok < 0 || (size_t)tok >= vocab) return -3; /* the reference reads out of bounds here */
+        const uint8_t* row = table + (size_t)tok * blocks_per_row * (size_t)f.bytes_per_block;
+        for (size_t d = 0; d < dim; d++) {
+            const uint8_t* blk = row + (d / (size_t)group) * (size_t)f.bytes_per_block;
+            uint16_t sb, zb;
+            memcpy(&sb, blk, 2);
+            memcpy(&zb, blk + 2, 2);
+            float q = (float)orc_unpack_code(blk + 4, (int)(d % (size_t)group), bits);
+            float prod = q * orc_f16_to_f32(sb); /* quantized * blockScale + blockZero */
+            float value = prod + orc_f16_to_f32(zb);
+            if (has_scale) value = value * embedding_scale;
+            out[pos * dim + d] = value;
+        }
+    }
+    return 0;
+}
+
 /* ---------------------------------------------------------------------- gemm */
 
 void orc_gemm_f64(const float* w, const float* x, size_t m, size_t n, size_t k, size_t x_stride,

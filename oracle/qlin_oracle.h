@@ -76,6 +76,15 @@ int orc_unpack_staf_codes(int bits, int group, size_t n_rows, size_t k, const ui
 int orc_unpack_plane_codes(int bits, size_t n_rows, size_t k, const uint32_t* codes,
                            uint8_t* out_codes);
 
+/* Quantized embedding gather (Sources/MetalCompiler/Generator/MetalSourceGenerator+Embedding.swift:79-153
+ * for q4, :229-322 for every format): out[pos, d] = (float(q) * scale + zero) [* embeddingScale] of row
+ * token_ids[pos], fp32, unfused.  Pinned by the reference's own vectors
+ * (Tests/MetalCompilerTests/Core/QuantizedEmbeddingKernelTests.swift:48-150, 229-270).  Returns -3 for a
+ * token id outside the table (the reference has no check). */
+int orc_embedding_lookup_staf_f32(int bits, int group, size_t vocab, size_t dim, const uint8_t* table,
+                                  const int32_t* token_ids, size_t sequence_length, int has_scale,
+                                  float embedding_scale, float* out);
+
 /* Sources/SwiftLM/CPUWeightStore.swift:141-172: w = scale*float(q) + zero, fp32, unfused. */
 int orc_dequant_staf_f32(int bits, int group, size_t n_rows, size_t k, const uint8_t* blocks,
                          float* out);

@@ -127,6 +127,7 @@ def library() -> C.CDLL:
         "mi355q_gemm_bf16": (i32, [vp, vp, vp, C.c_int, vp, vp, C.c_int, u32, u32, u32, u32, u32]),
         "mi355q_unpack_codes": (i32, [vp, vp, vp, vp]),
         "mi355q_argmax": (i32, [vp, vp, vp, C.c_int, u32, vp]),
+        "mi355q_embedding_lookup": (i32, [vp, vp, vp, vp, u32, vp, C.c_int, u32, C.c_int, C.c_float]),
         "mi355q_lmhead_argmax": (i32, [vp, vp, vp, vp, C.c_int, vp, vp, u32]),
         "mi355q_shape_family_resolve": (i32, [u32, u32, P(i32), P(u32), P(u32), C.c_char_p, sz]),
         "mi355q_plan_create": (i32, [vp, P(vp)]),
@@ -544,6 +545,14 @@ class Context:
     def gemm_bf16(self, a, a_dtype, b_bf16, c, c_dtype, m, n, k, a_row_stride=0, c_row_stride=0, stream=0):
         _check(library().mi355q_gemm_bf16(self.handle, stream, self._ptr(a), a_dtype, self._ptr(b_bf16),
                                           self._ptr(c), c_dtype, m, n, k, a_row_stride, c_row_stride))
+
+    def embedding_lookup(self, table: PackedWeight, token_ids, sequence_length, out, out_dtype, out_row_stride=0,
+                         embedding_scale=None, stream=0):
+        """Gather dequantised rows of a packed [vocabulary, embeddingDim] table (GatherFragment)."""
+        _check(library().mi355q_embedding_lookup(self.handle, stream, table.handle, self._ptr(token_ids),
+                                                 sequence_length, self._ptr(out), out_dtype, out_row_stride,
+                                                 0 if embedding_scale is None else 1,
+                                                 0.0 if embedding_scale is None else float(embedding_scale)))
 
     def unpack_codes(self, w: PackedWeight, out, stream=0):
         _check(library().mi355q_unpack_codes(self.handle, stream, w.handle, self._ptr(out)))

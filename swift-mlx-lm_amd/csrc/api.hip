@@ -222,6 +222,23 @@ mi355q_status mi355q_gemm_bf16(mi355q_context* ctx, void* stream, const void* a_
                                  c_dtype, m, n, k, a_row_stride, c_row_stride);
 }
 
+mi355q_status mi355q_embedding_lookup(mi355q_context* ctx, void* stream, const mi355q_weight* table,
+                                      const int32_t* token_ids_dev, uint32_t sequence_length, void* out_dev,
+                                      mi355q_dtype out_dtype, uint32_t out_row_stride, int has_embedding_scale,
+                                      float embedding_scale) {
+    if (mi355q_status s = check_launch(ctx, table)) return s;
+    if (!token_ids_dev || !out_dev) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null token or output pointer");
+    if (!dtype_ok(out_dtype)) return fail(MI355Q_ERR_INVALID_ARGUMENT, "bad dtype tag");
+    if (sequence_length == 0) return fail(MI355Q_ERR_INVALID_ARGUMENT, "sequence length must be >= 1");
+    if (sequence_length > 65535) return fail(MI355Q_ERR_SHAPE, "sequence length %u exceeds 65535", sequence_length);
+    if (out_row_stride == 0) out_row_stride = (uint32_t)table->k;
+    if (out_row_stride < table->k) return fail(MI355Q_ERR_SHAPE, "output row stride smaller than embeddingDim");
+    if ((uintptr_t)token_ids_dev % 4 || (uintptr_t)out_dev % (out_dtype == MI355Q_F32 ? 4 : 2))
+        return fail(MI355Q_ERR_INVALID_ARGUMENT, "misaligned pointer");
+    return launch_embedding_lookup((hipStream_t)stream, table->view(), token_ids_dev, sequence_length, out_dev, out_dtype,
+                                   out_row_stride, has_embedding_scale, embedding_scale);
+}
+
 mi355q_status mi355q_unpack_codes(mi355q_context* ctx, void* stream, const mi355q_weight* w,
                                   uint8_t* out_codes_dev) {
     if (mi355q_status s = check_launch(ctx, w)) return s;

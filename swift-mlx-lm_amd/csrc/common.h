@@ -112,6 +112,9 @@ mi355q_status launch_dequant_bf16(hipStream_t s, const WView& w, uint16_t* out);
 mi355q_status launch_gemv_generic(hipStream_t s, const WView& w, const void* x, int x_dtype,
                                   void* y, int y_dtype, uint32_t m, uint32_t x_stride,
                                   uint32_t y_stride);
+mi355q_status launch_embedding_lookup(hipStream_t s, const WView& w, const int32_t* token_ids, uint32_t sequence_length,
+                                      void* out, int out_dtype, uint32_t out_stride, int has_scale,
+                                      float embedding_scale);
 mi355q_status launch_argmax(hipStream_t s, const void* logits, int dtype, uint32_t n,
                             int32_t* token_out);
 mi355q_status launch_pack_sz(hipStream_t s, const uint16_t* scales, const uint16_t* biases, uint32_t* sz,

@@ -96,6 +96,49 @@ mi355q_status launch_tile16_pack(hipStream_t s, const WView& planes, uint32_t* t
     return MI355Q_OK;
 }
 
+// --------------------------------------------------------------------------- embedding lookup
+// out[pos, d] = (float(q) * scale + zero) [* embeddingScale] of table row token_ids[pos], rounded once to
+// the output type: embedding_lookup[_seq]_q{b}_g{g} of the reference
+// (Sources/MetalCompiler/Generator/MetalSourceGenerator+Embedding.swift:79-153, 229-322).  Any layout and
+// bit width; the two roundings (product, sum) are kept apart so the fp32 result is bit-identical to an
+// unfused host evaluation.  A token id outside the table yields a row of zeros (the reference reads out
+// of bounds there).
+__global__ __launch_bounds__(256) void embedding_lookup_kernel(WView w, const int32_t* __restrict__ token_ids,
+                                                               uint32_t sequence_length, void* __restrict__ out,
+                                                               uint32_t out_dtype, uint32_t out_stride, int has_scale,
+                                                               float embedding_scale) {
+    const uint32_t pos = blockIdx.y;
+    if (pos >= sequence_length) return;
+    const int32_t tok = token_ids[pos];
+    const bool valid = tok >= 0 && (uint32_t)tok < w.n;
+    for (uint32_t d = blockIdx.x * 256u + threadIdx.x; d < w.k; d += gridDim.x * 256u) {
+        float v = 0.0f;
+        if (valid) {
+            float scale, zero;
+            load_scale_zero(w, (uint32_t)tok, d / w.group, scale, zero);
+            const float q = (float)load_code(w, (uint32_t)tok, d);
+            v = __fadd_rn(__fmul_rn(q, scale), zero);
+            if (has_scale) v = __fmul_rn(v, embedding_scale);
+        }
+        const size_t o = (size_t)pos * out_stride + d;
+        if (out_dtype == MI355Q_F32) ((float*)out)[o] = v;
+        else if (out_dtype == MI355Q_BF16) ((uint16_t*)out)[o] = f32_to_bf16_rne(v);
+        else ((uint16_t*)out)[o] = f32_to_f16_rne(v);
+    }
+}
+
+mi355q_status launch_embedding_lookup(hipStream_t s, const WView& w, const int32_t* token_ids, uint32_t sequence_length,
+                                      void* out, int out_dtype, uint32_t out_stride, int has_scale,
+                                      float embedding_scale) {
+    uint32_t gx = (w.k + 255u) / 256u;
+    if (gx > 64u) gx = 64u;
+    embedding_lookup_kernel<<<dim3(gx, sequence_length), dim3(256), 0, s>>>(w, token_ids, sequence_length, out,
+                                                                           (uint32_t)out_dtype, out_stride, has_scale,
+                                                                           embedding_scale);
+    MI355Q_HIP(hipGetLastError());
+    return MI355Q_OK;
+}
+
 // ------------------------------------------------------------------------------ dequant bf16
 // One workgroup per row, 256 threads striding over the row, as the reference kernel does.
 // scale*q and +zero are kept as two roundings so the result is bit-identical to an unfused

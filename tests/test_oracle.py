@@ -363,3 +363,50 @@ def test_quantizer_formula_on_a_hand_group():
     # constant group: scale floors at 1e-10, codes all zero
     codes, s, z = oracle.quantize_affine(np.full((1, 64), 0.25, np.float32), 4, 64, oracle.F32)
     assert s[0, 0] == np.float32(1e-10) and not codes.any()
+
+
+# ------------------------------------------------------------------ quantized embedding gather (N1)
+def _q3_embedding_rows(v):
+    dim, group, rows = v["dim"], v["group"], v["rows"]
+    codes = np.array([[(i + 3 * g + 5 * t) % 8 for g in range(dim // group) for i in range(group)]
+                      for t in range(rows)], np.uint8)
+    s = np.array([[0.03125 * (g + 1) + 0.0078125 * t for g in range(dim // group)] for t in range(rows)])
+    z = np.array([[-0.125 + 0.0625 * t - 0.015625 * g for g in range(dim // group)] for t in range(rows)])
+    return codes, s, z
+
+
+def test_embedding_lookup_reference_vectors():
+    v = KATS["embedding_q4_row_of_twos"]
+    codes = np.array([[t] * v["dim"] for t in v["row_values"]], np.uint8)
+    blocks = kat.staf_blocks(codes, np.ones((2, 1)), np.zeros((2, 1)), 4, 64)
+    out = oracle.embedding_lookup_staf_f32(4, 64, 2, v["dim"], blocks, [v["token"]])
+    assert out.shape == (1, 64) and np.all(np.abs(out - v["expected"]) < 0.001)
+    out = oracle.embedding_lookup_staf_f32(4, 64, 2, v["dim"], blocks, [v["token"]], v["scale"])
+    assert np.all(np.abs(out - v["expected_scaled"]) < 0.001)
+
+    v = KATS["embedding_q3_sequence"]
+    codes, s, z = _q3_embedding_rows(v)
+    blocks = kat.staf_blocks(codes, s, z, 3, 64)
+    out = oracle.embedding_lookup_staf_f32(3, 64, v["rows"], v["dim"], blocks, v["tokens"])
+    for pos, t in enumerate(v["tokens"]):
+        want = (s[t].repeat(64).astype(np.float32) * codes[t].astype(np.float32) + z[t].repeat(64).astype(np.float32))
+        assert np.max(np.abs(out[pos] - want)) < v["bar"]                  # the reference's own bar
+
+
+def test_embedding_lookup_is_a_row_gather_of_the_dequantised_table():
+    """Independent of the gather loop: every output row equals the corresponding row of the CPU dequant
+    (itself pinned by the CPUWeightStore vector), times the scale; an id outside the table is an error."""
+    rng = np.random.default_rng(21)
+    for bits, group in [(4, 64), (8, 32), (3, 64), (6, 16), (2, 32), (5, 32)]:
+        vocab, dim = 37, group * 6
+        codes = rng.integers(0, 1 << bits, (vocab, dim), dtype=np.uint8)
+        s = rng.uniform(0.01, 0.1, (vocab, dim // group)); z = rng.uniform(-0.5, 0.5, (vocab, dim // group))
+        blocks = kat.staf_blocks(codes, s, z, bits, group)
+        table = oracle.dequant_staf_f32(bits, group, vocab, dim, blocks)
+        ids = rng.integers(0, vocab, 11)
+        assert np.array_equal(oracle.embedding_lookup_staf_f32(bits, group, vocab, dim, blocks, ids), table[ids])
+        scaled = oracle.embedding_lookup_staf_f32(bits, group, vocab, dim, blocks, ids, 1.75)
+        assert np.array_equal(scaled, table[ids] * np.float32(1.75))
+    with pytest.raises(ValueError):
+        oracle.embedding_lookup_staf_f32(4, 64, 2, 64, kat.staf_blocks(np.zeros((2, 64), np.uint8), np.ones((2, 1)),
+                                                                        np.zeros((2, 1)), 4, 64), [2])
