@@ -24,6 +24,14 @@
 
 #include "device_utils.h"
 
+// Weights are read exactly once per launch: non-temporal loads keep them from displacing the
+// activations and each other in the caches.
+#ifdef MI355Q_GEMV_NO_NT
+#define MI355Q_STREAM_LOAD(p) (*(p))
+#else
+#define MI355Q_STREAM_LOAD(p) __builtin_nontemporal_load(p)
+#endif
+
 namespace mi355q {
 
 constexpr int kGemvMaxSegments = 3;
@@ -157,18 +165,18 @@ void gemv_planes_kernel(GemvArgs a) {
             const uint32_t* rowp = seg_codes + (size_t)row * a.code_stride;    // scalar
             const uint32_t* szp = seg_sz + (size_t)row * a.sz_stride;          // scalar
             if constexpr (WPL == 4) {
-                const u32x4 v = *(const u32x4*)(rowp + code_off);
+                const u32x4 v = MI355Q_STREAM_LOAD((const u32x4*)(rowp + code_off));
                 p.w[r][0] = v.x; p.w[r][1] = v.y; p.w[r][2] = v.z; p.w[r][3] = v.w;
             } else {
 #pragma unroll
-                for (int i = 0; i < WPL; i++) p.w[r][i] = rowp[code_off + i];
+                for (int i = 0; i < WPL; i++) p.w[r][i] = MI355Q_STREAM_LOAD(rowp + code_off + i);
             }
 #pragma unroll
             for (int sr = 0; sr < NSR; sr++) {
 #ifdef MI355Q_GEMV_EXPERIMENT
                 if (a.dbg & 1) { p.sz[r][sr] = 0x38003C00u; continue; }
 #endif
-                p.sz[r][sr] = szp[sz_off[sr]];
+                p.sz[r][sr] = MI355Q_STREAM_LOAD(szp + sz_off[sr]);
             }
         }
     };
