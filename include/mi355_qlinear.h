@@ -51,8 +51,11 @@ enum {
     MI355Q_ERR_DEVICE = -5,             /* MetalCompilerError.deviceSetupFailed */
     MI355Q_ERR_OUT_OF_MEMORY = -6,
     MI355Q_ERR_KERNEL_NOT_FOUND = -7,   /* MetalCompilerError.kernelNotFound */
-    MI355Q_ERR_SIZE_MISMATCH = -8       /* payload size != rows*blocksPerRow*bytesPerBlock
+    MI355Q_ERR_SIZE_MISMATCH = -8,      /* payload size != rows*blocksPerRow*bytesPerBlock
                                            (Sources/SwiftLM/CPUWeightStore.swift:133-138) */
+    MI355Q_ERR_INVALID_FILE = -9,       /* STAFLoadError.invalidFile (MC/STAF/STAFLoader.swift:318-330) */
+    MI355Q_ERR_IO = -10,                /* STAFLoadError.mmapFailed, file system errors */
+    MI355Q_ERR_NOT_FOUND = -11          /* entries[name] == nil */
 };
 
 /* BufferPrecision (MC/MetalDispatchTypes.swift:13-37) */
@@ -437,6 +440,87 @@ MI355Q_API mi355q_status mi355q_plan_graph_launch(mi355q_plan* plan, void* strea
  * traffic counters).  Both pointers 16-byte aligned, bytes a multiple of 16. */
 MI355Q_API mi355q_status mi355q_buffer_copy(mi355q_context* ctx, void* stream, void* dst_dev,
                                             const void* src_dev, size_t bytes);
+
+/* ------------------------------------------------------------------------------------------
+ * STAF container (model.staf): reader, validator, writer
+ * ---------------------------------------------------------------------------------------- */
+/* STAFLoader.load (MC/STAF/STAFLoader.swift:19-198): maps the file read-only and parses header, section
+ * table, string table and metadata table (MC/STAF/STAFFormat.swift:10-80, 84-167).  Rejects what the
+ * reference rejects (missing or <= 64-byte file, bad magic, a format version other than 0 or 2, a payload
+ * that leaves the file, malformed metadata, no tensors) with MI355Q_ERR_INVALID_FILE, and also tables
+ * that leave the file, which the reference reads unchecked. */
+typedef struct mi355q_staf mi355q_staf;
+/* STAFSectionEntry / STAFTensorEntry (STAFFormat.swift:132-167, STAFLoader.swift:299-311).  `name` points
+ * into the mapping: name_length bytes of UTF-8, valid until mi355q_staf_close. */
+typedef struct mi355q_staf_entry {
+    const char* name;
+    uint32_t name_length;
+    uint8_t scheme_identifier, semantic_role, original_dtype, dimension_count;
+    uint32_t shape[8];
+    uint64_t payload_offset;   /* from the start of the file */
+    uint64_t payload_size;
+    uint64_t buffer_offset;    /* STAFTensorEntry.bufferOffset: from the start of the payload region */
+    uint32_t alignment, block_size, group_size, checksum, shard_index;
+} mi355q_staf_entry;
+/* STAFMetadataValueType (MC/STAF/STAFMetadataValue.swift:12-19) */
+enum { MI355Q_STAF_BOOL = 1, MI355Q_STAF_UINT32 = 2, MI355Q_STAF_UINT64 = 3, MI355Q_STAF_FLOAT32 = 4,
+       MI355Q_STAF_FLOAT64 = 5, MI355Q_STAF_STRING = 6 };
+/* One file-level metadata value (STAFMetadataValue).  payload0 holds the bool, the integer or the bit
+ * pattern of the float; strings are text[0, text_length). */
+typedef struct mi355q_staf_metadata {
+    const char* key;
+    uint8_t type;
+    uint64_t payload0;
+    const char* text;
+    uint32_t text_length;
+} mi355q_staf_metadata;
+/* One tensor handed to the writer (STAFConversionEntry + its converted payload). */
+typedef struct mi355q_staf_tensor {
+    const char* name;
+    uint8_t scheme_identifier, semantic_role, original_dtype;
+    uint32_t dimension_count;
+    uint32_t shape[8];         /* packed tensors: the MLX shape [N, K*bits/32] */
+    const void* payload;
+    uint64_t payload_size;
+    uint32_t shard_index;
+} mi355q_staf_tensor;
+
+MI355Q_API mi355q_status mi355q_staf_open(const char* path, mi355q_staf** out);
+MI355Q_API void mi355q_staf_close(mi355q_staf* staf);
+MI355Q_API uint32_t mi355q_staf_format_version(const mi355q_staf* staf);
+MI355Q_API uint32_t mi355q_staf_tensor_count(const mi355q_staf* staf);
+MI355Q_API mi355q_status mi355q_staf_tensor_at(const mi355q_staf* staf, uint32_t index, mi355q_staf_entry* out);
+/* STAFWeightStore.entries[name]; MI355Q_ERR_NOT_FOUND when absent. */
+MI355Q_API mi355q_status mi355q_staf_find(const mi355q_staf* staf, const char* name, mi355q_staf_entry* out);
+/* The payload region in host memory: first tensor to end of file, the span of the single MTLBuffer
+ * (STAFLoader.swift:160-197). */
+MI355Q_API const void* mi355q_staf_payload_region(const mi355q_staf* staf, uint64_t* bytes);
+MI355Q_API uint32_t mi355q_staf_metadata_count(const mi355q_staf* staf);
+MI355Q_API mi355q_status mi355q_staf_metadata_at(const mi355q_staf* staf, uint32_t index,
+                                                 mi355q_staf_metadata* out);
+/* STAFValidator.isValid (MC/STAF/STAFValidator.swift:5-78): format version 2, section table right after
+ * the header, metadata table in bounds, every expected value present and equal, no source file newer than
+ * the container.  *valid = 1 or 0; an unreadable path is MI355Q_ERR_IO (the reference throws). */
+MI355Q_API mi355q_status mi355q_staf_is_valid(const char* staf_path, const char* const* source_paths,
+                                              uint32_t source_count, const mi355q_staf_metadata* expected,
+                                              uint32_t expected_count, int32_t* valid);
+/* STAFWriter.write (MC/STAF/STAFWriter.swift:11-269) for payloads that are already converted: header,
+ * section table, metadata table sorted by key, de-duplicated string table, payload region from the next
+ * 4096-byte boundary with every tensor on a 256-byte one.  A payload whose size is not what its shape and
+ * scheme imply (computePayloadSize, :240-262) is MI355Q_ERR_SIZE_MISMATCH. */
+MI355Q_API mi355q_status mi355q_staf_write(const char* path, const mi355q_staf_tensor* tensors,
+                                           uint32_t tensor_count, const mi355q_staf_metadata* metadata,
+                                           uint32_t metadata_count);
+/* The single device buffer of STAFWeightStore: copies the payload region to device memory (one
+ * allocation, released with mi355q_buffer_free).  Tensor `t` then lives at *base_dev_out + t.buffer_offset. */
+MI355Q_API mi355q_status mi355q_staf_upload(mi355q_context* ctx, const mi355q_staf* staf, void** base_dev_out,
+                                            uint64_t* bytes_out);
+/* resolvedBufferAccess for one packed 2-D tensor (STAFLoader.swift:213-299): MI355Q_LAYOUT_STAF_BLOCKS
+ * borrows the bytes inside the uploaded region (zero copy); MI355Q_LAYOUT_PLANES / _TILE16 build this
+ * library's specialized copy from the mapping, as STAFSpecializedWeightStoreBuilder does
+ * (MC/STAF/STAFSpecializedWeightStoreBuilder.swift:15-31).  N = shape[0], K = shape[1] * 32 / bits. */
+MI355Q_API mi355q_status mi355q_staf_weight(mi355q_context* ctx, const mi355q_staf* staf, const void* base_dev,
+                                            const char* name, mi355q_layout layout, mi355q_weight** out);
 
 #ifdef __cplusplus
 }

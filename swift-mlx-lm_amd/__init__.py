@@ -24,7 +24,8 @@ LAYOUT_STAF_BLOCKS, LAYOUT_PLANES, LAYOUT_TILE16 = 0, 1, 2
 FLAG_NONE, FLAG_FORCE_GENERIC, FLAG_FORCE_SMALL_M, FLAG_FORCE_MFMA = 0, 1, 2, 4
 
 STATUS_NAMES = {0: "OK", -1: "INVALID_ARGUMENT", -2: "UNSUPPORTED_FORMAT", -3: "SHAPE", -4: "NULL_HANDLE",
-                -5: "DEVICE", -6: "OUT_OF_MEMORY", -7: "KERNEL_NOT_FOUND", -8: "SIZE_MISMATCH"}
+                -5: "DEVICE", -6: "OUT_OF_MEMORY", -7: "KERNEL_NOT_FOUND", -8: "SIZE_MISMATCH",
+                -9: "INVALID_FILE", -10: "IO", -11: "NOT_FOUND"}
 FALLBACK_NAMES = {0: None, 1: "inputStrideMismatch", 2: "lastTokenProjectionUsesDecodeKernel",
                   3: "disabledByEnvironment", 4: "unavailableAcceleration"}
 PATH_NAMES = {0: "prefillProjection", 1: "decodeProjection"}
@@ -48,6 +49,25 @@ class _Format(C.Structure):
                 ("block_struct_name", C.c_char * 32), ("gemv_kernel_name", C.c_char * 32),
                 ("gemm_kernel_name_f32s", C.c_char * 32), ("gemm_kernel_name", C.c_char * 32),
                 ("dequant_to_bfloat_kernel_name", C.c_char * 32), ("embedding_lookup_token", C.c_char * 16)]
+
+
+class _StafEntry(C.Structure):
+    _fields_ = [("name", C.c_void_p), ("name_length", C.c_uint32), ("scheme_identifier", C.c_uint8),
+                ("semantic_role", C.c_uint8), ("original_dtype", C.c_uint8), ("dimension_count", C.c_uint8),
+                ("shape", C.c_uint32 * 8), ("payload_offset", C.c_uint64), ("payload_size", C.c_uint64),
+                ("buffer_offset", C.c_uint64), ("alignment", C.c_uint32), ("block_size", C.c_uint32),
+                ("group_size", C.c_uint32), ("checksum", C.c_uint32), ("shard_index", C.c_uint32)]
+
+
+class _StafMetadata(C.Structure):
+    _fields_ = [("key", C.c_char_p), ("type", C.c_uint8), ("payload0", C.c_uint64), ("text", C.c_void_p),
+                ("text_length", C.c_uint32)]
+
+
+class _StafTensor(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("scheme_identifier", C.c_uint8), ("semantic_role", C.c_uint8),
+                ("original_dtype", C.c_uint8), ("dimension_count", C.c_uint32), ("shape", C.c_uint32 * 8),
+                ("payload", C.c_void_p), ("payload_size", C.c_uint64), ("shard_index", C.c_uint32)]
 
 
 class _DeviceInfo(C.Structure):
@@ -142,6 +162,19 @@ def library() -> C.CDLL:
         "mi355q_plan_graph_build": (i32, [vp, vp]),
         "mi355q_plan_graph_launch": (i32, [vp, vp]),
         "mi355q_buffer_copy": (i32, [vp, vp, vp, vp, sz]),
+        "mi355q_staf_open": (i32, [C.c_char_p, P(vp)]),
+        "mi355q_staf_close": (None, [vp]),
+        "mi355q_staf_format_version": (u32, [vp]),
+        "mi355q_staf_tensor_count": (u32, [vp]),
+        "mi355q_staf_tensor_at": (i32, [vp, u32, P(_StafEntry)]),
+        "mi355q_staf_find": (i32, [vp, C.c_char_p, P(_StafEntry)]),
+        "mi355q_staf_payload_region": (vp, [vp, P(u64)]),
+        "mi355q_staf_metadata_count": (u32, [vp]),
+        "mi355q_staf_metadata_at": (i32, [vp, u32, P(_StafMetadata)]),
+        "mi355q_staf_is_valid": (i32, [C.c_char_p, P(C.c_char_p), u32, P(_StafMetadata), u32, P(i32)]),
+        "mi355q_staf_write": (i32, [C.c_char_p, P(_StafTensor), u32, P(_StafMetadata), u32]),
+        "mi355q_staf_upload": (i32, [vp, vp, P(vp), P(u64)]),
+        "mi355q_staf_weight": (i32, [vp, vp, vp, C.c_char_p, C.c_int, P(vp)]),
         "mi355q_plan_decode_step": (i32, [vp, u32, C.c_int, u32, P(_Step)]),
         "mi355q_plan_prefill_steps": (i32, [vp, u32, u32, C.c_int, C.c_int, u32, P(_Step), P(u32)]),
     }
@@ -403,6 +436,165 @@ class DispatchPlan:
         if self.handle:
             _check(library().mi355q_plan_destroy(self.handle))
             self.handle = 0
+
+
+
+# --------------------------------------------------------------------------------- STAF container
+# STAFMetadataValueType
+STAF_BOOL, STAF_UINT32, STAF_UINT64, STAF_FLOAT32, STAF_FLOAT64, STAF_STRING = 1, 2, 3, 4, 5, 6
+
+
+@dataclass(frozen=True)
+class STAFTensorEntry:
+    """STAFTensorEntry (MC/STAF/STAFLoader.swift:299-311)."""
+    name: str
+    payload_offset: int
+    payload_size: int
+    scheme_identifier: int
+    semantic_role: int
+    original_dtype: int
+    shape: tuple
+    block_size: int
+    group_size: int
+    buffer_offset: int
+    alignment: int
+    checksum: int
+    shard_index: int
+
+
+def _entry_from_c(e: _StafEntry) -> STAFTensorEntry:
+    name = C.string_at(e.name, e.name_length).decode("utf-8", "replace") if e.name else ""
+    return STAFTensorEntry(name, e.payload_offset, e.payload_size, e.scheme_identifier, e.semantic_role,
+                           e.original_dtype, tuple(e.shape[:e.dimension_count]), e.block_size, e.group_size,
+                           e.buffer_offset, e.alignment, e.checksum, e.shard_index)
+
+
+def _metadata_to_c(values: dict):
+    """{key: (type, value)} -> array of mi355q_staf_metadata (plus the byte strings that back it)."""
+    import struct
+    arr = (_StafMetadata * max(1, len(values)))()
+    keep = []
+    for i, (key, (typ, value)) in enumerate(values.items()):
+        kb = key.encode()
+        keep.append(kb)
+        arr[i].key, arr[i].type = kb, typ
+        if typ == STAF_STRING:
+            vb = value.encode()
+            buf = C.create_string_buffer(vb, len(vb) + 1)
+            keep.append(buf)
+            arr[i].text, arr[i].text_length, arr[i].payload0 = C.addressof(buf), len(vb), 0
+        elif typ == STAF_FLOAT32:
+            arr[i].payload0 = struct.unpack("<I", struct.pack("<f", value))[0]
+        elif typ == STAF_FLOAT64:
+            arr[i].payload0 = struct.unpack("<Q", struct.pack("<d", value))[0]
+        else:
+            arr[i].payload0 = int(value)
+    return arr, keep
+
+
+class STAFFile:
+    """An opened model.staf (STAFLoader.load + STAFWeightStore, MC/STAF/STAFLoader.swift:19-299)."""
+
+    def __init__(self, path: str):
+        h = C.c_void_p()
+        _check(library().mi355q_staf_open(os.fsencode(path), C.byref(h)))
+        self.handle = h.value
+
+    def close(self):
+        if self.handle:
+            library().mi355q_staf_close(self.handle)
+            self.handle = None
+
+    @property
+    def format_version(self) -> int:
+        return library().mi355q_staf_format_version(self.handle)
+
+    @property
+    def entries(self) -> list:
+        out = []
+        for i in range(library().mi355q_staf_tensor_count(self.handle)):
+            e = _StafEntry()
+            _check(library().mi355q_staf_tensor_at(self.handle, i, C.byref(e)))
+            out.append(_entry_from_c(e))
+        return out
+
+    def find(self, name: str) -> STAFTensorEntry:
+        e = _StafEntry()
+        _check(library().mi355q_staf_find(self.handle, name.encode(), C.byref(e)))
+        return _entry_from_c(e)
+
+    @property
+    def metadata(self) -> dict:
+        import struct
+        out = {}
+        for i in range(library().mi355q_staf_metadata_count(self.handle)):
+            m = _StafMetadata()
+            _check(library().mi355q_staf_metadata_at(self.handle, i, C.byref(m)))
+            if m.type == STAF_STRING:
+                v = C.string_at(m.text, m.text_length).decode("utf-8", "replace") if m.text else ""
+            elif m.type == STAF_BOOL:
+                v = m.payload0 != 0
+            elif m.type == STAF_UINT32:
+                v = m.payload0 & 0xFFFFFFFF
+            elif m.type == STAF_FLOAT32:
+                v = struct.unpack("<f", struct.pack("<I", m.payload0 & 0xFFFFFFFF))[0]
+            elif m.type == STAF_FLOAT64:
+                v = struct.unpack("<d", struct.pack("<Q", m.payload0))[0]
+            else:
+                v = m.payload0
+            out[m.key.decode()] = (m.type, v)
+        return out
+
+    def payload_region(self) -> np.ndarray:
+        """Copy of the payload region (first tensor to end of file) as bytes."""
+        n = C.c_uint64()
+        p = library().mi355q_staf_payload_region(self.handle, C.byref(n))
+        return np.frombuffer(C.string_at(p, n.value), dtype=np.uint8)
+
+    def payload(self, entry: STAFTensorEntry) -> np.ndarray:
+        return self.payload_region()[entry.buffer_offset:entry.buffer_offset + entry.payload_size]
+
+    def upload(self, ctx: "Context") -> "DeviceBuffer":
+        """The single device buffer of the weight store; tensors live at .ptr + entry.buffer_offset."""
+        p, n = C.c_void_p(), C.c_uint64()
+        _check(library().mi355q_staf_upload(ctx.handle, self.handle, C.byref(p), C.byref(n)))
+        return DeviceBuffer(ctx, p.value, n.value)
+
+    def weight(self, ctx: "Context", name: str, layout: int = LAYOUT_STAF_BLOCKS,
+               region: "DeviceBuffer | None" = None) -> "PackedWeight":
+        h = C.c_void_p()
+        _check(library().mi355q_staf_weight(ctx.handle, self.handle, region.ptr if region is not None else None,
+                                            name.encode(), layout, C.byref(h)))
+        return PackedWeight(ctx, h.value, keepalive=(region, self) if region is not None else (self,))
+
+
+def staf_write(path: str, tensors: list, metadata: dict | None = None):
+    """STAFWriter.write for converted payloads.  tensors: dicts with name, scheme_identifier, shape, payload
+    (bytes-like) and optionally semantic_role, original_dtype, shard_index; metadata: {key: (type, value)}."""
+    arr = (_StafTensor * max(1, len(tensors)))()
+    keep = []
+    for i, t in enumerate(tensors):
+        nb = t["name"].encode()
+        pb = np.ascontiguousarray(np.frombuffer(bytes(t["payload"]), dtype=np.uint8))
+        keep += [nb, pb]
+        arr[i].name, arr[i].scheme_identifier = nb, t["scheme_identifier"]
+        arr[i].semantic_role, arr[i].original_dtype = t.get("semantic_role", 0), t.get("original_dtype", 0xFF)
+        arr[i].dimension_count = len(t["shape"])
+        for d, v in enumerate(t["shape"][:8]):
+            arr[i].shape[d] = v
+        arr[i].payload, arr[i].payload_size = pb.ctypes.data if pb.size else None, pb.size
+        arr[i].shard_index = t.get("shard_index", 0)
+    md, keep_md = _metadata_to_c(metadata or {})
+    _check(library().mi355q_staf_write(os.fsencode(path), arr, len(tensors), md, len(metadata or {})))
+
+
+def staf_is_valid(path: str, sources=(), expected: dict | None = None) -> bool:
+    """STAFValidator.isValid (MC/STAF/STAFValidator.swift:5-78)."""
+    src = (C.c_char_p * max(1, len(sources)))(*[os.fsencode(s) for s in sources])
+    md, keep = _metadata_to_c(expected or {})
+    ok = C.c_int32()
+    _check(library().mi355q_staf_is_valid(os.fsencode(path), src, len(sources), md, len(expected or {}), C.byref(ok)))
+    return bool(ok.value)
 
 
 def shape_family(output_dimension: int, input_dimension: int):

@@ -589,4 +589,48 @@ mi355q_status mi355q_weight_destroy(mi355q_weight* w) {
     return MI355Q_OK;
 }
 
+// ---- STAF container on the device ----------------------------------------------------------------
+mi355q_status mi355q_staf_upload(mi355q_context* ctx, const mi355q_staf* staf, void** base_dev_out, uint64_t* bytes_out) {
+    if (!base_dev_out) return fail(MI355Q_ERR_INVALID_ARGUMENT, "output pointer is null");
+    *base_dev_out = nullptr;
+    if (!ctx || !staf) return fail(MI355Q_ERR_NULL_HANDLE, "context or container is null");
+    uint64_t bytes = 0;
+    const void* region = mi355q_staf_payload_region(staf, &bytes);
+    void* dev = nullptr;
+    if (mi355q_status st = mi355q_buffer_alloc(ctx, (size_t)bytes, &dev)) return st;
+    // pageable host memory (the file mapping): a synchronous copy, staged by the runtime
+    const hipError_t e = hipMemcpy(dev, region, (size_t)bytes, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        (void)hipFree(dev);
+        return fail(MI355Q_ERR_DEVICE, "copy of the payload region failed: %s", hipGetErrorString(e));
+    }
+    *base_dev_out = dev;
+    if (bytes_out) *bytes_out = bytes;
+    return MI355Q_OK;
+}
+
+mi355q_status mi355q_staf_weight(mi355q_context* ctx, const mi355q_staf* staf, const void* base_dev, const char* name,
+                                 mi355q_layout layout, mi355q_weight** out) {
+    if (!out) return fail(MI355Q_ERR_INVALID_ARGUMENT, "weight out pointer is null");
+    *out = nullptr;
+    if (!ctx || !staf) return fail(MI355Q_ERR_NULL_HANDLE, "context or container is null");
+    mi355q_staf_entry t;
+    if (mi355q_status st = mi355q_staf_find(staf, name, &t)) return st;
+    const mi355q_format* f = find_format_scheme(t.scheme_identifier);
+    if (!f) return fail(MI355Q_ERR_UNSUPPORTED_FORMAT, "tensor '%s' has scheme 0x%02x, which is not a packed format", name,
+                        (unsigned)t.scheme_identifier);
+    if (t.dimension_count != 2)
+        return fail(MI355Q_ERR_SHAPE, "tensor '%s' has %u dimensions; a packed projection has 2", name, (unsigned)t.dimension_count);
+    const uint64_t n = t.shape[0], k = (uint64_t)t.shape[1] * 32 / f->bits;      // STAFWriter.swift:250-258
+    if (layout == MI355Q_LAYOUT_STAF_BLOCKS) {
+        if (!base_dev) return fail(MI355Q_ERR_INVALID_ARGUMENT, "the row-major layout needs the uploaded payload region");
+        return mi355q_weight_wrap_staf(ctx, t.scheme_identifier, n, k, (const char*)base_dev + t.buffer_offset,
+                                       (size_t)t.payload_size, out);
+    }
+    uint64_t bytes = 0;
+    const uint8_t* region = (const uint8_t*)mi355q_staf_payload_region(staf, &bytes);
+    return mi355q_weight_prepare_staf(ctx, t.scheme_identifier, n, k, region + t.buffer_offset, (size_t)t.payload_size,
+                                      layout, out);
+}
+
 }  // extern "C"

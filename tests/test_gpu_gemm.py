@@ -181,6 +181,15 @@ def test_config3_prefill_gate_up_and_down(pkg, ctx, m, n, k):
     assert rel < 5e-4
 
 
+def test_mfma_gemm_many_tiles_ragged_last_column_tile(pkg, ctx):
+    """2048 x 14286: more 256 x 256 tiles than CUs (two rounds), the last column tile cut at column 14286,
+    padded output rows."""
+    m, n, k = 2048, 14286, 128
+    sample = _tile_edge_sample(n, 77)
+    _seeded_gemm(pkg, ctx, 960, m, n, k, 4, 64, sample=sample)
+    _seeded_gemm(pkg, ctx, 961, m, n, k, 8, 32, sample=sample, y_pad=2)
+
+
 @pytest.mark.parametrize("bits,group", [f for f in MFMA_FORMATS if f != (4, 64)])
 def test_mfma_gemm_other_formats_seeded(pkg, ctx, bits, group):
     _seeded_gemm(pkg, ctx, 800 + bits + group, 200, 384, 1024, bits, group)
