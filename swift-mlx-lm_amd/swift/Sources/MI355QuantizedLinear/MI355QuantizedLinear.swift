@@ -8,6 +8,7 @@
 //
 // Errors keep the reference's convention: plan/compile-time failures throw, programmer errors trap.
 import CMI355QLinear
+import Foundation
 
 public enum MI355QError: Error, CustomStringConvertible {
     case invalidArgument(String), unsupportedQuantization(String), inconsistentShape(String)
@@ -38,6 +39,7 @@ public enum BufferPrecision: UInt32 {
 public enum WeightLayout: UInt32 {
     case rowMajorBlocks = 0      // canonical STAF interleaved blocks
     case splitPlanes = 1         // specialized layout of this backend
+    case tile16 = 2              // matrix-core decode layout (q4 g64): 1...16 sequences per launch
     var c: mi355q_layout { mi355q_layout(rawValue) }
 }
 
@@ -121,6 +123,12 @@ public final class PackedWeight {
         self.context = context
     }
 
+    /// Takes ownership of a handle made by the library (a tensor of an opened container).
+    init(context: MI355Context, owning handle: OpaquePointer) {
+        self.handle = handle
+        self.context = context
+    }
+
     deinit { _ = mi355q_weight_destroy(handle) }
 
     /// Plan record of the decode step of this projection (kernel name, grid, shape family,
@@ -155,5 +163,73 @@ public extension MI355Context {
                                 precision: BufferPrecision, logits: UnsafeMutablePointer<Float>?,
                                 token: UnsafeMutablePointer<Int32>) throws {
         try MI355QError.check(mi355q_lmhead_argmax(handle, stream, weight.handle, hidden, precision.c, logits, token, 0))
+    }
+}
+
+/// An opened `model.staf` with its payload region resident in HBM: the analogue of `STAFWeightStore`
+/// (one buffer, entries by name, file-level metadata).
+public final class MI355STAFStore {
+    let handle: OpaquePointer
+    public let context: MI355Context
+    /// Device address of the payload region; tensor `t` lives at `base + t.buffer_offset`.
+    public let base: UnsafeMutableRawPointer
+
+    public init(context: MI355Context, url: URL) throws {
+        var h: OpaquePointer?
+        try MI355QError.check(mi355q_staf_open(url.path, &h))
+        var dev: UnsafeMutableRawPointer?
+        var bytes: UInt64 = 0
+        let status = mi355q_staf_upload(context.handle, h, &dev, &bytes)
+        if status != 0 {
+            mi355q_staf_close(h)
+            try MI355QError.check(status)
+        }
+        handle = h!
+        base = dev!
+        self.context = context
+    }
+
+    deinit {
+        _ = mi355q_buffer_free(context.handle, base)
+        mi355q_staf_close(handle)
+    }
+
+    /// `entries[name]`
+    public func entry(named name: String) -> mi355q_staf_entry? {
+        var e = mi355q_staf_entry()
+        return mi355q_staf_find(handle, name, &e) == 0 ? e : nil
+    }
+
+    /// `resolvedBufferAccess(for:)`: the row-major bytes in place, or this library's specialized copy.
+    public func weight(named name: String, layout: WeightLayout = .rowMajorBlocks) throws -> PackedWeight {
+        var w: OpaquePointer?
+        try MI355QError.check(mi355q_staf_weight(context.handle, handle, base, name, layout.c, &w))
+        return PackedWeight(context: context, owning: w!)
+    }
+
+    /// `STAFValidator.isValid`
+    public static func isValid(stafURL: URL, safetensorsURLs: [URL]) throws -> Bool {
+        var valid: Int32 = 0
+        var paths = safetensorsURLs.map { strdup($0.path) }
+        defer { paths.forEach { free($0) } }
+        let status = paths.withUnsafeMutableBufferPointer { buf -> mi355q_status in
+            buf.withMemoryRebound(to: UnsafePointer<CChar>?.self) { p in
+                mi355q_staf_is_valid(stafURL.path, p.baseAddress, UInt32(p.count), nil, 0, &valid)
+            }
+        }
+        try MI355QError.check(status)
+        return valid != 0
+    }
+}
+
+public extension MI355Context {
+    /// Embedding gather (tokenIDs, table, output, embeddingDim, sequenceLength bindings of
+    /// `embedding_lookup[_seq]_q{b}_g{g}`); the table may be the tied output head.
+    func encodeEmbeddingLookup(stream: UnsafeMutableRawPointer?, table: PackedWeight, tokenIDs: UnsafePointer<Int32>,
+                               sequenceLength: Int, output: UnsafeMutableRawPointer, precision: BufferPrecision,
+                               embeddingScale: Float? = nil) throws {
+        try MI355QError.check(mi355q_embedding_lookup(handle, stream, table.handle, tokenIDs, UInt32(sequenceLength),
+                                                      output, precision.c, 0, embeddingScale == nil ? 0 : 1,
+                                                      embeddingScale ?? 1))
     }
 }
