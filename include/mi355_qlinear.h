@@ -522,6 +522,40 @@ MI355Q_API mi355q_status mi355q_staf_upload(mi355q_context* ctx, const mi355q_st
 MI355Q_API mi355q_status mi355q_staf_weight(mi355q_context* ctx, const mi355q_staf* staf, const void* base_dev,
                                             const char* name, mi355q_layout layout, mi355q_weight** out);
 
+/* ------------------------------------------------------------------------------------------
+ * Quantized KV cache (the step on the other side of the attention projections)
+ * ---------------------------------------------------------------------------------------- */
+/* QuantizationSchemeIdentifier.isSupportedForKVCache (MC/STAF/STAFFormat.swift:239-262) for the schemes this
+ * library writes and reads: dense 0x00 / 0x01 / 0x02, 8-bit 0x10-0x12, 4-bit 0x40-0x42.  The rotor schemes
+ * (0x70, 0x71) need the Clifford pre-rotation, which is outside this path: 0. */
+MI355Q_API int32_t mi355q_kv_scheme_is_supported(uint8_t scheme_identifier);
+/* KVCacheSpecification.bytesPerHeadSlot (MC/Buffer/MetalGraphAllocator.swift:60-114): ceil(headDim /
+ * weightsPerBlock) blocks rounded up to 64 bytes (packed) or 256 bytes (dense); every registered format is
+ * sizable, also those without kernels; rotor schemes size as their base scheme; 0 = no registered format. */
+MI355Q_API uint32_t mi355q_kv_bytes_per_head_slot(uint8_t scheme_identifier, uint32_t head_dimension);
+/* The uniforms of the cache kernels (kvHeadCount, headDimension, maxSequenceLength, layoutMode, k/vQuantScheme,
+ * k/vHeadSlotBytes; MC/Generator/MetalSourceGenerator+Attention.swift:1199-1216).  layout_mode 0 =
+ * [head][position] (sequence-major), 1 = [position][head] (head-major); one layer's K or V buffer. */
+typedef struct mi355q_kv_layout {
+    uint8_t scheme;
+    uint8_t layout_mode;
+    uint16_t reserved0;
+    uint32_t kv_head_count, head_dimension, maximum_sequence_length, head_slot_bytes;
+} mi355q_kv_layout;
+/* write_kv_quantized / write_kv_element_dense for positions [first_position, +sequence_length) of every head
+ * (:2057-2180, :1958-1971; addressing :762-769): src is [sequence_length, input_row_stride] with head h at
+ * columns [h * headDim, +headDim) (0 = dense rows).  Per group: scale = (max - min) / levels (at least 1e-10),
+ * header f16(scale), f16(min), codes round((v - min) / scale) clamped. */
+MI355Q_API mi355q_status mi355q_kv_cache_write(mi355q_context* ctx, void* stream, const mi355q_kv_layout* layout,
+                                               void* cache_dev, const void* src_dev, mi355q_dtype src_dtype,
+                                               uint32_t input_row_stride, uint32_t first_position,
+                                               uint32_t sequence_length);
+/* read_kv_element (:1923-1956) over whole slots: out is [sequence_length, out_row_stride] in out_dtype. */
+MI355Q_API mi355q_status mi355q_kv_cache_read(mi355q_context* ctx, void* stream, const mi355q_kv_layout* layout,
+                                              const void* cache_dev, void* out_dev, mi355q_dtype out_dtype,
+                                              uint32_t out_row_stride, uint32_t first_position,
+                                              uint32_t sequence_length);
+
 #ifdef __cplusplus
 }
 #endif

@@ -59,6 +59,10 @@ def lib():
         L.orc_dequant_planes_f32.argtypes = [i32, i32, sz, sz, vp, vp, vp, i32, vp]
         L.orc_dequant_staf_bf16.argtypes = [i32, i32, sz, sz, vp, vp]
         L.orc_embedding_lookup_staf_f32.argtypes = [i32, i32, sz, sz, vp, vp, sz, i32, C.c_float, vp]
+        L.orc_kv_quant_bits.argtypes = [i32]; L.orc_kv_quant_group.argtypes = [i32]
+        L.orc_kv_bytes_per_head_slot.argtypes = [i32, sz]; L.orc_kv_bytes_per_head_slot.restype = sz
+        L.orc_kv_write_slot.argtypes = [i32, vp, sz, vp]; L.orc_kv_read_slot.argtypes = [i32, vp, sz, vp]
+        L.orc_kv_slot_offset.argtypes = [i32, sz, sz, sz, sz, sz]; L.orc_kv_slot_offset.restype = sz
         L.orc_gemm_f64.argtypes = [vp, vp, sz, sz, sz, sz, vp]; L.orc_gemm_f64.restype = None
         L.orc_qgemm_staf_ref_f32.argtypes = [i32, i32, vp, vp, sz, sz, sz, sz, vp, i32]
         L.orc_qgemm_planes_ref_f32.argtypes = [i32, i32, vp, vp, vp, i32, vp, sz, sz, sz, sz, vp, i32]
@@ -209,6 +213,52 @@ def embedding_lookup_staf_f32(bits, group, vocab, dim, table, token_ids, embeddi
                                                0 if embedding_scale is None else 1,
                                                0.0 if embedding_scale is None else float(embedding_scale), _p(out)),
            "embedding_lookup_staf_f32")
+    return out
+
+
+# --------------------------------------------------------------------- KV cache
+def kv_bytes_per_head_slot(scheme: int, head_dim: int) -> int:
+    return int(lib().orc_kv_bytes_per_head_slot(scheme, head_dim))
+
+
+def kv_write_slot(scheme: int, src, slot=None) -> np.ndarray:
+    """Quantise one head vector into a slot (a fresh zeroed slot unless one is given)."""
+    src = _c(src, np.float32)
+    if slot is None:
+        slot = np.zeros(kv_bytes_per_head_slot(scheme, src.size), np.uint8)
+    _check(lib().orc_kv_write_slot(scheme, _p(src), src.size, _p(slot)), "kv_write_slot")
+    return slot
+
+
+def kv_read_slot(scheme: int, slot, head_dim: int) -> np.ndarray:
+    slot = _c(slot, np.uint8)
+    out = np.zeros(head_dim, np.float32)
+    _check(lib().orc_kv_read_slot(scheme, _p(slot), head_dim, _p(out)), "kv_read_slot")
+    return out
+
+
+def kv_cache_write(scheme, layout_mode, kv_heads, head_dim, max_positions, src, first_position, cache=None):
+    """src [positions, kv_heads * head_dim] fp32 -> cache bytes; the reference's fill loop
+    (MC/Generator/MetalSourceGenerator+Attention.swift:1233-1250, slot addressing :762-769)."""
+    src = _c(src, np.float32).reshape(-1, kv_heads * head_dim)
+    slot = kv_bytes_per_head_slot(scheme, head_dim)
+    if cache is None:
+        cache = np.zeros(kv_heads * max_positions * slot, np.uint8)
+    for p in range(src.shape[0]):
+        for h in range(kv_heads):
+            off = int(lib().orc_kv_slot_offset(layout_mode, h, first_position + p, kv_heads, max_positions, slot))
+            kv_write_slot(scheme, src[p, h * head_dim:(h + 1) * head_dim], cache[off:off + slot])
+    return cache
+
+
+def kv_cache_read(scheme, layout_mode, kv_heads, head_dim, max_positions, cache, first_position, count):
+    cache = _c(cache, np.uint8)
+    slot = kv_bytes_per_head_slot(scheme, head_dim)
+    out = np.zeros((count, kv_heads * head_dim), np.float32)
+    for p in range(count):
+        for h in range(kv_heads):
+            off = int(lib().orc_kv_slot_offset(layout_mode, h, first_position + p, kv_heads, max_positions, slot))
+            out[p, h * head_dim:(h + 1) * head_dim] = kv_read_slot(scheme, cache[off:off + slot], head_dim)
     return out
 
 

@@ -542,3 +542,109 @@ int orc_quantize_affine(const float* w, size_t n_rows, size_t k, int bits, int g
     free(tmp);
     return 0;
 }
+
+
+/* ---- quantized KV cache ---------------------------------------------------------------------------- */
+/* MC/Generator/MetalSourceGenerator+Attention.swift:1894-1921 */
+int orc_kv_quant_bits(int scheme) {
+    if (scheme == 0x10 || scheme == 0x11 || scheme == 0x12) return 8;
+    if (scheme == 0x40 || scheme == 0x41 || scheme == 0x42) return 4;
+    return 0;
+}
+int orc_kv_quant_group(int scheme) {
+    switch (scheme) {
+    case 0x10: return 32;
+    case 0x11: return 64;
+    case 0x12: return 128;
+    case 0x40: return 64;
+    case 0x41: case 0x42: return 128;
+    default: return 0;
+    }
+}
+
+/* MC/Buffer/MetalGraphAllocator.swift:60-114 */
+size_t orc_kv_bytes_per_head_slot(int scheme, size_t head_dim) {
+    size_t weights_per_block, bytes_per_block, alignment;
+    if (scheme == 0x00 || scheme == 0x01 || scheme == 0xFF) { weights_per_block = 1; bytes_per_block = 2; alignment = 256; }
+    else if (scheme == 0x02) { weights_per_block = 1; bytes_per_block = 4; alignment = 256; }
+    else {
+        orc_format f;
+        if (scheme == 0x70) scheme = 0x10;           /* rotor schemes size as their base scheme */
+        if (scheme == 0x71) scheme = 0x40;
+        if (orc_format_for_scheme(scheme, &f) != 0 || !f.in_reference) return 0;
+        weights_per_block = (size_t)f.group; bytes_per_block = (size_t)f.bytes_per_block; alignment = 64;
+    }
+    const size_t raw = (head_dim + weights_per_block - 1) / weights_per_block * bytes_per_block;
+    return (raw + alignment - 1) / alignment * alignment;
+}
+
+size_t orc_kv_slot_offset(int layout_mode, size_t head, size_t position, size_t kv_heads, size_t max_positions,
+                          size_t head_slot_bytes) {
+    return layout_mode == 0 ? head * max_positions * head_slot_bytes + position * head_slot_bytes
+                            : position * kv_heads * head_slot_bytes + head * head_slot_bytes;
+}
+
+/* MC/Generator/MetalSourceGenerator+Attention.swift:2057-2157 (packed), :1958-1971 (dense) */
+int orc_kv_write_slot(int scheme, const float* src, size_t head_dim, uint8_t* slot) {
+    if (scheme == 0x00) { for (size_t d = 0; d < head_dim; d++) ((uint16_t*)slot)[d] = orc_f16_from_f32(src[d]); return 0; }
+    if (scheme == 0x01) { for (size_t d = 0; d < head_dim; d++) ((uint16_t*)slot)[d] = orc_bf16_from_f32(src[d]); return 0; }
+    if (scheme == 0x02) { memcpy(slot, src, head_dim * 4); return 0; }
+    const int bits = orc_kv_quant_bits(scheme);
+    const size_t group = (size_t)orc_kv_quant_group(scheme);
+    if (!bits) return -1;
+    const size_t bytes_per_block = 4 + group * (size_t)bits / 8;
+    const float levels = bits == 8 ? 255.0f : 15.0f;
+    const int top = bits == 8 ? 255 : 15;
+    for (size_t g = 0; g * group < head_dim; g++) {
+        const size_t start = g * group;
+        float lo = HUGE_VALF, hi = -HUGE_VALF;
+        for (size_t i = 0; i < group && start + i < head_dim; i++) {
+            lo = fminf(lo, src[start + i]);
+            hi = fmaxf(hi, src[start + i]);
+        }
+        float scale = (hi - lo) / levels;
+        if (scale < 1e-10f) scale = 1e-10f;
+        uint8_t* block = slot + g * bytes_per_block;
+        const uint16_t hs = orc_f16_from_f32(scale), hz = orc_f16_from_f32(lo);
+        memcpy(block, &hs, 2);
+        memcpy(block + 2, &hz, 2);
+        if (bits == 8) {
+            for (size_t i = 0; i < group && start + i < head_dim; i++) {
+                int q = (int)roundf((src[start + i] - lo) / scale);
+                block[4 + i] = (uint8_t)(q < 0 ? 0 : q > top ? top : q);
+            }
+        } else {
+            for (size_t i = 0; i < group / 2 && start + 2 * i < head_dim; i++) {
+                const float v0 = src[start + 2 * i];
+                const float v1 = start + 2 * i + 1 < head_dim ? src[start + 2 * i + 1] : 0.0f;
+                int q0 = (int)roundf((v0 - lo) / scale), q1 = (int)roundf((v1 - lo) / scale);
+                q0 = q0 < 0 ? 0 : q0 > top ? top : q0;
+                q1 = q1 < 0 ? 0 : q1 > top ? top : q1;
+                block[4 + i] = (uint8_t)(q0 | (q1 << 4));
+            }
+        }
+    }
+    return 0;
+}
+
+/* MC/Generator/MetalSourceGenerator+Attention.swift:1923-1956 */
+int orc_kv_read_slot(int scheme, const uint8_t* slot, size_t head_dim, float* out) {
+    if (scheme == 0x00) { for (size_t d = 0; d < head_dim; d++) out[d] = orc_f16_to_f32(((const uint16_t*)slot)[d]); return 0; }
+    if (scheme == 0x01) { for (size_t d = 0; d < head_dim; d++) out[d] = orc_bf16_to_f32(((const uint16_t*)slot)[d]); return 0; }
+    if (scheme == 0x02) { memcpy(out, slot, head_dim * 4); return 0; }
+    const int bits = orc_kv_quant_bits(scheme);
+    const size_t group = (size_t)orc_kv_quant_group(scheme);
+    if (!bits) return -1;
+    const size_t bytes_per_block = 4 + group * (size_t)bits / 8;
+    for (size_t d = 0; d < head_dim; d++) {
+        const uint8_t* block = slot + d / group * bytes_per_block;
+        const size_t i = d % group;
+        uint16_t hs, hz;
+        memcpy(&hs, block, 2);
+        memcpy(&hz, block + 2, 2);
+        const float scale = orc_f16_to_f32(hs), zero = orc_f16_to_f32(hz);
+        const unsigned q = bits == 8 ? block[4 + i] : (i % 2 == 0 ? (block[4 + i / 2] & 0x0Fu) : (block[4 + i / 2] >> 4));
+        out[d] = scale * (float)q + zero;
+    }
+    return 0;
+}

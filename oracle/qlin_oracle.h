@@ -17,6 +17,9 @@
  *   orc_gemm_f64 / *_ref_f32   pinned: closed-form KATs (192.0 / 320.0, integer dot products)
  *   orc_bf16_from_f32          pinned: RNE rule + known bit patterns
  *   orc_f16_from_f32           pinned: exhaustive round trip over all 65536 half patterns vs numpy
+ *   orc_embedding_lookup_*     pinned: the reference's two embedding vectors + row gather of the pinned dequant
+ *   orc_kv_*                   pinned: head-slot sizes, the q8 round-trip vector and the unsigned-byte read
+ *                              vector of the reference's tests; exact rational arithmetic for the codes
  *   orc_argmax_lowest          PARITY UNPINNED against the reference (it holds no argmax value
  *                              test); pinned only by brute force against numpy on tiny vectors
  *   orc_quantize_affine        PARITY UNPINNED (the reference has no weight quantizer; this is an
@@ -115,6 +118,26 @@ int32_t orc_argmax_lowest(const float* v, size_t n);
  * 1e-10 floor as MC/Generator/MetalSourceGenerator+Quantized.swift:427-433). */
 int orc_quantize_affine(const float* w, size_t n_rows, size_t k, int bits, int group, int sb_dtype,
                         uint32_t* codes, void* scales, void* biases);
+
+/* ---- quantized KV cache (MC/Generator/MetalSourceGenerator+Attention.swift) ------------------------- */
+/* kv_quant_bits / kv_quant_group_size / kv_quant_bytes_per_block (:1894-1921): 8-bit g32/64/128, 4-bit g64/128/128z;
+ * 0 for every other scheme.  Dense 0x00 / 0x01 / 0x02 are handled by the read / write functions. */
+int orc_kv_quant_bits(int scheme);
+int orc_kv_quant_group(int scheme);
+/* KVCacheSpecification.bytesPerHeadSlot (MC/Buffer/MetalGraphAllocator.swift:60-114): ceil(headDim / weightsPerBlock)
+ * blocks, rounded up to 64 bytes for packed formats and 256 for dense ones; every registered format is sizable.
+ * 0 for a scheme without a registered format. */
+size_t orc_kv_bytes_per_head_slot(int scheme, size_t head_dim);
+/* write_kv_quantized_q8 / _q4 (:2057-2157) and write_kv_element_dense (:1958-1971) for one head vector:
+ * per group min/max, scale = (max - min) / levels clamped to 1e-10, header = f16(scale), f16(min),
+ * q = clamp(round((v - min) / scale), 0, levels) with the unrounded fp32 scale.  Bytes of the slot that the
+ * reference does not write are left as they are.  Returns 0, or -1 for a scheme the kernels do not write. */
+int orc_kv_write_slot(int scheme, const float* src, size_t head_dim, uint8_t* slot);
+/* read_kv_element (:1923-1956) for elements [0, head_dim) of one slot. */
+int orc_kv_read_slot(int scheme, const uint8_t* slot, size_t head_dim, float* out);
+/* Byte offset of the slot of (head, position): layoutMode 0 = [head][position], 1 = [position][head] (:762-769). */
+size_t orc_kv_slot_offset(int layout_mode, size_t head, size_t position, size_t kv_heads, size_t max_positions,
+                          size_t head_slot_bytes);
 
 #ifdef __cplusplus
 }

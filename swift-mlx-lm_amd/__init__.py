@@ -70,6 +70,12 @@ class _StafTensor(C.Structure):
                 ("payload", C.c_void_p), ("payload_size", C.c_uint64), ("shard_index", C.c_uint32)]
 
 
+class _KvLayout(C.Structure):
+    _fields_ = [("scheme", C.c_uint8), ("layout_mode", C.c_uint8), ("reserved0", C.c_uint16),
+                ("kv_head_count", C.c_uint32), ("head_dimension", C.c_uint32),
+                ("maximum_sequence_length", C.c_uint32), ("head_slot_bytes", C.c_uint32)]
+
+
 class _DeviceInfo(C.Structure):
     _fields_ = [("name", C.c_char * 64), ("arch", C.c_char * 32), ("compute_units", C.c_int32),
                 ("wavefront_size", C.c_int32), ("lds_bytes_per_workgroup", C.c_int32), ("reserved0", C.c_int32),
@@ -162,6 +168,10 @@ def library() -> C.CDLL:
         "mi355q_plan_graph_build": (i32, [vp, vp]),
         "mi355q_plan_graph_launch": (i32, [vp, vp]),
         "mi355q_buffer_copy": (i32, [vp, vp, vp, vp, sz]),
+        "mi355q_kv_scheme_is_supported": (i32, [u8]),
+        "mi355q_kv_bytes_per_head_slot": (u32, [u8, u32]),
+        "mi355q_kv_cache_write": (i32, [vp, vp, P(_KvLayout), vp, vp, C.c_int, u32, u32, u32]),
+        "mi355q_kv_cache_read": (i32, [vp, vp, P(_KvLayout), vp, vp, C.c_int, u32, u32, u32]),
         "mi355q_staf_open": (i32, [C.c_char_p, P(vp)]),
         "mi355q_staf_close": (None, [vp]),
         "mi355q_staf_format_version": (u32, [vp]),
@@ -597,6 +607,51 @@ def staf_is_valid(path: str, sources=(), expected: dict | None = None) -> bool:
     return bool(ok.value)
 
 
+
+# --------------------------------------------------------------------------------- KV cache
+KV_SEQUENCE_MAJOR, KV_HEAD_MAJOR = 0, 1      # KVCacheLayoutMode
+
+
+def kv_scheme_is_supported(scheme_identifier: int) -> bool:
+    return bool(library().mi355q_kv_scheme_is_supported(scheme_identifier))
+
+
+def kv_bytes_per_head_slot(scheme_identifier: int, head_dimension: int) -> int:
+    return library().mi355q_kv_bytes_per_head_slot(scheme_identifier, head_dimension)
+
+
+@dataclass(frozen=True)
+class KVCacheSpecification:
+    """One layer's K or V cache (KVCacheSpecification, MC/Buffer/MetalGraphAllocator.swift:7-175)."""
+    scheme_identifier: int
+    layout_mode: int
+    kv_head_count: int
+    head_dimension: int
+    maximum_sequence_length: int
+
+    @property
+    def bytes_per_head_slot(self) -> int:
+        return kv_bytes_per_head_slot(self.scheme_identifier, self.head_dimension)
+
+    @property
+    def bytes_per_token_slot(self) -> int:
+        return self.kv_head_count * self.bytes_per_head_slot
+
+    @property
+    def bytes_per_layer(self) -> int:
+        return self.maximum_sequence_length * self.bytes_per_token_slot
+
+    def offset(self, head: int, position: int) -> int:
+        slot = self.bytes_per_head_slot
+        if self.layout_mode == KV_SEQUENCE_MAJOR:
+            return head * self.maximum_sequence_length * slot + position * slot
+        return position * self.kv_head_count * slot + head * slot
+
+    def _c(self) -> _KvLayout:
+        return _KvLayout(self.scheme_identifier, self.layout_mode, 0, self.kv_head_count, self.head_dimension,
+                         self.maximum_sequence_length, self.bytes_per_head_slot)
+
+
 def shape_family(output_dimension: int, input_dimension: int):
     """DecodeProjectionShapeFamily.resolve -> (family, preferredSimdgroups, tileElements, kernelBaseName)."""
     fam, sg, tile = C.c_int32(), C.c_uint32(), C.c_uint32()
@@ -693,6 +748,18 @@ class Context:
         _check(library().mi355q_weight_prepare_staf(self.handle, fmt.scheme_identifier, n, k, blocks.ctypes.data,
                                                     blocks.size, layout, C.byref(h)))
         return PackedWeight(self, h.value)
+
+    def kv_cache_write(self, spec: "KVCacheSpecification", cache, src, src_dtype: int, first_position: int,
+                       sequence_length: int, input_row_stride: int = 0, stream: int = 0):
+        lay = spec._c()
+        _check(library().mi355q_kv_cache_write(self.handle, stream, C.byref(lay), self._ptr(cache), self._ptr(src),
+                                               src_dtype, input_row_stride, first_position, sequence_length))
+
+    def kv_cache_read(self, spec: "KVCacheSpecification", cache, out, out_dtype: int, first_position: int,
+                      sequence_length: int, out_row_stride: int = 0, stream: int = 0):
+        lay = spec._c()
+        _check(library().mi355q_kv_cache_read(self.handle, stream, C.byref(lay), self._ptr(cache), self._ptr(out),
+                                              out_dtype, out_row_stride, first_position, sequence_length))
 
     def weight_wrap_staf(self, fmt: QuantizationFormat, n: int, k: int, blocks: DeviceBuffer,
                          byte_offset: int = 0, payload_bytes: int | None = None) -> PackedWeight:
