@@ -78,7 +78,8 @@ enum {
     MI355Q_FLAG_NONE = 0,
     MI355Q_FLAG_FORCE_GENERIC = 1, /* run the reference-shaped per-code kernel (A/B and tests) */
     MI355Q_FLAG_FORCE_SMALL_M = 2, /* qgemm: use the small-M GEMV-style kernel whatever M is */
-    MI355Q_FLAG_FORCE_MFMA = 4     /* qgemm: use the MFMA kernel whatever M is */
+    MI355Q_FLAG_FORCE_MFMA = 4,    /* qgemm: use the MFMA kernel whatever M is */
+    MI355Q_FLAG_PROBE_CLOCK = 8    /* qgemm on the MFMA kernel: record the clock probe (mi355q_clock_probe_read) */
 };
 
 /* ------------------------------------------------------------------------------------------
@@ -253,6 +254,14 @@ MI355Q_API mi355q_status mi355q_qgemm(mi355q_context* ctx, void* stream, const m
                                       const void* x_dev, mi355q_dtype x_dtype, void* y_dev,
                                       mi355q_dtype y_dtype, uint32_t m, uint32_t x_row_stride,
                                       uint32_t y_row_stride, uint32_t flags);
+
+/* Measurement aid without a counterpart in the reference: after an mi355q_qgemm call with
+ * MI355Q_FLAG_PROBE_CLOCK that ran on the matrix cores has completed, returns what the first wavefront of
+ * workgroup 0 counted while it was in the kernel: shader-clock cycles and ticks of the constant 100 MHz
+ * counter.  cycles / ticks / 10 is the clock in GHz the kernel ran at (it depends on the operand data:
+ * the part lowers its clock under matrix-core load).  Synchronises with the device. */
+MI355Q_API mi355q_status mi355q_clock_probe_read(mi355q_context* ctx, uint64_t* shader_cycles,
+                                                 uint64_t* realtime_ticks);
 
 /* batched_gemm_q4_g64_{2,3} (:166-338; bindings MC/Compiler/MetalPrefillStepBuilder.swift:928-955):
  * 2 or 3 projections sharing one input (gate+up, q+k+v) in one launch.  All weights must share

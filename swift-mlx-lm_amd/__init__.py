@@ -21,7 +21,7 @@ F16, BF16, F32 = 0, 1, 2
 # STAFWeightLayout
 LAYOUT_STAF_BLOCKS, LAYOUT_PLANES, LAYOUT_TILE16 = 0, 1, 2
 # launch flags
-FLAG_NONE, FLAG_FORCE_GENERIC, FLAG_FORCE_SMALL_M, FLAG_FORCE_MFMA = 0, 1, 2, 4
+FLAG_NONE, FLAG_FORCE_GENERIC, FLAG_FORCE_SMALL_M, FLAG_FORCE_MFMA, FLAG_PROBE_CLOCK = 0, 1, 2, 4, 8
 
 STATUS_NAMES = {0: "OK", -1: "INVALID_ARGUMENT", -2: "UNSUPPORTED_FORMAT", -3: "SHAPE", -4: "NULL_HANDLE",
                 -5: "DEVICE", -6: "OUT_OF_MEMORY", -7: "KERNEL_NOT_FOUND", -8: "SIZE_MISMATCH",
@@ -168,6 +168,7 @@ def library() -> C.CDLL:
         "mi355q_plan_graph_build": (i32, [vp, vp]),
         "mi355q_plan_graph_launch": (i32, [vp, vp]),
         "mi355q_buffer_copy": (i32, [vp, vp, vp, vp, sz]),
+        "mi355q_clock_probe_read": (i32, [vp, P(u64), P(u64)]),
         "mi355q_kv_scheme_is_supported": (i32, [u8]),
         "mi355q_kv_bytes_per_head_slot": (u32, [u8, u32]),
         "mi355q_kv_cache_write": (i32, [vp, vp, P(_KvLayout), vp, vp, C.c_int, u32, u32, u32]),
@@ -748,6 +749,12 @@ class Context:
         _check(library().mi355q_weight_prepare_staf(self.handle, fmt.scheme_identifier, n, k, blocks.ctypes.data,
                                                     blocks.size, layout, C.byref(h)))
         return PackedWeight(self, h.value)
+
+    def clock_probe_ghz(self) -> float:
+        """Shader clock of the last MFMA GEMM launched with FLAG_PROBE_CLOCK (0.0 if none ran)."""
+        c, t = C.c_uint64(), C.c_uint64()
+        _check(library().mi355q_clock_probe_read(self.handle, C.byref(c), C.byref(t)))
+        return c.value / (t.value * 10.0) if t.value else 0.0
 
     def kv_cache_write(self, spec: "KVCacheSpecification", cache, src, src_dtype: int, first_position: int,
                        sequence_length: int, input_row_stride: int = 0, stream: int = 0):

@@ -94,14 +94,16 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
         return fail(MI355Q_ERR_INVALID_ARGUMENT, "contradictory kernel selection flags");
     const WView v = w->view();
     const bool mfma_ok = gemm_mfma_eligible(v, x_dtype, m, xs);
+    // the clock probe cell lives behind the argmax cells of the context's scratch
+    unsigned long long* const probe = (flags & MI355Q_FLAG_PROBE_CLOCK) ? ctx->argmax_scratch + 16 : nullptr;
     if (flags & MI355Q_FLAG_FORCE_MFMA) {
         if (!mfma_ok)
             return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the MFMA GEMM does not accept this format, layout or stride");
-        return launch_qgemm_mfma(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
+        return launch_qgemm_mfma(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys, probe);
     }
     const bool small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) || m <= 8 || !mfma_ok;
     if (small) return run_small_m(ctx, s, w, x, x_dtype, y, y_dtype, m, xs, ys, flags);
-    return launch_qgemm_mfma(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
+    return launch_qgemm_mfma(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys, probe);
 }
 
 // Two or three projections that read the same activations (q+k+v, gate+up).  For M <= 8 on the
@@ -260,6 +262,17 @@ mi355q_status mi355q_lmhead_argmax(mi355q_context* ctx, void* stream, const mi35
                                    uint32_t flags) {
     if (mi355q_status s = check_launch(ctx, w)) return s;
     return dispatch_output_head(ctx, (hipStream_t)stream, w, x_dev, x_dtype, logits_f32_dev, token_out_dev, flags);
+}
+
+mi355q_status mi355q_clock_probe_read(mi355q_context* ctx, uint64_t* shader_cycles, uint64_t* realtime_ticks) {
+    if (!ctx) return fail(MI355Q_ERR_NULL_HANDLE, "context is null");
+    if (!shader_cycles || !realtime_ticks) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null output");
+    unsigned long long cell[2] = {0, 0};
+    MI355Q_HIP(hipDeviceSynchronize());
+    MI355Q_HIP(hipMemcpy(cell, ctx->argmax_scratch + 16, sizeof cell, hipMemcpyDeviceToHost));
+    *shader_cycles = cell[0];
+    *realtime_ticks = cell[1];
+    return MI355Q_OK;
 }
 
 }  // extern "C"

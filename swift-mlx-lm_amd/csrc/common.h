@@ -171,7 +171,7 @@ mi355q_status ensure_workspace(mi355q_context* ctx, size_t bytes);
 bool gemm_mfma_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
 mi355q_status launch_qgemm_mfma(hipStream_t s, mi355q_context* ctx, const WView& w,
                                 const void* x, int x_dtype, void* y, int y_dtype, uint32_t m,
-                                uint32_t x_stride, uint32_t y_stride);
+                                uint32_t x_stride, uint32_t y_stride, unsigned long long* probe = nullptr);
 mi355q_status launch_gemm_bf16_mfma(hipStream_t s, mi355q_context* ctx, const void* a,
                                     int a_dtype, const uint16_t* b, void* c, int c_dtype,
                                     uint32_t m, uint32_t n, uint32_t k, uint32_t a_stride,

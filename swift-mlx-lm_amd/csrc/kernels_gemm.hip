@@ -42,6 +42,7 @@ struct GemmArgs {
     float* partial;          // split-K: fp32 [splits][M][N] partial results (null when K is not split)
     uint32_t kt_per_split;   // K-tiles per split (blockIdx.y indexes the split)
     uint32_t dbg;            // tuning builds only: bit0 fetch only the first K-tile, bit1 fill LDS only once
+    unsigned long long* probe;   // optional: [0] shader cycles, [1] 100 MHz ticks that workgroup 0 spent in the kernel
 };
 
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
@@ -95,6 +96,11 @@ __global__ __launch_bounds__(WAVES * 64, (STAGES == 1 ? 2 : 1)) void qgemm_mfma_
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t wm = wave / WN, wn = wave % WN;
+    // clock probe: the first wavefront of workgroup 0 times itself with the shader-clock counter and the
+    // constant 100 MHz counter; their ratio is the clock the matrix cores actually ran at
+    const bool probing = a.probe != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && wave == 0;
+    unsigned long long probe_c0 = 0, probe_r0 = 0;
+    if (probing) { probe_c0 = __builtin_readcyclecounter(); probe_r0 = __builtin_amdgcn_s_memrealtime(); }
 
     // ---- global -> register fetch and register -> LDS fill of one K-tile, in NP parts -----------
     // Part p covers X-tile passes [p*AP, (p+1)*AP) and weight chunks [p*BC, (p+1)*BC) (a chunk is 8
@@ -335,6 +341,10 @@ __global__ __launch_bounds__(WAVES * 64, (STAGES == 1 ? 2 : 1)) void qgemm_mfma_
         }
     }
 
+    if (probing) {
+        const unsigned long long c1 = __builtin_readcyclecounter(), r1 = __builtin_amdgcn_s_memrealtime();
+        if (lane == 0) { a.probe[0] = c1 - probe_c0; a.probe[1] = r1 - probe_r0; }
+    }
     // ---- epilogue: one rounding, to the output type --------------------------------------------
 #pragma unroll
     for (int i = 0; i < TM; i++)
@@ -482,7 +492,8 @@ bool gemm_mfma_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stri
 }
 
 mi355q_status launch_qgemm_mfma(hipStream_t s, mi355q_context* ctx, const WView& w, const void* x, int x_dtype,
-                                void* y, int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride) {
+                                void* y, int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride,
+                                unsigned long long* probe) {
     if (x_dtype != MI355Q_BF16) return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the MFMA GEMM takes bf16 activations");
     if ((uintptr_t)x % 16) return fail(MI355Q_ERR_INVALID_ARGUMENT, "activation pointer must be 16-byte aligned");
     GemmArgs a{};
@@ -492,6 +503,7 @@ mi355q_status launch_qgemm_mfma(hipStream_t s, mi355q_context* ctx, const WView&
     a.code_stride = w.code_stride; a.sz_stride = w.sz_stride;
     a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = w.sb_dtype;
     a.dbg = (uint32_t)env_int_cached("MI355Q_GEMM_DBG", 0);
+    a.probe = probe;
     switch (w.bits * 1000 + w.group) {
     case 4064: return launch_shape<4, 64, true>(s, ctx, a);
     case 4128: return launch_shape<4, 128, true>(s, ctx, a);
