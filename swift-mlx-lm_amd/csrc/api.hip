@@ -101,7 +101,9 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
             return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the MFMA GEMM does not accept this format, layout or stride");
         return launch_qgemm_mfma(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys, probe);
     }
-    const bool small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) || m <= 8 || !mfma_ok;
+    // the decode kernels take up to 8 rows per launch on the planes, 16 on TILE16 records
+    const uint32_t small_rows = v.layout == MI355Q_LAYOUT_TILE16 ? 16u : 8u;
+    const bool small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) || m <= small_rows || !mfma_ok;
     if (small) return run_small_m(ctx, s, w, x, x_dtype, y, y_dtype, m, xs, ys, flags);
     return launch_qgemm_mfma(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys, probe);
 }

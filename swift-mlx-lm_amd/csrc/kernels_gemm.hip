@@ -31,6 +31,7 @@ typedef float float2_v __attribute__((ext_vector_type(2)));
 
 struct GemmArgs {
     const uint32_t* codes;   // QUANT: [N, K*bits/32]
+    const uint32_t* tiles;   // QUANT on the TILE16 layout: records of 16 rows x 128 codes + 32 (scale, bias) words
     const uint32_t* sz;      // QUANT: packed (scale | bias << 16) per group
     const uint16_t* bdense;  // !QUANT: bf16 [N, K]
     const uint16_t* x;       // bf16 [M, xs]
@@ -39,6 +40,7 @@ struct GemmArgs {
     uint32_t code_stride, sz_stride;   // 32-bit words between consecutive rows
     uint32_t y_dtype, sb_dtype;
     uint32_t tiles_m, tiles_n;
+    uint32_t kblocks;        // TILE16: K / 128
     float* partial;          // split-K: fp32 [splits][M][N] partial results (null when K is not split)
     uint32_t kt_per_split;   // K-tiles per split (blockIdx.y indexes the split)
     uint32_t dbg;            // tuning builds only: bit0 fetch only the first K-tile, bit1 fill LDS only once
@@ -67,7 +69,7 @@ __device__ __forceinline__ uint32_t lds_off(uint32_t row, uint32_t chunk) {
 // dequantisation, LDS fill and barrier.
 // WAVES = 4: wavefronts 2 x 2 over the tile, one per SIMD.  WAVES = 8: 2 x 4, two per SIMD, so that
 // one wavefront's LDS waits and barrier skew are covered by the other's MFMAs.
-template <int BITS, int GROUP, int BM, int BN, bool QUANT, int STAGES, bool SB_BF16, int WAVES>
+template <int BITS, int GROUP, int BM, int BN, bool QUANT, int STAGES, bool SB_BF16, int WAVES, bool T16>
 __global__ __launch_bounds__(WAVES * 64, (STAGES == 1 ? 2 : 1)) void qgemm_mfma_kernel(GemmArgs a) {
     constexpr int NT = WAVES * 64;                        // threads
     constexpr int WN = WAVES / 2;                         // wavefronts along N (2 along M)
@@ -81,6 +83,8 @@ __global__ __launch_bounds__(WAVES * 64, (STAGES == 1 ? 2 : 1)) void qgemm_mfma_
     constexpr int NGT = QUANT ? (CPT > GROUP ? CPT / GROUP : 1) : 0;   // groups a thread touches
     constexpr int B_DENSE_PASSES = BN / RPP;
     static_assert(TPR >= 1 && CPT % 8 == 0, "weight tile does not split over the threads");
+    // TILE16 operand: 4-bit g64 records; a thread takes 32 codes (two 16-code quarters) of one row per K-tile
+    static_assert(!T16 || (QUANT && BITS == 4 && GROUP == 64 && CPT == 32), "the TILE16 fetch is written for q4 g64, 32 codes per thread");
 
     extern __shared__ uint4 smem_q[];
     char* lds = (char*)smem_q;
@@ -142,7 +146,18 @@ __global__ __launch_bounds__(WAVES * 64, (STAGES == 1 ? 2 : 1)) void qgemm_mfma_
     // packed words + (scale, bias) words of K-tile kt into (w, sz)
     auto fetch_codes = [&](uint32_t kt, uint32_t (&w)[QUANT ? WPT : 1], uint32_t (&sz)[QUANT ? NGT : 1])
                            __attribute__((always_inline)) {
-        if constexpr (QUANT) {
+        if constexpr (T16) {
+            // K-tile kt is half h of record kt / 2; row b_grow is row n of row tile rt.  Quarter kq of the half
+            // sits with lane kq * 16 + n: its words 2h and 2h + 1 hold codes kq * 16 .. + 16 of the K-tile.
+            const uint32_t rt = b_grow >> 4, n = b_grow & 15u, h = kt & 1u;
+            const uint32_t* rec = a.tiles + ((size_t)rt * a.kblocks + (kt >> 1)) * 288u;
+#pragma unroll
+            for (int q = 0; q < 2; q++) {
+                const u32x2 v = *(const u32x2*)(rec + ((b_part * 2 + q) * 16 + n) * 4 + h * 2);
+                w[2 * q] = v.x; w[2 * q + 1] = v.y;
+            }
+            sz[0] = rec[256 + n * 2 + h];
+        } else if constexpr (QUANT) {
             const uint32_t k0 = kt * kTileK;
             const uint32_t* src = a.codes + (size_t)b_grow * a.code_stride + (size_t)kt * (kTileK * BITS / 32) +
                                   b_part * WPT;
@@ -209,8 +224,16 @@ __global__ __launch_bounds__(WAVES * 64, (STAGES == 1 ? 2 : 1)) void qgemm_mfma_
                     asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(q[5]) : "v"(hi));
                     asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(q[6]) : "v"(lo));
                     asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(q[7]) : "v"(hi));
+                    if constexpr (T16) {
+                        // q[i] is nibble i of the word; record words keep their nibbles in the order
+                        // (c0,c2,c4,c6,c1,c3,c5,c7), so code e sits in nibble at[e]
+                        constexpr int at[8] = {0, 4, 1, 5, 2, 6, 3, 7};
 #pragma unroll
-                    for (int e = 0; e < 8; e++) f[e] = __builtin_fmaf(s, q[e], z);
+                        for (int e = 0; e < 8; e++) f[e] = __builtin_fmaf(s, q[at[e]], z);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 8; e++) f[e] = __builtin_fmaf(s, q[e], z);
+                    }
                 } else {
                     f[0] = __builtin_fmaf(s, (float)extract_code<(ci * 8 + 0) * BITS, BITS, (WPT ? WPT : 1)>(wreg), z);
                     f[1] = __builtin_fmaf(s, (float)extract_code<(ci * 8 + 1) * BITS, BITS, (WPT ? WPT : 1)>(wreg), z);
@@ -421,14 +444,14 @@ GemmLaunchShape gemm_mfma_shape(const mi355q_context* ctx, uint32_t m, uint32_t 
 
 namespace {
 
-template <int BITS, int GROUP, int BM, int BN, bool QUANT, int STAGES, bool SB_BF16, int WAVES>
+template <int BITS, int GROUP, int BM, int BN, bool QUANT, int STAGES, bool SB_BF16, int WAVES, bool T16>
 mi355q_status launch_tile_sb(hipStream_t s, GemmArgs a) {
     a.tiles_m = (a.m + BM - 1) / BM;
     a.tiles_n = (a.n + BN - 1) / BN;
     const uint32_t total = a.tiles_m * a.tiles_n;
     const uint32_t grid = (total + 7) / 8 * 8;
     constexpr size_t lds = (size_t)STAGES * (BM + BN) * kRowBytes;
-    auto kern = qgemm_mfma_kernel<BITS, GROUP, BM, BN, QUANT, STAGES, SB_BF16, WAVES>;
+    auto kern = qgemm_mfma_kernel<BITS, GROUP, BM, BN, QUANT, STAGES, SB_BF16, WAVES, T16>;
     static bool lds_limit_raised = false;      // per instantiation; the library drives one device
     if (!lds_limit_raised) {
         MI355Q_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
@@ -451,10 +474,16 @@ mi355q_status launch_tile_sb(hipStream_t s, GemmArgs a) {
 
 template <int BITS, int GROUP, int BM, int BN, bool QUANT, int STAGES, int WAVES = 4>
 mi355q_status launch_tile(hipStream_t s, const GemmArgs& a) {
-    if constexpr (QUANT) {
-        if (a.sb_dtype == MI355Q_BF16) return launch_tile_sb<BITS, GROUP, BM, BN, QUANT, STAGES, true, WAVES>(s, a);
+    if constexpr (QUANT && BITS == 4 && GROUP == 64 && STAGES == 2) {
+        if (a.tiles) {
+            if (a.sb_dtype == MI355Q_BF16) return launch_tile_sb<BITS, GROUP, BM, BN, QUANT, STAGES, true, WAVES, true>(s, a);
+            return launch_tile_sb<BITS, GROUP, BM, BN, QUANT, STAGES, false, WAVES, true>(s, a);
+        }
     }
-    return launch_tile_sb<BITS, GROUP, BM, BN, QUANT, STAGES, false, WAVES>(s, a);
+    if constexpr (QUANT) {
+        if (a.sb_dtype == MI355Q_BF16) return launch_tile_sb<BITS, GROUP, BM, BN, QUANT, STAGES, true, WAVES, false>(s, a);
+    }
+    return launch_tile_sb<BITS, GROUP, BM, BN, QUANT, STAGES, false, WAVES, false>(s, a);
 }
 
 template <int BITS, int GROUP, bool QUANT>
@@ -479,8 +508,10 @@ mi355q_status launch_shape(hipStream_t s, mi355q_context* ctx, GemmArgs a) {
 }  // namespace
 
 bool gemm_mfma_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
-    if (w.layout != MI355Q_LAYOUT_PLANES || x_dtype != MI355Q_BF16 || !w.sz) return false;
-    if (m < 1) return false;
+    if (x_dtype != MI355Q_BF16 || m < 1) return false;
+    if (w.layout == MI355Q_LAYOUT_TILE16)        // q4 g64 records, K % 128 == 0 by construction
+        return w.tiles && w.bits == 4 && w.group == 64 && w.k % 128 == 0 && x_stride % 8 == 0;
+    if (w.layout != MI355Q_LAYOUT_PLANES || !w.sz) return false;
     if (w.k % kTileK) return false;
     if (x_stride % 8) return false;                       // 128-bit activation loads
     if ((uintptr_t)w.codes % 16 || w.code_stride % 4) return false;
@@ -498,6 +529,7 @@ mi355q_status launch_qgemm_mfma(hipStream_t s, mi355q_context* ctx, const WView&
     if ((uintptr_t)x % 16) return fail(MI355Q_ERR_INVALID_ARGUMENT, "activation pointer must be 16-byte aligned");
     GemmArgs a{};
     a.codes = w.codes; a.sz = w.sz; a.bdense = nullptr;
+    if (w.layout == MI355Q_LAYOUT_TILE16) { a.tiles = w.tiles; a.kblocks = w.k / 128; }
     a.x = (const uint16_t*)x; a.y = y;
     a.m = m; a.n = w.n; a.k = w.k; a.xs = x_stride; a.ys = y_stride;
     a.code_stride = w.code_stride; a.sz_stride = w.sz_stride;

@@ -132,7 +132,8 @@ mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w, uint32_t maximum
     }
 
     const uint32_t m = maximum_sequence_length;
-    const bool want_small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) || m <= 8;
+    const uint32_t small_rows = v.layout == MI355Q_LAYOUT_TILE16 ? 16u : 8u;      // rows the decode kernels take per launch
+    const bool want_small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) || m <= small_rows;
     const bool mfma_ok = gemm_mfma_eligible(v, x_dtype, m, input_row_stride);
     fill_common(w, m, s);
     s->path = MI355Q_PATH_PREFILL_PROJECTION;

@@ -99,7 +99,9 @@ def test_tile16_ragged_shapes_and_long_batches(pkg, ctx):
             x = act_rounded(kat.seeded_activations(2400 + i + m, m, k), pkg.BF16, pkg)
             say(f"tile16 ragged {k}->{n} M={m}")
             got = _run(ctx, pkg, w, x, pkg.F32, use_qgemm=m > 8)
-            assert_within_tolerance(got, oracle.gemm_f64(wq, x), f"{k}->{n} M={m}")
+            # beyond 16 rows the projection runs on the prefill kernel, whose weights are rounded to bf16
+            ref_w = wq if m <= 16 else oracle.bf16_to_f32(oracle.bf16_from_f32(wq)).reshape(wq.shape)
+            assert_within_tolerance(got, oracle.gemm_f64(ref_w, x), f"{k}->{n} M={m}")
         w.destroy()
     # f16 scale words (STAF source)
     rng = np.random.default_rng(5)
@@ -194,6 +196,38 @@ def test_tile16_lm_head_fused_argmax(pkg, ctx):
     w.destroy()
     for b in (xd, logits, tok, xd2, lg2):
         b.free()
+
+
+def test_tile16_prefill_runs_on_the_matrix_cores(pkg, ctx):
+    """Above 16 rows a TILE16 weight feeds the prefill GEMM directly from its records.  The arithmetic is that of
+    the same kernel on the split planes (same bf16 weights, same contraction order): identical bits; the plan
+    record names the matrix-core kernel."""
+    for i, (m, n, k) in enumerate([(17, 130, 2048 + 128), (64, 4099, 384), (300, 257, 128), (512, 4096, 4096),
+                                   (2048, 1024, 512)]):
+        words, s, z, wq = seeded_case(2700 + i, n, k, 4, 64)
+        wt = ctx.weight_prepare_mlx(_fmt(pkg), words, s, z, pkg.BF16, pkg.LAYOUT_TILE16)
+        wp = ctx.weight_prepare_mlx(_fmt(pkg), words, s, z, pkg.BF16, pkg.LAYOUT_PLANES)
+        x = act_rounded(kat.seeded_activations(2750 + i, m, k), pkg.BF16, pkg)
+        say(f"tile16 prefill {k}->{n} M={m}")
+        got = _run(ctx, pkg, wt, x, pkg.F32, use_qgemm=True)
+        same = _run(ctx, pkg, wp, x, pkg.F32, use_qgemm=True, flags=pkg.FLAG_FORCE_MFMA)
+        assert np.array_equal(got, same), f"{k}->{n} M={m}: records and planes disagree"
+        if m * n * k <= 2 ** 28:
+            wb = oracle.bf16_to_f32(oracle.bf16_from_f32(wq)).reshape(wq.shape)
+            assert_within_tolerance(got, oracle.gemm_f64(wb, x), f"{k}->{n} M={m}")
+        st = wt.plan_prefill_steps(m)[0]
+        assert st.device_kernel == "qgemm_mfma_q4_g64" and not st.used_fallback
+        wt.destroy(); wp.destroy()
+    # f16 scale words (a STAF source)
+    rng = np.random.default_rng(6)
+    n, k, m = 96, 256, 40
+    case = Case(4, 64, rng.integers(0, 16, (n, k), dtype=np.uint8), rng.choice([0.0625, 0.125], (n, k // 64)),
+                rng.integers(-8, 8, (n, k // 64)) * 0.0625)
+    wt = ctx.weight_prepare_staf(_fmt(pkg), n, k, case.staf_blocks(), pkg.LAYOUT_TILE16)
+    x = act_rounded(kat.seeded_activations(2790, m, k), pkg.BF16, pkg)
+    wq = (case.scales.repeat(64, axis=1) * case.codes + case.zeros.repeat(64, axis=1)).astype(np.float32)
+    assert_within_tolerance(_run(ctx, pkg, wt, x, pkg.F32, use_qgemm=True), oracle.gemm_f64(wq, x), "f16 scales")   # exact in bf16
+    wt.destroy()
 
 
 def test_tile16_errors_and_plan_records(pkg, ctx):
