@@ -270,6 +270,19 @@ def main():
     log(f"  copy  {gate_bytes} B: {ms_copy * 1e3:.2f} us/launch, {2 * gate_bytes / (ms_copy * 1e-3) / 1e9:.1f} GB/s "
         "read+write")
 
+    # ---- what HBM delivers to one launch of the dominant launch's size: a kernel that only reads that many bytes
+    # (cold: eight buffers in rotation, as the weights of the layer copies are)
+    probe_copies = 8
+    pbuf = ctx.alloc(probe_copies * dom_bytes)
+    ctx.fill(pbuf, 0x01020304, stream)
+    ctx.synchronize(stream)
+    ms_read = time_region(ctx, lambda i: ctx.read_probe(pbuf.ptr + (i % probe_copies) * dom_bytes, dom_bytes, stream),
+                          64, stream)
+    stream_read = {"bytes": dom_bytes, "us": round(ms_read * 1e3, 2), "GBps": round(dom_bytes / (ms_read * 1e-3) / 1e9, 1)}
+    log(f"  read-only launch of {dom_bytes} B: {stream_read['us']} us, {stream_read['GBps']} GB/s "
+        f"(the {dom} launch reaches {achieved / stream_read['GBps'] * 100:.0f} % of it)")
+    pbuf.free()
+
     # ---- secondary figure: the prefill GEMM of the same layer's gate projection (not the metric)
     prefill = None
     if not a.no_prefill:
@@ -325,7 +338,7 @@ def main():
                    "weight_bytes_per_step": layer_bytes, "layers_resident": a.layers,
                    "replay": mode, "replay_GBps": replay_gbps,
                    "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2), "per_shape": per_shape,
-                   "batch_sweep": batch_sweep, "prefill_gemm_gate": prefill},
+                   "batch_sweep": batch_sweep, "stream_read_probe": stream_read, "prefill_gemm_gate": prefill},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": TRAFFIC_BYTES[dom],
                      "algorithmic_bytes": dom_bytes,

@@ -449,6 +449,11 @@ MI355Q_API mi355q_status mi355q_plan_graph_launch(mi355q_plan* plan, void* strea
  * traffic counters).  Both pointers 16-byte aligned, bytes a multiple of 16. */
 MI355Q_API mi355q_status mi355q_buffer_copy(mi355q_context* ctx, void* stream, void* dst_dev,
                                             const void* src_dev, size_t bytes);
+/* Measurement aid without a counterpart in the reference: one launch that only reads `bytes` of device memory
+ * with the load instructions the decode kernels use for weights.  Its duration is what HBM delivers to a launch of
+ * that size on this part: the practical ceiling the decode GEMV is compared with.  16-byte aligned pointer and size. */
+MI355Q_API mi355q_status mi355q_buffer_read_probe(mi355q_context* ctx, void* stream, const void* src_dev,
+                                                  size_t bytes);
 
 /* ------------------------------------------------------------------------------------------
  * STAF container (model.staf): reader, validator, writer

@@ -168,6 +168,7 @@ def library() -> C.CDLL:
         "mi355q_plan_graph_build": (i32, [vp, vp]),
         "mi355q_plan_graph_launch": (i32, [vp, vp]),
         "mi355q_buffer_copy": (i32, [vp, vp, vp, vp, sz]),
+        "mi355q_buffer_read_probe": (i32, [vp, vp, vp, sz]),
         "mi355q_clock_probe_read": (i32, [vp, P(u64), P(u64)]),
         "mi355q_kv_scheme_is_supported": (i32, [u8]),
         "mi355q_kv_bytes_per_head_slot": (u32, [u8, u32]),
@@ -692,6 +693,10 @@ class Context:
         if a.nbytes:
             b.upload(a)
         return b
+
+    def read_probe(self, src, nbytes: int, stream: int = 0):
+        """One launch that only streams `nbytes` of `src` from HBM (the ceiling a decode launch is compared with)."""
+        _check(library().mi355q_buffer_read_probe(self.handle, stream, self._ptr(src), nbytes))
 
     def copy(self, dst, src, nbytes: int, stream: int = 0):
         _check(library().mi355q_buffer_copy(self.handle, stream, self._ptr(dst), self._ptr(src), nbytes))

@@ -6,6 +6,7 @@
 #include <vector>
 
 #include "common.h"
+#include "device_utils.h"
 
 using namespace mi355q;
 
@@ -247,6 +248,36 @@ __global__ void copy_kernel(uint4* __restrict__ dst, const uint4* __restrict__ s
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     for (; i < n_vec; i += stride) dst[i] = src[i];
+}
+
+// Streaming read of a buffer with the loads the decode kernels use for weights (128-bit, non-temporal, four in
+// flight per lane) and nothing else: what HBM delivers to a launch of this size on this part.
+__global__ __launch_bounds__(256) void read_probe_kernel(const mi355q::u32x4* __restrict__ src, size_t n_vec, uint32_t* __restrict__ sink) {
+    const size_t base = (size_t)blockIdx.x * 1024 + threadIdx.x;
+    mi355q::u32x4 v[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const size_t idx = base + (size_t)i * 256;
+        v[i] = __builtin_nontemporal_load(src + (idx < n_vec ? idx : 0));
+    }
+    uint32_t acc = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) acc ^= v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
+    if (acc == 0x9E3779B9u) sink[0] = acc;      // keeps the loads alive; practically never taken
+}
+
+mi355q_status mi355q_buffer_read_probe(mi355q_context* ctx, void* stream, const void* src_dev, size_t bytes) {
+    if (!ctx) return fail(MI355Q_ERR_NULL_HANDLE, "context is null");
+    if (!src_dev || bytes == 0 || bytes % 16 || (uintptr_t)src_dev % 16)
+        return fail(MI355Q_ERR_INVALID_ARGUMENT, "read_probe needs a 16-byte aligned pointer and a positive size that is a multiple of 16");
+    MI355Q_HIP(hipSetDevice(ctx->device));
+    const size_t n_vec = bytes / 16;
+    const size_t blocks = (n_vec + 1023) / 1024;
+    if (blocks > 0x7FFFFFFFull) return fail(MI355Q_ERR_INVALID_ARGUMENT, "buffer too large for one launch");
+    read_probe_kernel<<<dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream>>>(
+        (const mi355q::u32x4*)src_dev, n_vec, (uint32_t*)(ctx->argmax_scratch + 24));
+    MI355Q_HIP(hipGetLastError());
+    return MI355Q_OK;
 }
 
 mi355q_status mi355q_buffer_copy(mi355q_context* ctx, void* stream, void* dst_dev, const void* src_dev, size_t bytes) {
