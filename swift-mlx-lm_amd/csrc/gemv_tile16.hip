@@ -17,9 +17,9 @@
 // A wavefront reads a record with one 128-bit and one 64-bit load per lane and feeds four
 // v_mfma_f32_16x16x32_bf16 per group pair: codes become bf16 (128 + q) with one and-or each, the
 // activations are the A operand straight from LDS (natural order, no permutation), the matrix core
-// does every multiply-add, and a second MFMA against a tile of ones gives sum(x) over the same k.
-// Per group the VALU applies the affine form once per kept output row:
-//   acc += s * D + (z - 128 s) * D1        (D = sum (128+q) x,  D1 = sum x).
+// does every multiply-add; sum(x) per group and activation row is computed once per workgroup while the
+// activations are staged.  Per group the VALU applies the affine form once per kept output row:
+//   acc += s * D + (z - 128 s) * SX        (D = sum (128+q) x,  SX = sum x).
 // The accumulator of lane (kq, n) holds output rows m = 4 kq .. 4 kq + 3 of weight row n, so there is
 // no cross-lane reduction at all; the WAVES wavefronts of a workgroup split K and add their partial
 // tiles through LDS at the end.
@@ -29,6 +29,12 @@ namespace mi355q {
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4_t;
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float float2_t;
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 t16_bf16x2_t;
+
+__device__ __forceinline__ float t16_dot2(uint32_t a, uint32_t b, float acc) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(t16_bf16x2_t, a), __builtin_bit_cast(t16_bf16x2_t, b), acc, false);
+}
 
 struct T16Args {
     const uint32_t* tiles[kTile16MaxSegments];   // TILE16 buffers of up to three matrices sharing x
@@ -117,14 +123,30 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
     static_for<D>([&](auto J) { issue(b_first + decltype(J)::value, ring[decltype(J)::value]); });
 
     // ---- 3. stage the activations (waits only for the loads of step 1) --------------------------
+    // With each 16-byte chunk goes its share of sum(x): eight consecutive lanes hold the eight chunks of one
+    // 64-element group of one row, so three xor-shuffles give the group sum, kept as sxs[group][row].
+    float* const sxs = (float*)(lds + (size_t)a.m * a.lds_row_bytes);
     {
         const uint32_t total = a.m * chunks;
+        auto stage = [&](uint32_t idx, const u32x4& v) {
+            float p = t16_dot2(v.x, 0x3F803F80u, 0.0f);
+            p = t16_dot2(v.y, 0x3F803F80u, p);
+            p = t16_dot2(v.z, 0x3F803F80u, p);
+            p = t16_dot2(v.w, 0x3F803F80u, p);
+            p += __shfl_xor(p, 1);
+            p += __shfl_xor(p, 2);
+            p += __shfl_xor(p, 4);
+            if (idx < total) {
+                *x_dst(idx) = v;
+                uint32_t m, c;
+                x_row(idx, m, c);
+                if ((c & 7u) == 0) sxs[(c >> 3) * 16 + m] = p;
+            }
+        };
 #pragma unroll
-        for (int t = 0; t < XC; t++) {
-            const uint32_t idx = tid + t * WAVES * 64;
-            if (idx < total) *x_dst(idx) = xe[t];
-        }
-        for (uint32_t idx = tid + XC * WAVES * 64; idx < total; idx += WAVES * 64) *x_dst(idx) = *x_src(idx);
+        for (int t = 0; t < XC; t++) stage(tid + t * WAVES * 64, xe[t]);
+        // whole wavefronts take part in the shuffles: the loop bound is rounded up to the workgroup size
+        for (uint32_t base = XC * WAVES * 64; base < total; base += WAVES * 64) stage(base + tid, *x_src(base + tid));
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __builtin_amdgcn_s_barrier();
@@ -134,11 +156,6 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
     uint32_t k_mask = 0x000F000Fu, k_magic = 0x43004300u;   // opaque: keeps (w & mask) | magic one v_and_or_b32
     asm volatile("" : "+s"(k_mask));
     asm volatile("" : "+v"(k_magic));
-    bf16x8_t ones;
-    {
-        u32x4 o = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
-        ones = __builtin_bit_cast(bf16x8_t, o);
-    }
     floatx4_t zero4 = {0.f, 0.f, 0.f, 0.f};
     float acc[MR];
 #pragma unroll
@@ -166,8 +183,12 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
             const bf16x8_t b1 = unpack(g == 0 ? r.w.y : r.w.w);
             floatx4_t d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, b0, zero4, 0, 0, 0);
             d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b1, d, 0, 0, 0);
-            floatx4_t d1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, ones, zero4, 0, 0, 0);
-            d1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, ones, d1, 0, 0, 0);
+            // sum(x) of this group for output rows 4 kq .. 4 kq + MR - 1
+            const float* const sxp = sxs + (size_t)(b * 2 + g) * 16 + 4 * kq;
+            float sx[MR];
+            if constexpr (MR == 4) { const floatx4_t t = *(const floatx4_t*)sxp; sx[0] = t[0]; sx[1] = t[1]; sx[2] = t[2]; sx[3] = t[3]; }
+            else if constexpr (MR == 2) { const float2_t t = *(const float2_t*)sxp; sx[0] = t[0]; sx[1] = t[1]; }
+            else sx[0] = sxp[0];
             const uint32_t szw = g == 0 ? r.sz.x : r.sz.y;
             float s, z;
             if (a.sb_dtype == MI355Q_BF16) {                // wavefront-uniform
@@ -179,7 +200,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
             }
             const float zc = z - 128.0f * s;
 #pragma unroll
-            for (int q = 0; q < MR; q++) acc[q] += s * d[q] + zc * d1[q];
+            for (int q = 0; q < MR; q++) acc[q] += s * d[q] + zc * sx[q];
         });
     };
 
@@ -289,7 +310,7 @@ bool gemv_tile16_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_st
     if (m < 1 || m > 16) return false;
     if (w.bits != 4 || w.group != 64 || w.k % 128) return false;
     if (x_stride % 8) return false;                                   // 128-bit activation loads
-    return (size_t)m * ((size_t)w.k * 2 + 16) <= kT16LdsBudget;       // staged activations fit in LDS
+    return (size_t)m * ((size_t)w.k * 2 + 16) + w.k <= kT16LdsBudget; // staged activations and their group sums fit in LDS
 }
 
 Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_total_tiles, uint32_t k, uint32_t m) {
@@ -319,7 +340,7 @@ Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_total_
     g.blocks_per_wave = (kblocks + ks - 1) / ks;
     g.grid = (n_total_tiles + tpw - 1) / tpw;
     g.block = g.waves * 64;
-    const size_t x_bytes = (size_t)m * ((size_t)k * 2 + 16);
+    const size_t x_bytes = (size_t)m * ((size_t)k * 2 + 16) + k;     // rows, then sum(x) per group: [K/64][16] floats
     const size_t red_bytes = (size_t)g.waves * 4 * 64 * 4;
     g.lds_bytes = (uint32_t)(x_bytes > red_bytes ? x_bytes : red_bytes);
     return g;
