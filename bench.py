@@ -89,6 +89,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-parity", action="store_true")
     ap.add_argument("--no-prefill", action="store_true", help="skip the secondary prefill-GEMM figure")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip the secondary per-launch figures of BASELINE configs 0, 2 and 4")
     ap.add_argument("--no-batch-sweep", action="store_true", help="skip the secondary M = 1, 2, 4, 8 figures")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -270,6 +272,54 @@ def main():
     log(f"  copy  {gate_bytes} B: {ms_copy * 1e3:.2f} us/launch, {2 * gate_bytes / (ms_copy * 1e-3) / 1e9:.1f} GB/s "
         "read+write")
 
+    # ---- secondary: one launch each of BASELINE config 0 (2048->8192), config 2 (4096->14336 at 8, 6, 3 and 2 bits)
+    # and config 4 (LM head 2048->65536 fused with argmax), over rotating copies of more than 512 MB in total
+    other = None
+    if not a.no_other_configs:
+        other = {}
+        cases = [("config0 q4g64 2048->8192", 4, 64, 8192, 2048, False), ("config2 q8g32 4096->14336", 8, 32, 14336, 4096, False),
+                 ("config2 q6g64 4096->14336", 6, 64, 14336, 4096, False), ("config2 q3g64 4096->14336", 3, 64, 14336, 4096, False),
+                 ("config2 q2g64 4096->14336", 2, 64, 14336, 4096, False), ("config4 q4g64 lm head 2048->65536 + argmax", 4, 64, 65536, 2048, True)]
+        for ci, (label, bits, group, n, k, head) in enumerate(cases):
+            f2 = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(bits, group)
+            words, s, z = oracle.quantize_affine(kat.seeded_weights(3000 + ci, n, k), bits, group, oracle.BF16)
+            nbytes = n * (k // group) * (4 + group * bits // 8)
+            copies = max(2, min(64, int(5.4e8 // nbytes) + 1))
+            ws = [ctx.weight_prepare_mlx(f2, words, s, z, pkg.BF16, pkg.LAYOUT_PLANES) for _ in range(copies)]
+            x1 = oracle.bf16_to_f32(oracle.bf16_from_f32(kat.seeded_activations(3100 + ci, 1, k))).reshape(1, k)
+            xd1 = ctx.upload(oracle.bf16_from_f32(x1))
+            yd1, logits, tok = ctx.alloc(n * 2), ctx.alloc(n * 4), ctx.alloc(16)
+            pl = pkg.DispatchPlan(ctx)
+            for w in ws:
+                if head:
+                    pl.add_output_head(w, xd1, pkg.BF16, logits, tok)
+                else:
+                    pl.add_linear(w, xd1, pkg.BF16, yd1, pkg.BF16, 1)
+            pl.encode(stream)
+            ctx.synchronize(stream)
+            if not a.skip_parity:                       # the launch just timed is checked before its number is used
+                wq = oracle.dequant_planes_f32(bits, group, n, k, words, s, z, oracle.BF16)
+                want = oracle.gemm_f64(wq, x1)[0]
+                if head:
+                    got = logits.download(np.float32)
+                    t = int(tok.download(np.int32)[0])
+                    if t != oracle.argmax_lowest(got):
+                        sys.exit(f"bench.py: {label}: token {t} is not the lowest-index argmax of the logits")
+                else:
+                    got = oracle.bf16_to_f32(yd1.download(np.uint16))
+                    want = oracle.bf16_to_f32(oracle.bf16_from_f32(want.astype(np.float32)))
+                rel = float(np.linalg.norm(got - want) / np.linalg.norm(want))
+                if rel > (1e-3 if head else 4e-3):      # bf16 outputs carry their own rounding
+                    sys.exit(f"bench.py: parity gate failed on {label}: rel-L2 {rel:.3e}")
+            ms = time_region(ctx, lambda i: pl.encode(stream), 6, stream) / copies
+            other[label] = {"us": round(ms * 1e3, 2), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1), "weight_bytes": nbytes}
+            log(f"  {label}: {other[label]['us']} us/launch, {other[label]['GBps']} GB/s")
+            pl.destroy()
+            for w in ws:
+                w.destroy()
+            for b in (xd1, yd1, logits, tok):
+                b.free()
+
     # ---- what HBM delivers to one launch of the dominant launch's size: a kernel that only reads that many bytes
     # (cold: eight buffers in rotation, as the weights of the layer copies are)
     probe_copies = 8
@@ -338,7 +388,8 @@ def main():
                    "weight_bytes_per_step": layer_bytes, "layers_resident": a.layers,
                    "replay": mode, "replay_GBps": replay_gbps,
                    "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2), "per_shape": per_shape,
-                   "batch_sweep": batch_sweep, "stream_read_probe": stream_read, "prefill_gemm_gate": prefill},
+                   "batch_sweep": batch_sweep, "other_configs": other, "stream_read_probe": stream_read,
+                   "prefill_gemm_gate": prefill},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": TRAFFIC_BYTES[dom],
                      "algorithmic_bytes": dom_bytes,

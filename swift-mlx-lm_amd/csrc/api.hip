@@ -159,12 +159,12 @@ mi355q_status dispatch_output_head(mi355q_context* ctx, hipStream_t s, const mi3
     const uint32_t xs = (uint32_t)w->k;
     if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && gemv_fast_eligible(v, x_dtype, 1, xs) && (uintptr_t)x % 16 == 0)
         return launch_gemv_fast(s, ctx, v, x, nullptr, MI355Q_F32, 1, xs, (uint32_t)w->n, logits, token,
-                                ctx->argmax_scratch);
+                                ctx->argmax_partials);
     if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && gemv_tile16_eligible(v, x_dtype, 1, xs) && (uintptr_t)x % 16 == 0) {
         void* none[1] = {nullptr};
         const uint32_t strides[1] = {(uint32_t)w->n};
         return launch_gemv_tile16_multi(s, ctx, 1, &v, x, none, strides, MI355Q_F32, 1, xs, logits, token,
-                                        ctx->argmax_scratch);
+                                        ctx->argmax_partials);
     }
     // two dispatches, as the reference runs the head: projection to fp32 logits, then argmax
     if (!logits)

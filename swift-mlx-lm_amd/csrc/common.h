@@ -54,8 +54,10 @@ struct WView {
 struct mi355q_context {
     int device;
     hipDeviceProp_t props;
-    // scratch of the fused LM-head/argmax launch: [0] packed (key,~index) maximum, [1] ticket
+    // small cells: [16..17] clock probe of the prefill GEMM, [24] sink of the read-only probe launch
     unsigned long long* argmax_scratch;
+    // fused output head: one packed (ordered value, ~row) key per workgroup of the projection launch
+    unsigned long long* argmax_partials;
     // split-K partial results of the prefill GEMM: grown on demand, never shrunk
     void* workspace;
     size_t workspace_bytes;
@@ -115,6 +117,9 @@ mi355q_status launch_gemv_generic(hipStream_t s, const WView& w, const void* x, 
 mi355q_status launch_embedding_lookup(hipStream_t s, const WView& w, const int32_t* token_ids, uint32_t sequence_length,
                                       void* out, int out_dtype, uint32_t out_stride, int has_scale,
                                       float embedding_scale);
+// Partial keys of the fused output head: one per workgroup of the projection launch.
+constexpr uint32_t kArgmaxPartialCapacity = 65536;
+mi355q_status launch_argmax_finish(hipStream_t s, const unsigned long long* partial, uint32_t count, int32_t* token_out);
 mi355q_status launch_argmax(hipStream_t s, const void* logits, int dtype, uint32_t n,
                             int32_t* token_out);
 mi355q_status launch_pack_sz(hipStream_t s, const uint16_t* scales, const uint16_t* biases, uint32_t* sz,

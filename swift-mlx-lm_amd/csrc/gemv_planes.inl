@@ -50,7 +50,7 @@ struct GemvArgs {
     const uint16_t* x;       // bf16 [M, x_stride]
     float* logits;           // optional fp32 [N] copy (M == 1, single segment)
     int32_t* token_out;      // ARGMAX only
-    unsigned long long* scratch;  // ARGMAX only: [0] packed max, [1] ticket
+    unsigned long long* scratch;  // ARGMAX only: one packed (ordered value, ~row) key per workgroup; 0 = no candidate
     uint32_t k, m;
     uint32_t x_stride;
     uint32_t code_stride, sz_stride;   // 32-bit words between consecutive rows
@@ -552,10 +552,11 @@ void gemv_planes_kernel(GemvArgs a) {
     }
 
     if constexpr (ARGMAX) {
-        // Per-lane candidates -> wavefront maximum (butterfly on the packed 64-bit key), one atomic
-        // per wavefront, then a ticket: the workgroup that draws the last ticket publishes the
-        // token and leaves the scratch cells zeroed again.
-        __shared__ uint32_t s_last;
+        // Per-lane candidates -> wavefront maximum (butterfly on the packed 64-bit key) -> workgroup maximum
+        // through LDS -> one plain store per workgroup into the partial-key array.  A one-workgroup launch
+        // (argmax_finish_kernel) then picks the token: same-address atomics from thousands of workgroups
+        // serialise across the XCDs and would cost more than the projection itself.
+        __shared__ unsigned long long s_best[WAVES];
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) {
             const uint32_t hi = (uint32_t)__shfl_xor((int)(best >> 32), off, 64);
@@ -563,19 +564,13 @@ void gemv_planes_kernel(GemvArgs a) {
             const unsigned long long o = ((unsigned long long)hi << 32) | lo;
             best = o > best ? o : best;
         }
-        if (lane == 0 && best) atomicMax(&a.scratch[0], best);
-        __threadfence();
+        if (lane == 0) s_best[wave] = best;
         __syncthreads();
         if (tid == 0) {
-            const unsigned long long t = atomicAdd(&a.scratch[1], 1ull);
-            s_last = (t == (unsigned long long)gridDim.x - 1ull) ? 1u : 0u;
-        }
-        __syncthreads();
-        if (s_last && tid == 0) {
-            __threadfence();
-            const unsigned long long pk = atomicExch(&a.scratch[0], 0ull);
-            a.token_out[0] = pk ? (int32_t)(0xFFFFFFFFu - (uint32_t)(pk & 0xFFFFFFFFull)) : 0;
-            atomicExch(&a.scratch[1], 0ull);
+            unsigned long long m = s_best[0];
+#pragma unroll
+            for (int w2 = 1; w2 < WAVES; w2++) m = s_best[w2] > m ? s_best[w2] : m;
+            a.scratch[blockIdx.x] = m;
         }
     }
 }

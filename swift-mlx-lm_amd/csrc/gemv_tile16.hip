@@ -45,7 +45,7 @@ struct T16Args {
     const uint16_t* x;                           // bf16 [M, x_stride]
     float* logits;                               // optional fp32 [N] copy (M == 1, one matrix)
     int32_t* token_out;                          // ARGMAX only
-    unsigned long long* scratch;                 // ARGMAX only: [0] packed max, [1] ticket
+    unsigned long long* scratch;                 // ARGMAX only: one packed key per workgroup; 0 = no candidate
     uint32_t k, m, x_stride;
     uint32_t kblocks;                            // K / 128
     uint32_t blocks_per_wave;                    // K-blocks per wavefront (K split over the workgroup)
@@ -248,31 +248,23 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
         }
     }
     if constexpr (ARGMAX) {
-        // wavefront maximum of the packed (ordered value, ~row) key, one atomic per workgroup, then a
-        // ticket: the workgroup that draws the last ticket publishes the token and re-zeroes the cells
-        __shared__ uint32_t s_last;
-        if (slice == 0) {
+        // wavefront maximum of the packed (ordered value, ~row) key, workgroup maximum through LDS, one plain
+        // store per workgroup; argmax_finish_kernel picks the token from the partial keys
+        __shared__ unsigned long long s_best[WAVES];
 #pragma unroll
-            for (int off = 32; off > 0; off >>= 1) {
-                const uint32_t hi = (uint32_t)__shfl_xor((int)(best >> 32), off, 64);
-                const uint32_t lo = (uint32_t)__shfl_xor((int)(best & 0xFFFFFFFFull), off, 64);
-                const unsigned long long o = ((unsigned long long)hi << 32) | lo;
-                best = o > best ? o : best;
-            }
-            if (lane == 0 && best) atomicMax(&a.scratch[0], best);
+        for (int off = 32; off > 0; off >>= 1) {
+            const uint32_t hi = (uint32_t)__shfl_xor((int)(best >> 32), off, 64);
+            const uint32_t lo = (uint32_t)__shfl_xor((int)(best & 0xFFFFFFFFull), off, 64);
+            const unsigned long long o = ((unsigned long long)hi << 32) | lo;
+            best = o > best ? o : best;
         }
-        __threadfence();
+        if (lane == 0) s_best[wave] = best;               // 0 for the wavefronts that hold no result rows
         __syncthreads();
         if (tid == 0) {
-            const unsigned long long t = atomicAdd(&a.scratch[1], 1ull);
-            s_last = (t == (unsigned long long)gridDim.x - 1ull) ? 1u : 0u;
-        }
-        __syncthreads();
-        if (s_last && tid == 0) {
-            __threadfence();
-            const unsigned long long pk = atomicExch(&a.scratch[0], 0ull);
-            a.token_out[0] = pk ? (int32_t)(0xFFFFFFFFu - (uint32_t)(pk & 0xFFFFFFFFull)) : 0;
-            atomicExch(&a.scratch[1], 0ull);
+            unsigned long long m = s_best[0];
+#pragma unroll
+            for (int w2 = 1; w2 < WAVES; w2++) m = s_best[w2] > m ? s_best[w2] : m;
+            a.scratch[blockIdx.x] = m;
         }
     }
 }
@@ -376,7 +368,13 @@ mi355q_status launch_gemv_tile16_multi(hipStream_t s, const mi355q_context* ctx,
     a.lds_row_bytes = w[0].k * 2 + 16;
     a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = w[0].sb_dtype;
     const int mr = m == 1 ? 1 : m == 2 ? 2 : 4;
-    if (argmax) return launch_t16_shape<1, true>(s, a, g);
+    if (argmax) {
+        if (g.grid > kArgmaxPartialCapacity)
+            return fail(MI355Q_ERR_SHAPE, "the fused output head keeps one partial key per workgroup: %u workgroups exceed %u",
+                        g.grid, kArgmaxPartialCapacity);
+        if (mi355q_status st = launch_t16_shape<1, true>(s, a, g)) return st;
+        return launch_argmax_finish(s, argmax_scratch, g.grid, token_out);
+    }
     if (mr == 1) return launch_t16_shape<1, false>(s, a, g);
     if (mr == 2) return launch_t16_shape<2, false>(s, a, g);
     return launch_t16_shape<4, false>(s, a, g);

@@ -176,6 +176,9 @@ mi355q_status launch_gemv_fast_multi(hipStream_t s, const mi355q_context* ctx, u
         a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = all.sb_dtype;
         a.dbg = (uint32_t)env_int("MI355Q_GEMV_DBG", 0);
         c.grid = grid;                        // whole wavefronts per matrix: a few more than rows / rows_per_wave
+        if (argmax && grid > kArgmaxPartialCapacity)
+            return fail(MI355Q_ERR_SHAPE, "the fused output head keeps one partial key per workgroup: %u workgroups exceed %u",
+                        grid, kArgmaxPartialCapacity);
         mi355q_status st;
         switch (all.bits) {
         case 2: st = launch_gemv_planes_q2(s, a, (int)all.group, c); break;
@@ -187,6 +190,8 @@ mi355q_status launch_gemv_fast_multi(hipStream_t s, const mi355q_context* ctx, u
         default: st = fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no split-plane GEMV for %u-bit codes", all.bits);
         }
         if (st != MI355Q_OK) return st;
+        if (argmax)
+            if (mi355q_status fin = launch_argmax_finish(s, argmax_scratch, grid, token_out)) return fin;
     }
     return MI355Q_OK;
 }

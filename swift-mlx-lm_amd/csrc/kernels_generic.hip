@@ -238,6 +238,38 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const void* __restrict__ l
     }
 }
 
+// Second step of the fused output head: the maximum of the packed (ordered value, ~row) keys the projection's
+// workgroups left behind, one key each; 0 means "no finite candidate".  Keys order by value first and by lower
+// row second, so the plain maximum is the lowest index holding the maximum.
+__global__ __launch_bounds__(1024) void argmax_finish_kernel(const unsigned long long* __restrict__ partial, uint32_t count,
+                                                             int32_t* __restrict__ result) {
+    __shared__ unsigned long long s_key[16];
+    unsigned long long best = 0ull;
+    for (uint32_t i = threadIdx.x; i < count; i += 1024) {
+        const unsigned long long k = partial[i];
+        best = k > best ? k : best;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const uint32_t hi = (uint32_t)__shfl_xor((int)(best >> 32), off, 64);
+        const uint32_t lo = (uint32_t)__shfl_xor((int)(best & 0xFFFFFFFFull), off, 64);
+        const unsigned long long o = ((unsigned long long)hi << 32) | lo;
+        best = o > best ? o : best;
+    }
+    if ((threadIdx.x & 63) == 0) s_key[threadIdx.x >> 6] = best;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int i = 1; i < 16; i++) best = s_key[i] > best ? s_key[i] : best;
+        result[0] = best ? (int32_t)(0xFFFFFFFFu - (uint32_t)(best & 0xFFFFFFFFull)) : 0;
+    }
+}
+
+mi355q_status launch_argmax_finish(hipStream_t s, const unsigned long long* partial, uint32_t count, int32_t* token_out) {
+    argmax_finish_kernel<<<dim3(1), dim3(1024), 0, s>>>(partial, count, token_out);
+    MI355Q_HIP(hipGetLastError());
+    return MI355Q_OK;
+}
+
 mi355q_status launch_argmax(hipStream_t s, const void* logits, int dtype, uint32_t n, int32_t* token_out) {
     switch (dtype) {
     case MI355Q_F16: argmax_kernel<MI355Q_F16><<<dim3(1), dim3(1024), 0, s>>>(logits, n, token_out); break;
