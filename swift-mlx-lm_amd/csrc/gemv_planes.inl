@@ -118,7 +118,9 @@ void gemv_planes_kernel(GemvArgs a) {
     constexpr int SR = CPL < GROUP ? CPL : GROUP;       // codes of one group inside a lane chunk
     constexpr int NSR = CPL / SR;                       // sub-runs (groups touched) per lane chunk
     constexpr int KC = 64 * CPL;                        // codes per wavefront K-step
-    constexpr float OFS = G::PAIRS ? 128.0f : 0.0f;     // magic offset carried by the bf16 codes
+    // 3-, 5- and 6-bit codes are also fed to v_dot2 as bf16 (128 + q): the field fits the 7 mantissa bits
+    constexpr bool SMALL_FIELD = BITS == 3 || BITS == 5 || BITS == 6;
+    constexpr float OFS = (G::PAIRS || SMALL_FIELD) ? 128.0f : 0.0f;     // magic offset carried by the bf16 codes
     constexpr int XC = XREG ? XREG : 1;                 // K-steps cached in registers
     static_assert(XREG == 0 || (MT == 1 && R == 1), "register-resident activations are for M == 1, R == 1");
     static_assert(XREG == 0 || D % XREG == 0, "ring depth must be a multiple of the K-steps per row");
@@ -420,6 +422,29 @@ void gemv_planes_kernel(GemvArgs a) {
                         pr[2] = ((wv >> 4) & k_mask) | k_magic;
                         pr[3] = ((wv >> 6) & k_mask) | k_magic;
                     }
+#pragma unroll
+                    for (int m = 0; m < MT; m++) {
+                        float dsum = dot[r][m][sr];
+                        dsum = dot2_bf16(pr[0], xv[m].x, dsum);
+                        dsum = dot2_bf16(pr[1], xv[m].y, dsum);
+                        dsum = dot2_bf16(pr[2], xv[m].z, dsum);
+                        dsum = dot2_bf16(pr[3], xv[m].w, dsum);
+                        dot[r][m][sr] = dsum;
+                    }
+                }
+            } else if constexpr (SMALL_FIELD) {
+                // codes 2i and 2i+1 of this piece side by side as bf16 (128 + q): two field extracts (funnel
+                // shifts where a code straddles words), one shift-or and the magic, then v_dot2 against the
+                // activation pair in natural order -- no int->float conversion and no bf16->fp32 unpack of x
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    uint32_t pr[4];
+                    static_for<4>([&](auto I) {
+                        constexpr int i = decltype(I)::value;
+                        const uint32_t qa = extract_code<(p * 8 + 2 * i) * BITS, BITS, WPL>(cur.w[r]);
+                        const uint32_t qb = extract_code<(p * 8 + 2 * i + 1) * BITS, BITS, WPL>(cur.w[r]);
+                        pr[i] = ((qb << 16) | qa) | k_magic;
+                    });
 #pragma unroll
                     for (int m = 0; m < MT; m++) {
                         float dsum = dot[r][m][sr];

@@ -474,12 +474,13 @@ mi355q_status launch_tile_sb(hipStream_t s, GemmArgs a) {
 
 template <int BITS, int GROUP, int BM, int BN, bool QUANT, int STAGES, int WAVES = 4>
 mi355q_status launch_tile(hipStream_t s, const GemmArgs& a) {
-    if constexpr (QUANT && BITS == 4 && GROUP == 64 && STAGES == 2) {
+    if constexpr (QUANT && BITS == 4 && GROUP == 64 && STAGES == 2 && WAVES * 64 == 2 * BN) {
         if (a.tiles) {
             if (a.sb_dtype == MI355Q_BF16) return launch_tile_sb<BITS, GROUP, BM, BN, QUANT, STAGES, true, WAVES, true>(s, a);
             return launch_tile_sb<BITS, GROUP, BM, BN, QUANT, STAGES, false, WAVES, true>(s, a);
         }
     }
+    if (a.tiles) return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "this tile shape does not read TILE16 records");
     if constexpr (QUANT) {
         if (a.sb_dtype == MI355Q_BF16) return launch_tile_sb<BITS, GROUP, BM, BN, QUANT, STAGES, true, WAVES, false>(s, a);
     }

@@ -62,12 +62,13 @@ GemvCfg choose(const mi355q_context* ctx, const WView& w, uint32_t m, bool argma
     const uint64_t weight_bytes = (uint64_t)w.n * (w.k / w.group) * (4 + w.group * w.bits / 8);
     const bool big = weight_bytes >= (24ull << 20);
     if (c.mt == 1) {
-        // Measured on MI355X (q4 g64): rows of one K-step keep their activation slice in registers;
-        // longer rows read it from LDS.  Large matrices of short rows run best with 4 wavefronts
-        // per workgroup, everything else with 8.
-        c.xreg = c.nc == 1 ? 1 : 0;
+        // Measured on MI355X (q4 g64): large matrices of short rows (one or two K-steps) run best with 4
+        // wavefronts per workgroup, and with rows of one K-step they keep their activation slice in
+        // registers; everything else runs best with 8 wavefronts reading the slice from LDS
+        // (2048 -> 8192: 4.3 us against 5.5 us with the large-matrix shape).
+        c.xreg = (c.nc == 1 && big) ? 1 : 0;
         c.r = 1;
-        c.waves = (c.nc == 1 || (c.nc == 2 && big)) ? 4 : 8;
+        c.waves = (c.nc <= 2 && big) ? 4 : 8;
     } else {
         c.xreg = 0;
         c.r = 2;
