@@ -146,6 +146,7 @@ mi355q_status launch_gemv_fast_multi(hipStream_t s, const mi355q_context* ctx, u
 constexpr int kTile16MaxSegments = 3;
 struct Tile16LaunchShape {
     uint32_t ksplit, tiles_per_wg, waves, blocks_per_wave, grid, block, lds_bytes;
+    uint32_t passes;     // row tiles a wavefront walks on one staged copy of the activations
 };
 bool gemv_tile16_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
 Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_total_tiles, uint32_t k, uint32_t m);

@@ -49,6 +49,7 @@ struct T16Args {
     uint32_t k, m, x_stride;
     uint32_t kblocks;                            // K / 128
     uint32_t blocks_per_wave;                    // K-blocks per wavefront (K split over the workgroup)
+    uint32_t passes;                             // row tiles a wavefront walks, one after the other, on one staged copy of x
     uint32_t lds_row_bytes;                      // K*2 + 16: staged activation row pitch
     uint32_t y_dtype, sb_dtype;
 };
@@ -67,18 +68,35 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t n_in = lane & 15, kq = lane >> 4;
 
-    // ---- matrix and row tile of this wavefront (scalar select chain, once) ----------------------
+    // ---- matrix and row tile of this wavefront in pass `pass` (scalar select chain) ---------------
     const uint32_t slice = wave % KSPLIT;                   // share of K
-    uint32_t gt = blockIdx.x * TPW + wave / KSPLIT;
-    const bool tile_valid = gt < a.tile_end[kTile16MaxSegments - 1];
-    gt = tile_valid ? gt : a.tile_end[kTile16MaxSegments - 1] - 1;       // idle wavefronts re-read the last tile
-    const bool in1 = gt >= a.tile_end[0], in2 = gt >= a.tile_end[1];
-    const uint32_t* const seg_tiles = in2 ? a.tiles[2] : in1 ? a.tiles[1] : a.tiles[0];
-    void* const seg_y = in2 ? a.y[2] : in1 ? a.y[1] : a.y[0];
-    const uint32_t seg_ys = in2 ? a.y_stride[2] : in1 ? a.y_stride[1] : a.y_stride[0];
-    const uint32_t seg_n = in2 ? a.seg_rows[2] : in1 ? a.seg_rows[1] : a.seg_rows[0];
-    const uint32_t lt = gt - (in2 ? a.tile_end[1] : in1 ? a.tile_end[0] : 0u);
-    const uint32_t n0 = lt * 16;
+    struct Tile {
+        const uint32_t* base;      // first record of the row tile
+        void* y;
+        uint32_t ys, rows, n0, nb, b_first, b_last;
+        bool valid;
+    };
+    auto select_tile = [&](uint32_t pass) {
+        Tile t;
+        uint32_t gt = (blockIdx.x * a.passes + pass) * TPW + wave / KSPLIT;
+        t.valid = gt < a.tile_end[kTile16MaxSegments - 1];
+        gt = t.valid ? gt : a.tile_end[kTile16MaxSegments - 1] - 1;      // idle wavefronts re-read the last tile
+        const bool in1 = gt >= a.tile_end[0], in2 = gt >= a.tile_end[1];
+        const uint32_t* const seg_tiles = in2 ? a.tiles[2] : in1 ? a.tiles[1] : a.tiles[0];
+        t.y = in2 ? a.y[2] : in1 ? a.y[1] : a.y[0];
+        t.ys = in2 ? a.y_stride[2] : in1 ? a.y_stride[1] : a.y_stride[0];
+        t.rows = in2 ? a.seg_rows[2] : in1 ? a.seg_rows[1] : a.seg_rows[0];
+        const uint32_t lt = gt - (in2 ? a.tile_end[1] : in1 ? a.tile_end[0] : 0u);
+        t.n0 = lt * 16;
+        t.b_first = slice * a.blocks_per_wave;
+        uint32_t nb = a.kblocks > t.b_first ? a.kblocks - t.b_first : 0;      // blocks this wavefront owns
+        nb = nb < a.blocks_per_wave ? nb : a.blocks_per_wave;
+        t.nb = t.valid ? nb : 0;
+        t.b_last = t.nb ? t.b_first + t.nb - 1 : a.kblocks - 1;              // clamp target (always valid)
+        t.base = seg_tiles + (size_t)lt * a.kblocks * kT16RecordWords;
+        return t;
+    };
+    Tile tile = select_tile(0);
 
     // ---- 1. activation loads first (vector loads return in issue order) -------------------------
     // Raw copy of the M rows into LDS, row pitch K*2 + 16 bytes (the pad spreads the 16 rows of an
@@ -104,23 +122,16 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
 #pragma unroll
     for (int t = 0; t < XC; t++) xe[t] = *x_src(tid + t * WAVES * 64);
 
-    // ---- 2. the first D K-blocks of this wavefront's share of the row tile ----------------------
-    const uint32_t b_first = slice * a.blocks_per_wave;
-    uint32_t nb = a.kblocks > b_first ? a.kblocks - b_first : 0;          // blocks this wavefront owns
-    nb = nb < a.blocks_per_wave ? nb : a.blocks_per_wave;
-    nb = tile_valid ? nb : 0;
-    const uint32_t b_last = nb ? b_first + nb - 1 : a.kblocks - 1;        // clamp target (always valid)
-    const uint32_t* const tile_base = seg_tiles + (size_t)lt * a.kblocks * kT16RecordWords;
-
+    // ---- 2. the first D K-blocks of this wavefront's share of the first row tile -----------------
     struct Rec { u32x4 w; u32x2 sz; };
     Rec ring[D];
     auto issue = [&](uint32_t b, Rec& r) {
-        b = b < b_last ? b : b_last;                        // unconditional, clamped
-        const uint32_t* rec = tile_base + (size_t)b * kT16RecordWords;   // scalar
+        b = b < tile.b_last ? b : tile.b_last;              // unconditional, clamped
+        const uint32_t* rec = tile.base + (size_t)b * kT16RecordWords;   // scalar
         r.w = *((const u32x4*)rec + lane);
         r.sz = *((const u32x2*)(rec + 256) + n_in);
     };
-    static_for<D>([&](auto J) { issue(b_first + decltype(J)::value, ring[decltype(J)::value]); });
+    static_for<D>([&](auto J) { issue(tile.b_first + decltype(J)::value, ring[decltype(J)::value]); });
 
     // ---- 3. stage the activations (waits only for the loads of step 1) --------------------------
     // With each 16-byte chunk goes its share of sum(x): eight consecutive lanes hold the eight chunks of one
@@ -205,47 +216,54 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
     };
 
     const uint32_t rounds = (a.blocks_per_wave + D - 1) / D;            // same for every wavefront
-    for (uint32_t it = 0; it < rounds; it++) {
-        static_for<D>([&](auto J) {
-            constexpr int j = decltype(J)::value;
-            const uint32_t idx = it * D + j;                // block index inside this wavefront's share
-            if (idx < nb) compute(b_first + idx, ring[j]);
-            issue(b_first + idx + D, ring[j]);
-        });
-    }
-
-    // ---- 5. add the WAVES partial tiles through LDS, store -------------------------------------
-    // Activations are no longer needed: the reduction buffer overlays them.
-    __syncthreads();
-    float* red = (float*)lds;                               // [WAVES][MR][64]
-#pragma unroll
-    for (int r = 0; r < MR; r++) red[(wave * MR + r) * 64 + lane] = acc[r];
-    __syncthreads();
+    // partial tiles of the WAVES wavefronts, behind the activations and their group sums
+    float* const red = (float*)(lds + (size_t)a.m * a.lds_row_bytes + a.k);          // [WAVES][MR][64]
     unsigned long long best = 0ull;
-    if (slice == 0 && tile_valid) {                         // the first wavefront of each tile adds and stores
-        const uint32_t row = n0 + n_in;
+    for (uint32_t pass = 0; pass < a.passes; pass++) {
+        if (pass) {                                            // the first tile's loads were issued before staging
+            tile = select_tile(pass);
+            static_for<D>([&](auto J) { issue(tile.b_first + decltype(J)::value, ring[decltype(J)::value]); });
+        }
+        for (uint32_t it = 0; it < rounds; it++) {
+            static_for<D>([&](auto J) {
+                constexpr int j = decltype(J)::value;
+                const uint32_t idx = it * D + j;            // block index inside this wavefront's share
+                if (idx < tile.nb) compute(tile.b_first + idx, ring[j]);
+                issue(tile.b_first + idx + D, ring[j]);
+            });
+        }
+
+        // ---- 5. add the partial tiles of the wavefronts that share a row tile, store ----------------
 #pragma unroll
-        for (int r = 0; r < MR; r++) {
-            float v = 0.f;
-            for (uint32_t w2 = 0; w2 < (uint32_t)KSPLIT; w2++) v += red[((wave + w2) * MR + r) * 64 + lane];
-            const uint32_t m = 4 * kq + r;
-            if (m < a.m && row < seg_n) {
-                if (seg_y) {
-                    const size_t o = (size_t)m * seg_ys + row;
-                    if (a.y_dtype == MI355Q_F32) ((float*)seg_y)[o] = v;
-                    else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)seg_y)[o] = f32_to_bf16_rne(v);
-                    else ((uint16_t*)seg_y)[o] = f32_to_f16_rne(v);
-                }
-                if (a.logits && m == 0) a.logits[row] = v;
-                if constexpr (ARGMAX) {
-                    if (m == 0 && v > -INFINITY) {          // NaN and -inf never contribute
-                        const uint32_t u = __float_as_uint(v + 0.0f);   // -0 -> +0
-                        const uint32_t key = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
-                        best = ((unsigned long long)key << 32) | (unsigned long long)(0xFFFFFFFFu - row);
+        for (int r = 0; r < MR; r++) { red[(wave * MR + r) * 64 + lane] = acc[r]; acc[r] = 0.f; }
+        __syncthreads();
+        if (slice == 0 && tile.valid) {                     // the first wavefront of each tile adds and stores
+            const uint32_t row = tile.n0 + n_in;
+#pragma unroll
+            for (int r = 0; r < MR; r++) {
+                float v = 0.f;
+                for (uint32_t w2 = 0; w2 < (uint32_t)KSPLIT; w2++) v += red[((wave + w2) * MR + r) * 64 + lane];
+                const uint32_t m = 4 * kq + r;
+                if (m < a.m && row < tile.rows) {
+                    if (tile.y) {
+                        const size_t o = (size_t)m * tile.ys + row;
+                        if (a.y_dtype == MI355Q_F32) ((float*)tile.y)[o] = v;
+                        else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)tile.y)[o] = f32_to_bf16_rne(v);
+                        else ((uint16_t*)tile.y)[o] = f32_to_f16_rne(v);
+                    }
+                    if (a.logits && m == 0) a.logits[row] = v;
+                    if constexpr (ARGMAX) {
+                        if (m == 0 && v > -INFINITY) {      // NaN and -inf never contribute
+                            const uint32_t u = __float_as_uint(v + 0.0f);   // -0 -> +0
+                            const uint32_t key = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+                            const unsigned long long pk = ((unsigned long long)key << 32) | (unsigned long long)(0xFFFFFFFFu - row);
+                            best = pk > best ? pk : best;
+                        }
                     }
                 }
             }
         }
+        if (pass + 1 < a.passes) __syncthreads();           // the partial tiles are read before the next pass overwrites them
     }
     if constexpr (ARGMAX) {
         // wavefront maximum of the packed (ordered value, ~row) key, workgroup maximum through LDS, one plain
@@ -318,10 +336,13 @@ Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_total_
     const uint32_t want_tpw = m == 1 ? 1u : m <= 4 ? 2u : 4u;
     uint32_t tpw = 1;
     while (tpw < want_tpw && ks * tpw * 2 <= 16 && (n_total_tiles + tpw * 2 - 1) / (tpw * 2) >= cus / 2) tpw *= 2;
-    if ((size_t)m * ((size_t)k * 2 + 16) > 80 * 1024) {
-        // the staged activations leave room for one workgroup per CU: make it as large as possible
-        tpw = 1;
-        while (ks < 16 && kblocks / (ks * 2) >= 2) ks *= 2;
+    const bool one_wg_per_cu = (size_t)m * ((size_t)k * 2 + 16) > 80 * 1024;
+    if (one_wg_per_cu) {
+        // the staged activations leave room for one workgroup per CU: sixteen wavefronts, four row tiles at a time
+        // (each wavefront keeps a quarter of K: long enough a stream to fill its prefetch ring)
+        ks = kblocks >= 8 ? 4 : (kblocks >= 4 ? 2 : 1);
+        if (ks < 4) ks = 4;                                  // the built variants split K four ways at least
+        tpw = 4;
     }
     const int eks = env_int_cached("MI355Q_T16_KSPLIT", 0), etpw = env_int_cached("MI355Q_T16_TPW", 0);
     if (eks) ks = (uint32_t)eks;
@@ -330,11 +351,26 @@ Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_total_
     g.tiles_per_wg = tpw;
     g.waves = ks * tpw;
     g.blocks_per_wave = (kblocks + ks - 1) / ks;
-    g.grid = (n_total_tiles + tpw - 1) / tpw;
+    // A workgroup stages all M activation rows once.  When that is more than half of the weight bytes it streams
+    // (large batches: 131 KB of activations against 37 KB of weights per row tile at M = 16, K = 4096), its
+    // wavefronts walk several row tiles on the one staged copy -- as many as still leave a workgroup per CU.
+    {
+        const size_t staged = (size_t)m * ((size_t)k * 2 + 16);
+        const size_t per_pass = (size_t)tpw * 16 * (k / 64) * 36 / 2;
+        uint32_t want = (uint32_t)((staged + per_pass - 1) / per_pass);
+        // not more than leaves one workgroup per CU; with one workgroup per CU, exactly one round of workgroups
+        const uint32_t most = one_wg_per_cu ? (n_total_tiles + tpw * cus - 1) / (tpw * cus) : n_total_tiles / (tpw * cus);
+        if (want > most || one_wg_per_cu) want = most;
+        if (want > 16) want = 16;
+        g.passes = want ? want : 1;
+        const int ep = env_int_cached("MI355Q_T16_PASSES", 0);
+        if (ep) g.passes = (uint32_t)ep;
+    }
+    g.grid = (n_total_tiles + tpw * g.passes - 1) / (tpw * g.passes);
     g.block = g.waves * 64;
     const size_t x_bytes = (size_t)m * ((size_t)k * 2 + 16) + k;     // rows, then sum(x) per group: [K/64][16] floats
-    const size_t red_bytes = (size_t)g.waves * 4 * 64 * 4;
-    g.lds_bytes = (uint32_t)(x_bytes > red_bytes ? x_bytes : red_bytes);
+    const size_t red_bytes = (size_t)g.waves * 4 * 64 * 4;     // partial tiles, behind the activations
+    g.lds_bytes = (uint32_t)(x_bytes + red_bytes);
     return g;
 }
 
@@ -365,6 +401,7 @@ mi355q_status launch_gemv_tile16_multi(hipStream_t s, const mi355q_context* ctx,
     a.k = w[0].k; a.m = m; a.x_stride = x_stride;
     a.kblocks = w[0].k / 128;
     a.blocks_per_wave = g.blocks_per_wave;
+    a.passes = g.passes;
     a.lds_row_bytes = w[0].k * 2 + 16;
     a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = w[0].sb_dtype;
     const int mr = m == 1 ? 1 : m == 2 ? 2 : 4;
