@@ -60,6 +60,8 @@ mi355q_status run_small_m(mi355q_context* ctx, hipStream_t s, const mi355q_weigh
             st = launch_gemv_tile16_multi(s, ctx, 1, &v, xp, yv, strides, y_dtype, mm, xs, nullptr, nullptr, nullptr);
         } else if (!generic && gemv_fast_eligible(v, x_dtype, mm, xs) && (uintptr_t)xp % 16 == 0) {
             st = launch_gemv_fast(s, ctx, v, xp, yp, y_dtype, mm, xs, ys, nullptr, nullptr, nullptr);
+        } else if (!generic && gemv_staf_eligible(v, x_dtype, mm, xs) && (uintptr_t)xp % 16 == 0) {
+            st = launch_gemv_staf(s, ctx, v, xp, yp, y_dtype, mm, xs, ys);
         } else {
             st = launch_gemv_generic(s, v, xp, x_dtype, yp, y_dtype, mm, xs, ys);
         }
@@ -170,7 +172,11 @@ mi355q_status dispatch_output_head(mi355q_context* ctx, hipStream_t s, const mi3
     if (!logits)
         return fail(MI355Q_ERR_INVALID_ARGUMENT,
                     "a logits buffer is required when the fused head kernel does not accept the shape");
-    mi355q_status st = launch_gemv_generic(s, v, x, x_dtype, logits, MI355Q_F32, 1, xs, (uint32_t)w->n);
+    mi355q_status st;
+    if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && gemv_staf_eligible(v, x_dtype, 1, xs) && (uintptr_t)x % 16 == 0)
+        st = launch_gemv_staf(s, ctx, v, x, logits, MI355Q_F32, 1, xs, (uint32_t)w->n);
+    else
+        st = launch_gemv_generic(s, v, x, x_dtype, logits, MI355Q_F32, 1, xs, (uint32_t)w->n);
     if (st != MI355Q_OK) return st;
     return launch_argmax(s, logits, MI355Q_F32, (uint32_t)w->n, token);
 }

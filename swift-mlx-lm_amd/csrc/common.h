@@ -131,10 +131,15 @@ mi355q_status launch_gemv_fast(hipStream_t s, const mi355q_context* ctx, const W
                                const void* x, void* y, int y_dtype, uint32_t m,
                                uint32_t x_stride, uint32_t y_stride, float* logits_f32,
                                int32_t* token_out, unsigned long long* argmax_scratch);
+// Block-layout GEMV (gemv_staf.hip): reads STAF interleaved blocks in place.
+bool gemv_staf_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
+mi355q_status launch_gemv_staf(hipStream_t s, const mi355q_context* ctx, const WView& w, const void* x, void* y,
+                               int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride);
 struct GemvLaunchShape {
     uint32_t grid, block, lds_bytes, rows_per_workgroup;
     const char* kernel;
 };
+GemvLaunchShape gemv_staf_shape(const mi355q_context* ctx, const WView& w, uint32_t m);
 GemvLaunchShape gemv_fast_shape(const mi355q_context* ctx, const WView& w, uint32_t m);
 
 mi355q_status launch_gemv_fast_multi(hipStream_t s, const mi355q_context* ctx, uint32_t count, const WView* w,

@@ -48,7 +48,9 @@ mi355q_status launch_group(hipStream_t s, const GemvArgs& a, const GemvCfg& c) {
     MI355Q_TRY(1, 1, true, 4, 2, 0) MI355Q_TRY(1, 1, true, 4, 4, 0)
     MI355Q_TRY(1, 1, true, 8, 2, 0) MI355Q_TRY(1, 1, true, 8, 4, 0)
     // small batches (M = 2, 3-4)
-    MI355Q_TRY(2, 2, false, 4, 4, 0) MI355Q_TRY(2, 4, false, 4, 2, 0)
+    constexpr int R2 = gemv_batch_rows(BITS, GROUP, 2), R4 = gemv_batch_rows(BITS, GROUP, 4);
+    constexpr int D2 = gemv_batch_depth(BITS, GROUP, 2), D4 = gemv_batch_depth(BITS, GROUP, 4);
+    MI355Q_TRY(R2, 2, false, 4, D2, 0) MI355Q_TRY(R4, 4, false, 4, D4, 0)
     return fail(MI355Q_ERR_KERNEL_NOT_FOUND,
                 "no split-plane GEMV variant for q%d g%d R=%d MT=%d argmax=%d waves=%d depth=%d xreg=%d", BITS, GROUP,
                 c.r, c.mt, (int)c.argmax, c.waves, c.depth, c.xreg);

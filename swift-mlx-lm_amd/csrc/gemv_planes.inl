@@ -78,6 +78,17 @@ template <> struct GemvGeo<3> { static constexpr int WPL = 3, CPL = 32; static c
 template <> struct GemvGeo<6> { static constexpr int WPL = 3, CPL = 16; static constexpr bool PAIRS = false; };
 template <> struct GemvGeo<5> { static constexpr int WPL = 5, CPL = 32; static constexpr bool PAIRS = false; };
 
+// Small batches (MT = 2 or 4 activation rows): weight rows carried per pipeline step and ring depth.
+// Two rows per step halve the LDS reads of the activations, but only 4- and 6-bit codes leave room
+// for them in the register file at MT = 4 (the other widths would spill to scratch memory).
+constexpr int gemv_batch_rows(int bits, int group, int mt) {
+    if (mt == 2) return (bits == 2 && group == 16) ? 1 : 2;
+    return (bits == 4 || bits == 6) ? 2 : 1;
+}
+constexpr int gemv_batch_depth(int bits, int group, int mt) {
+    return (mt == 2 || gemv_batch_rows(bits, group, mt) == 1) ? 4 : 2;
+}
+
 // Element (within a lane chunk) that lands in half `which` of staged pair `i`.
 template <int BITS>
 __host__ __device__ constexpr int pair_elem(int i, int which) {

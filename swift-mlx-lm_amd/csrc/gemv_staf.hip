@@ -1,0 +1,414 @@
+// Decode GEMV that reads STAF interleaved blocks in place ([f16 scale][f16 zero][packed codes], one
+// block per group), bf16 activations, 1 <= M <= 8: the path of a weight that was wrapped or uploaded
+// from a model file without being repacked.
+//
+//   * a block is 4 + GROUP*BITS/8 bytes (36 for q4 g64), so a lane cannot fetch "its" block with one
+//     aligned vector load.  A wavefront instead copies a span of 64 consecutive blocks of one row --
+//     one contiguous byte range -- from memory straight into LDS with 128-bit direct-to-LDS loads
+//     (no register staging), and every lane then reads its own block back with 32-bit LDS reads:
+//     1 + GROUP*BITS/32 dwords at a stride that is odd for every supported format, so the reads are
+//     free of bank conflicts;
+//   * a wavefront owns a run of consecutive rows and keeps D spans in flight in a private LDS ring;
+//     the direct-to-LDS loads are invisible to the compiler's wait-counter bookkeeping, so the
+//     kernel waits on the vector-memory counter itself: every span is exactly NDMA load
+//     instructions, each issued with at least one lane active (lanes past the end of the buffer read
+//     a clamped address; their bytes belong to blocks no lane uses), which makes "at most NDMA
+//     loads outstanding per younger span" mean "the oldest span has landed";
+//   * arithmetic is that of the split-plane kernel: activations staged once per workgroup in LDS in
+//     the pair order the unpacker produces together with the per-block sums, 2..6-bit codes turned
+//     into bf16 (128+q) pairs for v_dot2_f32_bf16, 8-bit codes through fp32 FMA, the affine form
+//     s*sum(q*x) + z*sum(x) per block, one wavefront reduction per output row.
+//
+// Replaces gemv_q{b}_g{g} reading the STAF payload directly
+// (Sources/MetalCompiler/Generator/MetalSourceGenerator+Quantized.swift:496-575; block layout:
+// Sources/MetalCompiler/STAF/QuantizationFormat.swift:1284-1312).
+#include "gemv_planes.inl"
+
+namespace mi355q {
+
+namespace {
+
+#define MI355Q_LDS_PTR(p) ((__attribute__((address_space(3))) uint8_t*)(p))
+
+struct StafArgs {
+    const uint8_t* blocks;
+    const uint16_t* x;       // bf16 [M, x_stride]
+    void* y;                 // [M, y_stride] in y_dtype
+    uint64_t row_bytes;      // blocks_per_row * bytes per block (a multiple of 16)
+    uint64_t last_chunk;     // byte offset of the last whole 16-byte chunk of the weight buffer
+    uint32_t k, n, m;
+    uint32_t x_stride, y_stride, y_dtype;
+    uint32_t blocks_per_row;
+    uint32_t nsp;            // spans per row = ceil(blocks_per_row / 64)
+    uint32_t rows_per_wave;
+};
+
+template <int BITS, int GROUP>
+struct StafGeo {
+    static constexpr int WPB = GROUP * BITS / 32;           // code words per block
+    static constexpr int BW = 1 + WPB;                      // dwords per block
+    static constexpr int SPAN = 64 * BW * 4;                // bytes of 64 blocks
+    static constexpr int NDMA = (SPAN + 1023) / 1024;       // 64 lanes x 16 bytes per load instruction
+    static constexpr int SLOT = SPAN;                       // ring slot (a multiple of 256 bytes)
+    static constexpr int Q = GROUP / 8;                     // staged activation pieces (8 elements each) per block
+};
+
+template <int BITS, int GROUP, int MT, int WAVES, int D>
+__global__ __launch_bounds__(WAVES * 64) void gemv_staf_kernel(const StafArgs a) {
+    using G = StafGeo<BITS, GROUP>;
+    constexpr int WPB = G::WPB, BW = G::BW, SPAN = G::SPAN, NDMA = G::NDMA, SLOT = G::SLOT, Q = G::Q;
+    constexpr bool DOT2 = BITS <= 6;                        // 128 + q is exact in bf16
+    static_assert(GROUP * BITS % 32 == 0 && GROUP % 8 == 0, "blocks are whole words");
+    static_assert(NDMA * (D - 1) < 64, "the vector-memory counter has 6 bits");
+
+    extern __shared__ __align__(16) uint8_t lds[];
+    const uint32_t lane = threadIdx.x & 63u;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const uint32_t NSP = a.nsp;
+    u32x4* const xs = (u32x4*)lds;                                          // [m][span][piece][lane]
+    float* const sxs = (float*)(lds + (size_t)MT * NSP * Q * 1024);         // [m][span][lane]
+    uint8_t* const ring = lds + (size_t)MT * NSP * (Q * 1024 + 256) + (size_t)wave * D * SLOT;
+    const uint32_t ring_lds = (uint32_t)(uintptr_t)MI355Q_LDS_PTR(ring);
+
+    const uint32_t row0 = (blockIdx.x * WAVES + wave) * a.rows_per_wave;
+    const uint32_t nsteps = a.rows_per_wave * NSP;
+
+    // ---- 1. the first D spans go out before anything else ----------------------------------------
+    uint32_t irow = 0, isp = 0;                              // next span to issue
+    auto issue = [&](uint32_t slot) {
+        uint32_t row = row0 + irow;
+        row = row < a.n ? row : a.n - 1;                     // rows past the end of the matrix reload its last row
+        const uint64_t base = (uint64_t)row * a.row_bytes + (uint64_t)isp * SPAN + (uint64_t)lane * 16;
+#pragma unroll
+        for (int i = 0; i < NDMA; i++) {
+            uint64_t off = base + (uint64_t)i * 1024;
+            off = off < a.last_chunk ? off : a.last_chunk;
+            const uint8_t* g = a.blocks + off;
+            const uint32_t l = ring_lds + slot * SLOT + i * 1024;
+            // the last instruction of a span covers only part of the wavefront: the other lanes are masked
+            // off (never all of them, so the instruction is issued and counted every time)
+            if ((i + 1) * 1024 <= SPAN || lane < (uint32_t)(SPAN - i * 1024) / 16)
+                asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(l) : "memory");
+        }
+        if (++isp == NSP) { isp = 0; irow++; }
+    };
+#pragma unroll
+    for (int j = 0; j < D; j++)
+        if ((uint32_t)j < nsteps) issue(j);
+
+    // ---- 2. activations: loaded, permuted into pair order, summed per block, parked in LDS ---------
+    const uint32_t ntasks = a.m * NSP;
+    for (uint32_t t = wave; t < ntasks; t += WAVES) {
+        const uint32_t m = t / NSP, sp = t - m * NSP;
+        const uint32_t b = sp * 64 + lane;
+        const bool valid = b < a.blocks_per_row;
+        const u32x4* src = (const u32x4*)(a.x + (size_t)m * a.x_stride + (valid ? (size_t)b * GROUP : 0));
+        uint32_t d[GROUP / 2];
+#pragma unroll
+        for (int i = 0; i < Q; i++) {
+            const u32x4 v = src[i];
+            d[4 * i + 0] = valid ? v.x : 0; d[4 * i + 1] = valid ? v.y : 0;
+            d[4 * i + 2] = valid ? v.z : 0; d[4 * i + 3] = valid ? v.w : 0;
+        }
+        auto pairw = [&](auto I) -> uint32_t {
+            constexpr int i = decltype(I)::value;
+            constexpr int e0 = pair_elem<BITS>(i, 0), e1 = pair_elem<BITS>(i, 1);
+            if constexpr (e1 == e0 + 1 && (e0 & 1) == 0) return d[e0 >> 1];
+            else return __builtin_amdgcn_perm(d[e1 >> 1], d[e0 >> 1], (e0 & 1) ? 0x07060302u : 0x05040100u);
+        };
+        static_for<Q>([&](auto P) {
+            constexpr int i = decltype(P)::value;
+            u32x4 o;
+            o.x = pairw(std::integral_constant<int, 4 * i + 0>{});
+            o.y = pairw(std::integral_constant<int, 4 * i + 1>{});
+            o.z = pairw(std::integral_constant<int, 4 * i + 2>{});
+            o.w = pairw(std::integral_constant<int, 4 * i + 3>{});
+            xs[((size_t)(m * NSP + sp) * Q + i) * 64 + lane] = o;
+        });
+        float sx = 0.0f;
+#pragma unroll
+        for (int j = 0; j < GROUP / 2; j++) sx = dot2_bf16(d[j], 0x3F803F80u, sx);
+        sxs[(size_t)(m * NSP + sp) * 64 + lane] = sx;
+    }
+    __syncthreads();
+
+    uint32_t k_magic = 0x43004300u;                          // bf16 pair (128.0, 128.0)
+    uint32_t k_mask = BITS == 4 ? 0x000F000Fu : 0x00030003u;
+    asm volatile("" : "+v"(k_magic));
+    asm volatile("" : "+s"(k_mask));
+
+    float acc[MT], res[MT];
+#pragma unroll
+    for (int m = 0; m < MT; m++) acc[m] = res[m] = 0.0f;
+
+    auto flush = [&](uint32_t first_local, uint32_t count) {
+        const uint32_t row = row0 + first_local + lane;
+        if (lane < count && row < a.n) {
+#pragma unroll
+            for (int m = 0; m < MT; m++) {
+                if ((uint32_t)m < a.m) {
+                    const size_t o = (size_t)m * a.y_stride + row;
+                    if (a.y_dtype == MI355Q_F32) ((float*)a.y)[o] = res[m];
+                    else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)a.y)[o] = f32_to_bf16_rne(res[m]);
+                    else ((uint16_t*)a.y)[o] = f32_to_f16_rne(res[m]);
+                }
+            }
+        }
+    };
+
+    // ---- 3. one span per step: wait for the oldest slot, unpack it, refill it ------------------------
+    uint32_t lrow = 0, sp = 0;
+    for (uint32_t step = 0; step < nsteps; step++) {
+        const uint32_t slot = step % D;
+        // spans issued after this one: D-1 in the steady state, fewer over the last steps
+        const uint32_t younger = nsteps - 1 - step < (uint32_t)(D - 1) ? nsteps - 1 - step : (uint32_t)(D - 1);
+        static_for<D>([&](auto Y) {
+            constexpr int y = decltype(Y)::value;
+            if (younger == (uint32_t)y) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA * y) : "memory");
+        });
+        const uint32_t* blk = (const uint32_t*)(ring + (size_t)slot * SLOT) + lane * BW;
+        const bool valid = sp * 64 + lane < a.blocks_per_row;
+        uint32_t hdr = blk[0];
+        uint32_t w[WPB];
+#pragma unroll
+        for (int i = 0; i < WPB; i++) w[i] = blk[1 + i];
+        hdr = valid ? hdr : 0u;
+
+        float dot[MT];
+#pragma unroll
+        for (int m = 0; m < MT; m++) dot[m] = 0.0f;
+        static_for<Q>([&](auto P) {
+            constexpr int p = decltype(P)::value;
+            u32x4 xv[MT];
+#pragma unroll
+            for (int m = 0; m < MT; m++) xv[m] = xs[((size_t)(m * NSP + sp) * Q + p) * 64 + lane];
+            if constexpr (DOT2) {
+                uint32_t pr[4];
+                if constexpr (BITS == 4) {
+                    const uint32_t wv = w[p];
+                    pr[0] = (wv & k_mask) | k_magic;
+                    pr[1] = ((wv >> 4) & k_mask) | k_magic;
+                    pr[2] = ((wv >> 8) & k_mask) | k_magic;
+                    pr[3] = ((wv >> 12) & k_mask) | k_magic;
+                } else if constexpr (BITS == 2) {
+                    const uint32_t wv = w[p >> 1] >> (8 * (p & 1));
+                    pr[0] = (wv & k_mask) | k_magic;
+                    pr[1] = ((wv >> 2) & k_mask) | k_magic;
+                    pr[2] = ((wv >> 4) & k_mask) | k_magic;
+                    pr[3] = ((wv >> 6) & k_mask) | k_magic;
+                } else {
+                    static_for<4>([&](auto I) {
+                        constexpr int i = decltype(I)::value;
+                        const uint32_t qa = extract_code<(p * 8 + 2 * i) * BITS, BITS, WPB>(w);
+                        const uint32_t qb = extract_code<(p * 8 + 2 * i + 1) * BITS, BITS, WPB>(w);
+                        pr[i] = ((qb << 16) | qa) | k_magic;
+                    });
+                }
+#pragma unroll
+                for (int m = 0; m < MT; m++) {
+                    float dsum = dot[m];
+                    dsum = dot2_bf16(pr[0], xv[m].x, dsum);
+                    dsum = dot2_bf16(pr[1], xv[m].y, dsum);
+                    dsum = dot2_bf16(pr[2], xv[m].z, dsum);
+                    dsum = dot2_bf16(pr[3], xv[m].w, dsum);
+                    dot[m] = dsum;
+                }
+            } else {
+                float qf[8];
+                static_for<8>([&](auto E) {
+                    constexpr int e = decltype(E)::value;
+                    qf[e] = (float)extract_code<(p * 8 + e) * BITS, BITS, WPB>(w);
+                });
+#pragma unroll
+                for (int m = 0; m < MT; m++) {
+                    const uint32_t xw[4] = {xv[m].x, xv[m].y, xv[m].z, xv[m].w};
+                    float dsum = dot[m];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        dsum = __builtin_fmaf(qf[2 * e], __uint_as_float(xw[e] << 16), dsum);
+                        dsum = __builtin_fmaf(qf[2 * e + 1], __uint_as_float(xw[e] & 0xFFFF0000u), dsum);
+                    }
+                    dot[m] = dsum;
+                }
+            }
+        });
+        const float s = f16_to_f32((uint16_t)(hdr & 0xFFFFu)), z = f16_to_f32((uint16_t)(hdr >> 16));
+        const float zc = DOT2 ? z - 128.0f * s : z;
+#pragma unroll
+        for (int m = 0; m < MT; m++) acc[m] += s * dot[m] + zc * sxs[(size_t)(m * NSP + sp) * 64 + lane];
+
+        // the slot's LDS reads have been consumed by the arithmetic above: it can be overwritten
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (step + D < nsteps) issue(slot);
+
+        if (++sp == NSP) {                                   // row complete
+            sp = 0;
+#pragma unroll
+            for (int m = 0; m < MT; m++) {
+                const float total = wave_reduce_sum(acc[m]);
+                if (lane == (lrow & 63u)) res[m] = total;
+                acc[m] = 0.0f;
+            }
+            lrow++;
+            if ((lrow & 63u) == 0) flush(lrow - 64, 64);
+        }
+    }
+    if (lrow & 63u) flush(lrow & ~63u, lrow & 63u);
+}
+
+constexpr int kWaves = 4;
+
+// Ring depth and wavefronts per CU.  Tuning builds (MI355Q_GEMV_EXPERIMENT) read MI355Q_STAF_DEPTH and
+// MI355Q_STAF_WAVES_PER_CU; product builds ignore them.
+// Measured on MI355X (q4 g64, 14336x4096, M = 1): depth 2 with 8 wavefronts per CU 9.2 us, depth 4
+// 11.1 us; 4 wavefronts per CU 11.6 us, 16 and more 9.6 us and up.
+struct StafCfg { int depth; uint32_t per_cu; };
+StafCfg staf_cfg() {
+    StafCfg c{2, 8};
+    const int d = env_int_cached("MI355Q_STAF_DEPTH", 0), p = env_int_cached("MI355Q_STAF_WAVES_PER_CU", 0);
+    if (d == 2 || d == 4) c.depth = d;
+    if (p > 0) c.per_cu = (uint32_t)p;
+    return c;
+}
+
+size_t staf_lds_bytes(uint32_t span_slot, uint32_t q, uint32_t nsp, int mt, int depth) {
+    return (size_t)mt * nsp * (q * 1024 + 256) + (size_t)kWaves * depth * span_slot;
+}
+
+// When the staged activations leave room for a single workgroup per CU, its four wavefronts take the
+// CU's whole share of rows (every extra workgroup would stage the activations again).
+void staf_one_workgroup_per_cu(size_t lds, StafCfg& c) {
+    if (lds > 80 * 1024 && env_int_cached("MI355Q_STAF_WAVES_PER_CU", 0) == 0) c.per_cu = kWaves;
+}
+
+// Each wavefront owns a run of consecutive rows.
+uint32_t staf_rows_per_wave(const mi355q_context* ctx, uint32_t n, const StafCfg& c) {
+    const uint32_t target = (uint32_t)ctx->props.multiProcessorCount * c.per_cu;
+    const uint32_t rpw = (n + target - 1) / target;
+    return rpw ? rpw : 1;
+}
+
+template <int BITS, int GROUP>
+mi355q_status launch_for_format(hipStream_t s, const mi355q_context* ctx, const StafArgs& args, int mt) {
+    using G = StafGeo<BITS, GROUP>;
+    StafCfg c = staf_cfg();
+    const size_t lds = staf_lds_bytes(G::SLOT, G::Q, args.nsp, mt, c.depth);
+    staf_one_workgroup_per_cu(lds, c);
+    StafArgs a = args;
+    a.rows_per_wave = staf_rows_per_wave(ctx, a.n, c);
+    const uint32_t rows_per_wg = a.rows_per_wave * kWaves;
+    const uint32_t grid = (a.n + rows_per_wg - 1) / rows_per_wg;
+    auto go = [&](auto kernel) -> mi355q_status {
+        if (lds > 48 * 1024)
+            MI355Q_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(kWaves * 64), lds, s, a);
+        MI355Q_HIP(hipGetLastError());
+        return MI355Q_OK;
+    };
+    if (c.depth == 2) {
+        switch (mt) {
+        case 1: return go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 2>);
+        case 2: return go(gemv_staf_kernel<BITS, GROUP, 2, kWaves, 2>);
+        default: return go(gemv_staf_kernel<BITS, GROUP, 4, kWaves, 2>);
+        }
+    }
+    switch (mt) {
+    case 1: return go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 4>);
+    case 2: return go(gemv_staf_kernel<BITS, GROUP, 2, kWaves, 4>);
+    default: return go(gemv_staf_kernel<BITS, GROUP, 4, kWaves, 4>);
+    }
+}
+
+struct StafShape { uint32_t slot, q; };
+bool staf_shape(uint32_t bits, uint32_t group, StafShape& out) {
+#define MI355Q_STAF_CASE(B, GR) \
+    if (bits == B && group == GR) { out = {StafGeo<B, GR>::SLOT, StafGeo<B, GR>::Q}; return true; }
+    MI355Q_STAF_CASE(4, 64) MI355Q_STAF_CASE(4, 128) MI355Q_STAF_CASE(8, 32) MI355Q_STAF_CASE(8, 64)
+    MI355Q_STAF_CASE(2, 64) MI355Q_STAF_CASE(3, 64) MI355Q_STAF_CASE(5, 64) MI355Q_STAF_CASE(6, 64)
+#undef MI355Q_STAF_CASE
+    return false;
+}
+
+constexpr size_t kStafLdsBudget = 144 * 1024;
+
+int staf_max_mt(const WView& w, const StafShape& sh) {
+    const uint32_t nsp = (w.blocks_per_row + 63) / 64;
+    for (int mt = 4; mt >= 1; mt >>= 1)
+        if (staf_lds_bytes(sh.slot, sh.q, nsp, mt, staf_cfg().depth) <= kStafLdsBudget) return mt;
+    return 0;
+}
+
+}  // namespace
+
+bool gemv_staf_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
+    if (w.layout != MI355Q_LAYOUT_STAF_BLOCKS || x_dtype != MI355Q_BF16) return false;
+    if (m < 1 || m > 8 || !w.blocks) return false;
+    StafShape sh;
+    if (!staf_shape(w.bits, w.group, sh)) return false;
+    if (w.k % w.group) return false;
+    const uint64_t row_bytes = (uint64_t)w.blocks_per_row * w.bytes_per_block;
+    if (row_bytes % 16 || (uintptr_t)w.blocks % 16) return false;   // 128-bit loads of every row
+    if (x_stride % 8) return false;                                 // 128-bit activation loads
+    if ((uint64_t)w.n * row_bytes < 16) return false;
+    return staf_max_mt(w, sh) != 0;
+}
+
+GemvLaunchShape gemv_staf_shape(const mi355q_context* ctx, const WView& w, uint32_t m) {
+    GemvLaunchShape g{};
+    StafShape sh;
+    if (!staf_shape(w.bits, w.group, sh)) return g;
+    const int fit = staf_max_mt(w, sh);
+    int mt = m >= 3 ? 4 : (int)m;
+    if (mt > fit) mt = fit;
+    StafCfg c = staf_cfg();
+    g.lds_bytes = (uint32_t)staf_lds_bytes(sh.slot, sh.q, (w.blocks_per_row + 63) / 64, mt ? mt : 1, c.depth);
+    staf_one_workgroup_per_cu(g.lds_bytes, c);
+    const uint32_t rows_per_wg = staf_rows_per_wave(ctx, w.n, c) * kWaves;
+    g.grid = (w.n + rows_per_wg - 1) / rows_per_wg;
+    g.block = kWaves * 64;
+    g.rows_per_workgroup = rows_per_wg;
+    g.kernel = "gemv_staf";
+    return g;
+}
+
+mi355q_status launch_gemv_staf(hipStream_t s, const mi355q_context* ctx, const WView& w, const void* x, void* y,
+                               int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride) {
+    StafShape sh;
+    if (!staf_shape(w.bits, w.group, sh)) return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no block-layout GEMV for q%ug%u", w.bits, w.group);
+    const int fit = staf_max_mt(w, sh);
+    if (fit == 0) return fail(MI355Q_ERR_SHAPE, "K = %u is too long for the block-layout GEMV", w.k);
+    const size_t xsz = 2, ysz = y_dtype == MI355Q_F32 ? 4 : 2;
+    StafArgs a{};
+    a.blocks = w.blocks;
+    a.row_bytes = (uint64_t)w.blocks_per_row * w.bytes_per_block;
+    a.last_chunk = (uint64_t)w.n * a.row_bytes - 16;
+    a.k = w.k;
+    a.n = w.n;
+    a.x_stride = x_stride;
+    a.y_stride = y_stride;
+    a.y_dtype = (uint32_t)y_dtype;
+    a.blocks_per_row = w.blocks_per_row;
+    a.nsp = (w.blocks_per_row + 63) / 64;
+    for (uint32_t m0 = 0; m0 < m;) {
+        const uint32_t left = m - m0;
+        int mt = left >= 4 ? 4 : left >= 2 ? 2 : 1;          // 3 rows run as a 4-row launch with one row masked
+        if (left == 3) mt = 4;
+        if (mt > fit) mt = fit;
+        const uint32_t mm = left < (uint32_t)mt ? left : (uint32_t)mt;
+        a.x = (const uint16_t*)((const char*)x + (size_t)m0 * x_stride * xsz);
+        a.y = (char*)y + (size_t)m0 * y_stride * ysz;
+        a.m = mm;
+        mi355q_status st;
+#define MI355Q_STAF_LAUNCH(B, GR) \
+        if (w.bits == B && w.group == GR) st = launch_for_format<B, GR>(s, ctx, a, mt); else
+        MI355Q_STAF_LAUNCH(4, 64) MI355Q_STAF_LAUNCH(4, 128) MI355Q_STAF_LAUNCH(8, 32) MI355Q_STAF_LAUNCH(8, 64)
+        MI355Q_STAF_LAUNCH(2, 64) MI355Q_STAF_LAUNCH(3, 64) MI355Q_STAF_LAUNCH(5, 64) MI355Q_STAF_LAUNCH(6, 64)
+        st = MI355Q_ERR_KERNEL_NOT_FOUND;
+#undef MI355Q_STAF_LAUNCH
+        if (st != MI355Q_OK) return st;
+        m0 += mm;
+    }
+    return MI355Q_OK;
+}
+
+}  // namespace mi355q

@@ -44,7 +44,8 @@ int env_int(const char* name, int fallback) { return env_int_cached(name, fallba
 // Batches of 5 to 8 rows run as two launches: an 8-row variant of this kernel needs more registers
 // than a wavefront has.
 int max_mt(const WView& w) {
-    for (int mt = 4; mt >= 1; mt >>= 1)
+    // q2 g16 carries four scale groups per lane chunk: its 4-row variant does not fit the register file
+    for (int mt = (w.bits == 2 && w.group == 16) ? 2 : 4; mt >= 1; mt >>= 1)
         if (lds_bytes(w, mt) <= kLdsBudget) return mt;
     return 0;
 }
@@ -71,7 +72,7 @@ GemvCfg choose(const mi355q_context* ctx, const WView& w, uint32_t m, bool argma
         c.waves = (c.nc <= 2 && big) ? 4 : 8;
     } else {
         c.xreg = 0;
-        c.r = 2;
+        c.r = gemv_batch_rows((int)w.bits, (int)w.group, c.mt);
         c.waves = 4;
     }
     const int er = env_int("MI355Q_GEMV_R", 0), ew = env_int("MI355Q_GEMV_WAVES", 0),
@@ -93,7 +94,7 @@ GemvCfg choose(const mi355q_context* ctx, const WView& w, uint32_t m, bool argma
     // ring depth: four pipeline steps in flight, two when a wavefront only has two or three
     const uint32_t nsteps = rpw / (uint32_t)c.r * c.nc;
     if (c.mt == 1) c.depth = (nsteps >= 4 && (big || c.nc > 2)) ? 4 : 2;
-    else c.depth = c.mt == 2 ? 4 : 2;
+    else c.depth = gemv_batch_depth((int)w.bits, (int)w.group, c.mt);
     if (ed) c.depth = ed;
     const uint32_t rows_per_wg = rpw * (uint32_t)c.waves;
     c.grid = (w.n + rows_per_wg - 1) / rows_per_wg;

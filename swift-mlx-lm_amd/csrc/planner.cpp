@@ -63,6 +63,14 @@ void plan_small_m(const mi355q_weight* w, uint32_t m, int x_dtype, uint32_t x_st
         s->block[0] = g.block;
         s->lds_bytes = g.lds_bytes;
         s->rows_per_workgroup = g.rows_per_workgroup;
+    } else if (!forced && gemv_staf_eligible(v, x_dtype, m > 8 ? 8 : m, x_stride)) {
+        const GemvLaunchShape g = gemv_staf_shape(w->ctx, v, m > 8 ? 8 : m);
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_staf_q%u_g%u", (unsigned)w->fmt.bits,
+                      w->fmt.group_size);
+        s->grid[0] = g.grid;
+        s->block[0] = g.block;
+        s->lds_bytes = g.lds_bytes;
+        s->rows_per_workgroup = g.rows_per_workgroup;
     } else {
         std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_generic");
         s->grid[0] = (uint32_t)((w->n + 3) / 4);

@@ -1,0 +1,115 @@
+"""GPU parity tests of the decode GEMV that reads STAF interleaved blocks in place (no repacking),
+through the C ABI: the kernel a weight wrapped or uploaded straight from a model file runs
+(reference kernels gemv_q{b}_g{g}: MetalSourceGenerator+Quantized.swift:496-575, reading the block
+layout of QuantizationFormat.swift:1284-1312).
+
+Bars: fp32 outputs within relative L2 <= 1e-3 and max-abs <= 2e-2 of an fp64 accumulation of the
+same dequantised weights; bf16/f16 outputs equal the rounding of the fp32 outputs; the result of
+the per-code kernel (FLAG_FORCE_GENERIC) on the same buffers within the same bars.
+"""
+import sys
+
+import numpy as np
+import pytest
+
+import kat
+import oracle
+from gpu_util import Case, act_rounded, assert_within_tolerance, run_gemv
+
+pytestmark = pytest.mark.gpu
+
+# formats whose blocks are whole 32-bit words and that the in-place kernel is built for
+FORMATS = [(4, 64), (4, 128), (8, 32), (8, 64), (2, 64), (3, 64), (5, 64), (6, 64)]
+
+
+def say(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def _case(seed, n, k, bits, group):
+    rng = np.random.default_rng(seed)
+    codes = kat.random_codes(seed, n, k, bits)
+    scales = rng.integers(1, 400, size=(n, k // group)) / 16384.0       # exact in f16
+    zeros = rng.integers(-300, 300, size=(n, k // group)) / 8192.0
+    return Case(bits, group, codes, scales, zeros)
+
+
+def _row_alignment_k(bits, group):
+    """Smallest K whose row of blocks is a multiple of 16 bytes."""
+    bpb = 4 + group * bits // 8
+    blocks = 16 // int(np.gcd(16, bpb))
+    return blocks * group
+
+
+@pytest.mark.parametrize("bits,group", FORMATS)
+def test_in_place_gemv_formats_and_tails(pkg, ctx, bits, group):
+    """Rows shorter than one span of 64 blocks, exactly one span, one span plus a tail, several spans;
+    row counts that leave wavefronts partly or wholly past the end."""
+    unit = _row_alignment_k(bits, group)
+    ks = sorted({unit, 64 * group, 64 * group + unit, 3 * 64 * group + 2 * unit})
+    for ci, k in enumerate(ks):
+        for n in (1, 37, 700):
+            case = _case(3000 + bits * 7 + group + ci, n, k, bits, group)
+            w = case.device_weight(ctx, pkg, pkg.LAYOUT_STAF_BLOCKS)
+            wq = oracle.dequant_staf_f32(bits, group, n, k, case.staf_blocks())
+            for m in (1, 2, 3, 5, 8):
+                x = act_rounded(kat.seeded_activations(3100 + m + ci, m, k), pkg.BF16, pkg)
+                say(f"in-place q{bits}g{group} N={n} K={k} M={m}")
+                got = run_gemv(ctx, pkg, w, x, pkg.BF16, pkg.F32)
+                assert_within_tolerance(got, oracle.gemm_f64(wq, x), f"q{bits}g{group} N={n} K={k} M={m}")
+            w.destroy()
+
+
+def test_in_place_gemv_is_the_planned_kernel(pkg, ctx):
+    """The plan names the in-place kernel for a STAF-layout weight with bf16 activations, and the
+    per-code kernel when the row of blocks is not a multiple of 16 bytes or acceleration is off."""
+    case = _case(3200, 64, 4096, 4, 64)
+    w = case.device_weight(ctx, pkg, pkg.LAYOUT_STAF_BLOCKS)
+    step = w.plan_decode_step(1)
+    assert step.device_kernel == "gemv_staf_q4_g64" and not step.used_fallback, step.device_kernel
+    assert step.block[0] == 256 and step.grid[0] >= 1 and step.lds_bytes > 0
+    assert not w.plan_decode_step(1, pkg.F16).device_kernel.startswith("gemv_staf")   # bf16 activations only
+    forced = w.plan_decode_step(1, flags=pkg.FLAG_FORCE_GENERIC)
+    assert forced.device_kernel == "gemv_generic" and forced.used_fallback
+    w.destroy()
+    odd = _case(3201, 16, 64 * 3, 4, 64)                    # 108-byte rows
+    w = odd.device_weight(ctx, pkg, pkg.LAYOUT_STAF_BLOCKS)
+    assert w.plan_decode_step(1).device_kernel == "gemv_generic"
+    x = act_rounded(kat.seeded_activations(3202, 1, odd.k), pkg.BF16, pkg)
+    got = run_gemv(ctx, pkg, w, x, pkg.BF16, pkg.F32)
+    assert_within_tolerance(got, oracle.gemm_f64(oracle.dequant_staf_f32(4, 64, odd.n, odd.k, odd.staf_blocks()), x))
+    w.destroy()
+
+
+@pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336), (1024, 4096)])
+def test_in_place_gemv_llama_shapes(pkg, ctx, n, k):
+    """Llama-3-8B projection shapes at q4 g64, all output types, against the oracle and against the
+    per-code kernel on the same device buffers."""
+    case = _case(3300 + n % 97, n, k, 4, 64)
+    w = case.device_weight(ctx, pkg, pkg.LAYOUT_STAF_BLOCKS)
+    wq = oracle.dequant_staf_f32(4, 64, n, k, case.staf_blocks())
+    for m in (1, 4):
+        x = act_rounded(kat.seeded_activations(3310 + m, m, k), pkg.BF16, pkg)
+        say(f"in-place llama N={n} K={k} M={m}")
+        got = run_gemv(ctx, pkg, w, x, pkg.BF16, pkg.F32)
+        assert_within_tolerance(got, oracle.gemm_f64(wq, x), f"N={n} K={k} M={m}")
+        ref = run_gemv(ctx, pkg, w, x, pkg.BF16, pkg.F32, pkg.FLAG_FORCE_GENERIC)
+        assert_within_tolerance(got, ref, "against the per-code kernel")
+        gbf = run_gemv(ctx, pkg, w, x, pkg.BF16, pkg.BF16)
+        assert np.array_equal(oracle.bf16_from_f32(gbf), oracle.bf16_from_f32(got))
+        gh = run_gemv(ctx, pkg, w, x, pkg.BF16, pkg.F16)
+        assert np.array_equal(gh.astype(np.float16), got.astype(np.float16))
+    w.destroy()
+
+
+def test_in_place_gemv_strided_rows(pkg, ctx):
+    """Activation rows wider than K (x_row_stride > K): the padding is never read into the result."""
+    n, k, stride = 200, 4096, 4096 + 64
+    case = _case(3400, n, k, 4, 64)
+    w = case.device_weight(ctx, pkg, pkg.LAYOUT_STAF_BLOCKS)
+    wq = oracle.dequant_staf_f32(4, 64, n, k, case.staf_blocks())
+    x = np.full((3, stride), 1.0e6, np.float32)
+    x[:, :k] = act_rounded(kat.seeded_activations(3401, 3, k), pkg.BF16, pkg)
+    got = run_gemv(ctx, pkg, w, x, pkg.BF16, pkg.F32)
+    assert_within_tolerance(got, oracle.gemm_f64(wq, x[:, :k]), "strided rows")
+    w.destroy()
