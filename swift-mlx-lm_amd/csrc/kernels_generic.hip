@@ -96,6 +96,32 @@ mi355q_status launch_tile16_pack(hipStream_t s, const WView& planes, uint32_t* t
     return MI355Q_OK;
 }
 
+// Codes c0 .. c0+7 of a row (c0 a multiple of 8) as one little-endian bit string: code i sits at bit
+// i*bits.  A run of 8 codes starts on a byte boundary and spans at most 64 bits for every width.
+__device__ __forceinline__ uint64_t load_codes8(const WView& w, uint32_t row, uint32_t c0) {
+    uint64_t v = 0;
+    if (w.layout == MI355Q_LAYOUT_PLANES) {
+        const uint32_t* rowp = w.codes + (size_t)row * w.code_stride;
+        const uint32_t bit = c0 * w.bits, word = bit >> 5, sh = bit & 31u;
+        v = rowp[word];
+        if (sh + 8u * w.bits > 32u) v |= (uint64_t)rowp[word + 1] << 32;
+        v >>= sh;
+    } else if (w.layout == MI355Q_LAYOUT_STAF_BLOCKS) {
+        const uint32_t b = c0 / w.group, e = c0 - b * w.group;
+        const uint8_t* qs =
+            w.blocks + ((size_t)row * w.blocks_per_row + b) * w.bytes_per_block + 4 + ((e * w.bits) >> 3);
+        if (((uintptr_t)qs & 3u) == 0 && (w.bits & 3u) == 0) {
+            v = *(const uint32_t*)qs;
+            if (w.bits == 8) v |= (uint64_t)((const uint32_t*)qs)[1] << 32;
+        } else {
+            for (uint32_t i = 0; i < w.bits; i++) v |= (uint64_t)qs[i] << (8u * i);
+        }
+    } else {
+        for (uint32_t i = 0; i < 8; i++) v |= (uint64_t)load_code(w, row, c0 + i) << (i * w.bits);
+    }
+    return v;
+}
+
 // --------------------------------------------------------------------------- embedding lookup
 // out[pos, d] = (float(q) * scale + zero) [* embeddingScale] of table row token_ids[pos], rounded once to
 // the output type: embedding_lookup[_seq]_q{b}_g{g} of the reference
@@ -127,14 +153,70 @@ __global__ __launch_bounds__(256) void embedding_lookup_kernel(WView w, const in
     }
 }
 
+// The same lookup with eight consecutive dimensions per thread (one or two code loads, one scale/zero
+// pair, 128-bit stores): the variant for rows of whole 8-code runs and 16-byte aligned output rows.
+__global__ __launch_bounds__(256) void embedding_lookup_x8_kernel(WView w, const int32_t* __restrict__ token_ids,
+                                                                  uint32_t sequence_length, void* __restrict__ out,
+                                                                  uint32_t out_dtype, uint32_t out_stride, int has_scale,
+                                                                  float embedding_scale) {
+    const uint32_t per_row = w.k >> 3;
+    const uint64_t total = (uint64_t)sequence_length * per_row;
+    const uint32_t mask = (1u << w.bits) - 1u;
+    for (uint64_t t = (uint64_t)blockIdx.x * 256 + threadIdx.x; t < total; t += (uint64_t)gridDim.x * 256) {
+        const uint32_t pos = (uint32_t)(t / per_row), d0 = (uint32_t)(t - (uint64_t)pos * per_row) << 3;
+        const int32_t tok = token_ids[pos];
+        float f[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) f[i] = 0.0f;
+        if (tok >= 0 && (uint32_t)tok < w.n) {
+            const uint64_t v = load_codes8(w, (uint32_t)tok, d0);
+            float scale, zero;
+            load_scale_zero(w, (uint32_t)tok, d0 / w.group, scale, zero);
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const float q = (float)((uint32_t)(v >> (i * w.bits)) & mask);
+                f[i] = __fadd_rn(__fmul_rn(q, scale), zero);
+                if (has_scale) f[i] = __fmul_rn(f[i], embedding_scale);
+            }
+        }
+        const size_t o = (size_t)pos * out_stride + d0;
+        if (out_dtype == MI355Q_F32) {
+            typedef float f32x4 __attribute__((ext_vector_type(4)));
+            f32x4 a, b;
+            a.x = f[0]; a.y = f[1]; a.z = f[2]; a.w = f[3];
+            b.x = f[4]; b.y = f[5]; b.z = f[6]; b.w = f[7];
+            ((f32x4*)((float*)out + o))[0] = a;
+            ((f32x4*)((float*)out + o))[1] = b;
+        } else {
+            uint32_t h[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) h[i] = out_dtype == MI355Q_BF16 ? f32_to_bf16_rne(f[i]) : f32_to_f16_rne(f[i]);
+            u32x4 st;
+            st.x = h[0] | (h[1] << 16); st.y = h[2] | (h[3] << 16);
+            st.z = h[4] | (h[5] << 16); st.w = h[6] | (h[7] << 16);
+            *(u32x4*)((uint16_t*)out + o) = st;
+        }
+    }
+}
+
 mi355q_status launch_embedding_lookup(hipStream_t s, const WView& w, const int32_t* token_ids, uint32_t sequence_length,
                                       void* out, int out_dtype, uint32_t out_stride, int has_scale,
                                       float embedding_scale) {
-    uint32_t gx = (w.k + 255u) / 256u;
-    if (gx > 64u) gx = 64u;
-    embedding_lookup_kernel<<<dim3(gx, sequence_length), dim3(256), 0, s>>>(w, token_ids, sequence_length, out,
-                                                                           (uint32_t)out_dtype, out_stride, has_scale,
-                                                                           embedding_scale);
+    const size_t esz = out_dtype == MI355Q_F32 ? 4 : 2;
+    if (w.k % 8 == 0 && (uintptr_t)out % 16 == 0 && ((size_t)out_stride * esz) % 16 == 0) {
+        const uint64_t tasks = (uint64_t)sequence_length * (w.k / 8);
+        uint64_t blocks = (tasks + 255) / 256;
+        if (blocks > (1u << 20)) blocks = 1u << 20;
+        if (blocks == 0) blocks = 1;
+        embedding_lookup_x8_kernel<<<dim3((unsigned)blocks), dim3(256), 0, s>>>(
+            w, token_ids, sequence_length, out, (uint32_t)out_dtype, out_stride, has_scale, embedding_scale);
+    } else {
+        uint32_t gx = (w.k + 255u) / 256u;
+        if (gx > 64u) gx = 64u;
+        embedding_lookup_kernel<<<dim3(gx, sequence_length), dim3(256), 0, s>>>(w, token_ids, sequence_length, out,
+                                                                               (uint32_t)out_dtype, out_stride,
+                                                                               has_scale, embedding_scale);
+    }
     MI355Q_HIP(hipGetLastError());
     return MI355Q_OK;
 }
@@ -155,9 +237,44 @@ __global__ __launch_bounds__(256) void dequant_bf16_kernel(WView w, uint16_t* __
     }
 }
 
+// Eight consecutive codes per thread: one or two 32-bit loads of codes (a run of 8 codes starts on a
+// byte boundary and spans at most 64 bits for every width), one scale/zero pair (groups are multiples
+// of 8 codes), one 128-bit store.  Same arithmetic as the per-element kernel above.
+__global__ __launch_bounds__(256) void dequant_bf16_x8_kernel(WView w, uint16_t* __restrict__ out) {
+    const uint32_t per_row = w.k >> 3;
+    const uint64_t total = (uint64_t)w.n * per_row;
+    const uint32_t mask = (1u << w.bits) - 1u;
+    for (uint64_t t = (uint64_t)blockIdx.x * 256 + threadIdx.x; t < total; t += (uint64_t)gridDim.x * 256) {
+        const uint32_t row = (uint32_t)(t / per_row), c0 = (uint32_t)(t - (uint64_t)row * per_row) << 3;
+        const uint64_t v = load_codes8(w, row, c0);
+        float scale, zero;
+        load_scale_zero(w, row, c0 / w.group, scale, zero);
+        uint32_t o[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float q0 = (float)((uint32_t)(v >> ((2 * i) * w.bits)) & mask);
+            const float q1 = (float)((uint32_t)(v >> ((2 * i + 1) * w.bits)) & mask);
+            const uint32_t lo = f32_to_bf16_rne(__fadd_rn(__fmul_rn(scale, q0), zero));
+            const uint32_t hi = f32_to_bf16_rne(__fadd_rn(__fmul_rn(scale, q1), zero));
+            o[i] = lo | (hi << 16);
+        }
+        u32x4 st;
+        st.x = o[0]; st.y = o[1]; st.z = o[2]; st.w = o[3];
+        __builtin_nontemporal_store(st, (u32x4*)(out + (size_t)row * w.k + c0));
+    }
+}
+
 mi355q_status launch_dequant_bf16(hipStream_t s, const WView& w, uint16_t* out) {
-    unsigned blocks = w.n < 65535u * 16u ? w.n : 65535u * 16u;
-    dequant_bf16_kernel<<<dim3(blocks), dim3(256), 0, s>>>(w, out);
+    if (w.k % 8 == 0 && (uintptr_t)out % 16 == 0) {
+        const uint64_t tasks = (uint64_t)w.n * (w.k / 8);
+        uint64_t blocks = (tasks + 255) / 256;
+        if (blocks > (1u << 20)) blocks = 1u << 20;
+        if (blocks == 0) blocks = 1;
+        dequant_bf16_x8_kernel<<<dim3((unsigned)blocks), dim3(256), 0, s>>>(w, out);
+    } else {
+        unsigned blocks = w.n < 65535u * 16u ? w.n : 65535u * 16u;
+        dequant_bf16_kernel<<<dim3(blocks), dim3(256), 0, s>>>(w, out);
+    }
     MI355Q_HIP(hipGetLastError());
     return MI355Q_OK;
 }
