@@ -216,8 +216,11 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
     };
 
     const uint32_t rounds = (a.blocks_per_wave + D - 1) / D;            // same for every wavefront
-    // partial tiles of the WAVES wavefronts, behind the activations and their group sums
-    float* const red = (float*)(lds + (size_t)a.m * a.lds_row_bytes + a.k);          // [WAVES][MR][64]
+    // Partial tiles of the WAVES wavefronts, [WAVES][MR][64]: a single pass writes them over the staged activations
+    // once every wavefront is done reading those (the workgroup then needs no LDS beyond the activations, which
+    // decides how many workgroups share a CU); several passes keep them behind the activations and their sums.
+    const bool red_over_x = a.passes == 1;
+    float* const red = (float*)(red_over_x ? lds : lds + (size_t)a.m * a.lds_row_bytes + a.k);
     unsigned long long best = 0ull;
     for (uint32_t pass = 0; pass < a.passes; pass++) {
         if (pass) {                                            // the first tile's loads were issued before staging
@@ -234,6 +237,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
         }
 
         // ---- 5. add the partial tiles of the wavefronts that share a row tile, store ----------------
+        if (red_over_x) __syncthreads();
 #pragma unroll
         for (int r = 0; r < MR; r++) { red[(wave * MR + r) * 64 + lane] = acc[r]; acc[r] = 0.f; }
         __syncthreads();
@@ -336,13 +340,17 @@ Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_total_
     const uint32_t want_tpw = m == 1 ? 1u : m <= 4 ? 2u : 4u;
     uint32_t tpw = 1;
     while (tpw < want_tpw && ks * tpw * 2 <= 16 && (n_total_tiles + tpw * 2 - 1) / (tpw * 2) >= cus / 2) tpw *= 2;
-    const bool one_wg_per_cu = (size_t)m * ((size_t)k * 2 + 16) > 80 * 1024;
+    // The staged activations leave room for one workgroup per CU: sixteen wavefronts.  With at least three row tiles
+    // per CU they take four row tiles at a time (each wavefront keeps a quarter of K: long enough a stream to fill
+    // its prefetch ring) and walk further tiles in passes; with fewer, all sixteen share one row tile.
+    const bool big_x = (size_t)m * ((size_t)k * 2 + 16) > 80 * 1024;
+    const bool one_wg_per_cu = big_x && n_total_tiles >= 3 * cus;
     if (one_wg_per_cu) {
-        // the staged activations leave room for one workgroup per CU: sixteen wavefronts, four row tiles at a time
-        // (each wavefront keeps a quarter of K: long enough a stream to fill its prefetch ring)
-        ks = kblocks >= 8 ? 4 : (kblocks >= 4 ? 2 : 1);
-        if (ks < 4) ks = 4;                                  // the built variants split K four ways at least
+        ks = 4;
         tpw = 4;
+    } else if (big_x) {
+        tpw = 1;
+        while (ks < 16 && kblocks / (ks * 2) >= 2) ks *= 2;
     }
     const int eks = env_int_cached("MI355Q_T16_KSPLIT", 0), etpw = env_int_cached("MI355Q_T16_TPW", 0);
     if (eks) ks = (uint32_t)eks;
@@ -370,7 +378,7 @@ Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_total_
     g.block = g.waves * 64;
     const size_t x_bytes = (size_t)m * ((size_t)k * 2 + 16) + k;     // rows, then sum(x) per group: [K/64][16] floats
     const size_t red_bytes = (size_t)g.waves * 4 * 64 * 4;     // partial tiles, behind the activations
-    g.lds_bytes = (uint32_t)(x_bytes + red_bytes);
+    g.lds_bytes = (uint32_t)(g.passes > 1 ? x_bytes + red_bytes : (x_bytes > red_bytes ? x_bytes : red_bytes));
     return g;
 }
 

@@ -47,8 +47,15 @@ void plan_small_m(const mi355q_weight* w, uint32_t m, int x_dtype, uint32_t x_st
                   mi355q_step* s) {
     const WView v = w->view();
     const bool forced = flags & MI355Q_FLAG_FORCE_GENERIC;
-    if (!forced && gemv_tile16_eligible(v, x_dtype, m > 16 ? 16 : m, x_stride)) {
-        const Tile16LaunchShape g = gemv_tile16_shape(w->ctx, (uint32_t)((w->n + 15) / 16), (uint32_t)w->k, m > 16 ? 16 : m);
+    // rows per launch on the tile layout: 16, or fewer when K is so long that 16 staged rows overflow LDS
+    uint32_t t16_rows = m > 16 ? 16 : m;
+    if (!forced && v.layout == MI355Q_LAYOUT_TILE16) {
+        uint32_t step = 16;
+        while (step > 1 && !gemv_tile16_eligible(v, x_dtype, step, x_stride)) step >>= 1;
+        if (t16_rows > step) t16_rows = step;
+    }
+    if (!forced && gemv_tile16_eligible(v, x_dtype, t16_rows, x_stride)) {
+        const Tile16LaunchShape g = gemv_tile16_shape(w->ctx, (uint32_t)((w->n + 15) / 16), (uint32_t)w->k, t16_rows);
         std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_tile16_q%u_g%u", (unsigned)w->fmt.bits,
                       w->fmt.group_size);
         s->grid[0] = g.grid;
