@@ -69,7 +69,8 @@ typedef enum {
     MI355Q_LAYOUT_PLANES = 1,
     /* Matrix-core decode layout (4-bit, group 64, K % 128 == 0): records of 16 rows x 128 codes in
      * the order a wavefront loads them, each followed by its (scale, bias) words.  Serves
-     * 1 <= M <= 16 at the cost of M = 1; prefill on this layout runs in slices of 16 rows. */
+     * 1 <= M <= 16 per launch at nearly the cost of M = 1; the prefill GEMM on the matrix cores
+     * reads the same records. */
     MI355Q_LAYOUT_TILE16 = 2
 } mi355q_layout;
 
