@@ -277,15 +277,20 @@ def main():
     other = None
     if not a.no_other_configs:
         other = {}
-        cases = [("config0 q4g64 2048->8192", 4, 64, 8192, 2048, False), ("config2 q8g32 4096->14336", 8, 32, 14336, 4096, False),
-                 ("config2 q6g64 4096->14336", 6, 64, 14336, 4096, False), ("config2 q3g64 4096->14336", 3, 64, 14336, 4096, False),
-                 ("config2 q2g64 4096->14336", 2, 64, 14336, 4096, False), ("config4 q4g64 lm head 2048->65536 + argmax", 4, 64, 65536, 2048, True)]
-        for ci, (label, bits, group, n, k, head) in enumerate(cases):
+        P, S = pkg.LAYOUT_PLANES, pkg.LAYOUT_STAF_BLOCKS
+        cases = [("config0 q4g64 2048->8192", 4, 64, 8192, 2048, False, P), ("config2 q8g32 4096->14336", 8, 32, 14336, 4096, False, P),
+                 ("config2 q6g64 4096->14336", 6, 64, 14336, 4096, False, P), ("config2 q3g64 4096->14336", 3, 64, 14336, 4096, False, P),
+                 ("config2 q2g64 4096->14336", 2, 64, 14336, 4096, False, P),
+                 ("config4 q4g64 lm head 2048->65536 + argmax", 4, 64, 65536, 2048, True, P),
+                 # the same gate / down projections left in the reference's interleaved blocks (no re-layout at load)
+                 ("config1 gate q4g64 4096->14336, STAF blocks in place", 4, 64, 14336, 4096, False, S),
+                 ("config1 down q4g64 14336->4096, STAF blocks in place", 4, 64, 4096, 14336, False, S)]
+        for ci, (label, bits, group, n, k, head, layout) in enumerate(cases):
             f2 = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(bits, group)
             words, s, z = oracle.quantize_affine(kat.seeded_weights(3000 + ci, n, k), bits, group, oracle.BF16)
             nbytes = n * (k // group) * (4 + group * bits // 8)
             copies = max(2, min(64, int(5.4e8 // nbytes) + 1))
-            ws = [ctx.weight_prepare_mlx(f2, words, s, z, pkg.BF16, pkg.LAYOUT_PLANES) for _ in range(copies)]
+            ws = [ctx.weight_prepare_mlx(f2, words, s, z, pkg.BF16, layout) for _ in range(copies)]
             x1 = oracle.bf16_to_f32(oracle.bf16_from_f32(kat.seeded_activations(3100 + ci, 1, k))).reshape(1, k)
             xd1 = ctx.upload(oracle.bf16_from_f32(x1))
             yd1, logits, tok = ctx.alloc(n * 2), ctx.alloc(n * 4), ctx.alloc(16)

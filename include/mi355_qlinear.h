@@ -308,7 +308,9 @@ MI355Q_API mi355q_status mi355q_unpack_codes(mi355q_context* ctx, void* stream,
 /* argmax / argmax_f32 (generateArgmax, MC/Generator/MetalSourceGenerator+Sampling.swift:62-107;
  * bindings 0=logits 1=int* result 2=vocabularySize).  Strict '>' from -inf with index 0 as
  * the start value: NaN never wins; ties resolve to the LOWEST index (a rule this library adds:
- * the reference's reduction order does not define ties). */
+ * the reference's reduction order does not define ties).  Vocabulary-sized vectors run as two
+ * launches through a small scratch of the context, as the fused head below does: calls on one
+ * context that overlap in time (different streams) race on it; give each stream its own context. */
 MI355Q_API mi355q_status mi355q_argmax(mi355q_context* ctx, void* stream, const void* logits_dev,
                                        mi355q_dtype dtype, uint32_t vocabulary_size,
                                        int32_t* token_out_dev);

@@ -178,7 +178,7 @@ mi355q_status dispatch_output_head(mi355q_context* ctx, hipStream_t s, const mi3
     else
         st = launch_gemv_generic(s, v, x, x_dtype, logits, MI355Q_F32, 1, xs, (uint32_t)w->n);
     if (st != MI355Q_OK) return st;
-    return launch_argmax(s, logits, MI355Q_F32, (uint32_t)w->n, token);
+    return launch_argmax(s, logits, MI355Q_F32, (uint32_t)w->n, token, ctx->argmax_partials + kArgmaxPartialCapacity);
 }
 
 }  // namespace mi355q
@@ -262,7 +262,8 @@ mi355q_status mi355q_argmax(mi355q_context* ctx, void* stream, const void* logit
     if (!logits_dev || !token_out_dev) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null pointer");
     if (!dtype_ok(dtype)) return fail(MI355Q_ERR_INVALID_ARGUMENT, "bad dtype tag");
     MI355Q_HIP(hipSetDevice(ctx->device));
-    return launch_argmax((hipStream_t)stream, logits_dev, dtype, vocabulary_size, token_out_dev);
+    return launch_argmax((hipStream_t)stream, logits_dev, dtype, vocabulary_size, token_out_dev,
+                         ctx->argmax_partials + kArgmaxPartialCapacity);
 }
 
 mi355q_status mi355q_lmhead_argmax(mi355q_context* ctx, void* stream, const mi355q_weight* w, const void* x_dev,

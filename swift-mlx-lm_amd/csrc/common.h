@@ -57,6 +57,7 @@ struct mi355q_context {
     // small cells: [16..17] clock probe of the prefill GEMM, [24] sink of the read-only probe launch
     unsigned long long* argmax_scratch;
     // fused output head: one packed (ordered value, ~row) key per workgroup of the projection launch
+    // (kArgmaxPartialCapacity entries), then kArgmaxStandaloneKeys entries for the stand-alone argmax
     unsigned long long* argmax_partials;
     // split-K partial results of the prefill GEMM: grown on demand, never shrunk
     void* workspace;
@@ -120,8 +121,10 @@ mi355q_status launch_embedding_lookup(hipStream_t s, const WView& w, const int32
 // Partial keys of the fused output head: one per workgroup of the projection launch.
 constexpr uint32_t kArgmaxPartialCapacity = 65536;
 mi355q_status launch_argmax_finish(hipStream_t s, const unsigned long long* partial, uint32_t count, int32_t* token_out);
+// `partial`: 256 keys of scratch for the two-launch form taken by long vectors (null: always one workgroup).
+constexpr uint32_t kArgmaxStandaloneKeys = 256;
 mi355q_status launch_argmax(hipStream_t s, const void* logits, int dtype, uint32_t n,
-                            int32_t* token_out);
+                            int32_t* token_out, unsigned long long* partial);
 mi355q_status launch_pack_sz(hipStream_t s, const uint16_t* scales, const uint16_t* biases, uint32_t* sz,
                              size_t groups, uint32_t blocks_per_row, uint32_t sz_stride);
 

@@ -387,7 +387,52 @@ mi355q_status launch_argmax_finish(hipStream_t s, const unsigned long long* part
     return MI355Q_OK;
 }
 
-mi355q_status launch_argmax(hipStream_t s, const void* logits, int dtype, uint32_t n, int32_t* token_out) {
+// First step of the two-launch argmax for long vectors: one packed (ordered value, ~index) key per workgroup, the
+// same key the fused output head leaves behind (-0 counts as +0, NaN and -inf never contribute).
+template <int D>
+__global__ __launch_bounds__(256) void argmax_partial_kernel(const void* __restrict__ logits, uint32_t n,
+                                                             unsigned long long* __restrict__ partial) {
+    __shared__ unsigned long long s_key[4];
+    unsigned long long best = 0ull;
+    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < n; i += gridDim.x * 256u) {
+        const float v = load_act<D>(logits, i);
+        if (v > -INFINITY) {
+            const uint32_t u = __float_as_uint(v + 0.0f);
+            const uint32_t key = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+            const unsigned long long pk = ((unsigned long long)key << 32) | (unsigned long long)(0xFFFFFFFFu - i);
+            best = pk > best ? pk : best;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const uint32_t hi = (uint32_t)__shfl_xor((int)(best >> 32), off, 64);
+        const uint32_t lo = (uint32_t)__shfl_xor((int)(best & 0xFFFFFFFFull), off, 64);
+        const unsigned long long o = ((unsigned long long)hi << 32) | lo;
+        best = o > best ? o : best;
+    }
+    if ((threadIdx.x & 63) == 0) s_key[threadIdx.x >> 6] = best;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int i = 1; i < 4; i++) best = s_key[i] > best ? s_key[i] : best;
+        partial[blockIdx.x] = best;
+    }
+}
+
+// One workgroup for short vectors; for long ones (a vocabulary) up to 256 workgroups leave one key each in
+// `partial` (at least 256 entries; may be null, then the single workgroup runs) and a second launch picks the token.
+mi355q_status launch_argmax(hipStream_t s, const void* logits, int dtype, uint32_t n, int32_t* token_out,
+                            unsigned long long* partial) {
+    if (partial && n >= 16384) {
+        uint32_t groups = (n + 1023) / 1024;
+        if (groups > 256) groups = 256;
+        switch (dtype) {
+        case MI355Q_F16: argmax_partial_kernel<MI355Q_F16><<<dim3(groups), dim3(256), 0, s>>>(logits, n, partial); break;
+        case MI355Q_BF16: argmax_partial_kernel<MI355Q_BF16><<<dim3(groups), dim3(256), 0, s>>>(logits, n, partial); break;
+        default: argmax_partial_kernel<MI355Q_F32><<<dim3(groups), dim3(256), 0, s>>>(logits, n, partial); break;
+        }
+        MI355Q_HIP(hipGetLastError());
+        return launch_argmax_finish(s, partial, groups, token_out);
+    }
     switch (dtype) {
     case MI355Q_F16: argmax_kernel<MI355Q_F16><<<dim3(1), dim3(1024), 0, s>>>(logits, n, token_out); break;
     case MI355Q_BF16: argmax_kernel<MI355Q_BF16><<<dim3(1), dim3(1024), 0, s>>>(logits, n, token_out); break;

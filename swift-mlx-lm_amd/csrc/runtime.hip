@@ -217,7 +217,7 @@ mi355q_status mi355q_context_create(int device_index, mi355q_context** out) {
     }
     e = hipMalloc((void**)&ctx->argmax_scratch, 256);
     if (e == hipSuccess) e = hipMemset(ctx->argmax_scratch, 0, 256);
-    if (e == hipSuccess) e = hipMalloc((void**)&ctx->argmax_partials, (size_t)kArgmaxPartialCapacity * 8);
+    if (e == hipSuccess) e = hipMalloc((void**)&ctx->argmax_partials, (size_t)(kArgmaxPartialCapacity + kArgmaxStandaloneKeys) * 8);
     if (e != hipSuccess) {
         if (ctx->argmax_scratch) (void)hipFree(ctx->argmax_scratch);
         if (ctx->argmax_partials) (void)hipFree(ctx->argmax_partials);

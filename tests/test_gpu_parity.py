@@ -229,13 +229,21 @@ def test_argmax_ties_nan_and_boundaries(pkg, ctx):
                 np.array([np.nan, -np.inf, -np.inf], np.float32), np.zeros(70000, np.float32)]
     for v in specials:
         assert _argmax_dev(pkg, ctx, v, pkg.F32) == oracle.argmax_lowest(v)
-    for n in (1, 2, 63, 64, 65, 1023, 1024, 1025, 2049, 65536, 70001):
+    # vocabulary-sized vectors take the two-launch form: the same rules must hold across its workgroups
+    big = 40000
+    for v in (np.full(big, np.nan, np.float32), np.full(big, -np.inf, np.float32),
+              np.where(np.arange(big) % 2 == 0, -0.0, 0.0).astype(np.float32),
+              np.concatenate([np.full(big - 1, -np.inf, np.float32), [-3.0e38]]).astype(np.float32),
+              np.concatenate([np.full(big - 2, np.nan, np.float32), [np.inf, np.inf]]).astype(np.float32)):
+        assert _argmax_dev(pkg, ctx, v, pkg.F32) == oracle.argmax_lowest(v)
+    for n in (1, 2, 63, 64, 65, 1023, 1024, 1025, 2049, 16383, 16384, 16385, 65536, 70001, 262144):
         for _ in range(3):
             v = rng.integers(-3, 4, size=n).astype(np.float32)         # dense ties
             for dtype in (pkg.F32, pkg.BF16, pkg.F16):
                 assert _argmax_dev(pkg, ctx, v, dtype) == int(np.argmax(v)) == oracle.argmax_lowest(v)
         # one maximum duplicated across a lane / wavefront / workgroup-stride boundary
-        for a, b in [(0, n - 1), (n // 2, n - 1), (63 % n, 64 % n), (1023 % n, 1024 % n)]:
+        for a, b in [(0, n - 1), (n // 2, n - 1), (63 % n, 64 % n), (1023 % n, 1024 % n), (255 % n, 256 % n),
+                     (65535 % n, 65536 % n)]:
             v = rng.standard_normal(n).astype(np.float32)
             v[a] = v[b] = 100.0
             assert _argmax_dev(pkg, ctx, v, pkg.F32) == min(a, b)
