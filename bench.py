@@ -338,6 +338,42 @@ def main():
         f"(the {dom} launch reaches {achieved / stream_read['GBps'] * 100:.0f} % of it)")
     pbuf.free()
 
+    # ---- secondary: the same 4-launch step over weights left in the reference's interleaved STAF blocks (what a
+    # model.staf payload wrapped with no copy gives): 8 resident layer copies (1 GB), stream replay
+    staf_step = None
+    if not a.no_other_configs:
+        saved, layers = layers, []
+        for _ in range(8):
+            layers.append({name: ctx.weight_prepare_mlx(fmt, *host[name], pkg.BF16, pkg.LAYOUT_STAF_BLOCKS)
+                           for name, _, _ in LAYER_SHAPES})
+        if not a.skip_parity:
+            name, n, k = LAYER_SHAPES[-1]
+            words, s_, z_ = host[name]
+            want = oracle.gemm_f64(oracle.dequant_planes_f32(BITS, GROUP, n, k, words, s_, z_, oracle.BF16), xs[k])[0]
+            y32 = ctx.alloc(n * 4)
+            ctx.qgemv(layers[-1][name], xdev[k], pkg.BF16, y32, pkg.F32, 1)
+            ctx.synchronize()
+            got = y32.download(np.float32)
+            y32.free()
+            rel = float(np.linalg.norm(got - want) / np.linalg.norm(want))
+            if rel > 1e-3:
+                sys.exit(f"bench.py: parity gate failed on the in-place STAF {name} projection: rel-L2 {rel:.3e}")
+        plan = build_plan(True)
+        per_layer = len(plan) // len(layers)
+        for i in range(16):
+            plan.encode(stream, (i % 8) * per_layer, per_layer)
+        ctx.synchronize(stream)
+        ms = time_region(ctx, lambda i: plan.encode(stream, (i % 8) * per_layer, per_layer), 160, stream)
+        ctx.synchronize(stream)
+        staf_step = {"us_per_step": round(ms * 1e3, 2), "GBps": round(layer_bytes / (ms * 1e-3) / 1e9, 1),
+                     "kernel": plan.step(per_layer - 1)[0].device_kernel}
+        log(f"4-launch step on STAF blocks in place: {staf_step['us_per_step']} us/step, {staf_step['GBps']} GB/s")
+        plan.destroy()
+        for L in layers:
+            for w in L.values():
+                w.destroy()
+        layers = saved
+
     # ---- secondary figure: the prefill GEMM of the same layer's gate projection (not the metric)
     prefill = None
     if not a.no_prefill:
@@ -393,7 +429,8 @@ def main():
                    "weight_bytes_per_step": layer_bytes, "layers_resident": a.layers,
                    "replay": mode, "replay_GBps": replay_gbps,
                    "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2), "per_shape": per_shape,
-                   "batch_sweep": batch_sweep, "other_configs": other, "stream_read_probe": stream_read,
+                   "batch_sweep": batch_sweep, "other_configs": other, "staf_blocks_in_place_step": staf_step,
+                   "stream_read_probe": stream_read,
                    "prefill_gemm_gate": prefill},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": TRAFFIC_BYTES[dom],

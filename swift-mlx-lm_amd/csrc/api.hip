@@ -130,6 +130,7 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
     }
     bool fused = m <= 8 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
     bool tiled = m <= 16 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
+    bool in_place = m <= 8 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
     WView views[3];
     uint32_t strides[3];
     for (uint32_t i = 0; i < count; i++) {
@@ -140,12 +141,15 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
         views[i] = weights[i]->view();
         fused = fused && gemv_fast_eligible(views[i], x_dtype, m, xs) && views[i].sb_dtype == views[0].sb_dtype;
         tiled = tiled && gemv_tile16_eligible(views[i], x_dtype, m, xs) && views[i].sb_dtype == views[0].sb_dtype;
+        in_place = in_place && gemv_staf_eligible(views[i], x_dtype, m, xs);
     }
     if (fused && (uintptr_t)x % 16 == 0)
         return launch_gemv_fast_multi(s, ctx, count, views, x, ys, strides, y_dtype, m, xs, nullptr, nullptr, nullptr);
     if (tiled && (uintptr_t)x % 16 == 0)
         return launch_gemv_tile16_multi(s, ctx, count, views, x, ys, strides, y_dtype, m, xs, nullptr, nullptr,
                                         nullptr);
+    if (in_place && (uintptr_t)x % 16 == 0)
+        return launch_gemv_staf_multi(s, ctx, count, views, x, ys, strides, y_dtype, m, xs, nullptr, nullptr, nullptr);
     for (uint32_t i = 0; i < count; i++) {
         mi355q_status st = dispatch_linear(ctx, s, weights[i], x, x_dtype, ys[i], y_dtype, m, xs, 0, flags, false);
         if (st != MI355Q_OK) return st;
@@ -168,15 +172,17 @@ mi355q_status dispatch_output_head(mi355q_context* ctx, hipStream_t s, const mi3
         return launch_gemv_tile16_multi(s, ctx, 1, &v, x, none, strides, MI355Q_F32, 1, xs, logits, token,
                                         ctx->argmax_partials);
     }
+    if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && gemv_staf_eligible(v, x_dtype, 1, xs) && (uintptr_t)x % 16 == 0) {
+        void* none[1] = {nullptr};
+        const uint32_t strides[1] = {(uint32_t)w->n};
+        return launch_gemv_staf_multi(s, ctx, 1, &v, x, none, strides, MI355Q_F32, 1, xs, logits, token,
+                                      ctx->argmax_partials);
+    }
     // two dispatches, as the reference runs the head: projection to fp32 logits, then argmax
     if (!logits)
         return fail(MI355Q_ERR_INVALID_ARGUMENT,
                     "a logits buffer is required when the fused head kernel does not accept the shape");
-    mi355q_status st;
-    if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && gemv_staf_eligible(v, x_dtype, 1, xs) && (uintptr_t)x % 16 == 0)
-        st = launch_gemv_staf(s, ctx, v, x, logits, MI355Q_F32, 1, xs, (uint32_t)w->n);
-    else
-        st = launch_gemv_generic(s, v, x, x_dtype, logits, MI355Q_F32, 1, xs, (uint32_t)w->n);
+    mi355q_status st = launch_gemv_generic(s, v, x, x_dtype, logits, MI355Q_F32, 1, xs, (uint32_t)w->n);
     if (st != MI355Q_OK) return st;
     return launch_argmax(s, logits, MI355Q_F32, (uint32_t)w->n, token, ctx->argmax_partials + kArgmaxPartialCapacity);
 }

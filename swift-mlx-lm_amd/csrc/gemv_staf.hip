@@ -30,14 +30,20 @@ namespace {
 
 #define MI355Q_LDS_PTR(p) ((__attribute__((address_space(3))) uint8_t*)(p))
 
+// One launch covers up to three weight matrices that share K, format and activations (q+k+v, gate+up): wavefronts
+// are dealt to the matrices whole, matrix i owns the wavefronts [wave_end[i-1], wave_end[i]).
 struct StafArgs {
-    const uint8_t* blocks;
+    const uint8_t* blocks[kGemvMaxSegments];
+    void* y[kGemvMaxSegments];                 // [M, y_stride[i]] in y_dtype (may be null when only logits are wanted)
+    uint32_t wave_end[kGemvMaxSegments];       // cumulative wavefront counts; unused entries repeat the last
+    uint32_t seg_rows[kGemvMaxSegments];       // N_i
+    uint32_t y_stride[kGemvMaxSegments];
     const uint16_t* x;       // bf16 [M, x_stride]
-    void* y;                 // [M, y_stride] in y_dtype
+    float* logits;           // optional fp32 [N] copy (M == 1, single matrix)
+    unsigned long long* scratch;   // ARGMAX only: one packed (ordered value, ~row) key per workgroup
     uint64_t row_bytes;      // blocks_per_row * bytes per block (a multiple of 16)
-    uint64_t last_chunk;     // byte offset of the last whole 16-byte chunk of the weight buffer
-    uint32_t k, n, m;
-    uint32_t x_stride, y_stride, y_dtype;
+    uint32_t k, m;
+    uint32_t x_stride, y_dtype;
     uint32_t blocks_per_row;
     uint32_t nsp;            // spans per row = ceil(blocks_per_row / 64)
     uint32_t rows_per_wave;
@@ -53,7 +59,7 @@ struct StafGeo {
     static constexpr int Q = GROUP / 8;                     // staged activation pieces (8 elements each) per block
 };
 
-template <int BITS, int GROUP, int MT, int WAVES, int D>
+template <int BITS, int GROUP, int MT, int WAVES, int D, bool ARGMAX>
 __global__ __launch_bounds__(WAVES * 64) void gemv_staf_kernel(const StafArgs a) {
     using G = StafGeo<BITS, GROUP>;
     constexpr int WPB = G::WPB, BW = G::BW, SPAN = G::SPAN, NDMA = G::NDMA, SLOT = G::SLOT, Q = G::Q;
@@ -70,20 +76,30 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_staf_kernel(const StafArgs a)
     uint8_t* const ring = lds + (size_t)MT * NSP * (Q * 1024 + 256) + (size_t)wave * D * SLOT;
     const uint32_t ring_lds = (uint32_t)(uintptr_t)MI355Q_LDS_PTR(ring);
 
-    const uint32_t row0 = (blockIdx.x * WAVES + wave) * a.rows_per_wave;
+    // the matrix this wavefront works on (scalar select chain); wavefronts past the last matrix fall on rows past
+    // its end: their loads are clamped and nothing is stored
+    const uint32_t gw = blockIdx.x * WAVES + wave;
+    const uint32_t seg = gw < a.wave_end[0] ? 0u : (gw < a.wave_end[1] ? 1u : 2u);
+    const uint32_t first_wave = seg == 0 ? 0u : a.wave_end[seg - 1];
+    const uint8_t* const seg_blocks = seg == 0 ? a.blocks[0] : (seg == 1 ? a.blocks[1] : a.blocks[2]);
+    void* const seg_y = seg == 0 ? a.y[0] : (seg == 1 ? a.y[1] : a.y[2]);
+    const uint32_t seg_n = seg == 0 ? a.seg_rows[0] : (seg == 1 ? a.seg_rows[1] : a.seg_rows[2]);
+    const uint32_t seg_ys = seg == 0 ? a.y_stride[0] : (seg == 1 ? a.y_stride[1] : a.y_stride[2]);
+    const uint64_t last_chunk = (uint64_t)seg_n * a.row_bytes - 16;    // last whole 16-byte chunk of the matrix
+    const uint32_t row0 = gw < a.wave_end[kGemvMaxSegments - 1] ? (gw - first_wave) * a.rows_per_wave : seg_n;
     const uint32_t nsteps = a.rows_per_wave * NSP;
 
     // ---- 1. the first D spans go out before anything else ----------------------------------------
     uint32_t irow = 0, isp = 0;                              // next span to issue
     auto issue = [&](uint32_t slot) {
         uint32_t row = row0 + irow;
-        row = row < a.n ? row : a.n - 1;                     // rows past the end of the matrix reload its last row
+        row = row < seg_n ? row : seg_n - 1;                 // rows past the end of the matrix reload its last row
         const uint64_t base = (uint64_t)row * a.row_bytes + (uint64_t)isp * SPAN + (uint64_t)lane * 16;
 #pragma unroll
         for (int i = 0; i < NDMA; i++) {
             uint64_t off = base + (uint64_t)i * 1024;
-            off = off < a.last_chunk ? off : a.last_chunk;
-            const uint8_t* g = a.blocks + off;
+            off = off < last_chunk ? off : last_chunk;
+            const uint8_t* g = seg_blocks + off;
             const uint32_t l = ring_lds + slot * SLOT + i * 1024;
             // the last instruction of a span covers only part of the wavefront: the other lanes are masked
             // off (never all of them, so the instruction is issued and counted every time)
@@ -141,16 +157,29 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_staf_kernel(const StafArgs a)
 #pragma unroll
     for (int m = 0; m < MT; m++) acc[m] = res[m] = 0.0f;
 
+    unsigned long long best = 0ull;  // ARGMAX, per lane: packed (ordered value, ~row); 0 = nothing seen
     auto flush = [&](uint32_t first_local, uint32_t count) {
         const uint32_t row = row0 + first_local + lane;
-        if (lane < count && row < a.n) {
+        if (lane < count && row < seg_n) {
 #pragma unroll
             for (int m = 0; m < MT; m++) {
                 if ((uint32_t)m < a.m) {
-                    const size_t o = (size_t)m * a.y_stride + row;
-                    if (a.y_dtype == MI355Q_F32) ((float*)a.y)[o] = res[m];
-                    else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)a.y)[o] = f32_to_bf16_rne(res[m]);
-                    else ((uint16_t*)a.y)[o] = f32_to_f16_rne(res[m]);
+                    if (seg_y) {
+                        const size_t o = (size_t)m * seg_ys + row;
+                        if (a.y_dtype == MI355Q_F32) ((float*)seg_y)[o] = res[m];
+                        else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)seg_y)[o] = f32_to_bf16_rne(res[m]);
+                        else ((uint16_t*)seg_y)[o] = f32_to_f16_rne(res[m]);
+                    }
+                    if (a.logits && m == 0) a.logits[row] = res[m];
+                }
+            }
+            if constexpr (ARGMAX) {
+                const float v = res[0];
+                if (v > -INFINITY) {                         // NaN and -inf never contribute
+                    const uint32_t u = __float_as_uint(v + 0.0f);   // -0 -> +0
+                    const uint32_t key = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+                    const unsigned long long pk = ((unsigned long long)key << 32) | (unsigned long long)(0xFFFFFFFFu - row);
+                    best = pk > best ? pk : best;
                 }
             }
         }
@@ -254,6 +283,26 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_staf_kernel(const StafArgs a)
         }
     }
     if (lrow & 63u) flush(lrow & ~63u, lrow & 63u);
+    if constexpr (ARGMAX) {
+        // wavefront maximum of the packed keys, workgroup maximum through LDS, one plain store per workgroup;
+        // argmax_finish_kernel picks the token from the partial keys
+        __shared__ unsigned long long s_best[WAVES];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const uint32_t hi = (uint32_t)__shfl_xor((int)(best >> 32), off, 64);
+            const uint32_t lo = (uint32_t)__shfl_xor((int)(best & 0xFFFFFFFFull), off, 64);
+            const unsigned long long o = ((unsigned long long)hi << 32) | lo;
+            best = o > best ? o : best;
+        }
+        if (lane == 0) s_best[wave] = best;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            unsigned long long m = s_best[0];
+#pragma unroll
+            for (int w2 = 1; w2 < WAVES; w2++) m = s_best[w2] > m ? s_best[w2] : m;
+            a.scratch[blockIdx.x] = m;
+        }
+    }
 }
 
 constexpr int kWaves = 4;
@@ -288,16 +337,11 @@ uint32_t staf_rows_per_wave(const mi355q_context* ctx, uint32_t n, const StafCfg
     return rpw ? rpw : 1;
 }
 
+// `total_rows`: rows of all matrices of the launch; `grid`: workgroups (the caller has dealt the wavefronts).
 template <int BITS, int GROUP>
-mi355q_status launch_for_format(hipStream_t s, const mi355q_context* ctx, const StafArgs& args, int mt) {
+mi355q_status launch_for_format(hipStream_t s, const StafArgs& a, int mt, int depth, uint32_t grid, bool argmax) {
     using G = StafGeo<BITS, GROUP>;
-    StafCfg c = staf_cfg();
-    const size_t lds = staf_lds_bytes(G::SLOT, G::Q, args.nsp, mt, c.depth);
-    staf_one_workgroup_per_cu(lds, c);
-    StafArgs a = args;
-    a.rows_per_wave = staf_rows_per_wave(ctx, a.n, c);
-    const uint32_t rows_per_wg = a.rows_per_wave * kWaves;
-    const uint32_t grid = (a.n + rows_per_wg - 1) / rows_per_wg;
+    const size_t lds = staf_lds_bytes(G::SLOT, G::Q, a.nsp, mt, depth);
     auto go = [&](auto kernel) -> mi355q_status {
         if (lds > 48 * 1024)
             MI355Q_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
@@ -305,18 +349,36 @@ mi355q_status launch_for_format(hipStream_t s, const mi355q_context* ctx, const 
         MI355Q_HIP(hipGetLastError());
         return MI355Q_OK;
     };
-    if (c.depth == 2) {
+    if (argmax) return depth == 2 ? go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 2, true>)
+                                  : go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 4, true>);
+    if (depth == 2) {
         switch (mt) {
-        case 1: return go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 2>);
-        case 2: return go(gemv_staf_kernel<BITS, GROUP, 2, kWaves, 2>);
-        default: return go(gemv_staf_kernel<BITS, GROUP, 4, kWaves, 2>);
+        case 1: return go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 2, false>);
+        case 2: return go(gemv_staf_kernel<BITS, GROUP, 2, kWaves, 2, false>);
+        default: return go(gemv_staf_kernel<BITS, GROUP, 4, kWaves, 2, false>);
         }
     }
     switch (mt) {
-    case 1: return go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 4>);
-    case 2: return go(gemv_staf_kernel<BITS, GROUP, 2, kWaves, 4>);
-    default: return go(gemv_staf_kernel<BITS, GROUP, 4, kWaves, 4>);
+    case 1: return go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 4, false>);
+    case 2: return go(gemv_staf_kernel<BITS, GROUP, 2, kWaves, 4, false>);
+    default: return go(gemv_staf_kernel<BITS, GROUP, 4, kWaves, 4, false>);
     }
+}
+
+mi355q_status launch_by_format(hipStream_t s, uint32_t bits, uint32_t group, const StafArgs& a, int mt, int depth,
+                               uint32_t grid, bool argmax) {
+    switch (bits * 1000 + group) {
+    case 4064: return launch_for_format<4, 64>(s, a, mt, depth, grid, argmax);
+    case 4128: return launch_for_format<4, 128>(s, a, mt, depth, grid, argmax);
+    case 8032: return launch_for_format<8, 32>(s, a, mt, depth, grid, argmax);
+    case 8064: return launch_for_format<8, 64>(s, a, mt, depth, grid, argmax);
+    case 2064: return launch_for_format<2, 64>(s, a, mt, depth, grid, argmax);
+    case 3064: return launch_for_format<3, 64>(s, a, mt, depth, grid, argmax);
+    case 5064: return launch_for_format<5, 64>(s, a, mt, depth, grid, argmax);
+    case 6064: return launch_for_format<6, 64>(s, a, mt, depth, grid, argmax);
+    default: break;
+    }
+    return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no block-layout GEMV for q%ug%u", bits, group);
 }
 
 struct StafShape { uint32_t slot, q; };
@@ -371,44 +433,70 @@ GemvLaunchShape gemv_staf_shape(const mi355q_context* ctx, const WView& w, uint3
     return g;
 }
 
-mi355q_status launch_gemv_staf(hipStream_t s, const mi355q_context* ctx, const WView& w, const void* x, void* y,
-                               int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride) {
+// Up to three weights sharing K, format and activations in one launch; `w[0]` supplies the format, the caller has
+// checked that the others match.  `token_out` selects the fused arg-max tail (one weight, M == 1).
+mi355q_status launch_gemv_staf_multi(hipStream_t s, const mi355q_context* ctx, uint32_t count, const WView* w,
+                                     const void* x, void* const* y, const uint32_t* y_strides, int y_dtype,
+                                     uint32_t m, uint32_t x_stride, float* logits_f32, int32_t* token_out,
+                                     unsigned long long* argmax_scratch) {
+    if (count < 1 || count > (uint32_t)kGemvMaxSegments)
+        return fail(MI355Q_ERR_INVALID_ARGUMENT, "1..%d weights per fused launch", kGemvMaxSegments);
+    if ((uintptr_t)x % 16) return fail(MI355Q_ERR_INVALID_ARGUMENT, "activation pointer must be 16-byte aligned");
+    const bool argmax = token_out != nullptr;
+    if (argmax && (m != 1 || count != 1)) return fail(MI355Q_ERR_INVALID_ARGUMENT, "fused argmax needs M == 1");
+    if (logits_f32 && count != 1) return fail(MI355Q_ERR_INVALID_ARGUMENT, "fp32 logits need a single weight");
     StafShape sh;
-    if (!staf_shape(w.bits, w.group, sh)) return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no block-layout GEMV for q%ug%u", w.bits, w.group);
-    const int fit = staf_max_mt(w, sh);
-    if (fit == 0) return fail(MI355Q_ERR_SHAPE, "K = %u is too long for the block-layout GEMV", w.k);
-    const size_t xsz = 2, ysz = y_dtype == MI355Q_F32 ? 4 : 2;
+    if (!staf_shape(w[0].bits, w[0].group, sh))
+        return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no block-layout GEMV for q%ug%u", w[0].bits, w[0].group);
+    const int fit = staf_max_mt(w[0], sh);
+    if (fit == 0) return fail(MI355Q_ERR_SHAPE, "K = %u is too long for the block-layout GEMV", w[0].k);
+    uint64_t total = 0;
+    for (uint32_t i = 0; i < count; i++) total += w[i].n;
+    if (total > 0xFFFFFFFFull) return fail(MI355Q_ERR_SHAPE, "too many rows");
+    const size_t ysz = y_dtype == MI355Q_F32 ? 4 : 2;
     StafArgs a{};
-    a.blocks = w.blocks;
-    a.row_bytes = (uint64_t)w.blocks_per_row * w.bytes_per_block;
-    a.last_chunk = (uint64_t)w.n * a.row_bytes - 16;
-    a.k = w.k;
-    a.n = w.n;
+    a.row_bytes = (uint64_t)w[0].blocks_per_row * w[0].bytes_per_block;
+    a.k = w[0].k;
     a.x_stride = x_stride;
-    a.y_stride = y_stride;
     a.y_dtype = (uint32_t)y_dtype;
-    a.blocks_per_row = w.blocks_per_row;
-    a.nsp = (w.blocks_per_row + 63) / 64;
+    a.blocks_per_row = w[0].blocks_per_row;
+    a.nsp = (w[0].blocks_per_row + 63) / 64;
+    a.logits = logits_f32;
+    a.scratch = argmax_scratch;
     for (uint32_t m0 = 0; m0 < m;) {
         const uint32_t left = m - m0;
-        int mt = left >= 4 ? 4 : left >= 2 ? 2 : 1;          // 3 rows run as a 4-row launch with one row masked
-        if (left == 3) mt = 4;
+        int mt = left >= 3 ? 4 : (int)left;                  // 3 rows run as a 4-row launch with one row masked
         if (mt > fit) mt = fit;
         const uint32_t mm = left < (uint32_t)mt ? left : (uint32_t)mt;
-        a.x = (const uint16_t*)((const char*)x + (size_t)m0 * x_stride * xsz);
-        a.y = (char*)y + (size_t)m0 * y_stride * ysz;
+        StafCfg c = staf_cfg();
+        staf_one_workgroup_per_cu(staf_lds_bytes(sh.slot, sh.q, a.nsp, mt, c.depth), c);
+        a.rows_per_wave = staf_rows_per_wave(ctx, (uint32_t)total, c);
+        uint32_t waves = 0;
+        for (uint32_t i = 0; i < (uint32_t)kGemvMaxSegments; i++) {
+            const uint32_t j = i < count ? i : count - 1;
+            if (i < count) waves += (w[i].n + a.rows_per_wave - 1) / a.rows_per_wave;
+            a.blocks[i] = w[j].blocks;
+            a.y[i] = y[j] ? (void*)((char*)y[j] + (size_t)m0 * y_strides[j] * ysz) : nullptr;
+            a.y_stride[i] = y_strides[j];
+            a.seg_rows[i] = w[j].n;
+            a.wave_end[i] = waves;
+        }
+        const uint32_t grid = (waves + kWaves - 1) / kWaves;
+        if (argmax && grid > kArgmaxPartialCapacity) return fail(MI355Q_ERR_SHAPE, "too many workgroups for the fused argmax");
+        a.x = (const uint16_t*)x + (size_t)m0 * x_stride;
         a.m = mm;
-        mi355q_status st;
-#define MI355Q_STAF_LAUNCH(B, GR) \
-        if (w.bits == B && w.group == GR) st = launch_for_format<B, GR>(s, ctx, a, mt); else
-        MI355Q_STAF_LAUNCH(4, 64) MI355Q_STAF_LAUNCH(4, 128) MI355Q_STAF_LAUNCH(8, 32) MI355Q_STAF_LAUNCH(8, 64)
-        MI355Q_STAF_LAUNCH(2, 64) MI355Q_STAF_LAUNCH(3, 64) MI355Q_STAF_LAUNCH(5, 64) MI355Q_STAF_LAUNCH(6, 64)
-        st = MI355Q_ERR_KERNEL_NOT_FOUND;
-#undef MI355Q_STAF_LAUNCH
-        if (st != MI355Q_OK) return st;
+        if (mi355q_status st = launch_by_format(s, w[0].bits, w[0].group, a, mt, c.depth, grid, argmax)) return st;
+        if (argmax) return launch_argmax_finish(s, argmax_scratch, grid, token_out);
         m0 += mm;
     }
     return MI355Q_OK;
+}
+
+mi355q_status launch_gemv_staf(hipStream_t s, const mi355q_context* ctx, const WView& w, const void* x, void* y,
+                               int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride) {
+    void* ys[1] = {y};
+    const uint32_t strides[1] = {y_stride};
+    return launch_gemv_staf_multi(s, ctx, 1, &w, x, ys, strides, y_dtype, m, x_stride, nullptr, nullptr, nullptr);
 }
 
 }  // namespace mi355q

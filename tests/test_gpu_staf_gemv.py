@@ -113,3 +113,81 @@ def test_in_place_gemv_strided_rows(pkg, ctx):
     got = run_gemv(ctx, pkg, w, x, pkg.BF16, pkg.F32)
     assert_within_tolerance(got, oracle.gemm_f64(wq, x[:, :k]), "strided rows")
     w.destroy()
+
+
+def _run_batched(pkg, ctx, ws, ns, x, y_dtype):
+    from gpu_util import out_from_device
+    m = x.shape[0]
+    xd = ctx.upload(oracle.bf16_from_f32(x).reshape(x.shape))
+    esz = 4 if y_dtype == pkg.F32 else 2
+    yds = [ctx.alloc(m * n * esz) for n in ns]
+    for yd in yds:
+        ctx.fill(yd, 0x7FC00000 if y_dtype == pkg.F32 else 0x7FC07FC0)
+    ctx.batched_qgemm(ws, xd, pkg.BF16, yds, y_dtype, m)
+    ctx.synchronize()
+    out = [out_from_device(yd, y_dtype, (m, n), pkg) for yd, n in zip(yds, ns)]
+    xd.free()
+    for yd in yds:
+        yd.free()
+    return out
+
+
+@pytest.mark.parametrize("ns,k,bits,group", [((4096, 1024, 1024), 4096, 4, 64), ((14336, 14336), 4096, 4, 64),
+                                             ((5, 1, 3), 256, 4, 64), ((130, 67), 4096 + 256, 4, 64),
+                                             ((257, 63, 129), 1024, 8, 32), ((70, 200), 1024, 3, 64)])
+def test_in_place_batched_projections(pkg, ctx, ns, k, bits, group):
+    """q+k+v and gate+up left in STAF blocks as one launch each: wavefronts are dealt to the matrices whole, so
+    segment boundaries fall inside workgroups; every output against the per-projection oracle."""
+    cases = [_case(3500 + i + len(ns) * 10 + bits, n, k, bits, group) for i, n in enumerate(ns)]
+    ws = [c.device_weight(ctx, pkg, pkg.LAYOUT_STAF_BLOCKS) for c in cases]
+    wqs = [oracle.dequant_staf_f32(bits, group, c.n, k, c.staf_blocks()) for c in cases]
+    for m in (1, 3, 8):
+        x = act_rounded(kat.seeded_activations(3600 + m, m, k), pkg.BF16, pkg)
+        say(f"in-place batched {ns} K={k} q{bits}g{group} M={m}")
+        got = _run_batched(pkg, ctx, ws, ns, x, pkg.F32)
+        gbf = _run_batched(pkg, ctx, ws, ns, x, pkg.BF16)
+        for i in range(len(ns)):
+            assert_within_tolerance(got[i], oracle.gemm_f64(wqs[i], x), f"{ns} projection {i} M={m}")
+            assert np.array_equal(oracle.bf16_from_f32(gbf[i]), oracle.bf16_from_f32(got[i]))
+    for w in ws:
+        w.destroy()
+
+
+@pytest.mark.parametrize("n,k", [(65536, 2048), (1000, 4096), (37, 256)])
+def test_in_place_output_head(pkg, ctx, n, k):
+    """LM head over STAF blocks with the fused arg-max tail: fp32 logits within tolerance, the token is the
+    lowest-index maximum of the device's own logits, twice in a row (the partial keys need no reset), with and
+    without a logits buffer."""
+    case = _case(3700 + n % 89, n, k, 4, 64)
+    w = case.device_weight(ctx, pkg, pkg.LAYOUT_STAF_BLOCKS)
+    wq = oracle.dequant_staf_f32(4, 64, n, k, case.staf_blocks())
+    x = act_rounded(kat.seeded_activations(3701, 1, k), pkg.BF16, pkg)
+    want = oracle.gemm_f64(wq, x)[0]
+    xd = ctx.upload(oracle.bf16_from_f32(x))
+    logits = ctx.alloc(n * 4)
+    tok = ctx.upload(np.array([-7], np.int32))
+    for _ in range(2):
+        ctx.fill(logits, 0x7FC00000)
+        tok.upload(np.array([-7], np.int32))
+        ctx.lmhead_argmax(w, xd, pkg.BF16, logits, tok)
+        ctx.synchronize()
+        got = logits.download(np.float32)
+        assert_within_tolerance(got, want, "in-place head logits")
+        token = int(tok.download(np.int32)[0])
+        assert token == oracle.argmax_lowest(got)
+    tok.upload(np.array([-7], np.int32))
+    ctx.lmhead_argmax(w, xd, pkg.BF16, None, tok)
+    ctx.synchronize()
+    assert int(tok.download(np.int32)[0]) == token
+    # ties: identical rows give identical logits; the lowest row wins
+    dup = _case(3710, 512, 1024, 4, 64)
+    dup.codes[17] = 15; dup.scales[17] = 0.02; dup.zeros[17] = 0.0
+    dup.codes[300] = 15; dup.scales[300] = 0.02; dup.zeros[300] = 0.0
+    wd = dup.device_weight(ctx, pkg, pkg.LAYOUT_STAF_BLOCKS)
+    ones = ctx.upload(oracle.bf16_from_f32(np.ones((1, 1024), np.float32)))
+    ctx.lmhead_argmax(wd, ones, pkg.BF16, None, tok)
+    ctx.synchronize()
+    assert int(tok.download(np.int32)[0]) == 17
+    for b in (xd, logits, tok, ones):
+        b.free()
+    w.destroy(); wd.destroy()
