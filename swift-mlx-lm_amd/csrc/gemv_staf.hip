@@ -59,8 +59,11 @@ struct StafGeo {
     static constexpr int Q = GROUP / 8;                     // staged activation pieces (8 elements each) per block
 };
 
-template <int BITS, int GROUP, int MT, int WAVES, int D, bool ARGMAX>
+// XREG: rows are one span long (K <= 64 * GROUP) and M == 1: every lane keeps its block's activations and their sum
+// in registers instead of re-reading them from LDS at every row.
+template <int BITS, int GROUP, int MT, int WAVES, int D, bool ARGMAX, bool XREG>
 __global__ __launch_bounds__(WAVES * 64) void gemv_staf_kernel(const StafArgs a) {
+    static_assert(!XREG || MT == 1, "register-resident activations are for M == 1");
     using G = StafGeo<BITS, GROUP>;
     constexpr int WPB = G::WPB, BW = G::BW, SPAN = G::SPAN, NDMA = G::NDMA, SLOT = G::SLOT, Q = G::Q;
     constexpr bool DOT2 = BITS <= 6;                        // 128 + q is exact in bf16
@@ -148,6 +151,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_staf_kernel(const StafArgs a)
     }
     __syncthreads();
 
+    u32x4 xr[XREG ? Q : 1];
+    float sxr = 0.0f;
+    if constexpr (XREG) {
+#pragma unroll
+        for (int p = 0; p < Q; p++) xr[p] = xs[(size_t)p * 64 + lane];
+        sxr = sxs[lane];
+    }
+
     uint32_t k_magic = 0x43004300u;                          // bf16 pair (128.0, 128.0)
     uint32_t k_mask = BITS == 4 ? 0x000F000Fu : 0x00030003u;
     asm volatile("" : "+v"(k_magic));
@@ -209,8 +220,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_staf_kernel(const StafArgs a)
         static_for<Q>([&](auto P) {
             constexpr int p = decltype(P)::value;
             u32x4 xv[MT];
+            if constexpr (XREG) {
+                xv[0] = xr[p];
+            } else {
 #pragma unroll
-            for (int m = 0; m < MT; m++) xv[m] = xs[((size_t)(m * NSP + sp) * Q + p) * 64 + lane];
+                for (int m = 0; m < MT; m++) xv[m] = xs[((size_t)(m * NSP + sp) * Q + p) * 64 + lane];
+            }
             if constexpr (DOT2) {
                 uint32_t pr[4];
                 if constexpr (BITS == 4) {
@@ -264,7 +279,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_staf_kernel(const StafArgs a)
         const float s = f16_to_f32((uint16_t)(hdr & 0xFFFFu)), z = f16_to_f32((uint16_t)(hdr >> 16));
         const float zc = DOT2 ? z - 128.0f * s : z;
 #pragma unroll
-        for (int m = 0; m < MT; m++) acc[m] += s * dot[m] + zc * sxs[(size_t)(m * NSP + sp) * 64 + lane];
+        for (int m = 0; m < MT; m++) acc[m] += s * dot[m] + zc * (XREG ? sxr : sxs[(size_t)(m * NSP + sp) * 64 + lane]);
 
         // the slot's LDS reads have been consumed by the arithmetic above: it can be overwritten
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -342,6 +357,7 @@ template <int BITS, int GROUP>
 mi355q_status launch_for_format(hipStream_t s, const StafArgs& a, int mt, int depth, uint32_t grid, bool argmax) {
     using G = StafGeo<BITS, GROUP>;
     const size_t lds = staf_lds_bytes(G::SLOT, G::Q, a.nsp, mt, depth);
+    const bool xreg = mt == 1 && a.nsp == 1 && env_int_cached("MI355Q_STAF_XREG", 1) != 0;
     auto go = [&](auto kernel) -> mi355q_status {
         if (lds > 48 * 1024)
             MI355Q_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
@@ -349,20 +365,27 @@ mi355q_status launch_for_format(hipStream_t s, const StafArgs& a, int mt, int de
         MI355Q_HIP(hipGetLastError());
         return MI355Q_OK;
     };
-    if (argmax) return depth == 2 ? go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 2, true>)
-                                  : go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 4, true>);
     if (depth == 2) {
+        if (argmax) return xreg ? go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 2, true, true>)
+                                : go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 2, true, false>);
         switch (mt) {
-        case 1: return go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 2, false>);
-        case 2: return go(gemv_staf_kernel<BITS, GROUP, 2, kWaves, 2, false>);
-        default: return go(gemv_staf_kernel<BITS, GROUP, 4, kWaves, 2, false>);
+        case 1: return xreg ? go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 2, false, true>)
+                            : go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 2, false, false>);
+        case 2: return go(gemv_staf_kernel<BITS, GROUP, 2, kWaves, 2, false, false>);
+        default: return go(gemv_staf_kernel<BITS, GROUP, 4, kWaves, 2, false, false>);
         }
     }
+#ifdef MI355Q_GEMV_EXPERIMENT
+    // tuning builds: the deeper ring, selected with MI355Q_STAF_DEPTH
+    if (argmax) return go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 4, true, false>);
     switch (mt) {
-    case 1: return go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 4, false>);
-    case 2: return go(gemv_staf_kernel<BITS, GROUP, 2, kWaves, 4, false>);
-    default: return go(gemv_staf_kernel<BITS, GROUP, 4, kWaves, 4, false>);
+    case 1: return go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 4, false, false>);
+    case 2: return go(gemv_staf_kernel<BITS, GROUP, 2, kWaves, 4, false, false>);
+    default: return go(gemv_staf_kernel<BITS, GROUP, 4, kWaves, 4, false, false>);
     }
+#else
+    return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no block-layout GEMV with ring depth %d", depth);
+#endif
 }
 
 mi355q_status launch_by_format(hipStream_t s, uint32_t bits, uint32_t group, const StafArgs& a, int mt, int depth,
