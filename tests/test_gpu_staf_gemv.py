@@ -191,3 +191,42 @@ def test_in_place_output_head(pkg, ctx, n, k):
     for b in (xd, logits, tok, ones):
         b.free()
     w.destroy(); wd.destroy()
+
+
+def test_in_place_plan_replay_and_graph(pkg, ctx):
+    """A plan over STAF-layout weights (one fused q+k+v-style launch and the fused head) replayed from C and as a
+    HIP graph, with fills and uploads between the replays: every replay equals the eager launches bit for bit (the
+    direct-to-LDS loads, the partial keys of the head and its finishing launch carry no state between launches)."""
+    k = 1024
+    ns = (512, 256, 2048)
+    cases = [_case(3800 + i, n, k, 4, 64) for i, n in enumerate(ns)]
+    ws = [c.device_weight(ctx, pkg, pkg.LAYOUT_STAF_BLOCKS) for c in cases]
+    x = ctx.upload(oracle.bf16_from_f32(kat.seeded_activations(3810, 1, k)))
+    ys = [ctx.alloc(n * 4) for n in ns]
+    tok = ctx.upload(np.array([-3], np.int32))
+    ctx.batched_qgemm(ws[:2], x, pkg.BF16, ys[:2], pkg.F32, 1)
+    ctx.lmhead_argmax(ws[2], x, pkg.BF16, ys[2], tok)
+    ctx.synchronize()
+    eager = [y.download(np.float32) for y in ys]
+    etok = int(tok.download(np.int32)[0])
+    assert etok == oracle.argmax_lowest(eager[2])
+    plan = pkg.DispatchPlan(ctx)
+    plan.add_batched_linear(ws[:2], x, pkg.BF16, ys[:2], pkg.F32, 1)
+    plan.add_output_head(ws[2], x, pkg.BF16, ys[2], tok)
+    assert plan.step(0)[0].device_kernel == "gemv_staf_q4_g64"
+    stream = ctx.stream_create()
+    plan.graph_build(stream)
+    for rep in range(4):
+        for y in ys:
+            ctx.fill(y, 0x7FC00000, stream)
+        tok.upload(np.array([-3], np.int32))
+        plan.graph_launch(stream) if rep else plan.encode(stream)
+        ctx.synchronize(stream)
+        for y, want in zip(ys, eager):
+            assert np.array_equal(y.download(np.float32), want), rep
+        assert int(tok.download(np.int32)[0]) == etok
+    plan.destroy()
+    for b in ys + [x, tok]:
+        b.free()
+    for w in ws:
+        w.destroy()
