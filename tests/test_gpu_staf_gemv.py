@@ -41,6 +41,24 @@ def _row_alignment_k(bits, group):
     return blocks * group
 
 
+def _q4_blocks(case):
+    """STAF q4 blocks [N, row bytes] of a Case, vectorised (kat.staf_blocks walks every block in Python)."""
+    n, k, g = case.n, case.k, case.group
+    codes = case.codes.reshape(n, k // g, g // 2, 2)
+    packed = (codes[..., 0] | (codes[..., 1] << 4)).astype(np.uint8)                 # LSB-first: even code in the low nibble
+    hdr = np.stack([case.scales.astype(np.float16).view(np.uint16), case.zeros.astype(np.float16).view(np.uint16)], -1)
+    hdr = np.ascontiguousarray(hdr.astype("<u2")).view(np.uint8).reshape(n, k // g, 4)
+    return np.ascontiguousarray(np.concatenate([hdr, packed], axis=2).reshape(n, -1))
+
+
+def _device_and_reference(pkg, ctx, case):
+    """(STAF-layout device weight, dequantised fp32 reference weights); 4-bit cases use the vectorised block builder."""
+    blocks = _q4_blocks(case).reshape(-1) if case.bits == 4 else case.staf_blocks()
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(case.bits, case.group)
+    w = ctx.weight_prepare_staf(fmt, case.n, case.k, blocks, pkg.LAYOUT_STAF_BLOCKS)
+    return w, oracle.dequant_staf_f32(case.bits, case.group, case.n, case.k, blocks)
+
+
 @pytest.mark.parametrize("bits,group", FORMATS)
 def test_in_place_gemv_formats_and_tails(pkg, ctx, bits, group):
     """Rows shorter than one span of 64 blocks, exactly one span, one span plus a tail, several spans;
@@ -86,8 +104,7 @@ def test_in_place_gemv_llama_shapes(pkg, ctx, n, k):
     """Llama-3-8B projection shapes at q4 g64, all output types, against the oracle and against the
     per-code kernel on the same device buffers."""
     case = _case(3300 + n % 97, n, k, 4, 64)
-    w = case.device_weight(ctx, pkg, pkg.LAYOUT_STAF_BLOCKS)
-    wq = oracle.dequant_staf_f32(4, 64, n, k, case.staf_blocks())
+    w, wq = _device_and_reference(pkg, ctx, case)
     for m in (1, 4):
         x = act_rounded(kat.seeded_activations(3310 + m, m, k), pkg.BF16, pkg)
         say(f"in-place llama N={n} K={k} M={m}")
@@ -139,8 +156,8 @@ def test_in_place_batched_projections(pkg, ctx, ns, k, bits, group):
     """q+k+v and gate+up left in STAF blocks as one launch each: wavefronts are dealt to the matrices whole, so
     segment boundaries fall inside workgroups; every output against the per-projection oracle."""
     cases = [_case(3500 + i + len(ns) * 10 + bits, n, k, bits, group) for i, n in enumerate(ns)]
-    ws = [c.device_weight(ctx, pkg, pkg.LAYOUT_STAF_BLOCKS) for c in cases]
-    wqs = [oracle.dequant_staf_f32(bits, group, c.n, k, c.staf_blocks()) for c in cases]
+    pairs = [_device_and_reference(pkg, ctx, c) for c in cases]
+    ws, wqs = [p[0] for p in pairs], [p[1] for p in pairs]
     for m in (1, 3, 8):
         x = act_rounded(kat.seeded_activations(3600 + m, m, k), pkg.BF16, pkg)
         say(f"in-place batched {ns} K={k} q{bits}g{group} M={m}")
@@ -159,8 +176,7 @@ def test_in_place_output_head(pkg, ctx, n, k):
     lowest-index maximum of the device's own logits, twice in a row (the partial keys need no reset), with and
     without a logits buffer."""
     case = _case(3700 + n % 89, n, k, 4, 64)
-    w = case.device_weight(ctx, pkg, pkg.LAYOUT_STAF_BLOCKS)
-    wq = oracle.dequant_staf_f32(4, 64, n, k, case.staf_blocks())
+    w, wq = _device_and_reference(pkg, ctx, case)
     x = act_rounded(kat.seeded_activations(3701, 1, k), pkg.BF16, pkg)
     want = oracle.gemm_f64(wq, x)[0]
     xd = ctx.upload(oracle.bf16_from_f32(x))
@@ -230,3 +246,31 @@ def test_in_place_plan_replay_and_graph(pkg, ctx):
         b.free()
     for w in ws:
         w.destroy()
+
+
+def test_in_place_gemv_full_size_properties(pkg, ctx):
+    """Size-independent properties at the full gate shape (14336 x 4096, q4 g64), where the oracle is too slow to
+    be the checker for every element: scaling the activations by a power of two scales every output by the same
+    factor bit for bit, and permuting the weight rows permutes the outputs bit for bit (a row's result does not
+    depend on which wavefront, span slot or workgroup computes it)."""
+    n, k = 14336, 4096
+    case = _case(3900, n, k, 4, 64)
+    small = _case(3899, 3, 256, 4, 64)
+    assert np.array_equal(_q4_blocks(small).reshape(-1), small.staf_blocks())       # the fast builder below
+    blocks = _q4_blocks(case)
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+    w = ctx.weight_prepare_staf(fmt, n, k, blocks.reshape(-1), pkg.LAYOUT_STAF_BLOCKS)
+    x = act_rounded(kat.seeded_activations(3901, 1, k), pkg.BF16, pkg)
+    y = run_gemv(ctx, pkg, w, x, pkg.BF16, pkg.F32)
+    assert np.all(np.isfinite(y))
+    y4 = run_gemv(ctx, pkg, w, 4.0 * x, pkg.BF16, pkg.F32)
+    assert np.array_equal(y4, 4.0 * y)
+    perm = np.random.default_rng(3902).permutation(n)
+    wp = ctx.weight_prepare_staf(fmt, n, k, np.ascontiguousarray(blocks[perm]).reshape(-1), pkg.LAYOUT_STAF_BLOCKS)
+    yp = run_gemv(ctx, pkg, wp, x, pkg.BF16, pkg.F32)
+    assert np.array_equal(yp[0], y[0][perm])
+    # and a sample of rows against the oracle
+    rows = np.random.default_rng(3903).choice(n, 64, replace=False)
+    wq = oracle.dequant_staf_f32(4, 64, 64, k, np.ascontiguousarray(blocks[rows]).reshape(-1))
+    assert_within_tolerance(y[0][rows], oracle.gemm_f64(wq, x)[0], "sampled rows")
+    w.destroy(); wp.destroy()
