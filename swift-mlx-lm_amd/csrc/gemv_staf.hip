@@ -46,7 +46,8 @@ struct StafArgs {
     uint32_t x_stride, y_dtype;
     uint32_t blocks_per_row;
     uint32_t nsp;            // spans per row = ceil(blocks_per_row / 64)
-    uint32_t rows_per_wave;
+    uint32_t rows_per_span;  // 64 / blocks_per_row when a row is a power-of-two fraction of a span (then nsp == 1), else 1
+    uint32_t rows_per_wave;  // a multiple of rows_per_span
 };
 
 template <int BITS, int GROUP>
@@ -90,7 +91,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_staf_kernel(const StafArgs a)
     const uint32_t seg_ys = seg == 0 ? a.y_stride[0] : (seg == 1 ? a.y_stride[1] : a.y_stride[2]);
     const uint64_t last_chunk = (uint64_t)seg_n * a.row_bytes - 16;    // last whole 16-byte chunk of the matrix
     const uint32_t row0 = gw < a.wave_end[kGemvMaxSegments - 1] ? (gw - first_wave) * a.rows_per_wave : seg_n;
-    const uint32_t nsteps = a.rows_per_wave * NSP;
+    // Short rows share a span: RPS consecutive rows (contiguous in memory) fill the 64 lanes, lane l holding block
+    // l % blocks_per_row of row l / blocks_per_row.
+    const uint32_t RPS = a.rows_per_span;
+    const uint32_t nsteps = a.rows_per_wave / RPS * NSP;
 
     // ---- 1. the first D spans go out before anything else ----------------------------------------
     uint32_t irow = 0, isp = 0;                              // next span to issue
@@ -109,7 +113,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_staf_kernel(const StafArgs a)
             if ((i + 1) * 1024 <= SPAN || lane < (uint32_t)(SPAN - i * 1024) / 16)
                 asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(l) : "memory");
         }
-        if (++isp == NSP) { isp = 0; irow++; }
+        if (++isp == NSP) { isp = 0; irow += RPS; }
     };
 #pragma unroll
     for (int j = 0; j < D; j++)
@@ -119,7 +123,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_staf_kernel(const StafArgs a)
     const uint32_t ntasks = a.m * NSP;
     for (uint32_t t = wave; t < ntasks; t += WAVES) {
         const uint32_t m = t / NSP, sp = t - m * NSP;
-        const uint32_t b = sp * 64 + lane;
+        const uint32_t b = RPS > 1 ? lane % a.blocks_per_row : sp * 64 + lane;
         const bool valid = b < a.blocks_per_row;
         const u32x4* src = (const u32x4*)(a.x + (size_t)m * a.x_stride + (valid ? (size_t)b * GROUP : 0));
         uint32_t d[GROUP / 2];
@@ -207,7 +211,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_staf_kernel(const StafArgs a)
             if (younger == (uint32_t)y) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA * y) : "memory");
         });
         const uint32_t* blk = (const uint32_t*)(ring + (size_t)slot * SLOT) + lane * BW;
-        const bool valid = sp * 64 + lane < a.blocks_per_row;
+        const bool valid = RPS > 1 || sp * 64 + lane < a.blocks_per_row;
         uint32_t hdr = blk[0];
         uint32_t w[WPB];
 #pragma unroll
@@ -289,11 +293,21 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_staf_kernel(const StafArgs a)
             sp = 0;
 #pragma unroll
             for (int m = 0; m < MT; m++) {
-                const float total = wave_reduce_sum(acc[m]);
-                if (lane == (lrow & 63u)) res[m] = total;
+                float total;
+                if (RPS == 1) {
+                    total = wave_reduce_sum(acc[m]);
+                    if (lane == (lrow & 63u)) res[m] = total;
+                } else {
+                    // sum inside each run of blocks_per_row lanes, then hand the RPS row totals to their parking lanes
+                    total = acc[m];
+                    for (uint32_t off = a.blocks_per_row >> 1; off > 0; off >>= 1) total += __shfl_xor(total, (int)off, 64);
+                    const uint32_t park = (lane - lrow) & 63u;             // which row of this span parks here, if any
+                    const float moved = __shfl(total, (int)((park & (RPS - 1)) * a.blocks_per_row), 64);
+                    if (park < RPS) res[m] = moved;
+                }
                 acc[m] = 0.0f;
             }
-            lrow++;
+            lrow += RPS;
             if ((lrow & 63u) == 0) flush(lrow - 64, 64);
         }
     }
@@ -343,6 +357,12 @@ size_t staf_lds_bytes(uint32_t span_slot, uint32_t q, uint32_t nsp, int mt, int 
 // CU's whole share of rows (every extra workgroup would stage the activations again).
 void staf_one_workgroup_per_cu(size_t lds, StafCfg& c) {
     if (lds > 80 * 1024 && env_int_cached("MI355Q_STAF_WAVES_PER_CU", 0) == 0) c.per_cu = kWaves;
+}
+
+// Rows that are a power-of-two fraction of a span (32, 16, 8 ... blocks) share one.
+uint32_t staf_rows_per_span(uint32_t blocks_per_row) {
+    if (blocks_per_row >= 64 || (blocks_per_row & (blocks_per_row - 1)) != 0) return 1;
+    return 64 / blocks_per_row;
 }
 
 // Each wavefront owns a run of consecutive rows.
@@ -448,7 +468,8 @@ GemvLaunchShape gemv_staf_shape(const mi355q_context* ctx, const WView& w, uint3
     StafCfg c = staf_cfg();
     g.lds_bytes = (uint32_t)staf_lds_bytes(sh.slot, sh.q, (w.blocks_per_row + 63) / 64, mt ? mt : 1, c.depth);
     staf_one_workgroup_per_cu(g.lds_bytes, c);
-    const uint32_t rows_per_wg = staf_rows_per_wave(ctx, w.n, c) * kWaves;
+    const uint32_t rps = staf_rows_per_span(w.blocks_per_row);
+    const uint32_t rows_per_wg = (staf_rows_per_wave(ctx, w.n, c) + rps - 1) / rps * rps * kWaves;
     g.grid = (w.n + rows_per_wg - 1) / rows_per_wg;
     g.block = kWaves * 64;
     g.rows_per_workgroup = rows_per_wg;
@@ -484,6 +505,7 @@ mi355q_status launch_gemv_staf_multi(hipStream_t s, const mi355q_context* ctx, u
     a.y_dtype = (uint32_t)y_dtype;
     a.blocks_per_row = w[0].blocks_per_row;
     a.nsp = (w[0].blocks_per_row + 63) / 64;
+    a.rows_per_span = staf_rows_per_span(w[0].blocks_per_row);
     a.logits = logits_f32;
     a.scratch = argmax_scratch;
     for (uint32_t m0 = 0; m0 < m;) {
@@ -494,6 +516,7 @@ mi355q_status launch_gemv_staf_multi(hipStream_t s, const mi355q_context* ctx, u
         StafCfg c = staf_cfg();
         staf_one_workgroup_per_cu(staf_lds_bytes(sh.slot, sh.q, a.nsp, mt, c.depth), c);
         a.rows_per_wave = staf_rows_per_wave(ctx, (uint32_t)total, c);
+        a.rows_per_wave = (a.rows_per_wave + a.rows_per_span - 1) / a.rows_per_span * a.rows_per_span;
         uint32_t waves = 0;
         for (uint32_t i = 0; i < (uint32_t)kGemvMaxSegments; i++) {
             const uint32_t j = i < count ? i : count - 1;
