@@ -374,6 +374,61 @@ def main():
                 w.destroy()
         layers = saved
 
+    # ---- secondary: the rows either side of the projections (embedding gather, container load, KV cache), one
+    # figure each; HBM-bound byte movers, bytes = what the launch must read plus what it must write
+    next_rows = None
+    if not a.no_other_configs:
+        import tempfile
+        next_rows = {}
+        rng = np.random.default_rng(11)
+        table = layers[0]["gate"]                              # 14336 x 4096 q4 g64 as a vocabulary table
+        seq = 2048
+        ids = ctx.upload(rng.integers(0, 14336, seq).astype(np.int32))
+        emb = ctx.alloc(seq * 4096 * 2)
+        ctx.embedding_lookup(table, ids, seq, emb, pkg.BF16, 0, None, stream)
+        ctx.synchronize(stream)
+        ms = time_region(ctx, lambda i: ctx.embedding_lookup(table, ids, seq, emb, pkg.BF16, 0, None, stream), 20, stream)
+        moved = seq * (4096 // 64) * 36 + seq * 4096 * 2
+        next_rows["embedding gather 2048 tokens x 4096, q4 g64 -> bf16"] = {
+            "us": round(ms * 1e3, 2), "GBps": round(moved / (ms * 1e-3) / 1e9, 1), "bytes": moved}
+        ids.free(); emb.free()
+        spec = pkg.KVCacheSpecification(0x10, pkg.KV_SEQUENCE_MAJOR, 8, 128, 4096)
+        cache = ctx.alloc(spec.bytes_per_layer)
+        rows = ctx.upload(oracle.bf16_from_f32(rng.standard_normal((seq, 1024)).astype(np.float32)))
+        back = ctx.alloc(seq * 1024 * 2)
+        for label, fn, count in (("KV cache write q8 g32, 2048 positions x 8 heads x 128", lambda i: ctx.kv_cache_write(spec, cache, rows, pkg.BF16, 0, seq, 0, stream), seq),
+                                 ("KV cache read q8 g32, 2048 positions x 8 heads x 128", lambda i: ctx.kv_cache_read(spec, cache, back, pkg.BF16, 0, seq, 0, stream), seq),
+                                 ("KV cache append q8 g32, 1 position", lambda i: ctx.kv_cache_write(spec, cache, rows, pkg.BF16, seq, 1, 0, stream), 1)):
+            fn(0)
+            ctx.synchronize(stream)
+            ms = time_region(ctx, fn, 20, stream)
+            moved = count * 1024 * 2 + count * 8 * (128 // 32) * 36
+            next_rows[label] = {"us": round(ms * 1e3, 2), "GBps": round(moved / (ms * 1e-3) / 1e9, 1), "bytes": moved}
+        for b in (cache, rows, back):
+            b.free()
+        # container: one q4 g64 gate tensor written, opened, validated, uploaded as one device buffer, wrapped with no copy
+        words, s_, z_ = host["gate"]
+        blocks = pkg.repack_mlx_to_staf(fmt, words, s_, z_, pkg.BF16)
+        with tempfile.TemporaryDirectory() as tmp:
+            path = os.path.join(tmp, "bench.staf")
+            pkg.staf_write(path, [dict(name="layers.0.gate_proj.weight", scheme_identifier=fmt.scheme_identifier,
+                                       shape=[14336, 4096 * BITS // 32], payload=blocks.tobytes())], None)
+            t0 = time.perf_counter()
+            ok = pkg.staf_is_valid(path)
+            f = pkg.STAFFile(path)
+            t1 = time.perf_counter()
+            region = f.upload(ctx)
+            ctx.synchronize()
+            t2 = time.perf_counter()
+            w = f.weight(ctx, "layers.0.gate_proj.weight", pkg.LAYOUT_STAF_BLOCKS, region)
+            t3 = time.perf_counter()
+            next_rows["model.staf with one 33 MB q4 tensor (host side, ms)"] = {
+                "validate_and_open_ms": round((t1 - t0) * 1e3, 2), "upload_ms": round((t2 - t1) * 1e3, 2),
+                "wrap_zero_copy_ms": round((t3 - t2) * 1e3, 3), "valid": bool(ok)}
+            w.destroy(); region.free(); f.close()
+        for k_, v_ in next_rows.items():
+            log(f"  {k_}: {v_}")
+
     # ---- secondary figure: the prefill GEMM of the same layer's gate projection (not the metric)
     prefill = None
     if not a.no_prefill:
@@ -429,7 +484,7 @@ def main():
                    "weight_bytes_per_step": layer_bytes, "layers_resident": a.layers,
                    "replay": mode, "replay_GBps": replay_gbps,
                    "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2), "per_shape": per_shape,
-                   "batch_sweep": batch_sweep, "other_configs": other, "staf_blocks_in_place_step": staf_step,
+                   "batch_sweep": batch_sweep, "other_configs": other, "staf_blocks_in_place_step": staf_step, "next_rows": next_rows,
                    "stream_read_probe": stream_read,
                    "prefill_gemm_gate": prefill},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",

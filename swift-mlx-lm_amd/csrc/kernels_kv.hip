@@ -94,6 +94,46 @@ __global__ __launch_bounds__(256) void kv_cache_write_kernel(KvArgs a) {
     }
 }
 
+// The same quantiser for head vectors of exactly 128 elements (two per lane, read with one load) with all groups of
+// the vector in flight at once: minimum and maximum are taken inside the run of group/2 lanes that holds a group,
+// every lane then writes its own two codes.  Same operations per element as the kernel above, so the same bytes.
+__global__ __launch_bounds__(256) void kv_cache_write_hd128_kernel(KvArgs a) {
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t v = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (v >= a.count * a.kv_heads) return;               // wavefront-uniform
+    const uint32_t p = v / a.kv_heads, h = v - p * a.kv_heads;
+    uint8_t* slot = a.cache + kv_slot_offset(a, h, a.first_position + p);
+    const size_t src0 = (size_t)p * a.row_stride + (size_t)h * 128u + 2u * lane;
+    float x0, x1;
+    if (a.dtype == MI355Q_F32) {
+        const float2 t = *(const float2*)((const float*)a.src + src0);
+        x0 = t.x; x1 = t.y;
+    } else {
+        const uint32_t t = *(const uint32_t*)((const uint16_t*)a.src + src0);
+        if (a.dtype == MI355Q_BF16) { x0 = __uint_as_float(t << 16); x1 = __uint_as_float(t & 0xFFFF0000u); }
+        else { x0 = f16_to_f32((uint16_t)(t & 0xFFFFu)); x1 = f16_to_f32((uint16_t)(t >> 16)); }
+    }
+    float lo = fminf(x0, x1), hi = fmaxf(x0, x1);
+    for (uint32_t o = a.group >> 2; o >= 1; o >>= 1) {    // group / 2 lanes hold one group
+        lo = fminf(lo, __shfl_xor(lo, (int)o));
+        hi = fmaxf(hi, __shfl_xor(hi, (int)o));
+    }
+    const float levels = a.bits == 8 ? 255.0f : 15.0f;
+    const int top = a.bits == 8 ? 255 : 15;
+    float scale = __fdiv_rn(__fsub_rn(hi, lo), levels);
+    if (scale < 1e-10f) scale = 1e-10f;
+    const uint32_t d = 2u * lane, g = d / a.group, i = d - g * a.group;
+    uint8_t* block = slot + (size_t)g * a.bytes_per_block;
+    if (i == 0) *(uint32_t*)block = (uint32_t)f32_to_f16_rne(scale) | ((uint32_t)f32_to_f16_rne(lo) << 16);
+    auto code = [&](float x) {
+        const int q = (int)roundf(__fdiv_rn(__fsub_rn(x, lo), scale));
+        return (uint32_t)(q < 0 ? 0 : q > top ? top : q);
+    };
+    const uint32_t q0 = code(x0), q1 = code(x1);
+    if (a.bits == 8) *(uint16_t*)(block + 4 + i) = (uint16_t)(q0 | (q1 << 8));
+    else block[4 + (i >> 1)] = (uint8_t)(q0 | (q1 << 4));
+}
+
 // One thread per element of the output rows.
 __global__ __launch_bounds__(256) void kv_cache_read_kernel(KvArgs a) {
     const uint32_t row_elems = a.kv_heads * a.head_dim;
@@ -200,7 +240,13 @@ mi355q_status mi355q_kv_cache_write(mi355q_context* ctx, void* stream, const mi3
                                       sequence_length, &a)) return st;
     a.src = src_dev;
     const uint64_t vectors = (uint64_t)a.count * a.kv_heads;
-    kv_cache_write_kernel<<<dim3((unsigned)((vectors + 3) / 4)), dim3(256), 0, (hipStream_t)stream>>>(a);
+    const size_t esz = a.dtype == MI355Q_F32 ? 4 : 2;
+    const bool two_per_lane = a.bits != 0 && a.head_dim == 128 && a.row_stride % 2 == 0 &&
+                              (uintptr_t)src_dev % (2 * esz) == 0 && (a.group == 32 || a.group == 64 || a.group == 128);
+    if (two_per_lane)
+        kv_cache_write_hd128_kernel<<<dim3((unsigned)((vectors + 3) / 4)), dim3(256), 0, (hipStream_t)stream>>>(a);
+    else
+        kv_cache_write_kernel<<<dim3((unsigned)((vectors + 3) / 4)), dim3(256), 0, (hipStream_t)stream>>>(a);
     MI355Q_HIP(hipGetLastError());
     return MI355Q_OK;
 }
