@@ -117,7 +117,16 @@ __device__ __forceinline__ uint64_t load_codes8(const WView& w, uint32_t row, ui
             for (uint32_t i = 0; i < w.bits; i++) v |= (uint64_t)qs[i] << (8u * i);
         }
     } else {
-        for (uint32_t i = 0; i < 8; i++) v |= (uint64_t)load_code(w, row, c0 + i) << (i * w.bits);
+        // TILE16 (4-bit): the 8 codes are one record word, lane kq*16 + row%16, word j as in load_code; its nibbles are
+        // stored as (c0,c2,c4,c6,c1,c3,c5,c7): even codes in the low half, odd ones in the high half
+        const uint32_t o = c0 & 127u, g = o >> 6, in_g = o & 63u, kq = in_g >> 4, j = g * 2 + ((in_g >> 3) & 1u);
+        const uint32_t* rec = w.tiles + ((size_t)(row >> 4) * (w.k >> 7) + (c0 >> 7)) * 288u;
+        const uint32_t word = rec[(kq * 16u + (row & 15u)) * 4u + j];
+        auto spread = [](uint32_t x) {                       // nibble i of the low 16 bits -> nibble 2i
+            x = (x | (x << 8)) & 0x00FF00FFu;
+            return (x | (x << 4)) & 0x0F0F0F0Fu;
+        };
+        v = spread(word & 0xFFFFu) | (spread(word >> 16) << 4);
     }
     return v;
 }
