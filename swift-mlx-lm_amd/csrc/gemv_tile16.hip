@@ -337,6 +337,9 @@ Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_total_
     // traffic, as long as 16 wavefronts hold them and half the CUs still get a workgroup.
     uint32_t ks = 4;
     while (ks < 16 && n_total_tiles * ks < cus * 8 && kblocks / (ks * 2) >= 2) ks *= 2;
+    // long rows: at most 16 K-blocks per wavefront (28672 -> 8192 at M = 1: 48 us with a four-way split, 30 us
+    // with sixteen; 14336 -> 4096: 13.2 / 9.4 us), which leaves the four-way split to rows of up to 8192 codes
+    while (ks < 16 && kblocks / ks > 16) ks *= 2;
     const uint32_t want_tpw = m == 1 ? 1u : m <= 4 ? 2u : 4u;
     uint32_t tpw = 1;
     while (tpw < want_tpw && ks * tpw * 2 <= 16 && (n_total_tiles + tpw * 2 - 1) / (tpw * 2) >= cus / 2) tpw *= 2;
