@@ -310,6 +310,12 @@ def main():
                     t = int(tok.download(np.int32)[0])
                     if t != oracle.argmax_lowest(got):
                         sys.exit(f"bench.py: {label}: token {t} is not the lowest-index argmax of the logits")
+                    # and against the CPU reference logits: only a near-tie between the top two can differ
+                    top2 = np.sort(want)[-2:]
+                    head_check = {"token": t, "token_of_cpu_reference_logits": int(np.argmax(want)),
+                                  "top2_gap": float(top2[1] - top2[0])}
+                    if head_check["token"] != head_check["token_of_cpu_reference_logits"] and head_check["top2_gap"] > 1e-3:
+                        sys.exit(f"bench.py: {label}: token {t} differs from the CPU reference's {head_check}")
                 else:
                     got = oracle.bf16_to_f32(yd1.download(np.uint16))
                     want = oracle.bf16_to_f32(oracle.bf16_from_f32(want.astype(np.float32)))
@@ -318,6 +324,8 @@ def main():
                     sys.exit(f"bench.py: parity gate failed on {label}: rel-L2 {rel:.3e}")
             ms = time_region(ctx, lambda i: pl.encode(stream), 6, stream) / copies
             other[label] = {"us": round(ms * 1e3, 2), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1), "weight_bytes": nbytes}
+            if head and not a.skip_parity:
+                other[label]["argmax_parity"] = head_check
             log(f"  {label}: {other[label]['us']} us/launch, {other[label]['GBps']} GB/s")
             pl.destroy()
             for w in ws:
