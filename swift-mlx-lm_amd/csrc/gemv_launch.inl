@@ -42,11 +42,13 @@ mi355q_status launch_group(hipStream_t s, const GemvArgs& a, const GemvCfg& c) {
     MI355Q_TRY(1, 1, false, 4, 2, 1) MI355Q_TRY(1, 1, false, 4, 4, 1)
     MI355Q_TRY(1, 1, false, 4, 2, 0) MI355Q_TRY(1, 1, false, 4, 4, 0)
     MI355Q_TRY(1, 1, false, 8, 2, 0) MI355Q_TRY(1, 1, false, 8, 4, 0)
+    MI355Q_TRY(1, 1, false, 16, 2, 0) MI355Q_TRY(1, 1, false, 16, 4, 0)
 #endif
     // the same with the fused arg-max tail (LM head)
     MI355Q_TRY(1, 1, true, 4, 2, 1) MI355Q_TRY(1, 1, true, 4, 4, 1)
     MI355Q_TRY(1, 1, true, 4, 2, 0) MI355Q_TRY(1, 1, true, 4, 4, 0)
     MI355Q_TRY(1, 1, true, 8, 2, 0) MI355Q_TRY(1, 1, true, 8, 4, 0)
+    MI355Q_TRY(1, 1, true, 16, 2, 0) MI355Q_TRY(1, 1, true, 16, 4, 0)
     // small batches (M = 2, 3-4)
     constexpr int R2 = gemv_batch_rows(BITS, GROUP, 2), R4 = gemv_batch_rows(BITS, GROUP, 4);
     constexpr int D2 = gemv_batch_depth(BITS, GROUP, 2), D4 = gemv_batch_depth(BITS, GROUP, 4);
