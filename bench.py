@@ -217,7 +217,21 @@ def main():
         ms = time_region(ctx, lambda i: p1.encode(stream), reps, stream) / a.layers
         nbytes = sum(weight_bytes(*dims[n]) for n in names)
         per_shape[label] = {"us": round(ms * 1e3, 3), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1), "weight_bytes": nbytes}
-        log(f"  {label:8s}: {ms * 1e3:.2f} us/launch, {per_shape[label]['GBps']} GB/s")
+        # spread of single launches: one HIP event pair around each of 192 launches over the rotating copies
+        # (an event pair adds two to three microseconds to what it brackets; "us" above is the back-to-back figure)
+        singles = []
+        ea, eb = ctx.event_create(), ctx.event_create()
+        for i in range(192):
+            ctx.event_record(ea, stream)
+            p1.encode(stream, i % a.layers, 1)
+            ctx.event_record(eb, stream)
+            ctx.event_synchronize(eb)
+            singles.append(ctx.event_elapsed_ms(ea, eb) * 1e3)
+        singles.sort()
+        per_shape[label]["single_launch_us"] = {"median": round(singles[96], 2), "p10": round(singles[19], 2),
+                                                "p90": round(singles[172], 2)}
+        log(f"  {label:8s}: {ms * 1e3:.2f} us/launch, {per_shape[label]['GBps']} GB/s; single launches "
+            f"{per_shape[label]['single_launch_us']}")
         p1.destroy()
     # ---- secondary: the same layer step at M = 1, 2, 4, 8 activation rows (BASELINE config 1), on
     # the split-plane layout and on the matrix-core tile layout (4-launch schedule, stream replay)
