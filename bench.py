@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-linear hot path on one MI355X.
 
-Workload (BASELINE config 1 at M=1): one decode pass over the seven 4-bit g64 projections of a
+Workload (benchmark config 1 at M=1): one decode pass over the seven 4-bit g64 projections of a
 Llama-3-8B layer (q, k, v, o, gate, up, down).  One "step" = those seven GEMV launches on one
 stream.  `--layers` distinct copies of the layer's weights (default 32, 3.9 GB) are resident in
 HBM and steps rotate through them, so every launch streams its weights from HBM rather than
@@ -58,7 +58,7 @@ def time_region(ctx, fn, reps, stream=0):
 
 def cpu_baseline(seconds: float):
     """The reference's loop nest (row -> block -> k, fp32 accumulate) on the host cores, timed on
-    BASELINE config 0 (q4 g64, 2048 -> 8192, M=1) for a bounded number of passes."""
+    benchmark config 0 (q4 g64, 2048 -> 8192, M=1) for a bounded number of passes."""
     import kat
     import oracle
     n, k = 8192, 2048
@@ -90,7 +90,7 @@ def main():
     ap.add_argument("--skip-parity", action="store_true")
     ap.add_argument("--no-prefill", action="store_true", help="skip the secondary prefill-GEMM figure")
     ap.add_argument("--no-other-configs", action="store_true",
-                    help="skip the secondary per-launch figures of BASELINE configs 0, 2 and 4")
+                    help="skip the secondary per-launch figures of benchmark configs 0, 2 and 4")
     ap.add_argument("--no-batch-sweep", action="store_true", help="skip the secondary M = 1, 2, 4, 8 figures")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -233,7 +233,7 @@ def main():
         log(f"  {label:8s}: {ms * 1e3:.2f} us/launch, {per_shape[label]['GBps']} GB/s; single launches "
             f"{per_shape[label]['single_launch_us']}")
         p1.destroy()
-    # ---- secondary: the same layer step at M = 1, 2, 4, 8 activation rows (BASELINE config 1), on
+    # ---- secondary: the same layer step at M = 1, 2, 4, 8 activation rows (benchmark config 1), on
     # the split-plane layout and on the matrix-core tile layout (4-launch schedule, stream replay)
     batch_sweep = None
     if not a.no_batch_sweep:
@@ -286,7 +286,7 @@ def main():
     log(f"  copy  {gate_bytes} B: {ms_copy * 1e3:.2f} us/launch, {2 * gate_bytes / (ms_copy * 1e-3) / 1e9:.1f} GB/s "
         "read+write")
 
-    # ---- secondary: one launch each of BASELINE config 0 (2048->8192), config 2 (4096->14336 at 8, 6, 3 and 2 bits)
+    # ---- secondary: one launch each of benchmark config 0 (2048->8192), config 2 (4096->14336 at 8, 6, 3 and 2 bits)
     # and config 4 (LM head 2048->65536 fused with argmax), over rotating copies of more than 512 MB in total
     other = None
     if not a.no_other_configs:
@@ -501,7 +501,7 @@ def main():
         "dtype": "bf16 activations x u4 codes, fp32 accumulate",
         "data": "synthetic: W~N(0,0.02^2) quantised q4 g64 (bf16 scale/bias planes), x~N(0,1) bf16, seeded; "
                 f"{a.layers} resident copies of one layer's tensors",
-        "config": {"workload": "Llama-3-8B decode layer sweep (BASELINE config 1), M=1: q,k,v,o,gate,up,down "
+        "config": {"workload": "Llama-3-8B decode layer sweep (benchmark config 1), M=1: q,k,v,o,gate,up,down "
                                "GEMVs per step", "bits": BITS, "group_size": GROUP,
                    "weight_bytes_per_step": layer_bytes, "layers_resident": a.layers,
                    "replay": mode, "replay_GBps": replay_gbps,

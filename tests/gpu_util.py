@@ -107,7 +107,7 @@ def run_gemv(ctx, pkg, w, x_f32, x_dtype, y_dtype, flags=0, x_stride=None, use_q
 
 
 def seeded_case(seed, n, k, bits, group):
-    """BASELINE-style tensors: W ~ N(0, 0.02^2) quantised per group to bf16 scale/bias planes.
+    """benchmark-style tensors: W ~ N(0, 0.02^2) quantised per group to bf16 scale/bias planes.
     Returns (codes_words, scales_bf16, biases_bf16, dequantised fp32 weights)."""
     w = kat.seeded_weights(seed, n, k)
     words, s, z = oracle.quantize_affine(w, bits, group, oracle.BF16)

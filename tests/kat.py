@@ -14,7 +14,7 @@ import numpy as np
 
 _GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_kats.json")
 
-# every (bits, group) the reference registers, plus the two BASELINE additions
+# every (bits, group) the reference registers, plus the two formats the benchmark adds (q6 g64, q2 g64)
 REFERENCE_FORMATS = [(2, 16), (2, 32), (3, 16), (3, 32), (3, 64), (4, 64), (4, 128), (5, 32),
                      (5, 64), (6, 16), (6, 32), (8, 32), (8, 64), (8, 128)]
 NEW_FORMATS = [(2, 64), (6, 64)]
@@ -137,7 +137,7 @@ def roundtrip_case(bits, group, rows, blocks, scale_base, zero_base):
     return codes, scales, zeros
 
 
-# ---- seeded BASELINE-style inputs -----------------------------------------------------------
+# ---- seeded benchmark-style inputs -----------------------------------------------------------
 
 def seeded_weights(seed: int, n: int, k: int) -> np.ndarray:
     """W ~ N(0, 0.02^2) fp32, PCG64-seeded."""

@@ -173,8 +173,8 @@ def test_repack_error_paths():
 # ---- MetalCompileContext.swift:5-90: decode shape families ---------------------------------
 def test_shape_families():
     want = {
-        (8192, 2048): ("input20488192Dense", 8, 2048, "gemv_2048_8192"),     # BASELINE config 0
-        (65536, 2048): ("vocabDense", 16, 2048, "gemv_vocab"),                # BASELINE config 4
+        (8192, 2048): ("input20488192Dense", 8, 2048, "gemv_2048_8192"),     # benchmark config 0
+        (65536, 2048): ("vocabDense", 16, 2048, "gemv_vocab"),                # benchmark config 4
         (2048, 2048): ("input2048SquareDense", 8, 2048, "gemv_2048_sq"),
         (6144, 2048): ("input20486144Dense", 4, 2048, "gemv_2048_6144"),
         (4096, 2048): ("input2048ExpandedDense", 8, 2048, "gemv_2048"),

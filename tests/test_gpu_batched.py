@@ -51,7 +51,7 @@ def _run_batched(pkg, ctx, ws, ns, x, y_dtype, flags=0, x_stride=0):
 @pytest.mark.parametrize("ns,k", [((4096, 1024, 1024), 4096), ((14336, 14336), 4096)])
 @pytest.mark.parametrize("m", [1, 2, 8])
 def test_batched_llama_projections(pkg, ctx, ns, k, m):
-    """q+k+v and gate+up of a Llama-3-8B layer (BASELINE config 1 shapes) as one launch each."""
+    """q+k+v and gate+up of a Llama-3-8B layer (benchmark config 1 shapes) as one launch each."""
     ws, wqs = _prepare(pkg, ctx, 1300 + len(ns), ns, k, 4, 64, pkg.LAYOUT_PLANES)
     x = act_rounded(kat.seeded_activations(1310 + m, m, k), pkg.BF16, pkg)
     say(f"batched {ns} K={k} M={m}")

@@ -173,7 +173,7 @@ def _tile_edge_sample(n, seed, per_tile=2, tile=128):
 @pytest.mark.parametrize("m", [128, 512, 2048])
 @pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
 def test_config3_prefill_gate_up_and_down(pkg, ctx, m, n, k):
-    """BASELINE config 3 at full size.  Every one of the M output rows is checked, on a sample of
+    """benchmark config 3 at full size.  Every one of the M output rows is checked, on a sample of
     output columns that holds the first and last column of every 128-wide column tile plus two
     random ones (the CPU oracle on all 14336 columns would take minutes)."""
     sample = _tile_edge_sample(n, 31 * m + n)

@@ -124,7 +124,7 @@ def test_q4_gemm_with_padded_input_stride(pkg, ctx):
         w.destroy()
 
 
-# ---------------------------------------------------------- seeded BASELINE configurations
+# ---------------------------------------------------------- seeded benchmark configurations
 def _seeded_gemv_check(pkg, ctx, seed, n, k, bits, group, ms, layouts=("planes",), check_codes=False):
     words, s, z, wq = seeded_case(seed, n, k, bits, group)
     fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(bits, group)
@@ -151,7 +151,7 @@ def _seeded_gemv_check(pkg, ctx, seed, n, k, bits, group, ms, layouts=("planes",
 
 
 def test_config0_q4g64_2048_to_8192(pkg, ctx):
-    """BASELINE config 0, both layouts (bf16 scale planes and f16 STAF headers dequantise identically)."""
+    """benchmark config 0, both layouts (bf16 scale planes and f16 STAF headers dequantise identically)."""
     r = _seeded_gemv_check(pkg, ctx, 100, 8192, 2048, 4, 64, [1], layouts=("planes", "staf"), check_codes=True)
     assert max(v[0] for v in r.values()) < 1e-4
 

@@ -71,7 +71,7 @@ LLAMA = {"q_o": (4096, 4096), "k_v": (1024, 4096), "gate_up": (14336, 4096), "do
 
 @pytest.mark.parametrize("name", list(LLAMA))
 def test_tile16_llama_shapes_all_batch_sizes(pkg, ctx, name):
-    """BASELINE config 1 shapes, M = 1, 2, 4, 8 (and the sizes in between up to 16)."""
+    """benchmark config 1 shapes, M = 1, 2, 4, 8 (and the sizes in between up to 16)."""
     n, k = LLAMA[name]
     words, s, z, wq = seeded_case(2100 + n % 89, n, k, 4, 64)
     w = ctx.weight_prepare_mlx(_fmt(pkg), words, s, z, pkg.BF16, pkg.LAYOUT_TILE16)
@@ -165,7 +165,7 @@ def test_tile16_batched_projections_one_launch(pkg, ctx):
 
 
 def test_tile16_lm_head_fused_argmax(pkg, ctx):
-    """BASELINE config 4 (2048 -> 65536): token == lowest-index argmax of the GPU's own fp32 logits and
+    """benchmark config 4 (2048 -> 65536): token == lowest-index argmax of the GPU's own fp32 logits and
     of the CPU reference logits; ties resolve to the lowest index."""
     n, k = 65536, 2048
     words, s, z, wq = seeded_case(2800, n, k, 4, 64)

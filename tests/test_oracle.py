@@ -227,7 +227,7 @@ def test_cpu_weight_store_vector():
 
 
 def test_planes_and_staf_dequant_agree_with_bf16_scales():
-    """BASELINE-style bf16 scales are exact in f16 for the configured value range, so both
+    """benchmark-style bf16 scales are exact in f16 for the configured value range, so both
     layouts dequantise to identical fp32 weights."""
     w = kat.seeded_weights(7, 16, 256)
     for bits, group in [(4, 64), (8, 32), (6, 64), (3, 64), (2, 64)]:
