@@ -32,7 +32,7 @@ BITS, GROUP = 4, 64
 # HBM bytes per gate launch and per fused gate+up launch from the FETCH_SIZE and WRITE_SIZE counters, each scaled by what the
 # same counter reads for a plain copy of the same size (profiles/gemv_planes_q4_g64_gate_up_hbm_traffic_pmc.md).
 # Measured offline with the profiler; valid for the kernel variant named in `roofline.kernel`.
-TRAFFIC_BYTES = {"gate": 33244063, "gate_up": 66309001}
+TRAFFIC_BYTES = {"gate": 33260041, "gate_up": 66317409}
 
 
 def log(*a):
