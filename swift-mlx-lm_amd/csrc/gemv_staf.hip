@@ -6,8 +6,8 @@
 //     aligned vector load.  A wavefront instead copies a span of 64 consecutive blocks of one row --
 //     one contiguous byte range -- from memory straight into LDS with 128-bit direct-to-LDS loads
 //     (no register staging), and every lane then reads its own block back with 32-bit LDS reads:
-//     1 + GROUP*BITS/32 dwords at a stride that is odd for every supported format, so the reads are
-//     free of bank conflicts;
+//     1 + GROUP*BITS/32 dwords at a stride that is odd for the common formats (q4 and q8 at every
+//     group size, every width at g64), so their reads are free of bank conflicts;
 //   * a wavefront owns a run of consecutive rows and keeps D spans in flight in a private LDS ring;
 //     the direct-to-LDS loads are invisible to the compiler's wait-counter bookkeeping, so the
 //     kernel waits on the vector-memory counter itself: every span is exactly NDMA load
@@ -419,6 +419,13 @@ mi355q_status launch_by_format(hipStream_t s, uint32_t bits, uint32_t group, con
     case 3064: return launch_for_format<3, 64>(s, a, mt, depth, grid, argmax);
     case 5064: return launch_for_format<5, 64>(s, a, mt, depth, grid, argmax);
     case 6064: return launch_for_format<6, 64>(s, a, mt, depth, grid, argmax);
+    case 2016: return launch_for_format<2, 16>(s, a, mt, depth, grid, argmax);
+    case 2032: return launch_for_format<2, 32>(s, a, mt, depth, grid, argmax);
+    case 3032: return launch_for_format<3, 32>(s, a, mt, depth, grid, argmax);
+    case 5032: return launch_for_format<5, 32>(s, a, mt, depth, grid, argmax);
+    case 6016: return launch_for_format<6, 16>(s, a, mt, depth, grid, argmax);
+    case 6032: return launch_for_format<6, 32>(s, a, mt, depth, grid, argmax);
+    case 8128: return launch_for_format<8, 128>(s, a, mt, depth, grid, argmax);
     default: break;
     }
     return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no block-layout GEMV for q%ug%u", bits, group);
@@ -430,6 +437,8 @@ bool staf_shape(uint32_t bits, uint32_t group, StafShape& out) {
     if (bits == B && group == GR) { out = {StafGeo<B, GR>::SLOT, StafGeo<B, GR>::Q}; return true; }
     MI355Q_STAF_CASE(4, 64) MI355Q_STAF_CASE(4, 128) MI355Q_STAF_CASE(8, 32) MI355Q_STAF_CASE(8, 64)
     MI355Q_STAF_CASE(2, 64) MI355Q_STAF_CASE(3, 64) MI355Q_STAF_CASE(5, 64) MI355Q_STAF_CASE(6, 64)
+    MI355Q_STAF_CASE(2, 16) MI355Q_STAF_CASE(2, 32) MI355Q_STAF_CASE(3, 32) MI355Q_STAF_CASE(5, 32)
+    MI355Q_STAF_CASE(6, 16) MI355Q_STAF_CASE(6, 32) MI355Q_STAF_CASE(8, 128)
 #undef MI355Q_STAF_CASE
     return false;
 }

@@ -19,7 +19,8 @@ from gpu_util import Case, act_rounded, assert_within_tolerance, run_gemv
 pytestmark = pytest.mark.gpu
 
 # formats whose blocks are whole 32-bit words and that the in-place kernel is built for
-FORMATS = [(4, 64), (4, 128), (8, 32), (8, 64), (2, 64), (3, 64), (5, 64), (6, 64)]
+FORMATS = [(4, 64), (4, 128), (8, 32), (8, 64), (8, 128), (2, 16), (2, 32), (2, 64), (3, 32), (3, 64), (5, 32), (5, 64),
+           (6, 16), (6, 32), (6, 64)]
 
 
 def say(*a):
@@ -69,6 +70,7 @@ def test_in_place_gemv_formats_and_tails(pkg, ctx, bits, group):
         for n in (1, 37, 700):
             case = _case(3000 + bits * 7 + group + ci, n, k, bits, group)
             w = case.device_weight(ctx, pkg, pkg.LAYOUT_STAF_BLOCKS)
+            assert w.plan_decode_step(1).device_kernel == f"gemv_staf_q{bits}_g{group}"
             wq = oracle.dequant_staf_f32(bits, group, n, k, case.staf_blocks())
             for m in (1, 2, 3, 5, 8):
                 x = act_rounded(kat.seeded_activations(3100 + m + ci, m, k), pkg.BF16, pkg)
