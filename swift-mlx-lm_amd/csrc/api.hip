@@ -140,7 +140,8 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
         strides[i] = y_stride;
         views[i] = weights[i]->view();
         fused = fused && gemv_fast_eligible(views[i], x_dtype, m, xs) && views[i].sb_dtype == views[0].sb_dtype;
-        tiled = tiled && gemv_tile16_eligible(views[i], x_dtype, m, xs) && views[i].sb_dtype == views[0].sb_dtype;
+        tiled = tiled && gemv_tile16_eligible(views[i], x_dtype, m, xs) && gemv_tile16_k_parts(ctx, views[i], m) == 1 &&
+                views[i].sb_dtype == views[0].sb_dtype;
         in_place = in_place && gemv_staf_eligible(views[i], x_dtype, m, xs);
     }
     if (fused && (uintptr_t)x % 16 == 0)
@@ -166,7 +167,8 @@ mi355q_status dispatch_output_head(mi355q_context* ctx, hipStream_t s, const mi3
     if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && gemv_fast_eligible(v, x_dtype, 1, xs) && (uintptr_t)x % 16 == 0)
         return launch_gemv_fast(s, ctx, v, x, nullptr, MI355Q_F32, 1, xs, (uint32_t)w->n, logits, token,
                                 ctx->argmax_partials);
-    if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && gemv_tile16_eligible(v, x_dtype, 1, xs) && (uintptr_t)x % 16 == 0) {
+    if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && gemv_tile16_eligible(v, x_dtype, 1, xs) && gemv_tile16_k_parts(ctx, v, 1) == 1 &&
+        (uintptr_t)x % 16 == 0) {
         void* none[1] = {nullptr};
         const uint32_t strides[1] = {(uint32_t)w->n};
         return launch_gemv_tile16_multi(s, ctx, 1, &v, x, none, strides, MI355Q_F32, 1, xs, logits, token,
@@ -267,6 +269,7 @@ mi355q_status mi355q_argmax(mi355q_context* ctx, void* stream, const void* logit
     if (!ctx) return fail(MI355Q_ERR_NULL_HANDLE, "context is null");
     if (!logits_dev || !token_out_dev) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null pointer");
     if (!dtype_ok(dtype)) return fail(MI355Q_ERR_INVALID_ARGUMENT, "bad dtype tag");
+    if (vocabulary_size == 0) return fail(MI355Q_ERR_SHAPE, "argmax over an empty vector");
     MI355Q_HIP(hipSetDevice(ctx->device));
     return launch_argmax((hipStream_t)stream, logits_dev, dtype, vocabulary_size, token_out_dev,
                          ctx->argmax_partials + kArgmaxPartialCapacity);
@@ -283,6 +286,7 @@ mi355q_status mi355q_clock_probe_read(mi355q_context* ctx, uint64_t* shader_cycl
     if (!ctx) return fail(MI355Q_ERR_NULL_HANDLE, "context is null");
     if (!shader_cycles || !realtime_ticks) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null output");
     unsigned long long cell[2] = {0, 0};
+    MI355Q_HIP(hipSetDevice(ctx->device));
     MI355Q_HIP(hipDeviceSynchronize());
     MI355Q_HIP(hipMemcpy(cell, ctx->argmax_scratch + 16, sizeof cell, hipMemcpyDeviceToHost));
     *shader_cycles = cell[0];

@@ -59,10 +59,14 @@ struct mi355q_context {
     // fused output head: one packed (ordered value, ~row) key per workgroup of the projection launch
     // (kArgmaxPartialCapacity entries), then kArgmaxStandaloneKeys entries for the stand-alone argmax
     unsigned long long* argmax_partials;
-    // split-K partial results of the prefill GEMM: grown on demand, never shrunk
+    // fp32 partial results (split-K of the prefill GEMM, K parts of the tile kernel): grown on demand, never shrunk;
+    // outgrown buffers are kept until the context goes, because captured graphs hold their addresses
     void* workspace;
     size_t workspace_bytes;
+    void* retired[40];
+    int retired_count;
 };
+constexpr int kRetiredWorkspaces = 40;
 
 struct mi355q_weight {
     mi355q_context* ctx;
@@ -159,10 +163,14 @@ constexpr int kTile16MaxSegments = 3;
 struct Tile16LaunchShape {
     uint32_t ksplit, tiles_per_wg, waves, blocks_per_wave, grid, block, lds_bytes;
     uint32_t passes;     // row tiles a wavefront walks on one staged copy of the activations
+    uint32_t parts;      // K parts (1: whole rows); each part has wgs_per_part workgroups and stages only its columns
+    uint32_t wgs_per_part;
 };
 bool gemv_tile16_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
-Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_total_tiles, uint32_t k, uint32_t m);
-mi355q_status launch_gemv_tile16_multi(hipStream_t s, const mi355q_context* ctx, uint32_t count, const WView* w,
+// K parts a launch of M rows takes: 1 = whole rows (needed by fused q+k+v / gate+up launches and by the fused head)
+uint32_t gemv_tile16_k_parts(const mi355q_context* ctx, const WView& w, uint32_t m);
+Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_row_tiles, uint32_t k, uint32_t m);
+mi355q_status launch_gemv_tile16_multi(hipStream_t s, mi355q_context* ctx, uint32_t count, const WView* w,
                                        const void* x, void* const* y, const uint32_t* y_strides, int y_dtype,
                                        uint32_t m, uint32_t x_stride, float* logits_f32, int32_t* token_out,
                                        unsigned long long* argmax_scratch);
@@ -184,7 +192,7 @@ struct GemmLaunchShape {
     uint32_t bm, bn, stages, grid, block, lds_bytes, splits, kt_per_split;
 };
 GemmLaunchShape gemm_mfma_shape(const mi355q_context* ctx, uint32_t m, uint32_t n, uint32_t k);
-// Grows the context's scratch buffer (split-K partials); the buffer is kept until the context goes.
+// Grows the context's scratch buffer for fp32 partial results; nothing is released before the context goes.
 mi355q_status ensure_workspace(mi355q_context* ctx, size_t bytes);
 bool gemm_mfma_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
 mi355q_status launch_qgemm_mfma(hipStream_t s, mi355q_context* ctx, const WView& w,

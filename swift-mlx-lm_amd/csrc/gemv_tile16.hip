@@ -46,11 +46,15 @@ struct T16Args {
     float* logits;                               // optional fp32 [N] copy (M == 1, one matrix)
     int32_t* token_out;                          // ARGMAX only
     unsigned long long* scratch;                 // ARGMAX only: one packed key per workgroup; 0 = no candidate
+    float* partial;                              // K parts only: fp32 partial results [part][M][N] (one matrix)
     uint32_t k, m, x_stride;
     uint32_t kblocks;                            // K / 128
+    uint32_t parts;                              // K parts, each with workgroups of its own that stage only their columns
+    uint32_t part_blocks;                        // K-blocks per part (kblocks / parts)
+    uint32_t wgs_per_part;                       // workgroups of one part: blockIdx.x = part * wgs_per_part + index
     uint32_t blocks_per_wave;                    // K-blocks per wavefront (K split over the workgroup)
     uint32_t passes;                             // row tiles a wavefront walks, one after the other, on one staged copy of x
-    uint32_t lds_row_bytes;                      // K*2 + 16: staged activation row pitch
+    uint32_t lds_row_bytes;                      // part_blocks*256 + 16: staged activation row pitch
     uint32_t y_dtype, sb_dtype;
 };
 
@@ -67,6 +71,11 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t n_in = lane & 15, kq = lane >> 4;
+    // K part of this workgroup: K-blocks [kb0, kb0 + part_blocks), activation columns [kb0 * 128, ...)
+    const uint32_t part = a.parts > 1 ? blockIdx.x / a.wgs_per_part : 0u;
+    const uint32_t wg = blockIdx.x - part * a.wgs_per_part;
+    const uint32_t kb0 = part * a.part_blocks;
+    const uint32_t kp = a.part_blocks * 128;                // activation elements this workgroup stages per row
 
     // ---- matrix and row tile of this wavefront in pass `pass` (scalar select chain) ---------------
     const uint32_t slice = wave % KSPLIT;                   // share of K
@@ -78,7 +87,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
     };
     auto select_tile = [&](uint32_t pass) {
         Tile t;
-        uint32_t gt = (blockIdx.x * a.passes + pass) * TPW + wave / KSPLIT;
+        uint32_t gt = (wg * a.passes + pass) * TPW + wave / KSPLIT;
         t.valid = gt < a.tile_end[kTile16MaxSegments - 1];
         gt = t.valid ? gt : a.tile_end[kTile16MaxSegments - 1] - 1;      // idle wavefronts re-read the last tile
         const bool in1 = gt >= a.tile_end[0], in2 = gt >= a.tile_end[1];
@@ -88,11 +97,12 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
         t.rows = in2 ? a.seg_rows[2] : in1 ? a.seg_rows[1] : a.seg_rows[0];
         const uint32_t lt = gt - (in2 ? a.tile_end[1] : in1 ? a.tile_end[0] : 0u);
         t.n0 = lt * 16;
-        t.b_first = slice * a.blocks_per_wave;
-        uint32_t nb = a.kblocks > t.b_first ? a.kblocks - t.b_first : 0;      // blocks this wavefront owns
+        const uint32_t kb_end = kb0 + a.part_blocks;
+        t.b_first = kb0 + slice * a.blocks_per_wave;
+        uint32_t nb = kb_end > t.b_first ? kb_end - t.b_first : 0;            // blocks this wavefront owns
         nb = nb < a.blocks_per_wave ? nb : a.blocks_per_wave;
         t.nb = t.valid ? nb : 0;
-        t.b_last = t.nb ? t.b_first + t.nb - 1 : a.kblocks - 1;              // clamp target (always valid)
+        t.b_last = t.nb ? t.b_first + t.nb - 1 : kb_end - 1;                 // clamp target (always valid)
         t.base = seg_tiles + (size_t)lt * a.kblocks * kT16RecordWords;
         return t;
     };
@@ -101,7 +111,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
     // ---- 1. activation loads first (vector loads return in issue order) -------------------------
     // Raw copy of the M rows into LDS, row pitch K*2 + 16 bytes (the pad spreads the 16 rows of an
     // A-fragment read over all banks).  Each thread moves up to XC 16-byte chunks per row pass.
-    const uint32_t chunks = a.k / 8;                        // 16-byte chunks per activation row
+    const uint32_t chunks = kp / 8;                         // 16-byte chunks per staged activation row
     constexpr int XC = 2;
     u32x4 xe[XC];
     auto x_row = [&](uint32_t i, uint32_t& m, uint32_t& c) {   // chunk index -> (row, chunk in row)
@@ -112,7 +122,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
         const uint32_t total = a.m * chunks;
         uint32_t m, c;
         x_row(idx < total ? idx : 0, m, c);
-        return (const u32x4*)(a.x + (size_t)m * a.x_stride) + c;
+        return (const u32x4*)(a.x + (size_t)m * a.x_stride + (size_t)kb0 * 128) + c;
     };
     auto x_dst = [&](uint32_t idx) -> u32x4* {
         uint32_t m, c;
@@ -185,7 +195,8 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
         return __builtin_bit_cast(bf16x8_t, p);
     };
     auto compute = [&](uint32_t b, const Rec& r) {
-        const char* ab = a_lane + (size_t)b * 256;           // 128 codes = 256 bytes of activations
+        const uint32_t bl = b - kb0;                         // block inside the staged columns
+        const char* ab = a_lane + (size_t)bl * 256;          // 128 codes = 256 bytes of activations
         static_for<2>([&](auto G) {
             constexpr int g = decltype(G)::value;
             const bf16x8_t a0 = *(const bf16x8_t*)(ab + g * 128);
@@ -195,7 +206,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
             floatx4_t d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, b0, zero4, 0, 0, 0);
             d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b1, d, 0, 0, 0);
             // sum(x) of this group for output rows 4 kq .. 4 kq + MR - 1
-            const float* const sxp = sxs + (size_t)(b * 2 + g) * 16 + 4 * kq;
+            const float* const sxp = sxs + (size_t)(bl * 2 + g) * 16 + 4 * kq;
             float sx[MR];
             if constexpr (MR == 4) { const floatx4_t t = *(const floatx4_t*)sxp; sx[0] = t[0]; sx[1] = t[1]; sx[2] = t[2]; sx[3] = t[3]; }
             else if constexpr (MR == 2) { const float2_t t = *(const float2_t*)sxp; sx[0] = t[0]; sx[1] = t[1]; }
@@ -220,7 +231,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
     // once every wavefront is done reading those (the workgroup then needs no LDS beyond the activations, which
     // decides how many workgroups share a CU); several passes keep them behind the activations and their sums.
     const bool red_over_x = a.passes == 1;
-    float* const red = (float*)(red_over_x ? lds : lds + (size_t)a.m * a.lds_row_bytes + a.k);
+    float* const red = (float*)(red_over_x ? lds : lds + (size_t)a.m * a.lds_row_bytes + kp);
     unsigned long long best = 0ull;
     for (uint32_t pass = 0; pass < a.passes; pass++) {
         if (pass) {                                            // the first tile's loads were issued before staging
@@ -249,6 +260,10 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
                 for (uint32_t w2 = 0; w2 < (uint32_t)KSPLIT; w2++) v += red[((wave + w2) * MR + r) * 64 + lane];
                 const uint32_t m = 4 * kq + r;
                 if (m < a.m && row < tile.rows) {
+                    if (a.parts > 1) {                       // one matrix: the reduction launch converts and stores
+                        a.partial[((size_t)part * a.m + m) * tile.rows + row] = v;
+                        continue;
+                    }
                     if (tile.y) {
                         const size_t o = (size_t)m * tile.ys + row;
                         if (a.y_dtype == MI355Q_F32) ((float*)tile.y)[o] = v;
@@ -291,9 +306,50 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
     }
 }
 
+// Sum of the K parts, in part order, then the conversion the single-launch form does in its epilogue.
+__global__ __launch_bounds__(256) void tile16_sum_parts_kernel(const float* __restrict__ partial, uint32_t parts,
+                                                               uint32_t m, uint32_t n, void* __restrict__ y,
+                                                               uint32_t y_stride, uint32_t y_dtype,
+                                                               float* __restrict__ logits) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= m * n) return;
+    const uint32_t row = i / n, col = i - row * n;
+    float v = 0.f;
+    for (uint32_t p = 0; p < parts; p++) v += partial[((size_t)p * m + row) * n + col];
+    if (y) {
+        const size_t o = (size_t)row * y_stride + col;
+        if (y_dtype == MI355Q_F32) ((float*)y)[o] = v;
+        else if (y_dtype == MI355Q_BF16) ((uint16_t*)y)[o] = f32_to_bf16_rne(v);
+        else ((uint16_t*)y)[o] = f32_to_f16_rne(v);
+    }
+    if (logits && row == 0) logits[col] = v;
+}
+
 namespace {
 
 constexpr size_t kT16LdsBudget = 144 * 1024;
+
+size_t t16_staged_bytes(uint32_t m, uint32_t k) { return (size_t)m * ((size_t)k * 2 + 16) + k; }
+
+// K parts of a launch: 1 when the staged activations of whole rows fit in LDS; else a power of two that divides the
+// K-blocks and whose columns fit, 0 when none does.  Among those the smallest that leaves a workgroup either a small
+// staged copy (two workgroups per CU) or, with one workgroup per CU, at least three row tiles to walk on it (measured,
+// 14336 -> 4096: M = 8 in two parts 18.6 us, in four 14.2 us; M = 16 in four 16.4 us, in eight 17.6 us).
+uint32_t t16_parts(uint32_t k, uint32_t m, uint32_t n_row_tiles, uint32_t cus) {
+    const uint32_t kblocks = k / 128;
+    const int forced = env_int_cached("MI355Q_T16_PARTS", 0);
+    if (forced > 0 && kblocks % (uint32_t)forced == 0 && t16_staged_bytes(m, k / (uint32_t)forced) <= kT16LdsBudget)
+        return (uint32_t)forced;
+    if (t16_staged_bytes(m, k) <= kT16LdsBudget) return 1;
+    uint32_t first_fit = 0;
+    for (uint32_t p = 2; p <= 16 && kblocks % p == 0; p *= 2) {
+        const size_t staged = t16_staged_bytes(m, k / p);
+        if (staged > kT16LdsBudget) continue;
+        if (!first_fit) first_fit = p;
+        if (staged <= 80 * 1024 || (uint64_t)n_row_tiles * p >= 3ull * cus) return p;
+    }
+    return first_fit;
+}
 
 template <int MR, int KSPLIT, int TPW, bool ARGMAX>
 mi355q_status launch_t16(hipStream_t s, const T16Args& a, uint32_t grid, size_t lds) {
@@ -324,13 +380,24 @@ bool gemv_tile16_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_st
     if (m < 1 || m > 16) return false;
     if (w.bits != 4 || w.group != 64 || w.k % 128) return false;
     if (x_stride % 8) return false;                                   // 128-bit activation loads
-    return (size_t)m * ((size_t)w.k * 2 + 16) + w.k <= kT16LdsBudget; // staged activations and their group sums fit in LDS
+    return t16_parts(w.k, m, (w.n + 15) / 16, 256) != 0;              // staged activations and their group sums fit in LDS
 }
 
-Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_total_tiles, uint32_t k, uint32_t m) {
+uint32_t gemv_tile16_k_parts(const mi355q_context* ctx, const WView& w, uint32_t m) {
+    return t16_parts(w.k, m, (w.n + 15) / 16, (uint32_t)ctx->props.multiProcessorCount);
+}
+
+Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_row_tiles, uint32_t k_total, uint32_t m) {
     Tile16LaunchShape g{};
-    const uint32_t kblocks = k / 128;
+    // With K parts the launch is shaped as parts x as many row tiles of rows of K / parts codes: every workgroup
+    // belongs to one part, and the workgroups of a part cover all row tiles.
     const uint32_t cus = (uint32_t)ctx->props.multiProcessorCount;
+    uint32_t parts = t16_parts(k_total, m, n_row_tiles, cus);
+    if (!parts) parts = 1;
+    const uint32_t k = k_total / parts;
+    const uint32_t n_total_tiles = n_row_tiles * parts;
+    g.parts = parts;
+    const uint32_t kblocks = k / 128;
     // Measured on MI355X.  K split: the smallest of 4, 8, 16 that puts about eight wavefronts on
     // every CU (and leaves each wavefront at least two K-blocks).  Row tiles per workgroup: one for
     // M = 1; more for batches, where the staged activations are the larger share of a workgroup's
@@ -377,7 +444,8 @@ Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_total_
         const int ep = env_int_cached("MI355Q_T16_PASSES", 0);
         if (ep) g.passes = (uint32_t)ep;
     }
-    g.grid = (n_total_tiles + tpw * g.passes - 1) / (tpw * g.passes);
+    g.wgs_per_part = (n_row_tiles + tpw * g.passes - 1) / (tpw * g.passes);
+    g.grid = g.wgs_per_part * parts;
     g.block = g.waves * 64;
     const size_t x_bytes = (size_t)m * ((size_t)k * 2 + 16) + k;     // rows, then sum(x) per group: [K/64][16] floats
     const size_t red_bytes = (size_t)g.waves * 4 * 64 * 4;     // partial tiles, behind the activations
@@ -385,7 +453,7 @@ Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_total_
     return g;
 }
 
-mi355q_status launch_gemv_tile16_multi(hipStream_t s, const mi355q_context* ctx, uint32_t count, const WView* w,
+mi355q_status launch_gemv_tile16_multi(hipStream_t s, mi355q_context* ctx, uint32_t count, const WView* w,
                                        const void* x, void* const* y, const uint32_t* y_strides, int y_dtype,
                                        uint32_t m, uint32_t x_stride, float* logits_f32, int32_t* token_out,
                                        unsigned long long* argmax_scratch) {
@@ -411,9 +479,19 @@ mi355q_status launch_gemv_tile16_multi(hipStream_t s, const mi355q_context* ctx,
     a.logits = logits_f32; a.token_out = token_out; a.scratch = argmax_scratch;
     a.k = w[0].k; a.m = m; a.x_stride = x_stride;
     a.kblocks = w[0].k / 128;
+    a.parts = g.parts;
+    a.part_blocks = a.kblocks / g.parts;
+    a.wgs_per_part = g.wgs_per_part;
     a.blocks_per_wave = g.blocks_per_wave;
     a.passes = g.passes;
-    a.lds_row_bytes = w[0].k * 2 + 16;
+    a.lds_row_bytes = a.part_blocks * 256 + 16;
+    if (g.parts > 1) {
+        if (count != 1 || argmax)
+            return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "rows of %u codes at M = %u are split over K parts: one matrix, no fused argmax",
+                        w[0].k, m);
+        if (mi355q_status st = ensure_workspace(ctx, (size_t)g.parts * m * w[0].n * sizeof(float))) return st;
+        a.partial = (float*)ctx->workspace;
+    }
     a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = w[0].sb_dtype;
     const int mr = m == 1 ? 1 : m == 2 ? 2 : 4;
     if (argmax) {
@@ -423,9 +501,14 @@ mi355q_status launch_gemv_tile16_multi(hipStream_t s, const mi355q_context* ctx,
         if (mi355q_status st = launch_t16_shape<1, true>(s, a, g)) return st;
         return launch_argmax_finish(s, argmax_scratch, g.grid, token_out);
     }
-    if (mr == 1) return launch_t16_shape<1, false>(s, a, g);
-    if (mr == 2) return launch_t16_shape<2, false>(s, a, g);
-    return launch_t16_shape<4, false>(s, a, g);
+    mi355q_status st = mr == 1 ? launch_t16_shape<1, false>(s, a, g)
+                     : mr == 2 ? launch_t16_shape<2, false>(s, a, g) : launch_t16_shape<4, false>(s, a, g);
+    if (st != MI355Q_OK || g.parts == 1) return st;
+    const uint32_t cells = m * w[0].n;
+    tile16_sum_parts_kernel<<<dim3((cells + 255) / 256), dim3(256), 0, s>>>(a.partial, g.parts, m, w[0].n, y[0],
+                                                                            y_strides[0], (uint32_t)y_dtype, logits_f32);
+    MI355Q_HIP(hipGetLastError());
+    return MI355Q_OK;
 }
 
 }  // namespace mi355q

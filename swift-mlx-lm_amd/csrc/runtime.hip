@@ -10,14 +10,17 @@ namespace mi355q {
 
 mi355q_status ensure_workspace(mi355q_context* ctx, size_t bytes) {
     if (bytes <= ctx->workspace_bytes) return MI355Q_OK;
-    // launches that still read the old buffer must drain before it is released
-    MI355Q_HIP(hipDeviceSynchronize());
-    if (ctx->workspace) (void)hipFree(ctx->workspace);
-    ctx->workspace = nullptr;
-    ctx->workspace_bytes = 0;
-    const size_t rounded = (bytes + ((size_t)1 << 22) - 1) & ~(((size_t)1 << 22) - 1);
-    MI355Q_HIP(hipMalloc(&ctx->workspace, rounded));
-    ctx->workspace_bytes = rounded;
+    // A launch recorded in a HIP graph keeps the address it was captured with, so an outgrown buffer stays allocated
+    // until the context goes; growth at least doubles, which bounds the retired buffers to the size of the live one.
+    size_t want = bytes > 2 * ctx->workspace_bytes ? bytes : 2 * ctx->workspace_bytes;
+    want = (want + ((size_t)1 << 22) - 1) & ~(((size_t)1 << 22) - 1);
+    if (ctx->workspace && ctx->retired_count >= kRetiredWorkspaces)
+        return fail(MI355Q_ERR_OUT_OF_MEMORY, "scratch buffer outgrown %d times", kRetiredWorkspaces);
+    void* grown = nullptr;
+    MI355Q_HIP(hipMalloc(&grown, want));
+    if (ctx->workspace) ctx->retired[ctx->retired_count++] = ctx->workspace;
+    ctx->workspace = grown;
+    ctx->workspace_bytes = want;
     return MI355Q_OK;
 }
 
@@ -235,6 +238,7 @@ mi355q_status mi355q_context_destroy(mi355q_context* ctx) {
     if (ctx->argmax_scratch) (void)hipFree(ctx->argmax_scratch);
     if (ctx->argmax_partials) (void)hipFree(ctx->argmax_partials);
     if (ctx->workspace) (void)hipFree(ctx->workspace);
+    for (int i = 0; i < ctx->retired_count; i++) (void)hipFree(ctx->retired[i]);
     delete ctx;
     return MI355Q_OK;
 }

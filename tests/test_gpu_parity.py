@@ -355,6 +355,7 @@ def test_launch_argument_errors(pkg, ctx):
     assert status(ctx.qgemm, w, x, pkg.BF16, y, pkg.F32, 16, 0, 0, pkg.FLAG_FORCE_MFMA | pkg.FLAG_FORCE_GENERIC) \
         == "INVALID_ARGUMENT"
     assert status(ctx.batched_qgemm, [w], x, pkg.BF16, [y], pkg.F32, 1) == "KERNEL_NOT_FOUND"   # count 1
+    assert status(ctx.argmax, x, pkg.F32, 0, y) == "SHAPE"                                 # empty vector
     assert status(ctx.weight_prepare_mlx, fmt, np.zeros((2, 4), np.uint32), np.zeros((2, 1), np.uint16),
                   np.zeros((2, 1), np.uint16), pkg.BF16) == "SHAPE"                          # K=32 < group
     assert status(ctx.weight_prepare_staf, fmt, 2, 64, np.zeros(71, np.uint8)) == "SIZE_MISMATCH"

@@ -76,8 +76,6 @@ def test_tile16_llama_shapes_all_batch_sizes(pkg, ctx, name):
     words, s, z, wq = seeded_case(2100 + n % 89, n, k, 4, 64)
     w = ctx.weight_prepare_mlx(_fmt(pkg), words, s, z, pkg.BF16, pkg.LAYOUT_TILE16)
     for m in (1, 2, 3, 4, 5, 8, 13, 16):
-        if m * (k * 2 + 16) > 144 * 1024:
-            continue                                           # runs as several launches: covered below
         x = act_rounded(kat.seeded_activations(2200 + m, m, k), pkg.BF16, pkg)
         say(f"tile16 {name} M={m}")
         want = oracle.gemm_f64(wq, x)
@@ -115,6 +113,81 @@ def test_tile16_ragged_shapes_and_long_batches(pkg, ctx):
         x = act_rounded(kat.seeded_activations(2500 + m, m, k), pkg.BF16, pkg)
         assert_within_tolerance(_run(ctx, pkg, w, x, pkg.F32), oracle.gemm_f64(wq, x), f"f16 scales M={m}")
     w.destroy()
+
+
+def test_tile16_long_rows_split_over_k_parts(pkg, ctx):
+    """Rows too long for M staged activation rows in LDS (14336 codes from M = 5, 65536 codes at M = 1) run as one
+    launch whose workgroups each take a part of K, plus a launch that adds the parts: every output type, strided
+    rows, ragged N, agreement with the per-code kernel, the plan record, and replay from a HIP graph."""
+    for i, (n, k) in enumerate([(4096, 14336), (50, 14336), (33, 65536)]):
+        words, s, z, wq = seeded_case(2600 + i, n, k, 4, 64)
+        w = ctx.weight_prepare_mlx(_fmt(pkg), words, s, z, pkg.BF16, pkg.LAYOUT_TILE16)
+        for m in ((5, 8, 13, 16) if k == 14336 else (1, 2, 16)):
+            x = act_rounded(kat.seeded_activations(2650 + i + m, m, k), pkg.BF16, pkg)
+            say(f"tile16 K parts {k}->{n} M={m}")
+            st = w.plan_prefill_steps(m)[0] if m > 1 else w.plan_decode_step(1)
+            assert st.device_kernel == "gemv_tile16_q4_g64" and not st.used_fallback and st.lds_bytes <= 144 * 1024
+            want = oracle.gemm_f64(wq, x)
+            y32 = _run(ctx, pkg, w, x, pkg.F32, use_qgemm=True)
+            rel, _ = assert_within_tolerance(y32, want, f"{k}->{n} M={m}")
+            assert rel < 1e-4
+            assert np.array_equal(oracle.bf16_from_f32(_run(ctx, pkg, w, x, pkg.BF16, use_qgemm=True)), oracle.bf16_from_f32(y32))
+            if n <= 50:
+                y16 = _run(ctx, pkg, w, x, pkg.F16, use_qgemm=True)
+                assert np.array_equal(y16.astype(np.float16), y32.astype(np.float16))
+                assert_within_tolerance(_run(ctx, pkg, w, x, pkg.F32, True, pkg.FLAG_FORCE_GENERIC), want, "per-code kernel")
+        w.destroy()
+    # strided activation and output rows, then the same projection from a plan and its graph, three replays; on a
+    # context of its own, so that the scratch buffer of partial results starts small and a later, larger user of it
+    # (a split-K prefill projection) makes it grow while the graph still holds the address it was captured with
+    c2 = pkg.Context(0)
+    n, k, m, xs, ys = 200, 14336, 16, 14336 + 64, 200 + 24
+    words, s, z, wq = seeded_case(2690, n, k, 4, 64)
+    w = c2.weight_prepare_mlx(_fmt(pkg), words, s, z, pkg.BF16, pkg.LAYOUT_TILE16)
+    x = act_rounded(kat.seeded_activations(2691, m, k), pkg.BF16, pkg)
+    xh = np.zeros((m, xs), np.uint16); xh[:, :k] = oracle.bf16_from_f32(x).reshape(m, k)
+    xd = c2.upload(xh); yd = c2.alloc(m * ys * 4)
+    c2.fill(yd, 0x7FC00000)
+    c2.qgemm(w, xd, pkg.BF16, yd, pkg.F32, m, xs, ys); c2.synchronize()
+    got = yd.download(np.float32, (m, ys))
+    assert_within_tolerance(got[:, :n], oracle.gemm_f64(wq, x), "strided rows")
+    assert np.isnan(got[:, n:]).all()                         # nothing written between the rows
+    plan = pkg.DispatchPlan(c2)
+    plan.add_linear(w, xd, pkg.BF16, yd, pkg.F32, m, xs, ys)
+    stream = c2.stream_create()
+    plan.graph_build(stream)
+    rng = np.random.default_rng(2692)
+    for rep in range(4):
+        if rep == 3:
+            nb, mb = 4096, 2048
+            wb = c2.weight_prepare_mlx(_fmt(pkg), rng.integers(0, 2**32, (nb, k // 8), dtype=np.uint32),
+                                       np.full((nb, k // 64), 0x3C00, np.uint16), np.zeros((nb, k // 64), np.uint16), pkg.F16)
+            xb = c2.alloc(mb * k * 2); yb = c2.alloc(mb * nb * 2)
+            c2.fill(xb, 0x3C003C00)
+            say("tile16 K parts: a split-K prefill projection grows the scratch buffer")
+            c2.qgemm(wb, xb, pkg.BF16, yb, pkg.BF16, mb); c2.synchronize()
+            xb.free(); yb.free(); wb.destroy()
+        c2.fill(yd, 0x7FC00000, stream)
+        plan.graph_launch(stream) if rep else plan.encode(stream)
+        c2.synchronize(stream)
+        again = yd.download(np.float32, (m, ys))
+        assert np.array_equal(again[:, :n], got[:, :n]) and np.isnan(again[:, n:]).all(), rep
+    plan.destroy(); xd.free(); yd.free(); w.destroy(); c2.close()
+    # two long-row projections of one activation batch: no fused launch, each runs split, results as above
+    ws, wqs = [], []
+    for j, n2 in enumerate((48, 130)):
+        words, s, z, wq = seeded_case(2695 + j, n2, 14336, 4, 64)
+        ws.append(ctx.weight_prepare_mlx(_fmt(pkg), words, s, z, pkg.BF16, pkg.LAYOUT_TILE16)); wqs.append(wq)
+    x = act_rounded(kat.seeded_activations(2697, 8, 14336), pkg.BF16, pkg)
+    xd = ctx.upload(oracle.bf16_from_f32(x).reshape(x.shape)); yds = [ctx.alloc(8 * n2 * 4) for n2 in (48, 130)]
+    ctx.batched_qgemm(ws, xd, pkg.BF16, yds, pkg.F32, 8); ctx.synchronize()
+    for j, n2 in enumerate((48, 130)):
+        assert_within_tolerance(yds[j].download(np.float32, (8, n2)), oracle.gemm_f64(wqs[j], x), f"batched long rows {j}")
+    xd.free()
+    for b in yds:
+        b.free()
+    for w2 in ws:
+        w2.destroy()
 
 
 def test_tile16_exact_small_integers_and_scaling(pkg, ctx):
