@@ -244,7 +244,7 @@ def main():
                 pool = [{name: ctx.weight_prepare_mlx(fmt, *host[name], pkg.BF16, layout) for name, _, _ in LAYER_SHAPES}
                         for _ in range(n_t16)]
             batch_sweep[lname] = {}
-            for m in (1, 2, 4, 8):
+            for m in ((1, 2, 4, 8) if lname == "planes" else (1, 2, 4, 8, 16)):    # the tile kernel takes 16 rows a launch
                 xm = {k: ctx.alloc(m * k * 2) for k in (4096, 14336)}
                 for k in xm:
                     ctx.fill(xm[k], 0x3C003C00, stream)
