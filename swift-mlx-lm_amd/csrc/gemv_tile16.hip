@@ -367,6 +367,13 @@ mi355q_status launch_t16_shape(hipStream_t s, const T16Args& a, const Tile16Laun
     if (ks == 4 && tpw == 1) return launch_t16<MR, 4, 1, ARGMAX>(s, a, g.grid, g.lds_bytes);
     if (ks == 4 && tpw == 2) return launch_t16<MR, 4, 2, ARGMAX>(s, a, g.grid, g.lds_bytes);
     if (ks == 4 && tpw == 4) return launch_t16<MR, 4, 4, ARGMAX>(s, a, g.grid, g.lds_bytes);
+    if constexpr (!ARGMAX && MR == 4) {   // one round of workgroups with a CU's share of row tiles each (M >= 3)
+        if (ks == 4 && tpw == 3) return launch_t16<MR, 4, 3, false>(s, a, g.grid, g.lds_bytes);
+        if (ks == 2 && tpw == 5) return launch_t16<MR, 2, 5, false>(s, a, g.grid, g.lds_bytes);
+        if (ks == 2 && tpw == 6) return launch_t16<MR, 2, 6, false>(s, a, g.grid, g.lds_bytes);
+        if (ks == 2 && tpw == 7) return launch_t16<MR, 2, 7, false>(s, a, g.grid, g.lds_bytes);
+        if (ks == 2 && tpw == 8) return launch_t16<MR, 2, 8, false>(s, a, g.grid, g.lds_bytes);
+    }
     if (ks == 8 && tpw == 1) return launch_t16<MR, 8, 1, ARGMAX>(s, a, g.grid, g.lds_bytes);
     if (ks == 8 && tpw == 2) return launch_t16<MR, 8, 2, ARGMAX>(s, a, g.grid, g.lds_bytes);
     if (ks == 16 && tpw == 1) return launch_t16<MR, 16, 1, ARGMAX>(s, a, g.grid, g.lds_bytes);
@@ -414,8 +421,17 @@ Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_row_ti
     // per CU they take four row tiles at a time (each wavefront keeps a quarter of K: long enough a stream to fill
     // its prefetch ring) and walk further tiles in passes; with fewer, all sixteen share one row tile.
     const bool big_x = (size_t)m * ((size_t)k * 2 + 16) > 80 * 1024;
-    const bool one_wg_per_cu = big_x && n_total_tiles >= 3 * cus;
-    if (one_wg_per_cu) {
+    // From three activation rows and three row tiles per CU on, exactly one round of workgroups: each takes its CU's
+    // share of the row tiles at once when sixteen wavefronts can hold them two or four to a tile (28672 rows at M = 8,
+    // seven tiles per CU: 21.4 us as 4 x 4 wavefronts walking two passes on 224 CUs, 17.4 us as 2 x 7 on all 256; M = 4:
+    // 18.8 -> 16.3 us), else four tiles at a time in passes.
+    const uint32_t tiles_per_cu = (n_total_tiles + cus - 1) / cus;
+    const bool balanced = m >= 3 && n_total_tiles >= 3 * cus && tiles_per_cu <= 8;
+    const bool one_wg_per_cu = balanced || (big_x && n_total_tiles >= 3 * cus);
+    if (balanced) {
+        tpw = tiles_per_cu;
+        ks = tpw <= 4 ? 4 : 2;
+    } else if (one_wg_per_cu) {
         ks = 4;
         tpw = 4;
     } else if (big_x) {

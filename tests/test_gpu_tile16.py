@@ -115,6 +115,27 @@ def test_tile16_ragged_shapes_and_long_batches(pkg, ctx):
     w.destroy()
 
 
+@pytest.mark.parametrize("tiles_per_cu", [3, 5, 6, 7, 8])
+def test_tile16_one_round_workgroup_shapes(pkg, ctx, tiles_per_cu):
+    """From three activation rows on, a matrix with three to eight row tiles per CU runs as one round of workgroups that
+    each take their CU's share of row tiles (4 x 3, 2 x 5 ... 2 x 8 wavefronts): every such shape, ragged last tile,
+    K of one and of several blocks per wavefront, single and fused launches."""
+    cus = ctx.device_info().compute_units
+    # just past (tiles_per_cu - 1) tiles per CU with a ragged last tile; three per CU exist only as exactly 3 x CUs tiles
+    n = 16 * cus * 3 if tiles_per_cu == 3 else 16 * (cus * (tiles_per_cu - 1) + 3) + 5
+    for k in (128, 1280):
+        words, s, z, wq = seeded_case(2800 + tiles_per_cu + k, n, k, 4, 64)
+        w = ctx.weight_prepare_mlx(_fmt(pkg), words, s, z, pkg.BF16, pkg.LAYOUT_TILE16)
+        for m in (3, 8, 16):
+            st = w.plan_prefill_steps(m)[0]
+            assert st.device_kernel == "gemv_tile16_q4_g64" and st.grid[0] <= cus, (st.grid[0], cus)
+            assert st.block[0] == 64 * tiles_per_cu * (4 if tiles_per_cu <= 4 else 2), st.block[0]
+            x = act_rounded(kat.seeded_activations(2850 + m, m, k), pkg.BF16, pkg)
+            say(f"tile16 one round, {tiles_per_cu} tiles per CU, K={k} M={m}")
+            assert_within_tolerance(_run(ctx, pkg, w, x, pkg.F32, use_qgemm=True), oracle.gemm_f64(wq, x), f"{tiles_per_cu} K={k} M={m}")
+        w.destroy()
+
+
 def test_tile16_long_rows_split_over_k_parts(pkg, ctx):
     """Rows too long for M staged activation rows in LDS (14336 codes from M = 5, 65536 codes at M = 1) run as one
     launch whose workgroups each take a part of K, plus a launch that adds the parts: every output type, strided
