@@ -51,7 +51,6 @@ struct T16Args {
     uint32_t kblocks;                            // K / 128
     uint32_t parts;                              // K parts, each with workgroups of its own that stage only their columns
     uint32_t part_blocks;                        // K-blocks per part (kblocks / parts)
-    uint32_t wgs_per_part;                       // workgroups of one part: blockIdx.x = part * wgs_per_part + index
     uint32_t blocks_per_wave;                    // K-blocks per wavefront (K split over the workgroup)
     uint32_t passes;                             // row tiles a wavefront walks, one after the other, on one staged copy of x
     uint32_t lds_row_bytes;                      // part_blocks*256 + 16: staged activation row pitch
@@ -72,8 +71,9 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t n_in = lane & 15, kq = lane >> 4;
     // K part of this workgroup: K-blocks [kb0, kb0 + part_blocks), activation columns [kb0 * 128, ...)
-    const uint32_t part = a.parts > 1 ? blockIdx.x / a.wgs_per_part : 0u;
-    const uint32_t wg = blockIdx.x - part * a.wgs_per_part;
+    // (the part is the grid's second dimension: nothing is loaded or divided before the first weight loads go out)
+    const uint32_t part = blockIdx.y;
+    const uint32_t wg = blockIdx.x;
     const uint32_t kb0 = part * a.part_blocks;
     const uint32_t kp = a.part_blocks * 128;                // activation elements this workgroup stages per row
 
@@ -352,11 +352,11 @@ uint32_t t16_parts(uint32_t k, uint32_t m, uint32_t n_row_tiles, uint32_t cus) {
 }
 
 template <int MR, int KSPLIT, int TPW, bool ARGMAX>
-mi355q_status launch_t16(hipStream_t s, const T16Args& a, uint32_t grid, size_t lds) {
+mi355q_status launch_t16(hipStream_t s, const T16Args& a, uint32_t grid, size_t lds) {   // grid: workgroups of one K part
     auto kern = gemv_tile16_kernel<MR, KSPLIT, TPW, 4, ARGMAX>;
     if (lds > 64 * 1024)
         MI355Q_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    kern<<<dim3(grid), dim3(KSPLIT * TPW * 64), lds, s>>>(a);
+    kern<<<dim3(grid, a.parts), dim3(KSPLIT * TPW * 64), lds, s>>>(a);
     MI355Q_HIP(hipGetLastError());
     return MI355Q_OK;
 }
@@ -364,19 +364,19 @@ mi355q_status launch_t16(hipStream_t s, const T16Args& a, uint32_t grid, size_t 
 template <int MR, bool ARGMAX>
 mi355q_status launch_t16_shape(hipStream_t s, const T16Args& a, const Tile16LaunchShape& g) {
     const uint32_t ks = g.ksplit, tpw = g.tiles_per_wg;
-    if (ks == 4 && tpw == 1) return launch_t16<MR, 4, 1, ARGMAX>(s, a, g.grid, g.lds_bytes);
-    if (ks == 4 && tpw == 2) return launch_t16<MR, 4, 2, ARGMAX>(s, a, g.grid, g.lds_bytes);
-    if (ks == 4 && tpw == 4) return launch_t16<MR, 4, 4, ARGMAX>(s, a, g.grid, g.lds_bytes);
+    if (ks == 4 && tpw == 1) return launch_t16<MR, 4, 1, ARGMAX>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 4 && tpw == 2) return launch_t16<MR, 4, 2, ARGMAX>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 4 && tpw == 4) return launch_t16<MR, 4, 4, ARGMAX>(s, a, g.wgs_per_part, g.lds_bytes);
     if constexpr (!ARGMAX && MR == 4) {   // one round of workgroups with a CU's share of row tiles each (M >= 3)
-        if (ks == 4 && tpw == 3) return launch_t16<MR, 4, 3, false>(s, a, g.grid, g.lds_bytes);
-        if (ks == 2 && tpw == 5) return launch_t16<MR, 2, 5, false>(s, a, g.grid, g.lds_bytes);
-        if (ks == 2 && tpw == 6) return launch_t16<MR, 2, 6, false>(s, a, g.grid, g.lds_bytes);
-        if (ks == 2 && tpw == 7) return launch_t16<MR, 2, 7, false>(s, a, g.grid, g.lds_bytes);
-        if (ks == 2 && tpw == 8) return launch_t16<MR, 2, 8, false>(s, a, g.grid, g.lds_bytes);
+        if (ks == 4 && tpw == 3) return launch_t16<MR, 4, 3, false>(s, a, g.wgs_per_part, g.lds_bytes);
+        if (ks == 2 && tpw == 5) return launch_t16<MR, 2, 5, false>(s, a, g.wgs_per_part, g.lds_bytes);
+        if (ks == 2 && tpw == 6) return launch_t16<MR, 2, 6, false>(s, a, g.wgs_per_part, g.lds_bytes);
+        if (ks == 2 && tpw == 7) return launch_t16<MR, 2, 7, false>(s, a, g.wgs_per_part, g.lds_bytes);
+        if (ks == 2 && tpw == 8) return launch_t16<MR, 2, 8, false>(s, a, g.wgs_per_part, g.lds_bytes);
     }
-    if (ks == 8 && tpw == 1) return launch_t16<MR, 8, 1, ARGMAX>(s, a, g.grid, g.lds_bytes);
-    if (ks == 8 && tpw == 2) return launch_t16<MR, 8, 2, ARGMAX>(s, a, g.grid, g.lds_bytes);
-    if (ks == 16 && tpw == 1) return launch_t16<MR, 16, 1, ARGMAX>(s, a, g.grid, g.lds_bytes);
+    if (ks == 8 && tpw == 1) return launch_t16<MR, 8, 1, ARGMAX>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 8 && tpw == 2) return launch_t16<MR, 8, 2, ARGMAX>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 16 && tpw == 1) return launch_t16<MR, 16, 1, ARGMAX>(s, a, g.wgs_per_part, g.lds_bytes);
     return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no TILE16 variant for K-split %u x %u tiles per workgroup", ks, tpw);
 }
 
@@ -497,7 +497,6 @@ mi355q_status launch_gemv_tile16_multi(hipStream_t s, mi355q_context* ctx, uint3
     a.kblocks = w[0].k / 128;
     a.parts = g.parts;
     a.part_blocks = a.kblocks / g.parts;
-    a.wgs_per_part = g.wgs_per_part;
     a.blocks_per_wave = g.blocks_per_wave;
     a.passes = g.passes;
     a.lds_row_bytes = a.part_blocks * 256 + 16;
