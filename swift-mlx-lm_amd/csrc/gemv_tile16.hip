@@ -435,8 +435,14 @@ Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_row_ti
         ks = 4;
         tpw = 4;
     } else if (big_x) {
-        tpw = 1;
-        while (ks < 16 && kblocks / (ks * 2) >= 2) ks *= 2;
+        // one workgroup per CU and fewer than three row tiles per CU: all sixteen wavefronts on one row tile, or on the
+        // two or three a CU gets, so that the launch stays one round and the activations are staged once per CU
+        // (q+k+v 4096 -> 6144 at M = 16, 1.5 tiles per CU: 16.8 us with one tile per workgroup, 9.9 us with two)
+        tpw = tiles_per_cu < 3 || m < 3 ? (tiles_per_cu > 1 ? 2u : 1u) : 3u;
+        const uint32_t most_ks = tpw == 1 ? 16u : tpw == 2 ? 8u : 4u;
+        ks = tpw == 3 ? 4u : ks;
+        while (ks < most_ks && kblocks / (ks * 2) >= 2) ks *= 2;
+        if (ks > most_ks) ks = most_ks;
     }
     const int eks = env_int_cached("MI355Q_T16_KSPLIT", 0), etpw = env_int_cached("MI355Q_T16_TPW", 0);
     if (eks) ks = (uint32_t)eks;

@@ -136,6 +136,23 @@ def test_tile16_one_round_workgroup_shapes(pkg, ctx, tiles_per_cu):
         w.destroy()
 
 
+def test_tile16_large_batch_few_tiles_per_cu(pkg, ctx):
+    """Sixteen activation rows of 4096 (131 KB staged, one workgroup per CU) over matrices with one, two and three row
+    tiles per CU: sixteen wavefronts on one row tile, 8 x 2 and 4 x 3."""
+    cus = ctx.device_info().compute_units
+    k, m = 4096, 16
+    for i, tiles in enumerate((cus - 3, cus + cus // 2, 2 * cus + 9)):
+        n = 16 * tiles - 7
+        words, s, z, wq = seeded_case(2880 + i, n, k, 4, 64)
+        w = ctx.weight_prepare_mlx(_fmt(pkg), words, s, z, pkg.BF16, pkg.LAYOUT_TILE16)
+        st = w.plan_prefill_steps(m)[0]
+        assert st.device_kernel == "gemv_tile16_q4_g64" and st.grid[0] <= cus and st.block[0] == (1024, 1024, 768)[i], (st.grid[0], st.block[0])
+        x = act_rounded(kat.seeded_activations(2885 + i, m, k), pkg.BF16, pkg)
+        say(f"tile16 M=16, {tiles} row tiles on {cus} CUs")
+        assert_within_tolerance(_run(ctx, pkg, w, x, pkg.F32, use_qgemm=True), oracle.gemm_f64(wq, x), f"{tiles} tiles")
+        w.destroy()
+
+
 def test_tile16_long_rows_split_over_k_parts(pkg, ctx):
     """Rows too long for M staged activation rows in LDS (14336 codes from M = 5, 65536 codes at M = 1) run as one
     launch whose workgroups each take a part of K, plus a launch that adds the parts: every output type, strided
