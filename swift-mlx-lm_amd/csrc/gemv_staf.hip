@@ -84,11 +84,19 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_staf_kernel(const StafArgs a)
     // its end: their loads are clamped and nothing is stored
     const uint32_t gw = blockIdx.x * WAVES + wave;
     const uint32_t seg = gw < a.wave_end[0] ? 0u : (gw < a.wave_end[1] ? 1u : 2u);
-    const uint32_t first_wave = seg == 0 ? 0u : a.wave_end[seg - 1];
-    const uint8_t* const seg_blocks = seg == 0 ? a.blocks[0] : (seg == 1 ? a.blocks[1] : a.blocks[2]);
-    void* const seg_y = seg == 0 ? a.y[0] : (seg == 1 ? a.y[1] : a.y[2]);
-    const uint32_t seg_n = seg == 0 ? a.seg_rows[0] : (seg == 1 ? a.seg_rows[1] : a.seg_rows[2]);
-    const uint32_t seg_ys = seg == 0 ? a.y_stride[0] : (seg == 1 ? a.y_stride[1] : a.y_stride[2]);
+    // Mask arithmetic over all three entries instead of a select: a select of kernel-argument fields becomes one
+    // scalar load from a selected address, which waits for the load of wave_end first -- a second trip to the constant
+    // cache in front of the first weight loads.
+    const uint32_t k0 = seg == 0 ? ~0u : 0u, k1 = seg == 1 ? ~0u : 0u, k2 = seg == 2 ? ~0u : 0u;
+    const uint64_t q0 = seg == 0 ? ~0ull : 0ull, q1 = seg == 1 ? ~0ull : 0ull, q2 = seg == 2 ? ~0ull : 0ull;
+    const uint32_t first_wave = (a.wave_end[0] & k1) | (a.wave_end[1] & k2);
+    const uint8_t* const seg_blocks =
+        (const uint8_t*)(((uintptr_t)a.blocks[0] & q0) | ((uintptr_t)a.blocks[1] & q1) | ((uintptr_t)a.blocks[2] & q2));
+    void* const seg_y = (void*)(((uintptr_t)a.y[0] & q0) | ((uintptr_t)a.y[1] & q1) | ((uintptr_t)a.y[2] & q2));
+    const uint32_t seg_n = (a.seg_rows[0] & k0) | (a.seg_rows[1] & k1) | (a.seg_rows[2] & k2);
+    const uint32_t seg_ys = (a.y_stride[0] & k0) | (a.y_stride[1] & k1) | (a.y_stride[2] & k2);
+    // the remaining arguments of the prologue, asked for here so that they arrive with the same batch of scalar loads
+    asm volatile("" ::"s"(a.row_bytes), "s"(a.rows_per_wave), "s"(a.rows_per_span), "s"(a.blocks_per_row), "s"(a.m), "s"(a.x), "s"(a.x_stride));
     const uint64_t last_chunk = (uint64_t)seg_n * a.row_bytes - 16;    // last whole 16-byte chunk of the matrix
     const uint32_t row0 = gw < a.wave_end[kGemvMaxSegments - 1] ? (gw - first_wave) * a.rows_per_wave : seg_n;
     // Short rows share a span: RPS consecutive rows (contiguous in memory) fill the 64 lanes, lane l holding block

@@ -46,15 +46,15 @@ struct T16Args {
     float* logits;                               // optional fp32 [N] copy (M == 1, one matrix)
     int32_t* token_out;                          // ARGMAX only
     unsigned long long* scratch;                 // ARGMAX only: one packed key per workgroup; 0 = no candidate
-    float* partial;                              // K parts only: fp32 partial results [part][M][N] (one matrix)
     uint32_t k, m, x_stride;
     uint32_t kblocks;                            // K / 128
-    uint32_t parts;                              // K parts, each with workgroups of its own that stage only their columns
-    uint32_t part_blocks;                        // K-blocks per part (kblocks / parts)
     uint32_t blocks_per_wave;                    // K-blocks per wavefront (K split over the workgroup)
     uint32_t passes;                             // row tiles a wavefront walks, one after the other, on one staged copy of x
     uint32_t lds_row_bytes;                      // part_blocks*256 + 16: staged activation row pitch
     uint32_t y_dtype, sb_dtype;
+    uint32_t parts;                              // K parts, each with workgroups of its own that stage only their columns
+    uint32_t part_blocks;                        // K-blocks per part (kblocks / parts)
+    float* partial;                              // K parts only: fp32 partial results [part][M][N] (one matrix)
 };
 
 constexpr int kT16RecordWords = 288;             // 1152 bytes
