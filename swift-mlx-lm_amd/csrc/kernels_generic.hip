@@ -249,20 +249,25 @@ __global__ __launch_bounds__(256) void dequant_bf16_kernel(WView w, uint16_t* __
 // Eight consecutive codes per thread: one or two 32-bit loads of codes (a run of 8 codes starts on a
 // byte boundary and spans at most 64 bits for every width), one scale/zero pair (groups are multiples
 // of 8 codes), one 128-bit store.  Same arithmetic as the per-element kernel above.
+// BITS is a template argument (constant shifts on the 64-bit field) and the grid is two-dimensional -- x over the
+// 8-code chunks of a row, y over rows -- so that no thread divides a 64-bit index: with run-time width and a flat index
+// the kernel was bound by its integer arithmetic (42 us for 4096 -> 14336, against 26 us for a plain copy of as many bytes).
+template <int BITS>
 __global__ __launch_bounds__(256) void dequant_bf16_x8_kernel(WView w, uint16_t* __restrict__ out) {
-    const uint32_t per_row = w.k >> 3;
-    const uint64_t total = (uint64_t)w.n * per_row;
-    const uint32_t mask = (1u << w.bits) - 1u;
-    for (uint64_t t = (uint64_t)blockIdx.x * 256 + threadIdx.x; t < total; t += (uint64_t)gridDim.x * 256) {
-        const uint32_t row = (uint32_t)(t / per_row), c0 = (uint32_t)(t - (uint64_t)row * per_row) << 3;
+    const uint32_t c0 = (blockIdx.x * 256 + threadIdx.x) << 3;
+    if (c0 >= w.k) return;
+    constexpr uint32_t mask = (1u << BITS) - 1u;
+    const uint32_t g = c0 / w.group;
+#pragma unroll 2
+    for (uint32_t row = blockIdx.y; row < w.n; row += gridDim.y) {
         const uint64_t v = load_codes8(w, row, c0);
         float scale, zero;
-        load_scale_zero(w, row, c0 / w.group, scale, zero);
+        load_scale_zero(w, row, g, scale, zero);
         uint32_t o[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const float q0 = (float)((uint32_t)(v >> ((2 * i) * w.bits)) & mask);
-            const float q1 = (float)((uint32_t)(v >> ((2 * i + 1) * w.bits)) & mask);
+            const float q0 = (float)((uint32_t)(v >> ((2 * i) * BITS)) & mask);
+            const float q1 = (float)((uint32_t)(v >> ((2 * i + 1) * BITS)) & mask);
             const uint32_t lo = f32_to_bf16_rne(__fadd_rn(__fmul_rn(scale, q0), zero));
             const uint32_t hi = f32_to_bf16_rne(__fadd_rn(__fmul_rn(scale, q1), zero));
             o[i] = lo | (hi << 16);
@@ -275,11 +280,19 @@ __global__ __launch_bounds__(256) void dequant_bf16_x8_kernel(WView w, uint16_t*
 
 mi355q_status launch_dequant_bf16(hipStream_t s, const WView& w, uint16_t* out) {
     if (w.k % 8 == 0 && (uintptr_t)out % 16 == 0) {
-        const uint64_t tasks = (uint64_t)w.n * (w.k / 8);
-        uint64_t blocks = (tasks + 255) / 256;
-        if (blocks > (1u << 20)) blocks = 1u << 20;
-        if (blocks == 0) blocks = 1;
-        dequant_bf16_x8_kernel<<<dim3((unsigned)blocks), dim3(256), 0, s>>>(w, out);
+        // two to four rows per thread, at most 65535 workgroups along y
+        uint32_t gy = w.n > 4096 ? (w.n + 3) / 4 : (w.n + 1) / 2;
+        if (gy > 65535u) gy = 65535u;
+        const dim3 grid((w.k / 8 + 255) / 256, gy), block(256);
+        switch (w.bits) {
+        case 2: dequant_bf16_x8_kernel<2><<<grid, block, 0, s>>>(w, out); break;
+        case 3: dequant_bf16_x8_kernel<3><<<grid, block, 0, s>>>(w, out); break;
+        case 4: dequant_bf16_x8_kernel<4><<<grid, block, 0, s>>>(w, out); break;
+        case 5: dequant_bf16_x8_kernel<5><<<grid, block, 0, s>>>(w, out); break;
+        case 6: dequant_bf16_x8_kernel<6><<<grid, block, 0, s>>>(w, out); break;
+        case 8: dequant_bf16_x8_kernel<8><<<grid, block, 0, s>>>(w, out); break;
+        default: return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no dequantisation kernel for %u-bit codes", w.bits);
+        }
     } else {
         unsigned blocks = w.n < 65535u * 16u ? w.n : 65535u * 16u;
         dequant_bf16_kernel<<<dim3(blocks), dim3(256), 0, s>>>(w, out);
