@@ -163,16 +163,17 @@ __global__ __launch_bounds__(256) void embedding_lookup_kernel(WView w, const in
 }
 
 // The same lookup with eight consecutive dimensions per thread (one or two code loads, one scale/zero
-// pair, 128-bit stores): the variant for rows of whole 8-code runs and 16-byte aligned output rows.
+// pair, 128-bit stores): the variant for rows of whole 8-code runs and 16-byte aligned output rows.  The grid is
+// (chunks of a row) x (positions) and the bit width a template argument: no 64-bit division, constant shifts.
+template <int BITS>
 __global__ __launch_bounds__(256) void embedding_lookup_x8_kernel(WView w, const int32_t* __restrict__ token_ids,
                                                                   uint32_t sequence_length, void* __restrict__ out,
                                                                   uint32_t out_dtype, uint32_t out_stride, int has_scale,
                                                                   float embedding_scale) {
-    const uint32_t per_row = w.k >> 3;
-    const uint64_t total = (uint64_t)sequence_length * per_row;
-    const uint32_t mask = (1u << w.bits) - 1u;
-    for (uint64_t t = (uint64_t)blockIdx.x * 256 + threadIdx.x; t < total; t += (uint64_t)gridDim.x * 256) {
-        const uint32_t pos = (uint32_t)(t / per_row), d0 = (uint32_t)(t - (uint64_t)pos * per_row) << 3;
+    constexpr uint32_t mask = (1u << BITS) - 1u;
+    const uint32_t d0 = (blockIdx.x * 256 + threadIdx.x) << 3;
+    if (d0 >= w.k) return;
+    for (uint32_t pos = blockIdx.y; pos < sequence_length; pos += gridDim.y) {
         const int32_t tok = token_ids[pos];
         float f[8];
 #pragma unroll
@@ -183,7 +184,7 @@ __global__ __launch_bounds__(256) void embedding_lookup_x8_kernel(WView w, const
             load_scale_zero(w, (uint32_t)tok, d0 / w.group, scale, zero);
 #pragma unroll
             for (int i = 0; i < 8; i++) {
-                const float q = (float)((uint32_t)(v >> (i * w.bits)) & mask);
+                const float q = (float)((uint32_t)(v >> (i * BITS)) & mask);
                 f[i] = __fadd_rn(__fmul_rn(q, scale), zero);
                 if (has_scale) f[i] = __fmul_rn(f[i], embedding_scale);
             }
@@ -213,12 +214,18 @@ mi355q_status launch_embedding_lookup(hipStream_t s, const WView& w, const int32
                                       float embedding_scale) {
     const size_t esz = out_dtype == MI355Q_F32 ? 4 : 2;
     if (w.k % 8 == 0 && (uintptr_t)out % 16 == 0 && ((size_t)out_stride * esz) % 16 == 0) {
-        const uint64_t tasks = (uint64_t)sequence_length * (w.k / 8);
-        uint64_t blocks = (tasks + 255) / 256;
-        if (blocks > (1u << 20)) blocks = 1u << 20;
-        if (blocks == 0) blocks = 1;
-        embedding_lookup_x8_kernel<<<dim3((unsigned)blocks), dim3(256), 0, s>>>(
-            w, token_ids, sequence_length, out, (uint32_t)out_dtype, out_stride, has_scale, embedding_scale);
+        const dim3 grid((w.k / 8 + 255) / 256, sequence_length < 65535u ? sequence_length : 65535u), block(256);
+#define MI355Q_EMBED_CASE(B)                                                                                        \
+    case B:                                                                                                         \
+        embedding_lookup_x8_kernel<B><<<grid, block, 0, s>>>(w, token_ids, sequence_length, out, (uint32_t)out_dtype, \
+                                                             out_stride, has_scale, embedding_scale);               \
+        break;
+        switch (w.bits) {
+            MI355Q_EMBED_CASE(2) MI355Q_EMBED_CASE(3) MI355Q_EMBED_CASE(4) MI355Q_EMBED_CASE(5) MI355Q_EMBED_CASE(6)
+            MI355Q_EMBED_CASE(8)
+        default: return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no embedding kernel for %u-bit codes", w.bits);
+        }
+#undef MI355Q_EMBED_CASE
     } else {
         uint32_t gx = (w.k + 255u) / 256u;
         if (gx > 64u) gx = 64u;
