@@ -311,18 +311,19 @@ __global__ __launch_bounds__(256) void tile16_sum_parts_kernel(const float* __re
                                                                uint32_t m, uint32_t n, void* __restrict__ y,
                                                                uint32_t y_stride, uint32_t y_dtype,
                                                                float* __restrict__ logits) {
-    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
-    if (i >= m * n) return;
-    const uint32_t row = i / n, col = i - row * n;
-    float v = 0.f;
-    for (uint32_t p = 0; p < parts; p++) v += partial[((size_t)p * m + row) * n + col];
-    if (y) {
-        const size_t o = (size_t)row * y_stride + col;
-        if (y_dtype == MI355Q_F32) ((float*)y)[o] = v;
-        else if (y_dtype == MI355Q_BF16) ((uint16_t*)y)[o] = f32_to_bf16_rne(v);
-        else ((uint16_t*)y)[o] = f32_to_f16_rne(v);
+    // x over the columns of an activation row, y over the (at most 16) rows
+    const uint32_t row = blockIdx.y;
+    for (uint32_t col = blockIdx.x * 256 + threadIdx.x; col < n; col += gridDim.x * 256) {
+        float v = 0.f;
+        for (uint32_t p = 0; p < parts; p++) v += partial[((size_t)p * m + row) * n + col];
+        if (y) {
+            const size_t o = (size_t)row * y_stride + col;
+            if (y_dtype == MI355Q_F32) ((float*)y)[o] = v;
+            else if (y_dtype == MI355Q_BF16) ((uint16_t*)y)[o] = f32_to_bf16_rne(v);
+            else ((uint16_t*)y)[o] = f32_to_f16_rne(v);
+        }
+        if (logits && row == 0) logits[col] = v;
     }
-    if (logits && row == 0) logits[col] = v;
 }
 
 namespace {
@@ -533,8 +534,9 @@ mi355q_status launch_gemv_tile16_multi(hipStream_t s, mi355q_context* ctx, uint3
     mi355q_status st = mr == 1 ? launch_t16_shape<1, false>(s, a, g)
                      : mr == 2 ? launch_t16_shape<2, false>(s, a, g) : launch_t16_shape<4, false>(s, a, g);
     if (st != MI355Q_OK || g.parts == 1) return st;
-    const uint32_t cells = m * w[0].n;
-    tile16_sum_parts_kernel<<<dim3((cells + 255) / 256), dim3(256), 0, s>>>(a.partial, g.parts, m, w[0].n, y[0],
+    uint32_t sum_wgs = (w[0].n + 255) / 256;
+    if (sum_wgs > 65535u) sum_wgs = 65535u;
+    tile16_sum_parts_kernel<<<dim3(sum_wgs, m), dim3(256), 0, s>>>(a.partial, g.parts, m, w[0].n, y[0],
                                                                             y_strides[0], (uint32_t)y_dtype, logits_f32);
     MI355Q_HIP(hipGetLastError());
     return MI355Q_OK;
