@@ -413,13 +413,13 @@ Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_row_ti
     // long rows: at most 16 K-blocks per wavefront (28672 -> 8192 at M = 1: 48 us with a four-way split, 30 us
     // with sixteen; 14336 -> 4096: 13.2 / 9.4 us), which leaves the four-way split to rows of up to 8192 codes
     while (ks < 16 && kblocks / ks > 16) ks *= 2;
-    // Two row tiles per workgroup up to four activation rows, four above: at one row only while that leaves a
-    // workgroup and a half per CU (4096 -> 14336 at M = 1: 8.99 -> 8.36 us), for batches while it leaves one per two
-    // CUs.  A matrix with at most one row tile per CU keeps one tile per workgroup and, when every wavefront still
-    // gets two K-blocks (four up to M = 2), all sixteen wavefronts on it (14336 -> 4096 at M = 2: 12.3 -> 10.5 us;
+    // One row tile per workgroup at one activation row (two pay on 4096 -> 14336 alone, 8.99 -> 8.36 us, and cost the
+    // fused gate+up launch as much: 15.0 -> 16.0 us), two up to four rows, four above, while that leaves a workgroup
+    // per two CUs.  A matrix with at most one row tile per CU keeps one tile per workgroup and, when every wavefront
+    // still gets two K-blocks (four up to M = 2), all sixteen wavefronts on it (14336 -> 4096 at M = 2: 12.3 -> 10.5 us;
     // 4096 -> 4096: M = 2 5.8 -> 5.1 us with eight, M = 4 6.5 -> 6.2 us, M = 8 7.6 -> 7.2 us with sixteen).
-    const uint32_t want_tpw = m <= 4 ? 2u : 4u;
-    const uint32_t least_wgs = m == 1 ? cus + cus / 2 : cus / 2;
+    const uint32_t want_tpw = m == 1 ? 1u : m <= 4 ? 2u : 4u;
+    const uint32_t least_wgs = cus / 2;
     uint32_t tpw = 1;
     while (tpw < want_tpw && ks * tpw * 2 <= 16 && (n_total_tiles + tpw * 2 - 1) / (tpw * 2) >= least_wgs) tpw *= 2;
     if (n_total_tiles <= cus) {
