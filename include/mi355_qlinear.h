@@ -250,7 +250,11 @@ MI355Q_API mi355q_status mi355q_qgemv(mi355q_context* ctx, void* stream, const m
  * as ONE fused kernel: code tiles are dequantised to bf16 in LDS and contracted on MFMA with
  * fp32 accumulation.  Any M >= 1; M is a run-time value (the reference rebinds sequenceLength
  * per call, MC/Compiler/MetalPrefillStepBuilder.swift:728-732).  Small M routes to the
- * GEMV-style kernel unless flags say otherwise. */
+ * GEMV-style kernel unless flags say otherwise.  Launches that split K over workgroups (few output
+ * tiles at short M; on the TILE16 layout, rows too long for M staged activation rows) keep fp32
+ * partial results in a scratch buffer of the context, grown on first use: two such launches of one
+ * context must not overlap on different streams, and the first one of a size allocates (run a plan
+ * once before capturing it, as mi355q_plan_graph_build does). */
 MI355Q_API mi355q_status mi355q_qgemm(mi355q_context* ctx, void* stream, const mi355q_weight* w,
                                       const void* x_dev, mi355q_dtype x_dtype, void* y_dev,
                                       mi355q_dtype y_dtype, uint32_t m, uint32_t x_row_stride,
