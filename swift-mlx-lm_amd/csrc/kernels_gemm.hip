@@ -416,7 +416,23 @@ GemmLaunchShape gemm_mfma_shape(const mi355q_context* ctx, uint32_t m, uint32_t 
     auto tiles = [&](uint32_t bm, uint32_t bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
     GemmLaunchShape g{};
     int pick = env_int_cached("MI355Q_GEMM_TILE", 0);
-    if (pick == 0) pick = (m > 128 && 10 * tiles(256, 256) >= 9 * cus) ? 5 : 3;
+    const uint32_t kt = k / kTileK;
+    // 256 x 256 tiles on eight wavefronts when they fill the chip, alone or with K split so that tiles x splits comes
+    // to about one workgroup per CU and a split keeps sixteen K-tiles (M = 2048, 14336 -> 4096: 128 tiles, 333 us
+    // as 512 tiles of 128 x 128, 236 us as 128 x 2; M = 1024: 204 -> 131 us as 64 x 4; 4096 -> 14336 at M = 1024:
+    // 171 -> 126 us as 224 x 1); else 128 x 128 tiles, split over K when they leave half the CUs idle.
+    uint32_t wide_splits = 0;
+    if (pick == 0) {
+        const uint32_t t256 = tiles(256, 256);
+        if (m > 128 && 10 * t256 >= 9 * cus) {
+            pick = 5;
+        } else if (m >= 256) {
+            uint32_t sp = cus / t256;
+            while (sp > 1 && kt / sp < 16) sp--;
+            if (sp >= 1 && t256 * sp * 4 >= cus * 3) { pick = 5; wide_splits = sp; }
+        }
+        if (pick == 0) pick = 3;
+    }
     if (pick == 1) { g.bm = 256; g.bn = 256; g.stages = 2; }
     else if (pick == 5) { g.bm = 256; g.bn = 256; g.stages = 2; g.block = 512; }
     else if (pick == 2) { g.bm = 256; g.bn = 128; g.stages = 1; }
@@ -426,8 +442,7 @@ GemmLaunchShape gemm_mfma_shape(const mi355q_context* ctx, uint32_t m, uint32_t 
     if (!g.block) g.block = 256;
     // K is split over workgroups when the tiles alone leave most CUs idle (short M): each split writes
     // an fp32 partial, a second launch adds them.  At least 8 K-tiles per split.
-    g.splits = 1;
-    const uint32_t kt = k / kTileK;
+    g.splits = wide_splits ? wide_splits : 1;
     if (g.bm == 128 && tiles(128, 128) * 2 <= cus) {
         uint32_t want = (2 * cus) / tiles(128, 128);
         if (want > 16) want = 16;
