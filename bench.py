@@ -484,6 +484,21 @@ def main():
             f"(bf16 MFMA peak 2500 at 2.4 GHz); constant activations: {prefill['constant_activations']['TFLOPs']} TFLOP/s "
             f"at {ghz_c:.3f} GHz")
         xg.free(); yg.free()
+        # benchmark config 3: both MLP shapes at M = 128, 512, 2048 (as dispatched: tile shape and K split are the library's choice)
+        sweep = {}
+        for name, n, k in (("gate 4096->14336", 14336, 4096), ("down 14336->4096", 4096, 14336)):
+            wts = [L["gate" if n == 14336 else "down"] for L in layers[:4]]
+            for mm in (128, 512, 2048):
+                xb = ctx.alloc(mm * k * 2); yb = ctx.alloc(mm * n * 2)
+                ctx.fill(xb, 0x3C003C00, stream)
+                ctx.qgemm(wts[0], xb, pkg.BF16, yb, pkg.BF16, mm, 0, 0, 0, stream)
+                ctx.synchronize(stream)
+                ms = time_region(ctx, lambda i: ctx.qgemm(wts[i % len(wts)], xb, pkg.BF16, yb, pkg.BF16, mm, 0, 0, 0, stream), 8, stream)
+                sweep[f"{name} M={mm}"] = {"us": round(ms * 1e3, 1), "TFLOPs": round(2.0 * mm * n * k / (ms * 1e-3) / 1e12, 1)}
+                xb.free(); yb.free()
+        sweep["activations"] = "constant (the part clocks higher on them than on N(0,1) data: compare the two M=2048 gate figures above)"
+        prefill["config3"] = sweep
+        log("  prefill sweep: " + ", ".join(f"{k2} {v['us']} us" for k2, v in sweep.items() if isinstance(v, dict)))
 
     cpu = None if a.no_cpu else cpu_baseline(a.cpu_seconds)
 
