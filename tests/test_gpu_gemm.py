@@ -181,6 +181,16 @@ def test_config3_prefill_gate_up_and_down(pkg, ctx, m, n, k):
     assert rel < 5e-4
 
 
+def test_mfma_gemm_wide_tiles_with_k_split_ragged(pkg, ctx):
+    """Shapes whose 256 x 256 tiles alone leave CUs idle run with K split over workgroups (fp32 partials, then a sum
+    launch): M and N off the tile grid, padded output rows, 4- and 8-bit codes."""
+    for i, (m, n, k, bits, group, y_pad) in enumerate([(333, 14330, 4096, 4, 64, 0), (300, 7001, 4096, 8, 32, 3),
+                                                       (1000, 4100, 4096, 4, 64, 0)]):
+        fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(bits, group)
+        sample = _tile_edge_sample(n, 990 + i, per_tile=1, tile=256)
+        _seeded_gemm(pkg, ctx, 970 + i, m, n, k, bits, group, sample=sample, y_pad=y_pad)
+
+
 def test_mfma_gemm_many_tiles_ragged_last_column_tile(pkg, ctx):
     """2048 x 14286: more 256 x 256 tiles than CUs (two rounds), the last column tile cut at column 14286,
     padded output rows."""
