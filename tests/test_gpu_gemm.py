@@ -186,7 +186,6 @@ def test_mfma_gemm_wide_tiles_with_k_split_ragged(pkg, ctx):
     launch): M and N off the tile grid, padded output rows, 4- and 8-bit codes."""
     for i, (m, n, k, bits, group, y_pad) in enumerate([(333, 14330, 4096, 4, 64, 0), (300, 7001, 4096, 8, 32, 3),
                                                        (1000, 4100, 4096, 4, 64, 0)]):
-        fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(bits, group)
         sample = _tile_edge_sample(n, 990 + i, per_tile=1, tile=256)
         _seeded_gemm(pkg, ctx, 970 + i, m, n, k, bits, group, sample=sample, y_pad=y_pad)
 
