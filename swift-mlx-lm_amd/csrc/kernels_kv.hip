@@ -134,6 +134,55 @@ __global__ __launch_bounds__(256) void kv_cache_write_hd128_kernel(KvArgs a) {
     else block[4 + (i >> 1)] = (uint8_t)(q0 | (q1 << 4));
 }
 
+// Head vectors of 128 elements, four per lane: a wavefront quantises two vectors (one per half), a lane reads its
+// four elements with one load and writes its four codes with one store, and a group's minimum and maximum are
+// taken inside the run of group/4 lanes that holds it.  Same operations per element again, so the same bytes.
+__global__ __launch_bounds__(256) void kv_cache_write_hd128x4_kernel(KvArgs a) {
+    const uint32_t lane = threadIdx.x & 63, l = lane & 31;
+    const uint32_t total = a.count * a.kv_heads;
+    const uint32_t v_raw = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 2 + (lane >> 5);
+    const bool live = v_raw < total;                      // the last wavefront may hold a single vector
+    const uint32_t v = live ? v_raw : total - 1;          // its other half repeats that vector and stores nothing
+    const uint32_t p = v / a.kv_heads, h = v - p * a.kv_heads;
+    uint8_t* slot = a.cache + kv_slot_offset(a, h, a.first_position + p);
+    const size_t src0 = (size_t)p * a.row_stride + (size_t)h * 128u + 4u * l;
+    float x[4];
+    if (a.dtype == MI355Q_F32) {
+        const float4 t = *(const float4*)((const float*)a.src + src0);
+        x[0] = t.x; x[1] = t.y; x[2] = t.z; x[3] = t.w;
+    } else {
+        const uint2 t = *(const uint2*)((const uint16_t*)a.src + src0);
+        if (a.dtype == MI355Q_BF16) {
+            x[0] = __uint_as_float(t.x << 16); x[1] = __uint_as_float(t.x & 0xFFFF0000u);
+            x[2] = __uint_as_float(t.y << 16); x[3] = __uint_as_float(t.y & 0xFFFF0000u);
+        } else {
+            x[0] = f16_to_f32((uint16_t)(t.x & 0xFFFFu)); x[1] = f16_to_f32((uint16_t)(t.x >> 16));
+            x[2] = f16_to_f32((uint16_t)(t.y & 0xFFFFu)); x[3] = f16_to_f32((uint16_t)(t.y >> 16));
+        }
+    }
+    float lo = fminf(fminf(x[0], x[1]), fminf(x[2], x[3])), hi = fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3]));
+    for (uint32_t o = a.group >> 3; o >= 1; o >>= 1) {    // group / 4 lanes hold one group
+        lo = fminf(lo, __shfl_xor(lo, (int)o));
+        hi = fmaxf(hi, __shfl_xor(hi, (int)o));
+    }
+    const float levels = a.bits == 8 ? 255.0f : 15.0f;
+    const int top = a.bits == 8 ? 255 : 15;
+    float scale = __fdiv_rn(__fsub_rn(hi, lo), levels);
+    if (scale < 1e-10f) scale = 1e-10f;
+    const uint32_t d = 4u * l, g = d / a.group, i = d - g * a.group;
+    uint8_t* block = slot + (size_t)g * a.bytes_per_block;
+    if (!live) return;
+    if (i == 0) *(uint32_t*)block = (uint32_t)f32_to_f16_rne(scale) | ((uint32_t)f32_to_f16_rne(lo) << 16);
+    uint32_t q[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const int c = (int)roundf(__fdiv_rn(__fsub_rn(x[e], lo), scale));
+        q[e] = (uint32_t)(c < 0 ? 0 : c > top ? top : c);
+    }
+    if (a.bits == 8) *(uint32_t*)(block + 4 + i) = q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24);
+    else *(uint16_t*)(block + 4 + (i >> 1)) = (uint16_t)(q[0] | (q[1] << 4) | (q[2] << 8) | (q[3] << 12));
+}
+
 // One thread per element of the output rows.
 __global__ __launch_bounds__(256) void kv_cache_read_kernel(KvArgs a) {
     const uint32_t row_elems = a.kv_heads * a.head_dim;
@@ -157,6 +206,48 @@ __global__ __launch_bounds__(256) void kv_cache_read_kernel(KvArgs a) {
         if (a.dtype == MI355Q_F32) ((float*)a.out)[o] = x;
         else if (a.dtype == MI355Q_BF16) ((uint16_t*)a.out)[o] = f32_to_bf16_rne(x);
         else ((uint16_t*)a.out)[o] = f32_to_f16_rne(x);
+    }
+}
+
+// Quantized slots, four consecutive elements of a head vector per thread (they share a group: groups and head
+// dimensions are multiples of four here): one 32- or 16-bit load of codes, one header, one 8- or 16-byte store.
+// Same arithmetic per element as the kernel above.
+__global__ __launch_bounds__(256) void kv_cache_read_x4_kernel(KvArgs a) {
+    const uint32_t row_elems = a.kv_heads * a.head_dim;
+    const uint32_t p = blockIdx.y;
+    for (uint32_t e = (blockIdx.x * 256 + threadIdx.x) * 4; e < row_elems; e += gridDim.x * 1024) {
+        const uint32_t h = e / a.head_dim, d = e - h * a.head_dim;
+        const uint8_t* slot = a.cache + kv_slot_offset(a, h, a.first_position + p);
+        const uint8_t* block = slot + (size_t)(d / a.group) * a.bytes_per_block;
+        const uint32_t i = d % a.group;
+        const uint32_t hdr = *(const uint32_t*)block;
+        const float scale = f16_to_f32((uint16_t)(hdr & 0xFFFFu)), zero = f16_to_f32((uint16_t)(hdr >> 16));
+        uint32_t q[4];
+        if (a.bits == 8) {
+            const uint32_t w = *(const uint32_t*)(block + 4 + i);
+            q[0] = w & 0xFFu; q[1] = (w >> 8) & 0xFFu; q[2] = (w >> 16) & 0xFFu; q[3] = w >> 24;
+        } else {
+            const uint32_t w = *(const uint16_t*)(block + 4 + (i >> 1));
+            q[0] = w & 0xFu; q[1] = (w >> 4) & 0xFu; q[2] = (w >> 8) & 0xFu; q[3] = (w >> 12) & 0xFu;
+        }
+        float x[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) x[j] = __fadd_rn(__fmul_rn(scale, (float)q[j]), zero);
+        const size_t o = (size_t)p * a.row_stride + e;
+        if (a.dtype == MI355Q_F32) {
+            float4 t; t.x = x[0]; t.y = x[1]; t.z = x[2]; t.w = x[3];
+            *(float4*)((float*)a.out + o) = t;
+        } else {
+            uint2 t;
+            if (a.dtype == MI355Q_BF16) {
+                t.x = (uint32_t)f32_to_bf16_rne(x[0]) | ((uint32_t)f32_to_bf16_rne(x[1]) << 16);
+                t.y = (uint32_t)f32_to_bf16_rne(x[2]) | ((uint32_t)f32_to_bf16_rne(x[3]) << 16);
+            } else {
+                t.x = (uint32_t)f32_to_f16_rne(x[0]) | ((uint32_t)f32_to_f16_rne(x[1]) << 16);
+                t.y = (uint32_t)f32_to_f16_rne(x[2]) | ((uint32_t)f32_to_f16_rne(x[3]) << 16);
+            }
+            *(uint2*)((uint16_t*)a.out + o) = t;
+        }
     }
 }
 
@@ -243,7 +334,12 @@ mi355q_status mi355q_kv_cache_write(mi355q_context* ctx, void* stream, const mi3
     const size_t esz = a.dtype == MI355Q_F32 ? 4 : 2;
     const bool two_per_lane = a.bits != 0 && a.head_dim == 128 && a.row_stride % 2 == 0 &&
                               (uintptr_t)src_dev % (2 * esz) == 0 && (a.group == 32 || a.group == 64 || a.group == 128);
-    if (two_per_lane)
+    // four per lane needs 8- or 16-byte loads of the source and 4-byte aligned slots
+    const bool four_per_lane = two_per_lane && a.row_stride % 4 == 0 && (uintptr_t)src_dev % (4 * esz) == 0 &&
+                               a.slot_bytes % 4 == 0 && (uintptr_t)a.cache % 4 == 0;
+    if (four_per_lane)
+        kv_cache_write_hd128x4_kernel<<<dim3((unsigned)((vectors + 7) / 8)), dim3(256), 0, (hipStream_t)stream>>>(a);
+    else if (two_per_lane)
         kv_cache_write_hd128_kernel<<<dim3((unsigned)((vectors + 3) / 4)), dim3(256), 0, (hipStream_t)stream>>>(a);
     else
         kv_cache_write_kernel<<<dim3((unsigned)((vectors + 3) / 4)), dim3(256), 0, (hipStream_t)stream>>>(a);
@@ -259,6 +355,18 @@ mi355q_status mi355q_kv_cache_read(mi355q_context* ctx, void* stream, const mi35
                                       sequence_length, &a)) return st;
     a.out = out_dev;
     const uint32_t row = a.kv_heads * a.head_dim;
+    const size_t esz = a.dtype == MI355Q_F32 ? 4 : 2;
+    // four elements per thread: whole groups of four, 4-byte aligned slots and blocks, 8- or 16-byte aligned output rows
+    const bool four = a.bits != 0 && a.head_dim % 4 == 0 && a.group % 4 == 0 && a.slot_bytes % 4 == 0 &&
+                      a.bytes_per_block % 4 == 0 && (uintptr_t)a.cache % 4 == 0 && a.row_stride % 4 == 0 &&
+                      (uintptr_t)out_dev % (4 * esz) == 0;
+    if (four) {
+        uint32_t bx = (row / 4 + 255) / 256;
+        if (bx > 64) bx = 64;
+        kv_cache_read_x4_kernel<<<dim3(bx, a.count), dim3(256), 0, (hipStream_t)stream>>>(a);
+        MI355Q_HIP(hipGetLastError());
+        return MI355Q_OK;
+    }
     uint32_t bx = (row + 255) / 256;
     if (bx > 64) bx = 64;
     kv_cache_read_kernel<<<dim3(bx, a.count), dim3(256), 0, (hipStream_t)stream>>>(a);

@@ -55,8 +55,11 @@ def test_kv_cache_bytes_bit_exact(pkg, ctx, scheme):
             (pkg.KV_HEAD_MAJOR, 3, 80, 16, 3, 5, pkg.BF16),          # head dimension ends inside a group
             (pkg.KV_SEQUENCE_MAJOR, 1, 7, 4, 0, 4, pkg.F32),         # shorter than any group, odd
             (pkg.KV_HEAD_MAJOR, 4, 128, 32, 5, 9, pkg.F32),          # 128-element heads from fp32 rows
-            (pkg.KV_SEQUENCE_MAJOR, 4, 128, 32, 0, 6, pkg.BF16)]):   # the same with an odd row stride
-        pad = {1: 8, 6: 7}.get(i, 0)
+            (pkg.KV_SEQUENCE_MAJOR, 4, 128, 32, 0, 6, pkg.BF16),     # the same with an odd row stride
+            (pkg.KV_SEQUENCE_MAJOR, 3, 128, 16, 2, 5, pkg.BF16),     # an odd number of 128-element vectors
+            (pkg.KV_HEAD_MAJOR, 3, 128, 16, 0, 7, pkg.F16),          # row stride a multiple of two, not of four
+            (pkg.KV_HEAD_MAJOR, 1, 128, 8, 0, 1, pkg.F32)]):         # a single vector
+        pad = {1: 8, 6: 7, 8: 2}.get(i, 0)
         x, back = _roundtrip(pkg, ctx, scheme, layout, heads, hd, max_pos, first, count, dt, 100 * scheme + i, pad=pad)
         if scheme in (0x10, 0x11, 0x12):
             assert np.max(np.abs(back - x)) <= 0.51 * 8 * 30 / 255 + 0.02 * np.max(np.abs(x))
