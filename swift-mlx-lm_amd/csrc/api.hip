@@ -59,7 +59,7 @@ mi355q_status run_small_m(mi355q_context* ctx, hipStream_t s, const mi355q_weigh
             const uint32_t strides[1] = {ys};
             st = launch_gemv_tile16_multi(s, ctx, 1, &v, xp, yv, strides, y_dtype, mm, xs, nullptr, nullptr, nullptr);
         } else if (!generic && gemv_fast_eligible(v, x_dtype, mm, xs) && (uintptr_t)xp % 16 == 0) {
-            st = launch_gemv_fast(s, ctx, v, xp, yp, y_dtype, mm, xs, ys, nullptr, nullptr, nullptr);
+            st = launch_gemv_fast(s, ctx, v, xp, x_dtype, yp, y_dtype, mm, xs, ys, nullptr, nullptr, nullptr);
         } else if (!generic && gemv_staf_eligible(v, x_dtype, mm, xs) && (uintptr_t)xp % 16 == 0) {
             st = launch_gemv_staf(s, ctx, v, xp, yp, y_dtype, mm, xs, ys);
         } else {
@@ -145,7 +145,7 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
         in_place = in_place && gemv_staf_eligible(views[i], x_dtype, m, xs);
     }
     if (fused && (uintptr_t)x % 16 == 0)
-        return launch_gemv_fast_multi(s, ctx, count, views, x, ys, strides, y_dtype, m, xs, nullptr, nullptr, nullptr);
+        return launch_gemv_fast_multi(s, ctx, count, views, x, x_dtype, ys, strides, y_dtype, m, xs, nullptr, nullptr, nullptr);
     if (tiled && (uintptr_t)x % 16 == 0)
         return launch_gemv_tile16_multi(s, ctx, count, views, x, ys, strides, y_dtype, m, xs, nullptr, nullptr,
                                         nullptr);
@@ -165,7 +165,7 @@ mi355q_status dispatch_output_head(mi355q_context* ctx, hipStream_t s, const mi3
     const WView v = w->view();
     const uint32_t xs = (uint32_t)w->k;
     if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && gemv_fast_eligible(v, x_dtype, 1, xs) && (uintptr_t)x % 16 == 0)
-        return launch_gemv_fast(s, ctx, v, x, nullptr, MI355Q_F32, 1, xs, (uint32_t)w->n, logits, token,
+        return launch_gemv_fast(s, ctx, v, x, x_dtype, nullptr, MI355Q_F32, 1, xs, (uint32_t)w->n, logits, token,
                                 ctx->argmax_partials);
     if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && gemv_tile16_eligible(v, x_dtype, 1, xs) && gemv_tile16_k_parts(ctx, v, 1) == 1 &&
         (uintptr_t)x % 16 == 0) {

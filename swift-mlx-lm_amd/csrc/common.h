@@ -135,7 +135,7 @@ mi355q_status launch_pack_sz(hipStream_t s, const uint16_t* scales, const uint16
 // Fast split-plane GEMV (kernels_gemv.hip).  can_* say whether a shape is eligible.
 bool gemv_fast_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
 mi355q_status launch_gemv_fast(hipStream_t s, const mi355q_context* ctx, const WView& w,
-                               const void* x, void* y, int y_dtype, uint32_t m,
+                               const void* x, int x_dtype, void* y, int y_dtype, uint32_t m,
                                uint32_t x_stride, uint32_t y_stride, float* logits_f32,
                                int32_t* token_out, unsigned long long* argmax_scratch);
 // Block-layout GEMV (gemv_staf.hip): reads STAF interleaved blocks in place.
@@ -151,10 +151,10 @@ struct GemvLaunchShape {
     const char* kernel;
 };
 GemvLaunchShape gemv_staf_shape(const mi355q_context* ctx, const WView& w, uint32_t m);
-GemvLaunchShape gemv_fast_shape(const mi355q_context* ctx, const WView& w, uint32_t m);
+GemvLaunchShape gemv_fast_shape(const mi355q_context* ctx, const WView& w, uint32_t m, int x_dtype);
 
 mi355q_status launch_gemv_fast_multi(hipStream_t s, const mi355q_context* ctx, uint32_t count, const WView* w,
-                                     const void* x, void* const* y, const uint32_t* y_strides, int y_dtype,
+                                     const void* x, int x_dtype, void* const* y, const uint32_t* y_strides, int y_dtype,
                                      uint32_t m, uint32_t x_stride, float* logits_f32, int32_t* token_out,
                                      unsigned long long* argmax_scratch);
 

@@ -1,49 +1,40 @@
 // Instantiates the split-plane GEMV kernels for one bit width (QBITS) and exports one launcher.
 // Included by gemv_q{2,3,4,5,6,8}.hip so that the widths compile in parallel.
-#include "gemv_planes.inl"
+#include "gemv_rows.inl"
 
 namespace mi355q {
 
 namespace {
 
-template <int BITS, int GROUP, int R, int MT, bool ARGMAX, int WAVES, int D, int XREG>
-mi355q_status launch_one(hipStream_t s, const GemvArgs& a, uint32_t grid, size_t lds) {
-    auto kern = gemv_planes_kernel<BITS, GROUP, R, MT, ARGMAX, WAVES, D, XREG>;
+template <typename K>
+mi355q_status launch_kernel(K kern, hipStream_t s, const GemvArgs& a, uint32_t grid, uint32_t block, size_t lds) {
     if (lds > 64 * 1024) {
         // opt in to more than the default 64 KiB of dynamic LDS (gfx950 has 160 KiB per CU)
         MI355Q_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     }
-    kern<<<dim3(grid), dim3(WAVES * 64), lds, s>>>(a);
+    kern<<<dim3(grid), dim3(block), lds, s>>>(a);
     MI355Q_HIP(hipGetLastError());
     return MI355Q_OK;
 }
 
+// ---- the general kernel (any row length, small batches) ---------------------------------------------------
+template <int BITS, int GROUP, int R, int MT, bool ARGMAX, int WAVES, int D, int XREG>
+mi355q_status launch_one(hipStream_t s, const GemvArgs& a, const GemvCfg& c) {
+    if (c.xa) return launch_kernel(gemv_planes_kernel<BITS, GROUP, R, MT, ARGMAX, WAVES, D, XREG, 1>, s, a, c.grid, WAVES * 64, c.lds);
+    return launch_kernel(gemv_planes_kernel<BITS, GROUP, R, MT, ARGMAX, WAVES, D, XREG, 0>, s, a, c.grid, WAVES * 64, c.lds);
+}
+
 #define MI355Q_TRY(R_, MT_, AM_, WV_, D_, XR_)                                                            \
     if (c.r == R_ && c.mt == MT_ && c.argmax == AM_ && c.waves == WV_ && c.depth == D_ && c.xreg == XR_) \
-        return launch_one<BITS, GROUP, R_, MT_, AM_, WV_, D_, XR_>(s, a, c.grid, c.lds);
+        return launch_one<BITS, GROUP, R_, MT_, AM_, WV_, D_, XR_>(s, a, c);
 
 template <int BITS, int GROUP>
-mi355q_status launch_group(hipStream_t s, const GemvArgs& a, const GemvCfg& c) {
-#ifdef MI355Q_GEMV_EXPERIMENT
-    // tuning build: the (R, waves, depth, xreg) grid for one format
-    MI355Q_TRY(1, 1, false, 4, 2, 0) MI355Q_TRY(1, 1, false, 4, 4, 0) MI355Q_TRY(1, 1, false, 4, 8, 0)
-    MI355Q_TRY(2, 1, false, 4, 2, 0) MI355Q_TRY(2, 1, false, 4, 4, 0) MI355Q_TRY(2, 1, false, 4, 8, 0)
-    MI355Q_TRY(1, 1, false, 8, 2, 0) MI355Q_TRY(1, 1, false, 8, 4, 0) MI355Q_TRY(1, 1, false, 8, 8, 0)
-    MI355Q_TRY(2, 1, false, 8, 2, 0) MI355Q_TRY(2, 1, false, 8, 4, 0) MI355Q_TRY(2, 1, false, 8, 8, 0)
-    MI355Q_TRY(1, 1, false, 16, 2, 0) MI355Q_TRY(1, 1, false, 16, 4, 0) MI355Q_TRY(1, 1, false, 16, 8, 0)
-    MI355Q_TRY(1, 1, false, 4, 2, 1) MI355Q_TRY(1, 1, false, 4, 4, 1) MI355Q_TRY(1, 1, false, 4, 8, 1)
-    MI355Q_TRY(1, 1, false, 4, 2, 2) MI355Q_TRY(1, 1, false, 4, 4, 2) MI355Q_TRY(1, 1, false, 4, 8, 2)
-    MI355Q_TRY(1, 1, false, 8, 2, 1) MI355Q_TRY(1, 1, false, 8, 4, 1) MI355Q_TRY(1, 1, false, 8, 8, 1)
-    MI355Q_TRY(1, 1, false, 8, 2, 2) MI355Q_TRY(1, 1, false, 8, 4, 2) MI355Q_TRY(1, 1, false, 8, 8, 2)
-    MI355Q_TRY(1, 1, false, 16, 2, 1) MI355Q_TRY(1, 1, false, 16, 4, 1) MI355Q_TRY(1, 1, false, 16, 8, 1)
-    MI355Q_TRY(1, 1, false, 16, 2, 2) MI355Q_TRY(1, 1, false, 16, 4, 2) MI355Q_TRY(1, 1, false, 16, 8, 2)
-#else
+mi355q_status launch_general(hipStream_t s, const GemvArgs& a, const GemvCfg& c) {
     // M == 1 (decode): register-resident activations for rows of one K-step, LDS-resident otherwise
     MI355Q_TRY(1, 1, false, 4, 2, 1) MI355Q_TRY(1, 1, false, 4, 4, 1)
     MI355Q_TRY(1, 1, false, 4, 2, 0) MI355Q_TRY(1, 1, false, 4, 4, 0)
     MI355Q_TRY(1, 1, false, 8, 2, 0) MI355Q_TRY(1, 1, false, 8, 4, 0)
     MI355Q_TRY(1, 1, false, 16, 2, 0) MI355Q_TRY(1, 1, false, 16, 4, 0)
-#endif
     // the same with the fused arg-max tail (LM head)
     MI355Q_TRY(1, 1, true, 4, 2, 1) MI355Q_TRY(1, 1, true, 4, 4, 1)
     MI355Q_TRY(1, 1, true, 4, 2, 0) MI355Q_TRY(1, 1, true, 4, 4, 0)
@@ -59,6 +50,54 @@ mi355q_status launch_group(hipStream_t s, const GemvArgs& a, const GemvCfg& c) {
 }
 
 #undef MI355Q_TRY
+
+// ---- the static-structure kernel (M == 1, rows of 1, 2, 3, 4 or 7 K-steps) -----------------------------------
+template <int BITS, int GROUP, int NCT, int BR, int WAVES>
+mi355q_status launch_rows(hipStream_t s, const GemvArgs& a, const GemvCfg& c) {
+    const bool sbbf = a.sb_dtype == MI355Q_BF16;
+    const uint32_t block = WAVES * 64;
+    if (c.argmax) {
+        if constexpr (gemv_rows_has_argmax(NCT, BR)) {
+            if (c.xa) {
+                if constexpr (gemv_rows_has_f16(BITS, GROUP)) {
+                    if (sbbf) return launch_kernel(gemv_rows_kernel<BITS, GROUP, NCT, BR, WAVES, 1, true, true>, s, a, c.grid, block, c.lds);
+                    return launch_kernel(gemv_rows_kernel<BITS, GROUP, NCT, BR, WAVES, 1, false, true>, s, a, c.grid, block, c.lds);
+                }
+            } else {
+                if (sbbf) return launch_kernel(gemv_rows_kernel<BITS, GROUP, NCT, BR, WAVES, 0, true, true>, s, a, c.grid, block, c.lds);
+                return launch_kernel(gemv_rows_kernel<BITS, GROUP, NCT, BR, WAVES, 0, false, true>, s, a, c.grid, block, c.lds);
+            }
+        }
+        return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no fused arg-max variant of the row kernel for q%d g%d steps=%d rows=%d", BITS, GROUP, NCT, BR);
+    }
+    if (c.xa) {
+        if constexpr (gemv_rows_has_f16(BITS, GROUP)) {
+            if (sbbf) return launch_kernel(gemv_rows_kernel<BITS, GROUP, NCT, BR, WAVES, 1, true, false>, s, a, c.grid, block, c.lds);
+            return launch_kernel(gemv_rows_kernel<BITS, GROUP, NCT, BR, WAVES, 1, false, false>, s, a, c.grid, block, c.lds);
+        }
+        return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no f16 variant of the row kernel for q%d g%d", BITS, GROUP);
+    }
+    if (sbbf) return launch_kernel(gemv_rows_kernel<BITS, GROUP, NCT, BR, WAVES, 0, true, false>, s, a, c.grid, block, c.lds);
+    return launch_kernel(gemv_rows_kernel<BITS, GROUP, NCT, BR, WAVES, 0, false, false>, s, a, c.grid, block, c.lds);
+}
+
+#define MI355Q_TRY_ROWS(NCT_, BR_) \
+    if (c.nct == NCT_ && c.br == BR_) return launch_rows<BITS, GROUP, NCT_, BR_, gemv_rows_waves(NCT_)>(s, a, c);
+
+template <int BITS, int GROUP>
+mi355q_status launch_group(hipStream_t s, const GemvArgs& a, const GemvCfg& c) {
+    if (!c.rows) return launch_general<BITS, GROUP>(s, a, c);
+    if constexpr (gemv_rows_has_format(BITS, GROUP)) {
+        MI355Q_TRY_ROWS(1, 1) MI355Q_TRY_ROWS(1, 2) MI355Q_TRY_ROWS(1, 4) MI355Q_TRY_ROWS(1, 8)
+        MI355Q_TRY_ROWS(2, 1) MI355Q_TRY_ROWS(2, 2) MI355Q_TRY_ROWS(2, 4)
+        MI355Q_TRY_ROWS(3, 1) MI355Q_TRY_ROWS(3, 2)
+        MI355Q_TRY_ROWS(4, 1) MI355Q_TRY_ROWS(4, 2)
+        if constexpr (BITS != 8) { MI355Q_TRY_ROWS(7, 1) }   // 8-bit codes at sixteen wavefronts do not fit the register file
+    }
+    return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no row-kernel variant for q%d g%d steps=%d rows=%d", BITS, GROUP, c.nct, c.br);
+}
+
+#undef MI355Q_TRY_ROWS
 
 }  // namespace
 

@@ -1,5 +1,5 @@
 // Decode GEMV over the split-plane layout (uint32 code words + scale plane + bias plane),
-// bf16 activations, 1 <= M <= 8.  HBM-bound by design:
+// bf16 or f16 activations, 1 <= M <= 8.  HBM-bound by design:
 //
 //   * every lane owns one "lane chunk" of a row per K-step: WPL consecutive code words
 //     (128-bit load for 2/4/8-bit, 96-bit for 3/6-bit, so straddling codes never cross lanes);
@@ -8,9 +8,13 @@
 //     D pipeline steps ahead of the arithmetic in a register ring;
 //   * activations are staged once per workgroup in LDS, already permuted into the pair order
 //     the unpacker produces, laid out [m][k-step][piece][lane] so reads are conflict-free b128;
-//   * 2/4-bit codes become bf16 pairs (128+q) with one and-or each and go through
-//     v_dot2_f32_bf16 against the bf16 activation pairs (fp32 accumulate); other widths are
-//     extracted with bit-field/funnel ops and accumulated with fp32 FMA;
+//   * codes become 16-bit float pairs carrying a magic offset, with no int->float conversion, and go
+//     through v_dot2 against the staged activation pairs (fp32 accumulate).  XA = 0: bf16 pairs
+//     (128 + q) for bf16 activations.  XA = 1: f16 pairs for f16 activations.  In f16 a 4-bit field
+//     needs no shift when it sits in bits
+//     0-3 or 4-7 of a half-word ((w & 0x00F000F0) | 0x6400 is 1024 + 16 q), so a word of eight
+//     codes costs one shift and four and-ors instead of three and four; 2-bit fields take five
+//     positions per half-word unshifted; 8-bit codes become pairs with one byte permute;
 //   * the affine form is applied per lane chunk:  sum (s*q+z)*x = s*sum(q*x) + z*sum(x), with
 //     sum(x) per lane chunk precomputed at staging time;
 //   * one DPP/readlane reduction per output row at the end (split-K across the 64 lanes).
@@ -47,7 +51,7 @@ struct GemvArgs {
     uint32_t wave_end[kGemvMaxSegments];       // cumulative wavefront counts; unused entries repeat the last
     uint32_t seg_rows[kGemvMaxSegments];       // N_i
     uint32_t y_stride[kGemvMaxSegments];
-    const uint16_t* x;       // bf16 [M, x_stride]
+    const uint16_t* x;       // bf16 or f16 [M, x_stride]
     float* logits;           // optional fp32 [N] copy (M == 1, single segment)
     int32_t* token_out;      // ARGMAX only
     unsigned long long* scratch;  // ARGMAX only: one packed (ordered value, ~row) key per workgroup; 0 = no candidate
@@ -57,7 +61,7 @@ struct GemvArgs {
     uint32_t nc;             // K-steps per row = ceil(K / (64*CPL))
     uint32_t rows_per_wave;  // consecutive rows owned by one wavefront
     uint32_t y_dtype, sb_dtype;
-    uint32_t dbg;            // tuning builds only: bit0 no scale/bias loads, bit1 no arithmetic, bit2 no staging
+    uint32_t x_dtype;        // MI355Q_BF16 or MI355Q_F16 (f16 needs XA = 1)
 };
 
 // Host-side choice of kernel variant and launch shape.
@@ -66,9 +70,28 @@ struct GemvCfg {
     bool argmax;
     int waves, depth;   // wavefronts per workgroup, prefetch ring depth
     int xreg;           // 0: activations read from LDS each step; 1/2: register-resident (K-steps per row)
+    int xa;             // 0: bf16 activations and arithmetic; 1: f16
+    bool rows;          // the static-structure kernel (gemv_rows_kernel) with `nct` K-steps per row, `br` rows per pass
+    int nct, br;
     uint32_t grid, rows_per_wave, nc;
     size_t lds;
 };
+
+// Which instantiations of the static-structure kernel exist: the formats of the reference's default kernel set
+// plus the group-64 widths of the bit-width sweep; f16 activations for the default set; the fused arg-max tail
+// for rows of one or two K-steps (output heads have short rows and many of them).
+constexpr bool gemv_rows_has_format(int bits, int group) {
+    return (bits == 4 && (group == 64 || group == 128)) || (bits == 8 && (group == 32 || group == 64)) ||
+           ((bits == 2 || bits == 3 || bits == 6) && group == 64);
+}
+constexpr bool gemv_rows_has_f16(int bits, int group) { return (bits == 4 || bits == 8) && gemv_rows_has_format(bits, group); }
+constexpr bool gemv_rows_has_argmax(int nct, int br) { return (nct == 1 && br >= 4) || (nct == 2 && br >= 2); }
+constexpr bool gemv_rows_has_shape(int nct, int br) {
+    return (nct == 1 && (br == 1 || br == 2 || br == 4 || br == 8)) || (nct == 2 && (br == 1 || br == 2 || br == 4)) ||
+           ((nct == 3 || nct == 4) && (br == 1 || br == 2)) || (nct == 7 && br == 1);
+}
+// wavefronts per workgroup: the longer the row, the more wavefronts share one staged copy of the activations
+constexpr int gemv_rows_waves(int nct) { return nct <= 2 ? 4 : nct <= 4 ? 8 : 16; }
 
 template <int BITS> struct GemvGeo;
 template <> struct GemvGeo<2> { static constexpr int WPL = 4, CPL = 64; static constexpr bool PAIRS = true; };
@@ -97,11 +120,32 @@ __host__ __device__ constexpr int pair_elem(int i, int which) {
     return 2 * i + which;                                       // natural order
 }
 
+// f16 arithmetic on 2- and 4-bit codes: the field of staged pair i is used where it sits in its half-word, so
+// the f16 pair reads 1024 + mult * q.  mult by pair: 4-bit (1, 16, 1, 16); 2-bit (1, 4, 16, 64, 256, 1, 4, 16),
+// the last three after one shift by ten.  The dot products of pairs with the same mult share an accumulator
+// ("class"), and  sum q x = sum_c (dot_c - 1024 Sx_c) / mult_c.
+template <int BITS> __host__ __device__ constexpr int f16_classes() { return BITS == 4 ? 2 : BITS == 2 ? 5 : 1; }
+template <int BITS> __host__ __device__ constexpr int f16_pair_class(int i) {
+    if (BITS == 4) return i & 1;
+    if (BITS == 2) return (i % 8) < 5 ? (i % 8) : (i % 8) - 5;
+    return 0;
+}
+template <int BITS> __host__ __device__ constexpr int f16_class_shift(int c) { return BITS == 4 ? 4 * c : BITS == 2 ? 2 * c : 0; }
+
 typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 f16x2_t;
 
 __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float acc) {
     return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), acc,
                                            false);
+}
+__device__ __forceinline__ float dot2_f16(uint32_t a, uint32_t b, float acc) {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, a), __builtin_bit_cast(f16x2_t, b), acc, false);
+}
+template <int XA>
+__device__ __forceinline__ float dot2_x(uint32_t a, uint32_t b, float acc) {
+    if constexpr (XA == 1) return dot2_f16(a, b, acc);
+    else return dot2_bf16(a, b, acc);
 }
 
 // One wavefront owns `rows_per_wave` consecutive rows and walks them R at a time, one K-step
@@ -120,7 +164,8 @@ __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float acc) {
 // XREG = 1 or 2 means rows are exactly that many K-steps long and the wavefront keeps its
 // activation slice in registers; XREG = 0 re-reads the slice from LDS at every step
 // (conflict-free 128-bit reads shared by the R rows).
-template <int BITS, int GROUP, int R, int MT, bool ARGMAX, int WAVES, int D, int XREG>
+// XA = 0: bf16 activations and bf16 code pairs; XA = 1: f16 activations and f16 code pairs.
+template <int BITS, int GROUP, int R, int MT, bool ARGMAX, int WAVES, int D, int XREG, int XA>
 __global__ __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(MT == 1 ? 4 : 2)))
 void gemv_planes_kernel(GemvArgs a) {
     using G = GemvGeo<BITS>;
@@ -129,9 +174,13 @@ void gemv_planes_kernel(GemvArgs a) {
     constexpr int SR = CPL < GROUP ? CPL : GROUP;       // codes of one group inside a lane chunk
     constexpr int NSR = CPL / SR;                       // sub-runs (groups touched) per lane chunk
     constexpr int KC = 64 * CPL;                        // codes per wavefront K-step
-    // 3-, 5- and 6-bit codes are also fed to v_dot2 as bf16 (128 + q): the field fits the 7 mantissa bits
+    // 3-, 5- and 6-bit codes are fed to v_dot2 like the others: the field fits the mantissa next to the magic offset
     constexpr bool SMALL_FIELD = BITS == 3 || BITS == 5 || BITS == 6;
-    constexpr float OFS = (G::PAIRS || SMALL_FIELD) ? 128.0f : 0.0f;     // magic offset carried by the bf16 codes
+    constexpr bool DOT2 = XA == 1 || G::PAIRS || SMALL_FIELD;             // else (8-bit, bf16 arithmetic): fp32 FMA
+    constexpr bool MULTI = XA == 1 && G::PAIRS;                           // f16 arithmetic on fields used in place
+    constexpr int NCLS = MULTI ? f16_classes<BITS>() : 1;
+    constexpr int NF = MULTI ? 2 : 1;                   // staged floats per sub-run: Sx [, 1024 * sum_c Sx_c / mult_c]
+    constexpr float OFS = XA == 1 ? 1024.0f : DOT2 ? 128.0f : 0.0f;       // magic offset carried by the code pairs
     constexpr int XC = XREG ? XREG : 1;                 // K-steps cached in registers
     static_assert(XREG == 0 || (MT == 1 && R == 1), "register-resident activations are for M == 1, R == 1");
     static_assert(XREG == 0 || D % XREG == 0, "ring depth must be a multiple of the K-steps per row");
@@ -139,7 +188,7 @@ void gemv_planes_kernel(GemvArgs a) {
     extern __shared__ u32x4 smem[];
     const uint32_t NC = a.nc;
     u32x4* xs = smem;                                      // [MT][NC][Q][64]
-    float* sxs = (float*)(smem + (size_t)MT * NC * Q * 64); // [MT][NC][NSR][64]
+    float* sxs = (float*)(smem + (size_t)MT * NC * Q * 64); // [MT][NC][NSR][NF][64]
 
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     // the wavefront index is uniform: keep it (and everything derived from it) in scalar registers
@@ -185,12 +234,7 @@ void gemv_planes_kernel(GemvArgs a) {
                 for (int i = 0; i < WPL; i++) p.w[r][i] = MI355Q_STREAM_LOAD(rowp + code_off + i);
             }
 #pragma unroll
-            for (int sr = 0; sr < NSR; sr++) {
-#ifdef MI355Q_GEMV_EXPERIMENT
-                if (a.dbg & 1) { p.sz[r][sr] = 0x38003C00u; continue; }
-#endif
-                p.sz[r][sr] = MI355Q_STREAM_LOAD(szp + sz_off[sr]);
-            }
+            for (int sr = 0; sr < NSR; sr++) p.sz[r][sr] = MI355Q_STREAM_LOAD(szp + sz_off[sr]);
         }
     };
     // per-lane offsets of the K-steps a ring slot can hold, precomputed when rows are XREG steps long
@@ -224,10 +268,7 @@ void gemv_planes_kernel(GemvArgs a) {
         uint32_t m, cc;
         task_coords(tw, m, cc);
         const uint64_t kbase = (uint64_t)cc * KC + (uint64_t)lane * CPL;
-        bool valid = tw < nwt && m < a.m && kbase < a.k;
-#ifdef MI355Q_GEMV_EXPERIMENT
-        if (a.dbg & 8) valid = false;                       // every lane reads the same line
-#endif
+        const bool valid = tw < nwt && m < a.m && kbase < a.k;
         const u32x4* src = (const u32x4*)(a.x + (valid ? (size_t)m * a.x_stride + kbase : 0));
 #pragma unroll
         for (int i = 0; i < Q; i++) {
@@ -240,31 +281,49 @@ void gemv_planes_kernel(GemvArgs a) {
         if (tw >= nwt) return;                              // LDS writes only inside this (scalar) branch
         uint32_t m, cc;
         task_coords(tw, m, cc);
-        // staged pair i = (element e0, element e1) of the lane chunk: one byte permute of two dwords
-        auto pairw = [&](auto I) -> uint32_t {
-            constexpr int i = decltype(I)::value;
-            constexpr int e0 = pair_elem<BITS>(i, 0), e1 = pair_elem<BITS>(i, 1);
-            static_assert((e0 & 1) == (e1 & 1) || e1 == e0 + 1, "pair halves come from the same half-word");
-            if constexpr (e1 == e0 + 1 && (e0 & 1) == 0) return d[e0 >> 1];
-            else return __builtin_amdgcn_perm(d[e1 >> 1], d[e0 >> 1], (e0 & 1) ? 0x07060302u : 0x05040100u);
-        };
+        uint32_t pw[CPL / 2];                               // staged pairs, in the order the unpacker produces them
+        {
+            // 16-bit elements as they are: staged pair i = (element e0, element e1), one byte permute of two dwords
+            static_for<CPL / 2>([&](auto I) {
+                constexpr int i = decltype(I)::value;
+                constexpr int e0 = pair_elem<BITS>(i, 0), e1 = pair_elem<BITS>(i, 1);
+                static_assert((e0 & 1) == (e1 & 1) || e1 == e0 + 1, "pair halves come from the same half-word");
+                if constexpr (e1 == e0 + 1 && (e0 & 1) == 0) pw[i] = d[e0 >> 1];
+                else pw[i] = __builtin_amdgcn_perm(d[e1 >> 1], d[e0 >> 1], (e0 & 1) ? 0x07060302u : 0x05040100u);
+            });
+        }
         static_for<Q>([&](auto P) {
             constexpr int i = decltype(P)::value;
             u32x4 o;
-            o.x = pairw(std::integral_constant<int, 4 * i + 0>{});
-            o.y = pairw(std::integral_constant<int, 4 * i + 1>{});
-            o.z = pairw(std::integral_constant<int, 4 * i + 2>{});
-            o.w = pairw(std::integral_constant<int, 4 * i + 3>{});
+            o.x = pw[4 * i + 0]; o.y = pw[4 * i + 1]; o.z = pw[4 * i + 2]; o.w = pw[4 * i + 3];
             xs[((size_t)(m * NC + cc) * Q + i) * 64 + lane] = o;
         });
-        // sum of the activations of each sub-run: dot2 against the bf16 pair (1.0, 1.0)
-#pragma unroll
-        for (int sr = 0; sr < NSR; sr++) {
-            float sx = 0.0f;
-#pragma unroll
-            for (int j = 0; j < SR / 2; j++) sx = dot2_bf16(d[sr * (SR / 2) + j], 0x3F803F80u, sx);
-            sxs[((size_t)(m * NC + cc) * NSR + sr) * 64 + lane] = sx;
-        }
+        // per sub-run: the sum of its activations (dot2 against the pair (1, 1)) and, for fields used in place,
+        // 1024 * sum_c Sx_c / mult_c (dot2 against the pair (1024 / mult, 1024 / mult) of each staged pair)
+        constexpr uint32_t kOnes = XA == 1 ? 0x3C003C00u : 0x3F803F80u;
+        static_for<NSR>([&](auto S) {
+            constexpr int sr = decltype(S)::value;
+            float sx = 0.0f, px = 0.0f;
+            static_for<CPL / 2>([&](auto I) {
+                constexpr int i = decltype(I)::value;
+                if constexpr (pair_elem<BITS>(i, 0) / SR == sr) {
+                    sx = dot2_x<XA>(pw[i], kOnes, sx);
+                    if constexpr (MULTI) {
+                        // 1024 >> shift as an f16 pair: 1024 = 0x6400, each halving lowers the exponent field by one
+                        constexpr uint32_t h = 0x6400u - ((uint32_t)f16_class_shift<BITS>(f16_pair_class<BITS>(i)) << 10);
+                        px = dot2_f16(pw[i], h | (h << 16), px);
+                    }
+                }
+            });
+            float* const cell = sxs + ((size_t)(m * NC + cc) * NSR + sr) * NF * 64 + lane;
+            cell[0] = sx;
+            if constexpr (MULTI) cell[64] = px;
+        });
+    };
+    auto lds_barrier = [&]() {      // LDS-only: the weight loads in flight must not be waited for here
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
     };
 
     // ---- 1. activation loads first ------------------------------------------------------------
@@ -272,6 +331,7 @@ void gemv_planes_kernel(GemvArgs a) {
     uint32_t dearly[TE][CPL / 2];
 #pragma unroll
     for (int t = 0; t < TE; t++) stage_load(wave + t * WAVES, dearly[t]);
+    __builtin_amdgcn_sched_barrier(0);                      // pinned: the scheduler must not sink them below the weight loads
 
     // ---- 2. the first D steps of weight loads -------------------------------------------------
     // Steps past the last one repeat it (same addresses, so they hit in L2 and their data is
@@ -291,48 +351,41 @@ void gemv_planes_kernel(GemvArgs a) {
     });
 
     // ---- 3. permute the activations into LDS (waits only for the loads of step 1) -------------
-#ifdef MI355Q_GEMV_EXPERIMENT
-    if (!(a.dbg & 4))
-#endif
-    {
 #pragma unroll
-        for (int t = 0; t < TE; t++) stage_store(wave + t * WAVES, dearly[t]);
-        for (uint32_t tw = wave + TE * WAVES; tw < nwt; tw += WAVES) {
-            uint32_t dl[CPL / 2];                           // long rows / batches: the remaining tasks
-            stage_load(tw, dl);
-            stage_store(tw, dl);
-        }
+    for (int t = 0; t < TE; t++) stage_store(wave + t * WAVES, dearly[t]);
+    for (uint32_t tw = wave + TE * WAVES; tw < nwt; tw += WAVES) {
+        uint32_t dl[CPL / 2];                               // long rows / batches: the remaining tasks
+        stage_load(tw, dl);
+        stage_store(tw, dl);
     }
-    // LDS-only barrier: the weight loads in flight must not be waited for here
-#ifdef MI355Q_GEMV_EXPERIMENT
-    if (!(a.dbg & 16))
-#endif
-    {
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-        __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-    }
+    lds_barrier();
 
     // ---- optional register-resident activation slice (M == 1, rows of XREG K-steps) -----------
     u32x4 xr[XC][Q];
-    float sxr[XC][NSR];
+    float sxr[XC][NSR][NF];
     if constexpr (XREG != 0) {
 #pragma unroll
         for (int cc = 0; cc < XC; cc++) {
 #pragma unroll
             for (int p = 0; p < Q; p++) xr[cc][p] = xs[((size_t)cc * Q + p) * 64 + lane];
 #pragma unroll
-            for (int sr = 0; sr < NSR; sr++) sxr[cc][sr] = sxs[((size_t)cc * NSR + sr) * 64 + lane];
+            for (int sr = 0; sr < NSR; sr++)
+#pragma unroll
+                for (int f = 0; f < NF; f++) sxr[cc][sr][f] = sxs[(((size_t)cc * NSR + sr) * NF + f) * 64 + lane];
         }
     }
 
-    // The pair mask lives in an SGPR and the bf16 "128.0" pair in a VGPR, both opaque to the
-    // optimiser, so that (w & mask) | magic is one v_and_or_b32 instead of an AND and an OR with
-    // literals (a VOP3 instruction takes no literal and a single scalar operand on this target).
-    uint32_t k_magic = 0x43004300u;
-    uint32_t k_mask = BITS == 4 ? 0x000F000Fu : 0x00030003u;
+    // The pair masks live in SGPRs and the magic pair in a VGPR, all opaque to the optimiser, so that
+    // (w & mask) | magic is one v_and_or_b32 instead of an AND and an OR with literals (a VOP3
+    // instruction takes no literal and a single scalar operand on this target).
+    uint32_t k_magic = XA == 1 ? 0x64006400u : 0x43004300u;
     asm volatile("" : "+v"(k_magic));
-    asm volatile("" : "+s"(k_mask));
+    uint32_t k_mask[NCLS];
+#pragma unroll
+    for (int c = 0; c < NCLS; c++) {
+        k_mask[c] = (BITS == 4 ? 0x000F000Fu : 0x00030003u) << (MULTI ? f16_class_shift<BITS>(c) : 0);
+        asm volatile("" : "+s"(k_mask[c]));
+    }
 
     float acc[R][MT];
     float res[MT];                   // lane i parks the result of the wavefront's i-th row
@@ -358,13 +411,14 @@ void gemv_planes_kernel(GemvArgs a) {
 #pragma unroll
             for (int m = 0; m < MT; m++) {
                 if ((uint32_t)m < a.m) {
+                    const float v = res[m];
                     if (yb) {
                         const size_t o = (size_t)m * ys + lrow;
-                        if (a.y_dtype == MI355Q_F32) ((float*)yb)[o] = res[m];
-                        else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)yb)[o] = f32_to_bf16_rne(res[m]);
-                        else ((uint16_t*)yb)[o] = f32_to_f16_rne(res[m]);
+                        if (a.y_dtype == MI355Q_F32) ((float*)yb)[o] = v;
+                        else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)yb)[o] = f32_to_bf16_rne(v);
+                        else ((uint16_t*)yb)[o] = f32_to_f16_rne(v);
                     }
-                    if (a.logits && m == 0) a.logits[row] = res[m];
+                    if (a.logits && m == 0) a.logits[row] = v;
                 }
             }
             if constexpr (ARGMAX) {
@@ -384,26 +438,16 @@ void gemv_planes_kernel(GemvArgs a) {
     // constant (cj) and so is the slot at which a row completes.
     auto compute = [&](const Pref& cur, auto J) {
         constexpr int cj = XREG ? decltype(J)::value % XC : 0;
-#ifdef MI355Q_GEMV_EXPERIMENT
-        if (a.dbg & 2) {
-#pragma unroll
-            for (int r = 0; r < R; r++) {
-                uint32_t t = 0;
-#pragma unroll
-                for (int i = 0; i < WPL; i++) t ^= cur.w[r][i];
-                acc[r][0] += __uint_as_float(t & 0x3FFFFFFFu) + __uint_as_float(cur.sz[r][0] & 0x3FFFFFFFu);
-            }
-        } else
-#endif
-        {
         // ---- one K-step of R rows ----------------------------------------------------------
-        float dot[R][MT][NSR];
+        float dot[R][MT][NSR][NCLS];
 #pragma unroll
         for (int r = 0; r < R; r++)
 #pragma unroll
             for (int m = 0; m < MT; m++)
 #pragma unroll
-                for (int sr = 0; sr < NSR; sr++) dot[r][m][sr] = 0.0f;
+                for (int sr = 0; sr < NSR; sr++)
+#pragma unroll
+                    for (int cl = 0; cl < NCLS; cl++) dot[r][m][sr][cl] = 0.0f;
 
         static_for<Q>([&](auto P) {
             constexpr int p = decltype(P)::value;
@@ -416,54 +460,64 @@ void gemv_planes_kernel(GemvArgs a) {
                 for (int m = 0; m < MT; m++) xv[m] = xs[((size_t)(m * NC + c) * Q + p) * 64 + lane];
             }
 
-            if constexpr (G::PAIRS) {
+            if constexpr (DOT2) {
 #pragma unroll
                 for (int r = 0; r < R; r++) {
                     uint32_t pr[4];
-                    if constexpr (BITS == 4) {
+                    if constexpr (MULTI && BITS == 4) {
+                        // fields 0 and 1 of each half-word in place, fields 2 and 3 after one shift
+                        const uint32_t wv = cur.w[r][p], w8 = wv >> 8;
+                        pr[0] = (wv & k_mask[0]) | k_magic; pr[1] = (wv & k_mask[1]) | k_magic;
+                        pr[2] = (w8 & k_mask[0]) | k_magic; pr[3] = (w8 & k_mask[1]) | k_magic;
+                    } else if constexpr (MULTI && BITS == 2) {
+                        // word p/2; even pieces: fields 0..3 in place; odd pieces: field 4 in place, 5..7 after one shift
+                        const uint32_t wv = cur.w[r][p >> 1];
+                        if constexpr ((p & 1) == 0) {
+                            pr[0] = (wv & k_mask[0]) | k_magic; pr[1] = (wv & k_mask[1]) | k_magic;
+                            pr[2] = (wv & k_mask[2]) | k_magic; pr[3] = (wv & k_mask[3]) | k_magic;
+                        } else {
+                            const uint32_t w10 = wv >> 10;
+                            pr[0] = (wv & k_mask[4]) | k_magic; pr[1] = (w10 & k_mask[0]) | k_magic;
+                            pr[2] = (w10 & k_mask[1]) | k_magic; pr[3] = (w10 & k_mask[2]) | k_magic;
+                        }
+                    } else if constexpr (BITS == 4) {
                         const uint32_t wv = cur.w[r][p];
-                        pr[0] = (wv & k_mask) | k_magic;
-                        pr[1] = ((wv >> 4) & k_mask) | k_magic;
-                        pr[2] = ((wv >> 8) & k_mask) | k_magic;
-                        pr[3] = ((wv >> 12) & k_mask) | k_magic;
-                    } else {  // BITS == 2: word p/2, shifts 2*(4*(p&1) + i)
+                        pr[0] = (wv & k_mask[0]) | k_magic;
+                        pr[1] = ((wv >> 4) & k_mask[0]) | k_magic;
+                        pr[2] = ((wv >> 8) & k_mask[0]) | k_magic;
+                        pr[3] = ((wv >> 12) & k_mask[0]) | k_magic;
+                    } else if constexpr (BITS == 2) {   // word p/2, shifts 2*(4*(p&1) + i)
                         const uint32_t wv = cur.w[r][p >> 1] >> (8 * (p & 1));
-                        pr[0] = (wv & k_mask) | k_magic;
-                        pr[1] = ((wv >> 2) & k_mask) | k_magic;
-                        pr[2] = ((wv >> 4) & k_mask) | k_magic;
-                        pr[3] = ((wv >> 6) & k_mask) | k_magic;
+                        pr[0] = (wv & k_mask[0]) | k_magic;
+                        pr[1] = ((wv >> 2) & k_mask[0]) | k_magic;
+                        pr[2] = ((wv >> 4) & k_mask[0]) | k_magic;
+                        pr[3] = ((wv >> 6) & k_mask[0]) | k_magic;
+                    } else if constexpr (BITS == 8) {
+                        // f16 arithmetic: bytes (b0, 0x64, b1, 0x64), the 0x64 taken from the magic word, are the f16 pair (1024 + b0, 1024 + b1)
+                        const uint32_t w0 = cur.w[r][2 * p], w1 = cur.w[r][2 * p + 1];
+                        pr[0] = __builtin_amdgcn_perm(k_magic, w0, 0x05010500u);
+                        pr[1] = __builtin_amdgcn_perm(k_magic, w0, 0x05030502u);
+                        pr[2] = __builtin_amdgcn_perm(k_magic, w1, 0x05010500u);
+                        pr[3] = __builtin_amdgcn_perm(k_magic, w1, 0x05030502u);
+                    } else {
+                        // 3-, 5-, 6-bit: codes 2i and 2i+1 of this piece side by side: two field extracts (funnel
+                        // shifts where a code straddles words), one shift-or and the magic
+                        static_for<4>([&](auto I) {
+                            constexpr int i = decltype(I)::value;
+                            const uint32_t qa = extract_code<(p * 8 + 2 * i) * BITS, BITS, WPL>(cur.w[r]);
+                            const uint32_t qb = extract_code<(p * 8 + 2 * i + 1) * BITS, BITS, WPL>(cur.w[r]);
+                            pr[i] = ((qb << 16) | qa) | k_magic;
+                        });
                     }
+                    // accumulator of each of the piece's four pairs (its class; one accumulator otherwise)
+                    constexpr int c0 = MULTI ? f16_pair_class<BITS>(4 * p + 0) : 0, c1 = MULTI ? f16_pair_class<BITS>(4 * p + 1) : 0;
+                    constexpr int c2 = MULTI ? f16_pair_class<BITS>(4 * p + 2) : 0, c3 = MULTI ? f16_pair_class<BITS>(4 * p + 3) : 0;
 #pragma unroll
                     for (int m = 0; m < MT; m++) {
-                        float dsum = dot[r][m][sr];
-                        dsum = dot2_bf16(pr[0], xv[m].x, dsum);
-                        dsum = dot2_bf16(pr[1], xv[m].y, dsum);
-                        dsum = dot2_bf16(pr[2], xv[m].z, dsum);
-                        dsum = dot2_bf16(pr[3], xv[m].w, dsum);
-                        dot[r][m][sr] = dsum;
-                    }
-                }
-            } else if constexpr (SMALL_FIELD) {
-                // codes 2i and 2i+1 of this piece side by side as bf16 (128 + q): two field extracts (funnel
-                // shifts where a code straddles words), one shift-or and the magic, then v_dot2 against the
-                // activation pair in natural order -- no int->float conversion and no bf16->fp32 unpack of x
-#pragma unroll
-                for (int r = 0; r < R; r++) {
-                    uint32_t pr[4];
-                    static_for<4>([&](auto I) {
-                        constexpr int i = decltype(I)::value;
-                        const uint32_t qa = extract_code<(p * 8 + 2 * i) * BITS, BITS, WPL>(cur.w[r]);
-                        const uint32_t qb = extract_code<(p * 8 + 2 * i + 1) * BITS, BITS, WPL>(cur.w[r]);
-                        pr[i] = ((qb << 16) | qa) | k_magic;
-                    });
-#pragma unroll
-                    for (int m = 0; m < MT; m++) {
-                        float dsum = dot[r][m][sr];
-                        dsum = dot2_bf16(pr[0], xv[m].x, dsum);
-                        dsum = dot2_bf16(pr[1], xv[m].y, dsum);
-                        dsum = dot2_bf16(pr[2], xv[m].z, dsum);
-                        dsum = dot2_bf16(pr[3], xv[m].w, dsum);
-                        dot[r][m][sr] = dsum;
+                        dot[r][m][sr][c0] = dot2_x<XA>(pr[0], xv[m].x, dot[r][m][sr][c0]);
+                        dot[r][m][sr][c1] = dot2_x<XA>(pr[1], xv[m].y, dot[r][m][sr][c1]);
+                        dot[r][m][sr][c2] = dot2_x<XA>(pr[2], xv[m].z, dot[r][m][sr][c2]);
+                        dot[r][m][sr][c3] = dot2_x<XA>(pr[3], xv[m].w, dot[r][m][sr][c3]);
                     }
                 }
             } else {
@@ -488,24 +542,29 @@ void gemv_planes_kernel(GemvArgs a) {
                     qf[7] = (float)extract_code<(p * 8 + 7) * BITS, BITS, WPL>(cur.w[r]);
 #pragma unroll
                     for (int m = 0; m < MT; m++) {
-                        float dsum = dot[r][m][sr];
+                        float dsum = dot[r][m][sr][0];
 #pragma unroll
                         for (int e = 0; e < 8; e++) dsum = __builtin_fmaf(qf[e], xf[m][e], dsum);
-                        dot[r][m][sr] = dsum;
+                        dot[r][m][sr][0] = dsum;
                     }
                 }
             }
         });
 
-        // ---- affine form per sub-run: s*dot + (z - OFS*s)*sum(x) -----------------------------
+        // ---- affine form per sub-run: s * sum(q x) + z * sum(x) ---------------------------------
 #pragma unroll
         for (int sr = 0; sr < NSR; sr++) {
-            float sx[MT];
+            float sx[MT], px[MT];
             if constexpr (XREG != 0) {
-                sx[0] = sxr[cj][sr];
+                sx[0] = sxr[cj][sr][0];
+                px[0] = MULTI ? sxr[cj][sr][NF - 1] : 0.0f;
             } else {
 #pragma unroll
-                for (int m = 0; m < MT; m++) sx[m] = sxs[((size_t)(m * NC + c) * NSR + sr) * 64 + lane];
+                for (int m = 0; m < MT; m++) {
+                    const float* const cell = sxs + ((size_t)(m * NC + c) * NSR + sr) * NF * 64 + lane;
+                    sx[m] = cell[0];
+                    px[m] = MULTI ? cell[(NF - 1) * 64] : 0.0f;
+                }
             }
 #pragma unroll
             for (int r = 0; r < R; r++) {
@@ -518,11 +577,23 @@ void gemv_planes_kernel(GemvArgs a) {
                     asm volatile("" ::: "memory");
                     s = f16_to_f32((uint16_t)(szw & 0xFFFFu)); z = f16_to_f32((uint16_t)(szw >> 16));
                 }
-                const float zc = z - OFS * s;
+                if constexpr (MULTI) {
+                    // sum q x = sum_c dot_c / mult_c - px
 #pragma unroll
-                for (int m = 0; m < MT; m++) acc[r][m] += s * dot[r][m][sr] + zc * sx[m];
+                    for (int m = 0; m < MT; m++) {
+                        float t = dot[r][m][sr][0];
+#pragma unroll
+                        for (int cl = 1; cl < NCLS; cl++)
+                            t = __builtin_fmaf(dot[r][m][sr][cl], 1.0f / (float)(1 << f16_class_shift<BITS>(cl)), t);
+                        t -= px[m];
+                        acc[r][m] = __builtin_fmaf(s, t, __builtin_fmaf(z, sx[m], acc[r][m]));
+                    }
+                } else {
+                    const float zc = z - OFS * s;
+#pragma unroll
+                    for (int m = 0; m < MT; m++) acc[r][m] += s * dot[r][m][sr][0] + zc * sx[m];
+                }
             }
-        }
         }
         if constexpr (XREG != 0) {
             // ---- row complete at a known slot: keep its per-lane partial for the batched reduce -----

@@ -1,0 +1,336 @@
+// Decode GEMV over the split-plane layout for one activation row (M = 1) when a row is a small, known number
+// of K-steps: the fast path of gemv_q{b}_g{g}
+// (Sources/MetalCompiler/Generator/MetalSourceGenerator+Quantized.swift:496-575).
+//
+// Same arithmetic as gemv_planes_kernel (lane chunks, magic-offset code pairs into v_dot2, affine form per
+// sub-run, fp32 accumulation); what differs is the shape of the instruction stream:
+//   * NCT, the K-steps per row, is a template argument, and a wavefront walks its rows BR at a time ("pass"),
+//     so which ring slot holds which (row, K-step) is known at compile time: the steady loop has no index
+//     arithmetic, no selects and no branches besides its back edge.  The general kernel spends more scalar
+//     instructions and branches per K-step than vector ones, and the scalar unit issues one instruction per
+//     wavefront slot just like the vector unit: that bookkeeping, not the unpack, was its ceiling;
+//   * a wavefront whose share is at most eight K-steps issues ALL its weight loads before anything else
+//     (one pass).  Wavefronts are served oldest first, so the youngest ones get their first bytes late;
+//     with every load already in flight they need one memory round trip, not one per pass;
+//   * the activation loads are pinned ahead of the weight loads (vector loads return in issue order) and
+//     staged in LDS once per workgroup; rows re-read them from LDS (conflict-free 128-bit reads);
+//   * row sums are reduced BR at a time (transpose-reduce) and parked one per lane for one coalesced store.
+#pragma once
+
+#include "gemv_planes.inl"
+
+namespace mi355q {
+
+// XA = 0: bf16 activations, bf16 code pairs (128 + q).  XA = 1: f16 activations, f16 code pairs (1024 + mult q,
+// fields of 2- and 4-bit codes used where they sit in the half-word, see f16_classes).
+template <int BITS, int GROUP, int NCT, int BR, int WAVES, int XA, bool SBBF16, bool ARGMAX>
+__global__ __launch_bounds__(WAVES * 64) void gemv_rows_kernel(GemvArgs a) {
+    using G = GemvGeo<BITS>;
+    constexpr int WPL = G::WPL, CPL = G::CPL;
+    constexpr int Q = CPL / 8;
+    constexpr int SR = CPL < GROUP ? CPL : GROUP;
+    constexpr int NSR = CPL / SR;
+    constexpr int KC = 64 * CPL;
+    constexpr bool SMALL_FIELD = BITS == 3 || BITS == 5 || BITS == 6;
+    constexpr bool DOT2 = XA == 1 || G::PAIRS || SMALL_FIELD;
+    constexpr bool MULTI = XA == 1 && G::PAIRS;
+    constexpr int NCLS = MULTI ? f16_classes<BITS>() : 1;
+    constexpr int NF = MULTI ? 2 : 1;
+    constexpr float OFS = XA == 1 ? 1024.0f : DOT2 ? 128.0f : 0.0f;
+    static_assert(BR == 1 || BR == 2 || BR == 4 || BR == 8, "rows per pass: a power of two up to 8");
+
+    extern __shared__ u32x4 smem[];
+    u32x4* xs = smem;                                              // [NCT][Q][64]
+    float* sxs = (float*)(smem + (size_t)NCT * Q * 64);             // [NCT][NSR][NF][64]
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    // matrix of this wavefront (up to three share a launch), then its rows inside that matrix
+    const uint32_t gw = blockIdx.x * WAVES + wave;
+    const bool in1 = gw >= a.wave_end[0], in2 = gw >= a.wave_end[1];
+    const uint32_t* const seg_codes = in2 ? a.codes[2] : in1 ? a.codes[1] : a.codes[0];
+    const uint32_t* const seg_sz = in2 ? a.sz[2] : in1 ? a.sz[1] : a.sz[0];
+    void* const seg_y = in2 ? a.y[2] : in1 ? a.y[1] : a.y[0];
+    const uint32_t seg_n = in2 ? a.seg_rows[2] : in1 ? a.seg_rows[1] : a.seg_rows[0];
+    const uint32_t row0 = (gw - (in2 ? a.wave_end[1] : in1 ? a.wave_end[0] : 0u)) * a.rows_per_wave;
+    // rows this wavefront owns (0 for the wavefronts past the end of a matrix: they still stage and meet the barrier)
+    const uint32_t nrows = row0 < seg_n ? (seg_n - row0 < a.rows_per_wave ? seg_n - row0 : a.rows_per_wave) : 0u;
+    const uint32_t last = nrows ? nrows - 1 : 0u;                  // loads past the last row repeat it
+    const uint32_t rbase = nrows ? row0 : seg_n - 1;
+    const uint32_t cs_bytes = a.code_stride * 4, ss_bytes = a.sz_stride * 4;
+
+    struct Slot {
+        uint32_t w[WPL];
+        uint32_t sz[NSR];
+    };
+    // per-lane byte offsets of the lane chunk of every K-step (chunks past K are clamped: they meet activations staged as zero)
+    uint32_t voff[NCT], vsz[NCT][NSR];
+#pragma unroll
+    for (int c = 0; c < NCT; c++) {
+        uint32_t chunk = c * 64 + lane;
+        chunk = (uint64_t)chunk * CPL < a.k ? chunk : 0;
+        voff[c] = chunk * (WPL * 4);
+#pragma unroll
+        for (int sr = 0; sr < NSR; sr++) vsz[c][sr] = ((chunk * CPL + sr * SR) / GROUP) * 4;
+    }
+    auto row_ptrs = [&](uint32_t r, const char*& cp, const char*& zp) {    // r: row inside the wavefront's share (scalar)
+        r = r < last ? r : last;
+        const uint64_t row = rbase + r;
+        cp = (const char*)seg_codes + row * cs_bytes;
+        zp = (const char*)seg_sz + row * ss_bytes;
+    };
+    auto issue = [&](const char* cp, const char* zp, int c, Slot& s) {
+        if constexpr (WPL == 4) {
+            const u32x4 v = MI355Q_STREAM_LOAD((const u32x4*)(cp + voff[c]));
+            s.w[0] = v.x; s.w[1] = v.y; s.w[2] = v.z; s.w[3] = v.w;
+        } else {
+#pragma unroll
+            for (int i = 0; i < WPL; i++) s.w[i] = MI355Q_STREAM_LOAD((const uint32_t*)(cp + voff[c]) + i);
+        }
+#pragma unroll
+        for (int sr = 0; sr < NSR; sr++) s.sz[sr] = MI355Q_STREAM_LOAD((const uint32_t*)(zp + vsz[c][sr]));
+    };
+
+    // ---- staging: task cc = the 64 lane chunks of K-step cc, dealt to wavefronts whole ----------------------
+    auto stage_load = [&](uint32_t cc, uint32_t (&d)[CPL / 2]) {
+        const uint64_t kbase = (uint64_t)cc * KC + (uint64_t)lane * CPL;
+        const bool valid = cc < (uint32_t)NCT && kbase < a.k;
+        const u32x4* src = (const u32x4*)(a.x + (valid ? kbase : 0));
+#pragma unroll
+        for (int i = 0; i < Q; i++) {
+            const u32x4 v = src[i];                         // clamped address: always readable
+            d[4 * i + 0] = valid ? v.x : 0; d[4 * i + 1] = valid ? v.y : 0;
+            d[4 * i + 2] = valid ? v.z : 0; d[4 * i + 3] = valid ? v.w : 0;
+        }
+    };
+    auto stage_store = [&](uint32_t cc, const uint32_t (&d)[CPL / 2]) {
+        if (cc >= (uint32_t)NCT) return;
+        uint32_t pw[CPL / 2];                               // staged pairs in the order the unpacker produces them
+        static_for<CPL / 2>([&](auto I) {
+            constexpr int i = decltype(I)::value;
+            constexpr int e0 = pair_elem<BITS>(i, 0), e1 = pair_elem<BITS>(i, 1);
+            static_assert((e0 & 1) == (e1 & 1) || e1 == e0 + 1, "pair halves come from the same half-word");
+            if constexpr (e1 == e0 + 1 && (e0 & 1) == 0) pw[i] = d[e0 >> 1];
+            else pw[i] = __builtin_amdgcn_perm(d[e1 >> 1], d[e0 >> 1], (e0 & 1) ? 0x07060302u : 0x05040100u);
+        });
+        static_for<Q>([&](auto P) {
+            constexpr int i = decltype(P)::value;
+            u32x4 o;
+            o.x = pw[4 * i + 0]; o.y = pw[4 * i + 1]; o.z = pw[4 * i + 2]; o.w = pw[4 * i + 3];
+            xs[((size_t)cc * Q + i) * 64 + lane] = o;
+        });
+        constexpr uint32_t kOnes = XA == 1 ? 0x3C003C00u : 0x3F803F80u;
+        static_for<NSR>([&](auto S) {
+            constexpr int sr = decltype(S)::value;
+            float sx = 0.0f, px = 0.0f;
+            static_for<CPL / 2>([&](auto I) {
+                constexpr int i = decltype(I)::value;
+                if constexpr (pair_elem<BITS>(i, 0) / SR == sr) {
+                    sx = dot2_x<XA>(pw[i], kOnes, sx);
+                    if constexpr (MULTI) {
+                        constexpr uint32_t h = 0x6400u - ((uint32_t)f16_class_shift<BITS>(f16_pair_class<BITS>(i)) << 10);
+                        px = dot2_f16(pw[i], h | (h << 16), px);
+                    }
+                }
+            });
+            float* const cell = sxs + ((size_t)cc * NSR + sr) * NF * 64 + lane;
+            cell[0] = sx;
+            if constexpr (MULTI) cell[64] = px;
+        });
+    };
+
+    // ---- 1. activation loads, pinned ahead of the weight loads --------------------------------------------
+    uint32_t dearly[CPL / 2];
+    stage_load(wave, dearly);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- 2. the first pass of weight loads (for most launches: every load of this wavefront) ---------------
+    Slot ring[BR][NCT];
+    {
+        const char *cp[BR], *zp[BR];
+#pragma unroll
+        for (int j = 0; j < BR; j++) row_ptrs((uint32_t)j, cp[j], zp[j]);
+#pragma unroll
+        for (int j = 0; j < BR; j++)
+            static_for<NCT>([&](auto C) { issue(cp[j], zp[j], decltype(C)::value, ring[j][decltype(C)::value]); });
+    }
+
+    // ---- 3. stage the activations behind an LDS-only barrier ----------------------------------------------
+    stage_store(wave, dearly);
+    for (uint32_t cc = wave + WAVES; cc < (uint32_t)NCT; cc += WAVES) {
+        uint32_t dl[CPL / 2];
+        stage_load(cc, dl);
+        stage_store(cc, dl);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+
+    uint32_t k_magic = XA == 1 ? 0x64006400u : 0x43004300u;
+    asm volatile("" : "+v"(k_magic));
+    uint32_t k_mask[NCLS];
+#pragma unroll
+    for (int c = 0; c < NCLS; c++) {
+        k_mask[c] = (BITS == 4 ? 0x000F000Fu : 0x00030003u) << (MULTI ? f16_class_shift<BITS>(c) : 0);
+        asm volatile("" : "+s"(k_mask[c]));
+    }
+
+    // contribution of one K-step of one row: sum over its sub-runs of s * sum(q x) + z * sum(x)
+    auto step = [&](const Slot& cur, auto C) -> float {
+        constexpr int c = decltype(C)::value;
+        float dot[NSR][NCLS];
+#pragma unroll
+        for (int sr = 0; sr < NSR; sr++)
+#pragma unroll
+            for (int cl = 0; cl < NCLS; cl++) dot[sr][cl] = 0.0f;
+        static_for<Q>([&](auto P) {
+            constexpr int p = decltype(P)::value;
+            constexpr int sr = (p * 8) / SR;
+            const u32x4 xv = xs[((size_t)c * Q + p) * 64 + lane];
+            if constexpr (DOT2) {
+                uint32_t pr[4];
+                if constexpr (MULTI && BITS == 4) {
+                    const uint32_t wv = cur.w[p], w8 = wv >> 8;
+                    pr[0] = (wv & k_mask[0]) | k_magic; pr[1] = (wv & k_mask[1]) | k_magic;
+                    pr[2] = (w8 & k_mask[0]) | k_magic; pr[3] = (w8 & k_mask[1]) | k_magic;
+                } else if constexpr (MULTI && BITS == 2) {
+                    const uint32_t wv = cur.w[p >> 1];
+                    if constexpr ((p & 1) == 0) {
+                        pr[0] = (wv & k_mask[0]) | k_magic; pr[1] = (wv & k_mask[1]) | k_magic;
+                        pr[2] = (wv & k_mask[2]) | k_magic; pr[3] = (wv & k_mask[3]) | k_magic;
+                    } else {
+                        const uint32_t w10 = wv >> 10;
+                        pr[0] = (wv & k_mask[4]) | k_magic; pr[1] = (w10 & k_mask[0]) | k_magic;
+                        pr[2] = (w10 & k_mask[1]) | k_magic; pr[3] = (w10 & k_mask[2]) | k_magic;
+                    }
+                } else if constexpr (BITS == 4) {
+                    const uint32_t wv = cur.w[p];
+                    pr[0] = (wv & k_mask[0]) | k_magic;
+                    pr[1] = ((wv >> 4) & k_mask[0]) | k_magic;
+                    pr[2] = ((wv >> 8) & k_mask[0]) | k_magic;
+                    pr[3] = ((wv >> 12) & k_mask[0]) | k_magic;
+                } else if constexpr (BITS == 2) {
+                    const uint32_t wv = cur.w[p >> 1] >> (8 * (p & 1));
+                    pr[0] = (wv & k_mask[0]) | k_magic;
+                    pr[1] = ((wv >> 2) & k_mask[0]) | k_magic;
+                    pr[2] = ((wv >> 4) & k_mask[0]) | k_magic;
+                    pr[3] = ((wv >> 6) & k_mask[0]) | k_magic;
+                } else if constexpr (BITS == 8) {
+                    const uint32_t w0 = cur.w[2 * p], w1 = cur.w[2 * p + 1];
+                    pr[0] = __builtin_amdgcn_perm(k_magic, w0, 0x05010500u);
+                    pr[1] = __builtin_amdgcn_perm(k_magic, w0, 0x05030502u);
+                    pr[2] = __builtin_amdgcn_perm(k_magic, w1, 0x05010500u);
+                    pr[3] = __builtin_amdgcn_perm(k_magic, w1, 0x05030502u);
+                } else {
+                    static_for<4>([&](auto I) {
+                        constexpr int i = decltype(I)::value;
+                        const uint32_t qa = extract_code<(p * 8 + 2 * i) * BITS, BITS, WPL>(cur.w);
+                        const uint32_t qb = extract_code<(p * 8 + 2 * i + 1) * BITS, BITS, WPL>(cur.w);
+                        pr[i] = ((qb << 16) | qa) | k_magic;
+                    });
+                }
+                constexpr int c0 = MULTI ? f16_pair_class<BITS>(4 * p + 0) : 0, c1 = MULTI ? f16_pair_class<BITS>(4 * p + 1) : 0;
+                constexpr int c2 = MULTI ? f16_pair_class<BITS>(4 * p + 2) : 0, c3 = MULTI ? f16_pair_class<BITS>(4 * p + 3) : 0;
+                dot[sr][c0] = dot2_x<XA>(pr[0], xv.x, dot[sr][c0]);
+                dot[sr][c1] = dot2_x<XA>(pr[1], xv.y, dot[sr][c1]);
+                dot[sr][c2] = dot2_x<XA>(pr[2], xv.z, dot[sr][c2]);
+                dot[sr][c3] = dot2_x<XA>(pr[3], xv.w, dot[sr][c3]);
+            } else {
+                // 8-bit codes with bf16 activations: (128 + q) is not exact in bf16, so fp32 FMA on converted codes
+                const float xf[8] = {__uint_as_float(xv.x << 16), __uint_as_float(xv.x & 0xFFFF0000u),
+                                     __uint_as_float(xv.y << 16), __uint_as_float(xv.y & 0xFFFF0000u),
+                                     __uint_as_float(xv.z << 16), __uint_as_float(xv.z & 0xFFFF0000u),
+                                     __uint_as_float(xv.w << 16), __uint_as_float(xv.w & 0xFFFF0000u)};
+                float dsum = dot[sr][0];
+                static_for<8>([&](auto E) {
+                    constexpr int e = decltype(E)::value;
+                    dsum = __builtin_fmaf((float)extract_code<(p * 8 + e) * BITS, BITS, WPL>(cur.w), xf[e], dsum);
+                });
+                dot[sr][0] = dsum;
+            }
+        });
+        float out = 0.0f;
+#pragma unroll
+        for (int sr = 0; sr < NSR; sr++) {
+            const float* const cell = sxs + ((size_t)c * NSR + sr) * NF * 64 + lane;
+            const float sx = cell[0];
+            float s, z;
+            const uint32_t szw = cur.sz[sr];
+            if constexpr (SBBF16) { s = __uint_as_float(szw << 16); z = __uint_as_float(szw & 0xFFFF0000u); }
+            else { s = f16_to_f32((uint16_t)(szw & 0xFFFFu)); z = f16_to_f32((uint16_t)(szw >> 16)); }
+            if constexpr (MULTI) {
+                float t = dot[sr][0];
+#pragma unroll
+                for (int cl = 1; cl < NCLS; cl++) t = __builtin_fmaf(dot[sr][cl], 1.0f / (float)(1 << f16_class_shift<BITS>(cl)), t);
+                t -= cell[64];
+                out = __builtin_fmaf(s, t, __builtin_fmaf(z, sx, out));
+            } else {
+                out += s * dot[sr][0] + (z - OFS * s) * sx;
+            }
+        }
+        return out;
+    };
+
+    float res = 0.0f;                                        // lane i parks the result of the wavefront's i-th row
+    auto pass_body = [&](uint32_t pass, auto ISSUE_T) {
+        constexpr bool ISSUE = decltype(ISSUE_T)::value;
+        float acc[BR];
+#pragma unroll
+        for (int j = 0; j < BR; j++) {
+            const char *cp = nullptr, *zp = nullptr;
+            if constexpr (ISSUE) row_ptrs((pass + 1) * BR + j, cp, zp);
+            acc[j] = 0.0f;
+            static_for<NCT>([&](auto C) {
+                acc[j] += step(ring[j][decltype(C)::value], C);
+                if constexpr (ISSUE) issue(cp, zp, decltype(C)::value, ring[j][decltype(C)::value]);
+            });
+            asm volatile("" ::: "memory");                  // the next row reads the activations from LDS again (registers stay free)
+        }
+        const float v = transpose_reduce<BR>(acc, lane);    // lane l holds the sum of row (l & (BR - 1)) of this pass
+        res = ((lane & ~(uint32_t)(BR - 1)) == pass * BR) ? v : res;
+    };
+    const uint32_t passes = (nrows + BR - 1) / BR;
+    for (uint32_t pass = 0; pass + 1 < passes; pass++) pass_body(pass, std::true_type{});
+    if (passes) pass_body(passes - 1, std::false_type{});
+
+    // ---- one coalesced store of the parked results (rows_per_wave <= 64) ------------------------------------
+    unsigned long long best = 0ull;
+    if (lane < nrows) {
+        const uint32_t row = row0 + lane;
+        if (seg_y) {
+            if (a.y_dtype == MI355Q_F32) ((float*)seg_y)[row] = res;
+            else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)seg_y)[row] = f32_to_bf16_rne(res);
+            else ((uint16_t*)seg_y)[row] = f32_to_f16_rne(res);
+        }
+        if (a.logits) a.logits[row] = res;
+        if constexpr (ARGMAX) {
+            if (res > -INFINITY) {                           // NaN and -inf never contribute
+                const uint32_t u = __float_as_uint(res + 0.0f);     // -0 -> +0
+                const uint32_t key = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+                best = ((unsigned long long)key << 32) | (unsigned long long)(0xFFFFFFFFu - row);
+            }
+        }
+    }
+    if constexpr (ARGMAX) {
+        // wavefront maximum of the packed (ordered value, ~row) key, workgroup maximum through LDS, one plain store
+        // per workgroup; argmax_finish_kernel picks the token from the partial keys
+        __shared__ unsigned long long s_best[WAVES];
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const uint32_t hi = (uint32_t)__shfl_xor((int)(best >> 32), off, 64);
+            const uint32_t lo = (uint32_t)__shfl_xor((int)(best & 0xFFFFFFFFull), off, 64);
+            const unsigned long long o = ((unsigned long long)hi << 32) | lo;
+            best = o > best ? o : best;
+        }
+        if (lane == 0) s_best[wave] = best;
+        __syncthreads();
+        if (tid == 0) {
+            unsigned long long m = s_best[0];
+#pragma unroll
+            for (int w2 = 1; w2 < WAVES; w2++) m = s_best[w2] > m ? s_best[w2] : m;
+            a.scratch[blockIdx.x] = m;
+        }
+    }
+}
+
+}  // namespace mi355q

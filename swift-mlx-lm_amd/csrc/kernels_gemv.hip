@@ -29,16 +29,17 @@ Geo geo_for(uint32_t bits) {
     }
 }
 
-size_t lds_bytes(const WView& w, int mt) {
+// Staged activations of mt rows: pairs, then per sub-run the sum of the activations and, in f16 arithmetic on
+// 2- and 4-bit codes, the class-weighted sum next to it.
+size_t lds_bytes(const WView& w, int mt, int xa) {
     const Geo g = geo_for(w.bits);
     const size_t kc = 64 * (size_t)g.cpl;
     const size_t nc = (w.k + kc - 1) / kc;
     const size_t sr = (size_t)g.cpl < w.group ? g.cpl : w.group;
     const size_t nsr = g.cpl / sr;
-    return (size_t)mt * nc * 64 * ((size_t)(g.cpl / 8) * 16 + nsr * 4);
+    const size_t nf = (xa == 1 && (w.bits == 2 || w.bits == 4)) ? 2 : 1;
+    return (size_t)mt * nc * 64 * ((size_t)(g.cpl / 8) * 16 + nsr * nf * 4);
 }
-
-int env_int(const char* name, int fallback) { return env_int_cached(name, fallback); }
 
 // Largest activation batch per launch (1, 2 or 4) whose staged activations fit the LDS budget.
 // Batches of 5 to 8 rows run as two launches: an 8-row variant of this kernel needs more registers
@@ -46,20 +47,46 @@ int env_int(const char* name, int fallback) { return env_int_cached(name, fallba
 int max_mt(const WView& w) {
     // q2 g16 carries four scale groups per lane chunk: its 4-row variant does not fit the register file
     for (int mt = (w.bits == 2 && w.group == 16) ? 2 : 4; mt >= 1; mt >>= 1)
-        if (lds_bytes(w, mt) <= kLdsBudget) return mt;
+        if (lds_bytes(w, mt, 1) <= kLdsBudget) return mt;
     return 0;
 }
 
-// Variant and launch shape for one call.  In tuning builds (MI355Q_GEMV_EXPERIMENT) environment
-// variables override the heuristics (MI355Q_GEMV_R, _WAVES, _DEPTH, _XREG, _ROWS_PER_WAVE,
-// _WAVES_PER_CU); product builds ignore them.
-GemvCfg choose(const mi355q_context* ctx, const WView& w, uint32_t m, bool argmax) {
+// Variant and launch shape for one call (measured on MI355X).
+GemvCfg choose(const mi355q_context* ctx, const WView& w, uint32_t m, bool argmax, int x_dtype) {
     GemvCfg c{};
     c.argmax = argmax;
+    c.xa = x_dtype == MI355Q_F16 ? 1 : 0;
     c.mt = m <= 1 ? 1 : m <= 2 ? 2 : 4;
     const Geo g = geo_for(w.bits);
     const size_t kc = 64 * (size_t)g.cpl;
     c.nc = (uint32_t)((w.k + kc - 1) / kc);
+    // One activation row and rows of 1, 2, 3, 4 or 7 K-steps: the static-structure kernel.  About 28 wavefronts per
+    // CU, each owning a whole number of passes of `br` rows; a wavefront whose share is at most eight K-steps takes
+    // it in one pass, every load issued up front.
+    if (c.mt == 1 && gemv_rows_has_format((int)w.bits, (int)w.group) && (!c.xa || gemv_rows_has_f16((int)w.bits, (int)w.group)) &&
+        (c.nc <= 4 || (c.nc == 7 && w.bits != 8))) {
+        const uint32_t target = (uint32_t)ctx->props.multiProcessorCount * 28u;
+        uint32_t rpw = (w.n + target - 1) / target;
+        if (rpw < 1) rpw = 1;
+        const int most = c.nc == 1 ? 8 : c.nc == 2 ? 4 : c.nc <= 4 ? 2 : 1;       // rows per pass: up to eight K-steps in flight
+        int br = 1;
+        while (br * 2 <= most && (uint32_t)(br * 2) <= rpw) br *= 2;
+        if (argmax && !gemv_rows_has_argmax((int)c.nc, br)) br = c.nc == 1 ? 4 : 2;   // the head's variants
+        rpw = (rpw + br - 1) / br * br;
+        if (rpw <= 64 && gemv_rows_has_shape((int)c.nc, br) && (!argmax || gemv_rows_has_argmax((int)c.nc, br))) {
+            c.rows = true;
+            c.nct = (int)c.nc;
+            c.br = br;
+            c.r = 1;
+            c.waves = gemv_rows_waves(c.nct);
+            c.rows_per_wave = rpw;
+            c.lds = lds_bytes(w, 1, c.xa);
+            const uint32_t rows_per_wg = rpw * (uint32_t)c.waves;
+            c.grid = (w.n + rows_per_wg - 1) / rows_per_wg;
+            if (c.grid == 0) c.grid = 1;
+            return c;
+        }
+    }
     const uint64_t weight_bytes = (uint64_t)w.n * (w.k / w.group) * (4 + w.group * w.bits / 8);
     const bool big = weight_bytes >= (24ull << 20);
     if (c.mt == 1) {
@@ -78,19 +105,11 @@ GemvCfg choose(const mi355q_context* ctx, const WView& w, uint32_t m, bool argma
         c.r = gemv_batch_rows((int)w.bits, (int)w.group, c.mt);
         c.waves = 4;
     }
-    const int er = env_int("MI355Q_GEMV_R", 0), ew = env_int("MI355Q_GEMV_WAVES", 0),
-              ed = env_int("MI355Q_GEMV_DEPTH", 0), ex = env_int("MI355Q_GEMV_XREG", -1);
-    if (er) c.r = er;
-    if (ew) c.waves = ew;
-    if (ex >= 0) c.xreg = ex ? (int)c.nc : 0;
-    c.lds = lds_bytes(w, c.mt);
-    // rows per wavefront: aim for `per_cu` wavefronts on every CU (measured best: 32 for M = 1),
-    // each owning a whole number of R-row steps
-    const uint32_t per_cu = (uint32_t)env_int("MI355Q_GEMV_WAVES_PER_CU", c.mt == 1 ? 32 : 16);
-    const uint32_t target = (uint32_t)ctx->props.multiProcessorCount * (per_cu ? per_cu : 16);
+    c.lds = lds_bytes(w, c.mt, c.xa);
+    // rows per wavefront: aim for 32 wavefronts on every CU at M = 1, 16 for batches, each owning a whole
+    // number of R-row steps
+    const uint32_t target = (uint32_t)ctx->props.multiProcessorCount * (c.mt == 1 ? 32u : 16u);
     uint32_t rpw = (w.n + target - 1) / target;
-    const int forced = env_int("MI355Q_GEMV_ROWS_PER_WAVE", 0);
-    if (forced > 0) rpw = (uint32_t)forced;
     rpw = (rpw + c.r - 1) / c.r * c.r;
     if (rpw < (uint32_t)c.r) rpw = c.r;
     c.rows_per_wave = rpw;
@@ -98,7 +117,6 @@ GemvCfg choose(const mi355q_context* ctx, const WView& w, uint32_t m, bool argma
     const uint32_t nsteps = rpw / (uint32_t)c.r * c.nc;
     if (c.mt == 1) c.depth = (nsteps >= 4 && (big || c.nc > 2)) ? 4 : 2;
     else c.depth = gemv_batch_depth((int)w.bits, (int)w.group, c.mt);
-    if (ed) c.depth = ed;
     const uint32_t rows_per_wg = rpw * (uint32_t)c.waves;
     c.grid = (w.n + rows_per_wg - 1) / rows_per_wg;
     if (c.grid == 0) c.grid = 1;
@@ -108,7 +126,7 @@ GemvCfg choose(const mi355q_context* ctx, const WView& w, uint32_t m, bool argma
 }  // namespace
 
 bool gemv_fast_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
-    if (w.layout != MI355Q_LAYOUT_PLANES || x_dtype != MI355Q_BF16) return false;
+    if (w.layout != MI355Q_LAYOUT_PLANES || (x_dtype != MI355Q_BF16 && x_dtype != MI355Q_F16)) return false;
     if (m < 1 || m > 8) return false;
     const Geo g = geo_for(w.bits);
     if (!g.cpl) return false;
@@ -120,23 +138,23 @@ bool gemv_fast_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stri
     return true;
 }
 
-GemvLaunchShape gemv_fast_shape(const mi355q_context* ctx, const WView& w, uint32_t m) {
+GemvLaunchShape gemv_fast_shape(const mi355q_context* ctx, const WView& w, uint32_t m, int x_dtype) {
     const int fit = max_mt(w);
     const uint32_t mm = (fit && m > (uint32_t)fit) ? (uint32_t)fit : m;
-    const GemvCfg c = choose(ctx, w, mm, false);
+    const GemvCfg c = choose(ctx, w, mm, false, x_dtype);
     GemvLaunchShape s;
     s.grid = c.grid;
     s.block = (uint32_t)c.waves * 64;
     s.lds_bytes = (uint32_t)c.lds;
     s.rows_per_workgroup = c.rows_per_wave * (uint32_t)c.waves;
-    s.kernel = "gemv_planes_kernel";
+    s.kernel = c.rows ? "gemv_rows_kernel" : "gemv_planes_kernel";
     return s;
 }
 
 // Up to three weights sharing K, format and activations in one launch.  `w[0]` supplies the format;
 // the caller has checked that the others match.
 mi355q_status launch_gemv_fast_multi(hipStream_t s, const mi355q_context* ctx, uint32_t count, const WView* w,
-                                     const void* x, void* const* y, const uint32_t* y_strides, int y_dtype,
+                                     const void* x, int x_dtype, void* const* y, const uint32_t* y_strides, int y_dtype,
                                      uint32_t m, uint32_t x_stride, float* logits_f32, int32_t* token_out,
                                      unsigned long long* argmax_scratch) {
     if (count < 1 || count > (uint32_t)kGemvMaxSegments)
@@ -156,7 +174,7 @@ mi355q_status launch_gemv_fast_multi(hipStream_t s, const mi355q_context* ctx, u
     // activation batches larger than what fits in LDS are processed in slices of `fit` rows
     for (uint32_t m0 = 0; m0 < m; m0 += (uint32_t)fit) {
         const uint32_t mm = (m - m0) < (uint32_t)fit ? (m - m0) : (uint32_t)fit;
-        GemvCfg c = choose(ctx, all, mm, argmax);
+        GemvCfg c = choose(ctx, all, mm, argmax, x_dtype);
         GemvArgs a{};
         uint32_t waves = 0;
         for (uint32_t i = 0; i < (uint32_t)kGemvMaxSegments; i++) {
@@ -178,8 +196,7 @@ mi355q_status launch_gemv_fast_multi(hipStream_t s, const mi355q_context* ctx, u
         a.x_stride = x_stride;
         a.code_stride = all.code_stride; a.sz_stride = all.sz_stride;
         a.nc = c.nc; a.rows_per_wave = c.rows_per_wave;
-        a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = all.sb_dtype;
-        a.dbg = (uint32_t)env_int("MI355Q_GEMV_DBG", 0);
+        a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = all.sb_dtype; a.x_dtype = (uint32_t)x_dtype;
         c.grid = grid;                        // whole wavefronts per matrix: a few more than rows / rows_per_wave
         if (argmax && grid > kArgmaxPartialCapacity)
             return fail(MI355Q_ERR_SHAPE, "the fused output head keeps one partial key per workgroup: %u workgroups exceed %u",
@@ -201,12 +218,12 @@ mi355q_status launch_gemv_fast_multi(hipStream_t s, const mi355q_context* ctx, u
     return MI355Q_OK;
 }
 
-mi355q_status launch_gemv_fast(hipStream_t s, const mi355q_context* ctx, const WView& w, const void* x, void* y,
-                               int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride, float* logits_f32,
+mi355q_status launch_gemv_fast(hipStream_t s, const mi355q_context* ctx, const WView& w, const void* x, int x_dtype,
+                               void* y, int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride, float* logits_f32,
                                int32_t* token_out, unsigned long long* argmax_scratch) {
     void* ys[1] = {y};
     const uint32_t strides[1] = {y_stride};
-    return launch_gemv_fast_multi(s, ctx, 1, &w, x, ys, strides, y_dtype, m, x_stride, logits_f32, token_out,
+    return launch_gemv_fast_multi(s, ctx, 1, &w, x, x_dtype, ys, strides, y_dtype, m, x_stride, logits_f32, token_out,
                                   argmax_scratch);
 }
 

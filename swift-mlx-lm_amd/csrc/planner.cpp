@@ -63,7 +63,7 @@ void plan_small_m(const mi355q_weight* w, uint32_t m, int x_dtype, uint32_t x_st
         s->lds_bytes = g.lds_bytes;
         s->rows_per_workgroup = 16;
     } else if (!forced && gemv_fast_eligible(v, x_dtype, m > 8 ? 8 : m, x_stride)) {
-        const GemvLaunchShape g = gemv_fast_shape(w->ctx, v, m > 8 ? 8 : m);
+        const GemvLaunchShape g = gemv_fast_shape(w->ctx, v, m > 8 ? 8 : m, x_dtype);
         std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_planes_q%u_g%u", (unsigned)w->fmt.bits,
                       w->fmt.group_size);
         s->grid[0] = g.grid;
