@@ -29,10 +29,12 @@ HBM_PEAK_GBPS = 8000.0            # MI355X published HBM3E bandwidth
 LAYER_SHAPES = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4096, 4096),
                 ("gate", 14336, 4096), ("up", 14336, 4096), ("down", 4096, 14336)]
 BITS, GROUP = 4, 64
-# HBM bytes per gate launch and per fused gate+up launch from the FETCH_SIZE and WRITE_SIZE counters, each scaled by what the
-# same counter reads for a plain copy of the same size (profiles/gemv_planes_q4_g64_gate_up_hbm_traffic_pmc.md).
-# Measured offline with the profiler; valid for the kernel variant named in `roofline.kernel`.
-TRAFFIC_BYTES = {"gate": 33260041, "gate_up": 66317409}
+MFMA_BF16_PEAK_TFLOPS = 2500.0    # MI355X published dense bf16 matrix-core peak
+# HBM bytes per launch from the FETCH_SIZE and WRITE_SIZE counters, each scaled by what the same counter reads for a
+# plain copy of the same size (profiles/gemv_rows_q4_g64_gate_up_hbm_traffic_pmc.md).  Measured offline with the
+# profiler: the figure only holds for the kernel and launch shape it was measured on, so it is keyed by both and the
+# line carries null when the library picks anything else.
+TRAFFIC_BYTES = {("gemv_rows_kernel", "gate_up", 3584, 256): None, ("gemv_rows_kernel", "gate", 1792, 256): None}
 
 
 def log(*a):
@@ -64,7 +66,8 @@ def cpu_baseline(seconds: float):
     n, k = 8192, 2048
     words, s, z = oracle.quantize_affine(kat.seeded_weights(11, n, k), BITS, GROUP, oracle.BF16)
     x = oracle.bf16_to_f32(oracle.bf16_from_f32(kat.seeded_activations(12, 1, k))).reshape(1, k)
-    cores = min(os.cpu_count() or 1, 16)
+    host_cores = os.cpu_count() or 1
+    cores = min(host_cores, 16)           # the GPU box gives one job 16 cores' worth of CPU time, whatever it reports
     oracle.qgemm_planes_ref_f32(BITS, GROUP, words, s, z, oracle.BF16, x, n, k, threads=cores)  # warm-up
     passes, t0 = 0, time.perf_counter()
     while True:
@@ -74,16 +77,18 @@ def cpu_baseline(seconds: float):
         if dt >= seconds or passes >= 20000:
             break
     gbps = weight_bytes(n, k) * passes / dt / 1e9
-    return {"value": round(gbps, 4), "unit": "GB/s", "cores": cores, "kind": "port",
+    return {"value": round(gbps, 4), "unit": "GB/s", "cores": cores, "host_cores_reported": host_cores, "kind": "port",
             "sample": f"{passes} passes of config 0 (q4 g64 2048->8192, M=1, 9437184 weight bytes each) "
-                      f"in {dt:.1f} s, rows split over {cores} pthreads"}
+                      f"in {dt:.1f} s, rows split over {cores} pthreads (the host reports {host_cores} cores; "
+                      f"a job's CPU share on the GPU box is 16)"}
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=320)
-    ap.add_argument("--warmup", type=int, default=32)
+    ap.add_argument("--steps", type=int, default=320,
+                    help="timed steps; at least 256 are timed whatever is asked (rounded up to whole passes over the layer copies)")
+    ap.add_argument("--warmup", type=int, default=32, help="untimed warm-up steps; at least 32 are run")
     ap.add_argument("--layers", type=int, default=32, help="distinct weight copies resident in HBM")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -126,6 +131,11 @@ def main():
     log(f"resident: {a.layers} layers x {layer_bytes} B = {a.layers * layer_bytes / 1e9:.2f} GB")
 
     stream = ctx.stream_create()
+    # The headline must not depend on what the driver passes: at least 256 timed steps (1024 launches of the 4-launch
+    # schedule) after at least 32 warm-up steps, in whole passes over the resident layer copies.
+    steps = max(a.steps, 256)
+    steps = (steps + a.layers - 1) // a.layers * a.layers
+    warmup = max(a.warmup, 32)
 
     # ---- parity gate: no number is reported from a run whose outputs were not verified
     if not a.skip_parity:
@@ -166,7 +176,8 @@ def main():
                     lin(name, k)
         return plan
 
-    results = {}
+    results, spreads = {}, {}
+    group = 8                                              # steps per event pair of the spread measurement
     for label, fused in (("7-launch", False), ("4-launch", True)):
         plan = build_plan(fused)
         per_layer = len(plan) // a.layers
@@ -174,25 +185,52 @@ def main():
         def step(i, plan=plan, per_layer=per_layer):
             plan.encode(stream, (i % a.layers) * per_layer, per_layer)
 
-        for i in range(a.warmup):
+        for i in range(warmup):
             step(i)
         ctx.synchronize(stream)
-        ms = time_region(ctx, step, a.steps, stream)
+        ms = time_region(ctx, step, steps, stream)
         ctx.synchronize(stream)
         results[label + " stream"] = ms
-        log(f"{label} stream replay: {ms * 1e3:.2f} us/step, {layer_bytes / (ms * 1e-3) / 1e9:.1f} GB/s")
+        log(f"{label} stream replay: {ms * 1e3:.2f} us/step over {steps} steps, {layer_bytes / (ms * 1e-3) / 1e9:.1f} GB/s")
+        # spread: one HIP event pair around every `group` consecutive steps (a pair costs 2-3 us, so 0.3 us per step)
+        per_group = []
+        ea, eb = ctx.event_create(), ctx.event_create()
+        for g in range(steps // group):
+            ctx.event_record(ea, stream)
+            for i in range(group):
+                step(g * group + i)
+            ctx.event_record(eb, stream)
+            ctx.event_synchronize(eb)
+            per_group.append(ctx.event_elapsed_ms(ea, eb) / group)
+        ctx.event_destroy(ea); ctx.event_destroy(eb)
+        per_group.sort()
+        n_g = len(per_group)
+        spreads[label + " stream"] = {"median_us": round(per_group[n_g // 2] * 1e3, 2), "p10_us": round(per_group[n_g // 10] * 1e3, 2),
+                                      "p90_us": round(per_group[n_g * 9 // 10] * 1e3, 2), "samples": n_g, "steps_per_sample": group}
         # the same plan captured once into a HIP graph (one launch per pass over all layers)
-        if a.steps % a.layers == 0:
-            plan.graph_build(stream)
-            for _ in range(2):
-                plan.graph_launch(stream)
-            ctx.synchronize(stream)
-            passes = a.steps // a.layers
-            ms_pass = time_region(ctx, lambda i, plan=plan: plan.graph_launch(stream), passes, stream)
-            ctx.synchronize(stream)
-            results[label + " hip-graph"] = ms_pass / a.layers
-            log(f"{label} graph replay:  {ms_pass / a.layers * 1e3:.2f} us/step, "
-                f"{layer_bytes / (ms_pass / a.layers * 1e-3) / 1e9:.1f} GB/s")
+        plan.graph_build(stream)
+        for _ in range(2):
+            plan.graph_launch(stream)
+        ctx.synchronize(stream)
+        passes = steps // a.layers
+        ms_pass = time_region(ctx, lambda i, plan=plan: plan.graph_launch(stream), passes, stream)
+        ctx.synchronize(stream)
+        results[label + " hip-graph"] = ms_pass / a.layers
+        per_pass = []
+        ea, eb = ctx.event_create(), ctx.event_create()
+        for g in range(max(passes, 16)):
+            ctx.event_record(ea, stream)
+            plan.graph_launch(stream)
+            ctx.event_record(eb, stream)
+            ctx.event_synchronize(eb)
+            per_pass.append(ctx.event_elapsed_ms(ea, eb) / a.layers)
+        ctx.event_destroy(ea); ctx.event_destroy(eb)
+        per_pass.sort()
+        n_p = len(per_pass)
+        spreads[label + " hip-graph"] = {"median_us": round(per_pass[n_p // 2] * 1e3, 2), "p10_us": round(per_pass[n_p // 10] * 1e3, 2),
+                                         "p90_us": round(per_pass[n_p * 9 // 10] * 1e3, 2), "samples": n_p, "steps_per_sample": a.layers}
+        log(f"{label} graph replay:  {ms_pass / a.layers * 1e3:.2f} us/step, "
+            f"{layer_bytes / (ms_pass / a.layers * 1e-3) / 1e9:.1f} GB/s; spread {spreads[label + ' hip-graph']}")
         plan.destroy()
     mode = min(results, key=results.get)
     ms_step = results[mode]
@@ -213,7 +251,7 @@ def main():
                 p1.add_batched_linear([L[n] for n in names], xdev[k], pkg.BF16, [ydev[n] for n in names], pkg.BF16, 1)
         p1.encode(stream)
         ctx.synchronize(stream)
-        reps = max(1, max(a.steps, 4 * a.layers) // a.layers)
+        reps = max(1, max(steps, 8 * a.layers) // a.layers)      # at least 256 launches per figure
         ms = time_region(ctx, lambda i: p1.encode(stream), reps, stream) / a.layers
         # the same launches replayed from a HIP graph: for the small projections the host cannot issue stream
         # launches as fast as the GPU retires them, so the stream figure measures the host there
@@ -252,9 +290,7 @@ def main():
                         for _ in range(n_t16)]
             batch_sweep[lname] = {}
             for m in ((1, 2, 4, 8) if lname == "planes" else (1, 2, 4, 8, 16)):    # the tile kernel takes 16 rows a launch
-                xm = {k: ctx.alloc(m * k * 2) for k in (4096, 14336)}
-                for k in xm:
-                    ctx.fill(xm[k], 0x3C003C00, stream)
+                xm = {k: ctx.upload(oracle.bf16_from_f32(kat.seeded_activations(900 + m, m, k))) for k in (4096, 14336)}   # N(0,1)
                 ym = {name: ctx.alloc(m * n * 2) for name, n, _ in LAYER_SHAPES}
                 pl = pkg.DispatchPlan(ctx)
                 for L in pool:
@@ -265,13 +301,13 @@ def main():
                     pl.add_linear(L["down"], xm[14336], pkg.BF16, ym["down"], pkg.BF16, m)
                 pl.encode(stream)
                 ctx.synchronize(stream)
-                ms = time_region(ctx, lambda i: pl.encode(stream), 8, stream) / len(pool)
+                ms = time_region(ctx, lambda i: pl.encode(stream), 32, stream) / len(pool)     # 256 steps
                 batch_sweep[lname][f"M={m}"] = {"us_per_step": round(ms * 1e3, 2),
                                                 "GBps": round(layer_bytes / (ms * 1e-3) / 1e9, 1)}
                 pl.destroy()
                 for b in list(xm.values()) + list(ym.values()):
                     b.free()
-            log(f"  batch sweep {lname}: " + ", ".join(f"{k} {v['us_per_step']} us" for k, v in batch_sweep[lname].items()))
+            log(f"  batch sweep {lname} (N(0,1) activations): " + ", ".join(f"{k} {v['us_per_step']} us" for k, v in batch_sweep[lname].items()))
             if lname == "tile16":
                 for L in pool:
                     for w in L.values():
@@ -281,7 +317,16 @@ def main():
     dom = "gate_up" if mode.startswith("4-launch") else "gate"
     dom_bytes = per_shape[dom]["weight_bytes"]
     achieved = per_shape[dom]["GBps"]
-    dom_step = layers[0]["gate"].plan_decode_step(1)
+    # the kernel and launch shape of that launch, from the plan record of the step that ran it
+    pd = pkg.DispatchPlan(ctx)
+    if dom == "gate_up":
+        pd.add_batched_linear([layers[0]["gate"], layers[0]["up"]], xdev[4096], pkg.BF16, [ydev["gate"], ydev["up"]], pkg.BF16, 1)
+    else:
+        pd.add_linear(layers[0]["gate"], xdev[4096], pkg.BF16, ydev["gate"], pkg.BF16, 1)
+    dom_rec = pd.step(0)[0]
+    dom_kernel, dom_grid, dom_block = dom_rec.device_kernel, int(dom_rec.grid[0]), int(dom_rec.block[0])
+    pd.destroy()
+    traffic = TRAFFIC_BYTES.get((dom_kernel.split("_q")[0] if False else dom_kernel, dom, dom_grid, dom_block))
 
     # ---- plain copy of the gate tensor's size: the calibration launch for the HBM counters ------
     gate_bytes = weight_bytes(14336, 4096)
@@ -458,15 +503,35 @@ def main():
         for k_, v_ in next_rows.items():
             log(f"  {k_}: {v_}")
 
-    # ---- secondary figure: the prefill GEMM of the same layer's gate projection (not the metric)
-    prefill = None
+    # ---- the second half of the metric: the prefill GEMM (benchmark config 3) on N(0,1) activations ------------
+    # both MLP shapes at M = 128, 512, 2048, as dispatched (tile shape, K split and route are the library's choice),
+    # over four rotating weight copies; the M = 2048 gate projection is the roofline figure.
+    prefill, roofline_prefill = None, None
     if not a.no_prefill:
+        sweep = {}
+        for name, n, k in (("gate 4096->14336", 14336, 4096), ("down 14336->4096", 4096, 14336)):
+            wts = [L["gate" if n == 14336 else "down"] for L in layers[:4]]
+            for mm in (128, 512, 2048):
+                xb = ctx.upload(oracle.bf16_from_f32(kat.seeded_activations(500 + mm, mm, k)))        # N(0,1)
+                yb = ctx.alloc(mm * n * 2)
+                for i in range(4):
+                    ctx.qgemm(wts[i], xb, pkg.BF16, yb, pkg.BF16, mm, 0, 0, 0, stream)
+                ctx.synchronize(stream)
+                reps = 24 if mm == 2048 else 48
+                ms = time_region(ctx, lambda i: ctx.qgemm(wts[i % len(wts)], xb, pkg.BF16, yb, pkg.BF16, mm, 0, 0, 0, stream), reps, stream)
+                steps_p = wts[0].plan_prefill_steps(mm, k)
+                sweep[f"{name} M={mm}"] = {"us": round(ms * 1e3, 1), "TFLOPs": round(2.0 * mm * n * k / (ms * 1e-3) / 1e12, 1),
+                                           "route": " + ".join(st.device_kernel for st in steps_p)}
+                xb.free(); yb.free()
+        sweep["activations"] = "N(0,1) bf16, seeded"
+        log("  prefill sweep (N(0,1)): " + ", ".join(f"{k2} {v['us']} us ({v['TFLOPs']} TFLOP/s, {v['route']})"
+                                                   for k2, v in sweep.items() if isinstance(v, dict)))
+        # the same M = 2048 gate launch on the fused kernel with the in-kernel clock probe (what clock the matrix cores
+        # held), and on constant activations as a labelled aside (the part clocks higher when operand bits do not toggle)
         m = 2048
         xg = ctx.upload(oracle.bf16_from_f32(kat.seeded_activations(5, m, 4096)))
         yg = ctx.alloc(m * 14336 * 2)
         wg = layers[0]["gate"]
-        ctx.qgemm(wg, xg, pkg.BF16, yg, pkg.BF16, m, 0, 0, pkg.FLAG_FORCE_MFMA, stream)
-        ctx.synchronize(stream)
         probe = pkg.FLAG_FORCE_MFMA | pkg.FLAG_PROBE_CLOCK
 
         def gemm_figure(xbuf):
@@ -476,36 +541,25 @@ def main():
             return ms, ctx.clock_probe_ghz()
 
         ms_g, ghz = gemm_figure(xg)
-        # the same launch on constant activations: the part lowers its clock under matrix-core load by an amount
-        # that depends on how much the operand bits toggle, so this bounds what the N(0,1) figure loses to the clock
         xc = ctx.upload(np.full((m, 4096), 0x3F80, np.uint16))
         ms_c, ghz_c = gemm_figure(xc)
-        xc.free()
+        xc.free(); xg.free(); yg.free()
         flops = 2.0 * m * 14336 * 4096
-        prefill = {"m": m, "us": round(ms_g * 1e3, 1), "TFLOPs": round(flops / (ms_g * 1e-3) / 1e12, 1),
-                   "shader_clock_GHz": round(ghz, 3),
-                   "mfma_peak_at_that_clock_TFLOPs": round(2500.0 * ghz / 2.4, 1),
-                   "constant_activations": {"us": round(ms_c * 1e3, 1), "TFLOPs": round(flops / (ms_c * 1e-3) / 1e12, 1),
-                                            "shader_clock_GHz": round(ghz_c, 3)}}
-        log(f"  prefill GEMM M={m} 4096->14336: {prefill['us']} us, {prefill['TFLOPs']} TFLOP/s at {ghz:.3f} GHz "
-            f"(bf16 MFMA peak 2500 at 2.4 GHz); constant activations: {prefill['constant_activations']['TFLOPs']} TFLOP/s "
-            f"at {ghz_c:.3f} GHz")
-        xg.free(); yg.free()
-        # benchmark config 3: both MLP shapes at M = 128, 512, 2048 (as dispatched: tile shape and K split are the library's choice)
-        sweep = {}
-        for name, n, k in (("gate 4096->14336", 14336, 4096), ("down 14336->4096", 4096, 14336)):
-            wts = [L["gate" if n == 14336 else "down"] for L in layers[:4]]
-            for mm in (128, 512, 2048):
-                xb = ctx.alloc(mm * k * 2); yb = ctx.alloc(mm * n * 2)
-                ctx.fill(xb, 0x3C003C00, stream)
-                ctx.qgemm(wts[0], xb, pkg.BF16, yb, pkg.BF16, mm, 0, 0, 0, stream)
-                ctx.synchronize(stream)
-                ms = time_region(ctx, lambda i: ctx.qgemm(wts[i % len(wts)], xb, pkg.BF16, yb, pkg.BF16, mm, 0, 0, 0, stream), 8, stream)
-                sweep[f"{name} M={mm}"] = {"us": round(ms * 1e3, 1), "TFLOPs": round(2.0 * mm * n * k / (ms * 1e-3) / 1e12, 1)}
-                xb.free(); yb.free()
-        sweep["activations"] = "constant (the part clocks higher on them than on N(0,1) data: compare the two M=2048 gate figures above)"
-        prefill["config3"] = sweep
-        log("  prefill sweep: " + ", ".join(f"{k2} {v['us']} us" for k2, v in sweep.items() if isinstance(v, dict)))
+        prefill = {"config3": sweep,
+                   "fused_kernel_m2048_gate": {"us": round(ms_g * 1e3, 1), "TFLOPs": round(flops / (ms_g * 1e-3) / 1e12, 1),
+                                               "shader_clock_GHz": round(ghz, 3)},
+                   "aside_constant_activations_fused_kernel": {"us": round(ms_c * 1e3, 1), "TFLOPs": round(flops / (ms_c * 1e-3) / 1e12, 1),
+                                                               "shader_clock_GHz": round(ghz_c, 3)}}
+        log(f"  fused kernel M={m} gate: {prefill['fused_kernel_m2048_gate']}; constant activations (aside): "
+            f"{prefill['aside_constant_activations_fused_kernel']}")
+        best = sweep["gate 4096->14336 M=2048"]
+        roofline_prefill = {"bound": "mfma", "achieved": best["TFLOPs"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                            "frac": round(best["TFLOPs"] / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                            "kernel": best["route"], "m": 2048, "shape": "4096->14336", "us": best["us"],
+                            "flops": flops, "activations": "N(0,1) bf16",
+                            "down_14336_4096": {"TFLOPs": sweep["down 14336->4096 M=2048"]["TFLOPs"],
+                                                "frac": round(sweep["down 14336->4096 M=2048"]["TFLOPs"] / MFMA_BF16_PEAK_TFLOPS, 4),
+                                                "kernel": sweep["down 14336->4096 M=2048"]["route"]}}
 
     cpu = None if a.no_cpu else cpu_baseline(a.cpu_seconds)
 
@@ -514,8 +568,8 @@ def main():
         "value": round(value, 1),
         "unit": "GB/s",
         "n_gpus": 1,
-        "steps": a.steps,
-        "warmup": a.warmup,
+        "steps": steps,
+        "warmup": warmup,
         "ms_per_step": round(ms_step, 6),
         "higher_is_better": True,
         "scaling": "weak",
@@ -526,17 +580,20 @@ def main():
         "config": {"workload": "Llama-3-8B decode layer sweep (benchmark config 1), M=1: q,k,v,o,gate,up,down "
                                "GEMVs per step", "bits": BITS, "group_size": GROUP,
                    "weight_bytes_per_step": layer_bytes, "layers_resident": a.layers,
-                   "replay": mode, "replay_GBps": replay_gbps,
+                   "replay": mode, "replay_GBps": replay_gbps, "step_time_spread": spreads[mode],
+                   "step_time_spread_all": spreads, "steps_asked": a.steps, "warmup_asked": a.warmup,
                    "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2), "per_shape": per_shape,
                    "batch_sweep": batch_sweep, "other_configs": other, "staf_blocks_in_place_step": staf_step, "next_rows": next_rows,
                    "stream_read_probe": stream_read,
                    "prefill_gemm_gate": prefill},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": TRAFFIC_BYTES[dom],
-                     "algorithmic_bytes": dom_bytes,
-                     "kernel": f"{dom_step.device_kernel}: {dom} launch of the {mode} schedule, 4096->"
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+                     "algorithmic_bytes": dom_bytes, "us": per_shape[dom]["us"],
+                     "kernel": f"{dom_kernel} grid {dom_grid} x {dom_block}: {dom} launch of the {mode} schedule, 4096->"
                                f"{dom_bytes // weight_bytes(1, 4096)} rows, {dom_bytes} weight bytes/launch"},
     }
+    if roofline_prefill is not None:
+        out["roofline_prefill"] = roofline_prefill
     if cpu is not None:
         out["cpu_baseline"] = cpu
     print(json.dumps(out), flush=True)

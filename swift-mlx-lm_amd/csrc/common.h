@@ -186,6 +186,8 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
 mi355q_status dispatch_output_head(mi355q_context* ctx, hipStream_t s, const mi355q_weight* w, const void* x,
                                    int x_dtype, float* logits, int32_t* token, uint32_t flags);
 int env_int_cached(const char* name, int fallback);
+void plan_shared_launch_shape(const mi355q_weight* const* ws, uint32_t count, uint32_t m, int x_dtype, uint32_t x_stride,
+                              mi355q_step* s);
 
 // MFMA GEMM (kernels_gemm.hip)
 struct GemmLaunchShape {

@@ -90,8 +90,9 @@ constexpr bool gemv_rows_has_shape(int nct, int br) {
     return (nct == 1 && (br == 1 || br == 2 || br == 4 || br == 8)) || (nct == 2 && (br == 1 || br == 2 || br == 4)) ||
            ((nct == 3 || nct == 4) && (br == 1 || br == 2)) || (nct == 7 && br == 1);
 }
-// wavefronts per workgroup: the longer the row, the more wavefronts share one staged copy of the activations
-constexpr int gemv_rows_waves(int nct) { return nct <= 2 ? 4 : nct <= 4 ? 8 : 16; }
+// wavefronts per workgroup: four (measured best for rows of up to four K-steps at every bit width: with eight or
+// sixteen, more wavefronts wait at the staging barrier), eight for rows of seven K-steps, whose staged copy is 28 KiB
+constexpr int gemv_rows_waves(int nct) { return nct <= 4 ? 4 : 8; }
 
 template <int BITS> struct GemvGeo;
 template <> struct GemvGeo<2> { static constexpr int WPL = 4, CPL = 64; static constexpr bool PAIRS = true; };

@@ -60,19 +60,21 @@ GemvCfg choose(const mi355q_context* ctx, const WView& w, uint32_t m, bool argma
     const Geo g = geo_for(w.bits);
     const size_t kc = 64 * (size_t)g.cpl;
     c.nc = (uint32_t)((w.k + kc - 1) / kc);
-    // One activation row and rows of 1, 2, 3, 4 or 7 K-steps: the static-structure kernel.  About 28 wavefronts per
-    // CU, each owning a whole number of passes of `br` rows; a wavefront whose share is at most eight K-steps takes
-    // it in one pass, every load issued up front.
+    // One activation row and rows of 1, 2, 3, 4 or 7 K-steps: the static-structure kernel.  A wavefront takes two rows
+    // (four of one K-step) in one pass, every load issued up front, fewer while that would leave less than sixteen
+    // wavefronts per CU (measured, q4 g64: 28672 rows of two K-steps 12.1-12.3 us with two rows per wavefront,
+    // 12.4-14.0 with four, 13.8-14.1 with one; 14336 rows 7.5 / 8.2 / 8.0 us; 4096 rows 4.2 us either way; 14336 rows
+    // of four K-steps, q8 g32: 12.2 us with two rows, 14.4 with one; q6 g64 10.0 / 10.1; q3 g64 8.1 / 8.8).
     if (c.mt == 1 && gemv_rows_has_format((int)w.bits, (int)w.group) && (!c.xa || gemv_rows_has_f16((int)w.bits, (int)w.group)) &&
         (c.nc <= 4 || (c.nc == 7 && w.bits != 8))) {
-        const uint32_t target = (uint32_t)ctx->props.multiProcessorCount * 28u;
-        uint32_t rpw = (w.n + target - 1) / target;
-        if (rpw < 1) rpw = 1;
-        const int most = c.nc == 1 ? 8 : c.nc == 2 ? 4 : c.nc <= 4 ? 2 : 1;       // rows per pass: up to eight K-steps in flight
-        int br = 1;
-        while (br * 2 <= most && (uint32_t)(br * 2) <= rpw) br *= 2;
+        const uint32_t least_waves = (uint32_t)ctx->props.multiProcessorCount * 16u;
+        uint32_t rpw = c.nc == 1 ? 4 : c.nc <= 4 ? 2 : 1;
+        while (rpw > 1 && w.n / rpw < least_waves) rpw >>= 1;
+        int br = (int)rpw;                                                          // one pass
         if (argmax && !gemv_rows_has_argmax((int)c.nc, br)) br = c.nc == 1 ? 4 : 2;   // the head's variants
         rpw = (rpw + br - 1) / br * br;
+        // very tall matrices: more passes rather than more than 65535 workgroups
+        while ((w.n + rpw * 4 - 1) / (rpw * 4) > 65535u && rpw + br <= 64) rpw += br;
         if (rpw <= 64 && gemv_rows_has_shape((int)c.nc, br) && (!argmax || gemv_rows_has_argmax((int)c.nc, br))) {
             c.rows = true;
             c.nct = (int)c.nc;

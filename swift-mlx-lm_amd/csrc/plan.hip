@@ -160,6 +160,7 @@ mi355q_status mi355q_plan_add_batched_linear(mi355q_plan* plan, uint32_t count, 
         st.record = two[0];
     }
     if (rc != MI355Q_OK) return rc;
+    if (m <= 8) plan_shared_launch_shape(weights, count, m, x_dtype, st.xs, &st.record);   // one launch over the rows of all matrices
     std::snprintf(st.record.kernel_family, sizeof st.record.kernel_family, "batched%uQ%uG%u", count,
                   (unsigned)weights[0]->fmt.bits, weights[0]->fmt.group_size);
     plan->steps.push_back(st);

@@ -64,7 +64,8 @@ void plan_small_m(const mi355q_weight* w, uint32_t m, int x_dtype, uint32_t x_st
         s->rows_per_workgroup = 16;
     } else if (!forced && gemv_fast_eligible(v, x_dtype, m > 8 ? 8 : m, x_stride)) {
         const GemvLaunchShape g = gemv_fast_shape(w->ctx, v, m > 8 ? 8 : m, x_dtype);
-        std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_planes_q%u_g%u", (unsigned)w->fmt.bits,
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "%s_q%u_g%u",
+                      std::strcmp(g.kernel, "gemv_rows_kernel") == 0 ? "gemv_rows" : "gemv_planes", (unsigned)w->fmt.bits,
                       w->fmt.group_size);
         s->grid[0] = g.grid;
         s->block[0] = g.block;
@@ -90,6 +91,32 @@ void plan_small_m(const mi355q_weight* w, uint32_t m, int x_dtype, uint32_t x_st
 }
 
 }  // namespace
+
+namespace mi355q {
+
+// Launch shape of a shared launch (2 or 3 projections, one set of activations): the rows of all matrices together.
+void plan_shared_launch_shape(const mi355q_weight* const* ws, uint32_t count, uint32_t m, int x_dtype, uint32_t x_stride,
+                              mi355q_step* s) {
+    WView all = ws[0]->view();
+    uint64_t total = 0;
+    for (uint32_t i = 0; i < count; i++) {
+        const WView v = ws[i]->view();
+        if (v.layout != MI355Q_LAYOUT_PLANES || !gemv_fast_eligible(v, x_dtype, m > 8 ? 8 : m, x_stride)) return;
+        total += v.n;
+    }
+    if (m > 8 || total > 0xFFFFFFFFull) return;
+    all.n = (uint32_t)total;
+    const GemvLaunchShape g = gemv_fast_shape(ws[0]->ctx, all, m, x_dtype);
+    s->grid[0] = g.grid;
+    s->block[0] = g.block;
+    s->lds_bytes = g.lds_bytes;
+    s->rows_per_workgroup = g.rows_per_workgroup;
+    std::snprintf(s->device_kernel, sizeof s->device_kernel, "%s_q%u_g%u",
+                  std::strcmp(g.kernel, "gemv_rows_kernel") == 0 ? "gemv_rows" : "gemv_planes", (unsigned)ws[0]->fmt.bits,
+                  ws[0]->fmt.group_size);
+}
+
+}  // namespace mi355q
 
 extern "C" {
 

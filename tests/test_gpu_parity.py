@@ -375,7 +375,7 @@ def test_decode_and_prefill_plan_records(pkg, ctx):
     assert st.shape_family == "input20488192Dense" and st.reference_simdgroups == 8
     assert (st.input_dimension, st.output_dimension) == (2048, 8192)
     assert st.weight_bytes == 9_437_184 and st.flops == 2 * 2048 * 8192
-    assert st.device_kernel.startswith("gemv_planes") and st.block[0] in (256, 512) and st.grid[0] >= 1
+    assert st.device_kernel in ("gemv_rows_q4_g64", "gemv_planes_q4_g64") and st.block[0] in (256, 512) and st.grid[0] >= 1
     forced = w.plan_decode_step(1, flags=pkg.FLAG_FORCE_GENERIC)
     assert forced.used_fallback and forced.fallback_reason == "disabledByEnvironment"
     assert forced.device_kernel == "gemv_generic" and forced.grid[:2] == (2048, 1)
