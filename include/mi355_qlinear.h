@@ -327,6 +327,21 @@ MI355Q_API mi355q_status mi355q_lmhead_argmax(mi355q_context* ctx, void* stream,
                                               mi355q_dtype x_dtype, float* logits_f32_dev,
                                               int32_t* token_out_dev, uint32_t flags);
 
+/* mi355q_lmhead_argmax for callers that must not allocate.  No counterpart in the reference: it is for code that
+ * runs under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc.  Same arguments, kernels
+ * and results as mi355q_lmhead_argmax; the one partial key per workgroup that the head launch leaves for its
+ * finishing launch lives in a device array of the library image (258 KiB per GPU, held until the process ends)
+ * instead of the context's allocation, and the call makes no hipMalloc, hipFree or other allocating call.
+ * Limit: a head launch of more than mi355q_lmhead_argmax_static_capacity() = 32768 workgroups (524288 rows of up to
+ * 2048 4-bit codes, 262144 rows of up to 4096) is refused with MI355Q_ERR_SHAPE.  Every call on a GPU shares that
+ * GPU's array and overwrites the keys it uses (nothing has to be cleared between calls: a call reads back only the
+ * keys its own launch wrote): calls that overlap in time on one GPU race, whatever their contexts and streams. */
+MI355Q_API mi355q_status mi355q_lmhead_argmax_static(mi355q_context* ctx, void* stream,
+                                                     const mi355q_weight* w, const void* x_dev,
+                                                     mi355q_dtype x_dtype, float* logits_f32_dev,
+                                                     int32_t* token_out_dev, uint32_t flags);
+MI355Q_API uint32_t mi355q_lmhead_argmax_static_capacity(void);
+
 /* ------------------------------------------------------------------------------------------
  * Planner mirror: launch shapes, kernel selection and the quantization-plan record
  * ---------------------------------------------------------------------------------------- */

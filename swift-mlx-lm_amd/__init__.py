@@ -155,6 +155,8 @@ def library() -> C.CDLL:
         "mi355q_argmax": (i32, [vp, vp, vp, C.c_int, u32, vp]),
         "mi355q_embedding_lookup": (i32, [vp, vp, vp, vp, u32, vp, C.c_int, u32, C.c_int, C.c_float]),
         "mi355q_lmhead_argmax": (i32, [vp, vp, vp, vp, C.c_int, vp, vp, u32]),
+        "mi355q_lmhead_argmax_static": (i32, [vp, vp, vp, vp, C.c_int, vp, vp, u32]),
+        "mi355q_lmhead_argmax_static_capacity": (u32, []),
         "mi355q_shape_family_resolve": (i32, [u32, u32, P(i32), P(u32), P(u32), C.c_char_p, sz]),
         "mi355q_plan_create": (i32, [vp, P(vp)]),
         "mi355q_plan_destroy": (i32, [vp]),
@@ -835,3 +837,8 @@ class Context:
     def lmhead_argmax(self, w: PackedWeight, x, x_dtype, logits_f32, token_out, flags=0, stream=0):
         _check(library().mi355q_lmhead_argmax(self.handle, stream, w.handle, self._ptr(x), x_dtype,
                                               self._ptr(logits_f32), self._ptr(token_out), flags))
+
+    def lmhead_argmax_static(self, w: PackedWeight, x, x_dtype, logits_f32, token_out, flags=0, stream=0):
+        """The same head through the entry point that allocates nothing (its partial keys live in the library image)."""
+        _check(library().mi355q_lmhead_argmax_static(self.handle, stream, w.handle, self._ptr(x), x_dtype,
+                                                     self._ptr(logits_f32), self._ptr(token_out), flags))

@@ -57,9 +57,9 @@ mi355q_status run_small_m(mi355q_context* ctx, hipStream_t s, const mi355q_weigh
         if (!generic && gemv_tile16_eligible(v, x_dtype, mm, xs) && (uintptr_t)xp % 16 == 0) {
             void* yv[1] = {yp};
             const uint32_t strides[1] = {ys};
-            st = launch_gemv_tile16_multi(s, ctx, 1, &v, xp, yv, strides, y_dtype, mm, xs, nullptr, nullptr, nullptr);
+            st = launch_gemv_tile16_multi(s, ctx, 1, &v, xp, yv, strides, y_dtype, mm, xs, nullptr, nullptr, HeadKeys{});
         } else if (!generic && gemv_fast_eligible(v, x_dtype, mm, xs) && (uintptr_t)xp % 16 == 0) {
-            st = launch_gemv_fast(s, ctx, v, xp, x_dtype, yp, y_dtype, mm, xs, ys, nullptr, nullptr, nullptr);
+            st = launch_gemv_fast(s, ctx, v, xp, x_dtype, yp, y_dtype, mm, xs, ys, nullptr, nullptr, HeadKeys{});
         } else if (!generic && gemv_staf_eligible(v, x_dtype, mm, xs) && (uintptr_t)xp % 16 == 0) {
             st = launch_gemv_staf(s, ctx, v, xp, yp, y_dtype, mm, xs, ys);
         } else {
@@ -145,12 +145,12 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
         in_place = in_place && gemv_staf_eligible(views[i], x_dtype, m, xs);
     }
     if (fused && (uintptr_t)x % 16 == 0)
-        return launch_gemv_fast_multi(s, ctx, count, views, x, x_dtype, ys, strides, y_dtype, m, xs, nullptr, nullptr, nullptr);
+        return launch_gemv_fast_multi(s, ctx, count, views, x, x_dtype, ys, strides, y_dtype, m, xs, nullptr, nullptr, HeadKeys{});
     if (tiled && (uintptr_t)x % 16 == 0)
         return launch_gemv_tile16_multi(s, ctx, count, views, x, ys, strides, y_dtype, m, xs, nullptr, nullptr,
-                                        nullptr);
+                                        HeadKeys{});
     if (in_place && (uintptr_t)x % 16 == 0)
-        return launch_gemv_staf_multi(s, ctx, count, views, x, ys, strides, y_dtype, m, xs, nullptr, nullptr, nullptr);
+        return launch_gemv_staf_multi(s, ctx, count, views, x, ys, strides, y_dtype, m, xs, nullptr, nullptr, HeadKeys{});
     for (uint32_t i = 0; i < count; i++) {
         mi355q_status st = dispatch_linear(ctx, s, weights[i], x, x_dtype, ys[i], y_dtype, m, xs, 0, flags, false);
         if (st != MI355Q_OK) return st;
@@ -158,27 +158,29 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
     return MI355Q_OK;
 }
 
+// `keys`: kStaticHeadKeys or kArgmaxPartialCapacity keys for the fused head followed by kArgmaxStandaloneKeys for the
+// two-launch arg-max (the context's allocation, or the device array of the entry point that allocates nothing).
 mi355q_status dispatch_output_head(mi355q_context* ctx, hipStream_t s, const mi355q_weight* w, const void* x,
-                                   int x_dtype, float* logits, int32_t* token, uint32_t flags) {
+                                   int x_dtype, float* logits, int32_t* token, uint32_t flags, HeadKeys keys) {
     if (!x || !token) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null pointer");
     if (!dtype_ok(x_dtype)) return fail(MI355Q_ERR_INVALID_ARGUMENT, "bad dtype tag");
     const WView v = w->view();
     const uint32_t xs = (uint32_t)w->k;
     if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && gemv_fast_eligible(v, x_dtype, 1, xs) && (uintptr_t)x % 16 == 0)
         return launch_gemv_fast(s, ctx, v, x, x_dtype, nullptr, MI355Q_F32, 1, xs, (uint32_t)w->n, logits, token,
-                                ctx->argmax_partials);
+                                keys);
     if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && gemv_tile16_eligible(v, x_dtype, 1, xs) && gemv_tile16_k_parts(ctx, v, 1) == 1 &&
         (uintptr_t)x % 16 == 0) {
         void* none[1] = {nullptr};
         const uint32_t strides[1] = {(uint32_t)w->n};
         return launch_gemv_tile16_multi(s, ctx, 1, &v, x, none, strides, MI355Q_F32, 1, xs, logits, token,
-                                        ctx->argmax_partials);
+                                        keys);
     }
     if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && gemv_staf_eligible(v, x_dtype, 1, xs) && (uintptr_t)x % 16 == 0) {
         void* none[1] = {nullptr};
         const uint32_t strides[1] = {(uint32_t)w->n};
         return launch_gemv_staf_multi(s, ctx, 1, &v, x, none, strides, MI355Q_F32, 1, xs, logits, token,
-                                      ctx->argmax_partials);
+                                      keys);
     }
     // two dispatches, as the reference runs the head: projection to fp32 logits, then argmax
     if (!logits)
@@ -186,7 +188,7 @@ mi355q_status dispatch_output_head(mi355q_context* ctx, hipStream_t s, const mi3
                     "a logits buffer is required when the fused head kernel does not accept the shape");
     mi355q_status st = launch_gemv_generic(s, v, x, x_dtype, logits, MI355Q_F32, 1, xs, (uint32_t)w->n);
     if (st != MI355Q_OK) return st;
-    return launch_argmax(s, logits, MI355Q_F32, (uint32_t)w->n, token, ctx->argmax_partials + kArgmaxPartialCapacity);
+    return launch_argmax(s, logits, MI355Q_F32, (uint32_t)w->n, token, keys.ptr + keys.capacity);
 }
 
 }  // namespace mi355q
@@ -279,8 +281,23 @@ mi355q_status mi355q_lmhead_argmax(mi355q_context* ctx, void* stream, const mi35
                                    mi355q_dtype x_dtype, float* logits_f32_dev, int32_t* token_out_dev,
                                    uint32_t flags) {
     if (mi355q_status s = check_launch(ctx, w)) return s;
-    return dispatch_output_head(ctx, (hipStream_t)stream, w, x_dev, x_dtype, logits_f32_dev, token_out_dev, flags);
+    return dispatch_output_head(ctx, (hipStream_t)stream, w, x_dev, x_dtype, logits_f32_dev, token_out_dev, flags,
+                                HeadKeys{ctx->argmax_partials, kArgmaxPartialCapacity});
 }
+
+// The same head with its partial keys in a device array of the library image instead of the context's allocation: no
+// device memory is allocated or released on this path (the launches it makes need no workspace and no LDS opt-in).
+mi355q_status mi355q_lmhead_argmax_static(mi355q_context* ctx, void* stream, const mi355q_weight* w, const void* x_dev,
+                                          mi355q_dtype x_dtype, float* logits_f32_dev, int32_t* token_out_dev,
+                                          uint32_t flags) {
+    if (mi355q_status s = check_launch(ctx, w)) return s;
+    unsigned long long* const keys = static_head_keys(ctx->device);
+    if (!keys) return fail(MI355Q_ERR_DEVICE, "the static key array of device %d was not resolved", ctx->device);
+    return dispatch_output_head(ctx, (hipStream_t)stream, w, x_dev, x_dtype, logits_f32_dev, token_out_dev, flags,
+                                HeadKeys{keys, kStaticHeadKeys});
+}
+
+uint32_t mi355q_lmhead_argmax_static_capacity(void) { return kStaticHeadKeys; }
 
 mi355q_status mi355q_clock_probe_read(mi355q_context* ctx, uint64_t* shader_cycles, uint64_t* realtime_ticks) {
     if (!ctx) return fail(MI355Q_ERR_NULL_HANDLE, "context is null");

@@ -124,6 +124,16 @@ mi355q_status launch_embedding_lookup(hipStream_t s, const WView& w, const int32
                                       float embedding_scale);
 // Partial keys of the fused output head: one per workgroup of the projection launch.
 constexpr uint32_t kArgmaxPartialCapacity = 65536;
+// Where a fused head leaves its partial keys, and how many fit (null: the launch has no arg-max tail).
+struct HeadKeys {
+    unsigned long long* ptr = nullptr;
+    uint32_t capacity = 0;
+};
+// The entry point that allocates nothing keeps its keys in a device array of the library image: one pointer per device,
+// resolved when a context is created on that device (runtime.hip); null before that.  kStaticHeadKeys keys for the fused
+// head, then kArgmaxStandaloneKeys for the two-launch arg-max.
+constexpr uint32_t kStaticHeadKeys = 32768;
+unsigned long long* static_head_keys(int device);
 mi355q_status launch_argmax_finish(hipStream_t s, const unsigned long long* partial, uint32_t count, int32_t* token_out);
 // `partial`: 256 keys of scratch for the two-launch form taken by long vectors (null: always one workgroup).
 constexpr uint32_t kArgmaxStandaloneKeys = 256;
@@ -137,7 +147,7 @@ bool gemv_fast_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stri
 mi355q_status launch_gemv_fast(hipStream_t s, const mi355q_context* ctx, const WView& w,
                                const void* x, int x_dtype, void* y, int y_dtype, uint32_t m,
                                uint32_t x_stride, uint32_t y_stride, float* logits_f32,
-                               int32_t* token_out, unsigned long long* argmax_scratch);
+                               int32_t* token_out, HeadKeys keys);
 // Block-layout GEMV (gemv_staf.hip): reads STAF interleaved blocks in place.
 bool gemv_staf_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
 mi355q_status launch_gemv_staf(hipStream_t s, const mi355q_context* ctx, const WView& w, const void* x, void* y,
@@ -145,7 +155,7 @@ mi355q_status launch_gemv_staf(hipStream_t s, const mi355q_context* ctx, const W
 mi355q_status launch_gemv_staf_multi(hipStream_t s, const mi355q_context* ctx, uint32_t count, const WView* w,
                                      const void* x, void* const* y, const uint32_t* y_strides, int y_dtype,
                                      uint32_t m, uint32_t x_stride, float* logits_f32, int32_t* token_out,
-                                     unsigned long long* argmax_scratch);
+                                     HeadKeys keys);
 struct GemvLaunchShape {
     uint32_t grid, block, lds_bytes, rows_per_workgroup;
     const char* kernel;
@@ -156,7 +166,7 @@ GemvLaunchShape gemv_fast_shape(const mi355q_context* ctx, const WView& w, uint3
 mi355q_status launch_gemv_fast_multi(hipStream_t s, const mi355q_context* ctx, uint32_t count, const WView* w,
                                      const void* x, int x_dtype, void* const* y, const uint32_t* y_strides, int y_dtype,
                                      uint32_t m, uint32_t x_stride, float* logits_f32, int32_t* token_out,
-                                     unsigned long long* argmax_scratch);
+                                     HeadKeys keys);
 
 // Matrix-core decode kernel over the TILE16 layout (gemv_tile16.hip)
 constexpr int kTile16MaxSegments = 3;
@@ -173,7 +183,7 @@ Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_row_ti
 mi355q_status launch_gemv_tile16_multi(hipStream_t s, mi355q_context* ctx, uint32_t count, const WView* w,
                                        const void* x, void* const* y, const uint32_t* y_strides, int y_dtype,
                                        uint32_t m, uint32_t x_stride, float* logits_f32, int32_t* token_out,
-                                       unsigned long long* argmax_scratch);
+                                       HeadKeys keys);
 mi355q_status launch_tile16_pack(hipStream_t s, const WView& planes, uint32_t* tiles);
 
 // Validated dispatch shared by the direct entry points and by plan replay (api.hip)
@@ -184,7 +194,7 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
                               void* y, int y_dtype, uint32_t m, uint32_t xs, uint32_t ys, uint32_t flags,
                               bool small_m_only);
 mi355q_status dispatch_output_head(mi355q_context* ctx, hipStream_t s, const mi355q_weight* w, const void* x,
-                                   int x_dtype, float* logits, int32_t* token, uint32_t flags);
+                                   int x_dtype, float* logits, int32_t* token, uint32_t flags, HeadKeys keys);
 int env_int_cached(const char* name, int fallback);
 void plan_shared_launch_shape(const mi355q_weight* const* ws, uint32_t count, uint32_t m, int x_dtype, uint32_t x_stride,
                               mi355q_step* s);

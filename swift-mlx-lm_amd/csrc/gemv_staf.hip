@@ -499,7 +499,7 @@ GemvLaunchShape gemv_staf_shape(const mi355q_context* ctx, const WView& w, uint3
 mi355q_status launch_gemv_staf_multi(hipStream_t s, const mi355q_context* ctx, uint32_t count, const WView* w,
                                      const void* x, void* const* y, const uint32_t* y_strides, int y_dtype,
                                      uint32_t m, uint32_t x_stride, float* logits_f32, int32_t* token_out,
-                                     unsigned long long* argmax_scratch) {
+                                     HeadKeys keys) {
     if (count < 1 || count > (uint32_t)kGemvMaxSegments)
         return fail(MI355Q_ERR_INVALID_ARGUMENT, "1..%d weights per fused launch", kGemvMaxSegments);
     if ((uintptr_t)x % 16) return fail(MI355Q_ERR_INVALID_ARGUMENT, "activation pointer must be 16-byte aligned");
@@ -524,7 +524,7 @@ mi355q_status launch_gemv_staf_multi(hipStream_t s, const mi355q_context* ctx, u
     a.nsp = (w[0].blocks_per_row + 63) / 64;
     a.rows_per_span = staf_rows_per_span(w[0].blocks_per_row);
     a.logits = logits_f32;
-    a.scratch = argmax_scratch;
+    a.scratch = keys.ptr;
     for (uint32_t m0 = 0; m0 < m;) {
         const uint32_t left = m - m0;
         int mt = left >= 3 ? 4 : (int)left;                  // 3 rows run as a 4-row launch with one row masked
@@ -545,11 +545,11 @@ mi355q_status launch_gemv_staf_multi(hipStream_t s, const mi355q_context* ctx, u
             a.wave_end[i] = waves;
         }
         const uint32_t grid = (waves + kWaves - 1) / kWaves;
-        if (argmax && grid > kArgmaxPartialCapacity) return fail(MI355Q_ERR_SHAPE, "too many workgroups for the fused argmax");
+        if (argmax && grid > keys.capacity) return fail(MI355Q_ERR_SHAPE, "too many workgroups for the fused argmax");
         a.x = (const uint16_t*)x + (size_t)m0 * x_stride;
         a.m = mm;
         if (mi355q_status st = launch_by_format(s, w[0].bits, w[0].group, a, mt, c.depth, grid, argmax)) return st;
-        if (argmax) return launch_argmax_finish(s, argmax_scratch, grid, token_out);
+        if (argmax) return launch_argmax_finish(s, keys.ptr, grid, token_out);
         m0 += mm;
     }
     return MI355Q_OK;
@@ -559,7 +559,7 @@ mi355q_status launch_gemv_staf(hipStream_t s, const mi355q_context* ctx, const W
                                int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride) {
     void* ys[1] = {y};
     const uint32_t strides[1] = {y_stride};
-    return launch_gemv_staf_multi(s, ctx, 1, &w, x, ys, strides, y_dtype, m, x_stride, nullptr, nullptr, nullptr);
+    return launch_gemv_staf_multi(s, ctx, 1, &w, x, ys, strides, y_dtype, m, x_stride, nullptr, nullptr, HeadKeys{});
 }
 
 }  // namespace mi355q

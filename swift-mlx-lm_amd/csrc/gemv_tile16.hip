@@ -487,7 +487,7 @@ Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_row_ti
 mi355q_status launch_gemv_tile16_multi(hipStream_t s, mi355q_context* ctx, uint32_t count, const WView* w,
                                        const void* x, void* const* y, const uint32_t* y_strides, int y_dtype,
                                        uint32_t m, uint32_t x_stride, float* logits_f32, int32_t* token_out,
-                                       unsigned long long* argmax_scratch) {
+                                       HeadKeys keys) {
     if (count < 1 || count > (uint32_t)kTile16MaxSegments)
         return fail(MI355Q_ERR_INVALID_ARGUMENT, "1..%d weights per fused launch", kTile16MaxSegments);
     if ((uintptr_t)x % 16) return fail(MI355Q_ERR_INVALID_ARGUMENT, "activation pointer must be 16-byte aligned");
@@ -507,7 +507,7 @@ mi355q_status launch_gemv_tile16_multi(hipStream_t s, mi355q_context* ctx, uint3
     }
     const Tile16LaunchShape g = gemv_tile16_shape(ctx, tiles, w[0].k, m);
     a.x = (const uint16_t*)x;
-    a.logits = logits_f32; a.token_out = token_out; a.scratch = argmax_scratch;
+    a.logits = logits_f32; a.token_out = token_out; a.scratch = keys.ptr;
     a.k = w[0].k; a.m = m; a.x_stride = x_stride;
     a.kblocks = w[0].k / 128;
     a.parts = g.parts;
@@ -525,11 +525,11 @@ mi355q_status launch_gemv_tile16_multi(hipStream_t s, mi355q_context* ctx, uint3
     a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = w[0].sb_dtype;
     const int mr = m == 1 ? 1 : m == 2 ? 2 : 4;
     if (argmax) {
-        if (g.grid > kArgmaxPartialCapacity)
+        if (g.grid > keys.capacity)
             return fail(MI355Q_ERR_SHAPE, "the fused output head keeps one partial key per workgroup: %u workgroups exceed %u",
-                        g.grid, kArgmaxPartialCapacity);
+                        g.grid, keys.capacity);
         if (mi355q_status st = launch_t16_shape<1, true>(s, a, g)) return st;
-        return launch_argmax_finish(s, argmax_scratch, g.grid, token_out);
+        return launch_argmax_finish(s, keys.ptr, g.grid, token_out);
     }
     mi355q_status st = mr == 1 ? launch_t16_shape<1, false>(s, a, g)
                      : mr == 2 ? launch_t16_shape<2, false>(s, a, g) : launch_t16_shape<4, false>(s, a, g);

@@ -158,7 +158,7 @@ GemvLaunchShape gemv_fast_shape(const mi355q_context* ctx, const WView& w, uint3
 mi355q_status launch_gemv_fast_multi(hipStream_t s, const mi355q_context* ctx, uint32_t count, const WView* w,
                                      const void* x, int x_dtype, void* const* y, const uint32_t* y_strides, int y_dtype,
                                      uint32_t m, uint32_t x_stride, float* logits_f32, int32_t* token_out,
-                                     unsigned long long* argmax_scratch) {
+                                     HeadKeys keys) {
     if (count < 1 || count > (uint32_t)kGemvMaxSegments)
         return fail(MI355Q_ERR_INVALID_ARGUMENT, "1..%d weights per fused launch", kGemvMaxSegments);
     if ((uintptr_t)x % 16) return fail(MI355Q_ERR_INVALID_ARGUMENT, "activation pointer must be 16-byte aligned");
@@ -193,16 +193,16 @@ mi355q_status launch_gemv_fast_multi(hipStream_t s, const mi355q_context* ctx, u
         a.x = (const uint16_t*)x + (size_t)m0 * x_stride;
         a.logits = logits_f32;
         a.token_out = token_out;
-        a.scratch = argmax_scratch;
+        a.scratch = keys.ptr;
         a.k = all.k; a.m = mm;
         a.x_stride = x_stride;
         a.code_stride = all.code_stride; a.sz_stride = all.sz_stride;
         a.nc = c.nc; a.rows_per_wave = c.rows_per_wave;
         a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = all.sb_dtype; a.x_dtype = (uint32_t)x_dtype;
         c.grid = grid;                        // whole wavefronts per matrix: a few more than rows / rows_per_wave
-        if (argmax && grid > kArgmaxPartialCapacity)
+        if (argmax && grid > keys.capacity)
             return fail(MI355Q_ERR_SHAPE, "the fused output head keeps one partial key per workgroup: %u workgroups exceed %u",
-                        grid, kArgmaxPartialCapacity);
+                        grid, keys.capacity);
         mi355q_status st;
         switch (all.bits) {
         case 2: st = launch_gemv_planes_q2(s, a, (int)all.group, c); break;
@@ -215,18 +215,18 @@ mi355q_status launch_gemv_fast_multi(hipStream_t s, const mi355q_context* ctx, u
         }
         if (st != MI355Q_OK) return st;
         if (argmax)
-            if (mi355q_status fin = launch_argmax_finish(s, argmax_scratch, grid, token_out)) return fin;
+            if (mi355q_status fin = launch_argmax_finish(s, keys.ptr, grid, token_out)) return fin;
     }
     return MI355Q_OK;
 }
 
 mi355q_status launch_gemv_fast(hipStream_t s, const mi355q_context* ctx, const WView& w, const void* x, int x_dtype,
                                void* y, int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride, float* logits_f32,
-                               int32_t* token_out, unsigned long long* argmax_scratch) {
+                               int32_t* token_out, HeadKeys keys) {
     void* ys[1] = {y};
     const uint32_t strides[1] = {y_stride};
     return launch_gemv_fast_multi(s, ctx, 1, &w, x, x_dtype, ys, strides, y_dtype, m, x_stride, logits_f32, token_out,
-                                  argmax_scratch);
+                                  keys);
 }
 
 }  // namespace mi355q

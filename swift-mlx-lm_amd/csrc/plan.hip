@@ -56,7 +56,8 @@ mi355q_status encode_range(mi355q_plan* plan, hipStream_t s, uint32_t first, uin
             rc = dispatch_batched(plan->ctx, s, st.count, st.ws, st.x, st.x_dtype, st.ysv, st.y_dtype, st.m, st.xs,
                                   st.flags);
         else
-            rc = dispatch_output_head(plan->ctx, s, st.w, st.x, st.x_dtype, (float*)st.y, st.token, st.flags);
+            rc = dispatch_output_head(plan->ctx, s, st.w, st.x, st.x_dtype, (float*)st.y, st.token, st.flags,
+                                      HeadKeys{plan->ctx->argmax_partials, kArgmaxPartialCapacity});
         if (rc != MI355Q_OK) return rc;
     }
     return MI355Q_OK;

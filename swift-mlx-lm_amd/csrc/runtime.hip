@@ -1,10 +1,43 @@
 // Context, device memory, streams, events and packed-weight handles.
+#include <mutex>
 #include <new>
 #include <vector>
 
 #include "common.h"
 
 using namespace mi355q;
+
+// Partial keys of mi355q_lmhead_argmax_static, the entry point that allocates nothing: a device array in the library
+// image (each GPU the library runs on holds its own copy, 258 KiB, until the process ends).  Host code never uses the
+// array's name as an address: the address on a device is resolved once, with that device current, when the first context
+// is created there, and only that pointer is handed to kernels.
+static __device__ __align__(256) unsigned long long scratch[kStaticHeadKeys + kArgmaxStandaloneKeys];
+
+namespace {
+constexpr int kMaxDevices = 64;
+unsigned long long* g_static_keys[kMaxDevices] = {};
+std::mutex g_static_keys_mutex;
+
+// with `device` current
+mi355q_status resolve_static_keys(int device) {
+    if (device < 0 || device >= kMaxDevices) return fail(MI355Q_ERR_INVALID_ARGUMENT, "device index %d beyond %d", device, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_static_keys_mutex);
+    if (g_static_keys[device]) return MI355Q_OK;
+    void* ptr = nullptr;
+    MI355Q_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (!ptr) return fail(MI355Q_ERR_DEVICE, "hipGetSymbolAddress returned a null address for the static key array");
+    g_static_keys[device] = (unsigned long long*)ptr;
+    return MI355Q_OK;
+}
+}  // namespace
+
+namespace mi355q {
+unsigned long long* static_head_keys(int device) {
+    if (device < 0 || device >= kMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> lock(g_static_keys_mutex);
+    return g_static_keys[device];
+}
+}  // namespace mi355q
 
 namespace mi355q {
 
@@ -217,6 +250,10 @@ mi355q_status mi355q_context_create(int device_index, mi355q_context** out) {
         delete ctx;
         return fail(MI355Q_ERR_DEVICE, "device arch %s is not gfx950; the kernels are built for MI355X only",
                     arch.c_str());
+    }
+    if (mi355q_status st = resolve_static_keys(device_index)) {     // the device is current
+        delete ctx;
+        return st;
     }
     e = hipMalloc((void**)&ctx->argmax_scratch, 256);
     if (e == hipSuccess) e = hipMemset(ctx->argmax_scratch, 0, 256);
