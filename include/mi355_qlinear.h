@@ -282,6 +282,13 @@ MI355Q_API mi355q_status mi355q_batched_qgemm(mi355q_context* ctx, void* stream,
 MI355Q_API mi355q_status mi355q_dequant_bf16(mi355q_context* ctx, void* stream,
                                              const mi355q_weight* w, void* out_bf16_dev);
 
+/* CPUWeightStore.decodeQuantized (Sources/SwiftLM/CPUWeightStore.swift:109-174): the whole matrix as row-major fp32
+ * [N, K], each weight scale * float(q) + zero evaluated as the reference's host code does (:170): the product rounded
+ * to fp32, then the sum rounded to fp32, no fused multiply-add.  Any registered format and any layout (the reference
+ * decodes 4- and 8-bit blocks only, :156-166). */
+MI355Q_API mi355q_status mi355q_dequant_f32(mi355q_context* ctx, void* stream,
+                                            const mi355q_weight* w, float* out_f32_dev);
+
 /* gemm_bf16_f32s (generateMPPGEMM, MC/Generator/MetalSourceGenerator+Linear.swift:18-81):
  * C[M,N] = A[M, a_row_stride>=K] * B[N,K]^T with B dense bf16 (the dequant scratch), MFMA,
  * fp32 accumulation. */

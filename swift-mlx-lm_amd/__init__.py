@@ -150,6 +150,7 @@ def library() -> C.CDLL:
         "mi355q_qgemm": (i32, [vp, vp, vp, vp, C.c_int, vp, C.c_int, u32, u32, u32, u32]),
         "mi355q_batched_qgemm": (i32, [vp, vp, u32, P(vp), vp, C.c_int, P(vp), C.c_int, u32, u32, u32]),
         "mi355q_dequant_bf16": (i32, [vp, vp, vp, vp]),
+        "mi355q_dequant_f32": (i32, [vp, vp, vp, vp]),
         "mi355q_gemm_bf16": (i32, [vp, vp, vp, C.c_int, vp, vp, C.c_int, u32, u32, u32, u32, u32]),
         "mi355q_unpack_codes": (i32, [vp, vp, vp, vp]),
         "mi355q_argmax": (i32, [vp, vp, vp, C.c_int, u32, vp]),
@@ -814,6 +815,10 @@ class Context:
 
     def dequant_bf16(self, w: PackedWeight, out, stream=0):
         _check(library().mi355q_dequant_bf16(self.handle, stream, w.handle, self._ptr(out)))
+
+    def dequant_f32(self, w: PackedWeight, out, stream=0):
+        """CPUWeightStore.decodeQuantized on the device: row-major fp32 [N, K], scale * q then + zero, two roundings."""
+        _check(library().mi355q_dequant_f32(self.handle, stream, w.handle, self._ptr(out)))
 
     def gemm_bf16(self, a, a_dtype, b_bf16, c, c_dtype, m, n, k, a_row_stride=0, c_row_stride=0, stream=0):
         _check(library().mi355q_gemm_bf16(self.handle, stream, self._ptr(a), a_dtype, self._ptr(b_bf16),

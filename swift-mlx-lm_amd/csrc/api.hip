@@ -227,6 +227,12 @@ mi355q_status mi355q_dequant_bf16(mi355q_context* ctx, void* stream, const mi355
     return launch_dequant_bf16((hipStream_t)stream, w->view(), (uint16_t*)out_bf16_dev);
 }
 
+mi355q_status mi355q_dequant_f32(mi355q_context* ctx, void* stream, const mi355q_weight* w, float* out_f32_dev) {
+    if (mi355q_status s = check_launch(ctx, w)) return s;
+    if (!out_f32_dev || (uintptr_t)out_f32_dev % 4) return fail(MI355Q_ERR_INVALID_ARGUMENT, "bad output pointer");
+    return launch_dequant_f32((hipStream_t)stream, w->view(), out_f32_dev);
+}
+
 mi355q_status mi355q_gemm_bf16(mi355q_context* ctx, void* stream, const void* a_dev, mi355q_dtype a_dtype,
                                const void* b_bf16_dev, void* c_dev, mi355q_dtype c_dtype, uint32_t m, uint32_t n,
                                uint32_t k, uint32_t a_row_stride, uint32_t c_row_stride) {

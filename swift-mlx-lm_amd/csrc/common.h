@@ -116,6 +116,7 @@ namespace mi355q {
 // Each returns MI355Q_OK or a launch-time failure; all shape checks happen in api.hip before.
 mi355q_status launch_unpack_codes(hipStream_t s, const WView& w, uint8_t* out);
 mi355q_status launch_dequant_bf16(hipStream_t s, const WView& w, uint16_t* out);
+mi355q_status launch_dequant_f32(hipStream_t s, const WView& w, float* out);
 mi355q_status launch_gemv_generic(hipStream_t s, const WView& w, const void* x, int x_dtype,
                                   void* y, int y_dtype, uint32_t m, uint32_t x_stride,
                                   uint32_t y_stride);

@@ -237,18 +237,21 @@ mi355q_status launch_embedding_lookup(hipStream_t s, const WView& w, const int32
     return MI355Q_OK;
 }
 
-// ------------------------------------------------------------------------------ dequant bf16
+// ------------------------------------------------------------------------------ dequant to bf16 / fp32
 // One workgroup per row, 256 threads striding over the row, as the reference kernel does.
 // scale*q and +zero are kept as two roundings so the result is bit-identical to an unfused
-// host evaluation.
-__global__ __launch_bounds__(256) void dequant_bf16_kernel(WView w, uint16_t* __restrict__ out) {
+// host evaluation (the order CPUWeightStore.decodeQuantized evaluates, Sources/SwiftLM/CPUWeightStore.swift:170).
+// F32: the fp32 value itself is stored; else its bf16 rounding.
+template <bool F32>
+__global__ __launch_bounds__(256) void dequant_kernel(WView w, void* __restrict__ out) {
     for (uint32_t row = blockIdx.x; row < w.n; row += gridDim.x) {
-        uint16_t* orow = out + (size_t)row * w.k;
         for (uint32_t c = threadIdx.x; c < w.k; c += 256) {
             float scale, zero;
             load_scale_zero(w, row, c / w.group, scale, zero);
             const float q = (float)load_code(w, row, c);
-            orow[c] = f32_to_bf16_rne(__fadd_rn(__fmul_rn(scale, q), zero));
+            const float v = __fadd_rn(__fmul_rn(scale, q), zero);
+            if constexpr (F32) ((float*)out)[(size_t)row * w.k + c] = v;
+            else ((uint16_t*)out)[(size_t)row * w.k + c] = f32_to_bf16_rne(v);
         }
     }
 }
@@ -259,8 +262,8 @@ __global__ __launch_bounds__(256) void dequant_bf16_kernel(WView w, uint16_t* __
 // BITS is a template argument (constant shifts on the 64-bit field) and the grid is two-dimensional -- x over the
 // 8-code chunks of a row, y over rows -- so that no thread divides a 64-bit index: with run-time width and a flat index
 // the kernel was bound by its integer arithmetic (42 us for 4096 -> 14336, against 26 us for a plain copy of as many bytes).
-template <int BITS>
-__global__ __launch_bounds__(256) void dequant_bf16_x8_kernel(WView w, uint16_t* __restrict__ out) {
+template <int BITS, bool F32>
+__global__ __launch_bounds__(256) void dequant_x8_kernel(WView w, void* __restrict__ out) {
     const uint32_t c0 = (blockIdx.x * 256 + threadIdx.x) << 3;
     if (c0 >= w.k) return;
     constexpr uint32_t mask = (1u << BITS) - 1u;
@@ -270,43 +273,53 @@ __global__ __launch_bounds__(256) void dequant_bf16_x8_kernel(WView w, uint16_t*
         const uint64_t v = load_codes8(w, row, c0);
         float scale, zero;
         load_scale_zero(w, row, g, scale, zero);
-        uint32_t o[4];
+        float f[8];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const float q0 = (float)((uint32_t)(v >> ((2 * i) * BITS)) & mask);
-            const float q1 = (float)((uint32_t)(v >> ((2 * i + 1) * BITS)) & mask);
-            const uint32_t lo = f32_to_bf16_rne(__fadd_rn(__fmul_rn(scale, q0), zero));
-            const uint32_t hi = f32_to_bf16_rne(__fadd_rn(__fmul_rn(scale, q1), zero));
-            o[i] = lo | (hi << 16);
+        for (int i = 0; i < 8; i++) f[i] = __fadd_rn(__fmul_rn(scale, (float)((uint32_t)(v >> (i * BITS)) & mask)), zero);
+        if constexpr (F32) {
+            u32x4 lo, hi;
+            lo.x = __float_as_uint(f[0]); lo.y = __float_as_uint(f[1]); lo.z = __float_as_uint(f[2]); lo.w = __float_as_uint(f[3]);
+            hi.x = __float_as_uint(f[4]); hi.y = __float_as_uint(f[5]); hi.z = __float_as_uint(f[6]); hi.w = __float_as_uint(f[7]);
+            u32x4* dst = (u32x4*)((float*)out + (size_t)row * w.k + c0);
+            __builtin_nontemporal_store(lo, dst);
+            __builtin_nontemporal_store(hi, dst + 1);
+        } else {
+            u32x4 st;
+            st.x = f32_to_bf16_rne(f[0]) | ((uint32_t)f32_to_bf16_rne(f[1]) << 16);
+            st.y = f32_to_bf16_rne(f[2]) | ((uint32_t)f32_to_bf16_rne(f[3]) << 16);
+            st.z = f32_to_bf16_rne(f[4]) | ((uint32_t)f32_to_bf16_rne(f[5]) << 16);
+            st.w = f32_to_bf16_rne(f[6]) | ((uint32_t)f32_to_bf16_rne(f[7]) << 16);
+            __builtin_nontemporal_store(st, (u32x4*)((uint16_t*)out + (size_t)row * w.k + c0));
         }
-        u32x4 st;
-        st.x = o[0]; st.y = o[1]; st.z = o[2]; st.w = o[3];
-        __builtin_nontemporal_store(st, (u32x4*)(out + (size_t)row * w.k + c0));
     }
 }
 
-mi355q_status launch_dequant_bf16(hipStream_t s, const WView& w, uint16_t* out) {
-    if (w.k % 8 == 0 && (uintptr_t)out % 16 == 0) {
+template <bool F32>
+mi355q_status launch_dequant(hipStream_t s, const WView& w, void* out) {
+    if (w.k % 8 == 0 && (uintptr_t)out % 16 == 0 && (!F32 || w.k % 4 == 0)) {
         // two to four rows per thread, at most 65535 workgroups along y
         uint32_t gy = w.n > 4096 ? (w.n + 3) / 4 : (w.n + 1) / 2;
         if (gy > 65535u) gy = 65535u;
         const dim3 grid((w.k / 8 + 255) / 256, gy), block(256);
         switch (w.bits) {
-        case 2: dequant_bf16_x8_kernel<2><<<grid, block, 0, s>>>(w, out); break;
-        case 3: dequant_bf16_x8_kernel<3><<<grid, block, 0, s>>>(w, out); break;
-        case 4: dequant_bf16_x8_kernel<4><<<grid, block, 0, s>>>(w, out); break;
-        case 5: dequant_bf16_x8_kernel<5><<<grid, block, 0, s>>>(w, out); break;
-        case 6: dequant_bf16_x8_kernel<6><<<grid, block, 0, s>>>(w, out); break;
-        case 8: dequant_bf16_x8_kernel<8><<<grid, block, 0, s>>>(w, out); break;
+        case 2: dequant_x8_kernel<2, F32><<<grid, block, 0, s>>>(w, out); break;
+        case 3: dequant_x8_kernel<3, F32><<<grid, block, 0, s>>>(w, out); break;
+        case 4: dequant_x8_kernel<4, F32><<<grid, block, 0, s>>>(w, out); break;
+        case 5: dequant_x8_kernel<5, F32><<<grid, block, 0, s>>>(w, out); break;
+        case 6: dequant_x8_kernel<6, F32><<<grid, block, 0, s>>>(w, out); break;
+        case 8: dequant_x8_kernel<8, F32><<<grid, block, 0, s>>>(w, out); break;
         default: return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no dequantisation kernel for %u-bit codes", w.bits);
         }
     } else {
         unsigned blocks = w.n < 65535u * 16u ? w.n : 65535u * 16u;
-        dequant_bf16_kernel<<<dim3(blocks), dim3(256), 0, s>>>(w, out);
+        dequant_kernel<F32><<<dim3(blocks), dim3(256), 0, s>>>(w, out);
     }
     MI355Q_HIP(hipGetLastError());
     return MI355Q_OK;
 }
+
+mi355q_status launch_dequant_bf16(hipStream_t s, const WView& w, uint16_t* out) { return launch_dequant<false>(s, w, out); }
+mi355q_status launch_dequant_f32(hipStream_t s, const WView& w, float* out) { return launch_dequant<true>(s, w, out); }
 
 // ------------------------------------------------------------------------------ generic GEMV
 // grid (ceil(N/4), M); one wavefront per output row, lanes stride over the codes of the row.

@@ -63,6 +63,54 @@ def test_dequant_bf16_bit_exact(pkg, ctx, bits, group):
         out.free(); w.destroy()
 
 
+# ------------------------------------------------------------------- dequant -> fp32 (a11)
+@pytest.mark.parametrize("bits,group", kat.ALL_FORMATS)
+def test_dequant_f32_bit_exact(pkg, ctx, bits, group):
+    """CPUWeightStore.decodeQuantized (Sources/SwiftLM/CPUWeightStore.swift:109-174) on the device: every registered
+    format, STAF blocks and planes, bit for bit against the oracle's restatement (scale * q rounded, then + zero)."""
+    blocks_per_row = int(32 // np.gcd(32, group * bits)) * 3
+    k, n = group * blocks_per_row, 23
+    codes = kat.random_codes(2500 + bits * 5 + group, n, k, bits)
+    rng = np.random.default_rng(100 + bits + group)
+    scales = rng.integers(1, 400, size=(n, blocks_per_row)) / 4096.0      # exact in f16 and bf16, not powers of two
+    zeros = rng.integers(-127, 127, size=(n, blocks_per_row)) / 1024.0
+    case = Case(bits, group, codes, scales, zeros)
+    want = oracle.dequant_staf_f32(bits, group, n, k, case.staf_blocks())
+    for name, layout, sb in _layouts(pkg, case):
+        w = case.device_weight(ctx, pkg, layout, sb)
+        out = ctx.alloc(n * k * 4)
+        ctx.fill(out, 0x7FC00000)
+        ctx.dequant_f32(w, out)
+        ctx.synchronize()
+        assert np.array_equal(out.download(np.float32, (n, k)).view(np.uint32), want.view(np.uint32)), name
+        out.free(); w.destroy()
+
+
+def test_dequant_f32_reference_vector_and_seeded_tensor(pkg, ctx):
+    """The reference's own CPUWeightStore vector (Tests/SwiftLMTests/Core/TextEmbeddingRuntimeTests.swift:421-476:
+    scale 1, zero 0, byte i = (2i mod 16) | ((2i+1 mod 16) << 4) -> 0, 1, ..., 15, 0, ...), and a benchmark-style
+    tensor on all three layouts at a shape the eight-codes-per-thread kernel and the per-code kernel both see."""
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+    qs = np.array([((2 * i) % 16) | (((2 * i + 1) % 16) << 4) for i in range(32)], np.uint8)
+    block = np.concatenate([np.array([0x00, 0x3C, 0x00, 0x00], np.uint8), qs])
+    w = ctx.weight_prepare_staf(fmt, 1, 64, block, pkg.LAYOUT_STAF_BLOCKS)
+    out = ctx.alloc(64 * 4)
+    ctx.dequant_f32(w, out); ctx.synchronize()
+    assert out.download(np.float32, (64,)).tolist() == [float(i % 16) for i in range(64)]
+    out.free(); w.destroy()
+    n, k = 48, 512
+    words, s, z, wq = seeded_case(77, n, k, 4, 64)
+    for layout in (pkg.LAYOUT_PLANES, pkg.LAYOUT_TILE16, pkg.LAYOUT_STAF_BLOCKS):
+        w = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, layout)
+        out = ctx.alloc(n * k * 4 + 16)
+        for off in (0, 4):                                   # 16-byte aligned output, and one that is not
+            ctx.fill(out, 0x7FC00000)
+            ctx.dequant_f32(w, out.ptr + off); ctx.synchronize()
+            got = np.frombuffer(out.download(np.uint8)[off:off + n * k * 4].tobytes(), np.float32).reshape(n, k)
+            assert np.array_equal(got.view(np.uint32), wq.view(np.uint32)), (layout, off)
+        out.free(); w.destroy()
+
+
 # ------------------------------------------------------------- closed-form GEMV KATs (a4)
 def _check_kat(pkg, ctx, case, x, tol=2e-6):
     want = kat.exact_gemv(case.codes, case.scales, case.zeros, x, case.group)
