@@ -20,6 +20,14 @@
  *   - A context is thread-compatible, not thread-safe: callers serialise calls per context, as
  *     the reference serialises per MetalSubmissionContext
  *     (MC/Execution/MetalSubmissionContext.swift:56-120).
+ *   - PRECONDITION: one stream per context at a time.  A context owns device scratch that its
+ *     launches share (split-K partial sums of mi355q_qgemm, per-workgroup argmax keys of
+ *     mi355q_argmax / mi355q_lmhead_argmax, part sums of the matrix-core decode layout, the clock
+ *     probe).  Work enqueued through one context must therefore be ordered: on a single stream, or
+ *     on streams the caller has ordered with events.  Launches of one context that overlap in time
+ *     on different streams race on that scratch and return wrong results without an error; a
+ *     caller that wants concurrent streams creates one context per stream (contexts are cheap:
+ *     a few MB of scratch, grown on demand).
  *   - Shapes follow the reference: a weight is [N = outputDimension, K = inputDimension];
  *     K % groupSize == 0 is required (MC/Generator/MetalSourceGenerator+Quantized.swift:547);
  *     activations are [M = sequenceLength, x_row_stride >= K] in elements; outputs are [M, N].
@@ -79,8 +87,8 @@ enum {
     MI355Q_FLAG_NONE = 0,
     MI355Q_FLAG_FORCE_GENERIC = 1, /* run the reference-shaped per-code kernel (A/B and tests) */
     MI355Q_FLAG_FORCE_SMALL_M = 2, /* qgemm: use the small-M GEMV-style kernel whatever M is */
-    MI355Q_FLAG_FORCE_MFMA = 4,    /* qgemm: use the MFMA kernel whatever M is */
-    MI355Q_FLAG_PROBE_CLOCK = 8    /* qgemm on the MFMA kernel: record the clock probe (mi355q_clock_probe_read) */
+    MI355Q_FLAG_FORCE_MFMA = 4     /* qgemm: use the MFMA kernel whatever M is */
+    /* bit 3 (value 8) is taken by the measurement flag of mi355_qlinear_probe.h */
 };
 
 /* ------------------------------------------------------------------------------------------
@@ -201,8 +209,14 @@ typedef struct {
 } mi355q_weight_info;
 
 /* From MLX source planes in host memory (uint32 [N, K*bits/32]; scales/biases [N, K/g] in
- * sb_dtype; F32 scales are normalised to F16 as the converter does).  `layout` picks the
- * device layout; STAF_BLOCKS repacks on the host first (the reference's load path). */
+ * sb_dtype).  Whatever the layout, every scale and bias takes the value the converter's
+ * normalizeScaleToFloat16 gives it (MC/STAF/STAFConverter.swift:326-368): F32 and BF16 values are
+ * rounded to F16, round to nearest even, so values under the F16 normal range (6.1e-5) lose bits
+ * or flush and values over 65504 become infinite, exactly as in a model.staf the reference wrote.
+ * F32 planes are stored as F16; BF16 planes stay BF16 on the PLANES and TILE16 layouts, holding
+ * those rounded values (each has an exact BF16 spelling), and the block layout stores the F16
+ * header: one MLX tensor therefore decodes to the same weights on all three layouts.  `layout`
+ * picks the device layout; STAF_BLOCKS repacks on the host first (the reference's load path). */
 MI355Q_API mi355q_status mi355q_weight_prepare_mlx(mi355q_context* ctx, uint8_t scheme_identifier,
                                                    uint64_t n_rows, uint64_t k,
                                                    const uint32_t* codes_host,
@@ -259,14 +273,6 @@ MI355Q_API mi355q_status mi355q_qgemm(mi355q_context* ctx, void* stream, const m
                                       const void* x_dev, mi355q_dtype x_dtype, void* y_dev,
                                       mi355q_dtype y_dtype, uint32_t m, uint32_t x_row_stride,
                                       uint32_t y_row_stride, uint32_t flags);
-
-/* Measurement aid without a counterpart in the reference: after an mi355q_qgemm call with
- * MI355Q_FLAG_PROBE_CLOCK that ran on the matrix cores has completed, returns what the first wavefront of
- * workgroup 0 counted while it was in the kernel: shader-clock cycles and ticks of the constant 100 MHz
- * counter.  cycles / ticks / 10 is the clock in GHz the kernel ran at (it depends on the operand data:
- * the part lowers its clock under matrix-core load).  Synchronises with the device. */
-MI355Q_API mi355q_status mi355q_clock_probe_read(mi355q_context* ctx, uint64_t* shader_cycles,
-                                                 uint64_t* realtime_ticks);
 
 /* batched_gemm_q4_g64_{2,3} (:166-338; bindings MC/Compiler/MetalPrefillStepBuilder.swift:928-955):
  * 2 or 3 projections sharing one input (gate+up, q+k+v) in one launch.  All weights must share
@@ -478,11 +484,6 @@ MI355Q_API mi355q_status mi355q_plan_graph_launch(mi355q_plan* plan, void* strea
  * traffic counters).  Both pointers 16-byte aligned, bytes a multiple of 16. */
 MI355Q_API mi355q_status mi355q_buffer_copy(mi355q_context* ctx, void* stream, void* dst_dev,
                                             const void* src_dev, size_t bytes);
-/* Measurement aid without a counterpart in the reference: one launch that only reads `bytes` of device memory
- * with the load instructions the decode kernels use for weights.  Its duration is what HBM delivers to a launch of
- * that size on this part: the practical ceiling the decode GEMV is compared with.  16-byte aligned pointer and size. */
-MI355Q_API mi355q_status mi355q_buffer_read_probe(mi355q_context* ctx, void* stream, const void* src_dev,
-                                                  size_t bytes);
 
 /* ------------------------------------------------------------------------------------------
  * STAF container (model.staf): reader, validator, writer

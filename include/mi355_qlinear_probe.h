@@ -1,0 +1,35 @@
+/* Measurement aids of libmi355_qlinear: entry points without a counterpart in the reference, used by the
+ * benchmark and the profiles to price the kernels against the part itself.  They are exported by the same
+ * shared library but declared apart from mi355_qlinear.h on purpose: a host binding of the quantized
+ * projection path (the Swift module map, a ctypes or cgo stub) includes only mi355_qlinear.h and never sees
+ * them. */
+#ifndef MI355_QLINEAR_PROBE_H
+#define MI355_QLINEAR_PROBE_H
+
+#include "mi355_qlinear.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Launch flag for mi355q_qgemm (its `flags` argument, beside the MI355Q_FLAG_* values of mi355_qlinear.h): on
+ * the matrix-core kernel, the first wavefront of workgroup 0 records how long it was in the kernel. */
+enum { MI355Q_FLAG_PROBE_CLOCK = 8 };
+
+/* After an mi355q_qgemm call with MI355Q_FLAG_PROBE_CLOCK that ran on the matrix cores has completed, returns
+ * what that wavefront counted: shader-clock cycles and ticks of the constant 100 MHz counter.
+ * cycles / ticks / 10 is the clock in GHz the kernel ran at (it depends on the operand data: the part lowers
+ * its clock under matrix-core load).  Synchronises with the device. */
+MI355Q_API mi355q_status mi355q_clock_probe_read(mi355q_context* ctx, uint64_t* shader_cycles,
+                                                 uint64_t* realtime_ticks);
+
+/* One launch that only reads `bytes` of device memory with the load instructions the decode kernels use for
+ * weights.  Its duration is what HBM delivers to a launch of that size on this part: the practical ceiling the
+ * decode GEMV is compared with.  16-byte aligned pointer and size. */
+MI355Q_API mi355q_status mi355q_buffer_read_probe(mi355q_context* ctx, void* stream, const void* src_dev,
+                                                  size_t bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

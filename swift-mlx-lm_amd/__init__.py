@@ -204,11 +204,12 @@ EXPORTED_SYMBOLS = None  # filled lazily by exported_symbols()
 
 
 def exported_symbols():
-    """Names this binding expects the library to export (== every declaration of the C header)."""
+    """Names this binding expects the library to export (== every declaration of the C headers)."""
     import re
-    header = os.path.join(_HERE, "..", "include", "mi355_qlinear.h")
-    with open(header) as f:
-        text = f.read()
+    text = ""
+    for name in ("mi355_qlinear.h", "mi355_qlinear_probe.h"):
+        with open(os.path.join(_HERE, "..", "include", name)) as f:
+            text += f.read()
     return sorted(set(re.findall(r"MI355Q_API\s+[A-Za-z0-9_ ]+?\**\s*\b(mi355q_[a-z0-9_]+)\s*\(", text)))
 
 

@@ -22,7 +22,7 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
-] + os.environ.get("MI355Q_EXTRA_HIPCC_FLAGS", "").split()
+]
 
 
 def sources():
@@ -37,8 +37,8 @@ def _deps_mtime():
 def _compile(src: str, force: bool) -> str:
     obj = os.path.join(OBJ, src + ".o")
     srcp = os.path.join(CSRC, src)
-    newest = max(os.path.getmtime(srcp), _deps_mtime(),
-                 os.path.getmtime(os.path.join(HERE, "..", "include", "mi355_qlinear.h")))
+    inc = os.path.join(HERE, "..", "include")
+    newest = max(os.path.getmtime(srcp), _deps_mtime(), *(os.path.getmtime(os.path.join(inc, h)) for h in os.listdir(inc)))
     if not force and os.path.exists(obj) and os.path.getmtime(obj) >= newest:
         return obj
     cmd = [HIPCC, *FLAGS, "-x", "hip", "-c", srcp, "-o", obj]

@@ -48,6 +48,10 @@ mi355q_status run_small_m(mi355q_context* ctx, hipStream_t s, const mi355q_weigh
     if (!generic && v.layout == MI355Q_LAYOUT_TILE16) {
         step = 16;
         while (step > 1 && !gemv_tile16_eligible(v, x_dtype, step, xs)) step >>= 1;
+        // no row count the tile kernel takes (other activation type, stride): the per-code kernel takes all M at once
+        if (!gemv_tile16_eligible(v, x_dtype, step, xs)) step = m < 65535u ? m : 65535u;
+    } else if (generic || !(gemv_fast_eligible(v, x_dtype, 1, xs) || gemv_staf_eligible(v, x_dtype, 1, xs))) {
+        step = m < 65535u ? m : 65535u;   // the per-code kernel has no limit of 8 rows
     }
     for (uint32_t m0 = 0; m0 < m; m0 += step) {
         const uint32_t mm = m - m0 < step ? m - m0 : step;
@@ -73,16 +77,6 @@ mi355q_status run_small_m(mi355q_context* ctx, hipStream_t s, const mi355q_weigh
 }  // namespace
 
 namespace mi355q {
-
-int env_int_cached(const char* name, int fallback) {
-#ifdef MI355Q_GEMV_EXPERIMENT
-    const char* v = std::getenv(name);   // tuning builds re-read the environment at every launch
-    return (v && *v) ? std::atoi(v) : fallback;
-#else
-    (void)name;
-    return fallback;
-#endif
-}
 
 mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_weight* w, const void* x, int x_dtype,
                               void* y, int y_dtype, uint32_t m, uint32_t xs, uint32_t ys, uint32_t flags,

@@ -10,6 +10,7 @@
 #include <string>
 
 #include "../../include/mi355_qlinear.h"
+#include "../../include/mi355_qlinear_probe.h"
 
 namespace mi355q {
 
@@ -196,7 +197,6 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
                               bool small_m_only);
 mi355q_status dispatch_output_head(mi355q_context* ctx, hipStream_t s, const mi355q_weight* w, const void* x,
                                    int x_dtype, float* logits, int32_t* token, uint32_t flags, HeadKeys keys);
-int env_int_cached(const char* name, int fallback);
 void plan_shared_launch_shape(const mi355q_weight* const* ws, uint32_t count, uint32_t m, int x_dtype, uint32_t x_stride,
                               mi355q_step* s);
 

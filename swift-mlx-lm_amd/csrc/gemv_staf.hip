@@ -344,17 +344,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_staf_kernel(const StafArgs a)
 
 constexpr int kWaves = 4;
 
-// Ring depth and wavefronts per CU.  Tuning builds (MI355Q_GEMV_EXPERIMENT) read MI355Q_STAF_DEPTH and
-// MI355Q_STAF_WAVES_PER_CU; product builds ignore them.
+// Ring depth and wavefronts per CU.
 // Measured on MI355X (q4 g64, 14336x4096, M = 1): depth 2 with 8 wavefronts per CU 9.2 us, depth 4
 // 11.1 us; 4 wavefronts per CU 11.6 us, 16 and more 9.6 us and up.
 struct StafCfg { int depth; uint32_t per_cu; };
 StafCfg staf_cfg() {
-    StafCfg c{2, 8};
-    const int d = env_int_cached("MI355Q_STAF_DEPTH", 0), p = env_int_cached("MI355Q_STAF_WAVES_PER_CU", 0);
-    if (d == 2 || d == 4) c.depth = d;
-    if (p > 0) c.per_cu = (uint32_t)p;
-    return c;
+    return StafCfg{2, 8};
 }
 
 size_t staf_lds_bytes(uint32_t span_slot, uint32_t q, uint32_t nsp, int mt, int depth) {
@@ -364,7 +359,7 @@ size_t staf_lds_bytes(uint32_t span_slot, uint32_t q, uint32_t nsp, int mt, int 
 // When the staged activations leave room for a single workgroup per CU, its four wavefronts take the
 // CU's whole share of rows (every extra workgroup would stage the activations again).
 void staf_one_workgroup_per_cu(size_t lds, StafCfg& c) {
-    if (lds > 80 * 1024 && env_int_cached("MI355Q_STAF_WAVES_PER_CU", 0) == 0) c.per_cu = kWaves;
+    if (lds > 80 * 1024) c.per_cu = kWaves;
 }
 
 // Rows that are a power-of-two fraction of a span (32, 16, 8 ... blocks) share one.
@@ -385,7 +380,7 @@ template <int BITS, int GROUP>
 mi355q_status launch_for_format(hipStream_t s, const StafArgs& a, int mt, int depth, uint32_t grid, bool argmax) {
     using G = StafGeo<BITS, GROUP>;
     const size_t lds = staf_lds_bytes(G::SLOT, G::Q, a.nsp, mt, depth);
-    const bool xreg = mt == 1 && a.nsp == 1 && env_int_cached("MI355Q_STAF_XREG", 1) != 0;
+    const bool xreg = mt == 1 && a.nsp == 1;
     auto go = [&](auto kernel) -> mi355q_status {
         if (lds > 48 * 1024)
             MI355Q_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
@@ -403,17 +398,7 @@ mi355q_status launch_for_format(hipStream_t s, const StafArgs& a, int mt, int de
         default: return go(gemv_staf_kernel<BITS, GROUP, 4, kWaves, 2, false, false>);
         }
     }
-#ifdef MI355Q_GEMV_EXPERIMENT
-    // tuning builds: the deeper ring, selected with MI355Q_STAF_DEPTH
-    if (argmax) return go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 4, true, false>);
-    switch (mt) {
-    case 1: return go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 4, false, false>);
-    case 2: return go(gemv_staf_kernel<BITS, GROUP, 2, kWaves, 4, false, false>);
-    default: return go(gemv_staf_kernel<BITS, GROUP, 4, kWaves, 4, false, false>);
-    }
-#else
     return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no block-layout GEMV with ring depth %d", depth);
-#endif
 }
 
 mi355q_status launch_by_format(hipStream_t s, uint32_t bits, uint32_t group, const StafArgs& a, int mt, int depth,

@@ -338,9 +338,6 @@ size_t t16_staged_bytes(uint32_t m, uint32_t k) { return (size_t)m * ((size_t)k 
 // 14336 -> 4096: M = 8 in two parts 18.6 us, in four 14.2 us; M = 16 in four 16.4 us, in eight 17.6 us).
 uint32_t t16_parts(uint32_t k, uint32_t m, uint32_t n_row_tiles, uint32_t cus) {
     const uint32_t kblocks = k / 128;
-    const int forced = env_int_cached("MI355Q_T16_PARTS", 0);
-    if (forced > 0 && kblocks % (uint32_t)forced == 0 && t16_staged_bytes(m, k / (uint32_t)forced) <= kT16LdsBudget)
-        return (uint32_t)forced;
     if (t16_staged_bytes(m, k) <= kT16LdsBudget) return 1;
     uint32_t first_fit = 0;
     for (uint32_t p = 2; p <= 16 && kblocks % p == 0; p *= 2) {
@@ -453,9 +450,6 @@ Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_row_ti
         while (ks < most_ks && kblocks / (ks * 2) >= 2) ks *= 2;
         if (ks > most_ks) ks = most_ks;
     }
-    const int eks = env_int_cached("MI355Q_T16_KSPLIT", 0), etpw = env_int_cached("MI355Q_T16_TPW", 0);
-    if (eks) ks = (uint32_t)eks;
-    if (etpw) tpw = (uint32_t)etpw;
     g.ksplit = ks;
     g.tiles_per_wg = tpw;
     g.waves = ks * tpw;
@@ -472,8 +466,6 @@ Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_row_ti
         if (want > most || one_wg_per_cu) want = most;
         if (want > 16) want = 16;
         g.passes = want ? want : 1;
-        const int ep = env_int_cached("MI355Q_T16_PASSES", 0);
-        if (ep) g.passes = (uint32_t)ep;
     }
     g.wgs_per_part = (n_row_tiles + tpw * g.passes - 1) / (tpw * g.passes);
     g.grid = g.wgs_per_part * parts;

@@ -21,6 +21,7 @@
 //     the same M-tile: the activation rows they share stay in that XCD's L2;
 //   * fp32 accumulators are rounded once, to the output type, in the epilogue.
 #include "device_utils.h"
+#include <atomic>
 
 namespace mi355q {
 
@@ -43,7 +44,6 @@ struct GemmArgs {
     uint32_t kblocks;        // TILE16: K / 128
     float* partial;          // split-K: fp32 [splits][M][N] partial results (null when K is not split)
     uint32_t kt_per_split;   // K-tiles per split (blockIdx.y indexes the split)
-    uint32_t dbg;            // tuning builds only: bit0 fetch only the first K-tile, bit1 fill LDS only once
     unsigned long long* probe;   // optional: [0] shader cycles, [1] 100 MHz ticks that workgroup 0 spent in the kernel
 };
 
@@ -350,14 +350,8 @@ __global__ __launch_bounds__(WAVES * 64, (STAGES == 1 ? 2 : 1)) void qgemm_mfma_
         }
     } else {
         for (uint32_t kt = kt0; kt < KT; kt++) {
-#ifdef MI355Q_GEMV_EXPERIMENT
-            if (!(a.dbg & 2) || kt == kt0)
-#endif
             stash(0);
             __syncthreads();
-#ifdef MI355Q_GEMV_EXPERIMENT
-            if (!(a.dbg & 1))
-#endif
             if (kt + 1 < KT) fetch(kt + 1);      // in flight during the matrix-core phase
             multiply(0);
             __syncthreads();                     // every wavefront is done reading before the next fill
@@ -415,31 +409,24 @@ GemmLaunchShape gemm_mfma_shape(const mi355q_context* ctx, uint32_t m, uint32_t 
     const uint32_t cus = (uint32_t)ctx->props.multiProcessorCount;
     auto tiles = [&](uint32_t bm, uint32_t bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); };
     GemmLaunchShape g{};
-    int pick = env_int_cached("MI355Q_GEMM_TILE", 0);
     const uint32_t kt = k / kTileK;
     // 256 x 256 tiles on eight wavefronts when they fill the chip, alone or with K split so that tiles x splits comes
     // to about one workgroup per CU and a split keeps sixteen K-tiles (M = 2048, 14336 -> 4096: 128 tiles, 333 us
     // as 512 tiles of 128 x 128, 236 us as 128 x 2; M = 1024: 204 -> 131 us as 64 x 4; 4096 -> 14336 at M = 1024:
     // 171 -> 126 us as 224 x 1); else 128 x 128 tiles, split over K when they leave half the CUs idle.
     uint32_t wide_splits = 0;
-    if (pick == 0) {
-        const uint32_t t256 = tiles(256, 256);
-        if (m > 128 && 10 * t256 >= 9 * cus) {
-            pick = 5;
-        } else if (m >= 256) {
-            uint32_t sp = cus / t256;
-            while (sp > 1 && kt / sp < 16) sp--;
-            if (sp >= 1 && t256 * sp * 4 >= cus * 3) { pick = 5; wide_splits = sp; }
-        }
-        if (pick == 0) pick = 3;
+    bool wide = false;
+    const uint32_t t256 = tiles(256, 256);
+    if (m > 128 && 10 * t256 >= 9 * cus) {
+        wide = true;
+    } else if (m >= 256) {
+        uint32_t sp = cus / t256;
+        while (sp > 1 && kt / sp < 16) sp--;
+        if (sp >= 1 && t256 * sp * 4 >= cus * 3) { wide = true; wide_splits = sp; }
     }
-    if (pick == 1) { g.bm = 256; g.bn = 256; g.stages = 2; }
-    else if (pick == 5) { g.bm = 256; g.bn = 256; g.stages = 2; g.block = 512; }
-    else if (pick == 2) { g.bm = 256; g.bn = 128; g.stages = 1; }
-    else if (pick == 4) { g.bm = 128; g.bn = 128; g.stages = 1; }
-    else { g.bm = 128; g.bn = 128; g.stages = 2; }
+    if (wide) { g.bm = 256; g.bn = 256; g.stages = 2; g.block = 512; }
+    else { g.bm = 128; g.bn = 128; g.stages = 2; g.block = 256; }
     g.grid = (tiles(g.bm, g.bn) + 7) / 8 * 8;
-    if (!g.block) g.block = 256;
     // K is split over workgroups when the tiles alone leave most CUs idle (short M): each split writes
     // an fp32 partial, a second launch adds them.  At least 8 K-tiles per split.
     g.splits = wide_splits ? wide_splits : 1;
@@ -449,8 +436,6 @@ GemmLaunchShape gemm_mfma_shape(const mi355q_context* ctx, uint32_t m, uint32_t 
         while (want > 1 && kt / want < 8) want--;
         g.splits = want ? want : 1;
     }
-    const int es = env_int_cached("MI355Q_GEMM_SPLITK", 0);
-    if (es) g.splits = (uint32_t)es;
     g.kt_per_split = (kt + g.splits - 1) / g.splits;
     g.splits = (kt + g.kt_per_split - 1) / g.kt_per_split;
     g.lds_bytes = g.stages * (g.bm + g.bn) * (uint32_t)kRowBytes;
@@ -467,10 +452,14 @@ mi355q_status launch_tile_sb(hipStream_t s, GemmArgs a) {
     const uint32_t grid = (total + 7) / 8 * 8;
     constexpr size_t lds = (size_t)STAGES * (BM + BN) * kRowBytes;
     auto kern = qgemm_mfma_kernel<BITS, GROUP, BM, BN, QUANT, STAGES, SB_BF16, WAVES, T16>;
-    static bool lds_limit_raised = false;      // per instantiation; the library drives one device
-    if (!lds_limit_raised) {
+    // The attribute belongs to the function on one device: one bit per device and instantiation.
+    static std::atomic<uint64_t> lds_limit_raised{0};
+    int device = 0;
+    MI355Q_HIP(hipGetDevice(&device));
+    const uint64_t bit = 1ull << (device & 63);
+    if (!(lds_limit_raised.load(std::memory_order_relaxed) & bit)) {
         MI355Q_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        lds_limit_raised = true;
+        lds_limit_raised.fetch_or(bit, std::memory_order_relaxed);
     }
     const uint32_t kt = a.k / kTileK;
     const uint32_t splits = a.partial ? (kt + a.kt_per_split - 1) / a.kt_per_split : 1;
@@ -512,12 +501,6 @@ mi355q_status launch_shape(hipStream_t s, mi355q_context* ctx, GemmArgs a) {
         a.kt_per_split = g.kt_per_split;
     }
     if (g.bm == 256 && g.bn == 256 && g.block == 512) return launch_tile<BITS, GROUP, 256, 256, QUANT, 2, 8>(s, a);
-#ifdef MI355Q_GEMV_EXPERIMENT
-    // tuning builds: the other tile shapes, selected with MI355Q_GEMM_TILE
-    if (g.bm == 256 && g.bn == 256) return launch_tile<BITS, GROUP, 256, 256, QUANT, 2>(s, a);
-    if (g.bm == 256 && g.bn == 128) return launch_tile<BITS, GROUP, 256, 128, QUANT, 1>(s, a);
-    if (g.stages == 1) return launch_tile<BITS, GROUP, 128, 128, QUANT, 1>(s, a);
-#endif
     return launch_tile<BITS, GROUP, 128, 128, QUANT, 2>(s, a);
 }
 
@@ -550,7 +533,6 @@ mi355q_status launch_qgemm_mfma(hipStream_t s, mi355q_context* ctx, const WView&
     a.m = m; a.n = w.n; a.k = w.k; a.xs = x_stride; a.ys = y_stride;
     a.code_stride = w.code_stride; a.sz_stride = w.sz_stride;
     a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = w.sb_dtype;
-    a.dbg = (uint32_t)env_int_cached("MI355Q_GEMM_DBG", 0);
     a.probe = probe;
     switch (w.bits * 1000 + w.group) {
     case 4064: return launch_shape<4, 64, true>(s, ctx, a);
@@ -577,7 +559,6 @@ mi355q_status launch_gemm_bf16_mfma(hipStream_t s, mi355q_context* ctx, const vo
     a.x = (const uint16_t*)a_ptr; a.y = c;
     a.m = m; a.n = n; a.k = k; a.xs = a_stride; a.ys = c_stride;
     a.y_dtype = (uint32_t)c_dtype;
-    a.dbg = (uint32_t)env_int_cached("MI355Q_GEMM_DBG", 0);
     return launch_shape<4, 64, false>(s, ctx, a);
 }
 

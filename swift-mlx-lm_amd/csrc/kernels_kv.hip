@@ -186,7 +186,7 @@ __global__ __launch_bounds__(256) void kv_cache_write_hd128x4_kernel(KvArgs a) {
 // One thread per element of the output rows.
 __global__ __launch_bounds__(256) void kv_cache_read_kernel(KvArgs a) {
     const uint32_t row_elems = a.kv_heads * a.head_dim;
-    const uint32_t p = blockIdx.y;
+    for (uint32_t p = blockIdx.y; p < a.count; p += gridDim.y)     // positions beyond the grid's y limit wrap round
     for (uint32_t e = blockIdx.x * 256 + threadIdx.x; e < row_elems; e += gridDim.x * 256) {
         const uint32_t h = e / a.head_dim, d = e - h * a.head_dim;
         const uint8_t* slot = a.cache + kv_slot_offset(a, h, a.first_position + p);
@@ -214,7 +214,7 @@ __global__ __launch_bounds__(256) void kv_cache_read_kernel(KvArgs a) {
 // Same arithmetic per element as the kernel above.
 __global__ __launch_bounds__(256) void kv_cache_read_x4_kernel(KvArgs a) {
     const uint32_t row_elems = a.kv_heads * a.head_dim;
-    const uint32_t p = blockIdx.y;
+    for (uint32_t p = blockIdx.y; p < a.count; p += gridDim.y)
     for (uint32_t e = (blockIdx.x * 256 + threadIdx.x) * 4; e < row_elems; e += gridDim.x * 1024) {
         const uint32_t h = e / a.head_dim, d = e - h * a.head_dim;
         const uint8_t* slot = a.cache + kv_slot_offset(a, h, a.first_position + p);
@@ -356,6 +356,7 @@ mi355q_status mi355q_kv_cache_read(mi355q_context* ctx, void* stream, const mi35
     a.out = out_dev;
     const uint32_t row = a.kv_heads * a.head_dim;
     const size_t esz = a.dtype == MI355Q_F32 ? 4 : 2;
+    const uint32_t by = a.count < 65535u ? a.count : 65535u;     // grid y limit; the kernels stride over the rest
     // four elements per thread: whole groups of four, 4-byte aligned slots and blocks, 8- or 16-byte aligned output rows
     const bool four = a.bits != 0 && a.head_dim % 4 == 0 && a.group % 4 == 0 && a.slot_bytes % 4 == 0 &&
                       a.bytes_per_block % 4 == 0 && (uintptr_t)a.cache % 4 == 0 && a.row_stride % 4 == 0 &&
@@ -363,13 +364,13 @@ mi355q_status mi355q_kv_cache_read(mi355q_context* ctx, void* stream, const mi35
     if (four) {
         uint32_t bx = (row / 4 + 255) / 256;
         if (bx > 64) bx = 64;
-        kv_cache_read_x4_kernel<<<dim3(bx, a.count), dim3(256), 0, (hipStream_t)stream>>>(a);
+        kv_cache_read_x4_kernel<<<dim3(bx, by), dim3(256), 0, (hipStream_t)stream>>>(a);
         MI355Q_HIP(hipGetLastError());
         return MI355Q_OK;
     }
     uint32_t bx = (row + 255) / 256;
     if (bx > 64) bx = 64;
-    kv_cache_read_kernel<<<dim3(bx, a.count), dim3(256), 0, (hipStream_t)stream>>>(a);
+    kv_cache_read_kernel<<<dim3(bx, by), dim3(256), 0, (hipStream_t)stream>>>(a);
     MI355Q_HIP(hipGetLastError());
     return MI355Q_OK;
 }

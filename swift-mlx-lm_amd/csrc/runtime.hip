@@ -87,6 +87,22 @@ uint16_t host_f32_to_f16(float f) {
 
 float host_bf16_to_f32(uint16_t h) { return as_f32((uint32_t)h << 16); }
 
+float host_f16_to_f32(uint16_t h) {
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16, e = (h >> 10) & 0x1Fu, m = h & 0x3FFu;
+    if (e == 0x1Fu) return as_f32(sign | 0x7F800000u | (m << 13));
+    if (e) return as_f32(sign | ((e + 112u) << 23) | (m << 13));
+    const float v = (float)m * 5.9604644775390625e-8f;        // subnormal: m * 2^-24 (exact)
+    return sign ? -v : v;
+}
+
+// A bf16 scale or bias as the converter would store it (narrowed to f16, round to nearest even), written back as
+// bf16.  The narrowed value always has a bf16 spelling: inside the f16 normal range the 8 significant bits of a bf16
+// survive, below it rounding to the f16 subnormal grid can only drop bits, above it the result is infinity.  So a
+// plane of these values decodes to exactly what the f16 header of the block layout decodes to.
+uint16_t host_bf16_through_f16(uint16_t h) {
+    return (uint16_t)(as_u32(host_f16_to_f32(host_f32_to_f16(host_bf16_to_f32(h)))) >> 16);
+}
+
 float host_load_sb(const void* p, size_t i, int dtype) {
     if (dtype == MI355Q_F32) return ((const float*)p)[i];
     if (dtype == MI355Q_BF16) return host_bf16_to_f32(((const uint16_t*)p)[i]);
@@ -462,6 +478,15 @@ mi355q_status mi355q_weight_prepare_mlx(mi355q_context* ctx, uint8_t scheme_iden
                 w->sb_dtype = MI355Q_F16;
                 st = upload_new(&w->scales, s16.data(), w->sb_bytes);
                 if (st == MI355Q_OK) st = upload_new(&w->biases, z16.data(), w->sb_bytes);
+            } else if (sb_dtype == MI355Q_BF16) {  // kept as bf16, holding the values the converter's f16 would hold
+                std::vector<uint16_t> sb(groups), zb(groups);
+                for (size_t i = 0; i < groups; i++) {
+                    sb[i] = host_bf16_through_f16(((const uint16_t*)scales_host)[i]);
+                    zb[i] = host_bf16_through_f16(((const uint16_t*)biases_host)[i]);
+                }
+                w->sb_dtype = MI355Q_BF16;
+                st = upload_new(&w->scales, sb.data(), w->sb_bytes);
+                if (st == MI355Q_OK) st = upload_new(&w->biases, zb.data(), w->sb_bytes);
             } else {
                 w->sb_dtype = (uint8_t)sb_dtype;
                 st = upload_new(&w->scales, scales_host, w->sb_bytes);

@@ -107,3 +107,35 @@ def test_kv_cache_argument_errors(pkg, ctx):
     with pytest.raises(pkg.MI355QError):
         ctx.kv_cache_read(spec, cd, None, pkg.F32, 0, 1)
     cd.free(); xd.free()
+
+
+@pytest.mark.parametrize("scheme,out_dtype", [(0x40, 1), (0x10, 2), (0x01, 1)])
+def test_kv_cache_read_of_more_positions_than_one_grid_dimension(pkg, ctx, scheme, out_dtype):
+    """One read of 70 000 positions (more than the 65 535 workgroups a grid holds along y) returns what three
+    shorter reads return, and its last positions match the oracle."""
+    heads, hd, count = 1, 64, 70000
+    spec = pkg.KVCacheSpecification(scheme, pkg.KV_SEQUENCE_MAJOR, heads, hd, count)
+    rng = np.random.default_rng(scheme)
+    x = rng.standard_normal((count, hd)).astype(np.float32)
+    xd = ctx.upload(x)
+    cd = ctx.alloc(spec.bytes_per_layer); ctx.fill(cd, 0)
+    ctx.kv_cache_write(spec, cd, xd, pkg.F32, 0, count)
+    esz = 4 if out_dtype == pkg.F32 else 2
+    whole = ctx.alloc(count * hd * esz); ctx.fill(whole, 0x7FC07FC0)
+    parts = ctx.alloc(count * hd * esz); ctx.fill(parts, 0x7FC07FC0)
+    ctx.kv_cache_read(spec, cd, whole, out_dtype, 0, count)
+    for first, n in [(0, 30000), (30000, 30000), (60000, 10000)]:
+        ctx.kv_cache_read(spec, cd, pkg.DeviceBuffer(ctx, parts.ptr + first * hd * esz, n * hd * esz), out_dtype, first, n)
+    ctx.synchronize()
+    a = whole.download(np.uint8)
+    assert np.array_equal(a, parts.download(np.uint8))
+    tail_first, tail = 65530, 40
+    cache = cd.download(np.uint8, (spec.bytes_per_layer,))
+    ref = oracle.kv_cache_read(scheme, pkg.KV_SEQUENCE_MAJOR, heads, hd, count, cache, tail_first, tail)
+    got = out_from_device(whole, out_dtype, (count, hd), pkg)[tail_first:tail_first + tail]
+    if out_dtype == pkg.F32:
+        assert np.array_equal(got, ref)
+    else:
+        assert np.array_equal(oracle.bf16_from_f32(got), oracle.bf16_from_f32(ref))
+    for b in (xd, cd, whole, parts):
+        b.free()

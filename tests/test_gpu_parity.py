@@ -111,6 +111,47 @@ def test_dequant_f32_reference_vector_and_seeded_tensor(pkg, ctx):
         out.free(); w.destroy()
 
 
+def test_bf16_scales_outside_the_f16_range_decode_alike_on_every_layout(pkg, ctx):
+    """MLX planes with bf16 scales and biases below the f16 normal range (6.1e-5), on the f16 subnormal grid, below
+    it, and above 65504: the converter narrows them to f16 (STAFConverter.swift:326-368), so all three device layouts
+    must decode to what the oracle decodes from the converter's blocks, bit for bit, and a GEMV must agree too."""
+    bits, group, n, k = 4, 64, 32, 512
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(bits, group)
+    words = kat.mlx_planes(kat.random_codes(991, n, k, bits), bits)
+    rng = np.random.default_rng(992)
+    shape = (n, k // group)
+    mag = np.array([3.1e-5, 5.9e-5, 1.3e-6, 7.7e-8, 2.0e-8, 2.9e-8, 6.2e-5, 1.0e-3, 0.02])
+    s32 = (rng.choice(mag, shape) * rng.uniform(0.8, 1.2, shape)).astype(np.float32)
+    # biases also leave the range at the top (infinite after narrowing); scales stay finite so that no code 0 meets
+    # an infinite scale (whose NaN the host and the device may spell differently)
+    z32 = (rng.choice(np.concatenate([mag, [70000.0, 65504.0, 65519.0]]), shape) * rng.choice([-1.0, 1.0], shape))
+    s, z = oracle.bf16_from_f32(s32).reshape(shape), oracle.bf16_from_f32(z32.astype(np.float32)).reshape(shape)
+    with np.errstate(over="ignore"):
+        s16 = oracle.bf16_to_f32(s).astype(np.float16)           # numpy's cast is round to nearest even
+        z16 = oracle.bf16_to_f32(z).astype(np.float16)
+    assert np.any(s16 == 0) and np.any(np.isinf(z16)) and np.any((s16 != 0) & (np.abs(s16) < 6.1e-5))
+    blocks = oracle.repack_mlx_to_staf(bits, group, words, s, z, oracle.BF16)
+    hdr = blocks.reshape(n * (k // group), -1)[:, :4].copy().view(np.uint16)
+    assert np.array_equal(hdr[:, 0], s16.view(np.uint16).ravel())  # the oracle narrows like numpy does
+    assert np.array_equal(hdr[:, 1], z16.view(np.uint16).ravel())
+    want = oracle.dequant_staf_f32(bits, group, n, k, blocks)
+    x = kat.seeded_activations(993, 1, k)
+    ys = []
+    for layout in (pkg.LAYOUT_STAF_BLOCKS, pkg.LAYOUT_PLANES, pkg.LAYOUT_TILE16):
+        w = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, layout)
+        out = ctx.alloc(n * k * 4)
+        ctx.dequant_f32(w, out); ctx.synchronize()
+        got = out.download(np.float32, (n, k))
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), layout
+        ys.append(run_gemv(ctx, pkg, w, x, pkg.BF16, pkg.F32, 0))
+        out.free(); w.destroy()
+    finite = np.isfinite(ys[0])
+    assert np.array_equal(finite, np.isfinite(ys[1])) and np.array_equal(finite, np.isfinite(ys[2]))
+    scale = np.maximum(1e-30, np.abs(ys[0][finite]))
+    for y in ys[1:]:
+        assert np.max(np.abs(y[finite] - ys[0][finite]) / scale) < 1e-3
+
+
 # ------------------------------------------------------------- closed-form GEMV KATs (a4)
 def _check_kat(pkg, ctx, case, x, tol=2e-6):
     want = kat.exact_gemv(case.codes, case.scales, case.zeros, x, case.group)

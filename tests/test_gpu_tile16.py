@@ -13,7 +13,7 @@ import pytest
 
 import kat
 import oracle
-from gpu_util import Case, act_rounded, assert_within_tolerance, out_from_device, seeded_case
+from gpu_util import Case, act_rounded, assert_within_tolerance, out_from_device, run_gemv, seeded_case
 
 pytestmark = pytest.mark.gpu
 
@@ -397,3 +397,18 @@ def test_tile16_plan_replay_and_graph(pkg, ctx):
         b.free()
     for w in ws:
         w.destroy()
+
+
+@pytest.mark.parametrize("x_dtype_name", ["F16", "F32"])
+def test_tile16_other_activation_types_take_the_per_code_kernel_whole(pkg, ctx, x_dtype_name):
+    """The tile kernel reads bf16 activations only.  f16 and fp32 rows go to the per-code kernel, which takes all M
+    rows in one launch (no walk in steps of sixteen, eight ... one row)."""
+    x_dtype = getattr(pkg, x_dtype_name)
+    n, k = 96, 512
+    words, s, z, wq = seeded_case(2931, n, k, 4, 64)
+    w = ctx.weight_prepare_mlx(_fmt(pkg), words, s, z, pkg.BF16, pkg.LAYOUT_TILE16)
+    for m in (1, 13, 200):
+        x = act_rounded(kat.seeded_activations(2932 + m, m, k), x_dtype, pkg)
+        got = run_gemv(ctx, pkg, w, x, x_dtype, pkg.F32, 0, use_qgemm=True)
+        assert_within_tolerance(got, oracle.gemm_f64(wq, x), f"{x_dtype_name} M={m}")
+    w.destroy()
