@@ -87,8 +87,9 @@ enum {
     MI355Q_FLAG_NONE = 0,
     MI355Q_FLAG_FORCE_GENERIC = 1, /* run the reference-shaped per-code kernel (A/B and tests) */
     MI355Q_FLAG_FORCE_SMALL_M = 2, /* qgemm: use the small-M GEMV-style kernel whatever M is */
-    MI355Q_FLAG_FORCE_MFMA = 4     /* qgemm: use the MFMA kernel whatever M is */
+    MI355Q_FLAG_FORCE_MFMA = 4,    /* qgemm: use the fused MFMA kernel whatever M is */
     /* bit 3 (value 8) is taken by the measurement flag of mi355_qlinear_probe.h */
+    MI355Q_FLAG_FORCE_TWO_STEP = 16 /* qgemm: dequantise to bf16 scratch, then the dense library GEMM, whatever M is */
 };
 
 /* ------------------------------------------------------------------------------------------
@@ -260,11 +261,23 @@ MI355Q_API mi355q_status mi355q_qgemv(mi355q_context* ctx, void* stream, const m
                                       uint32_t y_row_stride, uint32_t flags);
 
 /* Prefill projection: gemm_q4_g64_f32s / gemm_q8_g32_f32s (:22-156) and the two-step
- * dequant_q*_bf16 + gemm_bf16_f32s path (:361-416, MC/Generator/MetalSourceGenerator+Linear.swift:18-81)
- * as ONE fused kernel: code tiles are dequantised to bf16 in LDS and contracted on MFMA with
- * fp32 accumulation.  Any M >= 1; M is a run-time value (the reference rebinds sequenceLength
- * per call, MC/Compiler/MetalPrefillStepBuilder.swift:728-732).  Small M routes to the
- * GEMV-style kernel unless flags say otherwise.  Launches that split K over workgroups (few output
+ * dequant_q*_bf16 + gemm_bf16_f32s path (:361-416, MC/Generator/MetalSourceGenerator+Linear.swift:18-81).
+ * Any M >= 1; M is a run-time value (the reference rebinds sequenceLength per call,
+ * MC/Compiler/MetalPrefillStepBuilder.swift:728-732).  Three routes, all with the weights rounded once
+ * to bf16 and fp32 accumulation, chosen by measured cost unless flags say otherwise
+ * (mi355q_plan_prefill_steps reports the choice):
+ *   - small M (up to 8 rows, 16 on TILE16): the GEMV-style decode kernels;
+ *   - ONE fused kernel: code tiles are dequantised to bf16 in LDS and contracted on MFMA (the planes
+ *     and TILE16 layouts, formats q4 g64/g128, q8 g32/g64, q6/q3/q2 g64, bf16 activations);
+ *   - two dispatches, as the reference's second route: the whole matrix is dequantised to bf16 in a
+ *     scratch matrix of the context (N*K*2 bytes, plus 64 MiB of library workspace) and multiplied by
+ *     the platform's dense GEMM library (hipBLASLt, opened with dlopen on first use; the reference
+ *     calls matmul2d there).  Serves every registered format on every layout: from 16 rows where the
+ *     fused kernel does not read the weight, from 2048 rows beside it (4096 when K > N).  bf16
+ *     activations, fp32 or bf16 output, K and the row stride multiples of 8, 16-byte aligned x.  The
+ *     first eager call of a shape times the library's candidate algorithms once (a few milliseconds)
+ *     and keeps the quickest.  When the library is absent or has no algorithm, the other routes serve.
+ * Launches that split K over workgroups (few output
  * tiles at short M; on the TILE16 layout, rows too long for M staged activation rows) keep fp32
  * partial results in a scratch buffer of the context, grown on first use: two such launches of one
  * context must not overlap on different streams, and the first one of a size allocates (run a plan
@@ -297,7 +310,9 @@ MI355Q_API mi355q_status mi355q_dequant_f32(mi355q_context* ctx, void* stream,
 
 /* gemm_bf16_f32s (generateMPPGEMM, MC/Generator/MetalSourceGenerator+Linear.swift:18-81):
  * C[M,N] = A[M, a_row_stride>=K] * B[N,K]^T with B dense bf16 (the dequant scratch), MFMA,
- * fp32 accumulation. */
+ * fp32 accumulation.  From 128 rows the product goes to the platform's dense GEMM library, as the
+ * reference's goes to matmul2d (bf16 A, fp32 or bf16 C, aligned operands); else, and when the
+ * library cannot serve, this library's own matrix-core kernel runs. */
 MI355Q_API mi355q_status mi355q_gemm_bf16(mi355q_context* ctx, void* stream, const void* a_dev,
                                           mi355q_dtype a_dtype, const void* b_bf16_dev,
                                           void* c_dev, mi355q_dtype c_dtype, uint32_t m,

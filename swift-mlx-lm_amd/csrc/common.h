@@ -52,6 +52,8 @@ struct WView {
 
 }  // namespace mi355q
 
+namespace mi355q { struct DenseLibrary; }
+
 struct mi355q_context {
     int device;
     hipDeviceProp_t props;
@@ -66,6 +68,9 @@ struct mi355q_context {
     size_t workspace_bytes;
     void* retired[40];
     int retired_count;
+    // the platform's dense GEMM library (second half of the two-dispatch prefill route), opened on first use
+    mi355q::DenseLibrary* dense_library;
+    bool dense_library_failed;
 };
 constexpr int kRetiredWorkspaces = 40;
 
@@ -211,6 +216,27 @@ bool gemm_mfma_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stri
 mi355q_status launch_qgemm_mfma(hipStream_t s, mi355q_context* ctx, const WView& w,
                                 const void* x, int x_dtype, void* y, int y_dtype, uint32_t m,
                                 uint32_t x_stride, uint32_t y_stride, unsigned long long* probe = nullptr);
+// Two-dispatch prefill route: dequantise the whole matrix to bf16 in the context's scratch, then the platform's
+// dense GEMM.  `dense_library_serves` answers whether the library can be opened and has an algorithm for the problem.
+constexpr size_t kDenseLibraryWorkspace = (size_t)64 << 20;
+bool dense_library_serves(mi355q_context* ctx, uint32_t m, uint32_t n, uint32_t k, uint32_t x_stride, uint32_t y_stride,
+                          int y_dtype);
+mi355q_status dense_library_gemm(hipStream_t s, mi355q_context* ctx, const uint16_t* x, const uint16_t* w_bf16, void* y,
+                                 int y_dtype, uint32_t m, uint32_t n, uint32_t k, uint32_t x_stride, uint32_t y_stride,
+                                 void* workspace);
+void dense_library_release(mi355q_context* ctx);
+// Rows from which the two-dispatch route is taken.  Beside the fused matrix-core kernel (measured, q4 g64, N(0,1)
+// activations, fused against two-dispatch): 4096 -> 14336 at M = 1024 131 against 140 us, M = 2048 282 against 244 us,
+// M = 4096 580 against 436 us; 14336 -> 4096 at M = 2048 262 against 271 us, M = 4096 477 against 386 us.  Where only
+// the decode kernels would serve (formats and layouts the fused kernel does not read; block layout, 4096 -> 14336:
+// M = 32 in four launches of eight rows 147 us, two-dispatch 47 us) it starts at sixteen rows.
+constexpr uint32_t kTwoStepMinRowsBesideFused = 2048, kTwoStepMinRowsLongK = 4096, kTwoStepMinRowsOtherwise = 16;
+// Rows from which mi355q_gemm_bf16 hands a plain dense product to the library.
+constexpr uint32_t kDenseLibraryMinRows = 128;
+bool gemm_two_step_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
+bool gemm_two_step_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride, uint32_t flags);
+mi355q_status launch_qgemm_two_step(hipStream_t s, mi355q_context* ctx, const WView& w, const void* x, void* y,
+                                    int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride);
 mi355q_status launch_gemm_bf16_mfma(hipStream_t s, mi355q_context* ctx, const void* a,
                                     int a_dtype, const uint16_t* b, void* c, int c_dtype,
                                     uint32_t m, uint32_t n, uint32_t k, uint32_t a_stride,

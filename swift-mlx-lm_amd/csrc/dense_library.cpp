@@ -1,0 +1,219 @@
+// Dense bf16 GEMM of the two-dispatch prefill route through hipBLASLt.
+//
+// The reference's second prefill route is  dequant_q{b}_g{g}_bf16  into a scratch matrix, then the platform's own
+// matmul2d primitive on the dense operands (Sources/MetalCompiler/Generator/MetalSourceGenerator+Linear.swift:18-81,
+// bindings Sources/MetalCompiler/Compiler/MetalPrefillStepBuilder.swift:928-955).  Here the dequantisation is this
+// library's kernel and the dense product is the platform's GEMM library.  hipBLASLt is opened with dlopen on first
+// use, so libmi355_qlinear.so itself has no link-time dependency on it and callers that never reach this route never
+// load it; when it cannot be opened the route reports itself unavailable and the fused kernel serves the call.
+//
+// Operands, in the library's column-major terms:  Y^T [N x M, ld ys] = W^T-as-stored [K x N, ld K]^T * X^T [K x M, ld xs].
+#include "common.h"
+
+#include <dlfcn.h>
+#include <hipblaslt/hipblaslt.h>
+
+#include <mutex>
+#include <vector>
+
+namespace mi355q {
+namespace {
+
+struct Api {
+    void* so = nullptr;
+    bool tried = false;
+    decltype(&hipblasLtCreate) create = nullptr;
+    decltype(&hipblasLtDestroy) destroy = nullptr;
+    decltype(&hipblasLtMatrixLayoutCreate) layout_create = nullptr;
+    decltype(&hipblasLtMatrixLayoutDestroy) layout_destroy = nullptr;
+    decltype(&hipblasLtMatmulDescCreate) desc_create = nullptr;
+    decltype(&hipblasLtMatmulDescDestroy) desc_destroy = nullptr;
+    decltype(&hipblasLtMatmulDescSetAttribute) desc_set = nullptr;
+    decltype(&hipblasLtMatmulPreferenceCreate) pref_create = nullptr;
+    decltype(&hipblasLtMatmulPreferenceDestroy) pref_destroy = nullptr;
+    decltype(&hipblasLtMatmulPreferenceSetAttribute) pref_set = nullptr;
+    decltype(&hipblasLtMatmulAlgoGetHeuristic) heuristic = nullptr;
+    decltype(&hipblasLtMatmul) matmul = nullptr;
+};
+
+Api g_api;
+std::mutex g_api_mu;
+
+template <typename F>
+bool resolve(void* so, const char* name, F& out) {
+    out = (F)dlsym(so, name);
+    return out != nullptr;
+}
+
+const Api* api() {
+    std::lock_guard<std::mutex> lock(g_api_mu);
+    if (g_api.tried) return g_api.so ? &g_api : nullptr;
+    g_api.tried = true;
+    void* so = dlopen("libhipblaslt.so.1", RTLD_NOW | RTLD_LOCAL);
+    if (!so) so = dlopen("/opt/rocm/lib/libhipblaslt.so.1", RTLD_NOW | RTLD_LOCAL);
+    if (!so) so = dlopen("libhipblaslt.so", RTLD_NOW | RTLD_LOCAL);
+    if (!so) return nullptr;
+    Api a;
+    const bool ok = resolve(so, "hipblasLtCreate", a.create) && resolve(so, "hipblasLtDestroy", a.destroy) &&
+                    resolve(so, "hipblasLtMatrixLayoutCreate", a.layout_create) &&
+                    resolve(so, "hipblasLtMatrixLayoutDestroy", a.layout_destroy) &&
+                    resolve(so, "hipblasLtMatmulDescCreate", a.desc_create) &&
+                    resolve(so, "hipblasLtMatmulDescDestroy", a.desc_destroy) &&
+                    resolve(so, "hipblasLtMatmulDescSetAttribute", a.desc_set) &&
+                    resolve(so, "hipblasLtMatmulPreferenceCreate", a.pref_create) &&
+                    resolve(so, "hipblasLtMatmulPreferenceDestroy", a.pref_destroy) &&
+                    resolve(so, "hipblasLtMatmulPreferenceSetAttribute", a.pref_set) &&
+                    resolve(so, "hipblasLtMatmulAlgoGetHeuristic", a.heuristic) &&
+                    resolve(so, "hipblasLtMatmul", a.matmul);
+    if (!ok) return nullptr;
+    a.so = so;
+    a.tried = true;
+    g_api = a;
+    return &g_api;
+}
+
+hipDataType data_type(int dtype) {
+    return dtype == MI355Q_F32 ? HIP_R_32F : dtype == MI355Q_BF16 ? HIP_R_16BF : HIP_R_16F;
+}
+
+constexpr int kCandidates = 8;
+
+// One problem the context has met: its descriptors and the algorithm the library's heuristic ranks first.
+struct Problem {
+    uint32_t m, n, k, xs, ys;
+    int y_dtype;
+    bool usable;
+    hipblasLtMatmulDesc_t desc;
+    hipblasLtMatrixLayout_t a, b, c;
+    hipblasLtMatmulAlgo_t algo;                       // the one in use: the heuristic's first until `timed`
+    hipblasLtMatmulAlgo_t ranked[kCandidates];        // what the heuristic returned, in its order
+    int candidates;
+    bool timed;                                       // the candidates have been timed on the device
+};
+
+}  // namespace
+
+struct DenseLibrary {
+    const Api* api;
+    hipblasLtHandle_t handle;
+    std::vector<Problem> problems;
+};
+
+namespace {
+
+DenseLibrary* library_of(mi355q_context* ctx) {
+    if (ctx->dense_library) return ctx->dense_library;
+    if (ctx->dense_library_failed) return nullptr;
+    const Api* a = api();
+    hipblasLtHandle_t h = nullptr;
+    if (!a || a->create(&h) != HIPBLAS_STATUS_SUCCESS) {
+        ctx->dense_library_failed = true;
+        return nullptr;
+    }
+    ctx->dense_library = new DenseLibrary{a, h, {}};
+    return ctx->dense_library;
+}
+
+Problem* find_problem(DenseLibrary* lib, uint32_t m, uint32_t n, uint32_t k, uint32_t xs, uint32_t ys, int y_dtype) {
+    for (Problem& p : lib->problems)
+        if (p.m == m && p.n == n && p.k == k && p.xs == xs && p.ys == ys && p.y_dtype == y_dtype) return &p;
+    const Api* a = lib->api;
+    Problem p{};
+    p.m = m; p.n = n; p.k = k; p.xs = xs; p.ys = ys; p.y_dtype = y_dtype;
+    const hipblasOperation_t op_t = HIPBLAS_OP_T, op_n = HIPBLAS_OP_N;
+    hipblasLtMatmulPreference_t pref = nullptr;
+    const uint64_t most = kDenseLibraryWorkspace;
+    bool ok = a->desc_create(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) == HIPBLAS_STATUS_SUCCESS &&
+              a->desc_set(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &op_t, sizeof op_t) == HIPBLAS_STATUS_SUCCESS &&
+              a->desc_set(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &op_n, sizeof op_n) == HIPBLAS_STATUS_SUCCESS &&
+              a->layout_create(&p.a, HIP_R_16BF, k, n, k) == HIPBLAS_STATUS_SUCCESS &&
+              a->layout_create(&p.b, HIP_R_16BF, k, m, xs) == HIPBLAS_STATUS_SUCCESS &&
+              a->layout_create(&p.c, data_type(y_dtype), n, m, ys) == HIPBLAS_STATUS_SUCCESS &&
+              a->pref_create(&pref) == HIPBLAS_STATUS_SUCCESS &&
+              a->pref_set(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &most, sizeof most) == HIPBLAS_STATUS_SUCCESS;
+    if (ok) {
+        hipblasLtMatmulHeuristicResult_t found[kCandidates];
+        int count = 0;
+        ok = a->heuristic(lib->handle, p.desc, p.a, p.b, p.c, p.c, pref, kCandidates, found, &count) == HIPBLAS_STATUS_SUCCESS;
+        p.candidates = 0;
+        for (int i = 0; ok && i < count; i++)
+            if (found[i].state == HIPBLAS_STATUS_SUCCESS && found[i].workspaceSize <= kDenseLibraryWorkspace)
+                p.ranked[p.candidates++] = found[i].algo;
+        ok = ok && p.candidates > 0;
+        if (ok) p.algo = p.ranked[0];
+    }
+    if (pref) a->pref_destroy(pref);
+    p.usable = ok;
+    lib->problems.push_back(p);      // an unusable problem is remembered too: the question is not asked again
+    return &lib->problems.back();
+}
+
+}  // namespace
+
+bool dense_library_serves(mi355q_context* ctx, uint32_t m, uint32_t n, uint32_t k, uint32_t x_stride, uint32_t y_stride,
+                          int y_dtype) {
+    DenseLibrary* lib = library_of(ctx);
+    if (!lib) return false;
+    return find_problem(lib, m, n, k, x_stride, y_stride, y_dtype)->usable;
+}
+
+mi355q_status dense_library_gemm(hipStream_t s, mi355q_context* ctx, const uint16_t* x, const uint16_t* w_bf16, void* y,
+                                 int y_dtype, uint32_t m, uint32_t n, uint32_t k, uint32_t x_stride, uint32_t y_stride,
+                                 void* workspace) {
+    DenseLibrary* lib = library_of(ctx);
+    if (!lib) return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the dense GEMM library (hipBLASLt) could not be opened");
+    Problem* p = find_problem(lib, m, n, k, x_stride, y_stride, y_dtype);
+    if (!p->usable)
+        return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the dense GEMM library has no algorithm for M=%u N=%u K=%u", m, n, k);
+    const float one = 1.0f, zero = 0.0f;
+    // First eager call of a problem: time the candidates the heuristic ranked (its first is often not the fastest at
+    // these shapes) on the caller's operands and keep the quickest.  Not while the stream is being captured: a
+    // capture takes the algorithm in use, so run a problem once before capturing it.
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    (void)hipStreamIsCapturing(s, &capture);
+    if (!p->timed && p->candidates > 1 && capture == hipStreamCaptureStatusNone) {
+        p->timed = true;
+        hipEvent_t e0 = nullptr, e1 = nullptr;
+        if (hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
+            float best = 0.f;
+            int best_i = -1;
+            for (int i = 0; i < p->candidates; i++) {
+                bool ran = true;
+                float ms = 0.f;
+                for (int rep = 0; rep < 3 && ran; rep++) {         // the first run warms up, the last two are timed
+                    if (rep == 1) (void)hipEventRecord(e0, s);
+                    ran = lib->api->matmul(lib->handle, p->desc, &one, w_bf16, p->a, x, p->b, &zero, y, p->c, y, p->c,
+                                           &p->ranked[i], workspace, kDenseLibraryWorkspace, s) == HIPBLAS_STATUS_SUCCESS;
+                }
+                if (!ran) continue;
+                if (hipEventRecord(e1, s) != hipSuccess || hipEventSynchronize(e1) != hipSuccess ||
+                    hipEventElapsedTime(&ms, e0, e1) != hipSuccess) continue;
+                if (best_i < 0 || ms < best) { best = ms; best_i = i; }
+            }
+            if (best_i >= 0) p->algo = p->ranked[best_i];
+        }
+        if (e0) (void)hipEventDestroy(e0);
+        if (e1) (void)hipEventDestroy(e1);
+    }
+    const hipblasStatus_t st = lib->api->matmul(lib->handle, p->desc, &one, w_bf16, p->a, x, p->b, &zero, y, p->c, y, p->c,
+                                                &p->algo, workspace, kDenseLibraryWorkspace, s);
+    if (st != HIPBLAS_STATUS_SUCCESS)
+        return fail(MI355Q_ERR_DEVICE, "hipblasLtMatmul failed with status %d (M=%u N=%u K=%u)", (int)st, m, n, k);
+    return MI355Q_OK;
+}
+
+void dense_library_release(mi355q_context* ctx) {
+    DenseLibrary* lib = ctx->dense_library;
+    if (!lib) return;
+    for (Problem& p : lib->problems) {
+        if (p.desc) lib->api->desc_destroy(p.desc);
+        if (p.a) lib->api->layout_destroy(p.a);
+        if (p.b) lib->api->layout_destroy(p.b);
+        if (p.c) lib->api->layout_destroy(p.c);
+    }
+    lib->api->destroy(lib->handle);
+    delete lib;
+    ctx->dense_library = nullptr;
+}
+
+}  // namespace mi355q

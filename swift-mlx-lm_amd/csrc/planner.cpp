@@ -177,6 +177,30 @@ mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w, uint32_t maximum
     const uint32_t small_rows = v.layout == MI355Q_LAYOUT_TILE16 ? 16u : 8u;      // rows the decode kernels take per launch
     const bool want_small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) || m <= small_rows;
     const bool mfma_ok = gemm_mfma_eligible(v, x_dtype, m, input_row_stride);
+    if (gemm_two_step_chosen(v, x_dtype, m, input_row_stride, flags)) {
+        // dequant_q{b}_g{g}_bf16 into the scratch matrix, then the dense GEMM (MetalPrefillStepBuilder's two-dispatch
+        // route; the dense product is the platform library's, as the reference's is matmul2d)
+        *out_count = 2;
+        mi355q_step* d = &out_steps[0];
+        fill_common(w, m, d);
+        d->path = MI355Q_PATH_PREFILL_PROJECTION;
+        d->input_row_stride = input_row_stride;
+        d->flops = 0;
+        std::snprintf(d->kernel_name, sizeof d->kernel_name, "%s", w->fmt.dequant_to_bfloat_kernel_name);
+        std::snprintf(d->device_kernel, sizeof d->device_kernel, "dequant_q%u_g%u_bf16", (unsigned)w->fmt.bits,
+                      w->fmt.group_size);
+        std::snprintf(d->kernel_family, sizeof d->kernel_family, "dequantToBFloat");
+        d->block[0] = 256;
+        s = &out_steps[1];
+        fill_common(w, m, s);
+        s->path = MI355Q_PATH_PREFILL_PROJECTION;
+        s->input_row_stride = input_row_stride;
+        s->weight_bytes = (uint64_t)w->n * w->k * 2;          // the dense operand it reads
+        std::snprintf(s->kernel_name, sizeof s->kernel_name, "gemm_bf16_f32s");
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "hipblaslt_gemm_bf16");
+        std::snprintf(s->kernel_family, sizeof s->kernel_family, "libraryGEMM");
+        return MI355Q_OK;
+    }
     fill_common(w, m, s);
     s->path = MI355Q_PATH_PREFILL_PROJECTION;
     s->input_row_stride = input_row_stride;

@@ -288,6 +288,7 @@ mi355q_status mi355q_context_destroy(mi355q_context* ctx) {
     if (!ctx) return fail(MI355Q_ERR_NULL_HANDLE, "context is null");
     (void)hipSetDevice(ctx->device);
     (void)hipDeviceSynchronize();
+    mi355q::dense_library_release(ctx);
     if (ctx->argmax_scratch) (void)hipFree(ctx->argmax_scratch);
     if (ctx->argmax_partials) (void)hipFree(ctx->argmax_partials);
     if (ctx->workspace) (void)hipFree(ctx->workspace);
