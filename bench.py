@@ -443,6 +443,22 @@ def main():
                      "kernel": plan.step(per_layer - 1)[0].device_kernel}
         log(f"4-launch step on STAF blocks in place: {staf_step['us_per_step']} us/step, {staf_step['GBps']} GB/s")
         plan.destroy()
+        if not a.no_prefill:
+            # prefill straight from the blocks: the gate projection over four rotating copies, as dispatched
+            staf_step["prefill_gate_4096_14336"] = {}
+            wts = [L["gate"] for L in layers[:4]]
+            for mm in (64, 512, 2048):
+                xb = ctx.upload(oracle.bf16_from_f32(kat.seeded_activations(500 + mm, mm, 4096)))
+                yb = ctx.alloc(mm * 14336 * 2)
+                for i in range(4):
+                    ctx.qgemm(wts[i], xb, pkg.BF16, yb, pkg.BF16, mm, 0, 0, 0, stream)
+                ctx.synchronize(stream)
+                ms = time_region(ctx, lambda i: ctx.qgemm(wts[i % 4], xb, pkg.BF16, yb, pkg.BF16, mm, 0, 0, 0, stream), 24, stream)
+                staf_step["prefill_gate_4096_14336"][f"M={mm}"] = {
+                    "us": round(ms * 1e3, 1), "TFLOPs": round(2.0 * mm * 14336 * 4096 / (ms * 1e-3) / 1e12, 1),
+                    "route": " + ".join(st.device_kernel for st in wts[0].plan_prefill_steps(mm, 4096))}
+                xb.free(); yb.free()
+            log(f"  prefill from the blocks (N(0,1)): {staf_step['prefill_gate_4096_14336']}")
         for L in layers:
             for w in L.values():
                 w.destroy()
@@ -504,20 +520,20 @@ def main():
             log(f"  {k_}: {v_}")
 
     # ---- the second half of the metric: the prefill GEMM (benchmark config 3) on N(0,1) activations ------------
-    # both MLP shapes at M = 128, 512, 2048, as dispatched (tile shape, K split and route are the library's choice),
+    # both MLP shapes at M = 128, 512, 2048, 4096, as dispatched (tile shape, K split and route are the library's choice),
     # over four rotating weight copies; the M = 2048 gate projection is the roofline figure.
     prefill, roofline_prefill = None, None
     if not a.no_prefill:
         sweep = {}
         for name, n, k in (("gate 4096->14336", 14336, 4096), ("down 14336->4096", 4096, 14336)):
             wts = [L["gate" if n == 14336 else "down"] for L in layers[:4]]
-            for mm in (128, 512, 2048):
+            for mm in (128, 512, 2048, 4096):
                 xb = ctx.upload(oracle.bf16_from_f32(kat.seeded_activations(500 + mm, mm, k)))        # N(0,1)
                 yb = ctx.alloc(mm * n * 2)
                 for i in range(4):
                     ctx.qgemm(wts[i], xb, pkg.BF16, yb, pkg.BF16, mm, 0, 0, 0, stream)
                 ctx.synchronize(stream)
-                reps = 24 if mm == 2048 else 48
+                reps = 24 if mm >= 2048 else 48
                 ms = time_region(ctx, lambda i: ctx.qgemm(wts[i % len(wts)], xb, pkg.BF16, yb, pkg.BF16, mm, 0, 0, 0, stream), reps, stream)
                 steps_p = wts[0].plan_prefill_steps(mm, k)
                 sweep[f"{name} M={mm}"] = {"us": round(ms * 1e3, 1), "TFLOPs": round(2.0 * mm * n * k / (ms * 1e-3) / 1e12, 1),

@@ -62,8 +62,18 @@ mi355q_status run_small_m(mi355q_context* ctx, hipStream_t s, const mi355q_weigh
             void* yv[1] = {yp};
             const uint32_t strides[1] = {ys};
             st = launch_gemv_tile16_multi(s, ctx, 1, &v, xp, yv, strides, y_dtype, mm, xs, nullptr, nullptr, HeadKeys{});
-        } else if (!generic && gemv_fast_eligible(v, x_dtype, mm, xs) && (uintptr_t)xp % 16 == 0) {
-            st = launch_gemv_fast(s, ctx, v, xp, x_dtype, yp, y_dtype, mm, xs, ys, nullptr, nullptr, HeadKeys{});
+        } else if (!generic && mm >= kMfmaPlanesMinRows && gemv_mfma_planes_eligible(v, x_dtype, mm, xs) &&
+                   (uintptr_t)xp % 16 == 0) {
+            void* yv[1] = {yp};
+            const uint32_t strides[1] = {ys};
+            st = launch_gemv_mfma_planes_multi(s, ctx, 1, &v, xp, yv, strides, y_dtype, mm, xs);
+        } else if (!generic && gemv_fast_eligible(v, x_dtype, mm > 8 ? 8 : mm, xs) && (uintptr_t)xp % 16 == 0) {
+            // the dot-product kernels take eight rows a launch
+            st = MI355Q_OK;
+            for (uint32_t r0 = 0; r0 < mm && st == MI355Q_OK; r0 += 8)
+                st = launch_gemv_fast(s, ctx, v, (const char*)xp + (size_t)r0 * xs * xsz, x_dtype,
+                                      (char*)yp + (size_t)r0 * ys * ysz, y_dtype, mm - r0 < 8 ? mm - r0 : 8, xs, ys, nullptr,
+                                      nullptr, HeadKeys{});
         } else if (!generic && gemv_staf_eligible(v, x_dtype, mm, xs) && (uintptr_t)xp % 16 == 0) {
             st = launch_gemv_staf(s, ctx, v, xp, yp, y_dtype, mm, xs, ys);
         } else {
@@ -110,10 +120,15 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
         return launch_qgemm_mfma(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys, probe);
     }
     // the decode kernels take up to 8 rows per launch on the planes, 16 on TILE16 records
-    const uint32_t small_rows = v.layout == MI355Q_LAYOUT_TILE16 ? 16u : 8u;
+    const uint32_t small_rows = small_batch_rows(v, x_dtype, xs);
     const bool small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) || m <= small_rows || !mfma_ok;
     if (small) return run_small_m(ctx, s, w, x, x_dtype, y, y_dtype, m, xs, ys, flags);
     return launch_qgemm_mfma(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys, probe);
+}
+
+uint32_t small_batch_rows(const WView& w, int x_dtype, uint32_t x_stride) {
+    (void)x_dtype; (void)x_stride;
+    return w.layout == MI355Q_LAYOUT_TILE16 ? 16 : 8;
 }
 
 bool gemm_two_step_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
@@ -161,6 +176,7 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
     bool fused = m <= 8 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
     bool tiled = m <= 16 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
     bool in_place = m <= 8 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
+    bool on_planes = m >= kMfmaPlanesMinRows && m <= 8 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
     WView views[3];
     uint32_t strides[3];
     for (uint32_t i = 0; i < count; i++) {
@@ -173,7 +189,12 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
         tiled = tiled && gemv_tile16_eligible(views[i], x_dtype, m, xs) && gemv_tile16_k_parts(ctx, views[i], m) == 1 &&
                 views[i].sb_dtype == views[0].sb_dtype;
         in_place = in_place && gemv_staf_eligible(views[i], x_dtype, m, xs);
+        on_planes = on_planes && gemv_mfma_planes_eligible(views[i], x_dtype, m, xs) &&
+                    gemv_mfma_planes_k_parts(ctx, views[i], m) == 1 && views[i].sb_dtype == views[0].sb_dtype &&
+                    views[i].code_stride == views[0].code_stride && views[i].group == views[0].group;
     }
+    if (on_planes && (uintptr_t)x % 16 == 0)
+        return launch_gemv_mfma_planes_multi(s, ctx, count, views, x, ys, strides, y_dtype, m, xs);
     if (fused && (uintptr_t)x % 16 == 0)
         return launch_gemv_fast_multi(s, ctx, count, views, x, x_dtype, ys, strides, y_dtype, m, xs, nullptr, nullptr, HeadKeys{});
     if (tiled && (uintptr_t)x % 16 == 0)

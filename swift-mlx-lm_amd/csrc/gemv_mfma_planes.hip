@@ -1,0 +1,430 @@
+// Small-batch projection on the matrix cores straight from the split planes (4-bit codes, groups of 64 or
+// 128), 2 <= M <= 8 activation rows per launch: the layout that serves M = 1 best also serves a batch.
+//
+// Stands in for gemv_q4_g{64,128} widened to the sequence signature and, at small sequence lengths, for gemm_q4_g64
+// (Sources/MetalCompiler/Generator/MetalSourceGenerator+Quantized.swift:496-575 and :22-156):
+//   y[m, n] = sum_g sum_{k in g} (s[n,g] * q[n,k] + z[n,g]) * x[m,k],  fp32 accumulation.
+//
+// A wavefront owns 16 consecutive weight rows and a share of K, walked in blocks of 128 codes.  One load instruction
+// takes 64 contiguous bytes of each of its 16 rows (four consecutive lanes per row); a cross-lane read per word then
+// gives lane (n = lane % 16, kq = lane / 16) the 32 codes at offset 32 kq of the block of row n, the order the matrix
+// core wants.  Four v_mfma_f32_16x16x32_bf16 consume such a load, one per 32-bit word: a
+// word's nibbles become the bf16 pairs (c0,c4) (c1,c5) (c2,c6) (c3,c7), each 128 + q, with one and-or per pair; the
+// activations are staged once per workgroup in LDS with every run of eight in that same order
+// (x0,x4,x1,x5,x2,x6,x3,x7), so they are the A operand as they lie.
+// The matrix core sums over all four kq, which for groups of 64 are two quantisation groups (kq 0,1 and kq 2,3).  They
+// are kept apart in the M dimension, which a batch of at most eight rows leaves half empty: A rows 0..7 carry the
+// activations only where kq < 2 (zeros elsewhere), rows 8..15 only where kq >= 2.  D rows 0..7 are then the first
+// group's sums, rows 8..15 the second's, and the accumulator of lane (n, kq), which holds D rows 4 kq .. 4 kq + 3, holds
+// sums of the very group whose codes and (scale, bias) word it loaded: the affine form
+//   acc += s * D + (z - 128 s) * SX        (D = sum (128 + q) x,  SX = sum x, computed while staging)
+// is applied lane by lane, once per block, and lanes kq and kq + 2 add their halves at the end.  The KSPLIT wavefronts
+// that share a row tile add their partial tiles through LDS.  (With groups of 128 both halves belong to one group and
+// the same code runs unchanged.)
+#include "device_utils.h"
+
+namespace mi355q {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 pm_bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float pm_floatx4_t;
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 pm_bf16x2_t;
+
+__device__ __forceinline__ float pm_dot2(uint32_t a, uint32_t b, float acc) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(pm_bf16x2_t, a), __builtin_bit_cast(pm_bf16x2_t, b), acc, false);
+}
+
+constexpr int kPmMaxSegments = 3;
+
+struct PmArgs {
+    const uint32_t* rows[kPmMaxSegments];      // code words of row 0 of up to three matrices sharing x
+    void* y[kPmMaxSegments];
+    uint32_t tile_end[kPmMaxSegments];         // cumulative 16-row tile counts; unused entries repeat the last
+    uint32_t seg_rows[kPmMaxSegments];         // N_i
+    uint32_t y_stride[kPmMaxSegments];
+    const uint16_t* x;                         // bf16 [M, x_stride]
+    uint32_t k, m, x_stride;
+    uint32_t row_words;                        // 32-bit words from one row to the next (codes, then the row's sz words)
+    uint32_t sz_offset;                        // words from a row's first code word to its first (scale, bias) word
+    uint32_t blocks_per_wave;                  // blocks of 128 codes per wavefront (K split over the workgroup)
+    uint32_t passes;                           // row tiles a wavefront walks, one after the other, on one staged copy of x
+    uint32_t lds_row_bytes;                    // part_blocks * 256 + 16: staged activation row pitch
+    uint32_t y_dtype, sb_dtype;
+    uint32_t parts;                            // K parts, each with workgroups of its own that stage only their columns
+    uint32_t part_blocks;                      // blocks per part
+    float* partial;                            // K parts only: fp32 partial results [part][M][N] (one matrix)
+};
+
+// GROUP: 64 or 128.  A workgroup of KSPLIT * TPW wavefronts covers TPW consecutive row tiles, each split over KSPLIT
+// wavefronts along K; all of them share one staged copy of the activations.
+template <int GROUP, int KSPLIT, int TPW, bool SBBF16>
+__global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmArgs a) {
+    constexpr int WAVES = KSPLIT * TPW;
+    constexpr int D = 4;                                    // blocks in flight per wavefront
+    constexpr int MR = 4;
+    extern __shared__ u32x4 smem_pm[];
+    char* lds = (char*)smem_pm;
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint32_t n_in = lane & 15, kq = lane >> 4;
+    const uint32_t part = blockIdx.y, wg = blockIdx.x;
+    const uint32_t b0 = part * a.part_blocks;               // first block of this workgroup's K part
+    const uint32_t kp = a.part_blocks * 128;                // activation elements staged per row
+
+    const uint32_t slice = wave % KSPLIT;
+    struct Tile {
+        const uint32_t* lane_row;  // this lane's row: first code word
+        void* y;
+        uint32_t ys, rows, n0, nb, b_first, b_last;
+        bool valid;
+    };
+    auto select_tile = [&](uint32_t pass) {
+        Tile t;
+        const uint32_t last = a.tile_end[kPmMaxSegments - 1];
+        uint32_t gt = (wg * a.passes + pass) * TPW + wave / KSPLIT;
+        t.valid = gt < last;
+        gt = t.valid ? gt : last - 1;                                     // idle wavefronts re-read the last tile
+        const bool in1 = gt >= a.tile_end[0], in2 = gt >= a.tile_end[1];
+        const uint32_t* const seg = in2 ? a.rows[2] : in1 ? a.rows[1] : a.rows[0];
+        t.y = in2 ? a.y[2] : in1 ? a.y[1] : a.y[0];
+        t.ys = in2 ? a.y_stride[2] : in1 ? a.y_stride[1] : a.y_stride[0];
+        t.rows = in2 ? a.seg_rows[2] : in1 ? a.seg_rows[1] : a.seg_rows[0];
+        const uint32_t lt = gt - (in2 ? a.tile_end[1] : in1 ? a.tile_end[0] : 0u);
+        t.n0 = lt * 16;
+        uint32_t row = t.n0 + (lane >> 2);                                // the row this lane LOADS (see `issue`)
+        row = row < t.rows ? row : t.rows - 1;                            // rows past the end re-read the last one
+        t.lane_row = seg + (size_t)row * a.row_words;
+        const uint32_t b_end = b0 + a.part_blocks;
+        t.b_first = b0 + slice * a.blocks_per_wave;
+        uint32_t nb = b_end > t.b_first ? b_end - t.b_first : 0;
+        nb = nb < a.blocks_per_wave ? nb : a.blocks_per_wave;
+        t.nb = t.valid ? nb : 0;
+        t.b_last = t.nb ? t.b_first + t.nb - 1 : b_end - 1;              // clamp target (always valid)
+        return t;
+    };
+    Tile tile = select_tile(0);
+
+    // ---- 1. activation loads first (vector loads return in issue order) -------------------------------------------
+    // The M x chunks 16-byte chunks of the staged columns are dealt to the threads in order, XB a thread at a time: a
+    // batch's loads all go out before its first chunk is staged, and the first batch goes out before the weight
+    // loads.  Row M of the staged copy is a row of zeros (the masked half of A).
+    const uint32_t chunks = kp / 8;                         // 16-byte chunks per staged activation row
+    constexpr uint32_t NT = WAVES * 64;
+    constexpr int XB = 8;
+    const uint32_t total = a.m * chunks;
+    const float inv_chunks = 1.0f / (float)chunks;
+    auto x_at = [&](uint32_t idx, uint32_t& m, uint32_t& c) -> bool {     // false: past the end
+        const bool has = idx < total;
+        idx = has ? idx : 0;
+        m = (uint32_t)(((float)idx + 0.5f) * inv_chunks);     // exact: idx < 2^20, chunks <= 2^13
+        c = idx - m * chunks;
+        return has;
+    };
+    auto x_load = [&](uint32_t idx) -> u32x4 {
+        uint32_t m, c;
+        x_at(idx, m, c);
+        return *((const u32x4*)(a.x + (size_t)m * a.x_stride + (size_t)b0 * 128) + c);
+    };
+    u32x4 xe[XB];
+#pragma unroll
+    for (int t = 0; t < XB; t++)
+        if ((uint32_t)t * NT < total) xe[t] = x_load(tid + (uint32_t)t * NT);     // wavefront-uniform: no load past the end
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- 2. the first D blocks of this wavefront's share of the first row tile ---------------------------------------
+    // Loads are issued with four consecutive lanes on one row (lane L: row L / 4, 16-byte piece L % 4), so that a
+    // load instruction is sixteen coalesced 64-byte requests; the matrix core wants lane kq * 16 + n to hold piece kq
+    // of row n, which `compute` arranges with one cross-lane read per 32-bit word.
+    const uint32_t piece = lane & 3u;
+    struct Rec { u32x4 w; };
+    Rec ring[D];
+    auto issue = [&](uint32_t b, Rec& r) {
+        b = b < tile.b_last ? b : tile.b_last;              // unconditional, clamped
+        r.w = __builtin_nontemporal_load((const u32x4*)(tile.lane_row + (size_t)b * 16 + piece * 4));
+    };
+    // (scale, bias) words, sixteen blocks of the wavefront's share at a time: this lane keeps those of blocks
+    // first + piece * 4 .. + 3 of the row it loads (one word per block and group of 64, so two for groups of 64)
+    constexpr int SZW = GROUP == 64 ? 2 : 1;
+    uint32_t szr[4][SZW];
+    auto issue_sz = [&](uint32_t first) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            uint32_t b = first + piece * 4 + i;
+            b = b < tile.b_last ? b : tile.b_last;
+            const uint32_t* q = tile.lane_row + a.sz_offset + (size_t)b * SZW;
+            if constexpr (SZW == 2) { const u32x2 t = *(const u32x2*)q; szr[i][0] = t.x; szr[i][1] = t.y; }
+            else szr[i][0] = *q;
+        }
+    };
+    static_for<D>([&](auto J) { issue(tile.b_first + decltype(J)::value, ring[decltype(J)::value]); });
+    issue_sz(tile.b_first);
+
+    // ---- 3. stage the activations: every run of eight as (x0,x4,x1,x5,x2,x6,x3,x7), and sum(x) per 64 and row ------
+    float* const sxs = (float*)(lds + (size_t)(a.m + 1) * a.lds_row_bytes);      // [run of 64 in part][8]
+    {
+        auto stage = [&](uint32_t idx, const u32x4& v) {
+            float p = pm_dot2(v.x, 0x3F803F80u, 0.0f);
+            p = pm_dot2(v.y, 0x3F803F80u, p);
+            p = pm_dot2(v.z, 0x3F803F80u, p);
+            p = pm_dot2(v.w, 0x3F803F80u, p);
+            p += __shfl_xor(p, 1);
+            p += __shfl_xor(p, 2);
+            p += __shfl_xor(p, 4);
+            uint32_t m, c;
+            if (x_at(idx, m, c)) {
+                u32x4 o;
+                o.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);    // (x0, x4)
+                o.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);    // (x1, x5)
+                o.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);    // (x2, x6)
+                o.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);    // (x3, x7)
+                *((u32x4*)(lds + (size_t)m * a.lds_row_bytes) + c) = o;
+                if ((c & 7u) == 0) sxs[(c >> 3) * 8 + m] = p;       // eight chunks: one run of 64
+            }
+        };
+        // whole wavefronts take part in the shuffles of every step: the walk is rounded up to whole batches
+#pragma unroll
+        for (int t = 0; t < XB; t++)
+            if ((uint32_t)t * NT < total) stage(tid + (uint32_t)t * NT, xe[t]);
+        for (uint32_t base = XB * NT; base < total; base += XB * NT) {
+#pragma unroll
+            for (int t = 0; t < XB; t++)
+                if (base + (uint32_t)t * NT < total) xe[t] = x_load(base + tid + (uint32_t)t * NT);
+#pragma unroll
+            for (int t = 0; t < XB; t++)
+                if (base + (uint32_t)t * NT < total) stage(base + tid + (uint32_t)t * NT, xe[t]);
+        }
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+        for (uint32_t c = tid; c < chunks; c += NT) *((u32x4*)(lds + (size_t)a.m * a.lds_row_bytes) + c) = zero;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+
+    // ---- 4. K loop --------------------------------------------------------------------------------------------------
+    uint32_t k_mask = 0x000F000Fu, k_magic = 0x43004300u;   // opaque: keeps (w & mask) | magic one v_and_or_b32
+    asm volatile("" : "+s"(k_mask));
+    asm volatile("" : "+v"(k_magic));
+    const pm_floatx4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+    float acc[MR];
+#pragma unroll
+    for (int r = 0; r < MR; r++) acc[r] = 0.f;
+
+    // A operand: lane (i = lane % 16, kq) stands for A row i.  Rows 0..7 are activation rows 0..7 where kq < 2, rows
+    // 8..15 are the same activation rows where kq >= 2; elsewhere the row of zeros.  Rows past M read row M-1 (their
+    // results are never stored).
+    const uint32_t xr = (n_in & 7u) < a.m ? (n_in & 7u) : a.m - 1;
+    const bool live = (n_in >> 3) == (kq >> 1);
+    const char* const a_lane = lds + (size_t)(live ? xr : a.m) * a.lds_row_bytes + kq * 64;
+
+    auto unpack = [&](uint32_t w) -> pm_bf16x8_t {
+        u32x4 p;
+        p.x = (w & k_mask) | k_magic;
+        p.y = ((w >> 4) & k_mask) | k_magic;
+        p.z = ((w >> 8) & k_mask) | k_magic;
+        p.w = ((w >> 12) & k_mask) | k_magic;
+        return __builtin_bit_cast(pm_bf16x8_t, p);
+    };
+    // this lane's D rows 4 kq .. 4 kq + 3 are activation rows 4 (kq & 1) .. + 3
+    const uint32_t sx_lane = (kq >> 1) * 8 + 4 * (kq & 1);
+    const int from_lane = (int)((4u * n_in + kq) * 4u);     // byte address of the lane that loaded (row n, piece kq)
+    auto compute = [&](uint32_t b, const Rec& r, const uint32_t (&sz_pair)[SZW], uint32_t sz_piece) {
+        const uint32_t bl = b - b0;                          // block inside the staged columns
+        const char* ab = a_lane + (size_t)bl * 256;          // 128 codes = 256 bytes of activations
+        // every LDS operation of the block goes out first: the cross-lane reads, the A operands, sum(x) over this lane
+        // half's run of 64 (runs 2 bl and 2 bl + 1 of the part): a group of 64, or half of a group of 128 whose other
+        // half the other lanes add
+        const uint32_t w0 = (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane, (int)r.w.x);
+        const uint32_t w1 = (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane, (int)r.w.y);
+        const uint32_t w2 = (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane, (int)r.w.z);
+        const uint32_t w3 = (uint32_t)__builtin_amdgcn_ds_bpermute(from_lane, (int)r.w.w);
+        // the block's (scale, bias) words sit with the lane that loaded piece `sz_piece` of this row
+        const int sz_from = (int)((4u * n_in + sz_piece) * 4u);
+        uint32_t szw = (uint32_t)__builtin_amdgcn_ds_bpermute(sz_from, (int)sz_pair[0]);
+        if constexpr (SZW == 2) {
+            const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute(sz_from, (int)sz_pair[1]);
+            szw = kq >> 1 ? hi : szw;
+        }
+        const pm_bf16x8_t a0 = *(const pm_bf16x8_t*)(ab), a1 = *(const pm_bf16x8_t*)(ab + 16);
+        const pm_bf16x8_t a2 = *(const pm_bf16x8_t*)(ab + 32), a3 = *(const pm_bf16x8_t*)(ab + 48);
+        const pm_floatx4_t sx = *(const pm_floatx4_t*)(sxs + (size_t)bl * 16 + sx_lane);
+        __builtin_amdgcn_sched_barrier(0);
+        pm_floatx4_t d = zero4;
+        d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, unpack(w0), d, 0, 0, 0);
+        d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, unpack(w1), d, 0, 0, 0);
+        d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2, unpack(w2), d, 0, 0, 0);
+        d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a3, unpack(w3), d, 0, 0, 0);
+        float s, z;
+        if constexpr (SBBF16) { s = __uint_as_float(szw << 16); z = __uint_as_float(szw & 0xFFFF0000u); }
+        else { s = f16_to_f32((uint16_t)(szw & 0xFFFFu)); z = f16_to_f32((uint16_t)(szw >> 16)); }
+        const float zc = z - 128.0f * s;
+#pragma unroll
+        for (int q = 0; q < MR; q++) acc[q] += s * d[q] + zc * sx[q];
+    };
+
+    const uint32_t rounds = (a.blocks_per_wave + D - 1) / D;              // same for every wavefront
+    // Partial tiles of the WAVES wavefronts, [WAVES][MR][64]: a single pass writes them over the staged activations
+    // once every wavefront is done reading those; several passes keep them behind the activations and their sums.
+    const bool red_over_x = a.passes == 1;
+    float* const red = (float*)(red_over_x ? lds : lds + (size_t)(a.m + 1) * a.lds_row_bytes + kp / 2);
+    for (uint32_t pass = 0; pass < a.passes; pass++) {
+        if (pass) {                                            // the first tile's loads were issued before staging
+            tile = select_tile(pass);
+            static_for<D>([&](auto J) { issue(tile.b_first + decltype(J)::value, ring[decltype(J)::value]); });
+            issue_sz(tile.b_first);
+        }
+        for (uint32_t it = 0; it < rounds; it++) {
+            if (it && (it & 3u) == 0) issue_sz(tile.b_first + it * D);       // the next sixteen blocks' words
+            static_for<D>([&](auto J) {
+                constexpr int j = decltype(J)::value;
+                const uint32_t idx = it * D + j;
+                if (idx < tile.nb) compute(tile.b_first + idx, ring[j], szr[j], it & 3u);
+                issue(tile.b_first + idx + D, ring[j]);
+            });
+        }
+
+        // ---- 5. add the partial tiles of the wavefronts that share a row tile, store ---------------------------------
+        if (red_over_x) __syncthreads();
+#pragma unroll
+        for (int r = 0; r < MR; r++) { red[(wave * MR + r) * 64 + lane] = acc[r]; acc[r] = 0.f; }
+        __syncthreads();
+        if (slice == 0 && tile.valid && kq < 2) {           // the first wavefront of each tile adds and stores
+            const uint32_t row = tile.n0 + n_in;
+#pragma unroll
+            for (int r = 0; r < MR; r++) {
+                float v = 0.f;
+                for (uint32_t w2 = 0; w2 < (uint32_t)KSPLIT; w2++)       // both halves of K of every wavefront's block
+                    v += red[((wave + w2) * MR + r) * 64 + lane] + red[((wave + w2) * MR + r) * 64 + lane + 32];
+                const uint32_t m = 4 * kq + r;
+                if (m < a.m && row < tile.rows) {
+                    if (a.parts > 1) {                       // one matrix: the reduction launch converts and stores
+                        a.partial[((size_t)part * a.m + m) * tile.rows + row] = v;
+                        continue;
+                    }
+                    const size_t o = (size_t)m * tile.ys + row;
+                    if (a.y_dtype == MI355Q_F32) ((float*)tile.y)[o] = v;
+                    else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)tile.y)[o] = f32_to_bf16_rne(v);
+                    else ((uint16_t*)tile.y)[o] = f32_to_f16_rne(v);
+                }
+            }
+        }
+        if (pass + 1 < a.passes) __syncthreads();           // the partial tiles are read before the next pass overwrites them
+    }
+}
+
+// Sum of the K parts, in part order, then the conversion the single-launch form does in its epilogue.
+__global__ __launch_bounds__(256) void pm_sum_parts_kernel(const float* __restrict__ partial, uint32_t parts, uint32_t m,
+                                                           uint32_t n, void* __restrict__ y, uint32_t y_stride,
+                                                           uint32_t y_dtype) {
+    const uint32_t row = blockIdx.y;
+    for (uint32_t col = blockIdx.x * 256 + threadIdx.x; col < n; col += gridDim.x * 256) {
+        float v = 0.f;
+        for (uint32_t p = 0; p < parts; p++) v += partial[((size_t)p * m + row) * n + col];
+        const size_t o = (size_t)row * y_stride + col;
+        if (y_dtype == MI355Q_F32) ((float*)y)[o] = v;
+        else if (y_dtype == MI355Q_BF16) ((uint16_t*)y)[o] = f32_to_bf16_rne(v);
+        else ((uint16_t*)y)[o] = f32_to_f16_rne(v);
+    }
+}
+
+namespace {
+
+template <int GROUP, int KSPLIT, int TPW>
+mi355q_status launch_pm(hipStream_t s, const PmArgs& a, uint32_t grid, size_t lds) {
+    auto kern = a.sb_dtype == MI355Q_BF16 ? gemv_mfma_planes_kernel<GROUP, KSPLIT, TPW, true>
+                                          : gemv_mfma_planes_kernel<GROUP, KSPLIT, TPW, false>;
+    if (lds > 64 * 1024)
+        MI355Q_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    kern<<<dim3(grid, a.parts), dim3(KSPLIT * TPW * 64), lds, s>>>(a);
+    MI355Q_HIP(hipGetLastError());
+    return MI355Q_OK;
+}
+
+template <int GROUP>
+mi355q_status launch_pm_shape(hipStream_t s, const PmArgs& a, const Tile16LaunchShape& g) {
+    const uint32_t ks = g.ksplit, tpw = g.tiles_per_wg;
+    if (ks == 4 && tpw == 1) return launch_pm<GROUP, 4, 1>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 4 && tpw == 2) return launch_pm<GROUP, 4, 2>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 4 && tpw == 3) return launch_pm<GROUP, 4, 3>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 4 && tpw == 4) return launch_pm<GROUP, 4, 4>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 2 && tpw == 5) return launch_pm<GROUP, 2, 5>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 2 && tpw == 6) return launch_pm<GROUP, 2, 6>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 2 && tpw == 7) return launch_pm<GROUP, 2, 7>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 2 && tpw == 8) return launch_pm<GROUP, 2, 8>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 8 && tpw == 1) return launch_pm<GROUP, 8, 1>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 8 && tpw == 2) return launch_pm<GROUP, 8, 2>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 16 && tpw == 1) return launch_pm<GROUP, 16, 1>(s, a, g.wgs_per_part, g.lds_bytes);
+    return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no matrix-core planes variant for K-split %u x %u tiles per workgroup", ks, tpw);
+}
+
+}  // namespace
+
+// The workgroups are shaped like those of the TILE16 kernel (16-row tiles walked in blocks of 128 codes, the same split
+// of K over wavefronts, tiles per workgroup, passes and K parts), for one staged row more: the row of zeros.  That
+// kernel's LDS sizes bound this one's ((M + 1) rows and K / 2 bytes of sums against (M + 1) rows and K bytes).
+bool gemv_mfma_planes_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
+    if (w.layout != MI355Q_LAYOUT_PLANES || !w.sz || x_dtype != MI355Q_BF16) return false;
+    if (m < 2 || m > 8) return false;
+    if (w.bits != 4 || (w.group != 64 && w.group != 128) || w.k % 128) return false;
+    if (x_stride % 8) return false;                                       // 128-bit activation loads
+    // a row is one stream: its sz words follow its code words at the same pitch; code words 16-byte aligned
+    if (w.sz_stride != w.code_stride || w.code_stride % 4 || (uintptr_t)w.codes % 16) return false;
+    if (w.sz < w.codes || (size_t)(w.sz - w.codes) >= w.code_stride || (w.sz - w.codes) % 2) return false;
+    return gemv_tile16_parts_for(w.k, m + 1, (w.n + 15) / 16, 256) != 0;
+}
+
+uint32_t gemv_mfma_planes_k_parts(const mi355q_context* ctx, const WView& w, uint32_t m) {
+    return gemv_tile16_parts_for(w.k, m + 1, (w.n + 15) / 16, (uint32_t)ctx->props.multiProcessorCount);
+}
+
+Tile16LaunchShape gemv_mfma_planes_shape(const mi355q_context* ctx, uint32_t n_row_tiles, uint32_t k_total, uint32_t m) {
+    return gemv_tile16_shape(ctx, n_row_tiles, k_total, m + 1);
+}
+
+mi355q_status launch_gemv_mfma_planes_multi(hipStream_t s, mi355q_context* ctx, uint32_t count, const WView* w,
+                                            const void* x, void* const* y, const uint32_t* y_strides, int y_dtype,
+                                            uint32_t m, uint32_t x_stride) {
+    if (count < 1 || count > (uint32_t)kPmMaxSegments)
+        return fail(MI355Q_ERR_INVALID_ARGUMENT, "1..%d weights per fused launch", kPmMaxSegments);
+    if ((uintptr_t)x % 16) return fail(MI355Q_ERR_INVALID_ARGUMENT, "activation pointer must be 16-byte aligned");
+    PmArgs a{};
+    uint32_t tiles = 0;
+    for (uint32_t i = 0; i < (uint32_t)kPmMaxSegments; i++) {
+        const uint32_t j = i < count ? i : count - 1;
+        if (i < count) tiles += (w[i].n + 15) / 16;
+        a.rows[i] = w[j].codes;
+        a.y[i] = y[j];
+        a.y_stride[i] = y_strides[j];
+        a.seg_rows[i] = w[j].n;
+        a.tile_end[i] = tiles;
+        if (w[j].code_stride != w[0].code_stride || (w[j].sz - w[j].codes) != (w[0].sz - w[0].codes) ||
+            w[j].k != w[0].k || w[j].group != w[0].group || w[j].sb_dtype != w[0].sb_dtype)
+            return fail(MI355Q_ERR_SHAPE, "fused projections must share K, group size, row pitch and scale type");
+    }
+    const Tile16LaunchShape g = gemv_mfma_planes_shape(ctx, tiles, w[0].k, m);
+    a.x = (const uint16_t*)x;
+    a.k = w[0].k; a.m = m; a.x_stride = x_stride;
+    a.row_words = w[0].code_stride;
+    a.sz_offset = (uint32_t)(w[0].sz - w[0].codes);
+    a.parts = g.parts;
+    a.part_blocks = w[0].k / 128 / g.parts;
+    a.blocks_per_wave = g.blocks_per_wave;
+    a.passes = g.passes;
+    a.lds_row_bytes = a.part_blocks * 256 + 16;
+    if (g.parts > 1) {
+        if (count != 1)
+            return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "rows of %u codes at M = %u are split over K parts: one matrix per launch",
+                        w[0].k, m);
+        if (mi355q_status st = ensure_workspace(ctx, (size_t)g.parts * m * w[0].n * sizeof(float))) return st;
+        a.partial = (float*)ctx->workspace;
+    }
+    a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = w[0].sb_dtype;
+    const mi355q_status st = w[0].group == 64 ? launch_pm_shape<64>(s, a, g) : launch_pm_shape<128>(s, a, g);
+    if (st != MI355Q_OK || g.parts == 1) return st;
+    uint32_t sum_wgs = (w[0].n + 255) / 256;
+    if (sum_wgs > 65535u) sum_wgs = 65535u;
+    pm_sum_parts_kernel<<<dim3(sum_wgs, m), dim3(256), 0, s>>>(a.partial, g.parts, m, w[0].n, y[0], y_strides[0],
+                                                                       (uint32_t)y_dtype);
+    MI355Q_HIP(hipGetLastError());
+    return MI355Q_OK;
+}
+
+}  // namespace mi355q

@@ -388,6 +388,10 @@ bool gemv_tile16_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_st
     return t16_parts(w.k, m, (w.n + 15) / 16, 256) != 0;              // staged activations and their group sums fit in LDS
 }
 
+uint32_t gemv_tile16_parts_for(uint32_t k, uint32_t m, uint32_t n_row_tiles, uint32_t cus) {
+    return t16_parts(k, m, n_row_tiles, cus);
+}
+
 uint32_t gemv_tile16_k_parts(const mi355q_context* ctx, const WView& w, uint32_t m) {
     return t16_parts(w.k, m, (w.n + 15) / 16, (uint32_t)ctx->props.multiProcessorCount);
 }

@@ -62,6 +62,16 @@ void plan_small_m(const mi355q_weight* w, uint32_t m, int x_dtype, uint32_t x_st
         s->block[0] = g.block;
         s->lds_bytes = g.lds_bytes;
         s->rows_per_workgroup = 16;
+    } else if (!forced && m >= kMfmaPlanesMinRows && gemv_mfma_planes_eligible(v, x_dtype, m > 8 ? 8 : m, x_stride)) {
+        const Tile16LaunchShape g = gemv_mfma_planes_shape(w->ctx, (uint32_t)((w->n + 15) / 16), (uint32_t)w->k,
+                                                           m > 8 ? 8 : m);
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_mfma_planes_q%u_g%u", (unsigned)w->fmt.bits,
+                      w->fmt.group_size);
+        s->grid[0] = g.wgs_per_part;
+        s->grid[1] = g.parts;
+        s->block[0] = g.block;
+        s->lds_bytes = g.lds_bytes;
+        s->rows_per_workgroup = 16 * g.tiles_per_wg * g.passes;
     } else if (!forced && gemv_fast_eligible(v, x_dtype, m > 8 ? 8 : m, x_stride)) {
         const GemvLaunchShape g = gemv_fast_shape(w->ctx, v, m > 8 ? 8 : m, x_dtype);
         std::snprintf(s->device_kernel, sizeof s->device_kernel, "%s_q%u_g%u",
@@ -174,7 +184,7 @@ mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w, uint32_t maximum
     }
 
     const uint32_t m = maximum_sequence_length;
-    const uint32_t small_rows = v.layout == MI355Q_LAYOUT_TILE16 ? 16u : 8u;      // rows the decode kernels take per launch
+    const uint32_t small_rows = small_batch_rows(v, x_dtype, input_row_stride);   // rows the decode kernels take per launch
     const bool want_small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) || m <= small_rows;
     const bool mfma_ok = gemm_mfma_eligible(v, x_dtype, m, input_row_stride);
     if (gemm_two_step_chosen(v, x_dtype, m, input_row_stride, flags)) {
