@@ -103,14 +103,14 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
     const WView v = w->view();
     if (flags & MI355Q_FLAG_FORCE_TWO_STEP) {
         if (!gemm_two_step_eligible(v, x_dtype, m, xs) || (uintptr_t)x % 16)
-            return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the two-dispatch route takes bf16 activations, 16-byte aligned, with K and the row stride multiples of 8");
-        return launch_qgemm_two_step(s, ctx, v, x, y, y_dtype, m, xs, ys);
+            return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the two-dispatch route takes 16-byte aligned activations, K and the row stride multiples of 8");
+        return launch_qgemm_two_step(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
     }
     // dequantise once, then the dense library GEMM: long prompts, and every format or layout the fused kernel does
     // not read.  When the library has no algorithm for the problem the routes below serve it.
     if (gemm_two_step_chosen(v, x_dtype, m, xs, flags) && (uintptr_t)x % 16 == 0 &&
-        dense_library_serves(ctx, m, (uint32_t)v.n, (uint32_t)v.k, xs, ys, y_dtype))
-        return launch_qgemm_two_step(s, ctx, v, x, y, y_dtype, m, xs, ys);
+        dense_library_serves(ctx, x_dtype, m, (uint32_t)v.n, (uint32_t)v.k, xs, ys, y_dtype))
+        return launch_qgemm_two_step(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
     const bool mfma_ok = gemm_mfma_eligible(v, x_dtype, m, xs);
     // the clock probe cell lives behind the argmax cells of the context's scratch
     unsigned long long* const probe = (flags & MI355Q_FLAG_PROBE_CLOCK) ? ctx->argmax_scratch + 16 : nullptr;
@@ -132,8 +132,9 @@ uint32_t small_batch_rows(const WView& w, int x_dtype, uint32_t x_stride) {
 }
 
 bool gemm_two_step_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
-    return x_dtype == MI355Q_BF16 && m >= 1 && w.k % 8 == 0 && x_stride % 8 == 0 &&
-           (uint64_t)w.n * w.k * 2 <= ((uint64_t)8 << 30);       // the bf16 copy lives in the context's scratch
+    (void)x_dtype;                                               // the dense copy takes the activations' type
+    return m >= 1 && w.k % 8 == 0 && x_stride % 8 == 0 &&
+           (uint64_t)w.n * w.k * 4 <= ((uint64_t)16 << 30);      // the dense copy lives in the context's scratch
 }
 
 bool gemm_two_step_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride, uint32_t flags) {
@@ -144,15 +145,19 @@ bool gemm_two_step_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_st
     return m >= (w.k > w.n ? kTwoStepMinRowsLongK : kTwoStepMinRowsBesideFused);
 }
 
-// The whole matrix as bf16 at the head of the context's scratch, the library's workspace behind it.
-mi355q_status launch_qgemm_two_step(hipStream_t s, mi355q_context* ctx, const WView& w, const void* x, void* y,
-                                    int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride) {
-    const size_t dense = (((size_t)w.n * w.k * 2) + 255) & ~(size_t)255;
+// The whole matrix in the activations' type at the head of the context's scratch, the library's workspace behind it.
+mi355q_status launch_qgemm_two_step(hipStream_t s, mi355q_context* ctx, const WView& w, const void* x, int x_dtype,
+                                    void* y, int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride) {
+    const size_t esz = x_dtype == MI355Q_F32 ? 4 : 2;
+    const size_t dense = (((size_t)w.n * w.k * esz) + 255) & ~(size_t)255;
     if (mi355q_status st = ensure_workspace(ctx, dense + kDenseLibraryWorkspace)) return st;
-    uint16_t* const w_bf16 = (uint16_t*)ctx->workspace;
-    if (mi355q_status st = launch_dequant_bf16(s, w, w_bf16)) return st;
-    return dense_library_gemm(s, ctx, (const uint16_t*)x, w_bf16, y, y_dtype, m, (uint32_t)w.n, (uint32_t)w.k, x_stride,
-                              y_stride, (char*)ctx->workspace + dense);
+    void* const w_dense = ctx->workspace;
+    const mi355q_status st = x_dtype == MI355Q_BF16 ? launch_dequant_bf16(s, w, (uint16_t*)w_dense)
+                           : x_dtype == MI355Q_F16 ? launch_dequant_f16(s, w, (uint16_t*)w_dense)
+                                                   : launch_dequant_f32(s, w, (float*)w_dense);
+    if (st != MI355Q_OK) return st;
+    return dense_library_gemm(s, ctx, x_dtype, x, w_dense, y, y_dtype, m, (uint32_t)w.n, (uint32_t)w.k, x_stride, y_stride,
+                              (char*)ctx->workspace + dense);
 }
 
 // Two or three projections that read the same activations (q+k+v, gate+up).  For M <= 8 on the
@@ -299,10 +304,10 @@ mi355q_status mi355q_gemm_bf16(mi355q_context* ctx, void* stream, const void* a_
     // library's own matrix-core kernel
     if (a_dtype == MI355Q_BF16 && m >= kDenseLibraryMinRows && k % 8 == 0 && a_row_stride % 8 == 0 &&
         (uintptr_t)a_dev % 16 == 0 && (uintptr_t)b_bf16_dev % 16 == 0 &&
-        dense_library_serves(ctx, m, n, k, a_row_stride, c_row_stride, c_dtype)) {
+        dense_library_serves(ctx, MI355Q_BF16, m, n, k, a_row_stride, c_row_stride, c_dtype)) {
         if (mi355q_status st = ensure_workspace(ctx, kDenseLibraryWorkspace)) return st;
-        return dense_library_gemm((hipStream_t)stream, ctx, (const uint16_t*)a_dev, (const uint16_t*)b_bf16_dev, c_dev,
-                                  c_dtype, m, n, k, a_row_stride, c_row_stride, ctx->workspace);
+        return dense_library_gemm((hipStream_t)stream, ctx, MI355Q_BF16, a_dev, b_bf16_dev, c_dev, c_dtype, m, n, k,
+                                  a_row_stride, c_row_stride, ctx->workspace);
     }
     return launch_gemm_bf16_mfma((hipStream_t)stream, ctx, a_dev, a_dtype, (const uint16_t*)b_bf16_dev, c_dev,
                                  c_dtype, m, n, k, a_row_stride, c_row_stride);

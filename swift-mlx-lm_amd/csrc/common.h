@@ -123,6 +123,7 @@ namespace mi355q {
 mi355q_status launch_unpack_codes(hipStream_t s, const WView& w, uint8_t* out);
 mi355q_status launch_dequant_bf16(hipStream_t s, const WView& w, uint16_t* out);
 mi355q_status launch_dequant_f32(hipStream_t s, const WView& w, float* out);
+mi355q_status launch_dequant_f16(hipStream_t s, const WView& w, uint16_t* out);
 mi355q_status launch_gemv_generic(hipStream_t s, const WView& w, const void* x, int x_dtype,
                                   void* y, int y_dtype, uint32_t m, uint32_t x_stride,
                                   uint32_t y_stride);
@@ -235,11 +236,12 @@ mi355q_status launch_qgemm_mfma(hipStream_t s, mi355q_context* ctx, const WView&
 // Two-dispatch prefill route: dequantise the whole matrix to bf16 in the context's scratch, then the platform's
 // dense GEMM.  `dense_library_serves` answers whether the library can be opened and has an algorithm for the problem.
 constexpr size_t kDenseLibraryWorkspace = (size_t)64 << 20;
-bool dense_library_serves(mi355q_context* ctx, uint32_t m, uint32_t n, uint32_t k, uint32_t x_stride, uint32_t y_stride,
-                          int y_dtype);
-mi355q_status dense_library_gemm(hipStream_t s, mi355q_context* ctx, const uint16_t* x, const uint16_t* w_bf16, void* y,
-                                 int y_dtype, uint32_t m, uint32_t n, uint32_t k, uint32_t x_stride, uint32_t y_stride,
-                                 void* workspace);
+// Both operands in `ab_dtype` (bf16, f16 or fp32), fp32 accumulation, output in y_dtype.
+bool dense_library_serves(mi355q_context* ctx, int ab_dtype, uint32_t m, uint32_t n, uint32_t k, uint32_t x_stride,
+                          uint32_t y_stride, int y_dtype);
+mi355q_status dense_library_gemm(hipStream_t s, mi355q_context* ctx, int ab_dtype, const void* x, const void* w_dense,
+                                 void* y, int y_dtype, uint32_t m, uint32_t n, uint32_t k, uint32_t x_stride,
+                                 uint32_t y_stride, void* workspace);
 void dense_library_release(mi355q_context* ctx);
 // Rows from which the two-dispatch route is taken.  Beside the fused matrix-core kernel (measured, q4 g64, N(0,1)
 // activations, fused against two-dispatch): 4096 -> 14336 at M = 1024 131 against 140 us, M = 2048 282 against 244 us,
@@ -251,8 +253,8 @@ constexpr uint32_t kTwoStepMinRowsBesideFused = 2048, kTwoStepMinRowsLongK = 409
 constexpr uint32_t kDenseLibraryMinRows = 128;
 bool gemm_two_step_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
 bool gemm_two_step_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride, uint32_t flags);
-mi355q_status launch_qgemm_two_step(hipStream_t s, mi355q_context* ctx, const WView& w, const void* x, void* y,
-                                    int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride);
+mi355q_status launch_qgemm_two_step(hipStream_t s, mi355q_context* ctx, const WView& w, const void* x, int x_dtype,
+                                    void* y, int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride);
 mi355q_status launch_gemm_bf16_mfma(hipStream_t s, mi355q_context* ctx, const void* a,
                                     int a_dtype, const uint16_t* b, void* c, int c_dtype,
                                     uint32_t m, uint32_t n, uint32_t k, uint32_t a_stride,

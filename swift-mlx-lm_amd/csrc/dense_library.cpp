@@ -1,4 +1,4 @@
-// Dense bf16 GEMM of the two-dispatch prefill route through hipBLASLt.
+// Dense GEMM (bf16, f16 or fp32 operands) of the two-dispatch prefill route through hipBLASLt.
 //
 // The reference's second prefill route is  dequant_q{b}_g{g}_bf16  into a scratch matrix, then the platform's own
 // matmul2d primitive on the dense operands (Sources/MetalCompiler/Generator/MetalSourceGenerator+Linear.swift:18-81,
@@ -81,7 +81,7 @@ constexpr int kCandidates = 8;
 // One problem the context has met: its descriptors and the algorithm the library's heuristic ranks first.
 struct Problem {
     uint32_t m, n, k, xs, ys;
-    int y_dtype;
+    int ab_dtype, y_dtype;
     bool usable;
     hipblasLtMatmulDesc_t desc;
     hipblasLtMatrixLayout_t a, b, c;
@@ -114,20 +114,22 @@ DenseLibrary* library_of(mi355q_context* ctx) {
     return ctx->dense_library;
 }
 
-Problem* find_problem(DenseLibrary* lib, uint32_t m, uint32_t n, uint32_t k, uint32_t xs, uint32_t ys, int y_dtype) {
+Problem* find_problem(DenseLibrary* lib, int ab_dtype, uint32_t m, uint32_t n, uint32_t k, uint32_t xs, uint32_t ys,
+                      int y_dtype) {
     for (Problem& p : lib->problems)
-        if (p.m == m && p.n == n && p.k == k && p.xs == xs && p.ys == ys && p.y_dtype == y_dtype) return &p;
+        if (p.m == m && p.n == n && p.k == k && p.xs == xs && p.ys == ys && p.ab_dtype == ab_dtype && p.y_dtype == y_dtype)
+            return &p;
     const Api* a = lib->api;
     Problem p{};
-    p.m = m; p.n = n; p.k = k; p.xs = xs; p.ys = ys; p.y_dtype = y_dtype;
+    p.m = m; p.n = n; p.k = k; p.xs = xs; p.ys = ys; p.ab_dtype = ab_dtype; p.y_dtype = y_dtype;
     const hipblasOperation_t op_t = HIPBLAS_OP_T, op_n = HIPBLAS_OP_N;
     hipblasLtMatmulPreference_t pref = nullptr;
     const uint64_t most = kDenseLibraryWorkspace;
     bool ok = a->desc_create(&p.desc, HIPBLAS_COMPUTE_32F, HIP_R_32F) == HIPBLAS_STATUS_SUCCESS &&
               a->desc_set(p.desc, HIPBLASLT_MATMUL_DESC_TRANSA, &op_t, sizeof op_t) == HIPBLAS_STATUS_SUCCESS &&
               a->desc_set(p.desc, HIPBLASLT_MATMUL_DESC_TRANSB, &op_n, sizeof op_n) == HIPBLAS_STATUS_SUCCESS &&
-              a->layout_create(&p.a, HIP_R_16BF, k, n, k) == HIPBLAS_STATUS_SUCCESS &&
-              a->layout_create(&p.b, HIP_R_16BF, k, m, xs) == HIPBLAS_STATUS_SUCCESS &&
+              a->layout_create(&p.a, data_type(ab_dtype), k, n, k) == HIPBLAS_STATUS_SUCCESS &&
+              a->layout_create(&p.b, data_type(ab_dtype), k, m, xs) == HIPBLAS_STATUS_SUCCESS &&
               a->layout_create(&p.c, data_type(y_dtype), n, m, ys) == HIPBLAS_STATUS_SUCCESS &&
               a->pref_create(&pref) == HIPBLAS_STATUS_SUCCESS &&
               a->pref_set(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &most, sizeof most) == HIPBLAS_STATUS_SUCCESS;
@@ -150,19 +152,19 @@ Problem* find_problem(DenseLibrary* lib, uint32_t m, uint32_t n, uint32_t k, uin
 
 }  // namespace
 
-bool dense_library_serves(mi355q_context* ctx, uint32_t m, uint32_t n, uint32_t k, uint32_t x_stride, uint32_t y_stride,
-                          int y_dtype) {
+bool dense_library_serves(mi355q_context* ctx, int ab_dtype, uint32_t m, uint32_t n, uint32_t k, uint32_t x_stride,
+                          uint32_t y_stride, int y_dtype) {
     DenseLibrary* lib = library_of(ctx);
     if (!lib) return false;
-    return find_problem(lib, m, n, k, x_stride, y_stride, y_dtype)->usable;
+    return find_problem(lib, ab_dtype, m, n, k, x_stride, y_stride, y_dtype)->usable;
 }
 
-mi355q_status dense_library_gemm(hipStream_t s, mi355q_context* ctx, const uint16_t* x, const uint16_t* w_bf16, void* y,
-                                 int y_dtype, uint32_t m, uint32_t n, uint32_t k, uint32_t x_stride, uint32_t y_stride,
-                                 void* workspace) {
+mi355q_status dense_library_gemm(hipStream_t s, mi355q_context* ctx, int ab_dtype, const void* x, const void* w_bf16,
+                                 void* y, int y_dtype, uint32_t m, uint32_t n, uint32_t k, uint32_t x_stride,
+                                 uint32_t y_stride, void* workspace) {
     DenseLibrary* lib = library_of(ctx);
     if (!lib) return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the dense GEMM library (hipBLASLt) could not be opened");
-    Problem* p = find_problem(lib, m, n, k, x_stride, y_stride, y_dtype);
+    Problem* p = find_problem(lib, ab_dtype, m, n, k, x_stride, y_stride, y_dtype);
     if (!p->usable)
         return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the dense GEMM library has no algorithm for M=%u N=%u K=%u", m, n, k);
     const float one = 1.0f, zero = 0.0f;

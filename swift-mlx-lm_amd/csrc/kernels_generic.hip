@@ -241,9 +241,15 @@ mi355q_status launch_embedding_lookup(hipStream_t s, const WView& w, const int32
 // One workgroup per row, 256 threads striding over the row, as the reference kernel does.
 // scale*q and +zero are kept as two roundings so the result is bit-identical to an unfused
 // host evaluation (the order CPUWeightStore.decodeQuantized evaluates, Sources/SwiftLM/CPUWeightStore.swift:170).
-// F32: the fp32 value itself is stored; else its bf16 rounding.
-template <bool F32>
+// OUT (an mi355q_dtype): F32 stores the fp32 value itself, BF16 and F16 its rounding to nearest even.
+template <int OUT>
+__device__ __forceinline__ uint16_t dequant_round16(float v) {
+    return OUT == MI355Q_BF16 ? f32_to_bf16_rne(v) : f32_to_f16_rne(v);
+}
+
+template <int OUT>
 __global__ __launch_bounds__(256) void dequant_kernel(WView w, void* __restrict__ out) {
+    constexpr bool F32 = OUT == MI355Q_F32;
     for (uint32_t row = blockIdx.x; row < w.n; row += gridDim.x) {
         for (uint32_t c = threadIdx.x; c < w.k; c += 256) {
             float scale, zero;
@@ -251,7 +257,7 @@ __global__ __launch_bounds__(256) void dequant_kernel(WView w, void* __restrict_
             const float q = (float)load_code(w, row, c);
             const float v = __fadd_rn(__fmul_rn(scale, q), zero);
             if constexpr (F32) ((float*)out)[(size_t)row * w.k + c] = v;
-            else ((uint16_t*)out)[(size_t)row * w.k + c] = f32_to_bf16_rne(v);
+            else ((uint16_t*)out)[(size_t)row * w.k + c] = dequant_round16<OUT>(v);
         }
     }
 }
@@ -262,8 +268,9 @@ __global__ __launch_bounds__(256) void dequant_kernel(WView w, void* __restrict_
 // BITS is a template argument (constant shifts on the 64-bit field) and the grid is two-dimensional -- x over the
 // 8-code chunks of a row, y over rows -- so that no thread divides a 64-bit index: with run-time width and a flat index
 // the kernel was bound by its integer arithmetic (42 us for 4096 -> 14336, against 26 us for a plain copy of as many bytes).
-template <int BITS, bool F32>
+template <int BITS, int OUT>
 __global__ __launch_bounds__(256) void dequant_x8_kernel(WView w, void* __restrict__ out) {
+    constexpr bool F32 = OUT == MI355Q_F32;
     const uint32_t c0 = (blockIdx.x * 256 + threadIdx.x) << 3;
     if (c0 >= w.k) return;
     constexpr uint32_t mask = (1u << BITS) - 1u;
@@ -285,41 +292,43 @@ __global__ __launch_bounds__(256) void dequant_x8_kernel(WView w, void* __restri
             __builtin_nontemporal_store(hi, dst + 1);
         } else {
             u32x4 st;
-            st.x = f32_to_bf16_rne(f[0]) | ((uint32_t)f32_to_bf16_rne(f[1]) << 16);
-            st.y = f32_to_bf16_rne(f[2]) | ((uint32_t)f32_to_bf16_rne(f[3]) << 16);
-            st.z = f32_to_bf16_rne(f[4]) | ((uint32_t)f32_to_bf16_rne(f[5]) << 16);
-            st.w = f32_to_bf16_rne(f[6]) | ((uint32_t)f32_to_bf16_rne(f[7]) << 16);
+            st.x = dequant_round16<OUT>(f[0]) | ((uint32_t)dequant_round16<OUT>(f[1]) << 16);
+            st.y = dequant_round16<OUT>(f[2]) | ((uint32_t)dequant_round16<OUT>(f[3]) << 16);
+            st.z = dequant_round16<OUT>(f[4]) | ((uint32_t)dequant_round16<OUT>(f[5]) << 16);
+            st.w = dequant_round16<OUT>(f[6]) | ((uint32_t)dequant_round16<OUT>(f[7]) << 16);
             __builtin_nontemporal_store(st, (u32x4*)((uint16_t*)out + (size_t)row * w.k + c0));
         }
     }
 }
 
-template <bool F32>
+template <int OUT>
 mi355q_status launch_dequant(hipStream_t s, const WView& w, void* out) {
+    constexpr bool F32 = OUT == MI355Q_F32;
     if (w.k % 8 == 0 && (uintptr_t)out % 16 == 0 && (!F32 || w.k % 4 == 0)) {
         // two to four rows per thread, at most 65535 workgroups along y
         uint32_t gy = w.n > 4096 ? (w.n + 3) / 4 : (w.n + 1) / 2;
         if (gy > 65535u) gy = 65535u;
         const dim3 grid((w.k / 8 + 255) / 256, gy), block(256);
         switch (w.bits) {
-        case 2: dequant_x8_kernel<2, F32><<<grid, block, 0, s>>>(w, out); break;
-        case 3: dequant_x8_kernel<3, F32><<<grid, block, 0, s>>>(w, out); break;
-        case 4: dequant_x8_kernel<4, F32><<<grid, block, 0, s>>>(w, out); break;
-        case 5: dequant_x8_kernel<5, F32><<<grid, block, 0, s>>>(w, out); break;
-        case 6: dequant_x8_kernel<6, F32><<<grid, block, 0, s>>>(w, out); break;
-        case 8: dequant_x8_kernel<8, F32><<<grid, block, 0, s>>>(w, out); break;
+        case 2: dequant_x8_kernel<2, OUT><<<grid, block, 0, s>>>(w, out); break;
+        case 3: dequant_x8_kernel<3, OUT><<<grid, block, 0, s>>>(w, out); break;
+        case 4: dequant_x8_kernel<4, OUT><<<grid, block, 0, s>>>(w, out); break;
+        case 5: dequant_x8_kernel<5, OUT><<<grid, block, 0, s>>>(w, out); break;
+        case 6: dequant_x8_kernel<6, OUT><<<grid, block, 0, s>>>(w, out); break;
+        case 8: dequant_x8_kernel<8, OUT><<<grid, block, 0, s>>>(w, out); break;
         default: return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no dequantisation kernel for %u-bit codes", w.bits);
         }
     } else {
         unsigned blocks = w.n < 65535u * 16u ? w.n : 65535u * 16u;
-        dequant_kernel<F32><<<dim3(blocks), dim3(256), 0, s>>>(w, out);
+        dequant_kernel<OUT><<<dim3(blocks), dim3(256), 0, s>>>(w, out);
     }
     MI355Q_HIP(hipGetLastError());
     return MI355Q_OK;
 }
 
-mi355q_status launch_dequant_bf16(hipStream_t s, const WView& w, uint16_t* out) { return launch_dequant<false>(s, w, out); }
-mi355q_status launch_dequant_f32(hipStream_t s, const WView& w, float* out) { return launch_dequant<true>(s, w, out); }
+mi355q_status launch_dequant_bf16(hipStream_t s, const WView& w, uint16_t* out) { return launch_dequant<MI355Q_BF16>(s, w, out); }
+mi355q_status launch_dequant_f32(hipStream_t s, const WView& w, float* out) { return launch_dequant<MI355Q_F32>(s, w, out); }
+mi355q_status launch_dequant_f16(hipStream_t s, const WView& w, uint16_t* out) { return launch_dequant<MI355Q_F16>(s, w, out); }
 
 // ------------------------------------------------------------------------------ generic GEMV
 // grid (ceil(N/4), M); one wavefront per output row, lanes stride over the codes of the row.

@@ -109,6 +109,26 @@ void plan_shared_launch_shape(const mi355q_weight* const* ws, uint32_t count, ui
                               mi355q_step* s) {
     WView all = ws[0]->view();
     uint64_t total = 0;
+    // four rows and more: the matrix-core kernel over the planes takes the rows of all matrices, in 16-row tiles
+    bool on_planes = m >= kMfmaPlanesMinRows && m <= 8;
+    uint32_t tiles = 0;
+    for (uint32_t i = 0; i < count && on_planes; i++) {
+        const WView v = ws[i]->view();
+        on_planes = gemv_mfma_planes_eligible(v, x_dtype, m, x_stride) && gemv_mfma_planes_k_parts(ws[0]->ctx, v, m) == 1 &&
+                    v.sb_dtype == all.sb_dtype && v.code_stride == all.code_stride && v.group == all.group;
+        tiles += (v.n + 15) / 16;
+    }
+    if (on_planes) {
+        const Tile16LaunchShape g = gemv_mfma_planes_shape(ws[0]->ctx, tiles, all.k, m);
+        s->grid[0] = g.wgs_per_part;
+        s->grid[1] = g.parts;
+        s->block[0] = g.block;
+        s->lds_bytes = g.lds_bytes;
+        s->rows_per_workgroup = 16 * g.tiles_per_wg * g.passes;
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_mfma_planes_q%u_g%u", (unsigned)ws[0]->fmt.bits,
+                      ws[0]->fmt.group_size);
+        return;
+    }
     for (uint32_t i = 0; i < count; i++) {
         const WView v = ws[i]->view();
         if (v.layout != MI355Q_LAYOUT_PLANES || !gemv_fast_eligible(v, x_dtype, m > 8 ? 8 : m, x_stride)) return;
@@ -196,18 +216,19 @@ mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w, uint32_t maximum
         d->path = MI355Q_PATH_PREFILL_PROJECTION;
         d->input_row_stride = input_row_stride;
         d->flops = 0;
+        const char* const type_name = x_dtype == MI355Q_BF16 ? "bf16" : x_dtype == MI355Q_F16 ? "f16" : "f32";
         std::snprintf(d->kernel_name, sizeof d->kernel_name, "%s", w->fmt.dequant_to_bfloat_kernel_name);
-        std::snprintf(d->device_kernel, sizeof d->device_kernel, "dequant_q%u_g%u_bf16", (unsigned)w->fmt.bits,
-                      w->fmt.group_size);
+        std::snprintf(d->device_kernel, sizeof d->device_kernel, "dequant_q%u_g%u_%s", (unsigned)w->fmt.bits,
+                      w->fmt.group_size, type_name);
         std::snprintf(d->kernel_family, sizeof d->kernel_family, "dequantToBFloat");
         d->block[0] = 256;
         s = &out_steps[1];
         fill_common(w, m, s);
         s->path = MI355Q_PATH_PREFILL_PROJECTION;
         s->input_row_stride = input_row_stride;
-        s->weight_bytes = (uint64_t)w->n * w->k * 2;          // the dense operand it reads
+        s->weight_bytes = (uint64_t)w->n * w->k * (x_dtype == MI355Q_F32 ? 4 : 2);          // the dense operand it reads
         std::snprintf(s->kernel_name, sizeof s->kernel_name, "gemm_bf16_f32s");
-        std::snprintf(s->device_kernel, sizeof s->device_kernel, "hipblaslt_gemm_bf16");
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "hipblaslt_gemm_%s", type_name);
         std::snprintf(s->kernel_family, sizeof s->kernel_family, "libraryGEMM");
         return MI355Q_OK;
     }

@@ -403,8 +403,9 @@ def test_tile16_plan_replay_and_graph(pkg, ctx):
 
 @pytest.mark.parametrize("x_dtype_name", ["F16", "F32"])
 def test_tile16_other_activation_types_take_the_per_code_kernel_whole(pkg, ctx, x_dtype_name):
-    """The tile kernel reads bf16 activations only.  f16 and fp32 rows go to the per-code kernel, which takes all M
-    rows in one launch (no walk in steps of sixteen, eight ... one row)."""
+    """The tile kernel reads bf16 activations only.  A few f16 or fp32 rows go to the per-code kernel, which takes all
+    of them in one launch (no walk in steps of sixteen, eight ... one row); from sixteen rows the two-dispatch route
+    serves (dequantised to the activations' type, then the dense library GEMM)."""
     x_dtype = getattr(pkg, x_dtype_name)
     n, k = 96, 512
     words, s, z, wq = seeded_case(2931, n, k, 4, 64)

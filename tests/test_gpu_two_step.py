@@ -14,7 +14,7 @@ import pytest
 
 import kat
 import oracle
-from gpu_util import Case, act_rounded, assert_within_tolerance, out_from_device, seeded_case
+from gpu_util import Case, act_rounded, act_to_device_array, assert_within_tolerance, out_from_device, seeded_case
 
 pytestmark = pytest.mark.gpu
 
@@ -202,3 +202,33 @@ def test_dense_entry_point_hands_long_products_to_the_library(pkg, ctx):
     assert_within_tolerance(yd.download(np.float32, (m, n)), oracle.gemm_f64(b, x), "dense entry point")
     for buf in (bd, xd, yd):
         buf.free()
+
+
+@pytest.mark.parametrize("x_dtype_name,y_dtype_names", [("F16", ("F32", "F16")), ("F32", ("F32",))])
+def test_two_step_f16_and_f32_activations(pkg, ctx, x_dtype_name, y_dtype_names):
+    """f16 and fp32 activations (the reference's gemm_q*_g* and gemm_q*_g*_f32s signatures): the matrix is dequantised
+    to the activations' type and the library multiplies in that type with fp32 accumulation.  Unforced, every layout
+    takes the route from sixteen rows (the fused kernel reads bf16 only)."""
+    x_dtype = getattr(pkg, x_dtype_name)
+    n, k = 200, 1024
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+    words, s, z, wq = seeded_case(3600, n, k, 4, 64)
+    w_round = wq.astype(np.float16).astype(np.float32) if x_dtype == pkg.F16 else wq
+    for layout in (pkg.LAYOUT_PLANES, pkg.LAYOUT_STAF_BLOCKS):
+        w = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, layout)
+        steps = w.plan_prefill_steps(64, x_dtype=x_dtype)
+        suffix = x_dtype_name.lower()
+        assert [st.device_kernel for st in steps] == [f"dequant_q4_g64_{suffix}", f"hipblaslt_gemm_{suffix}"]
+        for m in (16, 77, 300):
+            x = act_rounded(kat.seeded_activations(3610 + m, m, k), x_dtype, pkg)
+            want = oracle.gemm_f64(w_round, x)
+            for yname in y_dtype_names:
+                y_dtype = getattr(pkg, yname)
+                say(f"two-step {x_dtype_name} -> {yname} layout {layout} M={m}")
+                xd = ctx.upload(act_to_device_array(x, x_dtype, pkg))
+                yd = ctx.alloc(m * n * (4 if y_dtype == pkg.F32 else 2))
+                ctx.fill(yd, 0x7FC00000)
+                ctx.qgemm(w, xd, x_dtype, yd, y_dtype, m); ctx.synchronize()
+                assert_within_tolerance(out_from_device(yd, y_dtype, (m, n), pkg), want, f"{x_dtype_name}->{yname} M={m}")
+                xd.free(); yd.free()
+        w.destroy()
