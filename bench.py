@@ -31,10 +31,10 @@ LAYER_SHAPES = [("q", 4096, 4096), ("k", 1024, 4096), ("v", 1024, 4096), ("o", 4
 BITS, GROUP = 4, 64
 MFMA_BF16_PEAK_TFLOPS = 2500.0    # MI355X published dense bf16 matrix-core peak
 # HBM bytes per launch from the FETCH_SIZE and WRITE_SIZE counters, each scaled by what the same counter reads for a
-# plain copy of the same size (profiles/gemv_rows_q4_g64_gate_up_hbm_traffic_pmc.md).  Measured offline with the
+# plain copy of the same size (profiles/gemv_rows_q4_g64_gate_up_pmc_and_hbm_traffic.md).  Measured offline with the
 # profiler: the figure only holds for the kernel and launch shape it was measured on, so it is keyed by both and the
 # line carries null when the library picks anything else.
-TRAFFIC_BYTES = {("gemv_rows_kernel", "gate_up", 3584, 256): None, ("gemv_rows_kernel", "gate", 1792, 256): None}
+TRAFFIC_BYTES = {("gemv_rows_q4_g64", "gate_up", 3584, 256): 66171661 + 114688, ("gemv_rows_q4_g64", "gate", 1792, 256): 33159518 + 57344}
 
 
 def log(*a):
@@ -326,7 +326,7 @@ def main():
     dom_rec = pd.step(0)[0]
     dom_kernel, dom_grid, dom_block = dom_rec.device_kernel, int(dom_rec.grid[0]), int(dom_rec.block[0])
     pd.destroy()
-    traffic = TRAFFIC_BYTES.get((dom_kernel.split("_q")[0] if False else dom_kernel, dom, dom_grid, dom_block))
+    traffic = TRAFFIC_BYTES.get((dom_kernel, dom, dom_grid, dom_block))
 
     # ---- plain copy of the gate tensor's size: the calibration launch for the HBM counters ------
     gate_bytes = weight_bytes(14336, 4096)
@@ -573,6 +573,9 @@ def main():
                             "frac": round(best["TFLOPs"] / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
                             "kernel": best["route"], "m": 2048, "shape": "4096->14336", "us": best["us"],
                             "flops": flops, "activations": "N(0,1) bf16",
+                            "gate_m4096": {"TFLOPs": sweep["gate 4096->14336 M=4096"]["TFLOPs"],
+                                           "frac": round(sweep["gate 4096->14336 M=4096"]["TFLOPs"] / MFMA_BF16_PEAK_TFLOPS, 4),
+                                           "kernel": sweep["gate 4096->14336 M=4096"]["route"]},
                             "down_14336_4096": {"TFLOPs": sweep["down 14336->4096 M=2048"]["TFLOPs"],
                                                 "frac": round(sweep["down 14336->4096 M=2048"]["TFLOPs"] / MFMA_BF16_PEAK_TFLOPS, 4),
                                                 "kernel": sweep["down 14336->4096 M=2048"]["route"]}}

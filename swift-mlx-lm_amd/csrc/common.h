@@ -244,11 +244,12 @@ mi355q_status dense_library_gemm(hipStream_t s, mi355q_context* ctx, int ab_dtyp
                                  uint32_t y_stride, void* workspace);
 void dense_library_release(mi355q_context* ctx);
 // Rows from which the two-dispatch route is taken.  Beside the fused matrix-core kernel (measured, q4 g64, N(0,1)
-// activations, fused against two-dispatch): 4096 -> 14336 at M = 1024 131 against 140 us, M = 2048 282 against 244 us,
-// M = 4096 580 against 436 us; 14336 -> 4096 at M = 2048 262 against 271 us, M = 4096 477 against 386 us.  Where only
-// the decode kernels would serve (formats and layouts the fused kernel does not read; block layout, 4096 -> 14336:
-// M = 32 in four launches of eight rows 147 us, two-dispatch 47 us) it starts at sixteen rows.
-constexpr uint32_t kTwoStepMinRowsBesideFused = 2048, kTwoStepMinRowsLongK = 4096, kTwoStepMinRowsOtherwise = 16;
+// activations, fused against two-dispatch with the library's candidates timed): 4096 -> 14336 at M = 512 90-100
+// against 93-100 us, M = 1024 139-160 against 119-130 us, M = 2048 287-312 against 206-217 us; 14336 -> 4096 at
+// M = 1024 141-150 against 162-168 us, M = 2048 260-285 against 244-256 us, M = 4096 458-520 against 338-347 us.
+// Where only the decode kernels would serve (formats and layouts the fused kernel does not read; block layout,
+// 4096 -> 14336: M = 32 in four launches of eight rows 147 us, two-dispatch 47 us) it starts at sixteen rows.
+constexpr uint32_t kTwoStepMinRowsBesideFused = 1024, kTwoStepMinRowsLongK = 2048, kTwoStepMinRowsOtherwise = 16;
 // Rows from which mi355q_gemm_bf16 hands a plain dense product to the library.
 constexpr uint32_t kDenseLibraryMinRows = 128;
 bool gemm_two_step_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);

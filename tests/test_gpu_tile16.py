@@ -320,7 +320,7 @@ def test_tile16_prefill_runs_on_the_matrix_cores(pkg, ctx):
         wp = ctx.weight_prepare_mlx(_fmt(pkg), words, s, z, pkg.BF16, pkg.LAYOUT_PLANES)
         x = act_rounded(kat.seeded_activations(2750 + i, m, k), pkg.BF16, pkg)
         say(f"tile16 prefill {k}->{n} M={m}")
-        got = _run(ctx, pkg, wt, x, pkg.F32, use_qgemm=True, flags=0 if m < 2048 else pkg.FLAG_FORCE_MFMA)
+        got = _run(ctx, pkg, wt, x, pkg.F32, use_qgemm=True, flags=0 if m < 1024 else pkg.FLAG_FORCE_MFMA)
         same = _run(ctx, pkg, wp, x, pkg.F32, use_qgemm=True, flags=pkg.FLAG_FORCE_MFMA)
         assert np.array_equal(got, same), f"{k}->{n} M={m}: records and planes disagree"
         if m * n * k <= 2 ** 28:
@@ -329,7 +329,7 @@ def test_tile16_prefill_runs_on_the_matrix_cores(pkg, ctx):
         st = wt.plan_prefill_steps(m, flags=pkg.FLAG_FORCE_MFMA)[0]
         assert st.device_kernel == "qgemm_mfma_q4_g64" and not st.used_fallback
         unforced = [s.device_kernel for s in wt.plan_prefill_steps(m)]     # long prompts: dequantise once + dense GEMM
-        assert unforced == (["dequant_q4_g64_bf16", "hipblaslt_gemm_bf16"] if m >= 2048 else ["qgemm_mfma_q4_g64"])
+        assert unforced == (["dequant_q4_g64_bf16", "hipblaslt_gemm_bf16"] if m >= 1024 else ["qgemm_mfma_q4_g64"])
         wt.destroy(); wp.destroy()
     # f16 scale words (a STAF source)
     rng = np.random.default_rng(6)

@@ -102,7 +102,7 @@ def test_two_step_seeded_ragged_shapes_and_strides(pkg, ctx, bits, group, layout
 
 def test_two_step_is_chosen_where_measured_faster_and_planned_as_two_steps(pkg, ctx):
     """Without flags: the block layout (no fused matrix-core kernel) takes the route from sixteen rows; the planes keep
-    the fused kernel up to 2047 rows (long-K shapes up to 4095).  The planner reports dequant + GEMM as two steps."""
+    the fused kernel up to 1023 rows (shapes with K > N up to 2047).  The planner reports dequant + GEMM as two steps."""
     n, k = 192, 512
     words, s, z, wq = seeded_case(3300, n, k, 4, 64)
     fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
@@ -117,14 +117,14 @@ def test_two_step_is_chosen_where_measured_faster_and_planned_as_two_steps(pkg, 
     assert not steps[0].used_fallback and not steps[1].used_fallback
     assert len(ws.plan_prefill_steps(12)) == 1 and ws.plan_prefill_steps(12)[0].used_fallback
     assert len(ws.plan_prefill_steps(64, flags=pkg.FLAG_FORCE_SMALL_M)) == 1
-    assert [st.kernel_family for st in wp.plan_prefill_steps(2047)] == ["mfmaGEMM"]
-    assert [st.kernel_family for st in wp.plan_prefill_steps(2048)] == ["dequantToBFloat", "libraryGEMM"]
-    assert [st.kernel_family for st in wp.plan_prefill_steps(2048, flags=pkg.FLAG_FORCE_MFMA)] == ["mfmaGEMM"]
-    # K > N: the fused kernel keeps the shape up to 4095 rows
+    assert [st.kernel_family for st in wp.plan_prefill_steps(1023)] == ["mfmaGEMM"]
+    assert [st.kernel_family for st in wp.plan_prefill_steps(1024)] == ["dequantToBFloat", "libraryGEMM"]
+    assert [st.kernel_family for st in wp.plan_prefill_steps(1024, flags=pkg.FLAG_FORCE_MFMA)] == ["mfmaGEMM"]
+    # K > N: the fused kernel keeps the shape up to 2047 rows
     words2, s2, z2, _ = seeded_case(3301, 128, 1024, 4, 64)
     wl = ctx.weight_prepare_mlx(fmt, words2, s2, z2, pkg.BF16, pkg.LAYOUT_PLANES)
-    assert [st.kernel_family for st in wl.plan_prefill_steps(2048)] == ["mfmaGEMM"]
-    assert [st.kernel_family for st in wl.plan_prefill_steps(4096)] == ["dequantToBFloat", "libraryGEMM"]
+    assert [st.kernel_family for st in wl.plan_prefill_steps(2047)] == ["mfmaGEMM"]
+    assert [st.kernel_family for st in wl.plan_prefill_steps(2048)] == ["dequantToBFloat", "libraryGEMM"]
     wl.destroy()
     x = act_rounded(kat.seeded_activations(3302, 64, k), pkg.BF16, pkg)
     want = oracle.gemm_f64(wb, x)
