@@ -157,19 +157,21 @@ def main():
     # ---- the decode plans, built once, replayed from C -----------------------------------------
     #   "7-launch": one launch per projection, the reference's decode schedule
     #   "4-launch": q+k+v and gate+up share their input and run as one launch each
-    def build_plan(fused):
+    def build_plan(fused, xd=None, xt=None):
+        xd = xdev if xd is None else xd
+        xt = pkg.BF16 if xt is None else xt
         plan = pkg.DispatchPlan(ctx)
         for li, L in enumerate(layers):
             def lin(name, k):
-                plan.add_linear(L[name], xdev[k], pkg.BF16, ydev[name], pkg.BF16, 1, layer_index=li,
+                plan.add_linear(L[name], xd[k], xt, ydev[name], xt, 1, layer_index=li,
                                 tensor_name=f"layers.{li}.{name}_proj.weight")
             if fused:
-                plan.add_batched_linear([L["q"], L["k"], L["v"]], xdev[4096], pkg.BF16,
-                                        [ydev["q"], ydev["k"], ydev["v"]], pkg.BF16, 1, layer_index=li,
+                plan.add_batched_linear([L["q"], L["k"], L["v"]], xd[4096], xt,
+                                        [ydev["q"], ydev["k"], ydev["v"]], xt, 1, layer_index=li,
                                         tensor_name=f"layers.{li}.qkv_proj.weight")
                 lin("o", 4096)
-                plan.add_batched_linear([L["gate"], L["up"]], xdev[4096], pkg.BF16, [ydev["gate"], ydev["up"]],
-                                        pkg.BF16, 1, layer_index=li, tensor_name=f"layers.{li}.gate_up_proj.weight")
+                plan.add_batched_linear([L["gate"], L["up"]], xd[4096], xt, [ydev["gate"], ydev["up"]],
+                                        xt, 1, layer_index=li, tensor_name=f"layers.{li}.gate_up_proj.weight")
                 lin("down", 14336)
             else:
                 for name, n, k in LAYER_SHAPES:
@@ -232,6 +234,20 @@ def main():
         log(f"{label} graph replay:  {ms_pass / a.layers * 1e3:.2f} us/step, "
             f"{layer_bytes / (ms_pass / a.layers * 1e-3) / 1e9:.1f} GB/s; spread {spreads[label + ' hip-graph']}")
         plan.destroy()
+    # the reference decodes in f16: the same 4-launch step with f16 activations and outputs, graph replay
+    x16dev = {k: ctx.upload(v.astype(np.float16).view(np.uint16)) for k, v in xs.items()}
+    plan16 = build_plan(True, x16dev, pkg.F16)
+    f16_kernel = plan16.step(2)[0].device_kernel
+    plan16.graph_build(stream)
+    for _ in range(2):
+        plan16.graph_launch(stream)
+    ctx.synchronize(stream)
+    ms16 = time_region(ctx, lambda i: plan16.graph_launch(stream), max(1, steps // a.layers), stream) / a.layers
+    ctx.synchronize(stream)
+    plan16.destroy()
+    f16_step = {"us_per_step": round(ms16 * 1e3, 2), "GBps": round(layer_bytes / (ms16 * 1e-3) / 1e9, 1),
+                "gate_up_kernel": f16_kernel, "vs_bf16": round(ms16 / results["4-launch hip-graph"], 3)}
+    log(f"4-launch graph replay with f16 activations: {f16_step}")
     mode = min(results, key=results.get)
     ms_step = results[mode]
     value = layer_bytes / (ms_step * 1e-3) / 1e9
@@ -539,6 +555,20 @@ def main():
                 sweep[f"{name} M={mm}"] = {"us": round(ms * 1e3, 1), "TFLOPs": round(2.0 * mm * n * k / (ms * 1e-3) / 1e12, 1),
                                            "route": " + ".join(st.device_kernel for st in steps_p)}
                 xb.free(); yb.free()
+        # the reference prefills with f16 or fp32 activations: the two-dispatch route in those types, M = 2048 gate
+        for tname, xt, npdt in (("f16", pkg.F16, np.float16), ("f32", pkg.F32, np.float32)):
+            wts = [L["gate"] for L in layers[:4]]
+            xa = kat.seeded_activations(2548, 2048, 4096).astype(npdt)
+            xb = ctx.upload(xa.view(np.uint16) if tname == "f16" else xa)
+            yb = ctx.alloc(2048 * 14336 * 4)
+            for i in range(4):
+                ctx.qgemm(wts[i], xb, xt, yb, xt, 2048, 0, 0, 0, stream)
+            ctx.synchronize(stream)
+            ms = time_region(ctx, lambda i: ctx.qgemm(wts[i % 4], xb, xt, yb, xt, 2048, 0, 0, 0, stream), 12, stream)
+            sweep[f"gate 4096->14336 M=2048 {tname} activations"] = {
+                "us": round(ms * 1e3, 1), "TFLOPs": round(2.0 * 2048 * 14336 * 4096 / (ms * 1e-3) / 1e12, 1),
+                "route": " + ".join(st.device_kernel for st in wts[0].plan_prefill_steps(2048, 4096, x_dtype=xt))}
+            xb.free(); yb.free()
         sweep["activations"] = "N(0,1) bf16, seeded"
         log("  prefill sweep (N(0,1)): " + ", ".join(f"{k2} {v['us']} us ({v['TFLOPs']} TFLOP/s, {v['route']})"
                                                    for k2, v in sweep.items() if isinstance(v, dict)))
@@ -602,7 +632,7 @@ def main():
                    "replay": mode, "replay_GBps": replay_gbps, "step_time_spread": spreads[mode],
                    "step_time_spread_all": spreads, "steps_asked": a.steps, "warmup_asked": a.warmup,
                    "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2), "per_shape": per_shape,
-                   "batch_sweep": batch_sweep, "other_configs": other, "staf_blocks_in_place_step": staf_step, "next_rows": next_rows,
+                   "f16_activations_step": f16_step, "batch_sweep": batch_sweep, "other_configs": other, "staf_blocks_in_place_step": staf_step, "next_rows": next_rows,
                    "stream_read_probe": stream_read,
                    "prefill_gemm_gate": prefill},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
