@@ -75,7 +75,7 @@ mi355q_status run_small_m(mi355q_context* ctx, hipStream_t s, const mi355q_weigh
                                       (char*)yp + (size_t)r0 * ys * ysz, y_dtype, mm - r0 < 8 ? mm - r0 : 8, xs, ys, nullptr,
                                       nullptr, HeadKeys{});
         } else if (!generic && gemv_staf_eligible(v, x_dtype, mm, xs) && (uintptr_t)xp % 16 == 0) {
-            st = launch_gemv_staf(s, ctx, v, xp, yp, y_dtype, mm, xs, ys);
+            st = launch_gemv_staf(s, ctx, v, xp, x_dtype, yp, y_dtype, mm, xs, ys);
         } else {
             st = launch_gemv_generic(s, v, xp, x_dtype, yp, y_dtype, mm, xs, ys);
         }
@@ -206,7 +206,7 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
         return launch_gemv_tile16_multi(s, ctx, count, views, x, ys, strides, y_dtype, m, xs, nullptr, nullptr,
                                         HeadKeys{});
     if (in_place && (uintptr_t)x % 16 == 0)
-        return launch_gemv_staf_multi(s, ctx, count, views, x, ys, strides, y_dtype, m, xs, nullptr, nullptr, HeadKeys{});
+        return launch_gemv_staf_multi(s, ctx, count, views, x, x_dtype, ys, strides, y_dtype, m, xs, nullptr, nullptr, HeadKeys{});
     for (uint32_t i = 0; i < count; i++) {
         mi355q_status st = dispatch_linear(ctx, s, weights[i], x, x_dtype, ys[i], y_dtype, m, xs, 0, flags, false);
         if (st != MI355Q_OK) return st;
@@ -235,7 +235,7 @@ mi355q_status dispatch_output_head(mi355q_context* ctx, hipStream_t s, const mi3
     if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && gemv_staf_eligible(v, x_dtype, 1, xs) && (uintptr_t)x % 16 == 0) {
         void* none[1] = {nullptr};
         const uint32_t strides[1] = {(uint32_t)w->n};
-        return launch_gemv_staf_multi(s, ctx, 1, &v, x, none, strides, MI355Q_F32, 1, xs, logits, token,
+        return launch_gemv_staf_multi(s, ctx, 1, &v, x, x_dtype, none, strides, MI355Q_F32, 1, xs, logits, token,
                                       keys);
     }
     // two dispatches, as the reference runs the head: projection to fp32 logits, then argmax

@@ -158,10 +158,10 @@ mi355q_status launch_gemv_fast(hipStream_t s, const mi355q_context* ctx, const W
                                int32_t* token_out, HeadKeys keys);
 // Block-layout GEMV (gemv_staf.hip): reads STAF interleaved blocks in place.
 bool gemv_staf_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
-mi355q_status launch_gemv_staf(hipStream_t s, const mi355q_context* ctx, const WView& w, const void* x, void* y,
-                               int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride);
+mi355q_status launch_gemv_staf(hipStream_t s, const mi355q_context* ctx, const WView& w, const void* x, int x_dtype,
+                               void* y, int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride);
 mi355q_status launch_gemv_staf_multi(hipStream_t s, const mi355q_context* ctx, uint32_t count, const WView* w,
-                                     const void* x, void* const* y, const uint32_t* y_strides, int y_dtype,
+                                     const void* x, int x_dtype, void* const* y, const uint32_t* y_strides, int y_dtype,
                                      uint32_t m, uint32_t x_stride, float* logits_f32, int32_t* token_out,
                                      HeadKeys keys);
 struct GemvLaunchShape {

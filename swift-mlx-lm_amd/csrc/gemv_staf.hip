@@ -1,5 +1,5 @@
 // Decode GEMV that reads STAF interleaved blocks in place ([f16 scale][f16 zero][packed codes], one
-// block per group), bf16 activations, 1 <= M <= 8: the path of a weight that was wrapped or uploaded
+// block per group), bf16 or f16 activations, 1 <= M <= 8: the path of a weight that was wrapped or uploaded
 // from a model file without being repacked.
 //
 //   * a block is 4 + GROUP*BITS/8 bytes (36 for q4 g64), so a lane cannot fetch "its" block with one
@@ -17,7 +17,9 @@
 //   * arithmetic is that of the split-plane kernel: activations staged once per workgroup in LDS in
 //     the pair order the unpacker produces together with the per-block sums, 2..6-bit codes turned
 //     into bf16 (128+q) pairs for v_dot2_f32_bf16, 8-bit codes through fp32 FMA, the affine form
-//     s*sum(q*x) + z*sum(x) per block, one wavefront reduction per output row.
+//     s*sum(q*x) + z*sum(x) per block, one wavefront reduction per output row.  With f16 activations every
+//     width, 8 bits included, becomes f16 (1024+q) pairs (exact: one unit in the last place is 1 from 1024
+//     to 2048) for v_dot2_f32_f16.
 //
 // Replaces gemv_q{b}_g{g} reading the STAF payload directly
 // (Sources/MetalCompiler/Generator/MetalSourceGenerator+Quantized.swift:496-575; block layout:
@@ -38,7 +40,7 @@ struct StafArgs {
     uint32_t wave_end[kGemvMaxSegments];       // cumulative wavefront counts; unused entries repeat the last
     uint32_t seg_rows[kGemvMaxSegments];       // N_i
     uint32_t y_stride[kGemvMaxSegments];
-    const uint16_t* x;       // bf16 [M, x_stride]
+    const uint16_t* x;       // bf16 or f16 [M, x_stride] (the kernel's XA argument says which)
     float* logits;           // optional fp32 [N] copy (M == 1, single matrix)
     unsigned long long* scratch;   // ARGMAX only: one packed (ordered value, ~row) key per workgroup
     uint64_t row_bytes;      // blocks_per_row * bytes per block (a multiple of 16)
@@ -62,12 +64,15 @@ struct StafGeo {
 
 // XREG: rows are one span long (K <= 64 * GROUP) and M == 1: every lane keeps its block's activations and their sum
 // in registers instead of re-reading them from LDS at every row.
-template <int BITS, int GROUP, int MT, int WAVES, int D, bool ARGMAX, bool XREG>
+// XA = 0: bf16 activations.  XA = 1: f16 activations.
+template <int BITS, int GROUP, int MT, int WAVES, int D, bool ARGMAX, bool XREG, int XA>
 __global__ __launch_bounds__(WAVES * 64) void gemv_staf_kernel(const StafArgs a) {
     static_assert(!XREG || MT == 1, "register-resident activations are for M == 1");
     using G = StafGeo<BITS, GROUP>;
     constexpr int WPB = G::WPB, BW = G::BW, SPAN = G::SPAN, NDMA = G::NDMA, SLOT = G::SLOT, Q = G::Q;
-    constexpr bool DOT2 = BITS <= 6;                        // 128 + q is exact in bf16
+    constexpr bool DOT2 = BITS <= 6 || XA == 1;             // 128 + q is exact in bf16 up to 6 bits, 1024 + q in f16 up to 8
+    constexpr float OFS = XA == 1 ? 1024.0f : 128.0f;
+    constexpr uint32_t kOnes = XA == 1 ? 0x3C003C00u : 0x3F803F80u;
     static_assert(GROUP * BITS % 32 == 0 && GROUP % 8 == 0, "blocks are whole words");
     static_assert(NDMA * (D - 1) < 64, "the vector-memory counter has 6 bits");
 
@@ -158,7 +163,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_staf_kernel(const StafArgs a)
         });
         float sx = 0.0f;
 #pragma unroll
-        for (int j = 0; j < GROUP / 2; j++) sx = dot2_bf16(d[j], 0x3F803F80u, sx);
+        for (int j = 0; j < GROUP / 2; j++) sx = dot2_x<XA>(d[j], kOnes, sx);
         sxs[(size_t)(m * NSP + sp) * 64 + lane] = sx;
     }
     __syncthreads();
@@ -171,7 +176,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_staf_kernel(const StafArgs a)
         sxr = sxs[lane];
     }
 
-    uint32_t k_magic = 0x43004300u;                          // bf16 pair (128.0, 128.0)
+    uint32_t k_magic = XA == 1 ? 0x64006400u : 0x43004300u;  // f16 pair (1024.0, 1024.0) or bf16 pair (128.0, 128.0)
     uint32_t k_mask = BITS == 4 ? 0x000F000Fu : 0x00030003u;
     asm volatile("" : "+v"(k_magic));
     asm volatile("" : "+s"(k_mask));
@@ -263,10 +268,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_staf_kernel(const StafArgs a)
 #pragma unroll
                 for (int m = 0; m < MT; m++) {
                     float dsum = dot[m];
-                    dsum = dot2_bf16(pr[0], xv[m].x, dsum);
-                    dsum = dot2_bf16(pr[1], xv[m].y, dsum);
-                    dsum = dot2_bf16(pr[2], xv[m].z, dsum);
-                    dsum = dot2_bf16(pr[3], xv[m].w, dsum);
+                    dsum = dot2_x<XA>(pr[0], xv[m].x, dsum);
+                    dsum = dot2_x<XA>(pr[1], xv[m].y, dsum);
+                    dsum = dot2_x<XA>(pr[2], xv[m].z, dsum);
+                    dsum = dot2_x<XA>(pr[3], xv[m].w, dsum);
                     dot[m] = dsum;
                 }
             } else {
@@ -289,7 +294,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_staf_kernel(const StafArgs a)
             }
         });
         const float s = f16_to_f32((uint16_t)(hdr & 0xFFFFu)), z = f16_to_f32((uint16_t)(hdr >> 16));
-        const float zc = DOT2 ? z - 128.0f * s : z;
+        const float zc = DOT2 ? z - OFS * s : z;
 #pragma unroll
         for (int m = 0; m < MT; m++) acc[m] += s * dot[m] + zc * (XREG ? sxr : sxs[(size_t)(m * NSP + sp) * 64 + lane]);
 
@@ -376,7 +381,7 @@ uint32_t staf_rows_per_wave(const mi355q_context* ctx, uint32_t n, const StafCfg
 }
 
 // `total_rows`: rows of all matrices of the launch; `grid`: workgroups (the caller has dealt the wavefronts).
-template <int BITS, int GROUP>
+template <int BITS, int GROUP, int XA>
 mi355q_status launch_for_format(hipStream_t s, const StafArgs& a, int mt, int depth, uint32_t grid, bool argmax) {
     using G = StafGeo<BITS, GROUP>;
     const size_t lds = staf_lds_bytes(G::SLOT, G::Q, a.nsp, mt, depth);
@@ -389,38 +394,32 @@ mi355q_status launch_for_format(hipStream_t s, const StafArgs& a, int mt, int de
         return MI355Q_OK;
     };
     if (depth == 2) {
-        if (argmax) return xreg ? go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 2, true, true>)
-                                : go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 2, true, false>);
+        if (argmax) return xreg ? go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 2, true, true, XA>)
+                                : go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 2, true, false, XA>);
         switch (mt) {
-        case 1: return xreg ? go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 2, false, true>)
-                            : go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 2, false, false>);
-        case 2: return go(gemv_staf_kernel<BITS, GROUP, 2, kWaves, 2, false, false>);
-        default: return go(gemv_staf_kernel<BITS, GROUP, 4, kWaves, 2, false, false>);
+        case 1: return xreg ? go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 2, false, true, XA>)
+                            : go(gemv_staf_kernel<BITS, GROUP, 1, kWaves, 2, false, false, XA>);
+        case 2: return go(gemv_staf_kernel<BITS, GROUP, 2, kWaves, 2, false, false, XA>);
+        default: return go(gemv_staf_kernel<BITS, GROUP, 4, kWaves, 2, false, false, XA>);
         }
     }
     return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no block-layout GEMV with ring depth %d", depth);
 }
 
 mi355q_status launch_by_format(hipStream_t s, uint32_t bits, uint32_t group, const StafArgs& a, int mt, int depth,
-                               uint32_t grid, bool argmax) {
+                               uint32_t grid, bool argmax, int x_dtype) {
+#define MI355Q_STAF_LAUNCH(B, GR) \
+    case B * 1000 + GR: \
+        return x_dtype == MI355Q_F16 ? launch_for_format<B, GR, 1>(s, a, mt, depth, grid, argmax) \
+                                     : launch_for_format<B, GR, 0>(s, a, mt, depth, grid, argmax);
     switch (bits * 1000 + group) {
-    case 4064: return launch_for_format<4, 64>(s, a, mt, depth, grid, argmax);
-    case 4128: return launch_for_format<4, 128>(s, a, mt, depth, grid, argmax);
-    case 8032: return launch_for_format<8, 32>(s, a, mt, depth, grid, argmax);
-    case 8064: return launch_for_format<8, 64>(s, a, mt, depth, grid, argmax);
-    case 2064: return launch_for_format<2, 64>(s, a, mt, depth, grid, argmax);
-    case 3064: return launch_for_format<3, 64>(s, a, mt, depth, grid, argmax);
-    case 5064: return launch_for_format<5, 64>(s, a, mt, depth, grid, argmax);
-    case 6064: return launch_for_format<6, 64>(s, a, mt, depth, grid, argmax);
-    case 2016: return launch_for_format<2, 16>(s, a, mt, depth, grid, argmax);
-    case 2032: return launch_for_format<2, 32>(s, a, mt, depth, grid, argmax);
-    case 3032: return launch_for_format<3, 32>(s, a, mt, depth, grid, argmax);
-    case 5032: return launch_for_format<5, 32>(s, a, mt, depth, grid, argmax);
-    case 6016: return launch_for_format<6, 16>(s, a, mt, depth, grid, argmax);
-    case 6032: return launch_for_format<6, 32>(s, a, mt, depth, grid, argmax);
-    case 8128: return launch_for_format<8, 128>(s, a, mt, depth, grid, argmax);
+    MI355Q_STAF_LAUNCH(4, 64) MI355Q_STAF_LAUNCH(4, 128) MI355Q_STAF_LAUNCH(8, 32) MI355Q_STAF_LAUNCH(8, 64)
+    MI355Q_STAF_LAUNCH(2, 64) MI355Q_STAF_LAUNCH(3, 64) MI355Q_STAF_LAUNCH(5, 64) MI355Q_STAF_LAUNCH(6, 64)
+    MI355Q_STAF_LAUNCH(2, 16) MI355Q_STAF_LAUNCH(2, 32) MI355Q_STAF_LAUNCH(3, 32) MI355Q_STAF_LAUNCH(5, 32)
+    MI355Q_STAF_LAUNCH(6, 16) MI355Q_STAF_LAUNCH(6, 32) MI355Q_STAF_LAUNCH(8, 128)
     default: break;
     }
+#undef MI355Q_STAF_LAUNCH
     return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no block-layout GEMV for q%ug%u", bits, group);
 }
 
@@ -448,7 +447,7 @@ int staf_max_mt(const WView& w, const StafShape& sh) {
 }  // namespace
 
 bool gemv_staf_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
-    if (w.layout != MI355Q_LAYOUT_STAF_BLOCKS || x_dtype != MI355Q_BF16) return false;
+    if (w.layout != MI355Q_LAYOUT_STAF_BLOCKS || (x_dtype != MI355Q_BF16 && x_dtype != MI355Q_F16)) return false;
     if (m < 1 || m > 8 || !w.blocks) return false;
     StafShape sh;
     if (!staf_shape(w.bits, w.group, sh)) return false;
@@ -482,7 +481,7 @@ GemvLaunchShape gemv_staf_shape(const mi355q_context* ctx, const WView& w, uint3
 // Up to three weights sharing K, format and activations in one launch; `w[0]` supplies the format, the caller has
 // checked that the others match.  `token_out` selects the fused arg-max tail (one weight, M == 1).
 mi355q_status launch_gemv_staf_multi(hipStream_t s, const mi355q_context* ctx, uint32_t count, const WView* w,
-                                     const void* x, void* const* y, const uint32_t* y_strides, int y_dtype,
+                                     const void* x, int x_dtype, void* const* y, const uint32_t* y_strides, int y_dtype,
                                      uint32_t m, uint32_t x_stride, float* logits_f32, int32_t* token_out,
                                      HeadKeys keys) {
     if (count < 1 || count > (uint32_t)kGemvMaxSegments)
@@ -533,18 +532,18 @@ mi355q_status launch_gemv_staf_multi(hipStream_t s, const mi355q_context* ctx, u
         if (argmax && grid > keys.capacity) return fail(MI355Q_ERR_SHAPE, "too many workgroups for the fused argmax");
         a.x = (const uint16_t*)x + (size_t)m0 * x_stride;
         a.m = mm;
-        if (mi355q_status st = launch_by_format(s, w[0].bits, w[0].group, a, mt, c.depth, grid, argmax)) return st;
+        if (mi355q_status st = launch_by_format(s, w[0].bits, w[0].group, a, mt, c.depth, grid, argmax, x_dtype)) return st;
         if (argmax) return launch_argmax_finish(s, keys.ptr, grid, token_out);
         m0 += mm;
     }
     return MI355Q_OK;
 }
 
-mi355q_status launch_gemv_staf(hipStream_t s, const mi355q_context* ctx, const WView& w, const void* x, void* y,
-                               int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride) {
+mi355q_status launch_gemv_staf(hipStream_t s, const mi355q_context* ctx, const WView& w, const void* x, int x_dtype,
+                               void* y, int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride) {
     void* ys[1] = {y};
     const uint32_t strides[1] = {y_stride};
-    return launch_gemv_staf_multi(s, ctx, 1, &w, x, ys, strides, y_dtype, m, x_stride, nullptr, nullptr, HeadKeys{});
+    return launch_gemv_staf_multi(s, ctx, 1, &w, x, x_dtype, ys, strides, y_dtype, m, x_stride, nullptr, nullptr, HeadKeys{});
 }
 
 }  // namespace mi355q

@@ -77,18 +77,26 @@ def test_in_place_gemv_formats_and_tails(pkg, ctx, bits, group):
                 say(f"in-place q{bits}g{group} N={n} K={k} M={m}")
                 got = run_gemv(ctx, pkg, w, x, pkg.BF16, pkg.F32)
                 assert_within_tolerance(got, oracle.gemm_f64(wq, x), f"q{bits}g{group} N={n} K={k} M={m}")
+            # f16 activations (the reference's decode type): the same kernel with f16 code pairs, no fallback
+            assert w.plan_decode_step(1, pkg.F16).device_kernel == f"gemv_staf_q{bits}_g{group}"
+            for m in (1, 3, 8):
+                x = act_rounded(kat.seeded_activations(3150 + m + ci, m, k), pkg.F16, pkg)
+                got = run_gemv(ctx, pkg, w, x, pkg.F16, pkg.F32)
+                assert_within_tolerance(got, oracle.gemm_f64(wq, x), f"f16 q{bits}g{group} N={n} K={k} M={m}")
             w.destroy()
 
 
 def test_in_place_gemv_is_the_planned_kernel(pkg, ctx):
-    """The plan names the in-place kernel for a STAF-layout weight with bf16 activations, and the
+    """The plan names the in-place kernel for a STAF-layout weight with bf16 or f16 activations, and the
     per-code kernel when the row of blocks is not a multiple of 16 bytes or acceleration is off."""
     case = _case(3200, 64, 4096, 4, 64)
     w = case.device_weight(ctx, pkg, pkg.LAYOUT_STAF_BLOCKS)
     step = w.plan_decode_step(1)
     assert step.device_kernel == "gemv_staf_q4_g64" and not step.used_fallback, step.device_kernel
     assert step.block[0] == 256 and step.grid[0] >= 1 and step.lds_bytes > 0
-    assert not w.plan_decode_step(1, pkg.F16).device_kernel.startswith("gemv_staf")   # bf16 activations only
+    f16_step = w.plan_decode_step(1, pkg.F16)
+    assert f16_step.device_kernel == "gemv_staf_q4_g64" and not f16_step.used_fallback      # f16 activations too
+    assert not w.plan_decode_step(1, pkg.F32).device_kernel.startswith("gemv_staf")         # fp32: the per-code kernel
     forced = w.plan_decode_step(1, flags=pkg.FLAG_FORCE_GENERIC)
     assert forced.device_kernel == "gemv_generic" and forced.used_fallback
     w.destroy()
