@@ -124,6 +124,8 @@ mi355q_status launch_unpack_codes(hipStream_t s, const WView& w, uint8_t* out);
 mi355q_status launch_dequant_bf16(hipStream_t s, const WView& w, uint16_t* out);
 mi355q_status launch_dequant_f32(hipStream_t s, const WView& w, float* out);
 mi355q_status launch_dequant_f16(hipStream_t s, const WView& w, uint16_t* out);
+mi355q_status launch_split_f32_bf16x2(hipStream_t s, const float* x, uint32_t m, uint32_t k, uint32_t x_stride, uint16_t* hi,
+                                      uint16_t* lo);
 mi355q_status launch_gemv_generic(hipStream_t s, const WView& w, const void* x, int x_dtype,
                                   void* y, int y_dtype, uint32_t m, uint32_t x_stride,
                                   uint32_t y_stride);
@@ -239,9 +241,10 @@ constexpr size_t kDenseLibraryWorkspace = (size_t)64 << 20;
 // Both operands in `ab_dtype` (bf16, f16 or fp32), fp32 accumulation, output in y_dtype.
 bool dense_library_serves(mi355q_context* ctx, int ab_dtype, uint32_t m, uint32_t n, uint32_t k, uint32_t x_stride,
                           uint32_t y_stride, int y_dtype);
+// `accumulate`: Y += X W^T instead of Y = X W^T (the second half of a split-activation product).
 mi355q_status dense_library_gemm(hipStream_t s, mi355q_context* ctx, int ab_dtype, const void* x, const void* w_dense,
                                  void* y, int y_dtype, uint32_t m, uint32_t n, uint32_t k, uint32_t x_stride,
-                                 uint32_t y_stride, void* workspace);
+                                 uint32_t y_stride, void* workspace, bool accumulate = false);
 void dense_library_release(mi355q_context* ctx);
 // Rows from which the two-dispatch route is taken.  Beside the fused matrix-core kernel (measured, q4 g64, N(0,1)
 // activations, fused against two-dispatch with the library's candidates timed): 4096 -> 14336 at M = 512 90-100

@@ -161,19 +161,19 @@ bool dense_library_serves(mi355q_context* ctx, int ab_dtype, uint32_t m, uint32_
 
 mi355q_status dense_library_gemm(hipStream_t s, mi355q_context* ctx, int ab_dtype, const void* x, const void* w_bf16,
                                  void* y, int y_dtype, uint32_t m, uint32_t n, uint32_t k, uint32_t x_stride,
-                                 uint32_t y_stride, void* workspace) {
+                                 uint32_t y_stride, void* workspace, bool accumulate) {
     DenseLibrary* lib = library_of(ctx);
     if (!lib) return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the dense GEMM library (hipBLASLt) could not be opened");
     Problem* p = find_problem(lib, ab_dtype, m, n, k, x_stride, y_stride, y_dtype);
     if (!p->usable)
         return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the dense GEMM library has no algorithm for M=%u N=%u K=%u", m, n, k);
-    const float one = 1.0f, zero = 0.0f;
+    const float one = 1.0f, zero = accumulate ? 1.0f : 0.0f;     // `zero` is beta
     // First eager call of a problem: time the candidates the heuristic ranked (its first is often not the fastest at
     // these shapes) on the caller's operands and keep the quickest.  Not while the stream is being captured: a
     // capture takes the algorithm in use, so run a problem once before capturing it.
     hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
     (void)hipStreamIsCapturing(s, &capture);
-    if (!p->timed && p->candidates > 1 && capture == hipStreamCaptureStatusNone) {
+    if (!p->timed && p->candidates > 1 && capture == hipStreamCaptureStatusNone && !accumulate) {
         p->timed = true;
         hipEvent_t e0 = nullptr, e1 = nullptr;
         if (hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {

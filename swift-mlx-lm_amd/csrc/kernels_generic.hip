@@ -326,6 +326,39 @@ mi355q_status launch_dequant(hipStream_t s, const WView& w, void* out) {
     return MI355Q_OK;
 }
 
+// fp32 activations as two bf16 matrices: hi = bf16(x), lo = bf16(x - hi), so that hi + lo carries sixteen bits of x
+// (x - hi is exact in fp32).  Four elements per thread; x rows 16-byte aligned, K a multiple of 4.
+__global__ __launch_bounds__(256) void split_f32_bf16x2_kernel(const float* __restrict__ x, uint32_t m, uint32_t k,
+                                                               uint32_t x_stride, uint16_t* __restrict__ hi,
+                                                               uint16_t* __restrict__ lo) {
+    const uint32_t row = blockIdx.y;
+    for (uint32_t c = (blockIdx.x * 256 + threadIdx.x) * 4; c < k; c += gridDim.x * 1024) {
+        const float4 v = *(const float4*)(x + (size_t)row * x_stride + c);
+        const float f[4] = {v.x, v.y, v.z, v.w};
+        uint16_t h[4], l[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            h[i] = f32_to_bf16_rne(f[i]);
+            l[i] = f32_to_bf16_rne(f[i] - __uint_as_float((uint32_t)h[i] << 16));
+        }
+        uint2 hv, lv;
+        hv.x = h[0] | ((uint32_t)h[1] << 16); hv.y = h[2] | ((uint32_t)h[3] << 16);
+        lv.x = l[0] | ((uint32_t)l[1] << 16); lv.y = l[2] | ((uint32_t)l[3] << 16);
+        *(uint2*)(hi + (size_t)row * k + c) = hv;
+        *(uint2*)(lo + (size_t)row * k + c) = lv;
+    }
+}
+
+mi355q_status launch_split_f32_bf16x2(hipStream_t s, const float* x, uint32_t m, uint32_t k, uint32_t x_stride, uint16_t* hi,
+                                      uint16_t* lo) {
+    if (m > 65535u) return fail(MI355Q_ERR_SHAPE, "more than 65535 activation rows");
+    uint32_t gx = (k / 4 + 255) / 256;
+    if (gx > 64) gx = 64;
+    split_f32_bf16x2_kernel<<<dim3(gx, m), dim3(256), 0, s>>>(x, m, k, x_stride, hi, lo);
+    MI355Q_HIP(hipGetLastError());
+    return MI355Q_OK;
+}
+
 mi355q_status launch_dequant_bf16(hipStream_t s, const WView& w, uint16_t* out) { return launch_dequant<MI355Q_BF16>(s, w, out); }
 mi355q_status launch_dequant_f32(hipStream_t s, const WView& w, float* out) { return launch_dequant<MI355Q_F32>(s, w, out); }
 mi355q_status launch_dequant_f16(hipStream_t s, const WView& w, uint16_t* out) { return launch_dequant<MI355Q_F16>(s, w, out); }

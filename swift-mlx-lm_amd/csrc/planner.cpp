@@ -216,7 +216,8 @@ mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w, uint32_t maximum
         d->path = MI355Q_PATH_PREFILL_PROJECTION;
         d->input_row_stride = input_row_stride;
         d->flops = 0;
-        const char* const type_name = x_dtype == MI355Q_BF16 ? "bf16" : x_dtype == MI355Q_F16 ? "f16" : "f32";
+        // fp32 activations: bf16 weights against the activations split into two bf16 matrices (two library products)
+        const char* const type_name = x_dtype == MI355Q_F16 ? "f16" : "bf16";
         std::snprintf(d->kernel_name, sizeof d->kernel_name, "%s", w->fmt.dequant_to_bfloat_kernel_name);
         std::snprintf(d->device_kernel, sizeof d->device_kernel, "dequant_q%u_g%u_%s", (unsigned)w->fmt.bits,
                       w->fmt.group_size, type_name);
@@ -226,9 +227,10 @@ mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w, uint32_t maximum
         fill_common(w, m, s);
         s->path = MI355Q_PATH_PREFILL_PROJECTION;
         s->input_row_stride = input_row_stride;
-        s->weight_bytes = (uint64_t)w->n * w->k * (x_dtype == MI355Q_F32 ? 4 : 2);          // the dense operand it reads
+        s->weight_bytes = (uint64_t)w->n * w->k * 2;          // the dense operand it reads
         std::snprintf(s->kernel_name, sizeof s->kernel_name, "gemm_bf16_f32s");
-        std::snprintf(s->device_kernel, sizeof s->device_kernel, "hipblaslt_gemm_%s", type_name);
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, x_dtype == MI355Q_F32 ? "hipblaslt_gemm_%s_x2" : "hipblaslt_gemm_%s",
+                      type_name);
         std::snprintf(s->kernel_family, sizeof s->kernel_family, "libraryGEMM");
         return MI355Q_OK;
     }

@@ -206,19 +206,22 @@ def test_dense_entry_point_hands_long_products_to_the_library(pkg, ctx):
 
 @pytest.mark.parametrize("x_dtype_name,y_dtype_names", [("F16", ("F32", "F16")), ("F32", ("F32",))])
 def test_two_step_f16_and_f32_activations(pkg, ctx, x_dtype_name, y_dtype_names):
-    """f16 and fp32 activations (the reference's gemm_q*_g* and gemm_q*_g*_f32s signatures): the matrix is dequantised
-    to the activations' type and the library multiplies in that type with fp32 accumulation.  Unforced, every layout
-    takes the route from sixteen rows (the fused kernel reads bf16 only)."""
+    """f16 and fp32 activations (the reference's gemm_q*_g* and gemm_q*_g*_f32s signatures).  f16: the matrix is
+    dequantised to f16 and the library multiplies in f16 with fp32 accumulation.  fp32 into fp32: bf16 weights, as the
+    reference's gemm_bf16_f32s has them, against the activations split into two bf16 matrices (sixteen bits of every
+    activation; two library products, the second accumulating).  Unforced, every layout takes the route from sixteen
+    rows (the fused kernel reads bf16 only)."""
     x_dtype = getattr(pkg, x_dtype_name)
     n, k = 200, 1024
     fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
     words, s, z, wq = seeded_case(3600, n, k, 4, 64)
-    w_round = wq.astype(np.float16).astype(np.float32) if x_dtype == pkg.F16 else wq
+    w_round = wq.astype(np.float16).astype(np.float32) if x_dtype == pkg.F16 else bf16_round(wq)
     for layout in (pkg.LAYOUT_PLANES, pkg.LAYOUT_STAF_BLOCKS):
         w = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, layout)
         steps = w.plan_prefill_steps(64, x_dtype=x_dtype)
-        suffix = x_dtype_name.lower()
-        assert [st.device_kernel for st in steps] == [f"dequant_q4_g64_{suffix}", f"hipblaslt_gemm_{suffix}"]
+        want_kernels = (["dequant_q4_g64_f16", "hipblaslt_gemm_f16"] if x_dtype == pkg.F16
+                        else ["dequant_q4_g64_bf16", "hipblaslt_gemm_bf16_x2"])
+        assert [st.device_kernel for st in steps] == want_kernels
         for m in (16, 77, 300):
             x = act_rounded(kat.seeded_activations(3610 + m, m, k), x_dtype, pkg)
             want = oracle.gemm_f64(w_round, x)
