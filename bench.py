@@ -305,7 +305,7 @@ def main():
                 pool = [{name: ctx.weight_prepare_mlx(fmt, *host[name], pkg.BF16, layout) for name, _, _ in LAYER_SHAPES}
                         for _ in range(n_t16)]
             batch_sweep[lname] = {}
-            for m in ((1, 2, 4, 8) if lname == "planes" else (1, 2, 4, 8, 16)):    # the tile kernel takes 16 rows a launch
+            for m in (1, 2, 4, 8, 16):                      # both layouts take up to 16 rows a launch
                 xm = {k: ctx.upload(oracle.bf16_from_f32(kat.seeded_activations(900 + m, m, k))) for k in (4096, 14336)}   # N(0,1)
                 ym = {name: ctx.alloc(m * n * 2) for name, n, _ in LAYER_SHAPES}
                 pl = pkg.DispatchPlan(ctx)

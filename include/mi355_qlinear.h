@@ -266,7 +266,7 @@ MI355Q_API mi355q_status mi355q_qgemv(mi355q_context* ctx, void* stream, const m
  * MC/Compiler/MetalPrefillStepBuilder.swift:728-732).  Three routes, all with the weights rounded once
  * to bf16 and fp32 accumulation, chosen by measured cost unless flags say otherwise
  * (mi355q_plan_prefill_steps reports the choice):
- *   - small M (up to 8 rows, 16 on TILE16): the GEMV-style decode kernels;
+ *   - small M (up to 8 rows; 16 on TILE16 records and on q4 planes): the GEMV-style decode kernels;
  *   - ONE fused kernel: code tiles are dequantised to bf16 in LDS and contracted on MFMA (the planes
  *     and TILE16 layouts, formats q4 g64/g128, q8 g32/g64, q6/q3/q2 g64, bf16 activations);
  *   - two dispatches, as the reference's second route: the whole matrix is dequantised to bf16 in a

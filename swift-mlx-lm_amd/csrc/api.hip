@@ -44,7 +44,7 @@ mi355q_status run_small_m(mi355q_context* ctx, hipStream_t s, const mi355q_weigh
     const size_t xsz = x_dtype == MI355Q_F32 ? 4 : 2, ysz = y_dtype == MI355Q_F32 ? 4 : 2;
     const bool generic = flags & MI355Q_FLAG_FORCE_GENERIC;
     // rows per launch: 16 on the tile layout (fewer when K is so long that 16 staged rows overflow LDS), else 8
-    uint32_t step = 8;
+    uint32_t step = generic ? 8 : small_batch_rows(v, x_dtype, xs);
     if (!generic && v.layout == MI355Q_LAYOUT_TILE16) {
         step = 16;
         while (step > 1 && !gemv_tile16_eligible(v, x_dtype, step, xs)) step >>= 1;
@@ -129,8 +129,8 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
 }
 
 uint32_t small_batch_rows(const WView& w, int x_dtype, uint32_t x_stride) {
-    (void)x_dtype; (void)x_stride;
-    return w.layout == MI355Q_LAYOUT_TILE16 ? 16 : 8;
+    if (w.layout == MI355Q_LAYOUT_TILE16) return 16;
+    return gemv_mfma_planes_eligible(w, x_dtype, 16, x_stride) ? 16 : 8;
 }
 
 bool gemm_two_step_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
@@ -204,7 +204,7 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
     bool fused = m <= 8 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
     bool tiled = m <= 16 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
     bool in_place = m <= 8 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
-    bool on_planes = m >= kMfmaPlanesMinRows && m <= 8 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
+    bool on_planes = m >= kMfmaPlanesMinRows && m <= 16 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
     WView views[3];
     uint32_t strides[3];
     for (uint32_t i = 0; i < count; i++) {

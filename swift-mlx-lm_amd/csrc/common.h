@@ -198,7 +198,7 @@ mi355q_status launch_gemv_tile16_multi(hipStream_t s, mi355q_context* ctx, uint3
                                        HeadKeys keys);
 mi355q_status launch_tile16_pack(hipStream_t s, const WView& planes, uint32_t* tiles);
 
-// Matrix-core small-batch kernel over the split planes (gemv_mfma_planes.hip): 2 <= M <= 8, q4 g64 / g128.  Its
+// Matrix-core small-batch kernel over the split planes (gemv_mfma_planes.hip): 2 <= M <= 16, q4 g64 / g128.  Its
 // workgroups are shaped like those of the TILE16 kernel (16-row tiles, blocks of 128 codes).
 // Rows from which it is taken; below, the split-plane dot-product kernels are as fast or faster (measured, Llama-3-8B
 // layer step in four launches: M = 2 42 us against 48 us here, M = 4 59 against 56, M = 8 117 against 55).
@@ -209,7 +209,8 @@ Tile16LaunchShape gemv_mfma_planes_shape(const mi355q_context* ctx, uint32_t n_r
 mi355q_status launch_gemv_mfma_planes_multi(hipStream_t s, mi355q_context* ctx, uint32_t count, const WView* w,
                                             const void* x, void* const* y, const uint32_t* y_strides, int y_dtype,
                                             uint32_t m, uint32_t x_stride);
-// Rows one launch of the small-batch kernels takes for this weight: 16 on TILE16 records, else 8.
+// Rows one launch of the small-batch kernels takes for this weight: 16 on TILE16 records and on planes the
+// matrix-core kernel reads, else 8.
 uint32_t small_batch_rows(const WView& w, int x_dtype, uint32_t x_stride);
 
 // Validated dispatch shared by the direct entry points and by plan replay (api.hip)

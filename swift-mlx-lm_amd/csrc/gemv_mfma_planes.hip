@@ -1,5 +1,5 @@
 // Small-batch projection on the matrix cores straight from the split planes (4-bit codes, groups of 64 or
-// 128), 2 <= M <= 8 activation rows per launch: the layout that serves M = 1 best also serves a batch.
+// 128), 2 <= M <= 16 activation rows per launch: the layout that serves M = 1 best also serves a batch.
 //
 // Stands in for gemv_q4_g{64,128} widened to the sequence signature and, at small sequence lengths, for gemm_q4_g64
 // (Sources/MetalCompiler/Generator/MetalSourceGenerator+Quantized.swift:496-575 and :22-156):
@@ -56,8 +56,13 @@ struct PmArgs {
 
 // GROUP: 64 or 128.  A workgroup of KSPLIT * TPW wavefronts covers TPW consecutive row tiles, each split over KSPLIT
 // wavefronts along K; all of them share one staged copy of the activations.
-template <int GROUP, int KSPLIT, int TPW, bool SBBF16>
+// WIDE: nine to sixteen activation rows.  The M dimension then has no empty half, so the two groups of a block are
+// kept apart with two products per word instead: one whose A operand carries the activations only where kq < 2, one
+// only where kq >= 2 (groups of 128 need neither: one product with the whole A operand).  Every lane then holds rows
+// 4 kq .. 4 kq + 3 of both groups' sums and applies both (scale, bias) words.
+template <int GROUP, int KSPLIT, int TPW, bool SBBF16, bool WIDE>
 __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmArgs a) {
+    constexpr uint32_t SXR = WIDE ? 16 : 8;                 // activation rows per run of 64 in the staged sums
     constexpr int WAVES = KSPLIT * TPW;
     constexpr int D = 4;                                    // blocks in flight per wavefront
     constexpr int MR = 4;
@@ -159,7 +164,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
     issue_sz(tile.b_first);
 
     // ---- 3. stage the activations: every run of eight as (x0,x4,x1,x5,x2,x6,x3,x7), and sum(x) per 64 and row ------
-    float* const sxs = (float*)(lds + (size_t)(a.m + 1) * a.lds_row_bytes);      // [run of 64 in part][8]
+    float* const sxs = (float*)(lds + (size_t)(a.m + 1) * a.lds_row_bytes);      // [run of 64 in part][SXR]
     {
         auto stage = [&](uint32_t idx, const u32x4& v) {
             float p = pm_dot2(v.x, 0x3F803F80u, 0.0f);
@@ -177,7 +182,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
                 o.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);    // (x2, x6)
                 o.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);    // (x3, x7)
                 *((u32x4*)(lds + (size_t)m * a.lds_row_bytes) + c) = o;
-                if ((c & 7u) == 0) sxs[(c >> 3) * 8 + m] = p;       // eight chunks: one run of 64
+                if ((c & 7u) == 0) sxs[(c >> 3) * SXR + m] = p;     // eight chunks: one run of 64
             }
         };
         // whole wavefronts take part in the shuffles of every step: the walk is rounded up to whole batches
@@ -211,9 +216,12 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
     // A operand: lane (i = lane % 16, kq) stands for A row i.  Rows 0..7 are activation rows 0..7 where kq < 2, rows
     // 8..15 are the same activation rows where kq >= 2; elsewhere the row of zeros.  Rows past M read row M-1 (their
     // results are never stored).
-    const uint32_t xr = (n_in & 7u) < a.m ? (n_in & 7u) : a.m - 1;
-    const bool live = (n_in >> 3) == (kq >> 1);
-    const char* const a_lane = lds + (size_t)(live ? xr : a.m) * a.lds_row_bytes + kq * 64;
+    const uint32_t xi = WIDE ? n_in : (n_in & 7u);
+    const uint32_t xr = xi < a.m ? xi : a.m - 1;
+    const bool live = WIDE ? (kq < 2) : (n_in >> 3) == (kq >> 1);
+    const char* const a_lane = lds + (size_t)(live || (WIDE && GROUP == 128) ? xr : a.m) * a.lds_row_bytes + kq * 64;
+    // WIDE, groups of 64: the second product's operand, live where the first one's is not
+    const char* const a_lane_hi = lds + (size_t)(live ? a.m : xr) * a.lds_row_bytes + kq * 64;
 
     auto unpack = [&](uint32_t w) -> pm_bf16x8_t {
         u32x4 p;
@@ -224,7 +232,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
         return __builtin_bit_cast(pm_bf16x8_t, p);
     };
     // this lane's D rows 4 kq .. 4 kq + 3 are activation rows 4 (kq & 1) .. + 3
-    const uint32_t sx_lane = (kq >> 1) * 8 + 4 * (kq & 1);
+    const uint32_t sx_lane = WIDE ? 4 * kq : (kq >> 1) * 8 + 4 * (kq & 1);
     const int from_lane = (int)((4u * n_in + kq) * 4u);     // byte address of the lane that loaded (row n, piece kq)
     auto compute = [&](uint32_t b, const Rec& r, const uint32_t (&sz_pair)[SZW], uint32_t sz_piece) {
         const uint32_t bl = b - b0;                          // block inside the staged columns
@@ -239,32 +247,73 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
         // the block's (scale, bias) words sit with the lane that loaded piece `sz_piece` of this row
         const int sz_from = (int)((4u * n_in + sz_piece) * 4u);
         uint32_t szw = (uint32_t)__builtin_amdgcn_ds_bpermute(sz_from, (int)sz_pair[0]);
+        uint32_t szw_hi = szw;
         if constexpr (SZW == 2) {
-            const uint32_t hi = (uint32_t)__builtin_amdgcn_ds_bpermute(sz_from, (int)sz_pair[1]);
-            szw = kq >> 1 ? hi : szw;
+            szw_hi = (uint32_t)__builtin_amdgcn_ds_bpermute(sz_from, (int)sz_pair[1]);
+            if constexpr (!WIDE) szw = kq >> 1 ? szw_hi : szw;
         }
         const pm_bf16x8_t a0 = *(const pm_bf16x8_t*)(ab), a1 = *(const pm_bf16x8_t*)(ab + 16);
         const pm_bf16x8_t a2 = *(const pm_bf16x8_t*)(ab + 32), a3 = *(const pm_bf16x8_t*)(ab + 48);
-        const pm_floatx4_t sx = *(const pm_floatx4_t*)(sxs + (size_t)bl * 16 + sx_lane);
-        __builtin_amdgcn_sched_barrier(0);
-        pm_floatx4_t d = zero4;
-        d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, unpack(w0), d, 0, 0, 0);
-        d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, unpack(w1), d, 0, 0, 0);
-        d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2, unpack(w2), d, 0, 0, 0);
-        d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a3, unpack(w3), d, 0, 0, 0);
-        float s, z;
-        if constexpr (SBBF16) { s = __uint_as_float(szw << 16); z = __uint_as_float(szw & 0xFFFF0000u); }
-        else { s = f16_to_f32((uint16_t)(szw & 0xFFFFu)); z = f16_to_f32((uint16_t)(szw >> 16)); }
-        const float zc = z - 128.0f * s;
+        const pm_floatx4_t sx = *(const pm_floatx4_t*)(sxs + (size_t)bl * 2 * SXR + sx_lane);
+        auto scale_zero = [&](uint32_t word, float& sc, float& zc) {
+            float zr;
+            if constexpr (SBBF16) { sc = __uint_as_float(word << 16); zr = __uint_as_float(word & 0xFFFF0000u); }
+            else { sc = f16_to_f32((uint16_t)(word & 0xFFFFu)); zr = f16_to_f32((uint16_t)(word >> 16)); }
+            zc = zr - 128.0f * sc;
+        };
+        if constexpr (!WIDE) {
+            __builtin_amdgcn_sched_barrier(0);
+            pm_floatx4_t d = zero4;
+            d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, unpack(w0), d, 0, 0, 0);
+            d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, unpack(w1), d, 0, 0, 0);
+            d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2, unpack(w2), d, 0, 0, 0);
+            d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a3, unpack(w3), d, 0, 0, 0);
+            float sc, zc;
+            scale_zero(szw, sc, zc);
 #pragma unroll
-        for (int q = 0; q < MR; q++) acc[q] += s * d[q] + zc * sx[q];
+            for (int q = 0; q < MR; q++) acc[q] += sc * d[q] + zc * sx[q];
+        } else {
+            const pm_floatx4_t sx_hi = *(const pm_floatx4_t*)(sxs + (size_t)(bl * 2 + 1) * SXR + sx_lane);
+            const pm_bf16x8_t b0 = unpack(w0), b1 = unpack(w1), b2 = unpack(w2), b3 = unpack(w3);
+            if constexpr (GROUP == 128) {
+                __builtin_amdgcn_sched_barrier(0);
+                pm_floatx4_t d = zero4;
+                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, b0, d, 0, 0, 0);
+                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b1, d, 0, 0, 0);
+                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2, b2, d, 0, 0, 0);
+                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a3, b3, d, 0, 0, 0);
+                float sc, zc;
+                scale_zero(szw, sc, zc);
+#pragma unroll
+                for (int q = 0; q < MR; q++) acc[q] += sc * d[q] + zc * (sx[q] + sx_hi[q]);
+            } else {
+                const char* ah = a_lane_hi + (size_t)bl * 256;
+                const pm_bf16x8_t h0 = *(const pm_bf16x8_t*)(ah), h1 = *(const pm_bf16x8_t*)(ah + 16);
+                const pm_bf16x8_t h2 = *(const pm_bf16x8_t*)(ah + 32), h3 = *(const pm_bf16x8_t*)(ah + 48);
+                __builtin_amdgcn_sched_barrier(0);
+                pm_floatx4_t d = zero4, e = zero4;
+                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, b0, d, 0, 0, 0);
+                e = __builtin_amdgcn_mfma_f32_16x16x32_bf16(h0, b0, e, 0, 0, 0);
+                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, b1, d, 0, 0, 0);
+                e = __builtin_amdgcn_mfma_f32_16x16x32_bf16(h1, b1, e, 0, 0, 0);
+                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2, b2, d, 0, 0, 0);
+                e = __builtin_amdgcn_mfma_f32_16x16x32_bf16(h2, b2, e, 0, 0, 0);
+                d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a3, b3, d, 0, 0, 0);
+                e = __builtin_amdgcn_mfma_f32_16x16x32_bf16(h3, b3, e, 0, 0, 0);
+                float s0, z0, s1, z1;
+                scale_zero(szw, s0, z0);
+                scale_zero(szw_hi, s1, z1);
+#pragma unroll
+                for (int q = 0; q < MR; q++) acc[q] += (s0 * d[q] + z0 * sx[q]) + (s1 * e[q] + z1 * sx_hi[q]);
+            }
+        }
     };
 
     const uint32_t rounds = (a.blocks_per_wave + D - 1) / D;              // same for every wavefront
     // Partial tiles of the WAVES wavefronts, [WAVES][MR][64]: a single pass writes them over the staged activations
     // once every wavefront is done reading those; several passes keep them behind the activations and their sums.
     const bool red_over_x = a.passes == 1;
-    float* const red = (float*)(red_over_x ? lds : lds + (size_t)(a.m + 1) * a.lds_row_bytes + kp / 2);
+    float* const red = (float*)(red_over_x ? lds : lds + (size_t)(a.m + 1) * a.lds_row_bytes + (size_t)(kp / 64) * SXR * 4);
     for (uint32_t pass = 0; pass < a.passes; pass++) {
         if (pass) {                                            // the first tile's loads were issued before staging
             tile = select_tile(pass);
@@ -286,13 +335,15 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
 #pragma unroll
         for (int r = 0; r < MR; r++) { red[(wave * MR + r) * 64 + lane] = acc[r]; acc[r] = 0.f; }
         __syncthreads();
-        if (slice == 0 && tile.valid && kq < 2) {           // the first wavefront of each tile adds and stores
+        if (slice == 0 && tile.valid && (WIDE || kq < 2)) { // the first wavefront of each tile adds and stores
             const uint32_t row = tile.n0 + n_in;
 #pragma unroll
             for (int r = 0; r < MR; r++) {
                 float v = 0.f;
-                for (uint32_t w2 = 0; w2 < (uint32_t)KSPLIT; w2++)       // both halves of K of every wavefront's block
-                    v += red[((wave + w2) * MR + r) * 64 + lane] + red[((wave + w2) * MR + r) * 64 + lane + 32];
+                for (uint32_t w2 = 0; w2 < (uint32_t)KSPLIT; w2++) {     // (not WIDE: both halves of K of every block)
+                    v += red[((wave + w2) * MR + r) * 64 + lane];
+                    if constexpr (!WIDE) v += red[((wave + w2) * MR + r) * 64 + lane + 32];
+                }
                 const uint32_t m = 4 * kq + r;
                 if (m < a.m && row < tile.rows) {
                     if (a.parts > 1) {                       // one matrix: the reduction launch converts and stores
@@ -329,8 +380,10 @@ namespace {
 
 template <int GROUP, int KSPLIT, int TPW>
 mi355q_status launch_pm(hipStream_t s, const PmArgs& a, uint32_t grid, size_t lds) {
-    auto kern = a.sb_dtype == MI355Q_BF16 ? gemv_mfma_planes_kernel<GROUP, KSPLIT, TPW, true>
-                                          : gemv_mfma_planes_kernel<GROUP, KSPLIT, TPW, false>;
+    auto kern = a.m > 8 ? (a.sb_dtype == MI355Q_BF16 ? gemv_mfma_planes_kernel<GROUP, KSPLIT, TPW, true, true>
+                                                     : gemv_mfma_planes_kernel<GROUP, KSPLIT, TPW, false, true>)
+                        : (a.sb_dtype == MI355Q_BF16 ? gemv_mfma_planes_kernel<GROUP, KSPLIT, TPW, true, false>
+                                                     : gemv_mfma_planes_kernel<GROUP, KSPLIT, TPW, false, false>);
     if (lds > 64 * 1024)
         MI355Q_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     kern<<<dim3(grid, a.parts), dim3(KSPLIT * TPW * 64), lds, s>>>(a);
@@ -362,7 +415,7 @@ mi355q_status launch_pm_shape(hipStream_t s, const PmArgs& a, const Tile16Launch
 // kernel's LDS sizes bound this one's ((M + 1) rows and K / 2 bytes of sums against (M + 1) rows and K bytes).
 bool gemv_mfma_planes_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
     if (w.layout != MI355Q_LAYOUT_PLANES || !w.sz || x_dtype != MI355Q_BF16) return false;
-    if (m < 2 || m > 8) return false;
+    if (m < 2 || m > 16) return false;
     if (w.bits != 4 || (w.group != 64 && w.group != 128) || w.k % 128) return false;
     if (x_stride % 8) return false;                                       // 128-bit activation loads
     // a row is one stream: its sz words follow its code words at the same pitch; code words 16-byte aligned

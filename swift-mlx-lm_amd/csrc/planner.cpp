@@ -62,9 +62,9 @@ void plan_small_m(const mi355q_weight* w, uint32_t m, int x_dtype, uint32_t x_st
         s->block[0] = g.block;
         s->lds_bytes = g.lds_bytes;
         s->rows_per_workgroup = 16;
-    } else if (!forced && m >= kMfmaPlanesMinRows && gemv_mfma_planes_eligible(v, x_dtype, m > 8 ? 8 : m, x_stride)) {
+    } else if (!forced && m >= kMfmaPlanesMinRows && gemv_mfma_planes_eligible(v, x_dtype, m > 16 ? 16 : m, x_stride)) {
         const Tile16LaunchShape g = gemv_mfma_planes_shape(w->ctx, (uint32_t)((w->n + 15) / 16), (uint32_t)w->k,
-                                                           m > 8 ? 8 : m);
+                                                           m > 16 ? 16 : m);
         std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_mfma_planes_q%u_g%u", (unsigned)w->fmt.bits,
                       w->fmt.group_size);
         s->grid[0] = g.wgs_per_part;
@@ -110,7 +110,7 @@ void plan_shared_launch_shape(const mi355q_weight* const* ws, uint32_t count, ui
     WView all = ws[0]->view();
     uint64_t total = 0;
     // four rows and more: the matrix-core kernel over the planes takes the rows of all matrices, in 16-row tiles
-    bool on_planes = m >= kMfmaPlanesMinRows && m <= 8;
+    bool on_planes = m >= kMfmaPlanesMinRows && m <= 16;
     uint32_t tiles = 0;
     for (uint32_t i = 0; i < count && on_planes; i++) {
         const WView v = ws[i]->view();

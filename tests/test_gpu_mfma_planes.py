@@ -1,6 +1,7 @@
 """GPU parity tests of the small-batch matrix-core kernel over the split planes (4-bit, groups of 64 and 128), through
 the C ABI: the projections of gemv_q4_g64 / gemm_q4_g64 of the reference
-(MetalSourceGenerator+Quantized.swift:496-575, :22-156) for 4 <= M <= 8 rows per launch on the layout that serves M = 1.
+(MetalSourceGenerator+Quantized.swift:496-575, :22-156) for 4 <= M <= 16 rows per launch on the layout that serves M = 1
+(up to eight rows the two quantisation groups of a block are kept apart in the M dimension, above with two products).
 
 Bars: fp32 outputs within relative L2 <= 1e-3 and max-abs <= 2e-2 of an fp64 accumulation of the dequantised weights
 (exact codes, no rounding of the weights); bf16 outputs equal bf16_rne(fp32 outputs); exactly representable cases are
@@ -33,14 +34,14 @@ def test_mfma_planes_seeded_shapes(pkg, ctx, group):
     for i, (n, k) in enumerate([(96, 512), (200, 1024), (33, 128), (17, 256), (64, 14336), (4100, 4096)]):
         words, s, z, wq = seeded_case(4100 + i + group, n, k, 4, group)
         w = ctx.weight_prepare_mlx(_fmt(pkg, group), words, s, z, pkg.BF16, pkg.LAYOUT_PLANES)
-        for m in ((4, 5, 6, 7, 8) if n < 4000 else (4, 8)):
+        for m in ((4, 5, 6, 7, 8, 9, 11, 13, 16) if n < 4000 else (4, 8, 16)):
             say(f"mfma planes g{group} {k}->{n} M={m}")
             x = act_rounded(kat.seeded_activations(4200 + m, m, k), pkg.BF16, pkg)
-            st = w.plan_decode_step(m)
+            st = w.plan_decode_step(m) if m <= 8 else w.plan_prefill_steps(m)[0]
             assert st.device_kernel == f"gemv_mfma_planes_q4_g{group}" and not st.used_fallback
-            y32 = run_gemv(ctx, pkg, w, x, pkg.BF16, pkg.F32)
+            y32 = run_gemv(ctx, pkg, w, x, pkg.BF16, pkg.F32, use_qgemm=m > 8)
             assert_within_tolerance(y32, oracle.gemm_f64(wq, x), f"g{group} {k}->{n} M={m}")
-            ybf = run_gemv(ctx, pkg, w, x, pkg.BF16, pkg.BF16)
+            ybf = run_gemv(ctx, pkg, w, x, pkg.BF16, pkg.BF16, use_qgemm=m > 8)
             assert np.array_equal(oracle.bf16_from_f32(ybf), oracle.bf16_from_f32(y32))
         for m in (2, 3):                                        # below the threshold: the dot-product kernels
             assert w.plan_decode_step(m).device_kernel != f"gemv_mfma_planes_q4_g{group}"
@@ -59,13 +60,13 @@ def test_mfma_planes_exact_small_integers_f16_scales_and_strides(pkg, ctx):
     wq = scales.repeat(64, axis=1) * codes + zeros.repeat(64, axis=1)
     for name, w in (("f16", ctx.weight_prepare_staf(_fmt(pkg), n, k, case.staf_blocks(), pkg.LAYOUT_PLANES)),
                     ("bf16", ctx.weight_prepare_mlx(_fmt(pkg), *case.planes(pkg.BF16, pkg), pkg.BF16, pkg.LAYOUT_PLANES))):
-        for m, xpad, ypad in ((4, 0, 0), (5, 8, 0), (8, 16, 12)):
+        for m, xpad, ypad in ((4, 0, 0), (5, 8, 0), (8, 16, 12), (12, 8, 4), (16, 0, 0)):
             x = np.full((m, k + xpad), 512.0, np.float32)
             x[:, :k] = rng.integers(-8, 9, (m, k)).astype(np.float32) * 0.125
-            assert w.plan_decode_step(m).device_kernel == "gemv_mfma_planes_q4_g64"
             xd = ctx.upload(oracle.bf16_from_f32(x).reshape(x.shape))
             yd = ctx.alloc(m * (n + ypad) * 4); ctx.fill(yd, 0x7FC00000)
-            ctx.qgemv(w, xd, pkg.BF16, yd, pkg.F32, m, k + xpad, (n + ypad) if ypad else 0); ctx.synchronize()
+            (ctx.qgemv if m <= 8 else ctx.qgemm)(w, xd, pkg.BF16, yd, pkg.F32, m, k + xpad, (n + ypad) if ypad else 0)
+            ctx.synchronize()
             got = yd.download(np.float32, (m, n + ypad))
             assert np.array_equal(got[:, :n].astype(np.float64), x[:, :k].astype(np.float64) @ wq.T), (name, m)
             assert np.all(np.isnan(got[:, n:]))
@@ -80,14 +81,14 @@ def test_mfma_planes_batched_projections_one_launch(pkg, ctx):
         for i, n in enumerate(ns):
             words, s, z, wq = seeded_case(4400 + i + n % 13, n, k, 4, 64)
             ws.append(ctx.weight_prepare_mlx(_fmt(pkg), words, s, z, pkg.BF16, pkg.LAYOUT_PLANES)); wqs.append(wq)
-        for m in (4, 7, 8):
+        for m in (4, 7, 8, 10, 16):
             x = act_rounded(kat.seeded_activations(4500 + m, m, k), pkg.BF16, pkg)
             xd = ctx.upload(oracle.bf16_from_f32(x).reshape(x.shape))
             yds = [ctx.alloc(m * n * 4) for n in ns]
             ctx.batched_qgemm(ws, xd, pkg.BF16, yds, pkg.F32, m); ctx.synchronize()
             for j, n in enumerate(ns):
                 fused = yds[j].download(np.float32, (m, n))
-                alone = run_gemv(ctx, pkg, ws[j], x, pkg.BF16, pkg.F32)
+                alone = run_gemv(ctx, pkg, ws[j], x, pkg.BF16, pkg.F32, use_qgemm=m > 8)
                 assert np.array_equal(fused, alone), (ns, m, j)
                 assert_within_tolerance(fused, oracle.gemm_f64(wqs[j], x), f"batched {ns} M={m} #{j}")
             xd.free()
