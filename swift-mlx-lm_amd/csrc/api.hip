@@ -94,6 +94,14 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
     if (mi355q_status st = check_io(w, x, x_dtype, y, y_dtype, m, xs, ys)) return st;
     if (small_m_only) {
         if (m > 8) return fail(MI355Q_ERR_INVALID_ARGUMENT, "qgemv takes 1 <= M <= 8 (got %u); use qgemm", m);
+        // no decode kernel reads this layout with this activation type (fp32 anywhere, f16 on TILE16 records, block
+        // shapes the in-place kernel skips): dequantise once + the dense library product beats the per-code kernel
+        // from the second row (4096 -> 14336, fp32 activations: per-code kernel 123 us at M = 1, 195 at M = 2, 700 at
+        // M = 8; the route with fp32 weights 100-135 us whatever M)
+        const WView v = w->view();
+        if (gemm_two_step_chosen(v, x_dtype, m, xs, flags) && (uintptr_t)x % 16 == 0 &&
+            gemm_two_step_serves(ctx, v, x_dtype, y_dtype, m, xs, ys))
+            return launch_qgemm_two_step(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
         return run_small_m(ctx, s, w, x, x_dtype, y, y_dtype, m, xs, ys, flags);
     }
     const uint32_t forced = flags & (MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_TWO_STEP | MI355Q_FLAG_FORCE_SMALL_M |
@@ -108,10 +116,8 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
     }
     // dequantise once, then the dense library GEMM: long prompts, and every format or layout the fused kernel does
     // not read.  When the library has no algorithm for the problem the routes below serve it.
-    const bool split_f32 = x_dtype == MI355Q_F32 && y_dtype == MI355Q_F32;     // served as two bf16 products
     if (gemm_two_step_chosen(v, x_dtype, m, xs, flags) && (uintptr_t)x % 16 == 0 &&
-        (split_f32 ? dense_library_serves(ctx, MI355Q_BF16, m, (uint32_t)v.n, (uint32_t)v.k, (uint32_t)v.k, ys, MI355Q_F32)
-                   : dense_library_serves(ctx, x_dtype, m, (uint32_t)v.n, (uint32_t)v.k, xs, ys, y_dtype)))
+        gemm_two_step_serves(ctx, v, x_dtype, y_dtype, m, xs, ys))
         return launch_qgemm_two_step(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
     const bool mfma_ok = gemm_mfma_eligible(v, x_dtype, m, xs);
     // the clock probe cell lives behind the argmax cells of the context's scratch
@@ -133,6 +139,12 @@ uint32_t small_batch_rows(const WView& w, int x_dtype, uint32_t x_stride) {
     return gemv_mfma_planes_eligible(w, x_dtype, 16, x_stride) ? 16 : 8;
 }
 
+// Whether one of the decode kernels (not the per-code kernel) takes this layout with this activation type.
+bool decode_kernel_reads(const WView& w, int x_dtype, uint32_t x_stride) {
+    return gemv_tile16_eligible(w, x_dtype, 1, x_stride) || gemv_fast_eligible(w, x_dtype, 1, x_stride) ||
+           gemv_staf_eligible(w, x_dtype, 1, x_stride);
+}
+
 bool gemm_two_step_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
     (void)x_dtype;                                               // the dense copy takes the activations' type
     return m >= 1 && w.k % 8 == 0 && x_stride % 8 == 0 &&
@@ -143,21 +155,65 @@ bool gemm_two_step_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_st
     if (flags & (MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) return false;
     if (flags & MI355Q_FLAG_FORCE_TWO_STEP) return true;
     if (!gemm_two_step_eligible(w, x_dtype, m, x_stride)) return false;
-    if (!gemm_mfma_eligible(w, x_dtype, m, x_stride)) return m >= kTwoStepMinRowsOtherwise;
+    if (!gemm_mfma_eligible(w, x_dtype, m, x_stride))
+        return m >= kTwoStepMinRowsOtherwise || (m >= 2 && !decode_kernel_reads(w, x_dtype, x_stride));
     return m >= (w.k > w.n ? kTwoStepMinRowsLongK : kTwoStepMinRowsBesideFused);
 }
 
-// The whole matrix in the activations' type at the head of the context's scratch, the library's workspace behind it.
+// The three forms of the route, by rows and activation type:
+//   * below sixteen rows (only where no decode kernel reads the weight): fp32 weights, the activations widened to
+//     fp32, an fp32 product, the result narrowed to the output type -- the arithmetic of the decode kernels;
+//   * fp32 activations into an fp32 result from sixteen rows: bf16 weights, as the reference's gemm_bf16_f32s has
+//     them, against the activations split into two bf16 matrices (sixteen bits of every activation), two library
+//     products of which the second accumulates (M = 2048, 4096 -> 14336: 0.47 ms against 1.66 ms for an fp32 product);
+//   * otherwise: the matrix dequantised to the activations' type and one product in that type.
+namespace {
+enum class TwoStepForm { kExactF32, kSplitF32, kSameType };
+TwoStepForm two_step_form(int x_dtype, int y_dtype, uint32_t m, const WView& w, uint32_t x_stride) {
+    if (m < kTwoStepMinRowsOtherwise) return TwoStepForm::kExactF32;
+    if (x_dtype == MI355Q_F32 && y_dtype == MI355Q_F32 && w.k % 4 == 0 && x_stride % 4 == 0) return TwoStepForm::kSplitF32;
+    return TwoStepForm::kSameType;
+}
+}  // namespace
+
+bool gemm_two_step_serves(mi355q_context* ctx, const WView& w, int x_dtype, int y_dtype, uint32_t m, uint32_t x_stride,
+                          uint32_t y_stride) {
+    const uint32_t n = (uint32_t)w.n, k = (uint32_t)w.k;
+    switch (two_step_form(x_dtype, y_dtype, m, w, x_stride)) {
+    case TwoStepForm::kExactF32:
+        return dense_library_serves(ctx, MI355Q_F32, m, n, k, x_dtype == MI355Q_F32 ? x_stride : k,
+                                    y_dtype == MI355Q_F32 ? y_stride : n, MI355Q_F32);
+    case TwoStepForm::kSplitF32: return dense_library_serves(ctx, MI355Q_BF16, m, n, k, k, y_stride, MI355Q_F32);
+    default: return dense_library_serves(ctx, x_dtype, m, n, k, x_stride, y_stride, y_dtype);
+    }
+}
+
+// The dense matrix sits at the head of the context's scratch, converted activations and results behind it, the
+// library's workspace last.
 mi355q_status launch_qgemm_two_step(hipStream_t s, mi355q_context* ctx, const WView& w, const void* x, int x_dtype,
                                     void* y, int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride) {
-    // fp32 activations into an fp32 result: bf16 weights, as the reference's gemm_bf16_f32s has them, against the
-    // activations split into two bf16 matrices (sixteen bits of every activation), two library products of which the
-    // second accumulates: 3.8 times the speed of an fp32 product of fp32 weights (M = 2048, 4096 -> 14336: 0.44 against
-    // 1.66 ms).  Other output types of fp32 activations keep the fp32 product below.
-    if (x_dtype == MI355Q_F32 && y_dtype == MI355Q_F32 && w.k % 4 == 0 && x_stride % 4 == 0 &&
-        dense_library_serves(ctx, MI355Q_BF16, m, (uint32_t)w.n, (uint32_t)w.k, (uint32_t)w.k, y_stride, MI355Q_F32)) {
-        const size_t wbytes = (((size_t)w.n * w.k * 2) + 255) & ~(size_t)255;
-        const size_t xbytes = (((size_t)m * w.k * 2) + 255) & ~(size_t)255;
+    const uint32_t n = (uint32_t)w.n, k = (uint32_t)w.k;
+    auto round256 = [](size_t b) { return (b + 255) & ~(size_t)255; };
+    const TwoStepForm form = two_step_form(x_dtype, y_dtype, m, w, x_stride);
+    if (form == TwoStepForm::kExactF32) {
+        const bool widen = x_dtype != MI355Q_F32, narrow = y_dtype != MI355Q_F32;
+        const size_t wbytes = round256((size_t)n * k * 4), xbytes = widen ? round256((size_t)m * k * 4) : 0;
+        const size_t ybytes = narrow ? round256((size_t)m * n * 4) : 0;
+        if (mi355q_status st = ensure_workspace(ctx, wbytes + xbytes + ybytes + kDenseLibraryWorkspace)) return st;
+        char* const base = (char*)ctx->workspace;
+        float* const w32 = (float*)base;
+        float* const x32 = widen ? (float*)(base + wbytes) : (float*)const_cast<void*>(x);
+        float* const y32 = narrow ? (float*)(base + wbytes + xbytes) : (float*)y;
+        if (mi355q_status st = launch_dequant_f32(s, w, w32)) return st;
+        if (widen)
+            if (mi355q_status st = launch_convert_rows(s, x, x_dtype, x_stride, x32, MI355Q_F32, k, m, k)) return st;
+        if (mi355q_status st = dense_library_gemm(s, ctx, MI355Q_F32, x32, w32, y32, MI355Q_F32, m, n, k, widen ? k : x_stride,
+                                                  narrow ? n : y_stride, base + wbytes + xbytes + ybytes)) return st;
+        if (narrow) return launch_convert_rows(s, y32, MI355Q_F32, n, y, y_dtype, y_stride, m, n);
+        return MI355Q_OK;
+    }
+    if (form == TwoStepForm::kSplitF32) {
+        const size_t wbytes = round256((size_t)n * k * 2), xbytes = round256((size_t)m * k * 2);
         if (mi355q_status st = ensure_workspace(ctx, wbytes + 2 * xbytes + kDenseLibraryWorkspace)) return st;
         char* const base = (char*)ctx->workspace;
         uint16_t* const w_bf16 = (uint16_t*)base;
@@ -165,21 +221,20 @@ mi355q_status launch_qgemm_two_step(hipStream_t s, mi355q_context* ctx, const WV
         uint16_t* const lo = (uint16_t*)(base + wbytes + xbytes);
         void* const lib_ws = base + wbytes + 2 * xbytes;
         if (mi355q_status st = launch_dequant_bf16(s, w, w_bf16)) return st;
-        if (mi355q_status st = launch_split_f32_bf16x2(s, (const float*)x, m, (uint32_t)w.k, x_stride, hi, lo)) return st;
-        if (mi355q_status st = dense_library_gemm(s, ctx, MI355Q_BF16, hi, w_bf16, y, MI355Q_F32, m, (uint32_t)w.n,
-                                                  (uint32_t)w.k, (uint32_t)w.k, y_stride, lib_ws, false)) return st;
-        return dense_library_gemm(s, ctx, MI355Q_BF16, lo, w_bf16, y, MI355Q_F32, m, (uint32_t)w.n, (uint32_t)w.k,
-                                  (uint32_t)w.k, y_stride, lib_ws, true);
+        if (mi355q_status st = launch_split_f32_bf16x2(s, (const float*)x, m, k, x_stride, hi, lo)) return st;
+        if (mi355q_status st = dense_library_gemm(s, ctx, MI355Q_BF16, hi, w_bf16, y, MI355Q_F32, m, n, k, k, y_stride, lib_ws,
+                                                  false)) return st;
+        return dense_library_gemm(s, ctx, MI355Q_BF16, lo, w_bf16, y, MI355Q_F32, m, n, k, k, y_stride, lib_ws, true);
     }
     const size_t esz = x_dtype == MI355Q_F32 ? 4 : 2;
-    const size_t dense = (((size_t)w.n * w.k * esz) + 255) & ~(size_t)255;
+    const size_t dense = round256((size_t)n * k * esz);
     if (mi355q_status st = ensure_workspace(ctx, dense + kDenseLibraryWorkspace)) return st;
     void* const w_dense = ctx->workspace;
     const mi355q_status st = x_dtype == MI355Q_BF16 ? launch_dequant_bf16(s, w, (uint16_t*)w_dense)
                            : x_dtype == MI355Q_F16 ? launch_dequant_f16(s, w, (uint16_t*)w_dense)
                                                    : launch_dequant_f32(s, w, (float*)w_dense);
     if (st != MI355Q_OK) return st;
-    return dense_library_gemm(s, ctx, x_dtype, x, w_dense, y, y_dtype, m, (uint32_t)w.n, (uint32_t)w.k, x_stride, y_stride,
+    return dense_library_gemm(s, ctx, x_dtype, x, w_dense, y, y_dtype, m, n, k, x_stride, y_stride,
                               (char*)ctx->workspace + dense);
 }
 

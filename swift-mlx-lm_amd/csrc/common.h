@@ -256,6 +256,13 @@ void dense_library_release(mi355q_context* ctx);
 constexpr uint32_t kTwoStepMinRowsBesideFused = 1024, kTwoStepMinRowsLongK = 2048, kTwoStepMinRowsOtherwise = 16;
 // Rows from which mi355q_gemm_bf16 hands a plain dense product to the library.
 constexpr uint32_t kDenseLibraryMinRows = 128;
+bool decode_kernel_reads(const WView& w, int x_dtype, uint32_t x_stride);
+// whether the library has an algorithm for the product(s) the route would run for these types and rows
+bool gemm_two_step_serves(mi355q_context* ctx, const WView& w, int x_dtype, int y_dtype, uint32_t m, uint32_t x_stride,
+                          uint32_t y_stride);
+// rows of `cols` elements from one floating-point type to another (bf16, f16, fp32), strides in elements
+mi355q_status launch_convert_rows(hipStream_t s, const void* src, int src_dtype, uint32_t src_stride, void* dst, int dst_dtype,
+                                  uint32_t dst_stride, uint32_t rows, uint32_t cols);
 bool gemm_two_step_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
 bool gemm_two_step_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride, uint32_t flags);
 mi355q_status launch_qgemm_two_step(hipStream_t s, mi355q_context* ctx, const WView& w, const void* x, int x_dtype,

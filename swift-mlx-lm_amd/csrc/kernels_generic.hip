@@ -349,6 +349,33 @@ __global__ __launch_bounds__(256) void split_f32_bf16x2_kernel(const float* __re
     }
 }
 
+// Rows from one floating-point type to another, one element per thread (a handful of rows: the small-batch form of the
+// two-dispatch route widens its activations to fp32 and narrows its fp32 result).
+__global__ __launch_bounds__(256) void convert_rows_kernel(const void* __restrict__ src, int src_dtype, uint32_t src_stride,
+                                                           void* __restrict__ dst, int dst_dtype, uint32_t dst_stride,
+                                                           uint32_t cols) {
+    const uint32_t row = blockIdx.y;
+    for (uint32_t c = blockIdx.x * 256 + threadIdx.x; c < cols; c += gridDim.x * 256) {
+        const size_t i = (size_t)row * src_stride + c, o = (size_t)row * dst_stride + c;
+        const float v = src_dtype == MI355Q_F32 ? ((const float*)src)[i]
+                      : src_dtype == MI355Q_BF16 ? __uint_as_float((uint32_t)((const uint16_t*)src)[i] << 16)
+                                                 : f16_to_f32(((const uint16_t*)src)[i]);
+        if (dst_dtype == MI355Q_F32) ((float*)dst)[o] = v;
+        else if (dst_dtype == MI355Q_BF16) ((uint16_t*)dst)[o] = f32_to_bf16_rne(v);
+        else ((uint16_t*)dst)[o] = f32_to_f16_rne(v);
+    }
+}
+
+mi355q_status launch_convert_rows(hipStream_t s, const void* src, int src_dtype, uint32_t src_stride, void* dst, int dst_dtype,
+                                  uint32_t dst_stride, uint32_t rows, uint32_t cols) {
+    if (rows > 65535u) return fail(MI355Q_ERR_SHAPE, "more than 65535 rows");
+    uint32_t gx = (cols + 255) / 256;
+    if (gx > 256) gx = 256;
+    convert_rows_kernel<<<dim3(gx, rows), dim3(256), 0, s>>>(src, src_dtype, src_stride, dst, dst_dtype, dst_stride, cols);
+    MI355Q_HIP(hipGetLastError());
+    return MI355Q_OK;
+}
+
 mi355q_status launch_split_f32_bf16x2(hipStream_t s, const float* x, uint32_t m, uint32_t k, uint32_t x_stride, uint16_t* hi,
                                       uint16_t* lo) {
     if (m > 65535u) return fail(MI355Q_ERR_SHAPE, "more than 65535 activation rows");

@@ -89,6 +89,13 @@ void plan_small_m(const mi355q_weight* w, uint32_t m, int x_dtype, uint32_t x_st
         s->block[0] = g.block;
         s->lds_bytes = g.lds_bytes;
         s->rows_per_workgroup = g.rows_per_workgroup;
+    } else if (gemm_two_step_chosen(v, x_dtype, m, x_stride, flags)) {
+        // no decode kernel reads this layout with this activation type: dequantise once + the dense library product
+        // a few rows: fp32 weights and an fp32 product whatever the activation type (the decode kernels' arithmetic)
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "dequant_q%u_g%u_f32+hipblaslt_gemm_f32", (unsigned)w->fmt.bits,
+                      w->fmt.group_size);
+        std::snprintf(s->kernel_family, sizeof s->kernel_family, "libraryGEMM");
+        s->block[0] = 256;
     } else {
         std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_generic");
         s->grid[0] = (uint32_t)((w->n + 3) / 4);
@@ -216,8 +223,11 @@ mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w, uint32_t maximum
         d->path = MI355Q_PATH_PREFILL_PROJECTION;
         d->input_row_stride = input_row_stride;
         d->flops = 0;
-        // fp32 activations: bf16 weights against the activations split into two bf16 matrices (two library products)
-        const char* const type_name = x_dtype == MI355Q_F16 ? "f16" : "bf16";
+        // fp32 activations from sixteen rows: bf16 weights against the activations split into two bf16 matrices (two
+        // library products); below, an fp32 product of fp32 weights
+        const bool exact = m < kTwoStepMinRowsOtherwise;       // a few rows: fp32 weights, fp32 product, any activation type
+        const bool split = x_dtype == MI355Q_F32 && !exact;
+        const char* const type_name = exact ? "f32" : x_dtype == MI355Q_F16 ? "f16" : "bf16";
         std::snprintf(d->kernel_name, sizeof d->kernel_name, "%s", w->fmt.dequant_to_bfloat_kernel_name);
         std::snprintf(d->device_kernel, sizeof d->device_kernel, "dequant_q%u_g%u_%s", (unsigned)w->fmt.bits,
                       w->fmt.group_size, type_name);
@@ -227,10 +237,9 @@ mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w, uint32_t maximum
         fill_common(w, m, s);
         s->path = MI355Q_PATH_PREFILL_PROJECTION;
         s->input_row_stride = input_row_stride;
-        s->weight_bytes = (uint64_t)w->n * w->k * 2;          // the dense operand it reads
+        s->weight_bytes = (uint64_t)w->n * w->k * (exact ? 4 : 2);     // the dense operand it reads
         std::snprintf(s->kernel_name, sizeof s->kernel_name, "gemm_bf16_f32s");
-        std::snprintf(s->device_kernel, sizeof s->device_kernel, x_dtype == MI355Q_F32 ? "hipblaslt_gemm_%s_x2" : "hipblaslt_gemm_%s",
-                      type_name);
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, split ? "hipblaslt_gemm_%s_x2" : "hipblaslt_gemm_%s", type_name);
         std::snprintf(s->kernel_family, sizeof s->kernel_family, "libraryGEMM");
         return MI355Q_OK;
     }

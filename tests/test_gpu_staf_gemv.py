@@ -87,8 +87,8 @@ def test_in_place_gemv_formats_and_tails(pkg, ctx, bits, group):
 
 
 def test_in_place_gemv_is_the_planned_kernel(pkg, ctx):
-    """The plan names the in-place kernel for a STAF-layout weight with bf16 or f16 activations, and the
-    per-code kernel when the row of blocks is not a multiple of 16 bytes or acceleration is off."""
+    """The plan names the in-place kernel for a STAF-layout weight with bf16 or f16 activations, the small-batch form
+    of the two-dispatch route when the row of blocks is not a multiple of 16 bytes, the per-code kernel when forced."""
     case = _case(3200, 64, 4096, 4, 64)
     w = case.device_weight(ctx, pkg, pkg.LAYOUT_STAF_BLOCKS)
     step = w.plan_decode_step(1)
@@ -102,7 +102,11 @@ def test_in_place_gemv_is_the_planned_kernel(pkg, ctx):
     w.destroy()
     odd = _case(3201, 16, 64 * 3, 4, 64)                    # 108-byte rows
     w = odd.device_weight(ctx, pkg, pkg.LAYOUT_STAF_BLOCKS)
+    # no decode kernel reads 108-byte rows: the per-code kernel at one row; from two, fp32 weights into scratch + the
+    # library's fp32 product (or, forced, the per-code kernel)
     assert w.plan_decode_step(1).device_kernel == "gemv_generic"
+    assert w.plan_decode_step(2).device_kernel == "dequant_q4_g64_f32+hipblaslt_gemm_f32"
+    assert w.plan_decode_step(2, flags=pkg.FLAG_FORCE_GENERIC).device_kernel == "gemv_generic"
     x = act_rounded(kat.seeded_activations(3202, 1, odd.k), pkg.BF16, pkg)
     got = run_gemv(ctx, pkg, w, x, pkg.BF16, pkg.F32)
     assert_within_tolerance(got, oracle.gemm_f64(oracle.dequant_staf_f32(4, 64, odd.n, odd.k, odd.staf_blocks()), x))

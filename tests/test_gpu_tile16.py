@@ -403,9 +403,10 @@ def test_tile16_plan_replay_and_graph(pkg, ctx):
 
 @pytest.mark.parametrize("x_dtype_name", ["F16", "F32"])
 def test_tile16_other_activation_types_take_the_per_code_kernel_whole(pkg, ctx, x_dtype_name):
-    """The tile kernel reads bf16 activations only.  A few f16 or fp32 rows go to the per-code kernel, which takes all
-    of them in one launch (no walk in steps of sixteen, eight ... one row); from sixteen rows the two-dispatch route
-    serves (dequantised to the activations' type, then the dense library GEMM)."""
+    """The tile kernel reads bf16 activations only.  f16 and fp32 rows take the two-dispatch route from the second row
+    (the matrix dequantised to the activations' type, then the dense library GEMM; fp32 from sixteen rows: bf16
+    weights against split activations); forced, the per-code kernel takes all rows in one launch (no walk in steps
+    of sixteen, eight ... one row)."""
     x_dtype = getattr(pkg, x_dtype_name)
     n, k = 96, 512
     words, s, z, wq = seeded_case(2931, n, k, 4, 64)
@@ -413,7 +414,11 @@ def test_tile16_other_activation_types_take_the_per_code_kernel_whole(pkg, ctx, 
     for m in (1, 13, 200):
         x = act_rounded(kat.seeded_activations(2932 + m, m, k), x_dtype, pkg)
         got = run_gemv(ctx, pkg, w, x, x_dtype, pkg.F32, 0, use_qgemm=True)
-        # on the route, fp32 activations meet bf16 weights (the reference's gemm_bf16_f32s), f16 ones f16 weights
+        # from sixteen rows fp32 activations meet bf16 weights (the reference's gemm_bf16_f32s); f16 ones f16 weights
         weights = wq if m < 16 or x_dtype == pkg.F16 else oracle.bf16_to_f32(oracle.bf16_from_f32(wq)).reshape(wq.shape)
         assert_within_tolerance(got, oracle.gemm_f64(weights, x), f"{x_dtype_name} M={m}")
+        if m > 1:
+            assert w.plan_prefill_steps(m, x_dtype=x_dtype)[0].kernel_family in ("libraryGEMM", "dequantToBFloat")
+        slow = run_gemv(ctx, pkg, w, x, x_dtype, pkg.F32, pkg.FLAG_FORCE_GENERIC, use_qgemm=True)
+        assert_within_tolerance(slow, oracle.gemm_f64(wq, x), f"{x_dtype_name} M={m}, per-code kernel")
     w.destroy()
