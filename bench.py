@@ -408,7 +408,19 @@ def main():
             other[label] = {"us": round(ms * 1e3, 2), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1), "weight_bytes": nbytes}
             if head and not a.skip_parity:
                 other[label]["argmax_parity"] = head_check
-            log(f"  {label}: {other[label]['us']} us/launch, {other[label]['GBps']} GB/s")
+            if bits == 8:                                # the same matrix at eight activation rows, as dispatched
+                xb = ctx.upload(oracle.bf16_from_f32(kat.seeded_activations(3200 + ci, 8, k)))
+                yb = ctx.alloc(8 * n * 2)
+                for i in range(copies):
+                    ctx.qgemm(ws[i], xb, pkg.BF16, yb, pkg.BF16, 8, 0, 0, 0, stream)
+                ctx.synchronize(stream)
+                ms8 = time_region(ctx, lambda i: ctx.qgemm(ws[i % copies], xb, pkg.BF16, yb, pkg.BF16, 8, 0, 0, 0, stream),
+                                  6 * copies, stream)
+                other[label]["M=8"] = {"us": round(ms8 * 1e3, 2), "GBps": round(nbytes / (ms8 * 1e-3) / 1e9, 1),
+                                       "kernel": ws[0].plan_decode_step(8).device_kernel}
+                xb.free(); yb.free()
+            log(f"  {label}: {other[label]['us']} us/launch, {other[label]['GBps']} GB/s" +
+                (f"; M=8 {other[label]['M=8']}" if "M=8" in other[label] else ""))
             pl.destroy()
             for w in ws:
                 w.destroy()

@@ -266,7 +266,7 @@ MI355Q_API mi355q_status mi355q_qgemv(mi355q_context* ctx, void* stream, const m
  * MC/Compiler/MetalPrefillStepBuilder.swift:728-732).  Three routes, all with the weights rounded once
  * to bf16 and fp32 accumulation, chosen by measured cost unless flags say otherwise
  * (mi355q_plan_prefill_steps reports the choice):
- *   - small M (up to 8 rows; 16 on TILE16 records and on q4 planes): the GEMV-style decode kernels;
+ *   - small M (up to 8 rows; 16 on TILE16 records and on q4 / q8 planes): the GEMV-style decode kernels;
  *   - ONE fused kernel: code tiles are dequantised to bf16 in LDS and contracted on MFMA (the planes
  *     and TILE16 layouts, formats q4 g64/g128, q8 g32/g64, q6/q3/q2 g64, bf16 activations);
  *   - two dispatches, as the reference's second route: the whole matrix is dequantised to bf16 in a
@@ -279,6 +279,11 @@ MI355Q_API mi355q_status mi355q_qgemv(mi355q_context* ctx, void* stream, const m
  *     weights as in gemm_bf16_f32s, the activations split into bf16 high and low halves).  The
  *     first eager call of a shape times the library's candidate algorithms once (a few milliseconds)
  *     and keeps the quickest.  When the library is absent or has no algorithm, the other routes serve.
+ *     Batches of 2 to 15 rows whose layout or activation type no decode kernel reads (fp32 or f16
+ *     rows on TILE16 records, fp32 rows on planes and blocks, rows of the block layout that are not
+ *     whole 16-byte units) take it too, there with UNROUNDED fp32 weights (N*K*4 bytes of scratch),
+ *     the activations widened to fp32, the library's fp32 product and the result narrowed to y_dtype:
+ *     the result keeps the decode kernels' accuracy, at a cost that does not grow with M.
  * Launches that split K over workgroups (few output
  * tiles at short M; on the TILE16 layout, rows too long for M staged activation rows) keep fp32
  * partial results in a scratch buffer of the context, grown on first use: two such launches of one

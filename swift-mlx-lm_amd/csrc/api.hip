@@ -62,7 +62,7 @@ mi355q_status run_small_m(mi355q_context* ctx, hipStream_t s, const mi355q_weigh
             void* yv[1] = {yp};
             const uint32_t strides[1] = {ys};
             st = launch_gemv_tile16_multi(s, ctx, 1, &v, xp, yv, strides, y_dtype, mm, xs, nullptr, nullptr, HeadKeys{});
-        } else if (!generic && mm >= kMfmaPlanesMinRows && gemv_mfma_planes_eligible(v, x_dtype, mm, xs) &&
+        } else if (!generic && mm >= mfma_planes_min_rows(v.bits) && gemv_mfma_planes_eligible(v, x_dtype, mm, xs) &&
                    (uintptr_t)xp % 16 == 0) {
             void* yv[1] = {yp};
             const uint32_t strides[1] = {ys};
@@ -259,7 +259,7 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
     bool fused = m <= 8 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
     bool tiled = m <= 16 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
     bool in_place = m <= 8 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
-    bool on_planes = m >= kMfmaPlanesMinRows && m <= 16 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
+    bool on_planes = m >= mfma_planes_min_rows(weights[0]->fmt.bits) && m <= 16 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
     WView views[3];
     uint32_t strides[3];
     for (uint32_t i = 0; i < count; i++) {

@@ -202,10 +202,12 @@ mi355q_status launch_tile16_pack(hipStream_t s, const WView& planes, uint32_t* t
 // workgroups are shaped like those of the TILE16 kernel (16-row tiles, blocks of 128 codes).
 // Rows from which it is taken; below, the split-plane dot-product kernels are as fast or faster (measured, Llama-3-8B
 // layer step in four launches: M = 2 42 us against 48 us here, M = 4 59 against 56, M = 8 117 against 55).
-constexpr uint32_t kMfmaPlanesMinRows = 4;
+// fewest activation rows for which the matrix-core kernel beats the dot-product kernels on the same planes (measured;
+// 8 bits, 4096 -> 14336: two rows 16 us on the dot products, three 25 us, against 19 us on the matrix cores)
+inline uint32_t mfma_planes_min_rows(uint32_t bits) { return bits == 8 ? 3u : 4u; }
 bool gemv_mfma_planes_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
 uint32_t gemv_mfma_planes_k_parts(const mi355q_context* ctx, const WView& w, uint32_t m);
-Tile16LaunchShape gemv_mfma_planes_shape(const mi355q_context* ctx, uint32_t n_row_tiles, uint32_t k, uint32_t m);
+Tile16LaunchShape gemv_mfma_planes_shape(const mi355q_context* ctx, uint32_t n_row_tiles, uint32_t k, uint32_t bits, uint32_t m);
 mi355q_status launch_gemv_mfma_planes_multi(hipStream_t s, mi355q_context* ctx, uint32_t count, const WView* w,
                                             const void* x, void* const* y, const uint32_t* y_strides, int y_dtype,
                                             uint32_t m, uint32_t x_stride);

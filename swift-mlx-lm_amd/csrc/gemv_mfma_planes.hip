@@ -1,8 +1,9 @@
-// Small-batch projection on the matrix cores straight from the split planes (4-bit codes, groups of 64 or
-// 128), 2 <= M <= 16 activation rows per launch: the layout that serves M = 1 best also serves a batch.
+// Small-batch projection on the matrix cores straight from the split planes (4-bit codes in groups of 64 or 128,
+// 8-bit codes in groups of 32 or 64), 2 <= M <= 16 activation rows per launch: the layout that serves M = 1 best also
+// serves a batch.
 //
-// Stands in for gemv_q4_g{64,128} widened to the sequence signature and, at small sequence lengths, for gemm_q4_g64
-// (Sources/MetalCompiler/Generator/MetalSourceGenerator+Quantized.swift:496-575 and :22-156):
+// Stands in for gemv_q4_g{64,128} / gemv_q8_g{32,64} widened to the sequence signature and, at small sequence lengths,
+// for gemm_q4_g64 / gemm_q8_g32 (Sources/MetalCompiler/Generator/MetalSourceGenerator+Quantized.swift:496-575 and :22-156):
 //   y[m, n] = sum_g sum_{k in g} (s[n,g] * q[n,k] + z[n,g]) * x[m,k],  fp32 accumulation.
 //
 // A wavefront owns 16 consecutive weight rows and a share of K, walked in blocks of 128 codes.  One load instruction
@@ -21,6 +22,13 @@
 // is applied lane by lane, once per block, and lanes kq and kq + 2 add their halves at the end.  The KSPLIT wavefronts
 // that share a row tile add their partial tiles through LDS.  (With groups of 128 both halves belong to one group and
 // the same code runs unchanged.)
+//
+// 8-bit codes: a block is the same 64 bytes of a row, now 64 codes, and a lane's 16 bytes are 16 codes.  A code is
+// split into its nibbles, q = 16 h + l: the masks that pair up a 4-bit word's nibbles give, on an 8-bit word, the pairs
+// (l0,l2) (h0,h2) (l1,l3) (h1,h3), so two words make the B operand of one product over the low nibbles and one over the
+// high nibbles of eight codes, against the same A operand (activations staged as (x0,x2,x1,x3,x4,x6,x5,x7)):
+//   sum q x = D_l + 16 D_h - (128 + 16 * 128) SX.
+// Instructions per byte of weights are those of the 4-bit form; groups of 32 take the place of groups of 64.
 #include "device_utils.h"
 
 namespace mi355q {
@@ -45,23 +53,28 @@ struct PmArgs {
     uint32_t k, m, x_stride;
     uint32_t row_words;                        // 32-bit words from one row to the next (codes, then the row's sz words)
     uint32_t sz_offset;                        // words from a row's first code word to its first (scale, bias) word
-    uint32_t blocks_per_wave;                  // blocks of 128 codes per wavefront (K split over the workgroup)
+    uint32_t blocks_per_wave;                  // blocks (64 bytes of a row) per wavefront (K split over the workgroup)
     uint32_t passes;                           // row tiles a wavefront walks, one after the other, on one staged copy of x
-    uint32_t lds_row_bytes;                    // part_blocks * 256 + 16: staged activation row pitch
+    uint32_t lds_row_bytes;                    // part_blocks * (activation bytes per block) + 16: staged row pitch
     uint32_t y_dtype, sb_dtype;
     uint32_t parts;                            // K parts, each with workgroups of its own that stage only their columns
     uint32_t part_blocks;                      // blocks per part
     float* partial;                            // K parts only: fp32 partial results [part][M][N] (one matrix)
 };
 
-// GROUP: 64 or 128.  A workgroup of KSPLIT * TPW wavefronts covers TPW consecutive row tiles, each split over KSPLIT
+// BITS, GROUP: 4 with 64 or 128, 8 with 32 or 64.  A workgroup of KSPLIT * TPW wavefronts covers TPW consecutive row tiles, each split over KSPLIT
 // wavefronts along K; all of them share one staged copy of the activations.
 // WIDE: nine to sixteen activation rows.  The M dimension then has no empty half, so the two groups of a block are
 // kept apart with two products per word instead: one whose A operand carries the activations only where kq < 2, one
 // only where kq >= 2 (groups of 128 need neither: one product with the whole A operand).  Every lane then holds rows
 // 4 kq .. 4 kq + 3 of both groups' sums and applies both (scale, bias) words.
-template <int GROUP, int KSPLIT, int TPW, bool SBBF16, bool WIDE>
+template <int BITS, int GROUP, int KSPLIT, int TPW, bool SBBF16, bool WIDE>
 __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmArgs a) {
+    constexpr uint32_t BC = 512 / BITS;                     // codes per block: 64 bytes of a row
+    constexpr uint32_t XBYTES = BC * 2;                     // bytes of one activation row per block
+    constexpr uint32_t HALF = BC / 2;                       // codes of half a block: the run the staged sums cover
+    constexpr bool TWO = GROUP * 2 == (int)BC;              // a block holds two quantisation groups (else one)
+    static_assert((BITS == 4 || BITS == 8) && (TWO || GROUP == (int)BC), "4 bits: groups of 64 / 128; 8 bits: 32 / 64");
     constexpr uint32_t SXR = WIDE ? 16 : 8;                 // activation rows per run of 64 in the staged sums
     constexpr int WAVES = KSPLIT * TPW;
     constexpr int D = 4;                                    // blocks in flight per wavefront
@@ -73,7 +86,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
     const uint32_t n_in = lane & 15, kq = lane >> 4;
     const uint32_t part = blockIdx.y, wg = blockIdx.x;
     const uint32_t b0 = part * a.part_blocks;               // first block of this workgroup's K part
-    const uint32_t kp = a.part_blocks * 128;                // activation elements staged per row
+    const uint32_t kp = a.part_blocks * BC;                 // activation elements staged per row
 
     const uint32_t slice = wave % KSPLIT;
     struct Tile {
@@ -127,7 +140,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
     auto x_load = [&](uint32_t idx) -> u32x4 {
         uint32_t m, c;
         x_at(idx, m, c);
-        return *((const u32x4*)(a.x + (size_t)m * a.x_stride + (size_t)b0 * 128) + c);
+        return *((const u32x4*)(a.x + (size_t)m * a.x_stride + (size_t)b0 * BC) + c);
     };
     u32x4 xe[XB];
 #pragma unroll
@@ -147,8 +160,8 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
         r.w = __builtin_nontemporal_load((const u32x4*)(tile.lane_row + (size_t)b * 16 + piece * 4));
     };
     // (scale, bias) words, sixteen blocks of the wavefront's share at a time: this lane keeps those of blocks
-    // first + piece * 4 .. + 3 of the row it loads (one word per block and group of 64, so two for groups of 64)
-    constexpr int SZW = GROUP == 64 ? 2 : 1;
+    // first + piece * 4 .. + 3 of the row it loads (one word per group: two per block where a block holds two groups)
+    constexpr int SZW = TWO ? 2 : 1;
     uint32_t szr[4][SZW];
     auto issue_sz = [&](uint32_t first) {
 #pragma unroll
@@ -163,8 +176,10 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
     static_for<D>([&](auto J) { issue(tile.b_first + decltype(J)::value, ring[decltype(J)::value]); });
     issue_sz(tile.b_first);
 
-    // ---- 3. stage the activations: every run of eight as (x0,x4,x1,x5,x2,x6,x3,x7), and sum(x) per 64 and row ------
-    float* const sxs = (float*)(lds + (size_t)(a.m + 1) * a.lds_row_bytes);      // [run of 64 in part][SXR]
+    // ---- 3. stage the activations: every run of eight as (x0,x4,x1,x5,x2,x6,x3,x7) (8 bits: (x0,x2,x1,x3,x4,x6,x5,x7)),
+    //         and sum(x) per half block and row ----------------------------------------------------------------------
+    constexpr uint32_t CH = HALF / 8;                       // 16-byte chunks per half block
+    float* const sxs = (float*)(lds + (size_t)(a.m + 1) * a.lds_row_bytes);      // [half block in part][SXR]
     {
         auto stage = [&](uint32_t idx, const u32x4& v) {
             float p = pm_dot2(v.x, 0x3F803F80u, 0.0f);
@@ -173,16 +188,23 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
             p = pm_dot2(v.w, 0x3F803F80u, p);
             p += __shfl_xor(p, 1);
             p += __shfl_xor(p, 2);
-            p += __shfl_xor(p, 4);
+            if constexpr (CH == 8) p += __shfl_xor(p, 4);
             uint32_t m, c;
             if (x_at(idx, m, c)) {
                 u32x4 o;
-                o.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);    // (x0, x4)
-                o.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);    // (x1, x5)
-                o.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);    // (x2, x6)
-                o.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);    // (x3, x7)
+                if constexpr (BITS == 4) {
+                    o.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);    // (x0, x4)
+                    o.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);    // (x1, x5)
+                    o.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);    // (x2, x6)
+                    o.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);    // (x3, x7)
+                } else {
+                    o.x = __builtin_amdgcn_perm(v.y, v.x, 0x05040100u);    // (x0, x2)
+                    o.y = __builtin_amdgcn_perm(v.y, v.x, 0x07060302u);    // (x1, x3)
+                    o.z = __builtin_amdgcn_perm(v.w, v.z, 0x05040100u);    // (x4, x6)
+                    o.w = __builtin_amdgcn_perm(v.w, v.z, 0x07060302u);    // (x5, x7)
+                }
                 *((u32x4*)(lds + (size_t)m * a.lds_row_bytes) + c) = o;
-                if ((c & 7u) == 0) sxs[(c >> 3) * SXR + m] = p;     // eight chunks: one run of 64
+                if ((c & (CH - 1)) == 0) sxs[(c / CH) * SXR + m] = p;  // CH chunks: one half block
             }
         };
         // whole wavefronts take part in the shuffles of every step: the walk is rounded up to whole batches
@@ -219,9 +241,9 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
     const uint32_t xi = WIDE ? n_in : (n_in & 7u);
     const uint32_t xr = xi < a.m ? xi : a.m - 1;
     const bool live = WIDE ? (kq < 2) : (n_in >> 3) == (kq >> 1);
-    const char* const a_lane = lds + (size_t)(live || (WIDE && GROUP == 128) ? xr : a.m) * a.lds_row_bytes + kq * 64;
-    // WIDE, groups of 64: the second product's operand, live where the first one's is not
-    const char* const a_lane_hi = lds + (size_t)(live ? a.m : xr) * a.lds_row_bytes + kq * 64;
+    const char* const a_lane = lds + (size_t)(live || (WIDE && !TWO) ? xr : a.m) * a.lds_row_bytes + kq * (XBYTES / 4);
+    // WIDE, two groups per block: the second product's operand, live where the first one's is not
+    const char* const a_lane_hi = lds + (size_t)(live ? a.m : xr) * a.lds_row_bytes + kq * (XBYTES / 4);
 
     auto unpack = [&](uint32_t w) -> pm_bf16x8_t {
         u32x4 p;
@@ -231,12 +253,26 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
         p.w = ((w >> 12) & k_mask) | k_magic;
         return __builtin_bit_cast(pm_bf16x8_t, p);
     };
+    // 8 bits: the low (SH = 0) or high (SH = 4) nibbles of the eight codes of two words, in the order c0,c2,c1,c3 of each
+    auto unpack8 = [&](uint32_t wa, uint32_t wb, auto SH) -> pm_bf16x8_t {
+        constexpr int sh = decltype(SH)::value;
+        u32x4 p;
+        p.x = ((wa >> sh) & k_mask) | k_magic;
+        p.y = ((wa >> (8 + sh)) & k_mask) | k_magic;
+        p.z = ((wb >> sh) & k_mask) | k_magic;
+        p.w = ((wb >> (8 + sh)) & k_mask) | k_magic;
+        return __builtin_bit_cast(pm_bf16x8_t, p);
+    };
+    using Lo = std::integral_constant<int, 0>;
+    using Hi = std::integral_constant<int, 4>;
+    // sum (128 + q) x for 4 bits; for 8 bits sum (128 + l) x + 16 sum (128 + h) x: the offset the affine form takes back
+    constexpr float kOffset = BITS == 4 ? 128.0f : 128.0f * 17.0f;
     // this lane's D rows 4 kq .. 4 kq + 3 are activation rows 4 (kq & 1) .. + 3
     const uint32_t sx_lane = WIDE ? 4 * kq : (kq >> 1) * 8 + 4 * (kq & 1);
     const int from_lane = (int)((4u * n_in + kq) * 4u);     // byte address of the lane that loaded (row n, piece kq)
     auto compute = [&](uint32_t b, const Rec& r, const uint32_t (&sz_pair)[SZW], uint32_t sz_piece) {
         const uint32_t bl = b - b0;                          // block inside the staged columns
-        const char* ab = a_lane + (size_t)bl * 256;          // 128 codes = 256 bytes of activations
+        const char* ab = a_lane + (size_t)bl * XBYTES;       // this block's activations
         // every LDS operation of the block goes out first: the cross-lane reads, the A operands, sum(x) over this lane
         // half's run of 64 (runs 2 bl and 2 bl + 1 of the part): a group of 64, or half of a group of 128 whose other
         // half the other lanes add
@@ -253,15 +289,59 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
             if constexpr (!WIDE) szw = kq >> 1 ? szw_hi : szw;
         }
         const pm_bf16x8_t a0 = *(const pm_bf16x8_t*)(ab), a1 = *(const pm_bf16x8_t*)(ab + 16);
-        const pm_bf16x8_t a2 = *(const pm_bf16x8_t*)(ab + 32), a3 = *(const pm_bf16x8_t*)(ab + 48);
+        pm_bf16x8_t a2 = a0, a3 = a1;                       // (8 bits: a lane's share of a block is two operands)
+        if constexpr (BITS == 4) { a2 = *(const pm_bf16x8_t*)(ab + 32); a3 = *(const pm_bf16x8_t*)(ab + 48); }
         const pm_floatx4_t sx = *(const pm_floatx4_t*)(sxs + (size_t)bl * 2 * SXR + sx_lane);
         auto scale_zero = [&](uint32_t word, float& sc, float& zc) {
             float zr;
             if constexpr (SBBF16) { sc = __uint_as_float(word << 16); zr = __uint_as_float(word & 0xFFFF0000u); }
             else { sc = f16_to_f32((uint16_t)(word & 0xFFFFu)); zr = f16_to_f32((uint16_t)(word >> 16)); }
-            zc = zr - 128.0f * sc;
+            zc = zr - kOffset * sc;
         };
-        if constexpr (!WIDE) {
+        if constexpr (BITS == 8) {
+            // products over the low and the high nibbles share the A operands; WIDE with two groups per block: each
+            // against both masked operands
+            const pm_bf16x8_t l0 = unpack8(w0, w1, Lo{}), l1 = unpack8(w2, w3, Lo{});
+            const pm_bf16x8_t h0 = unpack8(w0, w1, Hi{}), h1 = unpack8(w2, w3, Hi{});
+            if constexpr (!(WIDE && TWO)) {
+                pm_floatx4_t sxv = sx;
+                if constexpr (WIDE) {
+                    const pm_floatx4_t sx_hi = *(const pm_floatx4_t*)(sxs + (size_t)(bl * 2 + 1) * SXR + sx_lane);
+                    sxv += sx_hi;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                pm_floatx4_t dl = zero4, dh = zero4;
+                dl = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, l0, dl, 0, 0, 0);
+                dh = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, h0, dh, 0, 0, 0);
+                dl = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, l1, dl, 0, 0, 0);
+                dh = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, h1, dh, 0, 0, 0);
+                float sc, zc;
+                scale_zero(szw, sc, zc);
+#pragma unroll
+                for (int q = 0; q < MR; q++) acc[q] += sc * __builtin_fmaf(16.0f, dh[q], dl[q]) + zc * sxv[q];
+            } else {
+                const pm_floatx4_t sx_hi = *(const pm_floatx4_t*)(sxs + (size_t)(bl * 2 + 1) * SXR + sx_lane);
+                const char* ah = a_lane_hi + (size_t)bl * XBYTES;
+                const pm_bf16x8_t g0 = *(const pm_bf16x8_t*)(ah), g1 = *(const pm_bf16x8_t*)(ah + 16);
+                __builtin_amdgcn_sched_barrier(0);
+                pm_floatx4_t dl = zero4, dh = zero4, el = zero4, eh = zero4;
+                dl = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, l0, dl, 0, 0, 0);
+                dh = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, h0, dh, 0, 0, 0);
+                el = __builtin_amdgcn_mfma_f32_16x16x32_bf16(g0, l0, el, 0, 0, 0);
+                eh = __builtin_amdgcn_mfma_f32_16x16x32_bf16(g0, h0, eh, 0, 0, 0);
+                dl = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, l1, dl, 0, 0, 0);
+                dh = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1, h1, dh, 0, 0, 0);
+                el = __builtin_amdgcn_mfma_f32_16x16x32_bf16(g1, l1, el, 0, 0, 0);
+                eh = __builtin_amdgcn_mfma_f32_16x16x32_bf16(g1, h1, eh, 0, 0, 0);
+                float s0, z0, s1, z1;
+                scale_zero(szw, s0, z0);
+                scale_zero(szw_hi, s1, z1);
+#pragma unroll
+                for (int q = 0; q < MR; q++)
+                    acc[q] += (s0 * __builtin_fmaf(16.0f, dh[q], dl[q]) + z0 * sx[q]) +
+                              (s1 * __builtin_fmaf(16.0f, eh[q], el[q]) + z1 * sx_hi[q]);
+            }
+        } else if constexpr (!WIDE) {
             __builtin_amdgcn_sched_barrier(0);
             pm_floatx4_t d = zero4;
             d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, unpack(w0), d, 0, 0, 0);
@@ -275,7 +355,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
         } else {
             const pm_floatx4_t sx_hi = *(const pm_floatx4_t*)(sxs + (size_t)(bl * 2 + 1) * SXR + sx_lane);
             const pm_bf16x8_t b0 = unpack(w0), b1 = unpack(w1), b2 = unpack(w2), b3 = unpack(w3);
-            if constexpr (GROUP == 128) {
+            if constexpr (!TWO) {
                 __builtin_amdgcn_sched_barrier(0);
                 pm_floatx4_t d = zero4;
                 d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0, b0, d, 0, 0, 0);
@@ -287,7 +367,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
 #pragma unroll
                 for (int q = 0; q < MR; q++) acc[q] += sc * d[q] + zc * (sx[q] + sx_hi[q]);
             } else {
-                const char* ah = a_lane_hi + (size_t)bl * 256;
+                const char* ah = a_lane_hi + (size_t)bl * XBYTES;
                 const pm_bf16x8_t h0 = *(const pm_bf16x8_t*)(ah), h1 = *(const pm_bf16x8_t*)(ah + 16);
                 const pm_bf16x8_t h2 = *(const pm_bf16x8_t*)(ah + 32), h3 = *(const pm_bf16x8_t*)(ah + 48);
                 __builtin_amdgcn_sched_barrier(0);
@@ -313,7 +393,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
     // Partial tiles of the WAVES wavefronts, [WAVES][MR][64]: a single pass writes them over the staged activations
     // once every wavefront is done reading those; several passes keep them behind the activations and their sums.
     const bool red_over_x = a.passes == 1;
-    float* const red = (float*)(red_over_x ? lds : lds + (size_t)(a.m + 1) * a.lds_row_bytes + (size_t)(kp / 64) * SXR * 4);
+    float* const red = (float*)(red_over_x ? lds : lds + (size_t)(a.m + 1) * a.lds_row_bytes + (size_t)(kp / HALF) * SXR * 4);
     for (uint32_t pass = 0; pass < a.passes; pass++) {
         if (pass) {                                            // the first tile's loads were issued before staging
             tile = select_tile(pass);
@@ -378,12 +458,12 @@ __global__ __launch_bounds__(256) void pm_sum_parts_kernel(const float* __restri
 
 namespace {
 
-template <int GROUP, int KSPLIT, int TPW>
+template <int BITS, int GROUP, int KSPLIT, int TPW>
 mi355q_status launch_pm(hipStream_t s, const PmArgs& a, uint32_t grid, size_t lds) {
-    auto kern = a.m > 8 ? (a.sb_dtype == MI355Q_BF16 ? gemv_mfma_planes_kernel<GROUP, KSPLIT, TPW, true, true>
-                                                     : gemv_mfma_planes_kernel<GROUP, KSPLIT, TPW, false, true>)
-                        : (a.sb_dtype == MI355Q_BF16 ? gemv_mfma_planes_kernel<GROUP, KSPLIT, TPW, true, false>
-                                                     : gemv_mfma_planes_kernel<GROUP, KSPLIT, TPW, false, false>);
+    auto kern = a.m > 8 ? (a.sb_dtype == MI355Q_BF16 ? gemv_mfma_planes_kernel<BITS, GROUP, KSPLIT, TPW, true, true>
+                                                     : gemv_mfma_planes_kernel<BITS, GROUP, KSPLIT, TPW, false, true>)
+                        : (a.sb_dtype == MI355Q_BF16 ? gemv_mfma_planes_kernel<BITS, GROUP, KSPLIT, TPW, true, false>
+                                                     : gemv_mfma_planes_kernel<BITS, GROUP, KSPLIT, TPW, false, false>);
     if (lds > 64 * 1024)
         MI355Q_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     kern<<<dim3(grid, a.parts), dim3(KSPLIT * TPW * 64), lds, s>>>(a);
@@ -391,20 +471,20 @@ mi355q_status launch_pm(hipStream_t s, const PmArgs& a, uint32_t grid, size_t ld
     return MI355Q_OK;
 }
 
-template <int GROUP>
+template <int BITS, int GROUP>
 mi355q_status launch_pm_shape(hipStream_t s, const PmArgs& a, const Tile16LaunchShape& g) {
     const uint32_t ks = g.ksplit, tpw = g.tiles_per_wg;
-    if (ks == 4 && tpw == 1) return launch_pm<GROUP, 4, 1>(s, a, g.wgs_per_part, g.lds_bytes);
-    if (ks == 4 && tpw == 2) return launch_pm<GROUP, 4, 2>(s, a, g.wgs_per_part, g.lds_bytes);
-    if (ks == 4 && tpw == 3) return launch_pm<GROUP, 4, 3>(s, a, g.wgs_per_part, g.lds_bytes);
-    if (ks == 4 && tpw == 4) return launch_pm<GROUP, 4, 4>(s, a, g.wgs_per_part, g.lds_bytes);
-    if (ks == 2 && tpw == 5) return launch_pm<GROUP, 2, 5>(s, a, g.wgs_per_part, g.lds_bytes);
-    if (ks == 2 && tpw == 6) return launch_pm<GROUP, 2, 6>(s, a, g.wgs_per_part, g.lds_bytes);
-    if (ks == 2 && tpw == 7) return launch_pm<GROUP, 2, 7>(s, a, g.wgs_per_part, g.lds_bytes);
-    if (ks == 2 && tpw == 8) return launch_pm<GROUP, 2, 8>(s, a, g.wgs_per_part, g.lds_bytes);
-    if (ks == 8 && tpw == 1) return launch_pm<GROUP, 8, 1>(s, a, g.wgs_per_part, g.lds_bytes);
-    if (ks == 8 && tpw == 2) return launch_pm<GROUP, 8, 2>(s, a, g.wgs_per_part, g.lds_bytes);
-    if (ks == 16 && tpw == 1) return launch_pm<GROUP, 16, 1>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 4 && tpw == 1) return launch_pm<BITS, GROUP, 4, 1>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 4 && tpw == 2) return launch_pm<BITS, GROUP, 4, 2>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 4 && tpw == 3) return launch_pm<BITS, GROUP, 4, 3>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 4 && tpw == 4) return launch_pm<BITS, GROUP, 4, 4>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 2 && tpw == 5) return launch_pm<BITS, GROUP, 2, 5>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 2 && tpw == 6) return launch_pm<BITS, GROUP, 2, 6>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 2 && tpw == 7) return launch_pm<BITS, GROUP, 2, 7>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 2 && tpw == 8) return launch_pm<BITS, GROUP, 2, 8>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 8 && tpw == 1) return launch_pm<BITS, GROUP, 8, 1>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 8 && tpw == 2) return launch_pm<BITS, GROUP, 8, 2>(s, a, g.wgs_per_part, g.lds_bytes);
+    if (ks == 16 && tpw == 1) return launch_pm<BITS, GROUP, 16, 1>(s, a, g.wgs_per_part, g.lds_bytes);
     return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no matrix-core planes variant for K-split %u x %u tiles per workgroup", ks, tpw);
 }
 
@@ -416,20 +496,25 @@ mi355q_status launch_pm_shape(hipStream_t s, const PmArgs& a, const Tile16Launch
 bool gemv_mfma_planes_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
     if (w.layout != MI355Q_LAYOUT_PLANES || !w.sz || x_dtype != MI355Q_BF16) return false;
     if (m < 2 || m > 16) return false;
-    if (w.bits != 4 || (w.group != 64 && w.group != 128) || w.k % 128) return false;
+    if (w.bits != 4 && w.bits != 8) return false;
+    const uint32_t bc = 512 / w.bits;                                     // codes per block
+    if ((w.group != bc && w.group * 2 != bc) || w.k % bc) return false;
     if (x_stride % 8) return false;                                       // 128-bit activation loads
     // a row is one stream: its sz words follow its code words at the same pitch; code words 16-byte aligned
     if (w.sz_stride != w.code_stride || w.code_stride % 4 || (uintptr_t)w.codes % 16) return false;
     if (w.sz < w.codes || (size_t)(w.sz - w.codes) >= w.code_stride || (w.sz - w.codes) % 2) return false;
-    return gemv_tile16_parts_for(w.k, m + 1, (w.n + 15) / 16, 256) != 0;
+    return gemv_tile16_parts_for(w.k * (w.bits / 4), m + 1, (w.n + 15) / 16, 256) != 0;
 }
 
 uint32_t gemv_mfma_planes_k_parts(const mi355q_context* ctx, const WView& w, uint32_t m) {
-    return gemv_tile16_parts_for(w.k, m + 1, (w.n + 15) / 16, (uint32_t)ctx->props.multiProcessorCount);
+    return gemv_tile16_parts_for(w.k * (w.bits / 4), m + 1, (w.n + 15) / 16, (uint32_t)ctx->props.multiProcessorCount);
 }
 
-Tile16LaunchShape gemv_mfma_planes_shape(const mi355q_context* ctx, uint32_t n_row_tiles, uint32_t k_total, uint32_t m) {
-    return gemv_tile16_shape(ctx, n_row_tiles, k_total, m + 1);
+// 8-bit rows are shaped as 4-bit rows of as many bytes (the same blocks; the staged activations take half the room
+// that shape reserves).
+Tile16LaunchShape gemv_mfma_planes_shape(const mi355q_context* ctx, uint32_t n_row_tiles, uint32_t k_total, uint32_t bits,
+                                         uint32_t m) {
+    return gemv_tile16_shape(ctx, n_row_tiles, k_total * (bits / 4), m + 1);
 }
 
 mi355q_status launch_gemv_mfma_planes_multi(hipStream_t s, mi355q_context* ctx, uint32_t count, const WView* w,
@@ -449,19 +534,20 @@ mi355q_status launch_gemv_mfma_planes_multi(hipStream_t s, mi355q_context* ctx, 
         a.seg_rows[i] = w[j].n;
         a.tile_end[i] = tiles;
         if (w[j].code_stride != w[0].code_stride || (w[j].sz - w[j].codes) != (w[0].sz - w[0].codes) ||
-            w[j].k != w[0].k || w[j].group != w[0].group || w[j].sb_dtype != w[0].sb_dtype)
-            return fail(MI355Q_ERR_SHAPE, "fused projections must share K, group size, row pitch and scale type");
+            w[j].k != w[0].k || w[j].bits != w[0].bits || w[j].group != w[0].group || w[j].sb_dtype != w[0].sb_dtype)
+            return fail(MI355Q_ERR_SHAPE, "fused projections must share K, format, row pitch and scale type");
     }
-    const Tile16LaunchShape g = gemv_mfma_planes_shape(ctx, tiles, w[0].k, m);
+    const Tile16LaunchShape g = gemv_mfma_planes_shape(ctx, tiles, w[0].k, w[0].bits, m);
+    const uint32_t bc = 512 / w[0].bits;
     a.x = (const uint16_t*)x;
     a.k = w[0].k; a.m = m; a.x_stride = x_stride;
     a.row_words = w[0].code_stride;
     a.sz_offset = (uint32_t)(w[0].sz - w[0].codes);
     a.parts = g.parts;
-    a.part_blocks = w[0].k / 128 / g.parts;
+    a.part_blocks = w[0].k / bc / g.parts;
     a.blocks_per_wave = g.blocks_per_wave;
     a.passes = g.passes;
-    a.lds_row_bytes = a.part_blocks * 256 + 16;
+    a.lds_row_bytes = a.part_blocks * bc * 2 + 16;
     if (g.parts > 1) {
         if (count != 1)
             return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "rows of %u codes at M = %u are split over K parts: one matrix per launch",
@@ -470,7 +556,8 @@ mi355q_status launch_gemv_mfma_planes_multi(hipStream_t s, mi355q_context* ctx, 
         a.partial = (float*)ctx->workspace;
     }
     a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = w[0].sb_dtype;
-    const mi355q_status st = w[0].group == 64 ? launch_pm_shape<64>(s, a, g) : launch_pm_shape<128>(s, a, g);
+    const mi355q_status st = w[0].bits == 4 ? (w[0].group == 64 ? launch_pm_shape<4, 64>(s, a, g) : launch_pm_shape<4, 128>(s, a, g))
+                                            : (w[0].group == 32 ? launch_pm_shape<8, 32>(s, a, g) : launch_pm_shape<8, 64>(s, a, g));
     if (st != MI355Q_OK || g.parts == 1) return st;
     uint32_t sum_wgs = (w[0].n + 255) / 256;
     if (sum_wgs > 65535u) sum_wgs = 65535u;

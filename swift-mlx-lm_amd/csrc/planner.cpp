@@ -62,9 +62,9 @@ void plan_small_m(const mi355q_weight* w, uint32_t m, int x_dtype, uint32_t x_st
         s->block[0] = g.block;
         s->lds_bytes = g.lds_bytes;
         s->rows_per_workgroup = 16;
-    } else if (!forced && m >= kMfmaPlanesMinRows && gemv_mfma_planes_eligible(v, x_dtype, m > 16 ? 16 : m, x_stride)) {
+    } else if (!forced && m >= mfma_planes_min_rows(v.bits) && gemv_mfma_planes_eligible(v, x_dtype, m > 16 ? 16 : m, x_stride)) {
         const Tile16LaunchShape g = gemv_mfma_planes_shape(w->ctx, (uint32_t)((w->n + 15) / 16), (uint32_t)w->k,
-                                                           m > 16 ? 16 : m);
+                                                           (uint32_t)w->fmt.bits, m > 16 ? 16 : m);
         std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_mfma_planes_q%u_g%u", (unsigned)w->fmt.bits,
                       w->fmt.group_size);
         s->grid[0] = g.wgs_per_part;
@@ -116,17 +116,17 @@ void plan_shared_launch_shape(const mi355q_weight* const* ws, uint32_t count, ui
                               mi355q_step* s) {
     WView all = ws[0]->view();
     uint64_t total = 0;
-    // four rows and more: the matrix-core kernel over the planes takes the rows of all matrices, in 16-row tiles
-    bool on_planes = m >= kMfmaPlanesMinRows && m <= 16;
+    // four rows and more (three at 8 bits): the matrix-core kernel over the planes takes the rows of all matrices, in 16-row tiles
+    bool on_planes = m >= mfma_planes_min_rows(all.bits) && m <= 16;
     uint32_t tiles = 0;
     for (uint32_t i = 0; i < count && on_planes; i++) {
         const WView v = ws[i]->view();
         on_planes = gemv_mfma_planes_eligible(v, x_dtype, m, x_stride) && gemv_mfma_planes_k_parts(ws[0]->ctx, v, m) == 1 &&
-                    v.sb_dtype == all.sb_dtype && v.code_stride == all.code_stride && v.group == all.group;
+                    v.sb_dtype == all.sb_dtype && v.code_stride == all.code_stride && v.group == all.group && v.bits == all.bits;
         tiles += (v.n + 15) / 16;
     }
     if (on_planes) {
-        const Tile16LaunchShape g = gemv_mfma_planes_shape(ws[0]->ctx, tiles, all.k, m);
+        const Tile16LaunchShape g = gemv_mfma_planes_shape(ws[0]->ctx, tiles, all.k, all.bits, m);
         s->grid[0] = g.wgs_per_part;
         s->grid[1] = g.parts;
         s->block[0] = g.block;

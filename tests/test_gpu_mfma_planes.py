@@ -1,5 +1,6 @@
-"""GPU parity tests of the small-batch matrix-core kernel over the split planes (4-bit, groups of 64 and 128), through
-the C ABI: the projections of gemv_q4_g64 / gemm_q4_g64 of the reference
+"""GPU parity tests of the small-batch matrix-core kernel over the split planes (4-bit codes in groups of 64 and 128,
+8-bit codes in groups of 32 and 64), through the C ABI: the projections of gemv_q4_g64 / gemm_q4_g64 and
+gemv_q8_g32 / gemm_q8_g32 of the reference
 (MetalSourceGenerator+Quantized.swift:496-575, :22-156) for 4 <= M <= 16 rows per launch on the layout that serves M = 1
 (up to eight rows the two quantisation groups of a block are kept apart in the M dimension, above with two products).
 
@@ -23,43 +24,46 @@ def say(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def _fmt(pkg, group=64):
-    return pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, group)
+def _fmt(pkg, group=64, bits=4):
+    return pkg.QuantizationFormatRegistry.format_for_mlx_quantization(bits, group)
 
 
-@pytest.mark.parametrize("group", [64, 128])
-def test_mfma_planes_seeded_shapes(pkg, ctx, group):
-    """Ragged row counts (tiles of sixteen rows end inside the matrix), one block of 128 codes up to rows of 14336
-    (sixteen wavefronts a tile), every M the kernel takes; the plan record names it."""
-    for i, (n, k) in enumerate([(96, 512), (200, 1024), (33, 128), (17, 256), (64, 14336), (4100, 4096)]):
-        words, s, z, wq = seeded_case(4100 + i + group, n, k, 4, group)
-        w = ctx.weight_prepare_mlx(_fmt(pkg, group), words, s, z, pkg.BF16, pkg.LAYOUT_PLANES)
-        for m in ((4, 5, 6, 7, 8, 9, 11, 13, 16) if n < 4000 else (4, 8, 16)):
-            say(f"mfma planes g{group} {k}->{n} M={m}")
+@pytest.mark.parametrize("bits,group", [(4, 64), (4, 128), (8, 32), (8, 64)])
+def test_mfma_planes_seeded_shapes(pkg, ctx, bits, group):
+    """Ragged row counts (tiles of sixteen rows end inside the matrix), one block (64 bytes of a row) up to rows of
+    14336 codes (sixteen wavefronts a tile), every M the kernel takes; the plan record names it."""
+    for i, (n, k) in enumerate([(96, 512), (200, 1024), (33, 128), (17, 256), (64, 14336), (4100, 4096), (40, 64 * 8 // bits * 3)]):
+        words, s, z, wq = seeded_case(4100 + i + group + bits, n, k, bits, group)
+        w = ctx.weight_prepare_mlx(_fmt(pkg, group, bits), words, s, z, pkg.BF16, pkg.LAYOUT_PLANES)
+        for m in (((4, 5, 6, 7, 8, 9, 11, 13, 16) if n < 4000 else (4, 8, 16)) + ((3,) if bits == 8 else ())):
+            say(f"mfma planes q{bits} g{group} {k}->{n} M={m}")
             x = act_rounded(kat.seeded_activations(4200 + m, m, k), pkg.BF16, pkg)
             st = w.plan_decode_step(m) if m <= 8 else w.plan_prefill_steps(m)[0]
-            assert st.device_kernel == f"gemv_mfma_planes_q4_g{group}" and not st.used_fallback
+            assert st.device_kernel == f"gemv_mfma_planes_q{bits}_g{group}" and not st.used_fallback
             y32 = run_gemv(ctx, pkg, w, x, pkg.BF16, pkg.F32, use_qgemm=m > 8)
-            assert_within_tolerance(y32, oracle.gemm_f64(wq, x), f"g{group} {k}->{n} M={m}")
+            assert_within_tolerance(y32, oracle.gemm_f64(wq, x), f"q{bits} g{group} {k}->{n} M={m}")
             ybf = run_gemv(ctx, pkg, w, x, pkg.BF16, pkg.BF16, use_qgemm=m > 8)
             assert np.array_equal(oracle.bf16_from_f32(ybf), oracle.bf16_from_f32(y32))
-        for m in (2, 3):                                        # below the threshold: the dot-product kernels
-            assert w.plan_decode_step(m).device_kernel != f"gemv_mfma_planes_q4_g{group}"
+        for m in ((2, 3) if bits == 4 else (2,)):               # below the threshold: the dot-product kernels
+            assert w.plan_decode_step(m).device_kernel != f"gemv_mfma_planes_q{bits}_g{group}"
         w.destroy()
 
 
-def test_mfma_planes_exact_small_integers_f16_scales_and_strides(pkg, ctx):
-    """Exactly representable case: every partial sum an integer multiple of 2^-6 below 2^20, so the result is exact
-    whatever the order of the sums; planes made from STAF blocks (f16 scale words) and from MLX planes (bf16); padded
-    activation and output rows."""
-    rng = np.random.default_rng(4300)
+@pytest.mark.parametrize("bits,group", [(4, 64), (8, 32), (8, 64)])
+def test_mfma_planes_exact_small_integers_f16_scales_and_strides(pkg, ctx, bits, group):
+    """Exactly representable case: every product and partial sum (those of the offset codes included: 128 + q, and for
+    8 bits 128 + l and 16 (128 + h)) is a multiple of 2^-6 that fits 24 bits, so the result is exact whatever the order
+    of the sums; planes made from STAF blocks (f16 scale words) and from MLX planes (bf16); padded activation and
+    output rows."""
+    rng = np.random.default_rng(4300 + bits + group)
     n, k = 100, 1024
-    codes = rng.integers(0, 16, (n, k), dtype=np.uint8)
-    scales = rng.choice([0.125, 0.25, 0.5], (n, k // 64)); zeros = rng.integers(-4, 5, (n, k // 64)) * 0.25
-    case = Case(4, 64, codes, scales, zeros)
-    wq = scales.repeat(64, axis=1) * codes + zeros.repeat(64, axis=1)
-    for name, w in (("f16", ctx.weight_prepare_staf(_fmt(pkg), n, k, case.staf_blocks(), pkg.LAYOUT_PLANES)),
-                    ("bf16", ctx.weight_prepare_mlx(_fmt(pkg), *case.planes(pkg.BF16, pkg), pkg.BF16, pkg.LAYOUT_PLANES))):
+    codes = rng.integers(0, 1 << bits, (n, k), dtype=np.uint8)
+    scales = rng.choice([0.125, 0.25, 0.5], (n, k // group)); zeros = rng.integers(-4, 5, (n, k // group)) * 0.25
+    case = Case(bits, group, codes, scales, zeros)
+    wq = scales.repeat(group, axis=1) * codes + zeros.repeat(group, axis=1)
+    fmt = _fmt(pkg, group, bits)
+    for name, w in (("f16", ctx.weight_prepare_staf(fmt, n, k, case.staf_blocks(), pkg.LAYOUT_PLANES)),
+                    ("bf16", ctx.weight_prepare_mlx(fmt, *case.planes(pkg.BF16, pkg), pkg.BF16, pkg.LAYOUT_PLANES))):
         for m, xpad, ypad in ((4, 0, 0), (5, 8, 0), (8, 16, 12), (12, 8, 4), (16, 0, 0)):
             x = np.full((m, k + xpad), 512.0, np.float32)
             x[:, :k] = rng.integers(-8, 9, (m, k)).astype(np.float32) * 0.125
@@ -76,11 +80,12 @@ def test_mfma_planes_exact_small_integers_f16_scales_and_strides(pkg, ctx):
 
 def test_mfma_planes_batched_projections_one_launch(pkg, ctx):
     """q+k+v and gate+up at 4 <= M <= 8 share one launch on the planes: identical bits to the separate launches."""
-    for ns, k in [((1024, 256, 256), 1024), ((1400, 1400), 512), ((5, 17, 130), 256)]:
+    for ns, k, bits, group in [((1024, 256, 256), 1024, 4, 64), ((1400, 1400), 512, 4, 64), ((5, 17, 130), 256, 4, 64),
+                               ((1024, 256, 256), 1024, 8, 32), ((300, 700), 448, 8, 64)]:
         ws, wqs = [], []
         for i, n in enumerate(ns):
-            words, s, z, wq = seeded_case(4400 + i + n % 13, n, k, 4, 64)
-            ws.append(ctx.weight_prepare_mlx(_fmt(pkg), words, s, z, pkg.BF16, pkg.LAYOUT_PLANES)); wqs.append(wq)
+            words, s, z, wq = seeded_case(4400 + i + n % 13, n, k, bits, group)
+            ws.append(ctx.weight_prepare_mlx(_fmt(pkg, group, bits), words, s, z, pkg.BF16, pkg.LAYOUT_PLANES)); wqs.append(wq)
         for m in (4, 7, 8, 10, 16):
             x = act_rounded(kat.seeded_activations(4500 + m, m, k), pkg.BF16, pkg)
             xd = ctx.upload(oracle.bf16_from_f32(x).reshape(x.shape))
