@@ -190,8 +190,10 @@ bool gemv_tile16_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_st
 // K parts a launch of M rows takes: 1 = whole rows (needed by fused q+k+v / gate+up launches and by the fused head)
 uint32_t gemv_tile16_k_parts(const mi355q_context* ctx, const WView& w, uint32_t m);
 // the same for a shape: 0 when no power-of-two split of K leaves M staged rows inside LDS
-uint32_t gemv_tile16_parts_for(uint32_t k, uint32_t m, uint32_t n_row_tiles, uint32_t cus);
-Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_row_tiles, uint32_t k, uint32_t m);
+// block_codes: codes in 64 bytes of a weight row (128 at 4 bits)
+uint32_t gemv_tile16_parts_for(uint32_t k, uint32_t m, uint32_t n_row_tiles, uint32_t cus, uint32_t block_codes = 128);
+Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_row_tiles, uint32_t k, uint32_t m,
+                                    uint32_t block_codes = 128);
 mi355q_status launch_gemv_tile16_multi(hipStream_t s, mi355q_context* ctx, uint32_t count, const WView* w,
                                        const void* x, void* const* y, const uint32_t* y_strides, int y_dtype,
                                        uint32_t m, uint32_t x_stride, float* logits_f32, int32_t* token_out,

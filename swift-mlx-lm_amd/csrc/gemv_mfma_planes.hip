@@ -503,18 +503,16 @@ bool gemv_mfma_planes_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t
     // a row is one stream: its sz words follow its code words at the same pitch; code words 16-byte aligned
     if (w.sz_stride != w.code_stride || w.code_stride % 4 || (uintptr_t)w.codes % 16) return false;
     if (w.sz < w.codes || (size_t)(w.sz - w.codes) >= w.code_stride || (w.sz - w.codes) % 2) return false;
-    return gemv_tile16_parts_for(w.k * (w.bits / 4), m + 1, (w.n + 15) / 16, 256) != 0;
+    return gemv_tile16_parts_for(w.k, m + 1, (w.n + 15) / 16, 256, bc) != 0;
 }
 
 uint32_t gemv_mfma_planes_k_parts(const mi355q_context* ctx, const WView& w, uint32_t m) {
-    return gemv_tile16_parts_for(w.k * (w.bits / 4), m + 1, (w.n + 15) / 16, (uint32_t)ctx->props.multiProcessorCount);
+    return gemv_tile16_parts_for(w.k, m + 1, (w.n + 15) / 16, (uint32_t)ctx->props.multiProcessorCount, 512 / w.bits);
 }
 
-// 8-bit rows are shaped as 4-bit rows of as many bytes (the same blocks; the staged activations take half the room
-// that shape reserves).
 Tile16LaunchShape gemv_mfma_planes_shape(const mi355q_context* ctx, uint32_t n_row_tiles, uint32_t k_total, uint32_t bits,
                                          uint32_t m) {
-    return gemv_tile16_shape(ctx, n_row_tiles, k_total * (bits / 4), m + 1);
+    return gemv_tile16_shape(ctx, n_row_tiles, k_total, m + 1, 512 / bits);
 }
 
 mi355q_status launch_gemv_mfma_planes_multi(hipStream_t s, mi355q_context* ctx, uint32_t count, const WView* w,

@@ -21,6 +21,26 @@
 
 namespace mi355q {
 
+// 3-bit codes with bf16 arithmetic, used where they lie.  A field whose lowest bit is bit a <= 4 of its half-word
+// stays inside the mantissa of the magic 0x4300, so (w & mask) | magic is the bf16 pair (128 + 2^a0 q0, 128 + 2^a1 q1)
+// with no shift; the activations are staged multiplied by 2^-a (exact), and
+//   sum (128 + 2^a q) (2^-a x) = sum q x + 128 sum 2^-a x,
+// the last sum computed once at staging.  One shift then serves every field it brings to a <= 4.  The 32 codes of a
+// lane chunk (three words) pair up as in the table below: thirteen pairs from eight shifts of the three words, one pair
+// from the outer half-words of words 0 and 2 (one byte permute), and the codes that straddle a half-word or word
+// boundary from two funnel shifts, which bring 5 and 10, 21 and 26 to bits 1 and 16: 27 instructions for 16 pairs
+// where extracting code by code took about 4 per pair more (4096 -> 14336: 8.4 -> 7.75 us).  (2-bit codes gain
+// nothing from the same treatment -- two shifts instead of seven per word, measured 7.6 us either way -- and pay for
+// the scaled staging: they keep their shifts.)
+struct InplacePair { int e0, a0, e1, a1; };                 // chunk elements of the low and high half, their bit positions
+__host__ __device__ constexpr InplacePair inplace_pair3(int i) {
+    constexpr InplacePair t[16] = {{1, 3, 6, 2},   {2, 3, 7, 2},   {3, 3, 8, 2},   {4, 3, 9, 2},      // word 0 >> 0, 3, 6, 9
+                                   {11, 1, 16, 0}, {12, 4, 17, 3}, {13, 1, 18, 0}, {14, 4, 19, 3},    // word 1 >> 0, 0, 6, 6
+                                   {15, 1, 20, 0}, {22, 2, 28, 4}, {23, 2, 29, 4}, {24, 2, 30, 4},    // word 1 >> 12; word 2 >> 0, 3, 6
+                                   {25, 2, 31, 4}, {0, 0, 27, 1},  {5, 1, 10, 0},  {21, 1, 26, 0}};   // word 2 >> 9; permute; funnel shifts
+    return t[i & 15];
+}
+
 // XA = 0: bf16 activations, bf16 code pairs (128 + q).  XA = 1: f16 activations, f16 code pairs (1024 + mult q,
 // fields of 2- and 4-bit codes used where they sit in the half-word, see f16_classes).
 template <int BITS, int GROUP, int NCT, int BR, int WAVES, int XA, bool SBBF16, bool ARGMAX>
@@ -34,8 +54,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_rows_kernel(GemvArgs a) {
     constexpr bool SMALL_FIELD = BITS == 3 || BITS == 5 || BITS == 6;
     constexpr bool DOT2 = XA == 1 || G::PAIRS || SMALL_FIELD;
     constexpr bool MULTI = XA == 1 && G::PAIRS;
+    constexpr bool INPLACE = XA == 0 && BITS == 3;                        // see inplace_pair3
+    static_assert(!INPLACE || CPL <= GROUP, "fields used in place: one group per lane chunk");
     constexpr int NCLS = MULTI ? f16_classes<BITS>() : 1;
-    constexpr int NF = MULTI ? 2 : 1;
+    constexpr int NF = MULTI || INPLACE ? 2 : 1;
     constexpr float OFS = XA == 1 ? 1024.0f : DOT2 ? 128.0f : 0.0f;
     static_assert(BR == 1 || BR == 2 || BR == 4 || BR == 8, "rows per pass: a power of two up to 8");
 
@@ -106,12 +128,25 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_rows_kernel(GemvArgs a) {
     auto stage_store = [&](uint32_t cc, const uint32_t (&d)[CPL / 2]) {
         if (cc >= (uint32_t)NCT) return;
         uint32_t pw[CPL / 2];                               // staged pairs in the order the unpacker produces them
+        float sx_true = 0.0f;                               // INPLACE: sum of the activations before they are scaled
         static_for<CPL / 2>([&](auto I) {
             constexpr int i = decltype(I)::value;
-            constexpr int e0 = pair_elem<BITS>(i, 0), e1 = pair_elem<BITS>(i, 1);
-            static_assert((e0 & 1) == (e1 & 1) || e1 == e0 + 1, "pair halves come from the same half-word");
+            constexpr int e0 = INPLACE ? inplace_pair3(i).e0 : pair_elem<BITS>(i, 0);
+            constexpr int e1 = INPLACE ? inplace_pair3(i).e1 : pair_elem<BITS>(i, 1);
             if constexpr (e1 == e0 + 1 && (e0 & 1) == 0) pw[i] = d[e0 >> 1];
-            else pw[i] = __builtin_amdgcn_perm(d[e1 >> 1], d[e0 >> 1], (e0 & 1) ? 0x07060302u : 0x05040100u);
+            else {
+                constexpr uint32_t h0 = 2 * (e0 & 1), h1 = 4 + 2 * (e1 & 1);      // first byte of each half in the permute
+                pw[i] = __builtin_amdgcn_perm(d[e1 >> 1], d[e0 >> 1], ((h1 + 1) << 24) | (h1 << 16) | ((h0 + 1) << 8) | h0);
+            }
+            if constexpr (INPLACE) {
+                sx_true = dot2_x<XA>(pw[i], 0x3F803F80u, sx_true);
+                constexpr int a0 = inplace_pair3(i).a0, a1 = inplace_pair3(i).a1;
+                if constexpr (a0 != 0 || a1 != 0) {
+                    const float lo = __uint_as_float(pw[i] << 16) * (1.0f / (float)(1 << a0));
+                    const float hi = __uint_as_float(pw[i] & 0xFFFF0000u) * (1.0f / (float)(1 << a1));
+                    pw[i] = __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
+                }
+            }
         });
         static_for<Q>([&](auto P) {
             constexpr int i = decltype(P)::value;
@@ -120,6 +155,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_rows_kernel(GemvArgs a) {
             xs[((size_t)cc * Q + i) * 64 + lane] = o;
         });
         constexpr uint32_t kOnes = XA == 1 ? 0x3C003C00u : 0x3F803F80u;
+        if constexpr (INPLACE) {                            // one group per lane chunk: sum x, and 128 sum 2^-a x
+            float px = 0.0f;
+            static_for<CPL / 2>([&](auto I) { px = dot2_x<XA>(pw[decltype(I)::value], 0x43004300u, px); });
+            float* const cell = sxs + (size_t)cc * NF * 64 + lane;
+            cell[0] = sx_true;
+            cell[64] = px;
+        } else
         static_for<NSR>([&](auto S) {
             constexpr int sr = decltype(S)::value;
             float sx = 0.0f, px = 0.0f;
@@ -174,6 +216,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_rows_kernel(GemvArgs a) {
         k_mask[c] = (BITS == 4 ? 0x000F000Fu : 0x00030003u) << (MULTI ? f16_class_shift<BITS>(c) : 0);
         asm volatile("" : "+s"(k_mask[c]));
     }
+    // INPLACE: the masks of the (low, high) field positions in use
+    auto ip_mask_value = [](int a0, int a1) constexpr -> uint32_t { return (7u << a0) | (7u << (16 + a1)); };
+    uint32_t m_a = ip_mask_value(3, 2), m_b = ip_mask_value(1, 0), m_c = ip_mask_value(4, 3);
+    uint32_t m_d = ip_mask_value(2, 4), m_e = ip_mask_value(0, 1);
+    if constexpr (INPLACE) {
+        asm volatile("" : "+s"(m_a)); asm volatile("" : "+s"(m_b)); asm volatile("" : "+s"(m_c));
+        asm volatile("" : "+s"(m_d)); asm volatile("" : "+s"(m_e));
+    }
 
     // contribution of one K-step of one row: sum over its sub-runs of s * sum(q x) + z * sum(x)
     auto step = [&](const Slot& cur, auto C) -> float {
@@ -215,6 +265,24 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_rows_kernel(GemvArgs a) {
                     pr[1] = ((wv >> 2) & k_mask[0]) | k_magic;
                     pr[2] = ((wv >> 4) & k_mask[0]) | k_magic;
                     pr[3] = ((wv >> 6) & k_mask[0]) | k_magic;
+                } else if constexpr (INPLACE) {
+                    const uint32_t w0 = cur.w[0], w1 = cur.w[1], w2 = cur.w[2];
+                    if constexpr (p == 0) {
+                        pr[0] = (w0 & m_a) | k_magic; pr[1] = ((w0 >> 3) & m_a) | k_magic;
+                        pr[2] = ((w0 >> 6) & m_a) | k_magic; pr[3] = ((w0 >> 9) & m_a) | k_magic;
+                    } else if constexpr (p == 1) {
+                        const uint32_t w6 = w1 >> 6;
+                        pr[0] = (w1 & m_b) | k_magic; pr[1] = (w1 & m_c) | k_magic;
+                        pr[2] = (w6 & m_b) | k_magic; pr[3] = (w6 & m_c) | k_magic;
+                    } else if constexpr (p == 2) {
+                        pr[0] = ((w1 >> 12) & m_b) | k_magic; pr[1] = (w2 & m_d) | k_magic;
+                        pr[2] = ((w2 >> 3) & m_d) | k_magic; pr[3] = ((w2 >> 6) & m_d) | k_magic;
+                    } else {
+                        pr[0] = ((w2 >> 9) & m_d) | k_magic;
+                        pr[1] = (__builtin_amdgcn_perm(w2, w0, 0x07060100u) & m_e) | k_magic;
+                        pr[2] = (__builtin_amdgcn_alignbit(w1, w0, 14) & m_b) | k_magic;
+                        pr[3] = (__builtin_amdgcn_alignbit(w2, w1, 30) & m_b) | k_magic;
+                    }
                 } else if constexpr (BITS == 8) {
                     const uint32_t w0 = cur.w[2 * p], w1 = cur.w[2 * p + 1];
                     pr[0] = __builtin_amdgcn_perm(k_magic, w0, 0x05010500u);
@@ -258,7 +326,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_rows_kernel(GemvArgs a) {
             const uint32_t szw = cur.sz[sr];
             if constexpr (SBBF16) { s = __uint_as_float(szw << 16); z = __uint_as_float(szw & 0xFFFF0000u); }
             else { s = f16_to_f32((uint16_t)(szw & 0xFFFFu)); z = f16_to_f32((uint16_t)(szw >> 16)); }
-            if constexpr (MULTI) {
+            if constexpr (INPLACE) {
+                out = __builtin_fmaf(s, dot[sr][0] - cell[64], __builtin_fmaf(z, sx, out));
+            } else if constexpr (MULTI) {
                 float t = dot[sr][0];
 #pragma unroll
                 for (int cl = 1; cl < NCLS; cl++) t = __builtin_fmaf(dot[sr][cl], 1.0f / (float)(1 << f16_class_shift<BITS>(cl)), t);

@@ -330,18 +330,19 @@ namespace {
 
 constexpr size_t kT16LdsBudget = 144 * 1024;
 
-size_t t16_staged_bytes(uint32_t m, uint32_t k) { return (size_t)m * ((size_t)k * 2 + 16) + k; }
+// M staged activation rows of k elements and the sums per half block (a block: 64 bytes of a weight row, bc codes)
+size_t t16_staged_bytes(uint32_t m, uint32_t k, uint32_t bc) { return (size_t)m * ((size_t)k * 2 + 16) + (size_t)(k / bc) * 128; }
 
 // K parts of a launch: 1 when the staged activations of whole rows fit in LDS; else a power of two that divides the
 // K-blocks and whose columns fit, 0 when none does.  Among those the smallest that leaves a workgroup either a small
 // staged copy (two workgroups per CU) or, with one workgroup per CU, at least three row tiles to walk on it (measured,
 // 14336 -> 4096: M = 8 in two parts 18.6 us, in four 14.2 us; M = 16 in four 16.4 us, in eight 17.6 us).
-uint32_t t16_parts(uint32_t k, uint32_t m, uint32_t n_row_tiles, uint32_t cus) {
-    const uint32_t kblocks = k / 128;
-    if (t16_staged_bytes(m, k) <= kT16LdsBudget) return 1;
+uint32_t t16_parts(uint32_t k, uint32_t m, uint32_t n_row_tiles, uint32_t cus, uint32_t bc = 128) {
+    const uint32_t kblocks = k / bc;
+    if (t16_staged_bytes(m, k, bc) <= kT16LdsBudget) return 1;
     uint32_t first_fit = 0;
     for (uint32_t p = 2; p <= 16 && kblocks % p == 0; p *= 2) {
-        const size_t staged = t16_staged_bytes(m, k / p);
+        const size_t staged = t16_staged_bytes(m, k / p, bc);
         if (staged > kT16LdsBudget) continue;
         if (!first_fit) first_fit = p;
         if (staged <= 80 * 1024 || (uint64_t)n_row_tiles * p >= 3ull * cus) return p;
@@ -388,25 +389,26 @@ bool gemv_tile16_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_st
     return t16_parts(w.k, m, (w.n + 15) / 16, 256) != 0;              // staged activations and their group sums fit in LDS
 }
 
-uint32_t gemv_tile16_parts_for(uint32_t k, uint32_t m, uint32_t n_row_tiles, uint32_t cus) {
-    return t16_parts(k, m, n_row_tiles, cus);
+uint32_t gemv_tile16_parts_for(uint32_t k, uint32_t m, uint32_t n_row_tiles, uint32_t cus, uint32_t block_codes) {
+    return t16_parts(k, m, n_row_tiles, cus, block_codes);
 }
 
 uint32_t gemv_tile16_k_parts(const mi355q_context* ctx, const WView& w, uint32_t m) {
     return t16_parts(w.k, m, (w.n + 15) / 16, (uint32_t)ctx->props.multiProcessorCount);
 }
 
-Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_row_tiles, uint32_t k_total, uint32_t m) {
+Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_row_tiles, uint32_t k_total, uint32_t m,
+                                    uint32_t block_codes) {
     Tile16LaunchShape g{};
     // With K parts the launch is shaped as parts x as many row tiles of rows of K / parts codes: every workgroup
     // belongs to one part, and the workgroups of a part cover all row tiles.
     const uint32_t cus = (uint32_t)ctx->props.multiProcessorCount;
-    uint32_t parts = t16_parts(k_total, m, n_row_tiles, cus);
+    uint32_t parts = t16_parts(k_total, m, n_row_tiles, cus, block_codes);
     if (!parts) parts = 1;
     const uint32_t k = k_total / parts;
     const uint32_t n_total_tiles = n_row_tiles * parts;
     g.parts = parts;
-    const uint32_t kblocks = k / 128;
+    const uint32_t kblocks = k / block_codes;
     // Measured on MI355X.  K split: the smallest of 4, 8, 16 that puts about eight wavefronts on
     // every CU (and leaves each wavefront at least two K-blocks).
     uint32_t ks = 4;
@@ -463,7 +465,7 @@ Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_row_ti
     // wavefronts walk several row tiles on the one staged copy -- as many as still leave a workgroup per CU.
     {
         const size_t staged = (size_t)m * ((size_t)k * 2 + 16);
-        const size_t per_pass = (size_t)tpw * 16 * (k / 64) * 36 / 2;
+        const size_t per_pass = (size_t)tpw * 16 * kblocks * 72 / 2;
         uint32_t want = (uint32_t)((staged + per_pass - 1) / per_pass);
         // not more than leaves one workgroup per CU; with one workgroup per CU, exactly one round of workgroups
         const uint32_t most = one_wg_per_cu ? (n_total_tiles + tpw * cus - 1) / (tpw * cus) : n_total_tiles / (tpw * cus);
@@ -474,7 +476,7 @@ Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_row_ti
     g.wgs_per_part = (n_row_tiles + tpw * g.passes - 1) / (tpw * g.passes);
     g.grid = g.wgs_per_part * parts;
     g.block = g.waves * 64;
-    const size_t x_bytes = (size_t)m * ((size_t)k * 2 + 16) + k;     // rows, then sum(x) per group: [K/64][16] floats
+    const size_t x_bytes = t16_staged_bytes(m, k, block_codes);      // rows, then sum(x) per half block: [2 kblocks][16] floats
     const size_t red_bytes = (size_t)g.waves * 4 * 64 * 4;     // partial tiles, behind the activations
     g.lds_bytes = (uint32_t)(g.passes > 1 ? x_bytes + red_bytes : (x_bytes > red_bytes ? x_bytes : red_bytes));
     return g;

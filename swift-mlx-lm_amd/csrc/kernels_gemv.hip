@@ -37,7 +37,8 @@ size_t lds_bytes(const WView& w, int mt, int xa) {
     const size_t nc = (w.k + kc - 1) / kc;
     const size_t sr = (size_t)g.cpl < w.group ? g.cpl : w.group;
     const size_t nsr = g.cpl / sr;
-    const size_t nf = (xa == 1 && (w.bits == 2 || w.bits == 4)) ? 2 : 1;
+    // two sums per lane chunk where fields are used in place (f16: 2 and 4 bits; bf16, rows kernel: 3 bits)
+    const size_t nf = ((xa == 1 && (w.bits == 2 || w.bits == 4)) || (xa == 0 && w.bits == 3)) ? 2 : 1;
     return (size_t)mt * nc * 64 * ((size_t)(g.cpl / 8) * 16 + nsr * nf * 4);
 }
 

@@ -279,6 +279,32 @@ def test_ragged_shapes(pkg, ctx):
     _seeded_gemv_check(pkg, ctx, 521, 67, 2048 + 256, 3, 64, [1, 2], layouts=("planes", "staf"))
 
 
+def test_q3_rows_every_code_position_and_row_length(pkg, ctx):
+    """3-bit codes on the planes are used where they lie in their words (pairs of fields picked with one mask, the
+    activations staged pre-scaled by powers of two).  One-hot activations single out every code position of a lane
+    chunk of 32 codes (and of a chunk further along the row, with a negative and a non-unit activation): each output
+    is s q x + z x exactly.  Then every row length the kernel is built for (1, 2, 3, 4 and 7 K-steps of 2048 codes)
+    against the oracle."""
+    rng = np.random.default_rng(530)
+    n, k = 70, 4096
+    codes = rng.integers(0, 8, (n, k), dtype=np.uint8)
+    scales = rng.choice([0.25, 0.5, 1.0], (n, k // 64)); zeros = rng.integers(-4, 5, (n, k // 64)) * 0.5
+    case = Case(3, 64, codes, scales, zeros)
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(3, 64)
+    w = ctx.weight_prepare_mlx(fmt, *case.planes(pkg.BF16, pkg), pkg.BF16, pkg.LAYOUT_PLANES)
+    assert w.plan_decode_step(1).device_kernel == "gemv_rows_q3_g64"
+    for base, val in ((0, 1.0), (2048 + 37 * 32, -1.0), (4096 - 32, 0.375)):
+        for j in range(32):
+            x = np.zeros((1, k), np.float32); x[0, base + j] = val
+            got = run_gemv(ctx, pkg, w, x, pkg.BF16, pkg.F32)[0]
+            g = (base + j) // 64
+            want = (scales[:, g] * codes[:, base + j] + zeros[:, g]) * val
+            assert np.array_equal(got.astype(np.float64), want), (base, j)
+    w.destroy()
+    for i, k in enumerate((2048, 4096, 6144, 8192, 14336, 4096 + 64, 2048 - 64)):
+        _seeded_gemv_check(pkg, ctx, 531 + i, 300, k, 3, 64, [1], layouts=("planes",))
+
+
 def test_linearity_and_scaling_at_full_size(pkg, ctx):
     """Size-independent properties at the full gate/up shape: y(2x) == 2*y(x) bit for bit
     (a power-of-two scale commutes with every rounding), and row i of the output only depends on
