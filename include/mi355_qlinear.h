@@ -254,7 +254,12 @@ MI355Q_API mi355q_status mi355q_weight_destroy(mi355q_weight* w);
  * 2=output 3=inputDimension 4=outputDimension, MC/Compiler/MetalDispatchStepBuilder.swift:679-688)
  * widened to the sequence signature for small M (5=sequenceLength 6=inputRowStride,
  * :116-153).  y[m*y_row_stride + n] = sum_k (scale*q + zero) * x[m*x_row_stride + k], fp32
- * accumulation, result rounded once to y_dtype.  1 <= M <= 8.  y_row_stride 0 means N. */
+ * accumulation, result rounded once to y_dtype.  1 <= M <= 8.  y_row_stride 0 means N.
+ * Activation types: bf16 and f16 rows are read by the decode kernels directly.  fp32 rows are split on the
+ * device into three bf16 rows each whose sum is the fp32 row exactly (8 + 8 + 8 significant bits); the bf16
+ * kernel of the layout runs on the 3 M rows (the matrix is still read once, every product is exact) and a small
+ * launch adds the three partial results of a row.  The split rows and partial results live in a scratch buffer
+ * of the context, grown on first use. */
 MI355Q_API mi355q_status mi355q_qgemv(mi355q_context* ctx, void* stream, const mi355q_weight* w,
                                       const void* x_dev, mi355q_dtype x_dtype, void* y_dev,
                                       mi355q_dtype y_dtype, uint32_t m, uint32_t x_row_stride,
@@ -279,9 +284,10 @@ MI355Q_API mi355q_status mi355q_qgemv(mi355q_context* ctx, void* stream, const m
  *     weights as in gemm_bf16_f32s, the activations split into bf16 high and low halves).  The
  *     first eager call of a shape times the library's candidate algorithms once (a few milliseconds)
  *     and keeps the quickest.  When the library is absent or has no algorithm, the other routes serve.
- *     Batches of 2 to 15 rows whose layout or activation type no decode kernel reads (fp32 or f16
- *     rows on TILE16 records, fp32 rows on planes and blocks, rows of the block layout that are not
- *     whole 16-byte units) take it too, there with UNROUNDED fp32 weights (N*K*4 bytes of scratch),
+ *     Batches of 2 to 15 rows whose layout or activation type no decode kernel reads (f16 rows on
+ *     TILE16 records, rows of the block layout that are not whole 16-byte units, fp32 rows beyond
+ *     those the three-way bf16 split of mi355q_qgemv serves: sixteen on TILE16 records and 4- / 8-bit
+ *     planes, two elsewhere) take it too, there with UNROUNDED fp32 weights (N*K*4 bytes of scratch),
  *     the activations widened to fp32, the library's fp32 product and the result narrowed to y_dtype:
  *     the result keeps the decode kernels' accuracy, at a cost that does not grow with M.
  * Launches that split K over workgroups (few output

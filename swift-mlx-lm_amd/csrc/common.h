@@ -68,6 +68,10 @@ struct mi355q_context {
     size_t workspace_bytes;
     void* retired[40];
     int retired_count;
+    // fp32 activations split into bf16 rows, and the partial projections of those rows (the decode kernels that run on
+    // them may use `workspace` themselves); grown and retired like `workspace`
+    void* split_buffer;
+    size_t split_bytes;
     // the platform's dense GEMM library (second half of the two-dispatch prefill route), opened on first use
     mi355q::DenseLibrary* dense_library;
     bool dense_library_failed;
@@ -124,6 +128,9 @@ mi355q_status launch_unpack_codes(hipStream_t s, const WView& w, uint8_t* out);
 mi355q_status launch_dequant_bf16(hipStream_t s, const WView& w, uint16_t* out);
 mi355q_status launch_dequant_f32(hipStream_t s, const WView& w, float* out);
 mi355q_status launch_dequant_f16(hipStream_t s, const WView& w, uint16_t* out);
+mi355q_status launch_split_f32_bf16x3(hipStream_t s, const float* x, uint32_t m, uint32_t k, uint32_t x_stride, uint16_t* out,
+                                      uint32_t out_stride);
+mi355q_status launch_sum3_rows(hipStream_t s, const float* y3, uint32_t m, uint32_t n, void* y, int y_dtype, uint32_t y_stride);
 mi355q_status launch_split_f32_bf16x2(hipStream_t s, const float* x, uint32_t m, uint32_t k, uint32_t x_stride, uint16_t* hi,
                                       uint16_t* lo);
 mi355q_status launch_gemv_generic(hipStream_t s, const WView& w, const void* x, int x_dtype,
@@ -236,6 +243,11 @@ struct GemmLaunchShape {
 GemmLaunchShape gemm_mfma_shape(const mi355q_context* ctx, uint32_t m, uint32_t n, uint32_t k);
 // Grows the context's scratch buffer for fp32 partial results; nothing is released before the context goes.
 mi355q_status ensure_workspace(mi355q_context* ctx, size_t bytes);
+mi355q_status ensure_split_buffer(mi355q_context* ctx, size_t bytes);
+// fp32 activations as three bf16 rows each on the bf16 decode kernels (api.hip): row pitch of the bf16 rows, and
+// whether a call takes that route
+inline uint32_t split_f32_row_stride(uint32_t k) { return (k + 7u) & ~7u; }
+bool split_f32_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t flags);
 bool gemm_mfma_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
 mi355q_status launch_qgemm_mfma(hipStream_t s, mi355q_context* ctx, const WView& w,
                                 const void* x, int x_dtype, void* y, int y_dtype, uint32_t m,

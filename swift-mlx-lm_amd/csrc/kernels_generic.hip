@@ -376,6 +376,61 @@ mi355q_status launch_convert_rows(hipStream_t s, const void* src, int src_dtype,
     return MI355Q_OK;
 }
 
+// fp32 activations as THREE bf16 rows each: hi = bf16(x), mid = bf16(x - hi), lo = x - hi - mid.  Both differences are
+// exact in fp32 and the last one fits bf16 (24 significant bits = 8 + 8 + 8, rounding to nearest leaves at most 16,
+// then at most 7), so hi + mid + lo == x exactly and a bf16 kernel run on the 3 M rows computes the fp32 projection with
+// exact products.  out: [3][M][out_stride].  A non-finite activation stays in hi alone.
+__global__ __launch_bounds__(256) void split_f32_bf16x3_kernel(const float* __restrict__ x, uint32_t m, uint32_t k,
+                                                               uint32_t x_stride, uint16_t* __restrict__ out,
+                                                               uint32_t out_stride) {
+    const uint32_t row = blockIdx.y;
+    for (uint32_t c = blockIdx.x * 256 + threadIdx.x; c < k; c += gridDim.x * 256) {
+        const float v = x[(size_t)row * x_stride + c];
+        const uint16_t hi = f32_to_bf16_rne(v);
+        uint16_t mid = 0, lo = 0;
+        if (v - v == 0.0f) {                                // finite
+            const float r1 = v - __uint_as_float((uint32_t)hi << 16);
+            mid = f32_to_bf16_rne(r1);
+            lo = f32_to_bf16_rne(r1 - __uint_as_float((uint32_t)mid << 16));
+        }
+        out[((size_t)0 * m + row) * out_stride + c] = hi;
+        out[((size_t)1 * m + row) * out_stride + c] = mid;
+        out[((size_t)2 * m + row) * out_stride + c] = lo;
+    }
+}
+
+// y[r] = (y3[2 M + r] + y3[M + r]) + y3[r]: the three partial projections of split_f32_bf16x3_kernel, smallest first
+__global__ __launch_bounds__(256) void sum3_rows_kernel(const float* __restrict__ y3, uint32_t m, uint32_t n,
+                                                        void* __restrict__ y, int y_dtype, uint32_t y_stride) {
+    const uint32_t row = blockIdx.y;
+    for (uint32_t c = blockIdx.x * 256 + threadIdx.x; c < n; c += gridDim.x * 256) {
+        const float v = (y3[((size_t)2 * m + row) * n + c] + y3[((size_t)m + row) * n + c]) + y3[(size_t)row * n + c];
+        const size_t o = (size_t)row * y_stride + c;
+        if (y_dtype == MI355Q_F32) ((float*)y)[o] = v;
+        else if (y_dtype == MI355Q_BF16) ((uint16_t*)y)[o] = f32_to_bf16_rne(v);
+        else ((uint16_t*)y)[o] = f32_to_f16_rne(v);
+    }
+}
+
+mi355q_status launch_split_f32_bf16x3(hipStream_t s, const float* x, uint32_t m, uint32_t k, uint32_t x_stride, uint16_t* out,
+                                      uint32_t out_stride) {
+    if (m > 65535u) return fail(MI355Q_ERR_SHAPE, "more than 65535 activation rows");
+    uint32_t gx = (k + 255) / 256;
+    if (gx > 256) gx = 256;
+    split_f32_bf16x3_kernel<<<dim3(gx, m), dim3(256), 0, s>>>(x, m, k, x_stride, out, out_stride);
+    MI355Q_HIP(hipGetLastError());
+    return MI355Q_OK;
+}
+
+mi355q_status launch_sum3_rows(hipStream_t s, const float* y3, uint32_t m, uint32_t n, void* y, int y_dtype, uint32_t y_stride) {
+    if (m > 65535u) return fail(MI355Q_ERR_SHAPE, "more than 65535 rows");
+    uint32_t gx = (n + 255) / 256;
+    if (gx > 256) gx = 256;
+    sum3_rows_kernel<<<dim3(gx, m), dim3(256), 0, s>>>(y3, m, n, y, y_dtype, y_stride);
+    MI355Q_HIP(hipGetLastError());
+    return MI355Q_OK;
+}
+
 mi355q_status launch_split_f32_bf16x2(hipStream_t s, const float* x, uint32_t m, uint32_t k, uint32_t x_stride, uint16_t* hi,
                                       uint16_t* lo) {
     if (m > 65535u) return fail(MI355Q_ERR_SHAPE, "more than 65535 activation rows");

@@ -47,6 +47,14 @@ void plan_small_m(const mi355q_weight* w, uint32_t m, int x_dtype, uint32_t x_st
                   mi355q_step* s) {
     const WView v = w->view();
     const bool forced = flags & MI355Q_FLAG_FORCE_GENERIC;
+    if (split_f32_chosen(v, x_dtype, m, flags)) {
+        // fp32 rows as three bf16 rows each on the bf16 decode kernel, then the sum of the three partial results
+        plan_small_m(w, 3 * m, MI355Q_BF16, split_f32_row_stride((uint32_t)w->k), flags, s);
+        char inner[sizeof s->device_kernel];
+        std::snprintf(inner, sizeof inner, "%s", s->device_kernel);
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "split_f32_bf16x3+%.30s", inner);
+        return;
+    }
     // rows per launch on the tile layout: 16, or fewer when K is so long that 16 staged rows overflow LDS
     uint32_t t16_rows = m > 16 ? 16 : m;
     if (!forced && v.layout == MI355Q_LAYOUT_TILE16) {
@@ -212,9 +220,10 @@ mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w, uint32_t maximum
 
     const uint32_t m = maximum_sequence_length;
     const uint32_t small_rows = small_batch_rows(v, x_dtype, input_row_stride);   // rows the decode kernels take per launch
-    const bool want_small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) || m <= small_rows;
+    const bool want_small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) || m <= small_rows ||
+                            split_f32_chosen(v, x_dtype, m, flags);
     const bool mfma_ok = gemm_mfma_eligible(v, x_dtype, m, input_row_stride);
-    if (gemm_two_step_chosen(v, x_dtype, m, input_row_stride, flags)) {
+    if (!split_f32_chosen(v, x_dtype, m, flags) && gemm_two_step_chosen(v, x_dtype, m, input_row_stride, flags)) {
         // dequant_q{b}_g{g}_bf16 into the scratch matrix, then the dense GEMM (MetalPrefillStepBuilder's two-dispatch
         // route; the dense product is the platform library's, as the reference's is matmul2d)
         *out_count = 2;

@@ -41,20 +41,30 @@ unsigned long long* static_head_keys(int device) {
 
 namespace mi355q {
 
-mi355q_status ensure_workspace(mi355q_context* ctx, size_t bytes) {
-    if (bytes <= ctx->workspace_bytes) return MI355Q_OK;
+namespace {
+mi355q_status grow_scratch(mi355q_context* ctx, void*& buffer, size_t& have, size_t bytes, size_t granule) {
+    if (bytes <= have) return MI355Q_OK;
     // A launch recorded in a HIP graph keeps the address it was captured with, so an outgrown buffer stays allocated
     // until the context goes; growth at least doubles, which bounds the retired buffers to the size of the live one.
-    size_t want = bytes > 2 * ctx->workspace_bytes ? bytes : 2 * ctx->workspace_bytes;
-    want = (want + ((size_t)1 << 22) - 1) & ~(((size_t)1 << 22) - 1);
-    if (ctx->workspace && ctx->retired_count >= kRetiredWorkspaces)
+    size_t want = bytes > 2 * have ? bytes : 2 * have;
+    want = (want + granule - 1) & ~(granule - 1);
+    if (buffer && ctx->retired_count >= kRetiredWorkspaces)
         return fail(MI355Q_ERR_OUT_OF_MEMORY, "scratch buffer outgrown %d times", kRetiredWorkspaces);
     void* grown = nullptr;
     MI355Q_HIP(hipMalloc(&grown, want));
-    if (ctx->workspace) ctx->retired[ctx->retired_count++] = ctx->workspace;
-    ctx->workspace = grown;
-    ctx->workspace_bytes = want;
+    if (buffer) ctx->retired[ctx->retired_count++] = buffer;
+    buffer = grown;
+    have = want;
     return MI355Q_OK;
+}
+}  // namespace
+
+mi355q_status ensure_workspace(mi355q_context* ctx, size_t bytes) {
+    return grow_scratch(ctx, ctx->workspace, ctx->workspace_bytes, bytes, (size_t)1 << 22);
+}
+
+mi355q_status ensure_split_buffer(mi355q_context* ctx, size_t bytes) {
+    return grow_scratch(ctx, ctx->split_buffer, ctx->split_bytes, bytes, (size_t)1 << 20);
 }
 
 }  // namespace mi355q
@@ -292,6 +302,7 @@ mi355q_status mi355q_context_destroy(mi355q_context* ctx) {
     if (ctx->argmax_scratch) (void)hipFree(ctx->argmax_scratch);
     if (ctx->argmax_partials) (void)hipFree(ctx->argmax_partials);
     if (ctx->workspace) (void)hipFree(ctx->workspace);
+    if (ctx->split_buffer) (void)hipFree(ctx->split_buffer);
     for (int i = 0; i < ctx->retired_count; i++) (void)hipFree(ctx->retired[i]);
     delete ctx;
     return MI355Q_OK;

@@ -1,0 +1,142 @@
+"""GPU parity tests of fp32 activations at a few rows (the f32s signatures of gemv_q{b}_g{g} / gemm_q{b}_g{g},
+Sources/MetalCompiler/Generator/MetalSourceGenerator+Quantized.swift:496-575, :22-156) through the C ABI.  Every fp32
+row is split on the device into three bf16 rows whose sum is the row exactly; the bf16 decode kernel of the layout runs
+on the 3 M rows and the three partial results of a row are added, so the matrix is read once and every product is exact.
+
+Bars: against an fp64 accumulation of the dequantised weights and the UNROUNDED fp32 activations, relative L2 <= 1e-5
+(rounding the activations to bf16 would give 1e-3); a case that needs all three parts and is exactly representable is
+compared exactly; padding of activation and output rows is neither read into the result nor written.
+"""
+import sys
+
+import numpy as np
+import pytest
+
+import kat
+import oracle
+from gpu_util import Case, out_from_device, rel_l2, seeded_case
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def run_f32(ctx, pkg, w, x, y_dtype=None, flags=0, xpad=0, ypad=0, use_qgemm=False):
+    y_dtype = pkg.F32 if y_dtype is None else y_dtype
+    m, k = x.shape
+    n = int(w.info.n_rows)
+    xh = np.full((m, k + xpad), 1e30, np.float32); xh[:, :k] = x
+    xd = ctx.upload(xh)
+    yd = ctx.alloc(m * (n + ypad) * (4 if y_dtype == pkg.F32 else 2))
+    ctx.fill(yd, 0x7FC07FC0 if y_dtype != pkg.F32 else 0x7FC00000)
+    (ctx.qgemm if use_qgemm else ctx.qgemv)(w, xd, pkg.F32, yd, y_dtype, m, k + xpad, (n + ypad) if ypad else 0, flags)
+    ctx.synchronize()
+    y = out_from_device(yd, y_dtype, (m, n + ypad), pkg)
+    xd.free(); yd.free()
+    assert np.all(np.isnan(y[:, n:]))
+    return y[:, :n]
+
+
+LAYOUTS = [("planes", 4, 64, 16), ("planes", 4, 128, 16), ("planes", 8, 32, 16), ("planes", 3, 64, 2), ("planes", 6, 64, 2),
+           ("tile16", 4, 64, 16), ("staf", 4, 64, 2), ("staf", 5, 32, 2)]
+
+
+@pytest.mark.parametrize("layout,bits,group,most", LAYOUTS, ids=lambda v: str(v))
+def test_f32_rows_full_mantissas(pkg, ctx, layout, bits, group, most):
+    """Seeded weights, activations with all 24 significant bits in use, every row count the route takes for the layout
+    (up to three launches of sixteen rows on TILE16 records and 4- / 8-bit planes, one launch of eight rows
+    elsewhere); one more row takes another route and still meets the common bar."""
+    lay = {"planes": pkg.LAYOUT_PLANES, "tile16": pkg.LAYOUT_TILE16, "staf": pkg.LAYOUT_STAF_BLOCKS}[layout]
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(bits, group)
+    for i, (n, k) in enumerate([(200, 1024), (70, 4096 + 256)]):
+        words, s, z, wq = seeded_case(5100 + i + bits + group, n, k, bits, group)
+        w = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, lay)
+        for m in ([1, 2, 3] if most == 2 else [1, 2, 5, 6, 11, 16, 17]):
+            say(f"f32 rows {layout} q{bits} g{group} {k}->{n} M={m}")
+            x = kat.seeded_activations(5200 + m, m, k).astype(np.float32)
+            x *= np.float32(1.0) + np.float32(2.0 ** -23) * (np.arange(k, dtype=np.float32) % 7)   # low mantissa bits in use
+            want = oracle.gemm_f64(wq, x)
+            st = w.plan_prefill_steps(m, x_dtype=pkg.F32)[0]
+            got = run_f32(ctx, pkg, w, x, use_qgemm=True)
+            if m <= most:
+                assert st.device_kernel.startswith("split_f32_bf16x3+"), st.device_kernel
+                assert rel_l2(got, want) <= 1e-5, (m, rel_l2(got, want))
+                if m <= 8:
+                    assert w.plan_decode_step(m, pkg.F32).device_kernel == st.device_kernel
+                    assert np.array_equal(run_f32(ctx, pkg, w, x), got)
+            else:
+                assert not st.device_kernel.startswith("split_f32_bf16x3+"), st.device_kernel
+                assert rel_l2(got, want) <= 3e-3        # from sixteen rows the weights are rounded to bf16 once
+        w.destroy()
+
+
+def test_f32_rows_exact_values_padding_and_output_types(pkg, ctx):
+    """Exact case: one activation per row is non-zero, v = (2^16 + odd) / 2^17, a value of 17 significant bits that
+    needs all three bf16 parts (8 + 8 + 1); with power-of-two scales and small integer zeros every product is exact and
+    y = (s q + z) v has at most 23 significant bits, so the fp32 result must equal it bit for bit.  Then seeded rows with
+    padded activation rows (poison behind K) and padded output rows (canary kept); bf16 and f16 outputs are the rounded
+    fp32 ones; forced, the per-code kernel agrees."""
+    rng = np.random.default_rng(5300)
+    n, k = 50, 512
+    codes = rng.integers(0, 16, (n, k), dtype=np.uint8)
+    scales = rng.choice([0.5, 1.0, 2.0], (n, k // 64)); zeros = rng.integers(-4, 5, (n, k // 64)).astype(np.float64)
+    case = Case(4, 64, codes, scales, zeros)
+    wq = scales.repeat(64, axis=1) * codes + zeros.repeat(64, axis=1)
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+    for layout in (pkg.LAYOUT_PLANES, pkg.LAYOUT_TILE16, pkg.LAYOUT_STAF_BLOCKS):
+        w = ctx.weight_prepare_mlx(fmt, *case.planes(pkg.BF16, pkg), pkg.BF16, layout)
+        for m, xpad, ypad in ((1, 0, 0), (2, 8, 3), (5, 4, 0)):
+            if 3 * m > 8 and layout == pkg.LAYOUT_STAF_BLOCKS:
+                continue
+            x = np.zeros((m, k), np.float32)
+            pos = rng.choice(k, m, replace=False)
+            for r in range(m):
+                x[r, pos[r]] = np.float32(((1 << 16) + 2 * int(rng.integers(0, 1 << 15)) + 1) / float(1 << 17)) * (-1) ** r
+            want = x.astype(np.float64) @ wq.T
+            assert np.array_equal(want.astype(np.float32).astype(np.float64), want)
+            got = run_f32(ctx, pkg, w, x, xpad=xpad, ypad=ypad)
+            assert np.array_equal(got.astype(np.float64), want), (layout, m)
+            x = kat.seeded_activations(5310 + m, m, k)
+            want = oracle.gemm_f64(wq, x)
+            got = run_f32(ctx, pkg, w, x, xpad=xpad, ypad=ypad)
+            assert rel_l2(got, want) <= 1e-5, (layout, m, rel_l2(got, want))
+            for yd in (pkg.BF16, pkg.F16):
+                low = run_f32(ctx, pkg, w, x, y_dtype=yd, xpad=xpad, ypad=ypad)
+                ref = oracle.bf16_to_f32(oracle.bf16_from_f32(got)).reshape(got.shape) if yd == pkg.BF16 \
+                    else got.astype(np.float16).astype(np.float32)
+                assert np.array_equal(low, ref), (layout, m, yd)
+            slow = run_f32(ctx, pkg, w, x, flags=pkg.FLAG_FORCE_GENERIC, xpad=xpad, ypad=ypad)
+            assert rel_l2(slow, want) <= 1e-5
+        w.destroy()
+
+
+def test_f32_rows_non_finite_activation_and_graph_replay(pkg, ctx):
+    """An infinite activation stays in the first bf16 part (the output row is non-finite where its weight is not zero,
+    finite rows are untouched); a plan with fp32 rows replays as a HIP graph with the same result every time."""
+    n, k, m = 64, 1024, 3
+    words, s, z, wq = seeded_case(5400, n, k, 4, 64)
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+    w = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, pkg.LAYOUT_PLANES)
+    x = kat.seeded_activations(5401, m, k).astype(np.float32)
+    x[1, 17] = np.inf
+    got = run_f32(ctx, pkg, w, x)
+    assert not np.any(np.isfinite(got[1][wq[:, 17] != 0]))
+    fin = oracle.gemm_f64(wq, x[[0, 2]])
+    assert rel_l2(got[[0, 2]], fin) <= 1e-5
+    x[1, 17] = 0.25
+    xd = ctx.upload(x); yd = ctx.alloc(m * n * 4)
+    plan = pkg.DispatchPlan(ctx)
+    plan.add_linear(w, xd, pkg.F32, yd, pkg.F32, m)
+    stream = ctx.stream_create()
+    plan.encode(stream); ctx.synchronize(stream)
+    eager = yd.download(np.float32, (m, n)).copy()
+    assert rel_l2(eager, oracle.gemm_f64(wq, x)) <= 1e-5
+    plan.graph_build(stream)
+    for _ in range(3):
+        ctx.fill(yd, 0x7FC00000, stream)
+        plan.graph_launch(stream); ctx.synchronize(stream)
+        assert np.array_equal(yd.download(np.float32, (m, n)), eager)
+    plan.destroy(); ctx.stream_destroy(stream)
+    xd.free(); yd.free(); w.destroy()
