@@ -258,8 +258,10 @@ MI355Q_API mi355q_status mi355q_weight_destroy(mi355q_weight* w);
  * Activation types: bf16 and f16 rows are read by the decode kernels directly.  fp32 rows are split on the
  * device into three bf16 rows each whose sum is the fp32 row exactly (8 + 8 + 8 significant bits); the bf16
  * kernel of the layout runs on the 3 M rows (the matrix is still read once, every product is exact) and a small
- * launch adds the three partial results of a row.  The split rows and partial results live in a scratch buffer
- * of the context, grown on first use. */
+ * launch adds the three partial results of a row.  f16 rows go the same way as two bf16 rows each (8 + 3 bits)
+ * where only a bf16 kernel reads the layout (TILE16 records) or the bf16 matrix-core kernel is the faster one
+ * (4- and 8-bit planes from five rows).  The split rows and partial results live in a scratch buffer of the
+ * context, grown on first use. */
 MI355Q_API mi355q_status mi355q_qgemv(mi355q_context* ctx, void* stream, const mi355q_weight* w,
                                       const void* x_dev, mi355q_dtype x_dtype, void* y_dev,
                                       mi355q_dtype y_dtype, uint32_t m, uint32_t x_row_stride,
@@ -284,10 +286,9 @@ MI355Q_API mi355q_status mi355q_qgemv(mi355q_context* ctx, void* stream, const m
  *     weights as in gemm_bf16_f32s, the activations split into bf16 high and low halves).  The
  *     first eager call of a shape times the library's candidate algorithms once (a few milliseconds)
  *     and keeps the quickest.  When the library is absent or has no algorithm, the other routes serve.
- *     Batches of 2 to 15 rows whose layout or activation type no decode kernel reads (f16 rows on
- *     TILE16 records, rows of the block layout that are not whole 16-byte units, fp32 rows beyond
- *     those the three-way bf16 split of mi355q_qgemv serves: sixteen on TILE16 records and 4- / 8-bit
- *     planes, two elsewhere) take it too, there with UNROUNDED fp32 weights (N*K*4 bytes of scratch),
+ *     Batches of 2 to 15 rows whose layout or activation type no decode kernel reads (rows of the
+ *     block layout that are not whole 16-byte units, fp32 rows beyond those the bf16 split of
+ *     mi355q_qgemv serves: sixteen on TILE16 records and 4- / 8-bit planes, two elsewhere) take it too, there with UNROUNDED fp32 weights (N*K*4 bytes of scratch),
  *     the activations widened to fp32, the library's fp32 product and the result narrowed to y_dtype:
  *     the result keeps the decode kernels' accuracy, at a cost that does not grow with M.
  * Launches that split K over workgroups (few output

@@ -84,36 +84,42 @@ mi355q_status run_small_m(mi355q_context* ctx, hipStream_t s, const mi355q_weigh
     return MI355Q_OK;
 }
 
-// fp32 activations, a few rows, on a weight the bf16 decode kernels read: every row becomes three bf16 rows whose sum is
-// the fp32 row exactly (split_f32_bf16x3_kernel), the bf16 kernels run on the 3 M rows, and the three partial results of
-// a row are added.  Products stay exact, the matrix is read once (4096 -> 14336 at one row: 123 us on the per-code
-// kernel, the only one that reads fp32 activations).
-mi355q_status run_split_f32(mi355q_context* ctx, hipStream_t s, const mi355q_weight* w, const void* x, void* y, int y_dtype,
-                            uint32_t m, uint32_t xs, uint32_t ys, uint32_t flags) {
-    const uint32_t n = (uint32_t)w->n, k = (uint32_t)w->k, kp = split_f32_row_stride(k);
-    const size_t xbytes = ((size_t)3 * m * kp * 2 + 255) & ~(size_t)255, ybytes = (size_t)3 * m * n * 4;
+// fp32 or f16 activations, a few rows, on a weight the bf16 decode kernels read: every row becomes three (fp32) or two
+// (f16) bf16 rows whose sum is the row exactly (split_rows_bf16_kernel), the bf16 kernels run on those rows, and the
+// partial results of a row are added.  Products stay exact, the matrix is read once per launch of sixteen or eight rows.
+mi355q_status run_split_rows(mi355q_context* ctx, hipStream_t s, const mi355q_weight* w, const void* x, int x_dtype, void* y,
+                             int y_dtype, uint32_t m, uint32_t xs, uint32_t ys, uint32_t flags) {
+    const uint32_t n = (uint32_t)w->n, k = (uint32_t)w->k, kp = split_rows_stride(k), parts = split_rows_parts(x_dtype);
+    const size_t xbytes = ((size_t)parts * m * kp * 2 + 255) & ~(size_t)255, ybytes = (size_t)parts * m * n * 4;
     if (mi355q_status st = ensure_split_buffer(ctx, xbytes + ybytes)) return st;
-    uint16_t* const x3 = (uint16_t*)ctx->split_buffer;
-    float* const y3 = (float*)((char*)ctx->split_buffer + xbytes);
-    if (mi355q_status st = launch_split_f32_bf16x3(s, (const float*)x, m, k, xs, x3, kp)) return st;
-    if (mi355q_status st = run_small_m(ctx, s, w, x3, MI355Q_BF16, y3, MI355Q_F32, 3 * m, kp, n, flags)) return st;
-    return launch_sum3_rows(s, y3, m, n, y, y_dtype, ys);
+    uint16_t* const xp = (uint16_t*)ctx->split_buffer;
+    float* const yp = (float*)((char*)ctx->split_buffer + xbytes);
+    if (mi355q_status st = launch_split_rows_bf16(s, x, x_dtype, m, k, xs, xp, kp)) return st;
+    if (mi355q_status st = run_small_m(ctx, s, w, xp, MI355Q_BF16, yp, MI355Q_F32, parts * m, kp, n, flags)) return st;
+    return launch_sum_parts_rows(s, yp, parts, m, n, y, y_dtype, ys);
 }
 
 }  // namespace
 
 namespace mi355q {
 
-// Whether fp32 activations of m rows are served as three bf16 rows each on the bf16 decode kernels: no kernel but the
-// per-code one reads fp32 activations, a bf16 decode kernel reads the weight, and the 3 m rows fit one launch of it --
-// three launches where a launch takes sixteen rows (4096 -> 14336 on 4-bit planes: 16-20 us up to five rows, where the
-// dequantise-once route takes 105 us whatever the rows; with launches of eight rows two rows already take 35 us).
-bool split_f32_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t flags) {
-    if (x_dtype != MI355Q_F32 || (flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_TWO_STEP)))
-        return false;
-    const uint32_t kp = split_f32_row_stride((uint32_t)w.k);
+// Whether m rows of fp32 or f16 activations are served as bf16 rows on the bf16 decode kernels.
+//   fp32: no kernel but the per-code one reads it; taken when a bf16 decode kernel reads the weight and the 3 m rows fit
+//   one launch of it -- three launches where a launch takes sixteen rows (4096 -> 14336 on 4-bit planes: 16-20 us up to
+//   five rows, 52 us at sixteen, where the dequantise-once route takes 105 us whatever the rows; with launches of eight
+//   rows two rows already take 35 us).
+//   f16: where no decode kernel reads f16 (TILE16 records), under the same limits; and on planes that the matrix-core
+//   kernel reads in bf16, from five rows (the f16 dot-product kernels take four rows a launch) to sixteen.
+bool split_rows_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride, uint32_t flags) {
+    const uint32_t parts = split_rows_parts(x_dtype);
+    if (!parts || (flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_TWO_STEP))) return false;
+    const uint32_t kp = split_rows_stride((uint32_t)w.k);
+    if (!decode_kernel_reads(w, MI355Q_BF16, kp)) return false;
     const uint32_t rows = small_batch_rows(w, MI355Q_BF16, kp);
-    return decode_kernel_reads(w, MI355Q_BF16, kp) && 3 * (uint64_t)m <= (rows >= 16 ? 3 * rows : rows);
+    const uint64_t most = rows >= 16 ? 3 * rows : rows;
+    if (x_dtype == MI355Q_F16 && decode_kernel_reads(w, MI355Q_F16, x_stride))
+        return rows >= 16 && m >= 5 && 2 * (uint64_t)m <= 2 * rows;
+    return (uint64_t)parts * m <= most;
 }
 
 mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_weight* w, const void* x, int x_dtype,
@@ -127,7 +133,7 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
         // from the second row (4096 -> 14336, fp32 activations: per-code kernel 123 us at M = 1, 195 at M = 2, 700 at
         // M = 8; the route with fp32 weights 100-135 us whatever M)
         const WView v = w->view();
-        if (split_f32_chosen(v, x_dtype, m, flags)) return run_split_f32(ctx, s, w, x, y, y_dtype, m, xs, ys, flags);
+        if (split_rows_chosen(v, x_dtype, m, xs, flags)) return run_split_rows(ctx, s, w, x, x_dtype, y, y_dtype, m, xs, ys, flags);
         if (gemm_two_step_chosen(v, x_dtype, m, xs, flags) && (uintptr_t)x % 16 == 0 &&
             gemm_two_step_serves(ctx, v, x_dtype, y_dtype, m, xs, ys))
             return launch_qgemm_two_step(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
@@ -143,8 +149,8 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
             return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the two-dispatch route takes 16-byte aligned activations, K and the row stride multiples of 8");
         return launch_qgemm_two_step(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
     }
-    if (split_f32_chosen(v, x_dtype, m, flags))
-        return run_split_f32(ctx, s, w, x, y, y_dtype, m, xs, ys, flags);
+    if (split_rows_chosen(v, x_dtype, m, xs, flags))
+        return run_split_rows(ctx, s, w, x, x_dtype, y, y_dtype, m, xs, ys, flags);
     // dequantise once, then the dense library GEMM: long prompts, and every format or layout the fused kernel does
     // not read.  When the library has no algorithm for the problem the routes below serve it.
     if (gemm_two_step_chosen(v, x_dtype, m, xs, flags) && (uintptr_t)x % 16 == 0 &&

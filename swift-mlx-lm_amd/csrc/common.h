@@ -128,9 +128,10 @@ mi355q_status launch_unpack_codes(hipStream_t s, const WView& w, uint8_t* out);
 mi355q_status launch_dequant_bf16(hipStream_t s, const WView& w, uint16_t* out);
 mi355q_status launch_dequant_f32(hipStream_t s, const WView& w, float* out);
 mi355q_status launch_dequant_f16(hipStream_t s, const WView& w, uint16_t* out);
-mi355q_status launch_split_f32_bf16x3(hipStream_t s, const float* x, uint32_t m, uint32_t k, uint32_t x_stride, uint16_t* out,
-                                      uint32_t out_stride);
-mi355q_status launch_sum3_rows(hipStream_t s, const float* y3, uint32_t m, uint32_t n, void* y, int y_dtype, uint32_t y_stride);
+mi355q_status launch_split_rows_bf16(hipStream_t s, const void* x, int x_dtype, uint32_t m, uint32_t k, uint32_t x_stride,
+                                     uint16_t* out, uint32_t out_stride);
+mi355q_status launch_sum_parts_rows(hipStream_t s, const float* yp, uint32_t parts, uint32_t m, uint32_t n, void* y, int y_dtype,
+                                    uint32_t y_stride);
 mi355q_status launch_split_f32_bf16x2(hipStream_t s, const float* x, uint32_t m, uint32_t k, uint32_t x_stride, uint16_t* hi,
                                       uint16_t* lo);
 mi355q_status launch_gemv_generic(hipStream_t s, const WView& w, const void* x, int x_dtype,
@@ -244,10 +245,11 @@ GemmLaunchShape gemm_mfma_shape(const mi355q_context* ctx, uint32_t m, uint32_t 
 // Grows the context's scratch buffer for fp32 partial results; nothing is released before the context goes.
 mi355q_status ensure_workspace(mi355q_context* ctx, size_t bytes);
 mi355q_status ensure_split_buffer(mi355q_context* ctx, size_t bytes);
-// fp32 activations as three bf16 rows each on the bf16 decode kernels (api.hip): row pitch of the bf16 rows, and
-// whether a call takes that route
-inline uint32_t split_f32_row_stride(uint32_t k) { return (k + 7u) & ~7u; }
-bool split_f32_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t flags);
+// fp32 / f16 activations as three / two bf16 rows each on the bf16 decode kernels (api.hip): row pitch of the bf16
+// rows, bf16 rows per activation row (0: the type is not split), and whether a call takes that route
+inline uint32_t split_rows_stride(uint32_t k) { return (k + 7u) & ~7u; }
+inline uint32_t split_rows_parts(int x_dtype) { return x_dtype == MI355Q_F32 ? 3u : x_dtype == MI355Q_F16 ? 2u : 0u; }
+bool split_rows_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride, uint32_t flags);
 bool gemm_mfma_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
 mi355q_status launch_qgemm_mfma(hipStream_t s, mi355q_context* ctx, const WView& w,
                                 const void* x, int x_dtype, void* y, int y_dtype, uint32_t m,

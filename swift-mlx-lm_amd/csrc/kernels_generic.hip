@@ -376,35 +376,41 @@ mi355q_status launch_convert_rows(hipStream_t s, const void* src, int src_dtype,
     return MI355Q_OK;
 }
 
-// fp32 activations as THREE bf16 rows each: hi = bf16(x), mid = bf16(x - hi), lo = x - hi - mid.  Both differences are
-// exact in fp32 and the last one fits bf16 (24 significant bits = 8 + 8 + 8, rounding to nearest leaves at most 16,
-// then at most 7), so hi + mid + lo == x exactly and a bf16 kernel run on the 3 M rows computes the fp32 projection with
-// exact products.  out: [3][M][out_stride].  A non-finite activation stays in hi alone.
-__global__ __launch_bounds__(256) void split_f32_bf16x3_kernel(const float* __restrict__ x, uint32_t m, uint32_t k,
-                                                               uint32_t x_stride, uint16_t* __restrict__ out,
-                                                               uint32_t out_stride) {
+// Activations as several bf16 rows each whose sum is the activation exactly.  fp32 (PARTS = 3): hi = bf16(x),
+// mid = bf16(x - hi), lo = x - hi - mid; both differences are exact in fp32 and the last one fits bf16 (24 significant
+// bits = 8 + 8 + 8, rounding to nearest leaves at most 16, then at most 7).  f16 (PARTS = 2): 11 significant bits =
+// 8 + 3, and every f16 value, subnormals included, lies inside bf16's exponent range.  A bf16 kernel run on the
+// PARTS * M rows then computes the projection with exact products.  out: [PARTS][M][out_stride].  A non-finite activation
+// stays in hi alone.
+template <int PARTS, bool F16IN>
+__global__ __launch_bounds__(256) void split_rows_bf16_kernel(const void* __restrict__ x, uint32_t m, uint32_t k,
+                                                              uint32_t x_stride, uint16_t* __restrict__ out,
+                                                              uint32_t out_stride) {
     const uint32_t row = blockIdx.y;
     for (uint32_t c = blockIdx.x * 256 + threadIdx.x; c < k; c += gridDim.x * 256) {
-        const float v = x[(size_t)row * x_stride + c];
-        const uint16_t hi = f32_to_bf16_rne(v);
-        uint16_t mid = 0, lo = 0;
+        const size_t i = (size_t)row * x_stride + c;
+        const float v = F16IN ? f16_to_f32(((const uint16_t*)x)[i]) : ((const float*)x)[i];
+        uint16_t part[3] = {f32_to_bf16_rne(v), 0, 0};
         if (v - v == 0.0f) {                                // finite
-            const float r1 = v - __uint_as_float((uint32_t)hi << 16);
-            mid = f32_to_bf16_rne(r1);
-            lo = f32_to_bf16_rne(r1 - __uint_as_float((uint32_t)mid << 16));
+            float r = v - __uint_as_float((uint32_t)part[0] << 16);
+#pragma unroll
+            for (int p = 1; p < PARTS; p++) {
+                part[p] = f32_to_bf16_rne(r);
+                r -= __uint_as_float((uint32_t)part[p] << 16);
+            }
         }
-        out[((size_t)0 * m + row) * out_stride + c] = hi;
-        out[((size_t)1 * m + row) * out_stride + c] = mid;
-        out[((size_t)2 * m + row) * out_stride + c] = lo;
+#pragma unroll
+        for (int p = 0; p < PARTS; p++) out[((size_t)p * m + row) * out_stride + c] = part[p];
     }
 }
 
-// y[r] = (y3[2 M + r] + y3[M + r]) + y3[r]: the three partial projections of split_f32_bf16x3_kernel, smallest first
-__global__ __launch_bounds__(256) void sum3_rows_kernel(const float* __restrict__ y3, uint32_t m, uint32_t n,
-                                                        void* __restrict__ y, int y_dtype, uint32_t y_stride) {
+// y[r] = the sum over the parts of split_rows_bf16_kernel of their partial projections, smallest part first
+__global__ __launch_bounds__(256) void sum_parts_rows_kernel(const float* __restrict__ yp, uint32_t parts, uint32_t m, uint32_t n,
+                                                             void* __restrict__ y, int y_dtype, uint32_t y_stride) {
     const uint32_t row = blockIdx.y;
     for (uint32_t c = blockIdx.x * 256 + threadIdx.x; c < n; c += gridDim.x * 256) {
-        const float v = (y3[((size_t)2 * m + row) * n + c] + y3[((size_t)m + row) * n + c]) + y3[(size_t)row * n + c];
+        float v = yp[((size_t)(parts - 1) * m + row) * n + c];
+        for (uint32_t p = parts - 1; p-- > 0;) v += yp[((size_t)p * m + row) * n + c];
         const size_t o = (size_t)row * y_stride + c;
         if (y_dtype == MI355Q_F32) ((float*)y)[o] = v;
         else if (y_dtype == MI355Q_BF16) ((uint16_t*)y)[o] = f32_to_bf16_rne(v);
@@ -412,21 +418,24 @@ __global__ __launch_bounds__(256) void sum3_rows_kernel(const float* __restrict_
     }
 }
 
-mi355q_status launch_split_f32_bf16x3(hipStream_t s, const float* x, uint32_t m, uint32_t k, uint32_t x_stride, uint16_t* out,
-                                      uint32_t out_stride) {
+mi355q_status launch_split_rows_bf16(hipStream_t s, const void* x, int x_dtype, uint32_t m, uint32_t k, uint32_t x_stride,
+                                     uint16_t* out, uint32_t out_stride) {
     if (m > 65535u) return fail(MI355Q_ERR_SHAPE, "more than 65535 activation rows");
     uint32_t gx = (k + 255) / 256;
     if (gx > 256) gx = 256;
-    split_f32_bf16x3_kernel<<<dim3(gx, m), dim3(256), 0, s>>>(x, m, k, x_stride, out, out_stride);
+    if (x_dtype == MI355Q_F32) split_rows_bf16_kernel<3, false><<<dim3(gx, m), dim3(256), 0, s>>>(x, m, k, x_stride, out, out_stride);
+    else if (x_dtype == MI355Q_F16) split_rows_bf16_kernel<2, true><<<dim3(gx, m), dim3(256), 0, s>>>(x, m, k, x_stride, out, out_stride);
+    else return fail(MI355Q_ERR_INVALID_ARGUMENT, "only f16 and fp32 rows are split into bf16 rows");
     MI355Q_HIP(hipGetLastError());
     return MI355Q_OK;
 }
 
-mi355q_status launch_sum3_rows(hipStream_t s, const float* y3, uint32_t m, uint32_t n, void* y, int y_dtype, uint32_t y_stride) {
+mi355q_status launch_sum_parts_rows(hipStream_t s, const float* yp, uint32_t parts, uint32_t m, uint32_t n, void* y, int y_dtype,
+                                    uint32_t y_stride) {
     if (m > 65535u) return fail(MI355Q_ERR_SHAPE, "more than 65535 rows");
     uint32_t gx = (n + 255) / 256;
     if (gx > 256) gx = 256;
-    sum3_rows_kernel<<<dim3(gx, m), dim3(256), 0, s>>>(y3, m, n, y, y_dtype, y_stride);
+    sum_parts_rows_kernel<<<dim3(gx, m), dim3(256), 0, s>>>(yp, parts, m, n, y, y_dtype, y_stride);
     MI355Q_HIP(hipGetLastError());
     return MI355Q_OK;
 }

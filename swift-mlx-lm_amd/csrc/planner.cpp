@@ -47,12 +47,14 @@ void plan_small_m(const mi355q_weight* w, uint32_t m, int x_dtype, uint32_t x_st
                   mi355q_step* s) {
     const WView v = w->view();
     const bool forced = flags & MI355Q_FLAG_FORCE_GENERIC;
-    if (split_f32_chosen(v, x_dtype, m, flags)) {
-        // fp32 rows as three bf16 rows each on the bf16 decode kernel, then the sum of the three partial results
-        plan_small_m(w, 3 * m, MI355Q_BF16, split_f32_row_stride((uint32_t)w->k), flags, s);
+    if (split_rows_chosen(v, x_dtype, m, x_stride, flags)) {
+        // fp32 / f16 rows as three / two bf16 rows each on the bf16 decode kernel, then the sum of the partial results
+        const uint32_t parts = split_rows_parts(x_dtype);
+        plan_small_m(w, parts * m, MI355Q_BF16, split_rows_stride((uint32_t)w->k), flags, s);
         char inner[sizeof s->device_kernel];
         std::snprintf(inner, sizeof inner, "%s", s->device_kernel);
-        std::snprintf(s->device_kernel, sizeof s->device_kernel, "split_f32_bf16x3+%.30s", inner);
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "split_%s_bf16x%u+%.30s", x_dtype == MI355Q_F32 ? "f32" : "f16",
+                      parts, inner);
         return;
     }
     // rows per launch on the tile layout: 16, or fewer when K is so long that 16 staged rows overflow LDS
@@ -221,9 +223,9 @@ mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w, uint32_t maximum
     const uint32_t m = maximum_sequence_length;
     const uint32_t small_rows = small_batch_rows(v, x_dtype, input_row_stride);   // rows the decode kernels take per launch
     const bool want_small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) || m <= small_rows ||
-                            split_f32_chosen(v, x_dtype, m, flags);
+                            split_rows_chosen(v, x_dtype, m, input_row_stride, flags);
     const bool mfma_ok = gemm_mfma_eligible(v, x_dtype, m, input_row_stride);
-    if (!split_f32_chosen(v, x_dtype, m, flags) && gemm_two_step_chosen(v, x_dtype, m, input_row_stride, flags)) {
+    if (!split_rows_chosen(v, x_dtype, m, input_row_stride, flags) && gemm_two_step_chosen(v, x_dtype, m, input_row_stride, flags)) {
         // dequant_q{b}_g{g}_bf16 into the scratch matrix, then the dense GEMM (MetalPrefillStepBuilder's two-dispatch
         // route; the dense product is the platform library's, as the reference's is matmul2d)
         *out_count = 2;

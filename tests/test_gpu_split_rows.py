@@ -1,7 +1,8 @@
-"""GPU parity tests of fp32 activations at a few rows (the f32s signatures of gemv_q{b}_g{g} / gemm_q{b}_g{g},
-Sources/MetalCompiler/Generator/MetalSourceGenerator+Quantized.swift:496-575, :22-156) through the C ABI.  Every fp32
-row is split on the device into three bf16 rows whose sum is the row exactly; the bf16 decode kernel of the layout runs
-on the 3 M rows and the three partial results of a row are added, so the matrix is read once and every product is exact.
+"""GPU parity tests of fp32 and f16 activations at a few rows on the bf16 decode kernels (the f32s and f16 signatures of
+gemv_q{b}_g{g} / gemm_q{b}_g{g}, Sources/MetalCompiler/Generator/MetalSourceGenerator+Quantized.swift:496-575, :22-156)
+through the C ABI.  Every fp32 row is split on the device into three bf16 rows whose sum is the row exactly (an f16 row
+into two); the bf16 decode kernel of the layout runs on those rows and the partial results of a row are added, so the
+matrix is read once per launch and every product is exact.
 
 Bars: against an fp64 accumulation of the dequantised weights and the UNROUNDED fp32 activations, relative L2 <= 1e-5
 (rounding the activations to bf16 would give 1e-3); a case that needs all three parts and is exactly representable is
@@ -23,15 +24,16 @@ def say(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def run_f32(ctx, pkg, w, x, y_dtype=None, flags=0, xpad=0, ypad=0, use_qgemm=False):
+def run_f32(ctx, pkg, w, x, y_dtype=None, flags=0, xpad=0, ypad=0, use_qgemm=False, x_dtype=None):
     y_dtype = pkg.F32 if y_dtype is None else y_dtype
+    x_dtype = pkg.F32 if x_dtype is None else x_dtype
     m, k = x.shape
     n = int(w.info.n_rows)
-    xh = np.full((m, k + xpad), 1e30, np.float32); xh[:, :k] = x
-    xd = ctx.upload(xh)
+    xh = np.full((m, k + xpad), 6e4, np.float32); xh[:, :k] = x
+    xd = ctx.upload(xh if x_dtype == pkg.F32 else xh.astype(np.float16).view(np.uint16))
     yd = ctx.alloc(m * (n + ypad) * (4 if y_dtype == pkg.F32 else 2))
     ctx.fill(yd, 0x7FC07FC0 if y_dtype != pkg.F32 else 0x7FC00000)
-    (ctx.qgemm if use_qgemm else ctx.qgemv)(w, xd, pkg.F32, yd, y_dtype, m, k + xpad, (n + ypad) if ypad else 0, flags)
+    (ctx.qgemm if use_qgemm else ctx.qgemv)(w, xd, x_dtype, yd, y_dtype, m, k + xpad, (n + ypad) if ypad else 0, flags)
     ctx.synchronize()
     y = out_from_device(yd, y_dtype, (m, n + ypad), pkg)
     xd.free(); yd.free()
@@ -140,3 +142,39 @@ def test_f32_rows_non_finite_activation_and_graph_replay(pkg, ctx):
         assert np.array_equal(yd.download(np.float32, (m, n)), eager)
     plan.destroy(); ctx.stream_destroy(stream)
     xd.free(); yd.free(); w.destroy()
+
+
+@pytest.mark.parametrize("layout", ["tile16", "planes"])
+def test_f16_rows_as_two_bf16_rows(pkg, ctx, layout):
+    """f16 activations where the bf16 matrix-core kernels are the faster or the only decode kernels: TILE16 records (no
+    kernel reads f16 there) from one row to twenty-four, 4-bit planes from five rows (below, the f16 dot-product
+    kernels) to sixteen.  One-hot rows with an 11-bit value (1024 + odd) / 2048, which needs both bf16 parts, must come
+    out bit for bit; seeded f16 rows to 1e-5 of the fp64 reference on the same f16 values."""
+    lay = {"planes": pkg.LAYOUT_PLANES, "tile16": pkg.LAYOUT_TILE16}[layout]
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+    rng = np.random.default_rng(5500)
+    n, k = 130, 1024
+    codes = rng.integers(0, 16, (n, k), dtype=np.uint8)
+    scales = rng.choice([0.5, 1.0, 2.0], (n, k // 64)); zeros = rng.integers(-4, 5, (n, k // 64)).astype(np.float64)
+    case = Case(4, 64, codes, scales, zeros)
+    wq = scales.repeat(64, axis=1) * codes + zeros.repeat(64, axis=1)
+    w = ctx.weight_prepare_mlx(fmt, *case.planes(pkg.BF16, pkg), pkg.BF16, lay)
+    split_ms = [1, 2, 5, 8, 13, 24] if layout == "tile16" else [5, 8, 13, 16]
+    other_ms = [25] if layout == "tile16" else [1, 4, 17]
+    for m in split_ms + other_ms:
+        say(f"f16 rows {layout} M={m}")
+        st = w.plan_prefill_steps(m, x_dtype=pkg.F16)[0]
+        assert st.device_kernel.startswith("split_f16_bf16x2+") == (m in split_ms), (m, st.device_kernel)
+        x = np.zeros((m, k), np.float32)
+        pos = rng.choice(k, m, replace=False)
+        for r in range(m):
+            x[r, pos[r]] = np.float32((1024 + 2 * int(rng.integers(0, 512)) + 1) / 2048.0) * (-1) ** r
+        want = x.astype(np.float64) @ wq.T
+        got = run_f32(ctx, pkg, w, x, use_qgemm=True, x_dtype=pkg.F16, xpad=8 if m % 2 else 0)
+        assert np.array_equal(got.astype(np.float64), want), (layout, m)
+        x = kat.seeded_activations(5510 + m, m, k).astype(np.float16).astype(np.float32)
+        got = run_f32(ctx, pkg, w, x, use_qgemm=True, x_dtype=pkg.F16)
+        assert rel_l2(got, oracle.gemm_f64(wq, x)) <= (1e-5 if m in split_ms else 1e-3), (layout, m)
+        if m <= 8:
+            assert np.array_equal(run_f32(ctx, pkg, w, x, x_dtype=pkg.F16), got)
+    w.destroy()

@@ -403,8 +403,8 @@ def test_tile16_plan_replay_and_graph(pkg, ctx):
 
 @pytest.mark.parametrize("x_dtype_name", ["F16", "F32"])
 def test_tile16_other_activation_types_take_the_per_code_kernel_whole(pkg, ctx, x_dtype_name):
-    """The tile kernel reads bf16 activations only.  Up to sixteen fp32 rows run on it as three bf16 rows each; beyond,
-    and f16 rows from the second on, take the two-dispatch route
+    """The tile kernel reads bf16 activations only.  Up to sixteen fp32 rows run on it as three bf16 rows each, up to
+    twenty-four f16 rows as two; beyond, rows take the two-dispatch route
     (the matrix dequantised to the activations' type, then the dense library GEMM; fp32 from sixteen rows: bf16
     weights against split activations); forced, the per-code kernel takes all rows in one launch (no walk in steps
     of sixteen, eight ... one row)."""
@@ -418,8 +418,9 @@ def test_tile16_other_activation_types_take_the_per_code_kernel_whole(pkg, ctx, 
         # from sixteen rows fp32 activations meet bf16 weights (the reference's gemm_bf16_f32s); f16 ones f16 weights
         weights = wq if m < 16 or x_dtype == pkg.F16 else oracle.bf16_to_f32(oracle.bf16_from_f32(wq)).reshape(wq.shape)
         assert_within_tolerance(got, oracle.gemm_f64(weights, x), f"{x_dtype_name} M={m}")
-        if x_dtype == pkg.F32 and m <= 16:
-            assert w.plan_prefill_steps(m, x_dtype=x_dtype)[0].device_kernel == "split_f32_bf16x3+gemv_tile16_q4_g64"
+        if m <= 16:
+            parts = "f32_bf16x3" if x_dtype == pkg.F32 else "f16_bf16x2"
+            assert w.plan_prefill_steps(m, x_dtype=x_dtype)[0].device_kernel == f"split_{parts}+gemv_tile16_q4_g64"
         elif m > 1:
             assert w.plan_prefill_steps(m, x_dtype=x_dtype)[0].kernel_family in ("libraryGEMM", "dequantToBFloat")
         slow = run_gemv(ctx, pkg, w, x, x_dtype, pkg.F32, pkg.FLAG_FORCE_GENERIC, use_qgemm=True)
