@@ -258,10 +258,10 @@ MI355Q_API mi355q_status mi355q_weight_destroy(mi355q_weight* w);
  * Activation types: bf16 and f16 rows are read by the decode kernels directly.  fp32 rows are split on the
  * device into three bf16 rows each whose sum is the fp32 row exactly (8 + 8 + 8 significant bits); the bf16
  * kernel of the layout runs on the 3 M rows (the matrix is still read once, every product is exact) and a small
- * launch adds the three partial results of a row.  f16 rows go the same way as two bf16 rows each (8 + 3 bits)
- * where only a bf16 kernel reads the layout (TILE16 records) or the bf16 matrix-core kernel is the faster one
- * (4- and 8-bit planes from five rows).  The split rows and partial results live in a scratch buffer of the
- * context, grown on first use. */
+ * launch adds the three partial results of a row (the split rows and partial results live in a scratch buffer
+ * of the context, grown on first use).  The matrix-core kernels (TILE16 records; 4- and 8-bit planes from three
+ * rows) split f16 rows into two bf16 rows each (8 + 3 bits) while staging them, and add the two results of a
+ * row before the store: eight f16 rows a launch. */
 MI355Q_API mi355q_status mi355q_qgemv(mi355q_context* ctx, void* stream, const mi355q_weight* w,
                                       const void* x_dev, mi355q_dtype x_dtype, void* y_dev,
                                       mi355q_dtype y_dtype, uint32_t m, uint32_t x_row_stride,
@@ -273,7 +273,8 @@ MI355Q_API mi355q_status mi355q_qgemv(mi355q_context* ctx, void* stream, const m
  * MC/Compiler/MetalPrefillStepBuilder.swift:728-732).  Three routes, all with the weights rounded once
  * to bf16 and fp32 accumulation, chosen by measured cost unless flags say otherwise
  * (mi355q_plan_prefill_steps reports the choice):
- *   - small M (up to 8 rows; 16 on TILE16 records and on q4 / q8 planes): the GEMV-style decode kernels;
+ *   - small M (up to 8 rows; 16 on TILE16 records and on q4 / q8 planes, and there up to 32 in two launches):
+ *     the GEMV-style decode kernels;
  *   - ONE fused kernel: code tiles are dequantised to bf16 in LDS and contracted on MFMA (the planes
  *     and TILE16 layouts, formats q4 g64/g128, q8 g32/g64, q6/q3/q2 g64, bf16 activations);
  *   - two dispatches, as the reference's second route: the whole matrix is dequantised to bf16 in a

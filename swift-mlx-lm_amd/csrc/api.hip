@@ -61,12 +61,12 @@ mi355q_status run_small_m(mi355q_context* ctx, hipStream_t s, const mi355q_weigh
         if (!generic && gemv_tile16_eligible(v, x_dtype, mm, xs) && (uintptr_t)xp % 16 == 0) {
             void* yv[1] = {yp};
             const uint32_t strides[1] = {ys};
-            st = launch_gemv_tile16_multi(s, ctx, 1, &v, xp, yv, strides, y_dtype, mm, xs, nullptr, nullptr, HeadKeys{});
-        } else if (!generic && mm >= mfma_planes_min_rows(v.bits) && gemv_mfma_planes_eligible(v, x_dtype, mm, xs) &&
+            st = launch_gemv_tile16_multi(s, ctx, 1, &v, xp, x_dtype, yv, strides, y_dtype, mm, xs, nullptr, nullptr, HeadKeys{});
+        } else if (!generic && mfma_planes_pays(v.bits, x_dtype, mm) && gemv_mfma_planes_eligible(v, x_dtype, mm, xs) &&
                    (uintptr_t)xp % 16 == 0) {
             void* yv[1] = {yp};
             const uint32_t strides[1] = {ys};
-            st = launch_gemv_mfma_planes_multi(s, ctx, 1, &v, xp, yv, strides, y_dtype, mm, xs);
+            st = launch_gemv_mfma_planes_multi(s, ctx, 1, &v, xp, x_dtype, yv, strides, y_dtype, mm, xs);
         } else if (!generic && gemv_fast_eligible(v, x_dtype, mm > 8 ? 8 : mm, xs) && (uintptr_t)xp % 16 == 0) {
             // the dot-product kernels take eight rows a launch
             st = MI355Q_OK;
@@ -84,9 +84,9 @@ mi355q_status run_small_m(mi355q_context* ctx, hipStream_t s, const mi355q_weigh
     return MI355Q_OK;
 }
 
-// fp32 or f16 activations, a few rows, on a weight the bf16 decode kernels read: every row becomes three (fp32) or two
-// (f16) bf16 rows whose sum is the row exactly (split_rows_bf16_kernel), the bf16 kernels run on those rows, and the
-// partial results of a row are added.  Products stay exact, the matrix is read once per launch of sixteen or eight rows.
+// fp32 activations, a few rows, on a weight the bf16 decode kernels read: every row becomes three bf16 rows whose sum
+// is the row exactly (split_rows_bf16_kernel), the bf16 kernels run on those rows, and the partial results of a row are
+// added.  Products stay exact, the matrix is read once per launch of sixteen or eight rows.
 mi355q_status run_split_rows(mi355q_context* ctx, hipStream_t s, const mi355q_weight* w, const void* x, int x_dtype, void* y,
                              int y_dtype, uint32_t m, uint32_t xs, uint32_t ys, uint32_t flags) {
     const uint32_t n = (uint32_t)w->n, k = (uint32_t)w->k, kp = split_rows_stride(k), parts = split_rows_parts(x_dtype);
@@ -103,23 +103,19 @@ mi355q_status run_split_rows(mi355q_context* ctx, hipStream_t s, const mi355q_we
 
 namespace mi355q {
 
-// Whether m rows of fp32 or f16 activations are served as bf16 rows on the bf16 decode kernels.
-//   fp32: no kernel but the per-code one reads it; taken when a bf16 decode kernel reads the weight and the 3 m rows fit
-//   one launch of it -- three launches where a launch takes sixteen rows (4096 -> 14336 on 4-bit planes: 16-20 us up to
-//   five rows, 52 us at sixteen, where the dequantise-once route takes 105 us whatever the rows; with launches of eight
-//   rows two rows already take 35 us).
-//   f16: where no decode kernel reads f16 (TILE16 records), under the same limits; and on planes that the matrix-core
-//   kernel reads in bf16, from five rows (the f16 dot-product kernels take four rows a launch) to sixteen.
+// Whether m rows of fp32 activations are served as three bf16 rows each on the bf16 decode kernels: no kernel but the
+// per-code one reads fp32; taken when a bf16 decode kernel reads the weight and the 3 m rows fit one launch of it --
+// three launches where a launch takes sixteen rows (4096 -> 14336 on 4-bit planes: 16-20 us up to five rows, 52 us at
+// sixteen, where the dequantise-once route takes 105 us whatever the rows; with launches of eight rows two rows already
+// take 35 us).  (f16 rows need no such route: the matrix-core kernels stage them as two bf16 rows themselves.)
 bool split_rows_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride, uint32_t flags) {
+    (void)x_stride;
     const uint32_t parts = split_rows_parts(x_dtype);
     if (!parts || (flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_TWO_STEP))) return false;
     const uint32_t kp = split_rows_stride((uint32_t)w.k);
     if (!decode_kernel_reads(w, MI355Q_BF16, kp)) return false;
     const uint32_t rows = small_batch_rows(w, MI355Q_BF16, kp);
-    const uint64_t most = rows >= 16 ? 3 * rows : rows;
-    if (x_dtype == MI355Q_F16 && decode_kernel_reads(w, MI355Q_F16, x_stride))
-        return rows >= 16 && m >= 5 && 2 * (uint64_t)m <= 2 * rows;
-    return (uint64_t)parts * m <= most;
+    return (uint64_t)parts * m <= (rows >= 16 ? 3 * rows : rows);
 }
 
 mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_weight* w, const void* x, int x_dtype,
@@ -164,16 +160,25 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
             return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the MFMA GEMM does not accept this format, layout or stride");
         return launch_qgemm_mfma(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys, probe);
     }
-    // the decode kernels take up to 8 rows per launch on the planes, 16 on TILE16 records
-    const uint32_t small_rows = small_batch_rows(v, x_dtype, xs);
-    const bool small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) || m <= small_rows || !mfma_ok;
+    // the decode kernels take up to 8 rows per launch, 16 on the matrix cores (and then pay for a second launch too)
+    const bool small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) ||
+                       m <= small_batch_limit(v, x_dtype, xs) || !mfma_ok;
     if (small) return run_small_m(ctx, s, w, x, x_dtype, y, y_dtype, m, xs, ys, flags);
     return launch_qgemm_mfma(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys, probe);
 }
 
+// Rows up to which the small-batch kernels, one launch after the other, beat the fused prefill kernel: two launches where
+// a launch takes sixteen rows (a Llama-3-8B layer step in bf16: 24 rows 124 us in two launches against 159 us on the
+// prefill kernel, 32 rows 136 against 161).
+uint32_t small_batch_limit(const WView& w, int x_dtype, uint32_t x_stride) {
+    const uint32_t rows = small_batch_rows(w, x_dtype, x_stride);
+    return rows >= 16 ? 2 * rows : rows;
+}
+
 uint32_t small_batch_rows(const WView& w, int x_dtype, uint32_t x_stride) {
-    if (w.layout == MI355Q_LAYOUT_TILE16) return 16;
-    return gemv_mfma_planes_eligible(w, x_dtype, 16, x_stride) ? 16 : 8;
+    const uint32_t most = x_dtype == MI355Q_F16 ? 8 : 16;      // sixteen staged rows: f16 rows are staged as two each
+    if (w.layout == MI355Q_LAYOUT_TILE16) return most;
+    return gemv_mfma_planes_eligible(w, x_dtype, most, x_stride) ? most : 8;
 }
 
 // Whether one of the decode kernels (not the per-code kernel) takes this layout with this activation type.
@@ -192,8 +197,14 @@ bool gemm_two_step_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_st
     if (flags & (MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) return false;
     if (flags & MI355Q_FLAG_FORCE_TWO_STEP) return true;
     if (!gemm_two_step_eligible(w, x_dtype, m, x_stride)) return false;
-    if (!gemm_mfma_eligible(w, x_dtype, m, x_stride))
-        return m >= kTwoStepMinRowsOtherwise || (m >= 2 && !decode_kernel_reads(w, x_dtype, x_stride));
+    if (!gemm_mfma_eligible(w, x_dtype, m, x_stride)) {
+        if (!decode_kernel_reads(w, x_dtype, x_stride)) return m >= 2;
+        // f16 rows on the matrix-core decode kernels, eight a launch: a Llama-3-8B layer step takes 56-67 us per eight
+        // rows there and 255-296 us on this route whatever the rows
+        const bool f16_on_matrix_cores = x_dtype == MI355Q_F16 && (gemv_tile16_eligible(w, x_dtype, 8, x_stride) ||
+                                                                   gemv_mfma_planes_eligible(w, x_dtype, 8, x_stride));
+        return m >= (f16_on_matrix_cores ? kTwoStepMinRowsF16Batches : kTwoStepMinRowsOtherwise);
+    }
     return m >= (w.k > w.n ? kTwoStepMinRowsLongK : kTwoStepMinRowsBesideFused);
 }
 
@@ -296,7 +307,7 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
     bool fused = m <= 8 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
     bool tiled = m <= 16 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
     bool in_place = m <= 8 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
-    bool on_planes = m >= mfma_planes_min_rows(weights[0]->fmt.bits) && m <= 16 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
+    bool on_planes = mfma_planes_pays(weights[0]->fmt.bits, x_dtype, m) && m <= 16 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
     WView views[3];
     uint32_t strides[3];
     for (uint32_t i = 0; i < count; i++) {
@@ -306,22 +317,63 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
         strides[i] = y_stride;
         views[i] = weights[i]->view();
         fused = fused && gemv_fast_eligible(views[i], x_dtype, m, xs) && views[i].sb_dtype == views[0].sb_dtype;
-        tiled = tiled && gemv_tile16_eligible(views[i], x_dtype, m, xs) && gemv_tile16_k_parts(ctx, views[i], m) == 1 &&
+        tiled = tiled && gemv_tile16_eligible(views[i], x_dtype, m, xs) &&
+                gemv_tile16_k_parts(ctx, views[i], staged_rows(x_dtype, m)) == 1 &&
                 views[i].sb_dtype == views[0].sb_dtype;
         in_place = in_place && gemv_staf_eligible(views[i], x_dtype, m, xs);
         on_planes = on_planes && gemv_mfma_planes_eligible(views[i], x_dtype, m, xs) &&
-                    gemv_mfma_planes_k_parts(ctx, views[i], m) == 1 && views[i].sb_dtype == views[0].sb_dtype &&
+                    gemv_mfma_planes_k_parts(ctx, views[i], staged_rows(x_dtype, m)) == 1 && views[i].sb_dtype == views[0].sb_dtype &&
                     views[i].code_stride == views[0].code_stride && views[i].group == views[0].group;
     }
     if (on_planes && (uintptr_t)x % 16 == 0)
-        return launch_gemv_mfma_planes_multi(s, ctx, count, views, x, ys, strides, y_dtype, m, xs);
+        return launch_gemv_mfma_planes_multi(s, ctx, count, views, x, x_dtype, ys, strides, y_dtype, m, xs);
     if (fused && (uintptr_t)x % 16 == 0)
         return launch_gemv_fast_multi(s, ctx, count, views, x, x_dtype, ys, strides, y_dtype, m, xs, nullptr, nullptr, HeadKeys{});
     if (tiled && (uintptr_t)x % 16 == 0)
-        return launch_gemv_tile16_multi(s, ctx, count, views, x, ys, strides, y_dtype, m, xs, nullptr, nullptr,
+        return launch_gemv_tile16_multi(s, ctx, count, views, x, x_dtype, ys, strides, y_dtype, m, xs, nullptr, nullptr,
                                         HeadKeys{});
     if (in_place && (uintptr_t)x % 16 == 0)
         return launch_gemv_staf_multi(s, ctx, count, views, x, x_dtype, ys, strides, y_dtype, m, xs, nullptr, nullptr, HeadKeys{});
+    // fp32 / f16 rows that go to the bf16 kernels as bf16 rows (split_rows_chosen): split once for all projections, one
+    // shared bf16 launch on those rows where they fit one, one sum per projection
+    const uint32_t parts = split_rows_parts(x_dtype);
+    bool split = parts && parts * (uint64_t)m <= 16;
+    for (uint32_t i = 0; i < count && split; i++) split = split_rows_chosen(views[i], x_dtype, m, xs, flags);
+    if (split) {
+        const uint32_t k = (uint32_t)views[0].k, kp = split_rows_stride(k);
+        const size_t xbytes = ((size_t)parts * m * kp * 2 + 255) & ~(size_t)255;
+        size_t ybytes[3] = {0, 0, 0}, total = xbytes;
+        for (uint32_t i = 0; i < count; i++) total += ybytes[i] = ((size_t)parts * m * views[i].n * 4 + 255) & ~(size_t)255;
+        if (mi355q_status st = ensure_split_buffer(ctx, total)) return st;
+        char* const base = (char*)ctx->split_buffer;
+        void* yps[3] = {nullptr, nullptr, nullptr};
+        size_t at = xbytes;
+        for (uint32_t i = 0; i < count; i++) { yps[i] = base + at; at += ybytes[i]; }
+        if (mi355q_status st = launch_split_rows_bf16(s, x, x_dtype, m, k, xs, (uint16_t*)base, kp)) return st;
+        if (mi355q_status st = dispatch_batched(ctx, s, count, weights, base, MI355Q_BF16, yps, MI355Q_F32, parts * m, kp, flags))
+            return st;
+        for (uint32_t i = 0; i < count; i++)
+            if (mi355q_status st = launch_sum_parts_rows(s, (const float*)yps[i], parts, m, (uint32_t)views[i].n, ys[i], y_dtype,
+                                                         strides[i])) return st;
+        return MI355Q_OK;
+    }
+    // more rows than one shared launch takes, served by the small-batch kernels all the same: the shared launch in steps
+    const uint32_t step = small_batch_rows(views[0], x_dtype, xs);
+    bool stepped = m > step && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_TWO_STEP));
+    for (uint32_t i = 0; i < count && stepped; i++)
+        stepped = decode_kernel_reads(views[i], x_dtype, xs) && !split_rows_chosen(views[i], x_dtype, m, xs, flags) &&
+                  !gemm_two_step_chosen(views[i], x_dtype, m, xs, flags) &&
+                  (m <= small_batch_limit(views[i], x_dtype, xs) || !gemm_mfma_eligible(views[i], x_dtype, m, xs));
+    if (stepped) {
+        const size_t xsz = x_dtype == MI355Q_F32 ? 4 : 2, ysz = y_dtype == MI355Q_F32 ? 4 : 2;
+        for (uint32_t m0 = 0; m0 < m; m0 += step) {
+            void* yc[3] = {nullptr, nullptr, nullptr};
+            for (uint32_t i = 0; i < count; i++) yc[i] = (char*)ys[i] + (size_t)m0 * strides[i] * ysz;
+            if (mi355q_status st = dispatch_batched(ctx, s, count, weights, (const char*)x + (size_t)m0 * xs * xsz, x_dtype, yc,
+                                                    y_dtype, m - m0 < step ? m - m0 : step, xs, flags)) return st;
+        }
+        return MI355Q_OK;
+    }
     for (uint32_t i = 0; i < count; i++) {
         mi355q_status st = dispatch_linear(ctx, s, weights[i], x, x_dtype, ys[i], y_dtype, m, xs, 0, flags, false);
         if (st != MI355Q_OK) return st;
@@ -340,11 +392,11 @@ mi355q_status dispatch_output_head(mi355q_context* ctx, hipStream_t s, const mi3
     if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && gemv_fast_eligible(v, x_dtype, 1, xs) && (uintptr_t)x % 16 == 0)
         return launch_gemv_fast(s, ctx, v, x, x_dtype, nullptr, MI355Q_F32, 1, xs, (uint32_t)w->n, logits, token,
                                 keys);
-    if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && gemv_tile16_eligible(v, x_dtype, 1, xs) && gemv_tile16_k_parts(ctx, v, 1) == 1 &&
-        (uintptr_t)x % 16 == 0) {
+    if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && x_dtype == MI355Q_BF16 && gemv_tile16_eligible(v, x_dtype, 1, xs) &&
+        gemv_tile16_k_parts(ctx, v, 1) == 1 && (uintptr_t)x % 16 == 0) {
         void* none[1] = {nullptr};
         const uint32_t strides[1] = {(uint32_t)w->n};
-        return launch_gemv_tile16_multi(s, ctx, 1, &v, x, none, strides, MI355Q_F32, 1, xs, logits, token,
+        return launch_gemv_tile16_multi(s, ctx, 1, &v, x, x_dtype, none, strides, MI355Q_F32, 1, xs, logits, token,
                                         keys);
     }
     if (!(flags & MI355Q_FLAG_FORCE_GENERIC) && gemv_staf_eligible(v, x_dtype, 1, xs) && (uintptr_t)x % 16 == 0) {

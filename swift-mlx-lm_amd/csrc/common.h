@@ -194,8 +194,11 @@ struct Tile16LaunchShape {
     uint32_t parts;      // K parts (1: whole rows); each part has wgs_per_part workgroups and stages only its columns
     uint32_t wgs_per_part;
 };
+// Rows the matrix-core decode kernels stage for m activation rows: an f16 row is staged as two bf16 rows (gemv_tile16.hip)
+inline uint32_t staged_rows(int x_dtype, uint32_t m) { return x_dtype == MI355Q_F16 ? 2 * m : m; }
 bool gemv_tile16_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
 // K parts a launch of M rows takes: 1 = whole rows (needed by fused q+k+v / gate+up launches and by the fused head)
+// (m: staged rows, see staged_rows)
 uint32_t gemv_tile16_k_parts(const mi355q_context* ctx, const WView& w, uint32_t m);
 // the same for a shape: 0 when no power-of-two split of K leaves M staged rows inside LDS
 // block_codes: codes in 64 bytes of a weight row (128 at 4 bits)
@@ -203,7 +206,7 @@ uint32_t gemv_tile16_parts_for(uint32_t k, uint32_t m, uint32_t n_row_tiles, uin
 Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_row_tiles, uint32_t k, uint32_t m,
                                     uint32_t block_codes = 128);
 mi355q_status launch_gemv_tile16_multi(hipStream_t s, mi355q_context* ctx, uint32_t count, const WView* w,
-                                       const void* x, void* const* y, const uint32_t* y_strides, int y_dtype,
+                                       const void* x, int x_dtype, void* const* y, const uint32_t* y_strides, int y_dtype,
                                        uint32_t m, uint32_t x_stride, float* logits_f32, int32_t* token_out,
                                        HeadKeys keys);
 mi355q_status launch_tile16_pack(hipStream_t s, const WView& planes, uint32_t* tiles);
@@ -215,15 +218,23 @@ mi355q_status launch_tile16_pack(hipStream_t s, const WView& planes, uint32_t* t
 // fewest activation rows for which the matrix-core kernel beats the dot-product kernels on the same planes (measured;
 // 8 bits, 4096 -> 14336: two rows 16 us on the dot products, three 25 us, against 19 us on the matrix cores)
 inline uint32_t mfma_planes_min_rows(uint32_t bits) { return bits == 8 ? 3u : 4u; }
+// f16 rows are staged as two bf16 rows each: three f16 rows (six staged) pay on the matrix cores, two stay on the f16
+// dot-product kernels (a Llama-3-8B layer step at two f16 rows: 42.6 us there)
+inline bool mfma_planes_pays(uint32_t bits, int x_dtype, uint32_t m) {
+    return x_dtype == MI355Q_F16 ? m >= 3 : m >= mfma_planes_min_rows(bits);
+}
 bool gemv_mfma_planes_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
+// (m below: staged rows, see staged_rows)
 uint32_t gemv_mfma_planes_k_parts(const mi355q_context* ctx, const WView& w, uint32_t m);
 Tile16LaunchShape gemv_mfma_planes_shape(const mi355q_context* ctx, uint32_t n_row_tiles, uint32_t k, uint32_t bits, uint32_t m);
 mi355q_status launch_gemv_mfma_planes_multi(hipStream_t s, mi355q_context* ctx, uint32_t count, const WView* w,
-                                            const void* x, void* const* y, const uint32_t* y_strides, int y_dtype,
+                                            const void* x, int x_dtype, void* const* y, const uint32_t* y_strides, int y_dtype,
                                             uint32_t m, uint32_t x_stride);
 // Rows one launch of the small-batch kernels takes for this weight: 16 on TILE16 records and on planes the
 // matrix-core kernel reads, else 8.
 uint32_t small_batch_rows(const WView& w, int x_dtype, uint32_t x_stride);
+// Rows up to which mi355q_qgemm stays on those kernels (launch after launch) before the fused prefill kernel takes over
+uint32_t small_batch_limit(const WView& w, int x_dtype, uint32_t x_stride);
 
 // Validated dispatch shared by the direct entry points and by plan replay (api.hip)
 mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t count, const mi355q_weight* const* weights,
@@ -245,10 +256,10 @@ GemmLaunchShape gemm_mfma_shape(const mi355q_context* ctx, uint32_t m, uint32_t 
 // Grows the context's scratch buffer for fp32 partial results; nothing is released before the context goes.
 mi355q_status ensure_workspace(mi355q_context* ctx, size_t bytes);
 mi355q_status ensure_split_buffer(mi355q_context* ctx, size_t bytes);
-// fp32 / f16 activations as three / two bf16 rows each on the bf16 decode kernels (api.hip): row pitch of the bf16
-// rows, bf16 rows per activation row (0: the type is not split), and whether a call takes that route
+// fp32 activations as three bf16 rows each on the bf16 decode kernels (api.hip): row pitch of the bf16 rows, bf16 rows
+// per activation row (0: the type is not split), and whether a call takes that route
 inline uint32_t split_rows_stride(uint32_t k) { return (k + 7u) & ~7u; }
-inline uint32_t split_rows_parts(int x_dtype) { return x_dtype == MI355Q_F32 ? 3u : x_dtype == MI355Q_F16 ? 2u : 0u; }
+inline uint32_t split_rows_parts(int x_dtype) { return x_dtype == MI355Q_F32 ? 3u : 0u; }
 bool split_rows_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride, uint32_t flags);
 bool gemm_mfma_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
 mi355q_status launch_qgemm_mfma(hipStream_t s, mi355q_context* ctx, const WView& w,
@@ -271,7 +282,9 @@ void dense_library_release(mi355q_context* ctx);
 // M = 1024 141-150 against 162-168 us, M = 2048 260-285 against 244-256 us, M = 4096 458-520 against 338-347 us.
 // Where only the decode kernels would serve (formats and layouts the fused kernel does not read; block layout,
 // 4096 -> 14336: M = 32 in four launches of eight rows 147 us, two-dispatch 47 us) it starts at sixteen rows.
+// f16 rows that the matrix-core decode kernels take eight a launch: from 32 rows.
 constexpr uint32_t kTwoStepMinRowsBesideFused = 1024, kTwoStepMinRowsLongK = 2048, kTwoStepMinRowsOtherwise = 16;
+constexpr uint32_t kTwoStepMinRowsF16Batches = 32;
 // Rows from which mi355q_gemm_bf16 hands a plain dense product to the library.
 constexpr uint32_t kDenseLibraryMinRows = 128;
 bool decode_kernel_reads(const WView& w, int x_dtype, uint32_t x_stride);

@@ -50,6 +50,26 @@ __device__ __forceinline__ uint16_t f32_to_f16_rne(float f) {
     return __builtin_bit_cast(uint16_t, (_Float16)f);
 }
 
+// Eight f16 values (four words) as two bf16 vectors whose sum is each value exactly: hi = the upper eight significant
+// bits (the fp32 form cut after its upper half), lo = value - hi (at most three significant bits, so its upper half is
+// all of it).  Non-finite values stay in hi alone.
+__device__ __forceinline__ void f16x8_to_bf16_hi_lo(const u32x4& v, u32x4& hi, u32x4& lo) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    uint32_t h[4], l[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float f0 = f16_to_f32((uint16_t)(w[i] & 0xFFFFu)), f1 = f16_to_f32((uint16_t)(w[i] >> 16));
+        const uint32_t h0 = __float_as_uint(f0) & 0xFFFF0000u, h1 = __float_as_uint(f1) & 0xFFFF0000u;
+        float l0 = f0 - __uint_as_float(h0), l1 = f1 - __uint_as_float(h1);
+        l0 = (f0 - f0 == 0.0f) ? l0 : 0.0f;
+        l1 = (f1 - f1 == 0.0f) ? l1 : 0.0f;
+        h[i] = __builtin_amdgcn_perm(h1, h0, 0x07060302u);
+        l[i] = __builtin_amdgcn_perm(__float_as_uint(l1), __float_as_uint(l0), 0x07060302u);
+    }
+    hi.x = h[0]; hi.y = h[1]; hi.z = h[2]; hi.w = h[3];
+    lo.x = l[0]; lo.y = l[1]; lo.z = l[2]; lo.w = l[3];
+}
+
 __device__ __forceinline__ float sb_to_f32(uint16_t h, uint32_t sb_dtype) {
     return sb_dtype == MI355Q_BF16 ? bf16_to_f32(h) : f16_to_f32(h);
 }

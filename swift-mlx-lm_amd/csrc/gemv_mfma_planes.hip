@@ -49,7 +49,9 @@ struct PmArgs {
     uint32_t tile_end[kPmMaxSegments];         // cumulative 16-row tile counts; unused entries repeat the last
     uint32_t seg_rows[kPmMaxSegments];         // N_i
     uint32_t y_stride[kPmMaxSegments];
-    const uint16_t* x;                         // bf16 [M, x_stride]
+    const uint16_t* x;                         // bf16 or f16 [M, x_stride]
+    uint32_t x_f16;                            // 1: f16 rows, staged as two bf16 rows each (upper eight bits, the rest)
+    uint32_t ms;                               // staged rows (2 M for f16): the M dimension the matrix core works on
     uint32_t k, m, x_stride;
     uint32_t row_words;                        // 32-bit words from one row to the next (codes, then the row's sz words)
     uint32_t sz_offset;                        // words from a row's first code word to its first (scale, bias) word
@@ -179,9 +181,9 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
     // ---- 3. stage the activations: every run of eight as (x0,x4,x1,x5,x2,x6,x3,x7) (8 bits: (x0,x2,x1,x3,x4,x6,x5,x7)),
     //         and sum(x) per half block and row ----------------------------------------------------------------------
     constexpr uint32_t CH = HALF / 8;                       // 16-byte chunks per half block
-    float* const sxs = (float*)(lds + (size_t)(a.m + 1) * a.lds_row_bytes);      // [half block in part][SXR]
+    float* const sxs = (float*)(lds + (size_t)(a.ms + 1) * a.lds_row_bytes);     // [half block in part][SXR]
     {
-        auto stage = [&](uint32_t idx, const u32x4& v) {
+        auto run_sum = [&](const u32x4& v) {
             float p = pm_dot2(v.x, 0x3F803F80u, 0.0f);
             p = pm_dot2(v.y, 0x3F803F80u, p);
             p = pm_dot2(v.z, 0x3F803F80u, p);
@@ -189,8 +191,12 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
             p += __shfl_xor(p, 1);
             p += __shfl_xor(p, 2);
             if constexpr (CH == 8) p += __shfl_xor(p, 4);
-            uint32_t m, c;
-            if (x_at(idx, m, c)) {
+            return p;
+        };
+        // one chunk of a staged row: every run of eight in the operand order of the unpacked codes, and its share of sum(x)
+        auto stage_row = [&](uint32_t m, uint32_t c, bool has, const u32x4& v) {
+            const float p = run_sum(v);
+            if (has) {
                 u32x4 o;
                 if constexpr (BITS == 4) {
                     o.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);    // (x0, x4)
@@ -207,6 +213,18 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
                 if ((c & (CH - 1)) == 0) sxs[(c / CH) * SXR + m] = p;  // CH chunks: one half block
             }
         };
+        auto stage = [&](uint32_t idx, const u32x4& v) {
+            uint32_t m, c;
+            const bool has = x_at(idx, m, c);
+            if (a.x_f16) {                                  // wavefront-uniform: an f16 row becomes staged rows 2 m, 2 m + 1
+                u32x4 hi, lo;
+                f16x8_to_bf16_hi_lo(v, hi, lo);
+                stage_row(2 * m, c, has, hi);
+                stage_row(2 * m + 1, c, has, lo);
+            } else {
+                stage_row(m, c, has, v);
+            }
+        };
         // whole wavefronts take part in the shuffles of every step: the walk is rounded up to whole batches
 #pragma unroll
         for (int t = 0; t < XB; t++)
@@ -220,7 +238,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
                 if (base + (uint32_t)t * NT < total) stage(base + tid + (uint32_t)t * NT, xe[t]);
         }
         const u32x4 zero = {0u, 0u, 0u, 0u};
-        for (uint32_t c = tid; c < chunks; c += NT) *((u32x4*)(lds + (size_t)a.m * a.lds_row_bytes) + c) = zero;
+        for (uint32_t c = tid; c < chunks; c += NT) *((u32x4*)(lds + (size_t)a.ms * a.lds_row_bytes) + c) = zero;
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __builtin_amdgcn_s_barrier();
@@ -239,11 +257,11 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
     // 8..15 are the same activation rows where kq >= 2; elsewhere the row of zeros.  Rows past M read row M-1 (their
     // results are never stored).
     const uint32_t xi = WIDE ? n_in : (n_in & 7u);
-    const uint32_t xr = xi < a.m ? xi : a.m - 1;
+    const uint32_t xr = xi < a.ms ? xi : a.ms - 1;
     const bool live = WIDE ? (kq < 2) : (n_in >> 3) == (kq >> 1);
-    const char* const a_lane = lds + (size_t)(live || (WIDE && !TWO) ? xr : a.m) * a.lds_row_bytes + kq * (XBYTES / 4);
+    const char* const a_lane = lds + (size_t)(live || (WIDE && !TWO) ? xr : a.ms) * a.lds_row_bytes + kq * (XBYTES / 4);
     // WIDE, two groups per block: the second product's operand, live where the first one's is not
-    const char* const a_lane_hi = lds + (size_t)(live ? a.m : xr) * a.lds_row_bytes + kq * (XBYTES / 4);
+    const char* const a_lane_hi = lds + (size_t)(live ? a.ms : xr) * a.lds_row_bytes + kq * (XBYTES / 4);
 
     auto unpack = [&](uint32_t w) -> pm_bf16x8_t {
         u32x4 p;
@@ -393,7 +411,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
     // Partial tiles of the WAVES wavefronts, [WAVES][MR][64]: a single pass writes them over the staged activations
     // once every wavefront is done reading those; several passes keep them behind the activations and their sums.
     const bool red_over_x = a.passes == 1;
-    float* const red = (float*)(red_over_x ? lds : lds + (size_t)(a.m + 1) * a.lds_row_bytes + (size_t)(kp / HALF) * SXR * 4);
+    float* const red = (float*)(red_over_x ? lds : lds + (size_t)(a.ms + 1) * a.lds_row_bytes + (size_t)(kp / HALF) * SXR * 4);
     for (uint32_t pass = 0; pass < a.passes; pass++) {
         if (pass) {                                            // the first tile's loads were issued before staging
             tile = select_tile(pass);
@@ -417,14 +435,22 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
         __syncthreads();
         if (slice == 0 && tile.valid && (WIDE || kq < 2)) { // the first wavefront of each tile adds and stores
             const uint32_t row = tile.n0 + n_in;
+            float vv[MR];
 #pragma unroll
             for (int r = 0; r < MR; r++) {
-                float v = 0.f;
+                vv[r] = 0.f;
                 for (uint32_t w2 = 0; w2 < (uint32_t)KSPLIT; w2++) {     // (not WIDE: both halves of K of every block)
-                    v += red[((wave + w2) * MR + r) * 64 + lane];
-                    if constexpr (!WIDE) v += red[((wave + w2) * MR + r) * 64 + lane + 32];
+                    vv[r] += red[((wave + w2) * MR + r) * 64 + lane];
+                    if constexpr (!WIDE) vv[r] += red[((wave + w2) * MR + r) * 64 + lane + 32];
                 }
-                const uint32_t m = 4 * kq + r;
+            }
+            // f16 rows: staged rows 2 m and 2 m + 1, both in this lane, are the two parts of activation row m
+            const bool fold = a.x_f16;
+#pragma unroll
+            for (int r = 0; r < MR; r++) {
+                if (fold && r >= MR / 2) break;
+                const float v = fold ? vv[(2 * r + 1) % MR] + vv[(2 * r) % MR] : vv[r];
+                const uint32_t m = fold ? 2 * kq + r : 4 * kq + r;
                 if (m < a.m && row < tile.rows) {
                     if (a.parts > 1) {                       // one matrix: the reduction launch converts and stores
                         a.partial[((size_t)part * a.m + m) * tile.rows + row] = v;
@@ -460,7 +486,7 @@ namespace {
 
 template <int BITS, int GROUP, int KSPLIT, int TPW>
 mi355q_status launch_pm(hipStream_t s, const PmArgs& a, uint32_t grid, size_t lds) {
-    auto kern = a.m > 8 ? (a.sb_dtype == MI355Q_BF16 ? gemv_mfma_planes_kernel<BITS, GROUP, KSPLIT, TPW, true, true>
+    auto kern = a.ms > 8 ? (a.sb_dtype == MI355Q_BF16 ? gemv_mfma_planes_kernel<BITS, GROUP, KSPLIT, TPW, true, true>
                                                      : gemv_mfma_planes_kernel<BITS, GROUP, KSPLIT, TPW, false, true>)
                         : (a.sb_dtype == MI355Q_BF16 ? gemv_mfma_planes_kernel<BITS, GROUP, KSPLIT, TPW, true, false>
                                                      : gemv_mfma_planes_kernel<BITS, GROUP, KSPLIT, TPW, false, false>);
@@ -494,8 +520,9 @@ mi355q_status launch_pm_shape(hipStream_t s, const PmArgs& a, const Tile16Launch
 // of K over wavefronts, tiles per workgroup, passes and K parts), for one staged row more: the row of zeros.  That
 // kernel's LDS sizes bound this one's ((M + 1) rows and K / 2 bytes of sums against (M + 1) rows and K bytes).
 bool gemv_mfma_planes_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
-    if (w.layout != MI355Q_LAYOUT_PLANES || !w.sz || x_dtype != MI355Q_BF16) return false;
-    if (m < 2 || m > 16) return false;
+    if (w.layout != MI355Q_LAYOUT_PLANES || !w.sz || (x_dtype != MI355Q_BF16 && x_dtype != MI355Q_F16)) return false;
+    const uint32_t ms = staged_rows(x_dtype, m);                           // f16 rows are staged as two bf16 rows each
+    if (ms < 2 || ms > 16) return false;
     if (w.bits != 4 && w.bits != 8) return false;
     const uint32_t bc = 512 / w.bits;                                     // codes per block
     if ((w.group != bc && w.group * 2 != bc) || w.k % bc) return false;
@@ -503,7 +530,7 @@ bool gemv_mfma_planes_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t
     // a row is one stream: its sz words follow its code words at the same pitch; code words 16-byte aligned
     if (w.sz_stride != w.code_stride || w.code_stride % 4 || (uintptr_t)w.codes % 16) return false;
     if (w.sz < w.codes || (size_t)(w.sz - w.codes) >= w.code_stride || (w.sz - w.codes) % 2) return false;
-    return gemv_tile16_parts_for(w.k, m + 1, (w.n + 15) / 16, 256, bc) != 0;
+    return gemv_tile16_parts_for(w.k, ms + 1, (w.n + 15) / 16, 256, bc) != 0;
 }
 
 uint32_t gemv_mfma_planes_k_parts(const mi355q_context* ctx, const WView& w, uint32_t m) {
@@ -516,7 +543,7 @@ Tile16LaunchShape gemv_mfma_planes_shape(const mi355q_context* ctx, uint32_t n_r
 }
 
 mi355q_status launch_gemv_mfma_planes_multi(hipStream_t s, mi355q_context* ctx, uint32_t count, const WView* w,
-                                            const void* x, void* const* y, const uint32_t* y_strides, int y_dtype,
+                                            const void* x, int x_dtype, void* const* y, const uint32_t* y_strides, int y_dtype,
                                             uint32_t m, uint32_t x_stride) {
     if (count < 1 || count > (uint32_t)kPmMaxSegments)
         return fail(MI355Q_ERR_INVALID_ARGUMENT, "1..%d weights per fused launch", kPmMaxSegments);
@@ -535,10 +562,13 @@ mi355q_status launch_gemv_mfma_planes_multi(hipStream_t s, mi355q_context* ctx, 
             w[j].k != w[0].k || w[j].bits != w[0].bits || w[j].group != w[0].group || w[j].sb_dtype != w[0].sb_dtype)
             return fail(MI355Q_ERR_SHAPE, "fused projections must share K, format, row pitch and scale type");
     }
-    const Tile16LaunchShape g = gemv_mfma_planes_shape(ctx, tiles, w[0].k, w[0].bits, m);
+    const uint32_t ms = staged_rows(x_dtype, m);
+    const Tile16LaunchShape g = gemv_mfma_planes_shape(ctx, tiles, w[0].k, w[0].bits, ms);
     const uint32_t bc = 512 / w[0].bits;
     a.x = (const uint16_t*)x;
     a.k = w[0].k; a.m = m; a.x_stride = x_stride;
+    a.x_f16 = x_dtype == MI355Q_F16 ? 1u : 0u;
+    a.ms = ms;
     a.row_words = w[0].code_stride;
     a.sz_offset = (uint32_t)(w[0].sz - w[0].codes);
     a.parts = g.parts;

@@ -23,6 +23,12 @@
 // The accumulator of lane (kq, n) holds output rows m = 4 kq .. 4 kq + 3 of weight row n, so there is
 // no cross-lane reduction at all; the WAVES wavefronts of a workgroup split K and add their partial
 // tiles through LDS at the end.
+//
+// f16 activations (the reference's decode type): a row is staged as TWO bf16 rows, hi = the upper eight significant
+// bits and lo = the remaining three (every f16 value, subnormals included, is their sum exactly and lies inside
+// bf16's exponent range), at rows 2 m and 2 m + 1.  The matrix core then works on 2 M rows with exact products, and
+// since a lane holds output rows 4 kq .. 4 kq + 3 the two partial results of a row are added in the lane that holds
+// them before the store: M <= 8 rows of f16 per launch at the cost of 2 M rows of bf16.
 #include "device_utils.h"
 
 namespace mi355q {
@@ -42,7 +48,9 @@ struct T16Args {
     uint32_t tile_end[kTile16MaxSegments];       // cumulative row-tile counts; unused entries repeat the last
     uint32_t seg_rows[kTile16MaxSegments];       // N_i
     uint32_t y_stride[kTile16MaxSegments];
-    const uint16_t* x;                           // bf16 [M, x_stride]
+    const uint16_t* x;                           // bf16 or f16 [M, x_stride]
+    uint32_t x_f16;                              // 1: f16 rows, staged as two bf16 rows each (ms = 2 m)
+    uint32_t ms;                                 // staged rows: the M dimension the matrix core works on
     float* logits;                               // optional fp32 [N] copy (M == 1, one matrix)
     int32_t* token_out;                          // ARGMAX only
     unsigned long long* scratch;                 // ARGMAX only: one packed key per workgroup; 0 = no candidate
@@ -146,10 +154,10 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
     // ---- 3. stage the activations (waits only for the loads of step 1) --------------------------
     // With each 16-byte chunk goes its share of sum(x): eight consecutive lanes hold the eight chunks of one
     // 64-element group of one row, so three xor-shuffles give the group sum, kept as sxs[group][row].
-    float* const sxs = (float*)(lds + (size_t)a.m * a.lds_row_bytes);
+    float* const sxs = (float*)(lds + (size_t)a.ms * a.lds_row_bytes);
     {
         const uint32_t total = a.m * chunks;
-        auto stage = [&](uint32_t idx, const u32x4& v) {
+        auto group_sum = [&](const u32x4& v) {
             float p = t16_dot2(v.x, 0x3F803F80u, 0.0f);
             p = t16_dot2(v.y, 0x3F803F80u, p);
             p = t16_dot2(v.z, 0x3F803F80u, p);
@@ -157,6 +165,23 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
             p += __shfl_xor(p, 1);
             p += __shfl_xor(p, 2);
             p += __shfl_xor(p, 4);
+            return p;
+        };
+        auto stage = [&](uint32_t idx, const u32x4& v) {
+            if (a.x_f16) {                                   // wavefront-uniform
+                u32x4 hi, lo;
+                f16x8_to_bf16_hi_lo(v, hi, lo);
+                const float ph = group_sum(hi), pl = group_sum(lo);
+                if (idx < total) {
+                    uint32_t m, c;
+                    x_row(idx, m, c);
+                    *((u32x4*)(lds + (size_t)(2 * m) * a.lds_row_bytes) + c) = hi;
+                    *((u32x4*)(lds + (size_t)(2 * m + 1) * a.lds_row_bytes) + c) = lo;
+                    if ((c & 7u) == 0) { sxs[(c >> 3) * 16 + 2 * m] = ph; sxs[(c >> 3) * 16 + 2 * m + 1] = pl; }
+                }
+                return;
+            }
+            const float p = group_sum(v);
             if (idx < total) {
                 *x_dst(idx) = v;
                 uint32_t m, c;
@@ -183,7 +208,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
     for (int r = 0; r < MR; r++) acc[r] = 0.f;
 
     // A operand: lane (m = lane & 15, kq) reads 8 consecutive bf16 of activation row min(m, M-1)
-    const uint32_t am = n_in < a.m ? n_in : a.m - 1;
+    const uint32_t am = n_in < a.ms ? n_in : a.ms - 1;
     const char* const a_lane = lds + (size_t)am * a.lds_row_bytes + kq * 32;
 
     auto unpack = [&](uint32_t w) -> bf16x8_t {
@@ -231,7 +256,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
     // once every wavefront is done reading those (the workgroup then needs no LDS beyond the activations, which
     // decides how many workgroups share a CU); several passes keep them behind the activations and their sums.
     const bool red_over_x = a.passes == 1;
-    float* const red = (float*)(red_over_x ? lds : lds + (size_t)a.m * a.lds_row_bytes + kp);
+    float* const red = (float*)(red_over_x ? lds : lds + (size_t)a.ms * a.lds_row_bytes + kp);
     unsigned long long best = 0ull;
     for (uint32_t pass = 0; pass < a.passes; pass++) {
         if (pass) {                                            // the first tile's loads were issued before staging
@@ -254,11 +279,20 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
         __syncthreads();
         if (slice == 0 && tile.valid) {                     // the first wavefront of each tile adds and stores
             const uint32_t row = tile.n0 + n_in;
+            float vv[MR];
 #pragma unroll
             for (int r = 0; r < MR; r++) {
-                float v = 0.f;
-                for (uint32_t w2 = 0; w2 < (uint32_t)KSPLIT; w2++) v += red[((wave + w2) * MR + r) * 64 + lane];
-                const uint32_t m = 4 * kq + r;
+                vv[r] = 0.f;
+                for (uint32_t w2 = 0; w2 < (uint32_t)KSPLIT; w2++) vv[r] += red[((wave + w2) * MR + r) * 64 + lane];
+            }
+            // f16 rows: staged rows 2 m and 2 m + 1 are the two parts of activation row m (smaller part first)
+            constexpr int OUT = MR >= 2 ? MR / 2 : 1;
+            const bool fold = MR >= 2 && a.x_f16;
+#pragma unroll
+            for (int r = 0; r < MR; r++) {
+                if (fold && r >= OUT) break;
+                const float v = fold ? vv[(2 * r + 1) % MR] + vv[(2 * r) % MR] : vv[r];
+                const uint32_t m = fold ? 2 * kq + r : 4 * kq + r;
                 if (m < a.m && row < tile.rows) {
                     if (a.parts > 1) {                       // one matrix: the reduction launch converts and stores
                         a.partial[((size_t)part * a.m + m) * tile.rows + row] = v;
@@ -382,11 +416,12 @@ mi355q_status launch_t16_shape(hipStream_t s, const T16Args& a, const Tile16Laun
 }  // namespace
 
 bool gemv_tile16_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
-    if (w.layout != MI355Q_LAYOUT_TILE16 || !w.tiles || x_dtype != MI355Q_BF16) return false;
-    if (m < 1 || m > 16) return false;
+    if (w.layout != MI355Q_LAYOUT_TILE16 || !w.tiles || (x_dtype != MI355Q_BF16 && x_dtype != MI355Q_F16)) return false;
+    const uint32_t ms = staged_rows(x_dtype, m);                      // f16 rows are staged as two bf16 rows each
+    if (m < 1 || ms > 16) return false;
     if (w.bits != 4 || w.group != 64 || w.k % 128) return false;
     if (x_stride % 8) return false;                                   // 128-bit activation loads
-    return t16_parts(w.k, m, (w.n + 15) / 16, 256) != 0;              // staged activations and their group sums fit in LDS
+    return t16_parts(w.k, ms, (w.n + 15) / 16, 256) != 0;             // staged activations and their group sums fit in LDS
 }
 
 uint32_t gemv_tile16_parts_for(uint32_t k, uint32_t m, uint32_t n_row_tiles, uint32_t cus, uint32_t block_codes) {
@@ -483,7 +518,7 @@ Tile16LaunchShape gemv_tile16_shape(const mi355q_context* ctx, uint32_t n_row_ti
 }
 
 mi355q_status launch_gemv_tile16_multi(hipStream_t s, mi355q_context* ctx, uint32_t count, const WView* w,
-                                       const void* x, void* const* y, const uint32_t* y_strides, int y_dtype,
+                                       const void* x, int x_dtype, void* const* y, const uint32_t* y_strides, int y_dtype,
                                        uint32_t m, uint32_t x_stride, float* logits_f32, int32_t* token_out,
                                        HeadKeys keys) {
     if (count < 1 || count > (uint32_t)kTile16MaxSegments)
@@ -503,8 +538,12 @@ mi355q_status launch_gemv_tile16_multi(hipStream_t s, mi355q_context* ctx, uint3
         a.seg_rows[i] = w[j].n;
         a.tile_end[i] = tiles;
     }
-    const Tile16LaunchShape g = gemv_tile16_shape(ctx, tiles, w[0].k, m);
+    const uint32_t ms = staged_rows(x_dtype, m);
+    if (argmax && x_dtype != MI355Q_BF16) return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the fused head on TILE16 records reads bf16 activations");
+    const Tile16LaunchShape g = gemv_tile16_shape(ctx, tiles, w[0].k, ms);
     a.x = (const uint16_t*)x;
+    a.x_f16 = x_dtype == MI355Q_F16 ? 1u : 0u;
+    a.ms = ms;
     a.logits = logits_f32; a.token_out = token_out; a.scratch = keys.ptr;
     a.k = w[0].k; a.m = m; a.x_stride = x_stride;
     a.kblocks = w[0].k / 128;
@@ -521,7 +560,7 @@ mi355q_status launch_gemv_tile16_multi(hipStream_t s, mi355q_context* ctx, uint3
         a.partial = (float*)ctx->workspace;
     }
     a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = w[0].sb_dtype;
-    const int mr = m == 1 ? 1 : m == 2 ? 2 : 4;
+    const int mr = ms == 1 ? 1 : ms == 2 ? 2 : 4;
     if (argmax) {
         if (g.grid > keys.capacity)
             return fail(MI355Q_ERR_SHAPE, "the fused output head keeps one partial key per workgroup: %u workgroups exceed %u",

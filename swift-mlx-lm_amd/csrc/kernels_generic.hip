@@ -376,31 +376,27 @@ mi355q_status launch_convert_rows(hipStream_t s, const void* src, int src_dtype,
     return MI355Q_OK;
 }
 
-// Activations as several bf16 rows each whose sum is the activation exactly.  fp32 (PARTS = 3): hi = bf16(x),
-// mid = bf16(x - hi), lo = x - hi - mid; both differences are exact in fp32 and the last one fits bf16 (24 significant
-// bits = 8 + 8 + 8, rounding to nearest leaves at most 16, then at most 7).  f16 (PARTS = 2): 11 significant bits =
-// 8 + 3, and every f16 value, subnormals included, lies inside bf16's exponent range.  A bf16 kernel run on the
-// PARTS * M rows then computes the projection with exact products.  out: [PARTS][M][out_stride].  A non-finite activation
-// stays in hi alone.
-template <int PARTS, bool F16IN>
-__global__ __launch_bounds__(256) void split_rows_bf16_kernel(const void* __restrict__ x, uint32_t m, uint32_t k,
+// fp32 activations as three bf16 rows each whose sum is the activation exactly: hi = bf16(x), mid = bf16(x - hi),
+// lo = x - hi - mid; both differences are exact in fp32 and the last one fits bf16 (24 significant bits = 8 + 8 + 8,
+// rounding to nearest leaves at most 16, then at most 7).  A bf16 kernel run on the 3 M rows then computes the fp32
+// projection with exact products.  out: [3][M][out_stride].  A non-finite activation stays in hi alone.
+__global__ __launch_bounds__(256) void split_rows_bf16_kernel(const float* __restrict__ x, uint32_t m, uint32_t k,
                                                               uint32_t x_stride, uint16_t* __restrict__ out,
                                                               uint32_t out_stride) {
     const uint32_t row = blockIdx.y;
     for (uint32_t c = blockIdx.x * 256 + threadIdx.x; c < k; c += gridDim.x * 256) {
-        const size_t i = (size_t)row * x_stride + c;
-        const float v = F16IN ? f16_to_f32(((const uint16_t*)x)[i]) : ((const float*)x)[i];
+        const float v = x[(size_t)row * x_stride + c];
         uint16_t part[3] = {f32_to_bf16_rne(v), 0, 0};
         if (v - v == 0.0f) {                                // finite
             float r = v - __uint_as_float((uint32_t)part[0] << 16);
 #pragma unroll
-            for (int p = 1; p < PARTS; p++) {
+            for (int p = 1; p < 3; p++) {
                 part[p] = f32_to_bf16_rne(r);
                 r -= __uint_as_float((uint32_t)part[p] << 16);
             }
         }
 #pragma unroll
-        for (int p = 0; p < PARTS; p++) out[((size_t)p * m + row) * out_stride + c] = part[p];
+        for (int p = 0; p < 3; p++) out[((size_t)p * m + row) * out_stride + c] = part[p];
     }
 }
 
@@ -423,9 +419,8 @@ mi355q_status launch_split_rows_bf16(hipStream_t s, const void* x, int x_dtype, 
     if (m > 65535u) return fail(MI355Q_ERR_SHAPE, "more than 65535 activation rows");
     uint32_t gx = (k + 255) / 256;
     if (gx > 256) gx = 256;
-    if (x_dtype == MI355Q_F32) split_rows_bf16_kernel<3, false><<<dim3(gx, m), dim3(256), 0, s>>>(x, m, k, x_stride, out, out_stride);
-    else if (x_dtype == MI355Q_F16) split_rows_bf16_kernel<2, true><<<dim3(gx, m), dim3(256), 0, s>>>(x, m, k, x_stride, out, out_stride);
-    else return fail(MI355Q_ERR_INVALID_ARGUMENT, "only f16 and fp32 rows are split into bf16 rows");
+    if (x_dtype != MI355Q_F32) return fail(MI355Q_ERR_INVALID_ARGUMENT, "only fp32 rows are split into bf16 rows");
+    split_rows_bf16_kernel<<<dim3(gx, m), dim3(256), 0, s>>>((const float*)x, m, k, x_stride, out, out_stride);
     MI355Q_HIP(hipGetLastError());
     return MI355Q_OK;
 }

@@ -48,33 +48,33 @@ void plan_small_m(const mi355q_weight* w, uint32_t m, int x_dtype, uint32_t x_st
     const WView v = w->view();
     const bool forced = flags & MI355Q_FLAG_FORCE_GENERIC;
     if (split_rows_chosen(v, x_dtype, m, x_stride, flags)) {
-        // fp32 / f16 rows as three / two bf16 rows each on the bf16 decode kernel, then the sum of the partial results
-        const uint32_t parts = split_rows_parts(x_dtype);
-        plan_small_m(w, parts * m, MI355Q_BF16, split_rows_stride((uint32_t)w->k), flags, s);
+        // fp32 rows as three bf16 rows each on the bf16 decode kernel, then the sum of the partial results
+        plan_small_m(w, split_rows_parts(x_dtype) * m, MI355Q_BF16, split_rows_stride((uint32_t)w->k), flags, s);
         char inner[sizeof s->device_kernel];
         std::snprintf(inner, sizeof inner, "%s", s->device_kernel);
-        std::snprintf(s->device_kernel, sizeof s->device_kernel, "split_%s_bf16x%u+%.30s", x_dtype == MI355Q_F32 ? "f32" : "f16",
-                      parts, inner);
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "split_f32_bf16x3+%.30s", inner);
         return;
     }
     // rows per launch on the tile layout: 16, or fewer when K is so long that 16 staged rows overflow LDS
-    uint32_t t16_rows = m > 16 ? 16 : m;
+    const uint32_t most = x_dtype == MI355Q_F16 ? 8 : 16;      // sixteen staged rows a launch; f16 rows are staged as two
+    uint32_t t16_rows = m > most ? most : m;
     if (!forced && v.layout == MI355Q_LAYOUT_TILE16) {
-        uint32_t step = 16;
+        uint32_t step = most;
         while (step > 1 && !gemv_tile16_eligible(v, x_dtype, step, x_stride)) step >>= 1;
         if (t16_rows > step) t16_rows = step;
     }
     if (!forced && gemv_tile16_eligible(v, x_dtype, t16_rows, x_stride)) {
-        const Tile16LaunchShape g = gemv_tile16_shape(w->ctx, (uint32_t)((w->n + 15) / 16), (uint32_t)w->k, t16_rows);
+        const Tile16LaunchShape g = gemv_tile16_shape(w->ctx, (uint32_t)((w->n + 15) / 16), (uint32_t)w->k,
+                                                      staged_rows(x_dtype, t16_rows));
         std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_tile16_q%u_g%u", (unsigned)w->fmt.bits,
                       w->fmt.group_size);
         s->grid[0] = g.grid;
         s->block[0] = g.block;
         s->lds_bytes = g.lds_bytes;
         s->rows_per_workgroup = 16;
-    } else if (!forced && m >= mfma_planes_min_rows(v.bits) && gemv_mfma_planes_eligible(v, x_dtype, m > 16 ? 16 : m, x_stride)) {
+    } else if (!forced && mfma_planes_pays(v.bits, x_dtype, m) && gemv_mfma_planes_eligible(v, x_dtype, m > most ? most : m, x_stride)) {
         const Tile16LaunchShape g = gemv_mfma_planes_shape(w->ctx, (uint32_t)((w->n + 15) / 16), (uint32_t)w->k,
-                                                           (uint32_t)w->fmt.bits, m > 16 ? 16 : m);
+                                                           (uint32_t)w->fmt.bits, staged_rows(x_dtype, m > most ? most : m));
         std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_mfma_planes_q%u_g%u", (unsigned)w->fmt.bits,
                       w->fmt.group_size);
         s->grid[0] = g.wgs_per_part;
@@ -127,16 +127,17 @@ void plan_shared_launch_shape(const mi355q_weight* const* ws, uint32_t count, ui
     WView all = ws[0]->view();
     uint64_t total = 0;
     // four rows and more (three at 8 bits): the matrix-core kernel over the planes takes the rows of all matrices, in 16-row tiles
-    bool on_planes = m >= mfma_planes_min_rows(all.bits) && m <= 16;
+    bool on_planes = mfma_planes_pays(all.bits, x_dtype, m) && m <= 16;
     uint32_t tiles = 0;
     for (uint32_t i = 0; i < count && on_planes; i++) {
         const WView v = ws[i]->view();
-        on_planes = gemv_mfma_planes_eligible(v, x_dtype, m, x_stride) && gemv_mfma_planes_k_parts(ws[0]->ctx, v, m) == 1 &&
+        on_planes = gemv_mfma_planes_eligible(v, x_dtype, m, x_stride) &&
+                    gemv_mfma_planes_k_parts(ws[0]->ctx, v, staged_rows(x_dtype, m)) == 1 &&
                     v.sb_dtype == all.sb_dtype && v.code_stride == all.code_stride && v.group == all.group && v.bits == all.bits;
         tiles += (v.n + 15) / 16;
     }
     if (on_planes) {
-        const Tile16LaunchShape g = gemv_mfma_planes_shape(ws[0]->ctx, tiles, all.k, all.bits, m);
+        const Tile16LaunchShape g = gemv_mfma_planes_shape(ws[0]->ctx, tiles, all.k, all.bits, staged_rows(x_dtype, m));
         s->grid[0] = g.wgs_per_part;
         s->grid[1] = g.parts;
         s->block[0] = g.block;
@@ -221,8 +222,9 @@ mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w, uint32_t maximum
     }
 
     const uint32_t m = maximum_sequence_length;
-    const uint32_t small_rows = small_batch_rows(v, x_dtype, input_row_stride);   // rows the decode kernels take per launch
-    const bool want_small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) || m <= small_rows ||
+    const uint32_t small_rows = small_batch_limit(v, x_dtype, input_row_stride);  // rows the decode kernels keep
+    const bool want_small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) ||
+                            (!(flags & MI355Q_FLAG_FORCE_MFMA) && m <= small_rows) ||
                             split_rows_chosen(v, x_dtype, m, input_row_stride, flags);
     const bool mfma_ok = gemm_mfma_eligible(v, x_dtype, m, input_row_stride);
     if (!split_rows_chosen(v, x_dtype, m, input_row_stride, flags) && gemm_two_step_chosen(v, x_dtype, m, input_row_stride, flags)) {

@@ -1,8 +1,9 @@
-"""GPU parity tests of fp32 and f16 activations at a few rows on the bf16 decode kernels (the f32s and f16 signatures of
-gemv_q{b}_g{g} / gemm_q{b}_g{g}, Sources/MetalCompiler/Generator/MetalSourceGenerator+Quantized.swift:496-575, :22-156)
-through the C ABI.  Every fp32 row is split on the device into three bf16 rows whose sum is the row exactly (an f16 row
-into two); the bf16 decode kernel of the layout runs on those rows and the partial results of a row are added, so the
-matrix is read once per launch and every product is exact.
+"""GPU parity tests of fp32 and f16 activations at a few rows on the kernels that compute in bf16 (the f32s and f16
+signatures of gemv_q{b}_g{g} / gemm_q{b}_g{g}, Sources/MetalCompiler/Generator/MetalSourceGenerator+Quantized.swift:496-575,
+:22-156) through the C ABI.  Every fp32 row is split on the device into three bf16 rows whose sum is the row exactly;
+the bf16 decode kernel of the layout runs on those rows and the partial results of a row are added.  f16 rows are
+split into two bf16 rows inside the matrix-core kernels themselves.  Either way the matrix is read once per launch and
+every product is exact.
 
 Bars: against an fp64 accumulation of the dequantised weights and the UNROUNDED fp32 activations, relative L2 <= 1e-5
 (rounding the activations to bf16 would give 1e-3); a case that needs all three parts and is exactly representable is
@@ -145,11 +146,13 @@ def test_f32_rows_non_finite_activation_and_graph_replay(pkg, ctx):
 
 
 @pytest.mark.parametrize("layout", ["tile16", "planes"])
-def test_f16_rows_as_two_bf16_rows(pkg, ctx, layout):
-    """f16 activations where the bf16 matrix-core kernels are the faster or the only decode kernels: TILE16 records (no
-    kernel reads f16 there) from one row to twenty-four, 4-bit planes from five rows (below, the f16 dot-product
-    kernels) to sixteen.  One-hot rows with an 11-bit value (1024 + odd) / 2048, which needs both bf16 parts, must come
-    out bit for bit; seeded f16 rows to 1e-5 of the fp64 reference on the same f16 values."""
+def test_f16_rows_on_the_matrix_core_kernels(pkg, ctx, layout):
+    """f16 activations (the reference's decode type) on the kernels that compute in bf16 on the matrix cores: a row is
+    staged inside the kernel as two bf16 rows (the upper eight significant bits, the remaining three) and the two
+    partial results are added before the store -- up to eight f16 rows a launch on TILE16 records, three to eight on
+    4-bit planes (below, the f16 dot-product kernels), more rows in steps of eight.  One-hot rows with an 11-bit value
+    (1024 + odd) / 2048, which needs both parts, must come out bit for bit; seeded f16 rows to 1e-5 of the fp64
+    reference on the same f16 values; padded rows; all output types."""
     lay = {"planes": pkg.LAYOUT_PLANES, "tile16": pkg.LAYOUT_TILE16}[layout]
     fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
     rng = np.random.default_rng(5500)
@@ -159,22 +162,74 @@ def test_f16_rows_as_two_bf16_rows(pkg, ctx, layout):
     case = Case(4, 64, codes, scales, zeros)
     wq = scales.repeat(64, axis=1) * codes + zeros.repeat(64, axis=1)
     w = ctx.weight_prepare_mlx(fmt, *case.planes(pkg.BF16, pkg), pkg.BF16, lay)
-    split_ms = [1, 2, 5, 8, 13, 24] if layout == "tile16" else [5, 8, 13, 16]
-    other_ms = [25] if layout == "tile16" else [1, 4, 17]
-    for m in split_ms + other_ms:
+    fast = "gemv_tile16_q4_g64" if layout == "tile16" else "gemv_mfma_planes_q4_g64"
+    for m in (1, 2, 3, 4, 5, 7, 8, 9, 13, 15):
         say(f"f16 rows {layout} M={m}")
         st = w.plan_prefill_steps(m, x_dtype=pkg.F16)[0]
-        assert st.device_kernel.startswith("split_f16_bf16x2+") == (m in split_ms), (m, st.device_kernel)
+        assert (st.device_kernel == fast) == (layout == "tile16" or m >= 3), (m, st.device_kernel)
+        assert m > 8 or not st.used_fallback
         x = np.zeros((m, k), np.float32)
         pos = rng.choice(k, m, replace=False)
         for r in range(m):
             x[r, pos[r]] = np.float32((1024 + 2 * int(rng.integers(0, 512)) + 1) / 2048.0) * (-1) ** r
         want = x.astype(np.float64) @ wq.T
-        got = run_f32(ctx, pkg, w, x, use_qgemm=True, x_dtype=pkg.F16, xpad=8 if m % 2 else 0)
+        got = run_f32(ctx, pkg, w, x, use_qgemm=True, x_dtype=pkg.F16, xpad=8 if m % 2 else 0, ypad=3 if m % 3 == 0 else 0)
         assert np.array_equal(got.astype(np.float64), want), (layout, m)
         x = kat.seeded_activations(5510 + m, m, k).astype(np.float16).astype(np.float32)
         got = run_f32(ctx, pkg, w, x, use_qgemm=True, x_dtype=pkg.F16)
-        assert rel_l2(got, oracle.gemm_f64(wq, x)) <= (1e-5 if m in split_ms else 1e-3), (layout, m)
+        assert rel_l2(got, oracle.gemm_f64(wq, x)) <= 1e-5, (layout, m)
         if m <= 8:
             assert np.array_equal(run_f32(ctx, pkg, w, x, x_dtype=pkg.F16), got)
+            for yd in (pkg.BF16, pkg.F16):
+                low = run_f32(ctx, pkg, w, x, y_dtype=yd, x_dtype=pkg.F16)
+                ref = oracle.bf16_to_f32(oracle.bf16_from_f32(got)).reshape(got.shape) if yd == pkg.BF16 \
+                    else got.astype(np.float16).astype(np.float32)
+                assert np.array_equal(low, ref), (layout, m, yd)
     w.destroy()
+
+
+def test_f16_rows_long_k_parts_and_eight_bit_planes(pkg, ctx):
+    """Rows of 14336 codes at eight f16 rows (sixteen staged rows) overflow the staged copy: K parts with folded
+    partial results; 8-bit planes in groups of 32 take f16 rows on the same kernel."""
+    for lay, bits, group, n, k, ms in ((pkg.LAYOUT_TILE16, 4, 64, 48, 14336, (4, 8)), (pkg.LAYOUT_PLANES, 4, 64, 48, 14336, (4, 8)),
+                                       (pkg.LAYOUT_PLANES, 8, 32, 100, 2048, (3, 8)), (pkg.LAYOUT_PLANES, 4, 128, 100, 2048, (3, 6))):
+        fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(bits, group)
+        words, s, z, wq = seeded_case(5700 + bits + group, n, k, bits, group)
+        w = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, lay)
+        for m in ms:
+            say(f"f16 rows layout {lay} q{bits} g{group} {k}->{n} M={m}")
+            x = kat.seeded_activations(5710 + m, m, k).astype(np.float16).astype(np.float32)
+            got = run_f32(ctx, pkg, w, x, x_dtype=pkg.F16)
+            assert rel_l2(got, oracle.gemm_f64(wq, x)) <= 1e-5, (lay, bits, m, rel_l2(got, oracle.gemm_f64(wq, x)))
+        w.destroy()
+
+
+def test_batched_projections_other_activation_types(pkg, ctx):
+    """q+k+v / gate+up with f16 rows on TILE16 records (one shared launch that stages the f16 rows itself) and fp32 rows
+    on planes and blocks (split once into bf16 rows, one shared bf16 launch, one sum per projection): the same bits as
+    the separate calls."""
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+    for layout, x_dtype, npdt, ms in ((pkg.LAYOUT_TILE16, pkg.F16, np.float16, (1, 3, 8)),
+                                      (pkg.LAYOUT_PLANES, pkg.F32, np.float32, (1, 2, 5)),
+                                      (pkg.LAYOUT_STAF_BLOCKS, pkg.F32, np.float32, (1, 2))):
+        ns, k = (384, 96, 96), 1024
+        ws, wqs = [], []
+        for i, n in enumerate(ns):
+            words, s, z, wq = seeded_case(5600 + i, n, k, 4, 64)
+            ws.append(ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, layout)); wqs.append(wq)
+        for m in ms:
+            say(f"batched split layout {layout} dtype {x_dtype} M={m}")
+            x = kat.seeded_activations(5610 + m, m, k).astype(npdt)
+            xd = ctx.upload(x.view(np.uint16) if npdt == np.float16 else x)
+            yds = [ctx.alloc(m * n * 4) for n in ns]
+            ctx.batched_qgemm(ws, xd, x_dtype, yds, pkg.F32, m); ctx.synchronize()
+            for j, n in enumerate(ns):
+                fused = yds[j].download(np.float32, (m, n))
+                alone = run_f32(ctx, pkg, ws[j], x.astype(np.float32), x_dtype=x_dtype, use_qgemm=True)
+                assert np.array_equal(fused, alone), (layout, m, j)
+                assert rel_l2(fused, oracle.gemm_f64(wqs[j], x.astype(np.float32))) <= 1e-5
+            xd.free()
+            for b in yds:
+                b.free()
+        for w in ws:
+            w.destroy()

@@ -97,8 +97,8 @@ def test_tile16_ragged_shapes_and_long_batches(pkg, ctx):
             x = act_rounded(kat.seeded_activations(2400 + i + m, m, k), pkg.BF16, pkg)
             say(f"tile16 ragged {k}->{n} M={m}")
             got = _run(ctx, pkg, w, x, pkg.F32, use_qgemm=m > 8)
-            # beyond 16 rows the projection runs on the prefill kernel, whose weights are rounded to bf16
-            ref_w = wq if m <= 16 else oracle.bf16_to_f32(oracle.bf16_from_f32(wq)).reshape(wq.shape)
+            # beyond 32 rows (two launches) the projection runs on the prefill kernel, whose weights are rounded to bf16
+            ref_w = wq if m <= 32 else oracle.bf16_to_f32(oracle.bf16_from_f32(wq)).reshape(wq.shape)
             assert_within_tolerance(got, oracle.gemm_f64(ref_w, x), f"{k}->{n} M={m}")
         w.destroy()
     # f16 scale words (STAF source)
@@ -310,9 +310,9 @@ def test_tile16_lm_head_fused_argmax(pkg, ctx):
 
 
 def test_tile16_prefill_runs_on_the_matrix_cores(pkg, ctx):
-    """Above 16 rows a TILE16 weight feeds the prefill GEMM directly from its records.  The arithmetic is that of
-    the same kernel on the split planes (same bf16 weights, same contraction order): identical bits; the plan
-    record names the matrix-core kernel."""
+    """Above 32 rows (two launches of the small-batch kernel) a TILE16 weight feeds the prefill GEMM directly from its
+    records.  The arithmetic is that of the same kernel on the split planes (same bf16 weights, same contraction
+    order): identical bits; the plan record names the matrix-core kernel."""
     for i, (m, n, k) in enumerate([(17, 130, 2048 + 128), (64, 4099, 384), (300, 257, 128), (512, 4096, 4096),
                                    (2048, 1024, 512)]):
         words, s, z, wq = seeded_case(2700 + i, n, k, 4, 64)
@@ -320,7 +320,7 @@ def test_tile16_prefill_runs_on_the_matrix_cores(pkg, ctx):
         wp = ctx.weight_prepare_mlx(_fmt(pkg), words, s, z, pkg.BF16, pkg.LAYOUT_PLANES)
         x = act_rounded(kat.seeded_activations(2750 + i, m, k), pkg.BF16, pkg)
         say(f"tile16 prefill {k}->{n} M={m}")
-        got = _run(ctx, pkg, wt, x, pkg.F32, use_qgemm=True, flags=0 if m < 1024 else pkg.FLAG_FORCE_MFMA)
+        got = _run(ctx, pkg, wt, x, pkg.F32, use_qgemm=True, flags=0 if 32 < m < 1024 else pkg.FLAG_FORCE_MFMA)
         same = _run(ctx, pkg, wp, x, pkg.F32, use_qgemm=True, flags=pkg.FLAG_FORCE_MFMA)
         assert np.array_equal(got, same), f"{k}->{n} M={m}: records and planes disagree"
         if m * n * k <= 2 ** 28:
@@ -329,7 +329,10 @@ def test_tile16_prefill_runs_on_the_matrix_cores(pkg, ctx):
         st = wt.plan_prefill_steps(m, flags=pkg.FLAG_FORCE_MFMA)[0]
         assert st.device_kernel == "qgemm_mfma_q4_g64" and not st.used_fallback
         unforced = [s.device_kernel for s in wt.plan_prefill_steps(m)]     # long prompts: dequantise once + dense GEMM
-        assert unforced == (["dequant_q4_g64_bf16", "hipblaslt_gemm_bf16"] if m >= 1024 else ["qgemm_mfma_q4_g64"])
+        assert unforced == (["dequant_q4_g64_bf16", "hipblaslt_gemm_bf16"] if m >= 1024 else
+                            ["qgemm_mfma_q4_g64"] if m > 32 else ["gemv_tile16_q4_g64"])
+        if m <= 32:                                          # two launches of the small-batch kernel: unrounded weights
+            assert_within_tolerance(_run(ctx, pkg, wt, x, pkg.F32, use_qgemm=True), oracle.gemm_f64(wq, x), f"M={m} in steps")
         wt.destroy(); wp.destroy()
     # f16 scale words (a STAF source)
     rng = np.random.default_rng(6)
@@ -402,9 +405,9 @@ def test_tile16_plan_replay_and_graph(pkg, ctx):
 
 
 @pytest.mark.parametrize("x_dtype_name", ["F16", "F32"])
-def test_tile16_other_activation_types_take_the_per_code_kernel_whole(pkg, ctx, x_dtype_name):
-    """The tile kernel reads bf16 activations only.  Up to sixteen fp32 rows run on it as three bf16 rows each, up to
-    twenty-four f16 rows as two; beyond, rows take the two-dispatch route
+def test_tile16_other_activation_types(pkg, ctx, x_dtype_name):
+    """The tile kernel computes in bf16.  f16 rows are staged inside it as two bf16 rows each (eight rows a launch), up to
+    sixteen fp32 rows run on it as three bf16 rows each; from sixteen rows both take the two-dispatch route
     (the matrix dequantised to the activations' type, then the dense library GEMM; fp32 from sixteen rows: bf16
     weights against split activations); forced, the per-code kernel takes all rows in one launch (no walk in steps
     of sixteen, eight ... one row)."""
@@ -418,9 +421,9 @@ def test_tile16_other_activation_types_take_the_per_code_kernel_whole(pkg, ctx, 
         # from sixteen rows fp32 activations meet bf16 weights (the reference's gemm_bf16_f32s); f16 ones f16 weights
         weights = wq if m < 16 or x_dtype == pkg.F16 else oracle.bf16_to_f32(oracle.bf16_from_f32(wq)).reshape(wq.shape)
         assert_within_tolerance(got, oracle.gemm_f64(weights, x), f"{x_dtype_name} M={m}")
-        if m <= 16:
-            parts = "f32_bf16x3" if x_dtype == pkg.F32 else "f16_bf16x2"
-            assert w.plan_prefill_steps(m, x_dtype=x_dtype)[0].device_kernel == f"split_{parts}+gemv_tile16_q4_g64"
+        if m <= 15:
+            want_kernel = "split_f32_bf16x3+gemv_tile16_q4_g64" if x_dtype == pkg.F32 else "gemv_tile16_q4_g64"
+            assert w.plan_prefill_steps(m, x_dtype=x_dtype)[0].device_kernel == want_kernel
         elif m > 1:
             assert w.plan_prefill_steps(m, x_dtype=x_dtype)[0].kernel_family in ("libraryGEMM", "dequantToBFloat")
         slow = run_gemv(ctx, pkg, w, x, x_dtype, pkg.F32, pkg.FLAG_FORCE_GENERIC, use_qgemm=True)
