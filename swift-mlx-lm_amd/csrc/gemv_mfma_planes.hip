@@ -126,7 +126,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
     // ---- 1. activation loads first (vector loads return in issue order) -------------------------------------------
     // The M x chunks 16-byte chunks of the staged columns are dealt to the threads in order, XB a thread at a time: a
     // batch's loads all go out before its first chunk is staged, and the first batch goes out before the weight
-    // loads.  Row M of the staged copy is a row of zeros (the masked half of A).
+    // loads.  Behind the staged rows lie 256 bytes of zeros (the masked half of A).
     const uint32_t chunks = kp / 8;                         // 16-byte chunks per staged activation row
     constexpr uint32_t NT = WAVES * 64;
     constexpr int XB = 8;
@@ -181,7 +181,9 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
     // ---- 3. stage the activations: every run of eight as (x0,x4,x1,x5,x2,x6,x3,x7) (8 bits: (x0,x2,x1,x3,x4,x6,x5,x7)),
     //         and sum(x) per half block and row ----------------------------------------------------------------------
     constexpr uint32_t CH = HALF / 8;                       // 16-byte chunks per half block
-    float* const sxs = (float*)(lds + (size_t)(a.ms + 1) * a.lds_row_bytes);     // [half block in part][SXR]
+    // behind the staged rows: 256 bytes of zeros (the masked half of A reads them at every block), then the sums
+    char* const zero_block = lds + (size_t)a.ms * a.lds_row_bytes;
+    float* const sxs = (float*)(zero_block + 256);                            // [half block in part][SXR]
     {
         auto run_sum = [&](const u32x4& v) {
             float p = pm_dot2(v.x, 0x3F803F80u, 0.0f);
@@ -238,7 +240,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
                 if (base + (uint32_t)t * NT < total) stage(base + tid + (uint32_t)t * NT, xe[t]);
         }
         const u32x4 zero = {0u, 0u, 0u, 0u};
-        for (uint32_t c = tid; c < chunks; c += NT) *((u32x4*)(lds + (size_t)a.ms * a.lds_row_bytes) + c) = zero;
+        if (tid < 16) *((u32x4*)zero_block + tid) = zero;
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __builtin_amdgcn_s_barrier();
@@ -254,14 +256,17 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
     for (int r = 0; r < MR; r++) acc[r] = 0.f;
 
     // A operand: lane (i = lane % 16, kq) stands for A row i.  Rows 0..7 are activation rows 0..7 where kq < 2, rows
-    // 8..15 are the same activation rows where kq >= 2; elsewhere the row of zeros.  Rows past M read row M-1 (their
-    // results are never stored).
+    // 8..15 are the same activation rows where kq >= 2; elsewhere zeros, read from the same 64 bytes at every block (the
+    // lane's offset from block to block is masked away).  Rows past M read row M-1 (their results are never stored).
     const uint32_t xi = WIDE ? n_in : (n_in & 7u);
     const uint32_t xr = xi < a.ms ? xi : a.ms - 1;
     const bool live = WIDE ? (kq < 2) : (n_in >> 3) == (kq >> 1);
-    const char* const a_lane = lds + (size_t)(live || (WIDE && !TWO) ? xr : a.ms) * a.lds_row_bytes + kq * (XBYTES / 4);
+    const bool reads_x = live || (WIDE && !TWO);
+    const char* const a_lane = (reads_x ? lds + (size_t)xr * a.lds_row_bytes : zero_block) + kq * (XBYTES / 4);
+    const uint32_t a_mask = reads_x ? ~0u : 0u;            // (an and per block: a per-lane multiply is a slow instruction)
     // WIDE, two groups per block: the second product's operand, live where the first one's is not
-    const char* const a_lane_hi = lds + (size_t)(live ? a.ms : xr) * a.lds_row_bytes + kq * (XBYTES / 4);
+    const char* const a_lane_hi = (live ? zero_block : lds + (size_t)xr * a.lds_row_bytes) + kq * (XBYTES / 4);
+    const uint32_t a_mask_hi = live ? 0u : ~0u;
 
     auto unpack = [&](uint32_t w) -> pm_bf16x8_t {
         u32x4 p;
@@ -290,7 +295,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
     const int from_lane = (int)((4u * n_in + kq) * 4u);     // byte address of the lane that loaded (row n, piece kq)
     auto compute = [&](uint32_t b, const Rec& r, const uint32_t (&sz_pair)[SZW], uint32_t sz_piece) {
         const uint32_t bl = b - b0;                          // block inside the staged columns
-        const char* ab = a_lane + (size_t)bl * XBYTES;       // this block's activations
+        const char* ab = a_lane + ((bl * XBYTES) & a_mask);  // this block's activations
         // every LDS operation of the block goes out first: the cross-lane reads, the A operands, sum(x) over this lane
         // half's run of 64 (runs 2 bl and 2 bl + 1 of the part): a group of 64, or half of a group of 128 whose other
         // half the other lanes add
@@ -339,7 +344,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
                 for (int q = 0; q < MR; q++) acc[q] += sc * __builtin_fmaf(16.0f, dh[q], dl[q]) + zc * sxv[q];
             } else {
                 const pm_floatx4_t sx_hi = *(const pm_floatx4_t*)(sxs + (size_t)(bl * 2 + 1) * SXR + sx_lane);
-                const char* ah = a_lane_hi + (size_t)bl * XBYTES;
+                const char* ah = a_lane_hi + ((bl * XBYTES) & a_mask_hi);
                 const pm_bf16x8_t g0 = *(const pm_bf16x8_t*)(ah), g1 = *(const pm_bf16x8_t*)(ah + 16);
                 __builtin_amdgcn_sched_barrier(0);
                 pm_floatx4_t dl = zero4, dh = zero4, el = zero4, eh = zero4;
@@ -385,7 +390,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
 #pragma unroll
                 for (int q = 0; q < MR; q++) acc[q] += sc * d[q] + zc * (sx[q] + sx_hi[q]);
             } else {
-                const char* ah = a_lane_hi + (size_t)bl * XBYTES;
+                const char* ah = a_lane_hi + ((bl * XBYTES) & a_mask_hi);
                 const pm_bf16x8_t h0 = *(const pm_bf16x8_t*)(ah), h1 = *(const pm_bf16x8_t*)(ah + 16);
                 const pm_bf16x8_t h2 = *(const pm_bf16x8_t*)(ah + 32), h3 = *(const pm_bf16x8_t*)(ah + 48);
                 __builtin_amdgcn_sched_barrier(0);
@@ -411,7 +416,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
     // Partial tiles of the WAVES wavefronts, [WAVES][MR][64]: a single pass writes them over the staged activations
     // once every wavefront is done reading those; several passes keep them behind the activations and their sums.
     const bool red_over_x = a.passes == 1;
-    float* const red = (float*)(red_over_x ? lds : lds + (size_t)(a.ms + 1) * a.lds_row_bytes + (size_t)(kp / HALF) * SXR * 4);
+    float* const red = (float*)(red_over_x ? lds : (char*)sxs + (size_t)(kp / HALF) * SXR * 4);
     for (uint32_t pass = 0; pass < a.passes; pass++) {
         if (pass) {                                            // the first tile's loads were issued before staging
             tile = select_tile(pass);
@@ -517,8 +522,8 @@ mi355q_status launch_pm_shape(hipStream_t s, const PmArgs& a, const Tile16Launch
 }  // namespace
 
 // The workgroups are shaped like those of the TILE16 kernel (16-row tiles walked in blocks of 128 codes, the same split
-// of K over wavefronts, tiles per workgroup, passes and K parts), for one staged row more: the row of zeros.  That
-// kernel's LDS sizes bound this one's ((M + 1) rows and K / 2 bytes of sums against (M + 1) rows and K bytes).
+// of K over wavefronts, tiles per workgroup, passes and K parts), plus 256 bytes of zeros behind the staged rows.  That
+// kernel's LDS sizes bound this one's (M rows and K / 2 bytes of sums against M rows and K bytes).
 bool gemv_mfma_planes_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
     if (w.layout != MI355Q_LAYOUT_PLANES || !w.sz || (x_dtype != MI355Q_BF16 && x_dtype != MI355Q_F16)) return false;
     const uint32_t ms = staged_rows(x_dtype, m);                           // f16 rows are staged as two bf16 rows each
@@ -530,16 +535,18 @@ bool gemv_mfma_planes_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t
     // a row is one stream: its sz words follow its code words at the same pitch; code words 16-byte aligned
     if (w.sz_stride != w.code_stride || w.code_stride % 4 || (uintptr_t)w.codes % 16) return false;
     if (w.sz < w.codes || (size_t)(w.sz - w.codes) >= w.code_stride || (w.sz - w.codes) % 2) return false;
-    return gemv_tile16_parts_for(w.k, ms + 1, (w.n + 15) / 16, 256, bc) != 0;
+    return gemv_tile16_parts_for(w.k, ms, (w.n + 15) / 16, 256, bc) != 0;
 }
 
 uint32_t gemv_mfma_planes_k_parts(const mi355q_context* ctx, const WView& w, uint32_t m) {
-    return gemv_tile16_parts_for(w.k, m + 1, (w.n + 15) / 16, (uint32_t)ctx->props.multiProcessorCount, 512 / w.bits);
+    return gemv_tile16_parts_for(w.k, m, (w.n + 15) / 16, (uint32_t)ctx->props.multiProcessorCount, 512 / w.bits);
 }
 
 Tile16LaunchShape gemv_mfma_planes_shape(const mi355q_context* ctx, uint32_t n_row_tiles, uint32_t k_total, uint32_t bits,
                                          uint32_t m) {
-    return gemv_tile16_shape(ctx, n_row_tiles, k_total, m + 1, 512 / bits);
+    Tile16LaunchShape g = gemv_tile16_shape(ctx, n_row_tiles, k_total, m, 512 / bits);
+    g.lds_bytes += 256;                                                    // the block of zeros behind the staged rows
+    return g;
 }
 
 mi355q_status launch_gemv_mfma_planes_multi(hipStream_t s, mi355q_context* ctx, uint32_t count, const WView* w,
