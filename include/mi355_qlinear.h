@@ -270,9 +270,10 @@ MI355Q_API mi355q_status mi355q_qgemv(mi355q_context* ctx, void* stream, const m
 /* Prefill projection: gemm_q4_g64_f32s / gemm_q8_g32_f32s (:22-156) and the two-step
  * dequant_q*_bf16 + gemm_bf16_f32s path (:361-416, MC/Generator/MetalSourceGenerator+Linear.swift:18-81).
  * Any M >= 1; M is a run-time value (the reference rebinds sequenceLength per call,
- * MC/Compiler/MetalPrefillStepBuilder.swift:728-732).  Three routes, all with the weights rounded once
- * to bf16 and fp32 accumulation, chosen by measured cost unless flags say otherwise
- * (mi355q_plan_prefill_steps reports the choice):
+ * MC/Compiler/MetalPrefillStepBuilder.swift:728-732).  Three routes, all with fp32 accumulation, chosen by
+ * measured cost unless flags say otherwise (mi355q_plan_prefill_steps reports the choice); the first keeps
+ * the dequantised weights unrounded (the decode kernels' arithmetic), the other two round them once to bf16
+ * (the numerics of the reference's dequant -> bf16 -> GEMM route):
  *   - small M (up to 8 rows; 16 on TILE16 records and on q4 / q8 planes, and there up to 32 in two launches):
  *     the GEMV-style decode kernels;
  *   - ONE fused kernel: code tiles are dequantised to bf16 in LDS and contracted on MFMA (the planes
