@@ -97,6 +97,8 @@ def main():
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip the secondary per-launch figures of benchmark configs 0, 2 and 4")
     ap.add_argument("--no-batch-sweep", action="store_true", help="skip the secondary M = 1, 2, 4, 8 figures")
+    ap.add_argument("--all-formats", action="store_true",
+                    help="add 4096->14336 at M = 1 and 8 for every registered format, planes and blocks in place (half a minute)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (one process, one device); "
@@ -448,6 +450,33 @@ def main():
             for b in (xd1, yd1, logits, tok):
                 b.free()
 
+    # ---- on request: every registered format at the gate shape, one and eight rows, both decode layouts of the format
+    all_formats = None
+    if a.all_formats:
+        all_formats = {}
+        n, k = 14336, 4096
+        for bits, group in kat.ALL_FORMATS:
+            f2 = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(bits, group)
+            words, s, z = oracle.quantize_affine(kat.seeded_weights(3300 + bits + group, n, k), bits, group, oracle.BF16)
+            nbytes = n * (k // group) * (4 + group * bits // 8)
+            entry = {"weight_bytes": nbytes}
+            for lname, layout in (("planes", pkg.LAYOUT_PLANES), ("staf_blocks", pkg.LAYOUT_STAF_BLOCKS)):
+                ws = [ctx.weight_prepare_mlx(f2, words, s, z, pkg.BF16, layout) for _ in range(8)]
+                for m in (1, 8):
+                    xb = ctx.upload(oracle.bf16_from_f32(kat.seeded_activations(3400 + m, m, k)))
+                    yb = ctx.alloc(m * n * 2)
+                    for w in ws:
+                        ctx.qgemv(w, xb, pkg.BF16, yb, pkg.BF16, m, 0, 0, 0, stream)
+                    ctx.synchronize(stream)
+                    ms = time_region(ctx, lambda i: ctx.qgemv(ws[i % 8], xb, pkg.BF16, yb, pkg.BF16, m, 0, 0, 0, stream), 32, stream)
+                    entry[f"{lname} M={m}"] = {"us": round(ms * 1e3, 2), "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                                               "kernel": ws[0].plan_decode_step(m).device_kernel}
+                    xb.free(); yb.free()
+                for w in ws:
+                    w.destroy()
+            all_formats[f"q{bits} g{group}"] = entry
+            log(f"  q{bits} g{group}: " + ", ".join(f"{k2} {v['us']} us ({v['kernel']})" for k2, v in entry.items() if isinstance(v, dict)))
+
     # ---- what HBM delivers to one launch of the dominant launch's size: a kernel that only reads that many bytes
     # (cold: eight buffers in rotation, as the weights of the layer copies are)
     probe_copies = 8
@@ -665,7 +694,7 @@ def main():
                    "replay": mode, "replay_GBps": replay_gbps, "step_time_spread": spreads[mode],
                    "step_time_spread_all": spreads, "steps_asked": a.steps, "warmup_asked": a.warmup,
                    "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2), "per_shape": per_shape,
-                   "f16_activations_step": f16_step, "batch_sweep": batch_sweep, "other_configs": other, "staf_blocks_in_place_step": staf_step, "next_rows": next_rows,
+                   "f16_activations_step": f16_step, "batch_sweep": batch_sweep, "other_configs": other, "all_formats": all_formats, "staf_blocks_in_place_step": staf_step, "next_rows": next_rows,
                    "stream_read_probe": stream_read,
                    "prefill_gemm_gate": prefill},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",

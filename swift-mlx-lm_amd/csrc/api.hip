@@ -198,7 +198,10 @@ bool gemm_two_step_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_st
     if (flags & MI355Q_FLAG_FORCE_TWO_STEP) return true;
     if (!gemm_two_step_eligible(w, x_dtype, m, x_stride)) return false;
     if (!gemm_mfma_eligible(w, x_dtype, m, x_stride)) {
-        if (!decode_kernel_reads(w, x_dtype, x_stride)) return m >= 2;
+        // no decode kernel reads the weight: from the second row; from the first where the per-code kernel leaves most
+        // of its lanes idle (a lane per code of a group: q3 g16 blocks, 4096 -> 14336, take it 465 us at one row
+        // against 120 us on this route)
+        if (!decode_kernel_reads(w, x_dtype, x_stride)) return m >= 2 || w.group < 64;
         // f16 rows on the matrix-core decode kernels, eight a launch: a Llama-3-8B layer step takes 56-67 us per eight
         // rows there and 255-296 us on this route whatever the rows
         const bool f16_on_matrix_cores = x_dtype == MI355Q_F16 && (gemv_tile16_eligible(w, x_dtype, 8, x_stride) ||
