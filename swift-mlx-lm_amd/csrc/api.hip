@@ -206,7 +206,9 @@ bool gemm_two_step_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_st
         // rows there and 255-296 us on this route whatever the rows
         const bool f16_on_matrix_cores = x_dtype == MI355Q_F16 && (gemv_tile16_eligible(w, x_dtype, 8, x_stride) ||
                                                                    gemv_mfma_planes_eligible(w, x_dtype, 8, x_stride));
-        return m >= (f16_on_matrix_cores ? kTwoStepMinRowsF16Batches : kTwoStepMinRowsOtherwise);
+        const uint32_t least = f16_on_matrix_cores ? kTwoStepMinRowsF16Batches : kTwoStepMinRowsOtherwise;
+        const uint32_t one_launch = small_batch_rows(w, x_dtype, x_stride);      // what one small-batch launch still takes
+        return m >= least && m > one_launch;
     }
     return m >= (w.k > w.n ? kTwoStepMinRowsLongK : kTwoStepMinRowsBesideFused);
 }

@@ -64,7 +64,7 @@ struct PmArgs {
     float* partial;                            // K parts only: fp32 partial results [part][M][N] (one matrix)
 };
 
-// BITS, GROUP: 4 with 64 or 128, 8 with 32 or 64.  A workgroup of KSPLIT * TPW wavefronts covers TPW consecutive row tiles, each split over KSPLIT
+// BITS, GROUP: 4 with 64 or 128, 8 with 32, 64 or 128 (a group of two blocks: both blocks apply the group's word).  A workgroup of KSPLIT * TPW wavefronts covers TPW consecutive row tiles, each split over KSPLIT
 // wavefronts along K; all of them share one staged copy of the activations.
 // WIDE: nine to sixteen activation rows.  The M dimension then has no empty half, so the two groups of a block are
 // kept apart with two products per word instead: one whose A operand carries the activations only where kq < 2, one
@@ -76,7 +76,8 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
     constexpr uint32_t XBYTES = BC * 2;                     // bytes of one activation row per block
     constexpr uint32_t HALF = BC / 2;                       // codes of half a block: the run the staged sums cover
     constexpr bool TWO = GROUP * 2 == (int)BC;              // a block holds two quantisation groups (else one)
-    static_assert((BITS == 4 || BITS == 8) && (TWO || GROUP == (int)BC), "4 bits: groups of 64 / 128; 8 bits: 32 / 64");
+    constexpr bool PAIR = GROUP == 2 * (int)BC;             // a quantisation group spans two blocks (8 bits, groups of 128)
+    static_assert((BITS == 4 || BITS == 8) && (TWO || PAIR || GROUP == (int)BC), "4 bits: groups of 64 / 128; 8 bits: 32 / 64 / 128");
     constexpr uint32_t SXR = WIDE ? 16 : 8;                 // activation rows per run of 64 in the staged sums
     constexpr int WAVES = KSPLIT * TPW;
     constexpr int D = 4;                                    // blocks in flight per wavefront
@@ -170,7 +171,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
         for (int i = 0; i < 4; i++) {
             uint32_t b = first + piece * 4 + i;
             b = b < tile.b_last ? b : tile.b_last;
-            const uint32_t* q = tile.lane_row + a.sz_offset + (size_t)b * SZW;
+            const uint32_t* q = tile.lane_row + a.sz_offset + (size_t)(PAIR ? b >> 1 : b) * SZW;
             if constexpr (SZW == 2) { const u32x2 t = *(const u32x2*)q; szr[i][0] = t.x; szr[i][1] = t.y; }
             else szr[i][0] = *q;
         }
@@ -530,7 +531,7 @@ bool gemv_mfma_planes_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t
     if (ms < 2 || ms > 16) return false;
     if (w.bits != 4 && w.bits != 8) return false;
     const uint32_t bc = 512 / w.bits;                                     // codes per block
-    if ((w.group != bc && w.group * 2 != bc) || w.k % bc) return false;
+    if ((w.group != bc && w.group * 2 != bc && !(w.bits == 8 && w.group == 2 * bc)) || w.k % w.group || w.k % bc) return false;
     if (x_stride % 8) return false;                                       // 128-bit activation loads
     // a row is one stream: its sz words follow its code words at the same pitch; code words 16-byte aligned
     if (w.sz_stride != w.code_stride || w.code_stride % 4 || (uintptr_t)w.codes % 16) return false;
@@ -592,7 +593,8 @@ mi355q_status launch_gemv_mfma_planes_multi(hipStream_t s, mi355q_context* ctx, 
     }
     a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = w[0].sb_dtype;
     const mi355q_status st = w[0].bits == 4 ? (w[0].group == 64 ? launch_pm_shape<4, 64>(s, a, g) : launch_pm_shape<4, 128>(s, a, g))
-                                            : (w[0].group == 32 ? launch_pm_shape<8, 32>(s, a, g) : launch_pm_shape<8, 64>(s, a, g));
+                                            : (w[0].group == 32 ? launch_pm_shape<8, 32>(s, a, g)
+                                               : w[0].group == 64 ? launch_pm_shape<8, 64>(s, a, g) : launch_pm_shape<8, 128>(s, a, g));
     if (st != MI355Q_OK || g.parts == 1) return st;
     uint32_t sum_wgs = (w[0].n + 255) / 256;
     if (sum_wgs > 65535u) sum_wgs = 65535u;

@@ -1,5 +1,5 @@
 """GPU parity tests of the small-batch matrix-core kernel over the split planes (4-bit codes in groups of 64 and 128,
-8-bit codes in groups of 32 and 64), through the C ABI: the projections of gemv_q4_g64 / gemm_q4_g64 and
+8-bit codes in groups of 32, 64 and 128), through the C ABI: the projections of gemv_q4_g64 / gemm_q4_g64 and
 gemv_q8_g32 / gemm_q8_g32 of the reference
 (MetalSourceGenerator+Quantized.swift:496-575, :22-156) for 4 <= M <= 16 rows per launch on the layout that serves M = 1
 (up to eight rows the two quantisation groups of a block are kept apart in the M dimension, above with two products).
@@ -28,11 +28,11 @@ def _fmt(pkg, group=64, bits=4):
     return pkg.QuantizationFormatRegistry.format_for_mlx_quantization(bits, group)
 
 
-@pytest.mark.parametrize("bits,group", [(4, 64), (4, 128), (8, 32), (8, 64)])
+@pytest.mark.parametrize("bits,group", [(4, 64), (4, 128), (8, 32), (8, 64), (8, 128)])
 def test_mfma_planes_seeded_shapes(pkg, ctx, bits, group):
     """Ragged row counts (tiles of sixteen rows end inside the matrix), one block (64 bytes of a row) up to rows of
     14336 codes (sixteen wavefronts a tile), every M the kernel takes; the plan record names it."""
-    for i, (n, k) in enumerate([(96, 512), (200, 1024), (33, 128), (17, 256), (64, 14336), (4100, 4096), (40, 64 * 8 // bits * 3)]):
+    for i, (n, k) in enumerate([(96, 512), (200, 1024), (33, 128), (17, 256), (64, 14336), (4100, 4096), (40, max(group, 512 // bits) * 3)]):
         words, s, z, wq = seeded_case(4100 + i + group + bits, n, k, bits, group)
         w = ctx.weight_prepare_mlx(_fmt(pkg, group, bits), words, s, z, pkg.BF16, pkg.LAYOUT_PLANES)
         for m in (((4, 5, 6, 7, 8, 9, 11, 13, 16) if n < 4000 else (4, 8, 16)) + ((3,) if bits == 8 else ())):
@@ -49,7 +49,7 @@ def test_mfma_planes_seeded_shapes(pkg, ctx, bits, group):
         w.destroy()
 
 
-@pytest.mark.parametrize("bits,group", [(4, 64), (8, 32), (8, 64)])
+@pytest.mark.parametrize("bits,group", [(4, 64), (8, 32), (8, 64), (8, 128)])
 def test_mfma_planes_exact_small_integers_f16_scales_and_strides(pkg, ctx, bits, group):
     """Exactly representable case: every product and partial sum (those of the offset codes included: 128 + q, and for
     8 bits 128 + l and 16 (128 + h)) is a multiple of 2^-6 that fits 24 bits, so the result is exact whatever the order
