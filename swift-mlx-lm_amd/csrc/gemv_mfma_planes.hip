@@ -1,5 +1,5 @@
 // Small-batch projection on the matrix cores straight from the split planes (4-bit codes in groups of 64 or 128,
-// 8-bit codes in groups of 32 or 64), 2 <= M <= 16 activation rows per launch: the layout that serves M = 1 best also
+// 8-bit codes in groups of 32, 64 or 128), 2 <= M <= 16 activation rows per launch: the layout that serves M = 1 best also
 // serves a batch.
 //
 // Stands in for gemv_q4_g{64,128} / gemv_q8_g{32,64} widened to the sequence signature and, at small sequence lengths,
