@@ -22,8 +22,9 @@
  *     (MC/Execution/MetalSubmissionContext.swift:56-120).
  *   - PRECONDITION: one stream per context at a time.  A context owns device scratch that its
  *     launches share (split-K partial sums of mi355q_qgemm, per-workgroup argmax keys of
- *     mi355q_argmax / mi355q_lmhead_argmax, part sums of the matrix-core decode layout, the clock
- *     probe).  Work enqueued through one context must therefore be ordered: on a single stream, or
+ *     mi355q_argmax / mi355q_lmhead_argmax, part sums of the matrix-core decode kernels, the dequantised
+ *     matrix of the two-dispatch prefill route, the bf16 rows that fp32 activations are split into, the
+ *     clock probe).  Work enqueued through one context must therefore be ordered: on a single stream, or
  *     on streams the caller has ordered with events.  Launches of one context that overlap in time
  *     on different streams race on that scratch and return wrong results without an error; a
  *     caller that wants concurrent streams creates one context per stream (contexts are cheap:
