@@ -216,8 +216,9 @@ mi355q_status launch_tile16_pack(hipStream_t s, const WView& planes, uint32_t* t
 // Rows from which it is taken; below, the split-plane dot-product kernels are as fast or faster (measured, Llama-3-8B
 // layer step in four launches: M = 2 42 us against 48 us here, M = 4 59 against 56, M = 8 117 against 55).
 // fewest activation rows for which the matrix-core kernel beats the dot-product kernels on the same planes (measured;
-// 8 bits, 4096 -> 14336: two rows 16 us on the dot products, three 25 us, against 19 us on the matrix cores)
-inline uint32_t mfma_planes_min_rows(uint32_t bits) { return bits == 8 ? 3u : 4u; }
+// 8 bits, 4096 -> 14336: two rows 16 us on the dot products, three 25 us, against 19 us on the matrix cores; 4 bits, a
+// Llama-3-8B layer step: two rows 42 us on the dot products, three 58-61 us, against 52-55 us on the matrix cores)
+inline uint32_t mfma_planes_min_rows(uint32_t bits) { (void)bits; return 3u; }
 // f16 rows are staged as two bf16 rows each: three f16 rows (six staged) pay on the matrix cores, two stay on the f16
 // dot-product kernels (a Llama-3-8B layer step at two f16 rows: 42.6 us there)
 inline bool mfma_planes_pays(uint32_t bits, int x_dtype, uint32_t m) {

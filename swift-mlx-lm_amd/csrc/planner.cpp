@@ -126,7 +126,7 @@ void plan_shared_launch_shape(const mi355q_weight* const* ws, uint32_t count, ui
                               mi355q_step* s) {
     WView all = ws[0]->view();
     uint64_t total = 0;
-    // four rows and more (three at 8 bits): the matrix-core kernel over the planes takes the rows of all matrices, in 16-row tiles
+    // three rows and more: the matrix-core kernel over the planes takes the rows of all matrices, in 16-row tiles
     bool on_planes = mfma_planes_pays(all.bits, x_dtype, m) && m <= 16;
     uint32_t tiles = 0;
     for (uint32_t i = 0; i < count && on_planes; i++) {

@@ -35,7 +35,7 @@ def test_mfma_planes_seeded_shapes(pkg, ctx, bits, group):
     for i, (n, k) in enumerate([(96, 512), (200, 1024), (33, 128), (17, 256), (64, 14336), (4100, 4096), (40, max(group, 512 // bits) * 3)]):
         words, s, z, wq = seeded_case(4100 + i + group + bits, n, k, bits, group)
         w = ctx.weight_prepare_mlx(_fmt(pkg, group, bits), words, s, z, pkg.BF16, pkg.LAYOUT_PLANES)
-        for m in (((4, 5, 6, 7, 8, 9, 11, 13, 16) if n < 4000 else (4, 8, 16)) + ((3,) if bits == 8 else ())):
+        for m in ((3, 4, 5, 6, 7, 8, 9, 11, 13, 16) if n < 4000 else (3, 4, 8, 16)):
             say(f"mfma planes q{bits} g{group} {k}->{n} M={m}")
             x = act_rounded(kat.seeded_activations(4200 + m, m, k), pkg.BF16, pkg)
             st = w.plan_decode_step(m) if m <= 8 else w.plan_prefill_steps(m)[0]
@@ -44,7 +44,7 @@ def test_mfma_planes_seeded_shapes(pkg, ctx, bits, group):
             assert_within_tolerance(y32, oracle.gemm_f64(wq, x), f"q{bits} g{group} {k}->{n} M={m}")
             ybf = run_gemv(ctx, pkg, w, x, pkg.BF16, pkg.BF16, use_qgemm=m > 8)
             assert np.array_equal(oracle.bf16_from_f32(ybf), oracle.bf16_from_f32(y32))
-        for m in ((2, 3) if bits == 4 else (2,)):               # below the threshold: the dot-product kernels
+        for m in (2,):                                          # below the threshold: the dot-product kernels
             assert w.plan_decode_step(m).device_kernel != f"gemv_mfma_planes_q{bits}_g{group}"
         w.destroy()
 
