@@ -366,7 +366,10 @@ MI355Q_API mi355q_status mi355q_argmax(mi355q_context* ctx, void* stream, const 
 
 /* OutputHeadFragment = LinearFragment + ArgmaxFragment (MC/Compilable/OutputHeadFragment.swift:5-8)
  * fused into one launch: fp32 logits [N] (optional, may be NULL) and the greedy token index.
- * M = 1 (the reference runs the head in lastToken mode, MC/Compiler/MetalPrefillStepBuilder.swift:493-507). */
+ * M = 1 (the reference runs the head in lastToken mode, MC/Compiler/MetalPrefillStepBuilder.swift:493-507).
+ * The fused kernels read bf16 activations on every layout and f16 ones on planes and blocks; fp32 activations
+ * (the prefill's last token) and f16 ones on TILE16 records run the projection on its own fast route into the
+ * logits buffer, which is then required, and an arg-max launch picks the token. */
 MI355Q_API mi355q_status mi355q_lmhead_argmax(mi355q_context* ctx, void* stream,
                                               const mi355q_weight* w, const void* x_dev,
                                               mi355q_dtype x_dtype, float* logits_f32_dev,

@@ -414,7 +414,13 @@ mi355q_status dispatch_output_head(mi355q_context* ctx, hipStream_t s, const mi3
     if (!logits)
         return fail(MI355Q_ERR_INVALID_ARGUMENT,
                     "a logits buffer is required when the fused head kernel does not accept the shape");
-    mi355q_status st = launch_gemv_generic(s, v, x, x_dtype, logits, MI355Q_F32, 1, xs, (uint32_t)w->n);
+    // fp32 activations (three bf16 rows on the bf16 decode kernel) and f16 ones on TILE16 records: the projection's own
+    // route for one row (2048 -> 65536 with fp32 activations: the per-code kernel takes hundreds of microseconds)
+    const bool routed = !(flags & MI355Q_FLAG_FORCE_GENERIC) && (uintptr_t)x % 16 == 0 &&
+                        (split_rows_chosen(v, x_dtype, 1, xs, flags) ||
+                         (x_dtype == MI355Q_F16 && gemv_tile16_eligible(v, x_dtype, 1, xs)));
+    mi355q_status st = routed ? dispatch_linear(ctx, s, w, x, x_dtype, logits, MI355Q_F32, 1, xs, (uint32_t)w->n, flags, true)
+                              : launch_gemv_generic(s, v, x, x_dtype, logits, MI355Q_F32, 1, xs, (uint32_t)w->n);
     if (st != MI355Q_OK) return st;
     return launch_argmax(s, logits, MI355Q_F32, (uint32_t)w->n, token, keys.ptr + keys.capacity);
 }

@@ -233,3 +233,31 @@ def test_batched_projections_other_activation_types(pkg, ctx):
                 b.free()
         for w in ws:
             w.destroy()
+
+
+def test_output_head_with_fp32_and_f16_rows(pkg, ctx):
+    """The output head with activation types the fused head kernels do not read (fp32 anywhere, f16 on TILE16 records):
+    the projection takes its fast route to fp32 logits, an arg-max launch picks the token.  Logits to 1e-5 of the fp64
+    reference on the unrounded activations, token = lowest-index argmax of the device's logits and of the reference."""
+    n, k = 8192, 2048
+    words, s, z, wq = seeded_case(5800, n, k, 4, 64)
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+    for layout, x_dtype in ((pkg.LAYOUT_PLANES, pkg.F32), (pkg.LAYOUT_TILE16, pkg.F32), (pkg.LAYOUT_TILE16, pkg.F16),
+                            (pkg.LAYOUT_STAF_BLOCKS, pkg.F32)):
+        w = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, layout)
+        x = kat.seeded_activations(5801, 1, k)
+        if x_dtype == pkg.F16:
+            x = x.astype(np.float16).astype(np.float32)
+        want = oracle.gemm_f64(wq, x)[0]
+        top2 = np.sort(want)[-2:]
+        assert top2[1] - top2[0] > 1e-3, "seed gives a near-tie; pick another"
+        xd = ctx.upload(x if x_dtype == pkg.F32 else x.astype(np.float16).view(np.uint16))
+        logits = ctx.alloc(n * 4); ctx.fill(logits, 0x7FC00000)
+        tok = ctx.upload(np.array([-7], np.int32))
+        for _ in range(2):
+            ctx.lmhead_argmax(w, xd, x_dtype, logits, tok); ctx.synchronize()
+            got = logits.download(np.float32)
+            assert rel_l2(got, want) <= 1e-5, (layout, x_dtype, rel_l2(got, want))
+            token = int(tok.download(np.int32)[0])
+            assert token == oracle.argmax_lowest(got) == int(np.argmax(want))
+        w.destroy(); xd.free(); logits.free(); tok.free()
