@@ -283,7 +283,7 @@ MI355Q_API mi355q_status mi355q_qgemv(mi355q_context* ctx, void* stream, const m
  *     scratch matrix of the context (N*K*2 bytes, plus 64 MiB of library workspace) and multiplied by
  *     the platform's dense GEMM library (hipBLASLt, opened with dlopen on first use; the reference
  *     calls matmul2d there).  Serves every registered format on every layout: from 16 rows where the
- *     fused kernel does not read the weight, from 1024 rows beside it (2048 when K > N).  bf16
+ *     fused kernel does not read the weight; beside it from 512 rows (768 when N >= 8192, 2048 when K > N).  bf16
  *     activations, fp32 or bf16 output, K and the row stride multiples of 8, 16-byte aligned x; f16
  *     activations likewise in f16; fp32 activations into an fp32 result as two bf16 products (bf16
  *     weights as in gemm_bf16_f32s, the activations split into bf16 high and low halves).  The

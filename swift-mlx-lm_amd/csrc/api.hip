@@ -210,7 +210,7 @@ bool gemm_two_step_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_st
         const uint32_t one_launch = small_batch_rows(w, x_dtype, x_stride);      // what one small-batch launch still takes
         return m >= least && m > one_launch;
     }
-    return m >= (w.k > w.n ? kTwoStepMinRowsLongK : kTwoStepMinRowsBesideFused);
+    return m >= (w.k > w.n ? kTwoStepMinRowsLongK : w.n >= kTwoStepWideColumns ? kTwoStepMinRowsWide : kTwoStepMinRowsBesideFused);
 }
 
 // The three forms of the route, by rows and activation type:

@@ -277,14 +277,17 @@ mi355q_status dense_library_gemm(hipStream_t s, mi355q_context* ctx, int ab_dtyp
                                  void* y, int y_dtype, uint32_t m, uint32_t n, uint32_t k, uint32_t x_stride,
                                  uint32_t y_stride, void* workspace, bool accumulate = false);
 void dense_library_release(mi355q_context* ctx);
-// Rows from which the two-dispatch route is taken.  Beside the fused matrix-core kernel (measured, q4 g64, N(0,1)
-// activations, fused against two-dispatch with the library's candidates timed): 4096 -> 14336 at M = 512 90-100
-// against 93-100 us, M = 1024 139-160 against 119-130 us, M = 2048 287-312 against 206-217 us; 14336 -> 4096 at
-// M = 1024 141-150 against 162-168 us, M = 2048 260-285 against 244-256 us, M = 4096 458-520 against 338-347 us.
+// Rows from which the two-dispatch route is taken.  Beside the fused matrix-core kernel (measured at sustained load,
+// q4 g64, N(0,1) activations, fused against two-dispatch with the library's candidates timed): 4096 -> 14336 at M = 512
+// 83 against 86 us, M = 768 136 against 101, M = 1024 126 against 115, M = 2048 242 against 199; 4096 -> 4096 at
+// M = 256 32 against 33 us, M = 512 46 against 41, M = 1024 61 against 53, M = 2048 92 against 67; 14336 -> 4096 at
+// M = 1024 133 against 153 us, M = 2048 234 against 236, M = 3072 349 against 289.  So: rows longer than the matrix
+// is tall (K > N) from 2048, wide matrices (N >= 8192) from 768, the others from 512.
 // Where only the decode kernels would serve (formats and layouts the fused kernel does not read; block layout,
 // 4096 -> 14336: M = 32 in four launches of eight rows 147 us, two-dispatch 47 us) it starts at sixteen rows.
 // f16 rows that the matrix-core decode kernels take eight a launch: from 32 rows.
-constexpr uint32_t kTwoStepMinRowsBesideFused = 1024, kTwoStepMinRowsLongK = 2048, kTwoStepMinRowsOtherwise = 16;
+constexpr uint32_t kTwoStepMinRowsLongK = 2048, kTwoStepMinRowsWide = 768, kTwoStepMinRowsBesideFused = 512;
+constexpr uint32_t kTwoStepWideColumns = 8192, kTwoStepMinRowsOtherwise = 16;
 constexpr uint32_t kTwoStepMinRowsF16Batches = 32;
 // Rows from which mi355q_gemm_bf16 hands a plain dense product to the library.
 constexpr uint32_t kDenseLibraryMinRows = 128;

@@ -320,7 +320,8 @@ def test_tile16_prefill_runs_on_the_matrix_cores(pkg, ctx):
         wp = ctx.weight_prepare_mlx(_fmt(pkg), words, s, z, pkg.BF16, pkg.LAYOUT_PLANES)
         x = act_rounded(kat.seeded_activations(2750 + i, m, k), pkg.BF16, pkg)
         say(f"tile16 prefill {k}->{n} M={m}")
-        got = _run(ctx, pkg, wt, x, pkg.F32, use_qgemm=True, flags=0 if 32 < m < 1024 else pkg.FLAG_FORCE_MFMA)
+        two_step_from = 2048 if k > n else 768 if n >= 8192 else 512       # rows from which dequantise once + dense GEMM
+        got = _run(ctx, pkg, wt, x, pkg.F32, use_qgemm=True, flags=0 if 32 < m < two_step_from else pkg.FLAG_FORCE_MFMA)
         same = _run(ctx, pkg, wp, x, pkg.F32, use_qgemm=True, flags=pkg.FLAG_FORCE_MFMA)
         assert np.array_equal(got, same), f"{k}->{n} M={m}: records and planes disagree"
         if m * n * k <= 2 ** 28:
@@ -329,7 +330,7 @@ def test_tile16_prefill_runs_on_the_matrix_cores(pkg, ctx):
         st = wt.plan_prefill_steps(m, flags=pkg.FLAG_FORCE_MFMA)[0]
         assert st.device_kernel == "qgemm_mfma_q4_g64" and not st.used_fallback
         unforced = [s.device_kernel for s in wt.plan_prefill_steps(m)]     # long prompts: dequantise once + dense GEMM
-        assert unforced == (["dequant_q4_g64_bf16", "hipblaslt_gemm_bf16"] if m >= 1024 else
+        assert unforced == (["dequant_q4_g64_bf16", "hipblaslt_gemm_bf16"] if m >= two_step_from else
                             ["qgemm_mfma_q4_g64"] if m > 32 else ["gemv_tile16_q4_g64"])
         if m <= 32:                                          # two launches of the small-batch kernel: unrounded weights
             assert_within_tolerance(_run(ctx, pkg, wt, x, pkg.F32, use_qgemm=True), oracle.gemm_f64(wq, x), f"M={m} in steps")

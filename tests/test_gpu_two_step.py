@@ -103,7 +103,7 @@ def test_two_step_seeded_ragged_shapes_and_strides(pkg, ctx, bits, group, layout
 
 def test_two_step_is_chosen_where_measured_faster_and_planned_as_two_steps(pkg, ctx):
     """Without flags: the block layout (no fused matrix-core kernel) takes the route from sixteen rows; the planes keep
-    the fused kernel up to 1023 rows (shapes with K > N up to 2047).  The planner reports dequant + GEMM as two steps."""
+    the fused kernel up to 511 rows (wide matrices, N >= 8192, up to 767; shapes with K > N up to 2047).  The planner reports dequant + GEMM as two steps."""
     n, k = 192, 512
     words, s, z, wq = seeded_case(3300, n, k, 4, 64)
     fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
@@ -118,9 +118,14 @@ def test_two_step_is_chosen_where_measured_faster_and_planned_as_two_steps(pkg, 
     assert not steps[0].used_fallback and not steps[1].used_fallback
     assert len(ws.plan_prefill_steps(12)) == 1 and ws.plan_prefill_steps(12)[0].used_fallback
     assert len(ws.plan_prefill_steps(64, flags=pkg.FLAG_FORCE_SMALL_M)) == 1
-    assert [st.kernel_family for st in wp.plan_prefill_steps(1023)] == ["mfmaGEMM"]
-    assert [st.kernel_family for st in wp.plan_prefill_steps(1024)] == ["dequantToBFloat", "libraryGEMM"]
+    assert [st.kernel_family for st in wp.plan_prefill_steps(511)] == ["mfmaGEMM"]
+    assert [st.kernel_family for st in wp.plan_prefill_steps(512)] == ["dequantToBFloat", "libraryGEMM"]
     assert [st.kernel_family for st in wp.plan_prefill_steps(1024, flags=pkg.FLAG_FORCE_MFMA)] == ["mfmaGEMM"]
+    words3, s3, z3, _ = seeded_case(3304, 8192, 64, 4, 64)                # wide: N >= 8192
+    ww = ctx.weight_prepare_mlx(fmt, words3, s3, z3, pkg.BF16, pkg.LAYOUT_PLANES)
+    assert [st.kernel_family for st in ww.plan_prefill_steps(767)] == ["mfmaGEMM"]
+    assert [st.kernel_family for st in ww.plan_prefill_steps(768)] == ["dequantToBFloat", "libraryGEMM"]
+    ww.destroy()
     # K > N: the fused kernel keeps the shape up to 2047 rows
     words2, s2, z2, _ = seeded_case(3301, 128, 1024, 4, 64)
     wl = ctx.weight_prepare_mlx(fmt, words2, s2, z2, pkg.BF16, pkg.LAYOUT_PLANES)
