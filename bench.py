@@ -625,7 +625,7 @@ def main():
             for mm in (128, 512, 2048, 4096):
                 xb = ctx.upload(oracle.bf16_from_f32(kat.seeded_activations(500 + mm, mm, k)))        # N(0,1)
                 yb = ctx.alloc(mm * n * 2)
-                for i in range(4):
+                for i in range(len(wts)):
                     ctx.qgemm(wts[i], xb, pkg.BF16, yb, pkg.BF16, mm, 0, 0, 0, stream)
                 ctx.synchronize(stream)
                 reps = 24 if mm >= 2048 else 48
@@ -642,10 +642,10 @@ def main():
             xa = kat.seeded_activations(2548, 2048, 4096).astype(npdt)
             xb = ctx.upload(xa.view(np.uint16) if tname == "f16" else xa)
             yb = ctx.alloc(2048 * 14336 * 4)
-            for i in range(4):
+            for i in range(len(wts)):
                 ctx.qgemm(wts[i], xb, xt, yb, xt, 2048, 0, 0, 0, stream)
             ctx.synchronize(stream)
-            ms, ms_first, taken = steady_region(ctx, lambda i: ctx.qgemm(wts[i % 4], xb, xt, yb, xt, 2048, 0, 0, 0, stream), 12, stream)
+            ms, ms_first, taken = steady_region(ctx, lambda i: ctx.qgemm(wts[i % len(wts)], xb, xt, yb, xt, 2048, 0, 0, 0, stream), 12, stream)
             sweep[f"gate 4096->14336 M=2048 {tname} activations"] = {
                 "us": round(ms * 1e3, 1), "TFLOPs": round(2.0 * 2048 * 14336 * 4096 / (ms * 1e-3) / 1e12, 1),
                 "first_sample_us": round(ms_first * 1e3, 1), "samples_of": [taken, 12],
