@@ -1,0 +1,113 @@
+"""GPU parity sweep over the dispatcher's choices through the C ABI: seeded random combinations of format, device
+layout, activation type, output type, row count (1 to 70, across every small-batch, stepping, split and prefill
+threshold), row strides with padding, and entry point (mi355q_qgemv up to eight rows, mi355q_qgemm, the shared launch
+of two or three projections), each against the CPU oracle on the same inputs
+(gemv_q{b}_g{g} / gemm_q{b}_g{g}[_f32s] / batched_gemm_q4_g64_{2,3},
+Sources/MetalCompiler/Generator/MetalSourceGenerator+Quantized.swift:22-338, 496-575).
+
+Bar: relative L2 <= 2.5e-3 and max-abs <= 2e-2 of an fp64 accumulation of the dequantised weights and the activations as
+rounded to their type (the prefill routes round the weights to bf16 once, which alone is 1.5e-3; the decode routes
+meet 1e-3 and are tested at that bar elsewhere); poisoned padding of the activation rows must not reach the result,
+the canary behind the output rows must survive, 16-bit outputs are within one rounding of the fp32 result.
+"""
+import sys
+
+import numpy as np
+import pytest
+
+import kat
+import oracle
+from gpu_util import act_rounded, act_to_device_array, out_from_device, rel_l2, seeded_case
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+FORMATS = [(4, 64), (4, 128), (8, 32), (8, 64), (8, 128), (3, 64), (2, 64), (6, 64), (5, 32), (3, 16)]
+
+
+def _one_case(pkg, ctx, rng, idx):
+    bits, group = FORMATS[int(rng.integers(len(FORMATS)))]
+    layouts = [pkg.LAYOUT_PLANES, pkg.LAYOUT_STAF_BLOCKS] + ([pkg.LAYOUT_TILE16] if (bits, group) == (4, 64) else [])
+    layout = layouts[int(rng.integers(len(layouts)))]
+    k = int(rng.choice([128, 256, 384, 512, 1024, 2048 + 128])) // group * group or group
+    k = max(k, 128) // 128 * 128
+    n = int(rng.choice([1, 17, 48, 100, 257, 300]))
+    m = int(rng.choice([1, 2, 3, 4, 5, 7, 8, 9, 12, 15, 16, 17, 24, 31, 32, 33, 40, 70]))
+    x_dtype = [pkg.BF16, pkg.F16, pkg.F32][int(rng.integers(3))]
+    y_dtype = [pkg.F32, pkg.BF16, pkg.F16][int(rng.integers(3))]
+    xpad = int(rng.choice([0, 0, 8, 24]))
+    ypad = int(rng.choice([0, 0, 5]))
+    entry = "qgemv" if m <= 8 and rng.integers(2) else "qgemm"
+    what = f"#{idx} q{bits} g{group} layout {layout} {k}->{n} M={m} x{x_dtype} y{y_dtype} xpad {xpad} ypad {ypad} {entry}"
+    say(what)
+    words, s, z, wq = seeded_case(9000 + idx, n, k, bits, group)
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(bits, group)
+    w = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, layout)
+    x = act_rounded(kat.seeded_activations(9500 + idx, m, k), x_dtype, pkg)
+    xh = np.full((m, k + xpad), 3.0e4, np.float32); xh[:, :k] = x
+    xd = ctx.upload(act_to_device_array(xh, x_dtype, pkg))
+    ysz = 4 if y_dtype == pkg.F32 else 2
+    if (m * (n + ypad) * ysz) % 4:                           # the canary fill writes whole 32-bit words
+        ypad += 1
+    yd = ctx.alloc(m * (n + ypad) * ysz)
+    ctx.fill(yd, 0x7FC07FC0 if ysz == 2 else 0x7FC00000)
+    getattr(ctx, entry)(w, xd, x_dtype, yd, y_dtype, m, k + xpad, (n + ypad) if ypad else 0, 0)
+    ctx.synchronize()
+    got = out_from_device(yd, y_dtype, (m, n + ypad), pkg)
+    assert np.all(np.isnan(got[:, n:])), what
+    got = got[:, :n]
+    want = oracle.gemm_f64(wq, x)
+    assert np.all(np.isfinite(got)), what
+    tol16 = {pkg.F32: 0.0, pkg.BF16: 2.0 ** -8, pkg.F16: 2.0 ** -11}[y_dtype]
+    r = rel_l2(got, want)
+    assert r <= 2.5e-3 + tol16, f"{what}: rel-L2 {r:.3e}"
+    assert float(np.max(np.abs(got - want))) <= 2e-2 + tol16 * float(np.max(np.abs(want))), what
+    w.destroy(); xd.free(); yd.free()
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_random_dispatch_combinations(pkg, ctx, seed):
+    rng = np.random.default_rng(7700 + seed)
+    for i in range(45):
+        _one_case(pkg, ctx, rng, seed * 100 + i)
+
+
+def test_random_shared_launches(pkg, ctx):
+    """Two or three projections on one set of activations, every type and row count: the same bits as the separate
+    calls of mi355q_qgemm."""
+    rng = np.random.default_rng(7800)
+    for i in range(30):
+        bits, group = [(4, 64), (4, 64), (8, 32), (3, 64), (4, 128)][int(rng.integers(5))]
+        layouts = [pkg.LAYOUT_PLANES, pkg.LAYOUT_STAF_BLOCKS] + ([pkg.LAYOUT_TILE16] if (bits, group) == (4, 64) else [])
+        layout = layouts[int(rng.integers(len(layouts)))]
+        k = int(rng.choice([256, 512, 1024]))
+        ns = [int(v) for v in rng.choice([16, 40, 96, 130, 256], int(rng.integers(2, 4)))]
+        m = int(rng.choice([1, 2, 3, 5, 8, 9, 13, 16, 17, 24, 33]))
+        x_dtype = [pkg.BF16, pkg.F16, pkg.F32][int(rng.integers(3))]
+        y_dtype = [pkg.F32, pkg.BF16][int(rng.integers(2))]
+        say(f"shared #{i} q{bits} g{group} layout {layout} K={k} N={ns} M={m} x{x_dtype} y{y_dtype}")
+        fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(bits, group)
+        ws = []
+        for j, n in enumerate(ns):
+            words, s, z, _ = seeded_case(9800 + 10 * i + j, n, k, bits, group)
+            ws.append(ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, layout))
+        x = act_rounded(kat.seeded_activations(9900 + i, m, k), x_dtype, pkg)
+        xd = ctx.upload(act_to_device_array(x, x_dtype, pkg))
+        ysz = 4 if y_dtype == pkg.F32 else 2
+        yds = [ctx.alloc(m * n * ysz) for n in ns]
+        ctx.batched_qgemm(ws, xd, x_dtype, yds, y_dtype, m); ctx.synchronize()
+        for j, n in enumerate(ns):
+            fused = out_from_device(yds[j], y_dtype, (m, n), pkg)
+            alone = ctx.alloc(m * n * ysz)
+            ctx.qgemm(ws[j], xd, x_dtype, alone, y_dtype, m, 0, 0, 0); ctx.synchronize()
+            assert np.array_equal(fused, out_from_device(alone, y_dtype, (m, n), pkg)), (i, j)
+            alone.free()
+        xd.free()
+        for b in yds:
+            b.free()
+        for w in ws:
+            w.destroy()
