@@ -90,7 +90,8 @@ enum {
     MI355Q_FLAG_FORCE_SMALL_M = 2, /* qgemm: use the small-M GEMV-style kernel whatever M is */
     MI355Q_FLAG_FORCE_MFMA = 4,    /* qgemm: use the fused MFMA kernel whatever M is */
     /* bit 3 (value 8) is taken by the measurement flag of mi355_qlinear_probe.h */
-    MI355Q_FLAG_FORCE_TWO_STEP = 16 /* qgemm: dequantise to bf16 scratch, then the dense library GEMM, whatever M is */
+    MI355Q_FLAG_FORCE_TWO_STEP = 16, /* qgemm: dequantise to bf16 scratch, then the dense library GEMM, whatever M is */
+    MI355Q_FLAG_FORCE_STREAM = 32  /* qgemm: the streamed-weight matrix-core kernel (4-bit planes, bf16 rows, M <= 96) */
 };
 
 /* ------------------------------------------------------------------------------------------

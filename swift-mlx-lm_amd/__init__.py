@@ -22,6 +22,7 @@ F16, BF16, F32 = 0, 1, 2
 LAYOUT_STAF_BLOCKS, LAYOUT_PLANES, LAYOUT_TILE16 = 0, 1, 2
 # launch flags
 FLAG_NONE, FLAG_FORCE_GENERIC, FLAG_FORCE_SMALL_M, FLAG_FORCE_MFMA, FLAG_PROBE_CLOCK, FLAG_FORCE_TWO_STEP = 0, 1, 2, 4, 8, 16
+FLAG_FORCE_STREAM = 32
 
 STATUS_NAMES = {0: "OK", -1: "INVALID_ARGUMENT", -2: "UNSUPPORTED_FORMAT", -3: "SHAPE", -4: "NULL_HANDLE",
                 -5: "DEVICE", -6: "OUT_OF_MEMORY", -7: "KERNEL_NOT_FOUND", -8: "SIZE_MISMATCH",

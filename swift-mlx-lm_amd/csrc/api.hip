@@ -140,6 +140,10 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
     if ((forced & (MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_TWO_STEP)) && (forced & (forced - 1)))
         return fail(MI355Q_ERR_INVALID_ARGUMENT, "contradictory kernel selection flags");
     const WView v = w->view();
+    if (flags & MI355Q_FLAG_FORCE_STREAM) {
+        if (forced) return fail(MI355Q_ERR_INVALID_ARGUMENT, "contradictory kernel selection flags");
+        return launch_qgemm_stream(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
+    }
     if (flags & MI355Q_FLAG_FORCE_TWO_STEP) {
         if (!gemm_two_step_eligible(v, x_dtype, m, xs) || (uintptr_t)x % 16)
             return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the two-dispatch route takes 16-byte aligned activations, K and the row stride multiples of 8");
@@ -160,6 +164,9 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
             return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the MFMA GEMM does not accept this format, layout or stride");
         return launch_qgemm_mfma(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys, probe);
     }
+    // a few dozen rows on 4-bit planes: weights streamed through registers, activations alone through LDS
+    if (!forced && gemm_stream_chosen(v, x_dtype, m, xs) && (uintptr_t)x % 16 == 0)
+        return launch_qgemm_stream(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
     // the decode kernels take up to 8 rows per launch, 16 on the matrix cores (and then pay for a second launch too)
     const bool small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) ||
                        m <= small_batch_limit(v, x_dtype, xs) || !mfma_ok;
@@ -172,7 +179,16 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
 // prefill kernel, 32 rows 136 against 161).
 uint32_t small_batch_limit(const WView& w, int x_dtype, uint32_t x_stride) {
     const uint32_t rows = small_batch_rows(w, x_dtype, x_stride);
+    if (gemm_stream_eligible(w, x_dtype, rows + 1, x_stride)) return rows;     // the streamed-weight kernel takes over
     return rows >= 16 ? 2 * rows : rows;
+}
+
+// Rows the streamed-weight kernel serves: beyond one small-batch launch, up to its own limit (4096 -> 14336 q4 g64:
+// 17 rows 16.6 us where two small-batch launches take 25.8 and the tiled kernel 30.2; 32 rows 17.1 against 33.1 and
+// 29.6; 64 rows 21.1 against 33.2 tiled; 96 rows 26.5 against 35.0; 14336 -> 4096: 32 rows 19.3 against 31.4, 96 rows
+// 28.0 against 35.4; 4096 -> 4096: 32 rows 12.4 against 17.6, 96 rows 17.9 against 22.7).
+bool gemm_stream_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
+    return m <= kStreamMaxRows && gemm_stream_eligible(w, x_dtype, m, x_stride) && m > small_batch_limit(w, x_dtype, x_stride);
 }
 
 uint32_t small_batch_rows(const WView& w, int x_dtype, uint32_t x_stride) {
@@ -194,7 +210,7 @@ bool gemm_two_step_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_
 }
 
 bool gemm_two_step_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride, uint32_t flags) {
-    if (flags & (MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) return false;
+    if (flags & (MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_STREAM)) return false;
     if (flags & MI355Q_FLAG_FORCE_TWO_STEP) return true;
     if (!gemm_two_step_eligible(w, x_dtype, m, x_stride)) return false;
     if (!gemm_mfma_eligible(w, x_dtype, m, x_stride)) {

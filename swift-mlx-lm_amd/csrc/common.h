@@ -266,6 +266,20 @@ bool gemm_mfma_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stri
 mi355q_status launch_qgemm_mfma(hipStream_t s, mi355q_context* ctx, const WView& w,
                                 const void* x, int x_dtype, void* y, int y_dtype, uint32_t m,
                                 uint32_t x_stride, uint32_t y_stride, unsigned long long* probe = nullptr);
+// Streamed-weight matrix-core kernel (gemm_stream.hip): 4-bit planes, bf16 activations, at most 96 rows.
+constexpr uint32_t kStreamMaxRows = 96;
+struct StreamLaunchShape {
+    uint32_t row_blocks;       // workgroups along N (64 weight rows each)
+    uint32_t parts;            // K parts (workgroups along K; fp32 partial results added by a second launch)
+    uint32_t iters_per_part;   // iterations of 256 columns per part
+    uint32_t m_blocks;         // 32-row blocks of activations
+    uint32_t lds_bytes;
+};
+bool gemm_stream_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
+bool gemm_stream_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
+StreamLaunchShape gemm_stream_shape(const mi355q_context* ctx, uint32_t m, uint32_t n, uint32_t k);
+mi355q_status launch_qgemm_stream(hipStream_t s, mi355q_context* ctx, const WView& w, const void* x, int x_dtype, void* y,
+                                  int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride);
 // Two-dispatch prefill route: dequantise the whole matrix to bf16 in the context's scratch, then the platform's
 // dense GEMM.  `dense_library_serves` answers whether the library can be opened and has an algorithm for the problem.
 constexpr size_t kDenseLibraryWorkspace = (size_t)64 << 20;

@@ -1,0 +1,345 @@
+// Projection of 17 to 96 activation rows on the matrix cores with the weights streamed through registers:
+//   Y[M,N] = X[M,K] * W[N,K]^T,  W = 4-bit group-affine codes on the split planes, bf16 activations.
+//
+// Stands in, at these sequence lengths, for the reference's direct quantized GEMM gemm_q4_g64 / gemm_q4_g128
+// (Sources/MetalCompiler/Generator/MetalSourceGenerator+Quantized.swift:22-156) and for its dequant + matmul2d pair
+// (MetalSourceGenerator+Linear.swift:18-81).  The tiled prefill kernel dequantises a weight K-tile into LDS once per
+// workgroup and spends a barrier round trip on it whatever M is; with at most three 32-row blocks of activations the
+// whole M extent fits one wavefront's accumulators, so here nothing but the activations goes through LDS:
+//   * eight wavefronts of a workgroup own 64 weight rows: two blocks of 32 rows, each walked by four wavefronts
+//     that take every fourth 64-code K-tile (K slice s takes tiles 4 i + s), so the four touch one 128-byte line of
+//     a row together;
+//   * lane (n, h) of a wavefront loads 16 bytes = words 4h .. 4h+3 of row n's K-tile and uses word j in k-step j:
+//     the eight codes of a word become the B operand of v_mfma_f32_32x32x16_bf16 in registers (byte-lane convert,
+//     fp32 fma with the group's scale and bias, one rounding to bf16: the weights of the tiled kernel, bit for bit);
+//     the A operand is the activations' chunk 4h + j of that K-tile, read from LDS;
+//   * per iteration four more wavefronts of the workgroup stage [32 MB rows][256 columns] of activations
+//     (XOR-swizzled 128-byte rows per K slice) two iterations ahead into the third of three LDS stages, copied
+//     global -> LDS directly; the multiplying wavefronts fetch weight words six iterations ahead and wait for nothing
+//     else; one barrier per iteration;
+//   * the four K slices of a row block add their accumulators through LDS at the end; with K split over workgroups
+//     (few rows, long K) fp32 partial results go to scratch and a second launch adds them.
+#include "device_utils.h"
+#include <atomic>
+
+namespace mi355q {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 st_bf16x8_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float st_floatx16_t;
+typedef __bf16 st_bf16x2_v __attribute__((ext_vector_type(2)));
+typedef float st_float2_v __attribute__((ext_vector_type(2)));
+
+struct StreamArgs {
+    const uint32_t* codes;     // [N][code_stride] words, eight codes a word
+    const uint32_t* sz;        // [N][sz_stride] words: scale | bias << 16 per group
+    const uint16_t* x;         // bf16 [M][xs]
+    void* y;
+    float* partial;            // K split over workgroups: fp32 [parts][M][N]; else null
+    uint32_t m, n, k, xs, ys;
+    uint32_t code_stride, sz_stride;
+    uint32_t y_dtype;
+    uint32_t iters_per_part;   // iterations (256 columns each) per K part; blockIdx.y is the part
+};
+
+constexpr int kStreamIterK = 256;      // columns of K per iteration: one 64-code K-tile per K slice
+constexpr int kStreamRows = 64;        // weight rows per workgroup
+constexpr int kStreamAhead = 6;        // iterations the weight words are fetched ahead (and the loop's unroll)
+constexpr int kStreamThreads = 768;    // eight multiplying wavefronts and four that stage the activations
+
+__device__ __forceinline__ uint32_t st_pack_bf16(float lo, float hi) {
+    st_float2_v v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, st_bf16x2_v));
+}
+
+// Byte offset of 16-byte chunk `chunk` of row `row` in a [rows][128 bytes] array: the chunk position is rotated by
+// (row / 2) % 8, so sixteen consecutive rows reading or writing one logical chunk touch sixteen different bank groups.
+__device__ __forceinline__ uint32_t st_lds_off(uint32_t row, uint32_t chunk) {
+    return row * 128u + ((chunk ^ ((row >> 1) & 7u)) << 4);
+}
+
+template <int GROUP, int MB, bool SB_BF16>
+__global__ __launch_bounds__(kStreamThreads) void qgemm_stream_kernel(StreamArgs a) {
+    constexpr int MPAD = 32 * MB;                         // staged activation rows
+    constexpr int SLICE_BYTES = MPAD * 128;               // one K slice of a stage: [MPAD][64] bf16
+    constexpr int STAGE = 4 * SLICE_BYTES;
+    constexpr int XP = 4 * MB;                            // copy instructions (eight rows of a K slice each) per stage
+    constexpr int U = kStreamAhead;
+    extern __shared__ u32x4 smem_st[];
+    char* const lds = (char*)smem_st;
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const bool stager = wave >= 8;                        // wavefronts 8..11 move the activations, 0..7 multiply
+    const uint32_t rb = (wave >> 2) & 1u, slice = wave & 3u;     // row block, K slice
+    const uint32_t ln = lane & 31, lh = lane >> 5;
+    const uint32_t n0 = blockIdx.x * kStreamRows + rb * 32;
+
+    const uint32_t KT = a.k / 64;                         // K-tiles
+    const uint32_t it_all = (a.k + kStreamIterK - 1) / kStreamIterK;
+    const uint32_t it_begin = blockIdx.y * a.iters_per_part;
+    const uint32_t it_end = it_begin + a.iters_per_part < it_all ? it_begin + a.iters_per_part : it_all;
+
+    st_floatx16_t acc[MB];
+#pragma unroll
+    for (int i = 0; i < MB; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[i][r] = 0.0f;
+
+    if (stager) {
+        // Activations, global -> LDS without a register in between (global_load_lds_dwordx4: lane L's 16 bytes land at
+        // the base in M0 + 16 L), two iterations ahead into the third stage.  Staging wavefront w moves K slice w: one
+        // instruction covers eight rows of the slice, and lane L fetches the chunk that belongs at its position after
+        // the rotation of st_lds_off.  These wavefronts wait on nothing but their own copies (which hit the L2): were
+        // the multiplying wavefronts to stage the activations themselves, every wait for a staged chunk would also
+        // wait for the older weight loads, and the distance the weights are fetched ahead would shrink to that of the
+        // activations.
+        const uint32_t xs_slice = wave - 8;
+        const uint32_t lds_base = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) uint8_t*)lds) + xs_slice * SLICE_BYTES;
+        const uint32_t xrow = lane >> 3;
+        auto issue = [&](uint32_t stage, uint32_t it) __attribute__((always_inline)) {
+            uint32_t col0 = it * kStreamIterK + xs_slice * 64;
+            col0 = col0 + 64 <= a.k ? col0 : a.k - 64;    // a K slice past K has no tile there: what it stages is not read
+#pragma unroll
+            for (int q = 0; q < XP; q++) {
+                const uint32_t row = 8 * q + xrow;
+                const uint32_t chunk = (lane & 7u) ^ ((row >> 1) & 7u);
+                const uint32_t r = row < a.m ? row : a.m - 1;
+                const uint16_t* const g = a.x + (size_t)r * a.xs + col0 + chunk * 8;
+                const uint32_t l = lds_base + stage * STAGE + q * 1024;
+                asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(l) : "memory");
+            }
+        };
+        issue(0, it_begin);
+        if (it_begin + 1 < it_end) {
+            issue(1, it_begin + 1);
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(XP) : "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        __syncthreads();
+        for (uint32_t it0 = it_begin; it0 < it_end; it0 += 3) {
+            static_for<3>([&](auto I) __attribute__((always_inline)) {
+                constexpr int i = decltype(I)::value;
+                const uint32_t it = it0 + i;
+                if (it < it_end) {
+                    // the stage iteration it - 1 was read from is free since the last barrier; iteration it + 1 must
+                    // have landed before the next one
+                    if (it + 2 < it_end) {
+                        issue((i + 2) % 3, it + 2);
+                        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(XP) : "memory");
+                    } else {
+                        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    }
+                    __syncthreads();
+                }
+            });
+        }
+    } else {
+        uint32_t wrow = n0 + ln;
+        wrow = wrow < a.n ? wrow : a.n - 1;               // rows past the end re-read the last one
+        const uint32_t* const crow = a.codes + (size_t)wrow * a.code_stride + 4 * lh;
+        const uint32_t* const szrow = a.sz + (size_t)wrow * a.sz_stride;
+        // weight words and (scale, bias) word of this wavefront's K-tile of iteration `it`
+        u32x4 ring[U];
+        uint32_t szring[U];
+        auto load_w = [&](auto I, uint32_t it) __attribute__((always_inline)) {
+            constexpr int i = decltype(I)::value;
+            uint32_t t = it * 4 + slice;
+            t = t < KT ? t : KT - 1;
+            ring[i] = *(const u32x4*)(crow + (size_t)t * 8);
+            szring[i] = szrow[(t * 64) / GROUP];
+        };
+        static_for<U>([&](auto I) __attribute__((always_inline)) { load_w(I, it_begin + decltype(I)::value); });
+        __syncthreads();
+        for (uint32_t it0 = it_begin; it0 < it_end; it0 += U) {
+            static_for<U>([&](auto I) __attribute__((always_inline)) {
+                constexpr int i = decltype(I)::value;
+                constexpr int stage = i % 3;
+                const uint32_t it = it0 + i;
+                if (it < it_end) {                        // the same for every wavefront of the workgroup
+                    const u32x4 w = ring[i];
+                    const uint32_t szw = szring[i];
+                    load_w(I, it + U);
+                    if (it * 4 + slice < KT) {
+                        float s, z;
+                        if constexpr (SB_BF16) {
+                            s = __uint_as_float(szw << 16); z = __uint_as_float(szw & 0xFFFF0000u);
+                        } else {
+                            s = f16_to_f32((uint16_t)(szw & 0xFFFFu)); z = f16_to_f32((uint16_t)(szw >> 16));
+                        }
+                        const char* const xs_lds = lds + stage * STAGE + slice * SLICE_BYTES;
+                        static_for<4>([&](auto J) __attribute__((always_inline)) {
+                            constexpr int j = decltype(J)::value;
+                            const uint32_t word = j == 0 ? w.x : j == 1 ? w.y : j == 2 ? w.z : w.w;
+                            const uint32_t lo = word & 0x0F0F0F0Fu, hi = (word >> 4) & 0x0F0F0F0Fu;
+                            float q[8];
+                            asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(q[0]) : "v"(lo));
+                            asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(q[1]) : "v"(hi));
+                            asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(q[2]) : "v"(lo));
+                            asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(q[3]) : "v"(hi));
+                            asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(q[4]) : "v"(lo));
+                            asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(q[5]) : "v"(hi));
+                            asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(q[6]) : "v"(lo));
+                            asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(q[7]) : "v"(hi));
+                            u32x4 o;
+                            o.x = st_pack_bf16(__builtin_fmaf(s, q[0], z), __builtin_fmaf(s, q[1], z));
+                            o.y = st_pack_bf16(__builtin_fmaf(s, q[2], z), __builtin_fmaf(s, q[3], z));
+                            o.z = st_pack_bf16(__builtin_fmaf(s, q[4], z), __builtin_fmaf(s, q[5], z));
+                            o.w = st_pack_bf16(__builtin_fmaf(s, q[6], z), __builtin_fmaf(s, q[7], z));
+                            const st_bf16x8_t bw = __builtin_bit_cast(st_bf16x8_t, o);
+#pragma unroll
+                            for (int b = 0; b < MB; b++) {
+                                const st_bf16x8_t ax = *(const st_bf16x8_t*)(xs_lds + st_lds_off(b * 32 + ln, 4 * lh + j));
+                                acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ax, bw, acc[b], 0, 0, 0);
+                            }
+                            if constexpr (MB >= 3) __builtin_amdgcn_sched_barrier(0);   // one word at a time: registers
+                        });
+                    }
+                    __syncthreads();
+                }
+            });
+        }
+    }
+
+    // ---- the four K slices of a row block add up through LDS (the staged activations are done with) ----------------
+    float* const red = (float*)lds;
+    if (!stager && slice != 0) {
+        float* const mine = red + (size_t)(rb * 3 + slice - 1) * (16 * MB * 64);
+#pragma unroll
+        for (int b = 0; b < MB; b++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) mine[(b * 16 + r) * 64 + lane] = acc[b][r];
+    }
+    __syncthreads();
+    if (stager || slice != 0) return;
+#pragma nounroll
+    for (int sl = 0; sl < 3; sl++) {
+        const float* const other = red + (size_t)(rb * 3 + sl) * (16 * MB * 64);
+#pragma unroll
+        for (int b = 0; b < MB; b++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[b][r] += other[(b * 16 + r) * 64 + lane];
+    }
+    const uint32_t col = n0 + ln;
+    if (col >= a.n) return;
+#pragma unroll
+    for (int b = 0; b < MB; b++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const uint32_t row = b * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
+            if (row >= a.m) continue;
+            const float v = acc[b][r];
+            if (a.partial) {
+                a.partial[((size_t)blockIdx.y * a.m + row) * a.n + col] = v;
+                continue;
+            }
+            const size_t o = (size_t)row * a.ys + col;
+            if (a.y_dtype == MI355Q_F32) ((float*)a.y)[o] = v;
+            else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)a.y)[o] = f32_to_bf16_rne(v);
+            else ((uint16_t*)a.y)[o] = f32_to_f16_rne(v);
+        }
+}
+
+// y = the sum of the K parts' fp32 partial results, part 0 first, rounded once to the output type
+__global__ __launch_bounds__(256) void stream_sum_parts_kernel(const float* __restrict__ partial, void* __restrict__ y,
+                                                               uint32_t m, uint32_t n, uint32_t ys, uint32_t parts,
+                                                               uint32_t y_dtype) {
+    const size_t total = (size_t)m * n;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        float v = 0.f;
+        for (uint32_t p = 0; p < parts; p++) v += partial[(size_t)p * total + i];
+        const size_t row = i / n, col = i - row * n;
+        const size_t o = row * ys + col;
+        if (y_dtype == MI355Q_F32) ((float*)y)[o] = v;
+        else if (y_dtype == MI355Q_BF16) ((uint16_t*)y)[o] = f32_to_bf16_rne(v);
+        else ((uint16_t*)y)[o] = f32_to_f16_rne(v);
+    }
+}
+
+bool gemm_stream_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
+    if (x_dtype != MI355Q_BF16 || m < 1 || m > kStreamMaxRows) return false;
+    if (w.layout != MI355Q_LAYOUT_PLANES || !w.sz || !w.codes) return false;
+    if (w.bits != 4 || (w.group != 64 && w.group != 128)) return false;
+    if (w.k % 64 || w.k < 64 || x_stride % 8) return false;
+    if ((uintptr_t)w.codes % 16 || w.code_stride % 4) return false;
+    return true;
+}
+
+StreamLaunchShape gemm_stream_shape(const mi355q_context* ctx, uint32_t m, uint32_t n, uint32_t k) {
+    StreamLaunchShape g{};
+    const uint32_t cus = (uint32_t)ctx->props.multiProcessorCount;
+    g.row_blocks = (n + kStreamRows - 1) / kStreamRows;
+    const uint32_t it_all = (k + kStreamIterK - 1) / kStreamIterK;
+    // K parts while the row blocks alone leave half the CUs idle and a part keeps four iterations
+    uint32_t parts = 1;
+    while (g.row_blocks * parts * 2 <= cus && it_all / (parts * 2) >= 4) parts *= 2;
+    g.iters_per_part = (it_all + parts - 1) / parts;
+    g.parts = (it_all + g.iters_per_part - 1) / g.iters_per_part;
+    g.m_blocks = (m + 31) / 32;
+    g.lds_bytes = 3u * 4u * g.m_blocks * 32u * 128u;       // three stages of [32 m_blocks][256] bf16
+    return g;
+}
+
+namespace {
+
+template <int GROUP, int MB, bool SB_BF16>
+mi355q_status launch_stream_mb(hipStream_t s, const StreamArgs& a, const StreamLaunchShape& g) {
+    auto kern = qgemm_stream_kernel<GROUP, MB, SB_BF16>;
+    if (g.lds_bytes > 64u * 1024u) {
+        // the attribute belongs to the function on one device: one bit per device and instantiation
+        static std::atomic<uint64_t> lds_limit_raised{0};
+        int device = 0;
+        MI355Q_HIP(hipGetDevice(&device));
+        const uint64_t bit = 1ull << (device & 63);
+        if (!(lds_limit_raised.load(std::memory_order_relaxed) & bit)) {
+            MI355Q_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)g.lds_bytes));
+            lds_limit_raised.fetch_or(bit, std::memory_order_relaxed);
+        }
+    }
+    kern<<<dim3(g.row_blocks, g.parts), dim3(kStreamThreads), g.lds_bytes, s>>>(a);
+    MI355Q_HIP(hipGetLastError());
+    return MI355Q_OK;
+}
+
+template <int GROUP, bool SB_BF16>
+mi355q_status launch_stream_group(hipStream_t s, const StreamArgs& a, const StreamLaunchShape& g) {
+    switch (g.m_blocks) {
+    case 1: return launch_stream_mb<GROUP, 1, SB_BF16>(s, a, g);
+    case 2: return launch_stream_mb<GROUP, 2, SB_BF16>(s, a, g);
+    case 3: return launch_stream_mb<GROUP, 3, SB_BF16>(s, a, g);
+    default: break;
+    }
+    return fail(MI355Q_ERR_SHAPE, "the streamed-weight kernel takes at most %u rows", kStreamMaxRows);
+}
+
+}  // namespace
+
+mi355q_status launch_qgemm_stream(hipStream_t s, mi355q_context* ctx, const WView& w, const void* x, int x_dtype, void* y,
+                                  int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride) {
+    if (!gemm_stream_eligible(w, x_dtype, m, x_stride))
+        return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the streamed-weight kernel does not take this weight or these activations");
+    if ((uintptr_t)x % 16) return fail(MI355Q_ERR_INVALID_ARGUMENT, "activation pointer must be 16-byte aligned");
+    const StreamLaunchShape g = gemm_stream_shape(ctx, m, w.n, w.k);
+    StreamArgs a{};
+    a.codes = w.codes; a.sz = w.sz; a.x = (const uint16_t*)x; a.y = y;
+    a.m = m; a.n = w.n; a.k = w.k; a.xs = x_stride; a.ys = y_stride;
+    a.code_stride = w.code_stride; a.sz_stride = w.sz_stride;
+    a.y_dtype = (uint32_t)y_dtype;
+    a.iters_per_part = g.iters_per_part;
+    if (g.parts > 1) {
+        if (mi355q_status st = ensure_workspace(ctx, (size_t)g.parts * m * w.n * sizeof(float))) return st;
+        a.partial = (float*)ctx->workspace;
+    }
+    const bool bf = w.sb_dtype == MI355Q_BF16;
+    const mi355q_status st = w.group == 64 ? (bf ? launch_stream_group<64, true>(s, a, g) : launch_stream_group<64, false>(s, a, g))
+                                           : (bf ? launch_stream_group<128, true>(s, a, g) : launch_stream_group<128, false>(s, a, g));
+    if (st != MI355Q_OK || g.parts == 1) return st;
+    const size_t total = (size_t)m * w.n;
+    size_t blocks = (total + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    stream_sum_parts_kernel<<<dim3((unsigned)blocks), dim3(256), 0, s>>>(a.partial, y, m, w.n, y_stride, g.parts, (uint32_t)y_dtype);
+    MI355Q_HIP(hipGetLastError());
+    return MI355Q_OK;
+}
+
+}  // namespace mi355q

@@ -259,6 +259,23 @@ mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w, uint32_t maximum
     fill_common(w, m, s);
     s->path = MI355Q_PATH_PREFILL_PROJECTION;
     s->input_row_stride = input_row_stride;
+    if (!(flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA)) &&
+        !split_rows_chosen(v, x_dtype, m, input_row_stride, flags) &&
+        ((flags & MI355Q_FLAG_FORCE_STREAM) ? gemm_stream_eligible(v, x_dtype, m, input_row_stride)
+                                            : gemm_stream_chosen(v, x_dtype, m, input_row_stride))) {
+        // weights streamed through registers into the matrix cores: the direct quantized GEMM at a few dozen rows
+        std::snprintf(s->kernel_name, sizeof s->kernel_name, "%s", w->fmt.gemm_kernel_name_f32s);
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "qgemm_stream_q%u_g%u", (unsigned)w->fmt.bits,
+                      w->fmt.group_size);
+        std::snprintf(s->kernel_family, sizeof s->kernel_family, "mfmaGEMM");
+        const StreamLaunchShape g = gemm_stream_shape(w->ctx, m, (uint32_t)w->n, (uint32_t)w->k);
+        s->block[0] = 768;
+        s->grid[0] = g.row_blocks;
+        s->grid[1] = g.parts;
+        s->lds_bytes = g.lds_bytes;
+        s->rows_per_workgroup = 64;
+        return MI355Q_OK;
+    }
     if (!want_small && mfma_ok) {
         // fused dequant + matrix-core contraction: the stand-in for dequant_q*_bf16 + gemm_bf16_f32s
         std::snprintf(s->kernel_name, sizeof s->kernel_name, "%s", w->fmt.gemm_kernel_name_f32s);

@@ -216,7 +216,7 @@ def test_mfma_gemm_ragged_shapes(pkg, ctx):
 def test_qgemm_selects_matrix_cores_above_eight_rows(pkg, ctx):
     """Without flags, M > 8 goes to the matrix-core kernel when the weight is eligible and to the
     per-row kernel otherwise; both agree within the tolerance, and the plan record names the choice."""
-    m, n, k = 64, 256, 512
+    m, n, k = 200, 256, 512
     got_auto, _ = _seeded_gemm(pkg, ctx, 920, m, n, k, 4, 64, flags=0)
     got_mfma, _ = _seeded_gemm(pkg, ctx, 920, m, n, k, 4, 64)
     assert np.array_equal(got_auto, got_mfma)
@@ -224,8 +224,9 @@ def test_qgemm_selects_matrix_cores_above_eight_rows(pkg, ctx):
     fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
     w = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, pkg.LAYOUT_PLANES)
     step = w.plan_prefill_steps(m)[0]
-    assert step.kernel_family == "mfmaGEMM" and not step.used_fallback
+    assert step.kernel_family == "mfmaGEMM" and not step.used_fallback and step.device_kernel == "qgemm_mfma_q4_g64"
     assert step.block[0] in (256, 512) and step.grid[0] >= 1
+    m = 64
     ws = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, pkg.LAYOUT_STAF_BLOCKS)
     step = ws.plan_prefill_steps(m, flags=pkg.FLAG_FORCE_SMALL_M)[0]       # unforced, the two-dispatch route serves it
     assert step.kernel_family != "mfmaGEMM"

@@ -1,0 +1,118 @@
+"""Streamed-weight matrix-core kernel (gemm_stream.hip): 17 to 96 bf16 activation rows on 4-bit planes, the weights
+dequantised in registers straight into the matrix cores' operand, the activations alone staged through LDS.
+
+The kernel rounds every weight to bf16 exactly as the tiled prefill kernel does
+(Sources/MetalCompiler/Generator/MetalSourceGenerator+Quantized.swift:361-416 writes bf16 weights for gemm_bf16_f32s), so
+its results equal the tiled kernel's up to the order of the fp32 sums; both are checked against the fp64 oracle."""
+import numpy as np
+import pytest
+
+import kat
+import oracle
+import sys
+
+from gpu_util import act_rounded, act_to_device_array, out_from_device, rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def _case(seed, n, k, group, sb):
+    w = kat.seeded_weights(seed, n, k)
+    words, s, z = oracle.quantize_affine(w, 4, group, sb)
+    return words, s, z, oracle.dequant_planes_f32(4, group, n, k, words, s, z, sb)
+
+
+def _run(ctx, pkg, w, x, m, n, y_dtype, flags, ypad=0, xpad=0):
+    k = x.shape[1]
+    xh = np.zeros((m, k + xpad), dtype=np.float32)
+    xh[:, :k] = x
+    xd = ctx.upload(act_to_device_array(xh, pkg.BF16, pkg))
+    ysz = 4 if y_dtype == pkg.F32 else 2
+    if (m * (n + ypad) * ysz) % 4:
+        ypad += 1
+    yd = ctx.alloc(m * (n + ypad) * ysz)
+    ctx.fill(yd, 0x7FC07FC0 if ysz == 2 else 0x7FC00000)
+    ctx.qgemm(w, xd, pkg.BF16, yd, y_dtype, m, k + xpad, n + ypad, flags)
+    ctx.synchronize()
+    got = out_from_device(yd, y_dtype, (m, n + ypad), pkg)
+    xd.free(); yd.free()
+    assert np.isnan(got[:, n:]).all(), "output padding overwritten"
+    return got[:, :n]
+
+
+@pytest.mark.parametrize("group,sb", [(64, "bf16"), (64, "f16"), (128, "bf16"), (128, "f16")])
+def test_stream_kernel_against_oracle_and_tiled_kernel(pkg, ctx, group, sb):
+    """Row counts across the three block counts, N off the 64-row workgroups and the 32-row blocks, K with and
+    without whole 256-column iterations and split into parts (few rows, long K), padded strides."""
+    sbo, sbp = (oracle.BF16, pkg.BF16) if sb == "bf16" else (oracle.F16, pkg.F16)
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, group)
+    shapes = [(17, 64, 128), (32, 1000, 320), (33, 130, 2112), (64, 4096, 1024), (65, 31, 4096), (96, 200, 8192 + 128),
+              (90, 257, 256), (48, 64, 14336)]
+    for i, (m, n, k) in enumerate(shapes):
+        k += 64 if k % group else 0                      # 320 and 2112 columns: whole groups of 128 take 64 more
+        say(f"stream q4 g{group} {sb} M={m} {k}->{n}")
+        words, s, z, wq = _case(1300 + i, n, k, group, sbo)
+        w = ctx.weight_prepare_mlx(fmt, words, s, z, sbp, pkg.LAYOUT_PLANES)
+        x = act_rounded(kat.seeded_activations(1400 + i, m, k), pkg.BF16, pkg)
+        want = oracle.gemm_f64(wq, x)
+        got = _run(ctx, pkg, w, x, m, n, pkg.F32, pkg.FLAG_FORCE_STREAM, ypad=i % 3, xpad=8 * (i % 2))
+        tiled = _run(ctx, pkg, w, x, m, n, pkg.F32, pkg.FLAG_FORCE_MFMA)
+        # bf16-rounded weights: 2^-9 relative per weight, 1.5e-3 in the L2 norm at most
+        assert rel_l2(got, want) < 2.5e-3, (m, n, k, rel_l2(got, want))
+        # the same rounded weights as the tiled kernel: only the order of the fp32 sums differs
+        assert rel_l2(got, tiled) < 2e-6, (m, n, k, rel_l2(got, tiled))
+        auto = _run(ctx, pkg, w, x, m, n, pkg.F32, 0)
+        assert np.array_equal(auto, got), "rows 17 to 96 on eligible planes take the streamed-weight kernel unforced"
+        step = w.plan_prefill_steps(m)[0]
+        assert step.device_kernel == f"qgemm_stream_q4_g{group}" and step.kernel_family == "mfmaGEMM"
+        assert not step.used_fallback and step.block[0] == 768
+        for y_dtype in (pkg.BF16, pkg.F16):
+            low = _run(ctx, pkg, w, x, m, n, y_dtype, pkg.FLAG_FORCE_STREAM, ypad=1)
+            ref = act_rounded(got, y_dtype, pkg)
+            assert np.array_equal(low, ref), "16-bit outputs are the fp32 results rounded once"
+        w.destroy()
+
+
+def test_stream_kernel_exact_on_integer_weights(pkg, ctx):
+    """Weights and activations that bf16 holds exactly and sums that fp32 holds exactly: the result is the integer
+    sum, whatever the order -- a dropped K-tile, a swapped word or a wrong row would show as a whole number off."""
+    rng = np.random.default_rng(31)
+    m, n, k = 70, 192, 1280
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+    q = rng.integers(0, 16, size=(n, k)).astype(np.uint32)
+    scales = np.ones((n, k // 64), dtype=np.float32) * 2.0
+    biases = -rng.integers(0, 8, size=(n, k // 64)).astype(np.float32)
+    words = (q.reshape(n, k // 8, 8) << (4 * np.arange(8, dtype=np.uint32))).sum(axis=2).astype(np.uint32)
+    w = ctx.weight_prepare_mlx(fmt, words, oracle.bf16_from_f32(scales), oracle.bf16_from_f32(biases), pkg.BF16,
+                               pkg.LAYOUT_PLANES)
+    x = rng.integers(-3, 4, size=(m, k)).astype(np.float32)
+    wq = 2.0 * q.astype(np.float64) + np.repeat(biases.astype(np.float64), 64, axis=1)
+    want = x.astype(np.float64) @ wq.T
+    got = _run(ctx, pkg, w, x, m, n, pkg.F32, pkg.FLAG_FORCE_STREAM)
+    assert np.array_equal(got.astype(np.float64), want)
+    w.destroy()
+
+
+def test_stream_kernel_refuses_what_it_does_not_read(pkg, ctx):
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+    words, s, z, _ = _case(1500, 64, 128, 64, oracle.BF16)
+    w = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, pkg.LAYOUT_PLANES)
+    x = act_rounded(kat.seeded_activations(1, 97, 128), pkg.BF16, pkg)
+    with pytest.raises(pkg.MI355QError):
+        _run(ctx, pkg, w, x, 97, 64, pkg.F32, pkg.FLAG_FORCE_STREAM)           # more than 96 rows
+    with pytest.raises(pkg.MI355QError):
+        _run(ctx, pkg, w, x[:20], 20, 64, pkg.F32, pkg.FLAG_FORCE_STREAM | pkg.FLAG_FORCE_MFMA)
+    ws = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, pkg.LAYOUT_STAF_BLOCKS)
+    with pytest.raises(pkg.MI355QError):
+        _run(ctx, pkg, ws, x[:20], 20, 64, pkg.F32, pkg.FLAG_FORCE_STREAM)     # block layout
+    fmt8 = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(8, 64)
+    words8, s8, z8 = oracle.quantize_affine(kat.seeded_weights(1501, 64, 128), 8, 64, oracle.BF16)
+    w8 = ctx.weight_prepare_mlx(fmt8, words8, s8, z8, pkg.BF16, pkg.LAYOUT_PLANES)
+    with pytest.raises(pkg.MI355QError):
+        _run(ctx, pkg, w8, x[:20], 20, 64, pkg.F32, pkg.FLAG_FORCE_STREAM)     # 8-bit codes
+    for t in (w, ws, w8):
+        t.destroy()
