@@ -313,7 +313,7 @@ def main():
         log(f"  {label:8s}: {ms * 1e3:.2f} us/launch, {per_shape[label]['GBps']} GB/s; single launches "
             f"{per_shape[label]['single_launch_us']}")
         p1.destroy()
-    # ---- secondary: the same layer step at M = 1, 2, 4, 8 activation rows (benchmark config 1), on
+    # ---- secondary: the same layer step at M = 1 to 64 activation rows (benchmark config 1), on
     # the split-plane layout and on the matrix-core tile layout (4-launch schedule, stream replay)
     batch_sweep = None
     if not a.no_batch_sweep:
@@ -324,7 +324,9 @@ def main():
                 pool = [{name: ctx.weight_prepare_mlx(fmt, *host[name], pkg.BF16, layout) for name, _, _ in LAYER_SHAPES}
                         for _ in range(n_t16)]
             batch_sweep[lname] = {}
-            for m in (1, 2, 4, 8, 16):                      # both layouts take up to 16 rows a launch
+            # both layouts take up to 16 rows a launch of the decode kernels; 32 and 64 rows on the planes run on the
+            # streamed-weight matrix-core kernel, on the records on the tiled prefill kernel
+            for m in (1, 2, 4, 8, 16, 32, 64):
                 xm = {k: ctx.upload(oracle.bf16_from_f32(kat.seeded_activations(900 + m, m, k))) for k in (4096, 14336)}   # N(0,1)
                 ym = {name: ctx.alloc(m * n * 2) for name, n, _ in LAYER_SHAPES}
                 pl = pkg.DispatchPlan(ctx)

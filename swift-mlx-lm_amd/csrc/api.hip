@@ -395,6 +395,14 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
         }
         return MI355Q_OK;
     }
+    // a few dozen rows on 4-bit planes: the streamed-weight kernel, one launch for the two or three matrices
+    if (!(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_TWO_STEP | MI355Q_FLAG_FORCE_SMALL_M)) &&
+        (uintptr_t)x % 16 == 0 && gemm_stream_multi_eligible(count, views, x_dtype, m, xs)) {
+        bool chosen = true;
+        for (uint32_t i = 0; i < count; i++)
+            chosen = chosen && ((flags & MI355Q_FLAG_FORCE_STREAM) || gemm_stream_chosen(views[i], x_dtype, m, xs));
+        if (chosen) return launch_qgemm_stream_multi(s, ctx, count, views, x, x_dtype, ys, strides, y_dtype, m, xs);
+    }
     for (uint32_t i = 0; i < count; i++) {
         mi355q_status st = dispatch_linear(ctx, s, weights[i], x, x_dtype, ys[i], y_dtype, m, xs, 0, flags, false);
         if (st != MI355Q_OK) return st;

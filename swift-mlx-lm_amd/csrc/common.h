@@ -280,6 +280,12 @@ bool gemm_stream_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stri
 StreamLaunchShape gemm_stream_shape(const mi355q_context* ctx, uint32_t m, uint32_t n, uint32_t k);
 mi355q_status launch_qgemm_stream(hipStream_t s, mi355q_context* ctx, const WView& w, const void* x, int x_dtype, void* y,
                                   int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride);
+// Up to three matrices that share the activations, K, the group size and the scale type, as one launch.
+StreamLaunchShape gemm_stream_shape_blocks(const mi355q_context* ctx, uint32_t m, uint32_t row_blocks, uint32_t k);
+bool gemm_stream_multi_eligible(uint32_t count, const WView* w, int x_dtype, uint32_t m, uint32_t x_stride);
+mi355q_status launch_qgemm_stream_multi(hipStream_t s, mi355q_context* ctx, uint32_t count, const WView* w, const void* x,
+                                        int x_dtype, void* const* y, const uint32_t* y_strides, int y_dtype, uint32_t m,
+                                        uint32_t x_stride);
 // Two-dispatch prefill route: dequantise the whole matrix to bf16 in the context's scratch, then the platform's
 // dense GEMM.  `dense_library_serves` answers whether the library can be opened and has an algorithm for the problem.
 constexpr size_t kDenseLibraryWorkspace = (size_t)64 << 20;

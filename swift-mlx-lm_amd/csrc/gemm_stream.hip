@@ -15,8 +15,10 @@
 //     the A operand is the activations' chunk 4h + j of that K-tile, read from LDS;
 //   * per iteration four more wavefronts of the workgroup stage [32 MB rows][256 columns] of activations
 //     (XOR-swizzled 128-byte rows per K slice) two iterations ahead into the third of three LDS stages, copied
-//     global -> LDS directly; the multiplying wavefronts fetch weight words six iterations ahead and wait for nothing
+//     global -> LDS directly; the multiplying wavefronts fetch weight words three or six iterations ahead and wait for nothing
 //     else; one barrier per iteration;
+//   * two or three matrices that share the activations (q+k+v, gate+up) run as one launch, each owning whole
+//     workgroups;
 //   * the four K slices of a row block add their accumulators through LDS at the end; with K split over workgroups
 //     (few rows, long K) fp32 partial results go to scratch and a second launch adds them.
 #include "device_utils.h"
@@ -29,21 +31,29 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float st_floatx16_t
 typedef __bf16 st_bf16x2_v __attribute__((ext_vector_type(2)));
 typedef float st_float2_v __attribute__((ext_vector_type(2)));
 
+constexpr int kStreamMaxSegments = 3;
+
 struct StreamArgs {
-    const uint32_t* codes;     // [N][code_stride] words, eight codes a word
-    const uint32_t* sz;        // [N][sz_stride] words: scale | bias << 16 per group
+    // up to three matrices that share the activations, K, the group size and the scale type (q+k+v, gate+up): matrix i
+    // owns the workgroups [wg_end[i-1], wg_end[i]) and the columns [col0[i], col0[i] + n[i]) of the fp32 partial results
+    const uint32_t* codes[kStreamMaxSegments];     // [N][code_stride] words, eight codes a word
+    const uint32_t* sz[kStreamMaxSegments];        // [N][sz_stride] words: scale | bias << 16 per group
+    void* y[kStreamMaxSegments];
+    uint32_t n[kStreamMaxSegments], ys[kStreamMaxSegments];
+    uint32_t code_stride[kStreamMaxSegments], sz_stride[kStreamMaxSegments];
+    uint32_t wg_end[kStreamMaxSegments], col0[kStreamMaxSegments];
     const uint16_t* x;         // bf16 [M][xs]
-    void* y;
-    float* partial;            // K split over workgroups: fp32 [parts][M][N]; else null
-    uint32_t m, n, k, xs, ys;
-    uint32_t code_stride, sz_stride;
+    float* partial;            // K split over workgroups: fp32 [parts][M][n_total]; else null
+    uint32_t m, k, xs, n_total;
     uint32_t y_dtype;
     uint32_t iters_per_part;   // iterations (256 columns each) per K part; blockIdx.y is the part
 };
 
 constexpr int kStreamIterK = 256;      // columns of K per iteration: one 64-code K-tile per K slice
 constexpr int kStreamRows = 64;        // weight rows per workgroup
-constexpr int kStreamAhead = 6;        // iterations the weight words are fetched ahead (and the loop's unroll)
+// iterations the weight words are fetched ahead (and the loop's unroll; a multiple of the three LDS stages): measured,
+// 4096 -> 14336 at 32 rows 16.6 us with three against 17.1 with six and 19.7 with twelve, at 64 rows 22.0 / 21.1 / 26.2
+constexpr int stream_ahead(int m_blocks) { return m_blocks == 1 ? 3 : 6; }
 constexpr int kStreamThreads = 768;    // eight multiplying wavefronts and four that stage the activations
 
 __device__ __forceinline__ uint32_t st_pack_bf16(float lo, float hi) {
@@ -63,7 +73,7 @@ __global__ __launch_bounds__(kStreamThreads) void qgemm_stream_kernel(StreamArgs
     constexpr int SLICE_BYTES = MPAD * 128;               // one K slice of a stage: [MPAD][64] bf16
     constexpr int STAGE = 4 * SLICE_BYTES;
     constexpr int XP = 4 * MB;                            // copy instructions (eight rows of a K slice each) per stage
-    constexpr int U = kStreamAhead;
+    constexpr int U = stream_ahead(MB);
     extern __shared__ u32x4 smem_st[];
     char* const lds = (char*)smem_st;
 
@@ -72,7 +82,9 @@ __global__ __launch_bounds__(kStreamThreads) void qgemm_stream_kernel(StreamArgs
     const bool stager = wave >= 8;                        // wavefronts 8..11 move the activations, 0..7 multiply
     const uint32_t rb = (wave >> 2) & 1u, slice = wave & 3u;     // row block, K slice
     const uint32_t ln = lane & 31, lh = lane >> 5;
-    const uint32_t n0 = blockIdx.x * kStreamRows + rb * 32;
+    const bool in1 = blockIdx.x >= a.wg_end[0], in2 = blockIdx.x >= a.wg_end[1];      // the matrix of this workgroup
+    const uint32_t seg_n = in2 ? a.n[2] : in1 ? a.n[1] : a.n[0];
+    const uint32_t n0 = (blockIdx.x - (in2 ? a.wg_end[1] : in1 ? a.wg_end[0] : 0u)) * kStreamRows + rb * 32;
 
     const uint32_t KT = a.k / 64;                         // K-tiles
     const uint32_t it_all = (a.k + kStreamIterK - 1) / kStreamIterK;
@@ -136,9 +148,11 @@ __global__ __launch_bounds__(kStreamThreads) void qgemm_stream_kernel(StreamArgs
         }
     } else {
         uint32_t wrow = n0 + ln;
-        wrow = wrow < a.n ? wrow : a.n - 1;               // rows past the end re-read the last one
-        const uint32_t* const crow = a.codes + (size_t)wrow * a.code_stride + 4 * lh;
-        const uint32_t* const szrow = a.sz + (size_t)wrow * a.sz_stride;
+        wrow = wrow < seg_n ? wrow : seg_n - 1;           // rows past the end re-read the last one
+        const uint32_t* const crow = (in2 ? a.codes[2] : in1 ? a.codes[1] : a.codes[0]) +
+                                     (size_t)wrow * (in2 ? a.code_stride[2] : in1 ? a.code_stride[1] : a.code_stride[0]) + 4 * lh;
+        const uint32_t* const szrow = (in2 ? a.sz[2] : in1 ? a.sz[1] : a.sz[0]) +
+                                      (size_t)wrow * (in2 ? a.sz_stride[2] : in1 ? a.sz_stride[1] : a.sz_stride[0]);
         // weight words and (scale, bias) word of this wavefront's K-tile of iteration `it`
         u32x4 ring[U];
         uint32_t szring[U];
@@ -221,7 +235,10 @@ __global__ __launch_bounds__(kStreamThreads) void qgemm_stream_kernel(StreamArgs
             for (int r = 0; r < 16; r++) acc[b][r] += other[(b * 16 + r) * 64 + lane];
     }
     const uint32_t col = n0 + ln;
-    if (col >= a.n) return;
+    if (col >= seg_n) return;
+    void* const seg_y = in2 ? a.y[2] : in1 ? a.y[1] : a.y[0];
+    const uint32_t seg_ys = in2 ? a.ys[2] : in1 ? a.ys[1] : a.ys[0];
+    const uint32_t pcol = (in2 ? a.col0[2] : in1 ? a.col0[1] : a.col0[0]) + col;
 #pragma unroll
     for (int b = 0; b < MB; b++)
 #pragma unroll
@@ -230,28 +247,29 @@ __global__ __launch_bounds__(kStreamThreads) void qgemm_stream_kernel(StreamArgs
             if (row >= a.m) continue;
             const float v = acc[b][r];
             if (a.partial) {
-                a.partial[((size_t)blockIdx.y * a.m + row) * a.n + col] = v;
+                a.partial[((size_t)blockIdx.y * a.m + row) * a.n_total + pcol] = v;
                 continue;
             }
-            const size_t o = (size_t)row * a.ys + col;
-            if (a.y_dtype == MI355Q_F32) ((float*)a.y)[o] = v;
-            else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)a.y)[o] = f32_to_bf16_rne(v);
-            else ((uint16_t*)a.y)[o] = f32_to_f16_rne(v);
+            const size_t o = (size_t)row * seg_ys + col;
+            if (a.y_dtype == MI355Q_F32) ((float*)seg_y)[o] = v;
+            else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)seg_y)[o] = f32_to_bf16_rne(v);
+            else ((uint16_t*)seg_y)[o] = f32_to_f16_rne(v);
         }
 }
 
-// y = the sum of the K parts' fp32 partial results, part 0 first, rounded once to the output type
-__global__ __launch_bounds__(256) void stream_sum_parts_kernel(const float* __restrict__ partial, void* __restrict__ y,
-                                                               uint32_t m, uint32_t n, uint32_t ys, uint32_t parts,
-                                                               uint32_t y_dtype) {
-    const size_t total = (size_t)m * n;
+// y_i = the sum of the K parts' fp32 partial results over matrix i's columns, part 0 first, rounded once to the output type
+__global__ __launch_bounds__(256) void stream_sum_parts_kernel(StreamArgs a, uint32_t parts) {
+    const size_t total = (size_t)a.m * a.n_total;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
         float v = 0.f;
-        for (uint32_t p = 0; p < parts; p++) v += partial[(size_t)p * total + i];
-        const size_t row = i / n, col = i - row * n;
-        const size_t o = row * ys + col;
-        if (y_dtype == MI355Q_F32) ((float*)y)[o] = v;
-        else if (y_dtype == MI355Q_BF16) ((uint16_t*)y)[o] = f32_to_bf16_rne(v);
+        for (uint32_t p = 0; p < parts; p++) v += a.partial[(size_t)p * total + i];
+        const size_t row = i / a.n_total;
+        const uint32_t pcol = (uint32_t)(i - row * a.n_total);
+        const bool in1 = pcol >= a.col0[1], in2 = pcol >= a.col0[2];
+        void* const y = in2 ? a.y[2] : in1 ? a.y[1] : a.y[0];
+        const size_t o = row * (in2 ? a.ys[2] : in1 ? a.ys[1] : a.ys[0]) + (pcol - (in2 ? a.col0[2] : in1 ? a.col0[1] : 0u));
+        if (a.y_dtype == MI355Q_F32) ((float*)y)[o] = v;
+        else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)y)[o] = f32_to_bf16_rne(v);
         else ((uint16_t*)y)[o] = f32_to_f16_rne(v);
     }
 }
@@ -266,9 +284,13 @@ bool gemm_stream_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_st
 }
 
 StreamLaunchShape gemm_stream_shape(const mi355q_context* ctx, uint32_t m, uint32_t n, uint32_t k) {
+    return gemm_stream_shape_blocks(ctx, m, (n + kStreamRows - 1) / kStreamRows, k);
+}
+
+StreamLaunchShape gemm_stream_shape_blocks(const mi355q_context* ctx, uint32_t m, uint32_t row_blocks, uint32_t k) {
     StreamLaunchShape g{};
     const uint32_t cus = (uint32_t)ctx->props.multiProcessorCount;
-    g.row_blocks = (n + kStreamRows - 1) / kStreamRows;
+    g.row_blocks = row_blocks;
     const uint32_t it_all = (k + kStreamIterK - 1) / kStreamIterK;
     // K parts while the row blocks alone leave half the CUs idle and a part keeps four iterations
     uint32_t parts = 1;
@@ -316,28 +338,60 @@ mi355q_status launch_stream_group(hipStream_t s, const StreamArgs& a, const Stre
 
 mi355q_status launch_qgemm_stream(hipStream_t s, mi355q_context* ctx, const WView& w, const void* x, int x_dtype, void* y,
                                   int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride) {
-    if (!gemm_stream_eligible(w, x_dtype, m, x_stride))
-        return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the streamed-weight kernel does not take this weight or these activations");
+    void* ys[1] = {y};
+    const uint32_t strides[1] = {y_stride};
+    return launch_qgemm_stream_multi(s, ctx, 1, &w, x, x_dtype, ys, strides, y_dtype, m, x_stride);
+}
+
+bool gemm_stream_multi_eligible(uint32_t count, const WView* w, int x_dtype, uint32_t m, uint32_t x_stride) {
+    if (count < 1 || count > (uint32_t)kStreamMaxSegments) return false;
+    for (uint32_t i = 0; i < count; i++)
+        if (!gemm_stream_eligible(w[i], x_dtype, m, x_stride) || w[i].k != w[0].k || w[i].group != w[0].group ||
+            w[i].sb_dtype != w[0].sb_dtype)
+            return false;
+    return true;
+}
+
+mi355q_status launch_qgemm_stream_multi(hipStream_t s, mi355q_context* ctx, uint32_t count, const WView* w, const void* x,
+                                        int x_dtype, void* const* y, const uint32_t* y_strides, int y_dtype, uint32_t m,
+                                        uint32_t x_stride) {
+    if (!gemm_stream_multi_eligible(count, w, x_dtype, m, x_stride))
+        return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the streamed-weight kernel does not take these weights or activations");
     if ((uintptr_t)x % 16) return fail(MI355Q_ERR_INVALID_ARGUMENT, "activation pointer must be 16-byte aligned");
-    const StreamLaunchShape g = gemm_stream_shape(ctx, m, w.n, w.k);
     StreamArgs a{};
-    a.codes = w.codes; a.sz = w.sz; a.x = (const uint16_t*)x; a.y = y;
-    a.m = m; a.n = w.n; a.k = w.k; a.xs = x_stride; a.ys = y_stride;
-    a.code_stride = w.code_stride; a.sz_stride = w.sz_stride;
+    uint32_t blocks = 0, cols = 0;
+    for (uint32_t i = 0; i < (uint32_t)kStreamMaxSegments; i++) {
+        const uint32_t j = i < count ? i : count - 1;          // unused entries repeat the last matrix and own nothing
+        a.codes[i] = w[j].codes; a.sz[i] = w[j].sz; a.y[i] = y[j];
+        a.n[i] = w[j].n; a.ys[i] = y_strides[j];
+        a.code_stride[i] = w[j].code_stride; a.sz_stride[i] = w[j].sz_stride;
+        if (i < count) {
+            a.col0[i] = cols;
+            blocks += (w[i].n + kStreamRows - 1) / kStreamRows;
+            cols += w[i].n;
+            a.wg_end[i] = blocks;
+        } else {
+            a.col0[i] = 0xFFFFFFFFu;                           // no column and no workgroup reaches an unused entry
+            a.wg_end[i] = 0xFFFFFFFFu;
+        }
+    }
+    a.x = (const uint16_t*)x;
+    a.m = m; a.k = w[0].k; a.xs = x_stride; a.n_total = cols;
     a.y_dtype = (uint32_t)y_dtype;
+    const StreamLaunchShape g = gemm_stream_shape_blocks(ctx, m, blocks, w[0].k);
     a.iters_per_part = g.iters_per_part;
     if (g.parts > 1) {
-        if (mi355q_status st = ensure_workspace(ctx, (size_t)g.parts * m * w.n * sizeof(float))) return st;
+        if (mi355q_status st = ensure_workspace(ctx, (size_t)g.parts * m * cols * sizeof(float))) return st;
         a.partial = (float*)ctx->workspace;
     }
-    const bool bf = w.sb_dtype == MI355Q_BF16;
-    const mi355q_status st = w.group == 64 ? (bf ? launch_stream_group<64, true>(s, a, g) : launch_stream_group<64, false>(s, a, g))
-                                           : (bf ? launch_stream_group<128, true>(s, a, g) : launch_stream_group<128, false>(s, a, g));
+    const bool bf = w[0].sb_dtype == MI355Q_BF16;
+    const mi355q_status st = w[0].group == 64 ? (bf ? launch_stream_group<64, true>(s, a, g) : launch_stream_group<64, false>(s, a, g))
+                                              : (bf ? launch_stream_group<128, true>(s, a, g) : launch_stream_group<128, false>(s, a, g));
     if (st != MI355Q_OK || g.parts == 1) return st;
-    const size_t total = (size_t)m * w.n;
-    size_t blocks = (total + 255) / 256;
-    if (blocks > 4096) blocks = 4096;
-    stream_sum_parts_kernel<<<dim3((unsigned)blocks), dim3(256), 0, s>>>(a.partial, y, m, w.n, y_stride, g.parts, (uint32_t)y_dtype);
+    const size_t total = (size_t)m * cols;
+    size_t sum_blocks = (total + 255) / 256;
+    if (sum_blocks > 4096) sum_blocks = 4096;
+    stream_sum_parts_kernel<<<dim3((unsigned)sum_blocks), dim3(256), 0, s>>>(a, g.parts);
     MI355Q_HIP(hipGetLastError());
     return MI355Q_OK;
 }

@@ -116,3 +116,35 @@ def test_stream_kernel_refuses_what_it_does_not_read(pkg, ctx):
         _run(ctx, pkg, w8, x[:20], 20, 64, pkg.F32, pkg.FLAG_FORCE_STREAM)     # 8-bit codes
     for t in (w, ws, w8):
         t.destroy()
+
+
+@pytest.mark.parametrize("count,m", [(2, 40), (3, 24), (3, 96), (2, 70)])
+def test_stream_kernel_shared_launch_equals_separate_launches(pkg, ctx, count, m):
+    """Two or three matrices that share the activations (gate+up, q+k+v) as one launch of the streamed-weight kernel:
+    every output has the bits of its own launch; row counts off the 64-row workgroups, one and several K parts."""
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+    k = 1024 if count == 2 else 4096
+    ns = [300, 64, 130][:count] if count == 3 else [2048 + 40, 1000]
+    ws, wqs = [], []
+    for i, n in enumerate(ns):
+        words, s, z, wq = _case(1600 + 10 * count + i, n, k, 64, oracle.BF16)
+        ws.append(ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, pkg.LAYOUT_PLANES))
+        wqs.append(wq)
+    x = act_rounded(kat.seeded_activations(1700 + count, m, k), pkg.BF16, pkg)
+    xd = ctx.upload(act_to_device_array(x, pkg.BF16, pkg))
+    for y_dtype in (pkg.F32, pkg.BF16):
+        ysz = 4 if y_dtype == pkg.F32 else 2
+        say(f"shared launch of {count} M={m} K={k} N={ns} y {y_dtype}")
+        dense = [ctx.alloc(m * n * ysz) for n in ns]               # batched outputs are dense: row stride N_i
+        ctx.batched_qgemm(ws, xd, pkg.BF16, dense, y_dtype, m, 0, 0)
+        ctx.synchronize()
+        for w, wq, n, yd in zip(ws, wqs, ns, dense):
+            got = out_from_device(yd, y_dtype, (m, n), pkg)
+            alone = _run(ctx, pkg, w, x, m, n, y_dtype, pkg.FLAG_FORCE_STREAM)
+            assert np.array_equal(got, alone), (count, m, n)
+            assert rel_l2(got, oracle.gemm_f64(wq, x)) < (2.5e-3 if y_dtype == pkg.F32 else 5e-3)
+        for b in dense:
+            b.free()
+    xd.free()
+    for w in ws:
+        w.destroy()
