@@ -113,7 +113,8 @@ def main():
     ap.add_argument("--no-prefill", action="store_true", help="skip the secondary prefill-GEMM figure")
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip the secondary per-launch figures of benchmark configs 0, 2 and 4")
-    ap.add_argument("--no-batch-sweep", action="store_true", help="skip the secondary M = 1, 2, 4, 8 figures")
+    ap.add_argument("--no-batch-sweep", action="store_true", help="skip the secondary M = 1 to 64 figures")
+    ap.add_argument("--no-f16-step", action="store_true", help="skip the layer step with f16 activations")
     ap.add_argument("--all-formats", action="store_true",
                     help="add 4096->14336 at M = 1 and 8 for every registered format, planes and blocks in place (half a minute)")
     a = ap.parse_args()
@@ -254,19 +255,21 @@ def main():
             f"{layer_bytes / (ms_pass / a.layers * 1e-3) / 1e9:.1f} GB/s; spread {spreads[label + ' hip-graph']}")
         plan.destroy()
     # the reference decodes in f16: the same 4-launch step with f16 activations and outputs, graph replay
-    x16dev = {k: ctx.upload(v.astype(np.float16).view(np.uint16)) for k, v in xs.items()}
-    plan16 = build_plan(True, x16dev, pkg.F16)
-    f16_kernel = plan16.step(2)[0].device_kernel
-    plan16.graph_build(stream)
-    for _ in range(2):
-        plan16.graph_launch(stream)
-    ctx.synchronize(stream)
-    ms16 = time_region(ctx, lambda i: plan16.graph_launch(stream), max(1, steps // a.layers), stream) / a.layers
-    ctx.synchronize(stream)
-    plan16.destroy()
-    f16_step = {"us_per_step": round(ms16 * 1e3, 2), "GBps": round(layer_bytes / (ms16 * 1e-3) / 1e9, 1),
-                "gate_up_kernel": f16_kernel, "vs_bf16": round(ms16 / results["4-launch hip-graph"], 3)}
-    log(f"4-launch graph replay with f16 activations: {f16_step}")
+    f16_step = None
+    if not a.no_f16_step:
+        x16dev = {k: ctx.upload(v.astype(np.float16).view(np.uint16)) for k, v in xs.items()}
+        plan16 = build_plan(True, x16dev, pkg.F16)
+        f16_kernel = plan16.step(2)[0].device_kernel
+        plan16.graph_build(stream)
+        for _ in range(2):
+            plan16.graph_launch(stream)
+        ctx.synchronize(stream)
+        ms16 = time_region(ctx, lambda i: plan16.graph_launch(stream), max(1, steps // a.layers), stream) / a.layers
+        ctx.synchronize(stream)
+        plan16.destroy()
+        f16_step = {"us_per_step": round(ms16 * 1e3, 2), "GBps": round(layer_bytes / (ms16 * 1e-3) / 1e9, 1),
+                    "gate_up_kernel": f16_kernel, "vs_bf16": round(ms16 / results["4-launch hip-graph"], 3)}
+        log(f"4-launch graph replay with f16 activations: {f16_step}")
     mode = min(results, key=results.get)
     ms_step = results[mode]
     value = layer_bytes / (ms_step * 1e-3) / 1e9

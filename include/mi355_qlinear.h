@@ -272,12 +272,15 @@ MI355Q_API mi355q_status mi355q_qgemv(mi355q_context* ctx, void* stream, const m
 /* Prefill projection: gemm_q4_g64_f32s / gemm_q8_g32_f32s (:22-156) and the two-step
  * dequant_q*_bf16 + gemm_bf16_f32s path (:361-416, MC/Generator/MetalSourceGenerator+Linear.swift:18-81).
  * Any M >= 1; M is a run-time value (the reference rebinds sequenceLength per call,
- * MC/Compiler/MetalPrefillStepBuilder.swift:728-732).  Three routes, all with fp32 accumulation, chosen by
+ * MC/Compiler/MetalPrefillStepBuilder.swift:728-732).  Four routes, all with fp32 accumulation, chosen by
  * measured cost unless flags say otherwise (mi355q_plan_prefill_steps reports the choice); the first keeps
- * the dequantised weights unrounded (the decode kernels' arithmetic), the other two round them once to bf16
+ * the dequantised weights unrounded (the decode kernels' arithmetic), the others round them once to bf16
  * (the numerics of the reference's dequant -> bf16 -> GEMM route):
- *   - small M (up to 8 rows; 16 on TILE16 records and on q4 / q8 planes, and there up to 32 in two launches):
- *     the GEMV-style decode kernels;
+ *   - small M (up to 8 rows; 16 on TILE16 records and on q4 / q8 planes; up to 32 in two launches where the
+ *     next route does not read the weight): the GEMV-style decode kernels;
+ *   - 17 to 96 bf16 rows on 4-bit planes (groups of 64 or 128): the streamed-weight kernel -- weights
+ *     dequantised in registers straight into the matrix cores' operand, the activations alone staged in LDS;
+ *     through mi355q_batched_qgemm two or three matrices share one launch;
  *   - ONE fused kernel: code tiles are dequantised to bf16 in LDS and contracted on MFMA (the planes
  *     and TILE16 layouts, formats q4 g64/g128, q8 g32/g64, q6/q3/q2 g64, bf16 activations);
  *   - two dispatches, as the reference's second route: the whole matrix is dequantised to bf16 in a
