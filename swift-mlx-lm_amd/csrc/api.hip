@@ -213,6 +213,7 @@ bool gemm_two_step_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_st
     if (flags & (MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_STREAM)) return false;
     if (flags & MI355Q_FLAG_FORCE_TWO_STEP) return true;
     if (!gemm_two_step_eligible(w, x_dtype, m, x_stride)) return false;
+    if (gemm_stream_chosen(w, x_dtype, m, x_stride)) return false;      // a few dozen rows on 4- / 8-bit planes
     if (!gemm_mfma_eligible(w, x_dtype, m, x_stride)) {
         // no decode kernel reads the weight: from the second row; from the first where the per-code kernel leaves most
         // of its lanes idle (a lane per code of a group: q3 g16 blocks, 4096 -> 14336, take it 465 us at one row
@@ -383,7 +384,7 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
     bool stepped = m > step && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_TWO_STEP));
     for (uint32_t i = 0; i < count && stepped; i++)
         stepped = decode_kernel_reads(views[i], x_dtype, xs) && !split_rows_chosen(views[i], x_dtype, m, xs, flags) &&
-                  !gemm_two_step_chosen(views[i], x_dtype, m, xs, flags) &&
+                  !gemm_two_step_chosen(views[i], x_dtype, m, xs, flags) && !gemm_stream_chosen(views[i], x_dtype, m, xs) &&
                   (m <= small_batch_limit(views[i], x_dtype, xs) || !gemm_mfma_eligible(views[i], x_dtype, m, xs));
     if (stepped) {
         const size_t xsz = x_dtype == MI355Q_F32 ? 4 : 2, ysz = y_dtype == MI355Q_F32 ? 4 : 2;

@@ -30,6 +30,8 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 st_bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float st_floatx16_t;
 typedef __bf16 st_bf16x2_v __attribute__((ext_vector_type(2)));
 typedef float st_float2_v __attribute__((ext_vector_type(2)));
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 st_f16x8_t;
+typedef _Float16 st_f16x2_v __attribute__((ext_vector_type(2)));
 
 constexpr int kStreamMaxSegments = 3;
 
@@ -56,9 +58,12 @@ constexpr int kStreamRows = 64;        // weight rows per workgroup
 constexpr int stream_ahead(int m_blocks) { return m_blocks == 1 ? 3 : 6; }
 constexpr int kStreamThreads = 768;    // eight multiplying wavefronts and four that stage the activations
 
-__device__ __forceinline__ uint32_t st_pack_bf16(float lo, float hi) {
+// two fp32 values rounded (to nearest even) to the activations' 16-bit type, the first in the low half
+template <bool XF16>
+__device__ __forceinline__ uint32_t st_pack(float lo, float hi) {
     st_float2_v v = {lo, hi};
-    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, st_bf16x2_v));
+    if constexpr (XF16) return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, st_f16x2_v));
+    else return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, st_bf16x2_v));
 }
 
 // Byte offset of 16-byte chunk `chunk` of row `row` in a [rows][128 bytes] array: the chunk position is rotated by
@@ -67,8 +72,11 @@ __device__ __forceinline__ uint32_t st_lds_off(uint32_t row, uint32_t chunk) {
     return row * 128u + ((chunk ^ ((row >> 1) & 7u)) << 4);
 }
 
-template <int GROUP, int MB, bool SB_BF16>
+template <int BITS, int GROUP, int MB, bool SB_BF16, bool XF16>
 __global__ __launch_bounds__(kStreamThreads) void qgemm_stream_kernel(StreamArgs a) {
+    constexpr int LW = BITS;                              // words a lane loads per K-tile: 32 codes
+    constexpr int TW = 2 * LW;                            // words of a row's K-tile
+    static_assert(BITS == 4 || BITS == 8, "4- or 8-bit codes");
     constexpr int MPAD = 32 * MB;                         // staged activation rows
     constexpr int SLICE_BYTES = MPAD * 128;               // one K slice of a stage: [MPAD][64] bf16
     constexpr int STAGE = 4 * SLICE_BYTES;
@@ -150,18 +158,19 @@ __global__ __launch_bounds__(kStreamThreads) void qgemm_stream_kernel(StreamArgs
         uint32_t wrow = n0 + ln;
         wrow = wrow < seg_n ? wrow : seg_n - 1;           // rows past the end re-read the last one
         const uint32_t* const crow = (in2 ? a.codes[2] : in1 ? a.codes[1] : a.codes[0]) +
-                                     (size_t)wrow * (in2 ? a.code_stride[2] : in1 ? a.code_stride[1] : a.code_stride[0]) + 4 * lh;
+                                     (size_t)wrow * (in2 ? a.code_stride[2] : in1 ? a.code_stride[1] : a.code_stride[0]) + LW * lh;
         const uint32_t* const szrow = (in2 ? a.sz[2] : in1 ? a.sz[1] : a.sz[0]) +
                                       (size_t)wrow * (in2 ? a.sz_stride[2] : in1 ? a.sz_stride[1] : a.sz_stride[0]);
         // weight words and (scale, bias) word of this wavefront's K-tile of iteration `it`
-        u32x4 ring[U];
+        u32x4 ring[U][LW / 4];
         uint32_t szring[U];
         auto load_w = [&](auto I, uint32_t it) __attribute__((always_inline)) {
             constexpr int i = decltype(I)::value;
             uint32_t t = it * 4 + slice;
             t = t < KT ? t : KT - 1;
-            ring[i] = *(const u32x4*)(crow + (size_t)t * 8);
-            szring[i] = szrow[(t * 64) / GROUP];
+#pragma unroll
+            for (int v = 0; v < LW / 4; v++) ring[i][v] = *(const u32x4*)(crow + (size_t)t * TW + 4 * v);
+            szring[i] = szrow[(t * 64 + 32 * lh) / GROUP];     // the group of this lane's 32 codes
         };
         static_for<U>([&](auto I) __attribute__((always_inline)) { load_w(I, it_begin + decltype(I)::value); });
         __syncthreads();
@@ -171,7 +180,9 @@ __global__ __launch_bounds__(kStreamThreads) void qgemm_stream_kernel(StreamArgs
                 constexpr int stage = i % 3;
                 const uint32_t it = it0 + i;
                 if (it < it_end) {                        // the same for every wavefront of the workgroup
-                    const u32x4 w = ring[i];
+                    u32x4 w[LW / 4];
+#pragma unroll
+                    for (int v = 0; v < LW / 4; v++) w[v] = ring[i][v];
                     const uint32_t szw = szring[i];
                     load_w(I, it + U);
                     if (it * 4 + slice < KT) {
@@ -184,27 +195,40 @@ __global__ __launch_bounds__(kStreamThreads) void qgemm_stream_kernel(StreamArgs
                         const char* const xs_lds = lds + stage * STAGE + slice * SLICE_BYTES;
                         static_for<4>([&](auto J) __attribute__((always_inline)) {
                             constexpr int j = decltype(J)::value;
-                            const uint32_t word = j == 0 ? w.x : j == 1 ? w.y : j == 2 ? w.z : w.w;
-                            const uint32_t lo = word & 0x0F0F0F0Fu, hi = (word >> 4) & 0x0F0F0F0Fu;
+                            // the eight codes of k-step j as bytes: (c0,c2,c4,c6) and (c1,c3,c5,c7) of a 4-bit word,
+                            // (c0..c3) and (c4..c7) of two 8-bit words
+                            uint32_t lo, hi;
+                            if constexpr (BITS == 4) {
+                                const uint32_t word = w[0][j];
+                                lo = word & 0x0F0F0F0Fu; hi = (word >> 4) & 0x0F0F0F0Fu;
+                            } else {
+                                lo = w[j / 2][2 * (j % 2)]; hi = w[j / 2][2 * (j % 2) + 1];
+                            }
                             float q[8];
-                            asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(q[0]) : "v"(lo));
-                            asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(q[1]) : "v"(hi));
-                            asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(q[2]) : "v"(lo));
-                            asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(q[3]) : "v"(hi));
-                            asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(q[4]) : "v"(lo));
-                            asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(q[5]) : "v"(hi));
-                            asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(q[6]) : "v"(lo));
-                            asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(q[7]) : "v"(hi));
+                            constexpr int at0 = BITS == 4 ? 0 : 0, at1 = BITS == 4 ? 2 : 1, at2 = BITS == 4 ? 4 : 2, at3 = BITS == 4 ? 6 : 3;
+                            asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(q[at0]) : "v"(lo));
+                            asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(q[at1]) : "v"(lo));
+                            asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(q[at2]) : "v"(lo));
+                            asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(q[at3]) : "v"(lo));
+                            constexpr int bt0 = BITS == 4 ? 1 : 4, bt1 = BITS == 4 ? 3 : 5, bt2 = BITS == 4 ? 5 : 6, bt3 = 7;
+                            asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(q[bt0]) : "v"(hi));
+                            asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(q[bt1]) : "v"(hi));
+                            asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(q[bt2]) : "v"(hi));
+                            asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(q[bt3]) : "v"(hi));
                             u32x4 o;
-                            o.x = st_pack_bf16(__builtin_fmaf(s, q[0], z), __builtin_fmaf(s, q[1], z));
-                            o.y = st_pack_bf16(__builtin_fmaf(s, q[2], z), __builtin_fmaf(s, q[3], z));
-                            o.z = st_pack_bf16(__builtin_fmaf(s, q[4], z), __builtin_fmaf(s, q[5], z));
-                            o.w = st_pack_bf16(__builtin_fmaf(s, q[6], z), __builtin_fmaf(s, q[7], z));
-                            const st_bf16x8_t bw = __builtin_bit_cast(st_bf16x8_t, o);
+                            o.x = st_pack<XF16>(__builtin_fmaf(s, q[0], z), __builtin_fmaf(s, q[1], z));
+                            o.y = st_pack<XF16>(__builtin_fmaf(s, q[2], z), __builtin_fmaf(s, q[3], z));
+                            o.z = st_pack<XF16>(__builtin_fmaf(s, q[4], z), __builtin_fmaf(s, q[5], z));
+                            o.w = st_pack<XF16>(__builtin_fmaf(s, q[6], z), __builtin_fmaf(s, q[7], z));
 #pragma unroll
                             for (int b = 0; b < MB; b++) {
-                                const st_bf16x8_t ax = *(const st_bf16x8_t*)(xs_lds + st_lds_off(b * 32 + ln, 4 * lh + j));
-                                acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ax, bw, acc[b], 0, 0, 0);
+                                const u32x4 ax = *(const u32x4*)(xs_lds + st_lds_off(b * 32 + ln, 4 * lh + j));
+                                if constexpr (XF16)
+                                    acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(st_f16x8_t, ax),
+                                                                                    __builtin_bit_cast(st_f16x8_t, o), acc[b], 0, 0, 0);
+                                else
+                                    acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(st_bf16x8_t, ax),
+                                                                                     __builtin_bit_cast(st_bf16x8_t, o), acc[b], 0, 0, 0);
                             }
                             if constexpr (MB >= 3) __builtin_amdgcn_sched_barrier(0);   // one word at a time: registers
                         });
@@ -275,9 +299,10 @@ __global__ __launch_bounds__(256) void stream_sum_parts_kernel(StreamArgs a, uin
 }
 
 bool gemm_stream_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
-    if (x_dtype != MI355Q_BF16 || m < 1 || m > kStreamMaxRows) return false;
+    if ((x_dtype != MI355Q_BF16 && x_dtype != MI355Q_F16) || m < 1 || m > kStreamMaxRows) return false;
     if (w.layout != MI355Q_LAYOUT_PLANES || !w.sz || !w.codes) return false;
-    if (w.bits != 4 || (w.group != 64 && w.group != 128)) return false;
+    if (!((w.bits == 4 && (w.group == 64 || w.group == 128)) ||
+          (w.bits == 8 && (w.group == 32 || w.group == 64 || w.group == 128)))) return false;
     if (w.k % 64 || w.k < 64 || x_stride % 8) return false;
     if ((uintptr_t)w.codes % 16 || w.code_stride % 4) return false;
     return true;
@@ -304,9 +329,9 @@ StreamLaunchShape gemm_stream_shape_blocks(const mi355q_context* ctx, uint32_t m
 
 namespace {
 
-template <int GROUP, int MB, bool SB_BF16>
+template <int BITS, int GROUP, int MB, bool SB_BF16, bool XF16>
 mi355q_status launch_stream_mb(hipStream_t s, const StreamArgs& a, const StreamLaunchShape& g) {
-    auto kern = qgemm_stream_kernel<GROUP, MB, SB_BF16>;
+    auto kern = qgemm_stream_kernel<BITS, GROUP, MB, SB_BF16, XF16>;
     if (g.lds_bytes > 64u * 1024u) {
         // the attribute belongs to the function on one device: one bit per device and instantiation
         static std::atomic<uint64_t> lds_limit_raised{0};
@@ -323,15 +348,21 @@ mi355q_status launch_stream_mb(hipStream_t s, const StreamArgs& a, const StreamL
     return MI355Q_OK;
 }
 
-template <int GROUP, bool SB_BF16>
-mi355q_status launch_stream_group(hipStream_t s, const StreamArgs& a, const StreamLaunchShape& g) {
+template <int BITS, int GROUP, bool SB_BF16, bool XF16>
+mi355q_status launch_stream_blocks(hipStream_t s, const StreamArgs& a, const StreamLaunchShape& g) {
     switch (g.m_blocks) {
-    case 1: return launch_stream_mb<GROUP, 1, SB_BF16>(s, a, g);
-    case 2: return launch_stream_mb<GROUP, 2, SB_BF16>(s, a, g);
-    case 3: return launch_stream_mb<GROUP, 3, SB_BF16>(s, a, g);
+    case 1: return launch_stream_mb<BITS, GROUP, 1, SB_BF16, XF16>(s, a, g);
+    case 2: return launch_stream_mb<BITS, GROUP, 2, SB_BF16, XF16>(s, a, g);
+    case 3: return launch_stream_mb<BITS, GROUP, 3, SB_BF16, XF16>(s, a, g);
     default: break;
     }
     return fail(MI355Q_ERR_SHAPE, "the streamed-weight kernel takes at most %u rows", kStreamMaxRows);
+}
+
+template <int BITS, int GROUP>
+mi355q_status launch_stream_group(hipStream_t s, const StreamArgs& a, const StreamLaunchShape& g, bool sb_bf16, bool x_f16) {
+    if (sb_bf16) return x_f16 ? launch_stream_blocks<BITS, GROUP, true, true>(s, a, g) : launch_stream_blocks<BITS, GROUP, true, false>(s, a, g);
+    return x_f16 ? launch_stream_blocks<BITS, GROUP, false, true>(s, a, g) : launch_stream_blocks<BITS, GROUP, false, false>(s, a, g);
 }
 
 }  // namespace
@@ -347,7 +378,7 @@ bool gemm_stream_multi_eligible(uint32_t count, const WView* w, int x_dtype, uin
     if (count < 1 || count > (uint32_t)kStreamMaxSegments) return false;
     for (uint32_t i = 0; i < count; i++)
         if (!gemm_stream_eligible(w[i], x_dtype, m, x_stride) || w[i].k != w[0].k || w[i].group != w[0].group ||
-            w[i].sb_dtype != w[0].sb_dtype)
+            w[i].bits != w[0].bits || w[i].sb_dtype != w[0].sb_dtype)
             return false;
     return true;
 }
@@ -384,9 +415,16 @@ mi355q_status launch_qgemm_stream_multi(hipStream_t s, mi355q_context* ctx, uint
         if (mi355q_status st = ensure_workspace(ctx, (size_t)g.parts * m * cols * sizeof(float))) return st;
         a.partial = (float*)ctx->workspace;
     }
-    const bool bf = w[0].sb_dtype == MI355Q_BF16;
-    const mi355q_status st = w[0].group == 64 ? (bf ? launch_stream_group<64, true>(s, a, g) : launch_stream_group<64, false>(s, a, g))
-                                              : (bf ? launch_stream_group<128, true>(s, a, g) : launch_stream_group<128, false>(s, a, g));
+    const bool bf = w[0].sb_dtype == MI355Q_BF16, xf = x_dtype == MI355Q_F16;
+    mi355q_status st = MI355Q_ERR_KERNEL_NOT_FOUND;
+    switch (w[0].bits * 1000 + w[0].group) {
+    case 4064: st = launch_stream_group<4, 64>(s, a, g, bf, xf); break;
+    case 4128: st = launch_stream_group<4, 128>(s, a, g, bf, xf); break;
+    case 8032: st = launch_stream_group<8, 32>(s, a, g, bf, xf); break;
+    case 8064: st = launch_stream_group<8, 64>(s, a, g, bf, xf); break;
+    case 8128: st = launch_stream_group<8, 128>(s, a, g, bf, xf); break;
+    default: break;
+    }
     if (st != MI355Q_OK || g.parts == 1) return st;
     const size_t total = (size_t)m * cols;
     size_t sum_blocks = (total + 255) / 256;

@@ -1,4 +1,5 @@
-"""Streamed-weight matrix-core kernel (gemm_stream.hip): 17 to 96 bf16 activation rows on 4-bit planes, the weights
+"""Streamed-weight matrix-core kernel (gemm_stream.hip): 17 to 96 activation rows (bf16, or f16 from nine rows) on 4- and
+8-bit planes, the weights
 dequantised in registers straight into the matrix cores' operand, the activations alone staged through LDS.
 
 The kernel rounds every weight to bf16 exactly as the tiled prefill kernel does
@@ -20,23 +21,24 @@ def say(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def _case(seed, n, k, group, sb):
+def _case(seed, n, k, group, sb, bits=4):
     w = kat.seeded_weights(seed, n, k)
-    words, s, z = oracle.quantize_affine(w, 4, group, sb)
-    return words, s, z, oracle.dequant_planes_f32(4, group, n, k, words, s, z, sb)
+    words, s, z = oracle.quantize_affine(w, bits, group, sb)
+    return words, s, z, oracle.dequant_planes_f32(bits, group, n, k, words, s, z, sb)
 
 
-def _run(ctx, pkg, w, x, m, n, y_dtype, flags, ypad=0, xpad=0):
+def _run(ctx, pkg, w, x, m, n, y_dtype, flags, ypad=0, xpad=0, x_dtype=None):
+    x_dtype = pkg.BF16 if x_dtype is None else x_dtype
     k = x.shape[1]
     xh = np.zeros((m, k + xpad), dtype=np.float32)
     xh[:, :k] = x
-    xd = ctx.upload(act_to_device_array(xh, pkg.BF16, pkg))
+    xd = ctx.upload(act_to_device_array(xh, x_dtype, pkg))
     ysz = 4 if y_dtype == pkg.F32 else 2
     if (m * (n + ypad) * ysz) % 4:
         ypad += 1
     yd = ctx.alloc(m * (n + ypad) * ysz)
     ctx.fill(yd, 0x7FC07FC0 if ysz == 2 else 0x7FC00000)
-    ctx.qgemm(w, xd, pkg.BF16, yd, y_dtype, m, k + xpad, n + ypad, flags)
+    ctx.qgemm(w, xd, x_dtype, yd, y_dtype, m, k + xpad, n + ypad, flags)
     ctx.synchronize()
     got = out_from_device(yd, y_dtype, (m, n + ypad), pkg)
     xd.free(); yd.free()
@@ -109,11 +111,11 @@ def test_stream_kernel_refuses_what_it_does_not_read(pkg, ctx):
     ws = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, pkg.LAYOUT_STAF_BLOCKS)
     with pytest.raises(pkg.MI355QError):
         _run(ctx, pkg, ws, x[:20], 20, 64, pkg.F32, pkg.FLAG_FORCE_STREAM)     # block layout
-    fmt8 = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(8, 64)
-    words8, s8, z8 = oracle.quantize_affine(kat.seeded_weights(1501, 64, 128), 8, 64, oracle.BF16)
+    fmt8 = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(6, 64)
+    words8, s8, z8 = oracle.quantize_affine(kat.seeded_weights(1501, 64, 128), 6, 64, oracle.BF16)
     w8 = ctx.weight_prepare_mlx(fmt8, words8, s8, z8, pkg.BF16, pkg.LAYOUT_PLANES)
     with pytest.raises(pkg.MI355QError):
-        _run(ctx, pkg, w8, x[:20], 20, 64, pkg.F32, pkg.FLAG_FORCE_STREAM)     # 8-bit codes
+        _run(ctx, pkg, w8, x[:20], 20, 64, pkg.F32, pkg.FLAG_FORCE_STREAM)     # 6-bit codes
     for t in (w, ws, w8):
         t.destroy()
 
@@ -147,4 +149,52 @@ def test_stream_kernel_shared_launch_equals_separate_launches(pkg, ctx, count, m
             b.free()
     xd.free()
     for w in ws:
+        w.destroy()
+
+
+@pytest.mark.parametrize("bits,group", [(8, 32), (8, 64), (8, 128)])
+def test_stream_kernel_eight_bit_codes(pkg, ctx, bits, group):
+    """8-bit codes: a lane's 32 codes are eight words, two per k-step; groups of 32 give the two halves of a K-tile
+    their own (scale, bias) word.  Against the oracle, the tiled kernel (which reads q8 g32 / g64) and the plan record."""
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(bits, group)
+    for i, (m, n, k) in enumerate([(17, 64, 128), (40, 1000, 384), (96, 130, 2176), (64, 4096, 1024), (33, 64, 14336)]):
+        for sbo, sbp in ((oracle.BF16, pkg.BF16), (oracle.F16, pkg.F16)):
+            say(f"stream q8 g{group} M={m} {k}->{n} sb {sbp}")
+            words, s, z, wq = _case(1800 + i, n, k, group, sbo, bits=8)
+            w = ctx.weight_prepare_mlx(fmt, words, s, z, sbp, pkg.LAYOUT_PLANES)
+            x = act_rounded(kat.seeded_activations(1900 + i, m, k), pkg.BF16, pkg)
+            got = _run(ctx, pkg, w, x, m, n, pkg.F32, pkg.FLAG_FORCE_STREAM, ypad=i % 2, xpad=8 * (i % 2))
+            assert rel_l2(got, oracle.gemm_f64(wq, x)) < 2.5e-3
+            if group != 128:
+                tiled = _run(ctx, pkg, w, x, m, n, pkg.F32, pkg.FLAG_FORCE_MFMA)
+                assert rel_l2(got, tiled) < 2e-6
+            auto = _run(ctx, pkg, w, x, m, n, pkg.F32, 0)
+            assert np.array_equal(auto, got)
+            assert w.plan_prefill_steps(m)[0].device_kernel == f"qgemm_stream_q8_g{group}"
+            w.destroy()
+
+
+@pytest.mark.parametrize("bits,group", [(4, 64), (4, 128), (8, 32), (8, 64)])
+def test_stream_kernel_f16_activations(pkg, ctx, bits, group):
+    """f16 activations (the reference's decode type): the weights are rounded to f16 instead of bf16 and the f16 matrix
+    instruction multiplies; taken unforced from nine rows (one small-batch launch takes eight f16 rows)."""
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(bits, group)
+    for i, (m, n, k) in enumerate([(9, 64, 128), (16, 300, 1024), (31, 1000, 384), (64, 130, 4096), (96, 257, 2176)]):
+        say(f"stream f16 q{bits} g{group} M={m} {k}->{n}")
+        words, s, z, wq = _case(2000 + i, n, k, group, oracle.BF16, bits=bits)
+        w = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, pkg.LAYOUT_PLANES)
+        x = act_rounded(kat.seeded_activations(2100 + i, m, k), pkg.F16, pkg)
+        want = oracle.gemm_f64(wq, x)
+        got = _run(ctx, pkg, w, x, m, n, pkg.F32, pkg.FLAG_FORCE_STREAM, ypad=i % 2, x_dtype=pkg.F16)
+        # f16-rounded weights: 2^-12 relative per weight
+        assert rel_l2(got, want) < 4e-4, rel_l2(got, want)
+        two = _run(ctx, pkg, w, x, m, n, pkg.F32, pkg.FLAG_FORCE_TWO_STEP, x_dtype=pkg.F16) if m >= 16 else None
+        if two is not None:
+            assert rel_l2(got, two) < 2e-6            # the same f16 weights, another order of the fp32 sums
+        auto = _run(ctx, pkg, w, x, m, n, pkg.F32, 0, x_dtype=pkg.F16)
+        assert np.array_equal(auto, got), "nine to 96 f16 rows on eligible planes take the streamed-weight kernel"
+        low = _run(ctx, pkg, w, x, m, n, pkg.F16, pkg.FLAG_FORCE_STREAM, x_dtype=pkg.F16)
+        assert np.array_equal(low, act_rounded(got, pkg.F16, pkg))
+        step = w.plan_prefill_steps(m, x_dtype=pkg.F16)[0]
+        assert step.device_kernel == f"qgemm_stream_q{bits}_g{group}"
         w.destroy()

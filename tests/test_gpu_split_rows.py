@@ -150,7 +150,8 @@ def test_f16_rows_on_the_matrix_core_kernels(pkg, ctx, layout):
     """f16 activations (the reference's decode type) on the kernels that compute in bf16 on the matrix cores: a row is
     staged inside the kernel as two bf16 rows (the upper eight significant bits, the remaining three) and the two
     partial results are added before the store -- up to eight f16 rows a launch on TILE16 records, three to eight on
-    4-bit planes (below, the f16 dot-product kernels), more rows in steps of eight.  One-hot rows with an 11-bit value
+    4-bit planes (below, the f16 dot-product kernels), more rows in steps of eight on the records and on the
+    streamed-weight kernel on the planes.  One-hot rows with an 11-bit value
     (1024 + odd) / 2048, which needs both parts, must come out bit for bit; seeded f16 rows to 1e-5 of the fp64
     reference on the same f16 values; padded rows; all output types."""
     lay = {"planes": pkg.LAYOUT_PLANES, "tile16": pkg.LAYOUT_TILE16}[layout]
@@ -166,7 +167,10 @@ def test_f16_rows_on_the_matrix_core_kernels(pkg, ctx, layout):
     for m in (1, 2, 3, 4, 5, 7, 8, 9, 13, 15):
         say(f"f16 rows {layout} M={m}")
         st = w.plan_prefill_steps(m, x_dtype=pkg.F16)[0]
-        assert (st.device_kernel == fast) == (layout == "tile16" or m >= 3), (m, st.device_kernel)
+        if layout == "planes" and m > 8:        # beyond one launch of eight f16 rows: the streamed-weight kernel (f16 weights)
+            assert st.device_kernel == "qgemm_stream_q4_g64", (m, st.device_kernel)
+        else:
+            assert (st.device_kernel == fast) == (layout == "tile16" or m >= 3), (m, st.device_kernel)
         assert m > 8 or not st.used_fallback
         x = np.zeros((m, k), np.float32)
         pos = rng.choice(k, m, replace=False)
