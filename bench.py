@@ -348,10 +348,12 @@ def main():
                 for b in list(xm.values()) + list(ym.values()):
                     b.free()
             log(f"  batch sweep {lname} (N(0,1) activations): " + ", ".join(f"{k} {v['us_per_step']} us" for k, v in batch_sweep[lname].items()))
-            if lname == "tile16":
-                # the reference's decode type on the records: the kernel stages an f16 row as two bf16 rows
-                batch_sweep["tile16_f16_activations"] = {}
-                for m in (1, 8):
+            if True:
+                # the reference's decode type: the small-batch kernels stage an f16 row as two bf16 rows; from nine rows
+                # the planes run the streamed-weight kernel with f16 weights
+                key16 = lname + "_f16_activations"
+                batch_sweep[key16] = {}
+                for m in ((1, 8) if lname == "tile16" else (8, 32, 64)):
                     xm = {k: ctx.upload(kat.seeded_activations(950 + m, m, k).astype(np.float16).view(np.uint16)) for k in (4096, 14336)}
                     ym = {name: ctx.alloc(m * n * 2) for name, n, _ in LAYER_SHAPES}
                     pl = pkg.DispatchPlan(ctx)
@@ -363,13 +365,14 @@ def main():
                     pl.encode(stream)
                     ctx.synchronize(stream)
                     ms = time_region(ctx, lambda i: pl.encode(stream), 32, stream) / len(pool)
-                    batch_sweep["tile16_f16_activations"][f"M={m}"] = {
+                    batch_sweep[key16][f"M={m}"] = {
                         "us_per_step": round(ms * 1e3, 2), "GBps": round(layer_bytes / (ms * 1e-3) / 1e9, 1),
                         "kernel": pl.step(2)[0].device_kernel}
                     pl.destroy()
                     for b in list(xm.values()) + list(ym.values()):
                         b.free()
-                log(f"  batch sweep tile16, f16 activations: {batch_sweep['tile16_f16_activations']}")
+                log(f"  batch sweep {lname}, f16 activations: {batch_sweep[key16]}")
+            if lname == "tile16":
                 for L in pool:
                     for w in L.values():
                         w.destroy()

@@ -91,7 +91,7 @@ enum {
     MI355Q_FLAG_FORCE_MFMA = 4,    /* qgemm: use the fused MFMA kernel whatever M is */
     /* bit 3 (value 8) is taken by the measurement flag of mi355_qlinear_probe.h */
     MI355Q_FLAG_FORCE_TWO_STEP = 16, /* qgemm: dequantise to bf16 scratch, then the dense library GEMM, whatever M is */
-    MI355Q_FLAG_FORCE_STREAM = 32  /* qgemm: the streamed-weight matrix-core kernel (4-bit planes, bf16 rows, M <= 96) */
+    MI355Q_FLAG_FORCE_STREAM = 32  /* qgemm: the streamed-weight matrix-core kernel (4- / 8-bit planes, bf16 or f16 rows, M <= 96) */
 };
 
 /* ------------------------------------------------------------------------------------------
@@ -278,9 +278,10 @@ MI355Q_API mi355q_status mi355q_qgemv(mi355q_context* ctx, void* stream, const m
  * (the numerics of the reference's dequant -> bf16 -> GEMM route):
  *   - small M (up to 8 rows; 16 on TILE16 records and on q4 / q8 planes; up to 32 in two launches where the
  *     next route does not read the weight): the GEMV-style decode kernels;
- *   - 17 to 96 bf16 rows on 4-bit planes (groups of 64 or 128): the streamed-weight kernel -- weights
- *     dequantised in registers straight into the matrix cores' operand, the activations alone staged in LDS;
- *     through mi355q_batched_qgemm two or three matrices share one launch;
+ *   - 17 to 96 bf16 rows, or 9 to 96 f16 rows, on 4-bit planes (groups of 64 or 128) and 8-bit planes (groups
+ *     of 32, 64 or 128): the streamed-weight kernel -- weights dequantised in registers straight into the
+ *     matrix cores' operand (rounded to the activations' type), the activations alone staged in LDS; through
+ *     mi355q_batched_qgemm two or three matrices share one launch;
  *   - ONE fused kernel: code tiles are dequantised to bf16 in LDS and contracted on MFMA (the planes
  *     and TILE16 layouts, formats q4 g64/g128, q8 g32/g64, q6/q3/q2 g64, bf16 activations);
  *   - two dispatches, as the reference's second route: the whole matrix is dequantised to bf16 in a

@@ -266,7 +266,7 @@ bool gemm_mfma_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stri
 mi355q_status launch_qgemm_mfma(hipStream_t s, mi355q_context* ctx, const WView& w,
                                 const void* x, int x_dtype, void* y, int y_dtype, uint32_t m,
                                 uint32_t x_stride, uint32_t y_stride, unsigned long long* probe = nullptr);
-// Streamed-weight matrix-core kernel (gemm_stream.hip): 4-bit planes, bf16 activations, at most 96 rows.
+// Streamed-weight matrix-core kernel (gemm_stream.hip): 4- and 8-bit planes, bf16 or f16 activations, at most 96 rows.
 constexpr uint32_t kStreamMaxRows = 96;
 struct StreamLaunchShape {
     uint32_t row_blocks;       // workgroups along N (64 weight rows each)

@@ -1,8 +1,8 @@
 // Projection of 17 to 96 activation rows on the matrix cores with the weights streamed through registers:
-//   Y[M,N] = X[M,K] * W[N,K]^T,  W = 4-bit group-affine codes on the split planes, bf16 activations.
+//   Y[M,N] = X[M,K] * W[N,K]^T,  W = 4- or 8-bit group-affine codes on the split planes, bf16 or f16 activations.
 //
-// Stands in, at these sequence lengths, for the reference's direct quantized GEMM gemm_q4_g64 / gemm_q4_g128
-// (Sources/MetalCompiler/Generator/MetalSourceGenerator+Quantized.swift:22-156) and for its dequant + matmul2d pair
+// Stands in, at these sequence lengths, for the reference's direct quantized GEMM gemm_q4_g64 / gemm_q4_g128 /
+// gemm_q8_g32 / gemm_q8_g64 (Sources/MetalCompiler/Generator/MetalSourceGenerator+Quantized.swift:22-156) and for its dequant + matmul2d pair
 // (MetalSourceGenerator+Linear.swift:18-81).  The tiled prefill kernel dequantises a weight K-tile into LDS once per
 // workgroup and spends a barrier round trip on it whatever M is; with at most three 32-row blocks of activations the
 // whole M extent fits one wavefront's accumulators, so here nothing but the activations goes through LDS:
@@ -11,7 +11,8 @@
 //     a row together;
 //   * lane (n, h) of a wavefront loads 16 bytes = words 4h .. 4h+3 of row n's K-tile and uses word j in k-step j:
 //     the eight codes of a word become the B operand of v_mfma_f32_32x32x16_bf16 in registers (byte-lane convert,
-//     fp32 fma with the group's scale and bias, one rounding to bf16: the weights of the tiled kernel, bit for bit);
+//     fp32 fma with the group's scale and bias, one rounding to bf16: the weights of the tiled kernel, bit for bit;
+//     with f16 activations one rounding to f16 and the f16 instruction; 8-bit codes: eight words a lane, two a k-step);
 //     the A operand is the activations' chunk 4h + j of that K-tile, read from LDS;
 //   * per iteration four more wavefronts of the workgroup stage [32 MB rows][256 columns] of activations
 //     (XOR-swizzled 128-byte rows per K slice) two iterations ahead into the third of three LDS stages, copied
