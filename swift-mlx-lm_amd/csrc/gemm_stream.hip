@@ -44,6 +44,8 @@ struct StreamArgs {
     void* y[kStreamMaxSegments];
     uint32_t n[kStreamMaxSegments], ys[kStreamMaxSegments];
     uint32_t code_stride[kStreamMaxSegments], sz_stride[kStreamMaxSegments];
+    const uint8_t* blocks[kStreamMaxSegments];     // block layout: [N][row_bytes], a block = (scale f16, zero f16, codes)
+    uint64_t row_bytes;                            // block layout: bytes from one row to the next
     uint32_t wg_end[kStreamMaxSegments], col0[kStreamMaxSegments];
     const uint16_t* x;         // bf16 [M][xs]
     float* partial;            // K split over workgroups: fp32 [parts][M][n_total]; else null
@@ -73,7 +75,12 @@ __device__ __forceinline__ uint32_t st_lds_off(uint32_t row, uint32_t chunk) {
     return row * 128u + ((chunk ^ ((row >> 1) & 7u)) << 4);
 }
 
-template <int BITS, int GROUP, int MB, bool SB_BF16, bool XF16>
+// 16 bytes at an address that is a multiple of four
+typedef uint32_t st_u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+
+// BLOCKS: the weights lie in the reference's interleaved blocks (one (scale f16, zero f16) header and the codes of a group
+// each) instead of the planes; SB_BF16 is false then.
+template <int BITS, int GROUP, int MB, bool SB_BF16, bool XF16, bool BLOCKS>
 __global__ __launch_bounds__(kStreamThreads) void qgemm_stream_kernel(StreamArgs a) {
     constexpr int LW = BITS;                              // words a lane loads per K-tile: 32 codes
     constexpr int TW = 2 * LW;                            // words of a row's K-tile
@@ -158,10 +165,17 @@ __global__ __launch_bounds__(kStreamThreads) void qgemm_stream_kernel(StreamArgs
     } else {
         uint32_t wrow = n0 + ln;
         wrow = wrow < seg_n ? wrow : seg_n - 1;           // rows past the end re-read the last one
-        const uint32_t* const crow = (in2 ? a.codes[2] : in1 ? a.codes[1] : a.codes[0]) +
-                                     (size_t)wrow * (in2 ? a.code_stride[2] : in1 ? a.code_stride[1] : a.code_stride[0]) + LW * lh;
-        const uint32_t* const szrow = (in2 ? a.sz[2] : in1 ? a.sz[1] : a.sz[0]) +
-                                      (size_t)wrow * (in2 ? a.sz_stride[2] : in1 ? a.sz_stride[1] : a.sz_stride[0]);
+        const uint32_t* crow = nullptr;
+        const uint32_t* szrow = nullptr;
+        const uint8_t* brow = nullptr;
+        if constexpr (BLOCKS) {
+            brow = (in2 ? a.blocks[2] : in1 ? a.blocks[1] : a.blocks[0]) + (size_t)wrow * a.row_bytes;
+        } else {
+            crow = (in2 ? a.codes[2] : in1 ? a.codes[1] : a.codes[0]) +
+                   (size_t)wrow * (in2 ? a.code_stride[2] : in1 ? a.code_stride[1] : a.code_stride[0]) + LW * lh;
+            szrow = (in2 ? a.sz[2] : in1 ? a.sz[1] : a.sz[0]) +
+                    (size_t)wrow * (in2 ? a.sz_stride[2] : in1 ? a.sz_stride[1] : a.sz_stride[0]);
+        }
         // weight words and (scale, bias) word of this wavefront's K-tile of iteration `it`
         u32x4 ring[U][LW / 4];
         uint32_t szring[U];
@@ -169,9 +183,20 @@ __global__ __launch_bounds__(kStreamThreads) void qgemm_stream_kernel(StreamArgs
             constexpr int i = decltype(I)::value;
             uint32_t t = it * 4 + slice;
             t = t < KT ? t : KT - 1;
+            if constexpr (BLOCKS) {
+                // the lane's 32 codes start at code c0 of the row: block c0 / GROUP, behind its 4-byte header
+                constexpr uint32_t BLOCK_BYTES = 4 + GROUP * BITS / 8;
+                const uint32_t c0 = t * 64 + 32 * lh;
+                const uint8_t* const blk = brow + (size_t)(c0 / GROUP) * BLOCK_BYTES;
+                szring[i] = *(const uint32_t*)blk;
 #pragma unroll
-            for (int v = 0; v < LW / 4; v++) ring[i][v] = *(const u32x4*)(crow + (size_t)t * TW + 4 * v);
-            szring[i] = szrow[(t * 64 + 32 * lh) / GROUP];     // the group of this lane's 32 codes
+                for (int v = 0; v < LW / 4; v++)
+                    ring[i][v] = *(const st_u32x4_a4*)(blk + 4 + (c0 % GROUP) * BITS / 8 + 16 * v);
+            } else {
+#pragma unroll
+                for (int v = 0; v < LW / 4; v++) ring[i][v] = *(const u32x4*)(crow + (size_t)t * TW + 4 * v);
+                szring[i] = szrow[(t * 64 + 32 * lh) / GROUP];     // the group of this lane's 32 codes
+            }
         };
         static_for<U>([&](auto I) __attribute__((always_inline)) { load_w(I, it_begin + decltype(I)::value); });
         __syncthreads();
@@ -301,11 +326,15 @@ __global__ __launch_bounds__(256) void stream_sum_parts_kernel(StreamArgs a, uin
 
 bool gemm_stream_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
     if ((x_dtype != MI355Q_BF16 && x_dtype != MI355Q_F16) || m < 1 || m > kStreamMaxRows) return false;
-    if (w.layout != MI355Q_LAYOUT_PLANES || !w.sz || !w.codes) return false;
+    if (w.layout == MI355Q_LAYOUT_STAF_BLOCKS) {
+        if (!w.blocks || (uintptr_t)w.blocks % 4 || w.bytes_per_block != 4 + w.group * w.bits / 8) return false;
+    } else if (w.layout != MI355Q_LAYOUT_PLANES || !w.sz || !w.codes) {
+        return false;
+    }
     if (!((w.bits == 4 && (w.group == 64 || w.group == 128)) ||
           (w.bits == 8 && (w.group == 32 || w.group == 64 || w.group == 128)))) return false;
     if (w.k % 64 || w.k < 64 || x_stride % 8) return false;
-    if ((uintptr_t)w.codes % 16 || w.code_stride % 4) return false;
+    if (w.layout == MI355Q_LAYOUT_PLANES && ((uintptr_t)w.codes % 16 || w.code_stride % 4)) return false;
     return true;
 }
 
@@ -330,9 +359,9 @@ StreamLaunchShape gemm_stream_shape_blocks(const mi355q_context* ctx, uint32_t m
 
 namespace {
 
-template <int BITS, int GROUP, int MB, bool SB_BF16, bool XF16>
+template <int BITS, int GROUP, int MB, bool SB_BF16, bool XF16, bool BLOCKS>
 mi355q_status launch_stream_mb(hipStream_t s, const StreamArgs& a, const StreamLaunchShape& g) {
-    auto kern = qgemm_stream_kernel<BITS, GROUP, MB, SB_BF16, XF16>;
+    auto kern = qgemm_stream_kernel<BITS, GROUP, MB, SB_BF16, XF16, BLOCKS>;
     if (g.lds_bytes > 64u * 1024u) {
         // the attribute belongs to the function on one device: one bit per device and instantiation
         static std::atomic<uint64_t> lds_limit_raised{0};
@@ -349,21 +378,24 @@ mi355q_status launch_stream_mb(hipStream_t s, const StreamArgs& a, const StreamL
     return MI355Q_OK;
 }
 
-template <int BITS, int GROUP, bool SB_BF16, bool XF16>
+template <int BITS, int GROUP, bool SB_BF16, bool XF16, bool BLOCKS>
 mi355q_status launch_stream_blocks(hipStream_t s, const StreamArgs& a, const StreamLaunchShape& g) {
     switch (g.m_blocks) {
-    case 1: return launch_stream_mb<BITS, GROUP, 1, SB_BF16, XF16>(s, a, g);
-    case 2: return launch_stream_mb<BITS, GROUP, 2, SB_BF16, XF16>(s, a, g);
-    case 3: return launch_stream_mb<BITS, GROUP, 3, SB_BF16, XF16>(s, a, g);
+    case 1: return launch_stream_mb<BITS, GROUP, 1, SB_BF16, XF16, BLOCKS>(s, a, g);
+    case 2: return launch_stream_mb<BITS, GROUP, 2, SB_BF16, XF16, BLOCKS>(s, a, g);
+    case 3: return launch_stream_mb<BITS, GROUP, 3, SB_BF16, XF16, BLOCKS>(s, a, g);
     default: break;
     }
     return fail(MI355Q_ERR_SHAPE, "the streamed-weight kernel takes at most %u rows", kStreamMaxRows);
 }
 
 template <int BITS, int GROUP>
-mi355q_status launch_stream_group(hipStream_t s, const StreamArgs& a, const StreamLaunchShape& g, bool sb_bf16, bool x_f16) {
-    if (sb_bf16) return x_f16 ? launch_stream_blocks<BITS, GROUP, true, true>(s, a, g) : launch_stream_blocks<BITS, GROUP, true, false>(s, a, g);
-    return x_f16 ? launch_stream_blocks<BITS, GROUP, false, true>(s, a, g) : launch_stream_blocks<BITS, GROUP, false, false>(s, a, g);
+mi355q_status launch_stream_group(hipStream_t s, const StreamArgs& a, const StreamLaunchShape& g, bool sb_bf16, bool x_f16,
+                                  bool blocks) {
+    if (blocks)     // block headers are f16
+        return x_f16 ? launch_stream_blocks<BITS, GROUP, false, true, true>(s, a, g) : launch_stream_blocks<BITS, GROUP, false, false, true>(s, a, g);
+    if (sb_bf16) return x_f16 ? launch_stream_blocks<BITS, GROUP, true, true, false>(s, a, g) : launch_stream_blocks<BITS, GROUP, true, false, false>(s, a, g);
+    return x_f16 ? launch_stream_blocks<BITS, GROUP, false, true, false>(s, a, g) : launch_stream_blocks<BITS, GROUP, false, false, false>(s, a, g);
 }
 
 }  // namespace
@@ -379,7 +411,7 @@ bool gemm_stream_multi_eligible(uint32_t count, const WView* w, int x_dtype, uin
     if (count < 1 || count > (uint32_t)kStreamMaxSegments) return false;
     for (uint32_t i = 0; i < count; i++)
         if (!gemm_stream_eligible(w[i], x_dtype, m, x_stride) || w[i].k != w[0].k || w[i].group != w[0].group ||
-            w[i].bits != w[0].bits || w[i].sb_dtype != w[0].sb_dtype)
+            w[i].bits != w[0].bits || w[i].sb_dtype != w[0].sb_dtype || w[i].layout != w[0].layout)
             return false;
     return true;
 }
@@ -394,7 +426,7 @@ mi355q_status launch_qgemm_stream_multi(hipStream_t s, mi355q_context* ctx, uint
     uint32_t blocks = 0, cols = 0;
     for (uint32_t i = 0; i < (uint32_t)kStreamMaxSegments; i++) {
         const uint32_t j = i < count ? i : count - 1;          // unused entries repeat the last matrix and own nothing
-        a.codes[i] = w[j].codes; a.sz[i] = w[j].sz; a.y[i] = y[j];
+        a.codes[i] = w[j].codes; a.sz[i] = w[j].sz; a.blocks[i] = w[j].blocks; a.y[i] = y[j];
         a.n[i] = w[j].n; a.ys[i] = y_strides[j];
         a.code_stride[i] = w[j].code_stride; a.sz_stride[i] = w[j].sz_stride;
         if (i < count) {
@@ -407,6 +439,7 @@ mi355q_status launch_qgemm_stream_multi(hipStream_t s, mi355q_context* ctx, uint
             a.wg_end[i] = 0xFFFFFFFFu;
         }
     }
+    a.row_bytes = (uint64_t)w[0].blocks_per_row * w[0].bytes_per_block;
     a.x = (const uint16_t*)x;
     a.m = m; a.k = w[0].k; a.xs = x_stride; a.n_total = cols;
     a.y_dtype = (uint32_t)y_dtype;
@@ -416,14 +449,14 @@ mi355q_status launch_qgemm_stream_multi(hipStream_t s, mi355q_context* ctx, uint
         if (mi355q_status st = ensure_workspace(ctx, (size_t)g.parts * m * cols * sizeof(float))) return st;
         a.partial = (float*)ctx->workspace;
     }
-    const bool bf = w[0].sb_dtype == MI355Q_BF16, xf = x_dtype == MI355Q_F16;
+    const bool bf = w[0].sb_dtype == MI355Q_BF16, xf = x_dtype == MI355Q_F16, bl = w[0].layout == MI355Q_LAYOUT_STAF_BLOCKS;
     mi355q_status st = MI355Q_ERR_KERNEL_NOT_FOUND;
     switch (w[0].bits * 1000 + w[0].group) {
-    case 4064: st = launch_stream_group<4, 64>(s, a, g, bf, xf); break;
-    case 4128: st = launch_stream_group<4, 128>(s, a, g, bf, xf); break;
-    case 8032: st = launch_stream_group<8, 32>(s, a, g, bf, xf); break;
-    case 8064: st = launch_stream_group<8, 64>(s, a, g, bf, xf); break;
-    case 8128: st = launch_stream_group<8, 128>(s, a, g, bf, xf); break;
+    case 4064: st = launch_stream_group<4, 64>(s, a, g, bf, xf, bl); break;
+    case 4128: st = launch_stream_group<4, 128>(s, a, g, bf, xf, bl); break;
+    case 8032: st = launch_stream_group<8, 32>(s, a, g, bf, xf, bl); break;
+    case 8064: st = launch_stream_group<8, 64>(s, a, g, bf, xf, bl); break;
+    case 8128: st = launch_stream_group<8, 128>(s, a, g, bf, xf, bl); break;
     default: break;
     }
     if (st != MI355Q_OK || g.parts == 1) return st;

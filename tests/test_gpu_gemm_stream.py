@@ -108,9 +108,9 @@ def test_stream_kernel_refuses_what_it_does_not_read(pkg, ctx):
         _run(ctx, pkg, w, x, 97, 64, pkg.F32, pkg.FLAG_FORCE_STREAM)           # more than 96 rows
     with pytest.raises(pkg.MI355QError):
         _run(ctx, pkg, w, x[:20], 20, 64, pkg.F32, pkg.FLAG_FORCE_STREAM | pkg.FLAG_FORCE_MFMA)
-    ws = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, pkg.LAYOUT_STAF_BLOCKS)
+    ws = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, pkg.LAYOUT_TILE16)
     with pytest.raises(pkg.MI355QError):
-        _run(ctx, pkg, ws, x[:20], 20, 64, pkg.F32, pkg.FLAG_FORCE_STREAM)     # block layout
+        _run(ctx, pkg, ws, x[:20], 20, 64, pkg.F32, pkg.FLAG_FORCE_STREAM)     # tile records
     fmt8 = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(6, 64)
     words8, s8, z8 = oracle.quantize_affine(kat.seeded_weights(1501, 64, 128), 6, 64, oracle.BF16)
     w8 = ctx.weight_prepare_mlx(fmt8, words8, s8, z8, pkg.BF16, pkg.LAYOUT_PLANES)
@@ -197,4 +197,46 @@ def test_stream_kernel_f16_activations(pkg, ctx, bits, group):
         assert np.array_equal(low, act_rounded(got, pkg.F16, pkg))
         step = w.plan_prefill_steps(m, x_dtype=pkg.F16)[0]
         assert step.device_kernel == f"qgemm_stream_q{bits}_g{group}"
+        w.destroy()
+
+
+@pytest.mark.parametrize("bits,group", [(4, 64), (4, 128), (8, 32), (8, 64), (8, 128)])
+def test_stream_kernel_reads_staf_blocks_in_place(pkg, ctx, bits, group):
+    """Weights left in the reference's interleaved blocks (a model.staf payload, zero copy): the lane's 32 codes lie in
+    one block behind its (scale, zero) header, at a 4-byte aligned address.  Same results as from the planes bit for
+    bit (the same f16 scales), against the oracle, unforced from nine rows, bf16 and f16 activations, shared launch."""
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(bits, group)
+    for i, (m, n, k) in enumerate([(9, 64, 128), (17, 300, 1024), (40, 1000, 384), (96, 130, 2176), (64, 200, 14336)]):
+        words, s, z, wq = _case(2200 + i, n, k, group, oracle.F16, bits=bits)
+        wb = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.F16, pkg.LAYOUT_STAF_BLOCKS)
+        wp = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.F16, pkg.LAYOUT_PLANES)
+        for x_dtype in (pkg.BF16, pkg.F16):
+            say(f"stream from blocks q{bits} g{group} M={m} {k}->{n} x {x_dtype}")
+            x = act_rounded(kat.seeded_activations(2300 + i, m, k), x_dtype, pkg)
+            got = _run(ctx, pkg, wb, x, m, n, pkg.F32, pkg.FLAG_FORCE_STREAM, ypad=i % 2, xpad=8 * (i % 2), x_dtype=x_dtype)
+            ref = _run(ctx, pkg, wp, x, m, n, pkg.F32, pkg.FLAG_FORCE_STREAM, x_dtype=x_dtype)
+            assert np.array_equal(got, ref), "blocks and planes hold the same codes and f16 scales"
+            assert rel_l2(got, oracle.gemm_f64(wq, x)) < (2.5e-3 if x_dtype == pkg.BF16 else 4e-4)
+            auto = _run(ctx, pkg, wb, x, m, n, pkg.F32, 0, x_dtype=x_dtype)
+            assert np.array_equal(auto, got), "nine to 96 rows on blocks take the streamed-weight kernel unforced"
+            step = wb.plan_prefill_steps(m, x_dtype=x_dtype)[0]
+            assert step.device_kernel == f"qgemm_stream_q{bits}_g{group}" and not step.used_fallback
+        wb.destroy(); wp.destroy()
+    # two matrices in blocks sharing the activations: one launch, the bits of separate launches
+    m, k, ns = 33, 1024, [200, 1000]
+    ws, alone = [], []
+    x = act_rounded(kat.seeded_activations(2400, m, k), pkg.BF16, pkg)
+    for j, n in enumerate(ns):
+        words, s, z, _ = _case(2410 + j, n, k, group, oracle.F16, bits=bits)
+        ws.append(ctx.weight_prepare_mlx(fmt, words, s, z, pkg.F16, pkg.LAYOUT_STAF_BLOCKS))
+        alone.append(_run(ctx, pkg, ws[-1], x, m, n, pkg.F32, pkg.FLAG_FORCE_STREAM))
+    xd = ctx.upload(act_to_device_array(x, pkg.BF16, pkg))
+    yds = [ctx.alloc(m * n * 4) for n in ns]
+    ctx.batched_qgemm(ws, xd, pkg.BF16, yds, pkg.F32, m, 0, 0)
+    ctx.synchronize()
+    for yd, n, want in zip(yds, ns, alone):
+        assert np.array_equal(out_from_device(yd, pkg.F32, (m, n), pkg), want)
+        yd.free()
+    xd.free()
+    for w in ws:
         w.destroy()

@@ -102,7 +102,8 @@ def test_two_step_seeded_ragged_shapes_and_strides(pkg, ctx, bits, group, layout
 
 
 def test_two_step_is_chosen_where_measured_faster_and_planned_as_two_steps(pkg, ctx):
-    """Without flags: the block layout (no fused matrix-core kernel) takes the route from sixteen rows; the planes keep
+    """Without flags: the block layout (no fused matrix-core kernel) takes the route beyond the 96 rows of the
+    streamed-weight kernel; the planes keep
     the fused kernel up to 511 rows (wide matrices, N >= 8192, up to 767; shapes with K > N up to 2047).  The planner reports dequant + GEMM as two steps."""
     n, k = 192, 512
     words, s, z, wq = seeded_case(3300, n, k, 4, 64)
@@ -111,12 +112,14 @@ def test_two_step_is_chosen_where_measured_faster_and_planned_as_two_steps(pkg, 
     ws = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, pkg.LAYOUT_STAF_BLOCKS)
     words1, s1, z1, _ = seeded_case(3303, 512, 512, 4, 64)               # N >= K
     wp = ctx.weight_prepare_mlx(fmt, words1, s1, z1, pkg.BF16, pkg.LAYOUT_PLANES)
-    steps = ws.plan_prefill_steps(64)
+    steps = ws.plan_prefill_steps(100)
     assert [st.kernel_name for st in steps] == ["dequant_q4_g64_bf16", "gemm_bf16_f32s"]
     assert [st.kernel_family for st in steps] == ["dequantToBFloat", "libraryGEMM"]
-    assert steps[0].flops == 0 and steps[1].flops == 2 * 64 * n * k and steps[1].weight_bytes == n * k * 2
+    assert steps[0].flops == 0 and steps[1].flops == 2 * 100 * n * k and steps[1].weight_bytes == n * k * 2
     assert not steps[0].used_fallback and not steps[1].used_fallback
-    assert len(ws.plan_prefill_steps(12)) == 1 and ws.plan_prefill_steps(12)[0].used_fallback
+    assert [st.device_kernel for st in ws.plan_prefill_steps(64)] == ["qgemm_stream_q4_g64"]      # nine to 96 rows
+    assert [st.device_kernel for st in ws.plan_prefill_steps(12)] == ["qgemm_stream_q4_g64"]
+    assert len(ws.plan_prefill_steps(8)) == 1 and ws.plan_prefill_steps(8)[0].device_kernel == "gemv_staf_q4_g64"
     assert len(ws.plan_prefill_steps(64, flags=pkg.FLAG_FORCE_SMALL_M)) == 1
     assert [st.kernel_family for st in wp.plan_prefill_steps(511)] == ["mfmaGEMM"]
     assert [st.kernel_family for st in wp.plan_prefill_steps(512)] == ["dequantToBFloat", "libraryGEMM"]
@@ -142,8 +145,8 @@ def test_two_step_is_chosen_where_measured_faster_and_planned_as_two_steps(pkg, 
     with pytest.raises(pkg.MI355QError) as err:
         run_qgemm(ctx, pkg, ws, x, pkg.F16, pkg.FLAG_FORCE_TWO_STEP)
     assert err.value.status_name == "KERNEL_NOT_FOUND"
-    h = run_qgemm(ctx, pkg, ws, x, pkg.F16, 0)
-    assert_within_tolerance(h, oracle.gemm_f64(wq, x), "f16 output, no flags")
+    h = run_qgemm(ctx, pkg, ws, x, pkg.F16, 0)                              # 64 rows: the streamed-weight kernel, bf16 weights
+    assert_within_tolerance(h, want, "f16 output, no flags")
     for bad in (pkg.FLAG_FORCE_TWO_STEP | pkg.FLAG_FORCE_MFMA, pkg.FLAG_FORCE_TWO_STEP | pkg.FLAG_FORCE_GENERIC):
         with pytest.raises(pkg.MI355QError):
             run_qgemm(ctx, pkg, ws, x, pkg.F32, bad)
@@ -224,8 +227,8 @@ def test_two_step_f16_and_f32_activations(pkg, ctx, x_dtype_name, y_dtype_names)
     w_round = wq.astype(np.float16).astype(np.float32) if x_dtype == pkg.F16 else bf16_round(wq)
     for layout in (pkg.LAYOUT_PLANES, pkg.LAYOUT_STAF_BLOCKS):
         w = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, layout)
-        # f16 rows on 4-bit planes run on the streamed-weight kernel up to 96 rows (f16 weights there too)
-        steps = w.plan_prefill_steps(200 if x_dtype == pkg.F16 and layout == pkg.LAYOUT_PLANES else 64, x_dtype=x_dtype)
+        # f16 rows on 4-bit planes and blocks run on the streamed-weight kernel up to 96 rows (f16 weights there too)
+        steps = w.plan_prefill_steps(200 if x_dtype == pkg.F16 else 64, x_dtype=x_dtype)
         want_kernels = (["dequant_q4_g64_f16", "hipblaslt_gemm_f16"] if x_dtype == pkg.F16
                         else ["dequant_q4_g64_bf16", "hipblaslt_gemm_bf16_x2"])
         assert [st.device_kernel for st in steps] == want_kernels
