@@ -91,7 +91,7 @@ enum {
     MI355Q_FLAG_FORCE_MFMA = 4,    /* qgemm: use the fused MFMA kernel whatever M is */
     /* bit 3 (value 8) is taken by the measurement flag of mi355_qlinear_probe.h */
     MI355Q_FLAG_FORCE_TWO_STEP = 16, /* qgemm: dequantise to bf16 scratch, then the dense library GEMM, whatever M is */
-    MI355Q_FLAG_FORCE_STREAM = 32  /* qgemm: the streamed-weight matrix-core kernel (4- / 8-bit planes, bf16 or f16 rows, M <= 96) */
+    MI355Q_FLAG_FORCE_STREAM = 32  /* qgemm: the streamed-weight matrix-core kernel (4- / 8-bit planes or blocks, bf16 or f16 rows, M <= 96) */
 };
 
 /* ------------------------------------------------------------------------------------------
@@ -279,7 +279,8 @@ MI355Q_API mi355q_status mi355q_qgemv(mi355q_context* ctx, void* stream, const m
  *   - small M (up to 8 rows; 16 on TILE16 records and on q4 / q8 planes; up to 32 in two launches where the
  *     next route does not read the weight): the GEMV-style decode kernels;
  *   - 17 to 96 bf16 rows, or 9 to 96 f16 rows, on 4-bit planes (groups of 64 or 128) and 8-bit planes (groups
- *     of 32, 64 or 128): the streamed-weight kernel -- weights dequantised in registers straight into the
+ *     of 32, 64 or 128), and 9 to 96 rows of either type on the same formats left in STAF blocks: the
+ *     streamed-weight kernel -- weights dequantised in registers straight into the
  *     matrix cores' operand (rounded to the activations' type), the activations alone staged in LDS; through
  *     mi355q_batched_qgemm two or three matrices share one launch;
  *   - ONE fused kernel: code tiles are dequantised to bf16 in LDS and contracted on MFMA (the planes
