@@ -95,7 +95,13 @@ mi355q_status run_split_rows(mi355q_context* ctx, hipStream_t s, const mi355q_we
     uint16_t* const xp = (uint16_t*)ctx->split_buffer;
     float* const yp = (float*)((char*)ctx->split_buffer + xbytes);
     if (mi355q_status st = launch_split_rows_bf16(s, x, x_dtype, m, k, xs, xp, kp)) return st;
-    if (mi355q_status st = run_small_m(ctx, s, w, xp, MI355Q_BF16, yp, MI355Q_F32, parts * m, kp, n, flags)) return st;
+    const WView v = w->view();
+    if (!(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_SMALL_M)) && gemm_stream_chosen(v, MI355Q_BF16, parts * m, kp) &&
+        gemm_stream_unrounded(v, parts * m)) {
+        if (mi355q_status st = launch_qgemm_stream(s, ctx, v, xp, MI355Q_BF16, yp, MI355Q_F32, parts * m, kp, n)) return st;
+    } else if (mi355q_status st = run_small_m(ctx, s, w, xp, MI355Q_BF16, yp, MI355Q_F32, parts * m, kp, n, flags)) {
+        return st;
+    }
     return launch_sum_parts_rows(s, yp, parts, m, n, y, y_dtype, ys);
 }
 
@@ -133,6 +139,9 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
         if (gemm_two_step_chosen(v, x_dtype, m, xs, flags) && (uintptr_t)x % 16 == 0 &&
             gemm_two_step_serves(ctx, v, x_dtype, y_dtype, m, xs, ys))
             return launch_qgemm_two_step(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
+        if (!(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_SMALL_M)) && gemm_stream_chosen(v, x_dtype, m, xs) &&
+            gemm_stream_unrounded(v, m) && (uintptr_t)x % 16 == 0)
+            return launch_qgemm_stream(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
         return run_small_m(ctx, s, w, x, x_dtype, y, y_dtype, m, xs, ys, flags);
     }
     const uint32_t forced = flags & (MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_TWO_STEP | MI355Q_FLAG_FORCE_SMALL_M |
@@ -179,7 +188,14 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
 // prefill kernel, 32 rows 136 against 161).
 uint32_t small_batch_limit(const WView& w, int x_dtype, uint32_t x_stride) {
     const uint32_t rows = small_batch_rows(w, x_dtype, x_stride);
-    if (gemm_stream_eligible(w, x_dtype, rows + 1, x_stride)) return rows;     // the streamed-weight kernel takes over
+    if (gemm_stream_eligible(w, x_dtype, rows + 1, x_stride)) {                // the streamed-weight kernel takes over
+        // blocks in place: the in-place decode kernel costs 18.7 us at four rows and 35.7 at eight (4096 -> 14336 q4 g64;
+        // 31 and 60 on 14336 -> 4096), the streamed kernel with unrounded weights 15.6 and 17.6 whatever the rows
+        // (and from the first row where no decode kernel reads the blocks: rows that are not whole 16-byte units)
+        if (w.layout == MI355Q_LAYOUT_STAF_BLOCKS && gemm_stream_unrounded(w, kStreamBlocksFirstRows))
+            return gemv_staf_eligible(w, x_dtype, 1, x_stride) ? kStreamBlocksFirstRows - 1 : 0;
+        return rows;
+    }
     return rows >= 16 ? 2 * rows : rows;
 }
 
@@ -342,7 +358,7 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
         tiled = tiled && gemv_tile16_eligible(views[i], x_dtype, m, xs) &&
                 gemv_tile16_k_parts(ctx, views[i], staged_rows(x_dtype, m)) == 1 &&
                 views[i].sb_dtype == views[0].sb_dtype;
-        in_place = in_place && gemv_staf_eligible(views[i], x_dtype, m, xs);
+        in_place = in_place && gemv_staf_eligible(views[i], x_dtype, m, xs) && !gemm_stream_chosen(views[i], x_dtype, m, xs);
         on_planes = on_planes && gemv_mfma_planes_eligible(views[i], x_dtype, m, xs) &&
                     gemv_mfma_planes_k_parts(ctx, views[i], staged_rows(x_dtype, m)) == 1 && views[i].sb_dtype == views[0].sb_dtype &&
                     views[i].code_stride == views[0].code_stride && views[i].group == views[0].group;

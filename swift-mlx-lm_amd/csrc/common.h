@@ -268,6 +268,7 @@ mi355q_status launch_qgemm_mfma(hipStream_t s, mi355q_context* ctx, const WView&
                                 uint32_t x_stride, uint32_t y_stride, unsigned long long* probe = nullptr);
 // Streamed-weight matrix-core kernel (gemm_stream.hip): 4- and 8-bit planes, bf16 or f16 activations, at most 96 rows.
 constexpr uint32_t kStreamMaxRows = 96;
+constexpr uint32_t kStreamBlocksFirstRows = 3;     // blocks in place: rows from which it replaces the in-place decode kernel
 struct StreamLaunchShape {
     uint32_t row_blocks;       // workgroups along N (64 weight rows each)
     uint32_t parts;            // K parts (workgroups along K; fp32 partial results added by a second launch)
@@ -277,6 +278,9 @@ struct StreamLaunchShape {
 };
 bool gemm_stream_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
 bool gemm_stream_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
+// Whether the kernel keeps the weights unrounded at m rows (scale and bias applied to a K-tile's fp32 sums): one block
+// of activation rows, groups of whole K-tiles.
+bool gemm_stream_unrounded(const WView& w, uint32_t m);
 StreamLaunchShape gemm_stream_shape(const mi355q_context* ctx, uint32_t m, uint32_t n, uint32_t k);
 mi355q_status launch_qgemm_stream(hipStream_t s, mi355q_context* ctx, const WView& w, const void* x, int x_dtype, void* y,
                                   int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride);

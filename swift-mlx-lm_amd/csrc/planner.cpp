@@ -55,6 +55,19 @@ void plan_small_m(const mi355q_weight* w, uint32_t m, int x_dtype, uint32_t x_st
         std::snprintf(s->device_kernel, sizeof s->device_kernel, "split_f32_bf16x3+%.30s", inner);
         return;
     }
+    if (!(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_SMALL_M)) && gemm_stream_chosen(v, x_dtype, m, x_stride) &&
+        gemm_stream_unrounded(v, m)) {
+        // blocks in place from three rows: the streamed-weight kernel with unrounded weights
+        const StreamLaunchShape g = gemm_stream_shape(w->ctx, m, (uint32_t)w->n, (uint32_t)w->k);
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "qgemm_stream_q%u_g%u", (unsigned)w->fmt.bits,
+                      w->fmt.group_size);
+        s->grid[0] = g.row_blocks;
+        s->grid[1] = g.parts;
+        s->block[0] = 768;
+        s->lds_bytes = g.lds_bytes;
+        s->rows_per_workgroup = 64;
+        return;
+    }
     // rows per launch on the tile layout: 16, or fewer when K is so long that 16 staged rows overflow LDS
     const uint32_t most = x_dtype == MI355Q_F16 ? 8 : 16;      // sixteen staged rows a launch; f16 rows are staged as two
     uint32_t t16_rows = m > most ? most : m;

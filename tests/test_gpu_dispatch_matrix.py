@@ -104,7 +104,10 @@ def test_random_shared_launches(pkg, ctx):
             fused = out_from_device(yds[j], y_dtype, (m, n), pkg)
             alone = ctx.alloc(m * n * ysz)
             ctx.qgemm(ws[j], xd, x_dtype, alone, y_dtype, m, 0, 0, 0); ctx.synchronize()
-            assert np.array_equal(fused, out_from_device(alone, y_dtype, (m, n), pkg)), (i, j)
+            sep = out_from_device(alone, y_dtype, (m, n), pkg)
+            # the streamed-weight kernel splits K by the launch's workgroup count: a shared launch and a launch alone may
+            # add their fp32 parts in another order (and then round a 16-bit result the other way now and then)
+            assert np.array_equal(fused, sep) or rel_l2(fused, sep) <= (2e-6 if y_dtype == pkg.F32 else 1e-3), (i, j)
             alone.free()
         xd.free()
         for b in yds:

@@ -63,10 +63,15 @@ def test_stream_kernel_against_oracle_and_tiled_kernel(pkg, ctx, group, sb):
         want = oracle.gemm_f64(wq, x)
         got = _run(ctx, pkg, w, x, m, n, pkg.F32, pkg.FLAG_FORCE_STREAM, ypad=i % 3, xpad=8 * (i % 2))
         tiled = _run(ctx, pkg, w, x, m, n, pkg.F32, pkg.FLAG_FORCE_MFMA)
-        # bf16-rounded weights: 2^-9 relative per weight, 1.5e-3 in the L2 norm at most
-        assert rel_l2(got, want) < 2.5e-3, (m, n, k, rel_l2(got, want))
-        # the same rounded weights as the tiled kernel: only the order of the fp32 sums differs
-        assert rel_l2(got, tiled) < 2e-6, (m, n, k, rel_l2(got, tiled))
+        if m <= 32:
+            # one block of rows: the codes themselves in the operand, scale and bias applied to each K-tile's fp32 sums
+            assert rel_l2(got, want) < 1e-5, (m, n, k, rel_l2(got, want))
+            assert rel_l2(got, tiled) < 2.5e-3
+        else:
+            # bf16-rounded weights: 2^-9 relative per weight, 1.5e-3 in the L2 norm at most
+            assert rel_l2(got, want) < 2.5e-3, (m, n, k, rel_l2(got, want))
+            # the same rounded weights as the tiled kernel: only the order of the fp32 sums differs
+            assert rel_l2(got, tiled) < 2e-6, (m, n, k, rel_l2(got, tiled))
         auto = _run(ctx, pkg, w, x, m, n, pkg.F32, 0)
         assert np.array_equal(auto, got), "rows 17 to 96 on eligible planes take the streamed-weight kernel unforced"
         step = w.plan_prefill_steps(m)[0]
@@ -143,7 +148,8 @@ def test_stream_kernel_shared_launch_equals_separate_launches(pkg, ctx, count, m
         for w, wq, n, yd in zip(ws, wqs, ns, dense):
             got = out_from_device(yd, y_dtype, (m, n), pkg)
             alone = _run(ctx, pkg, w, x, m, n, y_dtype, pkg.FLAG_FORCE_STREAM)
-            assert np.array_equal(got, alone), (count, m, n)
+            # the K parts follow the launch's workgroup count, so the order of the fp32 sums may differ from a launch alone
+            assert rel_l2(got, alone) < (2e-6 if y_dtype == pkg.F32 else 1e-3), (count, m, n)
             assert rel_l2(got, oracle.gemm_f64(wq, x)) < (2.5e-3 if y_dtype == pkg.F32 else 5e-3)
         for b in dense:
             b.free()
@@ -164,10 +170,11 @@ def test_stream_kernel_eight_bit_codes(pkg, ctx, bits, group):
             w = ctx.weight_prepare_mlx(fmt, words, s, z, sbp, pkg.LAYOUT_PLANES)
             x = act_rounded(kat.seeded_activations(1900 + i, m, k), pkg.BF16, pkg)
             got = _run(ctx, pkg, w, x, m, n, pkg.F32, pkg.FLAG_FORCE_STREAM, ypad=i % 2, xpad=8 * (i % 2))
-            assert rel_l2(got, oracle.gemm_f64(wq, x)) < 2.5e-3
+            exact = m <= 32 and group % 64 == 0              # groups of 32 keep the rounded weights at every M
+            assert rel_l2(got, oracle.gemm_f64(wq, x)) < (1e-5 if exact else 2.5e-3)
             if group != 128:
                 tiled = _run(ctx, pkg, w, x, m, n, pkg.F32, pkg.FLAG_FORCE_MFMA)
-                assert rel_l2(got, tiled) < 2e-6
+                assert rel_l2(got, tiled) < (2.5e-3 if exact else 2e-6)
             auto = _run(ctx, pkg, w, x, m, n, pkg.F32, 0)
             assert np.array_equal(auto, got)
             assert w.plan_prefill_steps(m)[0].device_kernel == f"qgemm_stream_q8_g{group}"
@@ -186,11 +193,12 @@ def test_stream_kernel_f16_activations(pkg, ctx, bits, group):
         x = act_rounded(kat.seeded_activations(2100 + i, m, k), pkg.F16, pkg)
         want = oracle.gemm_f64(wq, x)
         got = _run(ctx, pkg, w, x, m, n, pkg.F32, pkg.FLAG_FORCE_STREAM, ypad=i % 2, x_dtype=pkg.F16)
-        # f16-rounded weights: 2^-12 relative per weight
-        assert rel_l2(got, want) < 4e-4, rel_l2(got, want)
+        exact = m <= 32 and group % 64 == 0
+        # f16-rounded weights: 2^-12 relative per weight; unrounded in the one-block variant
+        assert rel_l2(got, want) < (1e-5 if exact else 4e-4), rel_l2(got, want)
         two = _run(ctx, pkg, w, x, m, n, pkg.F32, pkg.FLAG_FORCE_TWO_STEP, x_dtype=pkg.F16) if m >= 16 else None
         if two is not None:
-            assert rel_l2(got, two) < 2e-6            # the same f16 weights, another order of the fp32 sums
+            assert rel_l2(got, two) < (4e-4 if exact else 2e-6)     # rounded: the same f16 weights, another order of the sums
         auto = _run(ctx, pkg, w, x, m, n, pkg.F32, 0, x_dtype=pkg.F16)
         assert np.array_equal(auto, got), "nine to 96 f16 rows on eligible planes take the streamed-weight kernel"
         low = _run(ctx, pkg, w, x, m, n, pkg.F16, pkg.FLAG_FORCE_STREAM, x_dtype=pkg.F16)
@@ -204,9 +212,12 @@ def test_stream_kernel_f16_activations(pkg, ctx, bits, group):
 def test_stream_kernel_reads_staf_blocks_in_place(pkg, ctx, bits, group):
     """Weights left in the reference's interleaved blocks (a model.staf payload, zero copy): the lane's 32 codes lie in
     one block behind its (scale, zero) header, at a 4-byte aligned address.  Same results as from the planes bit for
-    bit (the same f16 scales), against the oracle, unforced from nine rows, bf16 and f16 activations, shared launch."""
+    bit (the same f16 scales), against the oracle, unforced from three rows (unrounded weights up to 32 rows; groups of
+    32, which keep rounded weights, from nine), bf16 and f16 activations, shared launch."""
     fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(bits, group)
-    for i, (m, n, k) in enumerate([(9, 64, 128), (17, 300, 1024), (40, 1000, 384), (96, 130, 2176), (64, 200, 14336)]):
+    for i, (m, n, k) in enumerate([(3, 64, 128), (8, 300, 1024), (17, 300, 1024), (40, 1000, 384), (96, 130, 2176), (64, 200, 14336)]):
+        if m < 9 and group % 64:
+            continue                                     # groups of 32: from nine rows (rounded weights only)
         words, s, z, wq = _case(2200 + i, n, k, group, oracle.F16, bits=bits)
         wb = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.F16, pkg.LAYOUT_STAF_BLOCKS)
         wp = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.F16, pkg.LAYOUT_PLANES)
@@ -216,9 +227,9 @@ def test_stream_kernel_reads_staf_blocks_in_place(pkg, ctx, bits, group):
             got = _run(ctx, pkg, wb, x, m, n, pkg.F32, pkg.FLAG_FORCE_STREAM, ypad=i % 2, xpad=8 * (i % 2), x_dtype=x_dtype)
             ref = _run(ctx, pkg, wp, x, m, n, pkg.F32, pkg.FLAG_FORCE_STREAM, x_dtype=x_dtype)
             assert np.array_equal(got, ref), "blocks and planes hold the same codes and f16 scales"
-            assert rel_l2(got, oracle.gemm_f64(wq, x)) < (2.5e-3 if x_dtype == pkg.BF16 else 4e-4)
+            assert rel_l2(got, oracle.gemm_f64(wq, x)) < (1e-5 if m <= 32 and group % 64 == 0 else 2.5e-3 if x_dtype == pkg.BF16 else 4e-4)
             auto = _run(ctx, pkg, wb, x, m, n, pkg.F32, 0, x_dtype=x_dtype)
-            assert np.array_equal(auto, got), "nine to 96 rows on blocks take the streamed-weight kernel unforced"
+            assert np.array_equal(auto, got), "three to 96 rows on blocks take the streamed-weight kernel unforced"
             step = wb.plan_prefill_steps(m, x_dtype=x_dtype)[0]
             assert step.device_kernel == f"qgemm_stream_q{bits}_g{group}" and not step.used_fallback
         wb.destroy(); wp.destroy()
@@ -235,7 +246,7 @@ def test_stream_kernel_reads_staf_blocks_in_place(pkg, ctx, bits, group):
     ctx.batched_qgemm(ws, xd, pkg.BF16, yds, pkg.F32, m, 0, 0)
     ctx.synchronize()
     for yd, n, want in zip(yds, ns, alone):
-        assert np.array_equal(out_from_device(yd, pkg.F32, (m, n), pkg), want)
+        assert rel_l2(out_from_device(yd, pkg.F32, (m, n), pkg), want) < 2e-6
         yd.free()
     xd.free()
     for w in ws:

@@ -230,7 +230,12 @@ def test_batched_projections_other_activation_types(pkg, ctx):
             for j, n in enumerate(ns):
                 fused = yds[j].download(np.float32, (m, n))
                 alone = run_f32(ctx, pkg, ws[j], x.astype(np.float32), x_dtype=x_dtype, use_qgemm=True)
-                assert np.array_equal(fused, alone), (layout, m, j)
+                if layout == pkg.LAYOUT_STAF_BLOCKS:
+                    # the streamed-weight kernel: the K parts follow the launch's workgroup count, so the order of the
+                    # fp32 sums may differ between the shared launch and a launch alone
+                    assert rel_l2(fused, alone) <= 2e-6, (layout, m, j)
+                else:
+                    assert np.array_equal(fused, alone), (layout, m, j)
                 assert rel_l2(fused, oracle.gemm_f64(wqs[j], x.astype(np.float32))) <= 1e-5
             xd.free()
             for b in yds:

@@ -96,16 +96,18 @@ def test_in_place_gemv_is_the_planned_kernel(pkg, ctx):
     assert step.block[0] == 256 and step.grid[0] >= 1 and step.lds_bytes > 0
     f16_step = w.plan_decode_step(1, pkg.F16)
     assert f16_step.device_kernel == "gemv_staf_q4_g64" and not f16_step.used_fallback      # f16 activations too
-    assert w.plan_decode_step(1, pkg.F32).device_kernel == "split_f32_bf16x3+gemv_staf_q4_g64"   # fp32: three bf16 rows
+    # fp32: three bf16 rows, which the streamed-weight kernel takes from the blocks (unrounded weights)
+    assert w.plan_decode_step(1, pkg.F32).device_kernel == "split_f32_bf16x3+qgemm_stream_q4_g64"
+    assert w.plan_decode_step(2).device_kernel == "gemv_staf_q4_g64" and w.plan_decode_step(3).device_kernel == "qgemm_stream_q4_g64"
     forced = w.plan_decode_step(1, flags=pkg.FLAG_FORCE_GENERIC)
     assert forced.device_kernel == "gemv_generic" and forced.used_fallback
     w.destroy()
     odd = _case(3201, 16, 64 * 3, 4, 64)                    # 108-byte rows
     w = odd.device_weight(ctx, pkg, pkg.LAYOUT_STAF_BLOCKS)
-    # no decode kernel reads 108-byte rows: the per-code kernel at one row; from two, fp32 weights into scratch + the
-    # library's fp32 product (or, forced, the per-code kernel)
-    assert w.plan_decode_step(1).device_kernel == "gemv_generic"
-    assert w.plan_decode_step(2).device_kernel == "dequant_q4_g64_f32+hipblaslt_gemm_f32"
+    # the in-place decode kernel does not read 108-byte rows; the streamed-weight kernel does (4-byte aligned loads),
+    # with unrounded weights, from the first row (forced, the per-code kernel)
+    assert w.plan_decode_step(1).device_kernel == "qgemm_stream_q4_g64"
+    assert w.plan_decode_step(2).device_kernel == "qgemm_stream_q4_g64"
     assert w.plan_decode_step(2, flags=pkg.FLAG_FORCE_GENERIC).device_kernel == "gemv_generic"
     x = act_rounded(kat.seeded_activations(3202, 1, odd.k), pkg.BF16, pkg)
     got = run_gemv(ctx, pkg, w, x, pkg.BF16, pkg.F32)
