@@ -192,8 +192,14 @@ uint32_t small_batch_limit(const WView& w, int x_dtype, uint32_t x_stride) {
         // blocks in place: the in-place decode kernel costs 18.7 us at four rows and 35.7 at eight (4096 -> 14336 q4 g64;
         // 31 and 60 on 14336 -> 4096), the streamed kernel with unrounded weights 15.6 and 17.6 whatever the rows
         // (and from the first row where no decode kernel reads the blocks: rows that are not whole 16-byte units)
-        if (w.layout == MI355Q_LAYOUT_STAF_BLOCKS && gemm_stream_unrounded(w, kStreamBlocksFirstRows))
-            return gemv_staf_eligible(w, x_dtype, 1, x_stride) ? kStreamBlocksFirstRows - 1 : 0;
+        // Its cost has a floor of about 10 us (K parts and their sum launch on matrices of few rows), so smaller
+        // matrices change over later: 4096 -> 4096 at four rows 10.6 against 8.8 us, at six 10.6 against 14.5;
+        // 4096 -> 1024 at eight rows 9.8 against 10.0.
+        if (w.layout == MI355Q_LAYOUT_STAF_BLOCKS && gemm_stream_unrounded(w, 3)) {
+            const uint64_t codes = (uint64_t)w.n * w.k;
+            const uint32_t first = codes >= kStreamBlocksLargeCodes ? 3 : codes >= kStreamBlocksMediumCodes ? 5 : rows + 1;
+            return gemv_staf_eligible(w, x_dtype, 1, x_stride) ? first - 1 : 0;
+        }
         return rows;
     }
     return rows >= 16 ? 2 * rows : rows;
@@ -205,6 +211,14 @@ uint32_t small_batch_limit(const WView& w, int x_dtype, uint32_t x_stride) {
 // 28.0 against 35.4; 4096 -> 4096: 32 rows 12.4 against 17.6, 96 rows 17.9 against 22.7).
 bool gemm_stream_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
     return m <= kStreamMaxRows && gemm_stream_eligible(w, x_dtype, m, x_stride) && m > small_batch_limit(w, x_dtype, x_stride);
+}
+
+// The same for two or three matrices that would share a launch: the rows of all of them together decide.
+bool gemm_stream_chosen_multi(uint32_t count, const WView* w, int x_dtype, uint32_t m, uint32_t x_stride) {
+    if (m > kStreamMaxRows || !gemm_stream_multi_eligible(count, w, x_dtype, m, x_stride)) return false;
+    WView all = w[0];
+    for (uint32_t i = 1; i < count; i++) all.n += w[i].n;
+    return gemm_stream_chosen(all, x_dtype, m, x_stride);
 }
 
 uint32_t small_batch_rows(const WView& w, int x_dtype, uint32_t x_stride) {
@@ -358,11 +372,18 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
         tiled = tiled && gemv_tile16_eligible(views[i], x_dtype, m, xs) &&
                 gemv_tile16_k_parts(ctx, views[i], staged_rows(x_dtype, m)) == 1 &&
                 views[i].sb_dtype == views[0].sb_dtype;
-        in_place = in_place && gemv_staf_eligible(views[i], x_dtype, m, xs) && !gemm_stream_chosen(views[i], x_dtype, m, xs);
+        in_place = in_place && gemv_staf_eligible(views[i], x_dtype, m, xs);
         on_planes = on_planes && gemv_mfma_planes_eligible(views[i], x_dtype, m, xs) &&
                     gemv_mfma_planes_k_parts(ctx, views[i], staged_rows(x_dtype, m)) == 1 && views[i].sb_dtype == views[0].sb_dtype &&
                     views[i].code_stride == views[0].code_stride && views[i].group == views[0].group;
     }
+    // the streamed-weight kernel, one launch for the two or three matrices: a few dozen rows on 4- / 8-bit planes, and
+    // blocks in place from three to nine rows by the size of the matrices together
+    const bool no_stream = flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_TWO_STEP | MI355Q_FLAG_FORCE_SMALL_M);
+    const bool stream_multi = !no_stream && (uintptr_t)x % 16 == 0 &&
+                              ((flags & MI355Q_FLAG_FORCE_STREAM) ? gemm_stream_multi_eligible(count, views, x_dtype, m, xs)
+                                                                  : gemm_stream_chosen_multi(count, views, x_dtype, m, xs));
+    if (stream_multi) return launch_qgemm_stream_multi(s, ctx, count, views, x, x_dtype, ys, strides, y_dtype, m, xs);
     if (on_planes && (uintptr_t)x % 16 == 0)
         return launch_gemv_mfma_planes_multi(s, ctx, count, views, x, x_dtype, ys, strides, y_dtype, m, xs);
     if (fused && (uintptr_t)x % 16 == 0)
@@ -400,7 +421,7 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
     bool stepped = m > step && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_TWO_STEP));
     for (uint32_t i = 0; i < count && stepped; i++)
         stepped = decode_kernel_reads(views[i], x_dtype, xs) && !split_rows_chosen(views[i], x_dtype, m, xs, flags) &&
-                  !gemm_two_step_chosen(views[i], x_dtype, m, xs, flags) && !gemm_stream_chosen(views[i], x_dtype, m, xs) &&
+                  !gemm_two_step_chosen(views[i], x_dtype, m, xs, flags) &&
                   (m <= small_batch_limit(views[i], x_dtype, xs) || !gemm_mfma_eligible(views[i], x_dtype, m, xs));
     if (stepped) {
         const size_t xsz = x_dtype == MI355Q_F32 ? 4 : 2, ysz = y_dtype == MI355Q_F32 ? 4 : 2;
@@ -411,14 +432,6 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
                                                     y_dtype, m - m0 < step ? m - m0 : step, xs, flags)) return st;
         }
         return MI355Q_OK;
-    }
-    // a few dozen rows on 4-bit planes: the streamed-weight kernel, one launch for the two or three matrices
-    if (!(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_TWO_STEP | MI355Q_FLAG_FORCE_SMALL_M)) &&
-        (uintptr_t)x % 16 == 0 && gemm_stream_multi_eligible(count, views, x_dtype, m, xs)) {
-        bool chosen = true;
-        for (uint32_t i = 0; i < count; i++)
-            chosen = chosen && ((flags & MI355Q_FLAG_FORCE_STREAM) || gemm_stream_chosen(views[i], x_dtype, m, xs));
-        if (chosen) return launch_qgemm_stream_multi(s, ctx, count, views, x, x_dtype, ys, strides, y_dtype, m, xs);
     }
     for (uint32_t i = 0; i < count; i++) {
         mi355q_status st = dispatch_linear(ctx, s, weights[i], x, x_dtype, ys[i], y_dtype, m, xs, 0, flags, false);

@@ -268,7 +268,8 @@ mi355q_status launch_qgemm_mfma(hipStream_t s, mi355q_context* ctx, const WView&
                                 uint32_t x_stride, uint32_t y_stride, unsigned long long* probe = nullptr);
 // Streamed-weight matrix-core kernel (gemm_stream.hip): 4- and 8-bit planes, bf16 or f16 activations, at most 96 rows.
 constexpr uint32_t kStreamMaxRows = 96;
-constexpr uint32_t kStreamBlocksFirstRows = 3;     // blocks in place: rows from which it replaces the in-place decode kernel
+// blocks in place: codes (N x K) from which it replaces the in-place decode kernel at three rows / at five rows
+constexpr uint64_t kStreamBlocksLargeCodes = (uint64_t)1 << 25, kStreamBlocksMediumCodes = (uint64_t)1 << 23;
 struct StreamLaunchShape {
     uint32_t row_blocks;       // workgroups along N (64 weight rows each)
     uint32_t parts;            // K parts (workgroups along K; fp32 partial results added by a second launch)
@@ -278,6 +279,7 @@ struct StreamLaunchShape {
 };
 bool gemm_stream_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
 bool gemm_stream_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
+bool gemm_stream_chosen_multi(uint32_t count, const WView* w, int x_dtype, uint32_t m, uint32_t x_stride);
 // Whether the kernel keeps the weights unrounded at m rows (scale and bias applied to a K-tile's fp32 sums): one block
 // of activation rows, groups of whole K-tiles.
 bool gemm_stream_unrounded(const WView& w, uint32_t m);

@@ -230,7 +230,7 @@ def test_qgemm_selects_matrix_cores_above_eight_rows(pkg, ctx):
     ws = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, pkg.LAYOUT_STAF_BLOCKS)
     step = ws.plan_prefill_steps(m, flags=pkg.FLAG_FORCE_SMALL_M)[0]       # unforced, the two-dispatch route serves it
     assert step.kernel_family != "mfmaGEMM"
-    step = ws.plan_prefill_steps(12)[0]                  # three to 96 rows: the streamed-weight kernel reads the blocks
+    step = ws.plan_prefill_steps(12)[0]                  # nine to 96 rows: the streamed-weight kernel reads the blocks
     assert step.device_kernel == "qgemm_stream_q4_g64" and not step.used_fallback
     step = ws.plan_prefill_steps(2)[0]
     assert step.kernel_family != "mfmaGEMM"

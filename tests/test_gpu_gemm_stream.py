@@ -212,8 +212,8 @@ def test_stream_kernel_f16_activations(pkg, ctx, bits, group):
 def test_stream_kernel_reads_staf_blocks_in_place(pkg, ctx, bits, group):
     """Weights left in the reference's interleaved blocks (a model.staf payload, zero copy): the lane's 32 codes lie in
     one block behind its (scale, zero) header, at a 4-byte aligned address.  Same results as from the planes bit for
-    bit (the same f16 scales), against the oracle, unforced from three rows (unrounded weights up to 32 rows; groups of
-    32, which keep rounded weights, from nine), bf16 and f16 activations, shared launch."""
+    bit (the same f16 scales), against the oracle, unforced from nine rows (from three or five on large matrices, see the
+    test below), bf16 and f16 activations, shared launch."""
     fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(bits, group)
     for i, (m, n, k) in enumerate([(3, 64, 128), (8, 300, 1024), (17, 300, 1024), (40, 1000, 384), (96, 130, 2176), (64, 200, 14336)]):
         if m < 9 and group % 64:
@@ -228,10 +228,11 @@ def test_stream_kernel_reads_staf_blocks_in_place(pkg, ctx, bits, group):
             ref = _run(ctx, pkg, wp, x, m, n, pkg.F32, pkg.FLAG_FORCE_STREAM, x_dtype=x_dtype)
             assert np.array_equal(got, ref), "blocks and planes hold the same codes and f16 scales"
             assert rel_l2(got, oracle.gemm_f64(wq, x)) < (1e-5 if m <= 32 and group % 64 == 0 else 2.5e-3 if x_dtype == pkg.BF16 else 4e-4)
-            auto = _run(ctx, pkg, wb, x, m, n, pkg.F32, 0, x_dtype=x_dtype)
-            assert np.array_equal(auto, got), "three to 96 rows on blocks take the streamed-weight kernel unforced"
-            step = wb.plan_prefill_steps(m, x_dtype=x_dtype)[0]
-            assert step.device_kernel == f"qgemm_stream_q{bits}_g{group}" and not step.used_fallback
+            if m >= 9:                                   # matrices this small keep the in-place decode kernel up to eight rows
+                auto = _run(ctx, pkg, wb, x, m, n, pkg.F32, 0, x_dtype=x_dtype)
+                assert np.array_equal(auto, got), "nine to 96 rows on blocks take the streamed-weight kernel unforced"
+                step = wb.plan_prefill_steps(m, x_dtype=x_dtype)[0]
+                assert step.device_kernel == f"qgemm_stream_q{bits}_g{group}" and not step.used_fallback
         wb.destroy(); wp.destroy()
     # two matrices in blocks sharing the activations: one launch, the bits of separate launches
     m, k, ns = 33, 1024, [200, 1000]
@@ -247,6 +248,52 @@ def test_stream_kernel_reads_staf_blocks_in_place(pkg, ctx, bits, group):
     ctx.synchronize()
     for yd, n, want in zip(yds, ns, alone):
         assert rel_l2(out_from_device(yd, pkg.F32, (m, n), pkg), want) < 2e-6
+        yd.free()
+    xd.free()
+    for w in ws:
+        w.destroy()
+
+
+def test_blocks_in_place_change_over_to_the_stream_kernel_by_size(pkg, ctx):
+    """Blocks in place at a few rows: the in-place decode kernel re-reads the matrix for every four rows, the
+    streamed-weight kernel (unrounded weights up to 32 rows) costs the same whatever the rows but has a floor of about
+    10 us; matrices of 2^25 codes and more change over at three rows, of 2^23 at five, smaller ones at nine.  qgemv and
+    qgemm agree, the result holds the decode tolerance, and a shared launch decides on the matrices together."""
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+    for n, k, first in ((4096, 8192, 3), (2048, 4096, 5), (1024, 4096, 9)):
+        words, s, z, wq = _case(2500 + first, n, k, 64, oracle.F16)
+        w = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.F16, pkg.LAYOUT_STAF_BLOCKS)
+        for m in (first - 1, first):
+            want = "qgemm_stream_q4_g64" if m >= first else "gemv_staf_q4_g64"
+            if m <= 8:
+                assert w.plan_decode_step(m).device_kernel == want, (n, k, m)
+            assert w.plan_prefill_steps(m)[0].device_kernel == want, (n, k, m)
+            for x_dtype in (pkg.BF16, pkg.F16):
+                say(f"blocks {k}->{n} M={m} x {x_dtype}")
+                x = act_rounded(kat.seeded_activations(2600 + m, m, k), x_dtype, pkg)
+                got = _run(ctx, pkg, w, x, m, n, pkg.F32, 0, x_dtype=x_dtype)
+                # unrounded weights on either kernel (the in-place kernel's f16 dot products: pairs summed in fp32)
+                assert rel_l2(got, oracle.gemm_f64(wq, x)) < (1e-5 if m >= first else 1e-4)
+                if m <= 8:
+                    xd = ctx.upload(act_to_device_array(x, x_dtype, pkg)); yd = ctx.alloc(m * n * 4)
+                    ctx.qgemv(w, xd, x_dtype, yd, pkg.F32, m); ctx.synchronize()
+                    assert np.array_equal(out_from_device(yd, pkg.F32, (m, n), pkg), got)
+                    xd.free(); yd.free()
+        w.destroy()
+    # q + k + v of 2^23 + 2^21 + 2^21 codes at five rows: together 1.5 * 2^23, one shared launch of the stream kernel
+    ns, k, m = (2048, 512, 512), 4096, 5
+    ws, wqs = [], []
+    for j, n in enumerate(ns):
+        words, s, z, wq = _case(2700 + j, n, k, 64, oracle.F16)
+        ws.append(ctx.weight_prepare_mlx(fmt, words, s, z, pkg.F16, pkg.LAYOUT_STAF_BLOCKS)); wqs.append(wq)
+    x = act_rounded(kat.seeded_activations(2710, m, k), pkg.BF16, pkg)
+    xd = ctx.upload(act_to_device_array(x, pkg.BF16, pkg))
+    yds = [ctx.alloc(m * n * 4) for n in ns]
+    ctx.batched_qgemm(ws, xd, pkg.BF16, yds, pkg.F32, m); ctx.synchronize()
+    for yd, n, wq, w in zip(yds, ns, wqs, ws):
+        got = out_from_device(yd, pkg.F32, (m, n), pkg)
+        assert rel_l2(got, oracle.gemm_f64(wq, x)) < 1e-5
+        assert rel_l2(got, _run(ctx, pkg, w, x, m, n, pkg.F32, pkg.FLAG_FORCE_STREAM)) < 2e-6
         yd.free()
     xd.free()
     for w in ws:

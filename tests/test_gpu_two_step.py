@@ -117,7 +117,7 @@ def test_two_step_is_chosen_where_measured_faster_and_planned_as_two_steps(pkg, 
     assert [st.kernel_family for st in steps] == ["dequantToBFloat", "libraryGEMM"]
     assert steps[0].flops == 0 and steps[1].flops == 2 * 100 * n * k and steps[1].weight_bytes == n * k * 2
     assert not steps[0].used_fallback and not steps[1].used_fallback
-    assert [st.device_kernel for st in ws.plan_prefill_steps(64)] == ["qgemm_stream_q4_g64"]      # three to 96 rows
+    assert [st.device_kernel for st in ws.plan_prefill_steps(64)] == ["qgemm_stream_q4_g64"]      # nine to 96 rows
     assert [st.device_kernel for st in ws.plan_prefill_steps(12)] == ["qgemm_stream_q4_g64"]
     assert len(ws.plan_prefill_steps(2)) == 1 and ws.plan_prefill_steps(2)[0].device_kernel == "gemv_staf_q4_g64"
     assert len(ws.plan_prefill_steps(64, flags=pkg.FLAG_FORCE_SMALL_M)) == 1
