@@ -546,6 +546,26 @@ def main():
                      "kernel": plan.step(per_layer - 1)[0].device_kernel}
         log(f"4-launch step on STAF blocks in place: {staf_step['us_per_step']} us/step, {staf_step['GBps']} GB/s")
         plan.destroy()
+        # a batch of sequences on the blocks in place: the layer step at 8 and 32 rows (N(0,1) activations), as dispatched
+        staf_step["batch"] = {}
+        for m in (8, 32):
+            xm = {k: ctx.upload(oracle.bf16_from_f32(kat.seeded_activations(970 + m, m, k))) for k in (4096, 14336)}
+            ym = {name: ctx.alloc(m * n * 2) for name, n, _ in LAYER_SHAPES}
+            pl = pkg.DispatchPlan(ctx)
+            for L in layers:
+                pl.add_batched_linear([L["q"], L["k"], L["v"]], xm[4096], pkg.BF16, [ym["q"], ym["k"], ym["v"]], pkg.BF16, m)
+                pl.add_linear(L["o"], xm[4096], pkg.BF16, ym["o"], pkg.BF16, m)
+                pl.add_batched_linear([L["gate"], L["up"]], xm[4096], pkg.BF16, [ym["gate"], ym["up"]], pkg.BF16, m)
+                pl.add_linear(L["down"], xm[14336], pkg.BF16, ym["down"], pkg.BF16, m)
+            pl.encode(stream)
+            ctx.synchronize(stream)
+            ms_b = time_region(ctx, lambda i: pl.encode(stream), 32, stream) / len(layers)
+            staf_step["batch"][f"M={m}"] = {"us_per_step": round(ms_b * 1e3, 2), "GBps": round(layer_bytes / (ms_b * 1e-3) / 1e9, 1),
+                                            "down_kernel": layers[0]["down"].plan_prefill_steps(m, 14336)[0].device_kernel}
+            pl.destroy()
+            for b in list(xm.values()) + list(ym.values()):
+                b.free()
+        log(f"  batches on the blocks in place: {staf_step['batch']}")
         if not a.no_prefill:
             # prefill straight from the blocks: the gate projection over four rotating copies, as dispatched
             staf_step["prefill_gate_4096_14336"] = {}

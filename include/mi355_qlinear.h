@@ -279,10 +279,13 @@ MI355Q_API mi355q_status mi355q_qgemv(mi355q_context* ctx, void* stream, const m
  *   - small M (up to 8 rows; 16 on TILE16 records and on q4 / q8 planes; up to 32 in two launches where the
  *     next route does not read the weight): the GEMV-style decode kernels;
  *   - 17 to 96 bf16 rows, or 9 to 96 f16 rows, on 4-bit planes (groups of 64 or 128) and 8-bit planes (groups
- *     of 32, 64 or 128), and 9 to 96 rows of either type on the same formats left in STAF blocks: the
- *     streamed-weight kernel -- weights dequantised in registers straight into the
- *     matrix cores' operand (rounded to the activations' type), the activations alone staged in LDS; through
- *     mi355q_batched_qgemm two or three matrices share one launch;
+ *     of 32, 64 or 128), and on the same formats left in STAF blocks from 3, 5 or 9 rows by the size of the
+ *     matrix (mi355q_qgemv included): the streamed-weight kernel -- weights dequantised in registers
+ *     straight into the matrix cores' operand, the activations alone staged in LDS.  Up to 32 rows (groups of
+ *     64 or 128) it keeps the weights unrounded like the decode kernels; beyond, and with groups of 32, it
+ *     rounds them once to the activations' type.  Through mi355q_batched_qgemm two or three matrices share one
+ *     launch (whose split of K follows the launch's size: its fp32 sums may be ordered differently from those of
+ *     separate calls);
  *   - ONE fused kernel: code tiles are dequantised to bf16 in LDS and contracted on MFMA (the planes
  *     and TILE16 layouts, formats q4 g64/g128, q8 g32/g64, q6/q3/q2 g64, bf16 activations);
  *   - two dispatches, as the reference's second route: the whole matrix is dequantised to bf16 in a

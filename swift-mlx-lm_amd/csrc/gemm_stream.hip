@@ -18,6 +18,8 @@
 //     (XOR-swizzled 128-byte rows per K slice) two iterations ahead into the third of three LDS stages, copied
 //     global -> LDS directly; the multiplying wavefronts fetch weight words three or six iterations ahead and wait for nothing
 //     else; one barrier per iteration;
+//   * up to 32 rows (groups of whole K-tiles) the operand holds the codes themselves and scale and bias are applied to
+//     each K-tile's fp32 sums: unrounded weights, the decode kernels' arithmetic;
 //   * weights left in the reference's interleaved blocks are read in place: a lane's 32 codes lie in one block behind
 //     its (scale, zero) header (STAF payload, Sources/MetalCompiler/STAF/QuantizationFormat.swift:1121-1235);
 //   * two or three matrices that share the activations (q+k+v, gate+up) run as one launch, each owning whole
