@@ -298,3 +298,44 @@ def test_blocks_in_place_change_over_to_the_stream_kernel_by_size(pkg, ctx):
     xd.free()
     for w in ws:
         w.destroy()
+
+
+def test_stream_kernel_in_a_plan_replayed_as_a_graph(pkg, ctx):
+    """A shared launch (K split into parts: partial results in the context's scratch, a sum launch) and a single
+    projection on the kernel inside one plan, replayed eagerly and as a HIP graph with eager work between the replays:
+    every replay equals the first eager result bit for bit."""
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+    m, k = 40, 2048
+    ns = (192, 64, 64, 320)
+    ws = []
+    for i, n in enumerate(ns):
+        words, s, z, _ = _case(2800 + i, n, k, 64, oracle.BF16)
+        ws.append(ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, pkg.LAYOUT_PLANES))
+    xd = ctx.upload(oracle.bf16_from_f32(kat.seeded_activations(2810, m, k)))
+    ys = [ctx.alloc(m * n * 4) for n in ns]
+    stream = ctx.stream_create()
+    plan = pkg.DispatchPlan(ctx)
+    plan.add_batched_linear(ws[:3], xd, pkg.BF16, ys[:3], pkg.F32, m)
+    plan.add_linear(ws[3], xd, pkg.BF16, ys[3], pkg.F32, m)
+    assert ws[3].plan_prefill_steps(m)[0].device_kernel == "qgemm_stream_q4_g64"
+    plan.encode(stream); ctx.synchronize(stream)
+    eager = [y.download(np.float32) for y in ys]
+    assert all(np.all(np.isfinite(e)) for e in eager)
+
+    def scrub():
+        for y in ys:
+            ctx.fill(y, 0x7FC00000, stream)
+
+    plan.graph_build(stream)
+    for rep in range(4):
+        scrub(); plan.graph_launch(stream); ctx.synchronize(stream)
+        for y, want in zip(ys, eager):
+            assert np.array_equal(y.download(np.float32), want), f"graph replay {rep}"
+        ctx.qgemm(ws[0], xd, pkg.BF16, ys[0], pkg.F32, m, 0, 0, 0, stream)          # eager work between the replays
+        ctx.synchronize(stream)
+    plan.destroy()
+    for w in ws:
+        w.destroy()
+    xd.free()
+    for y in ys:
+        y.free()

@@ -157,7 +157,7 @@ def test_two_step_in_a_plan_replayed_as_a_graph(pkg, ctx):
     """Two projections on the route inside one plan (they share the context's scratch matrix, in stream order), replayed
     eagerly and as a HIP graph with eager work between the replays: every replay equals the first eager result."""
     fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
-    m = 96
+    m = 128                                       # beyond the 96 rows the streamed-weight kernel takes on blocks
     shapes = [(256, 512), (320, 1024)]
     ws, xs, ys = [], [], []
     for i, (n, k) in enumerate(shapes):
@@ -174,6 +174,7 @@ def test_two_step_in_a_plan_replayed_as_a_graph(pkg, ctx):
     plan = pkg.DispatchPlan(ctx)
     for i in range(2):
         plan.add_linear(ws[i], xs[i], pkg.BF16, ys[i], pkg.F32, m)
+        assert [st.kernel_family for st in ws[i].plan_prefill_steps(m)] == ["dequantToBFloat", "libraryGEMM"]
 
     def scrub():
         for y in ys:
