@@ -285,7 +285,7 @@ MI355Q_API mi355q_status mi355q_qgemv(mi355q_context* ctx, void* stream, const m
  *     64 or 128) it keeps the weights unrounded like the decode kernels; beyond, and with groups of 32, it
  *     rounds them once to the activations' type.  Through mi355q_batched_qgemm two or three matrices share one
  *     launch (whose split of K follows the launch's size: its fp32 sums may be ordered differently from those of
- *     separate calls);
+ *     separate calls); fp32 rows split into three bf16 rows each ride on it up to 32 fp32 rows;
  *   - ONE fused kernel: code tiles are dequantised to bf16 in LDS and contracted on MFMA (the planes
  *     and TILE16 layouts, formats q4 g64/g128, q8 g32/g64, q6/q3/q2 g64, bf16 activations);
  *   - two dispatches, as the reference's second route: the whole matrix is dequantised to bf16 in a

@@ -96,8 +96,7 @@ mi355q_status run_split_rows(mi355q_context* ctx, hipStream_t s, const mi355q_we
     float* const yp = (float*)((char*)ctx->split_buffer + xbytes);
     if (mi355q_status st = launch_split_rows_bf16(s, x, x_dtype, m, k, xs, xp, kp)) return st;
     const WView v = w->view();
-    if (!(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_SMALL_M)) && gemm_stream_chosen(v, MI355Q_BF16, parts * m, kp) &&
-        gemm_stream_unrounded(v, parts * m)) {
+    if (!(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_SMALL_M)) && split_rows_take_stream(v, x_dtype, m)) {
         if (mi355q_status st = launch_qgemm_stream(s, ctx, v, xp, MI355Q_BF16, yp, MI355Q_F32, parts * m, kp, n)) return st;
     } else if (mi355q_status st = run_small_m(ctx, s, w, xp, MI355Q_BF16, yp, MI355Q_F32, parts * m, kp, n, flags)) {
         return st;
@@ -118,10 +117,28 @@ bool split_rows_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_strid
     (void)x_stride;
     const uint32_t parts = split_rows_parts(x_dtype);
     if (!parts || (flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_TWO_STEP))) return false;
+    return split_rows_small_batch(w, parts, m) || split_rows_take_stream(w, x_dtype, m);
+}
+
+// The split rows fit the small-batch launches of a bf16 decode kernel.
+bool split_rows_small_batch(const WView& w, uint32_t parts, uint32_t m) {
     const uint32_t kp = split_rows_stride((uint32_t)w.k);
     if (!decode_kernel_reads(w, MI355Q_BF16, kp)) return false;
     const uint32_t rows = small_batch_rows(w, MI355Q_BF16, kp);
     return (uint64_t)parts * m <= (rows >= 16 ? 3 * rows : rows);
+}
+
+// The split rows go to the streamed-weight kernel: up to 32 of them with unrounded weights (blocks in place from three
+// fp32 rows' worth, where the dequantise-once route took 100-135 us; the planes from six fp32 rows, one launch instead
+// of two or three); more of them, with weights rounded to bf16, only where the small-batch launches do not serve and
+// the rows would otherwise take the dequantise-once route, which rounds the weights as well (from sixteen fp32 rows).
+bool split_rows_take_stream(const WView& w, int x_dtype, uint32_t m) {
+    const uint32_t parts = split_rows_parts(x_dtype);
+    if (!parts || (uint64_t)parts * m > kStreamMaxRows) return false;
+    const uint32_t pm = parts * m, kp = split_rows_stride((uint32_t)w.k);
+    if (!gemm_stream_chosen(w, MI355Q_BF16, pm, kp)) return false;
+    if (pm <= 32) return gemm_stream_unrounded(w, pm);
+    return !split_rows_small_batch(w, parts, m) && m >= kTwoStepMinRowsOtherwise;
 }
 
 mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_weight* w, const void* x, int x_dtype,

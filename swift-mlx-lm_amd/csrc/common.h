@@ -262,6 +262,8 @@ mi355q_status ensure_split_buffer(mi355q_context* ctx, size_t bytes);
 inline uint32_t split_rows_stride(uint32_t k) { return (k + 7u) & ~7u; }
 inline uint32_t split_rows_parts(int x_dtype) { return x_dtype == MI355Q_F32 ? 3u : 0u; }
 bool split_rows_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride, uint32_t flags);
+bool split_rows_small_batch(const WView& w, uint32_t parts, uint32_t m);
+bool split_rows_take_stream(const WView& w, int x_dtype, uint32_t m);
 bool gemm_mfma_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
 mi355q_status launch_qgemm_mfma(hipStream_t s, mi355q_context* ctx, const WView& w,
                                 const void* x, int x_dtype, void* y, int y_dtype, uint32_t m,

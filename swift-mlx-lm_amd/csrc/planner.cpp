@@ -47,6 +47,20 @@ void plan_small_m(const mi355q_weight* w, uint32_t m, int x_dtype, uint32_t x_st
                   mi355q_step* s) {
     const WView v = w->view();
     const bool forced = flags & MI355Q_FLAG_FORCE_GENERIC;
+    if (split_rows_chosen(v, x_dtype, m, x_stride, flags) && !(flags & MI355Q_FLAG_FORCE_SMALL_M) &&
+        split_rows_take_stream(v, x_dtype, m)) {
+        // fp32 rows as three bf16 rows each on the streamed-weight kernel, then the sum of the partial results
+        const uint32_t pm = split_rows_parts(x_dtype) * m;
+        const StreamLaunchShape g = gemm_stream_shape(w->ctx, pm, (uint32_t)w->n, (uint32_t)w->k);
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "split_f32_bf16x3+qgemm_stream_q%u_g%u", (unsigned)w->fmt.bits,
+                      w->fmt.group_size);
+        s->grid[0] = g.row_blocks;
+        s->grid[1] = g.parts;
+        s->block[0] = 768;
+        s->lds_bytes = g.lds_bytes;
+        s->rows_per_workgroup = 64;
+        return;
+    }
     if (split_rows_chosen(v, x_dtype, m, x_stride, flags)) {
         // fp32 rows as three bf16 rows each on the bf16 decode kernel, then the sum of the partial results
         plan_small_m(w, split_rows_parts(x_dtype) * m, MI355Q_BF16, split_rows_stride((uint32_t)w->k), flags, s);

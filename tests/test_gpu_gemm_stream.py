@@ -339,3 +339,37 @@ def test_stream_kernel_in_a_plan_replayed_as_a_graph(pkg, ctx):
     xd.free()
     for y in ys:
         y.free()
+
+
+@pytest.mark.parametrize("layout_name", ["planes", "blocks"])
+def test_fp32_rows_ride_on_the_stream_kernel(pkg, ctx, layout_name):
+    """fp32 activations (the reference's prefill type) split exactly into three bf16 rows each: up to ten fp32 rows (32
+    bf16 rows) the streamed-weight kernel keeps the weights unrounded; from sixteen fp32 rows, where the rows would
+    otherwise take the dequantise-once route with bf16 weights, it takes up to 32 of them with bf16 weights.  Eleven
+    to fifteen rows keep their earlier routes (unrounded weights)."""
+    layout = pkg.LAYOUT_PLANES if layout_name == "planes" else pkg.LAYOUT_STAF_BLOCKS
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+    n, k = 300, 2048
+    words, s, z, wq = _case(2900, n, k, 64, oracle.F16)
+    w = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.F16, layout)
+    wb = oracle.bf16_to_f32(oracle.bf16_from_f32(wq)).reshape(wq.shape)
+    for m in (3, 6, 10, 13, 16, 25, 32):
+        say(f"fp32 rows {layout_name} M={m}")
+        x = kat.seeded_activations(2910 + m, m, k)
+        xd = ctx.upload(x)
+        yd = ctx.alloc(m * n * 4)
+        ctx.qgemm(w, xd, pkg.F32, yd, pkg.F32, m); ctx.synchronize()
+        got = yd.download(np.float32, (m, n))
+        kernel = w.plan_prefill_steps(m, x_dtype=pkg.F32)[0].device_kernel
+        on_stream = kernel == "split_f32_bf16x3+qgemm_stream_q4_g64"
+        if m <= 10:
+            assert on_stream == (layout_name == "blocks" or m >= 6), (m, kernel)
+        elif m >= 16:
+            assert on_stream == (layout_name == "blocks" or m > 16), (m, kernel)
+        else:
+            assert not on_stream, (m, kernel)
+        rounded = on_stream and 3 * m > 32
+        want = oracle.gemm_f64(wb if rounded else wq, x)
+        assert rel_l2(got, want) < (2e-6 if not rounded else 1e-5), (m, kernel, rel_l2(got, want))
+        xd.free(); yd.free()
+    w.destroy()
