@@ -116,11 +116,11 @@ def test_stream_kernel_refuses_what_it_does_not_read(pkg, ctx):
     ws = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, pkg.LAYOUT_TILE16)
     with pytest.raises(pkg.MI355QError):
         _run(ctx, pkg, ws, x[:20], 20, 64, pkg.F32, pkg.FLAG_FORCE_STREAM)     # tile records
-    fmt8 = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(6, 64)
-    words8, s8, z8 = oracle.quantize_affine(kat.seeded_weights(1501, 64, 128), 6, 64, oracle.BF16)
+    fmt8 = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(6, 16)
+    words8, s8, z8 = oracle.quantize_affine(kat.seeded_weights(1501, 64, 128), 6, 16, oracle.BF16)
     w8 = ctx.weight_prepare_mlx(fmt8, words8, s8, z8, pkg.BF16, pkg.LAYOUT_PLANES)
     with pytest.raises(pkg.MI355QError):
-        _run(ctx, pkg, w8, x[:20], 20, 64, pkg.F32, pkg.FLAG_FORCE_STREAM)     # 6-bit codes
+        _run(ctx, pkg, w8, x[:20], 20, 64, pkg.F32, pkg.FLAG_FORCE_STREAM)     # groups of 16: two in a lane's 32 codes
     for t in (w, ws, w8):
         t.destroy()
 
@@ -373,3 +373,26 @@ def test_fp32_rows_ride_on_the_stream_kernel(pkg, ctx, layout_name):
         assert rel_l2(got, want) < (2e-6 if not rounded else 1e-5), (m, kernel, rel_l2(got, want))
         xd.free(); yd.free()
     w.destroy()
+
+
+@pytest.mark.parametrize("bits", [2, 3, 5, 6])
+def test_stream_kernel_other_widths(pkg, ctx, bits):
+    """2-, 3-, 5- and 6-bit codes in groups of 64 (fields that straddle words included): planes and blocks, bf16 and f16
+    rows; unrounded weights up to 32 rows, rounded to the activations' type beyond; the same bits from both layouts."""
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(bits, 64)
+    for i, (m, n, k) in enumerate([(5, 64, 128), (20, 300, 1024), (40, 1000, 384), (96, 130, 2176), (33, 70, 14336)]):
+        words, s, z, wq = _case(3000 + 10 * bits + i, n, k, 64, oracle.F16, bits=bits)
+        wp = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.F16, pkg.LAYOUT_PLANES)
+        wb = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.F16, pkg.LAYOUT_STAF_BLOCKS)
+        for x_dtype in (pkg.BF16, pkg.F16):
+            say(f"stream q{bits} g64 M={m} {k}->{n} x {x_dtype}")
+            x = act_rounded(kat.seeded_activations(3100 + i, m, k), x_dtype, pkg)
+            got = _run(ctx, pkg, wp, x, m, n, pkg.F32, pkg.FLAG_FORCE_STREAM, ypad=i % 2, xpad=8 * (i % 2), x_dtype=x_dtype)
+            bar = 1e-5 if m <= 32 else 2.5e-3 if x_dtype == pkg.BF16 else 4e-4
+            assert rel_l2(got, oracle.gemm_f64(wq, x)) < bar, (m, rel_l2(got, oracle.gemm_f64(wq, x)))
+            from_blocks = _run(ctx, pkg, wb, x, m, n, pkg.F32, pkg.FLAG_FORCE_STREAM, x_dtype=x_dtype)
+            assert np.array_equal(from_blocks, got)
+            if m >= 17:
+                assert wp.plan_prefill_steps(m, x_dtype=x_dtype)[0].device_kernel == f"qgemm_stream_q{bits}_g64"
+                assert np.array_equal(_run(ctx, pkg, wp, x, m, n, pkg.F32, 0, x_dtype=x_dtype), got)
+        wp.destroy(); wb.destroy()
