@@ -212,10 +212,19 @@ uint32_t small_batch_limit(const WView& w, int x_dtype, uint32_t x_stride) {
         // Its cost has a floor of about 10 us (K parts and their sum launch on matrices of few rows), so smaller
         // matrices change over later: 4096 -> 4096 at four rows 10.6 against 8.8 us, at six 10.6 against 14.5;
         // 4096 -> 1024 at eight rows 9.8 against 10.0.
-        if (w.layout == MI355Q_LAYOUT_STAF_BLOCKS && gemm_stream_unrounded(w, 3)) {
+        const bool other_width = w.bits != 4 && w.bits != 8;
+        if (w.layout == MI355Q_LAYOUT_STAF_BLOCKS && !other_width && gemm_stream_unrounded(w, 3)) {
             const uint64_t codes = (uint64_t)w.n * w.k;
             const uint32_t first = codes >= kStreamBlocksLargeCodes ? 3 : codes >= kStreamBlocksMediumCodes ? 5 : rows + 1;
             return gemv_staf_eligible(w, x_dtype, 1, x_stride) ? first - 1 : 0;
+        }
+        // 2, 3, 5 and 6 bits (planes and blocks): the decode kernels take four rows a launch there, so a fifth row is a
+        // second launch (4096 -> 14336 q6 g64: 19.4 us at four rows, 29.9 at five, 38.5 at eight, 77.7 at sixteen; the
+        // streamed kernel 20.6-21.1 throughout; 4096 -> 4096: 8.4 / 12.9 / 16.2 / 31.8 against 12.3-12.8)
+        if (other_width && gemm_stream_unrounded(w, 5)) {
+            const uint64_t codes = (uint64_t)w.n * w.k;
+            if (w.layout == MI355Q_LAYOUT_STAF_BLOCKS && !gemv_staf_eligible(w, x_dtype, 1, x_stride)) return 0;
+            return codes >= kStreamBlocksMediumCodes ? 4 : rows;
         }
         return rows;
     }

@@ -72,8 +72,8 @@ def test_f32_rows_full_mantissas(pkg, ctx, layout, bits, group, most):
                     assert np.array_equal(run_f32(ctx, pkg, w, x), got)
             else:
                 # beyond the small-batch launches: the split rows on the streamed-weight kernel where it reads the weight
-                # (4- / 8-bit planes and blocks: unrounded weights up to 32 bf16 rows, bf16 weights beyond), else another route
-                streams = bits in (4, 8) and layout != "tile16"
+                # (planes and blocks of the widths it takes: unrounded weights up to 32 bf16 rows, bf16 weights beyond), else another route
+                streams = layout != "tile16" and (bits in (4, 8) or group == 64)     # what the streamed-weight kernel reads
                 assert st.device_kernel.startswith("split_f32_bf16x3+qgemm_stream") == streams, st.device_kernel
                 if streams and 3 * m <= 32:
                     assert rel_l2(got, want) <= 1e-5, (m, rel_l2(got, want))
