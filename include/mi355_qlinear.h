@@ -279,8 +279,8 @@ MI355Q_API mi355q_status mi355q_qgemv(mi355q_context* ctx, void* stream, const m
  *   - small M (up to 8 rows; 16 on TILE16 records and on q4 / q8 planes; up to 32 in two launches where the
  *     next route does not read the weight): the GEMV-style decode kernels;
  *   - 17 to 96 bf16 rows, or 9 to 96 f16 rows, on 4-bit planes (groups of 64 or 128) and 8-bit planes (groups
- *     of 32, 64 or 128), and on the same formats left in STAF blocks from 3, 5 or 9 rows by the size of the
- *     matrix (mi355q_qgemv included): the streamed-weight kernel -- weights dequantised in registers
+ *     of 32, 64 or 128), on the same formats left in STAF blocks from 3, 5 or 9 rows by the size of the
+ *     matrix, and on 2-, 3-, 5- and 6-bit codes in groups of 64 (planes and blocks) from 5 rows (mi355q_qgemv included): the streamed-weight kernel -- weights dequantised in registers
  *     straight into the matrix cores' operand, the activations alone staged in LDS.  Up to 32 rows (groups of
  *     64 or 128) it keeps the weights unrounded like the decode kernels; beyond, and with groups of 32, it
  *     rounds them once to the activations' type.  Through mi355q_batched_qgemm two or three matrices share one
