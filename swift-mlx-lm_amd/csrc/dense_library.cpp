@@ -13,6 +13,7 @@
 #include <dlfcn.h>
 #include <hipblaslt/hipblaslt.h>
 
+#include <cmath>
 #include <mutex>
 #include <vector>
 
@@ -97,6 +98,7 @@ struct DenseLibrary {
     const Api* api;
     hipblasLtHandle_t handle;
     std::vector<Problem> problems;
+    float* check;                                     // two device cells: the sums a candidate's result is checked by
 };
 
 namespace {
@@ -110,8 +112,35 @@ DenseLibrary* library_of(mi355q_context* ctx) {
         ctx->dense_library_failed = true;
         return nullptr;
     }
-    ctx->dense_library = new DenseLibrary{a, h, {}};
+    float* check = nullptr;
+    if (hipMalloc((void**)&check, 2 * sizeof(float)) != hipSuccess) check = nullptr;      // without it no candidate is timed
+    ctx->dense_library = new DenseLibrary{a, h, {}, check};
     return ctx->dense_library;
+}
+
+// Two sums over a result matrix, a position-weighted one and one of magnitudes: what a timed candidate's result is
+// compared by with the result of the algorithm the library's heuristic ranks first.
+__global__ __launch_bounds__(256) void dense_result_sums_kernel(const void* __restrict__ y, int y_dtype, uint32_t m, uint32_t n,
+                                                               uint32_t ys, float* __restrict__ out) {
+    float weighted = 0.f, magnitude = 0.f;
+    const size_t total = (size_t)m * n;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+        const size_t row = i / n, col = i - row * n, at = row * ys + col;
+        float v;
+        if (y_dtype == MI355Q_F32) v = ((const float*)y)[at];
+        else if (y_dtype == MI355Q_BF16) v = __uint_as_float((uint32_t)((const uint16_t*)y)[at] << 16);
+        else v = (float)((const _Float16*)y)[at];
+        weighted += v * (float)(1 + (i % 7));
+        magnitude += v < 0.f ? -v : v;
+    }
+    __shared__ float part[2][256];
+    part[0][threadIdx.x] = weighted; part[1][threadIdx.x] = magnitude;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) { part[0][threadIdx.x] += part[0][threadIdx.x + w]; part[1][threadIdx.x] += part[1][threadIdx.x + w]; }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) { atomicAdd(out, part[0][0]); atomicAdd(out + 1, part[1][0]); }
 }
 
 Problem* find_problem(DenseLibrary* lib, int ab_dtype, uint32_t m, uint32_t n, uint32_t k, uint32_t xs, uint32_t ys,
@@ -176,9 +205,10 @@ mi355q_status dense_library_gemm(hipStream_t s, mi355q_context* ctx, int ab_dtyp
     if (!p->timed && p->candidates > 1 && capture == hipStreamCaptureStatusNone && !accumulate) {
         p->timed = true;
         hipEvent_t e0 = nullptr, e1 = nullptr;
-        if (hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
+        if (lib->check && hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
             float best = 0.f;
             int best_i = -1;
+            float reference[2] = {0.f, 0.f};
             for (int i = 0; i < p->candidates; i++) {
                 bool ran = true;
                 float ms = 0.f;
@@ -188,8 +218,23 @@ mi355q_status dense_library_gemm(hipStream_t s, mi355q_context* ctx, int ab_dtyp
                                            &p->ranked[i], workspace, kDenseLibraryWorkspace, s) == HIPBLAS_STATUS_SUCCESS;
                 }
                 if (!ran) continue;
-                if (hipEventRecord(e1, s) != hipSuccess || hipEventSynchronize(e1) != hipSuccess ||
+                if (hipEventRecord(e1, s) != hipSuccess) continue;
+                // A candidate is kept only if its result agrees with that of the heuristic's first algorithm: on small or
+                // odd shapes some of the ranked algorithms have returned wrong matrices (M = N = 17, K = 2176 in bf16).
+                float sums[2] = {0.f, 0.f};
+                if (hipMemsetAsync(lib->check, 0, sizeof sums, s) != hipSuccess) continue;
+                const size_t total = (size_t)m * n;
+                const unsigned blocks = (unsigned)(total / 256 + 1 < 1024 ? total / 256 + 1 : 1024);
+                dense_result_sums_kernel<<<dim3(blocks), dim3(256), 0, s>>>(y, y_dtype, m, n, y_stride, lib->check);
+                if (hipGetLastError() != hipSuccess || hipStreamSynchronize(s) != hipSuccess ||
+                    hipMemcpy(sums, lib->check, sizeof sums, hipMemcpyDeviceToHost) != hipSuccess ||
                     hipEventElapsedTime(&ms, e0, e1) != hipSuccess) continue;
+                if (i == 0) { reference[0] = sums[0]; reference[1] = sums[1]; }
+                const float slack = 2e-3f * reference[1] + 1e-30f;
+                const bool agrees = i == 0 || (sums[0] == sums[0] && sums[1] == sums[1] &&
+                                               std::fabs(sums[0] - reference[0]) <= 7.f * slack &&
+                                               std::fabs(sums[1] - reference[1]) <= slack);
+                if (!agrees) continue;
                 if (best_i < 0 || ms < best) { best = ms; best_i = i; }
             }
             if (best_i >= 0) p->algo = p->ranked[best_i];
@@ -213,6 +258,7 @@ void dense_library_release(mi355q_context* ctx) {
         if (p.b) lib->api->layout_destroy(p.b);
         if (p.c) lib->api->layout_destroy(p.c);
     }
+    if (lib->check) (void)hipFree(lib->check);
     lib->api->destroy(lib->handle);
     delete lib;
     ctx->dense_library = nullptr;

@@ -248,3 +248,27 @@ def test_two_step_f16_and_f32_activations(pkg, ctx, x_dtype_name, y_dtype_names)
                 assert_within_tolerance(out_from_device(yd, y_dtype, (m, n), pkg), want, f"{x_dtype_name}->{yname} M={m}")
                 xd.free(); yd.free()
         w.destroy()
+
+
+def test_timed_library_candidates_are_checked_against_the_first(pkg):
+    """The first eager call of a problem times the library's ranked algorithms; one of them has returned a wrong matrix
+    on a small odd problem (M = N = 17, K = 2176, bf16), so a candidate is kept only if its result agrees with that of
+    the heuristic's first algorithm.  Fresh contexts time the candidates anew: every one must give the right product."""
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(3, 16)
+    m, n, k = 17, 17, 2176
+    w32 = kat.seeded_weights(3700, n, k)
+    words, s, z = oracle.quantize_affine(w32, 3, 16, oracle.F16)
+    wq = bf16_round(oracle.dequant_planes_f32(3, 16, n, k, words, s, z, oracle.F16))
+    x = act_rounded(kat.seeded_activations(3701, m, k), pkg.BF16, pkg)
+    want = oracle.gemm_f64(wq, x)
+    for attempt in range(4):
+        c = pkg.Context(0)
+        w = c.weight_prepare_mlx(fmt, words, s, z, pkg.F16, pkg.LAYOUT_STAF_BLOCKS)
+        assert [st.kernel_family for st in w.plan_prefill_steps(m)] == ["dequantToBFloat", "libraryGEMM"]
+        xd = c.upload(act_to_device_array(x, pkg.BF16, pkg)); yd = c.alloc(m * n * 4)
+        for call in range(2):                       # the call that times the candidates, and one with the algorithm kept
+            c.fill(yd, 0x7FC00000)
+            c.qgemm(w, xd, pkg.BF16, yd, pkg.F32, m); c.synchronize()
+            got = yd.download(np.float32, (m, n))
+            assert_within_tolerance(got, want, f"context {attempt}, call {call}")
+        xd.free(); yd.free(); w.destroy(); c.close()
