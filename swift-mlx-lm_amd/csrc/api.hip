@@ -306,12 +306,43 @@ bool gemm_two_step_serves(mi355q_context* ctx, const WView& w, int x_dtype, int 
                           uint32_t y_stride) {
     const uint32_t n = (uint32_t)w.n, k = (uint32_t)w.k;
     switch (two_step_form(x_dtype, y_dtype, m, w, x_stride)) {
+    // (results of a padded stride are computed densely in scratch: the library is asked for stride N)
     case TwoStepForm::kExactF32:
-        return dense_library_serves(ctx, MI355Q_F32, m, n, k, x_dtype == MI355Q_F32 ? x_stride : k,
-                                    y_dtype == MI355Q_F32 ? y_stride : n, MI355Q_F32);
-    case TwoStepForm::kSplitF32: return dense_library_serves(ctx, MI355Q_BF16, m, n, k, k, y_stride, MI355Q_F32);
-    default: return dense_library_serves(ctx, x_dtype, m, n, k, x_stride, y_stride, y_dtype);
+        return dense_library_serves(ctx, MI355Q_F32, m, n, k, x_dtype == MI355Q_F32 ? x_stride : k, n, MI355Q_F32);
+    case TwoStepForm::kSplitF32: return dense_library_serves(ctx, MI355Q_BF16, m, n, k, k, n, MI355Q_F32);
+    default: return dense_library_serves(ctx, x_dtype, m, n, k, x_stride, n, y_dtype);
     }
+}
+
+// The library's product into a result whose row stride is not N: with long K (14336; not with 4224 or less) every
+// algorithm the library offers has returned a wrong matrix into such a result (M = 128, N = 64 or 2056, fp32 and bf16,
+// stride N + 5 or N + 8), while results of stride N are right.  So a padded result is computed densely in scratch and
+// copied row by row.  `free_ws` is scratch of dense_result_bytes() + kDenseLibraryWorkspace bytes; `x_second`, when
+// given, is a second activation matrix whose product is added to the first's (the low halves of split fp32 rows).
+size_t dense_result_bytes(uint32_t m, uint32_t n, uint32_t y_stride, int y_dtype) {
+    return y_stride == n ? 0 : (((size_t)m * n * (y_dtype == MI355Q_F32 ? 4 : 2)) + 255) & ~(size_t)255;
+}
+
+mi355q_status dense_gemm_into(hipStream_t s, mi355q_context* ctx, int ab_dtype, const void* x, const void* w_dense, void* y,
+                              int y_dtype, uint32_t m, uint32_t n, uint32_t k, uint32_t x_stride, uint32_t y_stride,
+                              char* free_ws, const void* x_second = nullptr) {
+    const size_t tmp_bytes = dense_result_bytes(m, n, y_stride, y_dtype);
+    void* const out = tmp_bytes ? (void*)free_ws : y;
+    const uint32_t out_stride = tmp_bytes ? n : y_stride;
+    void* const lib_ws = free_ws + tmp_bytes;
+    if (mi355q_status st = dense_library_gemm(s, ctx, ab_dtype, x, w_dense, out, y_dtype, m, n, k, x_stride, out_stride, lib_ws,
+                                              false)) return st;
+    if (x_second)
+        if (mi355q_status st = dense_library_gemm(s, ctx, ab_dtype, x_second, w_dense, out, y_dtype, m, n, k, x_stride, out_stride,
+                                                  lib_ws, true)) return st;
+    if (!tmp_bytes) return MI355Q_OK;
+    const size_t ysz = y_dtype == MI355Q_F32 ? 4 : 2;
+    for (uint32_t m0 = 0; m0 < m; m0 += 65535u) {
+        const uint32_t rows = m - m0 < 65535u ? m - m0 : 65535u;
+        if (mi355q_status st = launch_convert_rows(s, (const char*)out + (size_t)m0 * n * ysz, y_dtype, n,
+                                                   (char*)y + (size_t)m0 * y_stride * ysz, y_dtype, y_stride, rows, n)) return st;
+    }
+    return MI355Q_OK;
 }
 
 // The dense matrix sits at the head of the context's scratch, converted activations and results behind it, the
@@ -325,7 +356,8 @@ mi355q_status launch_qgemm_two_step(hipStream_t s, mi355q_context* ctx, const WV
         const bool widen = x_dtype != MI355Q_F32, narrow = y_dtype != MI355Q_F32;
         const size_t wbytes = round256((size_t)n * k * 4), xbytes = widen ? round256((size_t)m * k * 4) : 0;
         const size_t ybytes = narrow ? round256((size_t)m * n * 4) : 0;
-        if (mi355q_status st = ensure_workspace(ctx, wbytes + xbytes + ybytes + kDenseLibraryWorkspace)) return st;
+        const size_t dense_y = narrow ? 0 : dense_result_bytes(m, n, y_stride, MI355Q_F32);
+        if (mi355q_status st = ensure_workspace(ctx, wbytes + xbytes + ybytes + dense_y + kDenseLibraryWorkspace)) return st;
         char* const base = (char*)ctx->workspace;
         float* const w32 = (float*)base;
         float* const x32 = widen ? (float*)(base + wbytes) : (float*)const_cast<void*>(x);
@@ -333,35 +365,32 @@ mi355q_status launch_qgemm_two_step(hipStream_t s, mi355q_context* ctx, const WV
         if (mi355q_status st = launch_dequant_f32(s, w, w32)) return st;
         if (widen)
             if (mi355q_status st = launch_convert_rows(s, x, x_dtype, x_stride, x32, MI355Q_F32, k, m, k)) return st;
-        if (mi355q_status st = dense_library_gemm(s, ctx, MI355Q_F32, x32, w32, y32, MI355Q_F32, m, n, k, widen ? k : x_stride,
-                                                  narrow ? n : y_stride, base + wbytes + xbytes + ybytes)) return st;
+        if (mi355q_status st = dense_gemm_into(s, ctx, MI355Q_F32, x32, w32, y32, MI355Q_F32, m, n, k, widen ? k : x_stride,
+                                               narrow ? n : y_stride, base + wbytes + xbytes + ybytes)) return st;
         if (narrow) return launch_convert_rows(s, y32, MI355Q_F32, n, y, y_dtype, y_stride, m, n);
         return MI355Q_OK;
     }
     if (form == TwoStepForm::kSplitF32) {
         const size_t wbytes = round256((size_t)n * k * 2), xbytes = round256((size_t)m * k * 2);
-        if (mi355q_status st = ensure_workspace(ctx, wbytes + 2 * xbytes + kDenseLibraryWorkspace)) return st;
+        if (mi355q_status st = ensure_workspace(ctx, wbytes + 2 * xbytes + dense_result_bytes(m, n, y_stride, MI355Q_F32) +
+                                                         kDenseLibraryWorkspace)) return st;
         char* const base = (char*)ctx->workspace;
         uint16_t* const w_bf16 = (uint16_t*)base;
         uint16_t* const hi = (uint16_t*)(base + wbytes);
         uint16_t* const lo = (uint16_t*)(base + wbytes + xbytes);
-        void* const lib_ws = base + wbytes + 2 * xbytes;
         if (mi355q_status st = launch_dequant_bf16(s, w, w_bf16)) return st;
         if (mi355q_status st = launch_split_f32_bf16x2(s, (const float*)x, m, k, x_stride, hi, lo)) return st;
-        if (mi355q_status st = dense_library_gemm(s, ctx, MI355Q_BF16, hi, w_bf16, y, MI355Q_F32, m, n, k, k, y_stride, lib_ws,
-                                                  false)) return st;
-        return dense_library_gemm(s, ctx, MI355Q_BF16, lo, w_bf16, y, MI355Q_F32, m, n, k, k, y_stride, lib_ws, true);
+        return dense_gemm_into(s, ctx, MI355Q_BF16, hi, w_bf16, y, MI355Q_F32, m, n, k, k, y_stride, base + wbytes + 2 * xbytes, lo);
     }
     const size_t esz = x_dtype == MI355Q_F32 ? 4 : 2;
     const size_t dense = round256((size_t)n * k * esz);
-    if (mi355q_status st = ensure_workspace(ctx, dense + kDenseLibraryWorkspace)) return st;
+    if (mi355q_status st = ensure_workspace(ctx, dense + dense_result_bytes(m, n, y_stride, y_dtype) + kDenseLibraryWorkspace)) return st;
     void* const w_dense = ctx->workspace;
     const mi355q_status st = x_dtype == MI355Q_BF16 ? launch_dequant_bf16(s, w, (uint16_t*)w_dense)
                            : x_dtype == MI355Q_F16 ? launch_dequant_f16(s, w, (uint16_t*)w_dense)
                                                    : launch_dequant_f32(s, w, (float*)w_dense);
     if (st != MI355Q_OK) return st;
-    return dense_library_gemm(s, ctx, x_dtype, x, w_dense, y, y_dtype, m, n, k, x_stride, y_stride,
-                              (char*)ctx->workspace + dense);
+    return dense_gemm_into(s, ctx, x_dtype, x, w_dense, y, y_dtype, m, n, k, x_stride, y_stride, (char*)ctx->workspace + dense);
 }
 
 // Two or three projections that read the same activations (q+k+v, gate+up).  For M <= 8 on the
@@ -562,10 +591,10 @@ mi355q_status mi355q_gemm_bf16(mi355q_context* ctx, void* stream, const void* a_
     // library's own matrix-core kernel
     if (a_dtype == MI355Q_BF16 && m >= kDenseLibraryMinRows && k % 8 == 0 && a_row_stride % 8 == 0 &&
         (uintptr_t)a_dev % 16 == 0 && (uintptr_t)b_bf16_dev % 16 == 0 &&
-        dense_library_serves(ctx, MI355Q_BF16, m, n, k, a_row_stride, c_row_stride, c_dtype)) {
-        if (mi355q_status st = ensure_workspace(ctx, kDenseLibraryWorkspace)) return st;
-        return dense_library_gemm((hipStream_t)stream, ctx, MI355Q_BF16, a_dev, b_bf16_dev, c_dev, c_dtype, m, n, k,
-                                  a_row_stride, c_row_stride, ctx->workspace);
+        dense_library_serves(ctx, MI355Q_BF16, m, n, k, a_row_stride, n, c_dtype)) {
+        if (mi355q_status st = ensure_workspace(ctx, mi355q::dense_result_bytes(m, n, c_row_stride, c_dtype) + kDenseLibraryWorkspace)) return st;
+        return mi355q::dense_gemm_into((hipStream_t)stream, ctx, MI355Q_BF16, a_dev, b_bf16_dev, c_dev, c_dtype, m, n, k,
+                                       a_row_stride, c_row_stride, (char*)ctx->workspace);
     }
     return launch_gemm_bf16_mfma((hipStream_t)stream, ctx, a_dev, a_dtype, (const uint16_t*)b_bf16_dev, c_dev,
                                  c_dtype, m, n, k, a_row_stride, c_row_stride);

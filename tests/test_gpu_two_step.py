@@ -14,7 +14,7 @@ import pytest
 
 import kat
 import oracle
-from gpu_util import Case, act_rounded, act_to_device_array, assert_within_tolerance, out_from_device, seeded_case
+from gpu_util import rel_l2, Case, act_rounded, act_to_device_array, assert_within_tolerance, out_from_device, seeded_case
 
 pytestmark = pytest.mark.gpu
 
@@ -272,3 +272,47 @@ def test_timed_library_candidates_are_checked_against_the_first(pkg):
             got = yd.download(np.float32, (m, n))
             assert_within_tolerance(got, want, f"context {attempt}, call {call}")
         xd.free(); yd.free(); w.destroy(); c.close()
+
+
+@pytest.mark.parametrize("x_dtype_name", ["BF16", "F16", "F32"])
+def test_library_route_with_padded_result_rows_and_long_k(pkg, ctx, x_dtype_name):
+    """Results whose row stride is not N, with K = 14336: the library has returned wrong matrices into such results
+    (every algorithm it offers, strides N + 5 and N + 8 alike), so the route computes a padded result densely in
+    scratch and copies it row by row.  All three forms of the route, the dense entry point, canary behind the rows."""
+    x_dtype = getattr(pkg, x_dtype_name)
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+    n, k, m = 72, 14336, 128
+    words, s, z, wq = seeded_case(3800, n, k, 4, 64)
+    w = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, pkg.LAYOUT_PLANES)
+    w_round = wq.astype(np.float16).astype(np.float32) if x_dtype == pkg.F16 else bf16_round(wq)
+    x = act_rounded(kat.seeded_activations(3801, m, k), x_dtype, pkg)
+    want = oracle.gemm_f64(w_round, x)
+    xd = ctx.upload(act_to_device_array(x, x_dtype, pkg))
+    for ys in (n, n + 5, n + 8):
+        for y_dtype in ((pkg.F32,) if x_dtype == pkg.F32 else (pkg.F32, x_dtype)):
+            say(f"padded result rows: x {x_dtype_name} y {y_dtype} stride {ys}")
+            ysz = 4 if y_dtype == pkg.F32 else 2
+            yd = ctx.alloc((m * ys * ysz + 3) // 4 * 4)
+            ctx.fill(yd, 0x7FC00000 if ysz == 4 else 0x7FC07FC0)
+            ctx.qgemm(w, xd, x_dtype, yd, y_dtype, m, 0, ys, pkg.FLAG_FORCE_TWO_STEP); ctx.synchronize()
+            raw = yd.download(np.float32 if ysz == 4 else np.uint16)[: m * ys].reshape(m, ys)
+            got = raw if ysz == 4 else (oracle.bf16_to_f32(raw).reshape(m, ys) if y_dtype == pkg.BF16 else raw.view(np.float16).astype(np.float32))
+            assert np.all(np.isnan(got[:, n:])), "padding behind the rows overwritten"
+            if ysz == 4:
+                assert_within_tolerance(got[:, :n], want, f"x {x_dtype_name} y {y_dtype} stride {ys}")
+            else:                                     # a 16-bit result adds its own rounding (2^-9 for bf16)
+                assert rel_l2(got[:, :n], want) <= 3e-3, (x_dtype_name, y_dtype, ys)
+            yd.free()
+    if x_dtype == pkg.BF16:                        # the dense entry point on its own
+        dense = ctx.alloc(n * k * 2)
+        ctx.dequant_bf16(w, dense)
+        for ys in (n + 5, n + 8):
+            cd = ctx.alloc(m * ys * 4)
+            ctx.fill(cd, 0x7FC00000)
+            ctx.gemm_bf16(xd, pkg.BF16, dense, cd, pkg.F32, m, n, k, 0, ys); ctx.synchronize()
+            got = cd.download(np.float32, (m, ys))
+            assert np.all(np.isnan(got[:, n:]))
+            assert_within_tolerance(got[:, :n], want, f"gemm_bf16 stride {ys}")
+            cd.free()
+        dense.free()
+    xd.free(); w.destroy()
