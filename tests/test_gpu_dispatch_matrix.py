@@ -63,7 +63,10 @@ def _one_case(pkg, ctx, rng, idx):
     want = oracle.gemm_f64(wq, x)
     assert np.all(np.isfinite(got)), what
     tol16 = {pkg.F32: 0.0, pkg.BF16: 2.0 ** -8, pkg.F16: 2.0 ** -11}[y_dtype]
-    r = rel_l2(got, want)
+    # relative to the result, with a floor for results that are the small remainder of large terms (one output column
+    # whose products cancel: fp32 sums of |w x| = 12.7 leave an error of 3e-7 on a result of 8e-4)
+    terms = np.abs(wq.astype(np.float64)) @ np.abs(x.astype(np.float64)).T
+    r = float(np.sqrt(((got - want) ** 2).sum()) / (np.sqrt((want ** 2).sum()) + 1e-6 * np.sqrt((terms ** 2).sum())))
     assert r <= 2.5e-3 + tol16, f"{what}: rel-L2 {r:.3e}"
     assert float(np.max(np.abs(got - want))) <= 2e-2 + tol16 * float(np.max(np.abs(want))), what
     w.destroy(); xd.free(); yd.free()
