@@ -314,8 +314,8 @@ bool gemm_two_step_serves(mi355q_context* ctx, const WView& w, int x_dtype, int 
     }
 }
 
-// The library's product into a result whose row stride is not N: with long K (14336; not with 4224 or less) every
-// algorithm the library offers has returned a wrong matrix into such a result (M = 128, N = 64 or 2056, fp32 and bf16,
+// The library's product into a result whose row stride is not N: with long K (14336; not with 4224 or less) the
+// algorithm its heuristic ranks first has returned a wrong matrix into such a result (M = 128, N = 64 or 2056, fp32 and bf16,
 // stride N + 5 or N + 8), while results of stride N are right.  So a padded result is computed densely in scratch and
 // copied row by row.  `free_ws` is scratch of dense_result_bytes() + kDenseLibraryWorkspace bytes; `x_second`, when
 // given, is a second activation matrix whose product is added to the first's (the low halves of split fp32 rows).

@@ -277,7 +277,7 @@ def test_timed_library_candidates_are_checked_against_the_first(pkg):
 @pytest.mark.parametrize("x_dtype_name", ["BF16", "F16", "F32"])
 def test_library_route_with_padded_result_rows_and_long_k(pkg, ctx, x_dtype_name):
     """Results whose row stride is not N, with K = 14336: the library has returned wrong matrices into such results
-    (every algorithm it offers, strides N + 5 and N + 8 alike), so the route computes a padded result densely in
+    (the algorithm its heuristic ranks first, strides N + 5 and N + 8 alike), so the route computes a padded result densely in
     scratch and copies it row by row.  All three forms of the route, the dense entry point, canary behind the rows."""
     x_dtype = getattr(pkg, x_dtype_name)
     fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
