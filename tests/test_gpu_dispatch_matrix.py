@@ -29,14 +29,15 @@ def say(*a):
 FORMATS = [(4, 64), (4, 128), (8, 32), (8, 64), (8, 128), (3, 64), (2, 64), (6, 64), (5, 32), (3, 16)]
 
 
-def _one_case(pkg, ctx, rng, idx):
+def _one_case(pkg, ctx, rng, idx, ks=(128, 256, 384, 512, 1024, 2048 + 128), ns=(1, 17, 48, 100, 257, 300),
+              ms=(1, 2, 3, 4, 5, 7, 8, 9, 12, 15, 16, 17, 24, 31, 32, 33, 40, 70)):
     bits, group = FORMATS[int(rng.integers(len(FORMATS)))]
     layouts = [pkg.LAYOUT_PLANES, pkg.LAYOUT_STAF_BLOCKS] + ([pkg.LAYOUT_TILE16] if (bits, group) == (4, 64) else [])
     layout = layouts[int(rng.integers(len(layouts)))]
-    k = int(rng.choice([128, 256, 384, 512, 1024, 2048 + 128])) // group * group or group
+    k = int(rng.choice(list(ks))) // group * group or group
     k = max(k, 128) // 128 * 128
-    n = int(rng.choice([1, 17, 48, 100, 257, 300]))
-    m = int(rng.choice([1, 2, 3, 4, 5, 7, 8, 9, 12, 15, 16, 17, 24, 31, 32, 33, 40, 70]))
+    n = int(rng.choice(list(ns)))
+    m = int(rng.choice(list(ms)))
     x_dtype = [pkg.BF16, pkg.F16, pkg.F32][int(rng.integers(3))]
     y_dtype = [pkg.F32, pkg.BF16, pkg.F16][int(rng.integers(3))]
     xpad = int(rng.choice([0, 0, 8, 24]))
@@ -77,6 +78,15 @@ def test_random_dispatch_combinations(pkg, ctx, seed):
     rng = np.random.default_rng(7700 + seed)
     for i in range(45):
         _one_case(pkg, ctx, rng, seed * 100 + i)
+
+
+def test_random_dispatch_long_rows(pkg, ctx):
+    """The same sweep over long rows (K = 4224 and 14336) and more activation rows: the ranges of the streamed-weight
+    kernel, the tiled kernel and the library route, with padded result rows among them (a wider run of this sweep found
+    the library's wrong results into padded results at K = 14336)."""
+    rng = np.random.default_rng(7900)
+    for i in range(24):
+        _one_case(pkg, ctx, rng, 5000 + i, ks=(4224, 14336), ns=(1, 64, 129, 520), ms=(3, 9, 17, 48, 96, 100, 130, 260))
 
 
 def test_random_shared_launches(pkg, ctx):
