@@ -167,6 +167,12 @@ MI355Q_API int32_t mi355q_abi_version(void);
 MI355Q_API mi355q_status mi355q_context_create(int device_index, mi355q_context** out);
 MI355Q_API mi355q_status mi355q_context_destroy(mi355q_context* ctx);
 MI355Q_API mi355q_status mi355q_device_query(mi355q_context* ctx, mi355q_device_info* out);
+/* Whether launches through this context may hand a dense product to the platform's GEMM library (hipBLASLt, opened
+ * with dlopen on first use): the second half of the two-dispatch prefill route, as the reference's dense product is
+ * the platform's matmul2d (MC/Generator/MetalSourceGenerator+Linear.swift:18-81).  On by default; with 0 every
+ * launch stays on this library's own kernels (the fused, streamed-weight and decode kernels serve every shape, more
+ * slowly where the route was the quicker one), and the library is never opened. */
+MI355Q_API mi355q_status mi355q_context_set_library_use(mi355q_context* ctx, int enabled);
 
 MI355Q_API mi355q_status mi355q_buffer_alloc(mi355q_context* ctx, size_t bytes, void** out_dev);
 MI355Q_API mi355q_status mi355q_buffer_free(mi355q_context* ctx, void* dev);

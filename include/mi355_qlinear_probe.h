@@ -15,6 +15,11 @@ extern "C" {
 /* Launch flag for mi355q_qgemm (its `flags` argument, beside the MI355Q_FLAG_* values of mi355_qlinear.h): on
  * the matrix-core kernel, the first wavefront of workgroup 0 records how long it was in the kernel. */
 enum { MI355Q_FLAG_PROBE_CLOCK = 8 };
+/* Launch flag for mi355q_qgemm and mi355q_plan_prefill_steps: where the fused matrix-core route would take the wide-tile
+ * kernel (long prompts on 4-bit planes), keep the tiled kernel that dequantises into LDS (A/B runs). */
+enum { MI355Q_FLAG_PROBE_TILED = 64 };
+/* ... and the other way round: the wide-tile kernel wherever it reads the weight, whatever the size (tests of small shapes). */
+enum { MI355Q_FLAG_PROBE_WIDE = 128 };
 
 /* After an mi355q_qgemm call with MI355Q_FLAG_PROBE_CLOCK that ran on the matrix cores has completed, returns
  * what that wavefront counted: shader-clock cycles and ticks of the constant 100 MHz counter.

@@ -23,6 +23,8 @@ LAYOUT_STAF_BLOCKS, LAYOUT_PLANES, LAYOUT_TILE16 = 0, 1, 2
 # launch flags
 FLAG_NONE, FLAG_FORCE_GENERIC, FLAG_FORCE_SMALL_M, FLAG_FORCE_MFMA, FLAG_PROBE_CLOCK, FLAG_FORCE_TWO_STEP = 0, 1, 2, 4, 8, 16
 FLAG_FORCE_STREAM = 32
+FLAG_PROBE_TILED = 64      # measurement aid: the tiled fused kernel where the wide-tile one would be taken
+FLAG_PROBE_WIDE = 128      # ... the wide-tile kernel wherever it reads the weight, whatever the size
 
 STATUS_NAMES = {0: "OK", -1: "INVALID_ARGUMENT", -2: "UNSUPPORTED_FORMAT", -3: "SHAPE", -4: "NULL_HANDLE",
                 -5: "DEVICE", -6: "OUT_OF_MEMORY", -7: "KERNEL_NOT_FOUND", -8: "SIZE_MISMATCH",
@@ -128,6 +130,7 @@ def library() -> C.CDLL:
         "mi355q_context_create": (i32, [C.c_int, P(vp)]),
         "mi355q_context_destroy": (i32, [vp]),
         "mi355q_device_query": (i32, [vp, P(_DeviceInfo)]),
+        "mi355q_context_set_library_use": (i32, [vp, C.c_int]),
         "mi355q_buffer_alloc": (i32, [vp, sz, P(vp)]),
         "mi355q_buffer_free": (i32, [vp, vp]),
         "mi355q_buffer_upload": (i32, [vp, vp, vp, sz]),
@@ -680,6 +683,10 @@ class Context:
         if self.handle:
             library().mi355q_context_destroy(self.handle)
             self.handle = None
+
+    def set_library_use(self, enabled: bool):
+        """Whether launches may hand a dense product to the platform's GEMM library (on by default)."""
+        _check(library().mi355q_context_set_library_use(self.handle, 1 if enabled else 0))
 
     # ---- device info / memory / streams / events
     def device_info(self) -> _DeviceInfo:

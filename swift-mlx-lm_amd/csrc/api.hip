@@ -188,7 +188,7 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
     if (flags & MI355Q_FLAG_FORCE_MFMA) {
         if (!mfma_ok)
             return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the MFMA GEMM does not accept this format, layout or stride");
-        return launch_qgemm_mfma(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys, probe);
+        return launch_qgemm_mfma(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys, probe, flags);
     }
     // a few dozen rows on 4-bit planes: weights streamed through registers, activations alone through LDS
     if (!forced && gemm_stream_chosen(v, x_dtype, m, xs) && (uintptr_t)x % 16 == 0)
@@ -197,7 +197,7 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
     const bool small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) ||
                        m <= small_batch_limit(v, x_dtype, xs) || !mfma_ok;
     if (small) return run_small_m(ctx, s, w, x, x_dtype, y, y_dtype, m, xs, ys, flags);
-    return launch_qgemm_mfma(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys, probe);
+    return launch_qgemm_mfma(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys, probe, flags);
 }
 
 // Rows up to which the small-batch kernels, one launch after the other, beat the fused prefill kernel: two launches where
@@ -270,6 +270,7 @@ bool gemm_two_step_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_st
     if (flags & MI355Q_FLAG_FORCE_TWO_STEP) return true;
     if (!gemm_two_step_eligible(w, x_dtype, m, x_stride)) return false;
     if (gemm_stream_chosen(w, x_dtype, m, x_stride)) return false;      // a few dozen rows on 4- / 8-bit planes
+    if (gemm_wide_chosen(w, x_dtype, m, x_stride)) return false;        // long prompts on 4-bit planes: this library's own kernel
     if (!gemm_mfma_eligible(w, x_dtype, m, x_stride)) {
         // no decode kernel reads the weight: from the second row; from the first where the per-code kernel leaves most
         // of its lanes idle (a lane per code of a group: q3 g16 blocks, 4096 -> 14336, take it 465 us at one row

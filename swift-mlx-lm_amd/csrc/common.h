@@ -75,6 +75,7 @@ struct mi355q_context {
     // the platform's dense GEMM library (second half of the two-dispatch prefill route), opened on first use
     mi355q::DenseLibrary* dense_library;
     bool dense_library_failed;
+    bool dense_library_forbidden;      // mi355q_context_set_library_use(ctx, 0): in-tree kernels only
 };
 constexpr int kRetiredWorkspaces = 40;
 
@@ -265,9 +266,28 @@ bool split_rows_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_strid
 bool split_rows_small_batch(const WView& w, uint32_t parts, uint32_t m);
 bool split_rows_take_stream(const WView& w, int x_dtype, uint32_t m);
 bool gemm_mfma_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
+// `flags`: MI355Q_FLAG_PROBE_TILED keeps the tiled kernel where the wide-tile one (gemm_wide.hip) would be taken,
+// MI355Q_FLAG_PROBE_WIDE takes the wide-tile kernel wherever it reads the weight (A/B runs and tests)
 mi355q_status launch_qgemm_mfma(hipStream_t s, mi355q_context* ctx, const WView& w,
                                 const void* x, int x_dtype, void* y, int y_dtype, uint32_t m,
-                                uint32_t x_stride, uint32_t y_stride, unsigned long long* probe = nullptr);
+                                uint32_t x_stride, uint32_t y_stride, unsigned long long* probe = nullptr,
+                                uint32_t flags = 0);
+
+// Wide-tile MFMA GEMM for long prompts (gemm_wide.hip): 4-bit planes in groups of 64 / 128, bf16 activations; the weights
+// are dequantised in registers, only the activations pass through LDS.  Taken from kWideMinRows rows where its tiles
+// occupy three quarters of the CUs (measured against the tiled kernel and the two-dispatch route: see gemm_wide_chosen).
+constexpr uint32_t kWideMinRows = 384;
+bool gemm_wide_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
+bool gemm_wide_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
+GemmLaunchShape gemm_wide_shape(uint32_t m, uint32_t n, uint32_t k);
+uint32_t chip_cus();
+inline bool gemm_wide_taken(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride, uint32_t flags) {
+    if (flags & MI355Q_FLAG_PROBE_TILED) return false;
+    if (flags & MI355Q_FLAG_PROBE_WIDE) return gemm_wide_eligible(w, x_dtype, m, x_stride);
+    return gemm_wide_chosen(w, x_dtype, m, x_stride);
+}
+mi355q_status launch_qgemm_wide(hipStream_t s, mi355q_context* ctx, const WView& w, const void* x, int x_dtype, void* y,
+                                int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride, unsigned long long* probe = nullptr);
 // Streamed-weight matrix-core kernel (gemm_stream.hip): 4- and 8-bit planes, bf16 or f16 activations, at most 96 rows.
 constexpr uint32_t kStreamMaxRows = 96;
 // blocks in place: codes (N x K) from which it replaces the in-place decode kernel at three rows / at five rows

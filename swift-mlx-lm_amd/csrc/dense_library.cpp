@@ -105,7 +105,7 @@ namespace {
 
 DenseLibrary* library_of(mi355q_context* ctx) {
     if (ctx->dense_library) return ctx->dense_library;
-    if (ctx->dense_library_failed) return nullptr;
+    if (ctx->dense_library_failed || ctx->dense_library_forbidden) return nullptr;
     const Api* a = api();
     hipblasLtHandle_t h = nullptr;
     if (!a || a->create(&h) != HIPBLAS_STATUS_SUCCESS) {

@@ -309,7 +309,11 @@ mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w, uint32_t maximum
         std::snprintf(s->device_kernel, sizeof s->device_kernel, "qgemm_mfma_q%u_g%u", (unsigned)w->fmt.bits,
                       w->fmt.group_size);
         std::snprintf(s->kernel_family, sizeof s->kernel_family, "mfmaGEMM");
-        const GemmLaunchShape g = gemm_mfma_shape(w->ctx, m, (uint32_t)w->n, (uint32_t)w->k);
+        const bool wide = gemm_wide_taken(v, x_dtype, m, input_row_stride, flags);
+        if (wide)
+            std::snprintf(s->device_kernel, sizeof s->device_kernel, "qgemm_wide_q%u_g%u", (unsigned)w->fmt.bits, w->fmt.group_size);
+        const GemmLaunchShape g = wide ? gemm_wide_shape(m, (uint32_t)w->n, (uint32_t)w->k)
+                                       : gemm_mfma_shape(w->ctx, m, (uint32_t)w->n, (uint32_t)w->k);
         s->block[0] = g.block;
         s->grid[0] = g.grid;
         s->grid[1] = g.splits;

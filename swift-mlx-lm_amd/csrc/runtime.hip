@@ -294,6 +294,12 @@ mi355q_status mi355q_context_create(int device_index, mi355q_context** out) {
     return MI355Q_OK;
 }
 
+mi355q_status mi355q_context_set_library_use(mi355q_context* ctx, int enabled) {
+    if (!ctx) return fail(MI355Q_ERR_NULL_HANDLE, "context is null");
+    ctx->dense_library_forbidden = !enabled;
+    return MI355Q_OK;
+}
+
 mi355q_status mi355q_context_destroy(mi355q_context* ctx) {
     if (!ctx) return fail(MI355Q_ERR_NULL_HANDLE, "context is null");
     (void)hipSetDevice(ctx->device);

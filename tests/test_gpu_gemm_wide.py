@@ -1,0 +1,133 @@
+"""GPU parity tests of the wide-tile prefill GEMM (4-bit planes, weights dequantised in registers), through the C ABI.
+
+Numerics are those of the reference's dequant -> bf16 -> GEMM route
+(MetalSourceGenerator+Quantized.swift:361-416, MetalSourceGenerator+Linear.swift:18-81): the expected values are an
+fp64 accumulation of the bf16-rounded dequantised weights from the CPU oracle.  Bars as for the tiled kernel:
+relative L2 <= 1e-3 and max-abs <= 2e-2 on the fp32 output, 16-bit outputs equal to the rounding of the fp32 output,
+exactly representable cases compared exactly.  The kernel is forced with the probe flag where the shape is smaller
+than what the dispatcher gives it; BASELINE config 3 runs as dispatched.
+"""
+import sys
+
+import numpy as np
+import pytest
+
+import kat
+import oracle
+from gpu_util import Case, act_rounded, assert_within_tolerance, seeded_case
+from test_gpu_gemm import _tile_edge_sample, bf16_round, run_qgemm
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def wide(pkg):
+    return pkg.FLAG_FORCE_MFMA | pkg.FLAG_PROBE_WIDE
+
+
+@pytest.mark.parametrize("group", [64, 128])
+def test_wide_gemm_exact_small_integers(pkg, ctx, group):
+    """Every product and partial sum an integer multiple of 2^-6 below 2^17: any summation order is exact.  Rows
+    and columns off the tile grid (300 rows: a 256-row tile and a cut one; 530 columns: two whole column tiles and
+    one that ends inside a group of four), both scale types, all three output types, wide and narrow stores."""
+    rng = np.random.default_rng(4000 + group)
+    m, n, k = 300, 530, 3 * 256
+    codes = rng.integers(0, 16, (n, k), dtype=np.uint8)
+    scales = rng.choice([0.125, 0.25, 0.5], (n, k // group))
+    zeros = rng.integers(-4, 5, (n, k // group)) * 0.25
+    case = Case(4, group, codes, scales, zeros)
+    wq = scales.repeat(group, axis=1) * codes + zeros.repeat(group, axis=1)
+    assert np.array_equal(bf16_round(wq), wq.astype(np.float32))
+    x = rng.integers(-8, 9, (m, k)).astype(np.float32) * 0.125
+    want = x.astype(np.float64) @ wq.T
+    for sb in (pkg.F16, pkg.BF16):
+        w = case.device_weight(ctx, pkg, pkg.LAYOUT_PLANES, sb)
+        step = w.plan_prefill_steps(m, flags=wide(pkg))[0]
+        assert step.device_kernel == f"qgemm_wide_q4_g{group}" and step.block[0] == 256, step.device_kernel
+        for yd in (pkg.F32, pkg.BF16, pkg.F16):
+            for y_pad in (0, 2, 3):               # 532 columns a row: 16-byte rows; 533: the narrow stores
+                say(f"wide exact g{group} sb={sb} y={yd} pad={y_pad}")
+                got = run_qgemm(ctx, pkg, w, x, yd, wide(pkg), y_stride=(n + y_pad) if y_pad else None)
+                if y_pad:
+                    assert np.all(np.isnan(got[:, n:])), "padding of the output rows was written"
+                    got = got[:, :n]
+                if yd == pkg.F32:
+                    assert np.array_equal(got.astype(np.float64), want)
+                elif yd == pkg.BF16:
+                    assert np.array_equal(got, bf16_round(want.astype(np.float32)))
+                else:
+                    assert np.array_equal(got, want.astype(np.float16).astype(np.float32))
+        w.destroy()
+
+
+def _seeded(pkg, ctx, seed, m, n, k, group, flags, sample=None, x_pad=0, y_pad=0, sb=None):
+    words, s, z, wq = seeded_case(seed, n, k, 4, group)
+    wb = bf16_round(wq)
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, group)
+    w = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, pkg.LAYOUT_PLANES)
+    x = np.zeros((m, k + x_pad), np.float32)
+    x[:, :k] = act_rounded(kat.seeded_activations(seed + 1, m, k), pkg.BF16, pkg)
+    if x_pad:
+        x[:, k:] = 3.0e4
+    say(f"wide seeded g{group} M={m} {k}->{n} pads=({x_pad},{y_pad}) flags={flags}")
+    got = run_qgemm(ctx, pkg, w, x, pkg.F32, flags, y_stride=(n + y_pad) if y_pad else None)
+    if y_pad:
+        assert np.all(np.isnan(got[:, n:])), "padding of the output rows was written"
+        got = got[:, :n]
+    cols = np.arange(n) if sample is None else sample
+    want = oracle.gemm_f64(np.ascontiguousarray(wb[cols]), np.ascontiguousarray(x[:, :k]))
+    r = assert_within_tolerance(got[:, cols], want, f"wide g{group} M={m} {k}->{n}")
+    assert np.all(np.isfinite(got))
+    gb = run_qgemm(ctx, pkg, w, x, pkg.BF16, flags)
+    assert np.array_equal(oracle.bf16_from_f32(gb), oracle.bf16_from_f32(got)), "bf16 out != rne(fp32 out)"
+    return w, x, got, r
+
+
+def test_wide_gemm_ragged_shapes_against_the_oracle(pkg, ctx):
+    """One row, rows just past a tile, one column, columns off every grid, one group of four K-tiles and several, padded
+    rows on both sides; and the same weights through the tiled kernel: equal up to the order of the fp32 sums."""
+    for i, (m, n, k, group, x_pad, y_pad) in enumerate([(1, 1, 256, 64, 0, 0), (129, 257, 512, 64, 0, 0),
+                                                         (257, 70, 256, 128, 0, 0), (130, 515, 1024, 64, 64, 5),
+                                                         (600, 300, 768, 128, 8, 4), (33, 1030, 256, 64, 0, 1)]):
+        w, x, got, _ = _seeded(pkg, ctx, 4100 + i, m, n, k, group, wide(pkg), x_pad=x_pad, y_pad=y_pad)
+        tiled = run_qgemm(ctx, pkg, w, x, pkg.F32, pkg.FLAG_FORCE_MFMA | pkg.FLAG_PROBE_TILED)
+        assert np.max(np.abs(tiled - got)) <= 2e-5 * max(1.0, float(np.max(np.abs(got)))), "wide vs tiled kernel"
+        w.destroy()
+
+
+@pytest.mark.parametrize("m", [128, 512, 2048])
+@pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
+def test_config3_prefill_as_dispatched(pkg, ctx, m, n, k):
+    """BASELINE config 3 at full size with no flags: whatever route the library picks for the shape (the plan record
+    names it) is checked against the oracle on every row and the tile-edge column sample."""
+    sample = _tile_edge_sample(n, 17 * m + n, tile=256)
+    w, _, _, (rel, _) = _seeded(pkg, ctx, 4200 + m % 83, m, n, k, 64, 0, sample=sample)
+    steps = w.plan_prefill_steps(m)
+    say("as dispatched:", [s.device_kernel for s in steps])
+    if m == 2048:
+        # long prompts stay on this library's own kernel
+        assert len(steps) == 1 and steps[0].device_kernel == "qgemm_wide_q4_g64" and not steps[0].used_fallback
+    assert rel < 5e-4
+    w.destroy()
+
+
+def test_context_without_the_dense_library_keeps_in_tree_kernels(pkg):
+    """mi355q_context_set_library_use(ctx, 0): a long prompt on blocks in place, which the two-dispatch route would
+    serve, stays on this library's kernels, and the result holds the bar."""
+    c = pkg.Context(0)
+    try:
+        c.set_library_use(False)
+        m, n, k = 130, 96, 512
+        words, s, z = oracle.quantize_affine(kat.seeded_weights(4300, n, k), 4, 64, oracle.F16)
+        wq = oracle.dequant_planes_f32(4, 64, n, k, words, s, z, oracle.F16)
+        fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+        w = c.weight_prepare_mlx(fmt, words, s, z, pkg.F16, pkg.LAYOUT_STAF_BLOCKS)
+        x = act_rounded(kat.seeded_activations(4301, m, k), pkg.BF16, pkg)
+        got = run_qgemm(c, pkg, w, x, pkg.F32, 0)
+        assert_within_tolerance(got, oracle.gemm_f64(wq, x), "blocks in place, library forbidden")
+        w.destroy()
+    finally:
+        c.close()
