@@ -660,6 +660,23 @@ def main():
                 ms, ms_first, taken = steady_region(
                     ctx, lambda i: ctx.qgemm(wts[i % len(wts)], xb, pkg.BF16, yb, pkg.BF16, mm, 0, 0, 0, stream), reps, stream)
                 steps_p = wts[0].plan_prefill_steps(mm, k)
+                if mm == 2048 and not a.skip_parity:
+                    # parity gate on the output just timed (the last launch read copy (reps - 1) % 4, all copies hold the
+                    # same tensor): every row, 32 columns spread over the matrix, against an fp64 accumulation of the
+                    # bf16-rounded weights; the output is bf16, so the bar is that of a bf16 rounding (2^-9) on top
+                    ctx.synchronize(stream)
+                    cols = np.unique(np.concatenate([np.arange(0, n, n // 24), [1, 255, 256, n - 257, n - 2, n - 1]]))
+                    words, s_, z_ = host["gate" if n == 14336 else "down"]
+                    wq = oracle.dequant_planes_f32(BITS, GROUP, n, k, words, s_, z_, oracle.BF16)[cols]
+                    wb = oracle.bf16_to_f32(oracle.bf16_from_f32(wq)).reshape(wq.shape)
+                    xh = oracle.bf16_to_f32(oracle.bf16_from_f32(kat.seeded_activations(500 + mm, mm, k))).reshape(mm, k)
+                    want = oracle.gemm_f64(np.ascontiguousarray(wb), xh)
+                    got = oracle.bf16_to_f32(yb.download(np.uint16, (mm, n))[:, cols]).reshape(mm, len(cols))
+                    rel = float(np.linalg.norm(got - want) / np.linalg.norm(want))
+                    mx = float(np.max(np.abs(got - want)))
+                    if not (rel <= 3e-3 and mx <= 2e-2 + 4e-3 * float(np.max(np.abs(want)))):
+                        sys.exit(f"bench.py: prefill parity gate failed on {name} M={mm}: rel-L2 {rel:.3e} max-abs {mx:.3e}")
+                    log(f"  parity {name} M={mm} ({steps_p[0].device_kernel}): rel-L2 {rel:.2e} max-abs {mx:.2e} (bf16 output)")
                 sweep[f"{name} M={mm}"] = {"us": round(ms * 1e3, 1), "TFLOPs": round(2.0 * mm * n * k / (ms * 1e-3) / 1e12, 1),
                                            "route": " + ".join(st.device_kernel for st in steps_p),
                                            "first_sample_us": round(ms_first * 1e3, 1), "samples_of": [taken, reps]}
@@ -693,19 +710,27 @@ def main():
         probe = pkg.FLAG_FORCE_MFMA | pkg.FLAG_PROBE_CLOCK
 
         def gemm_figure(xbuf):
+            nonlocal probe
             ctx.qgemm(wg, xbuf, pkg.BF16, yg, pkg.BF16, m, 0, 0, probe, stream)
             ctx.synchronize(stream)
             ms, _, _ = steady_region(ctx, lambda i: ctx.qgemm(wg, xbuf, pkg.BF16, yg, pkg.BF16, m, 0, 0, probe, stream), 10, stream)
             return ms, ctx.clock_probe_ghz()
 
         ms_g, ghz = gemm_figure(xg)
+        probe |= pkg.FLAG_PROBE_TILED                     # the tiled kernel (weights dequantised into LDS) beside it
+        ms_t, ghz_t = gemm_figure(xg)
+        probe &= ~pkg.FLAG_PROBE_TILED
         xc = ctx.upload(np.full((m, 4096), 0x3F80, np.uint16))
         ms_c, ghz_c = gemm_figure(xc)
         xc.free(); xg.free(); yg.free()
         flops = 2.0 * m * 14336 * 4096
         prefill = {"config3": sweep,
                    "fused_kernel_m2048_gate": {"us": round(ms_g * 1e3, 1), "TFLOPs": round(flops / (ms_g * 1e-3) / 1e12, 1),
-                                               "shader_clock_GHz": round(ghz, 3)},
+                                               "shader_clock_GHz": round(ghz, 3),
+                                               "kernel": wg.plan_prefill_steps(m, 4096, flags=pkg.FLAG_FORCE_MFMA)[0].device_kernel},
+                   "tiled_kernel_m2048_gate": {"us": round(ms_t * 1e3, 1), "TFLOPs": round(flops / (ms_t * 1e-3) / 1e12, 1),
+                                               "shader_clock_GHz": round(ghz_t, 3),
+                                               "kernel": wg.plan_prefill_steps(m, 4096, flags=pkg.FLAG_FORCE_MFMA | pkg.FLAG_PROBE_TILED)[0].device_kernel},
                    "aside_constant_activations_fused_kernel": {"us": round(ms_c * 1e3, 1), "TFLOPs": round(flops / (ms_c * 1e-3) / 1e12, 1),
                                                                "shader_clock_GHz": round(ghz_c, 3)}}
         log(f"  fused kernel M={m} gate: {prefill['fused_kernel_m2048_gate']}; constant activations (aside): "
