@@ -94,6 +94,13 @@ enum {
     MI355Q_FLAG_FORCE_STREAM = 32  /* qgemm: the streamed-weight matrix-core kernel (4- / 8-bit planes or blocks, bf16 or f16 rows, M <= 96) */
 };
 
+/* ElementwiseFragment.ElementwiseKind of the gated MLP (MC/Compilable/MLPFragment.swift:16-27) and the activation its
+ * kernel applies to the gate (GatedActivation, MC/Generator/MetalSourceGenerator+NormAndElementwise.swift:175-207) */
+typedef enum {
+    MI355Q_GATED_SILU = 0,      /* .swiglu:    g / (1 + exp(-g)) * up */
+    MI355Q_GATED_GELU_TANH = 1  /* .geluGated: 0.5 g (1 + tanh(0.7978845608 (g + 0.044715 g^3))) * up */
+} mi355q_gated_activation;
+
 /* ------------------------------------------------------------------------------------------
  * Format descriptor: QuantizationFormat protocol (MC/STAF/QuantizationFormat.swift:25-153)
  * ---------------------------------------------------------------------------------------- */
@@ -318,6 +325,29 @@ MI355Q_API mi355q_status mi355q_qgemm(mi355q_context* ctx, void* stream, const m
                                       const void* x_dev, mi355q_dtype x_dtype, void* y_dev,
                                       mi355q_dtype y_dtype, uint32_t m, uint32_t x_row_stride,
                                       uint32_t y_row_stride, uint32_t flags);
+
+/* The elementwise step of the gated MLP, swiglu / gelu_gated (generateGatedActivation,
+ * MC/Generator/MetalSourceGenerator+NormAndElementwise.swift:196-249; ElementwiseFragment of
+ * MC/Compilable/MLPFragment.swift:7-14): out[s, i] = T(activation(float(gate[s, i])) * float(up[s, i])) for
+ * i < dimension, s < sequence_length, all three buffers of type T with rows `row_stride` elements apart
+ * (0 = dimension).  gate, up and out may alias. */
+MI355Q_API mi355q_status mi355q_gated_activation_apply(mi355q_context* ctx, void* stream, const void* gate_dev,
+                                                       const void* up_dev, void* out_dev, mi355q_dtype dtype,
+                                                       uint32_t dimension, uint32_t sequence_length,
+                                                       uint32_t row_stride, mi355q_gated_activation activation);
+
+/* MLPFragment's first two steps as one call (MC/Compilable/MLPFragment.swift:7-14): the batched gate_proj + up_proj
+ * projection of x and the gated activation, out[s, :] = activation(x[s] Wgate^T) * (x[s] Wup^T), one [M, N] result
+ * instead of two and no elementwise dispatch.  Both weights share N, K, scheme and layout.  The gate and up sums are
+ * rounded to y_dtype before the activation, as the reference's elementwise kernel reads them from buffers of that
+ * type, so the result is that of mi355q_batched_qgemm followed by mi355q_gated_activation_apply up to the order of
+ * the fp32 sums.  One activation row on split planes runs as ONE launch (a wavefront owns a gate row and the up row
+ * of the same index); other shapes run the projections into the context's scratch and then the elementwise kernel. */
+MI355Q_API mi355q_status mi355q_gated_qgemm(mi355q_context* ctx, void* stream, const mi355q_weight* w_gate,
+                                            const mi355q_weight* w_up, const void* x_dev, mi355q_dtype x_dtype,
+                                            void* y_dev, mi355q_dtype y_dtype, uint32_t m, uint32_t x_row_stride,
+                                            uint32_t y_row_stride, mi355q_gated_activation activation,
+                                            uint32_t flags);
 
 /* batched_gemm_q4_g64_{2,3} (:166-338; bindings MC/Compiler/MetalPrefillStepBuilder.swift:928-955):
  * 2 or 3 projections sharing one input (gate+up, q+k+v) in one launch.  All weights must share

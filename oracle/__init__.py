@@ -67,6 +67,7 @@ def lib():
         L.orc_qgemm_staf_ref_f32.argtypes = [i32, i32, vp, vp, sz, sz, sz, sz, vp, i32]
         L.orc_qgemm_planes_ref_f32.argtypes = [i32, i32, vp, vp, vp, i32, vp, sz, sz, sz, sz, vp, i32]
         L.orc_argmax_lowest.argtypes = [vp, sz]; L.orc_argmax_lowest.restype = C.c_int32
+        L.orc_gated_activation_f32.argtypes = [vp, vp, sz, i32, i32, vp]; L.orc_gated_activation_f32.restype = None
         L.orc_quantize_affine.argtypes = [vp, sz, sz, i32, i32, i32, vp, vp, vp]
         _lib = L
     return _lib
@@ -291,6 +292,17 @@ def qgemm_planes_ref_f32(bits, group, codes, scales, biases, sb_dtype, x, n, k, 
                                           _p(x), m, n, k, stride, _p(y), threads),
            "qgemm_planes_ref_f32")
     return y
+
+
+SILU, GELU_TANH = 0, 1
+
+
+def gated_activation_f32(gate, up, kind=SILU, dtype=F32):
+    """activation(T(gate)) * T(up), rounded to T: the gated MLP's elementwise step, fp32 arithmetic."""
+    gate = _c(gate, np.float32); up = _c(up, np.float32)
+    out = np.zeros(gate.shape, np.float32)
+    lib().orc_gated_activation_f32(_p(gate), _p(up), gate.size, kind, dtype, _p(out))
+    return out
 
 
 def argmax_lowest(v) -> int:

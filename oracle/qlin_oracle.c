@@ -488,6 +488,29 @@ int orc_qgemm_planes_ref_f32(int bits, int group, const uint32_t* codes, const v
     return run_ref(j, threads);
 }
 
+/* ---------------------------------------------------------- gated activation */
+
+static float round_to(float v, int dtype) {
+    if (dtype == ORC_BF16) return orc_bf16_to_f32(orc_bf16_from_f32(v));
+    if (dtype == ORC_F16) return orc_f16_to_f32(orc_f16_from_f32(v));
+    return v;
+}
+
+/* generateGatedActivation (MC/Generator/MetalSourceGenerator+NormAndElementwise.swift:196-249) */
+void orc_gated_activation_f32(const float* gate, const float* up, size_t n, int kind, int dtype, float* out) {
+    for (size_t i = 0; i < n; i++) {
+        const float g = round_to(gate[i], dtype), u = round_to(up[i], dtype);
+        float activated;
+        if (kind == 1) {
+            const float inner = 0.7978845608f * (g + 0.044715f * g * g * g);
+            activated = 0.5f * g * (1.0f + tanhf(inner));
+        } else {
+            activated = g * (1.0f / (1.0f + expf(-g)));
+        }
+        out[i] = round_to(activated * u, dtype);
+    }
+}
+
 /* -------------------------------------------------------------------- argmax */
 
 int32_t orc_argmax_lowest(const float* v, size_t n) {

@@ -20,6 +20,9 @@
  *   orc_embedding_lookup_*     pinned: the reference's two embedding vectors + row gather of the pinned dequant
  *   orc_kv_*                   pinned: head-slot sizes, the q8 round-trip vector and the unsigned-byte read
  *                              vector of the reference's tests; exact rational arithmetic for the codes
+ *   orc_gated_activation_f32   the reference holds no value test of its swiglu / gelu_gated kernels (only pipeline
+ *                              existence and benchmark tests): pinned by closed forms (g = 0, u = 0, large |g|,
+ *                              silu(1), gelu_tanh(1) to 1e-7 from their definitions) and by an fp64 evaluation
  *   orc_argmax_lowest          PARITY UNPINNED against the reference (it holds no argmax value
  *                              test); pinned only by brute force against numpy on tiny vectors
  *   orc_quantize_affine        PARITY UNPINNED (the reference has no weight quantizer; this is an
@@ -109,6 +112,13 @@ int orc_qgemm_staf_ref_f32(int bits, int group, const uint8_t* blocks, const flo
 int orc_qgemm_planes_ref_f32(int bits, int group, const uint32_t* codes, const void* scales,
                              const void* biases, int sb_dtype, const float* x, size_t m, size_t n,
                              size_t k, size_t x_stride, float* y, int threads);
+
+/* The gated MLP's elementwise step (generateGatedActivation,
+ * MC/Generator/MetalSourceGenerator+NormAndElementwise.swift:196-249): with T the buffer type `dtype`,
+ *   g = float(T(gate[i])), u = float(T(up[i])), activated = silu: g * (1 / (1 + exp(-g)))
+ *                                                           gelu: 0.5 g (1 + tanh(0.7978845608 (g + 0.044715 g g g)))
+ *   out[i] = float(T(activated * u)), all arithmetic in fp32.  kind 0 = silu (swiglu), 1 = gelu tanh (gelu_gated). */
+void orc_gated_activation_f32(const float* gate, const float* up, size_t n, int kind, int dtype, float* out);
 
 /* Strict '>' scan from index 0 (MC/Generator/MetalSourceGenerator+Sampling.swift:80-90):
  * NaN never wins, ties keep the lowest index, empty / all-NaN input yields 0. */

@@ -23,6 +23,7 @@ LAYOUT_STAF_BLOCKS, LAYOUT_PLANES, LAYOUT_TILE16 = 0, 1, 2
 # launch flags
 FLAG_NONE, FLAG_FORCE_GENERIC, FLAG_FORCE_SMALL_M, FLAG_FORCE_MFMA, FLAG_PROBE_CLOCK, FLAG_FORCE_TWO_STEP = 0, 1, 2, 4, 8, 16
 FLAG_FORCE_STREAM = 32
+GATED_SILU, GATED_GELU_TANH = 0, 1      # ElementwiseKind .swiglu / .geluGated
 FLAG_PROBE_TILED = 64      # measurement aid: the tiled fused kernel where the wide-tile one would be taken
 FLAG_PROBE_WIDE = 128      # ... the wide-tile kernel wherever it reads the weight, whatever the size
 
@@ -152,6 +153,8 @@ def library() -> C.CDLL:
         "mi355q_weight_destroy": (i32, [vp]),
         "mi355q_qgemv": (i32, [vp, vp, vp, vp, C.c_int, vp, C.c_int, u32, u32, u32, u32]),
         "mi355q_qgemm": (i32, [vp, vp, vp, vp, C.c_int, vp, C.c_int, u32, u32, u32, u32]),
+        "mi355q_gated_activation_apply": (i32, [vp, vp, vp, vp, vp, C.c_int, u32, u32, u32, C.c_int]),
+        "mi355q_gated_qgemm": (i32, [vp, vp, vp, vp, vp, C.c_int, vp, C.c_int, u32, u32, u32, C.c_int, u32]),
         "mi355q_batched_qgemm": (i32, [vp, vp, u32, P(vp), vp, C.c_int, P(vp), C.c_int, u32, u32, u32]),
         "mi355q_dequant_bf16": (i32, [vp, vp, vp, vp]),
         "mi355q_dequant_f32": (i32, [vp, vp, vp, vp]),
@@ -821,6 +824,19 @@ class Context:
         yh = (C.c_void_p * n)(*[self._ptr(y) for y in ys])
         _check(library().mi355q_batched_qgemm(self.handle, stream, n, wh, self._ptr(x), x_dtype, yh, y_dtype, m,
                                               x_row_stride, flags))
+
+    def gated_qgemm(self, w_gate, w_up, x, x_dtype, y, y_dtype, m, activation=GATED_SILU, x_row_stride=0,
+                    y_row_stride=0, flags=0, stream=0):
+        """MLPFragment's gate_proj + up_proj + swiglu / gelu_gated as one call: y = act(x Wgate^T) * (x Wup^T)."""
+        _check(library().mi355q_gated_qgemm(self.handle, stream, w_gate.handle, w_up.handle, self._ptr(x), x_dtype,
+                                            self._ptr(y), y_dtype, m, x_row_stride, y_row_stride, activation, flags))
+
+    def gated_activation(self, gate, up, out, dtype, dimension, sequence_length=1, row_stride=0,
+                         activation=GATED_SILU, stream=0):
+        """The elementwise step alone: out = act(gate) * up."""
+        _check(library().mi355q_gated_activation_apply(self.handle, stream, self._ptr(gate), self._ptr(up),
+                                                       self._ptr(out), dtype, dimension, sequence_length, row_stride,
+                                                       activation))
 
     def dequant_bf16(self, w: PackedWeight, out, stream=0):
         _check(library().mi355q_dequant_bf16(self.handle, stream, w.handle, self._ptr(out)))

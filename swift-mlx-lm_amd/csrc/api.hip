@@ -671,3 +671,55 @@ mi355q_status mi355q_clock_probe_read(mi355q_context* ctx, uint64_t* shader_cycl
 }
 
 }  // extern "C"
+
+// ---- gated MLP: gate_proj + up_proj + swiglu / gelu_gated --------------------------------------------------------
+extern "C" mi355q_status mi355q_gated_activation_apply(mi355q_context* ctx, void* stream, const void* gate_dev,
+                                                       const void* up_dev, void* out_dev, mi355q_dtype dtype,
+                                                       uint32_t dimension, uint32_t sequence_length,
+                                                       uint32_t row_stride, mi355q_gated_activation activation) {
+    if (!ctx) return fail(MI355Q_ERR_NULL_HANDLE, "context is null");
+    if (!gate_dev || !up_dev || !out_dev) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null buffer");
+    if (!dtype_ok(dtype)) return fail(MI355Q_ERR_INVALID_ARGUMENT, "bad dtype tag");
+    if (activation != MI355Q_GATED_SILU && activation != MI355Q_GATED_GELU_TANH)
+        return fail(MI355Q_ERR_INVALID_ARGUMENT, "unknown gated activation %d", (int)activation);
+    if (dimension == 0 || sequence_length == 0) return fail(MI355Q_ERR_INVALID_ARGUMENT, "dimension and sequence length must be >= 1");
+    if (row_stride == 0) row_stride = dimension;
+    if (row_stride < dimension) return fail(MI355Q_ERR_SHAPE, "row stride %u < dimension %u", row_stride, dimension);
+    hipError_t e = hipSetDevice(ctx->device);
+    if (e != hipSuccess) return fail(MI355Q_ERR_DEVICE, "hipSetDevice failed: %s", hipGetErrorString(e));
+    return launch_gated_activation((hipStream_t)stream, gate_dev, up_dev, out_dev, dtype, dimension, sequence_length, row_stride,
+                                   row_stride, row_stride, activation);
+}
+
+extern "C" mi355q_status mi355q_gated_qgemm(mi355q_context* ctx, void* stream, const mi355q_weight* w_gate,
+                                            const mi355q_weight* w_up, const void* x_dev, mi355q_dtype x_dtype,
+                                            void* y_dev, mi355q_dtype y_dtype, uint32_t m, uint32_t x_row_stride,
+                                            uint32_t y_row_stride, mi355q_gated_activation activation, uint32_t flags) {
+    if (mi355q_status st = check_launch(ctx, w_gate)) return st;
+    if (mi355q_status st = check_launch(ctx, w_up)) return st;
+    if (activation != MI355Q_GATED_SILU && activation != MI355Q_GATED_GELU_TANH)
+        return fail(MI355Q_ERR_INVALID_ARGUMENT, "unknown gated activation %d", (int)activation);
+    if (w_gate->n != w_up->n || w_gate->k != w_up->k || w_gate->fmt.scheme_identifier != w_up->fmt.scheme_identifier ||
+        w_gate->layout != w_up->layout)
+        return fail(MI355Q_ERR_SHAPE, "gate and up projections must share N, K, scheme and layout");
+    uint32_t xs = x_row_stride, ys = y_row_stride;
+    if (mi355q_status st = check_io(w_gate, x_dev, x_dtype, y_dev, y_dtype, m, xs, ys)) return st;
+    hipStream_t s = (hipStream_t)stream;
+    const WView g = w_gate->view(), u = w_up->view();
+    const uint32_t n = (uint32_t)w_gate->n;
+    if (!(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_TWO_STEP |
+                   MI355Q_FLAG_FORCE_STREAM)) &&
+        gemv_gated_eligible(ctx, g, u, x_dtype, m, xs) && (uintptr_t)x_dev % 16 == 0)
+        return launch_gemv_gated(s, ctx, g, u, x_dev, x_dtype, y_dev, y_dtype, xs, activation);
+    // elsewhere: the two projections as the batched entry point runs them, into scratch of the context, then the
+    // elementwise kernel (the reference's own sequence of dispatches)
+    const size_t esz = y_dtype == MI355Q_F32 ? 4 : 2;
+    const size_t half = ((size_t)m * n * esz + 255) & ~(size_t)255;
+    if (mi355q_status st = ensure_gated_buffer(ctx, 2 * half)) return st;
+    void* const gate_out = ctx->gated_buffer;
+    void* const up_out = (char*)ctx->gated_buffer + half;
+    const mi355q_weight* ws[2] = {w_gate, w_up};
+    void* ys2[2] = {gate_out, up_out};
+    if (mi355q_status st = dispatch_batched(ctx, s, 2, ws, x_dev, x_dtype, ys2, y_dtype, m, xs, flags)) return st;
+    return launch_gated_activation(s, gate_out, up_out, y_dev, y_dtype, n, m, n, n, ys, activation);
+}

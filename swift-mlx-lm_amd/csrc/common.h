@@ -66,18 +66,22 @@ struct mi355q_context {
     // outgrown buffers are kept until the context goes, because captured graphs hold their addresses
     void* workspace;
     size_t workspace_bytes;
-    void* retired[40];
+    void* retired[96];                 // shared by the three scratch buffers: each at most doubles ~30 times
     int retired_count;
     // fp32 activations split into bf16 rows, and the partial projections of those rows (the decode kernels that run on
     // them may use `workspace` themselves); grown and retired like `workspace`
     void* split_buffer;
     size_t split_bytes;
+    // gate and up sums of the gated projection where they do not stay in registers (its own buffer: the projections
+    // that fill it may use the other two)
+    void* gated_buffer;
+    size_t gated_bytes;
     // the platform's dense GEMM library (second half of the two-dispatch prefill route), opened on first use
     mi355q::DenseLibrary* dense_library;
     bool dense_library_failed;
     bool dense_library_forbidden;      // mi355q_context_set_library_use(ctx, 0): in-tree kernels only
 };
-constexpr int kRetiredWorkspaces = 40;
+constexpr int kRetiredWorkspaces = 96;
 
 struct mi355q_weight {
     mi355q_context* ctx;
@@ -167,6 +171,16 @@ mi355q_status launch_gemv_fast(hipStream_t s, const mi355q_context* ctx, const W
                                const void* x, int x_dtype, void* y, int y_dtype, uint32_t m,
                                uint32_t x_stride, uint32_t y_stride, float* logits_f32,
                                int32_t* token_out, HeadKeys keys);
+// Gate and up projection of one activation row with the gated activation as epilogue, one launch (rows kernel over row
+// pairs); `gemv_gated_eligible` says whether the pair of weights and the shape have such a launch.
+bool gemv_gated_eligible(const mi355q_context* ctx, const WView& gate, const WView& up, int x_dtype, uint32_t m, uint32_t x_stride);
+mi355q_status launch_gemv_gated(hipStream_t s, const mi355q_context* ctx, const WView& gate, const WView& up, const void* x,
+                                int x_dtype, void* y, int y_dtype, uint32_t x_stride, int activation);
+mi355q_status launch_gated_activation(hipStream_t s, const void* gate, const void* up, void* out, int dtype, uint32_t dimension,
+                                      uint32_t sequence_length, uint32_t gate_stride, uint32_t up_stride, uint32_t out_stride,
+                                      int activation);
+// Raises a kernel's dynamic-LDS limit above 64 KiB once per (kernel, device) instead of on every launch.
+mi355q_status raise_lds_limit(const void* kernel, size_t lds_bytes);
 // Block-layout GEMV (gemv_staf.hip): reads STAF interleaved blocks in place.
 bool gemv_staf_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
 mi355q_status launch_gemv_staf(hipStream_t s, const mi355q_context* ctx, const WView& w, const void* x, int x_dtype,
@@ -258,6 +272,7 @@ GemmLaunchShape gemm_mfma_shape(const mi355q_context* ctx, uint32_t m, uint32_t 
 // Grows the context's scratch buffer for fp32 partial results; nothing is released before the context goes.
 mi355q_status ensure_workspace(mi355q_context* ctx, size_t bytes);
 mi355q_status ensure_split_buffer(mi355q_context* ctx, size_t bytes);
+mi355q_status ensure_gated_buffer(mi355q_context* ctx, size_t bytes);
 // fp32 activations as three bf16 rows each on the bf16 decode kernels (api.hip): row pitch of the bf16 rows, bf16 rows
 // per activation row (0: the type is not split), and whether a call takes that route
 inline uint32_t split_rows_stride(uint32_t k) { return (k + 7u) & ~7u; }

@@ -70,6 +70,23 @@ __device__ __forceinline__ void f16x8_to_bf16_hi_lo(const u32x4& v, u32x4& hi, u
     lo.x = l[0]; lo.y = l[1]; lo.z = l[2]; lo.w = l[3];
 }
 
+// activation(gate) * up of the gated MLP (SwiGLU: silu; GEGLU: tanh-approximated GELU), on a gate and an up value that
+// are first rounded to the buffer type `dtype`, as the reference's elementwise kernel reads them from buffers of that
+// type (Sources/MetalCompiler/Generator/MetalSourceGenerator+NormAndElementwise.swift:196-249); fp32 arithmetic, the
+// caller rounds the product to the output type.
+__device__ __forceinline__ float round_to_dtype(float v, uint32_t dtype) {
+    if (dtype == MI355Q_BF16) return bf16_to_f32(f32_to_bf16_rne(v));
+    if (dtype == MI355Q_F16) return f16_to_f32(f32_to_f16_rne(v));
+    return v;
+}
+__device__ __forceinline__ float gated_value(float gate, float up, uint32_t activation, uint32_t dtype) {
+    const float g = round_to_dtype(gate, dtype), u = round_to_dtype(up, dtype);
+    float act;
+    if (activation == MI355Q_GATED_GELU_TANH) act = 0.5f * g * (1.0f + tanhf(0.7978845608f * (g + 0.044715f * g * g * g)));
+    else act = g * (1.0f / (1.0f + expf(-g)));
+    return act * u;
+}
+
 __device__ __forceinline__ float sb_to_f32(uint16_t h, uint32_t sb_dtype) {
     return sb_dtype == MI355Q_BF16 ? bf16_to_f32(h) : f16_to_f32(h);
 }

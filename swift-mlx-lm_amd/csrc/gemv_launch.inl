@@ -9,8 +9,8 @@ namespace {
 template <typename K>
 mi355q_status launch_kernel(K kern, hipStream_t s, const GemvArgs& a, uint32_t grid, uint32_t block, size_t lds) {
     if (lds > 64 * 1024) {
-        // opt in to more than the default 64 KiB of dynamic LDS (gfx950 has 160 KiB per CU)
-        MI355Q_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        // opt in to more than the default 64 KiB of dynamic LDS (gfx950 has 160 KiB per CU): once per kernel and device
+        if (mi355q_status st = raise_lds_limit((const void*)kern, lds)) return st;
     }
     kern<<<dim3(grid), dim3(block), lds, s>>>(a);
     MI355Q_HIP(hipGetLastError());
@@ -56,6 +56,18 @@ template <int BITS, int GROUP, int NCT, int BR, int WAVES>
 mi355q_status launch_rows(hipStream_t s, const GemvArgs& a, const GemvCfg& c) {
     const bool sbbf = a.sb_dtype == MI355Q_BF16;
     const uint32_t block = WAVES * 64;
+    if (c.gated) {
+        if (c.argmax) return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the gated row kernel has no arg-max tail");
+        if (c.xa) {
+            if constexpr (gemv_rows_has_f16(BITS, GROUP)) {
+                if (sbbf) return launch_kernel(gemv_rows_kernel<BITS, GROUP, NCT, BR, WAVES, 1, true, false, true>, s, a, c.grid, block, c.lds);
+                return launch_kernel(gemv_rows_kernel<BITS, GROUP, NCT, BR, WAVES, 1, false, false, true>, s, a, c.grid, block, c.lds);
+            }
+            return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no f16 variant of the row kernel for q%d g%d", BITS, GROUP);
+        }
+        if (sbbf) return launch_kernel(gemv_rows_kernel<BITS, GROUP, NCT, BR, WAVES, 0, true, false, true>, s, a, c.grid, block, c.lds);
+        return launch_kernel(gemv_rows_kernel<BITS, GROUP, NCT, BR, WAVES, 0, false, false, true>, s, a, c.grid, block, c.lds);
+    }
     if (c.argmax) {
         if constexpr (gemv_rows_has_argmax(NCT, BR)) {
             if (c.xa) {

@@ -497,7 +497,7 @@ mi355q_status launch_pm(hipStream_t s, const PmArgs& a, uint32_t grid, size_t ld
                         : (a.sb_dtype == MI355Q_BF16 ? gemv_mfma_planes_kernel<BITS, GROUP, KSPLIT, TPW, true, false>
                                                      : gemv_mfma_planes_kernel<BITS, GROUP, KSPLIT, TPW, false, false>);
     if (lds > 64 * 1024)
-        MI355Q_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        if (mi355q_status st = raise_lds_limit((const void*)kern, lds)) return st;
     kern<<<dim3(grid, a.parts), dim3(KSPLIT * TPW * 64), lds, s>>>(a);
     MI355Q_HIP(hipGetLastError());
     return MI355Q_OK;

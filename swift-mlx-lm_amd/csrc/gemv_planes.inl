@@ -62,6 +62,7 @@ struct GemvArgs {
     uint32_t rows_per_wave;  // consecutive rows owned by one wavefront
     uint32_t y_dtype, sb_dtype;
     uint32_t x_dtype;        // MI355Q_BF16 or MI355Q_F16 (f16 needs XA = 1)
+    uint32_t gated;          // gated launches (GATED kernels): mi355q_gated_activation of the epilogue
 };
 
 // Host-side choice of kernel variant and launch shape.
@@ -73,6 +74,7 @@ struct GemvCfg {
     int xa;             // 0: bf16 activations and arithmetic; 1: f16
     bool rows;          // the static-structure kernel (gemv_rows_kernel) with `nct` K-steps per row, `br` rows per pass
     int nct, br;
+    bool gated;         // rows kernel over (gate, up) row pairs with the gated activation as epilogue
     uint32_t grid, rows_per_wave, nc;
     size_t lds;
 };

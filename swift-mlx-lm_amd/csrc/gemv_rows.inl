@@ -43,8 +43,15 @@ __host__ __device__ constexpr InplacePair inplace_pair3(int i) {
 
 // XA = 0: bf16 activations, bf16 code pairs (128 + q).  XA = 1: f16 activations, f16 code pairs (1024 + mult q,
 // fields of 2- and 4-bit codes used where they sit in the half-word, see f16_classes).
-template <int BITS, int GROUP, int NCT, int BR, int WAVES, int XA, bool SBBF16, bool ARGMAX>
+// GATED: the launch covers two matrices of equal shape (gate_proj, up_proj: MLPFragment's batched projection,
+// Sources/MetalCompiler/Compilable/MLPFragment.swift:7-27).  A wavefront's rows are then "virtual rows" 2 r (row r of
+// the first matrix) and 2 r + 1 (row r of the second), so a wavefront that owns a gate row owns the up row of the same
+// index, their sums are parked in neighbouring lanes, and the epilogue stores activation(gate) * up: one output
+// vector instead of two, and no elementwise launch (generateGatedActivation,
+// Generator/MetalSourceGenerator+NormAndElementwise.swift:196-249).
+template <int BITS, int GROUP, int NCT, int BR, int WAVES, int XA, bool SBBF16, bool ARGMAX, bool GATED = false>
 __global__ __launch_bounds__(WAVES * 64) void gemv_rows_kernel(GemvArgs a) {
+    static_assert(!(GATED && ARGMAX), "the gated epilogue has no arg-max tail");
     using G = GemvGeo<BITS>;
     constexpr int WPL = G::WPL, CPL = G::CPL;
     constexpr int Q = CPL / 8;
@@ -97,6 +104,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_rows_kernel(GemvArgs a) {
     }
     auto row_ptrs = [&](uint32_t r, const char*& cp, const char*& zp) {    // r: row inside the wavefront's share (scalar)
         r = r < last ? r : last;
+        if constexpr (GATED) {
+            const uint32_t vrow = rbase + r;
+            const uint64_t row = vrow >> 1;
+            cp = (const char*)((vrow & 1u) ? a.codes[1] : a.codes[0]) + row * cs_bytes;
+            zp = (const char*)((vrow & 1u) ? a.sz[1] : a.sz[0]) + row * ss_bytes;
+            return;
+        }
         const uint64_t row = rbase + r;
         cp = (const char*)seg_codes + row * cs_bytes;
         zp = (const char*)seg_sz + row * ss_bytes;
@@ -364,6 +378,19 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_rows_kernel(GemvArgs a) {
     if (passes) pass_body(passes - 1, std::false_type{});
 
     // ---- one coalesced store of the parked results (rows_per_wave <= 64) ------------------------------------
+    if constexpr (GATED) {
+        // lanes 2 r and 2 r + 1 hold the gate and the up sum of output row (row0 / 2 + r): both are rounded to the
+        // output type first, as the reference's elementwise kernel reads them back from buffers of that type
+        const float up_sum = __shfl_down(res, 1, 64);
+        if (lane < nrows && !(lane & 1u)) {
+            const uint32_t row = (row0 + lane) >> 1;
+            const float v = gated_value(res, up_sum, a.gated, a.y_dtype);
+            if (a.y_dtype == MI355Q_F32) ((float*)seg_y)[row] = v;
+            else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)seg_y)[row] = f32_to_bf16_rne(v);
+            else ((uint16_t*)seg_y)[row] = f32_to_f16_rne(v);
+        }
+        return;
+    }
     unsigned long long best = 0ull;
     if (lane < nrows) {
         const uint32_t row = row0 + lane;

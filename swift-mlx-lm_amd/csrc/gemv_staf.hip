@@ -388,7 +388,7 @@ mi355q_status launch_for_format(hipStream_t s, const StafArgs& a, int mt, int de
     const bool xreg = mt == 1 && a.nsp == 1;
     auto go = [&](auto kernel) -> mi355q_status {
         if (lds > 48 * 1024)
-            MI355Q_HIP(hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            if (mi355q_status st = raise_lds_limit((const void*)kernel, lds)) return st;
         hipLaunchKernelGGL(kernel, dim3(grid), dim3(kWaves * 64), lds, s, a);
         MI355Q_HIP(hipGetLastError());
         return MI355Q_OK;

@@ -388,7 +388,7 @@ template <int MR, int KSPLIT, int TPW, bool ARGMAX>
 mi355q_status launch_t16(hipStream_t s, const T16Args& a, uint32_t grid, size_t lds) {   // grid: workgroups of one K part
     auto kern = gemv_tile16_kernel<MR, KSPLIT, TPW, 4, ARGMAX>;
     if (lds > 64 * 1024)
-        MI355Q_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        if (mi355q_status st = raise_lds_limit((const void*)kern, lds)) return st;
     kern<<<dim3(grid, a.parts), dim3(KSPLIT * TPW * 64), lds, s>>>(a);
     MI355Q_HIP(hipGetLastError());
     return MI355Q_OK;

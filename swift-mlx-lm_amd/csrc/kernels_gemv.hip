@@ -221,6 +221,69 @@ mi355q_status launch_gemv_fast_multi(hipStream_t s, const mi355q_context* ctx, u
     return MI355Q_OK;
 }
 
+// Gate and up projection of ONE activation row with the gated activation as epilogue: the rows kernel over 2 N
+// "virtual rows" (2 r = row r of gate, 2 r + 1 = row r of up), launch shape chosen as for a matrix of 2 N rows.
+namespace {
+bool gated_cfg(const mi355q_context* ctx, const WView& gate, const WView& up, int x_dtype, uint32_t x_stride, GemvCfg& c) {
+    if (!gemv_fast_eligible(gate, x_dtype, 1, x_stride) || !gemv_fast_eligible(up, x_dtype, 1, x_stride)) return false;
+    if (gate.n != up.n || gate.k != up.k || gate.bits != up.bits || gate.group != up.group || gate.sb_dtype != up.sb_dtype ||
+        gate.code_stride != up.code_stride || gate.sz_stride != up.sz_stride) return false;
+    if ((uint64_t)gate.n * 2 > 0xFFFFFFFFull) return false;
+    WView all = gate;
+    all.n = gate.n * 2;
+    c = choose(ctx, all, 1, false, x_dtype);
+    if (!c.rows) return false;                             // rows of a length the static-structure kernel does not take
+    if (c.rows_per_wave & 1u) {                            // a wavefront owns whole (gate, up) pairs
+        c.rows_per_wave += (uint32_t)c.br;
+        if ((c.rows_per_wave & 1u) || c.rows_per_wave > 64) return false;
+    }
+    c.gated = true;
+    return true;
+}
+}  // namespace
+
+bool gemv_gated_eligible(const mi355q_context* ctx, const WView& gate, const WView& up, int x_dtype, uint32_t m, uint32_t x_stride) {
+    GemvCfg c{};
+    return m == 1 && gated_cfg(ctx, gate, up, x_dtype, x_stride, c);
+}
+
+mi355q_status launch_gemv_gated(hipStream_t s, const mi355q_context* ctx, const WView& gate, const WView& up, const void* x,
+                                int x_dtype, void* y, int y_dtype, uint32_t x_stride, int activation) {
+    GemvCfg c{};
+    if (!gated_cfg(ctx, gate, up, x_dtype, x_stride, c))
+        return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no one-launch gated projection for these weights");
+    if ((uintptr_t)x % 16) return fail(MI355Q_ERR_INVALID_ARGUMENT, "activation pointer must be 16-byte aligned");
+    GemvArgs a{};
+    const uint32_t vrows = gate.n * 2;
+    const uint32_t waves = (vrows + c.rows_per_wave - 1) / c.rows_per_wave;
+    for (int i = 0; i < kGemvMaxSegments; i++) {
+        a.codes[i] = i == 0 ? gate.codes : up.codes;
+        a.sz[i] = i == 0 ? gate.sz : up.sz;
+        a.y[i] = y;
+        a.y_stride[i] = gate.n;
+        a.seg_rows[i] = vrows;
+        a.wave_end[i] = waves;
+    }
+    a.x = (const uint16_t*)x;
+    a.k = gate.k; a.m = 1;
+    a.x_stride = x_stride;
+    a.code_stride = gate.code_stride; a.sz_stride = gate.sz_stride;
+    a.nc = c.nc; a.rows_per_wave = c.rows_per_wave;
+    a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = gate.sb_dtype; a.x_dtype = (uint32_t)x_dtype;
+    a.gated = (uint32_t)activation;
+    c.grid = (waves + (uint32_t)c.waves - 1) / (uint32_t)c.waves;
+    switch (gate.bits) {
+    case 2: return launch_gemv_planes_q2(s, a, (int)gate.group, c);
+    case 3: return launch_gemv_planes_q3(s, a, (int)gate.group, c);
+    case 4: return launch_gemv_planes_q4(s, a, (int)gate.group, c);
+    case 5: return launch_gemv_planes_q5(s, a, (int)gate.group, c);
+    case 6: return launch_gemv_planes_q6(s, a, (int)gate.group, c);
+    case 8: return launch_gemv_planes_q8(s, a, (int)gate.group, c);
+    default: break;
+    }
+    return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no split-plane GEMV for %u-bit codes", gate.bits);
+}
+
 mi355q_status launch_gemv_fast(hipStream_t s, const mi355q_context* ctx, const WView& w, const void* x, int x_dtype,
                                void* y, int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride, float* logits_f32,
                                int32_t* token_out, HeadKeys keys) {

@@ -237,6 +237,38 @@ mi355q_status launch_embedding_lookup(hipStream_t s, const WView& w, const int32
     return MI355Q_OK;
 }
 
+// ------------------------------------------------------------------------------ gated activation (SwiGLU / GEGLU)
+// out[s, i] = T(activation(float(gate[s, i])) * float(up[s, i])): the reference's swiglu / gelu_gated elementwise kernel
+// (Sources/MetalCompiler/Generator/MetalSourceGenerator+NormAndElementwise.swift:196-249), one element per thread.
+__global__ __launch_bounds__(256) void gated_activation_kernel(const void* __restrict__ gate, const void* __restrict__ up,
+                                                              void* __restrict__ out, uint32_t dtype, uint32_t dimension,
+                                                              uint32_t sequence_length, uint32_t gate_stride,
+                                                              uint32_t up_stride, uint32_t out_stride, uint32_t activation) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= dimension) return;
+    for (uint32_t sq = blockIdx.y; sq < sequence_length; sq += gridDim.y) {
+        const size_t gi = (size_t)sq * gate_stride + i, ui = (size_t)sq * up_stride + i, oi = (size_t)sq * out_stride + i;
+        float g, u;
+        if (dtype == MI355Q_F32) { g = ((const float*)gate)[gi]; u = ((const float*)up)[ui]; }
+        else if (dtype == MI355Q_BF16) { g = bf16_to_f32(((const uint16_t*)gate)[gi]); u = bf16_to_f32(((const uint16_t*)up)[ui]); }
+        else { g = f16_to_f32(((const uint16_t*)gate)[gi]); u = f16_to_f32(((const uint16_t*)up)[ui]); }
+        const float v = gated_value(g, u, activation, MI355Q_F32);
+        if (dtype == MI355Q_F32) ((float*)out)[oi] = v;
+        else if (dtype == MI355Q_BF16) ((uint16_t*)out)[oi] = f32_to_bf16_rne(v);
+        else ((uint16_t*)out)[oi] = f32_to_f16_rne(v);
+    }
+}
+
+mi355q_status launch_gated_activation(hipStream_t s, const void* gate, const void* up, void* out, int dtype, uint32_t dimension,
+                                      uint32_t sequence_length, uint32_t gate_stride, uint32_t up_stride, uint32_t out_stride,
+                                      int activation) {
+    const dim3 grid((dimension + 255u) / 256u, sequence_length < 65535u ? sequence_length : 65535u);
+    gated_activation_kernel<<<grid, dim3(256), 0, s>>>(gate, up, out, (uint32_t)dtype, dimension, sequence_length, gate_stride,
+                                                       up_stride, out_stride, (uint32_t)activation);
+    MI355Q_HIP(hipGetLastError());
+    return MI355Q_OK;
+}
+
 // ------------------------------------------------------------------------------ dequant to bf16 / fp32
 // One workgroup per row, 256 threads striding over the row, as the reference kernel does.
 // scale*q and +zero are kept as two roundings so the result is bit-identical to an unfused

@@ -1,7 +1,9 @@
 // Context, device memory, streams, events and packed-weight handles.
-#include <mutex>
 #include <new>
 #include <vector>
+
+#include <mutex>
+#include <unordered_map>
 
 #include "common.h"
 
@@ -65,6 +67,10 @@ mi355q_status ensure_workspace(mi355q_context* ctx, size_t bytes) {
 
 mi355q_status ensure_split_buffer(mi355q_context* ctx, size_t bytes) {
     return grow_scratch(ctx, ctx->split_buffer, ctx->split_bytes, bytes, (size_t)1 << 20);
+}
+
+mi355q_status ensure_gated_buffer(mi355q_context* ctx, size_t bytes) {
+    return grow_scratch(ctx, ctx->gated_buffer, ctx->gated_bytes, bytes, (size_t)1 << 20);
 }
 
 }  // namespace mi355q
@@ -248,6 +254,23 @@ mi355q_status need_ctx(mi355q_context* ctx) {
 
 }  // namespace
 
+namespace mi355q {
+// hipFuncSetAttribute belongs to a function on one device: remember the largest size asked per (function, device)
+mi355q_status raise_lds_limit(const void* kernel, size_t lds_bytes) {
+    static std::mutex mu;
+    static std::unordered_map<uint64_t, size_t> raised;
+    int device = 0;
+    MI355Q_HIP(hipGetDevice(&device));
+    const uint64_t key = (uint64_t)(uintptr_t)kernel * 64u + (uint64_t)(device & 63);
+    std::lock_guard<std::mutex> lock(mu);
+    auto it = raised.find(key);
+    if (it != raised.end() && it->second >= lds_bytes) return MI355Q_OK;
+    MI355Q_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+    raised[key] = lds_bytes;
+    return MI355Q_OK;
+}
+}  // namespace mi355q
+
 extern "C" {
 
 // ---------------------------------------------------------------------------------- context
@@ -309,6 +332,7 @@ mi355q_status mi355q_context_destroy(mi355q_context* ctx) {
     if (ctx->argmax_partials) (void)hipFree(ctx->argmax_partials);
     if (ctx->workspace) (void)hipFree(ctx->workspace);
     if (ctx->split_buffer) (void)hipFree(ctx->split_buffer);
+    if (ctx->gated_buffer) (void)hipFree(ctx->gated_buffer);
     for (int i = 0; i < ctx->retired_count; i++) (void)hipFree(ctx->retired[i]);
     delete ctx;
     return MI355Q_OK;

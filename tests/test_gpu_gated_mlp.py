@@ -1,0 +1,176 @@
+"""GPU parity tests of the gated MLP's first half -- gate_proj + up_proj + swiglu / gelu_gated -- through the C ABI.
+
+Reference: MLPFragment (Sources/MetalCompiler/Compilable/MLPFragment.swift:7-27) = batched gate + up projection, then
+the elementwise kernel of Generator/MetalSourceGenerator+NormAndElementwise.swift:196-249, which reads gate and up back
+from buffers of the activation type.  Expected values: the oracle's fp64 projections, rounded to the buffer type, through
+the oracle's restatement of the elementwise kernel.  Bars: relative L2 <= 1e-3 and max-abs <= 2e-2 on fp32 results; a
+16-bit result may differ from the expected one by one step of its type where the fp32 sums differ in their last bits.
+"""
+import sys
+
+import numpy as np
+import pytest
+
+import kat
+import oracle
+from gpu_util import act_rounded, act_to_device_array, assert_within_tolerance, out_from_device, rel_l2, seeded_case
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def _o_dtype(pkg, d):
+    return {pkg.F32: oracle.F32, pkg.BF16: oracle.BF16, pkg.F16: oracle.F16}[d]
+
+
+def test_elementwise_kernel_closed_forms_and_oracle(pkg, ctx):
+    """The elementwise step alone: closed forms (silu(0) = 0, gelu(0) = 0, large g -> g * u, very negative g -> -0 * u,
+    u = 0 -> 0) and seeded values against the oracle, every buffer type, padded rows."""
+    g = np.array([0.0, 30.0, -100.0, 1.0, -1.0, 5.0, 0.5, 88.0], np.float32)
+    u = np.array([3.0, 2.0, 7.0, 1.0, 1.0, 0.0, -4.0, 0.5], np.float32)
+    for kind in (pkg.GATED_SILU, pkg.GATED_GELU_TANH):
+        gd, ud, od = ctx.upload(g), ctx.upload(u), ctx.alloc(g.size * 4)
+        ctx.gated_activation(gd, ud, od, pkg.F32, g.size, activation=kind)
+        ctx.synchronize()
+        got = od.download(np.float32)
+        assert got[0] == 0.0 and got[1] == 60.0 and got[5] == 0.0 and got[7] == 44.0
+        assert got[2] == 0.0                                            # silu(-100) = -100 / (1 + inf) = -0
+        want1 = 1.0 / (1.0 + np.exp(-1.0)) if kind == pkg.GATED_SILU else 0.5 * (1.0 + np.tanh(0.7978845608 * 1.044715))
+        assert abs(got[3] - want1) < 2e-7
+        assert np.allclose(got, oracle.gated_activation_f32(g, u, kind, oracle.F32), rtol=2e-6, atol=2e-6)
+        for b in (gd, ud, od):
+            b.free()
+    rng = np.random.default_rng(5)
+    seq, dim, stride = 3, 1000, 1008
+    for dt in (pkg.F32, pkg.BF16, pkg.F16):
+        gs = act_rounded((rng.standard_normal((seq, stride)) * 3).astype(np.float32), dt, pkg)
+        us = act_rounded(rng.standard_normal((seq, stride)).astype(np.float32), dt, pkg)
+        for kind in (pkg.GATED_SILU, pkg.GATED_GELU_TANH):
+            gd, ud = ctx.upload(act_to_device_array(gs, dt, pkg)), ctx.upload(act_to_device_array(us, dt, pkg))
+            od = ctx.alloc(seq * stride * (4 if dt == pkg.F32 else 2))
+            ctx.fill(od, 0x7FC07FC0 if dt != pkg.F32 else 0x7FC00000)
+            ctx.gated_activation(gd, ud, od, dt, dim, seq, stride, kind)
+            ctx.synchronize()
+            got = out_from_device(od, dt, (seq, stride), pkg)
+            assert np.all(np.isnan(got[:, dim:])), "row padding was written"
+            want = oracle.gated_activation_f32(gs[:, :dim], us[:, :dim], kind, _o_dtype(pkg, dt))
+            step = {pkg.F32: 2e-6, pkg.BF16: 2.0 ** -7, pkg.F16: 2.0 ** -10}[dt]     # at most one step of the type
+            # (1 + tanh cancels for negative g: the device's tanh and the host's differ by a few fp32 steps of |g u|)
+            slack = 1e-6 * np.abs(gs[:, :dim] * us[:, :dim])
+            assert np.all(np.abs(got[:, :dim] - want) <= step * np.maximum(np.abs(want), 1e-3) + slack), (dt, kind)
+            for b in (gd, ud, od):
+                b.free()
+
+
+def _expected(pkg, wq_g, wq_u, x, kind, y_dtype):
+    """Expected result and how far one step of the buffer type on the gate and up sums moves it."""
+    gate = oracle.gemm_f64(wq_g, x).astype(np.float32)
+    up = oracle.gemm_f64(wq_u, x).astype(np.float32)
+    od = _o_dtype(pkg, y_dtype)
+    want = oracle.gated_activation_f32(gate, up, kind, od)
+    step = {pkg.F32: 2.0 ** -22, pkg.BF16: 2.0 ** -8, pkg.F16: 2.0 ** -11}[y_dtype]
+    moved = np.zeros_like(want)
+    for sg in (1 - step, 1 + step):
+        for su in (1 - step, 1 + step):
+            moved = np.maximum(moved, np.abs(oracle.gated_activation_f32(gate * np.float32(sg), up * np.float32(su), kind, od) - want))
+    # ... and how far an absolute error of a few 1e-5 of the sums themselves (fp32 accumulation order; f16 code pairs with
+    # f16 activations) moves it: |d act(g) u| <= 1.13 (|u| dg + |du|)
+    moved += np.float32(4e-5) * (1.0 + np.abs(up))
+    return want, moved
+
+
+def _check(pkg, got, expected, y_dtype, what):
+    want, moved = expected
+    if y_dtype != pkg.F32:
+        # the gate and up sums are rounded to the buffer type before the activation: a sum whose last fp32 bits differ
+        # from the oracle's may round the other way, one step of the type, and the activation passes that on
+        step = 2.0 ** -7 if y_dtype == pkg.BF16 else 2.0 ** -10
+        # (a flipped rounding of the gate moves the product by up to two steps of the output, whose own rounding adds one)
+        assert np.all(np.abs(got - want) <= moved + 3 * step * np.abs(want)), what
+        assert rel_l2(got, want) <= 1e-3, what        # (max-abs 2e-2 is less than one bf16 step from |y| = 4 on)
+        return
+    assert_within_tolerance(got, want, what)
+
+
+@pytest.mark.parametrize("bits,group,n,k", [(4, 64, 14336, 4096), (4, 128, 1000, 2048), (8, 32, 520, 4096), (3, 64, 300, 4096),
+                                            (4, 64, 333, 8192)])
+def test_gated_projection_one_row(pkg, ctx, bits, group, n, k):
+    """M = 1 on split planes: one launch (a wavefront owns a gate row and the up row of the same index), every output
+    type, bf16 and f16 activations, both activations; Llama-3-8B's gate / up shape among the cases."""
+    wg, sg, zg, wq_g = seeded_case(6000 + bits, n, k, bits, group)
+    wu, su, zu, wq_u = seeded_case(6100 + bits, n, k, bits, group)
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(bits, group)
+    g = ctx.weight_prepare_mlx(fmt, wg, sg, zg, pkg.BF16, pkg.LAYOUT_PLANES)
+    u = ctx.weight_prepare_mlx(fmt, wu, su, zu, pkg.BF16, pkg.LAYOUT_PLANES)
+    for xd in ((pkg.BF16, pkg.F16) if bits in (4, 8) else (pkg.BF16,)):
+        x = act_rounded(kat.seeded_activations(6200 + k, 1, k), xd, pkg)
+        xdev = ctx.upload(act_to_device_array(x, xd, pkg))
+        for yd in (pkg.F32, pkg.BF16, pkg.F16):
+            for kind in (pkg.GATED_SILU, pkg.GATED_GELU_TANH):
+                say(f"gated q{bits}g{group} {k}->{n} x={xd} y={yd} act={kind}")
+                ydev = ctx.alloc(n * (4 if yd == pkg.F32 else 2))
+                ctx.gated_qgemm(g, u, xdev, xd, ydev, yd, 1, kind)
+                ctx.synchronize()
+                got = out_from_device(ydev, yd, (1, n), pkg) if yd != pkg.F32 else ydev.download(np.float32, (1, n))
+                _check(pkg, got, _expected(pkg, wq_g, wq_u, x, kind, yd), yd, f"gated q{bits}g{group} y={yd}")
+                ydev.free()
+        xdev.free()
+    g.destroy(); u.destroy()
+
+
+def test_gated_projection_equals_batched_projection_then_elementwise(pkg, ctx):
+    """Every other shape runs the two projections into scratch and then the elementwise kernel: M = 1 on blocks in place
+    and on TILE16 records, M = 5, 40 and 300 on planes -- equal, bit for bit, to mi355q_batched_qgemm followed by
+    mi355q_gated_activation_apply, and within the bar of the oracle."""
+    n, k = 520, 2048
+    wg, sg, zg, wq_g = seeded_case(6300, n, k, 4, 64)
+    wu, su, zu, wq_u = seeded_case(6301, n, k, 4, 64)
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+    for layout, ms in ((pkg.LAYOUT_PLANES, (5, 40, 300)), (pkg.LAYOUT_TILE16, (1, 9)), (pkg.LAYOUT_STAF_BLOCKS, (1, 3))):
+        sb = pkg.BF16
+        if layout == pkg.LAYOUT_STAF_BLOCKS:       # blocks keep f16 headers: quantise with f16 scales
+            wg2, sg2, zg2 = oracle.quantize_affine(kat.seeded_weights(6300, n, k), 4, 64, oracle.F16)
+            wu2, su2, zu2 = oracle.quantize_affine(kat.seeded_weights(6301, n, k), 4, 64, oracle.F16)
+            g = ctx.weight_prepare_mlx(fmt, wg2, sg2, zg2, pkg.F16, layout)
+            u = ctx.weight_prepare_mlx(fmt, wu2, su2, zu2, pkg.F16, layout)
+            dq_g = oracle.dequant_planes_f32(4, 64, n, k, wg2, sg2, zg2, oracle.F16)
+            dq_u = oracle.dequant_planes_f32(4, 64, n, k, wu2, su2, zu2, oracle.F16)
+        else:
+            g = ctx.weight_prepare_mlx(fmt, wg, sg, zg, sb, layout)
+            u = ctx.weight_prepare_mlx(fmt, wu, su, zu, sb, layout)
+            dq_g, dq_u = wq_g, wq_u
+        for m in ms:
+            x = act_rounded(kat.seeded_activations(6400 + m, m, k), pkg.BF16, pkg)
+            xdev = ctx.upload(act_to_device_array(x, pkg.BF16, pkg))
+            yd = pkg.BF16
+            say(f"gated layout={layout} M={m}")
+            fused, gate_b, up_b, two = ctx.alloc(m * n * 2), ctx.alloc(m * n * 2), ctx.alloc(m * n * 2), ctx.alloc(m * n * 2)
+            ctx.gated_qgemm(g, u, xdev, pkg.BF16, fused, yd, m, pkg.GATED_SILU)
+            ctx.batched_qgemm([g, u], xdev, pkg.BF16, [gate_b, up_b], yd, m)
+            ctx.gated_activation(gate_b, up_b, two, yd, n, m, 0, pkg.GATED_SILU)
+            ctx.synchronize()
+            a, b = fused.download(np.uint16, (m, n)), two.download(np.uint16, (m, n))
+            assert np.array_equal(a, b), "gated call != batched projection + elementwise kernel"
+            got = oracle.bf16_to_f32(a).reshape(m, n)
+            if m <= 32:      # few rows: unrounded weights on every route (beyond, the weights are rounded to bf16)
+                _check(pkg, got, _expected(pkg, dq_g, dq_u, x, pkg.GATED_SILU, yd), yd, f"layout {layout} M={m}")
+            for t in (xdev, fused, gate_b, up_b, two):
+                t.free()
+        g.destroy(); u.destroy()
+
+
+def test_gated_projection_rejects_mismatched_weights(pkg, ctx):
+    wa, sa, za, _ = seeded_case(6500, 64, 256, 4, 64)
+    wb, sb_, zb, _ = seeded_case(6501, 128, 256, 4, 64)
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+    a = ctx.weight_prepare_mlx(fmt, wa, sa, za, pkg.BF16, pkg.LAYOUT_PLANES)
+    b = ctx.weight_prepare_mlx(fmt, wb, sb_, zb, pkg.BF16, pkg.LAYOUT_PLANES)
+    x, y = ctx.alloc(256 * 2), ctx.alloc(128 * 4)
+    with pytest.raises(pkg.MI355QError):
+        ctx.gated_qgemm(a, b, x, pkg.BF16, y, pkg.F32, 1)
+    with pytest.raises(pkg.MI355QError):
+        ctx.gated_qgemm(a, a, x, pkg.BF16, y, pkg.F32, 1, activation=7)
+    a.destroy(); b.destroy(); x.free(); y.free()

@@ -410,3 +410,33 @@ def test_embedding_lookup_is_a_row_gather_of_the_dequantised_table():
     with pytest.raises(ValueError):
         oracle.embedding_lookup_staf_f32(4, 64, 2, 64, kat.staf_blocks(np.zeros((2, 64), np.uint8), np.ones((2, 1)),
                                                                         np.zeros((2, 1)), 4, 64), [2])
+
+
+# ------------------------------------------------------------------ gated activation (swiglu / gelu_gated)
+def test_gated_activation_closed_forms_and_fp64():
+    """The reference holds no value test of its gated-activation kernels, so the restatement is pinned by what the
+    formulas fix: act(0) = 0, u = 0 -> 0, large g -> g u exactly (sigmoid and tanh saturate to 1 in fp32), very negative
+    g -> 0 (exp overflows to inf), silu(1) and gelu_tanh(1) from their definitions, and an fp64 evaluation of both
+    formulas on seeded values; with a 16-bit buffer type, gate, up and the product are each rounded to it."""
+    g = np.array([0.0, 30.0, -100.0, 1.0, 5.0, 88.0, -0.0], np.float32)
+    u = np.array([3.0, 2.0, 7.0, 1.0, 0.0, 0.5, 2.0], np.float32)
+    for kind in (oracle.SILU, oracle.GELU_TANH):
+        out = oracle.gated_activation_f32(g, u, kind)
+        assert out[0] == 0.0 and out[1] == 60.0 and out[2] == 0.0 and out[4] == 0.0 and out[5] == 44.0 and out[6] == 0.0
+    assert abs(oracle.gated_activation_f32(g, u, oracle.SILU)[3] - 1.0 / (1.0 + np.exp(-1.0))) < 1e-7
+    assert abs(oracle.gated_activation_f32(g, u, oracle.GELU_TANH)[3] - 0.5 * (1.0 + np.tanh(0.7978845608 * 1.044715))) < 1e-7
+    rng = np.random.default_rng(12)
+    gs = (rng.standard_normal(4000) * 4).astype(np.float32)
+    us = rng.standard_normal(4000).astype(np.float32)
+    g64, u64 = gs.astype(np.float64), us.astype(np.float64)
+    silu = g64 / (1.0 + np.exp(-g64)) * u64
+    gelu = 0.5 * g64 * (1.0 + np.tanh(0.7978845608 * (g64 + 0.044715 * g64 ** 3))) * u64
+    assert np.allclose(oracle.gated_activation_f32(gs, us, oracle.SILU), silu, rtol=3e-6, atol=1e-7)
+    # 1 + tanh cancels for negative g: an absolute error of a few fp32 steps of |g u|
+    assert np.allclose(oracle.gated_activation_f32(gs, us, oracle.GELU_TANH), gelu, rtol=1e-5, atol=5e-6)
+    # a sign error, a dropped cubic term or a transposed operand moves these by far more than the bars above
+    assert not np.allclose(oracle.gated_activation_f32(gs, us, oracle.SILU), gelu, rtol=1e-3, atol=1e-4)
+    # buffer type bf16: inputs and output on the bf16 grid
+    gb = oracle.bf16_to_f32(oracle.bf16_from_f32(gs)); ub = oracle.bf16_to_f32(oracle.bf16_from_f32(us))
+    want = oracle.bf16_to_f32(oracle.bf16_from_f32(oracle.gated_activation_f32(gb, ub, oracle.SILU)))
+    assert np.array_equal(oracle.gated_activation_f32(gs, us, oracle.SILU, oracle.BF16), want)
