@@ -541,6 +541,15 @@ MI355Q_API mi355q_status mi355q_plan_add_batched_linear(mi355q_plan* plan, uint3
                                                         uint32_t m, uint32_t x_row_stride,
                                                         uint32_t flags, int32_t layer_index,
                                                         const char* tensor_name);
+/* One step for MLPFragment's gate_proj + up_proj + elementwise activation (bindings as mi355q_gated_qgemm;
+ * MC/Compilable/MLPFragment.swift:7-14).  The step record's kernel family is gatedFused... when the activation is the
+ * projection launch's epilogue, gatedBatched2... when the elementwise kernel follows the batched projection. */
+MI355Q_API mi355q_status mi355q_plan_add_gated_mlp(mi355q_plan* plan, const mi355q_weight* w_gate,
+                                                   const mi355q_weight* w_up, const void* x_dev,
+                                                   mi355q_dtype x_dtype, void* y_dev, mi355q_dtype y_dtype,
+                                                   uint32_t m, uint32_t x_row_stride, uint32_t y_row_stride,
+                                                   mi355q_gated_activation activation, uint32_t flags,
+                                                   int32_t layer_index, const char* tensor_name);
 /* One OutputHeadFragment step (bindings as mi355q_lmhead_argmax). */
 MI355Q_API mi355q_status mi355q_plan_add_output_head(mi355q_plan* plan, const mi355q_weight* w,
                                                      const void* x_dev, mi355q_dtype x_dtype,

@@ -171,6 +171,7 @@ def library() -> C.CDLL:
         "mi355q_plan_add_linear": (i32, [vp, vp, vp, C.c_int, vp, C.c_int, u32, u32, u32, u32, i32, C.c_char_p]),
         "mi355q_plan_add_batched_linear": (i32, [vp, u32, vp, vp, C.c_int, vp, C.c_int, u32, u32, u32, i32,
                                                   C.c_char_p]),
+        "mi355q_plan_add_gated_mlp": (i32, [vp, vp, vp, vp, C.c_int, vp, C.c_int, u32, u32, u32, C.c_int, u32, i32, C.c_char_p]),
         "mi355q_plan_add_output_head": (i32, [vp, vp, vp, C.c_int, vp, vp, u32, C.c_char_p]),
         "mi355q_plan_step_count": (i32, [vp]),
         "mi355q_plan_step_at": (i32, [vp, i32, P(_Step), P(i32), C.c_char_p, sz]),
@@ -429,6 +430,14 @@ class DispatchPlan:
                                                         x_row_stride, flags, layer_index,
                                                         tensor_name.encode() if tensor_name else None))
         self._keep.append((list(weights), x, list(ys)))
+
+    def add_gated_mlp(self, w_gate, w_up, x, x_dtype, y, y_dtype, m=1, activation=GATED_SILU, x_row_stride=0,
+                      y_row_stride=0, flags=0, layer_index=-1, tensor_name: str | None = None):
+        """gate_proj + up_proj + swiglu / gelu_gated as one step: y = act(x Wgate^T) * (x Wup^T)."""
+        _check(library().mi355q_plan_add_gated_mlp(self.handle, w_gate.handle, w_up.handle, Context._ptr(x), x_dtype,
+                                                   Context._ptr(y), y_dtype, m, x_row_stride, y_row_stride, activation,
+                                                   flags, layer_index, tensor_name.encode() if tensor_name else None))
+        self._keep.append(([w_gate, w_up], x, y))
 
     def add_output_head(self, w: "PackedWeight", x, x_dtype, logits_f32, token_out, flags=0,
                         tensor_name: str | None = None):

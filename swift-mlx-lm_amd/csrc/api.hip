@@ -691,20 +691,17 @@ extern "C" mi355q_status mi355q_gated_activation_apply(mi355q_context* ctx, void
                                    row_stride, row_stride, activation);
 }
 
-extern "C" mi355q_status mi355q_gated_qgemm(mi355q_context* ctx, void* stream, const mi355q_weight* w_gate,
-                                            const mi355q_weight* w_up, const void* x_dev, mi355q_dtype x_dtype,
-                                            void* y_dev, mi355q_dtype y_dtype, uint32_t m, uint32_t x_row_stride,
-                                            uint32_t y_row_stride, mi355q_gated_activation activation, uint32_t flags) {
-    if (mi355q_status st = check_launch(ctx, w_gate)) return st;
-    if (mi355q_status st = check_launch(ctx, w_up)) return st;
+namespace mi355q {
+mi355q_status dispatch_gated(mi355q_context* ctx, hipStream_t s, const mi355q_weight* w_gate, const mi355q_weight* w_up,
+                             const void* x_dev, int x_dtype, void* y_dev, int y_dtype, uint32_t m, uint32_t xs, uint32_t ys,
+                             int activation, uint32_t flags) {
     if (activation != MI355Q_GATED_SILU && activation != MI355Q_GATED_GELU_TANH)
-        return fail(MI355Q_ERR_INVALID_ARGUMENT, "unknown gated activation %d", (int)activation);
+        return fail(MI355Q_ERR_INVALID_ARGUMENT, "unknown gated activation %d", activation);
     if (w_gate->n != w_up->n || w_gate->k != w_up->k || w_gate->fmt.scheme_identifier != w_up->fmt.scheme_identifier ||
         w_gate->layout != w_up->layout)
         return fail(MI355Q_ERR_SHAPE, "gate and up projections must share N, K, scheme and layout");
-    uint32_t xs = x_row_stride, ys = y_row_stride;
+    if (x_dtype == MI355Q_F32) return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the gated projection takes bf16 or f16 activations");
     if (mi355q_status st = check_io(w_gate, x_dev, x_dtype, y_dev, y_dtype, m, xs, ys)) return st;
-    hipStream_t s = (hipStream_t)stream;
     const WView g = w_gate->view(), u = w_up->view();
     const uint32_t n = (uint32_t)w_gate->n;
     if (!(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_TWO_STEP |
@@ -722,4 +719,15 @@ extern "C" mi355q_status mi355q_gated_qgemm(mi355q_context* ctx, void* stream, c
     void* ys2[2] = {gate_out, up_out};
     if (mi355q_status st = dispatch_batched(ctx, s, 2, ws, x_dev, x_dtype, ys2, y_dtype, m, xs, flags)) return st;
     return launch_gated_activation(s, gate_out, up_out, y_dev, y_dtype, n, m, n, n, ys, activation);
+}
+}  // namespace mi355q
+
+extern "C" mi355q_status mi355q_gated_qgemm(mi355q_context* ctx, void* stream, const mi355q_weight* w_gate,
+                                            const mi355q_weight* w_up, const void* x_dev, mi355q_dtype x_dtype,
+                                            void* y_dev, mi355q_dtype y_dtype, uint32_t m, uint32_t x_row_stride,
+                                            uint32_t y_row_stride, mi355q_gated_activation activation, uint32_t flags) {
+    if (mi355q_status st = check_launch(ctx, w_gate)) return st;
+    if (mi355q_status st = check_launch(ctx, w_up)) return st;
+    return dispatch_gated(ctx, (hipStream_t)stream, w_gate, w_up, x_dev, x_dtype, y_dev, y_dtype, m, x_row_stride, y_row_stride,
+                          activation, flags);
 }

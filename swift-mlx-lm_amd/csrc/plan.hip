@@ -12,7 +12,7 @@ using namespace mi355q;
 
 namespace {
 
-enum StepKind { kLinear = 0, kOutputHead = 1, kBatched = 2 };
+enum StepKind { kLinear = 0, kOutputHead = 1, kBatched = 2, kGated = 3 };
 
 struct PlanStep {
     StepKind kind;
@@ -29,6 +29,7 @@ struct PlanStep {
     uint32_t count;
     const mi355q_weight* ws[3];
     void* ysv[3];
+    int activation;     // kGated: ws[0] = gate_proj, ws[1] = up_proj, y = the one output
 };
 
 }  // namespace
@@ -52,6 +53,9 @@ mi355q_status encode_range(mi355q_plan* plan, hipStream_t s, uint32_t first, uin
         if (st.kind == kLinear)
             rc = dispatch_linear(plan->ctx, s, st.w, st.x, st.x_dtype, st.y, st.y_dtype, st.m, st.xs, st.ys, st.flags,
                                  false);
+        else if (st.kind == kGated)
+            rc = dispatch_gated(plan->ctx, s, st.ws[0], st.ws[1], st.x, st.x_dtype, st.y, st.y_dtype, st.m, st.xs, st.ys,
+                                st.activation, st.flags);
         else if (st.kind == kBatched)
             rc = dispatch_batched(plan->ctx, s, st.count, st.ws, st.x, st.x_dtype, st.ysv, st.y_dtype, st.m, st.xs,
                                   st.flags);
@@ -164,6 +168,61 @@ mi355q_status mi355q_plan_add_batched_linear(mi355q_plan* plan, uint32_t count, 
     if (m <= 8) plan_shared_launch_shape(weights, count, m, x_dtype, st.xs, &st.record);   // one launch over the rows of all matrices
     std::snprintf(st.record.kernel_family, sizeof st.record.kernel_family, "batched%uQ%uG%u", count,
                   (unsigned)weights[0]->fmt.bits, weights[0]->fmt.group_size);
+    plan->steps.push_back(st);
+    return MI355Q_OK;
+}
+
+mi355q_status mi355q_plan_add_gated_mlp(mi355q_plan* plan, const mi355q_weight* w_gate, const mi355q_weight* w_up,
+                                        const void* x_dev, mi355q_dtype x_dtype, void* y_dev, mi355q_dtype y_dtype, uint32_t m,
+                                        uint32_t x_row_stride, uint32_t y_row_stride, mi355q_gated_activation activation,
+                                        uint32_t flags, int32_t layer_index, const char* tensor_name) {
+    if (!plan) return fail(MI355Q_ERR_NULL_HANDLE, "plan is null");
+    if (!w_gate || !w_up) return fail(MI355Q_ERR_NULL_HANDLE, "weight handle is null");
+    if (w_gate->ctx != plan->ctx || w_up->ctx != plan->ctx)
+        return fail(MI355Q_ERR_INVALID_ARGUMENT, "weight handle belongs to another context");
+    if (!x_dev || !y_dev) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null activation or output pointer");
+    if (m == 0) return fail(MI355Q_ERR_INVALID_ARGUMENT, "sequence length M must be >= 1");
+    if (activation != MI355Q_GATED_SILU && activation != MI355Q_GATED_GELU_TANH)
+        return fail(MI355Q_ERR_INVALID_ARGUMENT, "unknown gated activation %d", (int)activation);
+    if (w_gate->n != w_up->n || w_gate->k != w_up->k || w_gate->fmt.scheme_identifier != w_up->fmt.scheme_identifier ||
+        w_gate->layout != w_up->layout)
+        return fail(MI355Q_ERR_SHAPE, "gate and up projections must share N, K, scheme and layout");
+    if (plan->graph_exec) return fail(MI355Q_ERR_INVALID_ARGUMENT, "plan is frozen: its graph has been built");
+    PlanStep st{};
+    st.kind = kGated;
+    st.count = 2;
+    st.ws[0] = w_gate; st.ws[1] = w_up;
+    st.w = w_gate; st.x = x_dev; st.y = y_dev; st.token = nullptr;
+    st.x_dtype = x_dtype; st.y_dtype = y_dtype;
+    st.m = m;
+    st.xs = x_row_stride ? x_row_stride : (uint32_t)w_gate->k;
+    st.ys = y_row_stride ? y_row_stride : (uint32_t)w_gate->n;
+    st.flags = flags;
+    st.activation = activation;
+    st.layer_index = layer_index;
+    if (tensor_name) st.tensor_name = tensor_name;
+    mi355q_status rc;
+    if (m <= 8) {
+        rc = mi355q_plan_decode_step(w_gate, m, x_dtype, flags, &st.record);
+    } else {
+        mi355q_step two[2];
+        uint32_t cnt = 0;
+        rc = mi355q_plan_prefill_steps(w_gate, m, st.xs, x_dtype, 0, flags, two, &cnt);
+        st.record = two[0];
+    }
+    if (rc != MI355Q_OK) return rc;
+    const mi355q_weight* both[2] = {w_gate, w_up};
+    if (m <= 8) plan_shared_launch_shape(both, 2, m, x_dtype, st.xs, &st.record);
+    // one launch with the activation as its epilogue, or the batched projection followed by the elementwise kernel
+    const bool one_launch = !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_MFMA |
+                                       MI355Q_FLAG_FORCE_TWO_STEP | MI355Q_FLAG_FORCE_STREAM)) &&
+                            gemv_gated_eligible(plan->ctx, w_gate->view(), w_up->view(), x_dtype, m, st.xs);
+    const char* const act = activation == MI355Q_GATED_SILU ? "swiglu" : "gelu_gated";
+    char name[sizeof st.record.device_kernel];
+    std::snprintf(name, sizeof name, "%s%s%s", st.record.device_kernel, one_launch ? "+" : " ; ", act);
+    std::snprintf(st.record.device_kernel, sizeof st.record.device_kernel, "%s", name);
+    std::snprintf(st.record.kernel_family, sizeof st.record.kernel_family, "%sQ%uG%u", one_launch ? "gatedFused" : "gatedBatched2",
+                  (unsigned)w_gate->fmt.bits, w_gate->fmt.group_size);
     plan->steps.push_back(st);
     return MI355Q_OK;
 }

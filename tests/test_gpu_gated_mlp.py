@@ -174,3 +174,39 @@ def test_gated_projection_rejects_mismatched_weights(pkg, ctx):
     with pytest.raises(pkg.MI355QError):
         ctx.gated_qgemm(a, a, x, pkg.BF16, y, pkg.F32, 1, activation=7)
     a.destroy(); b.destroy(); x.free(); y.free()
+
+
+def test_gated_step_in_a_plan_replayed_as_a_graph(pkg, ctx):
+    """The gated projection as a plan step: the record names the fused launch, and eager replay, a captured graph and
+    the direct call give the same bits on every replay."""
+    n, k = 2048, 4096
+    wg, sg, zg, _ = seeded_case(6600, n, k, 4, 64)
+    wu, su, zu, _ = seeded_case(6601, n, k, 4, 64)
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+    g = ctx.weight_prepare_mlx(fmt, wg, sg, zg, pkg.BF16, pkg.LAYOUT_PLANES)
+    u = ctx.weight_prepare_mlx(fmt, wu, su, zu, pkg.BF16, pkg.LAYOUT_PLANES)
+    x = act_rounded(kat.seeded_activations(6602, 1, k), pkg.BF16, pkg)
+    xdev = ctx.upload(act_to_device_array(x, pkg.BF16, pkg))
+    direct, planned = ctx.alloc(n * 2), ctx.alloc(n * 2)
+    ctx.gated_qgemm(g, u, xdev, pkg.BF16, direct, pkg.BF16, 1, pkg.GATED_SILU)
+    plan = pkg.DispatchPlan(ctx)
+    plan.add_gated_mlp(g, u, xdev, pkg.BF16, planned, pkg.BF16, 1, pkg.GATED_SILU, layer_index=3, tensor_name="layers.3.mlp")
+    rec, layer, name = plan.step(0)
+    assert layer == 3 and name == "layers.3.mlp"
+    assert rec.kernel_family == "gatedFusedQ4G64" and rec.device_kernel.endswith("+swiglu"), (rec.kernel_family, rec.device_kernel)
+    stream = ctx.stream_create()
+    plan.encode(stream)
+    ctx.synchronize(stream)
+    ctx.synchronize()
+    want = direct.download(np.uint16)
+    assert np.array_equal(planned.download(np.uint16), want)
+    plan.graph_build(stream)
+    for _ in range(3):
+        ctx.fill(planned, 0x7FC07FC0, stream)
+        plan.graph_launch(stream)
+        ctx.synchronize(stream)
+        assert np.array_equal(planned.download(np.uint16), want)
+    plan.destroy()
+    for t in (xdev, direct, planned):
+        t.free()
+    g.destroy(); u.destroy()
