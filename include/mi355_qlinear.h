@@ -424,7 +424,11 @@ MI355Q_API mi355q_status mi355q_lmhead_argmax(mi355q_context* ctx, void* stream,
  * runs under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc.  Same arguments, kernels
  * and results as mi355q_lmhead_argmax; the one partial key per workgroup that the head launch leaves for its
  * finishing launch lives in a device array of the library image (258 KiB per GPU, held until the process ends)
- * instead of the context's allocation, and the call makes no hipMalloc, hipFree or other allocating call.
+ * instead of the context's allocation, and the call makes no hipMalloc, hipFree or other allocating call: where
+ * mi355q_lmhead_argmax would run the projection on a route that keeps scratch in the context (fp32 activations as
+ * three bf16 rows; f16 activations on TILE16 records), this entry point runs the per-code projection kernel and the
+ * arg-max launch instead (slower, same token up to ties between logits that differ in their last bits; a logits
+ * buffer is required there, as for every head that is not fused).
  * Limit: a head launch of more than mi355q_lmhead_argmax_static_capacity() = 32768 workgroups (524288 rows of up to
  * 2048 4-bit codes, 262144 rows of up to 4096) is refused with MI355Q_ERR_SHAPE.  Every call on a GPU shares that
  * GPU's array and overwrites the keys it uses (nothing has to be cleared between calls: a call reads back only the

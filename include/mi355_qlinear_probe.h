@@ -34,6 +34,11 @@ MI355Q_API mi355q_status mi355q_clock_probe_read(mi355q_context* ctx, uint64_t* 
 MI355Q_API mi355q_status mi355q_buffer_read_probe(mi355q_context* ctx, void* stream, const void* src_dev,
                                                   size_t bytes);
 
+/* Bytes of device scratch the context holds right now: [0] fp32 partial results / dense copies, [1] split activation
+ * rows, [2] gate and up sums of the gated projection.  A test of an entry point that must not allocate compares them
+ * before and after the call. */
+MI355Q_API mi355q_status mi355q_context_scratch_bytes(mi355q_context* ctx, uint64_t out_bytes[3]);
+
 #ifdef __cplusplus
 }
 #endif

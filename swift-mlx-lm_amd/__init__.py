@@ -181,6 +181,7 @@ def library() -> C.CDLL:
         "mi355q_buffer_copy": (i32, [vp, vp, vp, vp, sz]),
         "mi355q_buffer_read_probe": (i32, [vp, vp, vp, sz]),
         "mi355q_clock_probe_read": (i32, [vp, P(u64), P(u64)]),
+        "mi355q_context_scratch_bytes": (i32, [vp, P(u64)]),
         "mi355q_kv_scheme_is_supported": (i32, [u8]),
         "mi355q_kv_bytes_per_head_slot": (u32, [u8, u32]),
         "mi355q_kv_cache_write": (i32, [vp, vp, P(_KvLayout), vp, vp, C.c_int, u32, u32, u32]),
@@ -695,6 +696,12 @@ class Context:
         if self.handle:
             library().mi355q_context_destroy(self.handle)
             self.handle = None
+
+    def scratch_bytes(self):
+        """Bytes of device scratch the context holds (partial results, split rows, gated sums)."""
+        out = (C.c_uint64 * 3)()
+        _check(library().mi355q_context_scratch_bytes(self.handle, out))
+        return tuple(int(v) for v in out)
 
     def set_library_use(self, enabled: bool):
         """Whether launches may hand a dense product to the platform's GEMM library (on by default)."""

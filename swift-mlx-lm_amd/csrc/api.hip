@@ -499,7 +499,8 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
 // `keys`: kStaticHeadKeys or kArgmaxPartialCapacity keys for the fused head followed by kArgmaxStandaloneKeys for the
 // two-launch arg-max (the context's allocation, or the device array of the entry point that allocates nothing).
 mi355q_status dispatch_output_head(mi355q_context* ctx, hipStream_t s, const mi355q_weight* w, const void* x,
-                                   int x_dtype, float* logits, int32_t* token, uint32_t flags, HeadKeys keys) {
+                                   int x_dtype, float* logits, int32_t* token, uint32_t flags, HeadKeys keys,
+                                   bool no_allocation) {
     if (!x || !token) return fail(MI355Q_ERR_INVALID_ARGUMENT, "null pointer");
     if (!dtype_ok(x_dtype)) return fail(MI355Q_ERR_INVALID_ARGUMENT, "bad dtype tag");
     const WView v = w->view();
@@ -526,7 +527,8 @@ mi355q_status dispatch_output_head(mi355q_context* ctx, hipStream_t s, const mi3
                     "a logits buffer is required when the fused head kernel does not accept the shape");
     // fp32 activations (three bf16 rows on the bf16 decode kernel) and f16 ones on TILE16 records: the projection's own
     // route for one row (2048 -> 65536 with fp32 activations: the per-code kernel takes hundreds of microseconds)
-    const bool routed = !(flags & MI355Q_FLAG_FORCE_GENERIC) && (uintptr_t)x % 16 == 0 &&
+    // (the routed projections keep scratch in the context, grown on demand: not for the entry point that allocates nothing)
+    const bool routed = !no_allocation && !(flags & MI355Q_FLAG_FORCE_GENERIC) && (uintptr_t)x % 16 == 0 &&
                         (split_rows_chosen(v, x_dtype, 1, xs, flags) ||
                          (x_dtype == MI355Q_F16 && gemv_tile16_eligible(v, x_dtype, 1, xs)));
     mi355q_status st = routed ? dispatch_linear(ctx, s, w, x, x_dtype, logits, MI355Q_F32, 1, xs, (uint32_t)w->n, flags, true)
@@ -653,7 +655,7 @@ mi355q_status mi355q_lmhead_argmax_static(mi355q_context* ctx, void* stream, con
     unsigned long long* const keys = static_head_keys(ctx->device);
     if (!keys) return fail(MI355Q_ERR_DEVICE, "the static key array of device %d was not resolved", ctx->device);
     return dispatch_output_head(ctx, (hipStream_t)stream, w, x_dev, x_dtype, logits_f32_dev, token_out_dev, flags,
-                                HeadKeys{keys, kStaticHeadKeys});
+                                HeadKeys{keys, kStaticHeadKeys}, true);
 }
 
 uint32_t mi355q_lmhead_argmax_static_capacity(void) { return kStaticHeadKeys; }

@@ -263,7 +263,8 @@ mi355q_status dispatch_gated(mi355q_context* ctx, hipStream_t s, const mi355q_we
                              const void* x_dev, int x_dtype, void* y_dev, int y_dtype, uint32_t m, uint32_t xs, uint32_t ys,
                              int activation, uint32_t flags);
 mi355q_status dispatch_output_head(mi355q_context* ctx, hipStream_t s, const mi355q_weight* w, const void* x,
-                                   int x_dtype, float* logits, int32_t* token, uint32_t flags, HeadKeys keys);
+                                   int x_dtype, float* logits, int32_t* token, uint32_t flags, HeadKeys keys,
+                                   bool no_allocation = false);
 void plan_shared_launch_shape(const mi355q_weight* const* ws, uint32_t count, uint32_t m, int x_dtype, uint32_t x_stride,
                               mi355q_step* s);
 

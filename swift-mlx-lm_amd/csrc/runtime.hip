@@ -317,6 +317,14 @@ mi355q_status mi355q_context_create(int device_index, mi355q_context** out) {
     return MI355Q_OK;
 }
 
+mi355q_status mi355q_context_scratch_bytes(mi355q_context* ctx, uint64_t out_bytes[3]) {
+    if (!ctx || !out_bytes) return fail(MI355Q_ERR_NULL_HANDLE, "context or output is null");
+    out_bytes[0] = ctx->workspace_bytes;
+    out_bytes[1] = ctx->split_bytes;
+    out_bytes[2] = ctx->gated_bytes;
+    return MI355Q_OK;
+}
+
 mi355q_status mi355q_context_set_library_use(mi355q_context* ctx, int enabled) {
     if (!ctx) return fail(MI355Q_ERR_NULL_HANDLE, "context is null");
     ctx->dense_library_forbidden = !enabled;

@@ -64,3 +64,35 @@ def test_static_head_refuses_more_workgroups_than_keys(pkg, ctx):
     ctx.synchronize()
     assert int(tok.download(np.int32)[0]) >= 0
     w.destroy(); xd.free(); tok.free()
+
+
+@pytest.mark.parametrize("layout", ["LAYOUT_PLANES", "LAYOUT_TILE16", "LAYOUT_STAF_BLOCKS"])
+def test_static_head_allocates_nothing_with_f16_and_fp32_activations(pkg, layout):
+    """fp32 activations (and f16 ones on TILE16 records) reach mi355q_lmhead_argmax through routes that keep scratch in
+    the context; the entry point that allocates nothing must not take them.  On a fresh context, whose scratch buffers
+    do not exist yet: the context's scratch stays at zero bytes over both calls, the logits hold the bar against the
+    oracle, and the token is the lowest-index maximum of the logits the call returned."""
+    c = pkg.Context(0)
+    try:
+        fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+        for seed, n, k in ((830, 3000, 2048), (840, 520, 4096)):          # the second head is the smaller one
+            words, s, z = oracle.quantize_affine(kat.seeded_weights(seed, n, k), 4, 64, oracle.F16)
+            wq = oracle.dequant_planes_f32(4, 64, n, k, words, s, z, oracle.F16)
+            w = c.weight_prepare_mlx(fmt, words, s, z, pkg.F16, getattr(pkg, layout))
+            for xt, npdt in ((pkg.F32, np.float32), (pkg.F16, np.float16)):
+                xa = kat.seeded_activations(seed + 1, 1, k).astype(npdt)
+                xd = c.upload(xa.view(np.uint16) if xt == pkg.F16 else xa)
+                logits, tok = c.alloc(n * 4), c.upload(np.array([-7], np.int32))
+                before = c.scratch_bytes()
+                c.lmhead_argmax_static(w, xd, xt, logits, tok)
+                c.synchronize()
+                assert c.scratch_bytes() == before == (0, 0, 0), "the entry point that allocates nothing grew the context's scratch"
+                got, token = logits.download(np.float32), int(tok.download(np.int32)[0])
+                want = oracle.gemm_f64(wq, xa.astype(np.float32))[0]
+                assert np.linalg.norm(got - want) / np.linalg.norm(want) <= 1e-3
+                assert token == oracle.argmax_lowest(got)
+                for b in (xd, logits, tok):
+                    b.free()
+            w.destroy()
+    finally:
+        c.close()
