@@ -1,6 +1,6 @@
 """Builds libmi355_qlinear.so for gfx950 with hipcc (one object per translation unit, in parallel).
 
-Usage:  python swift-mlx-lm_amd/build.py [--force] [-j N]
+Usage:  python swift-mlx-lm_amd/build.py [--force] [-j N] [--timeline]
 The library is written to swift-mlx-lm_amd/lib/ (git-ignored, travels with the tree).
 """
 from __future__ import annotations
@@ -52,6 +52,21 @@ def _compile(src: str, force: bool) -> str:
     return obj
 
 
+def build_timeline(jobs: int | None = None) -> str:
+    """Measurement build: the library with per-workgroup time stamps in the decode rows kernel
+    (-DMI355Q_GEMV_TIMELINE), written beside the product library as libmi355_qlinear_timeline.so.
+    Used by decode_timeline.py only; the product library carries none of it."""
+    global OBJ, LIB, FLAGS
+    saved = (OBJ, LIB, FLAGS)
+    try:
+        OBJ = os.path.join(HERE, "build_timeline")
+        LIB = os.path.join(LIBDIR, "libmi355_qlinear_timeline.so")
+        FLAGS = FLAGS + ["-DMI355Q_GEMV_TIMELINE"]
+        return build(force=False, jobs=jobs)
+    finally:
+        OBJ, LIB, FLAGS = saved
+
+
 def build(force: bool = False, jobs: int | None = None) -> str:
     os.makedirs(OBJ, exist_ok=True)
     os.makedirs(LIBDIR, exist_ok=True)
@@ -78,5 +93,6 @@ if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--force", action="store_true")
     ap.add_argument("-j", type=int, default=None)
+    ap.add_argument("--timeline", action="store_true", help="the measurement build with per-workgroup time stamps (decode_timeline.py)")
     a = ap.parse_args()
-    print(build(force=a.force, jobs=a.j))
+    print(build_timeline(jobs=a.j) if a.timeline else build(force=a.force, jobs=a.j))

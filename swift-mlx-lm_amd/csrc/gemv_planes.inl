@@ -63,6 +63,9 @@ struct GemvArgs {
     uint32_t y_dtype, sb_dtype;
     uint32_t x_dtype;        // MI355Q_BF16 or MI355Q_F16 (f16 needs XA = 1)
     uint32_t gated;          // gated launches (GATED kernels): mi355q_gated_activation of the epilogue
+#ifdef MI355Q_GEMV_TIMELINE
+    unsigned long long* timeline;   // measurement build only: five 100 MHz time stamps and the hardware id per workgroup
+#endif
 };
 
 // Host-side choice of kernel variant and launch shape.

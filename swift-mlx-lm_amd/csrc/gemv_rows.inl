@@ -72,6 +72,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_rows_kernel(GemvArgs a) {
     u32x4* xs = smem;                                              // [NCT][Q][64]
     float* sxs = (float*)(smem + (size_t)NCT * Q * 64);             // [NCT][NSR][NF][64]
 
+#ifdef MI355Q_GEMV_TIMELINE
+    const unsigned long long tl_entry = __builtin_amdgcn_s_memrealtime();
+    unsigned long long tl_staged = 0, tl_first = 0;
+#endif
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     // matrix of this wavefront (up to three share a launch), then its rows inside that matrix
@@ -221,6 +225,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_rows_kernel(GemvArgs a) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+#ifdef MI355Q_GEMV_TIMELINE
+    tl_staged = __builtin_amdgcn_s_memrealtime();
+#endif
 
     uint32_t k_magic = XA == 1 ? 0x64006400u : 0x43004300u;
     asm volatile("" : "+v"(k_magic));
@@ -374,8 +381,25 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_rows_kernel(GemvArgs a) {
         res = ((lane & ~(uint32_t)(BR - 1)) == pass * BR) ? v : res;
     };
     const uint32_t passes = (nrows + BR - 1) / BR;
+#ifdef MI355Q_GEMV_TIMELINE
+    {   // when the first weight words of this wavefront are there
+        uint32_t first_word = ring[0][0].w[0];
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(first_word));
+        tl_first = __builtin_amdgcn_s_memrealtime();
+    }
+#endif
     for (uint32_t pass = 0; pass + 1 < passes; pass++) pass_body(pass, std::true_type{});
     if (passes) pass_body(passes - 1, std::false_type{});
+#ifdef MI355Q_GEMV_TIMELINE
+    if (a.timeline && wave == 0 && lane == 0) {
+        unsigned long long* const t = a.timeline + (size_t)blockIdx.x * 6;
+        uint32_t hw_id, xcc_id;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw_id));
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc_id));
+        t[0] = tl_entry; t[1] = tl_staged; t[2] = tl_first; t[3] = __builtin_amdgcn_s_memrealtime();
+        t[4] = hw_id; t[5] = xcc_id;
+    }
+#endif
 
     // ---- one coalesced store of the parked results (rows_per_wave <= 64) ------------------------------------
     if constexpr (GATED) {

@@ -12,6 +12,11 @@ mi355q_status launch_gemv_planes_q5(hipStream_t, const GemvArgs&, int, const Gem
 mi355q_status launch_gemv_planes_q6(hipStream_t, const GemvArgs&, int, const GemvCfg&);
 mi355q_status launch_gemv_planes_q8(hipStream_t, const GemvArgs&, int, const GemvCfg&);
 
+#ifdef MI355Q_GEMV_TIMELINE
+unsigned long long* g_gemv_timeline = nullptr;      // measurement build only
+extern "C" __attribute__((visibility("default"))) void mi355q_probe_set_timeline(unsigned long long* p) { g_gemv_timeline = p; }
+#endif
+
 namespace {
 
 constexpr size_t kLdsBudget = 144 * 1024;  // of the 160 KiB per CU; the rest is left for the runtime
@@ -72,6 +77,11 @@ GemvCfg choose(const mi355q_context* ctx, const WView& w, uint32_t m, bool argma
         uint32_t rpw = c.nc == 1 ? 4 : c.nc <= 4 ? 2 : 1;
         while (rpw > 1 && w.n / rpw < least_waves) rpw >>= 1;
         int br = (int)rpw;                                                          // one pass
+#ifdef MI355Q_GEMV_TIMELINE
+        if (const char* e = std::getenv("TL_RPW")) rpw = (uint32_t)std::atoi(e);      // measurement build only
+        br = (int)rpw;
+        if (const char* e = std::getenv("TL_BR")) br = std::atoi(e);
+#endif
         if (argmax && !gemv_rows_has_argmax((int)c.nc, br)) br = c.nc == 1 ? 4 : 2;   // the head's variants
         rpw = (rpw + br - 1) / br * br;
         // very tall matrices: more passes rather than more than 65535 workgroups
@@ -200,6 +210,9 @@ mi355q_status launch_gemv_fast_multi(hipStream_t s, const mi355q_context* ctx, u
         a.code_stride = all.code_stride; a.sz_stride = all.sz_stride;
         a.nc = c.nc; a.rows_per_wave = c.rows_per_wave;
         a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = all.sb_dtype; a.x_dtype = (uint32_t)x_dtype;
+#ifdef MI355Q_GEMV_TIMELINE
+        a.timeline = g_gemv_timeline;
+#endif
         c.grid = grid;                        // whole wavefronts per matrix: a few more than rows / rows_per_wave
         if (argmax && grid > keys.capacity)
             return fail(MI355Q_ERR_SHAPE, "the fused output head keeps one partial key per workgroup: %u workgroups exceed %u",
