@@ -39,6 +39,11 @@ MI355Q_API mi355q_status mi355q_buffer_read_probe(mi355q_context* ctx, void* str
  * before and after the call. */
 MI355Q_API mi355q_status mi355q_context_scratch_bytes(mi355q_context* ctx, uint64_t out_bytes[3]);
 
+/* A/B runs of the wide-tile prefill kernel: tile height (128 or 256 rows) and the number of parts K is split into
+ * (1 .. 4), for every later launch of the process; 0 leaves the choice to the library.  Values that do not fit a
+ * problem (fewer than sixteen K-tiles a part, N not a multiple of four) are ignored for it. */
+MI355Q_API void mi355q_probe_wide_shape(uint32_t tile_rows, uint32_t k_parts);
+
 #ifdef __cplusplus
 }
 #endif

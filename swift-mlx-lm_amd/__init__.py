@@ -182,6 +182,7 @@ def library() -> C.CDLL:
         "mi355q_buffer_read_probe": (i32, [vp, vp, vp, sz]),
         "mi355q_clock_probe_read": (i32, [vp, P(u64), P(u64)]),
         "mi355q_context_scratch_bytes": (i32, [vp, P(u64)]),
+        "mi355q_probe_wide_shape": (None, [u32, u32]),
         "mi355q_kv_scheme_is_supported": (i32, [u8]),
         "mi355q_kv_bytes_per_head_slot": (u32, [u8, u32]),
         "mi355q_kv_cache_write": (i32, [vp, vp, P(_KvLayout), vp, vp, C.c_int, u32, u32, u32]),
@@ -702,6 +703,11 @@ class Context:
         out = (C.c_uint64 * 3)()
         _check(library().mi355q_context_scratch_bytes(self.handle, out))
         return tuple(int(v) for v in out)
+
+    @staticmethod
+    def probe_wide_shape(tile_rows: int = 0, k_parts: int = 0):
+        """A/B runs: tile height and K parts of the wide-tile prefill kernel for the whole process (0: the library chooses)."""
+        library().mi355q_probe_wide_shape(tile_rows, k_parts)
 
     def set_library_use(self, enabled: bool):
         """Whether launches may hand a dense product to the platform's GEMM library (on by default)."""

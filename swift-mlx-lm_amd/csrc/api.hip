@@ -270,7 +270,10 @@ bool gemm_two_step_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_st
     if (flags & MI355Q_FLAG_FORCE_TWO_STEP) return true;
     if (!gemm_two_step_eligible(w, x_dtype, m, x_stride)) return false;
     if (gemm_stream_chosen(w, x_dtype, m, x_stride)) return false;      // a few dozen rows on 4- / 8-bit planes
-    if (gemm_wide_chosen(w, x_dtype, m, x_stride)) return false;        // long prompts on 4-bit planes: this library's own kernel
+    // long prompts on 4-bit planes: this library's own kernel, up to the rows from which the two dispatches are faster
+    // by a tenth and more (M = 3072: 4096 -> 14336 277 us against 314, 14336 -> 4096 282 against 307; M = 2048: 196-216
+    // against 202-216 and 224 against 210)
+    if (gemm_wide_chosen(w, x_dtype, m, x_stride) && m < kWideRowsBesideLibrary) return false;
     if (!gemm_mfma_eligible(w, x_dtype, m, x_stride)) {
         // no decode kernel reads the weight: from the second row; from the first where the per-code kernel leaves most
         // of its lanes idle (a lane per code of a group: q3 g16 blocks, 4096 -> 14336, take it 465 us at one row

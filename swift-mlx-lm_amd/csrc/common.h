@@ -295,11 +295,15 @@ mi355q_status launch_qgemm_mfma(hipStream_t s, mi355q_context* ctx, const WView&
 // Wide-tile MFMA GEMM for long prompts (gemm_wide.hip): 4-bit planes in groups of 64 / 128, bf16 activations; the weights
 // are dequantised in registers, only the activations pass through LDS.  Taken from kWideMinRows rows where its tiles
 // occupy three quarters of the CUs (measured against the tiled kernel and the two-dispatch route: see gemm_wide_chosen).
+// the dense library is forbidden for the context or could not be opened: the two-dispatch route serves nothing
+inline bool library_ruled_out(const mi355q_context* ctx) { return ctx->dense_library_failed || ctx->dense_library_forbidden; }
 constexpr uint32_t kWideMinRows = 384;
+constexpr uint32_t kWideRowsBesideLibrary = 2560;   // from here the two-dispatch route is taken where the dense library is there
 bool gemm_wide_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
 bool gemm_wide_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
 GemmLaunchShape gemm_wide_shape(uint32_t m, uint32_t n, uint32_t k);
 uint32_t chip_cus();
+void gemm_wide_force_shape(uint32_t bm, uint32_t splits);      // A/B runs (mi355q_probe_wide_shape)
 inline bool gemm_wide_taken(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride, uint32_t flags) {
     if (flags & MI355Q_FLAG_PROBE_TILED) return false;
     if (flags & MI355Q_FLAG_PROBE_WIDE) return gemm_wide_eligible(w, x_dtype, m, x_stride);

@@ -40,6 +40,7 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 wd_bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float wd_floatx16_t;
 typedef __bf16 wd_bf16x2_v __attribute__((ext_vector_type(2)));
 typedef float wd_float2_v __attribute__((ext_vector_type(2)));
+typedef float wd_float4_v __attribute__((ext_vector_type(4)));
 
 struct WideArgs {
     const uint32_t* codes;       // [N, K / 8] words, rows code_stride words apart
@@ -51,6 +52,8 @@ struct WideArgs {
     uint32_t tiles_m, tiles_n;
     uint32_t y_dtype;
     uint32_t wide_stores;        // rows of y are 16-byte aligned for every column that is a multiple of four
+    float* partial;              // K split over workgroups: fp32 [splits][M][N] partial results (null otherwise)
+    uint32_t splits, kt_per_split;   // K-tiles per split: a multiple of four
     unsigned long long* probe;   // optional: [0] shader cycles, [1] 100 MHz ticks that workgroup 0 spent in the kernel
 };
 
@@ -60,6 +63,14 @@ constexpr int kWideBN = 256;
 __device__ __forceinline__ uint32_t wd_pack_bf16(float lo, float hi) {
     wd_float2_v v = {lo, hi};
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, wd_bf16x2_v));
+}
+
+// A wave-uniform address as the scalar operand of hand-written memory instructions, wherever the compiler computed it
+__device__ __forceinline__ const char* wd_scalar(const char* p) {
+    const uint64_t v = (uint64_t)(uintptr_t)p;
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+    return (const char*)(uintptr_t)(((uint64_t)hi << 32) | lo);
 }
 
 template <int BM, bool SB_BF16, int GROUP>
@@ -76,17 +87,22 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
 
     // tile of this workgroup: the workgroups of one XCD (id % 8) take consecutive tiles, row tiles of one column tile
     // first, so that they share that column tile's weights and a few row tiles' activations in the XCD's L2
-    const uint32_t total = a.tiles_m * a.tiles_n;
+    // (with K split over workgroups: all tiles of the first part of K, then those of the second ...)
+    const uint32_t tiles = a.tiles_m * a.tiles_n;
+    const uint32_t total = tiles * a.splits;
     const uint32_t per_xcd = (total + 7) / 8;
     const uint32_t t_id = (blockIdx.x % 8u) * per_xcd + blockIdx.x / 8u;
     if (t_id >= total) return;
-    const uint32_t tn = t_id / a.tiles_m, tm = t_id % a.tiles_m;
-    const uint32_t m0 = tm * BM, n0 = tn * kWideBN;
+    const uint32_t split = (uint32_t)__builtin_amdgcn_readfirstlane((int)(t_id / tiles)), tile = t_id - split * tiles;
+    const uint32_t tn = tile / a.tiles_m, tm = tile % a.tiles_m;
+    const uint32_t m0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tm * BM)), n0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tn * kWideBN));
+    const uint32_t kt_begin = (uint32_t)__builtin_amdgcn_readfirstlane((int)(split * a.kt_per_split));
 
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t ln = lane & 31, lh = lane >> 5;
-    const uint32_t KT = a.k / 64;                   // a multiple of four
+    const uint32_t kt_left = a.k / 64 - kt_begin;
+    const uint32_t KT = (uint32_t)__builtin_amdgcn_readfirstlane((int)(kt_left < a.kt_per_split ? kt_left : a.kt_per_split));   // K-tiles of this workgroup: a multiple of four
 
     // ---- activations: global -> LDS ---------------------------------------------------------------
     // copy q of wavefront w covers tile rows 8 (AQ w + q) .. + 7; lane L lands at row L / 8, position L % 8, and
@@ -99,10 +115,10 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
         const uint32_t chunk = (lane & 7u) ^ ((row >> 1) & 7u);
         x_off[q] = (row < m_last ? row : m_last) * a.xs * 2 + chunk * 16;
     }
-    const char* const xg = (const char*)(a.x + (size_t)m0 * a.xs);
+    const char* const xg = (const char*)(a.x + (size_t)m0 * a.xs + (size_t)kt_begin * 64);
     auto copy_x = [&](uint32_t kt, auto Q0, auto CNT) __attribute__((always_inline)) {
         const uint32_t t = kt < KT ? kt : KT - 1;   // past the end: a copy nobody reads, so that the counts stay the same
-        const char* const g = xg + (size_t)t * 128;
+        const char* const g = wd_scalar(xg + (size_t)t * 128);
         const uint32_t as = lds_base + (kt % kWideStages) * A_STAGE + wave * (AQ * 1024);
 #pragma unroll
         for (int q = decltype(Q0)::value; q < decltype(Q0)::value + decltype(CNT)::value; q++) {
@@ -122,15 +138,15 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
         w_off[f] = gr * a.code_stride * 4 + lh * 16;
         sz_off[f] = gr * a.sz_stride * 4;
     }
-    const char* const cg = (const char*)(a.codes + (size_t)n0 * a.code_stride);
-    const char* const sg = (const char*)(a.sz + (size_t)n0 * a.sz_stride);
+    const char* const cg = (const char*)(a.codes + (size_t)n0 * a.code_stride) + (size_t)(kt_begin / 4) * 128;
+    const char* const sg = (const char*)(a.sz + (size_t)n0 * a.sz_stride) + (size_t)(kt_begin / 4) * (SZW * 4);
     using sz_vec = std::conditional_t<SZW == 4, u32x4, u32x2>;      // kept whole: the loads write them behind the compiler's back
     u32x4 wnext[2][4], wcur[2][4];
     sz_vec sznext[2], szcur[2];
     auto load_w = [&](uint32_t four) __attribute__((always_inline)) {
         const uint32_t p = four * 4 < KT ? four : KT / 4 - 1;
-        const char* const g = cg + (size_t)p * 128;
-        const char* const gs = sg + (size_t)p * (SZW * 4);
+        const char* const g = wd_scalar(cg + (size_t)p * 128);
+        const char* const gs = wd_scalar(sg + (size_t)p * (SZW * 4));
 #pragma unroll
         for (int f = 0; f < 2; f++) {
 #pragma unroll
@@ -213,7 +229,7 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
         constexpr int slot = decltype(SLOT)::value;
         const char* const xs_next = lds + (kt_next % kWideStages) * A_STAGE + a_rd[jn];
         const uint32_t tc = kt_copy < KT ? kt_copy : KT - 1;
-        const char* const gx = xg + (size_t)tc * 128;
+        const char* const gx = wd_scalar(xg + (size_t)tc * 128);
         const uint32_t lx = lds_base + (kt_copy % kWideStages) * A_STAGE + wave * (AQ * 1024);
         static_for<TM>([&](auto Q) __attribute__((always_inline)) {
             constexpr int q = decltype(Q)::value;
@@ -303,7 +319,7 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
     // ---- epilogue: one rounding, to the output type -----------------------------------------------------
     // lane (m, h) of accumulator (f, i) holds row m0 + 32 i + m, columns 32 f + 8 g + 4 h + (0 .. 3) for g = 0 .. 3.
     // One accumulator at a time (the fences keep the compiler from fetching all 256 registers first).
-    auto store_tiles = [&](auto DT) __attribute__((always_inline)) {
+    auto store_tiles = [&](auto DT, void* const y, const size_t ys, const bool wide) __attribute__((always_inline)) {
         constexpr int dt = decltype(DT)::value;
         static_for<2>([&](auto F) __attribute__((always_inline)) {
             static_for<TM>([&](auto I) __attribute__((always_inline)) {
@@ -317,25 +333,25 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
                     for (int g = 0; g < 4; g++) {
                         const uint32_t col = n0 + 64 * wave + 32 * f + 8 * g + 4 * lh;
                         const float v[4] = {acc[f][i][4 * g + 0], acc[f][i][4 * g + 1], acc[f][i][4 * g + 2], acc[f][i][4 * g + 3]};
-                        const size_t o = (size_t)row * a.ys + col;
-                        if (a.wide_stores && col + 3 < a.n) {
+                        const size_t o = (size_t)row * ys + col;
+                        if (wide && col + 3 < a.n) {
                             if constexpr (dt == MI355Q_F32) {
                                 const float4 t = {v[0], v[1], v[2], v[3]};
-                                *(float4*)((float*)a.y + o) = t;
+                                *(float4*)((float*)y + o) = t;
                             } else if constexpr (dt == MI355Q_BF16) {
                                 uint2 t;
                                 t.x = wd_pack_bf16(v[0], v[1]); t.y = wd_pack_bf16(v[2], v[3]);
-                                *(uint2*)((uint16_t*)a.y + o) = t;
+                                *(uint2*)((uint16_t*)y + o) = t;
                             } else {
                                 uint2 t;
                                 t.x = (uint32_t)f32_to_f16_rne(v[0]) | ((uint32_t)f32_to_f16_rne(v[1]) << 16);
                                 t.y = (uint32_t)f32_to_f16_rne(v[2]) | ((uint32_t)f32_to_f16_rne(v[3]) << 16);
-                                *(uint2*)((uint16_t*)a.y + o) = t;
+                                *(uint2*)((uint16_t*)y + o) = t;
                             }
                         } else {
 #pragma unroll
                             for (int e = 0; e < 4; e++)
-                                if (col + e < a.n) store_out<dt>(a.y, o + e, v[e]);
+                                if (col + e < a.n) store_out<dt>(y, o + e, v[e]);
                         }
                     }
                 }
@@ -343,16 +359,52 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
             });
         });
     };
-    if (a.y_dtype == MI355Q_BF16) store_tiles(std::integral_constant<int, MI355Q_BF16>{});
-    else if (a.y_dtype == MI355Q_F32) store_tiles(std::integral_constant<int, MI355Q_F32>{});
-    else store_tiles(std::integral_constant<int, MI355Q_F16>{});
+    if (a.partial)         // this part of K as fp32 (N is a multiple of four: 16-byte stores); wide_reduce_kernel adds the parts
+        store_tiles(std::integral_constant<int, MI355Q_F32>{}, a.partial + (size_t)split * a.m * a.n, a.n, true);
+    else if (a.y_dtype == MI355Q_BF16) store_tiles(std::integral_constant<int, MI355Q_BF16>{}, a.y, a.ys, a.wide_stores != 0);
+    else if (a.y_dtype == MI355Q_F32) store_tiles(std::integral_constant<int, MI355Q_F32>{}, a.y, a.ys, a.wide_stores != 0);
+    else store_tiles(std::integral_constant<int, MI355Q_F16>{}, a.y, a.ys, a.wide_stores != 0);
+}
+
+// Sum of the parts of a K-split launch in part order (deterministic), one rounding to the output type.  N is a
+// multiple of four; four columns per thread.
+__global__ __launch_bounds__(256) void wide_reduce_kernel(const wd_float4_v* __restrict__ partial, void* __restrict__ y, uint32_t m,
+                                                          uint32_t n, uint32_t ys, uint32_t splits, uint32_t y_dtype,
+                                                          uint32_t wide_stores) {
+    const size_t total = (size_t)m * n / 4;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        wd_float4_v v = __builtin_nontemporal_load(partial + i);
+        for (uint32_t s = 1; s < splits; s++) v += __builtin_nontemporal_load(partial + (size_t)s * total + i);
+        const size_t e = i * 4, row = e / n, col = e - row * n;
+        const size_t o = row * ys + col;
+        if (wide_stores) {
+            if (y_dtype == MI355Q_F32) *(wd_float4_v*)((float*)y + o) = v;
+            else if (y_dtype == MI355Q_BF16) {
+                uint2 t;
+                t.x = wd_pack_bf16(v.x, v.y); t.y = wd_pack_bf16(v.z, v.w);
+                *(uint2*)((uint16_t*)y + o) = t;
+            } else {
+                uint2 t;
+                t.x = (uint32_t)f32_to_f16_rne(v.x) | ((uint32_t)f32_to_f16_rne(v.y) << 16);
+                t.y = (uint32_t)f32_to_f16_rne(v.z) | ((uint32_t)f32_to_f16_rne(v.w) << 16);
+                *(uint2*)((uint16_t*)y + o) = t;
+            }
+        } else {
+            const float f[4] = {v.x, v.y, v.z, v.w};
+            for (int c = 0; c < 4; c++) {
+                if (y_dtype == MI355Q_F32) ((float*)y)[o + c] = f[c];
+                else if (y_dtype == MI355Q_BF16) ((uint16_t*)y)[o + c] = f32_to_bf16_rne(f[c]);
+                else ((uint16_t*)y)[o + c] = f32_to_f16_rne(f[c]);
+            }
+        }
+    }
 }
 
 template <int BM, bool SB_BF16, int GROUP>
 mi355q_status launch_wide_tile(hipStream_t s, WideArgs a) {
     a.tiles_m = (a.m + BM - 1) / BM;
     a.tiles_n = (a.n + kWideBN - 1) / kWideBN;
-    const uint32_t grid = (a.tiles_m * a.tiles_n + 7) / 8 * 8;
+    const uint32_t grid = (a.tiles_m * a.tiles_n * a.splits + 7) / 8 * 8;
     constexpr size_t lds = (size_t)kWideStages * BM * 128;
     auto kern = qgemm_wide_kernel<BM, SB_BF16, GROUP>;
     // the attribute belongs to the function on one device: one bit per device and instantiation
@@ -366,6 +418,13 @@ mi355q_status launch_wide_tile(hipStream_t s, WideArgs a) {
     }
     kern<<<dim3(grid), dim3(256), lds, s>>>(a);
     MI355Q_HIP(hipGetLastError());
+    if (a.partial) {
+        size_t blocks = ((size_t)a.m * a.n / 4 + 255) / 256;
+        if (blocks > 16384) blocks = 16384;
+        wide_reduce_kernel<<<dim3((unsigned)blocks), dim3(256), 0, s>>>((const wd_float4_v*)a.partial, a.y, a.m, a.n, a.ys, a.splits,
+                                                                        a.y_dtype, a.wide_stores);
+        MI355Q_HIP(hipGetLastError());
+    }
     return MI355Q_OK;
 }
 
@@ -391,7 +450,6 @@ bool gemm_wide_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stri
     return true;
 }
 
-// Tile height: 256 rows where such tiles come to at least 85 % of one per CU, else 128 rows (two workgroups a CU).
 // CUs of the current device (256 on an MI355X; fewer in a partitioned mode), asked once
 uint32_t chip_cus() {
     static std::atomic<uint32_t> cached{0};
@@ -407,19 +465,60 @@ uint32_t chip_cus() {
     return (uint32_t)count;
 }
 
+// A/B runs: tile height and K parts forced from outside (0: chosen here)
+static std::atomic<uint32_t> g_wide_forced_bm{0}, g_wide_forced_splits{0};
+void gemm_wide_force_shape(uint32_t bm, uint32_t splits) {
+    g_wide_forced_bm.store(bm == 128 || bm == 256 ? bm : 0, std::memory_order_relaxed);
+    g_wide_forced_splits.store(splits <= 8 ? splits : 0, std::memory_order_relaxed);
+}
+
+// Tile height and K parts.  What a wavefront spends on a K-tile depends on the tile height alone (the weights of its 64
+// columns are dequantised once per K-tile whatever the rows: about 2500 cycles at 256 rows, 1600 at 128, measured
+// under load), so 256-row tiles are the efficient ones and K is split into parts where they leave CUs idle: each part
+// writes fp32, a second launch adds the parts (about 3 us and the traffic of splits + 1 result matrices).
 GemmLaunchShape gemm_wide_shape(uint32_t m, uint32_t n, uint32_t k) {
     const uint32_t cus = chip_cus();
     const uint32_t tiles_n = (n + kWideBN - 1) / kWideBN;
-    const uint32_t t256 = ((m + 255) / 256) * tiles_n;
+    const uint32_t kt = k / 64;
     GemmLaunchShape g{};
-    g.bm = (m > 128 && 100 * t256 >= 85 * cus) ? 256 : 128;
+    double best = 0;
+    const uint32_t forced_bm = g_wide_forced_bm.load(std::memory_order_relaxed);
+    const uint32_t forced_splits = g_wide_forced_splits.load(std::memory_order_relaxed);
+    for (uint32_t bm : {256u, 128u}) {
+        if (forced_bm && bm != forced_bm) continue;
+        if (bm == 256 && m <= 128 && !forced_bm) continue;
+        for (uint32_t splits : {1u, 2u, 3u, 4u}) {
+            if (forced_splits && splits != forced_splits) continue;
+            if (splits > 1 && (n % 4 || kt / splits < 16)) continue;
+            const uint32_t per = (kt / 4 + splits - 1) / splits * 4;          // K-tiles a part, a multiple of four
+            const uint32_t parts = (kt + per - 1) / per;
+            if (parts != splits) continue;
+            const uint32_t wgs = ((m + bm - 1) / bm) * tiles_n * parts;
+            // cycles of a workgroup per K-tile, measured under load: 2500 at 256 rows (one workgroup a CU, whole rounds);
+            // 1600 at 128 rows alone on its CU, 2950 for the two that share one (a last round of at most one per CU
+            // runs alone)
+            double cycles;
+            if (bm == 256) {
+                cycles = (double)((wgs + cus - 1) / cus) * per * 2500.0;
+            } else {
+                const uint32_t full = wgs / (2 * cus), rest = wgs % (2 * cus);
+                cycles = (double)full * per * 2950.0 + (rest > cus ? per * 2950.0 : rest ? per * 1600.0 : 0.0);
+            }
+            const double rounds = bm == 256 ? (double)((wgs + cus - 1) / cus) : (double)((wgs + 2 * cus - 1) / (2 * cus));
+            double cost = cycles / 1750.0 + 8.0 * rounds;                       // us at the clock the part holds
+            if (parts > 1) cost += 3.0 + (double)(parts + 1) * m * n * 4.0 / 3.5e6;
+            if (best == 0 || cost < best) {
+                best = cost;
+                g.bm = bm; g.splits = parts; g.kt_per_split = per;
+            }
+        }
+    }
+    if (best == 0) { g.bm = 128; g.splits = 1; g.kt_per_split = kt; }       // forced values that do not fit
     g.bn = kWideBN;
     g.stages = kWideStages;
     g.block = 256;
-    g.grid = (((m + g.bm - 1) / g.bm) * tiles_n + 7) / 8 * 8;
+    g.grid = (((m + g.bm - 1) / g.bm) * tiles_n * g.splits + 7) / 8 * 8;
     g.lds_bytes = kWideStages * g.bm * 128;
-    g.splits = 1;
-    g.kt_per_split = k / 64;
     return g;
 }
 
@@ -428,8 +527,8 @@ GemmLaunchShape gemm_wide_shape(uint32_t m, uint32_t n, uint32_t k) {
 bool gemm_wide_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
     if (!gemm_wide_eligible(w, x_dtype, m, x_stride) || m < kWideMinRows) return false;
     const GemmLaunchShape g = gemm_wide_shape(m, w.n, w.k);
-    const uint32_t tiles = ((m + g.bm - 1) / g.bm) * ((w.n + kWideBN - 1) / kWideBN);
-    return 4 * tiles >= 3 * chip_cus();
+    const uint32_t wgs = ((m + g.bm - 1) / g.bm) * ((w.n + kWideBN - 1) / kWideBN) * g.splits;
+    return 4 * wgs >= 3 * chip_cus();
 }
 
 mi355q_status launch_qgemm_wide(hipStream_t s, mi355q_context* ctx, const WView& w, const void* x, int x_dtype, void* y,
@@ -445,8 +544,12 @@ mi355q_status launch_qgemm_wide(hipStream_t s, mi355q_context* ctx, const WView&
     a.y_dtype = (uint32_t)y_dtype;
     a.wide_stores = (y_stride % 4 == 0 && (uintptr_t)y % 16 == 0) ? 1u : 0u;
     a.probe = probe;
-    (void)ctx;
     const GemmLaunchShape g = gemm_wide_shape(m, w.n, w.k);
+    a.splits = g.splits; a.kt_per_split = g.kt_per_split;
+    if (g.splits > 1) {
+        if (mi355q_status st = ensure_workspace(ctx, (size_t)g.splits * m * w.n * sizeof(float))) return st;
+        a.partial = (float*)ctx->workspace;
+    }
     const bool sb_bf16 = w.sb_dtype == MI355Q_BF16;
     if (g.bm == 256) return launch_wide_bm<256>(s, a, w.group, sb_bf16);
     return launch_wide_bm<128>(s, a, w.group, sb_bf16);

@@ -126,7 +126,7 @@ void plan_small_m(const mi355q_weight* w, uint32_t m, int x_dtype, uint32_t x_st
         s->block[0] = g.block;
         s->lds_bytes = g.lds_bytes;
         s->rows_per_workgroup = g.rows_per_workgroup;
-    } else if (gemm_two_step_chosen(v, x_dtype, m, x_stride, flags)) {
+    } else if (gemm_two_step_chosen(v, x_dtype, m, x_stride, flags) && !library_ruled_out(w->ctx)) {
         // no decode kernel reads this layout with this activation type: dequantise once + the dense library product
         // a few rows: fp32 weights and an fp32 product whatever the activation type (the decode kernels' arithmetic)
         std::snprintf(s->device_kernel, sizeof s->device_kernel, "dequant_q%u_g%u_f32+hipblaslt_gemm_f32", (unsigned)w->fmt.bits,
@@ -254,7 +254,8 @@ mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w, uint32_t maximum
                             (!(flags & MI355Q_FLAG_FORCE_MFMA) && m <= small_rows) ||
                             split_rows_chosen(v, x_dtype, m, input_row_stride, flags);
     const bool mfma_ok = gemm_mfma_eligible(v, x_dtype, m, input_row_stride);
-    if (!split_rows_chosen(v, x_dtype, m, input_row_stride, flags) && gemm_two_step_chosen(v, x_dtype, m, input_row_stride, flags)) {
+    if (!split_rows_chosen(v, x_dtype, m, input_row_stride, flags) && gemm_two_step_chosen(v, x_dtype, m, input_row_stride, flags) &&
+        !library_ruled_out(w->ctx)) {
         // dequant_q{b}_g{g}_bf16 into the scratch matrix, then the dense GEMM (MetalPrefillStepBuilder's two-dispatch
         // route; the dense product is the platform library's, as the reference's is matmul2d)
         *out_count = 2;
@@ -316,7 +317,7 @@ mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w, uint32_t maximum
                                        : gemm_mfma_shape(w->ctx, m, (uint32_t)w->n, (uint32_t)w->k);
         s->block[0] = g.block;
         s->grid[0] = g.grid;
-        s->grid[1] = g.splits;
+        s->grid[1] = wide ? 1 : g.splits;            // the wide-tile kernel numbers the parts of K inside its one grid axis
         s->lds_bytes = g.lds_bytes;
         s->rows_per_workgroup = g.bn;
         return MI355Q_OK;

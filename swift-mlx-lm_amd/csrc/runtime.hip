@@ -325,6 +325,8 @@ mi355q_status mi355q_context_scratch_bytes(mi355q_context* ctx, uint64_t out_byt
     return MI355Q_OK;
 }
 
+void mi355q_probe_wide_shape(uint32_t tile_rows, uint32_t k_parts) { gemm_wide_force_shape(tile_rows, k_parts); }
+
 mi355q_status mi355q_context_set_library_use(mi355q_context* ctx, int enabled) {
     if (!ctx) return fail(MI355Q_ERR_NULL_HANDLE, "context is null");
     ctx->dense_library_forbidden = !enabled;

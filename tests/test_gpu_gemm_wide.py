@@ -98,6 +98,48 @@ def test_wide_gemm_ragged_shapes_against_the_oracle(pkg, ctx):
         w.destroy()
 
 
+@pytest.mark.parametrize("tile_rows,parts", [(256, 2), (256, 4), (128, 3), (128, 4)])
+def test_wide_gemm_with_k_in_parts(pkg, ctx, tile_rows, parts):
+    """K split over workgroups (fp32 partial results, summed in part order by a second launch): exact on small integers
+    for every output type and a padded result; seeded values against the oracle; the forced shape shows in the plan."""
+    rng = np.random.default_rng(4400 + parts)
+    m, n, k = 300, 264, 64 * 16 * parts + 256           # the last part is shorter than the others
+    codes = rng.integers(0, 16, (n, k), dtype=np.uint8)
+    scales = rng.choice([0.125, 0.25, 0.5], (n, k // 64))
+    zeros = rng.integers(-4, 5, (n, k // 64)) * 0.25
+    case = Case(4, 64, codes, scales, zeros)
+    wq = scales.repeat(64, axis=1) * codes + zeros.repeat(64, axis=1)
+    x = rng.integers(-8, 9, (m, k)).astype(np.float32) * 0.125
+    want = x.astype(np.float64) @ wq.T
+    pkg.Context.probe_wide_shape(tile_rows, parts)
+    try:
+        w = case.device_weight(ctx, pkg, pkg.LAYOUT_PLANES, pkg.BF16)
+        step = w.plan_prefill_steps(m, flags=wide(pkg))[0]
+        tiles = -(-m // tile_rows) * -(-n // 256)
+        assert step.device_kernel == "qgemm_wide_q4_g64" and step.grid[0] == -(-tiles * parts // 8) * 8, (step.grid, tiles)
+        for yd in (pkg.F32, pkg.BF16, pkg.F16):
+            for y_pad in (0, 3):
+                say(f"wide K parts {tile_rows}x{parts} y={yd} pad={y_pad}")
+                got = run_qgemm(ctx, pkg, w, x, yd, wide(pkg), y_stride=(n + y_pad) if y_pad else None)
+                if y_pad:
+                    assert np.all(np.isnan(got[:, n:])), "padding of the output rows was written"
+                    got = got[:, :n]
+                if yd == pkg.F32:
+                    assert np.array_equal(got.astype(np.float64), want)
+                elif yd == pkg.BF16:
+                    assert np.array_equal(got, bf16_round(want.astype(np.float32)))
+                else:
+                    assert np.array_equal(got, want.astype(np.float16).astype(np.float32))
+        w.destroy()
+        w, x, got, _ = _seeded(pkg, ctx, 4410 + parts, 257, 520, k, 64, wide(pkg))
+        pkg.Context.probe_wide_shape(0, 0)
+        whole = run_qgemm(ctx, pkg, w, x, pkg.F32, pkg.FLAG_FORCE_MFMA | pkg.FLAG_PROBE_TILED)
+        assert np.max(np.abs(whole - got)) <= 2e-5 * max(1.0, float(np.max(np.abs(got))))
+        w.destroy()
+    finally:
+        pkg.Context.probe_wide_shape(0, 0)
+
+
 @pytest.mark.parametrize("m", [128, 512, 2048])
 @pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
 def test_config3_prefill_as_dispatched(pkg, ctx, m, n, k):
@@ -126,6 +168,7 @@ def test_context_without_the_dense_library_keeps_in_tree_kernels(pkg):
         fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
         w = c.weight_prepare_mlx(fmt, words, s, z, pkg.F16, pkg.LAYOUT_STAF_BLOCKS)
         x = act_rounded(kat.seeded_activations(4301, m, k), pkg.BF16, pkg)
+        assert all(s.kernel_family != "libraryGEMM" for s in w.plan_prefill_steps(m)), "the plan names the library"
         got = run_qgemm(c, pkg, w, x, pkg.F32, 0)
         assert_within_tolerance(got, oracle.gemm_f64(wq, x), "blocks in place, library forbidden")
         w.destroy()
