@@ -182,7 +182,7 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
     if (gemm_two_step_chosen(v, x_dtype, m, xs, flags) && (uintptr_t)x % 16 == 0 &&
         gemm_two_step_serves(ctx, v, x_dtype, y_dtype, m, xs, ys))
         return launch_qgemm_two_step(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
-    const bool mfma_ok = gemm_mfma_eligible(v, x_dtype, m, xs);
+    const bool mfma_ok = gemm_mfma_eligible(v, x_dtype, m, xs) || gemm_wide_taken(v, x_dtype, m, xs, flags);
     // the clock probe cell lives behind the argmax cells of the context's scratch
     unsigned long long* const probe = (flags & MI355Q_FLAG_PROBE_CLOCK) ? ctx->argmax_scratch + 16 : nullptr;
     if (flags & MI355Q_FLAG_FORCE_MFMA) {
@@ -481,7 +481,8 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
     for (uint32_t i = 0; i < count && stepped; i++)
         stepped = decode_kernel_reads(views[i], x_dtype, xs) && !split_rows_chosen(views[i], x_dtype, m, xs, flags) &&
                   !gemm_two_step_chosen(views[i], x_dtype, m, xs, flags) &&
-                  (m <= small_batch_limit(views[i], x_dtype, xs) || !gemm_mfma_eligible(views[i], x_dtype, m, xs));
+                  (m <= small_batch_limit(views[i], x_dtype, xs) ||
+                   !(gemm_mfma_eligible(views[i], x_dtype, m, xs) || gemm_wide_taken(views[i], x_dtype, m, xs, flags)));
     if (stepped) {
         const size_t xsz = x_dtype == MI355Q_F32 ? 4 : 2, ysz = y_dtype == MI355Q_F32 ? 4 : 2;
         for (uint32_t m0 = 0; m0 < m; m0 += step) {

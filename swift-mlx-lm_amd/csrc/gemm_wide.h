@@ -1,0 +1,31 @@
+// Shared by gemm_wide.hip (choice of shape, launch, sum of K parts) and the two instantiation units of the kernel
+// (gemm_wide_bf16.hip, gemm_wide_f16.hip; kernel text in gemm_wide.inl).
+#pragma once
+#include "common.h"
+
+namespace mi355q {
+
+struct WideArgs {
+    const uint32_t* codes;       // planes: [N, K / 8] words, rows code_stride words apart
+    const uint32_t* sz;          // planes: (scale | bias << 16) per group, rows sz_stride words apart
+    const uint8_t* blocks;       // blocks in place: [f16 scale][f16 zero][codes] per group, rows row_bytes apart
+    const uint16_t* x;           // bf16 or f16 [M, xs]
+    void* y;
+    uint32_t m, n, k, xs, ys;
+    uint32_t code_stride, sz_stride, row_bytes;
+    uint32_t tiles_m, tiles_n;
+    uint32_t y_dtype;
+    uint32_t wide_stores;        // rows of y are 16-byte aligned for every column that is a multiple of four
+    float* partial;              // K split over workgroups: fp32 [splits][M][N] partial results (null otherwise)
+    uint32_t splits, kt_per_split;   // K-tiles per split: a multiple of four
+    unsigned long long* probe;   // optional: [0] shader cycles, [1] 100 MHz ticks that workgroup 0 spent in the kernel
+};
+
+constexpr int kWideStages = 4;   // LDS stages of activations
+constexpr int kWideBN = 256;
+
+// the kernel launch alone (tiles_m, tiles_n filled in here); activations bf16 / f16
+mi355q_status launch_wide_kernel_bf16(hipStream_t s, WideArgs a, uint32_t bm, uint32_t group, bool sb_bf16, bool blocks);
+mi355q_status launch_wide_kernel_f16(hipStream_t s, WideArgs a, uint32_t bm, uint32_t group, bool sb_bf16, bool blocks);
+
+}  // namespace mi355q

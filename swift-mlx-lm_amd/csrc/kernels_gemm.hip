@@ -524,10 +524,10 @@ bool gemm_mfma_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stri
 mi355q_status launch_qgemm_mfma(hipStream_t s, mi355q_context* ctx, const WView& w, const void* x, int x_dtype,
                                 void* y, int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride,
                                 unsigned long long* probe, uint32_t flags) {
-    if (x_dtype != MI355Q_BF16) return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the MFMA GEMM takes bf16 activations");
-    // long prompts on 4-bit planes: the wide-tile kernel with the weights dequantised in registers
+    // long prompts on 4-bit planes and blocks: the wide-tile kernel with the weights dequantised in registers
     if (gemm_wide_taken(w, x_dtype, m, x_stride, flags) && (uintptr_t)x % 16 == 0)
         return launch_qgemm_wide(s, ctx, w, x, x_dtype, y, y_dtype, m, x_stride, y_stride, probe);
+    if (x_dtype != MI355Q_BF16) return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the tiled MFMA GEMM takes bf16 activations");
     if ((uintptr_t)x % 16) return fail(MI355Q_ERR_INVALID_ARGUMENT, "activation pointer must be 16-byte aligned");
     GemmArgs a{};
     a.codes = w.codes; a.sz = w.sz; a.bdense = nullptr;

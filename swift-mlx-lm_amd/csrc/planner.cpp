@@ -253,7 +253,7 @@ mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w, uint32_t maximum
     const bool want_small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) ||
                             (!(flags & MI355Q_FLAG_FORCE_MFMA) && m <= small_rows) ||
                             split_rows_chosen(v, x_dtype, m, input_row_stride, flags);
-    const bool mfma_ok = gemm_mfma_eligible(v, x_dtype, m, input_row_stride);
+    const bool mfma_ok = gemm_mfma_eligible(v, x_dtype, m, input_row_stride) || gemm_wide_taken(v, x_dtype, m, input_row_stride, flags);
     if (!split_rows_chosen(v, x_dtype, m, input_row_stride, flags) && gemm_two_step_chosen(v, x_dtype, m, input_row_stride, flags) &&
         !library_ruled_out(w->ctx)) {
         // dequant_q{b}_g{g}_bf16 into the scratch matrix, then the dense GEMM (MetalPrefillStepBuilder's two-dispatch

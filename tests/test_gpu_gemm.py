@@ -16,7 +16,7 @@ import pytest
 
 import kat
 import oracle
-from gpu_util import Case, act_rounded, assert_within_tolerance, out_from_device, seeded_case
+from gpu_util import act_to_device_array, Case, act_rounded, assert_within_tolerance, out_from_device, seeded_case
 
 pytestmark = pytest.mark.gpu
 KATS = kat.load_kats()
@@ -33,15 +33,16 @@ def bf16_round(a):
     return oracle.bf16_to_f32(oracle.bf16_from_f32(a)).reshape(a.shape)
 
 
-def run_qgemm(ctx, pkg, w, x_f32, y_dtype, flags, x_stride=None, y_stride=None):
-    """x_f32 [M, x_stride] (bf16-representable) -> device result [M, y_stride] as float32."""
+def run_qgemm(ctx, pkg, w, x_f32, y_dtype, flags, x_stride=None, y_stride=None, x_dtype=None):
+    """x_f32 [M, x_stride] (representable in the activation type, bf16 unless given) -> device result [M, y_stride] as float32."""
     m, xs = x_f32.shape
     n = int(w.info.n_rows)
     ys = n if y_stride is None else y_stride
-    xd = ctx.upload(oracle.bf16_from_f32(x_f32).reshape(x_f32.shape))
+    x_dtype = pkg.BF16 if x_dtype is None else x_dtype
+    xd = ctx.upload(act_to_device_array(x_f32, x_dtype, pkg))
     yd = ctx.alloc(m * ys * (4 if y_dtype == pkg.F32 else 2))
     ctx.fill(yd, 0x7FC07FC0 if y_dtype != pkg.F32 else 0x7FC00000)      # NaN canary
-    ctx.qgemm(w, xd, pkg.BF16, yd, y_dtype, m, xs if x_stride is None else x_stride, ys if y_stride else 0, flags)
+    ctx.qgemm(w, xd, x_dtype, yd, y_dtype, m, xs if x_stride is None else x_stride, ys if y_stride else 0, flags)
     ctx.synchronize()
     y = out_from_device(yd, y_dtype, (m, ys), pkg)
     xd.free(); yd.free()

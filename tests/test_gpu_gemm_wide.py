@@ -63,17 +63,21 @@ def test_wide_gemm_exact_small_integers(pkg, ctx, group):
         w.destroy()
 
 
-def _seeded(pkg, ctx, seed, m, n, k, group, flags, sample=None, x_pad=0, y_pad=0, sb=None):
+def _seeded(pkg, ctx, seed, m, n, k, group, flags, sample=None, x_pad=0, y_pad=0, layout=None, x_dtype=None):
+    """Seeded weights and activations through the kernel: fp32 result against the fp64 product of the weights rounded
+    to the activation type (bf16 or f16), and the 16-bit result against the rounding of the fp32 one."""
+    layout = pkg.LAYOUT_PLANES if layout is None else layout
+    x_dtype = pkg.BF16 if x_dtype is None else x_dtype
     words, s, z, wq = seeded_case(seed, n, k, 4, group)
-    wb = bf16_round(wq)
+    wb = bf16_round(wq) if x_dtype == pkg.BF16 else wq.astype(np.float16).astype(np.float32)
     fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, group)
-    w = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, pkg.LAYOUT_PLANES)
+    w = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, layout)
     x = np.zeros((m, k + x_pad), np.float32)
-    x[:, :k] = act_rounded(kat.seeded_activations(seed + 1, m, k), pkg.BF16, pkg)
+    x[:, :k] = act_rounded(kat.seeded_activations(seed + 1, m, k), x_dtype, pkg)
     if x_pad:
         x[:, k:] = 3.0e4
-    say(f"wide seeded g{group} M={m} {k}->{n} pads=({x_pad},{y_pad}) flags={flags}")
-    got = run_qgemm(ctx, pkg, w, x, pkg.F32, flags, y_stride=(n + y_pad) if y_pad else None)
+    say(f"wide seeded g{group} M={m} {k}->{n} pads=({x_pad},{y_pad}) flags={flags} layout={layout} x={x_dtype}")
+    got = run_qgemm(ctx, pkg, w, x, pkg.F32, flags, y_stride=(n + y_pad) if y_pad else None, x_dtype=x_dtype)
     if y_pad:
         assert np.all(np.isnan(got[:, n:])), "padding of the output rows was written"
         got = got[:, :n]
@@ -81,7 +85,7 @@ def _seeded(pkg, ctx, seed, m, n, k, group, flags, sample=None, x_pad=0, y_pad=0
     want = oracle.gemm_f64(np.ascontiguousarray(wb[cols]), np.ascontiguousarray(x[:, :k]))
     r = assert_within_tolerance(got[:, cols], want, f"wide g{group} M={m} {k}->{n}")
     assert np.all(np.isfinite(got))
-    gb = run_qgemm(ctx, pkg, w, x, pkg.BF16, flags)
+    gb = run_qgemm(ctx, pkg, w, x, pkg.BF16, flags, x_dtype=x_dtype)
     assert np.array_equal(oracle.bf16_from_f32(gb), oracle.bf16_from_f32(got)), "bf16 out != rne(fp32 out)"
     return w, x, got, r
 
@@ -96,6 +100,67 @@ def test_wide_gemm_ragged_shapes_against_the_oracle(pkg, ctx):
         tiled = run_qgemm(ctx, pkg, w, x, pkg.F32, pkg.FLAG_FORCE_MFMA | pkg.FLAG_PROBE_TILED)
         assert np.max(np.abs(tiled - got)) <= 2e-5 * max(1.0, float(np.max(np.abs(got)))), "wide vs tiled kernel"
         w.destroy()
+
+
+@pytest.mark.parametrize("group", [64, 128])
+@pytest.mark.parametrize("blocks,f16", [(True, False), (False, True), (True, True)])
+def test_wide_gemm_blocks_in_place_and_f16_activations_exact(pkg, ctx, group, blocks, f16):
+    """The reference's interleaved blocks read in place (a lane's code bytes at 4-byte aligned addresses, scale and zero
+    from the block headers) and f16 activations (weights rounded to f16, f16 matrix instruction): small integers, so
+    every result is exact whatever the order of the sums; all three output types."""
+    rng = np.random.default_rng(4500 + group + 7 * blocks + 13 * f16)
+    m, n, k = 290, 300, 2 * 256
+    codes = rng.integers(0, 16, (n, k), dtype=np.uint8)
+    scales = rng.choice([0.125, 0.25, 0.5], (n, k // group))
+    zeros = rng.integers(-4, 5, (n, k // group)) * 0.25
+    case = Case(4, group, codes, scales, zeros)
+    wq = scales.repeat(group, axis=1) * codes + zeros.repeat(group, axis=1)
+    x = rng.integers(-8, 9, (m, k)).astype(np.float32) * 0.125
+    want = x.astype(np.float64) @ wq.T
+    x_dtype = pkg.F16 if f16 else pkg.BF16
+    w = case.device_weight(ctx, pkg, pkg.LAYOUT_STAF_BLOCKS if blocks else pkg.LAYOUT_PLANES, pkg.BF16)
+    step = w.plan_prefill_steps(m, x_dtype=x_dtype, flags=wide(pkg))[0]
+    assert step.device_kernel == f"qgemm_wide_q4_g{group}" and step.kernel_family == "mfmaGEMM", step.device_kernel
+    for yd in (pkg.F32, pkg.BF16, pkg.F16):
+        say(f"wide exact g{group} blocks={blocks} f16={f16} y={yd}")
+        got = run_qgemm(ctx, pkg, w, x, yd, wide(pkg), x_dtype=x_dtype)
+        if yd == pkg.F32:
+            assert np.array_equal(got.astype(np.float64), want)
+        elif yd == pkg.BF16:
+            assert np.array_equal(got, bf16_round(want.astype(np.float32)))
+        else:
+            assert np.array_equal(got, want.astype(np.float16).astype(np.float32))
+    w.destroy()
+
+
+def test_wide_gemm_blocks_and_f16_seeded_against_the_oracle(pkg, ctx):
+    """Seeded weights: blocks in place give the bits of the planes kernel (same codes, same f16 scales); f16
+    activations hold the bar against the fp64 product of f16-rounded weights."""
+    for i, (m, n, k, group) in enumerate([(257, 300, 512, 64), (130, 515, 768, 128)]):
+        wp, x, got_p, _ = _seeded(pkg, ctx, 4600 + i, m, n, k, group, wide(pkg))
+        wb, _, got_b, _ = _seeded(pkg, ctx, 4600 + i, m, n, k, group, wide(pkg), layout=pkg.LAYOUT_STAF_BLOCKS)
+        assert np.array_equal(got_p, got_b), "blocks in place and planes differ"
+        wp.destroy(); wb.destroy()
+        for layout in (pkg.LAYOUT_PLANES, pkg.LAYOUT_STAF_BLOCKS):
+            w, _, _, _ = _seeded(pkg, ctx, 4610 + i, m, n, k, group, wide(pkg), layout=layout, x_dtype=pkg.F16)
+            w.destroy()
+
+
+@pytest.mark.parametrize("layout_name,x_name", [("LAYOUT_STAF_BLOCKS", "BF16"), ("LAYOUT_PLANES", "F16"), ("LAYOUT_STAF_BLOCKS", "F16")])
+@pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
+def test_config3_on_blocks_and_f16_as_dispatched(pkg, ctx, layout_name, x_name, n, k):
+    """BASELINE config 3 at M = 2048 on the reference's block layout and with its f16 activations, no flags: the
+    plan names this library's matrix-core kernel, and the result holds the bar on the tile-edge column sample."""
+    m = 2048
+    layout, x_dtype = getattr(pkg, layout_name), getattr(pkg, x_name)
+    sample = _tile_edge_sample(n, 31 * m + n, tile=256)
+    w, _, _, (rel, _) = _seeded(pkg, ctx, 4700, m, n, k, 64, 0, sample=sample, layout=layout, x_dtype=x_dtype)
+    steps = w.plan_prefill_steps(m, x_dtype=x_dtype)
+    say("as dispatched:", [s.device_kernel for s in steps])
+    assert len(steps) == 1 and steps[0].device_kernel == "qgemm_wide_q4_g64" and steps[0].kernel_family == "mfmaGEMM"
+    assert not steps[0].used_fallback
+    assert rel < 5e-4
+    w.destroy()
 
 
 @pytest.mark.parametrize("tile_rows,parts", [(256, 2), (256, 4), (128, 3), (128, 4)])
