@@ -154,8 +154,11 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
         const WView v = w->view();
         if (split_rows_chosen(v, x_dtype, m, xs, flags)) return run_split_rows(ctx, s, w, x, x_dtype, y, y_dtype, m, xs, ys, flags);
         if (gemm_two_step_chosen(v, x_dtype, m, xs, flags) && (uintptr_t)x % 16 == 0 &&
-            gemm_two_step_serves(ctx, v, x_dtype, y_dtype, m, xs, ys))
-            return launch_qgemm_two_step(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
+            gemm_two_step_serves(ctx, v, x_dtype, y_dtype, m, xs, ys)) {
+            // (a library result that fails its check makes the problem unusable: the routes below serve the call)
+            const mi355q_status st = launch_qgemm_two_step(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
+            if (st != MI355Q_ERR_KERNEL_NOT_FOUND) return st;
+        }
         if (!(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_SMALL_M)) && gemm_stream_chosen(v, x_dtype, m, xs) &&
             gemm_stream_unrounded(v, m) && (uintptr_t)x % 16 == 0)
             return launch_qgemm_stream(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
@@ -180,8 +183,10 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
     // dequantise once, then the dense library GEMM: long prompts, and every format or layout the fused kernel does
     // not read.  When the library has no algorithm for the problem the routes below serve it.
     if (gemm_two_step_chosen(v, x_dtype, m, xs, flags) && (uintptr_t)x % 16 == 0 &&
-        gemm_two_step_serves(ctx, v, x_dtype, y_dtype, m, xs, ys))
-        return launch_qgemm_two_step(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
+        gemm_two_step_serves(ctx, v, x_dtype, y_dtype, m, xs, ys)) {
+        const mi355q_status st = launch_qgemm_two_step(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
+        if (st != MI355Q_ERR_KERNEL_NOT_FOUND) return st;
+    }
     const bool mfma_ok = gemm_mfma_eligible(v, x_dtype, m, xs) || gemm_wide_taken(v, x_dtype, m, xs, flags);
     // the clock probe cell lives behind the argmax cells of the context's scratch
     unsigned long long* const probe = (flags & MI355Q_FLAG_PROBE_CLOCK) ? ctx->argmax_scratch + 16 : nullptr;
@@ -318,11 +323,13 @@ bool gemm_two_step_serves(mi355q_context* ctx, const WView& w, int x_dtype, int 
     }
 }
 
-// The library's product into a result whose row stride is not N: with long K (14336; not with 4224 or less) the
-// algorithm its heuristic ranks first has returned a wrong matrix into such a result (M = 128, N = 64 or 2056, fp32 and bf16,
-// stride N + 5 or N + 8), while results of stride N are right.  So a padded result is computed densely in scratch and
-// copied row by row.  `free_ws` is scratch of dense_result_bytes() + kDenseLibraryWorkspace bytes; `x_second`, when
-// given, is a second activation matrix whose product is added to the first's (the low halves of split fp32 rows).
+// The library's product into a result whose row stride is not N: with long K (14336; not with 4224 or less) its
+// split-K algorithms, the heuristic's first among them, return a wrong matrix into such a result (M = 128, N = 64 or
+// 2056, fp32 and bf16, stride N + 5 or N + 8: every run, whatever the workspace holds before, and garbage placed in
+// the workspace shows up in the result -- the sum of the parts reads with another row stride than they were written
+// with), while results of stride N are right.  So a padded result is computed densely in scratch and copied row by
+// row.  `free_ws` is scratch of dense_result_bytes() bytes; `x_second`, when given, is a second activation matrix
+// whose product is added to the first's (the low halves of split fp32 rows).
 size_t dense_result_bytes(uint32_t m, uint32_t n, uint32_t y_stride, int y_dtype) {
     return y_stride == n ? 0 : (((size_t)m * n * (y_dtype == MI355Q_F32 ? 4 : 2)) + 255) & ~(size_t)255;
 }
@@ -333,12 +340,11 @@ mi355q_status dense_gemm_into(hipStream_t s, mi355q_context* ctx, int ab_dtype, 
     const size_t tmp_bytes = dense_result_bytes(m, n, y_stride, y_dtype);
     void* const out = tmp_bytes ? (void*)free_ws : y;
     const uint32_t out_stride = tmp_bytes ? n : y_stride;
-    void* const lib_ws = free_ws + tmp_bytes;
-    if (mi355q_status st = dense_library_gemm(s, ctx, ab_dtype, x, w_dense, out, y_dtype, m, n, k, x_stride, out_stride, lib_ws,
-                                              false)) return st;
+    if (mi355q_status st = dense_library_gemm(s, ctx, ab_dtype, x, w_dense, out, y_dtype, m, n, k, x_stride, out_stride, false))
+        return st;
     if (x_second)
         if (mi355q_status st = dense_library_gemm(s, ctx, ab_dtype, x_second, w_dense, out, y_dtype, m, n, k, x_stride, out_stride,
-                                                  lib_ws, true)) return st;
+                                                  true)) return st;
     if (!tmp_bytes) return MI355Q_OK;
     const size_t ysz = y_dtype == MI355Q_F32 ? 4 : 2;
     for (uint32_t m0 = 0; m0 < m; m0 += 65535u) {
@@ -361,7 +367,7 @@ mi355q_status launch_qgemm_two_step(hipStream_t s, mi355q_context* ctx, const WV
         const size_t wbytes = round256((size_t)n * k * 4), xbytes = widen ? round256((size_t)m * k * 4) : 0;
         const size_t ybytes = narrow ? round256((size_t)m * n * 4) : 0;
         const size_t dense_y = narrow ? 0 : dense_result_bytes(m, n, y_stride, MI355Q_F32);
-        if (mi355q_status st = ensure_workspace(ctx, wbytes + xbytes + ybytes + dense_y + kDenseLibraryWorkspace)) return st;
+        if (mi355q_status st = ensure_workspace(ctx, wbytes + xbytes + ybytes + dense_y)) return st;
         char* const base = (char*)ctx->workspace;
         float* const w32 = (float*)base;
         float* const x32 = widen ? (float*)(base + wbytes) : (float*)const_cast<void*>(x);
@@ -376,8 +382,7 @@ mi355q_status launch_qgemm_two_step(hipStream_t s, mi355q_context* ctx, const WV
     }
     if (form == TwoStepForm::kSplitF32) {
         const size_t wbytes = round256((size_t)n * k * 2), xbytes = round256((size_t)m * k * 2);
-        if (mi355q_status st = ensure_workspace(ctx, wbytes + 2 * xbytes + dense_result_bytes(m, n, y_stride, MI355Q_F32) +
-                                                         kDenseLibraryWorkspace)) return st;
+        if (mi355q_status st = ensure_workspace(ctx, wbytes + 2 * xbytes + dense_result_bytes(m, n, y_stride, MI355Q_F32))) return st;
         char* const base = (char*)ctx->workspace;
         uint16_t* const w_bf16 = (uint16_t*)base;
         uint16_t* const hi = (uint16_t*)(base + wbytes);
@@ -388,7 +393,7 @@ mi355q_status launch_qgemm_two_step(hipStream_t s, mi355q_context* ctx, const WV
     }
     const size_t esz = x_dtype == MI355Q_F32 ? 4 : 2;
     const size_t dense = round256((size_t)n * k * esz);
-    if (mi355q_status st = ensure_workspace(ctx, dense + dense_result_bytes(m, n, y_stride, y_dtype) + kDenseLibraryWorkspace)) return st;
+    if (mi355q_status st = ensure_workspace(ctx, dense + dense_result_bytes(m, n, y_stride, y_dtype))) return st;
     void* const w_dense = ctx->workspace;
     const mi355q_status st = x_dtype == MI355Q_BF16 ? launch_dequant_bf16(s, w, (uint16_t*)w_dense)
                            : x_dtype == MI355Q_F16 ? launch_dequant_f16(s, w, (uint16_t*)w_dense)
@@ -599,9 +604,10 @@ mi355q_status mi355q_gemm_bf16(mi355q_context* ctx, void* stream, const void* a_
     if (a_dtype == MI355Q_BF16 && m >= kDenseLibraryMinRows && k % 8 == 0 && a_row_stride % 8 == 0 &&
         (uintptr_t)a_dev % 16 == 0 && (uintptr_t)b_bf16_dev % 16 == 0 &&
         dense_library_serves(ctx, MI355Q_BF16, m, n, k, a_row_stride, n, c_dtype)) {
-        if (mi355q_status st = ensure_workspace(ctx, mi355q::dense_result_bytes(m, n, c_row_stride, c_dtype) + kDenseLibraryWorkspace)) return st;
-        return mi355q::dense_gemm_into((hipStream_t)stream, ctx, MI355Q_BF16, a_dev, b_bf16_dev, c_dev, c_dtype, m, n, k,
-                                       a_row_stride, c_row_stride, (char*)ctx->workspace);
+        if (mi355q_status st = ensure_workspace(ctx, mi355q::dense_result_bytes(m, n, c_row_stride, c_dtype))) return st;
+        const mi355q_status st = mi355q::dense_gemm_into((hipStream_t)stream, ctx, MI355Q_BF16, a_dev, b_bf16_dev, c_dev, c_dtype,
+                                                         m, n, k, a_row_stride, c_row_stride, (char*)ctx->workspace);
+        if (st != MI355Q_ERR_KERNEL_NOT_FOUND) return st;        // a library result that failed its check: this library's kernel
     }
     return launch_gemm_bf16_mfma((hipStream_t)stream, ctx, a_dev, a_dtype, (const uint16_t*)b_bf16_dev, c_dev,
                                  c_dtype, m, n, k, a_row_stride, c_row_stride);

@@ -339,14 +339,17 @@ mi355q_status launch_qgemm_stream_multi(hipStream_t s, mi355q_context* ctx, uint
                                         uint32_t x_stride);
 // Two-dispatch prefill route: dequantise the whole matrix to bf16 in the context's scratch, then the platform's
 // dense GEMM.  `dense_library_serves` answers whether the library can be opened and has an algorithm for the problem.
+// The library's workspace is its own allocation per context (zeroed once, written by nothing else).
 constexpr size_t kDenseLibraryWorkspace = (size_t)64 << 20;
 // Both operands in `ab_dtype` (bf16, f16 or fp32), fp32 accumulation, output in y_dtype.
 bool dense_library_serves(mi355q_context* ctx, int ab_dtype, uint32_t m, uint32_t n, uint32_t k, uint32_t x_stride,
                           uint32_t y_stride, int y_dtype);
-// `accumulate`: Y += X W^T instead of Y = X W^T (the second half of a split-activation product).
+// `accumulate`: Y += X W^T instead of Y = X W^T (the second half of a split-activation product).  The first eager call
+// of a problem checks sampled result elements against plain dot products (and synchronises the stream); a wrong
+// matrix makes the problem unusable and returns MI355Q_ERR_KERNEL_NOT_FOUND, on which callers take another route.
 mi355q_status dense_library_gemm(hipStream_t s, mi355q_context* ctx, int ab_dtype, const void* x, const void* w_dense,
                                  void* y, int y_dtype, uint32_t m, uint32_t n, uint32_t k, uint32_t x_stride,
-                                 uint32_t y_stride, void* workspace, bool accumulate = false);
+                                 uint32_t y_stride, bool accumulate = false);
 void dense_library_release(mi355q_context* ctx);
 // Rows from which the two-dispatch route is taken.  Beside the fused matrix-core kernel (measured at sustained load,
 // q4 g64, N(0,1) activations, fused against two-dispatch with the library's candidates timed): 4096 -> 14336 at M = 512

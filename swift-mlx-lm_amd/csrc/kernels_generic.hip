@@ -371,7 +371,11 @@ __global__ __launch_bounds__(256) void split_f32_bf16x2_kernel(const float* __re
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             h[i] = f32_to_bf16_rne(f[i]);
-            l[i] = f32_to_bf16_rne(f[i] - __uint_as_float((uint32_t)h[i] << 16));
+            // a finite value above the largest bf16 would round to infinity: the largest bf16 and a remainder instead;
+            // a non-finite one stands alone
+            const bool finite = f[i] - f[i] == 0.0f;
+            if (finite && (h[i] & 0x7FFFu) == 0x7F80u) h[i] = (uint16_t)((h[i] & 0x8000u) | 0x7F7Fu);
+            l[i] = finite ? f32_to_bf16_rne(f[i] - __uint_as_float((uint32_t)h[i] << 16)) : (uint16_t)0;
         }
         uint2 hv, lv;
         hv.x = h[0] | ((uint32_t)h[1] << 16); hv.y = h[2] | ((uint32_t)h[3] << 16);
@@ -419,8 +423,12 @@ __global__ __launch_bounds__(256) void split_rows_bf16_kernel(const float* __res
     for (uint32_t c = blockIdx.x * 256 + threadIdx.x; c < k; c += gridDim.x * 256) {
         const float v = x[(size_t)row * x_stride + c];
         uint16_t part[3] = {f32_to_bf16_rne(v), 0, 0};
+        // a finite v above the largest bf16 would round to infinity: its high part is the largest bf16 instead, and the
+        // remainder splits like any other
+        if (v - v == 0.0f && (part[0] & 0x7FFFu) == 0x7F80u) part[0] = (uint16_t)((part[0] & 0x8000u) | 0x7F7Fu);
+        const float high = __uint_as_float((uint32_t)part[0] << 16);
         if (v - v == 0.0f) {                                // finite
-            float r = v - __uint_as_float((uint32_t)part[0] << 16);
+            float r = v - high;
 #pragma unroll
             for (int p = 1; p < 3; p++) {
                 part[p] = f32_to_bf16_rne(r);

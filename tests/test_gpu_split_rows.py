@@ -123,18 +123,24 @@ def test_f32_rows_exact_values_padding_and_output_types(pkg, ctx):
 
 def test_f32_rows_non_finite_activation_and_graph_replay(pkg, ctx):
     """An infinite activation stays in the first bf16 part (the output row is non-finite where its weight is not zero,
-    finite rows are untouched); a plan with fp32 rows replays as a HIP graph with the same result every time."""
-    n, k, m = 64, 1024, 3
+    finite rows are untouched); a finite one above the largest bf16 (its rounding to bf16 is infinite) takes the largest
+    bf16 as its first part and a remainder, so its parts never cancel into NaN (the row overflows to infinity inside the
+    bf16 kernels, whose code values carry an offset of 128); a plan with fp32 rows replays as a HIP graph with the same
+    result every time."""
+    n, k, m = 64, 1024, 4
     words, s, z, wq = seeded_case(5400, n, k, 4, 64)
     fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
     w = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, pkg.LAYOUT_PLANES)
     x = kat.seeded_activations(5401, m, k).astype(np.float32)
     x[1, 17] = np.inf
+    x[3, 29] = 3.4e38
     got = run_f32(ctx, pkg, w, x)
     assert not np.any(np.isfinite(got[1][wq[:, 17] != 0]))
+    assert not np.any(np.isnan(got[3]))
     fin = oracle.gemm_f64(wq, x[[0, 2]])
     assert rel_l2(got[[0, 2]], fin) <= 1e-5
     x[1, 17] = 0.25
+    x[3, 29] = 0.5
     xd = ctx.upload(x); yd = ctx.alloc(m * n * 4)
     plan = pkg.DispatchPlan(ctx)
     plan.add_linear(w, xd, pkg.F32, yd, pkg.F32, m)
