@@ -63,7 +63,7 @@ mi355q_status run_small_m(mi355q_context* ctx, hipStream_t s, const mi355q_weigh
             const uint32_t strides[1] = {ys};
             st = launch_gemv_tile16_multi(s, ctx, 1, &v, xp, x_dtype, yv, strides, y_dtype, mm, xs, nullptr, nullptr, HeadKeys{});
         } else if (!generic && mfma_planes_pays(v.bits, x_dtype, mm) && gemv_mfma_planes_eligible(v, x_dtype, mm, xs) &&
-                   (uintptr_t)xp % 16 == 0) {
+                   !(gemv_rows_batch_pays(1, &v, x_dtype, mm) && gemv_fast_eligible(v, x_dtype, mm, xs)) && (uintptr_t)xp % 16 == 0) {
             void* yv[1] = {yp};
             const uint32_t strides[1] = {ys};
             st = launch_gemv_mfma_planes_multi(s, ctx, 1, &v, xp, x_dtype, yv, strides, y_dtype, mm, xs);
@@ -441,6 +441,7 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
                     gemv_mfma_planes_k_parts(ctx, views[i], staged_rows(x_dtype, m)) == 1 && views[i].sb_dtype == views[0].sb_dtype &&
                     views[i].code_stride == views[0].code_stride && views[i].group == views[0].group;
     }
+    if (fused && gemv_rows_batch_pays(count, views, x_dtype, m)) on_planes = false;      // small matrices, three or four rows
     // the streamed-weight kernel, one launch for the two or three matrices: a few dozen rows on 4- / 8-bit planes, and
     // blocks in place from three to nine rows by the size of the matrices together
     const bool no_stream = flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_TWO_STEP | MI355Q_FLAG_FORCE_SMALL_M);

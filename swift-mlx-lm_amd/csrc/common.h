@@ -239,6 +239,21 @@ inline uint32_t mfma_planes_min_rows(uint32_t bits) { (void)bits; return 3u; }
 inline bool mfma_planes_pays(uint32_t bits, int x_dtype, uint32_t m) {
     return x_dtype == MI355Q_F16 ? m >= 3 : m >= mfma_planes_min_rows(bits);
 }
+// Three or four bf16 rows on small 4-bit matrices (rows of two K-steps of the dot-product rows kernel; below 24 MB of
+// weights in the launch at three rows, below 12 MB at four) stay on that kernel, every row on each unpacked code
+// pair: its launch starts and ends faster than the matrix-core kernel's, whose workgroups stage the batch and add
+// partial tiles through LDS (Llama-3-8B: q+k+v 14 MB at three rows 7.5 us against 8.8 us, at four 9.4 against 9.0;
+// o 9 MB 6.1 against 8.7 and 6.8 against 8.8; gate+up and down stay on the matrix cores).
+inline bool gemv_rows_batch_pays(uint32_t count, const WView* v, int x_dtype, uint32_t m) {
+    if (x_dtype != MI355Q_BF16 || m < 3 || m > 4) return false;
+    uint64_t bytes = 0;
+    for (uint32_t i = 0; i < count; i++) {
+        if (v[i].layout != MI355Q_LAYOUT_PLANES || v[i].bits != 4 || (v[i].group != 64 && v[i].group != 128)) return false;
+        if (v[i].k <= 2048 || v[i].k > 4096) return false;
+        bytes += (uint64_t)v[i].n * (v[i].k / v[i].group) * (4 + v[i].group / 2);
+    }
+    return bytes < ((uint64_t)(m == 3 ? 24 : 12) << 20);
+}
 bool gemv_mfma_planes_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
 // (m below: staged rows, see staged_rows)
 uint32_t gemv_mfma_planes_k_parts(const mi355q_context* ctx, const WView& w, uint32_t m);

@@ -56,6 +56,27 @@ template <int BITS, int GROUP, int NCT, int BR, int WAVES>
 mi355q_status launch_rows(hipStream_t s, const GemvArgs& a, const GemvCfg& c) {
     const bool sbbf = a.sb_dtype == MI355Q_BF16;
     const uint32_t block = WAVES * 64;
+    if (c.mt > 1) {
+        if (!c.argmax && !c.gated && !c.xa) {
+            if constexpr (gemv_rows_has_batch(BITS, GROUP, NCT, BR, 2)) {
+                if (c.mt == 2) {
+                    if (sbbf) return launch_kernel(gemv_rows_kernel<BITS, GROUP, NCT, BR, WAVES, 0, true, false, false, 2>, s, a, c.grid, block, c.lds);
+                    return launch_kernel(gemv_rows_kernel<BITS, GROUP, NCT, BR, WAVES, 0, false, false, false, 2>, s, a, c.grid, block, c.lds);
+                }
+            }
+            if constexpr (gemv_rows_has_batch(BITS, GROUP, NCT, BR, 3)) {
+                if (c.mt == 3) {
+                    if (sbbf) return launch_kernel(gemv_rows_kernel<BITS, GROUP, NCT, BR, WAVES, 0, true, false, false, 3>, s, a, c.grid, block, c.lds);
+                    return launch_kernel(gemv_rows_kernel<BITS, GROUP, NCT, BR, WAVES, 0, false, false, false, 3>, s, a, c.grid, block, c.lds);
+                }
+                if (c.mt == 4) {
+                    if (sbbf) return launch_kernel(gemv_rows_kernel<BITS, GROUP, NCT, BR, WAVES, 0, true, false, false, 4>, s, a, c.grid, block, c.lds);
+                    return launch_kernel(gemv_rows_kernel<BITS, GROUP, NCT, BR, WAVES, 0, false, false, false, 4>, s, a, c.grid, block, c.lds);
+                }
+            }
+        }
+        return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no %d-row variant of the row kernel for q%d g%d steps=%d rows=%d", c.mt, BITS, GROUP, NCT, BR);
+    }
     if (c.gated) {
         if (c.argmax) return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the gated row kernel has no arg-max tail");
         if (c.xa) {

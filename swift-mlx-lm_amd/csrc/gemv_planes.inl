@@ -95,6 +95,16 @@ constexpr bool gemv_rows_has_shape(int nct, int br) {
     return (nct == 1 && (br == 1 || br == 2 || br == 4 || br == 8)) || (nct == 2 && (br == 1 || br == 2 || br == 4)) ||
            ((nct == 3 || nct == 4) && (br == 1 || br == 2)) || (nct == 7 && br == 1);
 }
+// Two to four activation rows on the static-structure kernel: 4-bit codes with bf16 activations.  Two rows: the shapes
+// the chooser gives whole matrices (one pass of four rows of one K-step, of two rows of two to four, one row of seven;
+// one row of two K-steps for matrices of few rows).  Three and four rows: rows of two K-steps (K up to 4096), where
+// matrices are small enough for this kernel's short start to beat the matrix-core kernel.
+constexpr bool gemv_rows_has_batch(int bits, int group, int nct, int br, int mt) {
+    if (bits != 4 || (group != 64 && group != 128)) return false;
+    if (mt == 2) return (nct == 1 && br == 4) || (nct >= 2 && nct <= 4 && br == 2) || (nct == 2 && br == 1) || (nct == 7 && br == 1);
+    if (mt == 3 || mt == 4) return nct == 2 && (br == 1 || br == 2);
+    return false;
+}
 // wavefronts per workgroup: four (measured best for rows of up to four K-steps at every bit width: with eight or
 // sixteen, more wavefronts wait at the staging barrier), eight for rows of seven K-steps, whose staged copy is 28 KiB
 constexpr int gemv_rows_waves(int nct) { return nct <= 4 ? 4 : 8; }

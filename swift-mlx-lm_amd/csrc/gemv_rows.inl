@@ -49,9 +49,12 @@ __host__ __device__ constexpr InplacePair inplace_pair3(int i) {
 // index, their sums are parked in neighbouring lanes, and the epilogue stores activation(gate) * up: one output
 // vector instead of two, and no elementwise launch (generateGatedActivation,
 // Generator/MetalSourceGenerator+NormAndElementwise.swift:196-249).
-template <int BITS, int GROUP, int NCT, int BR, int WAVES, int XA, bool SBBF16, bool ARGMAX, bool GATED = false>
+// MT: activation rows (1 to 4).  They share every unpacked code pair: the unpack, the scale / bias conversion and the
+// bookkeeping are paid once, the dot products per row, so a further row costs about a fifth of the first.
+template <int BITS, int GROUP, int NCT, int BR, int WAVES, int XA, bool SBBF16, bool ARGMAX, bool GATED = false, int MT = 1>
 __global__ __launch_bounds__(WAVES * 64) void gemv_rows_kernel(GemvArgs a) {
     static_assert(!(GATED && ARGMAX), "the gated epilogue has no arg-max tail");
+    static_assert(MT == 1 || (!GATED && !ARGMAX), "batches have neither the gated epilogue nor the arg-max tail");
     using G = GemvGeo<BITS>;
     constexpr int WPL = G::WPL, CPL = G::CPL;
     constexpr int Q = CPL / 8;
@@ -69,8 +72,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_rows_kernel(GemvArgs a) {
     static_assert(BR == 1 || BR == 2 || BR == 4 || BR == 8, "rows per pass: a power of two up to 8");
 
     extern __shared__ u32x4 smem[];
-    u32x4* xs = smem;                                              // [NCT][Q][64]
-    float* sxs = (float*)(smem + (size_t)NCT * Q * 64);             // [NCT][NSR][NF][64]
+    u32x4* xs = smem;                                              // [MT][NCT][Q][64]
+    float* sxs = (float*)(smem + (size_t)MT * NCT * Q * 64);        // [MT][NCT][NSR][NF][64]
 
 #ifdef MI355Q_GEMV_TIMELINE
     const unsigned long long tl_entry = __builtin_amdgcn_s_memrealtime();
@@ -131,11 +134,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_rows_kernel(GemvArgs a) {
         for (int sr = 0; sr < NSR; sr++) s.sz[sr] = MI355Q_STREAM_LOAD((const uint32_t*)(zp + vsz[c][sr]));
     };
 
-    // ---- staging: task cc = the 64 lane chunks of K-step cc, dealt to wavefronts whole ----------------------
+    // ---- staging: task cc = the 64 lane chunks of K-step cc % NCT of activation row cc / NCT, dealt to wavefronts whole
     auto stage_load = [&](uint32_t cc, uint32_t (&d)[CPL / 2]) {
-        const uint64_t kbase = (uint64_t)cc * KC + (uint64_t)lane * CPL;
-        const bool valid = cc < (uint32_t)NCT && kbase < a.k;
-        const u32x4* src = (const u32x4*)(a.x + (valid ? kbase : 0));
+        const uint32_t xrow = MT == 1 ? 0u : cc / (uint32_t)NCT, step_of = MT == 1 ? cc : cc % (uint32_t)NCT;
+        const uint64_t kbase = (uint64_t)step_of * KC + (uint64_t)lane * CPL;
+        const bool valid = cc < (uint32_t)(MT * NCT) && kbase < a.k;
+        const u32x4* src = (const u32x4*)(a.x + (valid ? (uint64_t)xrow * a.x_stride + kbase : 0));
 #pragma unroll
         for (int i = 0; i < Q; i++) {
             const u32x4 v = src[i];                         // clamped address: always readable
@@ -144,7 +148,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_rows_kernel(GemvArgs a) {
         }
     };
     auto stage_store = [&](uint32_t cc, const uint32_t (&d)[CPL / 2]) {
-        if (cc >= (uint32_t)NCT) return;
+        if (cc >= (uint32_t)(MT * NCT)) return;
         uint32_t pw[CPL / 2];                               // staged pairs in the order the unpacker produces them
         float sx_true = 0.0f;                               // INPLACE: sum of the activations before they are scaled
         static_for<CPL / 2>([&](auto I) {
@@ -217,7 +221,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_rows_kernel(GemvArgs a) {
 
     // ---- 3. stage the activations behind an LDS-only barrier ----------------------------------------------
     stage_store(wave, dearly);
-    for (uint32_t cc = wave + WAVES; cc < (uint32_t)NCT; cc += WAVES) {
+    for (uint32_t cc = wave + WAVES; cc < (uint32_t)(MT * NCT); cc += WAVES) {
         uint32_t dl[CPL / 2];
         stage_load(cc, dl);
         stage_store(cc, dl);
@@ -247,17 +251,19 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_rows_kernel(GemvArgs a) {
     }
 
     // contribution of one K-step of one row: sum over its sub-runs of s * sum(q x) + z * sum(x)
-    auto step = [&](const Slot& cur, auto C) -> float {
+    // (added to out[m] for each of the MT activation rows)
+    auto step = [&](const Slot& cur, auto C, float (&out)[MT]) {
         constexpr int c = decltype(C)::value;
-        float dot[NSR][NCLS];
+        float dot[MT][NSR][NCLS];
 #pragma unroll
-        for (int sr = 0; sr < NSR; sr++)
+        for (int m = 0; m < MT; m++)
 #pragma unroll
-            for (int cl = 0; cl < NCLS; cl++) dot[sr][cl] = 0.0f;
+            for (int sr = 0; sr < NSR; sr++)
+#pragma unroll
+                for (int cl = 0; cl < NCLS; cl++) dot[m][sr][cl] = 0.0f;
         static_for<Q>([&](auto P) {
             constexpr int p = decltype(P)::value;
             constexpr int sr = (p * 8) / SR;
-            const u32x4 xv = xs[((size_t)c * Q + p) * 64 + lane];
             if constexpr (DOT2) {
                 uint32_t pr[4];
                 if constexpr (MULTI && BITS == 4) {
@@ -320,65 +326,87 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_rows_kernel(GemvArgs a) {
                 }
                 constexpr int c0 = MULTI ? f16_pair_class<BITS>(4 * p + 0) : 0, c1 = MULTI ? f16_pair_class<BITS>(4 * p + 1) : 0;
                 constexpr int c2 = MULTI ? f16_pair_class<BITS>(4 * p + 2) : 0, c3 = MULTI ? f16_pair_class<BITS>(4 * p + 3) : 0;
-                dot[sr][c0] = dot2_x<XA>(pr[0], xv.x, dot[sr][c0]);
-                dot[sr][c1] = dot2_x<XA>(pr[1], xv.y, dot[sr][c1]);
-                dot[sr][c2] = dot2_x<XA>(pr[2], xv.z, dot[sr][c2]);
-                dot[sr][c3] = dot2_x<XA>(pr[3], xv.w, dot[sr][c3]);
+#pragma unroll
+                for (int m = 0; m < MT; m++) {
+                    const u32x4 xv = xs[((size_t)(m * NCT + c) * Q + p) * 64 + lane];
+                    dot[m][sr][c0] = dot2_x<XA>(pr[0], xv.x, dot[m][sr][c0]);
+                    dot[m][sr][c1] = dot2_x<XA>(pr[1], xv.y, dot[m][sr][c1]);
+                    dot[m][sr][c2] = dot2_x<XA>(pr[2], xv.z, dot[m][sr][c2]);
+                    dot[m][sr][c3] = dot2_x<XA>(pr[3], xv.w, dot[m][sr][c3]);
+                }
             } else {
                 // 8-bit codes with bf16 activations: (128 + q) is not exact in bf16, so fp32 FMA on converted codes
-                const float xf[8] = {__uint_as_float(xv.x << 16), __uint_as_float(xv.x & 0xFFFF0000u),
-                                     __uint_as_float(xv.y << 16), __uint_as_float(xv.y & 0xFFFF0000u),
-                                     __uint_as_float(xv.z << 16), __uint_as_float(xv.z & 0xFFFF0000u),
-                                     __uint_as_float(xv.w << 16), __uint_as_float(xv.w & 0xFFFF0000u)};
-                float dsum = dot[sr][0];
+                float qf[8];
                 static_for<8>([&](auto E) {
                     constexpr int e = decltype(E)::value;
-                    dsum = __builtin_fmaf((float)extract_code<(p * 8 + e) * BITS, BITS, WPL>(cur.w), xf[e], dsum);
+                    qf[e] = (float)extract_code<(p * 8 + e) * BITS, BITS, WPL>(cur.w);
                 });
-                dot[sr][0] = dsum;
+#pragma unroll
+                for (int m = 0; m < MT; m++) {
+                    const u32x4 xv = xs[((size_t)(m * NCT + c) * Q + p) * 64 + lane];
+                    const float xf[8] = {__uint_as_float(xv.x << 16), __uint_as_float(xv.x & 0xFFFF0000u),
+                                         __uint_as_float(xv.y << 16), __uint_as_float(xv.y & 0xFFFF0000u),
+                                         __uint_as_float(xv.z << 16), __uint_as_float(xv.z & 0xFFFF0000u),
+                                         __uint_as_float(xv.w << 16), __uint_as_float(xv.w & 0xFFFF0000u)};
+                    float dsum = dot[m][sr][0];
+#pragma unroll
+                    for (int e = 0; e < 8; e++) dsum = __builtin_fmaf(qf[e], xf[e], dsum);
+                    dot[m][sr][0] = dsum;
+                }
             }
         });
-        float out = 0.0f;
 #pragma unroll
         for (int sr = 0; sr < NSR; sr++) {
-            const float* const cell = sxs + ((size_t)c * NSR + sr) * NF * 64 + lane;
-            const float sx = cell[0];
             float s, z;
             const uint32_t szw = cur.sz[sr];
             if constexpr (SBBF16) { s = __uint_as_float(szw << 16); z = __uint_as_float(szw & 0xFFFF0000u); }
             else { s = f16_to_f32((uint16_t)(szw & 0xFFFFu)); z = f16_to_f32((uint16_t)(szw >> 16)); }
-            if constexpr (INPLACE) {
-                out = __builtin_fmaf(s, dot[sr][0] - cell[64], __builtin_fmaf(z, sx, out));
-            } else if constexpr (MULTI) {
-                float t = dot[sr][0];
 #pragma unroll
-                for (int cl = 1; cl < NCLS; cl++) t = __builtin_fmaf(dot[sr][cl], 1.0f / (float)(1 << f16_class_shift<BITS>(cl)), t);
-                t -= cell[64];
-                out = __builtin_fmaf(s, t, __builtin_fmaf(z, sx, out));
-            } else {
-                out += s * dot[sr][0] + (z - OFS * s) * sx;
+            for (int m = 0; m < MT; m++) {
+                const float* const cell = sxs + ((size_t)(m * NCT + c) * NSR + sr) * NF * 64 + lane;
+                const float sx = cell[0];
+                if constexpr (INPLACE) {
+                    out[m] = __builtin_fmaf(s, dot[m][sr][0] - cell[64], __builtin_fmaf(z, sx, out[m]));
+                } else if constexpr (MULTI) {
+                    float t = dot[m][sr][0];
+#pragma unroll
+                    for (int cl = 1; cl < NCLS; cl++)
+                        t = __builtin_fmaf(dot[m][sr][cl], 1.0f / (float)(1 << f16_class_shift<BITS>(cl)), t);
+                    t -= cell[64];
+                    out[m] = __builtin_fmaf(s, t, __builtin_fmaf(z, sx, out[m]));
+                } else {
+                    out[m] += s * dot[m][sr][0] + (z - OFS * s) * sx;
+                }
             }
         }
-        return out;
     };
 
-    float res = 0.0f;                                        // lane i parks the result of the wavefront's i-th row
+    float resm[MT];                                          // lane i parks the results of the wavefront's i-th row
+#pragma unroll
+    for (int m = 0; m < MT; m++) resm[m] = 0.0f;
     auto pass_body = [&](uint32_t pass, auto ISSUE_T) {
         constexpr bool ISSUE = decltype(ISSUE_T)::value;
-        float acc[BR];
+        float acc[MT][BR];
 #pragma unroll
         for (int j = 0; j < BR; j++) {
             const char *cp = nullptr, *zp = nullptr;
             if constexpr (ISSUE) row_ptrs((pass + 1) * BR + j, cp, zp);
-            acc[j] = 0.0f;
+            float o[MT];
+#pragma unroll
+            for (int m = 0; m < MT; m++) o[m] = 0.0f;
             static_for<NCT>([&](auto C) {
-                acc[j] += step(ring[j][decltype(C)::value], C);
+                step(ring[j][decltype(C)::value], C, o);
                 if constexpr (ISSUE) issue(cp, zp, decltype(C)::value, ring[j][decltype(C)::value]);
             });
+#pragma unroll
+            for (int m = 0; m < MT; m++) acc[m][j] = o[m];
             asm volatile("" ::: "memory");                  // the next row reads the activations from LDS again (registers stay free)
         }
-        const float v = transpose_reduce<BR>(acc, lane);    // lane l holds the sum of row (l & (BR - 1)) of this pass
-        res = ((lane & ~(uint32_t)(BR - 1)) == pass * BR) ? v : res;
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            const float v = transpose_reduce<BR>(acc[m], lane);    // lane l holds the sum of row (l & (BR - 1)) of this pass
+            resm[m] = ((lane & ~(uint32_t)(BR - 1)) == pass * BR) ? v : resm[m];
+        }
     };
     const uint32_t passes = (nrows + BR - 1) / BR;
 #ifdef MI355Q_GEMV_TIMELINE
@@ -402,6 +430,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_rows_kernel(GemvArgs a) {
 #endif
 
     // ---- one coalesced store of the parked results (rows_per_wave <= 64) ------------------------------------
+    const float res = resm[0];
+    if constexpr (MT > 1) {
+        const uint32_t ys = in2 ? a.y_stride[2] : in1 ? a.y_stride[1] : a.y_stride[0];
+        if (lane < nrows && seg_y) {
+#pragma unroll
+            for (int m = 0; m < MT; m++) {
+                const size_t o = (size_t)m * ys + row0 + lane;
+                if (a.y_dtype == MI355Q_F32) ((float*)seg_y)[o] = resm[m];
+                else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)seg_y)[o] = f32_to_bf16_rne(resm[m]);
+                else ((uint16_t*)seg_y)[o] = f32_to_f16_rne(resm[m]);
+            }
+        }
+        return;
+    }
     if constexpr (GATED) {
         // lanes 2 r and 2 r + 1 hold the gate and the up sum of output row (row0 / 2 + r): both are rounded to the
         // output type first, as the reference's elementwise kernel reads them back from buffers of that type

@@ -71,8 +71,13 @@ GemvCfg choose(const mi355q_context* ctx, const WView& w, uint32_t m, bool argma
     // wavefronts per CU (measured, q4 g64: 28672 rows of two K-steps 12.1-12.3 us with two rows per wavefront,
     // 12.4-14.0 with four, 13.8-14.1 with one; 14336 rows 7.5 / 8.2 / 8.0 us; 4096 rows 4.2 us either way; 14336 rows
     // of four K-steps, q8 g32: 12.2 us with two rows, 14.4 with one; q6 g64 10.0 / 10.1; q3 g64 8.1 / 8.8).
-    if (c.mt == 1 && gemv_rows_has_format((int)w.bits, (int)w.group) && (!c.xa || gemv_rows_has_f16((int)w.bits, (int)w.group)) &&
-        (c.nc <= 4 || (c.nc == 7 && w.bits != 8))) {
+    // Two to four activation rows (4 bits, bf16): the same kernel with every row on each unpacked code pair (28672 rows
+    // of two K-steps at two rows: 18.4 us on the general kernel, 15.7 us here; a further row costs the dot products
+    // alone).  Three and four rows where gemv_rows_batch_pays() says so (the callers ask).
+    const bool two_rows = m >= 2 && m <= 4 && !argmax && !c.xa && w.bits == 4;
+    if (two_rows) c.mt = (int)m;
+    if ((c.mt == 1 || two_rows) && gemv_rows_has_format((int)w.bits, (int)w.group) &&
+        (!c.xa || gemv_rows_has_f16((int)w.bits, (int)w.group)) && (c.nc <= 4 || (c.nc == 7 && w.bits != 8))) {
         const uint32_t least_waves = (uint32_t)ctx->props.multiProcessorCount * 16u;
         uint32_t rpw = c.nc == 1 ? 4 : c.nc <= 4 ? 2 : 1;
         while (rpw > 1 && w.n / rpw < least_waves) rpw >>= 1;
@@ -86,20 +91,22 @@ GemvCfg choose(const mi355q_context* ctx, const WView& w, uint32_t m, bool argma
         rpw = (rpw + br - 1) / br * br;
         // very tall matrices: more passes rather than more than 65535 workgroups
         while ((w.n + rpw * 4 - 1) / (rpw * 4) > 65535u && rpw + br <= 64) rpw += br;
-        if (rpw <= 64 && gemv_rows_has_shape((int)c.nc, br) && (!argmax || gemv_rows_has_argmax((int)c.nc, br))) {
+        if (rpw <= 64 && gemv_rows_has_shape((int)c.nc, br) && (!argmax || gemv_rows_has_argmax((int)c.nc, br)) &&
+            (!two_rows || (gemv_rows_has_batch((int)w.bits, (int)w.group, (int)c.nc, br, c.mt) && lds_bytes(w, c.mt, 0) <= kLdsBudget))) {
             c.rows = true;
             c.nct = (int)c.nc;
             c.br = br;
             c.r = 1;
             c.waves = gemv_rows_waves(c.nct);
             c.rows_per_wave = rpw;
-            c.lds = lds_bytes(w, 1, c.xa);
+            c.lds = lds_bytes(w, c.mt, c.xa);
             const uint32_t rows_per_wg = rpw * (uint32_t)c.waves;
             c.grid = (w.n + rows_per_wg - 1) / rows_per_wg;
             if (c.grid == 0) c.grid = 1;
             return c;
         }
     }
+    c.mt = m <= 1 ? 1 : m <= 2 ? 2 : 4;                      // the general kernel's batches
     const uint64_t weight_bytes = (uint64_t)w.n * (w.k / w.group) * (4 + w.group * w.bits / 8);
     const bool big = weight_bytes >= (24ull << 20);
     if (c.mt == 1) {

@@ -99,7 +99,8 @@ void plan_small_m(const mi355q_weight* w, uint32_t m, int x_dtype, uint32_t x_st
         s->block[0] = g.block;
         s->lds_bytes = g.lds_bytes;
         s->rows_per_workgroup = 16;
-    } else if (!forced && mfma_planes_pays(v.bits, x_dtype, m) && gemv_mfma_planes_eligible(v, x_dtype, m > most ? most : m, x_stride)) {
+    } else if (!forced && mfma_planes_pays(v.bits, x_dtype, m) && gemv_mfma_planes_eligible(v, x_dtype, m > most ? most : m, x_stride) &&
+               !(gemv_rows_batch_pays(1, &v, x_dtype, m) && gemv_fast_eligible(v, x_dtype, m, x_stride))) {
         const Tile16LaunchShape g = gemv_mfma_planes_shape(w->ctx, (uint32_t)((w->n + 15) / 16), (uint32_t)w->k,
                                                            (uint32_t)w->fmt.bits, staged_rows(x_dtype, m > most ? most : m));
         std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_mfma_planes_q%u_g%u", (unsigned)w->fmt.bits,
@@ -162,6 +163,15 @@ void plan_shared_launch_shape(const mi355q_weight* const* ws, uint32_t count, ui
                     gemv_mfma_planes_k_parts(ws[0]->ctx, v, staged_rows(x_dtype, m)) == 1 &&
                     v.sb_dtype == all.sb_dtype && v.code_stride == all.code_stride && v.group == all.group && v.bits == all.bits;
         tiles += (v.n + 15) / 16;
+    }
+    if (on_planes && m <= 4) {                               // small matrices at three or four rows: the dot-product rows kernel
+        WView views[3];
+        bool fast = count <= 3;
+        for (uint32_t i = 0; i < count && fast; i++) {
+            views[i] = ws[i]->view();
+            fast = gemv_fast_eligible(views[i], x_dtype, m, x_stride) && views[i].sb_dtype == all.sb_dtype;
+        }
+        if (fast && gemv_rows_batch_pays(count, views, x_dtype, m)) on_planes = false;
     }
     if (on_planes) {
         const Tile16LaunchShape g = gemv_mfma_planes_shape(ws[0]->ctx, tiles, all.k, all.bits, staged_rows(x_dtype, m));

@@ -254,6 +254,33 @@ def test_config1_llama3_8b_layer_shapes(pkg, ctx, name):
     _seeded_gemv_check(pkg, ctx, 200 + n % 97, n, k, 4, 64, [1, 2, 4, 8])
 
 
+@pytest.mark.parametrize("n,k,group", [(14336, 4096, 64), (4100, 4096, 128), (517, 14336, 64), (16387, 2048, 64), (3000, 2560, 64)])
+def test_activation_rows_share_the_unpacked_codes(pkg, ctx, n, k, group):
+    """M = 2 on 4-bit planes (and M = 3, 4 on small matrices with rows of two K-steps) runs on the static-structure
+    kernel with every activation row on each unpacked code pair: rows of one, two and seven K-steps, row counts off
+    every workgroup boundary, both group sizes; against the oracle and against the same rows taken one at a time."""
+    words, s, z, wq = seeded_case(270 + n % 89, n, k, 4, group)
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, group)
+    w = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, pkg.LAYOUT_PLANES)
+    small = 2048 < k <= 4096 and n * (k // group) * (4 + group // 2) < (12 << 20)
+    for m in ((2, 3, 4) if small else (2,)):
+        step = w.plan_decode_step(m)
+        if n >= 3000:
+            assert step.device_kernel == f"gemv_rows_q4_g{group}", (m, step.device_kernel)
+        x = act_rounded(kat.seeded_activations(271 + m, m, k), pkg.BF16, pkg)
+        want = oracle.gemm_f64(wq, x)
+        y32 = run_gemv(ctx, pkg, w, x, pkg.BF16, pkg.F32)
+        assert_within_tolerance(y32, want, f"M={m} {k}->{n}")
+        one = np.concatenate([run_gemv(ctx, pkg, w, x[i:i + 1], pkg.BF16, pkg.F32) for i in range(m)])
+        assert np.max(np.abs(one - y32)) <= 1e-5 * max(1.0, float(np.max(np.abs(y32)))), "rows together vs one at a time"
+        for yd in (pkg.BF16, pkg.F16):
+            y16 = run_gemv(ctx, pkg, w, x, pkg.BF16, yd)
+            want16 = (oracle.bf16_to_f32(oracle.bf16_from_f32(y32)).reshape(y32.shape) if yd == pkg.BF16
+                      else y32.astype(np.float16).astype(np.float32))
+            assert np.array_equal(y16, want16)
+    w.destroy()
+
+
 def test_config1_odd_batch_sizes(pkg, ctx):
     _seeded_gemv_check(pkg, ctx, 260, 1024, 4096, 4, 64, [3, 5, 6, 7])
 
