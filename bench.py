@@ -720,6 +720,14 @@ def main():
         probe |= pkg.FLAG_PROBE_TILED                     # the tiled kernel (weights dequantised into LDS) beside it
         ms_t, ghz_t = gemm_figure(xg)
         probe &= ~pkg.FLAG_PROBE_TILED
+        # the two-dispatch route (dequantise, then the platform's dense GEMM) on the same problem, where the library is there
+        ms_l = None
+        try:
+            ctx.qgemm(wg, xg, pkg.BF16, yg, pkg.BF16, m, 0, 0, pkg.FLAG_FORCE_TWO_STEP, stream)
+            ctx.synchronize(stream)
+            ms_l, _, _ = steady_region(ctx, lambda i: ctx.qgemm(wg, xg, pkg.BF16, yg, pkg.BF16, m, 0, 0, pkg.FLAG_FORCE_TWO_STEP, stream), 10, stream)
+        except pkg.MI355QError as e:
+            log(f"  two-dispatch route not available: {e}")
         xc = ctx.upload(np.full((m, 4096), 0x3F80, np.uint16))
         ms_c, ghz_c = gemm_figure(xc)
         xc.free(); xg.free(); yg.free()
@@ -731,6 +739,9 @@ def main():
                    "tiled_kernel_m2048_gate": {"us": round(ms_t * 1e3, 1), "TFLOPs": round(flops / (ms_t * 1e-3) / 1e12, 1),
                                                "shader_clock_GHz": round(ghz_t, 3),
                                                "kernel": wg.plan_prefill_steps(m, 4096, flags=pkg.FLAG_FORCE_MFMA | pkg.FLAG_PROBE_TILED)[0].device_kernel},
+                   "two_dispatch_route_m2048_gate": (None if ms_l is None else
+                                                     {"us": round(ms_l * 1e3, 1), "TFLOPs": round(flops / (ms_l * 1e-3) / 1e12, 1),
+                                                      "kernel": "+".join(st.device_kernel for st in wg.plan_prefill_steps(m, 4096, flags=pkg.FLAG_FORCE_TWO_STEP))}),
                    "aside_constant_activations_fused_kernel": {"us": round(ms_c * 1e3, 1), "TFLOPs": round(flops / (ms_c * 1e-3) / 1e12, 1),
                                                                "shader_clock_GHz": round(ghz_c, 3)}}
         log(f"  fused kernel M={m} gate: {prefill['fused_kernel_m2048_gate']}; constant activations (aside): "
