@@ -555,6 +555,8 @@ mi355q_status mi355q_qgemv(mi355q_context* ctx, void* stream, const mi355q_weigh
                            mi355q_dtype x_dtype, void* y_dev, mi355q_dtype y_dtype, uint32_t m,
                            uint32_t x_row_stride, uint32_t y_row_stride, uint32_t flags) {
     if (mi355q_status s = check_launch(ctx, w)) return s;
+    ScratchGuard guard(ctx, (hipStream_t)stream);
+    if (guard.status) return guard.status;
     return dispatch_linear(ctx, (hipStream_t)stream, w, x_dev, x_dtype, y_dev, y_dtype, m, x_row_stride,
                            y_row_stride, flags, true);
 }
@@ -563,6 +565,8 @@ mi355q_status mi355q_qgemm(mi355q_context* ctx, void* stream, const mi355q_weigh
                            mi355q_dtype x_dtype, void* y_dev, mi355q_dtype y_dtype, uint32_t m,
                            uint32_t x_row_stride, uint32_t y_row_stride, uint32_t flags) {
     if (mi355q_status s = check_launch(ctx, w)) return s;
+    ScratchGuard guard(ctx, (hipStream_t)stream);
+    if (guard.status) return guard.status;
     return dispatch_linear(ctx, (hipStream_t)stream, w, x_dev, x_dtype, y_dev, y_dtype, m, x_row_stride,
                            y_row_stride, flags, false);
 }
@@ -573,6 +577,8 @@ mi355q_status mi355q_batched_qgemm(mi355q_context* ctx, void* stream, uint32_t c
                                    uint32_t flags) {
     if (!ctx) return fail(MI355Q_ERR_NULL_HANDLE, "context is null");
     MI355Q_HIP(hipSetDevice(ctx->device));
+    ScratchGuard guard(ctx, (hipStream_t)stream);
+    if (guard.status) return guard.status;
     return dispatch_batched(ctx, (hipStream_t)stream, count, weights, x_dev, x_dtype, y_devs, y_dtype, m,
                             x_row_stride, flags);
 }
@@ -600,6 +606,8 @@ mi355q_status mi355q_gemm_bf16(mi355q_context* ctx, void* stream, const void* a_
     if (c_row_stride == 0) c_row_stride = n;
     if (a_row_stride < k || c_row_stride < n) return fail(MI355Q_ERR_SHAPE, "row stride smaller than the row");
     MI355Q_HIP(hipSetDevice(ctx->device));
+    ScratchGuard guard(ctx, (hipStream_t)stream);
+    if (guard.status) return guard.status;
     // long products go to the platform's GEMM library (the reference hands them to matmul2d), the rest to this
     // library's own matrix-core kernel
     if (a_dtype == MI355Q_BF16 && m >= kDenseLibraryMinRows && k % 8 == 0 && a_row_stride % 8 == 0 &&
@@ -645,6 +653,9 @@ mi355q_status mi355q_argmax(mi355q_context* ctx, void* stream, const void* logit
     if (!dtype_ok(dtype)) return fail(MI355Q_ERR_INVALID_ARGUMENT, "bad dtype tag");
     if (vocabulary_size == 0) return fail(MI355Q_ERR_SHAPE, "argmax over an empty vector");
     MI355Q_HIP(hipSetDevice(ctx->device));
+    ScratchGuard guard(ctx, (hipStream_t)stream);
+    if (guard.status) return guard.status;
+    ctx->scratch_touched = true;                              // the keys of the stand-alone arg-max
     return launch_argmax((hipStream_t)stream, logits_dev, dtype, vocabulary_size, token_out_dev,
                          ctx->argmax_partials + kArgmaxPartialCapacity);
 }
@@ -653,6 +664,9 @@ mi355q_status mi355q_lmhead_argmax(mi355q_context* ctx, void* stream, const mi35
                                    mi355q_dtype x_dtype, float* logits_f32_dev, int32_t* token_out_dev,
                                    uint32_t flags) {
     if (mi355q_status s = check_launch(ctx, w)) return s;
+    ScratchGuard guard(ctx, (hipStream_t)stream);
+    if (guard.status) return guard.status;
+    ctx->scratch_touched = true;                              // one key per workgroup of the head
     return dispatch_output_head(ctx, (hipStream_t)stream, w, x_dev, x_dtype, logits_f32_dev, token_out_dev, flags,
                                 HeadKeys{ctx->argmax_partials, kArgmaxPartialCapacity});
 }
@@ -741,6 +755,8 @@ extern "C" mi355q_status mi355q_gated_qgemm(mi355q_context* ctx, void* stream, c
                                             uint32_t y_row_stride, mi355q_gated_activation activation, uint32_t flags) {
     if (mi355q_status st = check_launch(ctx, w_gate)) return st;
     if (mi355q_status st = check_launch(ctx, w_up)) return st;
+    ScratchGuard guard(ctx, (hipStream_t)stream);
+    if (guard.status) return guard.status;
     return dispatch_gated(ctx, (hipStream_t)stream, w_gate, w_up, x_dev, x_dtype, y_dev, y_dtype, m, x_row_stride, y_row_stride,
                           activation, flags);
 }

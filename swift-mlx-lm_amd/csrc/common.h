@@ -80,6 +80,11 @@ struct mi355q_context {
     mi355q::DenseLibrary* dense_library;
     bool dense_library_failed;
     bool dense_library_forbidden;      // mi355q_context_set_library_use(ctx, 0): in-tree kernels only
+    // One stream per context at a time: the stream whose launches last used the scratch above, an event recorded
+    // behind them, and whether the entry point now running has touched the scratch (see ScratchGuard)
+    hipStream_t scratch_stream;
+    hipEvent_t scratch_event;
+    bool scratch_pending, scratch_touched;
 };
 constexpr int kRetiredWorkspaces = 96;
 
@@ -288,6 +293,20 @@ struct GemmLaunchShape {
     uint32_t bm, bn, stages, grid, block, lds_bytes, splits, kt_per_split;
 };
 GemmLaunchShape gemm_mfma_shape(const mi355q_context* ctx, uint32_t m, uint32_t n, uint32_t k);
+// Every entry point that enqueues work opens one of these first.  The context's scratch (partial results, dense
+// copies, split rows, gate / up sums, arg-max keys) is shared by its launches, so they must be ordered: when the scratch
+// was last used on ANOTHER stream and an event recorded behind that work has not completed, the entry point fails
+// with MI355Q_ERR_INVALID_ARGUMENT instead of racing (the null stream is ordered with every blocking stream and is let
+// through).  On the way out, if the call touched the scratch, the event is recorded again (not while capturing).
+struct ScratchGuard {
+    mi355q_context* ctx;
+    hipStream_t stream;
+    mi355q_status status;
+    ScratchGuard(mi355q_context* c, hipStream_t s);
+    ~ScratchGuard();
+    ScratchGuard(const ScratchGuard&) = delete;
+    ScratchGuard& operator=(const ScratchGuard&) = delete;
+};
 // Grows the context's scratch buffer for fp32 partial results; nothing is released before the context goes.
 mi355q_status ensure_workspace(mi355q_context* ctx, size_t bytes);
 mi355q_status ensure_split_buffer(mi355q_context* ctx, size_t bytes);

@@ -39,6 +39,8 @@ struct mi355q_plan {
     std::vector<PlanStep> steps;
     hipGraph_t graph;
     hipGraphExec_t graph_exec;
+    bool has_output_head;       // a step that keeps arg-max keys in the context's scratch
+    bool uses_scratch;          // the captured graph's launches use the context's scratch
 };
 
 namespace {
@@ -79,6 +81,8 @@ mi355q_status mi355q_plan_create(mi355q_context* ctx, mi355q_plan** out) {
     p->ctx = ctx;
     p->graph = nullptr;
     p->graph_exec = nullptr;
+    p->has_output_head = false;
+    p->uses_scratch = false;
     *out = p;
     return MI355Q_OK;
 }
@@ -237,6 +241,7 @@ mi355q_status mi355q_plan_add_output_head(mi355q_plan* plan, const mi355q_weight
     if (plan->graph_exec) return fail(MI355Q_ERR_INVALID_ARGUMENT, "plan is frozen: its graph has been built");
     PlanStep st{};
     st.kind = kOutputHead;
+    plan->has_output_head = true;
     st.w = w; st.x = x_dev; st.y = logits_f32_dev; st.token = token_out_dev;
     st.x_dtype = x_dtype; st.y_dtype = MI355Q_F32;
     st.m = 1; st.xs = (uint32_t)w->k; st.ys = (uint32_t)w->n;
@@ -268,7 +273,11 @@ mi355q_status mi355q_plan_step_at(const mi355q_plan* plan, int32_t index, mi355q
 mi355q_status mi355q_plan_encode(mi355q_plan* plan, void* stream, uint32_t first, uint32_t count) {
     if (!plan) return fail(MI355Q_ERR_NULL_HANDLE, "plan is null");
     MI355Q_HIP(hipSetDevice(plan->ctx->device));
-    return encode_range(plan, (hipStream_t)stream, first, count);
+    ScratchGuard guard(plan->ctx, (hipStream_t)stream);
+    if (guard.status) return guard.status;
+    const mi355q_status st = encode_range(plan, (hipStream_t)stream, first, count);
+    if (plan->has_output_head) plan->ctx->scratch_touched = true;          // one key per workgroup of the head
+    return st;
 }
 
 mi355q_status mi355q_plan_graph_build(mi355q_plan* plan, void* stream) {
@@ -277,8 +286,12 @@ mi355q_status mi355q_plan_graph_build(mi355q_plan* plan, void* stream) {
     if (plan->graph_exec) return MI355Q_OK;
     MI355Q_HIP(hipSetDevice(plan->ctx->device));
     hipStream_t s = (hipStream_t)stream;
+    ScratchGuard guard(plan->ctx, s);
+    if (guard.status) return guard.status;
     // One eager pass first: kernel attributes are set outside the capture.
     if (mi355q_status rc = encode_range(plan, s, 0, 0)) return rc;
+    if (plan->has_output_head) plan->ctx->scratch_touched = true;
+    plan->uses_scratch = plan->ctx->scratch_touched;
     MI355Q_HIP(hipStreamSynchronize(s));
     MI355Q_HIP(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
     mi355q_status rc = encode_range(plan, s, 0, 0);
@@ -301,7 +314,10 @@ mi355q_status mi355q_plan_graph_build(mi355q_plan* plan, void* stream) {
 mi355q_status mi355q_plan_graph_launch(mi355q_plan* plan, void* stream) {
     if (!plan) return fail(MI355Q_ERR_NULL_HANDLE, "plan is null");
     if (!plan->graph_exec) return fail(MI355Q_ERR_INVALID_ARGUMENT, "graph has not been built");
+    ScratchGuard guard(plan->ctx, (hipStream_t)stream);
+    if (guard.status) return guard.status;
     MI355Q_HIP(hipGraphLaunch(plan->graph_exec, (hipStream_t)stream));
+    plan->ctx->scratch_touched = plan->uses_scratch;           // the captured launches keep the scratch addresses
     return MI355Q_OK;
 }
 

@@ -61,15 +61,49 @@ mi355q_status grow_scratch(mi355q_context* ctx, void*& buffer, size_t& have, siz
 }
 }  // namespace
 
+ScratchGuard::ScratchGuard(mi355q_context* c, hipStream_t s) : ctx(c), stream(s), status(MI355Q_OK) {
+    if (!ctx) return;
+    ctx->scratch_touched = false;
+    if (!ctx->scratch_pending || ctx->scratch_stream == s || !s || !ctx->scratch_stream) return;
+    const hipError_t q = hipEventQuery(ctx->scratch_event);
+    if (q == hipErrorNotReady) {
+        (void)hipGetLastError();
+        status = fail(MI355Q_ERR_INVALID_ARGUMENT,
+                      "the context's scratch is still in use by work on another stream: one stream per context at a time "
+                      "(synchronise the first stream, or give each stream a context of its own)");
+        return;
+    }
+    (void)hipGetLastError();
+    ctx->scratch_pending = false;
+}
+
+ScratchGuard::~ScratchGuard() {
+    if (!ctx || status != MI355Q_OK || !ctx->scratch_touched || !ctx->scratch_event) return;
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (stream && (hipStreamIsCapturing(stream, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone)) {
+        (void)hipGetLastError();
+        return;
+    }
+    if (hipEventRecord(ctx->scratch_event, stream) == hipSuccess) {
+        ctx->scratch_stream = stream;
+        ctx->scratch_pending = true;
+    } else {
+        (void)hipGetLastError();
+    }
+}
+
 mi355q_status ensure_workspace(mi355q_context* ctx, size_t bytes) {
+    ctx->scratch_touched = true;
     return grow_scratch(ctx, ctx->workspace, ctx->workspace_bytes, bytes, (size_t)1 << 22);
 }
 
 mi355q_status ensure_split_buffer(mi355q_context* ctx, size_t bytes) {
+    ctx->scratch_touched = true;
     return grow_scratch(ctx, ctx->split_buffer, ctx->split_bytes, bytes, (size_t)1 << 20);
 }
 
 mi355q_status ensure_gated_buffer(mi355q_context* ctx, size_t bytes) {
+    ctx->scratch_touched = true;
     return grow_scratch(ctx, ctx->gated_buffer, ctx->gated_bytes, bytes, (size_t)1 << 20);
 }
 
@@ -307,7 +341,9 @@ mi355q_status mi355q_context_create(int device_index, mi355q_context** out) {
     e = hipMalloc((void**)&ctx->argmax_scratch, 256);
     if (e == hipSuccess) e = hipMemset(ctx->argmax_scratch, 0, 256);
     if (e == hipSuccess) e = hipMalloc((void**)&ctx->argmax_partials, (size_t)(kArgmaxPartialCapacity + kArgmaxStandaloneKeys) * 8);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&ctx->scratch_event, hipEventDisableTiming);
     if (e != hipSuccess) {
+        if (ctx->scratch_event) (void)hipEventDestroy(ctx->scratch_event);
         if (ctx->argmax_scratch) (void)hipFree(ctx->argmax_scratch);
         if (ctx->argmax_partials) (void)hipFree(ctx->argmax_partials);
         delete ctx;
@@ -338,6 +374,7 @@ mi355q_status mi355q_context_destroy(mi355q_context* ctx) {
     (void)hipSetDevice(ctx->device);
     (void)hipDeviceSynchronize();
     mi355q::dense_library_release(ctx);
+    if (ctx->scratch_event) (void)hipEventDestroy(ctx->scratch_event);
     if (ctx->argmax_scratch) (void)hipFree(ctx->argmax_scratch);
     if (ctx->argmax_partials) (void)hipFree(ctx->argmax_partials);
     if (ctx->workspace) (void)hipFree(ctx->workspace);

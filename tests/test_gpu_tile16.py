@@ -322,7 +322,7 @@ def test_tile16_prefill_runs_on_the_matrix_cores(pkg, ctx):
         say(f"tile16 prefill {k}->{n} M={m}")
         two_step_from = 2048 if k > n else 768 if n >= 8192 else 512       # rows from which dequantise once + dense GEMM
         got = _run(ctx, pkg, wt, x, pkg.F32, use_qgemm=True, flags=0 if 32 < m < two_step_from else pkg.FLAG_FORCE_MFMA)
-        same = _run(ctx, pkg, wp, x, pkg.F32, use_qgemm=True, flags=pkg.FLAG_FORCE_MFMA)
+        same = _run(ctx, pkg, wp, x, pkg.F32, use_qgemm=True, flags=pkg.FLAG_FORCE_MFMA | pkg.FLAG_PROBE_TILED)   # the same tiled kernel (long prompts on planes would take the wide-tile one)
         assert np.array_equal(got, same), f"{k}->{n} M={m}: records and planes disagree"
         if m * n * k <= 2 ** 28:
             wb = oracle.bf16_to_f32(oracle.bf16_from_f32(wq)).reshape(wq.shape)

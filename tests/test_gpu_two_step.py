@@ -316,3 +316,34 @@ def test_library_route_with_padded_result_rows_and_long_k(pkg, ctx, x_dtype_name
             cd.free()
         dense.free()
     xd.free(); w.destroy()
+
+
+def test_one_stream_per_context_is_enforced(pkg):
+    """The context's scratch is shared by its launches.  A launch that uses it on a second stream while work that used
+    it on a first stream is still running is refused (MI355Q_ERR_INVALID_ARGUMENT) instead of racing; once the first
+    stream has finished the second is served, and launches that keep to one stream never notice."""
+    c = pkg.Context(0)
+    try:
+        fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+        n, k, m = 4096, 4096, 2048
+        words, s, z = oracle.quantize_affine(kat.seeded_weights(3900, 64, k), 4, 64, oracle.BF16)
+        words = np.tile(words, (n // 64, 1)); s = np.tile(s.reshape(64, -1), (n // 64, 1)); z = np.tile(z.reshape(64, -1), (n // 64, 1))
+        w = c.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, pkg.LAYOUT_PLANES)
+        x = c.upload(oracle.bf16_from_f32(kat.seeded_activations(3901, m, k)))
+        y1 = c.alloc(m * n * 2); y2 = c.alloc(m * n * 2)
+        a, b = c.stream_create(), c.stream_create()
+        two = pkg.FLAG_FORCE_TWO_STEP                      # the dense copy of the matrix lives in the context's scratch
+        c.qgemm(w, x, pkg.BF16, y1, pkg.BF16, m, 0, 0, two, a); c.synchronize(a)      # (first call: timing, synchronous)
+        for _ in range(20):
+            c.qgemm(w, x, pkg.BF16, y1, pkg.BF16, m, 0, 0, two, a)                     # a few milliseconds of work on a
+        with pytest.raises(pkg.MI355QError) as err:
+            c.qgemm(w, x, pkg.BF16, y2, pkg.BF16, m, 0, 0, two, b)
+        assert "another stream" in str(err.value)
+        c.qgemm(w, x, pkg.BF16, y1, pkg.BF16, m, 0, 0, two, a)                         # the same stream goes on
+        c.synchronize(a)
+        c.qgemm(w, x, pkg.BF16, y2, pkg.BF16, m, 0, 0, two, b); c.synchronize(b)      # the first stream is done: served
+        assert np.array_equal(y1.download(np.uint16, (m, n)), y2.download(np.uint16, (m, n)))
+        c.stream_destroy(a); c.stream_destroy(b)
+        x.free(); y1.free(); y2.free(); w.destroy()
+    finally:
+        c.close()
