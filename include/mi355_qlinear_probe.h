@@ -44,6 +44,16 @@ MI355Q_API mi355q_status mi355q_context_scratch_bytes(mi355q_context* ctx, uint6
  * problem (fewer than sixteen K-tiles a part, N not a multiple of four) are ignored for it. */
 MI355Q_API void mi355q_probe_wide_shape(uint32_t tile_rows, uint32_t k_parts);
 
+/* The route table on a synthetic weight (no device needed): what the launcher would run for the problem
+ * ("route" or "route/kernel": split-rows, two-step, stream, small-batch/<kernel>, fused/wide, fused/tiled, error:...)
+ * and the device kernels the plan records name for it, joined by '+'.  Launcher and planner read the same table; the
+ * CPU test suite walks it.  layout: mi355q_layout; sb_dtype: scale type of planes; library_available: whether the
+ * dense library counts as usable; decode_entry: mi355q_qgemv / plan_decode_step, else mi355q_qgemm / plan_prefill_steps. */
+MI355Q_API mi355q_status mi355q_probe_route(uint8_t scheme_identifier, uint32_t layout, uint32_t sb_dtype, uint64_t n_rows,
+                                            uint64_t k, mi355q_dtype x_dtype, uint32_t m, uint32_t x_row_stride,
+                                            uint32_t flags, int decode_entry, int library_available, char* launcher_out,
+                                            char* planner_out, size_t cap);
+
 #ifdef __cplusplus
 }
 #endif

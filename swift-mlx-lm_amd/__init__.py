@@ -37,6 +37,16 @@ FAMILY_NAMES = {0: "generic", 1: "largeDense", 2: "input2048SquareDense", 3: "in
                 4: "input20488192Dense", 5: "input2048ExpandedDense", 6: "input8192Tiled", 7: "vocabDense"}
 
 
+def probe_route(fmt, layout, n, k, x_dtype, m, flags=0, decode_entry=False, library_available=True, sb_dtype=None,
+                x_row_stride=0):
+    """The route table on a synthetic weight (no device needed): (what the launcher would run, what the plan names)."""
+    a = C.create_string_buffer(128)
+    b = C.create_string_buffer(128)
+    _check(library().mi355q_probe_route(fmt.scheme_identifier, layout, BF16 if sb_dtype is None else sb_dtype, n, k, x_dtype, m,
+                                        x_row_stride, flags, int(decode_entry), int(library_available), a, b, 128))
+    return a.value.decode(), b.value.decode()
+
+
 class MI355QError(RuntimeError):
     def __init__(self, status: int, message: str):
         super().__init__(f"[{STATUS_NAMES.get(status, status)}] {message}")
@@ -183,6 +193,7 @@ def library() -> C.CDLL:
         "mi355q_clock_probe_read": (i32, [vp, P(u64), P(u64)]),
         "mi355q_context_scratch_bytes": (i32, [vp, P(u64)]),
         "mi355q_probe_wide_shape": (None, [u32, u32]),
+        "mi355q_probe_route": (i32, [u8, u32, u32, u64, u64, C.c_int, u32, u32, u32, C.c_int, C.c_int, C.c_char_p, C.c_char_p, sz]),
         "mi355q_kv_scheme_is_supported": (i32, [u8]),
         "mi355q_kv_bytes_per_head_slot": (u32, [u8, u32]),
         "mi355q_kv_cache_write": (i32, [vp, vp, P(_KvLayout), vp, vp, C.c_int, u32, u32, u32]),

@@ -42,42 +42,35 @@ mi355q_status run_small_m(mi355q_context* ctx, hipStream_t s, const mi355q_weigh
                           void* y, int y_dtype, uint32_t m, uint32_t xs, uint32_t ys, uint32_t flags) {
     const WView v = w->view();
     const size_t xsz = x_dtype == MI355Q_F32 ? 4 : 2, ysz = y_dtype == MI355Q_F32 ? 4 : 2;
-    const bool generic = flags & MI355Q_FLAG_FORCE_GENERIC;
-    // rows per launch: 16 on the tile layout (fewer when K is so long that 16 staged rows overflow LDS), else 8
-    uint32_t step = generic ? 8 : small_batch_rows(v, x_dtype, xs);
-    if (!generic && v.layout == MI355Q_LAYOUT_TILE16) {
-        step = 16;
-        while (step > 1 && !gemv_tile16_eligible(v, x_dtype, step, xs)) step >>= 1;
-        // no row count the tile kernel takes (other activation type, stride): the per-code kernel takes all M at once
-        if (!gemv_tile16_eligible(v, x_dtype, step, xs)) step = m < 65535u ? m : 65535u;
-    } else if (generic || !(gemv_fast_eligible(v, x_dtype, 1, xs) || gemv_staf_eligible(v, x_dtype, 1, xs))) {
-        step = m < 65535u ? m : 65535u;   // the per-code kernel has no limit of 8 rows
-    }
+    const uint32_t step = small_batch_step(v, x_dtype, m, xs, flags);
     for (uint32_t m0 = 0; m0 < m; m0 += step) {
         const uint32_t mm = m - m0 < step ? m - m0 : step;
         const void* xp = (const char*)x + (size_t)m0 * xs * xsz;
         void* yp = (char*)y + (size_t)m0 * ys * ysz;
         mi355q_status st;
-        if (!generic && gemv_tile16_eligible(v, x_dtype, mm, xs) && (uintptr_t)xp % 16 == 0) {
-            void* yv[1] = {yp};
-            const uint32_t strides[1] = {ys};
+        void* yv[1] = {yp};
+        const uint32_t strides[1] = {ys};
+        switch (small_kernel(v, x_dtype, mm, xs, flags, (uintptr_t)xp % 16 == 0)) {
+        case SmallKernel::kTile16:
             st = launch_gemv_tile16_multi(s, ctx, 1, &v, xp, x_dtype, yv, strides, y_dtype, mm, xs, nullptr, nullptr, HeadKeys{});
-        } else if (!generic && mfma_planes_pays(v.bits, x_dtype, mm) && gemv_mfma_planes_eligible(v, x_dtype, mm, xs) &&
-                   !(gemv_rows_batch_pays(1, &v, x_dtype, mm) && gemv_fast_eligible(v, x_dtype, mm, xs)) && (uintptr_t)xp % 16 == 0) {
-            void* yv[1] = {yp};
-            const uint32_t strides[1] = {ys};
+            break;
+        case SmallKernel::kMfmaPlanes:
             st = launch_gemv_mfma_planes_multi(s, ctx, 1, &v, xp, x_dtype, yv, strides, y_dtype, mm, xs);
-        } else if (!generic && gemv_fast_eligible(v, x_dtype, mm > 8 ? 8 : mm, xs) && (uintptr_t)xp % 16 == 0) {
+            break;
+        case SmallKernel::kDotPlanes:
             // the dot-product kernels take eight rows a launch
             st = MI355Q_OK;
             for (uint32_t r0 = 0; r0 < mm && st == MI355Q_OK; r0 += 8)
                 st = launch_gemv_fast(s, ctx, v, (const char*)xp + (size_t)r0 * xs * xsz, x_dtype,
                                       (char*)yp + (size_t)r0 * ys * ysz, y_dtype, mm - r0 < 8 ? mm - r0 : 8, xs, ys, nullptr,
                                       nullptr, HeadKeys{});
-        } else if (!generic && gemv_staf_eligible(v, x_dtype, mm, xs) && (uintptr_t)xp % 16 == 0) {
+            break;
+        case SmallKernel::kStafInPlace:
             st = launch_gemv_staf(s, ctx, v, xp, x_dtype, yp, y_dtype, mm, xs, ys);
-        } else {
+            break;
+        default:
             st = launch_gemv_generic(s, v, xp, x_dtype, yp, y_dtype, mm, xs, ys);
+            break;
         }
         if (st != MI355Q_OK) return st;
     }
@@ -117,7 +110,8 @@ bool split_rows_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_strid
     (void)x_stride;
     const uint32_t parts = split_rows_parts(x_dtype);
     if (!parts || (flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_TWO_STEP))) return false;
-    return split_rows_small_batch(w, parts, m) || split_rows_take_stream(w, x_dtype, m);
+    // (FORCE_SMALL_M keeps the rows off the streamed-weight kernel: then only the decode kernels count)
+    return split_rows_small_batch(w, parts, m) || (!(flags & MI355Q_FLAG_FORCE_SMALL_M) && split_rows_take_stream(w, x_dtype, m));
 }
 
 // The split rows fit the small-batch launches of a bf16 decode kernel.
@@ -145,64 +139,43 @@ mi355q_status dispatch_linear(mi355q_context* ctx, hipStream_t s, const mi355q_w
                               void* y, int y_dtype, uint32_t m, uint32_t xs, uint32_t ys, uint32_t flags,
                               bool small_m_only) {
     if (mi355q_status st = check_io(w, x, x_dtype, y, y_dtype, m, xs, ys)) return st;
-    if (small_m_only) {
-        if (m > 8) return fail(MI355Q_ERR_INVALID_ARGUMENT, "qgemv takes 1 <= M <= 8 (got %u); use qgemm", m);
-        // no decode kernel reads this layout with this activation type (fp32 anywhere, f16 on TILE16 records, block
-        // shapes the in-place kernel skips): dequantise once + the dense library product beats the per-code kernel
-        // from the second row (4096 -> 14336, fp32 activations: per-code kernel 123 us at M = 1, 195 at M = 2, 700 at
-        // M = 8; the route with fp32 weights 100-135 us whatever M)
-        const WView v = w->view();
-        if (split_rows_chosen(v, x_dtype, m, xs, flags)) return run_split_rows(ctx, s, w, x, x_dtype, y, y_dtype, m, xs, ys, flags);
-        if (gemm_two_step_chosen(v, x_dtype, m, xs, flags) && (uintptr_t)x % 16 == 0 &&
-            gemm_two_step_serves(ctx, v, x_dtype, y_dtype, m, xs, ys)) {
-            // (a library result that fails its check makes the problem unusable: the routes below serve the call)
-            const mi355q_status st = launch_qgemm_two_step(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
-            if (st != MI355Q_ERR_KERNEL_NOT_FOUND) return st;
-        }
-        if (!(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_SMALL_M)) && gemm_stream_chosen(v, x_dtype, m, xs) &&
-            gemm_stream_unrounded(v, m) && (uintptr_t)x % 16 == 0)
-            return launch_qgemm_stream(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
-        return run_small_m(ctx, s, w, x, x_dtype, y, y_dtype, m, xs, ys, flags);
-    }
-    const uint32_t forced = flags & (MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_TWO_STEP | MI355Q_FLAG_FORCE_SMALL_M |
-                                     MI355Q_FLAG_FORCE_GENERIC);
-    if ((forced & (MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_TWO_STEP)) && (forced & (forced - 1)))
-        return fail(MI355Q_ERR_INVALID_ARGUMENT, "contradictory kernel selection flags");
     const WView v = w->view();
-    if (flags & MI355Q_FLAG_FORCE_STREAM) {
-        if (forced) return fail(MI355Q_ERR_INVALID_ARGUMENT, "contradictory kernel selection flags");
-        return launch_qgemm_stream(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
-    }
-    if (flags & MI355Q_FLAG_FORCE_TWO_STEP) {
-        if (!gemm_two_step_eligible(v, x_dtype, m, xs) || (uintptr_t)x % 16)
-            return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the two-dispatch route takes 16-byte aligned activations, K and the row stride multiples of 8");
-        return launch_qgemm_two_step(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
-    }
-    if (split_rows_chosen(v, x_dtype, m, xs, flags))
-        return run_split_rows(ctx, s, w, x, x_dtype, y, y_dtype, m, xs, ys, flags);
-    // dequantise once, then the dense library GEMM: long prompts, and every format or layout the fused kernel does
-    // not read.  When the library has no algorithm for the problem the routes below serve it.
-    if (gemm_two_step_chosen(v, x_dtype, m, xs, flags) && (uintptr_t)x % 16 == 0 &&
-        gemm_two_step_serves(ctx, v, x_dtype, y_dtype, m, xs, ys)) {
-        const mi355q_status st = launch_qgemm_two_step(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
-        if (st != MI355Q_ERR_KERNEL_NOT_FOUND) return st;
-    }
-    const bool mfma_ok = gemm_mfma_eligible(v, x_dtype, m, xs) || gemm_wide_taken(v, x_dtype, m, xs, flags);
+    RouteFacts facts{};
+    facts.decode_entry = small_m_only;
+    facts.x_aligned = (uintptr_t)x % 16 == 0;
+    // (asked only where the route is a candidate: the question opens the library)
+    facts.library_ok = facts.x_aligned && ((flags & MI355Q_FLAG_FORCE_TWO_STEP) || gemm_two_step_chosen(v, x_dtype, m, xs, flags)) &&
+                       gemm_two_step_serves(ctx, v, x_dtype, y_dtype, m, xs, ys);
     // the clock probe cell lives behind the argmax cells of the context's scratch
     unsigned long long* const probe = (flags & MI355Q_FLAG_PROBE_CLOCK) ? ctx->argmax_scratch + 16 : nullptr;
-    if (flags & MI355Q_FLAG_FORCE_MFMA) {
-        if (!mfma_ok)
+    for (int attempt = 0; attempt < 2; attempt++) {
+        switch (linear_route(v, x_dtype, m, xs, flags, facts)) {
+        case LinearRoute::kErrorRows:
+            return fail(MI355Q_ERR_INVALID_ARGUMENT, "qgemv takes 1 <= M <= 8 (got %u); use qgemm", m);
+        case LinearRoute::kErrorFlags:
+            return fail(MI355Q_ERR_INVALID_ARGUMENT, "contradictory kernel selection flags");
+        case LinearRoute::kErrorTwoStepUnavailable:
+            return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the two-dispatch route takes 16-byte aligned activations, K and the row stride multiples of 8");
+        case LinearRoute::kErrorNoFusedKernel:
             return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the MFMA GEMM does not accept this format, layout or stride");
-        return launch_qgemm_mfma(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys, probe, flags);
+        case LinearRoute::kSplitRows:
+            return run_split_rows(ctx, s, w, x, x_dtype, y, y_dtype, m, xs, ys, flags);
+        case LinearRoute::kTwoStep: {
+            const mi355q_status st = launch_qgemm_two_step(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
+            // a library result that fails its check makes the problem unusable: the table is asked again without the library
+            if (st != MI355Q_ERR_KERNEL_NOT_FOUND || (flags & MI355Q_FLAG_FORCE_TWO_STEP)) return st;
+            facts.library_ok = false;
+            continue;
+        }
+        case LinearRoute::kStream:
+            return launch_qgemm_stream(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
+        case LinearRoute::kSmallBatch:
+            return run_small_m(ctx, s, w, x, x_dtype, y, y_dtype, m, xs, ys, flags);
+        case LinearRoute::kFused:
+            return launch_qgemm_mfma(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys, probe, flags);
+        }
     }
-    // a few dozen rows on 4-bit planes: weights streamed through registers, activations alone through LDS
-    if (!forced && gemm_stream_chosen(v, x_dtype, m, xs) && (uintptr_t)x % 16 == 0)
-        return launch_qgemm_stream(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys);
-    // the decode kernels take up to 8 rows per launch, 16 on the matrix cores (and then pay for a second launch too)
-    const bool small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) ||
-                       m <= small_batch_limit(v, x_dtype, xs) || !mfma_ok;
-    if (small) return run_small_m(ctx, s, w, x, x_dtype, y, y_dtype, m, xs, ys, flags);
-    return launch_qgemm_mfma(s, ctx, v, x, x_dtype, y, y_dtype, m, xs, ys, probe, flags);
+    return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "no route serves this projection");
 }
 
 // Rows up to which the small-batch kernels, one launch after the other, beat the fused prefill kernel: two launches where

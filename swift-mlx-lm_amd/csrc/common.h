@@ -293,6 +293,34 @@ struct GemmLaunchShape {
     uint32_t bm, bn, stages, grid, block, lds_bytes, splits, kt_per_split;
 };
 GemmLaunchShape gemm_mfma_shape(const mi355q_context* ctx, uint32_t m, uint32_t n, uint32_t k);
+// ---- the one table of routes (route.cpp) --------------------------------------------------------------------
+// Which route a linear projection takes is decided in ONE place, from the weight's view, the activation type, the
+// row count, the row stride and the caller's flags; dispatch_linear (api.hip) launches what it says and the planner
+// (planner.cpp) describes what it says, so a plan record cannot name a kernel the launch would not run.
+enum class LinearRoute : int {
+    kErrorRows = 0,            // the decode entry point takes at most eight rows
+    kErrorFlags,               // contradictory selection flags
+    kErrorTwoStepUnavailable,  // FORCE_TWO_STEP on a problem the route does not take
+    kErrorNoFusedKernel,       // FORCE_MFMA on a weight no fused matrix-core kernel reads
+    kSplitRows,                // fp32 rows as three bf16 rows each on the bf16 decode kernels, partial results added
+    kTwoStep,                  // dequantise once into scratch, then the platform's dense GEMM
+    kStream,                   // weights streamed through registers into the matrix cores (a few to 96 rows)
+    kSmallBatch,               // the decode kernels, eight or sixteen rows a launch (small_kernel() names the kernel)
+    kFused                     // fused dequantise + matrix-core GEMM: the wide-tile kernel where gemm_wide_taken(), else the tiled one
+};
+struct RouteFacts {
+    bool decode_entry;         // mi355q_qgemv / plan_decode_step (at most eight rows), else mi355q_qgemm / plan_prefill_steps
+    bool library_ok;           // the dense library can serve this problem (launcher: asked; planner: not ruled out for the context)
+    bool x_aligned;            // the activation pointer is 16-byte aligned (the planner assumes it)
+};
+LinearRoute linear_route(const WView& v, int x_dtype, uint32_t m, uint32_t x_stride, uint32_t flags, const RouteFacts& facts);
+const char* linear_route_name(LinearRoute r);
+// The decode kernel a small batch (or one slice of it) runs on.
+enum class SmallKernel : int { kTile16 = 0, kMfmaPlanes, kDotPlanes, kStafInPlace, kGeneric };
+SmallKernel small_kernel(const WView& v, int x_dtype, uint32_t rows, uint32_t x_stride, uint32_t flags, bool x_aligned);
+const char* small_kernel_name(SmallKernel k);
+uint32_t small_batch_step(const WView& v, int x_dtype, uint32_t m, uint32_t x_stride, uint32_t flags);
+
 // Every entry point that enqueues work opens one of these first.  The context's scratch (partial results, dense
 // copies, split rows, gate / up sums, arg-max keys) is shared by its launches, so they must be ordered: when the scratch
 // was last used on ANOTHER stream and an event recorded behind that work has not completed, the entry point fails

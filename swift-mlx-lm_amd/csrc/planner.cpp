@@ -43,75 +43,35 @@ void fill_common(const mi355q_weight* w, uint32_t m, mi355q_step* s) {
     s->grid[1] = s->grid[2] = s->block[1] = s->block[2] = 1;
 }
 
-void plan_small_m(const mi355q_weight* w, uint32_t m, int x_dtype, uint32_t x_stride, uint32_t flags,
-                  mi355q_step* s) {
+// Launch record of the decode kernel a small batch runs on: the first slice of the rows, as run_small_m (api.hip)
+// cuts them (small_batch_step), on the kernel small_kernel() names.
+void plan_small_kernel(const mi355q_weight* w, uint32_t m, int x_dtype, uint32_t x_stride, uint32_t flags, mi355q_step* s) {
     const WView v = w->view();
-    const bool forced = flags & MI355Q_FLAG_FORCE_GENERIC;
-    if (split_rows_chosen(v, x_dtype, m, x_stride, flags) && !(flags & MI355Q_FLAG_FORCE_SMALL_M) &&
-        split_rows_take_stream(v, x_dtype, m)) {
-        // fp32 rows as three bf16 rows each on the streamed-weight kernel, then the sum of the partial results
-        const uint32_t pm = split_rows_parts(x_dtype) * m;
-        const StreamLaunchShape g = gemm_stream_shape(w->ctx, pm, (uint32_t)w->n, (uint32_t)w->k);
-        std::snprintf(s->device_kernel, sizeof s->device_kernel, "split_f32_bf16x3+qgemm_stream_q%u_g%u", (unsigned)w->fmt.bits,
-                      w->fmt.group_size);
-        s->grid[0] = g.row_blocks;
-        s->grid[1] = g.parts;
-        s->block[0] = 768;
-        s->lds_bytes = g.lds_bytes;
-        s->rows_per_workgroup = 64;
-        return;
-    }
-    if (split_rows_chosen(v, x_dtype, m, x_stride, flags)) {
-        // fp32 rows as three bf16 rows each on the bf16 decode kernel, then the sum of the partial results
-        plan_small_m(w, split_rows_parts(x_dtype) * m, MI355Q_BF16, split_rows_stride((uint32_t)w->k), flags, s);
-        char inner[sizeof s->device_kernel];
-        std::snprintf(inner, sizeof inner, "%s", s->device_kernel);
-        std::snprintf(s->device_kernel, sizeof s->device_kernel, "split_f32_bf16x3+%.30s", inner);
-        return;
-    }
-    if (!(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_SMALL_M)) && gemm_stream_chosen(v, x_dtype, m, x_stride) &&
-        gemm_stream_unrounded(v, m)) {
-        // blocks in place from three rows: the streamed-weight kernel with unrounded weights
-        const StreamLaunchShape g = gemm_stream_shape(w->ctx, m, (uint32_t)w->n, (uint32_t)w->k);
-        std::snprintf(s->device_kernel, sizeof s->device_kernel, "qgemm_stream_q%u_g%u", (unsigned)w->fmt.bits,
-                      w->fmt.group_size);
-        s->grid[0] = g.row_blocks;
-        s->grid[1] = g.parts;
-        s->block[0] = 768;
-        s->lds_bytes = g.lds_bytes;
-        s->rows_per_workgroup = 64;
-        return;
-    }
-    // rows per launch on the tile layout: 16, or fewer when K is so long that 16 staged rows overflow LDS
-    const uint32_t most = x_dtype == MI355Q_F16 ? 8 : 16;      // sixteen staged rows a launch; f16 rows are staged as two
-    uint32_t t16_rows = m > most ? most : m;
-    if (!forced && v.layout == MI355Q_LAYOUT_TILE16) {
-        uint32_t step = most;
-        while (step > 1 && !gemv_tile16_eligible(v, x_dtype, step, x_stride)) step >>= 1;
-        if (t16_rows > step) t16_rows = step;
-    }
-    if (!forced && gemv_tile16_eligible(v, x_dtype, t16_rows, x_stride)) {
-        const Tile16LaunchShape g = gemv_tile16_shape(w->ctx, (uint32_t)((w->n + 15) / 16), (uint32_t)w->k,
-                                                      staged_rows(x_dtype, t16_rows));
-        std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_tile16_q%u_g%u", (unsigned)w->fmt.bits,
-                      w->fmt.group_size);
+    const uint32_t step = small_batch_step(v, x_dtype, m, x_stride, flags);
+    const uint32_t rows = m < step ? m : step;
+    switch (small_kernel(v, x_dtype, rows, x_stride, flags, true)) {
+    case SmallKernel::kTile16: {
+        const Tile16LaunchShape g = gemv_tile16_shape(w->ctx, (uint32_t)((w->n + 15) / 16), (uint32_t)w->k, staged_rows(x_dtype, rows));
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_tile16_q%u_g%u", (unsigned)w->fmt.bits, w->fmt.group_size);
         s->grid[0] = g.grid;
         s->block[0] = g.block;
         s->lds_bytes = g.lds_bytes;
         s->rows_per_workgroup = 16;
-    } else if (!forced && mfma_planes_pays(v.bits, x_dtype, m) && gemv_mfma_planes_eligible(v, x_dtype, m > most ? most : m, x_stride) &&
-               !(gemv_rows_batch_pays(1, &v, x_dtype, m) && gemv_fast_eligible(v, x_dtype, m, x_stride))) {
+        return;
+    }
+    case SmallKernel::kMfmaPlanes: {
         const Tile16LaunchShape g = gemv_mfma_planes_shape(w->ctx, (uint32_t)((w->n + 15) / 16), (uint32_t)w->k,
-                                                           (uint32_t)w->fmt.bits, staged_rows(x_dtype, m > most ? most : m));
-        std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_mfma_planes_q%u_g%u", (unsigned)w->fmt.bits,
-                      w->fmt.group_size);
+                                                           (uint32_t)w->fmt.bits, staged_rows(x_dtype, rows));
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_mfma_planes_q%u_g%u", (unsigned)w->fmt.bits, w->fmt.group_size);
         s->grid[0] = g.wgs_per_part;
         s->grid[1] = g.parts;
         s->block[0] = g.block;
         s->lds_bytes = g.lds_bytes;
         s->rows_per_workgroup = 16 * g.tiles_per_wg * g.passes;
-    } else if (!forced && gemv_fast_eligible(v, x_dtype, m > 8 ? 8 : m, x_stride)) {
-        const GemvLaunchShape g = gemv_fast_shape(w->ctx, v, m > 8 ? 8 : m, x_dtype);
+        return;
+    }
+    case SmallKernel::kDotPlanes: {
+        const GemvLaunchShape g = gemv_fast_shape(w->ctx, v, rows > 8 ? 8 : rows, x_dtype);
         std::snprintf(s->device_kernel, sizeof s->device_kernel, "%s_q%u_g%u",
                       std::strcmp(g.kernel, "gemv_rows_kernel") == 0 ? "gemv_rows" : "gemv_planes", (unsigned)w->fmt.bits,
                       w->fmt.group_size);
@@ -119,29 +79,71 @@ void plan_small_m(const mi355q_weight* w, uint32_t m, int x_dtype, uint32_t x_st
         s->block[0] = g.block;
         s->lds_bytes = g.lds_bytes;
         s->rows_per_workgroup = g.rows_per_workgroup;
-    } else if (!forced && gemv_staf_eligible(v, x_dtype, m > 8 ? 8 : m, x_stride)) {
-        const GemvLaunchShape g = gemv_staf_shape(w->ctx, v, m > 8 ? 8 : m);
-        std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_staf_q%u_g%u", (unsigned)w->fmt.bits,
-                      w->fmt.group_size);
+        return;
+    }
+    case SmallKernel::kStafInPlace: {
+        const GemvLaunchShape g = gemv_staf_shape(w->ctx, v, rows > 8 ? 8 : rows);
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_staf_q%u_g%u", (unsigned)w->fmt.bits, w->fmt.group_size);
         s->grid[0] = g.grid;
         s->block[0] = g.block;
         s->lds_bytes = g.lds_bytes;
         s->rows_per_workgroup = g.rows_per_workgroup;
-    } else if (gemm_two_step_chosen(v, x_dtype, m, x_stride, flags) && !library_ruled_out(w->ctx)) {
-        // no decode kernel reads this layout with this activation type: dequantise once + the dense library product
-        // a few rows: fp32 weights and an fp32 product whatever the activation type (the decode kernels' arithmetic)
-        std::snprintf(s->device_kernel, sizeof s->device_kernel, "dequant_q%u_g%u_f32+hipblaslt_gemm_f32", (unsigned)w->fmt.bits,
-                      w->fmt.group_size);
-        std::snprintf(s->kernel_family, sizeof s->kernel_family, "libraryGEMM");
-        s->block[0] = 256;
-    } else {
+        return;
+    }
+    default:
         std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_generic");
         s->grid[0] = (uint32_t)((w->n + 3) / 4);
         s->grid[1] = m;
         s->block[0] = 256;
         s->rows_per_workgroup = 4;
         s->used_fallback = 1;
-        s->fallback_reason = forced ? MI355Q_FALLBACK_DISABLED_BY_ENVIRONMENT : MI355Q_FALLBACK_UNAVAILABLE_ACCELERATION;
+        s->fallback_reason = (flags & MI355Q_FLAG_FORCE_GENERIC) ? MI355Q_FALLBACK_DISABLED_BY_ENVIRONMENT
+                                                                 : MI355Q_FALLBACK_UNAVAILABLE_ACCELERATION;
+        return;
+    }
+}
+
+void plan_stream(const mi355q_weight* w, uint32_t rows, const char* prefix, mi355q_step* s) {
+    const StreamLaunchShape g = gemm_stream_shape(w->ctx, rows, (uint32_t)w->n, (uint32_t)w->k);
+    std::snprintf(s->device_kernel, sizeof s->device_kernel, "%sqgemm_stream_q%u_g%u", prefix, (unsigned)w->fmt.bits, w->fmt.group_size);
+    s->grid[0] = g.row_blocks;
+    s->grid[1] = g.parts;
+    s->block[0] = 768;
+    s->lds_bytes = g.lds_bytes;
+    s->rows_per_workgroup = 64;
+}
+
+// Record of a route that runs on the decode kernels or beside them (what dispatch_linear does for the same route).
+void plan_small_m(const mi355q_weight* w, uint32_t m, int x_dtype, uint32_t x_stride, uint32_t flags, LinearRoute route,
+                  mi355q_step* s) {
+    const WView v = w->view();
+    switch (route) {
+    case LinearRoute::kSplitRows:
+        if (!(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_SMALL_M)) && split_rows_take_stream(v, x_dtype, m)) {
+            // fp32 rows as three bf16 rows each on the streamed-weight kernel, then the sum of the partial results
+            plan_stream(w, split_rows_parts(x_dtype) * m, "split_f32_bf16x3+", s);
+        } else {
+            // ... on the bf16 decode kernel
+            plan_small_kernel(w, split_rows_parts(x_dtype) * m, MI355Q_BF16, split_rows_stride((uint32_t)w->k), flags, s);
+            char inner[sizeof s->device_kernel];
+            std::snprintf(inner, sizeof inner, "%s", s->device_kernel);
+            std::snprintf(s->device_kernel, sizeof s->device_kernel, "split_f32_bf16x3+%.30s", inner);
+        }
+        return;
+    case LinearRoute::kStream:
+        plan_stream(w, m, "", s);      // blocks in place from three rows: the streamed-weight kernel with unrounded weights
+        return;
+    case LinearRoute::kTwoStep:
+        // no decode kernel reads this layout with this activation type: dequantise once + the dense library product
+        // a few rows: fp32 weights and an fp32 product whatever the activation type (the decode kernels' arithmetic)
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "dequant_q%u_g%u_f32+hipblaslt_gemm_f32", (unsigned)w->fmt.bits,
+                      w->fmt.group_size);
+        std::snprintf(s->kernel_family, sizeof s->kernel_family, "libraryGEMM");
+        s->block[0] = 256;
+        return;
+    default:
+        plan_small_kernel(w, m, x_dtype, x_stride, flags, s);
+        return;
     }
 }
 
@@ -228,7 +230,11 @@ mi355q_status mi355q_plan_decode_step(const mi355q_weight* w, uint32_t m, mi355q
     std::snprintf(out->kernel_name, sizeof out->kernel_name, "%s", w->fmt.gemv_kernel_name);
     std::snprintf(out->kernel_family, sizeof out->kernel_family, "q%uG%uGEMV", (unsigned)w->fmt.bits,
                   w->fmt.group_size);
-    plan_small_m(w, m, x_dtype, (uint32_t)w->k, flags, out);
+    RouteFacts facts{};
+    facts.decode_entry = true;
+    facts.library_ok = !library_ruled_out(w->ctx);
+    facts.x_aligned = true;
+    plan_small_m(w, m, x_dtype, (uint32_t)w->k, flags, linear_route(w->view(), x_dtype, m, (uint32_t)w->k, flags, facts), out);
     return MI355Q_OK;
 }
 
@@ -252,20 +258,24 @@ mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w, uint32_t maximum
         std::snprintf(s->kernel_name, sizeof s->kernel_name, "%s", w->fmt.gemv_kernel_name);
         std::snprintf(s->kernel_family, sizeof s->kernel_family, "q%uG%uGEMV", (unsigned)w->fmt.bits,
                       w->fmt.group_size);
-        plan_small_m(w, 1, x_dtype, input_row_stride, flags, s);
+        RouteFacts one{};
+        one.decode_entry = true;
+        one.library_ok = !library_ruled_out(w->ctx);
+        one.x_aligned = true;
+        plan_small_m(w, 1, x_dtype, input_row_stride, flags, linear_route(v, x_dtype, 1, input_row_stride, flags, one), s);
         s->used_fallback = 1;
         s->fallback_reason = MI355Q_FALLBACK_LAST_TOKEN_USES_DECODE_KERNEL;
         return MI355Q_OK;
     }
 
     const uint32_t m = maximum_sequence_length;
-    const uint32_t small_rows = small_batch_limit(v, x_dtype, input_row_stride);  // rows the decode kernels keep
-    const bool want_small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) ||
-                            (!(flags & MI355Q_FLAG_FORCE_MFMA) && m <= small_rows) ||
-                            split_rows_chosen(v, x_dtype, m, input_row_stride, flags);
-    const bool mfma_ok = gemm_mfma_eligible(v, x_dtype, m, input_row_stride) || gemm_wide_taken(v, x_dtype, m, input_row_stride, flags);
-    if (!split_rows_chosen(v, x_dtype, m, input_row_stride, flags) && gemm_two_step_chosen(v, x_dtype, m, input_row_stride, flags) &&
-        !library_ruled_out(w->ctx)) {
+    // the same table the launcher reads (route.cpp): the library counts as there unless it is ruled out for the context
+    RouteFacts facts{};
+    facts.decode_entry = false;
+    facts.library_ok = !library_ruled_out(w->ctx);
+    facts.x_aligned = true;
+    const LinearRoute route = linear_route(v, x_dtype, m, input_row_stride, flags, facts);
+    if (route == LinearRoute::kTwoStep) {
         // dequant_q{b}_g{g}_bf16 into the scratch matrix, then the dense GEMM (MetalPrefillStepBuilder's two-dispatch
         // route; the dense product is the platform library's, as the reference's is matmul2d)
         *out_count = 2;
@@ -297,10 +307,7 @@ mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w, uint32_t maximum
     fill_common(w, m, s);
     s->path = MI355Q_PATH_PREFILL_PROJECTION;
     s->input_row_stride = input_row_stride;
-    if (!(flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA)) &&
-        !split_rows_chosen(v, x_dtype, m, input_row_stride, flags) &&
-        ((flags & MI355Q_FLAG_FORCE_STREAM) ? gemm_stream_eligible(v, x_dtype, m, input_row_stride)
-                                            : gemm_stream_chosen(v, x_dtype, m, input_row_stride))) {
+    if (route == LinearRoute::kStream) {
         // weights streamed through registers into the matrix cores: the direct quantized GEMM at a few dozen rows
         std::snprintf(s->kernel_name, sizeof s->kernel_name, "%s", w->fmt.gemm_kernel_name_f32s);
         std::snprintf(s->device_kernel, sizeof s->device_kernel, "qgemm_stream_q%u_g%u", (unsigned)w->fmt.bits,
@@ -314,7 +321,7 @@ mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w, uint32_t maximum
         s->rows_per_workgroup = 64;
         return MI355Q_OK;
     }
-    if (!want_small && mfma_ok) {
+    if (route == LinearRoute::kFused) {
         // fused dequant + matrix-core contraction: the stand-in for dequant_q*_bf16 + gemm_bf16_f32s
         std::snprintf(s->kernel_name, sizeof s->kernel_name, "%s", w->fmt.gemm_kernel_name_f32s);
         std::snprintf(s->device_kernel, sizeof s->device_kernel, "qgemm_mfma_q%u_g%u", (unsigned)w->fmt.bits,
@@ -332,17 +339,89 @@ mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w, uint32_t maximum
         s->rows_per_workgroup = g.bn;
         return MI355Q_OK;
     }
-    // direct per-row kernel with the sequence signature (gemm_q{b}_g{g}[_f32s])
+    // the decode kernels with the sequence signature (gemm_q{b}_g{g}[_f32s]): small batches, split fp32 rows, and the
+    // weights no matrix-core kernel reads (recorded as a fallback, with the reference's reason)
     std::snprintf(s->kernel_name, sizeof s->kernel_name, "%s",
                   x_dtype == MI355Q_F32 ? w->fmt.gemm_kernel_name_f32s : w->fmt.gemm_kernel_name);
     std::snprintf(s->kernel_family, sizeof s->kernel_family, "q%uG%uGEMM", (unsigned)w->fmt.bits,
                   w->fmt.group_size);
-    plan_small_m(w, m, x_dtype, input_row_stride, flags, s);
-    if (!want_small && !mfma_ok) {
+    plan_small_m(w, m, x_dtype, input_row_stride, flags, route, s);
+    const bool want_small = (flags & (MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_GENERIC)) ||
+                            (!(flags & MI355Q_FLAG_FORCE_MFMA) && m <= small_batch_limit(v, x_dtype, input_row_stride)) ||
+                            route == LinearRoute::kSplitRows;
+    const bool fused_ok = gemm_mfma_eligible(v, x_dtype, m, input_row_stride) || gemm_wide_taken(v, x_dtype, m, input_row_stride, flags);
+    if (!want_small && !fused_ok) {
         s->used_fallback = 1;
         s->fallback_reason = (input_row_stride != w->k) ? MI355Q_FALLBACK_INPUT_STRIDE_MISMATCH
                                                         : MI355Q_FALLBACK_UNAVAILABLE_ACCELERATION;
     }
+    return MI355Q_OK;
+}
+
+// Measurement / test aid: the route table on a synthetic weight, no device needed.  `launcher_out` is what
+// dispatch_linear and run_small_m would run ("route" or "route/kernel"), `planner_out` the device kernels the plan
+// records name, joined by '+'.
+mi355q_status mi355q_probe_route(uint8_t scheme_identifier, uint32_t layout, uint32_t sb_dtype, uint64_t n_rows, uint64_t k,
+                                 mi355q_dtype x_dtype, uint32_t m, uint32_t x_row_stride, uint32_t flags, int decode_entry,
+                                 int library_available, char* launcher_out, char* planner_out, size_t cap) {
+    const mi355q_format* f = find_format_scheme(scheme_identifier);
+    if (!f) return fail(MI355Q_ERR_UNSUPPORTED_FORMAT, "unsupported scheme 0x%02x", scheme_identifier);
+    if (!launcher_out || !planner_out || cap < 16) return fail(MI355Q_ERR_INVALID_ARGUMENT, "output buffers");
+    if (!n_rows || !k || k % f->group_size) return fail(MI355Q_ERR_SHAPE, "K must be a whole number of groups");
+    if (layout != MI355Q_LAYOUT_STAF_BLOCKS && (k * f->bits) % 32) return fail(MI355Q_ERR_SHAPE, "planes need whole words per row");
+    if (layout == MI355Q_LAYOUT_TILE16 && (f->bits != 4 || f->group_size != 64 || k % 128))
+        return fail(MI355Q_ERR_UNSUPPORTED_FORMAT, "TILE16 holds q4 g64 with K %% 128 == 0");
+    if (x_row_stride == 0) x_row_stride = (uint32_t)k;
+    mi355q_context ctx;
+    std::memset((void*)&ctx, 0, sizeof ctx);
+    ctx.props.multiProcessorCount = 256;
+    ctx.dense_library_forbidden = !library_available;
+    mi355q_weight w;
+    std::memset((void*)&w, 0, sizeof w);
+    w.ctx = &ctx;
+    w.fmt = *f;
+    w.n = n_rows; w.k = k;
+    w.layout = (uint8_t)layout;
+    w.sb_dtype = layout == MI355Q_LAYOUT_STAF_BLOCKS ? (uint8_t)MI355Q_F16 : (uint8_t)sb_dtype;
+    uint32_t* const fake = (uint32_t*)(uintptr_t)0x10000000;     // aligned, never read
+    const uint32_t wpr = (uint32_t)(k * f->bits / 32), bpr = (uint32_t)(k / f->group_size);
+    if (layout == MI355Q_LAYOUT_STAF_BLOCKS) w.blocks = fake;
+    else if (layout == MI355Q_LAYOUT_TILE16) w.tiles = fake;
+    else {
+        w.codes = fake; w.sz = fake + wpr; w.scales = fake; w.biases = fake;
+        w.code_stride = w.sz_stride = (wpr + bpr + 3u) & ~3u;
+    }
+    const WView v = w.view();
+    RouteFacts facts{};
+    facts.decode_entry = decode_entry != 0;
+    facts.library_ok = library_available != 0;
+    facts.x_aligned = true;
+    const LinearRoute r = linear_route(v, x_dtype, m, x_row_stride, flags, facts);
+    const char* detail = "";
+    if (r == LinearRoute::kSmallBatch) {
+        const uint32_t step = small_batch_step(v, x_dtype, m, x_row_stride, flags);
+        detail = small_kernel_name(small_kernel(v, x_dtype, m < step ? m : step, x_row_stride, flags, true));
+    } else if (r == LinearRoute::kFused) {
+        detail = gemm_wide_taken(v, x_dtype, m, x_row_stride, flags) ? "wide" : "tiled";
+    } else if (r == LinearRoute::kSplitRows) {
+        if (!(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_SMALL_M)) && split_rows_take_stream(v, x_dtype, m)) detail = "stream";
+        else {
+            const uint32_t pm = split_rows_parts(x_dtype) * m, kp = split_rows_stride((uint32_t)k);
+            const uint32_t step = small_batch_step(v, MI355Q_BF16, pm, kp, flags);
+            detail = small_kernel_name(small_kernel(v, MI355Q_BF16, pm < step ? pm : step, kp, flags, true));
+        }
+    }
+    std::snprintf(launcher_out, cap, "%s%s%s", linear_route_name(r), *detail ? "/" : "", detail);
+    planner_out[0] = 0;
+    mi355q_step steps[2];
+    uint32_t count = 0;
+    mi355q_status st;
+    if (decode_entry) { st = mi355q_plan_decode_step(&w, m, x_dtype, flags, &steps[0]); count = 1; }
+    else st = mi355q_plan_prefill_steps(&w, m, x_row_stride, x_dtype, 0, flags, steps, &count);
+    if (st != MI355Q_OK) { std::snprintf(planner_out, cap, "error"); return MI355Q_OK; }
+    size_t at = 0;
+    for (uint32_t i = 0; i < count && at < cap; i++)
+        at += (size_t)std::snprintf(planner_out + at, cap - at, "%s%s", i ? "+" : "", steps[i].device_kernel);
     return MI355Q_OK;
 }
 
