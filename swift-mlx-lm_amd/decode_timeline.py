@@ -1,4 +1,4 @@
-"""Per-workgroup timeline of the decode launches (BASELINE config 1: 4-bit, groups of 64, M = 1).
+"""Per-workgroup timeline of the decode launches (benchmark config 1: 4-bit, groups of 64, M = 1).
 
 Runs the measurement build of the library (python swift-mlx-lm_amd/build.py --timeline), whose decode rows kernel
 writes four 100 MHz time stamps per workgroup (entry, activations staged, first weight words there, exit) and the

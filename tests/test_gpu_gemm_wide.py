@@ -5,7 +5,7 @@ Numerics are those of the reference's dequant -> bf16 -> GEMM route
 fp64 accumulation of the bf16-rounded dequantised weights from the CPU oracle.  Bars as for the tiled kernel:
 relative L2 <= 1e-3 and max-abs <= 2e-2 on the fp32 output, 16-bit outputs equal to the rounding of the fp32 output,
 exactly representable cases compared exactly.  The kernel is forced with the probe flag where the shape is smaller
-than what the dispatcher gives it; BASELINE config 3 runs as dispatched.
+than what the dispatcher gives it; benchmark config 3 runs as dispatched.
 """
 import sys
 
@@ -149,7 +149,7 @@ def test_wide_gemm_blocks_and_f16_seeded_against_the_oracle(pkg, ctx):
 @pytest.mark.parametrize("layout_name,x_name", [("LAYOUT_STAF_BLOCKS", "BF16"), ("LAYOUT_PLANES", "F16"), ("LAYOUT_STAF_BLOCKS", "F16")])
 @pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
 def test_config3_on_blocks_and_f16_as_dispatched(pkg, ctx, layout_name, x_name, n, k):
-    """BASELINE config 3 at M = 2048 on the reference's block layout and with its f16 activations, no flags: the
+    """benchmark config 3 at M = 2048 on the reference's block layout and with its f16 activations, no flags: the
     plan names this library's matrix-core kernel, and the result holds the bar on the tile-edge column sample."""
     m = 2048
     layout, x_dtype = getattr(pkg, layout_name), getattr(pkg, x_name)
@@ -208,7 +208,7 @@ def test_wide_gemm_with_k_in_parts(pkg, ctx, tile_rows, parts):
 @pytest.mark.parametrize("m", [128, 512, 2048])
 @pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
 def test_config3_prefill_as_dispatched(pkg, ctx, m, n, k):
-    """BASELINE config 3 at full size with no flags: whatever route the library picks for the shape (the plan record
+    """benchmark config 3 at full size with no flags: whatever route the library picks for the shape (the plan record
     names it) is checked against the oracle on every row and the tile-edge column sample."""
     sample = _tile_edge_sample(n, 17 * m + n, tile=256)
     w, _, _, (rel, _) = _seeded(pkg, ctx, 4200 + m % 83, m, n, k, 64, 0, sample=sample)
