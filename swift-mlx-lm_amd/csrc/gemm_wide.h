@@ -16,6 +16,7 @@ struct WideArgs {
     uint32_t tiles_m, tiles_n;
     uint32_t y_dtype;
     uint32_t wide_stores;        // rows of y are 16-byte aligned for every column that is a multiple of four
+    uint32_t line_stores;        // rows of y are 16-byte aligned at every tile's first column: whole lines through LDS
     float* partial;              // K split over workgroups: fp32 [splits][M][N] partial results (null otherwise)
     uint32_t splits, kt_per_split;   // K-tiles per split: a multiple of four
     unsigned long long* probe;   // optional: [0] shader cycles, [1] 100 MHz ticks that workgroup 0 spent in the kernel

@@ -196,6 +196,7 @@ mi355q_status launch_qgemm_wide(hipStream_t s, mi355q_context* ctx, const WView&
     a.code_stride = w.code_stride; a.sz_stride = w.sz_stride;
     a.y_dtype = (uint32_t)y_dtype;
     a.wide_stores = (y_stride % 4 == 0 && (uintptr_t)y % 16 == 0) ? 1u : 0u;
+    a.line_stores = ((size_t)y_stride * (y_dtype == MI355Q_F32 ? 4 : 2) % 16 == 0 && (uintptr_t)y % 16 == 0) ? 1u : 0u;
     a.probe = probe;
     const GemmLaunchShape g = gemm_wide_shape(m, w.n, w.k);
     a.splits = g.splits; a.kt_per_split = g.kt_per_split;

@@ -369,11 +369,72 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
             });
         });
     };
-    if (a.partial)         // this part of K as fp32 (N is a multiple of four: 16-byte stores); wide_reduce_kernel adds the parts
-        store_tiles(std::integral_constant<int, MI355Q_F32>{}, a.partial + (size_t)split * a.m * a.n, a.n, true);
-    else if (a.y_dtype == MI355Q_BF16) store_tiles(std::integral_constant<int, MI355Q_BF16>{}, a.y, a.ys, a.wide_stores != 0);
-    else if (a.y_dtype == MI355Q_F32) store_tiles(std::integral_constant<int, MI355Q_F32>{}, a.y, a.ys, a.wide_stores != 0);
-    else store_tiles(std::integral_constant<int, MI355Q_F16>{}, a.y, a.ys, a.wide_stores != 0);
+    // Whole cache lines instead: a wavefront's 32 rows x 64 columns of one accumulator row pass through LDS (the
+    // activation stages are free now), are read back eight (fp32: four) rows at a time with sixteen bytes per lane, and
+    // go out as full 128-byte lines.  (Stores of eight bytes per lane, 32 rows apart, as the loop above makes them,
+    // took 11 us per tile when every workgroup of a round stored at once; these take about 3.)  Taken when the tile's
+    // 256 columns lie inside the matrix and the rows of y are 16-byte aligned.
+    auto store_lines = [&](auto DT, void* const y, const size_t ys) __attribute__((always_inline)) {
+        constexpr int dt = decltype(DT)::value;
+        constexpr int ESZ = dt == MI355Q_F32 ? 4 : 2;
+        constexpr int PITCH = 64 * ESZ + 16;                       // a row of the staging block: 16 bytes of padding
+        constexpr int RPI = ESZ == 4 ? 4 : 8;                      // rows per read-back instruction
+        constexpr int LPR = 64 / RPI;                              // lanes per row
+        char* const stage = lds + wave * (32 * PITCH);
+        __builtin_amdgcn_s_barrier();                              // every wavefront is done with the activation stages
+        static_for<TM>([&](auto I) __attribute__((always_inline)) {
+            constexpr int i = decltype(I)::value;
+            asm volatile("" : "+v"(acc[0][i]), "+v"(acc[1][i]));
+#pragma unroll
+            for (int f = 0; f < 2; f++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const float v0 = acc[f][i][4 * g + 0], v1 = acc[f][i][4 * g + 1], v2 = acc[f][i][4 * g + 2], v3 = acc[f][i][4 * g + 3];
+                    char* const at = stage + ln * PITCH + (32 * f + 8 * g + 4 * lh) * ESZ;
+                    if constexpr (dt == MI355Q_F32) {
+                        const wd_float4_v t = {v0, v1, v2, v3};
+                        *(wd_float4_v*)at = t;
+                    } else {
+                        u32x2 t;
+                        t.x = dt == MI355Q_BF16 ? wd_pack_bf16(v0, v1) : wd_pack_f16(v0, v1);
+                        t.y = dt == MI355Q_BF16 ? wd_pack_bf16(v2, v3) : wd_pack_f16(v2, v3);
+                        *(u32x2*)at = t;
+                    }
+                }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int t = 0; t < 32 / RPI; t++) {
+                const uint32_t r = t * RPI + lane / LPR, piece = lane % LPR;
+                const u32x4 d = *(const u32x4*)(stage + r * PITCH + piece * 16);
+                const uint32_t row = m0 + i * 32 + r;
+                if (row < a.m)
+                    *(u32x4*)((char*)y + ((size_t)row * ys + n0 + 64 * wave) * ESZ + piece * 16) = d;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        });
+    };
+    const bool inner = n0 + kWideBN <= a.n;                        // (uniform over the workgroup)
+    if (a.partial) {       // this part of K as fp32 (N is a multiple of four: 16-byte stores); wide_reduce_kernel adds the parts
+        float* const part = a.partial + (size_t)split * a.m * a.n;
+        if (inner) store_lines(std::integral_constant<int, MI355Q_F32>{}, part, a.n);
+        else store_tiles(std::integral_constant<int, MI355Q_F32>{}, part, a.n, true);
+        return;
+    }
+    const bool lines = inner && a.line_stores;
+    if (a.y_dtype == MI355Q_BF16) {
+        if (lines) store_lines(std::integral_constant<int, MI355Q_BF16>{}, a.y, a.ys);
+        else store_tiles(std::integral_constant<int, MI355Q_BF16>{}, a.y, a.ys, a.wide_stores != 0);
+    } else if (a.y_dtype == MI355Q_F32) {
+        if (lines) store_lines(std::integral_constant<int, MI355Q_F32>{}, a.y, a.ys);
+        else store_tiles(std::integral_constant<int, MI355Q_F32>{}, a.y, a.ys, a.wide_stores != 0);
+    } else {
+        if (lines) store_lines(std::integral_constant<int, MI355Q_F16>{}, a.y, a.ys);
+        else store_tiles(std::integral_constant<int, MI355Q_F16>{}, a.y, a.ys, a.wide_stores != 0);
+    }
 }
 
 
