@@ -681,8 +681,8 @@ def main():
                                            "route": " + ".join(st.device_kernel for st in steps_p),
                                            "first_sample_us": round(ms_first * 1e3, 1), "samples_of": [taken, reps]}
                 xb.free(); yb.free()
-        # the reference prefills with f16 or fp32 activations: the two-dispatch route in those types, M = 2048 gate
-        for tname, xt, npdt in (("f16", pkg.F16, np.float16), ("f32", pkg.F32, np.float32)):  # fp32: two bf16 products
+        # the reference prefills with f16 or fp32 activations: the same launch in those types, as dispatched, M = 2048 gate
+        for tname, xt, npdt in (("f16", pkg.F16, np.float16), ("f32", pkg.F32, np.float32)):  # fp32: [hi | lo] bf16 halves, 2 K
             wts = [L["gate"] for L in layers[:4]]
             xa = kat.seeded_activations(2548, 2048, 4096).astype(npdt)
             xb = ctx.upload(xa.view(np.uint16) if tname == "f16" else xa)

@@ -142,8 +142,9 @@ mi355q_status launch_split_rows_bf16(hipStream_t s, const void* x, int x_dtype, 
                                      uint16_t* out, uint32_t out_stride);
 mi355q_status launch_sum_parts_rows(hipStream_t s, const float* yp, uint32_t parts, uint32_t m, uint32_t n, void* y, int y_dtype,
                                     uint32_t y_stride);
+// (`out_stride`: elements from one row of hi / lo to the next; 0 = k)
 mi355q_status launch_split_f32_bf16x2(hipStream_t s, const float* x, uint32_t m, uint32_t k, uint32_t x_stride, uint16_t* hi,
-                                      uint16_t* lo);
+                                      uint16_t* lo, uint32_t out_stride = 0);
 mi355q_status launch_gemv_generic(hipStream_t s, const WView& w, const void* x, int x_dtype,
                                   void* y, int y_dtype, uint32_t m, uint32_t x_stride,
                                   uint32_t y_stride);
@@ -363,7 +364,10 @@ constexpr uint32_t kWideMinRows = 384;
 constexpr uint32_t kWideRowsBesideLibrary = 2560;   // from here the two-dispatch route is taken where the dense library is there
 bool gemm_wide_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
 bool gemm_wide_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
+// `k`: the K the kernel walks (twice the weight's K for fp32 activations, see gemm_wide_k)
 GemmLaunchShape gemm_wide_shape(uint32_t m, uint32_t n, uint32_t k);
+// fp32 activations run as two bf16 halves side by side, hi = bf16(x) and lo = bf16(x - hi), against the weights twice
+inline uint32_t gemm_wide_k(uint32_t k, int x_dtype) { return x_dtype == MI355Q_F32 ? 2 * k : k; }
 uint32_t chip_cus();
 void gemm_wide_force_shape(uint32_t bm, uint32_t splits);      // A/B runs (mi355q_probe_wide_shape)
 inline bool gemm_wide_taken(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride, uint32_t flags) {

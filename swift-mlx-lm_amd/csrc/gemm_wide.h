@@ -19,6 +19,8 @@ struct WideArgs {
     uint32_t line_stores;        // rows of y are 16-byte aligned at every tile's first column: whole lines through LDS
     float* partial;              // K split over workgroups: fp32 [splits][M][N] partial results (null otherwise)
     uint32_t splits, kt_per_split;   // K-tiles per split: a multiple of four
+    uint32_t w_fours;                // groups of four K-tiles in a weight row: the walk over K wraps there (fp32 activations
+                                     // come as [hi | lo] rows of 2 K bf16 values against the same weights twice)
     unsigned long long* probe;   // optional: [0] shader cycles, [1] 100 MHz ticks that workgroup 0 spent in the kernel
 };
 

@@ -87,7 +87,8 @@ __global__ __launch_bounds__(256) void wide_reduce_kernel(const wd_float4_v* __r
 // of codes and of (scale, bias) words (a row's words of four K-tiles are one 16- or 8-byte load).  Blocks in place:
 // whole blocks of 4 + group / 2 bytes at a 4-byte aligned address.
 bool gemm_wide_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
-    if ((x_dtype != MI355Q_BF16 && x_dtype != MI355Q_F16) || m < 1) return false;
+    if ((x_dtype != MI355Q_BF16 && x_dtype != MI355Q_F16 && x_dtype != MI355Q_F32) || m < 1) return false;
+    if (x_dtype == MI355Q_F32 && x_stride % 4) return false;        // 16-byte loads of the rows that are split
     if (w.bits != 4 || (w.group != 64 && w.group != 128)) return false;
     if (w.k % 256 || x_stride % 8) return false;
     if ((uint64_t)x_stride * 2 * 256 >= (1ull << 32)) return false;               // offsets inside a tile are 32-bit
@@ -177,7 +178,7 @@ GemmLaunchShape gemm_wide_shape(uint32_t m, uint32_t n, uint32_t k) {
 // the two-dispatch route: enough tiles to occupy three quarters of the CUs.
 bool gemm_wide_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
     if (!gemm_wide_eligible(w, x_dtype, m, x_stride) || m < kWideMinRows) return false;
-    const GemmLaunchShape g = gemm_wide_shape(m, w.n, w.k);
+    const GemmLaunchShape g = gemm_wide_shape(m, w.n, gemm_wide_k(w.k, x_dtype));
     const uint32_t wgs = ((m + g.bm - 1) / g.bm) * ((w.n + kWideBN - 1) / kWideBN) * g.splits;
     return 4 * wgs >= 3 * chip_cus();
 }
@@ -187,21 +188,37 @@ mi355q_status launch_qgemm_wide(hipStream_t s, mi355q_context* ctx, const WView&
     if (!gemm_wide_eligible(w, x_dtype, m, x_stride))
         return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the wide-tile MFMA GEMM does not accept this format, layout or stride");
     if ((uintptr_t)x % 16) return fail(MI355Q_ERR_INVALID_ARGUMENT, "activation pointer must be 16-byte aligned");
+    const uint32_t k_walk = gemm_wide_k(w.k, x_dtype);
+    const GemmLaunchShape g = gemm_wide_shape(m, w.n, k_walk);
+    // fp32 activations (the reference's prefill type, gemm_q4_g*_f32s): every row becomes [hi | lo], hi = bf16(x) and
+    // lo = bf16(x - hi), sixteen bits of each activation, in scratch of the context; the kernel walks 2 K against the
+    // weights twice, so the two halves meet in the fp32 accumulators
+    const size_t split_bytes = x_dtype == MI355Q_F32 ? (((size_t)m * k_walk * 2 + 255) & ~(size_t)255) : 0;
+    const size_t part_bytes = g.splits > 1 ? (size_t)g.splits * m * w.n * sizeof(float) : 0;
+    const void* xk = x;
+    uint32_t xk_stride = x_stride;
+    if (split_bytes) {
+        if (mi355q_status st = ensure_split_buffer(ctx, split_bytes)) return st;
+        uint16_t* const hi = (uint16_t*)ctx->split_buffer;
+        if (mi355q_status st = launch_split_f32_bf16x2(s, (const float*)x, m, w.k, x_stride, hi, hi + w.k, k_walk)) return st;
+        xk = hi;
+        xk_stride = k_walk;
+    }
     WideArgs a{};
     const bool blocks = w.layout == MI355Q_LAYOUT_STAF_BLOCKS;
     a.codes = w.codes; a.sz = w.sz; a.blocks = w.blocks;
     a.row_bytes = w.blocks_per_row * w.bytes_per_block;
-    a.x = (const uint16_t*)x; a.y = y;
-    a.m = m; a.n = w.n; a.k = w.k; a.xs = x_stride; a.ys = y_stride;
+    a.x = (const uint16_t*)xk; a.y = y;
+    a.m = m; a.n = w.n; a.k = k_walk; a.xs = xk_stride; a.ys = y_stride;
+    a.w_fours = w.k / 256;
     a.code_stride = w.code_stride; a.sz_stride = w.sz_stride;
     a.y_dtype = (uint32_t)y_dtype;
     a.wide_stores = (y_stride % 4 == 0 && (uintptr_t)y % 16 == 0) ? 1u : 0u;
     a.line_stores = ((size_t)y_stride * (y_dtype == MI355Q_F32 ? 4 : 2) % 16 == 0 && (uintptr_t)y % 16 == 0) ? 1u : 0u;
     a.probe = probe;
-    const GemmLaunchShape g = gemm_wide_shape(m, w.n, w.k);
     a.splits = g.splits; a.kt_per_split = g.kt_per_split;
-    if (g.splits > 1) {
-        if (mi355q_status st = ensure_workspace(ctx, (size_t)g.splits * m * w.n * sizeof(float))) return st;
+    if (part_bytes) {
+        if (mi355q_status st = ensure_workspace(ctx, part_bytes)) return st;
         a.partial = (float*)ctx->workspace;
     }
     const bool sb_bf16 = w.sb_dtype == MI355Q_BF16;

@@ -109,16 +109,17 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
             sz_off[f] = gr * a.sz_stride * 4;
         }
     }
-    const char* const cg = BLOCKS ? (const char*)a.blocks + (size_t)n0 * a.row_bytes + (size_t)(kt_begin / 4) * FOUR_BYTES
-                                  : (const char*)(a.codes + (size_t)n0 * a.code_stride) + (size_t)(kt_begin / 4) * 128;
-    const char* const sg = BLOCKS ? cg : (const char*)(a.sz + (size_t)n0 * a.sz_stride) + (size_t)(kt_begin / 4) * (SZW * 4);
+    const char* const cg = BLOCKS ? (const char*)a.blocks + (size_t)n0 * a.row_bytes : (const char*)(a.codes + (size_t)n0 * a.code_stride);
+    const char* const sg = BLOCKS ? cg : (const char*)(a.sz + (size_t)n0 * a.sz_stride);
+    const uint32_t four_begin = kt_begin / 4;
     using sz_vec = std::conditional_t<SZW == 4, u32x4, u32x2>;      // kept whole: the loads write them behind the compiler's back
     u32x4 wnext[2][4], wcur[2][4];
     sz_vec sznext[2];
     uint32_t szone[2][SZW];                                         // blocks in place: one word per K-tile (g64) or per two
     uint32_t szcur[2][SZW];
     auto load_w = [&](uint32_t four) __attribute__((always_inline)) {
-        const uint32_t p = four * 4 < KT ? four : KT / 4 - 1;
+        uint32_t p = four_begin + (four * 4 < KT ? four : KT / 4 - 1);
+        p = p >= a.w_fours ? p - a.w_fours : p;      // the second half of [hi | lo] activations meets the same weights again
         const char* const g = wd_scalar(cg + (size_t)p * FOUR_BYTES);
         const char* const gs = BLOCKS ? g : wd_scalar(sg + (size_t)p * (SZW * 4));
 #pragma unroll

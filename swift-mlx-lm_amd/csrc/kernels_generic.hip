@@ -362,7 +362,7 @@ mi355q_status launch_dequant(hipStream_t s, const WView& w, void* out) {
 // (x - hi is exact in fp32).  Four elements per thread; x rows 16-byte aligned, K a multiple of 4.
 __global__ __launch_bounds__(256) void split_f32_bf16x2_kernel(const float* __restrict__ x, uint32_t m, uint32_t k,
                                                                uint32_t x_stride, uint16_t* __restrict__ hi,
-                                                               uint16_t* __restrict__ lo) {
+                                                               uint16_t* __restrict__ lo, uint32_t out_stride) {
     const uint32_t row = blockIdx.y;
     for (uint32_t c = (blockIdx.x * 256 + threadIdx.x) * 4; c < k; c += gridDim.x * 1024) {
         const float4 v = *(const float4*)(x + (size_t)row * x_stride + c);
@@ -380,8 +380,8 @@ __global__ __launch_bounds__(256) void split_f32_bf16x2_kernel(const float* __re
         uint2 hv, lv;
         hv.x = h[0] | ((uint32_t)h[1] << 16); hv.y = h[2] | ((uint32_t)h[3] << 16);
         lv.x = l[0] | ((uint32_t)l[1] << 16); lv.y = l[2] | ((uint32_t)l[3] << 16);
-        *(uint2*)(hi + (size_t)row * k + c) = hv;
-        *(uint2*)(lo + (size_t)row * k + c) = lv;
+        *(uint2*)(hi + (size_t)row * out_stride + c) = hv;
+        *(uint2*)(lo + (size_t)row * out_stride + c) = lv;
     }
 }
 
@@ -476,11 +476,12 @@ mi355q_status launch_sum_parts_rows(hipStream_t s, const float* yp, uint32_t par
 }
 
 mi355q_status launch_split_f32_bf16x2(hipStream_t s, const float* x, uint32_t m, uint32_t k, uint32_t x_stride, uint16_t* hi,
-                                      uint16_t* lo) {
+                                      uint16_t* lo, uint32_t out_stride) {
+    if (out_stride == 0) out_stride = k;
     if (m > 65535u) return fail(MI355Q_ERR_SHAPE, "more than 65535 activation rows");
     uint32_t gx = (k / 4 + 255) / 256;
     if (gx > 64) gx = 64;
-    split_f32_bf16x2_kernel<<<dim3(gx, m), dim3(256), 0, s>>>(x, m, k, x_stride, hi, lo);
+    split_f32_bf16x2_kernel<<<dim3(gx, m), dim3(256), 0, s>>>(x, m, k, x_stride, hi, lo, out_stride);
     MI355Q_HIP(hipGetLastError());
     return MI355Q_OK;
 }

@@ -329,8 +329,9 @@ mi355q_status mi355q_plan_prefill_steps(const mi355q_weight* w, uint32_t maximum
         std::snprintf(s->kernel_family, sizeof s->kernel_family, "mfmaGEMM");
         const bool wide = gemm_wide_taken(v, x_dtype, m, input_row_stride, flags);
         if (wide)
-            std::snprintf(s->device_kernel, sizeof s->device_kernel, "qgemm_wide_q%u_g%u", (unsigned)w->fmt.bits, w->fmt.group_size);
-        const GemmLaunchShape g = wide ? gemm_wide_shape(m, (uint32_t)w->n, (uint32_t)w->k)
+            std::snprintf(s->device_kernel, sizeof s->device_kernel, "%sqgemm_wide_q%u_g%u", x_dtype == MI355Q_F32 ? "split_f32_bf16x2+" : "",
+                          (unsigned)w->fmt.bits, w->fmt.group_size);
+        const GemmLaunchShape g = wide ? gemm_wide_shape(m, (uint32_t)w->n, gemm_wide_k((uint32_t)w->k, x_dtype))
                                        : gemm_mfma_shape(w->ctx, m, (uint32_t)w->n, (uint32_t)w->k);
         s->block[0] = g.block;
         s->grid[0] = g.grid;

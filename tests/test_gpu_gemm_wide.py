@@ -69,7 +69,8 @@ def _seeded(pkg, ctx, seed, m, n, k, group, flags, sample=None, x_pad=0, y_pad=0
     layout = pkg.LAYOUT_PLANES if layout is None else layout
     x_dtype = pkg.BF16 if x_dtype is None else x_dtype
     words, s, z, wq = seeded_case(seed, n, k, 4, group)
-    wb = bf16_round(wq) if x_dtype == pkg.BF16 else wq.astype(np.float16).astype(np.float32)
+    # fp32 activations meet bf16 weights, as in the reference's gemm_bf16_f32s
+    wb = wq.astype(np.float16).astype(np.float32) if x_dtype == pkg.F16 else bf16_round(wq)
     fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, group)
     w = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, layout)
     x = np.zeros((m, k + x_pad), np.float32)
@@ -146,18 +147,39 @@ def test_wide_gemm_blocks_and_f16_seeded_against_the_oracle(pkg, ctx):
             w.destroy()
 
 
-@pytest.mark.parametrize("layout_name,x_name", [("LAYOUT_STAF_BLOCKS", "BF16"), ("LAYOUT_PLANES", "F16"), ("LAYOUT_STAF_BLOCKS", "F16")])
+def test_wide_gemm_fp32_activations(pkg, ctx):
+    """fp32 activations (the reference's prefill type, gemm_q4_g*_f32s): every row is split into [hi | lo] bf16 halves
+    that carry sixteen bits of it, and the kernel walks 2 K against the weights twice; planes and blocks in place, K in
+    parts, against the fp64 product of bf16 weights and the fp32 activations."""
+    for i, (m, n, k, group, layout) in enumerate([(257, 300, 512, 64, pkg.LAYOUT_PLANES), (130, 515, 768, 128, pkg.LAYOUT_STAF_BLOCKS),
+                                                   (300, 264, 2304, 64, pkg.LAYOUT_PLANES)]):
+        w, x, got, _ = _seeded(pkg, ctx, 4800 + i, m, n, k, group, wide(pkg), layout=layout, x_dtype=pkg.F32)
+        step = w.plan_prefill_steps(m, x_dtype=pkg.F32, flags=wide(pkg))[0]
+        assert step.device_kernel == f"split_f32_bf16x2+qgemm_wide_q4_g{group}" and step.kernel_family == "mfmaGEMM"
+        if i == 2:
+            pkg.Context.probe_wide_shape(256, 3)
+            try:
+                parts = run_qgemm(ctx, pkg, w, x, pkg.F32, wide(pkg), x_dtype=pkg.F32)
+            finally:
+                pkg.Context.probe_wide_shape(0, 0)
+            assert np.max(np.abs(parts - got)) <= 2e-5 * max(1.0, float(np.max(np.abs(got))))
+        w.destroy()
+
+
+@pytest.mark.parametrize("layout_name,x_name", [("LAYOUT_STAF_BLOCKS", "BF16"), ("LAYOUT_PLANES", "F16"), ("LAYOUT_STAF_BLOCKS", "F16"),
+                                                ("LAYOUT_PLANES", "F32")])
 @pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
 def test_config3_on_blocks_and_f16_as_dispatched(pkg, ctx, layout_name, x_name, n, k):
-    """benchmark config 3 at M = 2048 on the reference's block layout and with its f16 activations, no flags: the
-    plan names this library's matrix-core kernel, and the result holds the bar on the tile-edge column sample."""
+    """benchmark config 3 at M = 2048 on the reference's block layout and with its f16 and fp32 activations, no flags:
+    the plan names this library's matrix-core kernel, and the result holds the bar on the tile-edge column sample."""
     m = 2048
     layout, x_dtype = getattr(pkg, layout_name), getattr(pkg, x_name)
     sample = _tile_edge_sample(n, 31 * m + n, tile=256)
     w, _, _, (rel, _) = _seeded(pkg, ctx, 4700, m, n, k, 64, 0, sample=sample, layout=layout, x_dtype=x_dtype)
     steps = w.plan_prefill_steps(m, x_dtype=x_dtype)
     say("as dispatched:", [s.device_kernel for s in steps])
-    assert len(steps) == 1 and steps[0].device_kernel == "qgemm_wide_q4_g64" and steps[0].kernel_family == "mfmaGEMM"
+    assert len(steps) == 1 and steps[0].device_kernel.endswith("qgemm_wide_q4_g64") and steps[0].kernel_family == "mfmaGEMM"
+    assert steps[0].device_kernel.startswith("split_f32_bf16x2+") == (x_dtype == pkg.F32)
     assert not steps[0].used_fallback
     assert rel < 5e-4
     w.destroy()

@@ -25,7 +25,7 @@ FLAG_SETS = {"none": 0, "mfma": pkg.FLAG_FORCE_MFMA, "two-step": pkg.FLAG_FORCE_
 PLAN_OF_ROUTE = {
     "two-step": r"^dequant_q\d_g\d+_(bf16|f16|f32)\+hipblaslt_gemm_(bf16|f16|f32)(_x2)?$",
     "stream": r"^qgemm_stream_q\d_g\d+$",
-    "fused/wide": r"^qgemm_wide_q\d_g\d+$",
+    "fused/wide": r"^(split_f32_bf16x2\+)?qgemm_wide_q\d_g\d+$",
     "fused/tiled": r"^qgemm_mfma_q\d_g\d+$",
     "small-batch/tile16": r"^gemv_tile16_q\d_g\d+$",
     "small-batch/mfma-planes": r"^gemv_mfma_planes_q\d_g\d+$",
@@ -133,7 +133,7 @@ def test_config_routes():
     assert r(q4, P, 4096, 4096, pkg.BF16, 3, decode_entry=True) == "small-batch/dot-planes"       # small matrix: rows kernel
     assert r(q4, P, 14336, 4096, pkg.BF16, 64) == "stream"
     assert r(q4, P, 14336, 4096, pkg.BF16, 128) == "fused/tiled"
-    for layout, xd in ((P, pkg.BF16), (B, pkg.BF16), (P, pkg.F16), (B, pkg.F16)):
+    for layout, xd in ((P, pkg.BF16), (B, pkg.BF16), (P, pkg.F16), (B, pkg.F16), (P, pkg.F32), (B, pkg.F32)):
         assert r(q4, layout, 14336, 4096, xd, 2048) == "fused/wide"
         assert r(q4, layout, 4096, 14336, xd, 2048) == "fused/wide"
         assert r(q4, layout, 14336, 4096, xd, 4096) == "two-step"
