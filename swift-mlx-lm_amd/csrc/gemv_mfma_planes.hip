@@ -62,7 +62,14 @@ struct PmArgs {
     uint32_t parts;                            // K parts, each with workgroups of its own that stage only their columns
     uint32_t part_blocks;                      // blocks per part
     float* partial;                            // K parts only: fp32 partial results [part][M][N] (one matrix)
+#ifdef MI355Q_GEMV_TIMELINE
+    unsigned long long* timeline;              // measurement build only: 100 MHz time stamps per workgroup
+#endif
 };
+
+#ifdef MI355Q_GEMV_TIMELINE
+extern unsigned long long* g_gemv_timeline;
+#endif
 
 // BITS, GROUP: 4 with 64 or 128, 8 with 32, 64 or 128 (a group of two blocks: both blocks apply the group's word).  A workgroup of KSPLIT * TPW wavefronts covers TPW consecutive row tiles, each split over KSPLIT
 // wavefronts along K; all of them share one staged copy of the activations.
@@ -84,6 +91,10 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
     constexpr int MR = 4;
     extern __shared__ u32x4 smem_pm[];
     char* lds = (char*)smem_pm;
+#ifdef MI355Q_GEMV_TIMELINE
+    const unsigned long long tl_entry = __builtin_amdgcn_s_memrealtime();
+    unsigned long long tl_staged = 0, tl_first = 0, tl_loop = 0;
+#endif
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t n_in = lane & 15, kq = lane >> 4;
@@ -191,9 +202,11 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
             p = pm_dot2(v.y, 0x3F803F80u, p);
             p = pm_dot2(v.z, 0x3F803F80u, p);
             p = pm_dot2(v.w, 0x3F803F80u, p);
-            p += __shfl_xor(p, 1);
-            p += __shfl_xor(p, 2);
-            if constexpr (CH == 8) p += __shfl_xor(p, 4);
+            // over the CH consecutive lanes of a half block, inside the vector unit (lane pairs, quads, then the mirror
+            // image inside eight lanes: every lane of a quad holds the quad's sum by then)
+            p += dpp_f32<0xB1>(p);                           // quad_perm [1,0,3,2]
+            p += dpp_f32<0x4E>(p);                           // quad_perm [2,3,0,1]
+            if constexpr (CH == 8) p += dpp_f32<0x141>(p);   // row_half_mirror
             return p;
         };
         // one chunk of a staged row: every run of eight in the operand order of the unpacked codes, and its share of sum(x)
@@ -246,6 +259,15 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+#ifdef MI355Q_GEMV_TIMELINE
+    tl_staged = __builtin_amdgcn_s_memrealtime();
+    {   // when the first weight words of this wavefront are there
+        uint32_t first_word = ring[0].w.x;
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(first_word));
+        ring[0].w.x = first_word;
+        tl_first = __builtin_amdgcn_s_memrealtime();
+    }
+#endif
 
     // ---- 4. K loop --------------------------------------------------------------------------------------------------
     uint32_t k_mask = 0x000F000Fu, k_magic = 0x43004300u;   // opaque: keeps (w & mask) | magic one v_and_or_b32
@@ -434,6 +456,9 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
             });
         }
 
+#ifdef MI355Q_GEMV_TIMELINE
+        if (pass + 1 == a.passes) tl_loop = __builtin_amdgcn_s_memrealtime();
+#endif
         // ---- 5. add the partial tiles of the wavefronts that share a row tile, store ---------------------------------
         if (red_over_x) __syncthreads();
 #pragma unroll
@@ -471,6 +496,15 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_mfma_planes_kernel(PmA
         }
         if (pass + 1 < a.passes) __syncthreads();           // the partial tiles are read before the next pass overwrites them
     }
+#ifdef MI355Q_GEMV_TIMELINE
+    if (a.timeline && wave == 0 && lane == 0) {
+        unsigned long long* const t = a.timeline + ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 6;
+        uint32_t hw_id;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw_id));
+        t[0] = tl_entry; t[1] = tl_staged; t[2] = tl_first; t[3] = __builtin_amdgcn_s_memrealtime();
+        t[4] = hw_id; t[5] = tl_loop;
+    }
+#endif
 }
 
 // Sum of the K parts, in part order, then the conversion the single-launch form does in its epilogue.
@@ -592,6 +626,9 @@ mi355q_status launch_gemv_mfma_planes_multi(hipStream_t s, mi355q_context* ctx, 
         a.partial = (float*)ctx->workspace;
     }
     a.y_dtype = (uint32_t)y_dtype; a.sb_dtype = w[0].sb_dtype;
+#ifdef MI355Q_GEMV_TIMELINE
+    a.timeline = g_gemv_timeline;
+#endif
     const mi355q_status st = w[0].bits == 4 ? (w[0].group == 64 ? launch_pm_shape<4, 64>(s, a, g) : launch_pm_shape<4, 128>(s, a, g))
                                             : (w[0].group == 32 ? launch_pm_shape<8, 32>(s, a, g)
                                                : w[0].group == 64 ? launch_pm_shape<8, 64>(s, a, g) : launch_pm_shape<8, 128>(s, a, g));

@@ -153,7 +153,7 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
 
     // ---- 3. stage the activations (waits only for the loads of step 1) --------------------------
     // With each 16-byte chunk goes its share of sum(x): eight consecutive lanes hold the eight chunks of one
-    // 64-element group of one row, so three xor-shuffles give the group sum, kept as sxs[group][row].
+    // 64-element group of one row, so three cross-lane adds give the group sum, kept as sxs[group][row].
     float* const sxs = (float*)(lds + (size_t)a.ms * a.lds_row_bytes);
     {
         const uint32_t total = a.m * chunks;
@@ -162,9 +162,9 @@ __global__ __launch_bounds__(KSPLIT * TPW * 64) void gemv_tile16_kernel(T16Args 
             p = t16_dot2(v.y, 0x3F803F80u, p);
             p = t16_dot2(v.z, 0x3F803F80u, p);
             p = t16_dot2(v.w, 0x3F803F80u, p);
-            p += __shfl_xor(p, 1);
-            p += __shfl_xor(p, 2);
-            p += __shfl_xor(p, 4);
+            p += dpp_f32<0xB1>(p);     // lane pairs (quad_perm [1,0,3,2]), quads ([2,3,0,1]), then the mirror image inside
+            p += dpp_f32<0x4E>(p);     // eight lanes (every lane of a quad holds the quad's sum by then): no trip through
+            p += dpp_f32<0x141>(p);    // LDS, an instruction each
             return p;
         };
         auto stage = [&](uint32_t idx, const u32x4& v) {

@@ -6,9 +6,11 @@ hardware ids of the CU it ran on.  The product library carries none of this.  Pr
 layer (fused gate+up, down, fused q+k+v, o): how workgroups enter over time, how long each waits for its
 activations and its first weights, how many are resident over time, and bytes delivered per phase.
 
-    python swift-mlx-lm_amd/decode_timeline.py [--rows-per-wave R --rows-per-pass B]
+    python swift-mlx-lm_amd/decode_timeline.py [--rows-per-wave R --rows-per-pass B] [--rows M]
 
-The two options override the launch shape of the rows kernel (measurement build only) for a sweep.
+The first two options override the launch shape of the rows kernel (measurement build only) for a sweep.  --rows M
+(5 .. 16) times the small-batch matrix-core kernel on M activation rows instead; its stamps are entry, activations
+staged (behind the barrier), first weight words there, end of the K loop, exit.
 """
 import argparse
 import ctypes as C
@@ -39,6 +41,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--rows-per-wave", type=int, default=0)
     ap.add_argument("--rows-per-pass", type=int, default=0)
+    ap.add_argument("--rows", type=int, default=1, help="activation rows of the launch")
     ap.add_argument("--brief", action="store_true", help="one line per launch")
     a = ap.parse_args()
     if a.rows_per_wave:
@@ -68,15 +71,15 @@ def main():
     for name, mats in shapes.items():
         ws = [[weight(n, k) for n, k in mats] for _ in range(copies)]
         k = mats[0][1]
-        x = ctx.upload(bf16_bits(rng.standard_normal((1, k)).astype(np.float32)))
-        ys = [ctx.alloc(n * 2) for n, _ in mats]
+        x = ctx.upload(bf16_bits(rng.standard_normal((a.rows, k)).astype(np.float32)))
+        ys = [ctx.alloc(a.rows * n * 2) for n, _ in mats]
         stream = ctx.stream_create()
 
         def launch(i):
             if len(mats) == 1:
-                ctx.qgemv(ws[i % copies][0], x, pkg.BF16, ys[0], pkg.BF16, 1, 0, 0, 0, stream)
+                ctx.qgemv(ws[i % copies][0], x, pkg.BF16, ys[0], pkg.BF16, a.rows, 0, 0, 0, stream)
             else:
-                ctx.batched_qgemm(ws[i % copies], x, pkg.BF16, ys, pkg.BF16, 1, 0, 0, stream)
+                ctx.batched_qgemm(ws[i % copies], x, pkg.BF16, ys, pkg.BF16, a.rows, 0, 0, stream)
 
         L.mi355q_probe_set_timeline(None)
         for i in range(12):
@@ -101,7 +104,7 @@ def main():
             runs.append(tl.download(np.uint64, (nwg, 6)).copy())
         L.mi355q_probe_set_timeline(None)
         if not all((t[:, 3] > 0).any() for t in runs):
-            print(f"== {name}: no time stamps: this launch shape is served by a kernel other than the rows kernel")
+            print(f"== {name}: no time stamps: this launch shape is served by a kernel that writes none")
             continue
         spans = [float((t[t[:, 3] > 0][:, 3].max() - t[t[:, 3] > 0][:, 0].min()) / 100.0) for t in runs]
         t = runs[int(np.argsort(spans)[len(spans) // 2])]
@@ -115,7 +118,7 @@ def main():
         exit_ = (t[:, 3] - t0) / 100.0
         end = float(exit_.max())
         total_bytes = sum(nn * (kk // 2 + kk // 64 * 4) for nn, kk in mats)
-        step = ws[0][0].plan_decode_step(1)
+        step = ws[0][0].plan_decode_step(a.rows)
         print(f"== {name}: {step.device_kernel}, {n} workgroups of {step.block[0]} threads, {total_bytes / 1e6:.1f} MB of weights; "
               f"{back_to_back:.2f} us a launch back to back; first entry to last exit {end:.2f} us "
               f"(five runs: {', '.join(f'{s:.2f}' for s in spans)})")
@@ -124,6 +127,9 @@ def main():
             print(f"   workgroups entered: 25% by {q(entry, 25):.2f}, 50% by {q(entry, 50):.2f}, 75% by {q(entry, 75):.2f}, all by {entry.max():.2f} us")
             print(f"   entry -> activations staged: median {q(staged, 50):.2f} (10% {q(staged, 10):.2f}, 90% {q(staged, 90):.2f}) us")
             print(f"   entry -> first weight words: median {q(first, 50):.2f} (10% {q(first, 10):.2f}, 90% {q(first, 90):.2f}) us")
+            if a.rows > 1:
+                loop = (t[:, 5] - t[:, 0]) / 100.0
+                print(f"   entry -> end of the K loop:  median {q(loop, 50):.2f} (10% {q(loop, 10):.2f}, 90% {q(loop, 90):.2f}) us")
             print(f"   entry -> exit:               median {q(life, 50):.2f} (10% {q(life, 10):.2f}, 90% {q(life, 90):.2f}) us")
             print(f"   first workgroup to exit leaves at {exit_.min():.2f} us")
             # bytes delivered over time: a workgroup's share of the weights counts as delivered when it exits
