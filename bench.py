@@ -34,6 +34,11 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0    # MI355X published dense bf16 matrix-core peak
 # plain copy of the same size (profiles/gemv_rows_q4_g64_gate_up_pmc_and_hbm_traffic.md).  Measured offline with the
 # profiler: the figure only holds for the kernel and launch shape it was measured on, so it is keyed by both and the
 # line carries null when the library picks anything else.
+# The same for the M = 2048 gate launch of the prefill GEMM (keyed by kernel and grid; FETCH_SIZE 180 400 and WRITE_SIZE
+# 69 080 per dispatch against 16 140 and 32 260 for a copy of 33 030 144 bytes: 369 MB read past the L2s, most of it the
+# activations once per round of column tiles and served by the last-level cache, and 71 MB written;
+# profiles/qgemm_wide_q4_g64_prefill_m2048_kernel_trace_pmc.md).
+PREFILL_TRAFFIC_BYTES = {("qgemm_wide_q4_g64", 448): 369_200_000 + 70_700_000}
 TRAFFIC_BYTES = {("gemv_rows_q4_g64", "gate_up", 3584, 256): 66171661 + 114688, ("gemv_rows_q4_g64", "gate", 1792, 256): 33159518 + 57344}
 
 
@@ -748,7 +753,8 @@ def main():
             f"{prefill['aside_constant_activations_fused_kernel']}")
         best = sweep["gate 4096->14336 M=2048"]
         roofline_prefill = {"bound": "mfma", "achieved": best["TFLOPs"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                            "frac": round(best["TFLOPs"] / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None,
+                            "frac": round(best["TFLOPs"] / MFMA_BF16_PEAK_TFLOPS, 4),
+                            "traffic": PREFILL_TRAFFIC_BYTES.get((best["route"], int(wg.plan_prefill_steps(2048, 4096)[0].grid[0]))),
                             "kernel": best["route"], "m": 2048, "shape": "4096->14336", "us": best["us"],
                             "flops": flops, "activations": "N(0,1) bf16",
                             "timing": "sustained load (see config.prefill_gemm_gate.config3.timing)",
