@@ -54,6 +54,14 @@ MI355Q_API mi355q_status mi355q_probe_route(uint8_t scheme_identifier, uint32_t 
                                             uint32_t flags, int decode_entry, int library_available, char* launcher_out,
                                             char* planner_out, size_t cap);
 
+/* The same for two or three projections that share their activations (mi355q_batched_qgemm, the shared steps of a plan):
+ * what the launcher would run ("shared/<kernel>" for one launch over the rows of all matrices, "split-rows", "steps",
+ * "separate") and the device kernel the plan record of that step names. */
+MI355Q_API mi355q_status mi355q_probe_shared_route(uint8_t scheme_identifier, uint32_t layout, uint32_t sb_dtype, uint32_t count,
+                                                   const uint64_t* n_rows, uint64_t k, mi355q_dtype x_dtype, uint32_t m,
+                                                   uint32_t x_row_stride, uint32_t flags, char* launcher_out,
+                                                   char* planner_out, size_t cap);
+
 #ifdef __cplusplus
 }
 #endif

@@ -47,6 +47,17 @@ def probe_route(fmt, layout, n, k, x_dtype, m, flags=0, decode_entry=False, libr
     return a.value.decode(), b.value.decode()
 
 
+def probe_shared_route(fmt, layout, ns, k, x_dtype, m, flags=0, sb_dtype=None, x_row_stride=0):
+    """The same for two or three projections of ns rows that share their activations: (what mi355q_batched_qgemm would
+    run, the device kernel the plan record of the shared step names)."""
+    a = C.create_string_buffer(128)
+    b = C.create_string_buffer(128)
+    rows = (C.c_uint64 * len(ns))(*ns)
+    _check(library().mi355q_probe_shared_route(fmt.scheme_identifier, layout, BF16 if sb_dtype is None else sb_dtype, len(ns), rows,
+                                               k, x_dtype, m, x_row_stride, flags, a, b, 128))
+    return a.value.decode(), b.value.decode()
+
+
 class MI355QError(RuntimeError):
     def __init__(self, status: int, message: str):
         super().__init__(f"[{STATUS_NAMES.get(status, status)}] {message}")
@@ -194,6 +205,7 @@ def library() -> C.CDLL:
         "mi355q_context_scratch_bytes": (i32, [vp, P(u64)]),
         "mi355q_probe_wide_shape": (None, [u32, u32]),
         "mi355q_probe_route": (i32, [u8, u32, u32, u64, u64, C.c_int, u32, u32, u32, C.c_int, C.c_int, C.c_char_p, C.c_char_p, sz]),
+        "mi355q_probe_shared_route": (i32, [u8, u32, u32, u32, P(u64), u64, C.c_int, u32, u32, u32, C.c_char_p, C.c_char_p, sz]),
         "mi355q_kv_scheme_is_supported": (i32, [u8]),
         "mi355q_kv_bytes_per_head_slot": (u32, [u8, u32]),
         "mi355q_kv_cache_write": (i32, [vp, vp, P(_KvLayout), vp, vp, C.c_int, u32, u32, u32]),

@@ -393,10 +393,6 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
             weights[i]->layout != weights[0]->layout)
             return fail(MI355Q_ERR_SHAPE, "batched projections must share K, scheme and layout");
     }
-    bool fused = m <= 8 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
-    bool tiled = m <= 16 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
-    bool in_place = m <= 8 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
-    bool on_planes = mfma_planes_pays(weights[0]->fmt.bits, x_dtype, m) && m <= 16 && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
     WView views[3];
     uint32_t strides[3];
     for (uint32_t i = 0; i < count; i++) {
@@ -405,38 +401,21 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
         xs = x_stride;
         strides[i] = y_stride;
         views[i] = weights[i]->view();
-        fused = fused && gemv_fast_eligible(views[i], x_dtype, m, xs) && views[i].sb_dtype == views[0].sb_dtype;
-        tiled = tiled && gemv_tile16_eligible(views[i], x_dtype, m, xs) &&
-                gemv_tile16_k_parts(ctx, views[i], staged_rows(x_dtype, m)) == 1 &&
-                views[i].sb_dtype == views[0].sb_dtype;
-        in_place = in_place && gemv_staf_eligible(views[i], x_dtype, m, xs);
-        on_planes = on_planes && gemv_mfma_planes_eligible(views[i], x_dtype, m, xs) &&
-                    gemv_mfma_planes_k_parts(ctx, views[i], staged_rows(x_dtype, m)) == 1 && views[i].sb_dtype == views[0].sb_dtype &&
-                    views[i].code_stride == views[0].code_stride && views[i].group == views[0].group;
     }
-    if (fused && gemv_rows_batch_pays(count, views, x_dtype, m)) on_planes = false;      // small matrices, three or four rows
-    // the streamed-weight kernel, one launch for the two or three matrices: a few dozen rows on 4- / 8-bit planes, and
-    // blocks in place from three to nine rows by the size of the matrices together
-    const bool no_stream = flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_TWO_STEP | MI355Q_FLAG_FORCE_SMALL_M);
-    const bool stream_multi = !no_stream && (uintptr_t)x % 16 == 0 &&
-                              ((flags & MI355Q_FLAG_FORCE_STREAM) ? gemm_stream_multi_eligible(count, views, x_dtype, m, xs)
-                                                                  : gemm_stream_chosen_multi(count, views, x_dtype, m, xs));
-    if (stream_multi) return launch_qgemm_stream_multi(s, ctx, count, views, x, x_dtype, ys, strides, y_dtype, m, xs);
-    if (on_planes && (uintptr_t)x % 16 == 0)
+    switch (shared_route(ctx, count, views, x_dtype, m, xs, flags, (uintptr_t)x % 16 == 0)) {
+    case SharedRoute::kStream:
+        return launch_qgemm_stream_multi(s, ctx, count, views, x, x_dtype, ys, strides, y_dtype, m, xs);
+    case SharedRoute::kMfmaPlanes:
         return launch_gemv_mfma_planes_multi(s, ctx, count, views, x, x_dtype, ys, strides, y_dtype, m, xs);
-    if (fused && (uintptr_t)x % 16 == 0)
+    case SharedRoute::kDotPlanes:
         return launch_gemv_fast_multi(s, ctx, count, views, x, x_dtype, ys, strides, y_dtype, m, xs, nullptr, nullptr, HeadKeys{});
-    if (tiled && (uintptr_t)x % 16 == 0)
+    case SharedRoute::kTile16:
         return launch_gemv_tile16_multi(s, ctx, count, views, x, x_dtype, ys, strides, y_dtype, m, xs, nullptr, nullptr,
                                         HeadKeys{});
-    if (in_place && (uintptr_t)x % 16 == 0)
+    case SharedRoute::kStafInPlace:
         return launch_gemv_staf_multi(s, ctx, count, views, x, x_dtype, ys, strides, y_dtype, m, xs, nullptr, nullptr, HeadKeys{});
-    // fp32 / f16 rows that go to the bf16 kernels as bf16 rows (split_rows_chosen): split once for all projections, one
-    // shared bf16 launch on those rows where they fit one, one sum per projection
-    const uint32_t parts = split_rows_parts(x_dtype);
-    bool split = parts && parts * (uint64_t)m <= 16;
-    for (uint32_t i = 0; i < count && split; i++) split = split_rows_chosen(views[i], x_dtype, m, xs, flags);
-    if (split) {
+    case SharedRoute::kSplitRows: {
+        const uint32_t parts = split_rows_parts(x_dtype);
         const uint32_t k = (uint32_t)views[0].k, kp = split_rows_stride(k);
         const size_t xbytes = ((size_t)parts * m * kp * 2 + 255) & ~(size_t)255;
         size_t ybytes[3] = {0, 0, 0}, total = xbytes;
@@ -454,15 +433,8 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
                                                          strides[i])) return st;
         return MI355Q_OK;
     }
-    // more rows than one shared launch takes, served by the small-batch kernels all the same: the shared launch in steps
-    const uint32_t step = small_batch_rows(views[0], x_dtype, xs);
-    bool stepped = m > step && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_TWO_STEP));
-    for (uint32_t i = 0; i < count && stepped; i++)
-        stepped = decode_kernel_reads(views[i], x_dtype, xs) && !split_rows_chosen(views[i], x_dtype, m, xs, flags) &&
-                  !gemm_two_step_chosen(views[i], x_dtype, m, xs, flags) &&
-                  (m <= small_batch_limit(views[i], x_dtype, xs) ||
-                   !(gemm_mfma_eligible(views[i], x_dtype, m, xs) || gemm_wide_taken(views[i], x_dtype, m, xs, flags)));
-    if (stepped) {
+    case SharedRoute::kSteps: {
+        const uint32_t step = small_batch_rows(views[0], x_dtype, xs);
         const size_t xsz = x_dtype == MI355Q_F32 ? 4 : 2, ysz = y_dtype == MI355Q_F32 ? 4 : 2;
         for (uint32_t m0 = 0; m0 < m; m0 += step) {
             void* yc[3] = {nullptr, nullptr, nullptr};
@@ -471,6 +443,9 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
                                                     y_dtype, m - m0 < step ? m - m0 : step, xs, flags)) return st;
         }
         return MI355Q_OK;
+    }
+    case SharedRoute::kSeparate:
+        break;
     }
     for (uint32_t i = 0; i < count; i++) {
         mi355q_status st = dispatch_linear(ctx, s, weights[i], x, x_dtype, ys[i], y_dtype, m, xs, 0, flags, false);

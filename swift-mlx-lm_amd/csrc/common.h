@@ -287,7 +287,7 @@ mi355q_status dispatch_output_head(mi355q_context* ctx, hipStream_t s, const mi3
                                    int x_dtype, float* logits, int32_t* token, uint32_t flags, HeadKeys keys,
                                    bool no_allocation = false);
 void plan_shared_launch_shape(const mi355q_weight* const* ws, uint32_t count, uint32_t m, int x_dtype, uint32_t x_stride,
-                              mi355q_step* s);
+                              uint32_t flags, mi355q_step* s);
 
 // MFMA GEMM (kernels_gemm.hip)
 struct GemmLaunchShape {
@@ -321,6 +321,22 @@ enum class SmallKernel : int { kTile16 = 0, kMfmaPlanes, kDotPlanes, kStafInPlac
 SmallKernel small_kernel(const WView& v, int x_dtype, uint32_t rows, uint32_t x_stride, uint32_t flags, bool x_aligned);
 const char* small_kernel_name(SmallKernel k);
 uint32_t small_batch_step(const WView& v, int x_dtype, uint32_t m, uint32_t x_stride, uint32_t flags);
+// What two or three projections that share their activations run as (q+k+v, gate+up): one launch over the rows of all
+// matrices on one of five kernels, the rows split first, the shared launch in steps, or a launch per projection.  Asked
+// by dispatch_batched (api.hip), which launches it, and by the planner, which describes it.
+enum class SharedRoute : int {
+    kStream = 0,       // the streamed-weight kernel over the matrices together
+    kMfmaPlanes,       // the small-batch matrix-core kernel over the planes
+    kDotPlanes,        // the dot-product decode kernels over the planes
+    kTile16,           // the matrix-core kernel over TILE16 records
+    kStafInPlace,      // the in-place kernel over the reference's blocks
+    kSplitRows,        // fp32 rows split into bf16 rows once for all projections, then one of the above on those
+    kSteps,            // more rows than one shared launch takes: the shared launch in steps
+    kSeparate,         // each projection on its own route (linear_route)
+};
+SharedRoute shared_route(const mi355q_context* ctx, uint32_t count, const WView* views, int x_dtype, uint32_t m, uint32_t xs,
+                         uint32_t flags, bool x_aligned);
+const char* shared_route_name(SharedRoute r);
 
 // Every entry point that enqueues work opens one of these first.  The context's scratch (partial results, dense
 // copies, split rows, gate / up sums, arg-max keys) is shared by its launches, so they must be ordered: when the scratch

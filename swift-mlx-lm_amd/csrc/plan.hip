@@ -169,7 +169,7 @@ mi355q_status mi355q_plan_add_batched_linear(mi355q_plan* plan, uint32_t count, 
         st.record = two[0];
     }
     if (rc != MI355Q_OK) return rc;
-    if (m <= 8) plan_shared_launch_shape(weights, count, m, x_dtype, st.xs, &st.record);   // one launch over the rows of all matrices
+    plan_shared_launch_shape(weights, count, m, x_dtype, st.xs, flags, &st.record);   // one launch over the rows of all matrices
     std::snprintf(st.record.kernel_family, sizeof st.record.kernel_family, "batched%uQ%uG%u", count,
                   (unsigned)weights[0]->fmt.bits, weights[0]->fmt.group_size);
     plan->steps.push_back(st);
@@ -216,7 +216,7 @@ mi355q_status mi355q_plan_add_gated_mlp(mi355q_plan* plan, const mi355q_weight* 
     }
     if (rc != MI355Q_OK) return rc;
     const mi355q_weight* both[2] = {w_gate, w_up};
-    if (m <= 8) plan_shared_launch_shape(both, 2, m, x_dtype, st.xs, &st.record);
+    plan_shared_launch_shape(both, 2, m, x_dtype, st.xs, flags, &st.record);
     // one launch with the activation as its epilogue, or the batched projection followed by the elementwise kernel
     const bool one_launch = !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_MFMA |
                                        MI355Q_FLAG_FORCE_TWO_STEP | MI355Q_FLAG_FORCE_STREAM)) &&

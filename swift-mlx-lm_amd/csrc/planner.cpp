@@ -151,59 +151,108 @@ void plan_small_m(const mi355q_weight* w, uint32_t m, int x_dtype, uint32_t x_st
 
 namespace mi355q {
 
-// Launch shape of a shared launch (2 or 3 projections, one set of activations): the rows of all matrices together.
+// Launch record of a shared launch (2 or 3 projections, one set of activations), where shared_route() gives the
+// projections one: the rows of all matrices together on the kernel it names.  Other routes leave the record of the
+// first projection as it is.
 void plan_shared_launch_shape(const mi355q_weight* const* ws, uint32_t count, uint32_t m, int x_dtype, uint32_t x_stride,
-                              mi355q_step* s) {
-    WView all = ws[0]->view();
+                              uint32_t flags, mi355q_step* s) {
+    if (count < 2 || count > 3) return;
+    WView views[3];
     uint64_t total = 0;
-    // three rows and more: the matrix-core kernel over the planes takes the rows of all matrices, in 16-row tiles
-    bool on_planes = mfma_planes_pays(all.bits, x_dtype, m) && m <= 16;
-    uint32_t tiles = 0;
-    for (uint32_t i = 0; i < count && on_planes; i++) {
-        const WView v = ws[i]->view();
-        on_planes = gemv_mfma_planes_eligible(v, x_dtype, m, x_stride) &&
-                    gemv_mfma_planes_k_parts(ws[0]->ctx, v, staged_rows(x_dtype, m)) == 1 &&
-                    v.sb_dtype == all.sb_dtype && v.code_stride == all.code_stride && v.group == all.group && v.bits == all.bits;
-        tiles += (v.n + 15) / 16;
+    uint32_t tiles = 0, row_blocks = 0;
+    for (uint32_t i = 0; i < count; i++) {
+        views[i] = ws[i]->view();
+        total += views[i].n;
+        tiles += (views[i].n + 15) / 16;
+        row_blocks += (views[i].n + 63) / 64;
     }
-    if (on_planes && m <= 4) {                               // small matrices at three or four rows: the dot-product rows kernel
-        WView views[3];
-        bool fast = count <= 3;
-        for (uint32_t i = 0; i < count && fast; i++) {
-            views[i] = ws[i]->view();
-            fast = gemv_fast_eligible(views[i], x_dtype, m, x_stride) && views[i].sb_dtype == all.sb_dtype;
-        }
-        if (fast && gemv_rows_batch_pays(count, views, x_dtype, m)) on_planes = false;
+    if (total > 0xFFFFFFFFull) return;
+    const mi355q_context* const ctx = ws[0]->ctx;
+    const unsigned bits = (unsigned)ws[0]->fmt.bits, group = ws[0]->fmt.group_size;
+    switch (shared_route(ctx, count, views, x_dtype, m, x_stride, flags, true)) {
+    case SharedRoute::kStream: {
+        const StreamLaunchShape g = gemm_stream_shape_blocks(ctx, m, row_blocks, views[0].k);
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "qgemm_stream_q%u_g%u", bits, group);
+        s->grid[0] = g.row_blocks;
+        s->grid[1] = g.parts;
+        s->block[0] = 768;
+        s->lds_bytes = g.lds_bytes;
+        s->rows_per_workgroup = 64;
+        return;
     }
-    if (on_planes) {
-        const Tile16LaunchShape g = gemv_mfma_planes_shape(ws[0]->ctx, tiles, all.k, all.bits, staged_rows(x_dtype, m));
+    case SharedRoute::kMfmaPlanes: {
+        const Tile16LaunchShape g = gemv_mfma_planes_shape(ctx, tiles, views[0].k, views[0].bits, staged_rows(x_dtype, m));
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_mfma_planes_q%u_g%u", bits, group);
         s->grid[0] = g.wgs_per_part;
         s->grid[1] = g.parts;
         s->block[0] = g.block;
         s->lds_bytes = g.lds_bytes;
         s->rows_per_workgroup = 16 * g.tiles_per_wg * g.passes;
-        std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_mfma_planes_q%u_g%u", (unsigned)ws[0]->fmt.bits,
-                      ws[0]->fmt.group_size);
         return;
     }
-    for (uint32_t i = 0; i < count; i++) {
-        const WView v = ws[i]->view();
-        if (v.layout != MI355Q_LAYOUT_PLANES || !gemv_fast_eligible(v, x_dtype, m > 8 ? 8 : m, x_stride)) return;
-        total += v.n;
+    case SharedRoute::kDotPlanes: {
+        WView all = views[0];
+        all.n = (uint32_t)total;
+        const GemvLaunchShape g = gemv_fast_shape(ctx, all, m, x_dtype);
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "%s_q%u_g%u",
+                      std::strcmp(g.kernel, "gemv_rows_kernel") == 0 ? "gemv_rows" : "gemv_planes", bits, group);
+        s->grid[0] = g.grid;
+        s->block[0] = g.block;
+        s->lds_bytes = g.lds_bytes;
+        s->rows_per_workgroup = g.rows_per_workgroup;
+        return;
     }
-    if (m > 8 || total > 0xFFFFFFFFull) return;
-    all.n = (uint32_t)total;
-    const GemvLaunchShape g = gemv_fast_shape(ws[0]->ctx, all, m, x_dtype);
-    s->grid[0] = g.grid;
-    s->block[0] = g.block;
-    s->lds_bytes = g.lds_bytes;
-    s->rows_per_workgroup = g.rows_per_workgroup;
-    std::snprintf(s->device_kernel, sizeof s->device_kernel, "%s_q%u_g%u",
-                  std::strcmp(g.kernel, "gemv_rows_kernel") == 0 ? "gemv_rows" : "gemv_planes", (unsigned)ws[0]->fmt.bits,
-                  ws[0]->fmt.group_size);
+    case SharedRoute::kTile16: {
+        const Tile16LaunchShape g = gemv_tile16_shape(ctx, tiles, views[0].k, staged_rows(x_dtype, m));
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_tile16_q%u_g%u", bits, group);
+        s->grid[0] = g.grid;
+        s->block[0] = g.block;
+        s->lds_bytes = g.lds_bytes;
+        s->rows_per_workgroup = 16;
+        return;
+    }
+    case SharedRoute::kStafInPlace: {
+        WView all = views[0];
+        all.n = (uint32_t)total;
+        const GemvLaunchShape g = gemv_staf_shape(ctx, all, m);
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_staf_q%u_g%u", bits, group);
+        s->grid[0] = g.grid;
+        s->block[0] = g.block;
+        s->lds_bytes = g.lds_bytes;
+        s->rows_per_workgroup = g.rows_per_workgroup;
+        return;
+    }
+    default:
+        return;
+    }
 }
 
 }  // namespace mi355q
+
+namespace {
+// A weight handle that describes a tensor without holding one (aligned addresses that are never read), on a context
+// of 256 CUs: enough for the route table and the planner.
+void synthetic_weight(mi355q_context* ctx, mi355q_weight* w, const mi355q_format* f, uint32_t layout, uint32_t sb_dtype,
+                      uint64_t n_rows, uint64_t k, bool library_available) {
+    std::memset((void*)ctx, 0, sizeof *ctx);
+    ctx->props.multiProcessorCount = 256;
+    ctx->dense_library_forbidden = !library_available;
+    std::memset((void*)w, 0, sizeof *w);
+    w->ctx = ctx;
+    w->fmt = *f;
+    w->n = n_rows; w->k = k;
+    w->layout = (uint8_t)layout;
+    w->sb_dtype = layout == MI355Q_LAYOUT_STAF_BLOCKS ? (uint8_t)MI355Q_F16 : (uint8_t)sb_dtype;
+    uint32_t* const fake = (uint32_t*)(uintptr_t)0x10000000;     // aligned, never read
+    const uint32_t wpr = (uint32_t)(k * f->bits / 32), bpr = (uint32_t)(k / f->group_size);
+    if (layout == MI355Q_LAYOUT_STAF_BLOCKS) w->blocks = fake;
+    else if (layout == MI355Q_LAYOUT_TILE16) w->tiles = fake;
+    else {
+        w->codes = fake; w->sz = fake + wpr; w->scales = fake; w->biases = fake;
+        w->code_stride = w->sz_stride = (wpr + bpr + 3u) & ~3u;
+    }
+}
+}  // namespace
 
 extern "C" {
 
@@ -374,24 +423,8 @@ mi355q_status mi355q_probe_route(uint8_t scheme_identifier, uint32_t layout, uin
         return fail(MI355Q_ERR_UNSUPPORTED_FORMAT, "TILE16 holds q4 g64 with K %% 128 == 0");
     if (x_row_stride == 0) x_row_stride = (uint32_t)k;
     mi355q_context ctx;
-    std::memset((void*)&ctx, 0, sizeof ctx);
-    ctx.props.multiProcessorCount = 256;
-    ctx.dense_library_forbidden = !library_available;
     mi355q_weight w;
-    std::memset((void*)&w, 0, sizeof w);
-    w.ctx = &ctx;
-    w.fmt = *f;
-    w.n = n_rows; w.k = k;
-    w.layout = (uint8_t)layout;
-    w.sb_dtype = layout == MI355Q_LAYOUT_STAF_BLOCKS ? (uint8_t)MI355Q_F16 : (uint8_t)sb_dtype;
-    uint32_t* const fake = (uint32_t*)(uintptr_t)0x10000000;     // aligned, never read
-    const uint32_t wpr = (uint32_t)(k * f->bits / 32), bpr = (uint32_t)(k / f->group_size);
-    if (layout == MI355Q_LAYOUT_STAF_BLOCKS) w.blocks = fake;
-    else if (layout == MI355Q_LAYOUT_TILE16) w.tiles = fake;
-    else {
-        w.codes = fake; w.sz = fake + wpr; w.scales = fake; w.biases = fake;
-        w.code_stride = w.sz_stride = (wpr + bpr + 3u) & ~3u;
-    }
+    synthetic_weight(&ctx, &w, f, layout, sb_dtype, n_rows, k, library_available != 0);
     const WView v = w.view();
     RouteFacts facts{};
     facts.decode_entry = decode_entry != 0;
@@ -423,6 +456,42 @@ mi355q_status mi355q_probe_route(uint8_t scheme_identifier, uint32_t layout, uin
     size_t at = 0;
     for (uint32_t i = 0; i < count && at < cap; i++)
         at += (size_t)std::snprintf(planner_out + at, cap - at, "%s%s", i ? "+" : "", steps[i].device_kernel);
+    return MI355Q_OK;
+}
+
+// The same for two or three projections that share their activations (q+k+v, gate+up): what dispatch_batched would run
+// (shared_route) and the device kernel the plan record of the shared launch names.
+mi355q_status mi355q_probe_shared_route(uint8_t scheme_identifier, uint32_t layout, uint32_t sb_dtype, uint32_t count,
+                                        const uint64_t* n_rows, uint64_t k, mi355q_dtype x_dtype, uint32_t m,
+                                        uint32_t x_row_stride, uint32_t flags, char* launcher_out, char* planner_out, size_t cap) {
+    const mi355q_format* f = find_format_scheme(scheme_identifier);
+    if (!f) return fail(MI355Q_ERR_UNSUPPORTED_FORMAT, "unsupported scheme 0x%02x", scheme_identifier);
+    if (!launcher_out || !planner_out || cap < 16 || !n_rows) return fail(MI355Q_ERR_INVALID_ARGUMENT, "output buffers");
+    if (count != 2 && count != 3) return fail(MI355Q_ERR_INVALID_ARGUMENT, "two or three projections");
+    if (!k || k % f->group_size) return fail(MI355Q_ERR_SHAPE, "K must be a whole number of groups");
+    if (layout != MI355Q_LAYOUT_STAF_BLOCKS && (k * f->bits) % 32) return fail(MI355Q_ERR_SHAPE, "planes need whole words per row");
+    if (layout == MI355Q_LAYOUT_TILE16 && (f->bits != 4 || f->group_size != 64 || k % 128))
+        return fail(MI355Q_ERR_UNSUPPORTED_FORMAT, "TILE16 holds q4 g64 with K %% 128 == 0");
+    if (x_row_stride == 0) x_row_stride = (uint32_t)k;
+    mi355q_context ctx;
+    mi355q_weight w[3];
+    const mi355q_weight* ws[3] = {&w[0], &w[1], &w[2]};
+    WView views[3];
+    for (uint32_t i = 0; i < count; i++) {
+        if (!n_rows[i]) return fail(MI355Q_ERR_SHAPE, "empty projection");
+        synthetic_weight(&ctx, &w[i], f, layout, sb_dtype, n_rows[i], k, true);
+        views[i] = w[i].view();
+    }
+    const SharedRoute r = shared_route(&ctx, count, views, x_dtype, m, x_row_stride, flags, true);
+    std::snprintf(launcher_out, cap, "%s", shared_route_name(r));
+    mi355q_step steps[2];
+    uint32_t n_steps = 0;
+    mi355q_status st;
+    if (m <= 8) { st = mi355q_plan_decode_step(&w[0], m, x_dtype, flags, &steps[0]); n_steps = 1; }
+    else st = mi355q_plan_prefill_steps(&w[0], m, x_row_stride, x_dtype, 0, flags, steps, &n_steps);
+    if (st != MI355Q_OK || !n_steps) { std::snprintf(planner_out, cap, "error"); return MI355Q_OK; }
+    plan_shared_launch_shape(ws, count, m, x_dtype, x_row_stride, flags, &steps[0]);
+    std::snprintf(planner_out, cap, "%s", steps[0].device_kernel);
     return MI355Q_OK;
 }
 

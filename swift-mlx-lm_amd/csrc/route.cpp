@@ -82,6 +82,68 @@ uint32_t small_batch_step(const WView& v, int x_dtype, uint32_t m, uint32_t xs, 
     return step ? step : 1;
 }
 
+SharedRoute shared_route(const mi355q_context* ctx, uint32_t count, const WView* views, int x_dtype, uint32_t m, uint32_t xs,
+                         uint32_t flags, bool x_aligned) {
+    // a forced route is each projection's own affair (honoured or refused there), except the streamed-weight kernel
+    // where it takes the matrices together
+    if (flags & MI355Q_FLAG_FORCE_TWO_STEP) return SharedRoute::kSeparate;
+    if (flags & MI355Q_FLAG_FORCE_STREAM)
+        return x_aligned && gemm_stream_multi_eligible(count, views, x_dtype, m, xs) ? SharedRoute::kStream : SharedRoute::kSeparate;
+    const bool decode_kernels = !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA));
+    bool fused = m <= 8 && decode_kernels, tiled = m <= 16 && decode_kernels, in_place = m <= 8 && decode_kernels;
+    bool on_planes = mfma_planes_pays(views[0].bits, x_dtype, m) && m <= 16 && decode_kernels;
+    for (uint32_t i = 0; i < count; i++) {
+        const WView& v = views[i];
+        fused = fused && gemv_fast_eligible(v, x_dtype, m, xs) && v.sb_dtype == views[0].sb_dtype;
+        tiled = tiled && gemv_tile16_eligible(v, x_dtype, m, xs) && gemv_tile16_k_parts(ctx, v, staged_rows(x_dtype, m)) == 1 &&
+                v.sb_dtype == views[0].sb_dtype;
+        in_place = in_place && gemv_staf_eligible(v, x_dtype, m, xs);
+        on_planes = on_planes && gemv_mfma_planes_eligible(v, x_dtype, m, xs) &&
+                    gemv_mfma_planes_k_parts(ctx, v, staged_rows(x_dtype, m)) == 1 && v.sb_dtype == views[0].sb_dtype &&
+                    v.code_stride == views[0].code_stride && v.group == views[0].group;
+    }
+    if (fused && gemv_rows_batch_pays(count, views, x_dtype, m)) on_planes = false;      // small matrices, three or four rows
+    // the streamed-weight kernel, one launch for the two or three matrices: a few dozen rows on 4- / 8-bit planes, and
+    // blocks in place from three to nine rows by the size of the matrices together
+    const bool no_stream = flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_SMALL_M);
+    if (!no_stream && x_aligned && gemm_stream_chosen_multi(count, views, x_dtype, m, xs)) return SharedRoute::kStream;
+    if (x_aligned) {
+        if (on_planes) return SharedRoute::kMfmaPlanes;
+        if (fused) return SharedRoute::kDotPlanes;
+        if (tiled) return SharedRoute::kTile16;
+        if (in_place) return SharedRoute::kStafInPlace;
+    }
+    // fp32 rows that go to the bf16 kernels as bf16 rows (split_rows_chosen): split once for all projections, one
+    // shared bf16 launch on those rows where they fit one, one sum per projection
+    const uint32_t parts = split_rows_parts(x_dtype);
+    bool split = parts && parts * (uint64_t)m <= 16;
+    for (uint32_t i = 0; i < count && split; i++) split = split_rows_chosen(views[i], x_dtype, m, xs, flags);
+    if (split) return SharedRoute::kSplitRows;
+    // more rows than one shared launch takes, served by the small-batch kernels all the same: the shared launch in steps
+    const uint32_t step = small_batch_rows(views[0], x_dtype, xs);
+    bool stepped = m > step && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_TWO_STEP));
+    for (uint32_t i = 0; i < count && stepped; i++)
+        stepped = decode_kernel_reads(views[i], x_dtype, xs) && !split_rows_chosen(views[i], x_dtype, m, xs, flags) &&
+                  !gemm_two_step_chosen(views[i], x_dtype, m, xs, flags) &&
+                  (m <= small_batch_limit(views[i], x_dtype, xs) ||
+                   !(gemm_mfma_eligible(views[i], x_dtype, m, xs) || gemm_wide_taken(views[i], x_dtype, m, xs, flags)));
+    return stepped ? SharedRoute::kSteps : SharedRoute::kSeparate;
+}
+
+const char* shared_route_name(SharedRoute r) {
+    switch (r) {
+    case SharedRoute::kStream: return "shared/stream";
+    case SharedRoute::kMfmaPlanes: return "shared/mfma-planes";
+    case SharedRoute::kDotPlanes: return "shared/dot-planes";
+    case SharedRoute::kTile16: return "shared/tile16";
+    case SharedRoute::kStafInPlace: return "shared/staf-in-place";
+    case SharedRoute::kSplitRows: return "split-rows";
+    case SharedRoute::kSteps: return "steps";
+    case SharedRoute::kSeparate: return "separate";
+    }
+    return "?";
+}
+
 const char* small_kernel_name(SmallKernel k) {
     switch (k) {
     case SmallKernel::kTile16: return "tile16";

@@ -165,3 +165,38 @@ def test_plan_with_batched_steps_replays_identically(pkg, ctx):
         b.free()
     for w in qkv + gu:
         w.destroy()
+
+
+def test_plan_records_of_shared_steps_name_the_kernel_that_runs(pkg, ctx):
+    """The record of a shared step names the kernel of the one launch over all matrices (launcher and planner ask the
+    same function): the dot-product, matrix-core, TILE16, in-place and streamed-weight kernels by layout and rows, and
+    the replayed step equals the eager call."""
+    k, ns = 1024, (1024, 256, 256)
+    cases = [(pkg.LAYOUT_PLANES, 1, r"gemv_(rows|planes)_q4_g64"), (pkg.LAYOUT_PLANES, 8, "gemv_mfma_planes_q4_g64"),
+             (pkg.LAYOUT_PLANES, 32, "qgemm_stream_q4_g64"), (pkg.LAYOUT_TILE16, 16, "gemv_tile16_q4_g64"),
+             (pkg.LAYOUT_STAF_BLOCKS, 2, "gemv_staf_q4_g64"), (pkg.LAYOUT_STAF_BLOCKS, 32, "qgemm_stream_q4_g64")]
+    import re
+    for layout, m, want in cases:
+        ws, _ = _prepare(pkg, ctx, 1900 + m, ns, k, 4, 64, layout)
+        fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+        route, planned = pkg.probe_shared_route(fmt, layout, ns, k, pkg.BF16, m)
+        x = ctx.upload(oracle.bf16_from_f32(kat.seeded_activations(1910 + m, m, k)))
+        ys = [ctx.alloc(m * n * 4) for n in ns]
+        ctx.batched_qgemm(ws, x, pkg.BF16, ys, pkg.F32, m)
+        ctx.synchronize()
+        eager = [y.download(np.float32) for y in ys]
+        plan = pkg.DispatchPlan(ctx)
+        plan.add_batched_linear(ws, x, pkg.BF16, ys, pkg.F32, m)
+        st, _, _ = plan.step(0)
+        assert re.fullmatch(want, st.device_kernel) and st.device_kernel == planned and route.startswith("shared/"), (layout, m, st.device_kernel, route)
+        for y in ys:
+            ctx.fill(y, 0x7FC00000)
+        plan.encode(0)
+        ctx.synchronize()
+        for y, e in zip(ys, eager):
+            assert np.array_equal(y.download(np.float32), e), (layout, m)
+        plan.destroy()
+        for b in ys + [x]:
+            b.free()
+        for w in ws:
+            w.destroy()

@@ -150,3 +150,74 @@ def test_every_route_has_a_gpu_parity_test():
         text = open(os.path.join(here, path)).read()
         assert re.search(rf"^def {func}\(", text, re.M), (route, test_id)
         assert "pytest.mark.gpu" in text, (route, path)
+
+
+# ---- two or three projections that share their activations (q+k+v, gate+up): shared_route, csrc/route.cpp -------------
+SHARED_SHAPES = [((14336, 14336), 4096), ((4096, 1024, 1024), 4096), ((1024, 256, 256), 1024), ((300, 700), 448), ((5, 17, 130), 256)]
+# the device kernel a shared launch's plan record must name
+PLAN_OF_SHARED_ROUTE = {
+    "shared/stream": r"^qgemm_stream_q\d_g\d+$",
+    "shared/mfma-planes": r"^gemv_mfma_planes_q\d_g\d+$",
+    "shared/dot-planes": r"^gemv_(rows|planes)_q\d_g\d+$",
+    "shared/tile16": r"^gemv_tile16_q\d_g\d+$",
+    "shared/staf-in-place": r"^gemv_staf_q\d_g\d+$",
+    "split-rows": r"^split_f32_bf16x3\+",          # the rows are split once, then the table is asked again for the bf16 rows
+    "steps": r".",                                    # the shared launch in steps: the record is the first projection's
+    "separate": r".",                                 # a launch per projection: the record is the first projection's own
+}
+PARITY_TEST_OF_SHARED_ROUTE = {
+    "shared/stream": "test_gpu_gemm_stream.py::test_stream_kernel_shared_launch_equals_separate_launches",
+    "shared/mfma-planes": "test_gpu_mfma_planes.py::test_mfma_planes_batched_projections_one_launch",
+    "shared/dot-planes": "test_gpu_batched.py::test_batched_llama_projections",
+    "shared/tile16": "test_gpu_tile16.py::test_tile16_batched_projections_one_launch",
+    "shared/staf-in-place": "test_gpu_staf_gemv.py::test_in_place_batched_projections",
+    "split-rows": "test_gpu_split_rows.py::test_batched_projections_other_activation_types",
+    "steps": "test_gpu_batched.py::test_batched_equals_separate_launches_on_other_routes",
+    "separate": "test_gpu_batched.py::test_batched_equals_separate_launches_on_other_routes",
+}
+
+
+def test_shared_launches_plan_what_the_launcher_runs_in_every_cell():
+    """mi355q_batched_qgemm and the shared steps of a plan ask one function what the projections run as; the plan record
+    of the step names the kernel of the shared launch wherever there is one."""
+    seen, count = {}, 0
+    for f in pkg.QuantizationFormatRegistry.all_formats():
+        for (lname, layout), (ns, k) in itertools.product(LAYOUTS.items(), SHARED_SHAPES):
+            if k % f.group_size or (layout != pkg.LAYOUT_STAF_BLOCKS and (k * f.bits) % 32):
+                continue
+            if layout == pkg.LAYOUT_TILE16 and not (f.bits == 4 and f.group_size == 64 and k % 128 == 0):
+                continue
+            for (xname, xd), m, fname in itertools.product(X_TYPES.items(), ROWS, FLAG_SETS):
+                launcher, plan = pkg.probe_shared_route(f, layout, ns, k, xd, m, flags=FLAG_SETS[fname])
+                cell = (f.bits, f.group_size, lname, ns, k, xname, m, fname)
+                count += 1
+                assert launcher in PLAN_OF_SHARED_ROUTE, (cell, launcher, plan)
+                if plan != "error":                       # contradictory flags: the launcher refuses the call as well
+                    assert re.match(PLAN_OF_SHARED_ROUTE[launcher], plan), (cell, launcher, plan)
+                if fname == "generic":
+                    assert not launcher.startswith("shared/"), (cell, launcher)
+                if fname in ("stream", "two-step"):         # forced: the matrices together on the stream kernel, or each on its own
+                    assert launcher in (("shared/stream", "separate") if fname == "stream" else ("separate",)), (cell, launcher)
+                seen.setdefault(launcher, cell)
+    assert count > 10000
+    assert set(seen) == set(PLAN_OF_SHARED_ROUTE), sorted(set(PLAN_OF_SHARED_ROUTE) - set(seen))
+    # the Llama-3-8B decode launches land where the measurements say they should
+    q4 = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+    r = lambda *a, **kw: pkg.probe_shared_route(*a, **kw)[0]
+    assert r(q4, pkg.LAYOUT_PLANES, (14336, 14336), 4096, pkg.BF16, 1) == "shared/dot-planes"
+    assert r(q4, pkg.LAYOUT_PLANES, (14336, 14336), 4096, pkg.BF16, 8) == "shared/mfma-planes"
+    assert r(q4, pkg.LAYOUT_PLANES, (4096, 1024, 1024), 4096, pkg.BF16, 3) == "shared/dot-planes"
+    assert r(q4, pkg.LAYOUT_PLANES, (14336, 14336), 4096, pkg.BF16, 32) == "shared/stream"
+    assert r(q4, pkg.LAYOUT_TILE16, (14336, 14336), 4096, pkg.BF16, 16) == "shared/tile16"
+    assert r(q4, pkg.LAYOUT_STAF_BLOCKS, (14336, 14336), 4096, pkg.BF16, 1) == "shared/staf-in-place"
+    assert r(q4, pkg.LAYOUT_STAF_BLOCKS, (14336, 14336), 4096, pkg.BF16, 8) == "shared/stream"
+
+
+def test_every_shared_route_has_a_gpu_parity_test():
+    here = os.path.dirname(os.path.abspath(__file__))
+    assert set(PARITY_TEST_OF_SHARED_ROUTE) == set(PLAN_OF_SHARED_ROUTE)
+    for route, test_id in PARITY_TEST_OF_SHARED_ROUTE.items():
+        path, func = test_id.split("::")
+        text = open(os.path.join(here, path)).read()
+        assert re.search(rf"^def {func}\(", text, re.M), (route, test_id)
+        assert "pytest.mark.gpu" in text, (route, path)
