@@ -372,11 +372,12 @@ mi355q_status launch_qgemm_mfma(hipStream_t s, mi355q_context* ctx, const WView&
                                 uint32_t flags = 0);
 
 // Wide-tile MFMA GEMM for long prompts (gemm_wide.hip): 4-bit planes in groups of 64 / 128, bf16 activations; the weights
-// are dequantised in registers, only the activations pass through LDS.  Taken from kWideMinRows rows where its tiles
-// occupy three quarters of the CUs (measured against the tiled kernel and the two-dispatch route: see gemm_wide_chosen).
+// are dequantised in registers, only the activations pass through LDS.  Taken from kWideMinRows rows (beyond what the
+// streamed-weight kernel takes) where its workgroups occupy five eighths of the CUs (measured against the tiled kernel and
+// the two-dispatch route: see gemm_wide_chosen).
 // the dense library is forbidden for the context or could not be opened: the two-dispatch route serves nothing
 inline bool library_ruled_out(const mi355q_context* ctx) { return ctx->dense_library_failed || ctx->dense_library_forbidden; }
-constexpr uint32_t kWideMinRows = 384;
+constexpr uint32_t kWideMinRows = 97;
 constexpr uint32_t kWideRowsBesideLibrary = 2560;   // from here the two-dispatch route is taken where the dense library is there
 bool gemm_wide_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
 bool gemm_wide_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);

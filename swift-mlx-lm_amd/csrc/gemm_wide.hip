@@ -175,12 +175,15 @@ GemmLaunchShape gemm_wide_shape(uint32_t m, uint32_t n, uint32_t k) {
 }
 
 // Rows from which this kernel is taken instead of the tiled one (which splits K over workgroups for short M) and of
-// the two-dispatch route: enough tiles to occupy three quarters of the CUs.
+// the two-dispatch route: enough workgroups (tiles x K parts) to occupy five eighths of the CUs.  4096 -> 14336: 34 us
+// at 128 rows (128-row tiles, K in four parts) against 41 us on the tiled kernel, 47 against 56-59 at 192 and 256, 57
+// against 78 at 320; 14336 -> 4096 has too few column tiles below 320 rows (59-62 us against 40-55) and changes over
+// there (63 against 78).
 bool gemm_wide_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride) {
     if (!gemm_wide_eligible(w, x_dtype, m, x_stride) || m < kWideMinRows) return false;
     const GemmLaunchShape g = gemm_wide_shape(m, w.n, gemm_wide_k(w.k, x_dtype));
     const uint32_t wgs = ((m + g.bm - 1) / g.bm) * ((w.n + kWideBN - 1) / kWideBN) * g.splits;
-    return 4 * wgs >= 3 * chip_cus();
+    return 8 * wgs >= 5 * chip_cus();
 }
 
 mi355q_status launch_qgemm_wide(hipStream_t s, mi355q_context* ctx, const WView& w, const void* x, int x_dtype, void* y,

@@ -132,7 +132,9 @@ def test_config_routes():
     assert r(q4, P, 14336, 4096, pkg.BF16, 8, decode_entry=True) == "small-batch/mfma-planes"
     assert r(q4, P, 4096, 4096, pkg.BF16, 3, decode_entry=True) == "small-batch/dot-planes"       # small matrix: rows kernel
     assert r(q4, P, 14336, 4096, pkg.BF16, 64) == "stream"
-    assert r(q4, P, 14336, 4096, pkg.BF16, 128) == "fused/tiled"
+    assert r(q4, P, 14336, 4096, pkg.BF16, 128) == "fused/wide"          # 56 column tiles x 4 K parts fill the CUs
+    assert r(q4, P, 4096, 14336, pkg.BF16, 128) == "fused/tiled"         # 16 column tiles do not
+    assert r(q4, P, 4096, 14336, pkg.BF16, 512) == "fused/wide"
     for layout, xd in ((P, pkg.BF16), (B, pkg.BF16), (P, pkg.F16), (B, pkg.F16), (P, pkg.F32), (B, pkg.F32)):
         assert r(q4, layout, 14336, 4096, xd, 2048) == "fused/wide"
         assert r(q4, layout, 4096, 14336, xd, 2048) == "fused/wide"
