@@ -183,7 +183,11 @@ bool gemm_wide_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride
     if (!gemm_wide_eligible(w, x_dtype, m, x_stride) || m < kWideMinRows) return false;
     const GemmLaunchShape g = gemm_wide_shape(m, w.n, gemm_wide_k(w.k, x_dtype));
     const uint32_t wgs = ((m + g.bm - 1) / g.bm) * ((w.n + kWideBN - 1) / kWideBN) * g.splits;
-    return 8 * wgs >= 5 * chip_cus();
+    // where the tiled kernel does not read the weight or the activation type (blocks in place, f16 and fp32 rows) the
+    // other route is the two-dispatch one, and half of the CUs are enough: 8192 -> 8192 on blocks with f16 rows 46-48 us at
+    // 100-128 rows against 66-72 us, 14336 -> 4096 70 against 82 at 256 rows, 4096 -> 4096 33-35 against 38 at 192-256
+    // (with a quarter of the CUs 14336 -> 4096 loses a tenth at 100-128 rows and 8192 -> 2048 a fifth throughout)
+    return 8 * wgs >= (gemm_mfma_eligible(w, x_dtype, m, x_stride) ? 5 : 4) * chip_cus();
 }
 
 mi355q_status launch_qgemm_wide(hipStream_t s, mi355q_context* ctx, const WView& w, const void* x, int x_dtype, void* y,
