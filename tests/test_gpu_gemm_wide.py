@@ -261,3 +261,27 @@ def test_context_without_the_dense_library_keeps_in_tree_kernels(pkg):
         w.destroy()
     finally:
         c.close()
+
+
+@pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
+def test_config3_full_size_properties_every_output(pkg, ctx, n, k):
+    """benchmark config 3 at M = 2048, as dispatched, every one of the M x N outputs through properties that need no
+    oracle pass over the matrix: y(2x) == 2 y(x) bit for bit (doubling is exact in bf16 and in every fp32 sum), rows of
+    x that are equal give rows of y that are equal, a zero row gives the zero row, and the fp32 and bf16 results agree
+    to one rounding."""
+    m = 2048
+    words, s, z, _ = seeded_case(4700 + n % 7, n, k, 4, 64)
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+    w = ctx.weight_prepare_mlx(fmt, words, s, z, pkg.BF16, pkg.LAYOUT_PLANES)
+    assert w.plan_prefill_steps(m)[0].device_kernel == "qgemm_wide_q4_g64"
+    x = act_rounded(kat.seeded_activations(4710, m, k), pkg.BF16, pkg)
+    x[5] = x[1900]                     # equal rows in different row tiles
+    x[300] = 0.0
+    y1 = run_qgemm(ctx, pkg, w, x, pkg.F32, 0)
+    y2 = run_qgemm(ctx, pkg, w, 2.0 * x, pkg.F32, 0)
+    assert np.all(np.isfinite(y1))
+    assert np.array_equal(2.0 * y1, y2)
+    assert np.array_equal(y1[5], y1[1900]) and not np.any(y1[300])
+    yb = run_qgemm(ctx, pkg, w, x, pkg.BF16, 0)
+    assert np.array_equal(oracle.bf16_from_f32(yb), oracle.bf16_from_f32(y1))
+    w.destroy()
