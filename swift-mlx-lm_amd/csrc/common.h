@@ -382,11 +382,24 @@ constexpr uint32_t kWideRowsBesideLibrary = 2560;   // from here the two-dispatc
 bool gemm_wide_eligible(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
 bool gemm_wide_chosen(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride);
 // `k`: the K the kernel walks (twice the weight's K for fp32 activations, see gemm_wide_k)
-GemmLaunchShape gemm_wide_shape(uint32_t m, uint32_t n, uint32_t k);
+GemmLaunchShape gemm_wide_shape(uint32_t m, uint32_t n, uint32_t k, bool one_part = false);
 // fp32 activations run as two bf16 halves side by side, hi = bf16(x) and lo = bf16(x - hi), against the weights twice
 inline uint32_t gemm_wide_k(uint32_t k, int x_dtype) { return x_dtype == MI355Q_F32 ? 2 * k : k; }
 uint32_t chip_cus();
 void gemm_wide_force_shape(uint32_t bm, uint32_t splits);      // A/B runs (mi355q_probe_wide_shape)
+// The gated MLP projection on the wide-tile kernel: gate_proj and up_proj as the two column fragments of every
+// wavefront, activation(gate) * up in the epilogue, one launch and no intermediate matrices.  Chosen under the same
+// rule as the plain kernel, over the 2 N columns of the two matrices, K in one part.
+bool gemm_wide_gated_eligible(const WView& gate, const WView& up, int x_dtype, uint32_t m, uint32_t x_stride);
+bool gemm_wide_gated_chosen(const WView& gate, const WView& up, int x_dtype, uint32_t m, uint32_t x_stride);
+// what dispatch_gated (api.hip) runs and the planner describes: the probe flag takes the kernel wherever it reads the
+// pair, other selection flags leave the gated projection to the separate launches they select; from the rows where the
+// two-dispatch route is ahead the projections go there and the activation stays a launch of its own
+bool gemm_wide_gated_taken(const mi355q_context* ctx, const WView& gate, const WView& up, int x_dtype, uint32_t m, uint32_t x_stride,
+                           uint32_t flags);
+mi355q_status launch_qgemm_wide_gated(hipStream_t s, mi355q_context* ctx, const WView& gate, const WView& up, const void* x,
+                                      int x_dtype, void* y, int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride,
+                                      int activation);
 inline bool gemm_wide_taken(const WView& w, int x_dtype, uint32_t m, uint32_t x_stride, uint32_t flags) {
     if (flags & MI355Q_FLAG_PROBE_TILED) return false;
     if (flags & MI355Q_FLAG_PROBE_WIDE) return gemm_wide_eligible(w, x_dtype, m, x_stride);

@@ -21,6 +21,13 @@ struct WideArgs {
     uint32_t splits, kt_per_split;   // K-tiles per split: a multiple of four
     uint32_t w_fours;                // groups of four K-tiles in a weight row: the walk over K wraps there (fp32 activations
                                      // come as [hi | lo] rows of 2 K bf16 values against the same weights twice)
+    // gated MLP projection (0: none; else 1 + mi355q_gated_activation): the second fragment of every wavefront reads
+    // up_proj where the first reads gate_proj (codes / sz / blocks above), a tile is 128 output columns wide, tiles_n
+    // counts those, and y receives activation(gate) * up; no K parts
+    uint32_t gated;
+    const uint32_t* codes_up;
+    const uint32_t* sz_up;
+    const uint8_t* blocks_up;
     unsigned long long* probe;   // optional: [0] shader cycles, [1] 100 MHz ticks that workgroup 0 spent in the kernel
 };
 

@@ -128,7 +128,7 @@ void gemm_wide_force_shape(uint32_t bm, uint32_t splits) {
 // columns are dequantised once per K-tile whatever the rows: about 2500 cycles at 256 rows, 1600 at 128, measured
 // under load), so 256-row tiles are the efficient ones and K is split into parts where they leave CUs idle: each part
 // writes fp32, a second launch adds the parts (about 3 us and the traffic of splits + 1 result matrices).
-GemmLaunchShape gemm_wide_shape(uint32_t m, uint32_t n, uint32_t k) {
+GemmLaunchShape gemm_wide_shape(uint32_t m, uint32_t n, uint32_t k, bool one_part) {
     const uint32_t cus = chip_cus();
     const uint32_t tiles_n = (n + kWideBN - 1) / kWideBN;
     const uint32_t kt = k / 64;
@@ -140,7 +140,7 @@ GemmLaunchShape gemm_wide_shape(uint32_t m, uint32_t n, uint32_t k) {
         if (forced_bm && bm != forced_bm) continue;
         if (bm == 256 && m <= 128 && !forced_bm) continue;
         for (uint32_t splits : {1u, 2u, 3u, 4u}) {
-            if (forced_splits && splits != forced_splits) continue;
+            if (one_part ? splits != 1 : forced_splits && splits != forced_splits) continue;
             if (splits > 1 && (n % 4 || kt / splits < 16)) continue;
             const uint32_t per = (kt / 4 + splits - 1) / splits * 4;          // K-tiles a part, a multiple of four
             const uint32_t parts = (kt + per - 1) / per;
@@ -240,6 +240,62 @@ mi355q_status launch_qgemm_wide(hipStream_t s, mi355q_context* ctx, const WView&
         MI355Q_HIP(hipGetLastError());
     }
     return MI355Q_OK;
+}
+
+// ---- gated MLP projection ------------------------------------------------------------------------------------------
+bool gemm_wide_gated_eligible(const WView& gate, const WView& up, int x_dtype, uint32_t m, uint32_t x_stride) {
+    if (x_dtype != MI355Q_BF16 && x_dtype != MI355Q_F16) return false;
+    if (!gemm_wide_eligible(gate, x_dtype, m, x_stride) || !gemm_wide_eligible(up, x_dtype, m, x_stride)) return false;
+    return gate.n == up.n && gate.k == up.k && gate.layout == up.layout && gate.group == up.group && gate.bits == up.bits &&
+           gate.sb_dtype == up.sb_dtype && gate.code_stride == up.code_stride && gate.sz_stride == up.sz_stride &&
+           gate.blocks_per_row == up.blocks_per_row && gate.bytes_per_block == up.bytes_per_block;
+}
+
+bool gemm_wide_gated_chosen(const WView& gate, const WView& up, int x_dtype, uint32_t m, uint32_t x_stride) {
+    if (!gemm_wide_gated_eligible(gate, up, x_dtype, m, x_stride) || m < kWideMinRows) return false;
+    const GemmLaunchShape g = gemm_wide_shape(m, 2 * gate.n, gate.k, true);
+    const uint32_t wgs = ((m + g.bm - 1) / g.bm) * ((gate.n + kWideBN / 2 - 1) / (kWideBN / 2));
+    // Up to two rounds of tiles.  The activation costs the matrix-core wavefronts about 10 us a tile (two roundings, an
+    // exponential and a division per output), which the elementwise launch it replaces (65 us at 2048 rows of 14336, bound
+    // by its 176 MB of traffic) spends beside nothing: 4096 -> 2 x 14336 at 256 rows 70 us against 102 for the two
+    // projections and the elementwise launch, at 512 rows 121 against 144, at 1024 rows 240 against 243, at 2048 rows
+    // (3.5 rounds) 484 against 475.
+    return 8 * wgs >= 5 * chip_cus() && wgs <= 2 * chip_cus();
+}
+
+bool gemm_wide_gated_taken(const mi355q_context* ctx, const WView& gate, const WView& up, int x_dtype, uint32_t m, uint32_t x_stride,
+                           uint32_t flags) {
+    if (flags & MI355Q_FLAG_PROBE_WIDE) return gemm_wide_gated_eligible(gate, up, x_dtype, m, x_stride);
+    if (flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_TWO_STEP |
+                 MI355Q_FLAG_FORCE_STREAM))
+        return false;
+    return gemm_wide_gated_chosen(gate, up, x_dtype, m, x_stride) && (m < kWideRowsBesideLibrary || library_ruled_out(ctx));
+}
+
+mi355q_status launch_qgemm_wide_gated(hipStream_t s, mi355q_context* ctx, const WView& gate, const WView& up, const void* x,
+                                      int x_dtype, void* y, int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride,
+                                      int activation) {
+    (void)ctx;
+    if (!gemm_wide_gated_eligible(gate, up, x_dtype, m, x_stride))
+        return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the wide-tile MFMA GEMM does not take this pair of weights as a gated projection");
+    if ((uintptr_t)x % 16) return fail(MI355Q_ERR_INVALID_ARGUMENT, "activation pointer must be 16-byte aligned");
+    const GemmLaunchShape g = gemm_wide_shape(m, 2 * gate.n, gate.k, true);
+    WideArgs a{};
+    const bool blocks = gate.layout == MI355Q_LAYOUT_STAF_BLOCKS;
+    a.codes = gate.codes; a.sz = gate.sz; a.blocks = gate.blocks;
+    a.codes_up = up.codes; a.sz_up = up.sz; a.blocks_up = up.blocks;
+    a.gated = 1u + (uint32_t)activation;
+    a.row_bytes = gate.blocks_per_row * gate.bytes_per_block;
+    a.x = (const uint16_t*)x; a.y = y;
+    a.m = m; a.n = gate.n; a.k = gate.k; a.xs = x_stride; a.ys = y_stride;
+    a.w_fours = gate.k / 256;
+    a.code_stride = gate.code_stride; a.sz_stride = gate.sz_stride;
+    a.y_dtype = (uint32_t)y_dtype;
+    a.line_stores = ((size_t)y_stride * (y_dtype == MI355Q_F32 ? 4 : 2) % 16 == 0 && (uintptr_t)y % 16 == 0) ? 1u : 0u;
+    a.splits = 1; a.kt_per_split = gate.k / 64;
+    const bool sb_bf16 = gate.sb_dtype == MI355Q_BF16;
+    return x_dtype == MI355Q_F16 ? launch_wide_kernel_f16(s, a, g.bm, gate.group, sb_bf16, blocks)
+                                 : launch_wide_kernel_bf16(s, a, g.bm, gate.group, sb_bf16, blocks);
 }
 
 }  // namespace mi355q

@@ -61,7 +61,10 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
     if (t_id >= total) return;
     const uint32_t split = (uint32_t)__builtin_amdgcn_readfirstlane((int)(t_id / tiles)), tile = t_id - split * tiles;
     const uint32_t tn = tile / a.tiles_m, tm = tile % a.tiles_m;
-    const uint32_t m0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tm * BM)), n0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tn * kWideBN));
+    // Gated (a.gated != 0): the two 32-column fragments of a wavefront are the same 32 output columns of gate_proj and of
+    // up_proj, so a tile is 128 output columns wide and activation(gate) * up is formed in the registers of the epilogue.
+    const uint32_t tile_cols = a.gated ? kWideBN / 2 : kWideBN;
+    const uint32_t m0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tm * BM)), n0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tn * tile_cols));
     const uint32_t kt_begin = (uint32_t)__builtin_amdgcn_readfirstlane((int)(split * a.kt_per_split));
 
     const uint32_t tid = threadIdx.x, lane = tid & 63;
@@ -99,7 +102,7 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
     uint32_t w_off[2], sz_off[2];
 #pragma unroll
     for (int f = 0; f < 2; f++) {
-        const uint32_t r = 64 * wave + 32 * f + ln;
+        const uint32_t r = a.gated ? 32 * wave + ln : 64 * wave + 32 * f + ln;
         const uint32_t gr = r < n_last ? r : n_last;
         if constexpr (BLOCKS) {
             sz_off[f] = gr * a.row_bytes;                 // the header of the row's first block
@@ -111,6 +114,10 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
     }
     const char* const cg = BLOCKS ? (const char*)a.blocks + (size_t)n0 * a.row_bytes : (const char*)(a.codes + (size_t)n0 * a.code_stride);
     const char* const sg = BLOCKS ? cg : (const char*)(a.sz + (size_t)n0 * a.sz_stride);
+    // the second fragment's matrix: up_proj where gated, else the same one
+    const char* const cg1 = !a.gated ? cg : BLOCKS ? (const char*)a.blocks_up + (size_t)n0 * a.row_bytes
+                                                   : (const char*)(a.codes_up + (size_t)n0 * a.code_stride);
+    const char* const sg1 = !a.gated ? sg : BLOCKS ? cg1 : (const char*)(a.sz_up + (size_t)n0 * a.sz_stride);
     const uint32_t four_begin = kt_begin / 4;
     using sz_vec = std::conditional_t<SZW == 4, u32x4, u32x2>;      // kept whole: the loads write them behind the compiler's back
     u32x4 wnext[2][4], wcur[2][4];
@@ -120,10 +127,12 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
     auto load_w = [&](uint32_t four) __attribute__((always_inline)) {
         uint32_t p = four_begin + (four * 4 < KT ? four : KT / 4 - 1);
         p = p >= a.w_fours ? p - a.w_fours : p;      // the second half of [hi | lo] activations meets the same weights again
-        const char* const g = wd_scalar(cg + (size_t)p * FOUR_BYTES);
-        const char* const gs = BLOCKS ? g : wd_scalar(sg + (size_t)p * (SZW * 4));
+        const char* const gb[2] = {wd_scalar(cg + (size_t)p * FOUR_BYTES), wd_scalar(cg1 + (size_t)p * FOUR_BYTES)};
+        const char* const gsb[2] = {BLOCKS ? gb[0] : wd_scalar(sg + (size_t)p * (SZW * 4)),
+                                    BLOCKS ? gb[1] : wd_scalar(sg1 + (size_t)p * (SZW * 4))};
 #pragma unroll
         for (int f = 0; f < 2; f++) {
+            const char* const g = gb[f];
 #pragma unroll
             for (int t = 0; t < 4; t++) {
                 // K-tile t of the four: 32 bytes on in the planes; in blocks, behind the header of its group
@@ -135,6 +144,7 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
         }
 #pragma unroll
         for (int f = 0; f < 2; f++) {
+            const char* const gs = gsb[f];
             if constexpr (BLOCKS) {
 #pragma unroll
                 for (int i = 0; i < SZW; i++)
@@ -418,6 +428,72 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         });
     };
+    // Gated: activation(gate) * up where the two accumulators of a row block meet (gate and up values rounded to the
+    // output type first, as the reference's elementwise kernel reads them from buffers of that type), the 32 x 32
+    // results of a wavefront through LDS and out in 16-byte pieces; tiles at the edge of the matrix element by element.
+    auto store_gated = [&](auto DT) __attribute__((always_inline)) {
+        constexpr int dt = decltype(DT)::value;
+        constexpr int ESZ = dt == MI355Q_F32 ? 4 : 2;
+        constexpr int PITCH = 32 * ESZ + 16;
+        constexpr int LPR = 32 * ESZ / 16;                         // lanes per row of the read-back
+        constexpr int RPI = 64 / LPR;                              // rows per read-back instruction
+        char* const stage = lds + wave * (32 * PITCH);
+        const bool whole = n0 + kWideBN / 2 <= a.n && a.line_stores;
+        const uint32_t act = a.gated - 1;
+        __builtin_amdgcn_s_barrier();                              // every wavefront is done with the activation stages
+        static_for<TM>([&](auto I) __attribute__((always_inline)) {
+            constexpr int i = decltype(I)::value;
+            asm volatile("" : "+v"(acc[0][i]), "+v"(acc[1][i]));
+            float v[16];
+#pragma unroll
+            for (int r = 0; r < 16; r++) v[r] = gated_value(acc[0][i][r], acc[1][i][r], act, (uint32_t)dt);
+            if (whole) {
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    char* const at = stage + ln * PITCH + (8 * g + 4 * lh) * ESZ;
+                    if constexpr (dt == MI355Q_F32) {
+                        const wd_float4_v t = {v[4 * g], v[4 * g + 1], v[4 * g + 2], v[4 * g + 3]};
+                        *(wd_float4_v*)at = t;
+                    } else {
+                        u32x2 t;
+                        t.x = dt == MI355Q_BF16 ? wd_pack_bf16(v[4 * g], v[4 * g + 1]) : wd_pack_f16(v[4 * g], v[4 * g + 1]);
+                        t.y = dt == MI355Q_BF16 ? wd_pack_bf16(v[4 * g + 2], v[4 * g + 3]) : wd_pack_f16(v[4 * g + 2], v[4 * g + 3]);
+                        *(u32x2*)at = t;
+                    }
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+                for (int t = 0; t < 32 / RPI; t++) {
+                    const uint32_t r = t * RPI + lane / LPR, piece = lane % LPR;
+                    const u32x4 d = *(const u32x4*)(stage + r * PITCH + piece * 16);
+                    const uint32_t row = m0 + i * 32 + r;
+                    if (row < a.m)
+                        *(u32x4*)((char*)a.y + ((size_t)row * a.ys + n0 + 32 * wave) * ESZ + piece * 16) = d;
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            } else {
+                const uint32_t row = m0 + i * 32 + ln;
+                if (row < a.m) {
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const uint32_t col = n0 + 32 * wave + 8 * (r / 4) + 4 * lh + r % 4;
+                        if (col < a.n) store_out<dt>(a.y, (size_t)row * a.ys + col, v[r]);
+                    }
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+    if (a.gated) {
+        if (a.y_dtype == MI355Q_BF16) store_gated(std::integral_constant<int, MI355Q_BF16>{});
+        else if (a.y_dtype == MI355Q_F32) store_gated(std::integral_constant<int, MI355Q_F32>{});
+        else store_gated(std::integral_constant<int, MI355Q_F16>{});
+        return;
+    }
     const bool inner = n0 + kWideBN <= a.n;                        // (uniform over the workgroup)
     if (a.partial) {       // this part of K as fp32 (N is a multiple of four: 16-byte stores); wide_reduce_kernel adds the parts
         float* const part = a.partial + (size_t)split * a.m * a.n;
@@ -442,7 +518,7 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
 template <int BM, bool SB_BF16, int GROUP, bool BLOCKS>
 mi355q_status launch_wide_tile(hipStream_t s, WideArgs a) {
     a.tiles_m = (a.m + BM - 1) / BM;
-    a.tiles_n = (a.n + kWideBN - 1) / kWideBN;
+    a.tiles_n = a.gated ? (a.n + kWideBN / 2 - 1) / (kWideBN / 2) : (a.n + kWideBN - 1) / kWideBN;
     const uint32_t grid = (a.tiles_m * a.tiles_n * a.splits + 7) / 8 * 8;
     constexpr size_t lds = (size_t)kWideStages * BM * 128;
     auto kern = qgemm_wide_kernel<BM, SB_BF16, GROUP, BLOCKS, WIDE_XF16 != 0>;

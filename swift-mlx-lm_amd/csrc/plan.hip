@@ -218,9 +218,21 @@ mi355q_status mi355q_plan_add_gated_mlp(mi355q_plan* plan, const mi355q_weight* 
     const mi355q_weight* both[2] = {w_gate, w_up};
     plan_shared_launch_shape(both, 2, m, x_dtype, st.xs, flags, &st.record);
     // one launch with the activation as its epilogue, or the batched projection followed by the elementwise kernel
-    const bool one_launch = !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_MFMA |
-                                       MI355Q_FLAG_FORCE_TWO_STEP | MI355Q_FLAG_FORCE_STREAM)) &&
-                            gemv_gated_eligible(plan->ctx, w_gate->view(), w_up->view(), x_dtype, m, st.xs);
+    bool one_launch = !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_MFMA |
+                                 MI355Q_FLAG_FORCE_TWO_STEP | MI355Q_FLAG_FORCE_STREAM)) &&
+                      gemv_gated_eligible(plan->ctx, w_gate->view(), w_up->view(), x_dtype, m, st.xs);
+    if (!one_launch && gemm_wide_gated_taken(plan->ctx, w_gate->view(), w_up->view(), x_dtype, m, st.xs, flags)) {
+        // the wide-tile prefill kernel over both matrices: tiles of 128 output columns, K in one part
+        one_launch = true;
+        const GemmLaunchShape g = gemm_wide_shape(m, 2 * (uint32_t)w_gate->n, (uint32_t)w_gate->k, true);
+        std::snprintf(st.record.device_kernel, sizeof st.record.device_kernel, "qgemm_wide_q%u_g%u", (unsigned)w_gate->fmt.bits,
+                      w_gate->fmt.group_size);
+        st.record.grid[0] = g.grid; st.record.grid[1] = 1;
+        st.record.block[0] = g.block;
+        st.record.lds_bytes = g.lds_bytes;
+        st.record.rows_per_workgroup = 128;
+        st.record.used_fallback = 0;
+    }
     const char* const act = activation == MI355Q_GATED_SILU ? "swiglu" : "gelu_gated";
     char name[sizeof st.record.device_kernel];
     std::snprintf(name, sizeof name, "%s%s%s", st.record.device_kernel, one_launch ? "+" : " ; ", act);

@@ -210,3 +210,86 @@ def test_gated_step_in_a_plan_replayed_as_a_graph(pkg, ctx):
     for t in (xdev, direct, planned):
         t.free()
     g.destroy(); u.destroy()
+
+
+@pytest.mark.parametrize("layout_name,x_name", [("LAYOUT_PLANES", "BF16"), ("LAYOUT_STAF_BLOCKS", "BF16"), ("LAYOUT_PLANES", "F16")])
+def test_gated_projection_on_the_prefill_kernel(pkg, ctx, layout_name, x_name):
+    """Prompts: gate_proj and up_proj as the two column fragments of every wavefront of the wide-tile matrix-core kernel,
+    activation(gate) * up in its epilogue, one launch.  Equal, bit for bit, to the two projections on that kernel
+    followed by the elementwise kernel (same sums, same roundings), for ragged rows and columns, groups of 64 and 128,
+    every output type, both activations and a padded result; the plan record says so."""
+    layout, xd = getattr(pkg, layout_name), getattr(pkg, x_name)
+    wide_flags = pkg.FLAG_FORCE_MFMA | pkg.FLAG_PROBE_WIDE
+    for i, (m, n, k, group) in enumerate([(300, 260, 512, 64), (130, 515, 768, 128), (258, 128, 256, 64)]):
+        fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, group)
+        sbo, sbp = (oracle.F16, pkg.F16) if layout == pkg.LAYOUT_STAF_BLOCKS else (oracle.BF16, pkg.BF16)
+        wg, sg, zg = oracle.quantize_affine(kat.seeded_weights(6500 + i, n, k), 4, group, sbo)
+        wu, su, zu = oracle.quantize_affine(kat.seeded_weights(6510 + i, n, k), 4, group, sbo)
+        g = ctx.weight_prepare_mlx(fmt, wg, sg, zg, sbp, layout)
+        u = ctx.weight_prepare_mlx(fmt, wu, su, zu, sbp, layout)
+        x = act_rounded(kat.seeded_activations(6520 + i, m, k), xd, pkg)
+        xdev = ctx.upload(act_to_device_array(x, xd, pkg))
+        for yd in (pkg.BF16, pkg.F32, pkg.F16):
+            esz = 4 if yd == pkg.F32 else 2
+            for kind in (pkg.GATED_SILU, pkg.GATED_GELU_TANH):
+                for y_pad in (0, 8, 3):
+                    say(f"gated wide {layout_name} x={x_name} {m}x{n}x{k} g{group} y={yd} act={kind} pad={y_pad}")
+                    ys = n + y_pad
+                    fused, gate_b, up_b, two = (ctx.alloc(m * ys * esz) for _ in range(4))
+                    ctx.fill(fused, 0x7FC07FC0 if esz == 2 else 0x7FC00000)
+                    ctx.fill(two, 0x7FC07FC0 if esz == 2 else 0x7FC00000)
+                    ctx.gated_qgemm(g, u, xdev, xd, fused, yd, m, kind, 0, ys if y_pad else 0, pkg.FLAG_PROBE_WIDE)
+                    ctx.qgemm(g, xdev, xd, gate_b, yd, m, 0, ys if y_pad else 0, wide_flags)
+                    ctx.qgemm(u, xdev, xd, up_b, yd, m, 0, ys if y_pad else 0, wide_flags)
+                    ctx.gated_activation(gate_b, up_b, two, yd, n, m, ys if y_pad else 0, kind)
+                    ctx.synchronize()
+                    dt = np.float32 if esz == 4 else np.uint16
+                    a, b = fused.download(dt, (m, ys)), two.download(dt, (m, ys))
+                    assert np.array_equal(a[:, :n], b[:, :n]), "one launch != two projections + elementwise kernel"
+                    if y_pad:
+                        pad = a[:, n:]
+                        assert np.all(np.isnan(pad)) if esz == 4 else np.all(pad == 0x7FC0), "padding of the output rows was written"
+                    for t in (fused, gate_b, up_b, two):
+                        t.free()
+        xdev.free(); g.destroy(); u.destroy()
+
+
+def test_gated_projection_llama_prompt_as_dispatched(pkg, ctx):
+    """Llama-3-8B's gate / up pair at 512 rows with no flags: one launch on the wide-tile kernel (the plan record names
+    it), equal to the two projections and the elementwise kernel, and within the bar of the oracle on a column sample;
+    at 2048 rows (more than two rounds of tiles) the plan keeps the projections and the elementwise launch apart."""
+    n, k, m = 14336, 4096, 512
+    wg, sg, zg, wq_g = seeded_case(6600, n, k, 4, 64)
+    wu, su, zu, wq_u = seeded_case(6601, n, k, 4, 64)
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+    g = ctx.weight_prepare_mlx(fmt, wg, sg, zg, pkg.BF16, pkg.LAYOUT_PLANES)
+    u = ctx.weight_prepare_mlx(fmt, wu, su, zu, pkg.BF16, pkg.LAYOUT_PLANES)
+    x = act_rounded(kat.seeded_activations(6602, m, k), pkg.BF16, pkg)
+    xdev = ctx.upload(act_to_device_array(x, pkg.BF16, pkg))
+    fused, gate_b, up_b, two = (ctx.alloc(m * n * 2) for _ in range(4))
+    plan = pkg.DispatchPlan(ctx)
+    plan.add_gated_mlp(g, u, xdev, pkg.BF16, fused, pkg.BF16, m, activation=pkg.GATED_SILU)
+    st, _, _ = plan.step(0)
+    assert st.device_kernel == "qgemm_wide_q4_g64+swiglu" and st.kernel_family == "gatedFusedQ4G64", (st.device_kernel, st.kernel_family)
+    far = pkg.DispatchPlan(ctx)
+    far.add_gated_mlp(g, u, xdev, pkg.BF16, fused, pkg.BF16, 2048, activation=pkg.GATED_SILU)     # (described, not run)
+    assert far.step(0)[0].kernel_family == "gatedBatched2Q4G64" and far.step(0)[0].device_kernel == "qgemm_wide_q4_g64 ; swiglu"
+    far.destroy()
+    plan.encode(0)
+    ctx.qgemm(g, xdev, pkg.BF16, gate_b, pkg.BF16, m)
+    ctx.qgemm(u, xdev, pkg.BF16, up_b, pkg.BF16, m)
+    ctx.gated_activation(gate_b, up_b, two, pkg.BF16, n, m, 0, pkg.GATED_SILU)
+    ctx.synchronize()
+    a, b = fused.download(np.uint16, (m, n)), two.download(np.uint16, (m, n))
+    assert np.array_equal(a, b)
+    cols = np.unique(np.concatenate([np.arange(0, n, n // 16), [1, 127, 128, n - 129, n - 1]]))
+    rows = np.unique(np.concatenate([np.arange(0, m, m // 8), [255, 256, m - 1]]))
+    bf = lambda w: oracle.bf16_to_f32(oracle.bf16_from_f32(w)).reshape(w.shape)
+    want = _expected(pkg, np.ascontiguousarray(bf(wq_g[cols])), np.ascontiguousarray(bf(wq_u[cols])), np.ascontiguousarray(x[rows]),
+                     pkg.GATED_SILU, pkg.BF16)
+    got = oracle.bf16_to_f32(a).reshape(m, n)[np.ix_(rows, cols)]
+    _check(pkg, got, want, pkg.BF16, "gated prompt")
+    plan.destroy()
+    for t in (xdev, fused, gate_b, up_b, two):
+        t.free()
+    g.destroy(); u.destroy()
