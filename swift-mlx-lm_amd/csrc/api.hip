@@ -686,6 +686,9 @@ mi355q_status dispatch_gated(mi355q_context* ctx, hipStream_t s, const mi355q_we
     // prompts on 4-bit weights: the wide-tile matrix-core kernel with the activation as its epilogue
     if (gemm_wide_gated_taken(ctx, g, u, x_dtype, m, xs, flags) && (uintptr_t)x_dev % 16 == 0)
         return launch_qgemm_wide_gated(s, ctx, g, u, x_dev, x_dtype, y_dev, y_dtype, m, xs, ys, activation);
+    // a few dozen rows: the streamed-weight kernel, gate_proj and up_proj as the two row blocks of every workgroup
+    if (gemm_stream_gated_taken(ctx, g, u, x_dtype, m, xs, flags) && (uintptr_t)x_dev % 16 == 0)
+        return launch_qgemm_stream_gated(s, ctx, g, u, x_dev, x_dtype, y_dev, y_dtype, m, xs, ys, activation);
     // elsewhere: the two projections as the batched entry point runs them, into scratch of the context, then the
     // elementwise kernel (the reference's own sequence of dispatches)
     const size_t esz = y_dtype == MI355Q_F32 ? 4 : 2;

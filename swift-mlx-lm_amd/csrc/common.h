@@ -433,6 +433,16 @@ bool gemm_stream_multi_eligible(uint32_t count, const WView* w, int x_dtype, uin
 mi355q_status launch_qgemm_stream_multi(hipStream_t s, mi355q_context* ctx, uint32_t count, const WView* w, const void* x,
                                         int x_dtype, void* const* y, const uint32_t* y_strides, int y_dtype, uint32_t m,
                                         uint32_t x_stride);
+// The gated MLP projection on the streamed-weight kernel: a workgroup's two row blocks read the same 32 rows of gate_proj
+// and up_proj, activation(gate) * up stored from its epilogue, one launch.  Taken where gate+up would share a launch of
+// this kernel (shared_route) and the workgroups of the gated form (32 output columns each) need no K parts; the flag
+// that forces the kernel takes it with K in one part whatever the shape.
+bool gemm_stream_gated_taken(const mi355q_context* ctx, const WView& gate, const WView& up, int x_dtype, uint32_t m,
+                             uint32_t x_stride, uint32_t flags);
+StreamLaunchShape gemm_stream_gated_shape(const mi355q_context* ctx, uint32_t m, uint32_t n, uint32_t k);
+mi355q_status launch_qgemm_stream_gated(hipStream_t s, mi355q_context* ctx, const WView& gate, const WView& up, const void* x,
+                                        int x_dtype, void* y, int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride,
+                                        int activation);
 // Two-dispatch prefill route: dequantise the whole matrix to bf16 in the context's scratch, then the platform's
 // dense GEMM.  `dense_library_serves` answers whether the library can be opened and has an algorithm for the problem.
 // The library's workspace is its own allocation per context (zeroed once, written by nothing else).

@@ -25,6 +25,10 @@ struct StreamArgs {
     uint32_t y_dtype;
     uint32_t iters_per_part;   // iterations (256 columns each) per K part; blockIdx.y is the part
     uint32_t exact;            // host side: the variant with unrounded weights (at most 32 rows, groups of 64 or 128)
+    // gated MLP projection (0: none; else 1 + mi355q_gated_activation): matrix 0 is gate_proj, matrix 1 up_proj, a
+    // workgroup owns rows 32 blockIdx.x .. + 31 of both (its two row blocks) and y[0] receives activation(gate) * up;
+    // K in one part
+    uint32_t gated;
 };
 
 constexpr int kStreamIterK = 256;      // columns of K per iteration: one 64-code K-tile per K slice

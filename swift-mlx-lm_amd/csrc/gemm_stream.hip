@@ -61,6 +61,23 @@ StreamLaunchShape gemm_stream_shape_blocks(const mi355q_context* ctx, uint32_t m
 }
 
 
+namespace {
+// the instantiation unit of the code width
+mi355q_status launch_stream_width(hipStream_t s, const StreamArgs& a, const StreamLaunchShape& g, const WView& w, int x_dtype) {
+    const bool bf = w.sb_dtype == MI355Q_BF16, xf = x_dtype == MI355Q_F16, bl = w.layout == MI355Q_LAYOUT_STAF_BLOCKS;
+    switch (w.bits) {
+    case 2: return launch_stream_q2(s, a, g, w.group, bf, xf, bl);
+    case 3: return launch_stream_q3(s, a, g, w.group, bf, xf, bl);
+    case 4: return launch_stream_q4(s, a, g, w.group, bf, xf, bl);
+    case 5: return launch_stream_q5(s, a, g, w.group, bf, xf, bl);
+    case 6: return launch_stream_q6(s, a, g, w.group, bf, xf, bl);
+    case 8: return launch_stream_q8(s, a, g, w.group, bf, xf, bl);
+    default: break;
+    }
+    return MI355Q_ERR_KERNEL_NOT_FOUND;
+}
+}  // namespace
+
 mi355q_status launch_qgemm_stream(hipStream_t s, mi355q_context* ctx, const WView& w, const void* x, int x_dtype, void* y,
                                   int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride) {
     void* ys[1] = {y};
@@ -113,17 +130,7 @@ mi355q_status launch_qgemm_stream_multi(hipStream_t s, mi355q_context* ctx, uint
         if (mi355q_status st = ensure_workspace(ctx, (size_t)g.parts * m * cols * sizeof(float))) return st;
         a.partial = (float*)ctx->workspace;
     }
-    const bool bf = w[0].sb_dtype == MI355Q_BF16, xf = x_dtype == MI355Q_F16, bl = w[0].layout == MI355Q_LAYOUT_STAF_BLOCKS;
-    mi355q_status st = MI355Q_ERR_KERNEL_NOT_FOUND;
-    switch (w[0].bits) {
-    case 2: st = launch_stream_q2(s, a, g, w[0].group, bf, xf, bl); break;
-    case 3: st = launch_stream_q3(s, a, g, w[0].group, bf, xf, bl); break;
-    case 4: st = launch_stream_q4(s, a, g, w[0].group, bf, xf, bl); break;
-    case 5: st = launch_stream_q5(s, a, g, w[0].group, bf, xf, bl); break;
-    case 6: st = launch_stream_q6(s, a, g, w[0].group, bf, xf, bl); break;
-    case 8: st = launch_stream_q8(s, a, g, w[0].group, bf, xf, bl); break;
-    default: break;
-    }
+    const mi355q_status st = launch_stream_width(s, a, g, w[0], x_dtype);
     if (st != MI355Q_OK || g.parts == 1) return st;
     const size_t total = (size_t)m * cols;
     size_t sum_blocks = (total + 255) / 256;
@@ -131,6 +138,48 @@ mi355q_status launch_qgemm_stream_multi(hipStream_t s, mi355q_context* ctx, uint
     stream_sum_parts_kernel<<<dim3((unsigned)sum_blocks), dim3(256), 0, s>>>(a, g.parts);
     MI355Q_HIP(hipGetLastError());
     return MI355Q_OK;
+}
+
+// ---- gated MLP projection ------------------------------------------------------------------------------------------
+StreamLaunchShape gemm_stream_gated_shape(const mi355q_context* ctx, uint32_t m, uint32_t n, uint32_t k) {
+    return gemm_stream_shape_blocks(ctx, m, (n + 31) / 32, k);
+}
+
+bool gemm_stream_gated_taken(const mi355q_context* ctx, const WView& gate, const WView& up, int x_dtype, uint32_t m,
+                             uint32_t x_stride, uint32_t flags) {
+    if (gate.n != up.n) return false;
+    const WView both[2] = {gate, up};
+    if (shared_route(ctx, 2, both, x_dtype, m, x_stride, flags, true) != SharedRoute::kStream) return false;
+    if (flags & MI355Q_FLAG_FORCE_STREAM) return true;
+    return gemm_stream_gated_shape(ctx, m, gate.n, gate.k).parts == 1;      // a partial sum cannot be gated
+}
+
+mi355q_status launch_qgemm_stream_gated(hipStream_t s, mi355q_context* ctx, const WView& gate, const WView& up, const void* x,
+                                        int x_dtype, void* y, int y_dtype, uint32_t m, uint32_t x_stride, uint32_t y_stride,
+                                        int activation) {
+    const WView w[2] = {gate, up};
+    if (gate.n != up.n || !gemm_stream_multi_eligible(2, w, x_dtype, m, x_stride))
+        return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the streamed-weight kernel does not take this pair of weights as a gated projection");
+    if ((uintptr_t)x % 16) return fail(MI355Q_ERR_INVALID_ARGUMENT, "activation pointer must be 16-byte aligned");
+    StreamArgs a{};
+    for (uint32_t i = 0; i < (uint32_t)kStreamMaxSegments; i++) {
+        const uint32_t j = i < 2 ? i : 1;
+        a.codes[i] = w[j].codes; a.sz[i] = w[j].sz; a.blocks[i] = w[j].blocks; a.y[i] = y;
+        a.n[i] = w[j].n; a.ys[i] = y_stride;
+        a.code_stride[i] = w[j].code_stride; a.sz_stride[i] = w[j].sz_stride;
+        a.col0[i] = 0xFFFFFFFFu; a.wg_end[i] = 0xFFFFFFFFu;     // (not read: a workgroup's row blocks name the matrices)
+    }
+    a.row_bytes = (uint64_t)gate.blocks_per_row * gate.bytes_per_block;
+    a.x = (const uint16_t*)x;
+    a.m = m; a.k = gate.k; a.xs = x_stride; a.n_total = gate.n;
+    a.y_dtype = (uint32_t)y_dtype;
+    a.gated = 1u + (uint32_t)activation;
+    StreamLaunchShape g = gemm_stream_gated_shape(ctx, m, gate.n, gate.k);
+    g.parts = 1;
+    g.iters_per_part = (gate.k + kStreamIterK - 1) / kStreamIterK;
+    a.iters_per_part = g.iters_per_part;
+    a.exact = gemm_stream_unrounded(gate, m);
+    return launch_stream_width(s, a, g, gate, x_dtype);
 }
 
 }  // namespace mi355q

@@ -23,9 +23,11 @@
 //   * weights left in the reference's interleaved blocks are read in place: a lane's 32 codes lie in one block behind
 //     its (scale, zero) header (STAF payload, Sources/MetalCompiler/STAF/QuantizationFormat.swift:1121-1235);
 //   * two or three matrices that share the activations (q+k+v, gate+up) run as one launch, each owning whole
-//     workgroups;
-//   * the four K slices of a row block add their accumulators through LDS at the end; with K split over workgroups
-//     (few rows, long K) fp32 partial results go to scratch and a second launch adds them.
+//     workgroups; the gated MLP projection (Sources/MetalCompiler/Compilable/MLPFragment.swift:7-27) gives a workgroup's
+//     first row block to gate_proj and its second to the same rows of up_proj and stores activation(gate) * up;
+//   * the four K slices of a row block add their accumulators through LDS at the end, all twelve wavefronts sharing the
+//     outputs; with K split over workgroups (few rows, long K) fp32 partial results go to scratch and a second launch
+//     adds them.
 #include "device_utils.h"
 #include "gemm_stream.h"
 #include <atomic>
@@ -92,9 +94,11 @@ __global__ __launch_bounds__(kStreamThreads) void qgemm_stream_kernel(StreamArgs
     const bool stager = wave >= 8;                        // wavefronts 8..11 move the activations, 0..7 multiply
     const uint32_t rb = (wave >> 2) & 1u, slice = wave & 3u;     // row block, K slice
     const uint32_t ln = lane & 31, lh = lane >> 5;
-    const bool in1 = blockIdx.x >= a.wg_end[0], in2 = blockIdx.x >= a.wg_end[1];      // the matrix of this workgroup
+    // the matrix of this workgroup; gated projection: of this row block (gate_proj, up_proj: rows n0 .. n0 + 31 of both)
+    const bool gated = a.gated != 0;
+    const bool in1 = gated ? rb == 1 : blockIdx.x >= a.wg_end[0], in2 = !gated && blockIdx.x >= a.wg_end[1];
     const uint32_t seg_n = in2 ? a.n[2] : in1 ? a.n[1] : a.n[0];
-    const uint32_t n0 = (blockIdx.x - (in2 ? a.wg_end[1] : in1 ? a.wg_end[0] : 0u)) * kStreamRows + rb * 32;
+    const uint32_t n0 = gated ? blockIdx.x * 32 : (blockIdx.x - (in2 ? a.wg_end[1] : in1 ? a.wg_end[0] : 0u)) * kStreamRows + rb * 32;
 
     const uint32_t KT = a.k / 64;                         // K-tiles
     const uint32_t it_all = (a.k + kStreamIterK - 1) / kStreamIterK;
@@ -308,45 +312,44 @@ __global__ __launch_bounds__(kStreamThreads) void qgemm_stream_kernel(StreamArgs
     }
 
     // ---- the four K slices of a row block add up through LDS (the staged activations are done with) ----------------
+    // Every multiplying wavefront parks its accumulators; then all twelve wavefronts, the staging ones too, share the
+    // outputs register by register (a lane's position in the 32 x 32 tile is the same in every wavefront): slice 0 + 1 +
+    // 2 + 3 in that order, then the store -- or, gated, activation(gate sums) * (up sums) of the two row blocks.  One
+    // wavefront a row block doing all of it costs 4 us a workgroup with the activation, 1 us without.
+    constexpr uint32_t T = 16 * MB * 64;                  // floats of one wavefront's accumulators
     float* const red = (float*)lds;
-    if (!stager && slice != 0) {
-        float* const mine = red + (size_t)(rb * 3 + slice - 1) * (16 * MB * 64);
+    if (!stager) {
+        float* const mine = red + (size_t)(rb * 4 + slice) * T;
 #pragma unroll
         for (int b = 0; b < MB; b++)
 #pragma unroll
             for (int r = 0; r < 16; r++) mine[(b * 16 + r) * 64 + lane] = acc[b][r];
     }
     __syncthreads();
-    if (stager || slice != 0) return;
+    const uint32_t wg_n0 = gated ? n0 : n0 - rb * 32;     // the workgroup's first weight row
+    void* const seg_y = in2 ? a.y[2] : (!gated && in1) ? a.y[1] : a.y[0];
+    const uint32_t seg_ys = in2 ? a.ys[2] : (!gated && in1) ? a.ys[1] : a.ys[0];
+    const uint32_t pcol0 = in2 ? a.col0[2] : (!gated && in1) ? a.col0[1] : a.col0[0];
 #pragma nounroll
-    for (int sl = 0; sl < 3; sl++) {
-        const float* const other = red + (size_t)(rb * 3 + sl) * (16 * MB * 64);
-#pragma unroll
-        for (int b = 0; b < MB; b++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) acc[b][r] += other[(b * 16 + r) * 64 + lane];
-    }
-    const uint32_t col = n0 + ln;
-    if (col >= seg_n) return;
-    void* const seg_y = in2 ? a.y[2] : in1 ? a.y[1] : a.y[0];
-    const uint32_t seg_ys = in2 ? a.ys[2] : in1 ? a.ys[1] : a.ys[0];
-    const uint32_t pcol = (in2 ? a.col0[2] : in1 ? a.col0[1] : a.col0[0]) + col;
-#pragma unroll
-    for (int b = 0; b < MB; b++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const uint32_t row = b * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
-            if (row >= a.m) continue;
-            const float v = acc[b][r];
-            if (a.partial) {
-                a.partial[((size_t)blockIdx.y * a.m + row) * a.n_total + pcol] = v;
-                continue;
-            }
-            const size_t o = (size_t)row * seg_ys + col;
-            if (a.y_dtype == MI355Q_F32) ((float*)seg_y)[o] = v;
-            else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)seg_y)[o] = f32_to_bf16_rne(v);
-            else ((uint16_t*)seg_y)[o] = f32_to_f16_rne(v);
+    for (uint32_t i = wave; i < (gated ? 1u : 2u) * 16u * MB; i += kStreamThreads / 64) {
+        const uint32_t rbx = i / (16u * MB), j = i - rbx * (16u * MB), r = j & 15u;
+        const uint32_t row = (j >> 4) * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
+        const uint32_t col = wg_n0 + rbx * 32 + ln;
+        if (row >= a.m || col >= seg_n) continue;
+        const float* const p = red + (size_t)(rbx * 4) * T + j * 64 + lane;
+        float v = ((p[0] + p[T]) + p[2 * T]) + p[3 * T];
+        if (gated) {
+            const float* const q = p + 4 * T;
+            v = gated_value(v, ((q[0] + q[T]) + q[2 * T]) + q[3 * T], a.gated - 1, a.y_dtype);
+        } else if (a.partial) {
+            a.partial[((size_t)blockIdx.y * a.m + row) * a.n_total + pcol0 + col] = v;
+            continue;
         }
+        const size_t o = (size_t)row * seg_ys + col;
+        if (a.y_dtype == MI355Q_F32) ((float*)seg_y)[o] = v;
+        else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)seg_y)[o] = f32_to_bf16_rne(v);
+        else ((uint16_t*)seg_y)[o] = f32_to_f16_rne(v);
+    }
 }
 
 namespace {

@@ -233,6 +233,18 @@ mi355q_status mi355q_plan_add_gated_mlp(mi355q_plan* plan, const mi355q_weight* 
         st.record.rows_per_workgroup = 128;
         st.record.used_fallback = 0;
     }
+    if (!one_launch && gemm_stream_gated_taken(plan->ctx, w_gate->view(), w_up->view(), x_dtype, m, st.xs, flags)) {
+        // the streamed-weight kernel, 32 output columns a workgroup, K in one part
+        one_launch = true;
+        const StreamLaunchShape g = gemm_stream_gated_shape(plan->ctx, m, (uint32_t)w_gate->n, (uint32_t)w_gate->k);
+        std::snprintf(st.record.device_kernel, sizeof st.record.device_kernel, "qgemm_stream_q%u_g%u", (unsigned)w_gate->fmt.bits,
+                      w_gate->fmt.group_size);
+        st.record.grid[0] = g.row_blocks; st.record.grid[1] = 1;
+        st.record.block[0] = 768;
+        st.record.lds_bytes = g.lds_bytes;
+        st.record.rows_per_workgroup = 32;
+        st.record.used_fallback = 0;
+    }
     const char* const act = activation == MI355Q_GATED_SILU ? "swiglu" : "gelu_gated";
     char name[sizeof st.record.device_kernel];
     std::snprintf(name, sizeof name, "%s%s%s", st.record.device_kernel, one_launch ? "+" : " ; ", act);

@@ -293,3 +293,100 @@ def test_gated_projection_llama_prompt_as_dispatched(pkg, ctx):
     for t in (xdev, fused, gate_b, up_b, two):
         t.free()
     g.destroy(); u.destroy()
+
+
+@pytest.mark.parametrize("layout_name,x_name", [("LAYOUT_PLANES", "BF16"), ("LAYOUT_STAF_BLOCKS", "BF16"), ("LAYOUT_PLANES", "F16")])
+def test_gated_projection_on_the_streamed_weight_kernel(pkg, ctx, layout_name, x_name):
+    """A few dozen rows: gate_proj and up_proj as the two row blocks of every workgroup of the streamed-weight kernel,
+    activation(gate) * up in its epilogue, one launch.  Equal, bit for bit, to the two projections on that kernel (K in
+    one part there too: K below 2048) followed by the elementwise kernel, for one to three blocks of 32 activation
+    rows (the first with unrounded weights), ragged columns, every code width the kernel reads, every output type, both
+    activations and a padded result."""
+    layout, xd = getattr(pkg, layout_name), getattr(pkg, x_name)
+    cases = [(40, 100, 512, 4, 64), (96, 70, 768, 4, 128), (18, 33, 256, 8, 32), (64, 96, 1024, 8, 64),
+             (34, 65, 320, 3, 64), (70, 40, 192, 6, 64), (20, 64, 128, 2, 64), (66, 31, 256, 5, 64)]
+    for i, (m, n, k, bits, group) in enumerate(cases):
+        fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(bits, group)
+        sbo, sbp = (oracle.F16, pkg.F16) if layout == pkg.LAYOUT_STAF_BLOCKS else (oracle.BF16, pkg.BF16)
+        wg, sg, zg = oracle.quantize_affine(kat.seeded_weights(6700 + i, n, k), bits, group, sbo)
+        wu, su, zu = oracle.quantize_affine(kat.seeded_weights(6720 + i, n, k), bits, group, sbo)
+        g = ctx.weight_prepare_mlx(fmt, wg, sg, zg, sbp, layout)
+        u = ctx.weight_prepare_mlx(fmt, wu, su, zu, sbp, layout)
+        x = act_rounded(kat.seeded_activations(6740 + i, m, k), xd, pkg)
+        xdev = ctx.upload(act_to_device_array(x, xd, pkg))
+        for yd in (pkg.BF16, pkg.F32, pkg.F16):
+            esz = 4 if yd == pkg.F32 else 2
+            for kind in (pkg.GATED_SILU, pkg.GATED_GELU_TANH):
+                for y_pad in (0, 5):
+                    say(f"gated stream {layout_name} x={x_name} {m}x{n}x{k} q{bits} g{group} y={yd} act={kind} pad={y_pad}")
+                    ys = n + y_pad
+                    fused, gate_b, up_b, two = (ctx.alloc(m * ys * esz) for _ in range(4))
+                    ctx.fill(fused, 0x7FC07FC0 if esz == 2 else 0x7FC00000)
+                    ctx.fill(two, 0x7FC07FC0 if esz == 2 else 0x7FC00000)
+                    ctx.gated_qgemm(g, u, xdev, xd, fused, yd, m, kind, 0, ys if y_pad else 0, pkg.FLAG_FORCE_STREAM)
+                    ctx.qgemm(g, xdev, xd, gate_b, yd, m, 0, ys if y_pad else 0, pkg.FLAG_FORCE_STREAM)
+                    ctx.qgemm(u, xdev, xd, up_b, yd, m, 0, ys if y_pad else 0, pkg.FLAG_FORCE_STREAM)
+                    ctx.gated_activation(gate_b, up_b, two, yd, n, m, ys if y_pad else 0, kind)
+                    ctx.synchronize()
+                    dt = np.float32 if esz == 4 else np.uint16
+                    a, b = fused.download(dt, (m, ys)), two.download(dt, (m, ys))
+                    assert np.array_equal(a[:, :n], b[:, :n]), "one launch != two projections + elementwise kernel"
+                    if y_pad:
+                        pad = a[:, n:]
+                        assert np.all(np.isnan(pad)) if esz == 4 else np.all(pad == 0x7FC0), "padding of the output rows was written"
+                    for t in (fused, gate_b, up_b, two):
+                        t.free()
+        plan = pkg.DispatchPlan(ctx)
+        out = ctx.alloc(m * n * 2)
+        plan.add_gated_mlp(g, u, xdev, xd, out, pkg.BF16, m, activation=pkg.GATED_SILU, flags=pkg.FLAG_FORCE_STREAM)
+        st = plan.step(0)[0]
+        assert st.device_kernel == f"qgemm_stream_q{bits}_g{group}+swiglu" and st.kernel_family == f"gatedFusedQ{bits}G{group}", \
+            (st.device_kernel, st.kernel_family)
+        assert tuple(st.grid)[:2] == ((n + 31) // 32, 1) and st.rows_per_workgroup == 32
+        plan.destroy()
+        out.free(); xdev.free(); g.destroy(); u.destroy()
+
+
+def test_gated_projection_llama_64_rows_as_dispatched(pkg, ctx):
+    """Llama-3-8B's gate / up pair at 64 rows with no flags: one launch of the streamed-weight kernel (the plan record
+    names it, a graph replays it), equal to the two projections on that kernel and the elementwise kernel, and within the
+    bar of the oracle on a column sample."""
+    n, k, m = 14336, 4096, 64
+    wg, sg, zg, wq_g = seeded_case(6800, n, k, 4, 64)
+    wu, su, zu, wq_u = seeded_case(6801, n, k, 4, 64)
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+    g = ctx.weight_prepare_mlx(fmt, wg, sg, zg, pkg.BF16, pkg.LAYOUT_PLANES)
+    u = ctx.weight_prepare_mlx(fmt, wu, su, zu, pkg.BF16, pkg.LAYOUT_PLANES)
+    x = act_rounded(kat.seeded_activations(6802, m, k), pkg.BF16, pkg)
+    xdev = ctx.upload(act_to_device_array(x, pkg.BF16, pkg))
+    fused, gate_b, up_b, two = (ctx.alloc(m * n * 2) for _ in range(4))
+    stream = ctx.stream_create()
+    plan = pkg.DispatchPlan(ctx)
+    plan.add_gated_mlp(g, u, xdev, pkg.BF16, fused, pkg.BF16, m, activation=pkg.GATED_SILU)
+    st, _, _ = plan.step(0)
+    assert st.device_kernel == "qgemm_stream_q4_g64+swiglu" and st.kernel_family == "gatedFusedQ4G64", (st.device_kernel, st.kernel_family)
+    assert tuple(st.grid)[:2] == (448, 1)
+    ctx.qgemm(g, xdev, pkg.BF16, gate_b, pkg.BF16, m, flags=pkg.FLAG_FORCE_STREAM)
+    ctx.qgemm(u, xdev, pkg.BF16, up_b, pkg.BF16, m, flags=pkg.FLAG_FORCE_STREAM)
+    ctx.gated_activation(gate_b, up_b, two, pkg.BF16, n, m, 0, pkg.GATED_SILU)
+    ctx.synchronize()
+    b = two.download(np.uint16, (m, n))
+    plan.graph_build(stream)
+    for _ in range(3):
+        ctx.fill(fused, 0x7FC07FC0, stream)
+        plan.graph_launch(stream)
+        ctx.synchronize(stream)
+        assert np.array_equal(fused.download(np.uint16, (m, n)), b)
+    a = fused.download(np.uint16, (m, n))
+    cols = np.unique(np.concatenate([np.arange(0, n, n // 16), [1, 31, 32, 63, 64, n - 33, n - 1]]))
+    rows = np.unique(np.concatenate([np.arange(0, m, m // 8), [31, 32, m - 1]]))
+    bf = lambda w: oracle.bf16_to_f32(oracle.bf16_from_f32(w)).reshape(w.shape)
+    want = _expected(pkg, np.ascontiguousarray(bf(wq_g[cols])), np.ascontiguousarray(bf(wq_u[cols])), np.ascontiguousarray(x[rows]),
+                     pkg.GATED_SILU, pkg.BF16)
+    got = oracle.bf16_to_f32(a).reshape(m, n)[np.ix_(rows, cols)]
+    _check(pkg, got, want, pkg.BF16, "gated 64 rows")
+    plan.destroy()
+    ctx.stream_destroy(stream)
+    for t in (xdev, fused, gate_b, up_b, two):
+        t.free()
+    g.destroy(); u.destroy()
