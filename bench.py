@@ -624,6 +624,39 @@ def main():
             next_rows[label] = {"us": round(ms * 1e3, 2), "GBps": round(moved / (ms * 1e-3) / 1e9, 1), "bytes": moved}
         for b in (cache, rows, back):
             b.free()
+        # the gated MLP projection (gate_proj + up_proj + SwiGLU, 4096 -> 2 x 14336) as dispatched, beside the batched
+        # projection followed by the elementwise launch; the plan names what the one call runs
+        gated = {}
+        for mm in (1, 8, 64, 512, 2048):
+            xg = ctx.upload(oracle.bf16_from_f32(kat.seeded_activations(900 + mm, mm, 4096)))
+            yg, gb, ub = (ctx.alloc(mm * 14336 * 2) for _ in range(3))
+            nl = min(len(layers), 4)
+            one = lambda i: ctx.gated_qgemm(layers[i % nl]["gate"], layers[i % nl]["up"], xg, pkg.BF16, yg, pkg.BF16, mm,
+                                            pkg.GATED_SILU, 0, 0, 0, stream)
+            def apart(i):
+                ctx.batched_qgemm([layers[i % nl]["gate"], layers[i % nl]["up"]], xg, pkg.BF16, [gb, ub], pkg.BF16, mm, 0, 0, stream)
+                ctx.gated_activation(gb, ub, yg, pkg.BF16, 14336, mm, 0, pkg.GATED_SILU, stream)
+            for fn in (one, apart):
+                for i in range(4):
+                    fn(i)
+            ctx.synchronize(stream)
+            # samples of the two forms in turn, medians (whichever form is timed first after a change of shape reads
+            # 5 to 10 % slow)
+            reps = 48 if mm <= 64 else 16
+            samples = ([], [])
+            for _ in range(7):
+                samples[0].append(time_region(ctx, one, reps, stream))
+                samples[1].append(time_region(ctx, apart, reps, stream))
+            t_one, t_apart = (sorted(v)[len(v) // 2] for v in samples)
+            probe = pkg.DispatchPlan(ctx)
+            probe.add_gated_mlp(layers[0]["gate"], layers[0]["up"], xg, pkg.BF16, yg, pkg.BF16, mm, activation=pkg.GATED_SILU)
+            rec = probe.step(0)[0]
+            gated[f"M={mm}"] = {"us": round(t_one * 1e3, 2), "projections_then_elementwise_us": round(t_apart * 1e3, 2),
+                                "kernel": rec.device_kernel, "family": rec.kernel_family}
+            probe.destroy()
+            for b in (xg, yg, gb, ub):
+                b.free()
+        next_rows["gated MLP projection 4096 -> 2 x 14336 q4 g64 + swiglu, bf16"] = gated
         # container: one q4 g64 gate tensor written, opened, validated, uploaded as one device buffer, wrapped with no copy
         words, s_, z_ = host["gate"]
         blocks = pkg.repack_mlx_to_staf(fmt, words, s_, z_, pkg.BF16)
