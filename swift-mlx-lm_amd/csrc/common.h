@@ -80,11 +80,12 @@ struct mi355q_context {
     mi355q::DenseLibrary* dense_library;
     bool dense_library_failed;
     bool dense_library_forbidden;      // mi355q_context_set_library_use(ctx, 0): in-tree kernels only
-    // One stream per context at a time: the stream whose launches last used the scratch above, an event recorded
-    // behind them, and whether the entry point now running has touched the scratch (see ScratchGuard)
+    // One stream per context at a time: the stream whose launches last used the scratch above, an event that is
+    // recorded behind them when another stream turns up (or when that stream is destroyed through this library:
+    // scratch_marked), and whether the entry point now running has touched the scratch (see ScratchGuard)
     hipStream_t scratch_stream;
     hipEvent_t scratch_event;
-    bool scratch_pending, scratch_touched;
+    bool scratch_pending, scratch_touched, scratch_marked;
 };
 constexpr int kRetiredWorkspaces = 96;
 

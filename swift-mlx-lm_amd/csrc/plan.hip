@@ -218,10 +218,12 @@ mi355q_status mi355q_plan_add_gated_mlp(mi355q_plan* plan, const mi355q_weight* 
     const mi355q_weight* both[2] = {w_gate, w_up};
     plan_shared_launch_shape(both, 2, m, x_dtype, st.xs, flags, &st.record);
     // one launch with the activation as its epilogue, or the batched projection followed by the elementwise kernel
-    bool one_launch = !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_MFMA |
-                                 MI355Q_FLAG_FORCE_TWO_STEP | MI355Q_FLAG_FORCE_STREAM)) &&
+    // (as dispatch_gated decides: the one-launch forms read 16-byte aligned activations)
+    const bool x_aligned = (uintptr_t)x_dev % 16 == 0;
+    bool one_launch = x_aligned && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_FORCE_MFMA |
+                                              MI355Q_FLAG_FORCE_TWO_STEP | MI355Q_FLAG_FORCE_STREAM)) &&
                       gemv_gated_eligible(plan->ctx, w_gate->view(), w_up->view(), x_dtype, m, st.xs);
-    if (!one_launch && gemm_wide_gated_taken(plan->ctx, w_gate->view(), w_up->view(), x_dtype, m, st.xs, flags)) {
+    if (!one_launch && x_aligned && gemm_wide_gated_taken(plan->ctx, w_gate->view(), w_up->view(), x_dtype, m, st.xs, flags)) {
         // the wide-tile prefill kernel over both matrices: tiles of 128 output columns, K in one part
         one_launch = true;
         const GemmLaunchShape g = gemm_wide_shape(m, 2 * (uint32_t)w_gate->n, (uint32_t)w_gate->k, true);
@@ -233,7 +235,7 @@ mi355q_status mi355q_plan_add_gated_mlp(mi355q_plan* plan, const mi355q_weight* 
         st.record.rows_per_workgroup = 128;
         st.record.used_fallback = 0;
     }
-    if (!one_launch && gemm_stream_gated_taken(plan->ctx, w_gate->view(), w_up->view(), x_dtype, m, st.xs, flags)) {
+    if (!one_launch && x_aligned && gemm_stream_gated_taken(plan->ctx, w_gate->view(), w_up->view(), x_dtype, m, st.xs, flags)) {
         // the streamed-weight kernel, 32 output columns a workgroup, K in one part
         one_launch = true;
         const StreamLaunchShape g = gemm_stream_gated_shape(plan->ctx, m, (uint32_t)w_gate->n, (uint32_t)w_gate->k);

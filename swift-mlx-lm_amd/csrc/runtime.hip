@@ -61,35 +61,47 @@ mi355q_status grow_scratch(mi355q_context* ctx, void*& buffer, size_t& have, siz
 }
 }  // namespace
 
+// An entry point that uses the scratch only notes its stream (an event recorded behind every such call costs a caller on
+// one stream about 3 us a call: the launches no longer run back to back).  When a call on a second stream arrives, the
+// first stream is asked whether it has run dry -- everything it holds by then, which is at least the work that used the
+// scratch.  A stream destroyed through this library leaves an event in its place (scratch_marked).
 ScratchGuard::ScratchGuard(mi355q_context* c, hipStream_t s) : ctx(c), stream(s), status(MI355Q_OK) {
     if (!ctx) return;
     ctx->scratch_touched = false;
     if (!ctx->scratch_pending || ctx->scratch_stream == s || !s || !ctx->scratch_stream) return;
-    const hipError_t q = hipEventQuery(ctx->scratch_event);
+    hipError_t q;
+    if (ctx->scratch_marked) {
+        q = hipEventQuery(ctx->scratch_event);
+    } else {
+        // a stream that is being captured runs nothing; one that is gone (destroyed by its owner, which the runtime
+        // answers with an error) has nothing left to order against
+        hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(ctx->scratch_stream, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone)
+            q = hipSuccess;
+        else
+            q = hipStreamQuery(ctx->scratch_stream);
+    }
+    (void)hipGetLastError();
     if (q == hipErrorNotReady) {
-        (void)hipGetLastError();
         status = fail(MI355Q_ERR_INVALID_ARGUMENT,
                       "the context's scratch is still in use by work on another stream: one stream per context at a time "
                       "(synchronise the first stream, or give each stream a context of its own)");
         return;
     }
-    (void)hipGetLastError();
     ctx->scratch_pending = false;
+    ctx->scratch_marked = false;
 }
 
 ScratchGuard::~ScratchGuard() {
-    if (!ctx || status != MI355Q_OK || !ctx->scratch_touched || !ctx->scratch_event) return;
+    if (!ctx || status != MI355Q_OK || !ctx->scratch_touched) return;
     hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
     if (stream && (hipStreamIsCapturing(stream, &capture) != hipSuccess || capture != hipStreamCaptureStatusNone)) {
         (void)hipGetLastError();
         return;
     }
-    if (hipEventRecord(ctx->scratch_event, stream) == hipSuccess) {
-        ctx->scratch_stream = stream;
-        ctx->scratch_pending = true;
-    } else {
-        (void)hipGetLastError();
-    }
+    ctx->scratch_stream = stream;
+    ctx->scratch_pending = true;
+    ctx->scratch_marked = false;
 }
 
 mi355q_status ensure_workspace(mi355q_context* ctx, size_t bytes) {
@@ -460,6 +472,19 @@ mi355q_status mi355q_stream_create(mi355q_context* ctx, void** out_stream) {
 }
 mi355q_status mi355q_stream_destroy(mi355q_context* ctx, void* stream) {
     if (mi355q_status s = need_ctx(ctx)) return s;
+    if (stream && ctx->scratch_pending && ctx->scratch_stream == (hipStream_t)stream && !ctx->scratch_marked) {
+        // the stream that last used the scratch goes: if it still holds work, an event takes its place
+        if (hipStreamQuery((hipStream_t)stream) != hipErrorNotReady) {
+            (void)hipGetLastError();
+            ctx->scratch_pending = false;
+        } else if (hipEventRecord(ctx->scratch_event, (hipStream_t)stream) == hipSuccess) {
+            ctx->scratch_marked = true;
+            ctx->scratch_stream = (hipStream_t)(uintptr_t)1;       // (no live stream: a new one may get the old address)
+        } else {
+            (void)hipGetLastError();
+            ctx->scratch_pending = false;
+        }
+    }
     if (stream) MI355Q_HIP(hipStreamDestroy((hipStream_t)stream));
     return MI355Q_OK;
 }
