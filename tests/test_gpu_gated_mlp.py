@@ -390,3 +390,34 @@ def test_gated_projection_llama_64_rows_as_dispatched(pkg, ctx):
     for t in (xdev, fused, gate_b, up_b, two):
         t.free()
     g.destroy(); u.destroy()
+
+
+def test_gated_projection_forced_onto_the_streamed_weight_kernel_keeps_k_in_one_part(pkg, ctx):
+    """Few outputs and a long K, where a projection alone splits K over workgroups: forced onto the streamed-weight kernel
+    the gated launch walks K in one part (a partial sum cannot be gated) and agrees with the two projections (K in
+    parts, another order of the fp32 sums) followed by the elementwise kernel to 1e-5 of the largest output."""
+    m, n, k = 48, 96, 4096
+    fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, 64)
+    wg, sg, zg = oracle.quantize_affine(kat.seeded_weights(6900, n, k), 4, 64, oracle.BF16)
+    wu, su, zu = oracle.quantize_affine(kat.seeded_weights(6901, n, k), 4, 64, oracle.BF16)
+    g = ctx.weight_prepare_mlx(fmt, wg, sg, zg, pkg.BF16, pkg.LAYOUT_PLANES)
+    u = ctx.weight_prepare_mlx(fmt, wu, su, zu, pkg.BF16, pkg.LAYOUT_PLANES)
+    assert g.plan_prefill_steps(m, 0, pkg.BF16, flags=pkg.FLAG_FORCE_STREAM)[0].grid[1] > 1, "the projection alone is meant to split K"
+    x = act_rounded(kat.seeded_activations(6902, m, k), pkg.BF16, pkg)
+    xdev = ctx.upload(act_to_device_array(x, pkg.BF16, pkg))
+    fused, gate_b, up_b, two = (ctx.alloc(m * n * 4) for _ in range(4))
+    ctx.gated_qgemm(g, u, xdev, pkg.BF16, fused, pkg.F32, m, pkg.GATED_SILU, 0, 0, pkg.FLAG_FORCE_STREAM)
+    ctx.qgemm(g, xdev, pkg.BF16, gate_b, pkg.F32, m, 0, 0, pkg.FLAG_FORCE_STREAM)
+    ctx.qgemm(u, xdev, pkg.BF16, up_b, pkg.F32, m, 0, 0, pkg.FLAG_FORCE_STREAM)
+    ctx.gated_activation(gate_b, up_b, two, pkg.F32, n, m, 0, pkg.GATED_SILU)
+    ctx.synchronize()
+    a, b = fused.download(np.float32, (m, n)), two.download(np.float32, (m, n))
+    assert np.all(np.isfinite(a)) and float(np.max(np.abs(a - b))) <= 1e-5 * float(np.max(np.abs(b))), float(np.max(np.abs(a - b)))
+    plan = pkg.DispatchPlan(ctx)
+    plan.add_gated_mlp(g, u, xdev, pkg.BF16, fused, pkg.F32, m, activation=pkg.GATED_SILU, flags=pkg.FLAG_FORCE_STREAM)
+    st = plan.step(0)[0]
+    assert st.device_kernel == "qgemm_stream_q4_g64+swiglu" and tuple(st.grid)[:2] == (3, 1), (st.device_kernel, tuple(st.grid))
+    plan.destroy()
+    for t in (xdev, fused, gate_b, up_b, two):
+        t.free()
+    g.destroy(); u.destroy()
