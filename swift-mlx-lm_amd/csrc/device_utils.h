@@ -79,12 +79,22 @@ __device__ __forceinline__ float round_to_dtype(float v, uint32_t dtype) {
     if (dtype == MI355Q_F16) return f16_to_f32(f32_to_f16_rne(v));
     return v;
 }
+// 1 / (1 + exp(-t)) on the hardware's 2^x and reciprocal (one unit in the last place each); the rounding of the product
+// t * log2(e), which would grow with |t|, is put back to first order.  Within 4e-7 relative of the formula; exp and
+// an IEEE division (45 instructions an output with the roundings, against 20) were what the activation cost the
+// epilogues of the matrix-core kernels.
+__device__ __forceinline__ float sigmoid_f32(float t) {
+    const float p = t * -1.4426950408889634f;
+    const float lost = __builtin_fmaf(t, -1.4426950408889634f, -p);        // exact: what the product's rounding dropped
+    const float e = __builtin_amdgcn_exp2f(p) * __builtin_fmaf(lost, 0.6931471805599453f, 1.0f);   // (inf stays inf)
+    return __builtin_amdgcn_rcpf(1.0f + e);
+}
+// swiglu: g * sigmoid(g) * u.  gelu_gated: 0.5 g (1 + tanh(y)) u with y = 0.7978845608 (g + 0.044715 g^3), which is
+// g * sigmoid(2 y) * u, the identity 0.5 (1 + tanh(y)) = sigmoid(2 y).
 __device__ __forceinline__ float gated_value(float gate, float up, uint32_t activation, uint32_t dtype) {
     const float g = round_to_dtype(gate, dtype), u = round_to_dtype(up, dtype);
-    float act;
-    if (activation == MI355Q_GATED_GELU_TANH) act = 0.5f * g * (1.0f + tanhf(0.7978845608f * (g + 0.044715f * g * g * g)));
-    else act = g * (1.0f / (1.0f + expf(-g)));
-    return act * u;
+    const float t = activation == MI355Q_GATED_GELU_TANH ? 1.5957691216f * (g + 0.044715f * g * g * g) : g;
+    return g * sigmoid_f32(t) * u;
 }
 
 __device__ __forceinline__ float sb_to_f32(uint16_t h, uint32_t sb_dtype) {

@@ -255,12 +255,13 @@ bool gemm_wide_gated_chosen(const WView& gate, const WView& up, int x_dtype, uin
     if (!gemm_wide_gated_eligible(gate, up, x_dtype, m, x_stride) || m < kWideMinRows) return false;
     const GemmLaunchShape g = gemm_wide_shape(m, 2 * gate.n, gate.k, true);
     const uint32_t wgs = ((m + g.bm - 1) / g.bm) * ((gate.n + kWideBN / 2 - 1) / (kWideBN / 2));
-    // Up to two rounds of tiles.  The activation costs the matrix-core wavefronts about 10 us a tile (two roundings, an
-    // exponential and a division per output), which the elementwise launch it replaces (65 us at 2048 rows of 14336, bound
-    // by its 176 MB of traffic) spends beside nothing: 4096 -> 2 x 14336 at 256 rows 70 us against 102 for the two
-    // projections and the elementwise launch, at 512 rows 121 against 144, at 1024 rows 240 against 243, at 2048 rows
-    // (3.5 rounds) 484 against 475.
-    return 8 * wgs >= 5 * chip_cus() && wgs <= 2 * chip_cus();
+    // K stays in one part (a partial sum cannot be gated), so the tiles alone must fill the chip.  The activation costs
+    // the matrix-core wavefronts about 5 us a round of tiles (two roundings, a 2^x and a reciprocal per output), the
+    // elementwise launch it replaces 65 us at 2048 rows of 14336: 4096 -> 2 x 14336 at 256 rows 66 us against 100 for
+    // the two projections and the elementwise launch, at 512 rows 108 against 144, at 1024 rows 209 against 236, at
+    // 2048 rows 422 against 463.  (With exp and an IEEE division in the activation, 10 us a round, the one launch won
+    // only up to two rounds of tiles: 484 against 475 at 2048 rows.)
+    return 8 * wgs >= 5 * chip_cus();
 }
 
 bool gemm_wide_gated_taken(const mi355q_context* ctx, const WView& gate, const WView& up, int x_dtype, uint32_t m, uint32_t x_stride,

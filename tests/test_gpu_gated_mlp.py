@@ -257,7 +257,7 @@ def test_gated_projection_on_the_prefill_kernel(pkg, ctx, layout_name, x_name):
 def test_gated_projection_llama_prompt_as_dispatched(pkg, ctx):
     """Llama-3-8B's gate / up pair at 512 rows with no flags: one launch on the wide-tile kernel (the plan record names
     it), equal to the two projections and the elementwise kernel, and within the bar of the oracle on a column sample;
-    at 2048 rows (more than two rounds of tiles) the plan keeps the projections and the elementwise launch apart."""
+    the plan of 2048 rows names the same launch over 896 tiles."""
     n, k, m = 14336, 4096, 512
     wg, sg, zg, wq_g = seeded_case(6600, n, k, 4, 64)
     wu, su, zu, wq_u = seeded_case(6601, n, k, 4, 64)
@@ -273,7 +273,9 @@ def test_gated_projection_llama_prompt_as_dispatched(pkg, ctx):
     assert st.device_kernel == "qgemm_wide_q4_g64+swiglu" and st.kernel_family == "gatedFusedQ4G64", (st.device_kernel, st.kernel_family)
     far = pkg.DispatchPlan(ctx)
     far.add_gated_mlp(g, u, xdev, pkg.BF16, fused, pkg.BF16, 2048, activation=pkg.GATED_SILU)     # (described, not run)
-    assert far.step(0)[0].kernel_family == "gatedBatched2Q4G64" and far.step(0)[0].device_kernel == "qgemm_wide_q4_g64 ; swiglu"
+    rec = far.step(0)[0]
+    assert rec.kernel_family == "gatedFusedQ4G64" and rec.device_kernel == "qgemm_wide_q4_g64+swiglu" and tuple(rec.grid)[:2] == (896, 1), \
+        (rec.kernel_family, rec.device_kernel, tuple(rec.grid))
     far.destroy()
     plan.encode(0)
     ctx.qgemm(g, xdev, pkg.BF16, gate_b, pkg.BF16, m)
