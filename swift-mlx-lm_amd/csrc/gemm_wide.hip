@@ -261,7 +261,11 @@ bool gemm_wide_gated_chosen(const WView& gate, const WView& up, int x_dtype, uin
     // the two projections and the elementwise launch, at 512 rows 108 against 144, at 1024 rows 209 against 236, at
     // 2048 rows 422 against 463.  (With exp and an IEEE division in the activation, 10 us a round, the one launch won
     // only up to two rounds of tiles: 484 against 475 at 2048 rows.)
-    return 8 * wgs >= 5 * chip_cus();
+    // One row of 128-row tiles (97 to 128 rows): from a quarter of the CUs, where the projections apart split K and
+    // add their parts (128 rows of 4096 -> 2 x N: N = 6144, 48 workgroups, 59 us either way; 8192 59 against 62;
+    // 11008 60 against 63; 14336 60 against 69).
+    const uint32_t eighths = g.bm == 128 && m <= 128 ? 2 : 5;
+    return 8 * wgs >= eighths * chip_cus();
 }
 
 bool gemm_wide_gated_taken(const mi355q_context* ctx, const WView& gate, const WView& up, int x_dtype, uint32_t m, uint32_t x_stride,

@@ -277,6 +277,12 @@ def test_gated_projection_llama_prompt_as_dispatched(pkg, ctx):
     assert rec.kernel_family == "gatedFusedQ4G64" and rec.device_kernel == "qgemm_wide_q4_g64+swiglu" and tuple(rec.grid)[:2] == (896, 1), \
         (rec.kernel_family, rec.device_kernel, tuple(rec.grid))
     far.destroy()
+    near = pkg.DispatchPlan(ctx)                  # one row of 128-row tiles: 112 workgroups, K in one part
+    near.add_gated_mlp(g, u, xdev, pkg.BF16, fused, pkg.BF16, 128, activation=pkg.GATED_SILU)
+    rec = near.step(0)[0]
+    assert rec.kernel_family == "gatedFusedQ4G64" and rec.device_kernel == "qgemm_wide_q4_g64+swiglu" and tuple(rec.grid)[:2] == (112, 1), \
+        (rec.kernel_family, rec.device_kernel, tuple(rec.grid))
+    near.destroy()
     plan.encode(0)
     ctx.qgemm(g, xdev, pkg.BF16, gate_b, pkg.BF16, m)
     ctx.qgemm(u, xdev, pkg.BF16, up_b, pkg.BF16, m)
