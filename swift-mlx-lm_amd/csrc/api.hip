@@ -414,6 +414,8 @@ mi355q_status dispatch_batched(mi355q_context* ctx, hipStream_t s, uint32_t coun
                                         HeadKeys{});
     case SharedRoute::kStafInPlace:
         return launch_gemv_staf_multi(s, ctx, count, views, x, x_dtype, ys, strides, y_dtype, m, xs, nullptr, nullptr, HeadKeys{});
+    case SharedRoute::kWide:
+        return launch_qgemm_wide_multi(s, ctx, count, views, x, x_dtype, ys, strides, y_dtype, m, xs);
     case SharedRoute::kSplitRows: {
         const uint32_t parts = split_rows_parts(x_dtype);
         const uint32_t k = (uint32_t)views[0].k, kp = split_rows_stride(k);

@@ -331,6 +331,7 @@ enum class SharedRoute : int {
     kDotPlanes,        // the dot-product decode kernels over the planes
     kTile16,           // the matrix-core kernel over TILE16 records
     kStafInPlace,      // the in-place kernel over the reference's blocks
+    kWide,             // prompts: the wide-tile prefill kernel over the column tiles of all matrices
     kSplitRows,        // fp32 rows split into bf16 rows once for all projections, then one of the above on those
     kSteps,            // more rows than one shared launch takes: the shared launch in steps
     kSeparate,         // each projection on its own route (linear_route)
@@ -388,6 +389,15 @@ GemmLaunchShape gemm_wide_shape(uint32_t m, uint32_t n, uint32_t k, bool one_par
 inline uint32_t gemm_wide_k(uint32_t k, int x_dtype) { return x_dtype == MI355Q_F32 ? 2 * k : k; }
 uint32_t chip_cus();
 void gemm_wide_force_shape(uint32_t bm, uint32_t splits);      // A/B runs (mi355q_probe_wide_shape)
+// Two or three matrices that share the activations as one launch of the wide-tile kernel: every column tile belongs to
+// one matrix (all but the last are whole numbers of 256-column tiles), K parts and their sum over the columns of all.
+// `chosen`: from the rows where the streamed-weight kernel ends (measured against a launch per projection).
+bool gemm_wide_multi_eligible(uint32_t count, const WView* w, int x_dtype, uint32_t m, uint32_t x_stride);
+bool gemm_wide_multi_chosen(uint32_t count, const WView* w, int x_dtype, uint32_t m, uint32_t x_stride);
+GemmLaunchShape gemm_wide_multi_shape(uint32_t count, const WView* w, uint32_t m);
+mi355q_status launch_qgemm_wide_multi(hipStream_t s, mi355q_context* ctx, uint32_t count, const WView* w, const void* x,
+                                      int x_dtype, void* const* y, const uint32_t* y_strides, int y_dtype, uint32_t m,
+                                      uint32_t x_stride);
 // The gated MLP projection on the wide-tile kernel: gate_proj and up_proj as the two column fragments of every
 // wavefront, activation(gate) * up in the epilogue, one launch and no intermediate matrices.  Chosen under the same
 // rule as the plain kernel, over the 2 N columns of the two matrices, K in one part.

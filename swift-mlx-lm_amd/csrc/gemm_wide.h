@@ -28,6 +28,16 @@ struct WideArgs {
     const uint32_t* codes_up;
     const uint32_t* sz_up;
     const uint8_t* blocks_up;
+    // two or three matrices that share the activations (q+k+v, gate+up) as one launch: `segments` > 1, the column tiles
+    // [0, seg_tile0[0]) belong to the matrix above, [seg_tile0[0], seg_tile0[1]) to seg_*[0], the rest to seg_*[1] (two
+    // matrices: seg_tile0[1] = tiles_n); every matrix but the last is a whole number of 256-column tiles; tiles_n is
+    // given; K parts land at column seg_col0 of fp32 rows of n_total columns
+    uint32_t segments;
+    uint32_t seg_tile0[2], seg_n[2], seg_ys[2], seg_col0[2], n_total;
+    const uint32_t* seg_codes[2];
+    const uint32_t* seg_sz[2];
+    const uint8_t* seg_blocks[2];
+    void* seg_y[2];
     unsigned long long* probe;   // optional: [0] shader cycles, [1] 100 MHz ticks that workgroup 0 spent in the kernel
 };
 

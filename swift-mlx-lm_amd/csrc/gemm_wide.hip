@@ -242,6 +242,127 @@ mi355q_status launch_qgemm_wide(hipStream_t s, mi355q_context* ctx, const WView&
     return MI355Q_OK;
 }
 
+// ---- two or three matrices that share the activations ----------------------------------------------------------------
+namespace {
+struct WideSumArgs {
+    const float* partial;      // [splits][m][n_total]
+    void* y[3];
+    uint32_t ys[3], col_end[3];
+    uint32_t m, n_total, splits, y_dtype;
+};
+// Sum of the K parts in part order, four columns a thread (every matrix is a multiple of four columns wide), each
+// matrix's columns to its own result.
+__global__ __launch_bounds__(256) void wide_reduce_multi_kernel(WideSumArgs a) {
+    const size_t total = (size_t)a.m * a.n_total / 4;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const wd_float4_v* const p = (const wd_float4_v*)a.partial + i;
+        wd_float4_v v = __builtin_nontemporal_load(p);
+        for (uint32_t s = 1; s < a.splits; s++) v += __builtin_nontemporal_load(p + (size_t)s * total);
+        const size_t e = i * 4, row = e / a.n_total;
+        const uint32_t pcol = (uint32_t)(e - row * a.n_total);
+        const uint32_t sg = pcol >= a.col_end[1] ? 2u : pcol >= a.col_end[0] ? 1u : 0u;
+        const uint32_t col = pcol - (sg == 2 ? a.col_end[1] : sg == 1 ? a.col_end[0] : 0u);
+        void* const y = sg == 2 ? a.y[2] : sg == 1 ? a.y[1] : a.y[0];
+        const size_t o = row * (sg == 2 ? a.ys[2] : sg == 1 ? a.ys[1] : a.ys[0]) + col;
+        const float f[4] = {v.x, v.y, v.z, v.w};
+        for (int c = 0; c < 4; c++) {
+            if (a.y_dtype == MI355Q_F32) ((float*)y)[o + c] = f[c];
+            else if (a.y_dtype == MI355Q_BF16) ((uint16_t*)y)[o + c] = f32_to_bf16_rne(f[c]);
+            else ((uint16_t*)y)[o + c] = f32_to_f16_rne(f[c]);
+        }
+    }
+}
+}  // namespace
+
+bool gemm_wide_multi_eligible(uint32_t count, const WView* w, int x_dtype, uint32_t m, uint32_t x_stride) {
+    if (count < 2 || count > 3 || (x_dtype != MI355Q_BF16 && x_dtype != MI355Q_F16)) return false;
+    uint64_t total = 0;
+    for (uint32_t i = 0; i < count; i++) {
+        if (!gemm_wide_eligible(w[i], x_dtype, m, x_stride)) return false;
+        if (w[i].k != w[0].k || w[i].layout != w[0].layout || w[i].group != w[0].group || w[i].bits != w[0].bits ||
+            w[i].sb_dtype != w[0].sb_dtype || w[i].code_stride != w[0].code_stride || w[i].sz_stride != w[0].sz_stride ||
+            w[i].blocks_per_row != w[0].blocks_per_row || w[i].bytes_per_block != w[0].bytes_per_block)
+            return false;
+        if (w[i].n % 4 || (i + 1 < count && w[i].n % kWideBN)) return false;     // whole tiles; K parts in 16-byte pieces
+        total += w[i].n;
+    }
+    return total < (1ull << 31);
+}
+
+GemmLaunchShape gemm_wide_multi_shape(uint32_t count, const WView* w, uint32_t m) {
+    uint32_t total = 0;
+    for (uint32_t i = 0; i < count; i++) total += w[i].n;
+    return gemm_wide_shape(m, total, w[0].k);
+}
+
+// From the rows where the streamed-weight kernel ends, whatever the size: against a launch per projection (each with
+// its own K parts and sum) the one launch took half the time wherever it was measured -- q+k+v 4096 -> 4096 + 1024 +
+// 1024 at 97 / 128 / 512 / 2048 rows 26 / 28 / 49 / 94 us against 57 / 58 / 88 / 135, 2048 + 512 + 512 at 97 to 384
+// rows 25-32 against 50-64, 1024 + 256 + 256 23-32 against 51-68, two of 256 columns 23-27 against 35-43, gate+up
+// 2 x 8192 at 97 to 384 rows 34-63 against 57-111, 2 x 14336 at 128 / 512 rows 50 / 107 against 65 / 131.
+bool gemm_wide_multi_chosen(uint32_t count, const WView* w, int x_dtype, uint32_t m, uint32_t x_stride) {
+    return gemm_wide_multi_eligible(count, w, x_dtype, m, x_stride) && m >= kWideMinRows;
+}
+
+mi355q_status launch_qgemm_wide_multi(hipStream_t s, mi355q_context* ctx, uint32_t count, const WView* w, const void* x,
+                                      int x_dtype, void* const* y, const uint32_t* y_strides, int y_dtype, uint32_t m,
+                                      uint32_t x_stride) {
+    if (!gemm_wide_multi_eligible(count, w, x_dtype, m, x_stride))
+        return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the wide-tile MFMA GEMM does not take these weights as one launch");
+    if ((uintptr_t)x % 16) return fail(MI355Q_ERR_INVALID_ARGUMENT, "activation pointer must be 16-byte aligned");
+    const GemmLaunchShape g = gemm_wide_multi_shape(count, w, m);
+    WideArgs a{};
+    const bool blocks = w[0].layout == MI355Q_LAYOUT_STAF_BLOCKS;
+    const size_t esz = y_dtype == MI355Q_F32 ? 4 : 2;
+    a.codes = w[0].codes; a.sz = w[0].sz; a.blocks = w[0].blocks;
+    a.y = y[0]; a.n = w[0].n; a.ys = y_strides[0];
+    a.segments = count;
+    a.wide_stores = 1; a.line_stores = 1;
+    uint32_t tiles = 0, cols = 0;
+    WideSumArgs sum{};
+    for (uint32_t i = 0; i < count; i++) {
+        if (i) {
+            a.seg_tile0[i - 1] = tiles; a.seg_col0[i - 1] = cols;
+            a.seg_codes[i - 1] = w[i].codes; a.seg_sz[i - 1] = w[i].sz; a.seg_blocks[i - 1] = w[i].blocks;
+            a.seg_y[i - 1] = y[i]; a.seg_n[i - 1] = w[i].n; a.seg_ys[i - 1] = y_strides[i];
+        }
+        tiles += (w[i].n + kWideBN - 1) / kWideBN;
+        cols += w[i].n;
+        sum.y[i] = y[i]; sum.ys[i] = y_strides[i]; sum.col_end[i] = cols;
+        if (y_strides[i] % 4 || (uintptr_t)y[i] % 16) a.wide_stores = 0;
+        if ((size_t)y_strides[i] * esz % 16 || (uintptr_t)y[i] % 16) a.line_stores = 0;
+    }
+    if (count == 2) {                                  // no third matrix: nothing reaches it
+        a.seg_tile0[1] = 0xFFFFFFFFu;
+        sum.y[2] = y[1]; sum.ys[2] = y_strides[1]; sum.col_end[1] = 0xFFFFFFFFu; sum.col_end[2] = 0xFFFFFFFFu;
+    }
+    a.tiles_n = tiles;
+    a.n_total = cols;
+    a.row_bytes = w[0].blocks_per_row * w[0].bytes_per_block;
+    a.x = (const uint16_t*)x;
+    a.m = m; a.k = w[0].k; a.xs = x_stride;
+    a.w_fours = w[0].k / 256;
+    a.code_stride = w[0].code_stride; a.sz_stride = w[0].sz_stride;
+    a.y_dtype = (uint32_t)y_dtype;
+    a.splits = g.splits; a.kt_per_split = g.kt_per_split;
+    if (g.splits > 1) {
+        if (mi355q_status st = ensure_workspace(ctx, (size_t)g.splits * m * cols * sizeof(float))) return st;
+        a.partial = (float*)ctx->workspace;
+    }
+    const bool sb_bf16 = w[0].sb_dtype == MI355Q_BF16;
+    if (mi355q_status st = x_dtype == MI355Q_F16 ? launch_wide_kernel_f16(s, a, g.bm, w[0].group, sb_bf16, blocks)
+                                                 : launch_wide_kernel_bf16(s, a, g.bm, w[0].group, sb_bf16, blocks))
+        return st;
+    if (a.partial) {
+        sum.partial = a.partial; sum.m = m; sum.n_total = cols; sum.splits = g.splits; sum.y_dtype = (uint32_t)y_dtype;
+        size_t wgs = ((size_t)m * cols / 4 + 255) / 256;
+        if (wgs > 16384) wgs = 16384;
+        wide_reduce_multi_kernel<<<dim3((unsigned)wgs), dim3(256), 0, s>>>(sum);
+        MI355Q_HIP(hipGetLastError());
+    }
+    return MI355Q_OK;
+}
+
 // ---- gated MLP projection ------------------------------------------------------------------------------------------
 bool gemm_wide_gated_eligible(const WView& gate, const WView& up, int x_dtype, uint32_t m, uint32_t x_stride) {
     if (x_dtype != MI355Q_BF16 && x_dtype != MI355Q_F16) return false;

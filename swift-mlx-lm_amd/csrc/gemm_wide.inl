@@ -60,7 +60,20 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
     const uint32_t t_id = (blockIdx.x % 8u) * per_xcd + blockIdx.x / 8u;
     if (t_id >= total) return;
     const uint32_t split = (uint32_t)__builtin_amdgcn_readfirstlane((int)(t_id / tiles)), tile = t_id - split * tiles;
-    const uint32_t tn = tile / a.tiles_m, tm = tile % a.tiles_m;
+    const uint32_t tn_all = tile / a.tiles_m, tm = tile % a.tiles_m;
+    // the matrix of this column tile (one of up to three that share the activations): its weights here, its result in
+    // the epilogue, which asks again -- nothing of the choice is kept in registers over the K loop but the tile's number
+    uint32_t tn = tn_all;
+    const uint32_t* seg_codes = a.codes;
+    const uint32_t* seg_sz = a.sz;
+    const uint8_t* seg_blocks = a.blocks;
+    uint32_t w_n = a.n;
+    if (a.segments > 1 && tn_all >= a.seg_tile0[0]) {
+        const uint32_t sg_ = tn_all >= a.seg_tile0[1] ? 1u : 0u;
+        seg_codes = a.seg_codes[sg_]; seg_sz = a.seg_sz[sg_]; seg_blocks = a.seg_blocks[sg_];
+        w_n = a.seg_n[sg_];
+        tn -= a.seg_tile0[sg_];
+    }
     // Gated (a.gated != 0): the two 32-column fragments of a wavefront are the same 32 output columns of gate_proj and of
     // up_proj, so a tile is 128 output columns wide and activation(gate) * up is formed in the registers of the epilogue.
     const uint32_t tile_cols = a.gated ? kWideBN / 2 : kWideBN;
@@ -98,7 +111,7 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
     };
     // ---- weights: global -> registers, four K-tiles at a time -------------------------------------------
     // lane (n, h) of fragment f holds codes 32 h .. 32 h + 31 of each K-tile of row 64 w + 32 f + n
-    const uint32_t n_last = a.n - 1 - n0;
+    const uint32_t n_last = w_n - 1 - n0;
     uint32_t w_off[2], sz_off[2];
 #pragma unroll
     for (int f = 0; f < 2; f++) {
@@ -112,8 +125,8 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
             sz_off[f] = gr * a.sz_stride * 4;
         }
     }
-    const char* const cg = BLOCKS ? (const char*)a.blocks + (size_t)n0 * a.row_bytes : (const char*)(a.codes + (size_t)n0 * a.code_stride);
-    const char* const sg = BLOCKS ? cg : (const char*)(a.sz + (size_t)n0 * a.sz_stride);
+    const char* const cg = BLOCKS ? (const char*)seg_blocks + (size_t)n0 * a.row_bytes : (const char*)(seg_codes + (size_t)n0 * a.code_stride);
+    const char* const sg = BLOCKS ? cg : (const char*)(seg_sz + (size_t)n0 * a.sz_stride);
     // the second fragment's matrix: up_proj where gated, else the same one
     const char* const cg1 = !a.gated ? cg : BLOCKS ? (const char*)a.blocks_up + (size_t)n0 * a.row_bytes
                                                    : (const char*)(a.codes_up + (size_t)n0 * a.code_stride);
@@ -338,6 +351,18 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
     }
 
     // ---- epilogue: one rounding, to the output type -----------------------------------------------------
+    // the result of this tile's matrix (asked again, from a copy of the tile's number the compiler takes for another)
+    uint32_t tn_again = tn_all;
+    asm volatile("" : "+s"(tn_again));
+    void* seg_y = a.y;
+    uint32_t seg_n = a.n, seg_ys = a.ys, part_col0 = 0, part_pitch = a.n;
+    if (a.segments > 1) {
+        part_pitch = a.n_total;
+        if (tn_again >= a.seg_tile0[0]) {
+            const uint32_t sg_ = tn_again >= a.seg_tile0[1] ? 1u : 0u;
+            seg_y = a.seg_y[sg_]; seg_n = a.seg_n[sg_]; seg_ys = a.seg_ys[sg_]; part_col0 = a.seg_col0[sg_];
+        }
+    }
     // lane (m, h) of accumulator (f, i) holds row m0 + 32 i + m, columns 32 f + 8 g + 4 h + (0 .. 3) for g = 0 .. 3.
     // One accumulator at a time (the fences keep the compiler from fetching all 256 registers first).
     auto store_tiles = [&](auto DT, void* const y, const size_t ys, const bool wide) __attribute__((always_inline)) {
@@ -355,7 +380,7 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
                         const uint32_t col = n0 + 64 * wave + 32 * f + 8 * g + 4 * lh;
                         const float v[4] = {acc[f][i][4 * g + 0], acc[f][i][4 * g + 1], acc[f][i][4 * g + 2], acc[f][i][4 * g + 3]};
                         const size_t o = (size_t)row * ys + col;
-                        if (wide && col + 3 < a.n) {
+                        if (wide && col + 3 < seg_n) {
                             if constexpr (dt == MI355Q_F32) {
                                 const float4 t = {v[0], v[1], v[2], v[3]};
                                 *(float4*)((float*)y + o) = t;
@@ -372,7 +397,7 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
                         } else {
 #pragma unroll
                             for (int e = 0; e < 4; e++)
-                                if (col + e < a.n) store_out<dt>(y, o + e, v[e]);
+                                if (col + e < seg_n) store_out<dt>(y, o + e, v[e]);
                         }
                     }
                 }
@@ -438,7 +463,7 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
         constexpr int LPR = 32 * ESZ / 16;                         // lanes per row of the read-back
         constexpr int RPI = 64 / LPR;                              // rows per read-back instruction
         char* const stage = lds + wave * (32 * PITCH);
-        const bool whole = n0 + kWideBN / 2 <= a.n && a.line_stores;
+        const bool whole = n0 + kWideBN / 2 <= seg_n && a.line_stores;
         const uint32_t act = a.gated - 1;
         __builtin_amdgcn_s_barrier();                              // every wavefront is done with the activation stages
         static_for<TM>([&](auto I) __attribute__((always_inline)) {
@@ -470,7 +495,7 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
                     const u32x4 d = *(const u32x4*)(stage + r * PITCH + piece * 16);
                     const uint32_t row = m0 + i * 32 + r;
                     if (row < a.m)
-                        *(u32x4*)((char*)a.y + ((size_t)row * a.ys + n0 + 32 * wave) * ESZ + piece * 16) = d;
+                        *(u32x4*)((char*)seg_y + ((size_t)row * seg_ys + n0 + 32 * wave) * ESZ + piece * 16) = d;
                 }
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                 __builtin_amdgcn_wave_barrier();
@@ -481,7 +506,7 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
 #pragma unroll
                     for (int r = 0; r < 16; r++) {
                         const uint32_t col = n0 + 32 * wave + 8 * (r / 4) + 4 * lh + r % 4;
-                        if (col < a.n) store_out<dt>(a.y, (size_t)row * a.ys + col, v[r]);
+                        if (col < seg_n) store_out<dt>(seg_y, (size_t)row * seg_ys + col, v[r]);
                     }
                 }
             }
@@ -494,23 +519,23 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
         else store_gated(std::integral_constant<int, MI355Q_F16>{});
         return;
     }
-    const bool inner = n0 + kWideBN <= a.n;                        // (uniform over the workgroup)
+    const bool inner = n0 + kWideBN <= seg_n;                        // (uniform over the workgroup)
     if (a.partial) {       // this part of K as fp32 (N is a multiple of four: 16-byte stores); wide_reduce_kernel adds the parts
-        float* const part = a.partial + (size_t)split * a.m * a.n;
-        if (inner) store_lines(std::integral_constant<int, MI355Q_F32>{}, part, a.n);
-        else store_tiles(std::integral_constant<int, MI355Q_F32>{}, part, a.n, true);
+        float* const part = a.partial + (size_t)split * a.m * part_pitch + part_col0;
+        if (inner) store_lines(std::integral_constant<int, MI355Q_F32>{}, part, part_pitch);
+        else store_tiles(std::integral_constant<int, MI355Q_F32>{}, part, part_pitch, true);
         return;
     }
     const bool lines = inner && a.line_stores;
     if (a.y_dtype == MI355Q_BF16) {
-        if (lines) store_lines(std::integral_constant<int, MI355Q_BF16>{}, a.y, a.ys);
-        else store_tiles(std::integral_constant<int, MI355Q_BF16>{}, a.y, a.ys, a.wide_stores != 0);
+        if (lines) store_lines(std::integral_constant<int, MI355Q_BF16>{}, seg_y, seg_ys);
+        else store_tiles(std::integral_constant<int, MI355Q_BF16>{}, seg_y, seg_ys, a.wide_stores != 0);
     } else if (a.y_dtype == MI355Q_F32) {
-        if (lines) store_lines(std::integral_constant<int, MI355Q_F32>{}, a.y, a.ys);
-        else store_tiles(std::integral_constant<int, MI355Q_F32>{}, a.y, a.ys, a.wide_stores != 0);
+        if (lines) store_lines(std::integral_constant<int, MI355Q_F32>{}, seg_y, seg_ys);
+        else store_tiles(std::integral_constant<int, MI355Q_F32>{}, seg_y, seg_ys, a.wide_stores != 0);
     } else {
-        if (lines) store_lines(std::integral_constant<int, MI355Q_F16>{}, a.y, a.ys);
-        else store_tiles(std::integral_constant<int, MI355Q_F16>{}, a.y, a.ys, a.wide_stores != 0);
+        if (lines) store_lines(std::integral_constant<int, MI355Q_F16>{}, seg_y, seg_ys);
+        else store_tiles(std::integral_constant<int, MI355Q_F16>{}, seg_y, seg_ys, a.wide_stores != 0);
     }
 }
 
@@ -518,7 +543,7 @@ __global__ __launch_bounds__(256, (BM == 128 ? 2 : 1)) void qgemm_wide_kernel(Wi
 template <int BM, bool SB_BF16, int GROUP, bool BLOCKS>
 mi355q_status launch_wide_tile(hipStream_t s, WideArgs a) {
     a.tiles_m = (a.m + BM - 1) / BM;
-    a.tiles_n = a.gated ? (a.n + kWideBN / 2 - 1) / (kWideBN / 2) : (a.n + kWideBN - 1) / kWideBN;
+    if (a.segments <= 1) a.tiles_n = a.gated ? (a.n + kWideBN / 2 - 1) / (kWideBN / 2) : (a.n + kWideBN - 1) / kWideBN;
     const uint32_t grid = (a.tiles_m * a.tiles_n * a.splits + 7) / 8 * 8;
     constexpr size_t lds = (size_t)kWideStages * BM * 128;
     auto kern = qgemm_wide_kernel<BM, SB_BF16, GROUP, BLOCKS, WIDE_XF16 != 0>;

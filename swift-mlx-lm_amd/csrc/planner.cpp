@@ -180,6 +180,17 @@ void plan_shared_launch_shape(const mi355q_weight* const* ws, uint32_t count, ui
         s->rows_per_workgroup = 64;
         return;
     }
+    case SharedRoute::kWide: {
+        const GemmLaunchShape g = gemm_wide_multi_shape(count, views, m);
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "qgemm_wide_q%u_g%u", bits, group);
+        s->grid[0] = g.grid;
+        s->grid[1] = 1;
+        s->block[0] = g.block;
+        s->lds_bytes = g.lds_bytes;
+        s->rows_per_workgroup = g.bn;
+        s->used_fallback = 0;
+        return;
+    }
     case SharedRoute::kMfmaPlanes: {
         const Tile16LaunchShape g = gemv_mfma_planes_shape(ctx, tiles, views[0].k, views[0].bits, staged_rows(x_dtype, m));
         std::snprintf(s->device_kernel, sizeof s->device_kernel, "gemv_mfma_planes_q%u_g%u", bits, group);

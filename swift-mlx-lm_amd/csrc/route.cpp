@@ -113,6 +113,15 @@ SharedRoute shared_route(const mi355q_context* ctx, uint32_t count, const WView*
         if (tiled) return SharedRoute::kTile16;
         if (in_place) return SharedRoute::kStafInPlace;
     }
+    // prompts: the wide-tile prefill kernel over the column tiles of all matrices, where it would take one matrix of
+    // their columns together (and the dense library is not the route: from kWideRowsBesideLibrary rows)
+    if (x_aligned && !(flags & (MI355Q_FLAG_FORCE_GENERIC | MI355Q_FLAG_FORCE_MFMA | MI355Q_FLAG_FORCE_SMALL_M | MI355Q_FLAG_PROBE_TILED))) {
+        if (flags & MI355Q_FLAG_PROBE_WIDE) {
+            if (gemm_wide_multi_eligible(count, views, x_dtype, m, xs)) return SharedRoute::kWide;
+        } else if (gemm_wide_multi_chosen(count, views, x_dtype, m, xs) && (m < kWideRowsBesideLibrary || library_ruled_out(ctx))) {
+            return SharedRoute::kWide;
+        }
+    }
     // fp32 rows that go to the bf16 kernels as bf16 rows (split_rows_chosen): split once for all projections, one
     // shared bf16 launch on those rows where they fit one, one sum per projection
     const uint32_t parts = split_rows_parts(x_dtype);
@@ -137,6 +146,7 @@ const char* shared_route_name(SharedRoute r) {
     case SharedRoute::kDotPlanes: return "shared/dot-planes";
     case SharedRoute::kTile16: return "shared/tile16";
     case SharedRoute::kStafInPlace: return "shared/staf-in-place";
+    case SharedRoute::kWide: return "shared/wide";
     case SharedRoute::kSplitRows: return "split-rows";
     case SharedRoute::kSteps: return "steps";
     case SharedRoute::kSeparate: return "separate";

@@ -7,6 +7,7 @@ relative L2 <= 1e-3 and max-abs <= 2e-2 on the fp32 output, 16-bit outputs equal
 exactly representable cases compared exactly.  The kernel is forced with the probe flag where the shape is smaller
 than what the dispatcher gives it; benchmark config 3 runs as dispatched.
 """
+import itertools
 import sys
 
 import numpy as np
@@ -285,3 +286,49 @@ def test_config3_full_size_properties_every_output(pkg, ctx, n, k):
     yb = run_qgemm(ctx, pkg, w, x, pkg.BF16, 0)
     assert np.array_equal(oracle.bf16_from_f32(yb), oracle.bf16_from_f32(y1))
     w.destroy()
+
+
+@pytest.mark.parametrize("layout_name,x_name", [("LAYOUT_PLANES", "BF16"), ("LAYOUT_STAF_BLOCKS", "BF16"), ("LAYOUT_PLANES", "F16")])
+def test_shared_launch_of_the_wide_kernel_equals_one_matrix_of_all_rows(pkg, ctx, layout_name, x_name):
+    """Two or three projections that share their activations (q+k+v, gate+up) as one launch of the wide-tile kernel: every
+    column tile belongs to one matrix.  Bit for bit the result of one matrix made of the rows of all of them (same
+    tiles, same K parts, same sums), for 128- and 256-row tiles, K in one part and in several, a ragged last matrix,
+    every output type, results whose rows are and are not 16-byte multiples; the plan record names the launch."""
+    layout, xd = getattr(pkg, layout_name), getattr(pkg, x_name)
+    sbo, sbp = (oracle.F16, pkg.F16) if layout == pkg.LAYOUT_STAF_BLOCKS else (oracle.BF16, pkg.BF16)
+    cases = [(100, (512, 256, 200), 1024, 64), (300, (768, 260), 512, 128), (700, (256, 256, 256), 2048, 64)]
+    for i, (m, ns, k, group) in enumerate(cases):
+        fmt = pkg.QuantizationFormatRegistry.format_for_mlx_quantization(4, group)
+        parts = [oracle.quantize_affine(kat.seeded_weights(7300 + 10 * i + j, n, k), 4, group, sbo) for j, n in enumerate(ns)]
+        ws = [ctx.weight_prepare_mlx(fmt, w_, s_, z_, sbp, layout) for (w_, s_, z_) in parts]
+        whole = ctx.weight_prepare_mlx(fmt, np.concatenate([p[0] for p in parts]), np.concatenate([p[1].reshape(n, -1) for p, n in zip(parts, ns)]),
+                                       np.concatenate([p[2].reshape(n, -1) for p, n in zip(parts, ns)]), sbp, layout)
+        x = act_rounded(kat.seeded_activations(7350 + i, m, k), xd, pkg)
+        xdev = ctx.upload(x.astype(np.float16).view(np.uint16) if xd == pkg.F16 else oracle.bf16_from_f32(x))
+        total = sum(ns)
+        shapes = [(0, 0)] + ([(128, 2), (256, 2)] if k >= 2048 else [])       # as chosen; K forced into two parts
+        for yd, (tile_rows, k_parts) in itertools.product((pkg.BF16, pkg.F32, pkg.F16), shapes):
+            esz = 4 if yd == pkg.F32 else 2
+            dt = np.float32 if esz == 4 else np.uint16
+            say(f"shared wide launch {layout_name} x={x_name} m={m} ns={ns} k={k} g{group} y={yd} tile {tile_rows} parts {k_parts}")
+            outs = [ctx.alloc(m * n * esz) for n in ns]
+            ref = ctx.alloc(m * total * esz)
+            pkg.Context.probe_wide_shape(tile_rows, k_parts)
+            try:
+                ctx.batched_qgemm(ws, xdev, xd, outs, yd, m, flags=pkg.FLAG_PROBE_WIDE)
+                ctx.qgemm(whole, xdev, xd, ref, yd, m, flags=pkg.FLAG_FORCE_MFMA | pkg.FLAG_PROBE_WIDE)
+            finally:
+                pkg.Context.probe_wide_shape(0, 0)
+            ctx.synchronize()
+            want = ref.download(dt, (m, total))
+            col = 0
+            for o, n in zip(outs, ns):
+                assert np.array_equal(o.download(dt, (m, n)), want[:, col:col + n]), (m, ns, k, yd, col)
+                col += n
+            for t in outs + [ref]:
+                t.free()
+        launcher, plan = pkg.probe_shared_route(fmt, layout, ns, k, xd, m, flags=pkg.FLAG_PROBE_WIDE, sb_dtype=sbp)
+        assert launcher == "shared/wide" and plan == f"qgemm_wide_q4_g{group}", (launcher, plan)
+        xdev.free(); whole.destroy()
+        for w in ws:
+            w.destroy()

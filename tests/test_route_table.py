@@ -163,6 +163,7 @@ PLAN_OF_SHARED_ROUTE = {
     "shared/dot-planes": r"^gemv_(rows|planes)_q\d_g\d+$",
     "shared/tile16": r"^gemv_tile16_q\d_g\d+$",
     "shared/staf-in-place": r"^gemv_staf_q\d_g\d+$",
+    "shared/wide": r"^qgemm_wide_q\d_g\d+$",
     "split-rows": r"^split_f32_bf16x3\+",          # the rows are split once, then the table is asked again for the bf16 rows
     "steps": r".",                                    # the shared launch in steps: the record is the first projection's
     "separate": r".",                                 # a launch per projection: the record is the first projection's own
@@ -173,6 +174,7 @@ PARITY_TEST_OF_SHARED_ROUTE = {
     "shared/dot-planes": "test_gpu_batched.py::test_batched_llama_projections",
     "shared/tile16": "test_gpu_tile16.py::test_tile16_batched_projections_one_launch",
     "shared/staf-in-place": "test_gpu_staf_gemv.py::test_in_place_batched_projections",
+    "shared/wide": "test_gpu_gemm_wide.py::test_shared_launch_of_the_wide_kernel_equals_one_matrix_of_all_rows",
     "split-rows": "test_gpu_split_rows.py::test_batched_projections_other_activation_types",
     "steps": "test_gpu_batched.py::test_batched_equals_separate_launches_on_other_routes",
     "separate": "test_gpu_batched.py::test_batched_equals_separate_launches_on_other_routes",
@@ -213,6 +215,11 @@ def test_shared_launches_plan_what_the_launcher_runs_in_every_cell():
     assert r(q4, pkg.LAYOUT_TILE16, (14336, 14336), 4096, pkg.BF16, 16) == "shared/tile16"
     assert r(q4, pkg.LAYOUT_STAF_BLOCKS, (14336, 14336), 4096, pkg.BF16, 1) == "shared/staf-in-place"
     assert r(q4, pkg.LAYOUT_STAF_BLOCKS, (14336, 14336), 4096, pkg.BF16, 8) == "shared/stream"
+    # prompts: q+k+v and gate+up on the wide-tile kernel as one launch, up to the rows where the dense library takes over
+    assert r(q4, pkg.LAYOUT_PLANES, (4096, 1024, 1024), 4096, pkg.BF16, 512) == "shared/wide"
+    assert r(q4, pkg.LAYOUT_PLANES, (14336, 14336), 4096, pkg.BF16, 2048) == "shared/wide"
+    assert r(q4, pkg.LAYOUT_STAF_BLOCKS, (4096, 1024, 1024), 4096, pkg.F16, 512) == "shared/wide"
+    assert r(q4, pkg.LAYOUT_PLANES, (4096, 1024, 1024), 4096, pkg.F32, 512) == "separate"
 
 
 def test_every_shared_route_has_a_gpu_parity_test():
