@@ -342,7 +342,10 @@ MI355Q_API mi355q_status mi355q_gated_activation_apply(mi355q_context* ctx, void
  * rounded to y_dtype before the activation, as the reference's elementwise kernel reads them from buffers of that
  * type, so the result is that of mi355q_batched_qgemm followed by mi355q_gated_activation_apply up to the order of
  * the fp32 sums.  One activation row on split planes runs as ONE launch (a wavefront owns a gate row and the up row
- * of the same index); other shapes run the projections into the context's scratch and then the elementwise kernel. */
+ * of the same index), and so do 17 to 96 rows on the streamed-weight kernel (a workgroup's two row blocks are the same
+ * rows of the two matrices) and, on 4-bit matrices, prompts from 97 rows on the wide-tile kernel (a wavefront's two
+ * column fragments are), the activation in their epilogues; other shapes run the projections into the context's
+ * scratch and then the elementwise kernel. */
 MI355Q_API mi355q_status mi355q_gated_qgemm(mi355q_context* ctx, void* stream, const mi355q_weight* w_gate,
                                             const mi355q_weight* w_up, const void* x_dev, mi355q_dtype x_dtype,
                                             void* y_dev, mi355q_dtype y_dtype, uint32_t m, uint32_t x_row_stride,
@@ -350,7 +353,9 @@ MI355Q_API mi355q_status mi355q_gated_qgemm(mi355q_context* ctx, void* stream, c
                                             uint32_t flags);
 
 /* batched_gemm_q4_g64_{2,3} (:166-338; bindings MC/Compiler/MetalPrefillStepBuilder.swift:928-955):
- * 2 or 3 projections sharing one input (gate+up, q+k+v) in one launch.  All weights must share
+ * 2 or 3 projections sharing one input (gate+up, q+k+v) in one launch: at decode and small batches on the decode
+ * kernels, at 17 to 96 rows on the streamed-weight kernel, from 97 rows (4-bit matrices whose widths but the last
+ * are multiples of 256) on the wide-tile prefill kernel; a launch per projection elsewhere.  All weights must share
  * K, scheme and layout.  Outputs are separate [M, N_i] buffers with row stride N_i. */
 MI355Q_API mi355q_status mi355q_batched_qgemm(mi355q_context* ctx, void* stream, uint32_t count,
                                               const mi355q_weight* const* weights,
