@@ -657,6 +657,33 @@ def main():
             for b in (xg, yg, gb, ub):
                 b.free()
         next_rows["gated MLP projection 4096 -> 2 x 14336 q4 g64 + swiglu, bf16"] = gated
+        # prompts: q+k+v (4096 -> 4096 + 1024 + 1024) through mi355q_batched_qgemm as dispatched, beside a call per
+        # projection; the table names what the projections run as together
+        shared = {}
+        for mm in (128, 512, 2048):
+            xq = ctx.upload(oracle.bf16_from_f32(kat.seeded_activations(950 + mm, mm, 4096)))
+            outs = [ctx.alloc(mm * n_ * 2) for n_ in (4096, 1024, 1024)]
+            nl = min(len(layers), 4)
+            qkv = lambda i: [layers[i % nl][t] for t in ("q", "k", "v")]
+            one = lambda i: ctx.batched_qgemm(qkv(i), xq, pkg.BF16, outs, pkg.BF16, mm, 0, 0, stream)
+            def apart(i):
+                for w_, o_ in zip(qkv(i), outs):
+                    ctx.qgemm(w_, xq, pkg.BF16, o_, pkg.BF16, mm, 0, 0, 0, stream)
+            for fn in (one, apart):
+                for i in range(4):
+                    fn(i)
+            ctx.synchronize(stream)
+            samples = ([], [])
+            for _ in range(7):
+                samples[0].append(time_region(ctx, one, 16, stream))
+                samples[1].append(time_region(ctx, apart, 16, stream))
+            t_one, t_apart = (sorted(v)[len(v) // 2] for v in samples)
+            route, kernel = pkg.probe_shared_route(fmt, pkg.LAYOUT_PLANES, (4096, 1024, 1024), 4096, pkg.BF16, mm)
+            shared[f"M={mm}"] = {"us": round(t_one * 1e3, 2), "a_call_per_projection_us": round(t_apart * 1e3, 2),
+                                 "route": route, "kernel": kernel}
+            for b in [xq] + outs:
+                b.free()
+        next_rows["q+k+v 4096 -> 4096 + 1024 + 1024 q4 g64 at prompts, bf16"] = shared
         # container: one q4 g64 gate tensor written, opened, validated, uploaded as one device buffer, wrapped with no copy
         words, s_, z_ = host["gate"]
         blocks = pkg.repack_mlx_to_staf(fmt, words, s_, z_, pkg.BF16)
