@@ -394,7 +394,7 @@ void gemm_wide_force_shape(uint32_t bm, uint32_t splits);      // A/B runs (mi35
 // `chosen`: from the rows where the streamed-weight kernel ends (measured against a launch per projection).
 bool gemm_wide_multi_eligible(uint32_t count, const WView* w, int x_dtype, uint32_t m, uint32_t x_stride);
 bool gemm_wide_multi_chosen(uint32_t count, const WView* w, int x_dtype, uint32_t m, uint32_t x_stride);
-GemmLaunchShape gemm_wide_multi_shape(uint32_t count, const WView* w, uint32_t m);
+GemmLaunchShape gemm_wide_multi_shape(uint32_t count, const WView* w, uint32_t m, int x_dtype);
 mi355q_status launch_qgemm_wide_multi(hipStream_t s, mi355q_context* ctx, uint32_t count, const WView* w, const void* x,
                                       int x_dtype, void* const* y, const uint32_t* y_strides, int y_dtype, uint32_t m,
                                       uint32_t x_stride);

@@ -275,7 +275,7 @@ __global__ __launch_bounds__(256) void wide_reduce_multi_kernel(WideSumArgs a) {
 }  // namespace
 
 bool gemm_wide_multi_eligible(uint32_t count, const WView* w, int x_dtype, uint32_t m, uint32_t x_stride) {
-    if (count < 2 || count > 3 || (x_dtype != MI355Q_BF16 && x_dtype != MI355Q_F16)) return false;
+    if (count < 2 || count > 3) return false;
     uint64_t total = 0;
     for (uint32_t i = 0; i < count; i++) {
         if (!gemm_wide_eligible(w[i], x_dtype, m, x_stride)) return false;
@@ -289,10 +289,10 @@ bool gemm_wide_multi_eligible(uint32_t count, const WView* w, int x_dtype, uint3
     return total < (1ull << 31);
 }
 
-GemmLaunchShape gemm_wide_multi_shape(uint32_t count, const WView* w, uint32_t m) {
+GemmLaunchShape gemm_wide_multi_shape(uint32_t count, const WView* w, uint32_t m, int x_dtype) {
     uint32_t total = 0;
     for (uint32_t i = 0; i < count; i++) total += w[i].n;
-    return gemm_wide_shape(m, total, w[0].k);
+    return gemm_wide_shape(m, total, gemm_wide_k(w[0].k, x_dtype));
 }
 
 // From the rows where the streamed-weight kernel ends, whatever the size: against a launch per projection (each with
@@ -310,7 +310,18 @@ mi355q_status launch_qgemm_wide_multi(hipStream_t s, mi355q_context* ctx, uint32
     if (!gemm_wide_multi_eligible(count, w, x_dtype, m, x_stride))
         return fail(MI355Q_ERR_KERNEL_NOT_FOUND, "the wide-tile MFMA GEMM does not take these weights as one launch");
     if ((uintptr_t)x % 16) return fail(MI355Q_ERR_INVALID_ARGUMENT, "activation pointer must be 16-byte aligned");
-    const GemmLaunchShape g = gemm_wide_multi_shape(count, w, m);
+    const GemmLaunchShape g = gemm_wide_multi_shape(count, w, m, x_dtype);
+    // fp32 activations: every row once as [hi | lo] bf16 halves for all the matrices (as launch_qgemm_wide does for one)
+    const uint32_t k_walk = gemm_wide_k(w[0].k, x_dtype);
+    const void* xk = x;
+    uint32_t xk_stride = x_stride;
+    if (x_dtype == MI355Q_F32) {
+        if (mi355q_status st = ensure_split_buffer(ctx, ((size_t)m * k_walk * 2 + 255) & ~(size_t)255)) return st;
+        uint16_t* const hi = (uint16_t*)ctx->split_buffer;
+        if (mi355q_status st = launch_split_f32_bf16x2(s, (const float*)x, m, w[0].k, x_stride, hi, hi + w[0].k, k_walk)) return st;
+        xk = hi;
+        xk_stride = k_walk;
+    }
     WideArgs a{};
     const bool blocks = w[0].layout == MI355Q_LAYOUT_STAF_BLOCKS;
     const size_t esz = y_dtype == MI355Q_F32 ? 4 : 2;
@@ -339,8 +350,8 @@ mi355q_status launch_qgemm_wide_multi(hipStream_t s, mi355q_context* ctx, uint32
     a.tiles_n = tiles;
     a.n_total = cols;
     a.row_bytes = w[0].blocks_per_row * w[0].bytes_per_block;
-    a.x = (const uint16_t*)x;
-    a.m = m; a.k = w[0].k; a.xs = x_stride;
+    a.x = (const uint16_t*)xk;
+    a.m = m; a.k = k_walk; a.xs = xk_stride;
     a.w_fours = w[0].k / 256;
     a.code_stride = w[0].code_stride; a.sz_stride = w[0].sz_stride;
     a.y_dtype = (uint32_t)y_dtype;

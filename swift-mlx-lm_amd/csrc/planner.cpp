@@ -181,8 +181,9 @@ void plan_shared_launch_shape(const mi355q_weight* const* ws, uint32_t count, ui
         return;
     }
     case SharedRoute::kWide: {
-        const GemmLaunchShape g = gemm_wide_multi_shape(count, views, m);
-        std::snprintf(s->device_kernel, sizeof s->device_kernel, "qgemm_wide_q%u_g%u", bits, group);
+        const GemmLaunchShape g = gemm_wide_multi_shape(count, views, m, x_dtype);
+        std::snprintf(s->device_kernel, sizeof s->device_kernel, "%sqgemm_wide_q%u_g%u", x_dtype == MI355Q_F32 ? "split_f32_bf16x2+" : "",
+                      bits, group);
         s->grid[0] = g.grid;
         s->grid[1] = 1;
         s->block[0] = g.block;

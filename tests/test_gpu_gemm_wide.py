@@ -288,12 +288,14 @@ def test_config3_full_size_properties_every_output(pkg, ctx, n, k):
     w.destroy()
 
 
-@pytest.mark.parametrize("layout_name,x_name", [("LAYOUT_PLANES", "BF16"), ("LAYOUT_STAF_BLOCKS", "BF16"), ("LAYOUT_PLANES", "F16")])
+@pytest.mark.parametrize("layout_name,x_name", [("LAYOUT_PLANES", "BF16"), ("LAYOUT_STAF_BLOCKS", "BF16"), ("LAYOUT_PLANES", "F16"),
+                                                ("LAYOUT_PLANES", "F32")])
 def test_shared_launch_of_the_wide_kernel_equals_one_matrix_of_all_rows(pkg, ctx, layout_name, x_name):
     """Two or three projections that share their activations (q+k+v, gate+up) as one launch of the wide-tile kernel: every
     column tile belongs to one matrix.  Bit for bit the result of one matrix made of the rows of all of them (same
     tiles, same K parts, same sums), for 128- and 256-row tiles, K in one part and in several, a ragged last matrix,
-    every output type, results whose rows are and are not 16-byte multiples; the plan record names the launch."""
+    every output type, results whose rows are and are not 16-byte multiples, fp32 activations (split once into bf16
+    halves for all the matrices); the plan record names the launch."""
     layout, xd = getattr(pkg, layout_name), getattr(pkg, x_name)
     sbo, sbp = (oracle.F16, pkg.F16) if layout == pkg.LAYOUT_STAF_BLOCKS else (oracle.BF16, pkg.BF16)
     cases = [(100, (512, 256, 200), 1024, 64), (300, (768, 260), 512, 128), (700, (256, 256, 256), 2048, 64)]
@@ -304,7 +306,8 @@ def test_shared_launch_of_the_wide_kernel_equals_one_matrix_of_all_rows(pkg, ctx
         whole = ctx.weight_prepare_mlx(fmt, np.concatenate([p[0] for p in parts]), np.concatenate([p[1].reshape(n, -1) for p, n in zip(parts, ns)]),
                                        np.concatenate([p[2].reshape(n, -1) for p, n in zip(parts, ns)]), sbp, layout)
         x = act_rounded(kat.seeded_activations(7350 + i, m, k), xd, pkg)
-        xdev = ctx.upload(x.astype(np.float16).view(np.uint16) if xd == pkg.F16 else oracle.bf16_from_f32(x))
+        xdev = ctx.upload(x.astype(np.float16).view(np.uint16) if xd == pkg.F16 else x.astype(np.float32) if xd == pkg.F32
+                          else oracle.bf16_from_f32(x))
         total = sum(ns)
         shapes = [(0, 0)] + ([(128, 2), (256, 2)] if k >= 2048 else [])       # as chosen; K forced into two parts
         for yd, (tile_rows, k_parts) in itertools.product((pkg.BF16, pkg.F32, pkg.F16), shapes):
@@ -328,7 +331,7 @@ def test_shared_launch_of_the_wide_kernel_equals_one_matrix_of_all_rows(pkg, ctx
             for t in outs + [ref]:
                 t.free()
         launcher, plan = pkg.probe_shared_route(fmt, layout, ns, k, xd, m, flags=pkg.FLAG_PROBE_WIDE, sb_dtype=sbp)
-        assert launcher == "shared/wide" and plan == f"qgemm_wide_q4_g{group}", (launcher, plan)
+        assert launcher == "shared/wide" and plan == ("split_f32_bf16x2+" if xd == pkg.F32 else "") + f"qgemm_wide_q4_g{group}", (launcher, plan)
         xdev.free(); whole.destroy()
         for w in ws:
             w.destroy()

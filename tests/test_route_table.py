@@ -163,7 +163,7 @@ PLAN_OF_SHARED_ROUTE = {
     "shared/dot-planes": r"^gemv_(rows|planes)_q\d_g\d+$",
     "shared/tile16": r"^gemv_tile16_q\d_g\d+$",
     "shared/staf-in-place": r"^gemv_staf_q\d_g\d+$",
-    "shared/wide": r"^qgemm_wide_q\d_g\d+$",
+    "shared/wide": r"^(split_f32_bf16x2\+)?qgemm_wide_q\d_g\d+$",
     "split-rows": r"^split_f32_bf16x3\+",          # the rows are split once, then the table is asked again for the bf16 rows
     "steps": r".",                                    # the shared launch in steps: the record is the first projection's
     "separate": r".",                                 # a launch per projection: the record is the first projection's own
@@ -219,7 +219,7 @@ def test_shared_launches_plan_what_the_launcher_runs_in_every_cell():
     assert r(q4, pkg.LAYOUT_PLANES, (4096, 1024, 1024), 4096, pkg.BF16, 512) == "shared/wide"
     assert r(q4, pkg.LAYOUT_PLANES, (14336, 14336), 4096, pkg.BF16, 2048) == "shared/wide"
     assert r(q4, pkg.LAYOUT_STAF_BLOCKS, (4096, 1024, 1024), 4096, pkg.F16, 512) == "shared/wide"
-    assert r(q4, pkg.LAYOUT_PLANES, (4096, 1024, 1024), 4096, pkg.F32, 512) == "separate"
+    assert pkg.probe_shared_route(q4, pkg.LAYOUT_PLANES, (4096, 1024, 1024), 4096, pkg.F32, 512) == ("shared/wide", "split_f32_bf16x2+qgemm_wide_q4_g64")
 
 
 def test_every_shared_route_has_a_gpu_parity_test():
